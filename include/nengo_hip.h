@@ -1,0 +1,168 @@
+/*
+ * nengo_hip.h -- C ABI of the MI355X (gfx950) timestep kernels.
+ *
+ * One simulator timestep of a Nengo model is a fixed sequence of "plans"
+ * (ragged gather-GEMV, neuron update, synapse filter, copies, probes ...).
+ * In the reference every plan is an OpenCL kernel generated from a Mako
+ * template and bound with `kernel.set_args(...)` inside a `plan_*` function;
+ * the entry points below are what those `plan_*` functions bind instead.
+ *
+ * Conventions (all entry points):
+ *   - `stream` is a `hipStream_t` passed as `void*` (NULL = default stream).
+ *   - every `*_data` / `X` / `Y` pointer is a DEVICE pointer to a flat float32
+ *     (or int32 where stated) buffer; all offsets inside the int32 work lists
+ *     are ELEMENT offsets into those buffers, exactly like the `*_starts`
+ *     arrays the reference kernels receive (nengo_ocl/raggedarray.py:31-236,
+ *     nengo_ocl/clraggedarray.py:65-184).
+ *   - work lists (`items`, `dots`, `tasks`, `blocks`, `desc`) are DEVICE int32
+ *     tables built once at plan time and owned by the caller; the library
+ *     only reads them during the launch.  Float scalars ride in them as raw
+ *     IEEE-754 bits.
+ *   - nothing here allocates, frees or synchronises (except where stated):
+ *     kernels are enqueued on `stream` and the call returns.
+ *   - return value: 0 on success, otherwise a `hipError_t` (or a negative
+ *     NHIP_E_* code for argument errors); `nhip_error_string` describes both.
+ *     No entry point throws or aborts.
+ *   - one stream per simulator; entry points are re-entrant but the caller
+ *     serialises work that touches the same buffers.
+ */
+#ifndef NENGO_HIP_H
+#define NENGO_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NHIP_ABI_VERSION 1
+
+#define NHIP_E_BADARG (-1)   /* null pointer / negative count / unknown mode   */
+#define NHIP_E_BADCLASS (-2) /* GEMV class (lanes-per-row, vector width) unknown */
+
+/* ---- library ---------------------------------------------------------- */
+int nhip_abi_version(void);
+const char *nhip_error_string(int err);
+/* device facts of the current device: compute units, wavefront size, LDS bytes
+ * per work-group, gcn arch name (copied, NUL-terminated, into `name`). */
+int nhip_device_info(int *n_cu, int *wave_size, int *lds_bytes, char *name, int name_len);
+
+/* ---- ragged gather-GEMV ------------------------------------------------
+ * For every output item b:
+ *     Y[b] = beta_b * Yin[b] + gamma_b + alpha_b * sum_d  A[b,d] @ X[b,d]
+ * replaces: clra_gemv.py `plan_block_gemv` / `block_impl` (:861-1175, kernels
+ * `fn` :1010-1060 and `reduce` :1122-1155), and the `ref_impl` /
+ * `reduce_impl` / `many_dots_impl` family (:264-858).  One launch computes
+ * the final Y directly (no partial-sum buffer, no second kernel).
+ *
+ *   items : int32[n_items][8]  {y_start, y_stride0, yin_start, yin_stride0,
+ *                               dot_begin, n_dots, M, 0}
+ *   coefs : float[n_items][4]  {alpha, beta, gamma, 0}
+ *   dots  : int32[n_dots][8]   {a_start, a_stride0, N, x_start, x_stride0,0,0,0}
+ *                               (A rows are contiguous: a_stride1 == 1)
+ *   tasks : int32[n_tasks][4]  {item, row0, n_rows, 0}
+ *
+ * `flavor` 0 = one work-group (256 threads) per task, X staged in LDS and
+ * shared by the group's four waves; rows per task <= nhip_gemv_rows_per_task.
+ * `flavor` 1 = one wave per task (four tasks per group), X read through L1;
+ * for many tiny items.  `lpr` = lanes cooperating on one row (1,2,...,64, or
+ * 256 for flavor 0); `vec` = 4 (16-byte loads; needs a_start % 4 == 0 and
+ * a_stride0 % 4 == 0 for every dot of the launch) or 1.  The host validates
+ * these preconditions; the kernel trusts them. */
+int nhip_gemv(void *stream, int flavor, int lpr, int vec, const int *items,
+              const float *coefs, const int *dots, const int *tasks, int n_tasks,
+              const float *A, const float *X, const float *Yin, float *Y);
+/* rows one task of the given class covers at most (0 if the class is unknown) */
+int nhip_gemv_rows_per_task(int flavor, int lpr, int vec);
+
+/* ---- neurons -----------------------------------------------------------
+ * LIF with refractory state and spike-time interpolation.
+ * replaces: clra_nonlinearities.py `plan_lif` (:1028-1146, non-adaptive,
+ * fastlif=False) through `_plan_template` (:1286-1483).
+ *   desc : int32[n_blocks][12] {j_start, v_start, w_start, s_start, count,
+ *                               tau, ref, amp, pflags, 0, 0, 0}
+ * `tau/ref/amp` are float bits, or (if bit 0/1/2 of pflags is set) element
+ * offsets into `TAU/REF/AMP` for per-neuron parameter vectors. */
+int nhip_lif(void *stream, const int *desc, int n_blocks, double dt, int upsample,
+             const float *J, float *V, float *W, float *S, const float *TAU,
+             const float *REF, const float *AMP);
+/* LIF rate curve.  replaces: `plan_lif_rate` (:1149-1197).
+ *   desc : int32[n_blocks][8] {j_start, r_start, count, tau, ref, amp, pflags, 0} */
+int nhip_lif_rate(void *stream, const int *desc, int n_blocks, const float *J, float *R,
+                  const float *TAU, const float *REF, const float *AMP);
+
+/* ---- synapses ----------------------------------------------------------
+ * Direct-form linear filter step  y <- sum_p b[p] x[n-p] - sum_p a[p] y[n-1-p]
+ * with ring buffers for orders > 1; fast paths for (na,nb) = (0,1) and (1,1).
+ * replaces: `plan_linearfilter` (:577-803) -- both its `linearfilter` kernel
+ * and the `linearfilter_inc` position kernel (positions advance in the same
+ * launch, after a block-wide barrier).
+ *   desc : int32[n_blocks][16] {x_start, x_stride0, x_stride1, y_start,
+ *          y_stride0, y_stride1, shape1, offset, count, na, nb, a_start,
+ *          b_start, xbuf_start, ybuf_start, size}
+ *   pos  : int32[n_blocks][2]  {xbuf_pos, ybuf_pos}   (read and advanced) */
+int nhip_linearfilter(void *stream, const int *desc, int *pos, int n_blocks, const float *X,
+                      float *Y, const float *A, const float *B, float *Xbuf, float *Ybuf);
+
+/* ---- element-wise ------------------------------------------------------ */
+/* Y (=|+=) alpha * A * X with scalar/row/column broadcasting, or outer product.
+ * replaces: `plan_elementwise_inc` (:414-574).
+ *   desc : int32[n_blocks][16] {a_start, a_shape0, a_shape1, a_stride0, x_start,
+ *          x_shape0, x_shape1, x_stride0, y_start, y_shape1, y_stride0, offset,
+ *          count, alpha_bits, flags(bit0 outer, bit1 inc), 0} */
+int nhip_elementwise_inc(void *stream, const int *desc, int n_blocks, const float *A,
+                         const float *X, float *Y);
+/* 2-D strided Y (=|+=) X.  replaces: `plan_copy` (:217-304).
+ *   desc : int32[n_blocks][8] {x_start, y_start, shape1, x_stride0, y_stride0,
+ *                              offset, count, inc} */
+int nhip_copy(void *stream, const int *desc, int n_blocks, const float *X, float *Y);
+/* gather/scatter  Y[yi[k]*ys] (=|+=) X[xi[k]*xs].  replaces: `plan_slicedcopy` (:307-411).
+ *   desc : int32[n_blocks][8] {x_start, x_stride0, y_start, y_stride0, xi_start,
+ *                              yi_start, count, inc} */
+int nhip_slicedcopy(void *stream, const int *desc, int n_blocks, const float *X, float *Y,
+                    const int *XI, const int *YI);
+/* constant fill.  replaces: `plan_reset` (:147-214).
+ *   blocks : int32[n_blocks][4] {start, count, value_bits, 0} */
+int nhip_reset(void *stream, const int *blocks, int n_blocks, float *Y);
+/* step += 1; time = dt * step (dt in double, rounded once).
+ * replaces: `plan_timeupdate` (:113-144). */
+int nhip_timeupdate(void *stream, float *step_data, int step_start, float *time_data,
+                    int time_start, double dt);
+
+/* ---- inputs and outputs ------------------------------------------------ */
+/* table playback  y = S[row(step) , :].  replaces: `plan_presentinput` (:1678-1759).
+ *   desc : int32[n][8] {y_start, m, t_start, s_start, nt, pt_bits, has_pt, 0} */
+int nhip_presentinput(void *stream, const int *desc, int n, float dt, float *Y, const float *T,
+                      const float *S);
+/* y[k] = f(x[k]) for a fixed table of unary functions (opcode: 0 identity, 1 sin,
+ * 2 cos, 3 tanh, 4 exp, 5 square).  replaces the generated `direct` kernel of
+ * `plan_direct` (:954-1025) for the expressions the function translator
+ * reduces to one of these.
+ *   desc : int32[n][4] {x_start, y_start, count, 0} */
+int nhip_direct_unary(void *stream, int opcode, const int *desc, int n, const float *X, float *Y);
+/* probe gather with per-probe float countdown.  replaces: `plan_probes` (:806-951).
+ *   desc : int32[n][8] {x_start, shape0, shape1, stride0, stride1, y_start, 0, 0} */
+int nhip_probes(void *stream, const int *desc, int n, float *countdowns, int *bufpositions,
+                const float *periods, const float *X, float *Y);
+/* fill an int32 device array (used to zero probe buffer positions without a
+ * memset node, so that it may also be recorded into a graph) */
+int nhip_fill_i32(void *stream, int *dst, int n, int value);
+
+/* ---- executor ----------------------------------------------------------
+ * replaces the Python launch loop of `Plans.enqueue_n_times` (plan.py:137-149):
+ * the plan sequence of one (or several) timesteps is recorded once from the
+ * stream into a graph and replayed. */
+int nhip_capture_begin(void *stream);
+int nhip_capture_end(void *stream, void **graph_exec_out);
+int nhip_graph_launch(void *graph_exec, void *stream, int n_times);
+int nhip_graph_destroy(void *graph_exec);
+int nhip_stream_sync(void *stream);
+
+/* events on `stream` (for per-plan and whole-run timing) */
+int nhip_event_create(void **event_out);
+int nhip_event_record(void *event, void *stream);
+int nhip_event_elapsed_ms(void *start, void *stop, float *ms_out); /* syncs on `stop` */
+int nhip_event_destroy(void *event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NENGO_HIP_H */

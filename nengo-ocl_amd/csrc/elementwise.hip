@@ -1,0 +1,377 @@
+// Streaming kernels of the timestep: reset, copy, sliced copy, element-wise
+// increment / outer product, linear-filter step, time update, table playback,
+// unary function nodes and probe gather.  All of them are one pass over
+// float32 data described by int32 block work lists: a "block" is a run of at
+// most a few thousand consecutive logical elements of one ragged item, handled
+// by one 256-thread group with a strided loop (consecutive threads touch
+// consecutive elements, so accesses coalesce whenever the item is contiguous).
+#include "nhip_common.h"
+
+namespace {
+
+// ---------------------------------------------------------------- reset
+// clra_nonlinearities.py:154-172 fills 16-element chunks; here a block is up to
+// 4096 elements of one contiguous item.
+__global__ __launch_bounds__(NHIP_WG) void reset_kernel(const int4* __restrict__ blocks,
+                                                        float* __restrict__ Y) {
+    const int4 b = blocks[blockIdx.x];  // {start, count, value_bits, 0}
+    const float v = nhip_bits(b.z);
+    float* y = Y + b.x;
+    for (int i = threadIdx.x; i < b.y; i += NHIP_WG) y[i] = v;
+}
+
+// ---------------------------------------------------------------- copy
+// 2-D strided Y (=|+=) X (clra_nonlinearities.py:225-262).
+struct CopyDesc { int x_start, y_start, shape1, x_stride0, y_stride0, offset, count, inc; };
+
+__global__ __launch_bounds__(NHIP_WG) void copy_kernel(const CopyDesc* __restrict__ desc,
+                                                       const float* X, float* Y) {
+    const CopyDesc d = desc[blockIdx.x];
+    const float* x = X + d.x_start;
+    float* y = Y + d.y_start;
+    const bool flat = (d.x_stride0 == d.shape1) && (d.y_stride0 == d.shape1);
+    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+        const int ij = d.offset + k;
+        size_t xo, yo;
+        if (flat) {
+            xo = yo = (size_t)ij;
+        } else {
+            const int i = ij / d.shape1, j = ij - i * d.shape1;
+            xo = (size_t)i * d.x_stride0 + j;
+            yo = (size_t)i * d.y_stride0 + j;
+        }
+        if (d.inc) y[yo] += x[xo];
+        else y[yo] = x[xo];
+    }
+}
+
+// ---------------------------------------------------------------- sliced copy
+// Y[yi[k]*ys] (=|+=) X[xi[k]*xs] (clra_nonlinearities.py:321-364); indices are
+// int32 and unique per item, so the scatter needs no atomics.
+struct SlicedDesc { int x_start, x_stride0, y_start, y_stride0, xi_start, yi_start, count, inc; };
+
+__global__ __launch_bounds__(NHIP_WG) void slicedcopy_kernel(const SlicedDesc* __restrict__ desc,
+                                                             const float* X, float* Y,
+                                                             const int* __restrict__ XI,
+                                                             const int* __restrict__ YI) {
+    const SlicedDesc d = desc[blockIdx.x];
+    const float* x = X + d.x_start;
+    float* y = Y + d.y_start;
+    const int* xi = XI + d.xi_start;
+    const int* yi = YI + d.yi_start;
+    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+        const float v = x[(size_t)xi[k] * d.x_stride0];
+        float* dst = y + (size_t)yi[k] * d.y_stride0;
+        if (d.inc) *dst += v;
+        else *dst = v;
+    }
+}
+
+// ---------------------------------------------------------------- elementwise inc
+// Y (=|+=) (alpha * A) * X with broadcasting, or Y[i,j] = alpha*A[i]*X[j]
+// (clra_nonlinearities.py:449-525; product order (alpha*a)*x as written there).
+struct EwDesc {
+    int a_start, a_shape0, a_shape1, a_stride0;
+    int x_start, x_shape0, x_shape1, x_stride0;
+    int y_start, y_shape1, y_stride0, offset;
+    int count, alpha_bits, flags, pad;
+};
+
+__device__ __forceinline__ float ew_element(const float* data, int shape0, int shape1,
+                                            int stride0, int i, int j) {
+    if (shape0 == 1 && shape1 == 1) return data[0];
+    if (shape0 == 1) return data[j];
+    if (shape1 == 1) return data[(size_t)i * stride0];
+    return data[(size_t)i * stride0 + j];
+}
+
+__global__ __launch_bounds__(NHIP_WG) void elementwise_inc_kernel(const EwDesc* __restrict__ desc,
+                                                                  const float* A, const float* X,
+                                                                  float* Y) {
+    const EwDesc d = desc[blockIdx.x];
+    const float* a = A + d.a_start;
+    const float* x = X + d.x_start;
+    float* y = Y + d.y_start;
+    const float alpha = nhip_bits(d.alpha_bits);
+    const bool outer = d.flags & 1, inc = d.flags & 2;
+    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+        const int ij = d.offset + k;
+        const int i = ij / d.y_shape1, j = ij - i * d.y_shape1;
+        float aa, xx;
+        if (outer) {
+            aa = ew_element(a, d.a_shape0, 1, d.a_stride0, i, 0);
+            xx = ew_element(x, d.x_shape0, 1, d.x_stride0, j, 0);
+        } else {
+            aa = ew_element(a, d.a_shape0, d.a_shape1, d.a_stride0, i, j);
+            xx = ew_element(x, d.x_shape0, d.x_shape1, d.x_stride0, i, j);
+        }
+        // two rounded multiplies then (for inc) one rounded add, never contracted,
+        // so the result is bit-identical to the float32 host restatement
+        const float prod = __fmul_rn(__fmul_rn(alpha, aa), xx);
+        float* dst = y + (size_t)i * d.y_stride0 + j;
+        if (inc) *dst = __fadd_rn(*dst, prod);
+        else *dst = prod;
+    }
+}
+
+// ---------------------------------------------------------------- linear filter
+// clra_nonlinearities.py:604-711.  Ring buffers: xbuf[(ix+p)%nb] holds x[n-p],
+// ybuf[(iy+p)%na] holds y[n-1-p] (p >= 1); positions step backwards once per call.
+struct LfDesc {
+    int x_start, x_stride0, x_stride1, y_start;
+    int y_stride0, y_stride1, shape1, offset;
+    int count, na, nb, a_start;
+    int b_start, xbuf_start, ybuf_start, size;
+};
+
+__global__ __launch_bounds__(NHIP_WG) void linearfilter_kernel(const LfDesc* __restrict__ desc,
+                                                               int2* pos, const float* X, float* Y,
+                                                               const float* __restrict__ A,
+                                                               const float* __restrict__ B,
+                                                               float* Xbuf, float* Ybuf) {
+    const LfDesc d = desc[blockIdx.x];
+    const float* a = A + d.a_start;
+    const float* b = B + d.b_start;
+    const int na = d.na, nb = d.nb;
+    const bool general = !(nb == 1 && na <= 1);
+    int ix = 0, iy = 0;
+    if (general) {
+        const int2 p = pos[blockIdx.x];
+        ix = p.x;
+        iy = p.y;
+    }
+    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+        const int ij = d.offset + k;
+        const int i = ij / d.shape1, j = ij - i * d.shape1;
+        const size_t xij = (size_t)d.x_start + (size_t)i * d.x_stride0 + (size_t)j * d.x_stride1;
+        const size_t yij = (size_t)d.y_start + (size_t)i * d.y_stride0 + (size_t)j * d.y_stride1;
+        if (!general) {
+            // y = b0*x           (na == 0)
+            // y = b0*x - a0*y    (na == 1): rounded products, rounded subtract
+            const float bx = __fmul_rn(b[0], X[xij]);
+            Y[yij] = (na == 0) ? bx : __fsub_rn(bx, __fmul_rn(a[0], Y[yij]));
+        } else {
+            float* xbuf = Xbuf + d.xbuf_start;
+            float* ybuf = Ybuf + d.ybuf_start;
+            const int iy1 = (iy > 0) ? iy - 1 : na - 1;
+            float yi = __fmul_rn(b[0], X[xij]);
+            if (nb > 1) {
+                xbuf[(size_t)ix * d.size + ij] = X[xij];
+                for (int p = 1; p < nb; ++p)
+                    yi = __fadd_rn(yi, __fmul_rn(b[p], xbuf[(size_t)((ix + p) % nb) * d.size + ij]));
+            }
+            if (na > 0) {
+                yi = __fsub_rn(yi, __fmul_rn(a[0], Y[yij]));
+                if (na > 1) {
+                    for (int p = 1; p < na; ++p)
+                        yi = __fsub_rn(yi, __fmul_rn(a[p], ybuf[(size_t)((iy + p) % na) * d.size + ij]));
+                    ybuf[(size_t)iy1 * d.size + ij] = yi;
+                }
+            }
+            Y[yij] = yi;
+        }
+    }
+    if (general) {
+        // every thread has read its position before anyone moves it
+        __syncthreads();
+        if (threadIdx.x == 0)
+            pos[blockIdx.x] = make_int2((ix > 0) ? ix - 1 : nb - 1, (iy > 0) ? iy - 1 : na - 1);
+    }
+}
+
+// ---------------------------------------------------------------- time update
+// clra_nonlinearities.py:119-133: the step counter is a float32 signal;
+// time = (float)(dt * (double)step) with dt a double literal.
+__global__ void timeupdate_kernel(float* step, float* time, double dt) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const float s = step[0] + 1.0f;
+        step[0] = s;
+        time[0] = (float)(dt * (double)s);
+    }
+}
+
+// ---------------------------------------------------------------- table playback
+// clra_nonlinearities.py:1694-1730: row index from the float32 step counter.
+struct PiDesc { int y_start, m, t_start, s_start, nt, pt_bits, has_pt, pad; };
+
+__global__ __launch_bounds__(NHIP_WG) void presentinput_kernel(const PiDesc* __restrict__ desc,
+                                                               float dt, float* Y, const float* T,
+                                                               const float* __restrict__ S) {
+    const PiDesc d = desc[blockIdx.x];
+    const int it = (int)T[d.t_start];
+    int ti;
+    if (d.has_pt) {
+        const float pt = nhip_bits(d.pt_bits);
+        ti = (int)(__fmul_rn((float)it - 0.5f, __fdiv_rn(dt, pt))) % d.nt;
+    } else {
+        ti = it % d.nt;
+    }
+    float* y = Y + d.y_start;
+    const float* s = S + d.s_start + (size_t)d.m * ti;
+    for (int i = threadIdx.x; i < d.m; i += NHIP_WG) y[i] = s[i];
+}
+
+// ---------------------------------------------------------------- unary function nodes
+__global__ __launch_bounds__(NHIP_WG) void direct_unary_kernel(int opcode,
+                                                               const int4* __restrict__ desc,
+                                                               const float* X, float* Y) {
+    const int4 d = desc[blockIdx.x];  // {x_start, y_start, count, 0}
+    for (int i = threadIdx.x; i < d.z; i += NHIP_WG) {
+        const float x = X[d.x + i];
+        float y;
+        switch (opcode) {
+            case 1: y = sinf(x); break;
+            case 2: y = cosf(x); break;
+            case 3: y = tanhf(x); break;
+            case 4: y = expf(x); break;
+            case 5: y = __fmul_rn(x, x); break;
+            default: y = x;
+        }
+        Y[d.y + i] = y;
+    }
+}
+
+// ---------------------------------------------------------------- probes
+// clra_nonlinearities.py:831-902.  One group per probe; the float32 countdown and
+// the buffer position are read by every thread before the barrier and written by
+// thread 0 after it.
+struct ProbeDesc { int x_start, shape0, shape1, stride0, stride1, y_start, p0, p1; };
+
+__global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __restrict__ desc,
+                                                         float* countdowns, int* bufpositions,
+                                                         const float* __restrict__ periods,
+                                                         const float* X, float* Y) {
+    const int n = blockIdx.x;
+    const float countdown = countdowns[n];
+    const bool fire = countdown <= 0.0f;
+    int bufpos = 0;
+    if (fire) {
+        const ProbeDesc d = desc[n];
+        bufpos = bufpositions[n];
+        const int n_dims = d.shape0 * d.shape1;
+        const float* x = X + d.x_start;
+        float* y = Y + d.y_start + (size_t)bufpos * n_dims;
+        for (int ij = threadIdx.x; ij < n_dims; ij += NHIP_WG) {
+            const int i = ij / d.shape1, j = ij - i * d.shape1;
+            y[ij] = x[(size_t)i * d.stride0 + (size_t)j * d.stride1];
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (fire) {
+            countdowns[n] = countdown + periods[n] - 1.0f;
+            bufpositions[n] = bufpos + 1;
+        } else {
+            countdowns[n] = countdown - 1.0f;
+        }
+    }
+}
+
+__global__ __launch_bounds__(NHIP_WG) void fill_i32_kernel(int* dst, int n, int value) {
+    const int i = blockIdx.x * NHIP_WG + threadIdx.x;
+    if (i < n) dst[i] = value;
+}
+
+}  // namespace
+
+#define NHIP_STREAM(s) static_cast<hipStream_t>(s)
+
+extern "C" int nhip_reset(void* stream, const int* blocks, int n_blocks, float* Y) {
+    if (n_blocks == 0) return 0;
+    if (n_blocks < 0 || !blocks || !Y) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(reset_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const int4*>(blocks), Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_copy(void* stream, const int* desc, int n_blocks, const float* X, float* Y) {
+    if (n_blocks == 0) return 0;
+    if (n_blocks < 0 || !desc || !X || !Y) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(copy_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const CopyDesc*>(desc), X, Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_slicedcopy(void* stream, const int* desc, int n_blocks, const float* X,
+                               float* Y, const int* XI, const int* YI) {
+    if (n_blocks == 0) return 0;
+    if (n_blocks < 0 || !desc || !X || !Y || !XI || !YI) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(slicedcopy_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const SlicedDesc*>(desc), X, Y, XI, YI);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_elementwise_inc(void* stream, const int* desc, int n_blocks, const float* A,
+                                    const float* X, float* Y) {
+    if (n_blocks == 0) return 0;
+    if (n_blocks < 0 || !desc || !A || !X || !Y) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(elementwise_inc_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), reinterpret_cast<const EwDesc*>(desc), A, X, Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_linearfilter(void* stream, const int* desc, int* pos, int n_blocks,
+                                 const float* X, float* Y, const float* A, const float* B,
+                                 float* Xbuf, float* Ybuf) {
+    if (n_blocks == 0) return 0;
+    if (n_blocks < 0 || !desc || !pos || !X || !Y || !A || !B) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(linearfilter_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const LfDesc*>(desc), reinterpret_cast<int2*>(pos), X, Y, A,
+                       B, Xbuf, Ybuf);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_timeupdate(void* stream, float* step_data, int step_start, float* time_data,
+                               int time_start, double dt) {
+    if (!step_data || !time_data || step_start < 0 || time_start < 0) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(timeupdate_kernel, dim3(1), dim3(NHIP_WAVE), 0, NHIP_STREAM(stream),
+                       step_data + step_start, time_data + time_start, dt);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_presentinput(void* stream, const int* desc, int n, float dt, float* Y,
+                                 const float* T, const float* S) {
+    if (n == 0) return 0;
+    if (n < 0 || !desc || !Y || !T || !S) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(presentinput_kernel, dim3(n), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const PiDesc*>(desc), dt, Y, T, S);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_direct_unary(void* stream, int opcode, const int* desc, int n, const float* X,
+                                 float* Y) {
+    if (n == 0) return 0;
+    if (n < 0 || !desc || !X || !Y || opcode < 0 || opcode > 5) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(direct_unary_kernel, dim3(n), dim3(NHIP_WG), 0, NHIP_STREAM(stream), opcode,
+                       reinterpret_cast<const int4*>(desc), X, Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_probes(void* stream, const int* desc, int n, float* countdowns,
+                           int* bufpositions, const float* periods, const float* X, float* Y) {
+    if (n == 0) return 0;
+    if (n < 0 || !desc || !countdowns || !bufpositions || !periods || !X || !Y)
+        return NHIP_E_BADARG;
+    hipLaunchKernelGGL(probes_kernel, dim3(n), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const ProbeDesc*>(desc), countdowns, bufpositions, periods,
+                       X, Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_fill_i32(void* stream, int* dst, int n, int value) {
+    if (n == 0) return 0;
+    if (n < 0 || !dst) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((n + NHIP_WG - 1) / NHIP_WG), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), dst, n, value);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}

@@ -1,0 +1,289 @@
+// Ragged gather-GEMV for gfx950 (wave64, no MFMA: the work is matrix-vector and
+// bound by HBM bandwidth).
+//
+//   Y[b] = beta_b * Yin[b] + gamma_b + alpha_b * sum_d A[b,d] @ X[b,d]
+//
+// for thousands of differently shaped (A, X) pairs that all live in one flat
+// float32 buffer and are described by int32 element offsets.  Semantics follow
+// the reference's block GEMV (clra_gemv.py:861-1175) but the decomposition is
+// different: a task owns complete rows of one output item, walks all of that
+// item's dot products and all of their columns, and writes the final Y once.
+// There is no partial-sum buffer and no second (reduce) launch, and the
+// summation order is fixed, so results are reproducible run to run.
+//
+// Two flavours, chosen per item by the host planner:
+//   wg   : one 256-thread group per task.  The gathered X vector is staged
+//          through LDS once per group (coalesced, stride-aware) and shared by
+//          the four waves.  LPR lanes cooperate on a row (LPR = 256: the whole
+//          group); every lane keeps P independent row accumulators so that P
+//          16-byte loads are in flight per lane.
+//   wave : one wave per task, four unrelated tasks per group, no LDS and no
+//          barrier; for the many tiny items (1 x 100, 100 x 1, ...) of
+//          networks with thousands of small ensembles.
+// Lanes of a row own interleaved column quads (lane l: columns 4l..4l+3, then
+// + 4*LPR ...), so one load instruction of a wave covers contiguous memory.
+#include "nhip_common.h"
+
+namespace {
+
+struct GemvItem { int y_start, y_stride0, yin_start, yin_stride0, dot_begin, n_dots, M, pad; };
+struct GemvDot { int a_start, a_stride0, N, x_start, x_stride0, p0, p1, p2; };
+struct GemvTask { int item, row0, n_rows, pad; };
+
+constexpr int XCHUNK = 4096;  // floats of X staged per pass: 16 KiB of the 160 KiB LDS
+
+// rows accumulated at once by each lane (independent loads in flight)
+template <int LPR> struct PassCount { static constexpr int value = 4; };
+template <> struct PassCount<16> { static constexpr int value = 8; };
+
+template <int LPR>
+__device__ __forceinline__ float row_reduce(float v) {
+    // butterfly over the LPR (<= 64) neighbouring lanes that share a row
+#pragma unroll
+    for (int off = LPR / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, NHIP_WAVE);
+    return v;
+}
+
+template <int LPR, int VEC>
+__global__ __launch_bounds__(NHIP_WG) void gemv_wg_kernel(
+    const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
+    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks,
+    const float* __restrict__ A, const float* __restrict__ X, const float* Yin, float* Y)
+{
+    constexpr bool WIDE = (LPR == 256);
+    constexpr int P = PassCount<LPR>::value;
+    constexpr int RPP = WIDE ? 1 : NHIP_WAVE / (WIDE ? 64 : LPR);  // rows per wave pass
+
+    __shared__ __attribute__((aligned(16))) float xs[XCHUNK];
+    __shared__ float red[NHIP_WG / NHIP_WAVE][P];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (NHIP_WAVE - 1);
+    const int wave = tid >> 6;
+    const int lir = WIDE ? tid : (lane % (WIDE ? 64 : LPR));  // lane index within the row
+
+    const GemvTask task = tasks[nhip_xcd_remap(blockIdx.x, gridDim.x)];
+    const GemvItem it = items[task.item];
+    const float4 cf = coefs[task.item];
+    const int row_end = task.row0 + task.n_rows;
+
+    int row[P];
+    bool valid[P];
+    float acc[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int r = WIDE ? task.row0 + p
+                           : task.row0 + (wave * P + p) * RPP + lane / (WIDE ? 64 : LPR);
+        valid[p] = r < row_end;
+        row[p] = valid[p] ? r : row_end - 1;  // clamp: loads stay in bounds, result dropped
+        acc[p] = 0.0f;
+    }
+
+    for (int d = 0; d < it.n_dots; ++d) {
+        const GemvDot dot = dots[it.dot_begin + d];
+        const float* xg = X + dot.x_start;
+        for (int c0 = 0; c0 < dot.N; c0 += XCHUNK) {
+            const int len = min(XCHUNK, dot.N - c0);
+            __syncthreads();  // everyone is done with the previous chunk
+            for (int k = tid; k < len; k += NHIP_WG)
+                xs[k] = xg[(size_t)(c0 + k) * dot.x_stride0];
+            __syncthreads();
+
+            const float* arow[P];
+#pragma unroll
+            for (int p = 0; p < P; ++p)
+                arow[p] = A + dot.a_start + (size_t)row[p] * dot.a_stride0 + c0;
+
+            if (VEC == 4) {
+                const int len4 = len & ~3;
+                for (int c = lir * 4; c < len4; c += LPR * 4) {
+                    const float4 x = *reinterpret_cast<const float4*>(&xs[c]);
+                    float4 a[P];
+#pragma unroll
+                    for (int p = 0; p < P; ++p)
+                        a[p] = *reinterpret_cast<const float4*>(arow[p] + c);
+#pragma unroll
+                    for (int p = 0; p < P; ++p) {
+                        acc[p] = fmaf(a[p].x, x.x, acc[p]);
+                        acc[p] = fmaf(a[p].y, x.y, acc[p]);
+                        acc[p] = fmaf(a[p].z, x.z, acc[p]);
+                        acc[p] = fmaf(a[p].w, x.w, acc[p]);
+                    }
+                }
+                for (int c = len4 + lir; c < len; c += LPR) {  // < 4 leftover columns
+                    const float x = xs[c];
+#pragma unroll
+                    for (int p = 0; p < P; ++p) acc[p] = fmaf(arow[p][c], x, acc[p]);
+                }
+            } else {
+                for (int c = lir; c < len; c += LPR) {
+                    const float x = xs[c];
+#pragma unroll
+                    for (int p = 0; p < P; ++p) acc[p] = fmaf(arow[p][c], x, acc[p]);
+                }
+            }
+        }
+    }
+
+    if (!WIDE) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const float s = row_reduce<WIDE ? 64 : LPR>(acc[p]);
+            if (lir == 0 && valid[p]) {
+                const float yin = Yin[it.yin_start + (size_t)row[p] * it.yin_stride0];
+                Y[it.y_start + (size_t)row[p] * it.y_stride0] = cf.y * yin + cf.z + cf.x * s;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const float s = row_reduce<64>(acc[p]);
+            if (lane == 0) red[wave][p] = s;
+        }
+        __syncthreads();
+        if (tid < P && task.row0 + tid < row_end) {
+            const int r = task.row0 + tid;
+            const float s = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+            const float yin = Yin[it.yin_start + (size_t)r * it.yin_stride0];
+            Y[it.y_start + (size_t)r * it.y_stride0] = cf.y * yin + cf.z + cf.x * s;
+        }
+    }
+}
+
+template <int LPR, int VEC>
+__global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
+    const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
+    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    const float* __restrict__ A, const float* __restrict__ X, const float* Yin, float* Y)
+{
+    constexpr int RPP = NHIP_WAVE / LPR;
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    const int t = blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6);
+    if (t >= n_tasks) return;  // wave-uniform; this kernel has no barrier
+
+    const GemvTask task = tasks[t];
+    const GemvItem it = items[task.item];
+    const float4 cf = coefs[task.item];
+    const int row_end = task.row0 + task.n_rows;
+    const int lir = lane % LPR;
+    const int sub = lane / LPR;
+
+    for (int r0 = task.row0; r0 < row_end; r0 += RPP) {
+        const bool valid = r0 + sub < row_end;
+        const int r = valid ? r0 + sub : row_end - 1;
+        float acc = 0.0f;
+        for (int d = 0; d < it.n_dots; ++d) {
+            const GemvDot dot = dots[it.dot_begin + d];
+            const float* arow = A + dot.a_start + (size_t)r * dot.a_stride0;
+            const float* xg = X + dot.x_start;
+            const size_t xs = (size_t)dot.x_stride0;
+            int c_tail = lir;
+            if (VEC == 4) {
+                const int n4 = dot.N & ~3;
+                for (int c = lir * 4; c < n4; c += LPR * 4) {
+                    const float4 a = *reinterpret_cast<const float4*>(arow + c);
+                    acc = fmaf(a.x, xg[(size_t)c * xs], acc);
+                    acc = fmaf(a.y, xg[(size_t)(c + 1) * xs], acc);
+                    acc = fmaf(a.z, xg[(size_t)(c + 2) * xs], acc);
+                    acc = fmaf(a.w, xg[(size_t)(c + 3) * xs], acc);
+                }
+                c_tail = n4 + lir;
+            }
+            for (int c = c_tail; c < dot.N; c += LPR)
+                acc = fmaf(arow[c], xg[(size_t)c * xs], acc);
+        }
+        const float s = row_reduce<LPR>(acc);
+        if (lir == 0 && valid) {
+            const float yin = Yin[it.yin_start + (size_t)r * it.yin_stride0];
+            Y[it.y_start + (size_t)r * it.y_stride0] = cf.y * yin + cf.z + cf.x * s;
+        }
+    }
+}
+
+template <int LPR, int VEC>
+int launch_wg(hipStream_t s, const int* items, const float* coefs, const int* dots,
+              const int* tasks, int n_tasks, const float* A, const float* X, const float* Yin,
+              float* Y) {
+    hipLaunchKernelGGL((gemv_wg_kernel<LPR, VEC>), dim3(n_tasks), dim3(NHIP_WG), 0, s,
+                       reinterpret_cast<const GemvItem*>(items),
+                       reinterpret_cast<const float4*>(coefs),
+                       reinterpret_cast<const GemvDot*>(dots),
+                       reinterpret_cast<const GemvTask*>(tasks), A, X, Yin, Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+template <int LPR, int VEC>
+int launch_wave(hipStream_t s, const int* items, const float* coefs, const int* dots,
+                const int* tasks, int n_tasks, const float* A, const float* X,
+                const float* Yin, float* Y) {
+    const int wpg = NHIP_WG / NHIP_WAVE;
+    hipLaunchKernelGGL((gemv_wave_kernel<LPR, VEC>), dim3((n_tasks + wpg - 1) / wpg),
+                       dim3(NHIP_WG), 0, s, reinterpret_cast<const GemvItem*>(items),
+                       reinterpret_cast<const float4*>(coefs),
+                       reinterpret_cast<const GemvDot*>(dots),
+                       reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int nhip_gemv_rows_per_task(int flavor, int lpr, int vec) {
+    if (vec != 1 && vec != 4) return 0;
+    if (flavor == 1) {
+        switch (lpr) { case 1: case 2: case 4: case 8: case 16: case 32: case 64: return 0x7fffffff; }
+        return 0;
+    }
+    if (flavor != 0) return 0;
+    switch (lpr) {
+        case 1: return 4 * PassCount<1>::value * 64;
+        case 2: return 4 * PassCount<2>::value * 32;
+        case 4: return 4 * PassCount<4>::value * 16;
+        case 8: return 4 * PassCount<8>::value * 8;
+        case 16: return 4 * PassCount<16>::value * 4;
+        case 32: return 4 * PassCount<32>::value * 2;
+        case 64: return 4 * PassCount<64>::value;
+        case 256: return PassCount<256>::value;
+    }
+    return 0;
+}
+
+#define NHIP_GEMV_CASE(FN, L)                                                            \
+    case L:                                                                              \
+        return vec == 4 ? FN<L, 4>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y)  \
+                        : FN<L, 1>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y);
+
+extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, const int* items,
+                         const float* coefs, const int* dots, const int* tasks, int n_tasks,
+                         const float* A, const float* X, const float* Yin, float* Y) {
+    if (n_tasks == 0) return 0;
+    if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
+        return NHIP_E_BADARG;
+    if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
+    if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (flavor == 0) {
+        switch (lpr) {
+            NHIP_GEMV_CASE(launch_wg, 1)
+            NHIP_GEMV_CASE(launch_wg, 2)
+            NHIP_GEMV_CASE(launch_wg, 4)
+            NHIP_GEMV_CASE(launch_wg, 8)
+            NHIP_GEMV_CASE(launch_wg, 16)
+            NHIP_GEMV_CASE(launch_wg, 32)
+            NHIP_GEMV_CASE(launch_wg, 64)
+            NHIP_GEMV_CASE(launch_wg, 256)
+        }
+    } else if (flavor == 1) {
+        switch (lpr) {
+            NHIP_GEMV_CASE(launch_wave, 1)
+            NHIP_GEMV_CASE(launch_wave, 2)
+            NHIP_GEMV_CASE(launch_wave, 4)
+            NHIP_GEMV_CASE(launch_wave, 8)
+            NHIP_GEMV_CASE(launch_wave, 16)
+            NHIP_GEMV_CASE(launch_wave, 32)
+            NHIP_GEMV_CASE(launch_wave, 64)
+        }
+    }
+    return NHIP_E_BADCLASS;
+}

@@ -1,0 +1,32 @@
+// Shared device/host helpers for the gfx950 timestep kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/nengo_hip.h"
+
+#define NHIP_WG 256    // threads per work-group: four wave64
+#define NHIP_WAVE 64
+#define NHIP_NXCD 8    // MI355X: 8 accelerator dies, each with its own L2
+
+#define NHIP_LAUNCH_CHECK()                 \
+    do {                                    \
+        hipError_t e_ = hipGetLastError();  \
+        if (e_ != hipSuccess) return (int)e_; \
+    } while (0)
+
+// Work-groups are handed to the 8 XCDs round-robin (group g runs on XCD g % 8).
+// This maps the hardware group id to a logical id such that every XCD works on
+// one contiguous range of logical ids; neighbouring tasks (row blocks of the
+// same matrix, which share the gathered X vector and the Y cache lines) then
+// hit the same L2.  The mapping is a bijection on [0, n_groups).
+__device__ __forceinline__ int nhip_xcd_remap(int bid, int n_groups) {
+    const int per = n_groups / NHIP_NXCD;
+    const int rem = n_groups % NHIP_NXCD;
+    const int xcd = bid % NHIP_NXCD;
+    const int idx = bid / NHIP_NXCD;
+    const int base = (xcd < rem) ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per;
+    return base + idx;
+}
+
+__device__ __forceinline__ float nhip_bits(int b) { return __int_as_float(b); }

@@ -1,0 +1,105 @@
+// Executor support: library identity, error strings, stream capture into an
+// executable graph, replay, and event timing.  The plan sequence of a timestep
+// never changes after construction (all device pointers and work lists are
+// fixed), so it is recorded once and replayed; this replaces the per-plan
+// Python launch loop of the reference executor (plan.py:137-149).
+#include <cstdio>
+#include <cstring>
+
+#include "nhip_common.h"
+
+extern "C" int nhip_abi_version(void) { return NHIP_ABI_VERSION; }
+
+extern "C" const char* nhip_error_string(int err) {
+    switch (err) {
+        case 0: return "success";
+        case NHIP_E_BADARG: return "nengo_hip: bad argument (null pointer, negative count or unknown mode)";
+        case NHIP_E_BADCLASS: return "nengo_hip: unknown GEMV kernel class (flavor, lanes per row, vector width)";
+    }
+    return hipGetErrorString(static_cast<hipError_t>(err));
+}
+
+extern "C" int nhip_device_info(int* n_cu, int* wave_size, int* lds_bytes, char* name,
+                                int name_len) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return (int)e;
+    if (n_cu) *n_cu = prop.multiProcessorCount;
+    if (wave_size) *wave_size = prop.warpSize;
+    if (lds_bytes) *lds_bytes = (int)prop.sharedMemPerBlock;
+    if (name && name_len > 0) {
+        std::strncpy(name, prop.gcnArchName, (size_t)name_len - 1);
+        name[name_len - 1] = '\0';
+    }
+    return 0;
+}
+
+extern "C" int nhip_capture_begin(void* stream) {
+    if (!stream) return NHIP_E_BADARG;  // the legacy default stream cannot be captured
+    // relaxed mode: other host threads (allocators, loggers) may keep calling
+    // the runtime while this stream records
+    return (int)hipStreamBeginCapture(static_cast<hipStream_t>(stream),
+                                      hipStreamCaptureModeRelaxed);
+}
+
+extern "C" int nhip_capture_end(void* stream, void** graph_exec_out) {
+    if (!stream || !graph_exec_out) return NHIP_E_BADARG;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(static_cast<hipStream_t>(stream), &graph);
+    if (e != hipSuccess) return (int)e;
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return (int)e;
+    *graph_exec_out = exec;
+    return 0;
+}
+
+extern "C" int nhip_graph_launch(void* graph_exec, void* stream, int n_times) {
+    if (!graph_exec || n_times < 0) return NHIP_E_BADARG;
+    for (int i = 0; i < n_times; ++i) {
+        hipError_t e = hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec),
+                                      static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return (int)e;
+    }
+    return 0;
+}
+
+extern "C" int nhip_graph_destroy(void* graph_exec) {
+    if (!graph_exec) return 0;
+    return (int)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec));
+}
+
+extern "C" int nhip_stream_sync(void* stream) {
+    return (int)hipStreamSynchronize(static_cast<hipStream_t>(stream));
+}
+
+extern "C" int nhip_event_create(void** event_out) {
+    if (!event_out) return NHIP_E_BADARG;
+    hipEvent_t ev = nullptr;
+    hipError_t e = hipEventCreate(&ev);
+    if (e != hipSuccess) return (int)e;
+    *event_out = ev;
+    return 0;
+}
+
+extern "C" int nhip_event_record(void* event, void* stream) {
+    if (!event) return NHIP_E_BADARG;
+    return (int)hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int nhip_event_elapsed_ms(void* start, void* stop, float* ms_out) {
+    if (!start || !stop || !ms_out) return NHIP_E_BADARG;
+    hipError_t e = hipEventSynchronize(static_cast<hipEvent_t>(stop));
+    if (e != hipSuccess) return (int)e;
+    return (int)hipEventElapsedTime(ms_out, static_cast<hipEvent_t>(start),
+                                    static_cast<hipEvent_t>(stop));
+}
+
+extern "C" int nhip_event_destroy(void* event) {
+    if (!event) return 0;
+    return (int)hipEventDestroy(static_cast<hipEvent_t>(event));
+}

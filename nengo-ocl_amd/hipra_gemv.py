@@ -1,0 +1,263 @@
+"""Plan builders for the ragged gather-GEMV on HIP.
+
+Counterpart of the dense half of the reference's ``nengo_ocl/clra_gemv.py``:
+``gemv_prog`` (:100-261), the planner classes ``plan_ref_gemv`` /
+``plan_many_dots_gemv`` / ``plan_reduce_gemv`` / ``plan_block_gemv`` /
+``plan_ragged_gather_gemv`` (:1178-1239) and the byte / flop accounting
+(``bw_from_geometry`` :49-70, ``flops_from_geometry`` :35-46).  Same call
+signature, same ``.plans`` attribute; what differs is the work decomposition:
+
+* every output item is cut into *tasks* of whole rows; a task walks all dot
+  products of its item and all their columns and writes final Y values, so a
+  GEMV group is ONE launch per kernel class instead of ``fn`` + ``reduce``;
+* items are sorted into kernel classes ``(flavor, lanes-per-row, vector width)``
+  by shape and alignment, one launch per class that occurs.
+
+For each item b:  ``Y[b] = beta[b]*Y_in[b] + gamma[b] + alpha[b] * sum_j A[A_js[b][j]] @ X[X_js[b][j]]``.
+"""
+
+from collections import defaultdict
+
+import numpy as np
+
+from . import _lib
+from .hipraggedarray import HIPRaggedArray, to_device
+from .plan import Plan
+from .utils import next_pow2
+
+# items with at most this many matrix elements go to the wave-per-task kernel
+SMALL_ITEM_ELEMS = 8192
+WG, WAVE = 256, 64
+
+
+def flops_from_geometry(geometry, items):
+    """2 flops per matrix element + 3 per output (clra_gemv.py:35-46)."""
+    flops = 0
+    for i in items:
+        g = geometry[i]
+        flops += 2 * g["y_len"] * sum(d["a_shape1"] for d in g["dots"]) + 3 * g["y_len"]
+    return int(flops)
+
+
+def bw_from_geometry(geometry, items):
+    """Algorithmic bytes: A and X of every dot, Y_in read, Y written, two scalars
+    (clra_gemv.py:49-70).  This is the figure achieved-GB/s numbers are quoted on."""
+    n_bytes = 0
+    for i in items:
+        g = geometry[i]
+        for d in g["dots"]:
+            n_bytes += 4 * d["a_shape1"] * g["y_len"] + 4 * d["a_shape1"]
+        n_bytes += 8 + 4 * g["y_len"] + 4 * g["y_len"]
+    return int(n_bytes)
+
+
+def _per_item_floats(arg, n, what):
+    """alpha/beta/gamma as a float32 vector of length n (scalar, list or ndarray)."""
+    if isinstance(arg, HIPRaggedArray):
+        raise NotImplementedError("%s given as a device ragged array" % what)
+    vec = np.asarray(arg, dtype=np.float32)
+    if vec.ndim == 0:
+        vec = np.full(n, vec, dtype=np.float32)
+    if vec.shape != (n,):
+        raise ValueError("%s must be a scalar or have one value per output" % what)
+    return vec
+
+
+class gemv_prog:
+    """Geometry + work lists of one ragged GEMV; subclasses pick the kernel classes."""
+
+    force_flavor = None  # None = by item size; 0 = work-group kernel; 1 = wave kernel
+    force_scalar = False  # one lane per output, 4-byte loads (the plain fallback)
+
+    def __init__(self, queue, alpha, A, A_js, X, X_js, beta, Y, Y_in=None, gamma=0.0, tag=None):
+        self.queue = queue
+        self.A, self.A_js, self.X, self.X_js = A, A_js, X, X_js
+        self.Y = Y
+        self.Y_in = Y if Y_in is None else Y_in
+        self.tag = str(tag)
+        n = len(Y)
+        self.alpha = _per_item_floats(alpha, n, "alpha")
+        self.beta = _per_item_floats(beta, n, "beta")
+        self.gamma = _per_item_floats(gamma, n, "gamma")
+        self.float_alpha = float(self.alpha[0]) if n and np.all(self.alpha == self.alpha[0]) else None
+        self.float_beta = float(self.beta[0]) if n and np.all(self.beta == self.beta[0]) else None
+        self.float_gamma = float(self.gamma[0]) if n and np.all(self.gamma == self.gamma[0]) else None
+
+        self.geometry = self._geometry()
+        self.plans = self.choose_plans()
+
+    # ------------------------------------------------------------ geometry
+    def _geometry(self):
+        A, X, Y, Y_in = self.A, self.X, self.Y, self.Y_in
+        if len(Y_in) != len(Y):
+            raise ValueError("Y_in and Y differ in length")
+        if self.A_js is None or self.X_js is None:
+            raise NotImplementedError("A_js / X_js are required")
+        if len(self.A_js) != len(Y) or len(self.X_js) != len(Y):
+            raise ValueError("need one A_js / X_js list per output")
+
+        geometry = []
+        for b in range(len(Y)):
+            M = int(Y.shape0s[b])
+            if int(Y.shape1s[b]) != 1 or int(Y_in.shape1s[b]) != 1:
+                raise NotImplementedError("outputs must be column vectors")
+            if int(Y_in.shape0s[b]) != M:
+                raise ValueError("Y_in[%d] and Y[%d] differ in length" % (b, b))
+            a_js = np.asarray(self.A_js[b]).ravel()
+            x_js = np.asarray(self.X_js[b]).ravel()
+            if a_js.size != x_js.size:
+                raise ValueError("A_js[%d] and X_js[%d] differ in length" % (b, b))
+            dots = []
+            for j, (aj, xj) in enumerate(zip(a_js.tolist(), x_js.tolist())):
+                if int(A.shape0s[aj]) != M:
+                    raise ValueError("A[%d] has %d rows, Y[%d] has %d" % (aj, A.shape0s[aj], b, M))
+                if int(A.shape1s[aj]) != int(X.shape0s[xj]) or int(X.shape1s[xj]) != 1:
+                    raise ValueError("A[%d] and X[%d] do not conform" % (aj, xj))
+                if int(A.stride1s[aj]) != 1 and int(A.shape1s[aj]) > 1:
+                    raise NotImplementedError("A rows must be contiguous (stride1 == 1)")
+                dots.append(
+                    {
+                        "j": j,
+                        "a_j": aj,
+                        "x_j": xj,
+                        "a_start": int(A.starts[aj]),
+                        "a_stride0": int(A.stride0s[aj]),
+                        "a_shape1": int(A.shape1s[aj]),
+                        "x_start": int(X.starts[xj]),
+                        "x_stride0": int(X.stride0s[xj]),
+                    }
+                )
+            geometry.append(
+                {
+                    "y_len": M,
+                    "dots": dots,
+                    "y_start": int(Y.starts[b]),
+                    "y_stride0": int(Y.stride0s[b]),
+                    "y_in_start": int(Y_in.starts[b]),
+                    "y_in_stride0": int(Y_in.stride0s[b]),
+                }
+            )
+        return geometry
+
+    def geometry_summary(self, items=None):
+        gg = self.geometry if items is None else [self.geometry[i] for i in items]
+        if not gg:
+            return "outputs: 0"
+        dots = np.array([len(g["dots"]) for g in gg])
+        m = np.array([g["y_len"] for g in gg])
+        n = np.array([d["a_shape1"] for g in gg for d in g["dots"]] or [0])
+        return "outputs: %d; dots: %0.1f [%d, %d]; shape: %0.1f [%d, %d] x %0.1f [%d, %d]" % (
+            len(gg), dots.mean(), dots.min(), dots.max(),
+            m.mean(), m.min(), m.max(), n.mean(), n.min(), n.max(),
+        )
+
+    # ------------------------------------------------------- class selection
+    def _item_class(self, g):
+        """(flavor, lanes per row, vector width) for one item."""
+        dots = g["dots"]
+        M = g["y_len"]
+        n_max = max([d["a_shape1"] for d in dots] or [1])
+        n_sum = sum(d["a_shape1"] for d in dots)
+        if self.force_scalar:
+            return (1, 1, 1)
+        vec = 4
+        if n_max < 4 or any(d["a_start"] % 4 or (d["a_stride0"] % 4 and M > 1) for d in dots):
+            vec = 1
+        flavor = self.force_flavor
+        if flavor is None:
+            flavor = 1 if M * n_sum <= SMALL_ITEM_ELEMS else 0
+        lpr = min(WAVE, next_pow2(-(-n_max // vec)))
+        if flavor == 0 and (n_max >= 2048 or (n_max >= 512 and M < 16)):
+            lpr = WG  # the whole group works on one row
+        return (flavor, lpr, vec)
+
+    def _build(self, items):
+        """Work lists for `items`; returns the list of plans (one per kernel class)."""
+        lib = self.queue.lib
+        geometry = self.geometry
+        n_items = len(geometry)
+
+        item_tab = np.zeros((max(n_items, 1), 8), dtype=np.int32)
+        coef_tab = np.zeros((max(n_items, 1), 4), dtype=np.float32)
+        dot_rows = []
+        for b, g in enumerate(geometry):
+            item_tab[b] = (g["y_start"], g["y_stride0"], g["y_in_start"], g["y_in_stride0"],
+                           len(dot_rows), len(g["dots"]), g["y_len"], 0)
+            coef_tab[b] = (self.alpha[b], self.beta[b], self.gamma[b], 0.0)
+            for d in g["dots"]:
+                dot_rows.append((d["a_start"], d["a_stride0"], d["a_shape1"], d["x_start"],
+                                 d["x_stride0"], 0, 0, 0))
+        dot_tab = np.array(dot_rows or [(0,) * 8], dtype=np.int32)
+
+        by_class = defaultdict(list)
+        for b in items:
+            if geometry[b]["y_len"] > 0:
+                by_class[self._item_class(geometry[b])].append(b)
+
+        dev_items = to_device(self.queue, item_tab)
+        dev_coefs = to_device(self.queue, coef_tab)
+        dev_dots = to_device(self.queue, dot_tab)
+
+        plans = []
+        for (flavor, lpr, vec), members in sorted(by_class.items()):
+            if flavor == 0:
+                rows = lib.nhip_gemv_rows_per_task(flavor, lpr, vec)
+            else:
+                rows = (WAVE // lpr) * 4
+            if rows <= 0:
+                raise _lib.HipError("unknown GEMV class %r" % ((flavor, lpr, vec),))
+            task_rows = []
+            for b in members:
+                M = geometry[b]["y_len"]
+                for r0 in range(0, M, rows):
+                    task_rows.append((b, r0, min(rows, M - r0), 0))
+            task_tab = np.array(task_rows, dtype=np.int32)
+            dev_tasks = to_device(self.queue, task_tab)
+            n_tasks = len(task_rows)
+            n_groups = n_tasks if flavor == 0 else -(-n_tasks // (WG // WAVE))
+            args = (flavor, lpr, vec, dev_items.ptr, dev_coefs.ptr, dev_dots.ptr, dev_tasks.ptr,
+                    n_tasks, self.A.ptr, self.X.ptr, self.Y_in.ptr, self.Y.ptr)
+            plan = Plan(
+                self.queue, lib.nhip_gemv, args, gsize=(WG * n_groups,), lsize=(WG,),
+                full_args=(dev_items, dev_coefs, dev_dots, dev_tasks, self.A.dev_buf,
+                           self.X.dev_buf, self.Y_in.dev_buf, self.Y.dev_buf),
+                name="hipra_gemv.%s" % ("wg" if flavor == 0 else "wave"),
+                tag="%s-lpr%d-v%d" % (self.tag, lpr, vec),
+                bw_per_call=bw_from_geometry(geometry, members),
+                flops_per_call=flops_from_geometry(geometry, members),
+            )
+            plan.description = self.geometry_summary(members)
+            plan.kernel_class = (flavor, lpr, vec)
+            plan.n_tasks = n_tasks
+            plans.append(plan)
+        return plans
+
+    def choose_plans(self):
+        return self._build(list(range(len(self.Y))))
+
+
+class plan_block_gemv(gemv_prog):
+    """The planner the Simulator uses (clra_gemv.py:1193-1195)."""
+
+
+class plan_ragged_gather_gemv(gemv_prog):
+    """Shape-driven choice between kernels (clra_gemv.py:1198-1239); here the
+    per-item class selection already does that."""
+
+
+class plan_reduce_gemv(gemv_prog):
+    """Few long dots per output: always the LDS-staged work-group kernel."""
+
+    force_flavor = 0
+
+
+class plan_many_dots_gemv(gemv_prog):
+    """Many shallow dots per output: always the wave-per-task kernel."""
+
+    force_flavor = 1
+
+
+class plan_ref_gemv(gemv_prog):
+    """One lane per output element, scalar loads: the plain fallback kernel."""
+
+    force_scalar = True

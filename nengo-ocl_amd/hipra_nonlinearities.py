@@ -1,0 +1,446 @@
+"""Plan builders for every non-GEMV step of the timestep, on HIP.
+
+Counterpart of the reference's ``nengo_ocl/clra_nonlinearities.py`` for the
+functions the timestep path uses; each keeps the reference's call signature
+(``queue`` is a `hipraggedarray.Queue`) and returns a `Plan`:
+
+=====================  =============================================  ==========
+this module            reference (clra_nonlinearities.py)             C entry
+=====================  =============================================  ==========
+plan_timeupdate        plan_timeupdate :113-144                       nhip_timeupdate
+plan_reset             plan_reset :147-214                            nhip_reset
+plan_copy              plan_copy :217-304                             nhip_copy
+plan_slicedcopy        plan_slicedcopy :307-411                       nhip_slicedcopy
+plan_elementwise_inc   plan_elementwise_inc :414-574                  nhip_elementwise_inc
+plan_linearfilter      plan_linearfilter :577-803                     nhip_linearfilter
+plan_probes            plan_probes :806-951                           nhip_probes
+plan_direct            plan_direct :954-1025 (unary table only)       nhip_direct_unary
+plan_lif               plan_lif :1028-1146 (non-adaptive)             nhip_lif
+plan_lif_rate          plan_lif_rate :1149-1197 (non-adaptive)        nhip_lif_rate
+plan_presentinput      plan_presentinput :1678-1759                   nhip_presentinput
+=====================  =============================================  ==========
+
+Where the reference's kernels index ``*_starts[n]`` device arrays, these build
+one int32 work list per plan (a row per block of <= ``BLOCK`` elements of one
+item) at plan time; argument checks raise the same exception types the
+reference's asserts / raises produce (AssertionError, NotImplementedError).
+"""
+
+import re
+
+import numpy as np
+
+from . import _lib
+from .hipraggedarray import DeviceArray, HIPRaggedArray, to_device
+from .plan import Plan
+from .utils import f32_bits, is_number
+
+WG = 256
+BLOCK = 1024  # elements of one item handled by one work-group
+
+
+def blockify(sizes, max_size=BLOCK):
+    """Cut items of the given sizes into blocks of <= max_size elements.
+
+    Returns int32 arrays ``(item index, offset inside the item, count)``, one
+    entry per block, items in order; empty items get no block.  (The
+    reference's ``blockify_ij`` / ``blockify_vectors`` :22-110 do this with
+    Python loops; this is the vectorised equivalent.)
+    """
+    sizes = np.asarray(sizes, dtype=np.int64).reshape(-1)
+    n_blocks = -(-sizes // max_size)
+    inds = np.repeat(np.arange(sizes.size), n_blocks)
+    first = np.cumsum(n_blocks) - n_blocks
+    k = np.arange(int(n_blocks.sum())) - np.repeat(first, n_blocks)
+    offsets = k * max_size
+    counts = np.minimum(sizes[inds] - offsets, max_size)
+    return inds.astype(np.int32), offsets.astype(np.int32), counts.astype(np.int32)
+
+
+def _description(ra):
+    sizes = ra.sizes
+    if len(sizes) == 0:
+        return "groups: 0"
+    return "groups: %d; items: %d; items/group: %0.1f [%d, %d]" % (
+        len(ra), sizes.sum(), sizes.mean(), sizes.min(), sizes.max())
+
+
+def _host(values):
+    return values.get() if isinstance(values, DeviceArray) else np.asarray(values)
+
+
+def _bits(values):
+    """float32 bit patterns of an array, as int32."""
+    return np.asarray(values, dtype=np.float32).view(np.int32)
+
+
+def _dev_table(queue, columns, width):
+    """Stack per-block int32 columns into a (n_blocks, width) device table."""
+    n = len(columns[0]) if columns else 0
+    table = np.zeros((max(n, 1), width), dtype=np.int32)
+    for c, col in enumerate(columns):
+        if n:
+            table[:n, c] = col
+    return to_device(queue, table), n
+
+
+# ---------------------------------------------------------------- time update
+def plan_timeupdate(queue, step, time, dt):
+    assert len(step) == len(time) == 1
+    assert step.ctype == time.ctype == "float"
+    assert step.shape0s[0] == step.shape1s[0] == 1
+    assert time.shape0s[0] == time.shape1s[0] == 1
+    args = (step.ptr, int(step.starts[0]), time.ptr, int(time.starts[0]), float(dt))
+    return Plan(queue, queue.lib.nhip_timeupdate, args, gsize=(64,), lsize=(64,),
+                full_args=(step.dev_buf, time.dev_buf), name="hip_timeupdate")
+
+
+# ---------------------------------------------------------------- reset
+def plan_reset(queue, Y, values, tag=None):
+    values = _host(values).astype(np.float32).reshape(-1)
+    assert len(Y) == len(values)
+    assert (Y.stride0s == Y.shape1s).all()
+    assert (Y.stride1s == 1).all()
+    assert Y.ctype == "float"
+
+    inds, offsets, counts = blockify(Y.sizes, 4 * BLOCK)
+    table, n = _dev_table(queue, [Y.starts[inds] + offsets, counts, _bits(values[inds])], 4)
+    plan = Plan(queue, queue.lib.nhip_reset, (table.ptr, n, Y.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,), full_args=(table, Y.dev_buf),
+                name="hip_reset", tag=tag)
+    plan.bw_per_call = Y.nbytes + values.nbytes + table.nbytes
+    plan.description = _description(Y)
+    return plan
+
+
+# ---------------------------------------------------------------- copy
+def plan_copy(queue, X, Y, incs, tag=None):
+    assert len(X) == len(Y)
+    assert (X.shape0s == Y.shape0s).all()
+    assert (X.shape1s == Y.shape1s).all()
+    assert (X.stride1s == 1).all()
+    assert (Y.stride1s == 1).all()
+    assert X.ctype == Y.ctype
+    incs = np.asarray(incs, dtype=np.int32).reshape(-1)
+    assert incs.shape == (len(X),)
+
+    inds, offsets, counts = blockify(Y.sizes)
+    table, n = _dev_table(queue, [X.starts[inds], Y.starts[inds], X.shape1s[inds],
+                                  X.stride0s[inds], Y.stride0s[inds], offsets, counts,
+                                  incs[inds]], 8)
+    plan = Plan(queue, queue.lib.nhip_copy, (table.ptr, n, X.ptr, Y.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, X.dev_buf, Y.dev_buf), name="hip_copy", tag=tag)
+    plan.bw_per_call = X.nbytes + Y.nbytes
+    plan.description = _description(X)
+    return plan
+
+
+# ---------------------------------------------------------------- sliced copy
+def plan_slicedcopy(queue, X, Y, Xinds, Yinds, incs, tag=None):
+    assert len(X) == len(Y) == len(Xinds) == len(Yinds)
+    for arr in [X, Y, Xinds, Yinds]:
+        assert (arr.shape1s == 1).all()
+        assert (arr.stride1s == 1).all()
+    for arr in [Xinds, Yinds]:
+        assert (arr.stride0s == 1).all()
+    assert (Xinds.shape0s == Yinds.shape0s).all()
+    assert X.ctype == Y.ctype
+    assert Xinds.ctype == Yinds.ctype == "int"
+    incs = np.asarray(incs, dtype=np.int32).reshape(-1)
+    assert incs.shape == (len(X),)
+
+    inds, offsets, counts = blockify(Xinds.shape0s)
+    table, n = _dev_table(queue, [X.starts[inds], X.stride0s[inds], Y.starts[inds],
+                                  Y.stride0s[inds], Xinds.starts[inds] + offsets,
+                                  Yinds.starts[inds] + offsets, counts, incs[inds]], 8)
+    plan = Plan(queue, queue.lib.nhip_slicedcopy,
+                (table.ptr, n, X.ptr, Y.ptr, Xinds.ptr, Yinds.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, X.dev_buf, Y.dev_buf, Xinds.dev_buf, Yinds.dev_buf),
+                name="hip_slicedcopy", tag=tag)
+    plan.bw_per_call = 2 * (Xinds.nbytes + int(Xinds.sizes.sum()) * X.dtype.itemsize)
+    plan.description = _description(Xinds)
+    return plan
+
+
+# ---------------------------------------------------------------- elementwise inc
+def plan_elementwise_inc(queue, A, X, Y, alpha=None, outer=False, inc=True, tag=None):
+    """``Y (+)= alpha * A * X`` element-wise with broadcasting, or (``outer``) the
+    outer product of vectors A and X."""
+    assert len(Y) == len(X) == len(A)
+    for arr in [A, X, Y]:
+        assert (arr.stride1s == 1).all()
+    if outer:
+        assert (A.shape1s == 1).all()
+        assert (X.shape1s == 1).all()
+        assert ((A.shape0s == 1) | (A.shape0s == Y.shape0s)).all()
+        assert ((X.shape0s == 1) | (X.shape0s == Y.shape1s)).all()
+    else:
+        assert ((X.shape0s == 1) | (X.shape0s == Y.shape0s)).all()
+        assert ((X.shape1s == 1) | (X.shape1s == Y.shape1s)).all()
+        assert ((A.shape0s == 1) | (A.shape0s == Y.shape0s)).all()
+        assert ((A.shape1s == 1) | (A.shape1s == Y.shape1s)).all()
+    assert X.ctype == Y.ctype
+    assert A.ctype == Y.ctype
+    if alpha is not None:
+        assert isinstance(alpha, np.ndarray)
+        assert alpha.shape == (len(Y),)
+        alphas = alpha.astype(np.float32)
+    else:
+        alphas = np.ones(len(Y), dtype=np.float32)
+
+    inds, offsets, counts = blockify(Y.sizes)
+    flags = np.full(len(inds), (1 if outer else 0) | (2 if inc else 0), dtype=np.int32)
+    table, n = _dev_table(queue, [
+        A.starts[inds], A.shape0s[inds], A.shape1s[inds], A.stride0s[inds],
+        X.starts[inds], X.shape0s[inds], X.shape1s[inds], X.stride0s[inds],
+        Y.starts[inds], Y.shape1s[inds], Y.stride0s[inds], offsets,
+        counts, _bits(alphas[inds]), flags], 16)
+    plan = Plan(queue, queue.lib.nhip_elementwise_inc, (table.ptr, n, A.ptr, X.ptr, Y.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, A.dev_buf, X.dev_buf, Y.dev_buf),
+                name="hip_elementwise_inc", tag=tag)
+    plan.flops_per_call = 2 * int(Y.sizes.sum())
+    plan.bw_per_call = A.nbytes + X.nbytes + Y.nbytes + (0 if alpha is None else alphas.nbytes)
+    plan.description = _description(Y)
+    return plan
+
+
+# ---------------------------------------------------------------- linear filter
+def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
+    """``y[n+1] + a[0] y[n] + ... = b[0] x[n] + ... + b[j] x[n-j]`` per element.
+
+    Returns a one-element list: the ring-buffer positions advance inside the
+    same launch (the reference returns a second ``linearfilter_inc`` plan when
+    any filter has order > 1, :781-803).
+    """
+    assert len(X) == len(Y) == len(A) == len(B) == len(Xbuf) == len(Ybuf)
+    assert (X.shape0s == Y.shape0s).all()
+    assert (X.shape1s == Y.shape1s).all()
+    for arr in [A, B, Xbuf, Ybuf]:
+        assert (arr.shape1s == arr.stride0s).all()
+        assert (arr.stride1s == 1).all()
+    for arr in [A, B]:
+        assert (arr.shape1s == 1).all()
+    assert (B.shape0s >= 1).all()
+    assert ((B.shape0s == 1) | (Xbuf.shape0s == B.shape0s)).all()
+    assert ((A.shape0s == 1) | (Ybuf.shape0s == A.shape0s)).all()
+    assert (Xbuf.shape1s == X.sizes).all()
+    assert (Ybuf.shape1s == Y.sizes).all()
+    assert X.ctype == Xbuf.ctype
+    assert Y.ctype == Ybuf.ctype
+
+    inds, offsets, counts = blockify(X.sizes)
+    table, n = _dev_table(queue, [
+        X.starts[inds], X.stride0s[inds], X.stride1s[inds], Y.starts[inds],
+        Y.stride0s[inds], Y.stride1s[inds], X.shape1s[inds], offsets,
+        counts, A.shape0s[inds], B.shape0s[inds], A.starts[inds],
+        B.starts[inds], Xbuf.starts[inds], Ybuf.starts[inds], X.sizes[inds]], 16)
+    pos = to_device(queue, np.zeros((max(n, 1), 2), dtype=np.int32))
+    plan = Plan(queue, queue.lib.nhip_linearfilter,
+                (table.ptr, pos.ptr, n, X.ptr, Y.ptr, A.ptr, B.ptr, Xbuf.ptr, Ybuf.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, pos, X.dev_buf, Y.dev_buf, A.dev_buf, B.dev_buf,
+                           Xbuf.dev_buf, Ybuf.dev_buf),
+                name="hip_linearfilter", tag=tag)
+    plan.bw_per_call = (X.nbytes + Y.nbytes + A.nbytes + B.nbytes + Xbuf.nbytes + Ybuf.nbytes)
+    plan.description = _description(Y)
+    plan.bufpos = pos  # zeroed again by Simulator.reset()
+    return [plan]
+
+
+# ---------------------------------------------------------------- probes
+def plan_probes(queue, periods, X, Y, tag=None):
+    """Every ``periods[i]`` steps copy signal ``X[i]`` into row ``bufpositions[i]``
+    of ``Y[i]`` (shape ``(buf_len, X[i].size)``)."""
+    assert len(X) == len(Y)
+    assert len(X) == len(periods)
+    assert X.ctype == Y.ctype
+    N = len(X)
+    assert (X.shape0s * X.shape1s == Y.shape1s).all()
+    assert (Y.stride0s == Y.shape1s).all()
+    assert (Y.stride1s == 1).all()
+
+    periods = np.asarray(periods, dtype=np.float32)
+    dev_periods = to_device(queue, periods)
+    dev_countdowns = to_device(queue, periods - 1)
+    dev_bufpositions = to_device(queue, np.zeros(N, dtype=np.int32))
+    table, n = _dev_table(queue, [X.starts, X.shape0s, X.shape1s, X.stride0s, X.stride1s,
+                                  Y.starts], 8)
+    plan = Plan(queue, queue.lib.nhip_probes,
+                (table.ptr, n, dev_countdowns.ptr, dev_bufpositions.ptr, dev_periods.ptr,
+                 X.ptr, Y.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, dev_countdowns, dev_bufpositions, dev_periods, X.dev_buf,
+                           Y.dev_buf), name="hip_probes", tag=tag)
+    plan.dev_bufpositions = dev_bufpositions
+    plan.cl_bufpositions = dev_bufpositions  # the reference's attribute name
+    plan.dev_countdowns = dev_countdowns
+    plan.periods = periods
+    plan.Y = Y
+    plan.bw_per_call = (2 * X.nbytes + dev_periods.nbytes + dev_countdowns.nbytes
+                        + dev_bufpositions.nbytes)
+    plan.description = _description(X)
+    return plan
+
+
+# ---------------------------------------------------------------- function nodes
+UNARY_OPCODES = {"identity": 0, "sin": 1, "cos": 2, "tanh": 3, "exp": 4, "square": 5}
+_DIRECT_RE = re.compile(
+    r"^\s*OUTPUT__\[0\]\s*=\s*(?P<fn>[a-z]+)\(\s*(?P<arg>\w+)\[0\]\s*\)\s*;\s*$")
+
+
+def plan_direct(queue, code, init, input_names, inputs, output, tag=None):
+    """Function nodes whose translated code is ``OUTPUT__[0] = f(name[0]);`` with f in
+    the unary table.  Anything else raises NotImplementedError, on which the
+    Simulator falls back to a host callback, as the reference does when its
+    translator fails (simulator.py:955-964)."""
+    assert len(input_names) == len(inputs)
+    for x in inputs:
+        assert len(x) == len(output)
+    for x in list(inputs) + [output]:
+        assert (x.shape1s == 1).all() and (x.stride1s == 1).all()
+        assert (x.stride0s == 1).all()
+    m = _DIRECT_RE.match(code or "")
+    if (init or "").strip() or m is None or m.group("fn") not in UNARY_OPCODES:
+        raise NotImplementedError("only single unary functions run on the device: %r" % code)
+    if m.group("arg") not in input_names:
+        raise NotImplementedError("unknown input %r" % m.group("arg"))
+    x = inputs[list(input_names).index(m.group("arg"))]
+    assert (x.shape0s == 1).all() and (output.shape0s == 1).all()
+
+    table, n = _dev_table(queue, [x.starts, output.starts, np.ones(len(output), np.int32)], 4)
+    plan = Plan(queue, queue.lib.nhip_direct_unary,
+                (UNARY_OPCODES[m.group("fn")], table.ptr, n, x.ptr, output.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, x.dev_buf, output.dev_buf), name="hip_direct", tag=tag)
+    plan.description = _description(output)
+    return plan
+
+
+# ---------------------------------------------------------------- neurons
+def _neuron_params(queue, params, sizes, inds, offsets):
+    """Pack tau/ref/amp for the block table.
+
+    A number, or a ragged array whose items are each constant, becomes float
+    bits in the table (one scalar per block, no per-neuron traffic).  Ragged
+    arrays with varying values stay on the device and the table holds offsets.
+    Returns (columns, pflags, device pointers, keepalive).
+    """
+    columns, ptrs, keep = [], [], []
+    pflags = 0
+    for k, p in enumerate(params):
+        if is_number(p):
+            columns.append(np.full(len(inds), f32_bits(p), dtype=np.int32))
+            ptrs.append(None)
+            continue
+        if not isinstance(p, HIPRaggedArray):
+            raise ValueError("Parameter must be a ragged device array or a float (got %s)" % type(p))
+        assert len(p) == len(sizes)
+        assert (p.shape1s == 1).all() and (p.stride1s == 1).all() and (p.stride0s == 1).all()
+        assert ((p.shape0s == sizes) | (p.shape0s == 1)).all()
+        host = p.to_host()
+        firsts = np.array([host[i][0, 0] if host.sizes[i] else 0.0 for i in range(len(host))],
+                          dtype=np.float32)
+        constant = all(np.all(host[i] == firsts[i]) for i in range(len(host)))
+        if constant:
+            columns.append(_bits(firsts[inds]))
+            ptrs.append(None)
+        else:
+            assert (p.shape0s == sizes).all(), "varying parameters need one value per neuron"
+            columns.append(p.starts[inds] + offsets)
+            ptrs.append(p.ptr)
+            keep.append(p.dev_buf)
+            pflags |= 1 << k
+    return columns, pflags, ptrs, keep
+
+
+def _check_vectors(ras):
+    first = ras[0]
+    for v in ras:
+        assert len(v) == len(first)
+        assert (v.shape0s == first.shape0s).all()
+        assert (v.stride0s == v.shape1s).all()
+        assert (v.stride1s == 1).all()
+        assert (v.shape1s == 1).all()
+
+
+def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, N=None, tau_n=None, inc_n=None,
+             upsample=1, fastlif=False, tag=None, **kwargs):
+    if N is not None or tau_n is not None or inc_n is not None:
+        raise NotImplementedError("adaptive LIF")
+    if fastlif:
+        raise NotImplementedError("fastlif approximation")
+    assert J.ctype == "float"
+    for x in [V, W, outS]:
+        assert x.ctype == J.ctype
+    _check_vectors([J, V, W, outS])
+
+    inds, offsets, counts = blockify(J.shape0s, 2 * WG)
+    pcols, pflags, pptrs, keep = _neuron_params(queue, [tau, ref, amp], J.shape0s, inds, offsets)
+    table, n = _dev_table(queue, [
+        J.starts[inds] + offsets, V.starts[inds] + offsets, W.starts[inds] + offsets,
+        outS.starts[inds] + offsets, counts, pcols[0], pcols[1], pcols[2],
+        np.full(len(inds), pflags, dtype=np.int32)], 12)
+    args = (table.ptr, n, float(dt), int(upsample), J.ptr, V.ptr, W.ptr, outS.ptr,
+            pptrs[0], pptrs[1], pptrs[2])
+    plan = Plan(queue, queue.lib.nhip_lif, args, gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, J.dev_buf, V.dev_buf, W.dev_buf, outS.dev_buf) + tuple(keep),
+                name="hip_lif", tag=tag)
+    n_vec = bin(pflags).count("1")
+    plan.bw_per_call = (J.nbytes + 2 * V.nbytes + 2 * W.nbytes + outS.nbytes + n_vec * J.nbytes)
+    plan.description = _description(J)
+    return plan
+
+
+def plan_lif_rate(queue, dt, J, R, ref, tau, amp, N=None, tau_n=None, inc_n=None, tag=None,
+                  **kwargs):
+    if N is not None or tau_n is not None or inc_n is not None:
+        raise NotImplementedError("adaptive LIF rate")
+    assert J.ctype == "float"
+    assert R.ctype == J.ctype
+    _check_vectors([J, R])
+
+    inds, offsets, counts = blockify(J.shape0s, 2 * WG)
+    pcols, pflags, pptrs, keep = _neuron_params(queue, [tau, ref, amp], J.shape0s, inds, offsets)
+    table, n = _dev_table(queue, [J.starts[inds] + offsets, R.starts[inds] + offsets, counts,
+                                  pcols[0], pcols[1], pcols[2],
+                                  np.full(len(inds), pflags, dtype=np.int32)], 8)
+    args = (table.ptr, n, J.ptr, R.ptr, pptrs[0], pptrs[1], pptrs[2])
+    plan = Plan(queue, queue.lib.nhip_lif_rate, args, gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, J.dev_buf, R.dev_buf) + tuple(keep), name="hip_lif_rate",
+                tag=tag)
+    plan.bw_per_call = J.nbytes + R.nbytes + bin(pflags).count("1") * J.nbytes
+    plan.description = _description(J)
+    return plan
+
+
+# ---------------------------------------------------------------- table playback
+def plan_presentinput(queue, Y, t, signals, dt, pres_t=None, tag=None):
+    """``Y[k] = signals[k][row]`` with the row picked by the float32 step counter
+    ``t[k]``: ``step % rows``, or ``int((step - 0.5) * (dt / pres_t)) % rows``."""
+    N = len(Y)
+    assert len(Y) == len(t) == len(signals)
+    pres = None if pres_t is None else _host(pres_t).astype(np.float32).reshape(-1)
+    assert pres is None or pres.shape == (N,)
+    for arr in [Y, t, signals]:
+        assert (arr.stride1s == 1).all()
+    assert (Y.shape1s == 1).all()
+    assert (Y.stride0s == 1).all()
+    assert (t.shape0s == 1).all()
+    assert (t.shape1s == 1).all()
+    assert (Y.shape0s == signals.shape1s).all()
+    assert (signals.stride0s == signals.shape1s).all()
+
+    table, n = _dev_table(queue, [
+        Y.starts, Y.shape0s, t.starts, signals.starts, signals.shape0s,
+        np.zeros(N, np.int32) if pres is None else _bits(pres),
+        np.full(N, 0 if pres is None else 1, dtype=np.int32)], 8)
+    plan = Plan(queue, queue.lib.nhip_presentinput,
+                (table.ptr, n, float(np.float32(dt)), Y.ptr, t.ptr, signals.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, Y.dev_buf, t.dev_buf, signals.dev_buf),
+                name="hip_presentinput", tag=tag)
+    plan.description = _description(Y)
+    return plan

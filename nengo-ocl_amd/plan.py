@@ -1,0 +1,243 @@
+"""Plans (bound kernel launches) and the executor that replays a timestep.
+
+Counterpart of the reference's ``nengo_ocl/plan.py`` (``BasePlan`` :12-38,
+``PythonPlan`` :41-53, ``Plan`` :56-108, ``Plans`` :111-149).  A `Plan` binds one
+C-ABI entry point of ``libnengo_hip.so`` to its arguments; the executor does
+not issue one driver call per plan per step from Python: the plan sequence is
+recorded once from the stream into a HIP graph and replayed ``n`` times by a
+single C call.  Host-callback plans (`PythonPlan`) cannot be recorded, so they
+split the sequence into graph segments with a stream sync on either side.
+"""
+
+import ctypes
+import time
+
+from . import _lib
+
+
+class BasePlan:
+    def __init__(self, name="", tag=None, flops_per_call=None, bw_per_call=None):
+        self.name = name
+        self.tag = tag
+        self.atimes = []  # queued -> submitted (always 0 here: HIP events time execution only)
+        self.btimes = []  # submitted -> started
+        self.ctimes = []  # started -> ended, seconds
+        self.n_calls = 0
+        self.flops_per_call = flops_per_call
+        self.bw_per_call = bw_per_call
+
+    def _label(self):
+        return "%s%s" % (self.name, ": %s" % self.tag if self.tag else "")
+
+    def __str__(self):
+        return "<%s>" % self._label()
+
+    def __repr__(self):
+        return "%s{%s}" % (type(self).__name__, self._label())
+
+    def update_profiling(self):
+        pass
+
+
+class PythonPlan(BasePlan):
+    """A host callback executed between device plans (forces a stream sync)."""
+
+    def __init__(self, function, **kwargs):
+        super().__init__(**kwargs)
+        self.function = function
+
+    def __call__(self, profiling=False):
+        t0 = time.time() if profiling else 0.0
+        self.function()
+        if profiling:
+            self.atimes.append(0)
+            self.btimes.append(0)
+            self.ctimes.append(time.time() - t0)
+            self.n_calls += 1
+
+
+class Plan(BasePlan):
+    """One kernel launch with all arguments bound.
+
+    ``kern`` is a ctypes function from ``libnengo_hip.so`` whose first parameter
+    is the stream; ``args`` are the remaining arguments.  ``gsize``/``lsize`` are
+    kept for display (grid in threads, group size), as in the reference.
+    ``full_args`` pins every device array the launch reads so that Python does
+    not free them.
+    """
+
+    def __init__(self, queue, kern, args, gsize, lsize=None, full_args=(), **kwargs):
+        super().__init__(**kwargs)
+        self.queue = queue
+        self.kern = kern
+        self.args = tuple(args)
+        self.gsize = self._format_size(gsize)
+        self.lsize = self._format_size(lsize) if lsize is not None else None
+        self.full_args = tuple(full_args)
+        self._events_to_profile = []
+
+    @staticmethod
+    def _format_size(size):
+        size = tuple(int(s) for s in size)
+        if len(size) == 0 or any(s <= 0 for s in size):
+            raise ValueError("launch sizes must be positive, got %r" % (size,))
+        return size
+
+    def enqueue(self, wait_for=None, profiling=False):
+        """Put the launch on the queue's stream; returns immediately."""
+        lib = self.queue.lib
+        if profiling:
+            ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
+            _lib.check(lib.nhip_event_create(ctypes.byref(ev0)))
+            _lib.check(lib.nhip_event_create(ctypes.byref(ev1)))
+            _lib.check(lib.nhip_event_record(ev0, self.queue.handle))
+        _lib.check(self.kern(self.queue.handle, *self.args), self.name)
+        if profiling:
+            _lib.check(lib.nhip_event_record(ev1, self.queue.handle))
+            self._events_to_profile.append((ev0, ev1))
+        return self
+
+    def wait(self):
+        self.queue.finish()
+
+    def __call__(self, profiling=False):
+        self.enqueue(profiling=profiling)
+        self.wait()
+
+    def update_profiling(self):
+        lib = self.queue.lib
+        for ev0, ev1 in self._events_to_profile:
+            ms = ctypes.c_float()
+            _lib.check(lib.nhip_event_elapsed_ms(ev0, ev1, ctypes.byref(ms)))
+            self.atimes.append(0.0)
+            self.btimes.append(0.0)
+            self.ctimes.append(1e-3 * ms.value)
+            self.n_calls += 1
+            lib.nhip_event_destroy(ev0)
+            lib.nhip_event_destroy(ev1)
+        self._events_to_profile[:] = []
+
+    def __str__(self):
+        return "<%s %s %s>" % (self._label(), self.gsize, self.lsize)
+
+    def __repr__(self):
+        return "%s{%s %s %s}" % (type(self).__name__, self._label(), self.gsize, self.lsize)
+
+
+class _GraphSegment:
+    """A run of consecutive device plans recorded into one executable graph."""
+
+    def __init__(self, queue, plans):
+        self.queue = queue
+        self.plans = list(plans)
+        self.exec = None
+
+    def capture(self):
+        lib = self.queue.lib
+        _lib.check(lib.nhip_capture_begin(self.queue.handle), "graph capture begin")
+        err = None
+        try:
+            for plan in self.plans:
+                plan.enqueue()
+        except Exception as e:  # close the capture before re-raising
+            err = e
+        handle = ctypes.c_void_p()
+        rc = lib.nhip_capture_end(self.queue.handle, ctypes.byref(handle))
+        if err is not None:
+            raise err
+        _lib.check(rc, "graph capture end")
+        self.exec = handle
+
+    def launch(self, n):
+        if self.exec is None:
+            self.capture()
+        _lib.check(self.queue.lib.nhip_graph_launch(self.exec, self.queue.handle, n), "graph launch")
+
+    def destroy(self):
+        if self.exec is not None:
+            self.queue.lib.nhip_graph_destroy(self.exec)
+            self.exec = None
+
+
+class Plans:
+    """The ordered plan list of one timestep and its executor."""
+
+    def __init__(self, planlist, profiling, use_graph=True):
+        self.plans = list(planlist)
+        self.profiling = profiling
+        self.use_graph = use_graph
+        self._segments = None  # list of _GraphSegment | PythonPlan
+
+    def __call__(self):
+        return self.call_n_times(1)
+
+    def __len__(self):
+        return len(self.plans)
+
+    def __getitem__(self, i):
+        return self.plans[i]
+
+    def __iter__(self):
+        return iter(self.plans)
+
+    def _queue(self):
+        for p in self.plans:
+            if hasattr(p, "queue"):
+                return p.queue
+        return None
+
+    def _build_segments(self):
+        segments, run = [], []
+        for plan in self.plans:
+            if hasattr(plan, "enqueue"):
+                run.append(plan)
+            else:
+                if run:
+                    segments.append(_GraphSegment(run[0].queue, run))
+                    run = []
+                segments.append(plan)
+        if run:
+            segments.append(_GraphSegment(run[0].queue, run))
+        self._segments = segments
+
+    def call_n_times(self, n):
+        """Run the whole plan sequence ``n`` times and wait for it to finish."""
+        self.enqueue_n_times(n)
+        queue = self._queue()
+        if queue is not None:
+            queue.finish()
+        if self.profiling:
+            for p in self.plans:
+                p.update_profiling()
+
+    def enqueue_n_times(self, n):
+        queue = self._queue()
+        if self.profiling or not self.use_graph:
+            # eager: one launch per plan, events around each when profiling
+            for _ in range(n):
+                for plan in self.plans:
+                    if hasattr(plan, "enqueue"):
+                        plan.enqueue(profiling=self.profiling)
+                    else:
+                        queue and queue.finish()
+                        plan(profiling=self.profiling)
+            return
+
+        if self._segments is None:
+            self._build_segments()
+        if len(self._segments) == 1 and isinstance(self._segments[0], _GraphSegment):
+            self._segments[0].launch(n)  # the common case: n replays, one C call
+            return
+        for _ in range(n):
+            for seg in self._segments:
+                if isinstance(seg, _GraphSegment):
+                    seg.launch(1)
+                else:
+                    queue and queue.finish()
+                    seg()
+
+    def close(self):
+        for seg in self._segments or []:
+            if isinstance(seg, _GraphSegment):
+                seg.destroy()
+        self._segments = None

@@ -1,0 +1,294 @@
+"""Python face of the CPU oracle (``oracle_kernels.c``).  TEST INFRASTRUCTURE ONLY.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and ``bench.py``'s cpu_baseline leg
+may import this module; it is the checker, never the thing shipped or measured.
+
+It offers the reference's ``plan_*`` call signatures
+(nengo_ocl/clra_gemv.py:1178-1195, nengo_ocl/clra_nonlinearities.py:113-1197,
+1678-1759) over HOST ragged arrays: ``queue`` is ignored (pass ``None``), every
+ragged argument is a ``RaggedArray`` whose ``buf`` is updated in place, and the
+returned object is a host-callback plan (``plan()`` runs the step once).
+Ragged metadata is handed to C exactly as the reference hands it to OpenCL
+(starts / shapes / strides per item), independent of the HIP work lists.
+"""
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+from nengo_ocl_amd.plan import PythonPlan
+from nengo_ocl_amd.raggedarray import RaggedArray
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile oracle_kernels.c with gcc (OpenMP, no contraction, no fast-math)."""
+    cmd = ["make", "-C", _HERE] + (["-B"] if force else [])
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("building the oracle failed:\n" + res.stdout + res.stderr)
+    return LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.orc_num_threads.restype = ctypes.c_int
+    return _lib
+
+
+def num_threads():
+    return lib().orc_num_threads()
+
+
+def set_num_threads(n):
+    lib().orc_set_num_threads(int(n))
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _per_item(arg, n, dtype):
+    v = np.asarray(arg, dtype=dtype)
+    if v.ndim == 0:
+        v = np.full(n, v, dtype=dtype)
+    assert v.shape == (n,)
+    return np.ascontiguousarray(v)
+
+
+def _param_per_item(p, n):
+    """tau/ref/amp: a number, or a ragged array constant within each item."""
+    if isinstance(p, RaggedArray):
+        vals = np.array([p[i].flat[0] for i in range(n)], dtype=np.float32)
+        for i in range(n):
+            assert np.all(p[i] == vals[i]), "the oracle takes one parameter value per item"
+        return vals
+    return _per_item(p, n, np.float32)
+
+
+def _plan(fn, name, keep, tag=None):
+    plan = PythonPlan(fn, name=name, tag=tag)
+    plan.keep = keep  # arrays whose memory the bound C call reads
+    return plan
+
+
+# --------------------------------------------------------------------- GEMV
+class plan_block_gemv:
+    """``Y = beta*Y_in + gamma + alpha * sum_j A[A_js[j]] @ X[X_js[j]]`` in the
+    block order of clra_gemv.py:861-1175 (32x128 tiles, 4 strided partial sums)."""
+
+    def __init__(self, queue, alpha, A, A_js, X, X_js, beta, Y, Y_in=None, gamma=0.0, tag=None):
+        Y_in = Y if Y_in is None else Y_in
+        n = len(Y)
+        dot_ptr = [0]
+        a_idx, x_idx = [], []
+        for b in range(n):
+            aj = np.asarray(A_js[b]).ravel().tolist()
+            xj = np.asarray(X_js[b]).ravel().tolist()
+            assert len(aj) == len(xj)
+            for a, x in zip(aj, xj):
+                assert A.shape0s[a] == Y.shape0s[b]
+                assert A.shape1s[a] == X.shape0s[x] and X.shape1s[x] == 1
+                assert A.stride1s[a] == 1 or A.shape1s[a] == 1
+            a_idx += aj
+            x_idx += xj
+            dot_ptr.append(len(a_idx))
+        a_idx = np.asarray(a_idx, dtype=np.int64)
+        x_idx = np.asarray(x_idx, dtype=np.int64)
+        args = [
+            _i32(Y.starts), _i32(Y.stride0s), _i32(Y.shape0s), _i32(Y_in.starts),
+            _i32(Y_in.stride0s), _i32(dot_ptr), _i32(A.starts[a_idx]), _i32(A.stride0s[a_idx]),
+            _i32(A.shape1s[a_idx]), _i32(X.starts[x_idx]), _i32(X.stride0s[x_idx]),
+            _per_item(alpha, n, np.float64), _per_item(beta, n, np.float64),
+            _per_item(gamma, n, np.float64),
+        ]
+        fn = lib().orc_gemv_block
+
+        def step():
+            fn(ctypes.c_int(n), *[_p(a) for a in args], _p(A.buf), _p(X.buf), _p(Y_in.buf),
+               _p(Y.buf))
+
+        self.plans = [_plan(step, "oracle_gemv_block", args, tag)]
+
+
+plan_ragged_gather_gemv = plan_block_gemv
+
+
+# ------------------------------------------------------------------ neurons
+def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, upsample=1, tag=None, **kwargs):
+    assert not kwargs.get("fastlif") and kwargs.get("N") is None
+    n = len(J)
+    args = [_i32(J.shape0s), _i32(J.starts), _i32(V.starts), _i32(W.starts), _i32(outS.starts),
+            _param_per_item(tau, n), _param_per_item(ref, n), _param_per_item(amp, n)]
+    fn = lib().orc_lif
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], ctypes.c_double(dt), ctypes.c_int(upsample),
+           _p(J.buf), _p(V.buf), _p(W.buf), _p(outS.buf))
+
+    return _plan(step, "oracle_lif", args, tag)
+
+
+def plan_lif_rate(queue, dt, J, R, ref, tau, amp, tag=None, **kwargs):
+    assert kwargs.get("N") is None
+    n = len(J)
+    args = [_i32(J.shape0s), _i32(J.starts), _i32(R.starts), _param_per_item(tau, n),
+            _param_per_item(ref, n), _param_per_item(amp, n)]
+    fn = lib().orc_lif_rate
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(J.buf), _p(R.buf))
+
+    return _plan(step, "oracle_lif_rate", args, tag)
+
+
+# ----------------------------------------------------------------- synapses
+def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
+    n = len(X)
+    xpos = np.zeros(n, dtype=np.int32)
+    ypos = np.zeros(n, dtype=np.int32)
+    args = [_i32(X.shape0s), _i32(X.shape1s), _i32(X.starts), _i32(X.stride0s), _i32(X.stride1s),
+            _i32(Y.starts), _i32(Y.stride0s), _i32(Y.stride1s), _i32(A.shape0s), _i32(A.starts),
+            _i32(B.shape0s), _i32(B.starts), _i32(Xbuf.starts), _i32(Ybuf.starts), xpos, ypos]
+    fn = lib().orc_linearfilter
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(X.buf), _p(Y.buf), _p(A.buf), _p(B.buf),
+           _p(Xbuf.buf), _p(Ybuf.buf))
+
+    plan = _plan(step, "oracle_linearfilter", args, tag)
+    plan.bufpos = (xpos, ypos)
+    return [plan]
+
+
+# -------------------------------------------------------------- elementwise
+def plan_elementwise_inc(queue, A, X, Y, alpha=None, outer=False, inc=True, tag=None):
+    n = len(Y)
+    alphas = _per_item(1.0 if alpha is None else alpha, n, np.float32)
+    args = [alphas, _i32(A.starts), _i32(A.shape0s), _i32(A.shape1s), _i32(A.stride0s),
+            _i32(X.starts), _i32(X.shape0s), _i32(X.shape1s), _i32(X.stride0s),
+            _i32(Y.starts), _i32(Y.shape0s), _i32(Y.shape1s), _i32(Y.stride0s)]
+    fn = lib().orc_elementwise_inc
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], ctypes.c_int(bool(outer)),
+           ctypes.c_int(bool(inc)), _p(A.buf), _p(X.buf), _p(Y.buf))
+
+    return _plan(step, "oracle_elementwise_inc", args, tag)
+
+
+def plan_copy(queue, X, Y, incs, tag=None):
+    n = len(X)
+    args = [_i32(X.shape0s), _i32(X.shape1s), _i32(X.starts), _i32(X.stride0s), _i32(Y.starts),
+            _i32(Y.stride0s), _i32(incs)]
+    fn = lib().orc_copy
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(X.buf), _p(Y.buf))
+
+    return _plan(step, "oracle_copy", args, tag)
+
+
+def plan_slicedcopy(queue, X, Y, Xinds, Yinds, incs, tag=None):
+    n = len(X)
+    args = [_i32(X.starts), _i32(X.stride0s), _i32(Y.starts), _i32(Y.stride0s),
+            _i32(Xinds.shape0s), _i32(Xinds.starts), _i32(Yinds.starts), _i32(incs)]
+    fn = lib().orc_slicedcopy
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(X.buf), _p(Y.buf), _p(Xinds.buf),
+           _p(Yinds.buf))
+
+    return _plan(step, "oracle_slicedcopy", args, tag)
+
+
+def plan_reset(queue, Y, values, tag=None):
+    n = len(Y)
+    args = [_i32(Y.starts), _i32(Y.sizes), _f32(values)]
+    fn = lib().orc_reset
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(Y.buf))
+
+    return _plan(step, "oracle_reset", args, tag)
+
+
+def plan_timeupdate(queue, step, time, dt):
+    fn = lib().orc_timeupdate
+    isz = 4
+
+    def run():
+        fn(ctypes.c_void_p(step.buf.ctypes.data + isz * int(step.starts[0])),
+           ctypes.c_void_p(time.buf.ctypes.data + isz * int(time.starts[0])),
+           ctypes.c_double(dt))
+
+    return _plan(run, "oracle_timeupdate", [])
+
+
+# --------------------------------------------------------- inputs / outputs
+def plan_presentinput(queue, Y, t, signals, dt, pres_t=None, tag=None):
+    n = len(Y)
+    pres = None if pres_t is None else _f32(pres_t)
+    args = [_i32(Y.starts), _i32(Y.shape0s), _i32(t.starts), _i32(signals.starts),
+            _i32(signals.shape0s)]
+    fn = lib().orc_presentinput
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(pres), ctypes.c_float(dt), _p(Y.buf),
+           _p(t.buf), _p(signals.buf))
+
+    return _plan(step, "oracle_presentinput", args + [pres], tag)
+
+
+UNARY_OPCODES = {"identity": 0, "sin": 1, "cos": 2, "tanh": 3, "exp": 4, "square": 5}
+
+
+def plan_direct_unary(queue, fn_name, x, output, tag=None):
+    """y[0] = f(x[0]) per item for a named function of the unary table."""
+    n = len(output)
+    args = [_i32(x.starts), _i32(output.starts)]
+    fn = lib().orc_direct_unary
+    opcode = UNARY_OPCODES[fn_name]
+
+    def step():
+        fn(ctypes.c_int(opcode), ctypes.c_int(n), *[_p(a) for a in args], _p(x.buf),
+           _p(output.buf))
+
+    return _plan(step, "oracle_direct", args, tag)
+
+
+def plan_probes(queue, periods, X, Y, tag=None):
+    n = len(X)
+    periods = _f32(periods)
+    countdowns = periods - np.float32(1)
+    bufpositions = np.zeros(n, dtype=np.int32)
+    args = [countdowns, bufpositions, periods, _i32(X.starts), _i32(X.shape0s), _i32(X.shape1s),
+            _i32(X.stride0s), _i32(X.stride1s), _i32(Y.starts)]
+    fn = lib().orc_probes
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(X.buf), _p(Y.buf))
+
+    plan = _plan(step, "oracle_probes", args, tag)
+    plan.bufpositions = bufpositions
+    plan.countdowns = countdowns
+    plan.periods = periods
+    plan.Y = Y
+    return plan

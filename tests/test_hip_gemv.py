@@ -1,0 +1,248 @@
+"""GPU parity of the ragged gather-GEMV against the CPU oracle.
+
+Shapes, seeds and parameters follow the reference's own GEMV tests
+(nengo_ocl/tests/test_clra_gemv.py: test_basic :60-93, _test_random :96-145,
+check_from_shapes :165-217 and the shape cases :220-289).  Every case runs
+through all planner classes.  Tolerance: rtol 1e-4 / atol 1e-5 against the
+oracle (block summation order of the reference) and against a float64
+accumulate; the summation order of the HIP kernels differs from the oracle's,
+so this comparison is tolerance based, not bit based.
+"""
+
+import numpy as np
+import pytest
+
+from helpers import RA, clone, to_dev
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def planners():
+    from nengo_ocl_amd import hipra_gemv as g
+
+    return [g.plan_block_gemv, g.plan_ragged_gather_gemv, g.plan_reduce_gemv,
+            g.plan_many_dots_gemv, g.plan_ref_gemv]
+
+
+PLANNER_NAMES = ["block", "ragged_gather", "reduce", "many_dots", "ref"]
+
+
+def run_case(queue, planner, alpha, beta, gamma, A, X, Y, A_js, X_js, Y_in=None):
+    from oracle import oracle as orc
+
+    # float64 expectation
+    expect = []
+    Yin_host = Y if Y_in is None else Y_in
+    for i in range(len(Y)):
+        acc = np.zeros(Y[i].shape, dtype=np.float64)
+        for aj, xj in zip(np.asarray(A_js[i]).ravel(), np.asarray(X_js[i]).ravel()):
+            acc += A[int(aj)].astype(np.float64) @ X[int(xj)].astype(np.float64)
+        a = np.asarray(alpha, dtype=np.float64).reshape(-1)
+        b = np.asarray(beta, dtype=np.float64).reshape(-1)
+        g = np.asarray(gamma, dtype=np.float64).reshape(-1)
+        expect.append(g[i % g.size] + b[i % b.size] * Yin_host[i].astype(np.float64)
+                      + a[i % a.size] * acc)
+
+    # oracle (reference block order, float32)
+    Yo = clone(Y)
+    Yo_in = Yo if Y_in is None else clone(Y_in)
+    orc.plan_block_gemv(None, alpha, A, A_js, X, X_js, beta, Yo, Y_in=Yo_in, gamma=gamma).plans[0]()
+
+    dA, dX, dY = to_dev(queue, A), to_dev(queue, X), to_dev(queue, Y)
+    dYin = None if Y_in is None else to_dev(queue, Y_in)
+    prog = planner(queue, alpha, dA, A_js, dX, X_js, beta, dY, Y_in=dYin, gamma=gamma)
+    assert len(prog.plans) >= 1
+    for plan in prog.plans:
+        plan()
+    got = dY.to_host()
+    for i in range(len(Y)):
+        scale = max(1.0, float(np.abs(expect[i]).max()) if expect[i].size else 1.0)
+        np.testing.assert_allclose(got[i], Yo[i], rtol=RTOL, atol=ATOL * scale)
+        np.testing.assert_allclose(got[i], expect[i], rtol=RTOL, atol=ATOL * scale)
+    # inputs untouched
+    assert np.array_equal(dA.buf, A.buf) and np.array_equal(dX.buf, X.buf)
+    return prog
+
+
+@pytest.mark.parametrize("pi", range(5), ids=PLANNER_NAMES)
+def test_basic_literal(queue, pi):
+    """Literal vectors of test_clra_gemv.py:60-93: Y0 = 4.5, Y1 = [3.3, 5.9]."""
+    A = RA([[[0.1, 0.2], [0.3, 0.4]], [[0.5, 0.6]]])
+    X = RA([[3, 5]])
+    Y = RA([[0.0], [2, 3]])
+    A_js = RA([[1], [0]], dtype=np.int32)
+    X_js = RA([[0], [0]], dtype=np.int32)
+    dA, dX, dY = to_dev(queue, A), to_dev(queue, X), to_dev(queue, Y)
+    prog = planners()[pi](queue, 1.0, dA, A_js, dX, X_js, 1.0, dY)
+    for plan in prog.plans:
+        plan()
+    np.testing.assert_allclose(dY[0].ravel(), [4.5], rtol=1e-6)
+    np.testing.assert_allclose(dY[1].ravel(), [3.3, 5.9], rtol=1e-6)
+
+
+def _random_case(queue, planner, k, p, m, n, align):
+    rng = np.random.RandomState(3294)
+    aa = [rng.normal(size=(m, n)) for _ in range(k)]
+    xx = [rng.normal(size=n) for _ in range(k)]
+    yy = [rng.normal(size=m) for _ in range(k)]
+    ajs = [rng.randint(k, size=p) for _ in range(k)]
+    xjs = [rng.randint(k, size=p) for _ in range(k)]
+    run_case(queue, planner, 0.5, 0.1, 0.0, RA(aa, align=align), RA(xx), RA(yy),
+             RA(ajs, dtype=np.int32), RA(xjs, dtype=np.int32))
+
+
+@pytest.mark.parametrize("align", [False, True], ids=["packed", "aligned"])
+@pytest.mark.parametrize("pi", range(5), ids=PLANNER_NAMES)
+@pytest.mark.parametrize("k,p,m,n", [(4, 1, 10, 10), (10, 1, 550, 550), (4, 4, 10, 10),
+                                     (4, 4, 2000, 1000)],
+                         ids=["small", "large", "many_dots_small", "many_dots_large"])
+def test_random(queue, pi, k, p, m, n, align):
+    _random_case(queue, planners()[pi], k, p, m, n, align)
+
+
+def _from_shapes(queue, planner, alpha, beta, gamma, A_shapes, X_shapes, A_js, X_js, align=False):
+    rng = np.random.RandomState(1234)
+    A = RA([0.1 + rng.rand(*shp) for shp in A_shapes], align=align)
+    X = RA([0.1 + rng.rand(*shp) for shp in X_shapes])
+    Y = RA([0.1 + rng.rand(A_shapes[A_js[i][0]][0], X_shapes[X_js[i][0]][1])
+            for i in range(len(A_js))])
+    run_case(queue, planner, alpha, beta, gamma, A, X, Y,
+             RA([list(a) for a in A_js], dtype=np.int32), RA([list(x) for x in X_js], dtype=np.int32))
+
+
+@pytest.mark.parametrize("pi", range(5), ids=PLANNER_NAMES)
+@pytest.mark.parametrize("rows", [1, 10, 2001])
+def test_one_segment(queue, pi, rows):
+    _from_shapes(queue, planners()[pi], 0.5, 0.6, 0.7, [(rows, 1)], [(1, 1)], [[0]], [[0]])
+
+
+@pytest.mark.parametrize("pi", range(5), ids=PLANNER_NAMES)
+@pytest.mark.parametrize("ND", [2, 20, 100])
+def test_one_short_segment_many_dots(queue, pi, ND):
+    _from_shapes(queue, planners()[pi], 0.5, 0.6, 0.7,
+                 [(10, 1 + i % 2) for i in range(ND)], [(1 + i % 2, 1) for i in range(ND)],
+                 [range(ND)], [range(ND)])
+
+
+@pytest.mark.parametrize("pi", range(5), ids=PLANNER_NAMES)
+@pytest.mark.parametrize("ND", [2, 20, 100])
+def test_one_short_segment_many_longer_dots(queue, pi, ND):
+    _from_shapes(queue, planners()[pi], 0.5, 0.6, 0.7,
+                 [(2000, i + 1) for i in range(ND)], [(i + 1, 1) for i in range(ND)],
+                 [range(ND)], [range(ND)], align=True)
+
+
+@pytest.mark.parametrize("pi", [0, 2, 3], ids=["block", "reduce", "many_dots"])
+def test_ensemble_shapes(queue, pi):
+    """The shapes the benchmark configurations produce: encoders (n x d, tall and
+    thin), decoders (d x n, short and wide), per-neuron scalars, single dots."""
+    rng = np.random.RandomState(7)
+    shapes = [(4096, 64), (64, 4096), (100, 1), (1, 100), (100, 2), (2, 100), (2000, 32),
+              (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000)]
+    A = RA([rng.normal(size=s) for s in shapes], align=True)
+    X = RA([rng.normal(size=s[1]) for s in shapes], align=True)
+    Y = RA([rng.normal(size=s[0]) for s in shapes], align=True)
+    js = RA([[i] for i in range(len(shapes))], dtype=np.int32)
+    prog = run_case(queue, planners()[pi], 1.0, 1.0, 0.0, A, X, Y, js, js)
+    if pi == 0:
+        classes = {p.kernel_class for p in prog.plans}
+        assert (0, 16, 4) in classes and (0, 256, 4) in classes and any(c[0] == 1 for c in classes)
+
+
+def test_strided_views_and_yin(queue):
+    """A is a column slice of a wider matrix (row stride > columns, one aligned and
+    one unaligned), X and Y are strided views of vectors, Y_in differs from Y, and
+    alpha / beta / gamma differ per item."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from nengo_ocl_amd.hipraggedarray import HIPRaggedArray
+    from nengo_ocl_amd.raggedarray import RaggedArray
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(11)
+    base = RA([rng.normal(size=(40, 96)), rng.normal(size=(200,)), rng.normal(size=(80,)),
+               rng.normal(size=(70,)), rng.normal(size=(70, 33))], align=True)
+    s = base.starts
+    # items 5..8: A0 = base0[:, 32:80]; X0 = base1[0::4][:48]; A1 = base4[:, 1:33]; X1 = base1[3::5][:32]
+    base.add_views([s[0] + 32, s[1], s[4] + 1, s[1] + 3], [40, 48, 70, 32], [48, 1, 32, 1],
+                   [96, 4, 33, 5], [1, 1, 1, 1])
+    A_js = RA([[5], [7]], dtype=np.int32)
+    X_js = RA([[6], [8]], dtype=np.int32)
+    y_meta = ([s[2], s[3]], [40, 70], [1, 1], [2, 1], [1, 1])  # Y0 = base2[::2], Y1 = base3
+    Yin = RA([rng.normal(size=40), rng.normal(size=70)])
+    alpha, beta, gamma = [0.5, -1.5], [1.0, 0.25], [0.0, 2.0]
+
+    host = clone(base)
+    Yo = RaggedArray.from_buffer(host.buf, *y_meta)
+    orc.plan_block_gemv(None, alpha, host, A_js, host, X_js, beta, Yo, Y_in=clone(Yin),
+                        gamma=gamma).plans[0]()
+
+    dbase = to_dev(queue, base)
+    dY = HIPRaggedArray.from_buffer(queue, dbase.dev_buf, *y_meta)
+    prog = g.plan_block_gemv(queue, alpha, dbase, A_js, dbase, X_js, beta, dY,
+                             Y_in=to_dev(queue, Yin), gamma=gamma)
+    for plan in prog.plans:
+        plan()
+    got = dbase.buf
+    np.testing.assert_allclose(got, host.buf, rtol=RTOL, atol=1e-4)
+    changed = got != base.buf
+    expect_changed = np.zeros_like(changed)
+    expect_changed[s[2]:s[2] + 80:2] = True
+    expect_changed[s[3]:s[3] + 70] = True
+    assert np.array_equal(changed, expect_changed)  # nothing outside Y was written
+
+
+def test_empty_dot_list_and_zero_rows(queue):
+    """An output with no dot products is just beta*Y_in + gamma; zero-length outputs are skipped."""
+    from nengo_ocl_amd import hipra_gemv as g
+
+    A = RA([np.ones((3, 2))])
+    X = RA([np.ones(2)])
+    Y = RA([np.arange(3.0), np.arange(5.0)])
+    A_js = [np.array([0], dtype=np.int32), np.array([], dtype=np.int32)]
+    X_js = [np.array([0], dtype=np.int32), np.array([], dtype=np.int32)]
+    dY = to_dev(queue, Y)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), A_js, to_dev(queue, X), X_js, 2.0, dY,
+                             gamma=1.0)
+    for plan in prog.plans:
+        plan()
+    np.testing.assert_allclose(dY[0].ravel(), 2 * np.arange(3.0) + 1 + 2)
+    np.testing.assert_allclose(dY[1].ravel(), 2 * np.arange(5.0) + 1)
+
+
+def test_bad_arguments_raise(queue):
+    from nengo_ocl_amd import hipra_gemv as g
+
+    A = to_dev(queue, RA([np.ones((3, 2))]))
+    X = to_dev(queue, RA([np.ones(3)]))
+    Y = to_dev(queue, RA([np.zeros(3)]))
+    js = RA([[0]], dtype=np.int32)
+    with pytest.raises(ValueError):
+        g.plan_block_gemv(queue, 1.0, A, js, X, js, 1.0, Y)  # 2 columns vs 3-vector
+
+
+def test_linearity_at_full_size(queue):
+    """Size-independent property at the large configuration's shapes: the GEMV is
+    linear in X, so A@(2x) - 2*(A@x) == 0 up to rounding, and A@e_k picks column k
+    bit-exactly (gather check)."""
+    from nengo_ocl_amd import hipra_gemv as g
+
+    rng = np.random.RandomState(5)
+    n_ens, n, d = 8, 4096, 64
+    enc = [rng.normal(size=(n, d)).astype(np.float32) for _ in range(n_ens)]
+    dec = [rng.normal(size=(d, n)).astype(np.float32) for _ in range(n_ens)]
+    k_enc, k_dec = 37, 2049
+    ex, dx = np.zeros(d, np.float32), np.zeros(n, np.float32)
+    ex[k_enc], dx[k_dec] = 1.0, 1.0
+    A = RA(enc + dec, align=True)
+    X = RA([ex] * n_ens + [dx] * n_ens, align=True)
+    Y = RA([np.zeros(n)] * n_ens + [np.zeros(d)] * n_ens, align=True)
+    js = RA([[i] for i in range(2 * n_ens)], dtype=np.int32)
+    dY = to_dev(queue, Y)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, 0.0, dY)
+    for plan in prog.plans:
+        plan()
+    for i in range(n_ens):
+        assert np.array_equal(dY[i].ravel(), enc[i][:, k_enc])
+        assert np.array_equal(dY[n_ens + i].ravel(), dec[i][:, k_dec])

@@ -1,0 +1,354 @@
+"""GPU parity of the non-GEMV timestep kernels against the CPU oracle.
+
+Cases follow nengo_ocl/tests/test_clra_nonlinearities.py: test_lif_step :35-91,
+test_lif_rate :141-173, test_copy :176-191, test_elementwise_inc :194-227,
+test_elementwise_inc_outer :230-251, test_reset :254-279, test_slicedcopy
+:282-326, test_linearfilter :329-406.  Index / copy / fill / single-rounding
+arithmetic is compared bit for bit; LIF state within 1e-6 wherever the spike
+decision agrees (device expm1/log1p differ from libm in the last ulp, so a
+neuron sitting exactly on the threshold may decide differently: the share of
+such neurons is bounded at 1e-4 and printed).
+"""
+
+import numpy as np
+import pytest
+
+from helpers import RA, clone, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def nl():
+    from nengo_ocl_amd import hipra_nonlinearities
+
+    return hipra_nonlinearities
+
+
+def orc():
+    from oracle import oracle
+
+    return oracle
+
+
+@pytest.mark.parametrize("param_kind", ["float", "ragged_const", "ragged_varying"])
+@pytest.mark.parametrize("upsample", [1, 4])
+def test_lif_step(queue, rng, upsample, param_kind):
+    dt = 1e-3
+    n_neurons = [12345, 23456, 34567]
+    J = RA([rng.normal(scale=1.2, size=n) for n in n_neurons])
+    V = RA([rng.uniform(low=0, high=1, size=n) for n in n_neurons])
+    W = RA([rng.uniform(low=-5 * dt, high=5 * dt, size=n) for n in n_neurons])
+    OS = RA([np.zeros(n) for n in n_neurons])
+    ref, amp = 2e-3, 1.0
+    taus = rng.uniform(low=15e-3, high=80e-3, size=len(n_neurons))
+
+    if param_kind == "ragged_varying":
+        # per-neuron taus: the oracle takes one value per item, so check each neuron
+        # against an oracle run on single-tau items instead
+        tau_arrays = [rng.choice([0.02, 0.05], size=n) for n in n_neurons]
+    else:
+        tau_arrays = [t * np.ones(n) for t, n in zip(taus, n_neurons)]
+
+    dJ, dV, dW, dOS = (to_dev(queue, x) for x in (J, V, W, OS))
+    if param_kind == "float":
+        taus = np.full(len(n_neurons), 0.02)
+        tau_arrays = [0.02 * np.ones(n) for n in n_neurons]
+        plan = nl().plan_lif(queue, dt, dJ, dV, dW, dOS, ref, 0.02, amp, upsample=upsample)
+    else:
+        dTau = to_dev(queue, RA(tau_arrays))
+        plan = nl().plan_lif(queue, dt, dJ, dV, dW, dOS, ref, dTau, amp, upsample=upsample)
+    plan()
+
+    # oracle: split every item by tau value so that each oracle item has one tau
+    Vo, Wo, So = clone(V), clone(W), clone(OS)
+    for i, n in enumerate(n_neurons):
+        for tau in np.unique(np.float32(tau_arrays[i])):
+            sel = np.nonzero(np.float32(tau_arrays[i]) == tau)[0]
+            j, v, w, s = (RA([x[i].ravel()[sel]]) for x in (J, V, W, OS))
+            orc().plan_lif(None, dt, j, v, w, s, ref, float(tau), amp, upsample=upsample)()
+            Vo[i][sel, 0], Wo[i][sel, 0], So[i][sel, 0] = v[0].ravel(), w[0].ravel(), s[0].ravel()
+
+    gV, gW, gS = dV.to_host(), dW.to_host(), dOS.to_host()
+    assert np.array_equal(dJ.buf, J.buf)
+    n_total = sum(n_neurons)
+    same = (gS.buf > 0) == (So.buf > 0)
+    n_diff = int(n_total - same.sum())
+    print("LIF spike decisions differing from the oracle: %d of %d" % (n_diff, n_total))
+    assert n_diff <= 1e-4 * n_total
+    assert So.buf.sum() > 0, "spiking mechanism not exercised"
+    np.testing.assert_allclose(gV.buf[same], Vo.buf[same], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(gW.buf[same], Wo.buf[same], rtol=1e-5, atol=1e-6)
+    assert np.array_equal(gS.buf[same], So.buf[same])
+    assert set(np.unique(gS.buf)) <= {0.0, np.float32(amp / dt)}
+
+
+def test_lif_rate(queue, rng):
+    n_neurons = [123459, 23456, 34567]
+    J = RA([rng.normal(loc=1, scale=10, size=n) for n in n_neurons])
+    R = RA([np.zeros(n) for n in n_neurons])
+    ref, amp = 2e-3, 1.0
+    taus = list(rng.uniform(low=15e-3, high=80e-3, size=len(n_neurons)))
+    tau_ra = RA([t * np.ones(n) for t, n in zip(taus, n_neurons)])
+
+    dJ, dR = to_dev(queue, J), to_dev(queue, R)
+    nl().plan_lif_rate(queue, 1e-3, dJ, dR, ref, to_dev(queue, tau_ra), amp)()
+    Ro = clone(R)
+    orc().plan_lif_rate(None, 1e-3, J, Ro, ref, tau_ra, amp)()
+    got = dR.to_host()
+    assert np.array_equal(dJ.buf, J.buf)
+    assert Ro.buf.sum() > 1.0
+    assert np.array_equal(got.buf == 0, Ro.buf == 0)  # silent below threshold, exactly
+    np.testing.assert_allclose(got.buf, Ro.buf, rtol=1e-5, atol=1e-4)
+
+
+def test_copy(queue, rng):
+    sizes = [(10, 1), (40, 64), (457, 342), (1, 100), (3000, 1)]
+    X = RA([rng.normal(size=s) for s in sizes])
+    Y0 = RA([rng.normal(size=s) for s in sizes])
+    incs = np.array([0, 1, 1, 0, 1], dtype=np.int32)
+    dX, dY = to_dev(queue, X), to_dev(queue, Y0)
+    nl().plan_copy(queue, dX, dY, incs)()
+    Yo = clone(Y0)
+    orc().plan_copy(None, X, Yo, incs)()
+    got = dY.to_host()
+    assert np.array_equal(got.buf, Yo.buf)
+    for i, inc in enumerate(incs):
+        assert np.array_equal(got[i], Y0[i] + X[i] if inc else X[i])
+
+
+def test_copy_strided_rows(queue, rng):
+    """Source and target are column slices of wider matrices (row stride > columns)."""
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    base = RA([rng.normal(size=(30, 50)), rng.normal(size=(30, 70))])
+    s = base.starts
+    X = RaggedArray.from_buffer(base.buf, [s[0] + 5], [30], [20], [50], [1])
+    Y = RaggedArray.from_buffer(base.buf, [s[1] + 40], [30], [20], [70], [1])
+    from nengo_ocl_amd.hipraggedarray import HIPRaggedArray
+
+    d = to_dev(queue, base)
+    dX = HIPRaggedArray.from_buffer(queue, d.dev_buf, X.starts, X.shape0s, X.shape1s, X.stride0s, X.stride1s)
+    dY = HIPRaggedArray.from_buffer(queue, d.dev_buf, Y.starts, Y.shape0s, Y.shape1s, Y.stride0s, Y.stride1s)
+    nl().plan_copy(queue, dX, dY, np.array([1], dtype=np.int32))()
+    expect = np.array(base.buf)
+    e = RaggedArray.from_buffer(expect, base.starts, base.shape0s, base.shape1s, base.stride0s, base.stride1s)
+    e[1][:, 40:60] += e[0][:, 5:25]
+    assert np.array_equal(d.buf, expect)
+
+
+@pytest.mark.parametrize("use_alpha", [False, True])
+@pytest.mark.parametrize("inc", [True, False])
+def test_elementwise_inc(queue, rng, inc, use_alpha):
+    Xsizes = [(3, 3), (32, 64), (457, 342), (1, 100)]
+    Asizes = [(3, 3), (1, 1), (457, 342), (100, 1)]
+    A = RA([rng.normal(size=s) for s in Asizes])
+    X = RA([rng.normal(size=s) for s in Xsizes])
+    alpha = rng.normal(size=len(Xsizes)).astype(np.float32) if use_alpha else None
+    Yshapes = [np.broadcast(A[i], X[i]).shape for i in range(len(Xsizes))]
+    Y = RA([rng.normal(size=s) for s in Yshapes])
+
+    dY = to_dev(queue, Y)
+    nl().plan_elementwise_inc(queue, to_dev(queue, A), to_dev(queue, X), dY, alpha=alpha, inc=inc)()
+    Yo = clone(Y)
+    orc().plan_elementwise_inc(None, A, X, Yo, alpha=alpha, inc=inc)()
+    got = dY.to_host()
+    assert np.array_equal(got.buf, Yo.buf)
+    for k in range(len(Y)):  # library expression, float32: (alpha*a)*x then one add
+        al = np.float32(1.0) if alpha is None else alpha[k]
+        ax = (al * A[k]) * X[k]
+        assert np.array_equal(got[k], Y[k] + ax if inc else ax), k
+
+
+def test_elementwise_inc_outer(queue, rng):
+    Xsizes = [3, 9, 15, 432]
+    Asizes = [9, 42, 10, 124]
+    alpha = rng.normal(size=len(Xsizes)).astype(np.float32)
+    A = RA([rng.normal(size=s) for s in Asizes])
+    X = RA([rng.normal(size=s) for s in Xsizes])
+    Y = RA([rng.normal(size=(a, x)) for a, x in zip(Asizes, Xsizes)])
+    for inc in (True, False):
+        dY = to_dev(queue, Y)
+        nl().plan_elementwise_inc(queue, to_dev(queue, A), to_dev(queue, X), dY, alpha=alpha,
+                                  outer=True, inc=inc)()
+        got = dY.to_host()
+        for k in range(len(Y)):
+            ax = np.outer(alpha[k] * A[k].ravel(), X[k].ravel())
+            assert np.array_equal(got[k], Y[k] + ax if inc else ax)
+
+
+def test_reset(queue, rng):
+    Yshapes = [(1000000,), (1000, 1700), (3, 3), (1,), (4097,)]
+    values = rng.uniform(size=len(Yshapes)).astype(np.float32)
+    dY = to_dev(queue, RA([np.ones(s) for s in Yshapes]))
+    nl().plan_reset(queue, dY, values)()
+    got = dY.to_host()
+    for i, v in enumerate(values):
+        assert np.all(got[i] == v)
+
+
+def test_slicedcopy(queue, rng):
+    sizes = rng.randint(20, 200, size=10)
+    A = RA([rng.normal(size=s) for s in sizes])
+    B = RA([rng.normal(size=s) for s in sizes])
+    incs = rng.randint(0, 2, size=len(sizes)).astype(np.int32)
+    Ainds, Binds = [], []
+    for k, size in enumerate(sizes):
+        r = np.arange(size, dtype=np.int32)
+        u = k % 3
+        if u == 0:
+            Ainds.append(r)
+            Binds.append(r)
+        elif u == 1:
+            Ainds.append(r[:10])
+            Binds.append(r[-10:])
+        else:
+            n = rng.randint(2, size - 2)
+            Ainds.append(rng.permutation(size)[:n])
+            Binds.append(rng.permutation(size)[:n])
+    Ainds, Binds = RA(Ainds, dtype=np.int32), RA(Binds, dtype=np.int32)
+
+    dB = to_dev(queue, B)
+    nl().plan_slicedcopy(queue, to_dev(queue, A), dB, to_dev(queue, Ainds), to_dev(queue, Binds), incs)()
+    Bo = clone(B)
+    orc().plan_slicedcopy(None, A, Bo, Ainds, Binds, incs)()
+    expect = clone(B)
+    for i in range(len(sizes)):
+        ai, bi = Ainds[i].ravel(), Binds[i].ravel()
+        if incs[i]:
+            expect[i][bi, 0] += A[i][ai, 0]
+        else:
+            expect[i][bi, 0] = A[i][ai, 0]
+    got = dB.to_host()
+    assert np.array_equal(got.buf, expect.buf)
+    assert np.array_equal(Bo.buf, expect.buf)
+
+
+def _filter_coefficients(kind, dt=1e-3):
+    """(num, den) of the discrete filter in the reference's packing
+    (simulator.py:1214-1227): zero-order-hold discretisation, leading zero of the
+    numerator and leading one of the denominator dropped."""
+    from scipy.signal import cont2discrete
+
+    if kind == "gain":
+        return np.array([2.0]), np.array([])
+    tau = 0.005
+    num, den = ([1.0], [tau, 1.0]) if kind == "lowpass" else ([1.0], [tau * tau, 2 * tau, 1.0])
+    numd, dend, _ = cont2discrete((num, den), dt, method="zoh")
+    numd = numd.ravel() / dend[0]
+    dend = dend / dend[0]
+    numd = numd[1:] if numd[0] == 0 else numd
+    return numd, dend[1:]
+
+
+@pytest.mark.parametrize("n_per_kind", [(100000, 0, 0), (0, 100000, 0), (0, 0, 100000),
+                                        (10000, 10000, 10000)])
+def test_linearfilter(queue, rng, n_per_kind):
+    from scipy.signal import lfilter
+
+    kinds = [(k, n) for k, n in zip(("gain", "lowpass", "alpha"), n_per_kind) if n > 0]
+    coefs = [_filter_coefficients(k) for k, _ in kinds]
+    A = RA([den for _, den in coefs])
+    B = RA([num for num, _ in coefs])
+    n_calls = 5
+    xs = [[rng.normal(size=n) for _, n in kinds] for _ in range(n_calls)]
+    X = RA(xs[0])
+    Y = RA([np.zeros(n) for _, n in kinds])
+    Xbuf = RA([np.zeros(s) for s in zip(B.sizes, X.sizes)])
+    Ybuf = RA([np.zeros(s) for s in zip(A.sizes, Y.sizes)])
+
+    dX, dY = to_dev(queue, X), to_dev(queue, Y)
+    plans = nl().plan_linearfilter(queue, dX, dY, to_dev(queue, A), to_dev(queue, B),
+                                   to_dev(queue, Xbuf), to_dev(queue, Ybuf))
+    Xo, Yo = clone(X), clone(Y)
+    oplans = orc().plan_linearfilter(None, Xo, Yo, A, B, clone(Xbuf), clone(Ybuf))
+    for c in range(n_calls):
+        for i in range(len(kinds)):
+            dX[i] = xs[c][i]
+            Xo[i] = xs[c][i][:, None]
+        for p in plans:
+            p()
+        for p in oplans:
+            p()
+        assert np.array_equal(dY.buf, Yo.buf), "call %d" % c
+
+    # independent check of the recurrence: scipy's direct-form filter in float64 on the
+    # float32-rounded coefficients.  The step maps x[n] to y[n] with no extra delay:
+    # y[n] = sum_p b[p] x[n-p] - sum_p a[p] y[n-1-p]  ==  lfilter(b, [1, a...], x)
+    got = dY.to_host()
+    for i, (kind, n) in enumerate(kinds):
+        num, den = (np.float32(c).astype(np.float64) for c in coefs[i])
+        m = min(n, 100)
+        x_hist = np.array([np.float32(xs[c][i][:m]) for c in range(n_calls)], dtype=np.float64)
+        y = lfilter(num, np.concatenate([[1.0], den]), x_hist, axis=0)
+        np.testing.assert_allclose(got[i][:m, 0], y[-1], rtol=1e-5, atol=1e-6)
+
+
+def test_timeupdate(queue):
+    sig = RA([np.zeros(1), np.zeros(1)])
+    d = to_dev(queue, sig)
+    plan = nl().plan_timeupdate(queue, d[[0]], d[[1]], 0.001)
+    for _ in range(1234):
+        plan.enqueue()
+    plan.wait()
+    assert d[0][0, 0] == np.float32(1234)
+    assert d[1][0, 0] == np.float32(0.001 * 1234)
+
+
+@pytest.mark.parametrize("with_pres_t", [False, True])
+def test_presentinput(queue, rng, with_pres_t):
+    dt = 0.001
+    tables = [rng.normal(size=(1000, 1)), rng.normal(size=(37, 32)), rng.normal(size=(5, 300))]
+    S = RA(tables)
+    Y = RA([np.zeros(t.shape[1]) for t in tables])
+    pres = np.array([0.01, 0.05, 0.003], dtype=np.float32) if with_pres_t else None
+    for step in [0, 1, 36, 37, 999, 1000, 123456]:
+        T = RA([np.array([step], dtype=np.float32)] * len(tables))
+        dY = to_dev(queue, Y)
+        nl().plan_presentinput(queue, dY, to_dev(queue, T), to_dev(queue, S), dt, pres_t=pres)()
+        Yo = clone(Y)
+        orc().plan_presentinput(None, Yo, T, S, dt, pres_t=pres)()
+        assert np.array_equal(dY.buf, Yo.buf)
+        if not with_pres_t:
+            for i, t in enumerate(tables):
+                assert np.array_equal(dY[i].ravel(), np.float32(t[step % t.shape[0]]))
+
+
+def test_direct_sin(queue):
+    t = RA([np.array([0.731], dtype=np.float32)])
+    y = RA([np.zeros(1)])
+    dy = to_dev(queue, y)
+    plan = nl().plan_direct(queue, "OUTPUT__[0] = sin(t[0]);", "", ["t"], [to_dev(queue, t)], dy)
+    plan()
+    np.testing.assert_allclose(dy[0][0, 0], np.sin(np.float32(0.731)), rtol=1e-6)
+    with pytest.raises(NotImplementedError):
+        nl().plan_direct(queue, "OUTPUT__[0] = t[0] * x[0];", "", ["t"], [to_dev(queue, t)], dy)
+
+
+def test_probes(queue, rng):
+    """Periods 1, 2.5 (non-integer) and 10 over 40 steps with 32 buffer rows; strided source."""
+    from nengo_ocl_amd.hipraggedarray import HIPRaggedArray
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    base = RA([np.zeros(7), np.zeros((6, 10)), np.zeros(300)])
+    s = base.starts
+    src_meta = ([s[0], s[1] + 2, s[2]], [7, 6, 300], [1, 4, 1], [1, 10, 1], [1, 1, 1])
+    periods = [1.0, 2.5, 10.0]
+    n_buf = 32
+    Xh = RaggedArray.from_buffer(base.buf, *src_meta)
+    Yh = RA([np.zeros((n_buf, 7)), np.zeros((n_buf, 24)), np.zeros((n_buf, 300))])
+    d = to_dev(queue, base)
+    dX = HIPRaggedArray.from_buffer(queue, d.dev_buf, *src_meta)
+    dYp = to_dev(queue, Yh)
+    plan = nl().plan_probes(queue, periods, dX, dYp)
+    oplan = orc().plan_probes(None, periods, Xh, Yh)
+    for step in range(30):
+        vals = rng.normal(size=base.buf.size).astype(np.float32)
+        base.buf[:] = vals
+        d.dev_buf.set(vals)
+        plan()
+        oplan()
+    pos = plan.dev_bufpositions.get()
+    assert np.array_equal(pos, oplan.bufpositions)
+    assert list(pos) == [30, 12, 3]
+    assert np.array_equal(plan.dev_countdowns.get(), oplan.countdowns)
+    assert np.array_equal(dYp.buf, Yh.buf)
