@@ -318,7 +318,7 @@ extern "C" int nhip_linearfilter(void* stream, const int* desc, int* pos, int n_
                                  const float* X, float* Y, const float* A, const float* B,
                                  float* Xbuf, float* Ybuf) {
     if (n_blocks == 0) return 0;
-    if (n_blocks < 0 || !desc || !pos || !X || !Y || !A || !B) return NHIP_E_BADARG;
+    if (n_blocks < 0 || !desc || !pos || !X || !Y || !B) return NHIP_E_BADARG;  // A, Xbuf, Ybuf may be empty
     hipLaunchKernelGGL(linearfilter_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
                        reinterpret_cast<const LfDesc*>(desc), reinterpret_cast<int2*>(pos), X, Y, A,
                        B, Xbuf, Ybuf);
