@@ -1,0 +1,183 @@
+#!/usr/bin/env python
+"""Benchmark of the simulator timestep on one MI355X.
+
+``python bench.py --gpus 1 --steps K --warmup W`` builds the large
+bandwidth-bound network (256 ensembles x 4096 LIF neurons x 64-D, 1,048,576
+neurons; `nengo_ocl_amd.configs.c3_large`), runs W untimed steps, then times
+exactly K steps of ``Simulator.run_steps`` (graph replay, probes drained every
+32 steps) between stream synchronisations and prints ONE JSON line:
+
+* ``value``: simulator steps per second (inputs resident in HBM);
+* ``roofline``: for the dominant kernel (the ragged gather-GEMV launch with the
+  largest share of the step), algorithmic bytes per launch (the reference's own
+  accounting: A + X per dot, Y_in, Y) divided by its average duration, measured
+  with HIP events on the simulator's stream in a separate eager pass over the
+  same state, against the 8 TB/s HBM peak;
+* ``cpu_baseline``: the CPU oracle (C restatement of the reference kernels,
+  OpenMP) stepping the same network on the host cores for a bounded sample.
+
+Other configurations: ``--config c0|c1|c2|c4``; ``--variant per-connection``
+gives c3 with one decoder matrix per connection.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def make_network(config, variant, scale):
+    from nengo_ocl_amd import configs
+
+    if config == "c0":
+        return configs.c0_readme(), "c0: README two-ensemble net, 200 LIF neurons"
+    if config == "c1":
+        return configs.c1_circconv(dims=64), "c1: circular convolution D=64, 13,200 LIF neurons"
+    if config == "c2":
+        return (configs.c2_watts_strogatz(),
+                "c2: Watts-Strogatz, 2048 ensembles x 100 LIF, 20,480 decoded edges")
+    if config == "c3":
+        n_ens = max(2, int(round(256 * scale)))
+        share = variant == "shared"
+        desc = ("c3: %d ensembles x 4096 LIF x 64-D, fan-out 4, %s, surrogate decoders"
+                % (n_ens, "one decoder matrix per ensemble (~%d MB of matrices per step)"
+                   % (n_ens * 2) if share else
+                   "one decoder matrix per connection (~%d MB of matrices per step)" % (n_ens * 5)))
+        return configs.c3_large(n_ens=n_ens, share_decoded=share), desc
+    if config == "c4":
+        n = max(1, int(round(64 * scale)))
+        return configs.c4_pes(n_triples=n), "c4: PES, %d triples x 2000 LIF x 32-D" % n
+    raise SystemExit("unknown config %r" % config)
+
+
+def gemv_summary(sim, profile_steps):
+    """Per-plan average durations from an eager pass with HIP events around each launch."""
+    plans = sim._plans
+    plans.profiling = True
+    for p in plans:
+        p.atimes[:], p.btimes[:], p.ctimes[:] = [], [], []
+        p.n_calls = 0
+    plans.call_n_times(profile_steps)
+    plans.profiling = False
+    rows = []
+    for p in plans:
+        if p.n_calls:
+            avg = sum(p.ctimes) / p.n_calls
+            rows.append(dict(plan=str(p), name=p.name, avg_us=1e6 * avg,
+                             bytes=p.bw_per_call,
+                             gbs=(1e-9 * p.bw_per_call / avg) if p.bw_per_call and avg > 0 else None))
+    return rows
+
+
+def cpu_baseline(config, variant, scale, budget_s, dt_gpu_step):
+    from oracle import oracle
+    from oracle.oracle_sim import OracleSimulator
+
+    (net, probes, _), _ = make_network(config, variant, scale)
+    sim = OracleSimulator(net, seed=1)
+    sim.run_steps(2)  # warm caches, first-touch
+    t0 = time.perf_counter()
+    sim.run_steps(3)
+    per_step = (time.perf_counter() - t0) / 3
+    n = int(max(5, min(2000, budget_s / max(per_step, 1e-6))))
+    t0 = time.perf_counter()
+    sim.run_steps(n)
+    elapsed = time.perf_counter() - t0
+    sim.close()
+    return dict(value=n / elapsed, unit="steps/s", cores=oracle.num_threads(), kind="port",
+                sample="%d steps of the same network on the CPU oracle (C restatement of the "
+                       "reference kernels, OpenMP over items), %.1f s" % (n, elapsed))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c3")
+    ap.add_argument("--variant", default="shared", choices=["shared", "per-connection"])
+    ap.add_argument("--scale", type=float, default=1.0, help="fraction of the ensembles (c3, c4)")
+    ap.add_argument("--profile-steps", type=int, default=100)
+    ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
+    ap.add_argument("--no-fuse", action="store_true")
+    ap.add_argument("--no-graph", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: the timestep of one simulator runs on a single "
+                         "MI355X and nothing here uses a second device (got --gpus %d)" % args.gpus)
+
+    import torch
+
+    from nengo_ocl_amd.simulator import Simulator
+
+    t0 = time.time()
+    (net, probes, _), workload = make_network(args.config, args.variant, args.scale)
+    sim = Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph)
+    build_s = time.time() - t0
+    n_plans = len(sim._plans)
+
+    sim.run_steps(args.warmup)
+    torch.cuda.synchronize()
+    sim.queue.finish()
+    t0 = time.perf_counter()
+    sim.run_steps(args.steps)
+    sim.queue.finish()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    steps_per_s = args.steps / elapsed
+
+    rows = gemv_summary(sim, args.profile_steps)
+    gemv_rows = [r for r in rows if r["name"].startswith("hipra_gemv") and r["bytes"]]
+    dom = max(gemv_rows, key=lambda r: r["avg_us"]) if gemv_rows else None
+    step_us_kernels = sum(r["avg_us"] for r in rows)
+    gemv_bytes = sum(r["bytes"] for r in gemv_rows)
+    gemv_us = sum(r["avg_us"] for r in gemv_rows)
+    roofline = None
+    if dom is not None:
+        roofline = dict(bound="hbm", achieved=dom["gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
+                        frac=dom["gbs"] / HBM_PEAK_GBS, traffic=None, kernel=dom["plan"],
+                        avg_us=dom["avg_us"], bytes_per_launch=dom["bytes"])
+
+    out = {
+        "metric": "sim steps/sec + ragged-GEMV HBM GB/s (% peak), 1M-neuron LIF net, 1 MI355X",
+        "value": steps_per_s,
+        "unit": "steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": 1e3 * elapsed / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": workload, "neurons": net.n_neurons, "plans_per_step": n_plans,
+                   "dt": 0.001, "graph": not args.no_graph, "fused_copies": not args.no_fuse},
+        "roofline": roofline,
+        "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,
+                     "gbs": 1e-3 * gemv_bytes / gemv_us if gemv_us else None,
+                     "frac_of_peak": (1e-3 * gemv_bytes / gemv_us / HBM_PEAK_GBS) if gemv_us else None},
+        "kernels": [{"plan": r["plan"], "avg_us": round(r["avg_us"], 2),
+                     "gbs": None if r["gbs"] is None else round(r["gbs"], 1)} for r in rows],
+        "kernel_us_per_step": step_us_kernels,
+        "build_s": build_s,
+    }
+    sim.close()
+    del sim
+    if args.cpu_budget > 0:
+        out["cpu_baseline"] = cpu_baseline(args.config, args.variant, args.scale, args.cpu_budget,
+                                           elapsed / args.steps)
+        out["cpu_baseline"]["host_cpu_count"] = os.cpu_count()
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

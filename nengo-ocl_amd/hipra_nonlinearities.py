@@ -323,8 +323,8 @@ def plan_direct(queue, code, init, input_names, inputs, output, tag=None):
 def _neuron_params(queue, params, sizes, inds, offsets):
     """Pack tau/ref/amp for the block table.
 
-    A number, or a ragged array whose items are each constant, becomes float
-    bits in the table (one scalar per block, no per-neuron traffic).  Ragged
+    A number, an ndarray with one value per item, or a ragged array whose items
+    are each constant, becomes float bits in the table (one scalar per block, no per-neuron traffic).  Ragged
     arrays with varying values stay on the device and the table holds offsets.
     Returns (columns, pflags, device pointers, keepalive).
     """
@@ -333,6 +333,10 @@ def _neuron_params(queue, params, sizes, inds, offsets):
     for k, p in enumerate(params):
         if is_number(p):
             columns.append(np.full(len(inds), f32_bits(p), dtype=np.int32))
+            ptrs.append(None)
+            continue
+        if isinstance(p, np.ndarray) and p.shape == (len(sizes),):  # one value per item
+            columns.append(_bits(p.astype(np.float32)[inds]))
             ptrs.append(None)
             continue
         if not isinstance(p, HIPRaggedArray):

@@ -1,0 +1,434 @@
+"""A small network front end that emits the operator graph nengo's builder emits.
+
+nengo (``nengo>=3.1.0``, the reference's dependency, reference setup.py:31) is
+what normally turns a ``Network`` into operators; it may be absent, so the
+benchmark configurations and the parity tests are built with this module
+instead.  It covers ensembles of LIF / LIFRate neurons, nodes (constant,
+function of time, process, passthrough), decoded connections with functions,
+transforms, slices and linear synapses, PES learning, and probes -- and emits,
+per object, the operator pattern of nengo 3.1's builder as it is recalled here
+(nengo's source is not available to check against, so equality with a real
+nengo build of "the same" network is not claimed):
+
+* ensemble:  ``Reset(in)``, ``Copy(bias -> J)``, ``DotInc(scaled_encoders, in, J)``,
+  ``SimNeurons(J -> out; voltage, refractory_time)``
+* decoded connection:  ``Reset(weighted)``, ``DotInc(transform @ decoders, out,
+  weighted)``, ``SimProcess(synapse, weighted -> filtered, mode="update")``,
+  ``Copy(filtered -> post.in[slice], inc=True)``
+* node connection:  no-op / ``ElementwiseInc`` / ``DotInc`` for transform None /
+  scalar / matrix, then the same synapse and copy
+* PES:  ``SimProcess(pre_synapse, pre.out -> pre_filtered)``, ``Reset(error)``,
+  ``SimPES(pre_filtered, error -> delta)``, ``Copy(delta -> weights, inc=True)``
+
+``share_decoded=True`` lets connections leaving one ensemble with the same
+function, transform and synapse share one decoder matrix, one decoded signal
+and one filter (what a passthrough node after the ensemble gives in nengo).
+"""
+
+import numpy as np
+
+from . import ir
+from .ir import LIF, Alpha, LIFRate, LinearFilter, Lowpass, PresentInput, WhiteSignal  # noqa: F401
+
+
+class _Sliceable:
+    def __getitem__(self, item):
+        return ObjView(self, item)
+
+
+class ObjView:
+    def __init__(self, obj, item):
+        self.obj, self.slice = obj, item
+
+
+class Node(_Sliceable):
+    def __init__(self, output=None, size_in=0, size_out=None, label=None):
+        self.output, self.size_in, self.label = output, size_in, label
+        if output is None:
+            self.size_out = size_in  # passthrough
+        elif callable(output) or isinstance(output, ir.Process):
+            if size_out is None:
+                size_out = 1 if callable(output) else None
+            if size_out is None:
+                raise ValueError("size_out is needed for process nodes")
+            self.size_out = int(size_out)
+        else:
+            self.output = np.atleast_1d(np.asarray(output, dtype=np.float64))
+            self.size_out = self.output.size
+
+
+class Neurons(_Sliceable):
+    def __init__(self, ensemble):
+        self.ensemble = ensemble
+        self.size_out = self.size_in = ensemble.n_neurons
+
+
+class Ensemble(_Sliceable):
+    def __init__(self, n_neurons, dimensions, radius=1.0, neuron_type=None, max_rates=(200, 400),
+                 intercepts=(-1, 1), encoders=None, label=None, seed=None):
+        self.n_neurons, self.dimensions, self.radius = int(n_neurons), int(dimensions), radius
+        self.neuron_type = LIF() if neuron_type is None else neuron_type
+        self.max_rates, self.intercepts, self.encoders = max_rates, intercepts, encoders
+        self.label, self.seed = label, seed
+        self.neurons = Neurons(self)
+        self.size_in = self.size_out = self.dimensions
+
+
+class PES:
+    def __init__(self, learning_rate=1e-4, pre_synapse=Lowpass(0.005)):
+        self.learning_rate, self.pre_synapse = learning_rate, pre_synapse
+        self.connection = None
+
+
+class Connection:
+    def __init__(self, pre, post, function=None, transform=None, synapse=Lowpass(0.005),
+                 learning_rule=None, reg=0.1, label=None):
+        self.pre, self.post, self.function, self.transform = pre, post, function, transform
+        self.synapse = Lowpass(synapse) if isinstance(synapse, (int, float)) else synapse
+        self.learning_rule, self.reg, self.label = learning_rule, reg, label
+        if learning_rule is not None:
+            learning_rule.connection = self
+
+
+class Probe(ir.Probe):
+    def __init__(self, target, synapse=None, sample_every=None, label=None):
+        super().__init__(target, sample_every=sample_every, label=label)
+        self.synapse = Lowpass(synapse) if isinstance(synapse, (int, float)) else synapse
+
+
+def _uniform(rng, spec, n):
+    if np.ndim(spec) == 1 and len(spec) == 2 and not isinstance(spec, np.ndarray):
+        return rng.uniform(spec[0], spec[1], size=n)
+    return np.broadcast_to(np.asarray(spec, dtype=np.float64), (n,)).copy()
+
+
+def sphere_surface(rng, n, d):
+    x = rng.normal(size=(n, d))
+    return x / np.linalg.norm(x, axis=1, keepdims=True)
+
+
+def ball(rng, n, d):
+    return sphere_surface(rng, n, d) * rng.uniform(size=(n, 1)) ** (1.0 / d)
+
+
+def lstsq_l2(A, Y, reg=0.1):
+    """Regularised least squares ``argmin |A D - Y|^2 + m sigma^2 |D|^2`` with
+    ``sigma = reg * max(A)``; solved in whichever of the two Gram forms is smaller."""
+    m, n = A.shape
+    sigma = reg * A.max()
+    lam = m * sigma * sigma
+    if m >= n:
+        G = A.T @ A
+        G[np.diag_indices(n)] += lam
+        return np.linalg.solve(G, A.T @ Y)
+    G = A @ A.T
+    G[np.diag_indices(m)] += lam
+    return A.T @ np.linalg.solve(G, Y)
+
+
+class Network:
+    """Collects objects; ``build_model(dt)`` produces an `ir.Model`.
+
+    ``solver``: "lstsq" solves decoders on sampled evaluation points;
+    "surrogate" draws seeded random decoders of a plausible scale (for timing
+    runs at sizes where hundreds of large solves would dominate start-up).
+    """
+
+    def __init__(self, seed=0, label=None, share_decoded=True, solver="lstsq",
+                 n_eval_points=None):
+        self.seed, self.label = seed, label
+        self.share_decoded, self.solver, self.n_eval_points = share_decoded, solver, n_eval_points
+        self.nodes, self.ensembles, self.connections, self.probes = [], [], [], []
+
+    # --- object creation (returns the object, like nengo's constructors inside `with`)
+    def Node(self, *args, **kwargs):
+        obj = Node(*args, **kwargs)
+        self.nodes.append(obj)
+        return obj
+
+    def Ensemble(self, *args, **kwargs):
+        obj = Ensemble(*args, **kwargs)
+        self.ensembles.append(obj)
+        return obj
+
+    def Connection(self, *args, **kwargs):
+        obj = Connection(*args, **kwargs)
+        self.connections.append(obj)
+        return obj
+
+    def Probe(self, *args, **kwargs):
+        obj = Probe(*args, **kwargs)
+        self.probes.append(obj)
+        return obj
+
+    @property
+    def n_neurons(self):
+        return sum(e.n_neurons for e in self.ensembles)
+
+    def __str__(self):
+        return "<minibuilder.Network %s>" % (self.label,)
+
+    # ================================================================ build
+    def build_model(self, dt=0.001):
+        model = ir.Model(dt=dt, label="%s, dt=%f" % (self, dt))
+        rng = np.random.RandomState(self.seed)
+        self._decoded_cache = {}
+        self._decoder_values = {}
+        for ens in self.ensembles:
+            self._build_ensemble(model, ens, rng)
+        for node in self.nodes:
+            self._build_node(model, node, rng)
+        # learning-rule error signals exist before connections target them
+        for conn in self.connections:
+            if conn.learning_rule is not None:
+                rule = conn.learning_rule
+                post_obj = conn.post.obj if isinstance(conn.post, ObjView) else conn.post
+                model.sig[rule] = {"in": ir.Signal(np.zeros(post_obj.size_in), name="PES:error")}
+                model.add_op(ir.Reset(model.sig[rule]["in"]))
+        for conn in self.connections:
+            self._build_connection(model, conn, rng)
+        for probe in self.probes:
+            self._build_probe(model, probe, rng)
+        del self._decoded_cache, self._decoder_values
+        return model
+
+    def _build_ensemble(self, model, ens, rng):
+        seed = ens.seed if ens.seed is not None else rng.randint(2 ** 31 - 1)
+        erng = np.random.RandomState(seed)
+        n, d = ens.n_neurons, ens.dimensions
+        if ens.encoders is None:
+            encoders = sphere_surface(erng, n, d)
+        else:
+            encoders = np.array(ens.encoders, dtype=np.float64).reshape(n, d)
+            encoders /= np.linalg.norm(encoders, axis=1, keepdims=True)
+        max_rates = _uniform(erng, ens.max_rates, n)
+        intercepts = _uniform(erng, ens.intercepts, n)
+        gain, bias = ens.neuron_type.gain_bias(max_rates, intercepts)
+        scaled_encoders = encoders * (gain / ens.radius)[:, None]
+
+        name = ens.label or "ens%d" % len(model.sig)
+        sig = {
+            "in": ir.Signal(np.zeros(d), name="%s.signal" % name),
+            "encoders": ir.Signal(scaled_encoders, name="%s.scaled_encoders" % name, readonly=True),
+        }
+        nsig = {
+            "in": ir.Signal(np.zeros(n), name="%s.neuron_in" % name),
+            "out": ir.Signal(np.zeros(n), name="%s.neuron_out" % name),
+            "bias": ir.Signal(bias, name="%s.bias" % name, readonly=True),
+        }
+        model.sig[ens], model.sig[ens.neurons] = sig, nsig
+        model.params[ens] = dict(encoders=encoders, gain=gain, bias=bias, max_rates=max_rates,
+                                 intercepts=intercepts, scaled_encoders=scaled_encoders, seed=seed)
+        model.add_op(ir.Reset(sig["in"]))
+        model.add_op(ir.Copy(nsig["bias"], nsig["in"]))
+        model.add_op(ir.DotInc(sig["encoders"], sig["in"], nsig["in"], tag="%s encoding" % name))
+        if type(ens.neuron_type).__name__ == "LIF":
+            state = {"voltage": ir.Signal(np.zeros(n), name="%s.voltage" % name),
+                     "refractory_time": ir.Signal(np.zeros(n), name="%s.refractory_time" % name)}
+        else:
+            state = {}
+        model.add_op(ir.SimNeurons(ens.neuron_type, nsig["in"], nsig["out"], state=state))
+
+    def _build_node(self, model, node, rng):
+        name = node.label or "node%d" % len(model.sig)
+        if node.output is None:  # passthrough: in == out
+            sig_in = ir.Signal(np.zeros(node.size_in), name="<Node %s>.in" % name)
+            model.sig[node] = {"in": sig_in, "out": sig_in}
+            model.add_op(ir.Reset(sig_in))
+            return
+        if node.size_in:
+            raise NotImplementedError("nodes with both input and output function")
+        if isinstance(node.output, np.ndarray):
+            out = ir.Signal(node.output, name="<Node %s>.out" % name)
+            model.sig[node] = {"in": None, "out": out}
+            return
+        out = ir.Signal(np.zeros(node.size_out), name="<Node %s>.out" % name)
+        model.sig[node] = {"in": None, "out": out}
+        if isinstance(node.output, ir.Process):
+            if node.output.seed is None and hasattr(node.output, "table"):
+                node.output.seed = int(rng.randint(2 ** 31 - 1))
+            model.add_op(ir.SimProcess(node.output, None, out, model.time, mode="set"))
+        else:
+            model.add_op(ir.SimPyFunc(out, node.output, model.time, None))
+
+    # --- decoders
+    def _eval_activities(self, model, ens, rng):
+        p = model.params[ens]
+        n, d = ens.n_neurons, ens.dimensions
+        m = self.n_eval_points
+        if m is None:
+            m = int(max(np.clip(500 * d, 750, 2500), 2 * n))
+        pts = ball(rng, m, d) * ens.radius
+        J = p["gain"] * (pts @ p["encoders"].T / ens.radius) + p["bias"]
+        return pts, ens.neuron_type.rates_from_current(J)
+
+    def _decoders(self, model, conn, ens, function, size_mid, rng):
+        """Decoders (size_mid x n) for ``function`` of the ensemble's value.
+
+        Solved values are cached per (ensemble, function): connections that do not
+        share a decoded signal still get equal decoder *values* (nengo would sample
+        new evaluation points per connection)."""
+        n = ens.n_neurons
+        key = (ens, function)
+        if key in self._decoder_values:
+            return self._decoder_values[key]
+        if self.solver == "surrogate":
+            # seeded random decoders of the magnitude real ones have (~ 1 / (n * rate));
+            # a function that is identically zero keeps zero decoders
+            probe = np.atleast_1d(function(rng.normal(size=ens.dimensions))) if function else None
+            if probe is not None and not np.any(probe):
+                dec = np.zeros((size_mid, n))
+            else:
+                dec = rng.normal(scale=2.0 / (100.0 * n), size=(size_mid, n))
+        else:
+            pts, acts = self._eval_activities(model, ens, rng)
+            targets = pts if function is None else np.array(
+                [np.atleast_1d(function(x)) for x in pts])
+            dec = lstsq_l2(acts, targets, reg=conn.reg if conn is not None else 0.1).T
+        self._decoder_values[key] = dec
+        return dec
+
+    # --- connections
+    @staticmethod
+    def _split(target):
+        if isinstance(target, ObjView):
+            return target.obj, target.slice
+        return target, None
+
+    def _apply_synapse(self, model, signal, synapse, name):
+        if synapse is None:
+            return signal
+        filtered = ir.Signal(np.zeros(signal.shape), name="%s.filtered" % name)
+        model.add_op(ir.SimProcess(synapse, signal, filtered, model.time, mode="update"))
+        return filtered
+
+    def _build_connection(self, model, conn, rng, into_signal=None):
+        pre, pre_slice = self._split(conn.pre)
+        post, post_slice = self._split(conn.post)
+        crng = np.random.RandomState(rng.randint(2 ** 31 - 1))
+        name = conn.label or "conn%d" % len(model.sig)
+        transform = None if conn.transform is None else np.asarray(conn.transform, dtype=np.float64)
+
+        if isinstance(pre, Ensemble):
+            if pre_slice is not None:
+                sel = np.arange(pre.dimensions)[pre_slice]
+                base_fn = conn.function
+                function = (lambda x, f=base_fn, s=sel: (x if f is None else np.atleast_1d(f(x)))[s])
+            else:
+                function = conn.function
+            learned = conn.learning_rule is not None
+            key = (pre, conn.function, None if transform is None else transform.tobytes(),
+                   repr(pre_slice), self._synapse_key(conn.synapse))
+            cached = self._decoded_cache.get(key) if (self.share_decoded and not learned) else None
+            if cached is not None:
+                signal = cached
+            else:
+                probe_x = np.zeros(pre.dimensions)
+                size_mid = pre.dimensions if function is None else np.atleast_1d(function(probe_x)).size
+                decoders = self._decoders(model, conn, pre, function, size_mid, crng)
+                if transform is None:
+                    weights = decoders
+                elif transform.ndim == 0:
+                    weights = transform * decoders
+                elif transform.ndim == 1:
+                    weights = transform[:, None] * decoders
+                else:
+                    weights = transform @ decoders
+                wsig = ir.Signal(weights, name="%s.weights" % name, readonly=not learned)
+                model.sig[conn] = {"weights": wsig}
+                model.params[conn] = dict(weights=weights)
+                weighted = ir.Signal(np.zeros(weights.shape[0]), name="%s.weighted" % name)
+                model.add_op(ir.Reset(weighted))
+                model.add_op(ir.DotInc(wsig, model.sig[pre.neurons]["out"], weighted,
+                                       tag="%s.weights_dotinc" % name))
+                signal = self._apply_synapse(model, weighted, conn.synapse, name)
+                if self.share_decoded and not learned:
+                    self._decoded_cache[key] = signal
+                if learned:
+                    self._build_pes(model, conn, pre, wsig, name)
+        elif isinstance(pre, Neurons):
+            signal = model.sig[pre]["out"]
+            if pre_slice is not None:
+                signal = signal[pre_slice]
+            signal = self._apply_synapse(model, signal, conn.synapse, name)
+        elif isinstance(pre, Node):
+            signal = model.sig[pre]["out"]
+            if pre_slice is not None:
+                signal = signal[pre_slice]
+            if conn.function is not None:
+                raise NotImplementedError("functions on node connections")
+            if transform is not None:
+                if transform.ndim == 0:
+                    tsig = ir.Signal(transform, name="%s.transform" % name, readonly=True)
+                    weighted = ir.Signal(np.zeros(signal.shape), name="%s.weighted" % name)
+                    model.add_op(ir.Reset(weighted))
+                    model.add_op(ir.ElementwiseInc(tsig, signal, weighted))
+                else:
+                    t2 = np.diag(transform) if transform.ndim == 1 else transform
+                    tsig = ir.Signal(t2, name="%s.transform" % name, readonly=True)
+                    weighted = ir.Signal(np.zeros(t2.shape[0]), name="%s.weighted" % name)
+                    model.add_op(ir.Reset(weighted))
+                    model.add_op(ir.DotInc(tsig, signal, weighted, tag="%s.transform" % name))
+                signal = weighted
+            signal = self._apply_synapse(model, signal, conn.synapse, name)
+        else:
+            raise TypeError("cannot connect from %r" % (pre,))
+
+        # --- deliver
+        if into_signal is not None:
+            target = into_signal
+        elif isinstance(post, Ensemble):
+            target = model.sig[post]["in"]
+        elif isinstance(post, Neurons):
+            target = model.sig[post]["in"]
+        elif isinstance(post, Node):
+            if post.output is not None:
+                raise NotImplementedError("connections into function nodes")
+            target = model.sig[post]["in"]
+        elif isinstance(post, PES):
+            target = model.sig[post]["in"]
+        else:
+            raise TypeError("cannot connect to %r" % (post,))
+        n_target = target.size if post_slice is None else np.arange(target.size)[post_slice].size
+        if signal.size != n_target:
+            raise ValueError("%s: %d values into %d slots" % (name, signal.size, n_target))
+        model.add_op(ir.Copy(signal, target, dst_slice=post_slice, inc=True, tag="%s" % name))
+
+    @staticmethod
+    def _synapse_key(synapse):
+        if synapse is None:
+            return None
+        return (type(synapse).__name__, tuple(synapse.num), tuple(synapse.den), synapse.analog)
+
+    def _build_pes(self, model, conn, pre, wsig, name):
+        rule = conn.learning_rule
+        acts = model.sig[pre.neurons]["out"]
+        pre_filtered = self._apply_synapse(model, acts, rule.pre_synapse, "%s.pes_pre" % name)
+        delta = ir.Signal(np.zeros(wsig.shape), name="%s.Delta" % name)
+        model.add_op(ir.SimPES(pre_filtered, model.sig[rule]["in"], delta, rule.learning_rate))
+        model.add_op(ir.Copy(delta, wsig, inc=True, tag="%s += delta" % name))
+        model.sig[rule]["delta"] = delta
+
+    # --- probes
+    def _build_probe(self, model, probe, rng):
+        target, tslice = self._split(probe.target)
+        if isinstance(target, Ensemble):
+            sig_in = ir.Signal(np.zeros(target.dimensions if tslice is None else
+                                        np.arange(target.dimensions)[tslice].size),
+                               name="probe(%s)" % (target.label,))
+            model.sig[probe] = {"in": sig_in}
+            model.add_op(ir.Reset(sig_in))
+            conn = Connection(probe.target, None, synapse=probe.synapse, label="probe_conn")
+            self._build_connection(model, conn, rng, into_signal=sig_in)
+        elif isinstance(target, (Node, Neurons)):
+            src = model.sig[target]["out"]
+            if tslice is not None:
+                src = src[tslice]
+            if probe.synapse is None:
+                model.sig[probe] = {"in": src}
+            else:
+                filtered = self._apply_synapse(model, src, probe.synapse, "probe")
+                model.sig[probe] = {"in": filtered}
+        else:
+            raise TypeError("cannot probe %r" % (target,))
+        model.probes.append(probe)

@@ -1,0 +1,328 @@
+"""Graph rewrites that feed the ragged GEMV: MultiDotInc and op simplification.
+
+Counterpart of the reference's ``nengo_ocl/operators.py``: ``MultiDotInc``
+(:19-194: ``convert_to`` :51, ``compress`` :112, ``get_views`` :159),
+``signal_io_dicts`` (:197), ``remove_unmodified_resets`` (:226),
+``remove_zero_incs`` (:265), ``simplify_operators`` / ``simplifications``
+(:334-350).  Operator kinds are recognised by class name so that operators
+built by nengo and by `ir` are treated alike.
+"""
+
+import numpy as np
+
+from . import ir
+
+
+def _is(op, name):
+    return type(op).__name__ == name
+
+
+class MultiDotInc(ir.Operator):
+    r"""``Y <- gamma + beta * Y_in + \sum_i dot(A_i, X_i)``"""
+
+    def __init__(self, Y, Y_in, beta, gamma, tag=None):
+        super().__init__(tag=tag)
+        if Y.ndim != 1:
+            raise ValueError("Y must be a vector")
+        if Y.shape != Y_in.shape:
+            raise TypeError("Y and Y_in differ in shape")
+        self.Y, self.Y_in = Y, Y_in
+
+        if hasattr(beta, "shape") and hasattr(beta, "base"):  # a Signal
+            if beta.shape != Y.shape:
+                raise NotImplementedError("", (beta.shape, Y.shape))
+            self._float_beta, self._signal_beta = None, beta
+        else:
+            self._float_beta = float(getattr(beta, "value", beta))
+            self._signal_beta = None
+
+        self.gamma = float(gamma)
+        self.As, self.Xs = [], []
+        self._incs_Y = self._signal_beta is None and self._float_beta == 1 and Y_in is Y
+
+    @classmethod
+    def convert_to(cls, op):
+        """A plain DotInc becomes ``MultiDotInc(Y, Y, beta=1, gamma=0)`` with one pair."""
+        if _is(op, "BsrDotInc"):
+            raise NotImplementedError("BsrDotInc operations are not supported")
+        if not _is(op, "DotInc"):
+            return op
+        new = cls(op.Y, op.Y, beta=1, gamma=0, tag=op.tag)
+        new.add_AX(op.A, op.X)
+        assert set(op.reads).issuperset(new.reads)
+        assert list(new.incs) == list(op.incs) and list(new.sets) == list(op.sets)
+        assert all(s.size for s in new.all_signals), op
+        return new
+
+    def add_AX(self, A, X):
+        if X.ndim != 1:
+            raise ValueError("X must be a vector")
+        self.As.append(A)
+        self.Xs.append(X)
+
+    # sets / incs / reads are derived from the current state
+    @property
+    def reads(self):
+        r = list(self.As) + list(self.Xs)
+        if not self._incs_Y:
+            if self._signal_beta is not None:
+                r.append(self._signal_beta)
+                if self.Y_in is not self.Y:
+                    r.append(self.Y_in)
+            elif self._float_beta != 0 and self.Y_in is not self.Y:
+                r.append(self.Y_in)
+        return r
+
+    @reads.setter
+    def reads(self, value):
+        pass
+
+    @property
+    def incs(self):
+        return [self.Y] if self._incs_Y else []
+
+    @incs.setter
+    def incs(self, value):
+        pass
+
+    @property
+    def sets(self):
+        return [] if self._incs_Y else [self.Y]
+
+    @sets.setter
+    def sets(self, value):
+        pass
+
+    @property
+    def updates(self):
+        return []
+
+    @updates.setter
+    def updates(self, value):
+        pass
+
+    def __repr__(self):
+        beta = self._float_beta if self._signal_beta is None else self._signal_beta
+        dots = ", ".join("dot(%s, %s)" % (A, X) for A, X in zip(self.As, self.Xs))
+        return "<MultiDotInc(tag=%s, Y=%s, Y_in=%s, beta=%s, gamma=%s, dots=[%s]) at 0x%x>" % (
+            self.tag, self.Y, self.Y_in, beta, self.gamma, dots, id(self))
+
+    @classmethod
+    def compress(cls, operators):
+        """Merge MultiDotIncs that write the same Signal object into one op.
+
+        Increments are folded into the op that sets the same signal, if any;
+        the remaining increments on one signal are folded together.  Other
+        operators keep their order and come first, as in the reference.
+        """
+        setters, incrementers, rest = {}, {}, []
+        for op in operators:
+            if not isinstance(op, cls):
+                rest.append(op)
+            elif op.sets:
+                assert len(op.sets) == 1 and not op.incs
+                setters.setdefault(op.sets[0], []).append(op)
+            else:
+                assert len(op.incs) == 1 and not op.sets
+                incrementers.setdefault(op.incs[0], []).append(op)
+
+        for view, set_ops in setters.items():
+            (set_op,) = set_ops
+            for inc_op in incrementers.pop(view, []):
+                set_op.As.extend(inc_op.As)
+                set_op.Xs.extend(inc_op.Xs)
+            rest.append(set_op)
+
+        for view, inc_ops in incrementers.items():
+            first = inc_ops[0]
+            for other in inc_ops[1:]:
+                first.As.extend(other.As)
+                first.Xs.extend(other.Xs)
+            rest.append(first)
+        return rest
+
+    @staticmethod
+    def _as2d(view):
+        if view.ndim == 0:
+            return view.reshape(1, 1)
+        if view.ndim == 1:
+            return view.reshape(view.shape[0], 1)
+        if view.ndim == 2:
+            return view
+        raise ValueError("No support for tensors with %d dimensions" % view.ndim)
+
+    def get_views(self):
+        """2-D views ``(A_views, X_views, Y, Y_in, beta)`` in kernel orientation.
+
+        A vector A with a vector X is a 1 x n row; a 1 x 1 (scalar) A is swapped
+        with its X, so ``y += a * x`` runs as the GEMV ``x[n x 1] @ a[1]``.
+        """
+        Y_view, Y_in_view = self._as2d(self.Y), self._as2d(self.Y_in)
+        beta_view = None if self._signal_beta is None else self._as2d(self._signal_beta)
+        A_views, X_views = [], []
+        for A, X in zip(self.As, self.Xs):
+            X_view = self._as2d(X)
+            A_view = A.reshape((1, A.shape[0])) if (A.ndim == 1 and X.ndim == 1) else self._as2d(A)
+            if A_view.shape == (1, 1):
+                A_view, X_view = X_view, A_view
+            elif not (X_view.shape[0] == A_view.shape[1] and X_view.shape[1] == Y_view.shape[1]
+                      and A_view.shape[0] == Y_view.shape[0]):
+                raise ValueError("shape mismach (A: %s, X: %s, Y: %s)" % (A.shape, X.shape, self.Y.shape))
+            A_views.append(A_view)
+            X_views.append(X_view)
+        return A_views, X_views, Y_view, Y_in_view, beta_view
+
+
+def signal_io_dicts(operators):
+    """Four dicts base-signal -> [ops that set / inc / read / update part of it]."""
+    bases = {s.base for op in operators for s in op.all_signals}
+    sets, incs, reads, updates = ({b: [] for b in bases} for _ in range(4))
+    for op in operators:
+        for table, sigs in ((sets, op.sets), (incs, op.incs), (reads, op.reads), (updates, op.updates)):
+            for s in sigs:
+                table[s.base].append(op)
+    return sets, incs, reads, updates
+
+
+def _overwrite_initial_value(sig, value):
+    arr = sig.initial_value
+    owner = sig.base.initial_value
+    owner.setflags(write=True)
+    arr.setflags(write=True)
+    arr[...] = value
+    arr.setflags(write=False)
+    owner.setflags(write=False)
+
+
+def remove_unmodified_resets(operators):
+    """Drop every Reset whose target is never incremented or updated: the reset
+    value becomes the signal's initial value instead."""
+    _, incs, _, updates = signal_io_dicts(operators)
+    kept = []
+    for op in operators:
+        if _is(op, "Reset") and not incs[op.dst.base] and not updates[op.dst.base]:
+            _overwrite_initial_value(op.dst, op.value)
+        else:
+            kept.append(op)
+    return kept
+
+
+def remove_zero_incs(operators):
+    """Drop DotInc / ElementwiseInc / Copy / ConvInc ops with an input known to be
+    zero forever (only written by a ``Reset(0)``, or constant zero).  A dropped op
+    that *set* its target is replaced by a Reset of that target.  Node outputs are
+    never treated as constant."""
+
+    def constant_zero(sig):
+        data = sig.initial_value
+        if getattr(sig, "sparse", False):
+            data = data.tocoo().data if hasattr(data, "tocoo") else data.data
+        return np.all(np.asarray(data) == 0)
+
+    sets, incs, _, updates = signal_io_dicts(operators)
+    kept = []
+    for op in operators:
+        if type(op).__name__ not in ("DotInc", "ElementwiseInc", "Copy", "ConvInc"):
+            kept.append(op)
+            continue
+        for src in op.reads:
+            if str(src.name).startswith("<Node"):
+                continue
+            writers = sets[src.base] + incs[src.base] + updates[src.base]
+            if len(writers) == 1:
+                w = writers[0]
+                zero = _is(w, "Reset") and np.all(w.value == 0)
+            else:
+                zero = len(writers) == 0 and constant_zero(src)
+            if zero:
+                if len(op.sets) > 0:
+                    kept.append(_make_reset(op, op.sets[0]))
+                break
+        else:
+            kept.append(op)
+    return kept
+
+
+def _make_reset(like, dst):
+    """A Reset of the same family (nengo's or `ir`'s) as operator ``like``."""
+    if type(like).__module__.startswith("nengo."):
+        from nengo.builder.operator import Reset
+
+        return Reset(dst)
+    return ir.Reset(dst)
+
+
+def fuse_into_multidotinc(operators):
+    """Express vector copies and resets that surround a GEMV as part of that GEMV.
+
+    ``MultiDotInc`` computes ``Y = beta*Y_in + gamma + sum_i A_i @ X_i`` with
+    ``Y_in`` allowed to differ from ``Y``; three common operator patterns are
+    special cases of it and are rewritten so that `MultiDotInc.compress` can
+    fold them into one operator per target (one kernel work item instead of
+    several dependent launches):
+
+    * ``Copy(src -> dst[slice], inc=True)`` on vectors is ``dst[slice] += src * 1``:
+      a MultiDotInc with the pair ``(A = scalar one, X = src)`` (the scalar-A
+      form of `get_views`).  All increments into one target then merge, where
+      the planner would otherwise run colliding increments one group at a time.
+    * ``Reset(dst, v)`` of a vector that receives MultiDotInc increments is the
+      setter ``dst = 0*dst + v + sum(...)``.
+    * ``Copy(src -> dst)`` (e.g. bias into the neuron input) of a vector that
+      receives MultiDotInc increments is the setter ``dst = 1*src + 0 + sum(...)``.
+
+    The order of floating-point additions per element is unchanged: first the
+    set value, then the increments in operator order.
+    """
+    one = None
+    views = {}
+
+    def view_of(sig, sl):
+        if sl is None:
+            return sig
+        key = (id(sig), sl.start, sl.stop, sl.step)
+        if key not in views:
+            views[key] = sig[sl]
+        return views[key]
+
+    basic = lambda sl: sl is None or isinstance(sl, slice)
+    out = []
+    for op in operators:
+        if (_is(op, "Copy") and op.inc and basic(op.src_slice) and basic(op.dst_slice)
+                and op.src.ndim == 1 and op.dst.ndim == 1):
+            if one is None:
+                one = type(op.src)(np.array(1.0), name="one", readonly=True)
+            y = view_of(op.dst, op.dst_slice)
+            new = MultiDotInc(y, y, beta=1, gamma=0, tag=op.tag)
+            new.add_AX(one, view_of(op.src, op.src_slice))
+            out.append(new)
+        else:
+            out.append(op)
+
+    targets = {op.Y for op in out if isinstance(op, MultiDotInc) and op._incs_Y}
+    setters = {}
+    for op in out:
+        if not isinstance(op, MultiDotInc):
+            for sig in op.sets:
+                setters.setdefault(sig, []).append(op)
+    fused = []
+    for op in out:
+        if _is(op, "Reset") and op.dst in targets and op.dst.ndim == 1 and len(setters[op.dst]) == 1:
+            fused.append(MultiDotInc(op.dst, op.dst, beta=0, gamma=op.value, tag=op.tag))
+        elif (_is(op, "Copy") and not op.inc and op.src_slice is None and op.dst_slice is None
+              and op.dst in targets and op.dst.ndim == 1 and op.src.shape == op.dst.shape
+              and len(setters[op.dst]) == 1):
+            fused.append(MultiDotInc(op.dst, op.src, beta=1, gamma=0, tag=op.tag))
+        else:
+            fused.append(op)
+    return fused
+
+
+def simplify_operators(operators):
+    """Apply every function in ``simplifications`` in turn."""
+    for simplification in simplifications:
+        operators = simplification(operators)
+    return operators
+
+
+# Modify this module-level list to change which simplifications run.
+simplifications = [remove_unmodified_resets, remove_zero_incs]
