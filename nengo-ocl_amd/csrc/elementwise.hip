@@ -220,10 +220,10 @@ __global__ __launch_bounds__(NHIP_WG) void direct_unary_kernel(int opcode,
         const float x = X[d.x + i];
         float y;
         switch (opcode) {
-            case 1: y = sinf(x); break;
-            case 2: y = cosf(x); break;
-            case 3: y = tanhf(x); break;
-            case 4: y = expf(x); break;
+            case 1: y = (float)sin((double)x); break;   // double, rounded once: library independent
+            case 2: y = (float)cos((double)x); break;
+            case 3: y = (float)tanh((double)x); break;
+            case 4: y = (float)exp((double)x); break;
             case 5: y = __fmul_rn(x, x); break;
             default: y = x;
         }

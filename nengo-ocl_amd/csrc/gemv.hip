@@ -11,7 +11,8 @@
 // There is no partial-sum buffer and no second (reduce) launch, and the
 // summation order is fixed, so results are reproducible run to run.
 //
-// Two flavours, chosen per item by the host planner:
+// Three flavours, chosen per item by the host planner (the third, "wave_ref", is
+// the wave flavour in the reference's summation order, see below):
 //   wg   : one 256-thread group per task.  The gathered X vector is staged
 //          through LDS once per group (coalesced, stride-aware) and shared by
 //          the four waves.  LPR lanes cooperate on a row (LPR = 256: the whole
@@ -200,6 +201,53 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
     }
 }
 
+// Wave-per-task kernel in the summation order of the reference's block GEMV
+// (clra_gemv.py:1040-1058 and :1148-1153): per row and per 128-column tile, lane
+// j of four sums columns j, j+4, ... left to right (product and sum rounded
+// separately), the four partial sums combine as (s0+s2)+(s1+s3), and tile sums
+// are added one after the other onto beta*y_in; gamma comes last.  Used for the
+// small items of networks with thousands of tiny ensembles, where the order costs
+// nothing and makes the result bit-identical to a float32 restatement of the
+// reference; sixteen rows are in flight per wave.
+__global__ __launch_bounds__(NHIP_WG) void gemv_wave_ref_kernel(
+    const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
+    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    const float* __restrict__ A, const float* __restrict__ X, const float* Yin, float* Y)
+{
+    constexpr int TILE = 128;
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    const int t = blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6);
+    if (t >= n_tasks) return;  // wave-uniform; this kernel has no barrier
+
+    const GemvTask task = tasks[t];
+    const GemvItem it = items[task.item];
+    const float4 cf = coefs[task.item];
+    const int row_end = task.row0 + task.n_rows;
+    const int lir = lane & 3;
+    const int sub = lane >> 2;
+
+    for (int r0 = task.row0; r0 < row_end; r0 += NHIP_WAVE / 4) {
+        const bool valid = r0 + sub < row_end;
+        const int r = valid ? r0 + sub : row_end - 1;
+        float sum = cf.y * Yin[it.yin_start + (size_t)r * it.yin_stride0];
+        for (int d = 0; d < it.n_dots; ++d) {
+            const GemvDot dot = dots[it.dot_begin + d];
+            const float* arow = A + dot.a_start + (size_t)r * dot.a_stride0;
+            const float* xg = X + dot.x_start;
+            const size_t xs = (size_t)dot.x_stride0;
+            for (int c0 = 0; c0 < dot.N; c0 += TILE) {
+                const int c1 = min(c0 + TILE, dot.N);
+                float s = 0.0f;
+                for (int c = c0 + lir; c < c1; c += 4) s = s + arow[c] * xg[(size_t)c * xs];
+                s = s + __shfl_xor(s, 2, NHIP_WAVE);
+                s = s + __shfl_xor(s, 1, NHIP_WAVE);
+                sum = sum + cf.x * s;
+            }
+        }
+        if (lir == 0 && valid) Y[it.y_start + (size_t)r * it.y_stride0] = sum + cf.z;
+    }
+}
+
 template <int LPR, int VEC>
 int launch_wg(hipStream_t s, const int* items, const float* coefs, const int* dots,
               const int* tasks, int n_tasks, const float* A, const float* X, const float* Yin,
@@ -231,6 +279,7 @@ int launch_wave(hipStream_t s, const int* items, const float* coefs, const int* 
 
 extern "C" int nhip_gemv_rows_per_task(int flavor, int lpr, int vec) {
     if (vec != 1 && vec != 4) return 0;
+    if (flavor == 2) return (lpr == 4 && vec == 1) ? 0x7fffffff : 0;
     if (flavor == 1) {
         switch (lpr) { case 1: case 2: case 4: case 8: case 16: case 32: case 64: return 0x7fffffff; }
         return 0;
@@ -274,6 +323,16 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, const int* 
             NHIP_GEMV_CASE(launch_wg, 64)
             NHIP_GEMV_CASE(launch_wg, 256)
         }
+    } else if (flavor == 2) {
+        if (lpr != 4 || vec != 1) return NHIP_E_BADCLASS;
+        const int wpg = NHIP_WG / NHIP_WAVE;
+        hipLaunchKernelGGL(gemv_wave_ref_kernel, dim3((n_tasks + wpg - 1) / wpg), dim3(NHIP_WG), 0,
+                           s, reinterpret_cast<const GemvItem*>(items),
+                           reinterpret_cast<const float4*>(coefs),
+                           reinterpret_cast<const GemvDot*>(dots),
+                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
+        NHIP_LAUNCH_CHECK();
+        return 0;
     } else if (flavor == 1) {
         switch (lpr) {
             NHIP_GEMV_CASE(launch_wave, 1)

@@ -20,6 +20,10 @@ __device__ __forceinline__ float lif_param(int word, bool is_vector, const float
 // exponential-Euler voltage step, threshold test with spike-time interpolation.
 // Sums that follow a product are written with explicit rounded operations so
 // that the compiler cannot fuse them differently from one build to the next.
+// expm1 and log1p are evaluated in double and rounded once to float: that is the
+// correctly rounded float32 value (the best any float implementation can return),
+// so every conforming host or device math library gives the same bits and spike
+// decisions do not depend on the library.
 __global__ __launch_bounds__(NHIP_WG) void lif_kernel(const LifDesc* __restrict__ desc, float dt,
                                                       float dt_inv, int upsample, const float* J,
                                                       float* V, float* W, float* S,
@@ -39,11 +43,11 @@ __global__ __launch_bounds__(NHIP_WG) void lif_kernel(const LifDesc* __restrict_
         for (int u = 0; u < upsample; ++u) {
             w -= dtu;
             const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
-            const float dv = __fmul_rn(-expm1f(__fdiv_rn(-delta_t, tau)), j - v);
+            const float dv = __fmul_rn(-(float)expm1((double)__fdiv_rn(-delta_t, tau)), j - v);
             v = __fadd_rn(v, dv);
             if (v > 1.0f) {
                 const float t_spike =
-                    __fadd_rn(dtu, __fmul_rn(tau, log1pf(__fdiv_rn(-(v - 1.0f), j - 1.0f))));
+                    __fadd_rn(dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
                 w = ref + t_spike;
                 v = 0.0f;
                 spiked = true;
@@ -71,7 +75,7 @@ __global__ __launch_bounds__(NHIP_WG) void lif_rate_kernel(const RateDesc* __res
         const float ref = lif_param(d.ref, d.pflags & 2, REF, i);
         const float amp = lif_param(d.amp, d.pflags & 4, AMP, i);
         const float j = fmaxf(J[(size_t)d.j_start + i] - 1.0f, 0.0f);
-        const float denom = __fadd_rn(ref, __fmul_rn(tau, log1pf(__fdiv_rn(1.0f, j))));
+        const float denom = __fadd_rn(ref, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(1.0f, j))));
         R[(size_t)d.r_start + i] = __fdiv_rn(amp, denom);
     }
 }

@@ -27,6 +27,8 @@ from .utils import next_pow2
 
 # items with at most this many matrix elements go to the wave-per-task kernel
 SMALL_ITEM_ELEMS = 8192
+# ... and among those, rows up to this length use the reference-order wave kernel
+REF_ORDER_MAX_COLS = 512
 WG, WAVE = 256, 64
 
 
@@ -166,6 +168,8 @@ class gemv_prog:
         flavor = self.force_flavor
         if flavor is None:
             flavor = 1 if M * n_sum <= SMALL_ITEM_ELEMS else 0
+            if flavor == 1 and n_max <= REF_ORDER_MAX_COLS:
+                return (2, 4, 1)  # small item: the reference's summation order, bit for bit
         lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         if flavor == 0 and (n_max >= 2048 or (n_max >= 512 and M < 16)):
             lpr = WG  # the whole group works on one row
@@ -203,7 +207,7 @@ class gemv_prog:
             if flavor == 0:
                 rows = lib.nhip_gemv_rows_per_task(flavor, lpr, vec)
             else:
-                rows = (WAVE // lpr) * 4
+                rows = (WAVE // lpr) * 4  # four passes of a wave
             if rows <= 0:
                 raise _lib.HipError("unknown GEMV class %r" % ((flavor, lpr, vec),))
             task_rows = []
@@ -221,7 +225,7 @@ class gemv_prog:
                 self.queue, lib.nhip_gemv, args, gsize=(WG * n_groups,), lsize=(WG,),
                 full_args=(dev_items, dev_coefs, dev_dots, dev_tasks, self.A.dev_buf,
                            self.X.dev_buf, self.Y_in.dev_buf, self.Y.dev_buf),
-                name="hipra_gemv.%s" % ("wg" if flavor == 0 else "wave"),
+                name="hipra_gemv.%s" % ("wg", "wave", "wave_ref")[flavor],
                 tag="%s-lpr%d-v%d" % (self.tag, lpr, vec),
                 bw_per_call=bw_from_geometry(geometry, members),
                 flops_per_call=flops_from_geometry(geometry, members),

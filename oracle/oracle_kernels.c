@@ -93,7 +93,10 @@ void orc_gemv_block(int n_items, const int *y_starts, const int *y_stride0s, con
  * fastlif off) inside `_plan_template` :1367-1417.  tau/ref/amp are per-neuron
  * arrays there (simulator.py:1054-1062); here one value per item, which is what
  * those arrays hold.  dtu = dt/upsample, dt_inv = 1/dt are double literals
- * rounded to float at declaration.
+ * rounded to float at declaration.  The kernel text calls the float built-ins
+ * expm1 / log1p, whose last bit OpenCL leaves to the implementation; here they
+ * are the correctly rounded float values (evaluated in double, rounded once),
+ * which every conforming implementation approximates.
  */
 void orc_lif(int n_items, const int *sizes, const int *j_starts, const int *v_starts,
              const int *w_starts, const int *s_starts, const float *taus, const float *refs,
@@ -112,10 +115,10 @@ void orc_lif(int n_items, const int *sizes, const int *j_starts, const int *v_st
             for (int u = 0; u < upsample; ++u) {
                 w = w - dtu;
                 const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
-                const float dv = -expm1f(-delta_t / tau) * (j - v);
+                const float dv = -(float)expm1((double)(-delta_t / tau)) * (j - v);
                 v = v + dv;
                 if (v > 1.0f) {
-                    const float t_spike = dtu + tau * log1pf(-(v - 1.0f) / (j - 1.0f));
+                    const float t_spike = dtu + tau * (float)log1p((double)(-(v - 1.0f) / (j - 1.0f)));
                     w = ref + t_spike;
                     v = 0.0f;
                     spiked = 1;
@@ -139,7 +142,7 @@ void orc_lif_rate(int n_items, const int *sizes, const int *j_starts, const int 
         for (int i = 0; i < sizes[n]; ++i) {
             float j = J[(size_t)j_starts[n] + i] - 1.0f;
             j = (j > 0.0f) ? j : 0.0f;
-            R[(size_t)r_starts[n] + i] = amps[n] / (refs[n] + taus[n] * log1pf(1.0f / j));
+            R[(size_t)r_starts[n] + i] = amps[n] / (refs[n] + taus[n] * (float)log1p((double)(1.0f / j)));
         }
     }
 }
@@ -351,10 +354,10 @@ void orc_direct_unary(int opcode, int n_items, const int *x_starts, const int *y
         const float x = X[x_starts[n]];
         float y;
         switch (opcode) {
-            case 1: y = sinf(x); break;
-            case 2: y = cosf(x); break;
-            case 3: y = tanhf(x); break;
-            case 4: y = expf(x); break;
+            case 1: y = (float)sin((double)x); break;
+            case 2: y = (float)cos((double)x); break;
+            case 3: y = (float)tanh((double)x); break;
+            case 4: y = (float)exp((double)x); break;
             case 5: y = x * x; break;
             default: y = x;
         }
