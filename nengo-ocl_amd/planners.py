@@ -50,6 +50,26 @@ def operator_dependency_graph(operators):
 
 
 def greedy_planner(operators):
+    """The reference's rule (planners.py:39-91): among the ready types take the one
+    with the most ready operators (ties: the type that became ready last)."""
+    return _plan(operators, completing=False)
+
+
+def batching_planner(operators):
+    """Like `greedy_planner`, but a type all of whose remaining operators are ready is
+    scheduled first (smallest such type first).
+
+    Taking the largest ready set can split a type into several groups when a few
+    of its operators sit behind a small group of another type (ensembles without
+    input whose bias copy is the only Copy left, for instance): the large group
+    goes first, the stragglers need a second launch of every later type.
+    Finishing complete types first removes those splits and never adds a group
+    for the type that is completed.  This is the Simulator's default.
+    """
+    return _plan(operators, completing=True)
+
+
+def _plan(operators, completing):
     """Group operators by type into as few sequential groups as dependencies and
     write-overlap allow.
 
@@ -71,12 +91,20 @@ def greedy_planner(operators):
         if n_waiting[op] == 0:
             ready.setdefault(type(op), {})[op] = None
 
+    n_of_type = defaultdict(int)  # operators of each type not yet scheduled
+    for op in operators:
+        n_of_type[type(op)] += 1
+
     groups = []
     n_left = len(operators)
     while n_left > 0:
         if not ready:
             raise ValueError("Cycles in the op graph")
         chosen_type = sorted(ready.items(), key=lambda kv: len(kv[1]))[-1][0]
+        if completing:
+            complete = [t for t, ops in ready.items() if len(ops) == n_of_type[t]]
+            if complete:
+                chosen_type = min(complete, key=lambda t: n_of_type[t])
 
         written = (defaultdict(list), defaultdict(list), defaultdict(list))
         chosen = []
@@ -102,6 +130,7 @@ def greedy_planner(operators):
                 if n_waiting[post] == 0:
                     ready.setdefault(type(post), {})[post] = None
         n_left -= len(chosen)
+        n_of_type[chosen_type] -= len(chosen)
 
     assert sum(len(ops) for _, ops in groups) == len(operators)
     return groups

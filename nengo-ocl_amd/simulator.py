@@ -34,7 +34,7 @@ import numpy as np
 from . import operators as ops_mod
 from .operators import MultiDotInc
 from .plan import BasePlan, Plans, PythonPlan
-from .planners import greedy_planner
+from .planners import batching_planner, greedy_planner  # noqa: F401
 from .raggedarray import RaggedArray
 from .utils import get_closures, groupby, indent, split, stable_unique
 
@@ -189,7 +189,7 @@ class Simulator:
 
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
                  n_prealloc_probes=32, profiling=None, if_python_code="none",
-                 planner=greedy_planner, progress_bar=True, backend=None, use_graph=True,
+                 planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
                  fuse=True):
         self.closed = False
         self.model = None
