@@ -63,7 +63,7 @@ def gemv_summary(sim, profile_steps):
     for p in plans:
         p.atimes[:], p.btimes[:], p.ctimes[:] = [], [], []
         p.n_calls = 0
-    plans.call_n_times(profile_steps)
+    sim.run_steps(profile_steps)  # run_steps drains the probe buffers between batches
     plans.profiling = False
     rows = []
     for p in plans:

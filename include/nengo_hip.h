@@ -142,7 +142,9 @@ int nhip_presentinput(void *stream, const int *desc, int n, float dt, float *Y, 
  *   desc : int32[n][4] {x_start, y_start, count, 0} */
 int nhip_direct_unary(void *stream, int opcode, const int *desc, int n, const float *X, float *Y);
 /* probe gather with per-probe float countdown.  replaces: `plan_probes` (:806-951).
- *   desc : int32[n][8] {x_start, shape0, shape1, stride0, stride1, y_start, 0, 0} */
+ *   desc : int32[n][8] {x_start, shape0, shape1, stride0, stride1, y_start, capacity, 0}
+ * `capacity` = rows of Y[i]; a sample that would land beyond it is dropped (the
+ * position still advances), so an undrained buffer can never be overrun. */
 int nhip_probes(void *stream, const int *desc, int n, float *countdowns, int *bufpositions,
                 const float *periods, const float *X, float *Y);
 /* fill an int32 device array (used to zero probe buffer positions without a

@@ -232,10 +232,10 @@ __global__ __launch_bounds__(NHIP_WG) void direct_unary_kernel(int opcode,
 }
 
 // ---------------------------------------------------------------- probes
-// clra_nonlinearities.py:831-902.  One group per probe; the float32 countdown and
+// clra_nonlinearities.py:831-902 (plus a capacity guard).  One group per probe; the float32 countdown and
 // the buffer position are read by every thread before the barrier and written by
 // thread 0 after it.
-struct ProbeDesc { int x_start, shape0, shape1, stride0, stride1, y_start, p0, p1; };
+struct ProbeDesc { int x_start, shape0, shape1, stride0, stride1, y_start, capacity, p1; };
 
 __global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __restrict__ desc,
                                                          float* countdowns, int* bufpositions,
@@ -245,9 +245,11 @@ __global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __rest
     const float countdown = countdowns[n];
     const bool fire = countdown <= 0.0f;
     int bufpos = 0;
-    if (fire) {
+    // a full buffer (the host did not drain it in time) drops the sample instead of
+    // writing past the end; the position keeps counting so the host can tell
+    if (fire) bufpos = bufpositions[n];
+    if (fire && bufpos < desc[n].capacity) {
         const ProbeDesc d = desc[n];
-        bufpos = bufpositions[n];
         const int n_dims = d.shape0 * d.shape1;
         const float* x = X + d.x_start;
         float* y = Y + d.y_start + (size_t)bufpos * n_dims;

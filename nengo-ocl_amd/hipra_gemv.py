@@ -98,6 +98,10 @@ class gemv_prog:
         if len(self.A_js) != len(Y) or len(self.X_js) != len(Y):
             raise ValueError("need one A_js / X_js list per output")
 
+        # kernels trust these offsets: fail on the host if a view leaves its buffer
+        for name, ra in (("A", A), ("X", X), ("Y", Y), ("Y_in", Y_in)):
+            ra.check_bounds(name)
+
         geometry = []
         for b in range(len(Y)):
             M = int(Y.shape0s[b])
@@ -206,6 +210,8 @@ class gemv_prog:
         for (flavor, lpr, vec), members in sorted(by_class.items()):
             if flavor == 0:
                 rows = lib.nhip_gemv_rows_per_task(flavor, lpr, vec)
+            elif flavor == 2:
+                rows = WAVE // lpr  # one pass: these items are latency bound, spread them
             else:
                 rows = (WAVE // lpr) * 4  # four passes of a wave
             if rows <= 0:

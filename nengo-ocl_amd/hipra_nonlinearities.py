@@ -57,6 +57,13 @@ def blockify(sizes, max_size=BLOCK):
     return inds.astype(np.int32), offsets.astype(np.int32), counts.astype(np.int32)
 
 
+def _check(*named):
+    """Bounds-check ragged operands on the host before any kernel is bound to them."""
+    for name, ra in named:
+        if isinstance(ra, HIPRaggedArray):
+            ra.check_bounds(name)
+
+
 def _description(ra):
     sizes = ra.sizes
     if len(sizes) == 0:
@@ -90,6 +97,7 @@ def plan_timeupdate(queue, step, time, dt):
     assert step.ctype == time.ctype == "float"
     assert step.shape0s[0] == step.shape1s[0] == 1
     assert time.shape0s[0] == time.shape1s[0] == 1
+    _check(("step", step), ("time", time))
     args = (step.ptr, int(step.starts[0]), time.ptr, int(time.starts[0]), float(dt))
     return Plan(queue, queue.lib.nhip_timeupdate, args, gsize=(64,), lsize=(64,),
                 full_args=(step.dev_buf, time.dev_buf), name="hip_timeupdate")
@@ -102,6 +110,7 @@ def plan_reset(queue, Y, values, tag=None):
     assert (Y.stride0s == Y.shape1s).all()
     assert (Y.stride1s == 1).all()
     assert Y.ctype == "float"
+    _check(("Y", Y))
 
     inds, offsets, counts = blockify(Y.sizes, 4 * BLOCK)
     table, n = _dev_table(queue, [Y.starts[inds] + offsets, counts, _bits(values[inds])], 4)
@@ -123,6 +132,7 @@ def plan_copy(queue, X, Y, incs, tag=None):
     assert X.ctype == Y.ctype
     incs = np.asarray(incs, dtype=np.int32).reshape(-1)
     assert incs.shape == (len(X),)
+    _check(("X", X), ("Y", Y))
 
     inds, offsets, counts = blockify(Y.sizes)
     table, n = _dev_table(queue, [X.starts[inds], Y.starts[inds], X.shape1s[inds],
@@ -149,6 +159,12 @@ def plan_slicedcopy(queue, X, Y, Xinds, Yinds, incs, tag=None):
     assert Xinds.ctype == Yinds.ctype == "int"
     incs = np.asarray(incs, dtype=np.int32).reshape(-1)
     assert incs.shape == (len(X),)
+    _check(("X", X), ("Y", Y), ("Xinds", Xinds), ("Yinds", Yinds))
+    xi_host, yi_host = Xinds.to_host(), Yinds.to_host()
+    for k in range(len(X)):  # every index must address an element of its vector
+        if Xinds.shape0s[k]:
+            assert 0 <= xi_host[k].min() and xi_host[k].max() < X.shape0s[k], "Xinds[%d] out of range" % k
+            assert 0 <= yi_host[k].min() and yi_host[k].max() < Y.shape0s[k], "Yinds[%d] out of range" % k
 
     inds, offsets, counts = blockify(Xinds.shape0s)
     table, n = _dev_table(queue, [X.starts[inds], X.stride0s[inds], Y.starts[inds],
@@ -189,6 +205,7 @@ def plan_elementwise_inc(queue, A, X, Y, alpha=None, outer=False, inc=True, tag=
         alphas = alpha.astype(np.float32)
     else:
         alphas = np.ones(len(Y), dtype=np.float32)
+    _check(("A", A), ("X", X), ("Y", Y))
 
     inds, offsets, counts = blockify(Y.sizes)
     flags = np.full(len(inds), (1 if outer else 0) | (2 if inc else 0), dtype=np.int32)
@@ -230,6 +247,7 @@ def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
     assert (Ybuf.shape1s == Y.sizes).all()
     assert X.ctype == Xbuf.ctype
     assert Y.ctype == Ybuf.ctype
+    _check(("X", X), ("Y", Y), ("A", A), ("B", B), ("Xbuf", Xbuf), ("Ybuf", Ybuf))
 
     inds, offsets, counts = blockify(X.sizes)
     table, n = _dev_table(queue, [
@@ -261,13 +279,14 @@ def plan_probes(queue, periods, X, Y, tag=None):
     assert (X.shape0s * X.shape1s == Y.shape1s).all()
     assert (Y.stride0s == Y.shape1s).all()
     assert (Y.stride1s == 1).all()
+    _check(("X", X), ("Y", Y))
 
     periods = np.asarray(periods, dtype=np.float32)
     dev_periods = to_device(queue, periods)
     dev_countdowns = to_device(queue, periods - 1)
     dev_bufpositions = to_device(queue, np.zeros(N, dtype=np.int32))
     table, n = _dev_table(queue, [X.starts, X.shape0s, X.shape1s, X.stride0s, X.stride1s,
-                                  Y.starts], 8)
+                                  Y.starts, Y.shape0s], 8)
     plan = Plan(queue, queue.lib.nhip_probes,
                 (table.ptr, n, dev_countdowns.ptr, dev_bufpositions.ptr, dev_periods.ptr,
                  X.ptr, Y.ptr),
@@ -309,6 +328,7 @@ def plan_direct(queue, code, init, input_names, inputs, output, tag=None):
         raise NotImplementedError("unknown input %r" % m.group("arg"))
     x = inputs[list(input_names).index(m.group("arg"))]
     assert (x.shape0s == 1).all() and (output.shape0s == 1).all()
+    _check(("input", x), ("output", output))
 
     table, n = _dev_table(queue, [x.starts, output.starts, np.ones(len(output), np.int32)], 4)
     plan = Plan(queue, queue.lib.nhip_direct_unary,
@@ -380,6 +400,7 @@ def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, N=None, tau_n=None, inc_n=
     for x in [V, W, outS]:
         assert x.ctype == J.ctype
     _check_vectors([J, V, W, outS])
+    _check(("J", J), ("V", V), ("W", W), ("outS", outS), ("tau", tau), ("ref", ref), ("amp", amp))
 
     inds, offsets, counts = blockify(J.shape0s, 2 * WG)
     pcols, pflags, pptrs, keep = _neuron_params(queue, [tau, ref, amp], J.shape0s, inds, offsets)
@@ -405,6 +426,7 @@ def plan_lif_rate(queue, dt, J, R, ref, tau, amp, N=None, tau_n=None, inc_n=None
     assert J.ctype == "float"
     assert R.ctype == J.ctype
     _check_vectors([J, R])
+    _check(("J", J), ("R", R), ("tau", tau), ("ref", ref), ("amp", amp))
 
     inds, offsets, counts = blockify(J.shape0s, 2 * WG)
     pcols, pflags, pptrs, keep = _neuron_params(queue, [tau, ref, amp], J.shape0s, inds, offsets)
@@ -436,6 +458,7 @@ def plan_presentinput(queue, Y, t, signals, dt, pres_t=None, tag=None):
     assert (t.shape1s == 1).all()
     assert (Y.shape0s == signals.shape1s).all()
     assert (signals.stride0s == signals.shape1s).all()
+    _check(("Y", Y), ("t", t), ("signals", signals))
 
     table, n = _dev_table(queue, [
         Y.starts, Y.shape0s, t.starts, signals.starts, signals.shape0s,

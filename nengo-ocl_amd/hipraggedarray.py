@@ -207,6 +207,28 @@ class HIPRaggedArray:
     def __len__(self):
         return int(self.starts.size)
 
+    def check_bounds(self, what="ragged array"):
+        """Raise if any item reaches outside the device buffer.
+
+        Kernels trust the int32 offsets they are given; every plan builder calls
+        this on its operands so that a bad view fails on the host, at plan time,
+        instead of as a memory fault on the device."""
+        if len(self) == 0:
+            return
+        m = self.shape0s.astype(np.int64)
+        n = self.shape1s.astype(np.int64)
+        last = (self.starts.astype(np.int64) + np.maximum(m - 1, 0) * self.stride0s
+                + np.maximum(n - 1, 0) * self.stride1s)
+        used = (m * n) > 0
+        if np.any(self.starts < 0) or np.any(self.stride0s < 0) or np.any(self.stride1s < 0):
+            raise ValueError("%s: negative start or stride" % what)
+        if used.any() and int(last[used].max()) >= self.dev_buf.size:
+            bad = int(np.nonzero(used & (last >= self.dev_buf.size))[0][0])
+            raise ValueError("%s: item %d (start %d, shape %dx%d, strides %d,%d) runs past the "
+                             "end of its %d-element buffer" % (
+                                 what, bad, self.starts[bad], m[bad], n[bad], self.stride0s[bad],
+                                 self.stride1s[bad], self.dev_buf.size))
+
     # ------------------------------------------------------------- host access
     def _span(self, i):
         m, n = int(self.shape0s[i]), int(self.shape1s[i])
