@@ -95,6 +95,27 @@ def cpu_baseline(config, variant, scale, budget_s, dt_gpu_step):
                        "reference kernels, OpenMP over items), %.1f s" % (n, elapsed))
 
 
+def calibrate_copy(n_floats=64 * 1024 * 1024, repeats=20):
+    """Plain device copy of a known size through the library's copy kernel: reads
+    256 MiB and writes 256 MiB per launch.  Profiling this gives the scale of the
+    FETCH_SIZE / WRITE_SIZE counters for a kernel whose traffic is known."""
+    import numpy as np
+
+    from nengo_ocl_amd.hipra_nonlinearities import plan_copy
+    from nengo_ocl_amd.hipraggedarray import HIPRaggedArray, Queue
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    queue = Queue(0)
+    X = HIPRaggedArray(queue, RaggedArray([np.ones(n_floats, dtype=np.float32)]))
+    Y = HIPRaggedArray(queue, RaggedArray([np.zeros(n_floats, dtype=np.float32)]))
+    plan = plan_copy(queue, X, Y, np.zeros(1, dtype=np.int32))
+    for _ in range(repeats):
+        plan.enqueue()
+    queue.finish()
+    print(json.dumps({"kernel": "copy_kernel", "launches": repeats,
+                      "read_bytes_per_launch": 4 * n_floats, "write_bytes_per_launch": 4 * n_floats}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,7 +128,12 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
     ap.add_argument("--no-fuse", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run the plain copy kernel on 256 MiB (1 GiB of traffic per 2 "
+                         "launches) 20 times: the known-size reference for HBM counters")
     args = ap.parse_args()
+    if args.calibrate_copy:
+        return calibrate_copy()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the timestep of one simulator runs on a single "
                          "MI355X and nothing here uses a second device (got --gpus %d)" % args.gpus)

@@ -1,0 +1,70 @@
+"""The C ABI: the library loads and exports every entry point the header declares
+(no GPU needed, no compute call is made)."""
+
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "nengo_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nhip_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_symbols()
+    for required in ("nhip_gemv", "nhip_lif", "nhip_lif_rate", "nhip_linearfilter",
+                     "nhip_elementwise_inc", "nhip_copy", "nhip_slicedcopy", "nhip_reset",
+                     "nhip_timeupdate", "nhip_presentinput", "nhip_probes", "nhip_capture_begin",
+                     "nhip_graph_launch"):
+        assert required in names
+
+
+def test_library_exports_every_declared_symbol():
+    from nengo_ocl_amd import _lib
+
+    assert os.path.exists(_lib.LIB_PATH), "build with __graft_entry__.build()"
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(handle, name), "%s declared in nengo_hip.h but not exported" % name
+
+
+def test_binding_covers_header_and_versions_match():
+    import nengo_ocl_amd
+    from nengo_ocl_amd import _lib
+
+    bound = set(_lib.SIGNATURES) | {"nhip_error_string"}
+    assert bound == set(declared_symbols())
+    lib = _lib.lib()
+    assert lib.nhip_abi_version() == nengo_ocl_amd.ABI_VERSION
+    assert b"bad argument" in lib.nhip_error_string(-1)
+    assert lib.nhip_gemv_rows_per_task(0, 16, 4) == 128
+    assert lib.nhip_gemv_rows_per_task(0, 256, 4) == 4
+    assert lib.nhip_gemv_rows_per_task(0, 3, 4) == 0
+
+
+def test_product_does_not_import_the_oracle():
+    """Nothing under the package may reach into oracle/ (the checker is not a fallback)."""
+    pkg = os.path.join(ROOT, "nengo-ocl_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text, f
+                assert "liboracle" not in text, f
+
+
+def test_no_device_no_fallback():
+    """Without a HIP device the device layer raises instead of computing elsewhere."""
+    import pytest
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    from nengo_ocl_amd.hipraggedarray import Queue
+
+    with pytest.raises(RuntimeError):
+        Queue(0)

@@ -1,0 +1,243 @@
+"""Host logic above the plan_* boundary, run on the CPU oracle backend: operator
+rewrites, dependency graph, planners, the Simulator's run / probe / reset logic.
+
+Literal answers come from the reference's tests (tests/test_simulator.py:14-38,
+tests/test_planners.py:13-47, tests/test_operators.py:30,54,82).
+"""
+
+import numpy as np
+import pytest
+
+from nengo_ocl_amd import configs, ir, minibuilder
+from nengo_ocl_amd import operators as ops_mod
+from nengo_ocl_amd.operators import MultiDotInc
+from nengo_ocl_amd.planners import batching_planner, greedy_planner, operator_dependency_graph
+from oracle.oracle_sim import OracleSimulator
+
+
+def literal_model():
+    a = ir.Signal([0, 0], name="a")
+    b = ir.Signal([0, 0], name="b")
+    A = ir.Signal([[1, 2], [0, 1]], name="A")
+    B = ir.Signal([[2, 1], [-1, 1]], name="B")
+    x = ir.Signal([1, 1], name="x")
+    y = ir.Signal([1, -1], name="y")
+    m = ir.Model(dt=0.001)
+    m.operators += [ir.Reset(a), ir.DotInc(A, x, a), ir.DotInc(B, y, a)]
+    m.operators += [ir.DotInc(A, y, b), ir.DotInc(B, x, b)]
+    return m, a, b
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_multidotinc_compress_literal(fuse):
+    """tests/test_simulator.py:14-38: a = [4, -1]; b = [2, -1] then [4, -2]."""
+    m, a, b = literal_model()
+    with OracleSimulator(None, model=m, fuse=fuse) as sim:
+        n_mdi = sum(isinstance(op, MultiDotInc) for op in sim.operators)
+        assert n_mdi == 2  # four DotIncs folded onto two targets
+        sim.step()
+        assert np.allclose(sim.signals[a], [4, -1])
+        assert np.allclose(sim.signals[b], [2, -1])
+        sim.step()
+        assert np.allclose(sim.signals[a], [4, -1])
+        assert np.allclose(sim.signals[b], [4, -2])
+
+
+def test_get_views_scalar_swap_and_shapes():
+    y = ir.Signal(np.zeros(5), name="y")
+    x = ir.Signal(np.ones(5), name="x")
+    a = ir.Signal(np.array(2.0), name="a")
+    op = MultiDotInc(y, y, beta=1, gamma=0)
+    op.add_AX(a, x)
+    A_views, X_views, Y_view, Y_in_view, beta_view = op.get_views()
+    assert A_views[0].shape == (5, 1) and X_views[0].shape == (1, 1)  # scalar A swapped with X
+    assert Y_view.shape == (5, 1) and beta_view is None
+    assert op.incs == [y] and op.sets == []
+    bad = MultiDotInc(y, y, beta=1, gamma=0)
+    bad.add_AX(ir.Signal(np.zeros((4, 5))), x)
+    with pytest.raises(ValueError):
+        bad.get_views()
+    setter = MultiDotInc(y, x, beta=1, gamma=0)
+    assert setter.sets == [y] and x in setter.reads
+
+
+def feedforward_network(n=5):
+    """The shape of tests/test_planners.py:22-38: n nodes -> n ensembles, probed."""
+    net = minibuilder.Network(seed=0)
+    probes = []
+    for i in range(n):
+        node = net.Node(minibuilder.WhiteSignal(1.0, 5.0, seed=i), size_out=1)
+        ens = net.Ensemble(10, 1)
+        net.Connection(node, ens, synapse=None)
+        probes.append(net.Probe(ens, synapse=0.01))
+    return net, probes
+
+
+@pytest.mark.parametrize("planner", [greedy_planner, batching_planner])
+@pytest.mark.parametrize("fuse", [True, False])
+def test_planner_groups(planner, fuse):
+    net, _ = feedforward_network()
+    with OracleSimulator(net, planner=planner, fuse=fuse) as sim:
+        names = [t.__name__ for t, _ in sim.op_groups]
+        assert names.count("Reset") <= 1  # all resets planned together (test_planners.py:18)
+        assert names.count("SimNeurons") == 1
+        assert sum(len(ops) for _, ops in sim.op_groups) == len(sim.operators)
+        # every op runs after all of its predecessors
+        edges = operator_dependency_graph(sim.operators)
+        position = {op: k for k, (_, ops) in enumerate(sim.op_groups) for op in ops}
+        for pre, posts in edges.items():
+            for post in posts:
+                assert position[pre] < position[post]
+        # no two ops of a group write overlapping memory
+        for _, ops in sim.op_groups:
+            written = [s for op in ops for s in list(op.sets) + list(op.incs) + list(op.updates)]
+            for i, s in enumerate(written):
+                for s2 in written[i + 1:]:
+                    assert not (s is s2 or s.may_share_memory(s2))
+
+
+def test_fusion_cuts_groups_and_keeps_results():
+    make = lambda: configs.c2_watts_strogatz(n_ens=48, n_driven=6)
+    sims = []
+    for fuse in (True, False):
+        net, probes, _ = make()
+        sim = OracleSimulator(net, seed=1, fuse=fuse)
+        sim.run_steps(200)
+        sims.append((sim, probes))
+    (fused, pf), (plain, pp) = sims
+    assert len(fused.op_groups) < len(plain.op_groups) and len(fused.op_groups) <= 8
+    for k in pf:
+        assert np.array_equal(fused.data[pf[k]], plain.data[pp[k]])  # same additions, same order
+
+
+def test_cycle_is_reported():
+    a, b = ir.Signal(np.zeros(2), name="a"), ir.Signal(np.zeros(2), name="b")
+    ops = [ir.Copy(a, b), ir.Copy(b, a)]  # a set-before-read cycle
+    with pytest.raises(ValueError):
+        greedy_planner(ops)
+
+
+def test_simplifications_remove_ops():
+    """remove_unmodified_resets drops 1 op, remove_zero_incs 1, both 2
+    (tests/test_operators.py:30, :54, :82: an ensemble without input)."""
+    def n_ops(simps):
+        net = minibuilder.Network(seed=0)
+        ens = net.Ensemble(10, 2)
+        net.Probe(ens, synapse=0.01)
+        model = net.build_model()
+        old = ops_mod.simplifications
+        ops_mod.simplifications = simps
+        try:
+            return len(ops_mod.simplify_operators(list(model.operators)))
+        finally:
+            ops_mod.simplifications = old
+
+    base = n_ops([])
+    assert n_ops([ops_mod.remove_unmodified_resets]) == base - 1
+    assert n_ops([ops_mod.remove_zero_incs]) == base - 1
+    assert n_ops([ops_mod.remove_unmodified_resets, ops_mod.remove_zero_incs]) == base - 2
+
+
+def test_run_probe_reset_semantics():
+    net, probes, _ = configs.c0_readme()
+    with OracleSimulator(net, n_prealloc_probes=4, seed=1) as sim:
+        assert sim._max_steps_between_probes == 4
+        sim.run_steps(37)
+        first = np.array(sim.data[probes["a"]])
+        assert first.shape == (37, 1) and sim.n_steps == 37 and abs(sim.time - 0.037) < 1e-9
+        assert np.allclose(sim.trange(), 0.001 * np.arange(1, 38))
+        assert np.allclose(sim.trange(sample_every=0.005), 0.001 * np.arange(5, 38, 5))
+        sim.reset()
+        assert sim.n_steps == 0 and len(sim.data[probes["a"]]) == 0
+        sim.run(0.0366)  # rounds to 37 steps
+        assert np.array_equal(first, sim.data[probes["a"]])
+        sim.clear_probes()
+        sim.run_steps(5)
+        assert len(sim.data[probes["a"]]) == 5 and sim.n_steps == 42
+        with pytest.raises(ValueError):
+            sim.run_steps(-1)
+        with pytest.raises(ValueError):
+            sim.run_steps(2 ** 24)
+        with pytest.raises(ValueError):
+            sim.run(-1.0)
+        with pytest.raises(NotImplementedError):
+            sim.reset(seed=3)
+    from nengo_ocl_amd.simulator import SimulatorClosed
+
+    with pytest.raises(SimulatorClosed):
+        sim.run_steps(1)
+    with pytest.raises(SimulatorClosed):
+        sim.reset()
+    with pytest.raises(NotImplementedError):
+        sim.__getstate__()
+
+
+def test_probe_sample_every():
+    net, _, _ = configs.c4_pes(n_triples=1, n_neurons=50, dims=2, solver="lstsq", sample_every=0.01)
+    p_fast = net.Probe(net.ensembles[0], synapse=0.01)
+    p_slow = net.probes[0]
+    with OracleSimulator(net, seed=1) as sim:
+        assert sim._max_steps_between_probes == 32  # 32 buffer rows x the shortest period (1 step)
+        sim.run_steps(95)
+        assert len(sim.data[p_fast]) == 95 and len(sim.data[p_slow]) == 9
+        assert len(sim.trange(sample_every=0.01)) == 9
+
+
+def test_python_function_fallback_and_if_python_code():
+    def make(fn):
+        net = minibuilder.Network(seed=0)
+        node = net.Node(fn, label="f")
+        ens = net.Ensemble(20, 1)
+        net.Connection(node, ens, synapse=None)
+        return net, net.Probe(node)
+
+    net, p = make(lambda t: np.cos(3 * t))
+    with OracleSimulator(net) as sim:
+        assert any(plan.name == "python_fn" for plan in sim._plans)
+        sim.run_steps(20)
+        t = sim.trange()
+        assert np.allclose(sim.data[p][:, 0], np.cos(3 * t), atol=1e-6)
+    with pytest.raises(RuntimeError):
+        OracleSimulator(make(lambda t: t)[0], if_python_code="error")
+    with pytest.warns(RuntimeWarning):
+        OracleSimulator(make(lambda t: t)[0], if_python_code="warn").close()
+    net, p = make(np.sin)  # in the unary table: no host callback
+    with OracleSimulator(net, if_python_code="error") as sim:
+        sim.run_steps(10)
+        assert np.allclose(sim.data[p][:, 0], np.sin(sim.trange()), atol=1e-6)
+
+
+def test_circconv_transforms_exact():
+    for dims in (4, 16, 64):
+        tr_a, tr_b, tr_out = configs.circconv_transforms(dims)
+        rng = np.random.RandomState(dims)
+        a, b = rng.normal(size=dims), rng.normal(size=dims)
+        expect = np.fft.irfft(np.fft.rfft(a) * np.fft.rfft(b), n=dims)
+        assert np.allclose(tr_out @ ((tr_a @ a) * (tr_b @ b)), expect)
+        assert tr_a.shape == (4 * (dims // 2 + 1), dims)
+
+
+def test_watts_strogatz_edges():
+    rng = np.random.RandomState(0)
+    edges = configs.watts_strogatz_edges(200, 10, 0.1, rng)
+    assert len(edges) == 2000 and len(set(edges)) == 2000
+    assert all(i != j for i, j in edges)
+    lattice = sum(1 for i, j in edges if min((i - j) % 200, (j - i) % 200) <= 5)
+    assert 0.8 * 2000 < lattice < 2000  # about 10 % rewired
+
+
+def test_decoders_decode():
+    """LstsqL2 decoders of the mini-builder reproduce x and x**2 from rate activities."""
+    net = minibuilder.Network(seed=3)
+    ens = net.Ensemble(200, 1)
+    out = net.Node(size_in=2)
+    net.Connection(ens, out[0:1], synapse=None)
+    net.Connection(ens, out[1:2], function=lambda x: x ** 2, synapse=None)
+    model = net.build_model()
+    p = model.params[ens]
+    xs = np.linspace(-1, 1, 21)[:, None]
+    acts = ens.neuron_type.rates_from_current(p["gain"] * (xs @ p["encoders"].T) + p["bias"])
+    ws = [model.params[c]["weights"] for c in net.connections]
+    assert np.abs(acts @ ws[0].T - xs).max() < 0.05
+    assert np.abs(acts @ ws[1].T - xs ** 2).max() < 0.05
+    assert np.all(acts.max(axis=0) <= 400.5)

@@ -1,0 +1,332 @@
+"""Pins for the CPU oracle: each restated kernel is checked against something that
+does not share its code -- literal vectors held by the reference's own tests,
+closed forms, float64 brute force, library routines (numpy / scipy).
+
+The reference itself cannot be imported here (nengo, pyopencl and mako are not
+installed), so these are what fix the oracle's behaviour; the GPU tests then
+compare the HIP kernels with the oracle.
+"""
+
+import numpy as np
+import pytest
+
+from helpers import RA, clone
+from oracle import oracle as orc
+
+
+# ------------------------------------------------------------------ GEMV
+def test_gemv_literal_vectors():
+    """nengo_ocl/tests/test_clra_gemv.py:60-93: Y0 = 4.5, Y1 = [3.3, 5.9]."""
+    A = RA([[[0.1, 0.2], [0.3, 0.4]], [[0.5, 0.6]]])
+    X = RA([[3, 5]])
+    Y = RA([[0.0], [2, 3]])
+    A_js = RA([[1], [0]], dtype=np.int32)
+    X_js = RA([[0], [0]], dtype=np.int32)
+    orc.plan_block_gemv(None, 1.0, A, A_js, X, X_js, 1.0, Y).plans[0]()
+    np.testing.assert_allclose(Y[0].ravel(), [4.5], rtol=1e-6)
+    np.testing.assert_allclose(Y[1].ravel(), [3.3, 5.9], rtol=1e-6)
+
+
+@pytest.mark.parametrize("k,p,m,n", [(4, 1, 10, 10), (10, 1, 550, 550), (4, 4, 10, 10),
+                                     (4, 4, 500, 300)])
+def test_gemv_seeded_random_against_float64(k, p, m, n):
+    """The seeded sweep of test_clra_gemv.py:96-145 (RandomState(3294), alpha 0.5, beta 0.1)."""
+    rng = np.random.RandomState(3294)
+    aa = [rng.normal(size=(m, n)) for _ in range(k)]
+    xx = [rng.normal(size=n) for _ in range(k)]
+    yy = [rng.normal(size=m) for _ in range(k)]
+    ajs = [rng.randint(k, size=p) for _ in range(k)]
+    xjs = [rng.randint(k, size=p) for _ in range(k)]
+    A, X, Y = RA(aa), RA(xx), RA(yy)
+    Y0 = clone(Y)
+    orc.plan_block_gemv(None, 0.5, A, RA(ajs, dtype=np.int32), X, RA(xjs, dtype=np.int32), 0.1, Y).plans[0]()
+    for i in range(k):
+        ref = 0.1 * Y0[i].astype(np.float64)
+        for aj, xj in zip(ajs[i], xjs[i]):
+            ref += 0.5 * (A[aj].astype(np.float64) @ X[xj].astype(np.float64))
+        np.testing.assert_allclose(Y[i], ref, rtol=1e-4, atol=1e-4)
+
+
+def test_gemv_gamma_yin_and_strides():
+    """gamma, a Y_in different from Y, a transposed-stride X and a row-strided A: a dropped
+    term, a swapped operand or a wrong stride changes the result."""
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    rng = np.random.RandomState(1234)
+    base = RA([rng.rand(6, 10), rng.rand(40), rng.rand(6), rng.rand(6)])
+    s = base.starts
+    base.add_views([s[0] + 2, s[1] + 1], [6, 7], [7, 1], [10, 5], [1, 1])  # A = M[:, 2:9], x = v[1::5][:7]
+    Y = RaggedArray.from_buffer(base.buf, [s[2]], [6], [1], [1], [1])
+    Yin = RaggedArray.from_buffer(base.buf, [s[3]], [6], [1], [1], [1])
+    expect = 0.7 + 0.6 * base[3][:, 0].astype(np.float64) + 0.5 * (
+        base[0][:, 2:9].astype(np.float64) @ base[1][1::5][:7, 0].astype(np.float64))
+    orc.plan_block_gemv(None, 0.5, base, [np.array([4])], base, [np.array([5])], 0.6, Y, Y_in=Yin,
+                        gamma=0.7).plans[0]()
+    np.testing.assert_allclose(Y[0][:, 0], expect, rtol=1e-6)
+
+
+def test_gemv_block_order_is_the_reference_order():
+    """The four strided partial sums per 128-column tile, (s0+s2)+(s1+s3), tiles in
+    order (clra_gemv.py:1043-1058, :1148-1153), replayed step by step in numpy float32."""
+    rng = np.random.RandomState(5)
+    n = 300  # three tiles: 128, 128, 44
+    a = rng.normal(size=(1, n)).astype(np.float32)
+    x = rng.normal(size=n).astype(np.float32)
+    y0 = np.float32(0.25)
+    Y = RA([[y0]])
+    orc.plan_block_gemv(None, 1.0, RA([a]), [np.array([0])], RA([x]), [np.array([0])], 1.0, Y).plans[0]()
+    total = y0
+    for c0 in range(0, n, 128):
+        s = np.zeros(4, dtype=np.float32)
+        for jj in range(min(128, n - c0)):
+            s[jj % 4] = np.float32(s[jj % 4] + np.float32(a[0, c0 + jj] * x[c0 + jj]))
+        total = np.float32(total + np.float32(np.float32(s[0] + s[2]) + np.float32(s[1] + s[3])))
+    assert Y[0][0, 0] == total
+
+
+# ------------------------------------------------------------------- LIF
+def lif_step_float64(dt, J, V, W, tau_rc, tau_ref, amplitude=1.0):
+    """nengo's LIF.step as the reference's test_lif_step (:35-91) runs it on the host:
+    refractory countdown, exponential integration over the non-refractory part of the
+    step, spike with interpolated spike time."""
+    W = W - dt
+    delta_t = np.clip(dt - W, 0, dt)
+    V = V - (J - V) * np.expm1(-delta_t / tau_rc)
+    spiked = V > 1
+    out = spiked * (amplitude / dt)
+    t_spike = dt + tau_rc * np.log1p(-(V[spiked] - 1) / (J[spiked] - 1))
+    V[V < 0] = 0
+    V[spiked] = 0
+    W[spiked] = tau_ref + t_spike
+    return V, W, out
+
+
+def test_lif_step_against_float64():
+    rng = np.random.RandomState(8)
+    dt, ref, amp = 1e-3, 2e-3, 1.0
+    n_neurons = [12345, 23456, 34567]
+    taus = rng.uniform(15e-3, 80e-3, size=3)
+    J = RA([rng.normal(scale=1.2, size=n) for n in n_neurons])
+    V = RA([rng.uniform(0, 1, size=n) for n in n_neurons])
+    W = RA([rng.uniform(-5 * dt, 5 * dt, size=n) for n in n_neurons])
+    S = RA([np.zeros(n) for n in n_neurons])
+    V0, W0 = clone(V), clone(W)
+    orc.plan_lif(None, dt, J, V, W, S, ref, RA([t * np.ones(n) for t, n in zip(taus, n_neurons)]), amp)()
+    n_spikes = 0
+    for i in range(3):
+        v, w, s = lif_step_float64(dt, J[i][:, 0].astype(np.float64), V0[i][:, 0].astype(np.float64),
+                                   W0[i][:, 0].astype(np.float64), taus[i], ref, amp)
+        agree = (S[i][:, 0] > 0) == (s > 0)
+        assert agree.mean() > 0.9999  # a float32 voltage within rounding of the threshold may differ
+        np.testing.assert_allclose(V[i][agree, 0], v[agree], atol=1e-5)
+        np.testing.assert_allclose(W[i][agree, 0], w[agree], atol=1e-6)
+        np.testing.assert_allclose(S[i][agree, 0], s[agree])
+        n_spikes += int((s > 0).sum())
+    assert n_spikes > 50  # the spike branch is exercised
+
+
+def test_lif_constant_input_rate_and_bounds():
+    """Constant J: the spike count over 1 s is rate(J) within one spike, where
+    rate = 1/(tau_ref + tau_rc*log1p(1/(J-1))); J <= 1 never spikes and V -> J;
+    V stays in [0, 1] and S takes two values."""
+    dt, tau_rc, tau_ref, amp = 1e-3, 0.02, 0.002, 1.0
+    Jv = np.array([0.5, 0.99, 1.0, 1.05, 1.5, 2.0, 5.0, 10.0, 40.0], dtype=np.float32)
+    J, V, W, S = RA([Jv]), RA([np.zeros(Jv.size)]), RA([np.zeros(Jv.size)]), RA([np.zeros(Jv.size)])
+    plan = orc.plan_lif(None, dt, J, V, W, S, tau_ref, tau_rc, amp)
+    counts = np.zeros(Jv.size)
+    for _ in range(1000):
+        plan()
+        counts += S[0][:, 0] * dt
+        assert np.all(V[0] >= 0) and np.all(V[0] <= 1)
+        assert set(np.unique(S[0])) <= {0.0, np.float32(1000.0)}
+    rate = np.zeros(Jv.size)
+    m = Jv > 1
+    rate[m] = 1.0 / (tau_ref + tau_rc * np.log1p(1.0 / (Jv[m].astype(np.float64) - 1)))
+    assert np.all(counts[~m] == 0)
+    assert np.all(np.abs(counts - rate) <= 1.0 + 1e-9)
+    np.testing.assert_allclose(V[0][:2, 0], Jv[:2], rtol=1e-4)  # subthreshold voltage settles at J
+
+
+def test_lif_upsample_equals_substeps():
+    rng = np.random.RandomState(2)
+    dt = 1e-3
+    J = RA([rng.normal(1.5, 1.0, size=500)])
+    V = RA([rng.uniform(0, 1, size=500)])
+    W = RA([rng.uniform(-2 * dt, 2 * dt, size=500)])
+    S = RA([np.zeros(500)])
+    V2, W2, S2 = clone(V), clone(W), clone(S)
+    orc.plan_lif(None, dt, J, V, W, S, 2e-3, 0.02, 1.0, upsample=4)()
+    any_spike = np.zeros(500, dtype=bool)
+    sub = orc.plan_lif(None, dt / 4, J, V2, W2, S2, 2e-3, 0.02, 1.0)
+    for _ in range(4):
+        sub()
+        any_spike |= S2[0][:, 0] > 0
+    np.testing.assert_allclose(V[0], V2[0], atol=1e-6)
+    np.testing.assert_allclose(W[0], W2[0], atol=1e-7)
+    assert np.array_equal(S[0][:, 0] > 0, any_spike)
+    assert set(np.unique(S[0])) <= {0.0, np.float32(1000.0)}  # amp/dt, not amp/(dt/4)
+
+
+def test_lif_rate_closed_form():
+    rng = np.random.RandomState(3)
+    Jv = rng.normal(1, 10, size=5000).astype(np.float32)
+    J, R = RA([Jv]), RA([np.zeros(Jv.size)])
+    orc.plan_lif_rate(None, 1e-3, J, R, 2e-3, 0.03, 1.5)()
+    j = np.maximum(Jv.astype(np.float64) - 1, 0)
+    with np.errstate(divide="ignore"):
+        expect = 1.5 / (2e-3 + 0.03 * np.log1p(1.0 / j))
+    np.testing.assert_allclose(R[0][:, 0], expect, rtol=2e-6, atol=1e-6)
+    assert np.all(R[0][Jv <= 1] == 0)
+    assert np.array_equal(J[0][:, 0], Jv)
+
+
+# --------------------------------------------------------------- filters
+def test_lowpass_step_response():
+    """y[n] = a y[n-1] + (1-a) x[n], a = exp(-dt/tau): unit step gives 1 - a^n."""
+    dt, tau = 1e-3, 0.005
+    a = np.exp(-dt / tau)
+    X, Y = RA([np.ones(7)]), RA([np.zeros(7)])
+    A, B = RA([[-a]]), RA([[1 - a]])
+    (plan,) = orc.plan_linearfilter(None, X, Y, A, B, RA([np.zeros((1, 7))]), RA([np.zeros((1, 7))]))
+    for n in range(1, 60):
+        plan()
+        np.testing.assert_allclose(Y[0][:, 0], 1 - a ** n, rtol=2e-6)
+
+
+def test_general_filter_against_scipy():
+    """Second-order (alpha) synapse, zero-order hold, in the reference's packing
+    (simulator.py:1214-1227) against scipy.signal.lfilter; also a 2-D strided signal."""
+    from scipy.signal import cont2discrete, lfilter
+
+    dt, tau = 1e-3, 0.005
+    numd, dend, _ = cont2discrete(([1.0], [tau * tau, 2 * tau, 1.0]), dt, method="zoh")
+    num, den = numd.ravel()[1:], dend[1:]
+    rng = np.random.RandomState(4)
+    n_steps, shape = 50, (3, 4)
+    xs = rng.normal(size=(n_steps,) + shape).astype(np.float32)
+    base = RA([np.zeros((3, 6)), np.zeros(shape)])
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    X = RaggedArray.from_buffer(base.buf, [base.starts[0] + 1], [3], [4], [6], [1])  # columns 1..4 of a 3x6
+    Y = base[[1]]
+    (plan,) = orc.plan_linearfilter(None, X, Y, RA([den]), RA([num]), RA([np.zeros((2, 12))]),
+                                    RA([np.zeros((2, 12))]))
+    ys = []
+    for n in range(n_steps):
+        base[0][:, 1:5] = xs[n]
+        plan()
+        ys.append(np.array(Y[0]))
+    expect = lfilter(np.float32(num).astype(np.float64), np.concatenate([[1.0], np.float32(den)]),
+                     xs.astype(np.float64), axis=0)
+    np.testing.assert_allclose(np.array(ys), expect, rtol=1e-4, atol=1e-6)
+
+
+def test_gain_only_filter():
+    X, Y = RA([[1.0, -2.0, 3.0]]), RA([np.zeros(3)])
+    (plan,) = orc.plan_linearfilter(None, X, Y, RA([[]]), RA([[2.0]]), RA([np.zeros((1, 3))]),
+                                    RA([np.zeros((0, 3))]))
+    plan()
+    assert np.array_equal(Y[0][:, 0], [2.0, -4.0, 6.0])
+
+
+# ------------------------------------------------- element-wise and copies
+def test_elementwise_inc_against_numpy():
+    rng = np.random.RandomState(6)
+    Xs = [(3, 3), (32, 64), (45, 34), (1, 100)]
+    As = [(3, 3), (1, 1), (45, 34), (100, 1)]
+    A, X = RA([rng.normal(size=s) for s in As]), RA([rng.normal(size=s) for s in Xs])
+    alpha = rng.normal(size=4).astype(np.float32)
+    Y = RA([rng.normal(size=np.broadcast(A[i], X[i]).shape) for i in range(4)])
+    for inc in (True, False):
+        Yo = clone(Y)
+        orc.plan_elementwise_inc(None, A, X, Yo, alpha=alpha, inc=inc)()
+        for k in range(4):
+            ax = (alpha[k] * A[k]) * X[k]
+            assert np.array_equal(Yo[k], Y[k] + ax if inc else ax)
+
+
+def test_outer_product_pes_form():
+    rng = np.random.RandomState(7)
+    err, pre = rng.normal(size=5).astype(np.float32), rng.normal(size=40).astype(np.float32)
+    delta = RA([rng.normal(size=(5, 40))])
+    alpha = np.array([-1e-4 * 1e-3 / 40], dtype=np.float32)
+    orc.plan_elementwise_inc(None, RA([err]), RA([pre]), delta, alpha=alpha, outer=True, inc=False)()
+    assert np.array_equal(delta[0], np.outer(alpha[0] * err, pre))
+
+
+def test_copy_slicedcopy_reset_against_numpy():
+    rng = np.random.RandomState(9)
+    sizes = [(10, 1), (40, 64), (1, 100)]
+    X, Y = RA([rng.normal(size=s) for s in sizes]), RA([rng.normal(size=s) for s in sizes])
+    Y0 = clone(Y)
+    orc.plan_copy(None, X, Y, np.array([1, 0, 1]))()
+    for i, inc in enumerate([1, 0, 1]):
+        assert np.array_equal(Y[i], Y0[i] + X[i] if inc else X[i])
+
+    A, B = RA([rng.normal(size=30), rng.normal(size=50)]), RA([rng.normal(size=30), rng.normal(size=50)])
+    ai = [rng.permutation(30)[:12].astype(np.int32), np.arange(10, dtype=np.int32)]
+    bi = [rng.permutation(30)[:12].astype(np.int32), np.arange(40, 50, dtype=np.int32)]
+    expect = clone(B)
+    expect[0][bi[0], 0] += A[0][ai[0], 0]
+    expect[1][bi[1], 0] = A[1][ai[1], 0]
+    orc.plan_slicedcopy(None, A, B, RA(ai, dtype=np.int32), RA(bi, dtype=np.int32), np.array([1, 0]))()
+    assert np.array_equal(B.buf, expect.buf)
+
+    Z = RA([np.ones(1000), np.ones((10, 17)), np.ones((3, 3))])
+    vals = np.array([0.5, -2.0, 7.0], dtype=np.float32)
+    orc.plan_reset(None, Z, vals)()
+    for i, v in enumerate(vals):
+        assert np.all(Z[i] == v)
+
+
+# ------------------------------------------------------- time, inputs, probes
+def test_timeupdate_float32_counter():
+    sig = RA([np.zeros(1), np.zeros(1)])
+    plan = orc.plan_timeupdate(None, sig[[0]], sig[[1]], 0.001)
+    for n in range(1, 3001):
+        plan()
+        assert sig[0][0, 0] == np.float32(n)
+        assert sig[1][0, 0] == np.float32(0.001 * n)  # double product, rounded once
+
+
+def test_presentinput_rows():
+    rng = np.random.RandomState(10)
+    tables = [rng.normal(size=(1000, 1)), rng.normal(size=(37, 5))]
+    S, Y = RA(tables), RA([np.zeros(1), np.zeros(5)])
+    for step in [0, 1, 36, 37, 999, 1000, 4321]:
+        T = RA([[float(step)], [float(step)]])
+        orc.plan_presentinput(None, Y, T, S, 0.001)()
+        for i, t in enumerate(tables):
+            assert np.array_equal(Y[i][:, 0], np.float32(t[step % t.shape[0]]))
+    # with a presentation time: row = int((step - 0.5) * dt / pt) mod rows
+    T = RA([[250.0], [250.0]])
+    orc.plan_presentinput(None, Y, T, S, 0.001, pres_t=np.array([0.01, 0.05], dtype=np.float32))()
+    assert np.array_equal(Y[0][:, 0], np.float32(tables[0][24]))
+    assert np.array_equal(Y[1][:, 0], np.float32(tables[1][4]))
+
+
+def test_probe_schedule_matches_trange_rule():
+    """A probe with period p (in steps) fires at the steps n with n % p < 1
+    (simulator.py:700-702), for integer and non-integer periods."""
+    periods = [1.0, 2.0, 2.5, 10.0]
+    X = RA([np.zeros(1)] * len(periods))
+    Y = RA([np.zeros((64, 1))] * len(periods))
+    plan = orc.plan_probes(None, periods, X, Y)
+    fired = [[] for _ in periods]
+    for n in range(1, 41):
+        X.buf[:] = n
+        before = plan.bufpositions.copy()
+        plan()
+        for i in range(len(periods)):
+            if plan.bufpositions[i] > before[i]:
+                fired[i].append(n)
+    steps = np.arange(1, 41)
+    for i, p in enumerate(periods):
+        assert fired[i] == list(steps[steps % p < 1]), p
+        assert np.array_equal(Y[i][: len(fired[i]), 0], fired[i])  # the sampled values, in order
+
+
+def test_direct_unary():
+    x, y = RA([[0.731], [2.5]]), RA([[0.0], [0.0]])
+    orc.plan_direct_unary(None, "sin", x, y)()
+    np.testing.assert_allclose(y.buf, np.sin(np.float32([0.731, 2.5])), rtol=1e-6)
