@@ -68,13 +68,30 @@ int nhip_device_info(int *n_cu, int *wave_size, int *lds_bytes, char *name, int 
  * tiles added in order; lpr must be 4 and vec 1): bit-identical to a float32
  * restatement of that kernel.  `lpr` = lanes cooperating on one row (1,2,...,64, or
  * 256 for flavor 0); `vec` = 4 (16-byte loads; needs a_start % 4 == 0 and
- * a_stride0 % 4 == 0 for every dot of the launch) or 1.  The host validates
- * these preconditions; the kernel trusts them. */
-int nhip_gemv(void *stream, int flavor, int lpr, int vec, const int *items,
+ * a_stride0 % 4 == 0 for every dot of the launch) or 1.  `passes` (flavor 0) =
+ * rows each lane accumulates at once, i.e. independent loads in flight: 2, 4, 8,
+ * or 0 for the class default.  The host validates these preconditions; the
+ * kernel trusts them. */
+int nhip_gemv(void *stream, int flavor, int lpr, int vec, int passes, const int *items,
               const float *coefs, const int *dots, const int *tasks, int n_tasks,
               const float *A, const float *X, const float *Yin, float *Y);
 /* rows one task of the given class covers at most (0 if the class is unknown) */
-int nhip_gemv_rows_per_task(int flavor, int lpr, int vec);
+int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
+
+/* The same operation and the same four tables, summed in the ORDER of the
+ * reference's block kernel (clra_gemv.py:1043-1058, :1148-1153: four strided
+ * partial sums per 128-column tile, (s0+s2)+(s1+s3), tiles added in order, products
+ * rounded separately), for large items: a wave owns the rows of one task (four tasks
+ * per 256-thread group) and streams the matrix through a wave-private LDS block of
+ * `blk_words` float32 (a multiple of 4, >= 1056; 2176 = 8.5 KiB by default), so the
+ * result is bit-identical to a float32 restatement of that kernel while HBM is
+ * still read in whole lines.  A task may cover at most
+ * nhip_gemv_tile_rows(N, blk_words) rows for every dot product (N columns) of its
+ * item.  `vec` as for nhip_gemv. */
+int nhip_gemv_tile(void *stream, int vec, int blk_words, const int *items, const float *coefs,
+                   const int *dots, const int *tasks, int n_tasks, const float *A,
+                   const float *X, const float *Yin, float *Y);
+int nhip_gemv_tile_rows(int n_cols, int blk_words);
 
 /* ---- neurons -----------------------------------------------------------
  * LIF with refractory state and spike-time interpolation.

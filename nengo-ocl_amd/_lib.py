@@ -11,7 +11,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libnengo_hip.so")
+# NENGO_HIP_LIBRARY points at an alternative build of the same ABI (kernel experiments)
+LIB_PATH = os.environ.get("NENGO_HIP_LIBRARY") or os.path.join(_HERE, "libnengo_hip.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 c_int = ctypes.c_int
@@ -24,8 +25,10 @@ P = ctypes.c_void_p  # every device pointer crosses the boundary as void*
 SIGNATURES = {
     "nhip_abi_version": [],
     "nhip_device_info": [P, P, P, ctypes.c_char_p, c_int],
-    "nhip_gemv": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P],
-    "nhip_gemv_rows_per_task": [c_int, c_int, c_int],
+    "nhip_gemv": [P, c_int, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P],
+    "nhip_gemv_rows_per_task": [c_int, c_int, c_int, c_int],
+    "nhip_gemv_tile": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P],
+    "nhip_gemv_tile_rows": [c_int, c_int],
     "nhip_lif": [P, P, c_int, c_double, c_int, P, P, P, P, P, P, P],
     "nhip_lif_rate": [P, P, c_int, P, P, P, P, P],
     "nhip_linearfilter": [P, P, P, c_int, P, P, P, P, P, P],

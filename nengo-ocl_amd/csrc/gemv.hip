@@ -24,18 +24,39 @@
 // Lanes of a row own interleaved column quads (lane l: columns 4l..4l+3, then
 // + 4*LPR ...), so one load instruction of a wave covers contiguous memory.
 #include "nhip_common.h"
+#include "gemv_types.h"
 
 namespace {
 
-struct GemvItem { int y_start, y_stride0, yin_start, yin_stride0, dot_begin, n_dots, M, pad; };
-struct GemvDot { int a_start, a_stride0, N, x_start, x_stride0, p0, p1, p2; };
-struct GemvTask { int item, row0, n_rows, pad; };
 
 constexpr int XCHUNK = 4096;  // floats of X staged per pass: 16 KiB of the 160 KiB LDS
 
 // rows accumulated at once by each lane (independent loads in flight)
-template <int LPR> struct PassCount { static constexpr int value = 4; };
-template <> struct PassCount<16> { static constexpr int value = 8; };
+// default rows per lane, measured on MI355X (256 matrices of 4096 x 64 and of
+// 64 x 4096, alternating)
+template <int LPR> struct PassCount { static constexpr int value = 2; };
+template <> struct PassCount<8> { static constexpr int value = 4; };
+template <> struct PassCount<16> { static constexpr int value = 4; };
+template <> struct PassCount<256> { static constexpr int value = 4; };
+
+// Matrix elements are read exactly once per launch, so they are loaded with the
+// non-temporal hint: the lines do not displace the gathered X vectors, the state
+// vectors and the work lists in L2 / Infinity Cache.  Measured on MI355X with the
+// encoders and decoders of 256 ensembles alternating (536 MB working set): 5.0 ->
+// 5.8 TB/s.  A wave load instruction must then consume whole 128-byte lines of a
+// row by itself (>= 8 lanes x 16 bytes per row), because a line is not kept for a
+// later iteration; the host planner picks the lanes-per-row class accordingly.
+#ifndef NHIP_TEMPORAL_LOADS
+typedef float nhip_f4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 nhip_load_a4(const float* p) {
+    const nhip_f4 v = __builtin_nontemporal_load(reinterpret_cast<const nhip_f4*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+#else
+__device__ __forceinline__ float4 nhip_load_a4(const float* p) {
+    return *reinterpret_cast<const float4*>(p);
+}
+#endif
 
 template <int LPR>
 __device__ __forceinline__ float row_reduce(float v) {
@@ -45,14 +66,13 @@ __device__ __forceinline__ float row_reduce(float v) {
     return v;
 }
 
-template <int LPR, int VEC>
+template <int LPR, int VEC, int P>
 __global__ __launch_bounds__(NHIP_WG) void gemv_wg_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks,
     const float* __restrict__ A, const float* __restrict__ X, const float* Yin, float* Y)
 {
     constexpr bool WIDE = (LPR == 256);
-    constexpr int P = PassCount<LPR>::value;
     constexpr int RPP = WIDE ? 1 : NHIP_WAVE / (WIDE ? 64 : LPR);  // rows per wave pass
 
     __shared__ __attribute__((aligned(16))) float xs[XCHUNK];
@@ -102,7 +122,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wg_kernel(
                     float4 a[P];
 #pragma unroll
                     for (int p = 0; p < P; ++p)
-                        a[p] = *reinterpret_cast<const float4*>(arow[p] + c);
+                        a[p] = nhip_load_a4(arow[p] + c);
 #pragma unroll
                     for (int p = 0; p < P; ++p) {
                         acc[p] = fmaf(a[p].x, x.x, acc[p]);
@@ -203,8 +223,8 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
 
 // Wave-per-task kernel in the summation order of the reference's block GEMV
 // (clra_gemv.py:1040-1058 and :1148-1153): per row and per 128-column tile, lane
-// j of four sums columns j, j+4, ... left to right (product and sum rounded
-// separately), the four partial sums combine as (s0+s2)+(s1+s3), and tile sums
+// j of four sums columns j, j+4, ... left to right (fused multiply-add, as an
+// OpenCL compiler contracts the reference's `+=`), the four partial sums combine as (s0+s2)+(s1+s3), and tile sums
 // are added one after the other onto beta*y_in; gamma comes last.  Used for the
 // small items of networks with thousands of tiny ensembles, where the order costs
 // nothing and makes the result bit-identical to a float32 restatement of the
@@ -238,7 +258,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_ref_kernel(
             for (int c0 = 0; c0 < dot.N; c0 += TILE) {
                 const int c1 = min(c0 + TILE, dot.N);
                 float s = 0.0f;
-                for (int c = c0 + lir; c < c1; c += 4) s = s + arow[c] * xg[(size_t)c * xs];
+                for (int c = c0 + lir; c < c1; c += 4) s = fmaf(arow[c], xg[(size_t)c * xs], s);
                 s = s + __shfl_xor(s, 2, NHIP_WAVE);
                 s = s + __shfl_xor(s, 1, NHIP_WAVE);
                 sum = sum + cf.x * s;
@@ -248,17 +268,29 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_ref_kernel(
     }
 }
 
-template <int LPR, int VEC>
-int launch_wg(hipStream_t s, const int* items, const float* coefs, const int* dots,
-              const int* tasks, int n_tasks, const float* A, const float* X, const float* Yin,
-              float* Y) {
-    hipLaunchKernelGGL((gemv_wg_kernel<LPR, VEC>), dim3(n_tasks), dim3(NHIP_WG), 0, s,
+template <int LPR, int VEC, int P>
+int launch_wg_p(hipStream_t s, const int* items, const float* coefs, const int* dots,
+                const int* tasks, int n_tasks, const float* A, const float* X, const float* Yin,
+                float* Y) {
+    hipLaunchKernelGGL((gemv_wg_kernel<LPR, VEC, P>), dim3(n_tasks), dim3(NHIP_WG), 0, s,
                        reinterpret_cast<const GemvItem*>(items),
                        reinterpret_cast<const float4*>(coefs),
                        reinterpret_cast<const GemvDot*>(dots),
                        reinterpret_cast<const GemvTask*>(tasks), A, X, Yin, Y);
     NHIP_LAUNCH_CHECK();
     return 0;
+}
+
+template <int LPR, int VEC>
+int launch_wg(hipStream_t s, int passes, const int* items, const float* coefs, const int* dots,
+              const int* tasks, int n_tasks, const float* A, const float* X, const float* Yin,
+              float* Y) {
+    switch (passes ? passes : PassCount<LPR>::value) {
+        case 2: return launch_wg_p<LPR, VEC, 2>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y);
+        case 4: return launch_wg_p<LPR, VEC, 4>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y);
+        case 8: return launch_wg_p<LPR, VEC, 8>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y);
+    }
+    return NHIP_E_BADCLASS;
 }
 
 template <int LPR, int VEC>
@@ -277,33 +309,44 @@ int launch_wave(hipStream_t s, const int* items, const float* coefs, const int* 
 
 }  // namespace
 
-extern "C" int nhip_gemv_rows_per_task(int flavor, int lpr, int vec) {
+static int default_passes(int lpr) {
+    switch (lpr) {
+        case 1: return PassCount<1>::value;
+        case 2: return PassCount<2>::value;
+        case 4: return PassCount<4>::value;
+        case 8: return PassCount<8>::value;
+        case 16: return PassCount<16>::value;
+        case 32: return PassCount<32>::value;
+        case 64: return PassCount<64>::value;
+        case 256: return PassCount<256>::value;
+    }
+    return 0;
+}
+
+extern "C" int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes) {
     if (vec != 1 && vec != 4) return 0;
     if (flavor == 2) return (lpr == 4 && vec == 1) ? 0x7fffffff : 0;
     if (flavor == 1) {
         switch (lpr) { case 1: case 2: case 4: case 8: case 16: case 32: case 64: return 0x7fffffff; }
         return 0;
     }
-    if (flavor != 0) return 0;
-    switch (lpr) {
-        case 1: return 4 * PassCount<1>::value * 64;
-        case 2: return 4 * PassCount<2>::value * 32;
-        case 4: return 4 * PassCount<4>::value * 16;
-        case 8: return 4 * PassCount<8>::value * 8;
-        case 16: return 4 * PassCount<16>::value * 4;
-        case 32: return 4 * PassCount<32>::value * 2;
-        case 64: return 4 * PassCount<64>::value;
-        case 256: return PassCount<256>::value;
-    }
-    return 0;
+    if (flavor != 0 || default_passes(lpr) == 0) return 0;
+    if (passes == 0) passes = default_passes(lpr);
+    if (passes != 2 && passes != 4 && passes != 8) return 0;
+    return lpr == 256 ? passes : (NHIP_WG / NHIP_WAVE) * passes * (NHIP_WAVE / lpr);
 }
 
-#define NHIP_GEMV_CASE(FN, L)                                                            \
-    case L:                                                                              \
-        return vec == 4 ? FN<L, 4>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y)  \
-                        : FN<L, 1>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y);
+#define NHIP_WG_CASE(L)                                                                         \
+    case L:                                                                                     \
+        return vec == 4                                                                         \
+                   ? launch_wg<L, 4>(s, passes, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y) \
+                   : launch_wg<L, 1>(s, passes, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y);
+#define NHIP_WAVE_CASE(L)                                                                   \
+    case L:                                                                                 \
+        return vec == 4 ? launch_wave<L, 4>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y) \
+                        : launch_wave<L, 1>(s, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y);
 
-extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, const int* items,
+extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes, const int* items,
                          const float* coefs, const int* dots, const int* tasks, int n_tasks,
                          const float* A, const float* X, const float* Yin, float* Y) {
     if (n_tasks == 0) return 0;
@@ -314,14 +357,14 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, const int* 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (flavor == 0) {
         switch (lpr) {
-            NHIP_GEMV_CASE(launch_wg, 1)
-            NHIP_GEMV_CASE(launch_wg, 2)
-            NHIP_GEMV_CASE(launch_wg, 4)
-            NHIP_GEMV_CASE(launch_wg, 8)
-            NHIP_GEMV_CASE(launch_wg, 16)
-            NHIP_GEMV_CASE(launch_wg, 32)
-            NHIP_GEMV_CASE(launch_wg, 64)
-            NHIP_GEMV_CASE(launch_wg, 256)
+            NHIP_WG_CASE(1)
+            NHIP_WG_CASE(2)
+            NHIP_WG_CASE(4)
+            NHIP_WG_CASE(8)
+            NHIP_WG_CASE(16)
+            NHIP_WG_CASE(32)
+            NHIP_WG_CASE(64)
+            NHIP_WG_CASE(256)
         }
     } else if (flavor == 2) {
         if (lpr != 4 || vec != 1) return NHIP_E_BADCLASS;
@@ -335,13 +378,13 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, const int* 
         return 0;
     } else if (flavor == 1) {
         switch (lpr) {
-            NHIP_GEMV_CASE(launch_wave, 1)
-            NHIP_GEMV_CASE(launch_wave, 2)
-            NHIP_GEMV_CASE(launch_wave, 4)
-            NHIP_GEMV_CASE(launch_wave, 8)
-            NHIP_GEMV_CASE(launch_wave, 16)
-            NHIP_GEMV_CASE(launch_wave, 32)
-            NHIP_GEMV_CASE(launch_wave, 64)
+            NHIP_WAVE_CASE(1)
+            NHIP_WAVE_CASE(2)
+            NHIP_WAVE_CASE(4)
+            NHIP_WAVE_CASE(8)
+            NHIP_WAVE_CASE(16)
+            NHIP_WAVE_CASE(32)
+            NHIP_WAVE_CASE(64)
         }
     }
     return NHIP_E_BADCLASS;

@@ -1,0 +1,352 @@
+// Ragged gather-GEMV in the summation order of the reference, at streaming speed.
+//
+// The reference's block GEMV (clra_gemv.py:1010-1060, :1122-1155) fixes the
+// float32 result of every output: per row and per 128-column tile, four partial
+// sums (columns j, j+4, ... for j = 0..3) each accumulated left to right (one fused
+// multiply-add per element), combined as (s0+s2)+(s1+s3), scaled by alpha; tile
+// sums are then added in order (dot products in list order, tiles left to right)
+// onto beta*y_in, and gamma is added last.  Spiking networks amplify one-ulp
+// differences in a neuron's input into different spike counts, so the large
+// matrices are summed in exactly that order here, which makes the result
+// bit-identical to a float32 restatement of the reference kernel.
+//
+// How that order is had without giving up coalesced HBM streaming:
+//   * a wave owns n_rows rows of one output item (four independent waves per
+//     group, no group barrier anywhere); it walks the dot products and, per dot
+//     product, column stages of up to 512 columns;
+//   * a block (about 8 KiB of the matrix: 4 rows x 512 columns, or 32 rows x 64
+//     columns, ...) is read with 16-byte non-temporal loads, consecutive lanes on
+//     consecutive addresses of a row, into registers; two stages are in flight per
+//     wave (two register sets) while an earlier one is summed;
+//   * the stage is written to a wave-private LDS block in which every 128-column
+//     tile is padded by 4 words, so that lane (row, tile, j) can walk "its" partial
+//     sum -- elements j, j+4, ... of the tile, in order, times the matching elements
+//     of the gathered X vector, which is staged in LDS once per column stage and
+//     reused by all row blocks of the task -- without bank conflicts (consecutive
+//     lanes: consecutive j, then tiles, rows);
+//   * the four j-lanes of a tile combine with two wave shuffles; one lane per row
+//     adds the tile sums of the stage in order.
+// The arithmetic is tiny next to the memory traffic (2 flops per 4 bytes), so the
+// serial order inside a lane costs nothing; parallelism comes from the
+// rows x tiles x 4 partial sums of a stage and from the many independent waves.
+#include "nhip_common.h"
+#include "gemv_types.h"
+
+namespace {
+
+constexpr int TILE = 128;          // columns per tile of the reference kernel
+constexpr int TILE_LDS = TILE + 4; // words per tile in LDS (bank rotation)
+constexpr int STAGE_COLS = 512;    // columns per column stage
+constexpr int MAX_PF = 9;          // 16-byte loads per lane and block (one register set)
+constexpr int TSUM_WORDS = 64;     // tile sums of one block (rows x tiles <= 64)
+constexpr int MAX_CHAIN = TILE / 4;  // elements of one partial sum: 32
+constexpr int X_PF = STAGE_COLS / NHIP_WAVE;  // gathered X elements per lane and column stage
+constexpr int XBLK_WORDS = (STAGE_COLS / TILE) * TILE_LDS;  // X block of a wave in LDS
+constexpr int ROW_SLOTS = 4;       // row sums per lane: a task covers <= 256 rows
+
+typedef float tile_f4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ tile_f4 load_nt4(const float* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const tile_f4*>(p));
+}
+
+// a / b for small non-negative a and positive b (both < 2^20), without the long
+// integer-division sequence
+__device__ __forceinline__ int small_div(int a, int b) {
+    int q = (int)((float)a * __frcp_rn((float)b));
+    if ((q + 1) * b <= a) ++q;
+    if (q * b > a) --q;
+    return q;
+}
+
+// words one matrix row occupies in LDS for a dot product with n columns
+__host__ __device__ __forceinline__ int row_words(int n) {
+    const int cols = n < STAGE_COLS ? n : STAGE_COLS;
+    return n >= TILE ? ((cols + TILE - 1) / TILE) * TILE_LDS : ((n + 3) & ~3) + 4;
+}
+
+// Rows of one block (what a wave stages through LDS at a time) for a dot product
+// with n columns: bounded by the LDS block, by one register set, and by one partial
+// sum per lane (two when a row is a single tile).
+__host__ __device__ __forceinline__ int block_rows(int n, int blk_words) {
+    const int cols = n < STAGE_COLS ? n : STAGE_COLS;
+    const int tiles = (cols + TILE - 1) / TILE;
+    int rows = blk_words / row_words(n);
+    const int by_regs = (MAX_PF * NHIP_WAVE) / ((cols + 3) / 4);
+    if (rows > by_regs) rows = by_regs;
+    const int by_lanes = tiles == 1 ? 2 * (NHIP_WAVE / 4) : (NHIP_WAVE / 4) / tiles;
+    if (rows > by_lanes) rows = by_lanes;
+    return rows;
+}
+
+// word offset of column c (relative to the stage) inside a row of the LDS block
+__device__ __forceinline__ int col_word(int c, bool tiled) {
+    return tiled ? (c >> 7) * TILE_LDS + (c & (TILE - 1)) : c;
+}
+
+// LDS written by some lanes of the wave is read by others: order it at wave scope
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+struct Stage {
+    int d;    // index of the dot product inside the item, -1 = none
+    int c0;   // first column of the column stage
+    int b;    // row block inside the task
+    int rb;   // rows per block for this dot product
+    GemvDot dot;
+};
+
+template <int VEC>
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3))) void gemv_tile_kernel(
+    const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
+    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
+    float* Y)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    float* ab = lds + wave * (blk_words + TSUM_WORDS + XBLK_WORDS);  // this wave's block
+    float* tsum = ab + blk_words;                                    // [row of the block][tile]
+    float* xb = tsum + TSUM_WORDS;  // gathered X of the current column stage, tiles padded
+
+    const int t = nhip_xcd_remap(blockIdx.x, gridDim.x) * (NHIP_WG / NHIP_WAVE) + wave;
+    if (t >= n_tasks) return;  // wave-uniform; the kernel has no group barrier
+
+    const GemvTask task = tasks[t];
+    const GemvItem it = items[task.item];
+    const float4 cf = coefs[task.item];
+    const int n_rows = task.n_rows;
+
+    // lane l carries the running sums of rows l, l + 64, ... of the task
+    float sum[ROW_SLOTS];
+#pragma unroll
+    for (int k = 0; k < ROW_SLOTS; ++k) {
+        const int r = lane + k * NHIP_WAVE;
+        sum[k] = r < n_rows ? cf.y * Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0]
+                            : 0.0f;
+    }
+
+    // ---- the blocks of a task in order: dot product, column stage, row block
+    auto first_stage = [&]() {
+        Stage s;
+        s.d = it.n_dots > 0 ? 0 : -1;
+        s.c0 = 0;
+        s.b = 0;
+        s.rb = 1;
+        if (s.d >= 0) {
+            s.dot = dots[it.dot_begin];
+            s.rb = block_rows(s.dot.N, blk_words);
+        }
+        return s;
+    };
+    auto next_stage = [&](const Stage& s) {
+        Stage n = s;
+        if (s.d < 0) return n;
+        n.b = s.b + 1;
+        if (n.b * s.rb >= n_rows) {
+            n.b = 0;
+            n.c0 = s.c0 + STAGE_COLS;
+            if (n.c0 >= s.dot.N) {
+                n.c0 = 0;
+                n.d = s.d + 1;
+                if (n.d < it.n_dots) {
+                    n.dot = dots[it.dot_begin + n.d];
+                    n.rb = block_rows(n.dot.N, blk_words);
+                } else {
+                    n.d = -1;
+                }
+            }
+        }
+        return n;
+    };
+
+    // global -> registers (non-temporal 16-byte loads, whole lines per instruction)
+    auto load_stage = [&](tile_f4 (&pf)[MAX_PF], float (&xq)[X_PF], const Stage& s) {
+        const int ncs = min(STAGE_COLS, s.dot.N - s.c0);
+        const int f4_per_row = (ncs + 3) >> 2;
+        const int rows = min(s.rb, n_rows - s.b * s.rb);
+        const int n_f4 = rows * f4_per_row;
+        const float* base = A + s.dot.a_start
+                            + (size_t)(task.row0 + s.b * s.rb) * s.dot.a_stride0 + s.c0;
+        const int step_r = small_div(NHIP_WAVE, f4_per_row);
+        const int step_q = NHIP_WAVE - step_r * f4_per_row;
+        int r = small_div(lane, f4_per_row), q = lane - r * f4_per_row;
+#pragma unroll
+        for (int i = 0; i < MAX_PF; ++i) {
+            tile_f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (lane + i * NHIP_WAVE < n_f4) {
+                const float* p = base + r * s.dot.a_stride0 + 4 * q;
+                if (VEC == 4 && 4 * q + 3 < ncs) {
+                    v = load_nt4(p);
+                } else {  // unaligned rows, or the last columns of a row
+                    if (4 * q + 0 < ncs) v.x = p[0];
+                    if (4 * q + 1 < ncs) v.y = p[1];
+                    if (4 * q + 2 < ncs) v.z = p[2];
+                    if (4 * q + 3 < ncs) v.w = p[3];
+                }
+            }
+            pf[i] = v;
+            r += step_r;
+            q += step_q;
+            if (q >= f4_per_row) { q -= f4_per_row; ++r; }
+        }
+        if (s.b == 0) {  // first row block of a column stage: its gathered X travels along
+            const float* xg = X + s.dot.x_start + (size_t)s.c0 * s.dot.x_stride0;
+#pragma unroll
+            for (int i = 0; i < X_PF; ++i) {
+                const int k = lane + i * NHIP_WAVE;
+                xq[i] = k < ncs ? xg[(size_t)k * s.dot.x_stride0] : 0.0f;
+            }
+        }
+    };
+
+    // registers -> this wave's LDS block (and X block, at the start of a column stage)
+    auto store_stage = [&](const tile_f4 (&pf)[MAX_PF], const float (&xq)[X_PF], const Stage& s) {
+        const int ncs = min(STAGE_COLS, s.dot.N - s.c0);
+        const bool tiled = s.dot.N >= TILE;
+        const int roww = row_words(s.dot.N);
+        const int f4_per_row = (ncs + 3) >> 2;
+        const int rows = min(s.rb, n_rows - s.b * s.rb);
+        const int n_f4 = rows * f4_per_row;
+        const int step_r = small_div(NHIP_WAVE, f4_per_row);
+        const int step_q = NHIP_WAVE - step_r * f4_per_row;
+        int r = small_div(lane, f4_per_row), q = lane - r * f4_per_row;
+        wave_sync();  // every lane is done reading the previous block
+#pragma unroll
+        for (int i = 0; i < MAX_PF; ++i) {
+            if (lane + i * NHIP_WAVE < n_f4)
+                *reinterpret_cast<tile_f4*>(ab + r * roww + col_word(4 * q, tiled)) = pf[i];
+            r += step_r;
+            q += step_q;
+            if (q >= f4_per_row) { q -= f4_per_row; ++r; }
+        }
+        if (s.b == 0) {
+#pragma unroll
+            for (int i = 0; i < X_PF; ++i) {
+                const int k = lane + i * NHIP_WAVE;
+                if (k < ncs) xb[col_word(k, tiled)] = xq[i];
+            }
+        }
+        wave_sync();
+    };
+
+    // partial sums of the block in LDS, then the row sums
+    auto sum_stage = [&](const Stage& s) {
+        const int ncs = min(STAGE_COLS, s.dot.N - s.c0);
+        const bool tiled = s.dot.N >= TILE;
+        const int roww = row_words(s.dot.N);
+        const int tiles_s = (ncs + TILE - 1) / TILE;
+        const int rows = min(s.rb, n_rows - s.b * s.rb);
+        const int n_chains = rows * tiles_s * 4;
+        const int j = lane & 3;
+        const int tl = (lane >> 2) % tiles_s;
+        const int w = min(TILE, ncs - tl * TILE);
+        const int count = max(0, (w - j + 3) >> 2);
+        const int cmax = (min(TILE, ncs) + 3) >> 2;  // longest partial sum of the block (uniform)
+        const bool all_full = (ncs & (TILE - 1)) == 0;  // every tile has 128 columns
+        for (int ch0 = 0; ch0 < n_chains; ch0 += NHIP_WAVE) {
+            const bool live = ch0 + lane < n_chains;
+            const int rt = live ? ((ch0 + lane) >> 2) : 0;
+            const int r = small_div(rt, tiles_s);
+            const float* ap = ab + r * roww + (tiled ? tl * TILE_LDS : 0) + j;
+            const float* xp = xb + (tiled ? tl * TILE_LDS : 0) + j;
+            float acc = 0.0f;
+            if (all_full) {
+#pragma unroll
+                for (int m = 0; m < MAX_CHAIN; ++m) acc = fmaf(ap[4 * m], xp[4 * m], acc);
+            } else {
+#pragma unroll
+                for (int m = 0; m < MAX_CHAIN; ++m)
+                    if (m < cmax) {  // uniform
+                        if (m < count) acc = fmaf(ap[4 * m], xp[4 * m], acc);
+                    }
+            }
+            acc = acc + __shfl_xor(acc, 2, NHIP_WAVE);
+            acc = acc + __shfl_xor(acc, 1, NHIP_WAVE);
+            if (live && j == 0) tsum[rt] = acc;
+        }
+        wave_sync();
+        // tile sums of the block, in order, onto the sums of its rows
+        const int r_first = s.b * s.rb;  // first row of the block inside the task
+#pragma unroll
+        for (int k = 0; k < ROW_SLOTS; ++k) {
+            const int rl = lane + k * NHIP_WAVE - r_first;  // row of this slot inside the block
+            if (rl >= 0 && rl < rows) {
+                const float* ts = tsum + rl * tiles_s;
+                for (int q = 0; q < tiles_s; ++q) sum[k] = sum[k] + cf.x * ts[q];
+            }
+        }
+    };
+
+    tile_f4 pf0[MAX_PF], pf1[MAX_PF];
+    float xq0[X_PF], xq1[X_PF];
+    Stage sa = first_stage();
+    Stage sb = next_stage(sa);
+    if (sa.d >= 0) load_stage(pf0, xq0, sa);
+    if (sb.d >= 0) load_stage(pf1, xq1, sb);
+    while (sa.d >= 0) {
+        store_stage(pf0, xq0, sa);
+        const Stage sc = next_stage(sb);
+        if (sc.d >= 0) load_stage(pf0, xq0, sc);
+        sum_stage(sa);
+        if (sb.d < 0) break;
+        store_stage(pf1, xq1, sb);
+        const Stage sd = next_stage(sc);
+        if (sd.d >= 0) load_stage(pf1, xq1, sd);
+        sum_stage(sb);
+        sa = sc;
+        sb = sd;
+    }
+
+#pragma unroll
+    for (int k = 0; k < ROW_SLOTS; ++k) {
+        const int r = lane + k * NHIP_WAVE;
+        if (r < n_rows) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = sum[k] + cf.z;
+    }
+}
+
+}  // namespace
+
+// Rows of one block for a dot product with n columns (the host sizes tasks as a
+// multiple of this; any task size up to 256 rows is legal).
+extern "C" int nhip_gemv_tile_rows(int n_cols, int blk_words) {
+    if (n_cols <= 0 || blk_words <= 0) return 0;
+    return block_rows(n_cols, blk_words);
+}
+
+extern "C" int nhip_gemv_tile(void* stream, int vec, int blk_words, const int* items,
+                              const float* coefs, const int* dots, const int* tasks, int n_tasks,
+                              const float* A, const float* X, const float* Yin, float* Y) {
+    if (n_tasks == 0) return 0;
+    if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
+        return NHIP_E_BADARG;
+    if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
+    if (blk_words < (STAGE_COLS / TILE) * TILE_LDS || (blk_words & 3)) return NHIP_E_BADARG;
+    if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
+    const int waves = NHIP_WG / NHIP_WAVE;
+    const size_t lds_bytes = sizeof(float) * waves * ((size_t)blk_words + TSUM_WORDS + XBLK_WORDS);
+    if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
+    const int n_groups = (n_tasks + waves - 1) / waves;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vec == 4) {
+        hipLaunchKernelGGL(gemv_tile_kernel<4>, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+                           reinterpret_cast<const GemvItem*>(items),
+                           reinterpret_cast<const float4*>(coefs),
+                           reinterpret_cast<const GemvDot*>(dots),
+                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, blk_words, A, X, Yin,
+                           Y);
+    } else {
+        hipLaunchKernelGGL(gemv_tile_kernel<1>, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+                           reinterpret_cast<const GemvItem*>(items),
+                           reinterpret_cast<const float4*>(coefs),
+                           reinterpret_cast<const GemvDot*>(dots),
+                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, blk_words, A, X, Yin,
+                           Y);
+    }
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}

@@ -1,0 +1,7 @@
+// Work-list records of the ragged GEMV (rows of the int32 tables described in
+// include/nengo_hip.h), shared by the GEMV kernels.
+#pragma once
+
+struct GemvItem { int y_start, y_stride0, yin_start, yin_stride0, dot_begin, n_dots, M, pad; };
+struct GemvDot { int a_start, a_stride0, N, x_start, x_stride0, p0, p1, p2; };
+struct GemvTask { int item, row0, n_rows, pad; };

@@ -16,6 +16,7 @@ signature, same ``.plans`` attribute; what differs is the work decomposition:
 For each item b:  ``Y[b] = beta[b]*Y_in[b] + gamma[b] + alpha[b] * sum_j A[A_js[b][j]] @ X[X_js[b][j]]``.
 """
 
+import os
 from collections import defaultdict
 
 import numpy as np
@@ -29,6 +30,10 @@ from .utils import next_pow2
 SMALL_ITEM_ELEMS = 8192
 # ... and among those, rows up to this length use the reference-order wave kernel
 REF_ORDER_MAX_COLS = 512
+# float32 words of one wave's LDS block in the reference-order kernel for large items
+TILE_STAGE_WORDS = int(os.environ.get("NENGO_HIP_TILE_WORDS", 2176))
+# the reference-order kernel wants at least this many (wave) tasks per launch
+MIN_TILE_TASKS = 4096
 WG, WAVE = 256, 64
 
 
@@ -65,10 +70,19 @@ def _per_item_floats(arg, n, what):
     return vec
 
 
+def _balanced_rows(M, cap):
+    """Rows per task so that the tasks of an item are equally full (M = 4096, cap = 128
+    stays 128; M = 100, cap = 64 becomes 50 instead of 64 + 36)."""
+    n_tasks = -(-M // cap)
+    return -(-M // n_tasks)
+
+
 class gemv_prog:
     """Geometry + work lists of one ragged GEMV; subclasses pick the kernel classes."""
 
-    force_flavor = None  # None = by item size; 0 = work-group kernel; 1 = wave kernel
+    # None = reference summation order (kernels "wave_ref" and "tile"); 0 = work-group
+    # kernel and 1 = wave kernel with their own, faster-to-reduce order
+    force_flavor = None
     force_scalar = False  # one lane per output, 4-byte loads (the plain fallback)
 
     def __init__(self, queue, alpha, A, A_js, X, X_js, beta, Y, Y_in=None, gamma=0.0, tag=None):
@@ -171,12 +185,26 @@ class gemv_prog:
             vec = 1
         flavor = self.force_flavor
         if flavor is None:
-            flavor = 1 if M * n_sum <= SMALL_ITEM_ELEMS else 0
-            if flavor == 1 and n_max <= REF_ORDER_MAX_COLS:
-                return (2, 4, 1)  # small item: the reference's summation order, bit for bit
-        lpr = min(WAVE, next_pow2(-(-n_max // vec)))
-        if flavor == 0 and (n_max >= 2048 or (n_max >= 512 and M < 16)):
-            lpr = WG  # the whole group works on one row
+            # default: the reference's summation order, bit for bit -- small items one
+            # wave per task, large items staged through LDS by a work-group
+            if M * n_sum <= SMALL_ITEM_ELEMS and n_max <= REF_ORDER_MAX_COLS:
+                return (2, 4, 1)
+            return (3, 0, vec)
+        if flavor == 0:
+            # Matrix loads are non-temporal, so one wave instruction should take whole
+            # 128-byte lines of a row: at least 8 lanes x 16 bytes per row, each lane then
+            # walking further column quads of its row.  Measured on MI355X, encoders and
+            # decoders of 256 ensembles alternating: 4096 x 64 -> 8 lanes per row, 5.75 TB/s;
+            # 64 x 4096 -> the whole group per row, 5.85 TB/s.
+            if vec == 4:
+                lpr = min(WAVE, max(8, next_pow2(n_max // 16))) if n_max >= 32 else next_pow2(
+                    -(-n_max // 4))
+            else:
+                lpr = min(WAVE, next_pow2(-(-n_max // 4)))
+            if n_max >= 2048 and M <= 256:
+                lpr = WG  # few, long rows: the whole group works on one row
+        else:
+            lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         return (flavor, lpr, vec)
 
     def _build(self, items):
@@ -207,37 +235,59 @@ class gemv_prog:
         dev_dots = to_device(self.queue, dot_tab)
 
         plans = []
-        for (flavor, lpr, vec), members in sorted(by_class.items()):
-            if flavor == 0:
-                rows = lib.nhip_gemv_rows_per_task(flavor, lpr, vec)
+        for cls, members in sorted(by_class.items()):
+            flavor, lpr, vec = cls[:3]
+            passes = cls[3] if len(cls) > 3 else 0  # 0 = the class default
+            if flavor == 3:
+                rows = None  # per item, below
+            elif flavor == 0:
+                rows = lib.nhip_gemv_rows_per_task(flavor, lpr, vec, passes)
             elif flavor == 2:
                 rows = WAVE // lpr  # one pass: these items are latency bound, spread them
             else:
                 rows = (WAVE // lpr) * 4  # four passes of a wave
-            if rows <= 0:
-                raise _lib.HipError("unknown GEMV class %r" % ((flavor, lpr, vec),))
+            if rows is not None and rows <= 0:
+                raise _lib.HipError("unknown GEMV class %r" % (cls,))
             task_rows = []
+            if flavor == 3:
+                # rows one wave stages through LDS at a time, per item (smallest over its dots)
+                blk = {b: min([lib.nhip_gemv_tile_rows(dd["a_shape1"], TILE_STAGE_WORDS)
+                               for dd in geometry[b]["dots"]] or [WAVE]) for b in members}
+                n_blocks = sum(-(-geometry[b]["y_len"] // blk[b]) for b in members)
+                # several row blocks per task reuse the gathered X registers, as long as
+                # enough tasks remain to fill the device
+                per_task = next((k for k in (4, 2) if n_blocks // k >= MIN_TILE_TASKS), 1)
             for b in members:
                 M = geometry[b]["y_len"]
-                for r0 in range(0, M, rows):
-                    task_rows.append((b, r0, min(rows, M - r0), 0))
+                item_rows = rows
+                if flavor == 3:
+                    assert blk[b] > 0
+                    item_rows = min(blk[b] * per_task, 256)
+                    item_rows = blk[b] * max(1, _balanced_rows(M, item_rows) // blk[b]) \
+                        if M > item_rows else item_rows
+                for r0 in range(0, M, item_rows):
+                    task_rows.append((b, r0, min(item_rows, M - r0), 0))
             task_tab = np.array(task_rows, dtype=np.int32)
             dev_tasks = to_device(self.queue, task_tab)
             n_tasks = len(task_rows)
             n_groups = n_tasks if flavor == 0 else -(-n_tasks // (WG // WAVE))
-            args = (flavor, lpr, vec, dev_items.ptr, dev_coefs.ptr, dev_dots.ptr, dev_tasks.ptr,
-                    n_tasks, self.A.ptr, self.X.ptr, self.Y_in.ptr, self.Y.ptr)
+            tail = (dev_items.ptr, dev_coefs.ptr, dev_dots.ptr, dev_tasks.ptr, n_tasks, self.A.ptr,
+                    self.X.ptr, self.Y_in.ptr, self.Y.ptr)
+            if flavor == 3:
+                kern, args = lib.nhip_gemv_tile, (vec, TILE_STAGE_WORDS) + tail
+            else:
+                kern, args = lib.nhip_gemv, (flavor, lpr, vec, passes) + tail
             plan = Plan(
-                self.queue, lib.nhip_gemv, args, gsize=(WG * n_groups,), lsize=(WG,),
+                self.queue, kern, args, gsize=(WG * n_groups,), lsize=(WG,),
                 full_args=(dev_items, dev_coefs, dev_dots, dev_tasks, self.A.dev_buf,
                            self.X.dev_buf, self.Y_in.dev_buf, self.Y.dev_buf),
-                name="hipra_gemv.%s" % ("wg", "wave", "wave_ref")[flavor],
+                name="hipra_gemv.%s" % ("wg", "wave", "wave_ref", "tile")[flavor],
                 tag="%s-lpr%d-v%d" % (self.tag, lpr, vec),
                 bw_per_call=bw_from_geometry(geometry, members),
                 flops_per_call=flops_from_geometry(geometry, members),
             )
             plan.description = self.geometry_summary(members)
-            plan.kernel_class = (flavor, lpr, vec)
+            plan.kernel_class = cls
             plan.n_tasks = n_tasks
             plans.append(plan)
         return plans

@@ -47,7 +47,12 @@ void orc_set_num_threads(int n) {
  * Block GEMV: clra_gemv.py `block_impl` :861-1175.
  *   kernel `fn`     :1010-1060  per (32-row x 128-col) tile, four partial sums
  *                               per row (lane j takes columns j, j+4, ...),
- *                               combined as (s0+s2)+(s1+s3), times alpha
+ *                               combined as (s0+s2)+(s1+s3), times alpha.
+ *                               The accumulation `sums[i][j] += A[..] * x[..]` is one
+ *                               expression; OpenCL C lets the compiler contract it and
+ *                               LLVM-based implementations do on devices with FMA, so
+ *                               it is a fused multiply-add here (the one place in this
+ *                               file where contraction is applied, explicitly).
  *   kernel `reduce` :1122-1155  y = beta*yin + sum over tiles (dots in A_js
  *                               order, column tiles left to right) + gamma
  * dot_ptr[b] .. dot_ptr[b+1] index the per-dot arrays of output item b.
@@ -73,10 +78,8 @@ void orc_gemv_block(int n_items, const int *y_starts, const int *y_stride0s, con
                 for (int c0 = 0; c0 < N; c0 += BLOCK_X) {
                     const int w = (N - c0 < BLOCK_X) ? N - c0 : BLOCK_X;
                     float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-                    for (int jj = 0; jj < w; ++jj) {
-                        const float prod = arow[c0 + jj] * x[(size_t)(c0 + jj) * xs];
-                        s[jj & 3] = s[jj & 3] + prod;
-                    }
+                    for (int jj = 0; jj < w; ++jj)
+                        s[jj & 3] = fmaf(arow[c0 + jj], x[(size_t)(c0 + jj) * xs], s[jj & 3]);
                     s[0] = s[0] + s[2];
                     s[1] = s[1] + s[3];
                     const float tile = (float)(alphas[b] * (double)(s[0] + s[1]));

@@ -41,9 +41,10 @@ def test_binding_covers_header_and_versions_match():
     lib = _lib.lib()
     assert lib.nhip_abi_version() == nengo_ocl_amd.ABI_VERSION
     assert b"bad argument" in lib.nhip_error_string(-1)
-    assert lib.nhip_gemv_rows_per_task(0, 16, 4) == 128
-    assert lib.nhip_gemv_rows_per_task(0, 256, 4) == 4
-    assert lib.nhip_gemv_rows_per_task(0, 3, 4) == 0
+    assert lib.nhip_gemv_rows_per_task(0, 16, 4, 0) == 64
+    assert lib.nhip_gemv_rows_per_task(0, 4, 4, 0) == 128
+    assert lib.nhip_gemv_rows_per_task(0, 256, 4, 8) == 8
+    assert lib.nhip_gemv_rows_per_task(0, 3, 4, 0) == 0
 
 
 def test_product_does_not_import_the_oracle():

@@ -66,8 +66,9 @@ def test_gemv_gamma_yin_and_strides():
 
 
 def test_gemv_block_order_is_the_reference_order():
-    """The four strided partial sums per 128-column tile, (s0+s2)+(s1+s3), tiles in
-    order (clra_gemv.py:1043-1058, :1148-1153), replayed step by step in numpy float32."""
+    """The four strided partial sums per 128-column tile (fused multiply-add per
+    element), (s0+s2)+(s1+s3), tiles in order (clra_gemv.py:1043-1058, :1148-1153),
+    replayed step by step in numpy."""
     rng = np.random.RandomState(5)
     n = 300  # three tiles: 128, 128, 44
     a = rng.normal(size=(1, n)).astype(np.float32)
@@ -78,8 +79,9 @@ def test_gemv_block_order_is_the_reference_order():
     total = y0
     for c0 in range(0, n, 128):
         s = np.zeros(4, dtype=np.float32)
-        for jj in range(min(128, n - c0)):
-            s[jj % 4] = np.float32(s[jj % 4] + np.float32(a[0, c0 + jj] * x[c0 + jj]))
+        for jj in range(min(128, n - c0)):  # fused multiply-add: exact product, one rounding
+            s[jj % 4] = np.float32(np.longdouble(a[0, c0 + jj]) * np.longdouble(x[c0 + jj])
+                                   + np.longdouble(s[jj % 4]))
         total = np.float32(total + np.float32(np.float32(s[0] + s[2]) + np.float32(s[1] + s[3])))
     assert Y[0][0, 0] == total
 
