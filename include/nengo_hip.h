@@ -56,8 +56,12 @@ int nhip_device_info(int *n_cu, int *wave_size, int *lds_bytes, char *name, int 
  *   items : int32[n_items][8]  {y_start, y_stride0, yin_start, yin_stride0,
  *                               dot_begin, n_dots, M, 0}
  *   coefs : float[n_items][4]  {alpha, beta, gamma, 0}
- *   dots  : int32[n_dots][8]   {a_start, a_stride0, N, x_start, x_stride0,0,0,0}
- *                               (A rows are contiguous: a_stride1 == 1)
+ *   dots  : int32[n_dots][8]   {a_start, a_stride0, N, x_start, x_stride0,
+ *                               tile_rows, log2_N, 0}
+ *                               (A rows are contiguous: a_stride1 == 1; the last
+ *                               two are read by nhip_gemv_tile only: tile_rows =
+ *                               nhip_gemv_tile_rows(N, blk_words), log2_N = the
+ *                               exponent when N is a power of two, else -1)
  *   tasks : int32[n_tasks][4]  {item, row0, n_rows, 0}
  *
  * `flavor` 0 = one work-group (256 threads) per task, X staged in LDS and
@@ -80,17 +84,20 @@ int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
 
 /* The same operation and the same four tables, summed in the ORDER of the
  * reference's block kernel (clra_gemv.py:1043-1058, :1148-1153: four strided
- * partial sums per 128-column tile, (s0+s2)+(s1+s3), tiles added in order, products
- * rounded separately), for large items: a wave owns the rows of one task (four tasks
- * per 256-thread group) and streams the matrix through a wave-private LDS block of
- * `blk_words` float32 (a multiple of 4, >= 1056; 2176 = 8.5 KiB by default), so the
- * result is bit-identical to a float32 restatement of that kernel while HBM is
- * still read in whole lines.  A task may cover at most
- * nhip_gemv_tile_rows(N, blk_words) rows for every dot product (N columns) of its
- * item.  `vec` as for nhip_gemv. */
-int nhip_gemv_tile(void *stream, int vec, int blk_words, const int *items, const float *coefs,
-                   const int *dots, const int *tasks, int n_tasks, const float *A,
-                   const float *X, const float *Yin, float *Y);
+ * partial sums per 128-column tile, one fused multiply-add per element,
+ * (s0+s2)+(s1+s3), tiles added in order), for large items: a wave owns the rows
+ * of one task (four tasks per 256-thread group, at most 256 rows per task) and
+ * streams the matrix through a wave-private LDS block of `blk_words` float32 (a
+ * multiple of 4, >= 528; 2176 = 8.5 KiB by default), so the result is
+ * bit-identical to a float32 restatement of that kernel while HBM is still read in
+ * whole lines.  nhip_gemv_tile_rows(N, blk_words) = rows of a dot product with N
+ * columns that fit one LDS block (a power of two; goes into the dots table).
+ * `vec` as for nhip_gemv.  `pow2_cols` = 1 selects the streamlined kernel for
+ * launches in which every dot product has a power-of-two column count >= 4
+ * (log2_N set), vec == 4 and a_stride0 < 2^22; 0 = any shape. */
+int nhip_gemv_tile(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
+                   const float *coefs, const int *dots, const int *tasks, int n_tasks,
+                   const float *A, const float *X, const float *Yin, float *Y);
 int nhip_gemv_tile_rows(int n_cols, int blk_words);
 
 /* ---- neurons -----------------------------------------------------------

@@ -67,7 +67,7 @@ __host__ __device__ __forceinline__ int row_words(int n) {
 
 // Rows of one block (what a wave stages through LDS at a time) for a dot product
 // with n columns: bounded by the LDS block, by one register set, and by one partial
-// sum per lane (two when a row is a single tile).
+// sum per lane (two when a row is a single tile); rounded down to a power of two.
 __host__ __device__ __forceinline__ int block_rows(int n, int blk_words) {
     const int cols = n < STAGE_COLS ? n : STAGE_COLS;
     const int tiles = (cols + TILE - 1) / TILE;
@@ -76,6 +76,7 @@ __host__ __device__ __forceinline__ int block_rows(int n, int blk_words) {
     if (rows > by_regs) rows = by_regs;
     const int by_lanes = tiles == 1 ? 2 * (NHIP_WAVE / 4) : (NHIP_WAVE / 4) / tiles;
     if (rows > by_lanes) rows = by_lanes;
+    while (rows & (rows - 1)) rows &= rows - 1;  // a power of two: blocks never straddle 64 rows
     return rows;
 }
 
@@ -100,7 +101,7 @@ struct Stage {
 };
 
 template <int VEC>
-__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3))) void gemv_tile_kernel(
+__global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
@@ -108,7 +109,9 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3))) vo
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
-    const int wave = threadIdx.x >> 6;
+    // readfirstlane: the compiler then keeps everything derived from the wave's task in
+    // scalar registers and on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     float* ab = lds + wave * (blk_words + TSUM_WORDS + XBLK_WORDS);  // this wave's block
     float* tsum = ab + blk_words;                                    // [row of the block][tile]
     float* xb = tsum + TSUM_WORDS;  // gathered X of the current column stage, tiles padded
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3))) vo
         s.rb = 1;
         if (s.d >= 0) {
             s.dot = dots[it.dot_begin];
-            s.rb = block_rows(s.dot.N, blk_words);
+            s.rb = s.dot.p0;
         }
         return s;
     };
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3))) vo
                 n.d = s.d + 1;
                 if (n.d < it.n_dots) {
                     n.dot = dots[it.dot_begin + n.d];
-                    n.rb = block_rows(n.dot.N, blk_words);
+                    n.rb = n.dot.p0;
                 } else {
                     n.d = -1;
                 }
@@ -309,6 +312,229 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3))) vo
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same algorithm for dot products whose column counts are powers of two
+// (>= 4) with 16-byte aligned rows: every lane-to-element mapping is a shift or a
+// mask of wave-uniform values, stages and tiles are always full, and a block is at
+// most 8 loads per lane.  This is the streaming path of the big encoder / decoder
+// matrices; its instruction count per byte is a fraction of the general kernel's.
+constexpr int P2_PF = 8;         // 16-byte loads per lane and block
+constexpr int YSUM_WORDS = 256;  // running sums of the task's rows, in LDS
+
+__device__ __forceinline__ float quad_xor(float v, int ctrl_sel) {
+    // lanes exchange inside groups of four: xor 2 = [2,3,0,1], xor 1 = [1,0,3,2]
+    const int r = ctrl_sel == 2
+        ? __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true)
+        : __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true);
+    return __int_as_float(r);
+}
+
+struct P2Stage {
+    int d;    // index of the dot product inside the item, -1 = none
+    int c0;   // first column of the column stage
+    int b;    // row block inside the task
+    GemvDot dot;  // p0 = rows per block, p1 = log2(columns)
+};
+
+__global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
+    const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
+    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
+    float* Y)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    // readfirstlane: the compiler then keeps everything derived from the wave's task in
+    // scalar registers and on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float* ab = lds + wave * (blk_words + TSUM_WORDS + XBLK_WORDS + YSUM_WORDS);
+    float* tsum = ab + blk_words;
+    float* xb = tsum + TSUM_WORDS;
+    float* ys = xb + XBLK_WORDS;  // running sum of row r of the task
+
+    const int t = nhip_xcd_remap(blockIdx.x, gridDim.x) * (NHIP_WG / NHIP_WAVE) + wave;
+    if (t >= n_tasks) return;  // wave-uniform; the kernel has no group barrier
+
+    const GemvTask task = tasks[t];
+    const GemvItem it = items[task.item];
+    const float4 cf = coefs[task.item];
+    const int n_rows = task.n_rows;
+
+#pragma unroll
+    for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
+        const int r = lane + k * NHIP_WAVE;
+        if (r < n_rows)
+            ys[r] = cf.y * Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0];
+    }
+
+    auto first_stage = [&]() {
+        P2Stage s;
+        s.d = it.n_dots > 0 ? 0 : -1;
+        s.c0 = 0;
+        s.b = 0;
+        if (s.d >= 0) s.dot = dots[it.dot_begin];
+        return s;
+    };
+    auto next_stage = [&](const P2Stage& s) {
+        P2Stage n = s;
+        if (s.d < 0) return n;
+        n.b = s.b + 1;
+        if (n.b * s.dot.p0 >= n_rows) {
+            n.b = 0;
+            n.c0 = s.c0 + STAGE_COLS;
+            if (n.c0 >= s.dot.N) {
+                n.c0 = 0;
+                n.d = s.d + 1;
+                if (n.d < it.n_dots) n.dot = dots[it.dot_begin + n.d];
+                else n.d = -1;
+            }
+        }
+        return n;
+    };
+
+    // Wave-uniform shape of a stage.  lgq: log2 of the lanes side by side in a row
+    // (each on one 16-byte quad); a row of the stage takes 1 << lg_lpr load
+    // instructions, one instruction covers rpl rows.
+#define P2_GEOMETRY(s)                                                              \
+    const int lgn = (s).dot.p1;                                                     \
+    const int lgc = lgn < 9 ? lgn : 9;               /* log2 columns of the stage */ \
+    const int lgq = lgc - 2 < 6 ? lgc - 2 : 6;                                      \
+    const int lg_lpr = lgc - 2 - lgq;                                               \
+    const int rpl = NHIP_WAVE >> lgq;                                               \
+    const int lgt = lgc > 7 ? lgc - 7 : 0;           /* log2 tiles of the stage */  \
+    const int roww = lgn >= 7 ? (TILE_LDS << lgt) : (1 << lgn) + 4;                 \
+    const int rb = (s).dot.p0;                                                      \
+    const int rows = min(rb, n_rows - (s).b * rb);                                  \
+    const int lane_r = lane >> lgq;                                                 \
+    const int lane_q = lane & ((1 << lgq) - 1);
+
+    auto load_stage = [&](tile_f4 (&pf)[P2_PF], float (&xq)[X_PF], const P2Stage& s) {
+        P2_GEOMETRY(s)
+        (void)lgt; (void)roww;
+        const char* base = reinterpret_cast<const char*>(
+            A + s.dot.a_start + (size_t)(task.row0 + s.b * rb) * s.dot.a_stride0 + s.c0);
+        const unsigned lane_off = 4u * (unsigned)(lane_r * s.dot.a_stride0 + 4 * lane_q);
+        const size_t load_pitch = (size_t)rpl * s.dot.a_stride0 * 4u;  // bytes between loads
+#pragma unroll
+        for (int i = 0; i < P2_PF; ++i) {
+            const int ri = (i >> lg_lpr) * rpl;                  // uniform
+            const int part = i & ((1 << lg_lpr) - 1);            // uniform: which 256 columns
+            if (ri < rows) {                                     // uniform
+                if (ri + lane_r < rows)
+                    pf[i] = load_nt4(reinterpret_cast<const float*>(
+                        base + ((size_t)(i >> lg_lpr) * load_pitch + (size_t)part * 1024u) + lane_off));
+            }
+        }
+        if (s.b == 0) {  // first row block of a column stage: its gathered X travels along
+            const int ncs = 1 << lgc;
+            const float* xg = X + s.dot.x_start + (size_t)s.c0 * s.dot.x_stride0;
+            const int lane_x = lane * s.dot.x_stride0;
+#pragma unroll
+            for (int i = 0; i < X_PF; ++i)
+                if (i * NHIP_WAVE < ncs) {                       // uniform
+                    if (lane + i * NHIP_WAVE < ncs)
+                        xq[i] = xg[(size_t)i * NHIP_WAVE * s.dot.x_stride0 + lane_x];
+                }
+        }
+    };
+
+    auto store_stage = [&](const tile_f4 (&pf)[P2_PF], const float (&xq)[X_PF], const P2Stage& s) {
+        P2_GEOMETRY(s)
+        (void)lgt;
+        // word of this lane's quad inside the block: tiles are padded by 4 words
+        const int lane_l = lane_r * roww + (lane_q >> 5) * TILE_LDS + ((lane_q & 31) << 2);
+        wave_sync();  // every lane is done reading the previous block
+#pragma unroll
+        for (int i = 0; i < P2_PF; ++i) {
+            const int ri = (i >> lg_lpr) * rpl;
+            const int part = i & ((1 << lg_lpr) - 1);
+            if (ri < rows) {
+                if (ri + lane_r < rows)
+                    *reinterpret_cast<tile_f4*>(ab + lane_l + ri * roww + part * (2 * TILE_LDS)) = pf[i];
+            }
+        }
+        if (s.b == 0) {
+            const int ncs = 1 << lgc;
+#pragma unroll
+            for (int i = 0; i < X_PF; ++i)
+                if (i * NHIP_WAVE < ncs) {
+                    if (lane + i * NHIP_WAVE < ncs)
+                        xb[lane + (i >> 1) * TILE_LDS + (i & 1) * NHIP_WAVE] = xq[i];
+                }
+        }
+        wave_sync();
+    };
+
+    auto sum_stage = [&](const P2Stage& s) {
+        P2_GEOMETRY(s)
+        (void)lane_r; (void)lane_q; (void)lg_lpr; (void)rpl;
+        const int cmax = lgn >= 7 ? MAX_CHAIN : (1 << lgn) >> 2;  // elements per partial sum
+        const int n_rt = rows << lgt;                             // (row, tile) pairs of the block
+        const int j = lane & 3;
+        const int rt = lane >> 2;
+        const int tl = rt & ((1 << lgt) - 1);
+        const float* ap = ab + (rt >> lgt) * roww + tl * TILE_LDS + j;
+        const float* xp = xb + tl * TILE_LDS + j;
+        const int pass_words = (16 >> lgt) * roww;
+        for (int rt0 = 0; rt0 < n_rt; rt0 += 16, ap += pass_words) {
+            float acc = 0.0f;
+            if (cmax == MAX_CHAIN) {
+#pragma unroll
+                for (int m = 0; m < MAX_CHAIN; ++m) acc = fmaf(ap[4 * m], xp[4 * m], acc);
+            } else if (cmax == MAX_CHAIN / 2) {
+#pragma unroll
+                for (int m = 0; m < MAX_CHAIN / 2; ++m) acc = fmaf(ap[4 * m], xp[4 * m], acc);
+            } else {
+                for (int m = 0; m < cmax; ++m) acc = fmaf(ap[4 * m], xp[4 * m], acc);
+            }
+            acc = acc + quad_xor(acc, 2);
+            acc = acc + quad_xor(acc, 1);
+            if (j == 0 && rt0 + rt < n_rt) tsum[rt0 + rt] = acc;
+        }
+        wave_sync();
+        // tile sums of the block, in order, onto the running sums of its rows
+        if (lane < rows) {
+            const float* ts = tsum + (lane << lgt);
+            float* yp = ys + s.b * rb + lane;
+            float v = *yp;
+            for (int q = 0; q < (1 << lgt); ++q) v = v + cf.x * ts[q];
+            *yp = v;
+        }
+    };
+#undef P2_GEOMETRY
+
+    tile_f4 pf0[P2_PF], pf1[P2_PF];
+    float xq0[X_PF], xq1[X_PF];
+#pragma unroll
+    for (int i = 0; i < P2_PF; ++i) pf0[i] = pf1[i] = tile_f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < X_PF; ++i) xq0[i] = xq1[i] = 0.0f;
+    P2Stage sa = first_stage();
+    P2Stage sb = next_stage(sa);
+    if (sa.d >= 0) load_stage(pf0, xq0, sa);
+    if (sb.d >= 0) load_stage(pf1, xq1, sb);
+    while (sa.d >= 0) {
+        store_stage(pf0, xq0, sa);
+        const P2Stage sc = next_stage(sb);
+        if (sc.d >= 0) load_stage(pf0, xq0, sc);
+        sum_stage(sa);
+        if (sb.d < 0) break;
+        store_stage(pf1, xq1, sb);
+        const P2Stage sd = next_stage(sc);
+        if (sd.d >= 0) load_stage(pf1, xq1, sd);
+        sum_stage(sb);
+        sa = sc;
+        sb = sd;
+    }
+
+    wave_sync();
+#pragma unroll
+    for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
+        const int r = lane + k * NHIP_WAVE;
+        if (r < n_rows) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = ys[r] + cf.z;
+    }
+}
+
 }  // namespace
 
 // Rows of one block for a dot product with n columns (the host sizes tasks as a
@@ -318,35 +544,34 @@ extern "C" int nhip_gemv_tile_rows(int n_cols, int blk_words) {
     return block_rows(n_cols, blk_words);
 }
 
-extern "C" int nhip_gemv_tile(void* stream, int vec, int blk_words, const int* items,
-                              const float* coefs, const int* dots, const int* tasks, int n_tasks,
-                              const float* A, const float* X, const float* Yin, float* Y) {
+extern "C" int nhip_gemv_tile(void* stream, int vec, int pow2_cols, int blk_words,
+                              const int* items, const float* coefs, const int* dots,
+                              const int* tasks, int n_tasks, const float* A, const float* X,
+                              const float* Yin, float* Y) {
     if (n_tasks == 0) return 0;
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
+    if (pow2_cols != 0 && (pow2_cols != 1 || vec != 4)) return NHIP_E_BADCLASS;
     if (blk_words < (STAGE_COLS / TILE) * TILE_LDS || (blk_words & 3)) return NHIP_E_BADARG;
     if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
     const int waves = NHIP_WG / NHIP_WAVE;
-    const size_t lds_bytes = sizeof(float) * waves * ((size_t)blk_words + TSUM_WORDS + XBLK_WORDS);
+    const size_t wave_words = (size_t)blk_words + TSUM_WORDS + XBLK_WORDS + (pow2_cols ? YSUM_WORDS : 0);
+    const size_t lds_bytes = sizeof(float) * waves * wave_words;
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
     const int n_groups = (n_tasks + waves - 1) / waves;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (vec == 4) {
-        hipLaunchKernelGGL(gemv_tile_kernel<4>, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
                            reinterpret_cast<const GemvItem*>(items),
                            reinterpret_cast<const float4*>(coefs),
                            reinterpret_cast<const GemvDot*>(dots),
                            reinterpret_cast<const GemvTask*>(tasks), n_tasks, blk_words, A, X, Yin,
                            Y);
-    } else {
-        hipLaunchKernelGGL(gemv_tile_kernel<1>, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
-                           reinterpret_cast<const GemvItem*>(items),
-                           reinterpret_cast<const float4*>(coefs),
-                           reinterpret_cast<const GemvDot*>(dots),
-                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, blk_words, A, X, Yin,
-                           Y);
-    }
+    };
+    if (pow2_cols) launch(gemv_tile_p2_kernel);
+    else if (vec == 4) launch(gemv_tile_kernel<4>);
+    else launch(gemv_tile_kernel<1>);
     NHIP_LAUNCH_CHECK();
     return 0;
 }

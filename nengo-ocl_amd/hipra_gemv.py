@@ -33,7 +33,9 @@ REF_ORDER_MAX_COLS = 512
 # float32 words of one wave's LDS block in the reference-order kernel for large items
 TILE_STAGE_WORDS = int(os.environ.get("NENGO_HIP_TILE_WORDS", 2176))
 # the reference-order kernel wants at least this many (wave) tasks per launch
-MIN_TILE_TASKS = 4096
+MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
+TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
+    "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
 WG, WAVE = 256, 64
 
 
@@ -189,7 +191,10 @@ class gemv_prog:
             # wave per task, large items staged through LDS by a work-group
             if M * n_sum <= SMALL_ITEM_ELEMS and n_max <= REF_ORDER_MAX_COLS:
                 return (2, 4, 1)
-            return (3, 0, vec)
+            pow2 = vec == 4 and all(
+                d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0
+                and d["a_stride0"] < 2 ** 22 for d in dots)
+            return (3, int(pow2), vec)  # second entry: 1 = every column count a power of two
         if flavor == 0:
             # Matrix loads are non-temporal, so one wave instruction should take whole
             # 128-byte lines of a row: at least 8 lanes x 16 bytes per row, each lane then
@@ -207,6 +212,45 @@ class gemv_prog:
             lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         return (flavor, lpr, vec)
 
+    def _tile_tasks(self, members):
+        """Tasks (item, first row, rows, 0) of the reference-order kernel for large items.
+
+        A task is the rows one wave carries through all columns, a few row blocks of
+        what fits its LDS stage.  Larger tasks reuse the gathered X more often; but all
+        groups of a launch are resident at once (up to three per compute unit) and take
+        about as long as the launch itself, so the device is only busy to the end when
+        the groups spread evenly over the compute units.  Among the task sizes that
+        give enough tasks, the one with the least uneven spread wins.
+        """
+        lib, geometry = self.queue.lib, self.geometry
+        blk = {b: min([lib.nhip_gemv_tile_rows(dd["a_shape1"], TILE_STAGE_WORDS)
+                       for dd in geometry[b]["dots"]] or [WAVE]) for b in members}
+
+        def tasks_for(per_task):
+            out = []
+            for b in members:
+                M = geometry[b]["y_len"]
+                item_rows = max(1, min(int(blk[b] * per_task), 256))
+                if M > item_rows:
+                    item_rows = _balanced_rows(M, item_rows)
+                    if item_rows >= 2 * blk[b]:
+                        item_rows -= item_rows % blk[b]
+                for r0 in range(0, M, item_rows):
+                    out.append((b, r0, min(item_rows, M - r0), 0))
+            return out
+
+        n_cu = self.queue.n_compute_units
+        best = None
+        for per_task in TILE_TASK_BLOCKS:
+            tasks = tasks_for(per_task)
+            rounds = -(-len(tasks) // (WG // WAVE)) / float(n_cu)  # groups per compute unit
+            uneven = -(-rounds // 1) / rounds
+            enough = len(tasks) >= MIN_TILE_TASKS
+            key = (not enough, round(uneven, 2))
+            if best is None or key < best[0]:
+                best = (key, tasks)
+        return best[1]
+
     def _build(self, items):
         """Work lists for `items`; returns the list of plans (one per kernel class)."""
         lib = self.queue.lib
@@ -221,8 +265,10 @@ class gemv_prog:
                            len(dot_rows), len(g["dots"]), g["y_len"], 0)
             coef_tab[b] = (self.alpha[b], self.beta[b], self.gamma[b], 0.0)
             for d in g["dots"]:
-                dot_rows.append((d["a_start"], d["a_stride0"], d["a_shape1"], d["x_start"],
-                                 d["x_stride0"], 0, 0, 0))
+                n = d["a_shape1"]
+                log2_n = n.bit_length() - 1 if n > 0 and n & (n - 1) == 0 else -1
+                dot_rows.append((d["a_start"], d["a_stride0"], n, d["x_start"], d["x_stride0"],
+                                 lib.nhip_gemv_tile_rows(n, TILE_STAGE_WORDS), log2_n, 0))
         dot_tab = np.array(dot_rows or [(0,) * 8], dtype=np.int32)
 
         by_class = defaultdict(list)
@@ -248,25 +294,14 @@ class gemv_prog:
                 rows = (WAVE // lpr) * 4  # four passes of a wave
             if rows is not None and rows <= 0:
                 raise _lib.HipError("unknown GEMV class %r" % (cls,))
-            task_rows = []
             if flavor == 3:
-                # rows one wave stages through LDS at a time, per item (smallest over its dots)
-                blk = {b: min([lib.nhip_gemv_tile_rows(dd["a_shape1"], TILE_STAGE_WORDS)
-                               for dd in geometry[b]["dots"]] or [WAVE]) for b in members}
-                n_blocks = sum(-(-geometry[b]["y_len"] // blk[b]) for b in members)
-                # several row blocks per task reuse the gathered X registers, as long as
-                # enough tasks remain to fill the device
-                per_task = next((k for k in (4, 2) if n_blocks // k >= MIN_TILE_TASKS), 1)
-            for b in members:
-                M = geometry[b]["y_len"]
-                item_rows = rows
-                if flavor == 3:
-                    assert blk[b] > 0
-                    item_rows = min(blk[b] * per_task, 256)
-                    item_rows = blk[b] * max(1, _balanced_rows(M, item_rows) // blk[b]) \
-                        if M > item_rows else item_rows
-                for r0 in range(0, M, item_rows):
-                    task_rows.append((b, r0, min(item_rows, M - r0), 0))
+                task_rows = self._tile_tasks(members)
+            else:
+                task_rows = []
+                for b in members:
+                    M = geometry[b]["y_len"]
+                    for r0 in range(0, M, rows):
+                        task_rows.append((b, r0, min(rows, M - r0), 0))
             task_tab = np.array(task_rows, dtype=np.int32)
             dev_tasks = to_device(self.queue, task_tab)
             n_tasks = len(task_rows)
@@ -274,7 +309,7 @@ class gemv_prog:
             tail = (dev_items.ptr, dev_coefs.ptr, dev_dots.ptr, dev_tasks.ptr, n_tasks, self.A.ptr,
                     self.X.ptr, self.Y_in.ptr, self.Y.ptr)
             if flavor == 3:
-                kern, args = lib.nhip_gemv_tile, (vec, TILE_STAGE_WORDS) + tail
+                kern, args = lib.nhip_gemv_tile, (vec, lpr, TILE_STAGE_WORDS) + tail
             else:
                 kern, args = lib.nhip_gemv, (flavor, lpr, vec, passes) + tail
             plan = Plan(

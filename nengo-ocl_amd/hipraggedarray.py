@@ -43,6 +43,13 @@ class Queue:
         self.stream = torch.cuda.Stream(device=self.device)
         self.handle = ctypes.c_void_p(self.stream.cuda_stream)
         self.lib = _lib.lib()
+        n_cu, wave, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        name = ctypes.create_string_buffer(64)
+        with torch.cuda.device(self.device):
+            _lib.check(self.lib.nhip_device_info(ctypes.byref(n_cu), ctypes.byref(wave),
+                                                 ctypes.byref(lds), name, 64), "device info")
+        self.n_compute_units = max(1, n_cu.value)
+        self.arch = name.value.decode()
 
     def finish(self):
         _lib.check(self.lib.nhip_stream_sync(self.handle), "stream sync")

@@ -11,7 +11,10 @@ Differences from the reference, all deliberate:
 
 * ``align=True`` pads every item start to a multiple of ``align_elems``
   (default 16 floats = 64 B) so that rows of matrices whose row stride is a
-  multiple of 4 can be read with 16-byte vector loads on the GPU.  The
+  multiple of 4 can be read with 16-byte vector loads on the GPU; items of 1024
+  elements or more start on a multiple of 64 elements (256 B), and matrices of
+  65536 elements or more are skewed against each other inside 16 KiB windows (HBM
+  channel spreading, see ``SKEW_ITEM_ELEMS``).  The
   reference's policy (16 for size >= 16, 4 for size >= 8, raggedarray.py:46-55)
   is available as ``align="reference"``.
 * the five metadata vectors live in one ``(5, n)`` int32 table, exposed through
@@ -23,6 +26,21 @@ from io import StringIO
 import numpy as np
 
 from .utils import is_iterable, round_up
+
+# items this large start on a 256-byte boundary, so that a wave's 1 KiB load
+# instruction covers whole 128-byte memory lines of the matrix
+BIG_ITEM_ELEMS = 1024
+BIG_ITEM_ALIGN = 64
+# Matrices of this size or more are additionally skewed against each other: the
+# k-th one starts (9 k mod 64) * 256 bytes past a 16 KiB boundary.  Many waves
+# stream rows of many such matrices at the same column offset at the same time; when
+# all rows are congruent modulo the memory channel interleave (row strides of 4 KiB
+# multiples, bases 512 B or 4 KiB apart) the traffic piles up on a few HBM channels.
+# Measured on MI355X, 256 matrices of 64 x 4096: 78 us per pass with bases 1 MiB +
+# 4 KiB apart, 66 us at + 512 B, 51 us with this skew.
+SKEW_ITEM_ELEMS = 65536
+SKEW_WINDOW = 4096     # elements: 16 KiB
+SKEW_STEP = 9 * 64     # elements: 2304 bytes
 
 _FIELDS = ("starts", "shape0s", "shape1s", "stride0s", "stride1s")
 
@@ -58,13 +76,17 @@ class RaggedArray:
         sizes = [a.size for a in arrays]
         starts = []
         cursor = 0
+        n_skewed = 0
         for size in sizes:
             if align == "reference":
                 unit = 16 if size >= 16 else 4 if size >= 8 else 1
             elif align:
-                unit = align_elems if size >= 4 else 1
+                unit = BIG_ITEM_ALIGN if size >= BIG_ITEM_ELEMS else align_elems if size >= 4 else 1
             else:
                 unit = 1
+            if align is True and size >= SKEW_ITEM_ELEMS:
+                cursor = round_up(cursor, SKEW_WINDOW) + (n_skewed * SKEW_STEP) % SKEW_WINDOW
+                n_skewed += 1
             cursor = round_up(cursor, unit)
             starts.append(cursor)
             cursor += size

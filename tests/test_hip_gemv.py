@@ -148,7 +148,7 @@ def test_ensemble_shapes(queue, pi):
     prog = run_case(queue, planners()[pi], 1.0, 1.0, 0.0, A, X, Y, js, js)
     if pi == 0:
         classes = {p.kernel_class for p in prog.plans}
-        assert classes == {(3, 0, 4), (2, 4, 1)}
+        assert classes == {(3, 1, 4), (3, 0, 4), (2, 4, 1)}  # power-of-two widths, any width, small
 
 
 def test_strided_views_and_yin(queue):
@@ -307,3 +307,53 @@ def test_large_items_bit_exact(queue, beta):
         got = dY.to_host()
         for i in range(len(Y)):
             assert np.array_equal(got[i], Yo[i]), (i, use_yin)
+
+
+@pytest.mark.parametrize("beta", [1.0, 0.5])
+def test_pow2_items_bit_exact(queue, beta):
+    """Power-of-two column counts take the streamlined staged kernel: every width from
+    4 to 8192, row counts that leave partial row blocks and partial tasks, outputs that
+    sum dot products of different power-of-two widths, and matrix views with a row
+    stride larger than the width -- bit-identical to the oracle."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(777)
+    shapes = [(5001, 4), (3003, 8), (1111, 16), (999, 32), (4096, 64), (777, 64), (301, 128),
+              (130, 256), (67, 512), (33, 1024), (64, 4096), (9, 8192), (1, 16384), (257, 2048)]
+    multi = (64, 128, 1024, 4, 512)
+    mats = [rng.normal(size=s) for s in shapes] + [rng.normal(size=(300, n)) for n in multi]
+    A = RA(mats, align=True)
+    X = RA([rng.normal(size=m.shape[1]) for m in mats], align=True)
+    Y = RA([rng.normal(size=s[0]) for s in shapes] + [rng.normal(size=300)], align=True)
+    n = len(shapes)
+    js = [np.array([i], dtype=np.int32) for i in range(n)] + [np.arange(n, n + len(multi), dtype=np.int32)]
+    Yo = clone(Y)
+    orc.plan_block_gemv(None, 1.0, A, js, X, js, beta, Yo).plans[0]()
+    dY = to_dev(queue, Y)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY)
+    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4)}
+    for plan in prog.plans:
+        plan()
+    got = dY.to_host()
+    for i in range(len(Y)):
+        assert np.array_equal(got[i], Yo[i]), i
+
+    # column blocks of a wider matrix: row stride 640, widths 128 and 512
+    wide = rng.normal(size=(700, 640)).astype(np.float32)
+    Aw = RA([wide], align=True)
+    Av = Aw[[0]]  # shares the buffer
+    Av.add_views([Aw.starts[0], Aw.starts[0] + 128], [700, 700], [128, 512], [640, 640], [1, 1])
+    Xw = RA([rng.normal(size=128), rng.normal(size=512)], align=True)
+    Yw = RA([rng.normal(size=700)], align=True)
+    jA, jX = [np.array([1, 2], dtype=np.int32)], [np.array([0, 1], dtype=np.int32)]
+    Yo = clone(Yw)
+    orc.plan_block_gemv(None, 1.0, Av, jA, Xw, jX, beta, Yo).plans[0]()
+    dY = to_dev(queue, Yw)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, Av), jA, to_dev(queue, Xw), jX, beta, dY)
+    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4)}
+    for plan in prog.plans:
+        plan()
+    assert np.array_equal(dY.to_host()[0], Yo[0])
+    expect = beta * Yw[0][:, 0] + wide[:, :128] @ Xw[0][:, 0] + wide[:, 128:] @ Xw[1][:, 0]
+    assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
