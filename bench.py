@@ -128,6 +128,9 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
     ap.add_argument("--no-fuse", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--branches", action="store_true",
+                    help="record kernels that touch different memory as side-by-side graph "
+                         "branches instead of one chain")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run the plain copy kernel on 256 MiB (1 GiB of traffic per 2 "
                          "launches) 20 times: the known-size reference for HBM counters")
@@ -144,7 +147,8 @@ def main():
 
     t0 = time.time()
     (net, probes, _), workload = make_network(args.config, args.variant, args.scale)
-    sim = Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph)
+    sim = Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph,
+                    branches=args.branches)
     build_s = time.time() - t0
     n_plans = len(sim._plans)
 
@@ -184,7 +188,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": workload, "neurons": net.n_neurons, "plans_per_step": n_plans,
-                   "dt": 0.001, "graph": not args.no_graph, "fused_copies": not args.no_fuse},
+                   "dt": 0.001, "graph": not args.no_graph, "graph_branches": args.branches,
+                   "fused_copies": not args.no_fuse},
         "roofline": roofline,
         "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,
                      "gbs": 1e-3 * gemv_bytes / gemv_us if gemv_us else None,

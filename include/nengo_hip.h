@@ -99,6 +99,21 @@ int nhip_gemv_tile(void *stream, int vec, int pow2_cols, int blk_words, const in
                    const float *coefs, const int *dots, const int *tasks, int n_tasks,
                    const float *A, const float *X, const float *Yin, float *Y);
 int nhip_gemv_tile_rows(int n_cols, int blk_words);
+/* nhip_gemv_tile followed by nhip_lif on its outputs, in one launch: replaces
+ * `plan_block_gemv` (clra_gemv.py:1193-1195) + `plan_lif`
+ * (clra_nonlinearities.py:1028-1146) when the GEMV output is the neurons' input
+ * current.  Row r of item b is the current of neuron r of population b:
+ *   pops : int32[n_items][8] {v_start, w_start, s_start, enabled, tau, ref, amp, pflags}
+ * (tau / ref / amp: float bits, or with bit 0/1/2 of pflags set the element offset
+ * of a per-neuron vector in TAU / REF / AMP; items with enabled == 0 only get Y).
+ * Y is still written.  V, W, S must not overlap anything the launch reads through
+ * A, X or Yin; dt, upsample as for nhip_lif.  Results are bit-identical to the two
+ * separate calls. */
+int nhip_gemv_tile_lif(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
+                       const float *coefs, const int *dots, const int *tasks, int n_tasks,
+                       const float *A, const float *X, const float *Yin, float *Y,
+                       const int *pops, double dt, int upsample, float *V, float *W, float *S,
+                       const float *TAU, const float *REF, const float *AMP);
 
 /* ---- neurons -----------------------------------------------------------
  * LIF with refractory state and spike-time interpolation.
@@ -184,6 +199,15 @@ int nhip_capture_end(void *stream, void **graph_exec_out);
 int nhip_graph_launch(void *graph_exec, void *stream, int n_times);
 int nhip_graph_destroy(void *graph_exec);
 int nhip_stream_sync(void *stream);
+/* Branches of a timestep that do not depend on each other (the reference runs its
+ * plans strictly in order on one in-order queue, plan.py:137-149) are recorded on
+ * side streams: a side stream joins the recording by waiting on an event recorded
+ * on a stream that is already being captured, and the capturing stream waits on
+ * an event of every side stream before nhip_capture_end.  The graph keeps only
+ * these dependencies; replays run independent kernels side by side. */
+int nhip_stream_create(void **stream_out); /* non-blocking, default priority */
+int nhip_stream_destroy(void *stream);
+int nhip_stream_wait_event(void *stream, void *event);
 
 /* events on `stream` (for per-plan and whole-run timing) */
 int nhip_event_create(void **event_out);

@@ -28,6 +28,8 @@ SIGNATURES = {
     "nhip_gemv": [P, c_int, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P],
     "nhip_gemv_rows_per_task": [c_int, c_int, c_int, c_int],
     "nhip_gemv_tile": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P],
+    "nhip_gemv_tile_lif": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
+                           P, ctypes.c_double, c_int, P, P, P, P, P, P],
     "nhip_gemv_tile_rows": [c_int, c_int],
     "nhip_lif": [P, P, c_int, c_double, c_int, P, P, P, P, P, P, P],
     "nhip_lif_rate": [P, P, c_int, P, P, P, P, P],
@@ -46,6 +48,9 @@ SIGNATURES = {
     "nhip_graph_launch": [P, P, c_int],
     "nhip_graph_destroy": [P],
     "nhip_stream_sync": [P],
+    "nhip_stream_create": [ctypes.POINTER(c_void_p)],
+    "nhip_stream_destroy": [P],
+    "nhip_stream_wait_event": [P, P],
     "nhip_event_create": [ctypes.POINTER(c_void_p)],
     "nhip_event_record": [P, P],
     "nhip_event_elapsed_ms": [P, P, ctypes.POINTER(c_float)],

@@ -31,6 +31,7 @@
 // rows x tiles x 4 partial sums of a stage and from the many independent waves.
 #include "nhip_common.h"
 #include "gemv_types.h"
+#include "neuron_math.h"
 
 namespace {
 
@@ -100,12 +101,12 @@ struct Stage {
     GemvDot dot;
 };
 
-template <int VEC>
+template <int VEC, bool LIF>
 __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
-    float* Y)
+    float* Y, LifArgs lif)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
@@ -305,10 +306,18 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
         sb = sd;
     }
 
+    // the finished rows; with LIF, row r of the item is also the input current of
+    // neuron r of the item's population, which is updated on the spot
+    LifPop pop = {};
+    if (LIF) pop = lif.pops[task.item];
 #pragma unroll
     for (int k = 0; k < ROW_SLOTS; ++k) {
         const int r = lane + k * NHIP_WAVE;
-        if (r < n_rows) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = sum[k] + cf.z;
+        if (r < n_rows) {
+            const float y = sum[k] + cf.z;
+            Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
+            if (LIF && pop.enabled) lif_epilogue(lif, pop, task.row0 + r, y);
+        }
     }
 }
 
@@ -336,11 +345,12 @@ struct P2Stage {
     GemvDot dot;  // p0 = rows per block, p1 = log2(columns)
 };
 
+template <bool LIF>
 __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
-    float* Y)
+    float* Y, LifArgs lif)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
@@ -528,10 +538,16 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     }
 
     wave_sync();
+    LifPop pop = {};
+    if (LIF) pop = lif.pops[task.item];
 #pragma unroll
     for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
         const int r = lane + k * NHIP_WAVE;
-        if (r < n_rows) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = ys[r] + cf.z;
+        if (r < n_rows) {
+            const float y = ys[r] + cf.z;
+            Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
+            if (LIF && pop.enabled) lif_epilogue(lif, pop, task.row0 + r, y);
+        }
     }
 }
 
@@ -544,10 +560,11 @@ extern "C" int nhip_gemv_tile_rows(int n_cols, int blk_words) {
     return block_rows(n_cols, blk_words);
 }
 
-extern "C" int nhip_gemv_tile(void* stream, int vec, int pow2_cols, int blk_words,
-                              const int* items, const float* coefs, const int* dots,
-                              const int* tasks, int n_tasks, const float* A, const float* X,
-                              const float* Yin, float* Y) {
+namespace {
+
+int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* items,
+                const float* coefs, const int* dots, const int* tasks, int n_tasks, const float* A,
+                const float* X, const float* Yin, float* Y, const LifArgs* lif) {
     if (n_tasks == 0) return 0;
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
@@ -561,17 +578,56 @@ extern "C" int nhip_gemv_tile(void* stream, int vec, int pow2_cols, int blk_word
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
     const int n_groups = (n_tasks + waves - 1) / waves;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const LifArgs args = lif ? *lif : LifArgs{};
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
                            reinterpret_cast<const GemvItem*>(items),
                            reinterpret_cast<const float4*>(coefs),
                            reinterpret_cast<const GemvDot*>(dots),
                            reinterpret_cast<const GemvTask*>(tasks), n_tasks, blk_words, A, X, Yin,
-                           Y);
+                           Y, args);
     };
-    if (pow2_cols) launch(gemv_tile_p2_kernel);
-    else if (vec == 4) launch(gemv_tile_kernel<4>);
-    else launch(gemv_tile_kernel<1>);
+    if (lif) {
+        if (pow2_cols) launch(gemv_tile_p2_kernel<true>);
+        else if (vec == 4) launch(gemv_tile_kernel<4, true>);
+        else launch(gemv_tile_kernel<1, true>);
+    } else {
+        if (pow2_cols) launch(gemv_tile_p2_kernel<false>);
+        else if (vec == 4) launch(gemv_tile_kernel<4, false>);
+        else launch(gemv_tile_kernel<1, false>);
+    }
     NHIP_LAUNCH_CHECK();
     return 0;
+}
+
+}  // namespace
+
+extern "C" int nhip_gemv_tile(void* stream, int vec, int pow2_cols, int blk_words,
+                              const int* items, const float* coefs, const int* dots,
+                              const int* tasks, int n_tasks, const float* A, const float* X,
+                              const float* Yin, float* Y) {
+    return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
+                       Yin, Y, nullptr);
+}
+
+extern "C" int nhip_gemv_tile_lif(void* stream, int vec, int pow2_cols, int blk_words,
+                                  const int* items, const float* coefs, const int* dots,
+                                  const int* tasks, int n_tasks, const float* A, const float* X,
+                                  const float* Yin, float* Y, const int* pops, double dt,
+                                  int upsample, float* V, float* W, float* S, const float* TAU,
+                                  const float* REF, const float* AMP) {
+    if (!pops || !V || !W || !S || upsample < 1 || !(dt > 0.0)) return NHIP_E_BADARG;
+    LifArgs lif;
+    lif.pops = reinterpret_cast<const LifPop*>(pops);
+    lif.dtu = (float)(dt / (double)upsample);  // formed in double and rounded once, as in nhip_lif
+    lif.dt_inv = (float)(1.0 / dt);
+    lif.upsample = upsample;
+    lif.V = V;
+    lif.W = W;
+    lif.S = S;
+    lif.TAU = TAU;
+    lif.REF = REF;
+    lif.AMP = AMP;
+    return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
+                       Yin, Y, &lif);
 }

@@ -1,0 +1,72 @@
+// Per-neuron update rules shared by the neuron kernels and by GEMV epilogues.
+#pragma once
+
+#include "nhip_common.h"
+
+// One population of LIF neurons driven by one output item of a GEMV: element
+// offsets of its state, and its parameters as float bits or (pflags bit set) as the
+// element offset of a per-neuron vector.
+struct LifPop {
+    int v_start, w_start, s_start, enabled;
+    int tau, ref, amp, pflags;  // bit 0/1/2 of pflags: tau/ref/amp is a per-neuron vector
+};
+
+// State arrays and constants of a fused LIF update (all populations of a launch).
+struct LifArgs {
+    const LifPop* pops;  // one per GEMV item
+    float dtu, dt_inv;   // dt / upsample, 1 / dt
+    int upsample;
+    float* V;
+    float* W;
+    float* S;
+    const float* TAU;
+    const float* REF;
+    const float* AMP;
+};
+
+__device__ __forceinline__ float lif_param(int word, bool is_vector, const float* data, int i) {
+    return is_vector ? data[(size_t)word + i] : nhip_bits(word);
+}
+
+// The update follows the reference kernel text (clra_nonlinearities.py:1086-1133)
+// operation by operation: refractory countdown, partial-step integration time,
+// exponential-Euler voltage step, threshold test with spike-time interpolation.
+// Sums that follow a product are written with explicit rounded operations so
+// that the compiler cannot fuse them differently from one build to the next.
+// expm1 and log1p are evaluated in double and rounded once to float: that is the
+// correctly rounded float32 value (the best any float implementation can return),
+// so every conforming host or device math library gives the same bits and spike
+// decisions do not depend on the library.  Returns whether the neuron spiked.
+__device__ __forceinline__ bool lif_step(float j, float& v, float& w, float tau, float ref,
+                                         float dtu, int upsample) {
+    bool spiked = false;
+    for (int u = 0; u < upsample; ++u) {
+        w -= dtu;
+        const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
+        const float dv = __fmul_rn(-(float)expm1((double)__fdiv_rn(-delta_t, tau)), j - v);
+        v = __fadd_rn(v, dv);
+        if (v > 1.0f) {
+            const float t_spike =
+                __fadd_rn(dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
+            w = ref + t_spike;
+            v = 0.0f;
+            spiked = true;
+        } else if (v < 0.0f) {
+            v = 0.0f;
+        }
+    }
+    return spiked;
+}
+
+// LIF update of neuron i of population p with input current j (GEMV epilogue)
+__device__ __forceinline__ void lif_epilogue(const LifArgs& a, const LifPop& p, int i, float j) {
+    float v = a.V[(size_t)p.v_start + i];
+    float w = a.W[(size_t)p.w_start + i];
+    const float tau = lif_param(p.tau, p.pflags & 1, a.TAU, i);
+    const float ref = lif_param(p.ref, p.pflags & 2, a.REF, i);
+    const float amp = lif_param(p.amp, p.pflags & 4, a.AMP, i);
+    const bool spiked = lif_step(j, v, w, tau, ref, a.dtu, a.upsample);
+    a.V[(size_t)p.v_start + i] = v;
+    a.W[(size_t)p.w_start + i] = w;
+    a.S[(size_t)p.s_start + i] = spiked ? __fmul_rn(amp, a.dt_inv) : 0.0f;
+}

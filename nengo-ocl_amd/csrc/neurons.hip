@@ -2,6 +2,7 @@
 // One thread per neuron, consecutive threads on consecutive neurons of a block
 // (a run of <= 1024 neurons of one population), float32 throughout.
 #include "nhip_common.h"
+#include "neuron_math.h"
 
 namespace {
 
@@ -11,19 +12,7 @@ struct LifDesc {
     int pflags, p0, p1, p2;    // bit 0/1/2: tau/ref/amp is a per-neuron vector
 };
 
-__device__ __forceinline__ float lif_param(int word, bool is_vector, const float* data, int i) {
-    return is_vector ? data[(size_t)word + i] : nhip_bits(word);
-}
-
-// The update follows the reference kernel text (clra_nonlinearities.py:1086-1133)
-// operation by operation: refractory countdown, partial-step integration time,
-// exponential-Euler voltage step, threshold test with spike-time interpolation.
-// Sums that follow a product are written with explicit rounded operations so
-// that the compiler cannot fuse them differently from one build to the next.
-// expm1 and log1p are evaluated in double and rounded once to float: that is the
-// correctly rounded float32 value (the best any float implementation can return),
-// so every conforming host or device math library gives the same bits and spike
-// decisions do not depend on the library.
+// One thread per neuron; the update itself is `lif_step` (neuron_math.h).
 __global__ __launch_bounds__(NHIP_WG) void lif_kernel(const LifDesc* __restrict__ desc, float dt,
                                                       float dt_inv, int upsample, const float* J,
                                                       float* V, float* W, float* S,
@@ -39,22 +28,7 @@ __global__ __launch_bounds__(NHIP_WG) void lif_kernel(const LifDesc* __restrict_
         const float tau = lif_param(d.tau, d.pflags & 1, TAU, i);
         const float ref = lif_param(d.ref, d.pflags & 2, REF, i);
         const float amp = lif_param(d.amp, d.pflags & 4, AMP, i);
-        bool spiked = false;
-        for (int u = 0; u < upsample; ++u) {
-            w -= dtu;
-            const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
-            const float dv = __fmul_rn(-(float)expm1((double)__fdiv_rn(-delta_t, tau)), j - v);
-            v = __fadd_rn(v, dv);
-            if (v > 1.0f) {
-                const float t_spike =
-                    __fadd_rn(dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
-                w = ref + t_spike;
-                v = 0.0f;
-                spiked = true;
-            } else if (v < 0.0f) {
-                v = 0.0f;
-            }
-        }
+        const bool spiked = lif_step(j, v, w, tau, ref, dtu, upsample);
         V[(size_t)d.v_start + i] = v;
         W[(size_t)d.w_start + i] = w;
         S[(size_t)d.s_start + i] = spiked ? __fmul_rn(amp, dt_inv) : 0.0f;

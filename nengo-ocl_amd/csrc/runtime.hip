@@ -77,6 +77,28 @@ extern "C" int nhip_stream_sync(void* stream) {
     return (int)hipStreamSynchronize(static_cast<hipStream_t>(stream));
 }
 
+// Side streams carry the branches of a timestep that do not depend on each other
+// while the step is recorded; the recorded graph keeps only the dependencies.
+extern "C" int nhip_stream_create(void** stream_out) {
+    if (!stream_out) return NHIP_E_BADARG;
+    hipStream_t s = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);  // default priority
+    if (e != hipSuccess) return (int)e;
+    *stream_out = s;
+    return 0;
+}
+
+extern "C" int nhip_stream_destroy(void* stream) {
+    if (!stream) return 0;
+    return (int)hipStreamDestroy(static_cast<hipStream_t>(stream));
+}
+
+extern "C" int nhip_stream_wait_event(void* stream, void* event) {
+    if (!stream || !event) return NHIP_E_BADARG;
+    return (int)hipStreamWaitEvent(static_cast<hipStream_t>(stream),
+                                   static_cast<hipEvent_t>(event), 0);
+}
+
 extern "C" int nhip_event_create(void** event_out) {
     if (!event_out) return NHIP_E_BADARG;
     hipEvent_t ev = nullptr;

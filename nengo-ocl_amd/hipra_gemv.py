@@ -87,8 +87,10 @@ class gemv_prog:
     force_flavor = None
     force_scalar = False  # one lane per output, 4-byte loads (the plain fallback)
 
-    def __init__(self, queue, alpha, A, A_js, X, X_js, beta, Y, Y_in=None, gamma=0.0, tag=None):
+    def __init__(self, queue, alpha, A, A_js, X, X_js, beta, Y, Y_in=None, gamma=0.0, tag=None,
+                 tile_items=()):
         self.queue = queue
+        self.tile_items = frozenset(tile_items)  # items that take the large-item kernel regardless
         self.A, self.A_js, self.X, self.X_js = A, A_js, X, X_js
         self.Y = Y
         self.Y_in = Y if Y_in is None else Y_in
@@ -151,6 +153,7 @@ class gemv_prog:
                 )
             geometry.append(
                 {
+                    "index": b,
                     "y_len": M,
                     "dots": dots,
                     "y_start": int(Y.starts[b]),
@@ -176,6 +179,8 @@ class gemv_prog:
     # ------------------------------------------------------- class selection
     def _item_class(self, g):
         """(flavor, lanes per row, vector width) for one item."""
+        if g["index"] in self.tile_items and not g["dots"]:
+            return (3, 1, 4)  # no dot products: only Y = beta Y_in + gamma and the epilogue
         dots = g["dots"]
         M = g["y_len"]
         n_max = max([d["a_shape1"] for d in dots] or [1])
@@ -324,6 +329,8 @@ class gemv_prog:
             plan.description = self.geometry_summary(members)
             plan.kernel_class = cls
             plan.n_tasks = n_tasks
+            plan.members = list(members)
+            plan.prog = self
             plans.append(plan)
         return plans
 
@@ -356,3 +363,153 @@ class plan_ref_gemv(gemv_prog):
     """One lane per output element, scalar loads: the plain fallback kernel."""
 
     force_scalar = True
+
+
+def _overlaps(a, b):
+    """Does any half-open interval of `a` overlap one of `b`?  (lists of (lo, hi))"""
+    if not a or not b:
+        return False
+    b = sorted(b)
+    los = np.array([lo for lo, _ in b])
+    his = np.maximum.accumulate(np.array([hi for _, hi in b]))
+    for lo, hi in a:
+        k = np.searchsorted(los, hi, side="left")  # intervals of b starting before hi
+        if k > 0 and his[k - 1] > lo:
+            return True
+    return False
+
+
+def _span(ra, i):
+    """Half-open element interval item i of a ragged array may touch."""
+    m, n = int(ra.shape0s[i]), int(ra.shape1s[i])
+    if m == 0 or n == 0:
+        return None
+    lo = int(ra.starts[i])
+    return lo, lo + (m - 1) * int(ra.stride0s[i]) + (n - 1) * int(ra.stride1s[i]) + 1
+
+
+def _concat(ras):
+    """Items of several views of one device buffer, as one ragged view."""
+    first = ras[0]
+    fields = [np.concatenate([getattr(ra, f) for ra in ras])
+              for f in ("starts", "shape0s", "shape1s", "stride0s", "stride1s")]
+    return HIPRaggedArray.from_buffer(first.queue, first.dev_buf, *fields)
+
+
+def _subset_param(param, idx):
+    """tau / ref / amp of `plan_lif` restricted to the populations `idx`."""
+    if isinstance(param, HIPRaggedArray):
+        return param[list(idx)]
+    if isinstance(param, np.ndarray) and param.ndim == 1:
+        return param[list(idx)]
+    return param
+
+
+def fuse_lif(prog, lif_plan):
+    """Fewer launches for "J = GEMV(...); LIF(J)" (clra_gemv.py `plan_block_gemv` followed
+    by clra_nonlinearities.py `plan_lif`): the reference-order kernel for large items
+    updates the neurons of a row block as soon as its currents are final, so the
+    currents are not read back and the neuron kernel is not launched.
+
+    A population is fused when its J is exactly the output of one large item of
+    `prog`.  Populations whose J no item of `prog` writes (neurons without input
+    connections) ride along as items without dot products.  Populations fed by small
+    items keep a neuron launch of their own.  Nothing is fused when a state the
+    update writes (voltage, refractory time, spikes) is read by a dot product of
+    `prog`.  Returns the plans that replace ``prog.plans + [lif_plan]`` (same results
+    bit for bit), or None.
+    """
+    from .hipra_nonlinearities import lif_population_table, plan_lif
+
+    spec = getattr(lif_plan, "lif_spec", None)
+    if spec is None or not prog.plans:
+        return None
+    queue, lib = prog.queue, prog.queue.lib
+    J, V, W, S = spec["J"], spec["V"], spec["W"], spec["outS"]
+    Y = prog.Y
+    if any(ra.ptr.value != Y.ptr.value for ra in (J, V, W, S)):
+        return None  # different device buffers: nothing to match offsets against
+    large = {}
+    for plan in prog.plans:
+        if plan.kernel_class[0] == 3:
+            for b in plan.members:
+                if int(Y.stride0s[b]) == 1:
+                    large[(int(Y.starts[b]), int(Y.shape0s[b]))] = b
+    y_spans = [iv for iv in (_span(Y, b) for b in range(len(Y))) if iv]
+    matched, idle, rest = [], [], []
+    for p in range(len(J)):
+        b = large.get((int(J.starts[p]), int(J.shape0s[p])))
+        if b is not None:
+            matched.append((p, b))
+        elif _span(J, p) and not _overlaps([_span(J, p)], y_spans):
+            idle.append(p)
+        else:
+            rest.append(p)
+    if not matched or len({b for _, b in matched}) != len(matched):
+        return None
+
+    # the update must not write what the launch still reads elsewhere
+    fused_pops = [p for p, _ in matched] + idle
+    written = [iv for ra in (V, W, S) for iv in (_span(ra, p) for p in fused_pops) if iv]
+    read = []
+    for g in prog.geometry:
+        for d in g["dots"]:
+            if prog.A.ptr.value == Y.ptr.value:
+                read.append(_span(prog.A, d["a_j"]))
+            if prog.X.ptr.value == Y.ptr.value:
+                read.append(_span(prog.X, d["x_j"]))
+    if prog.Y_in.ptr.value == Y.ptr.value:
+        for b in range(len(Y)):
+            if int(prog.Y_in.starts[b]) != int(Y.starts[b]):
+                read.append(_span(prog.Y_in, b))
+    written += y_spans  # and the currents themselves
+    if _overlaps(written, [iv for iv in read if iv]):
+        return None
+
+    if idle:
+        # the same GEMV with one more item per input-less population: Y = 1 * J + 0, no dots
+        n_old = len(Y)
+        extra = J[idle]
+        none = np.zeros(0, dtype=np.int32)
+        prog = type(prog)(
+            queue, np.concatenate([prog.alpha, np.ones(len(idle), np.float32)]),
+            prog.A, list(prog.A_js) + [none] * len(idle), prog.X, list(prog.X_js) + [none] * len(idle),
+            np.concatenate([prog.beta, np.ones(len(idle), np.float32)]),
+            _concat([Y, extra]), Y_in=_concat([prog.Y_in, extra]),
+            gamma=np.concatenate([prog.gamma, np.zeros(len(idle), np.float32)]), tag=prog.tag,
+            tile_items=range(n_old, n_old + len(idle)))
+        matched = matched + [(p, n_old + k) for k, p in enumerate(idle)]
+        Y = prog.Y
+
+    cols, pptrs, keep = lif_population_table(queue, spec)
+    table = np.zeros((len(Y), 8), dtype=np.int32)
+    for p, b in matched:
+        table[b] = (cols["v_start"][p], cols["w_start"][p], cols["s_start"][p], 1,
+                    cols["tau"][p], cols["ref"][p], cols["amp"][p], cols["pflags"][p])
+    dev_pops = to_device(queue, table)
+    lif_args = (dev_pops.ptr, spec["dt"], spec["upsample"], V.ptr, W.ptr, S.ptr,
+                pptrs[0], pptrs[1], pptrs[2])
+    pop_of = {b: p for p, b in matched}
+    out = []
+    for plan in prog.plans:
+        if plan.kernel_class[0] != 3 or not any(b in pop_of for b in plan.members):
+            out.append(plan)
+            continue
+        lif_bytes = sum(4 * int(J.shape0s[pop_of[b]]) for b in plan.members if b in pop_of)
+        fused = Plan(queue, lib.nhip_gemv_tile_lif, plan.args + lif_args, gsize=plan.gsize,
+                     lsize=plan.lsize,
+                     full_args=plan.full_args + (dev_pops, V.dev_buf, W.dev_buf, S.dev_buf) + tuple(keep),
+                     name="hipra_gemv.tile_lif", tag=plan.tag,
+                     bw_per_call=plan.bw_per_call + 5 * lif_bytes,  # V and W in and out, spikes out
+                     flops_per_call=plan.flops_per_call)
+        fused.description = plan.description
+        fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
+        fused.members, fused.prog = plan.members, prog
+        fused.gemv_bytes = plan.bw_per_call
+        out.append(fused)
+    if rest:
+        out.append(plan_lif(queue, spec["dt"], J[rest], V[rest], W[rest], S[rest],
+                            _subset_param(spec["ref"], rest), _subset_param(spec["tau"], rest),
+                            _subset_param(spec["amp"], rest), upsample=spec["upsample"],
+                            tag=lif_plan.tag))
+    return out

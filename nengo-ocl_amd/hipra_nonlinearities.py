@@ -416,7 +416,25 @@ def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, N=None, tau_n=None, inc_n=
     n_vec = bin(pflags).count("1")
     plan.bw_per_call = (J.nbytes + 2 * V.nbytes + 2 * W.nbytes + outS.nbytes + n_vec * J.nbytes)
     plan.description = _description(J)
+    # what a GEMV that produces J needs to run this update as its epilogue
+    plan.lif_spec = dict(dt=float(dt), upsample=int(upsample), J=J, V=V, W=W, outS=outS,
+                         ref=ref, tau=tau, amp=amp)
     return plan
+
+
+def lif_population_table(queue, spec):
+    """Per-population rows {v_start, w_start, s_start, tau, ref, amp, pflags} (int32
+    columns) of a `plan_lif` call, plus the parameter pointers and keep-alives."""
+    J = spec["J"]
+    n = len(J)
+    inds = np.arange(n)
+    zeros = np.zeros(n, dtype=np.int64)
+    pcols, pflags, pptrs, keep = _neuron_params(
+        queue, [spec["tau"], spec["ref"], spec["amp"]], J.shape0s, inds, zeros)
+    cols = dict(v_start=spec["V"].starts, w_start=spec["W"].starts, s_start=spec["outS"].starts,
+                tau=pcols[0], ref=pcols[1], amp=pcols[2],
+                pflags=np.full(n, pflags, dtype=np.int32))
+    return cols, pptrs, keep
 
 
 def plan_lif_rate(queue, dt, J, R, ref, tau, amp, N=None, tau_n=None, inc_n=None, tag=None,

@@ -83,17 +83,19 @@ class Plan(BasePlan):
             raise ValueError("launch sizes must be positive, got %r" % (size,))
         return size
 
-    def enqueue(self, wait_for=None, profiling=False):
-        """Put the launch on the queue's stream; returns immediately."""
+    def enqueue(self, wait_for=None, profiling=False, stream=None):
+        """Put the launch on the queue's stream (or on `stream`, a raw handle, while a
+        timestep with independent branches is being recorded); returns immediately."""
         lib = self.queue.lib
+        handle = self.queue.handle if stream is None else stream
         if profiling:
             ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
             _lib.check(lib.nhip_event_create(ctypes.byref(ev0)))
             _lib.check(lib.nhip_event_create(ctypes.byref(ev1)))
-            _lib.check(lib.nhip_event_record(ev0, self.queue.handle))
-        _lib.check(self.kern(self.queue.handle, *self.args), self.name)
+            _lib.check(lib.nhip_event_record(ev0, handle))
+        _lib.check(self.kern(handle, *self.args), self.name)
         if profiling:
-            _lib.check(lib.nhip_event_record(ev1, self.queue.handle))
+            _lib.check(lib.nhip_event_record(ev1, handle))
             self._events_to_profile.append((ev0, ev1))
         return self
 
@@ -124,29 +126,128 @@ class Plan(BasePlan):
         return "%s{%s %s %s}" % (type(self).__name__, self._label(), self.gsize, self.lsize)
 
 
-class _GraphSegment:
-    """A run of consecutive device plans recorded into one executable graph."""
+def plan_dependencies(plans):
+    """For every plan, the earlier plans it has to wait for (indices into `plans`),
+    transitively reduced.
 
-    def __init__(self, queue, plans):
+    Two plans conflict when one writes memory the other reads or writes; `reads_mem`
+    and `writes_mem` of a plan are sets of hashable memory-block keys (the Simulator
+    uses the base signals of the operators behind the plan).  A plan without them is
+    ordered against everything.  The list order of `plans` is a valid execution
+    order, so a conflict always means "the later one waits for the earlier one".
+    """
+    deps, ancestors = [], []
+    for i, p in enumerate(plans):
+        ri, wi = getattr(p, "reads_mem", None), getattr(p, "writes_mem", None)
+        direct = set()
+        for j in range(i):
+            rj, wj = getattr(plans[j], "reads_mem", None), getattr(plans[j], "writes_mem", None)
+            if ri is None or wi is None or rj is None or wj is None:
+                direct.add(j)
+            elif (wj & ri) or (wj & wi) or (rj & wi):
+                direct.add(j)
+        reduced, anc = set(), set()
+        for j in sorted(direct, reverse=True):
+            if j not in anc:
+                reduced.add(j)
+                anc.add(j)
+                anc |= ancestors[j]
+        deps.append(reduced)
+        ancestors.append(anc)
+    return deps
+
+
+class _GraphSegment:
+    """A run of consecutive device plans recorded into one executable graph.
+
+    With `deps` (see `plan_dependencies`) the plans are recorded on several streams so
+    that the graph holds their true dependencies only: kernels of one timestep that
+    do not touch the same memory run side by side when the graph is replayed, which
+    takes the short launch-latency-bound kernels (clock, inputs, filters, probes)
+    off the critical path of the long ones.
+    """
+
+    MAX_SIDE_STREAMS = 7
+
+    def __init__(self, queue, plans, deps=None):
         self.queue = queue
         self.plans = list(plans)
+        self.deps = deps
         self.exec = None
+        self._side_streams = []
+        self.n_streams_used = 1
 
     def capture(self):
         lib = self.queue.lib
         _lib.check(lib.nhip_capture_begin(self.queue.handle), "graph capture begin")
         err = None
+        events = []
         try:
-            for plan in self.plans:
-                plan.enqueue()
+            if self.deps is None:
+                for plan in self.plans:
+                    plan.enqueue()
+            else:
+                self._record_branches(events)
         except Exception as e:  # close the capture before re-raising
             err = e
         handle = ctypes.c_void_p()
         rc = lib.nhip_capture_end(self.queue.handle, ctypes.byref(handle))
+        for ev in events:
+            lib.nhip_event_destroy(ev)
         if err is not None:
             raise err
         _lib.check(rc, "graph capture end")
         self.exec = handle
+
+    def _record_branches(self, events):
+        lib = self.queue.lib
+        streams = [self.queue.handle]
+
+        def new_event(stream):
+            ev = ctypes.c_void_p()
+            _lib.check(lib.nhip_event_create(ctypes.byref(ev)), "event create")
+            events.append(ev)
+            _lib.check(lib.nhip_event_record(ev, stream), "event record")
+            return ev
+
+        def side_stream():
+            k = len(streams) - 1
+            if k == len(self._side_streams):
+                s = ctypes.c_void_p()
+                _lib.check(lib.nhip_stream_create(ctypes.byref(s)), "stream create")
+                self._side_streams.append(s)
+            streams.append(self._side_streams[k])
+            return len(streams) - 1
+
+        fork = new_event(streams[0])  # start of the step: what a branch without inputs waits for
+        tail = {0: None}   # stream -> plan recorded last on it
+        where, done = {}, {}
+        for i, plan in enumerate(self.plans):
+            deps = self.deps[i]
+            si = None
+            for d in sorted(deps, reverse=True):  # continue the stream of a dependency
+                if tail[where[d]] == d:
+                    si = where[d]
+                    break
+            if si is None:
+                if tail[0] is None and not deps:
+                    si = 0
+                elif len(streams) <= self.MAX_SIDE_STREAMS:
+                    si = side_stream()
+                    tail[si] = None
+                    _lib.check(lib.nhip_stream_wait_event(streams[si], fork), "fork")
+                else:  # out of streams: queue behind the oldest tail (an extra, harmless edge)
+                    si = min(tail, key=lambda k: -1 if tail[k] is None else tail[k])
+            for d in deps:
+                if where[d] != si:
+                    _lib.check(lib.nhip_stream_wait_event(streams[si], done[d]), "join")
+            plan.enqueue(stream=streams[si])
+            done[i] = new_event(streams[si])
+            tail[si], where[i] = i, si
+        for k, last in tail.items():
+            if k != 0 and last is not None:
+                _lib.check(lib.nhip_stream_wait_event(streams[0], done[last]), "join")
+        self.n_streams_used = len(streams)
 
     def launch(self, n):
         if self.exec is None:
@@ -157,15 +258,19 @@ class _GraphSegment:
         if self.exec is not None:
             self.queue.lib.nhip_graph_destroy(self.exec)
             self.exec = None
+        for s in self._side_streams:
+            self.queue.lib.nhip_stream_destroy(s)
+        self._side_streams = []
 
 
 class Plans:
     """The ordered plan list of one timestep and its executor."""
 
-    def __init__(self, planlist, profiling, use_graph=True):
+    def __init__(self, planlist, profiling, use_graph=True, branches=True):
         self.plans = list(planlist)
         self.profiling = profiling
         self.use_graph = use_graph
+        self.branches = branches  # record independent plans as parallel graph branches
         self._segments = None  # list of _GraphSegment | PythonPlan
 
     def __call__(self):
@@ -188,16 +293,20 @@ class Plans:
 
     def _build_segments(self):
         segments, run = [], []
+
+        def close_run():
+            if run:
+                deps = plan_dependencies(run) if self.branches else None
+                segments.append(_GraphSegment(run[0].queue, run, deps))
+
         for plan in self.plans:
             if hasattr(plan, "enqueue"):
                 run.append(plan)
             else:
-                if run:
-                    segments.append(_GraphSegment(run[0].queue, run))
-                    run = []
+                close_run()
+                run = []
                 segments.append(plan)
-        if run:
-            segments.append(_GraphSegment(run[0].queue, run))
+        close_run()
         self._segments = segments
 
     def call_n_times(self, n):

@@ -68,6 +68,15 @@ class HipBackend:
                      "plan_lif", "plan_lif_rate", "plan_presentinput"):
             setattr(self, name, getattr(hipra_nonlinearities, name))
         self.plan_block_gemv = hipra_gemv.plan_block_gemv
+        self._fuse_lif = hipra_gemv.fuse_lif
+
+    def fuse_gemv_neurons(self, gemv_plans, neuron_plans):
+        """Plans replacing ``gemv_plans + neuron_plans`` by launches that update the
+        neurons in the epilogue of the GEMV that produces their input, or None."""
+        progs = {id(getattr(p, "prog", None)) for p in gemv_plans}
+        if len(neuron_plans) != 1 or len(progs) != 1 or not hasattr(gemv_plans[0], "prog"):
+            return None
+        return self._fuse_lif(gemv_plans[0].prog, neuron_plans[0])
 
     def upload(self, host_ragged):
         return self._ra.HIPRaggedArray(self.queue, host_ragged)
@@ -184,13 +193,15 @@ class Simulator:
     (the CPU oracle used by the tests plugs in there); ``use_graph=False`` runs
     the plan list as an eager launch loop; ``fuse=False`` keeps vector copies and
     resets as separate operators instead of folding them into the GEMVs
-    (`operators.fuse_into_multidotinc`).
+    (`operators.fuse_into_multidotinc`); ``branches=False`` records the timestep as
+    one chain of kernels instead of a graph in which kernels that touch different
+    memory run side by side.
     """
 
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
                  n_prealloc_probes=32, profiling=None, if_python_code="none",
                  planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
-                 fuse=True):
+                 fuse=True, branches=False):
         self.closed = False
         self.model = None
 
@@ -289,12 +300,35 @@ class Simulator:
         self._filter_positions = []
         self._python_rngs = {}
         plans = []
+        previous = None  # (type, plans) of the group planned last
         for op_type, op_list in op_groups:
-            plans.extend(self._plan_op_group(op_type, op_list))
-        plans.extend(self._plan_probes())
+            group_plans = self._plan_op_group(op_type, op_list)
+            # memory blocks the group's kernels touch, for the executor's dependency graph
+            reads = {sig.base for op in op_list for sig in list(op.reads) + list(op.incs)}
+            writes = {sig.base for op in op_list
+                      for sig in list(op.sets) + list(op.incs) + list(op.updates)}
+            if (fuse and op_type.__name__ == "SimNeurons" and previous is not None
+                    and previous[0].__name__ == "MultiDotInc" and previous[1]
+                    and hasattr(self.backend, "fuse_gemv_neurons")):
+                # neurons right behind the GEMV that computes their input current
+                fused = self.backend.fuse_gemv_neurons(previous[1], group_plans)
+                if fused is not None:
+                    reads = reads | previous[1][0].reads_mem
+                    writes = writes | previous[1][0].writes_mem
+                    del plans[len(plans) - len(previous[1]):]
+                    group_plans = fused
+            for plan in group_plans:
+                plan.reads_mem, plan.writes_mem = reads, writes
+            plans.extend(group_plans)
+            previous = (op_type, group_plans)
+        probe_plans = self._plan_probes()
+        for plan in probe_plans:  # sample buffers and counters are the plan's own
+            plan.reads_mem = {self.model.sig[p]["in"].base for p in self.model.probes}
+            plan.writes_mem = set()
+        plans.extend(probe_plans)
         logger.info("Plans in %0.3f s", _time.time() - t0)
 
-        self._plans = Plans(plans, self.profiling, use_graph=use_graph)
+        self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches)
         self.rng = None
         self._reset_probes()
 

@@ -241,3 +241,27 @@ def test_decoders_decode():
     assert np.abs(acts @ ws[0].T - xs).max() < 0.05
     assert np.abs(acts @ ws[1].T - xs ** 2).max() < 0.05
     assert np.all(acts.max(axis=0) <= 400.5)
+
+
+def test_plan_dependencies():
+    """Conflicts order plans, independent plans stay unordered, edges implied by others
+    are dropped, and a plan without memory sets is ordered against everything."""
+    from nengo_ocl_amd.plan import plan_dependencies
+
+    class P:
+        def __init__(self, reads=None, writes=None):
+            if reads is not None:
+                self.reads_mem, self.writes_mem = set(reads), set(writes)
+
+    plans = [P("", "t"),      # 0 clock
+             P("a", "b"),     # 1 reads a, writes b
+             P("b", "c"),     # 2 after 1 (read after write)
+             P("t", "d"),     # 3 after 0 only
+             P("c", "a"),     # 4 after 2 (c) and after 1 (write after read of a): 1 implied by 2
+             P("dc", "")]     # 5 after 3 and 2; 4 does not write c or d
+    assert plan_dependencies(plans) == [set(), set(), {1}, {0}, {2}, {2, 3}]
+    plans.insert(3, P())      # unknown memory: a barrier
+    deps = plan_dependencies(plans)
+    assert deps[3] == {0, 2} and deps[4] == {3} and deps[5] == {3}
+    plans = [P("", "x"), P("", "x"), P("x", "")]  # two writers of x stay in order
+    assert plan_dependencies(plans) == [set(), {0}, {1}]

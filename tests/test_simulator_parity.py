@@ -153,6 +153,9 @@ def test_c3_large_reduced_spiking(queue, share):
 
     gpu, cpu, pg, pc, _ = build_pair(make)
     with gpu, cpu:
+        # the neurons are updated by the GEMV that computes their input current
+        assert any(p.name == "hipra_gemv.tile_lif" for p in gpu._plans)
+        assert not any(p.name == "hip_lif" for p in gpu._plans)
         check_spiking(gpu, cpu, pg["spikes"], pc["spikes"], 1000, "c3 reduced (8 x 1024 x 64-D)")
 
 
@@ -206,24 +209,41 @@ def test_run_steps_batches_and_reset(queue):
         assert len(sim.data[probes["a"]]) == 5 and sim.n_steps == 42
 
 
-def test_graph_replay_equals_eager(queue):
-    """The recorded graph and the eager launch loop give bit-identical state, also when
-    the graph is replayed in several batches with host work in between."""
+def _graph_cases():
     from nengo_ocl_amd import configs
+
+    return {
+        "c2": lambda: configs.c2_watts_strogatz(n_ens=32, n_driven=4),
+        "c1": lambda: configs.c1_circconv(dims=8, n_per_dim=30),
+        "c4": lambda: configs.c4_pes(n_triples=3, n_neurons=100, dims=4),
+        "c3": lambda: configs.c3_large(n_ens=6, n_neurons=256, dims=16, fan_out=2),
+    }
+
+
+@pytest.mark.parametrize("case", ["c2", "c1", "c4", "c3"])
+def test_graph_replay_equals_eager(queue, case):
+    """The recorded graph -- with independent kernels as side-by-side branches, and as
+    one chain -- and the eager launch loop give bit-identical state, also when the
+    graph is replayed in several batches with host work in between."""
     from nengo_ocl_amd.simulator import Simulator
 
     results = []
-    for use_graph in (True, False):
-        net, probes, _ = configs.c2_watts_strogatz(n_ens=32, n_driven=4)
-        with Simulator(net, seed=1, use_graph=use_graph, n_prealloc_probes=8) as sim:
+    for use_graph, branches in ((True, True), (True, False), (False, False)):
+        net, probes, _ = _graph_cases()[case]()
+        with Simulator(net, seed=1, use_graph=use_graph, branches=branches,
+                       n_prealloc_probes=8) as sim:
             for chunk in (3, 8, 21, 1, 40):
                 sim.run_steps(chunk)
                 _ = sim.signals[sim.model.time]
+            if use_graph and branches:
+                segs = [g for g in sim._plans._segments if hasattr(g, "n_streams_used")]
+                assert segs and all(g.deps is not None for g in segs)
             results.append((np.array(sim.all_data.buf), {k: np.array(sim.data[p])
                                                          for k, p in probes.items()}))
-    assert np.array_equal(results[0][0], results[1][0])
-    for k in results[0][1]:
-        assert np.array_equal(results[0][1][k], results[1][1][k])
+    for other in results[1:]:
+        assert np.array_equal(results[0][0], other[0])
+        for k in results[0][1]:
+            assert np.array_equal(results[0][1][k], other[1][k])
 
 
 def test_multidotinc_compress_literal(queue):
