@@ -190,6 +190,41 @@ int nhip_probes(void *stream, const int *desc, int n, float *countdowns, int *bu
  * memset node, so that it may also be recorded into a graph) */
 int nhip_fill_i32(void *stream, int *dst, int n, int value);
 
+/* ---- several small operations in one launch ------------------------------
+ * One 256-thread group runs the given operations one after the other (a group
+ * barrier in between), each exactly as its own entry point would: for the short
+ * operations of a step (clock, inputs, small copies and filters, probes), whose
+ * cost is the launch, not the work.  The reference launches each of them
+ * separately (plan.py:137-149).  `ops` is a DEVICE array of NhipSeqOp; the pointer
+ * slots hold the device-pointer arguments of the matching nhip_* call in order:
+ *   RESET {blocks, Y}   COPY {desc, X, Y}   SLICEDCOPY {desc, X, Y, XI, YI}
+ *   ELEMENTWISE_INC {desc, A, X, Y}   LINEARFILTER {desc, pos, X, Y, A, B, Xbuf, Ybuf}
+ *   TIMEUPDATE {step_data + step_start, time_data + time_start} (d0 = dt)
+ *   PRESENTINPUT {desc, Y, T, S} (d0 = dt)   DIRECT_UNARY {desc, X, Y} (i0 = opcode)
+ *   PROBES {desc, countdowns, bufpositions, periods, X, Y} */
+enum {
+    NHIP_SEQ_RESET = 1,
+    NHIP_SEQ_COPY = 2,
+    NHIP_SEQ_SLICEDCOPY = 3,
+    NHIP_SEQ_ELEMENTWISE_INC = 4,
+    NHIP_SEQ_LINEARFILTER = 5,
+    NHIP_SEQ_TIMEUPDATE = 6,
+    NHIP_SEQ_PRESENTINPUT = 7,
+    NHIP_SEQ_DIRECT_UNARY = 8,
+    NHIP_SEQ_PROBES = 9
+};
+typedef struct NhipSeqOp {
+    int kind;                /* NHIP_SEQ_* */
+    int n_blocks;            /* rows of the operation's work list (1 for TIMEUPDATE) */
+    int i0;                  /* DIRECT_UNARY: opcode */
+    int reserved;
+    double d0;               /* TIMEUPDATE, PRESENTINPUT: dt */
+    unsigned long long p[8]; /* device pointers, see above */
+} NhipSeqOp;                 /* 88 bytes */
+/* at most 16 operations with at most 32 work-list rows in all; n_rows = the sum of
+ * n_blocks over `ops` (the library cannot read the device table to check it) */
+int nhip_sequence(void *stream, const void *ops, int n_ops, int n_rows);
+
 /* ---- executor ----------------------------------------------------------
  * replaces the Python launch loop of `Plans.enqueue_n_times` (plan.py:137-149):
  * the plan sequence of one (or several) timesteps is recorded once from the

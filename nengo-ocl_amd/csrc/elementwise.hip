@@ -9,28 +9,34 @@
 
 namespace {
 
+// Every operation is written as a "block" function: what one 256-thread group does
+// for one row of its work list.  The plain kernels below run one block per group;
+// the sequence kernel at the end of this file runs the blocks of several small
+// operations one after the other inside a single group.
+
 // ---------------------------------------------------------------- reset
 // clra_nonlinearities.py:154-172 fills 16-element chunks; here a block is up to
 // 4096 elements of one contiguous item.
-__global__ __launch_bounds__(NHIP_WG) void reset_kernel(const int4* __restrict__ blocks,
-                                                        float* __restrict__ Y) {
-    const int4 b = blocks[blockIdx.x];  // {start, count, value_bits, 0}
+__device__ __forceinline__ void reset_block(const int4 b, float* Y, int tid) {
+    // b = {start, count, value_bits, 0}
     const float v = nhip_bits(b.z);
     float* y = Y + b.x;
-    for (int i = threadIdx.x; i < b.y; i += NHIP_WG) y[i] = v;
+    for (int i = tid; i < b.y; i += NHIP_WG) y[i] = v;
+}
+
+__global__ __launch_bounds__(NHIP_WG) void reset_kernel(const int4* __restrict__ blocks, float* Y) {
+    reset_block(blocks[blockIdx.x], Y, threadIdx.x);
 }
 
 // ---------------------------------------------------------------- copy
 // 2-D strided Y (=|+=) X (clra_nonlinearities.py:225-262).
 struct CopyDesc { int x_start, y_start, shape1, x_stride0, y_stride0, offset, count, inc; };
 
-__global__ __launch_bounds__(NHIP_WG) void copy_kernel(const CopyDesc* __restrict__ desc,
-                                                       const float* X, float* Y) {
-    const CopyDesc d = desc[blockIdx.x];
+__device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, float* Y, int tid) {
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const bool flat = (d.x_stride0 == d.shape1) && (d.y_stride0 == d.shape1);
-    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+    for (int k = tid; k < d.count; k += NHIP_WG) {
         const int ij = d.offset + k;
         size_t xo, yo;
         if (flat) {
@@ -45,26 +51,36 @@ __global__ __launch_bounds__(NHIP_WG) void copy_kernel(const CopyDesc* __restric
     }
 }
 
+__global__ __launch_bounds__(NHIP_WG) void copy_kernel(const CopyDesc* __restrict__ desc,
+                                                       const float* X, float* Y) {
+    copy_block(desc[blockIdx.x], X, Y, threadIdx.x);
+}
+
 // ---------------------------------------------------------------- sliced copy
 // Y[yi[k]*ys] (=|+=) X[xi[k]*xs] (clra_nonlinearities.py:321-364); indices are
 // int32 and unique per item, so the scatter needs no atomics.
 struct SlicedDesc { int x_start, x_stride0, y_start, y_stride0, xi_start, yi_start, count, inc; };
 
-__global__ __launch_bounds__(NHIP_WG) void slicedcopy_kernel(const SlicedDesc* __restrict__ desc,
-                                                             const float* X, float* Y,
-                                                             const int* __restrict__ XI,
-                                                             const int* __restrict__ YI) {
-    const SlicedDesc d = desc[blockIdx.x];
+__device__ __forceinline__ void slicedcopy_block(const SlicedDesc d, const float* X, float* Y,
+                                                 const int* __restrict__ XI,
+                                                 const int* __restrict__ YI, int tid) {
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const int* xi = XI + d.xi_start;
     const int* yi = YI + d.yi_start;
-    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+    for (int k = tid; k < d.count; k += NHIP_WG) {
         const float v = x[(size_t)xi[k] * d.x_stride0];
         float* dst = y + (size_t)yi[k] * d.y_stride0;
         if (d.inc) *dst += v;
         else *dst = v;
     }
+}
+
+__global__ __launch_bounds__(NHIP_WG) void slicedcopy_kernel(const SlicedDesc* __restrict__ desc,
+                                                             const float* X, float* Y,
+                                                             const int* __restrict__ XI,
+                                                             const int* __restrict__ YI) {
+    slicedcopy_block(desc[blockIdx.x], X, Y, XI, YI, threadIdx.x);
 }
 
 // ---------------------------------------------------------------- elementwise inc
@@ -85,16 +101,14 @@ __device__ __forceinline__ float ew_element(const float* data, int shape0, int s
     return data[(size_t)i * stride0 + j];
 }
 
-__global__ __launch_bounds__(NHIP_WG) void elementwise_inc_kernel(const EwDesc* __restrict__ desc,
-                                                                  const float* A, const float* X,
-                                                                  float* Y) {
-    const EwDesc d = desc[blockIdx.x];
+__device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const float* A,
+                                                      const float* X, float* Y, int tid) {
     const float* a = A + d.a_start;
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const float alpha = nhip_bits(d.alpha_bits);
     const bool outer = d.flags & 1, inc = d.flags & 2;
-    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+    for (int k = tid; k < d.count; k += NHIP_WG) {
         const int ij = d.offset + k;
         const int i = ij / d.y_shape1, j = ij - i * d.y_shape1;
         float aa, xx;
@@ -114,6 +128,12 @@ __global__ __launch_bounds__(NHIP_WG) void elementwise_inc_kernel(const EwDesc* 
     }
 }
 
+__global__ __launch_bounds__(NHIP_WG) void elementwise_inc_kernel(const EwDesc* __restrict__ desc,
+                                                                  const float* A, const float* X,
+                                                                  float* Y) {
+    elementwise_inc_block(desc[blockIdx.x], A, X, Y, threadIdx.x);
+}
+
 // ---------------------------------------------------------------- linear filter
 // clra_nonlinearities.py:604-711.  Ring buffers: xbuf[(ix+p)%nb] holds x[n-p],
 // ybuf[(iy+p)%na] holds y[n-1-p] (p >= 1); positions step backwards once per call.
@@ -124,23 +144,21 @@ struct LfDesc {
     int b_start, xbuf_start, ybuf_start, size;
 };
 
-__global__ __launch_bounds__(NHIP_WG) void linearfilter_kernel(const LfDesc* __restrict__ desc,
-                                                               int2* pos, const float* X, float* Y,
-                                                               const float* __restrict__ A,
-                                                               const float* __restrict__ B,
-                                                               float* Xbuf, float* Ybuf) {
-    const LfDesc d = desc[blockIdx.x];
+__device__ __forceinline__ void linearfilter_block(const LfDesc d, int2* pos, const float* X,
+                                                   float* Y, const float* __restrict__ A,
+                                                   const float* __restrict__ B, float* Xbuf,
+                                                   float* Ybuf, int block, int tid) {
     const float* a = A + d.a_start;
     const float* b = B + d.b_start;
     const int na = d.na, nb = d.nb;
     const bool general = !(nb == 1 && na <= 1);
     int ix = 0, iy = 0;
     if (general) {
-        const int2 p = pos[blockIdx.x];
+        const int2 p = pos[block];
         ix = p.x;
         iy = p.y;
     }
-    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+    for (int k = tid; k < d.count; k += NHIP_WG) {
         const int ij = d.offset + k;
         const int i = ij / d.shape1, j = ij - i * d.shape1;
         const size_t xij = (size_t)d.x_start + (size_t)i * d.x_stride0 + (size_t)j * d.x_stride1;
@@ -174,30 +192,41 @@ __global__ __launch_bounds__(NHIP_WG) void linearfilter_kernel(const LfDesc* __r
     if (general) {
         // every thread has read its position before anyone moves it
         __syncthreads();
-        if (threadIdx.x == 0)
-            pos[blockIdx.x] = make_int2((ix > 0) ? ix - 1 : nb - 1, (iy > 0) ? iy - 1 : na - 1);
+        if (tid == 0)
+            pos[block] = make_int2((ix > 0) ? ix - 1 : nb - 1, (iy > 0) ? iy - 1 : na - 1);
     }
+}
+
+__global__ __launch_bounds__(NHIP_WG) void linearfilter_kernel(const LfDesc* __restrict__ desc,
+                                                               int2* pos, const float* X, float* Y,
+                                                               const float* __restrict__ A,
+                                                               const float* __restrict__ B,
+                                                               float* Xbuf, float* Ybuf) {
+    linearfilter_block(desc[blockIdx.x], pos, X, Y, A, B, Xbuf, Ybuf, blockIdx.x, threadIdx.x);
 }
 
 // ---------------------------------------------------------------- time update
 // clra_nonlinearities.py:119-133: the step counter is a float32 signal;
 // time = (float)(dt * (double)step) with dt a double literal.
-__global__ void timeupdate_kernel(float* step, float* time, double dt) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
+__device__ __forceinline__ void timeupdate_block(float* step, float* time, double dt, int tid) {
+    if (tid == 0) {
         const float s = step[0] + 1.0f;
         step[0] = s;
         time[0] = (float)(dt * (double)s);
     }
 }
 
+__global__ void timeupdate_kernel(float* step, float* time, double dt) {
+    if (blockIdx.x == 0) timeupdate_block(step, time, dt, threadIdx.x);
+}
+
 // ---------------------------------------------------------------- table playback
 // clra_nonlinearities.py:1694-1730: row index from the float32 step counter.
 struct PiDesc { int y_start, m, t_start, s_start, nt, pt_bits, has_pt, pad; };
 
-__global__ __launch_bounds__(NHIP_WG) void presentinput_kernel(const PiDesc* __restrict__ desc,
-                                                               float dt, float* Y, const float* T,
-                                                               const float* __restrict__ S) {
-    const PiDesc d = desc[blockIdx.x];
+__device__ __forceinline__ void presentinput_block(const PiDesc d, float dt, float* Y,
+                                                   const float* T, const float* __restrict__ S,
+                                                   int tid) {
     const int it = (int)T[d.t_start];
     int ti;
     if (d.has_pt) {
@@ -208,15 +237,20 @@ __global__ __launch_bounds__(NHIP_WG) void presentinput_kernel(const PiDesc* __r
     }
     float* y = Y + d.y_start;
     const float* s = S + d.s_start + (size_t)d.m * ti;
-    for (int i = threadIdx.x; i < d.m; i += NHIP_WG) y[i] = s[i];
+    for (int i = tid; i < d.m; i += NHIP_WG) y[i] = s[i];
+}
+
+__global__ __launch_bounds__(NHIP_WG) void presentinput_kernel(const PiDesc* __restrict__ desc,
+                                                               float dt, float* Y, const float* T,
+                                                               const float* __restrict__ S) {
+    presentinput_block(desc[blockIdx.x], dt, Y, T, S, threadIdx.x);
 }
 
 // ---------------------------------------------------------------- unary function nodes
-__global__ __launch_bounds__(NHIP_WG) void direct_unary_kernel(int opcode,
-                                                               const int4* __restrict__ desc,
-                                                               const float* X, float* Y) {
-    const int4 d = desc[blockIdx.x];  // {x_start, y_start, count, 0}
-    for (int i = threadIdx.x; i < d.z; i += NHIP_WG) {
+__device__ __forceinline__ void direct_unary_block(int opcode, const int4 d, const float* X,
+                                                   float* Y, int tid) {
+    // d = {x_start, y_start, count, 0}
+    for (int i = tid; i < d.z; i += NHIP_WG) {
         const float x = X[d.x + i];
         float y;
         switch (opcode) {
@@ -231,35 +265,39 @@ __global__ __launch_bounds__(NHIP_WG) void direct_unary_kernel(int opcode,
     }
 }
 
+__global__ __launch_bounds__(NHIP_WG) void direct_unary_kernel(int opcode,
+                                                               const int4* __restrict__ desc,
+                                                               const float* X, float* Y) {
+    direct_unary_block(opcode, desc[blockIdx.x], X, Y, threadIdx.x);
+}
+
 // ---------------------------------------------------------------- probes
-// clra_nonlinearities.py:831-902 (plus a capacity guard).  One group per probe; the float32 countdown and
-// the buffer position are read by every thread before the barrier and written by
-// thread 0 after it.
+// clra_nonlinearities.py:831-902 (plus a capacity guard).  One block per probe; the
+// float32 countdown and the buffer position are read by every thread before the
+// barrier and written by thread 0 after it.
 struct ProbeDesc { int x_start, shape0, shape1, stride0, stride1, y_start, capacity, p1; };
 
-__global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __restrict__ desc,
-                                                         float* countdowns, int* bufpositions,
-                                                         const float* __restrict__ periods,
-                                                         const float* X, float* Y) {
-    const int n = blockIdx.x;
+__device__ __forceinline__ void probes_block(const ProbeDesc d, float* countdowns,
+                                             int* bufpositions, const float* __restrict__ periods,
+                                             const float* X, float* Y, int block, int tid) {
+    const int n = block;
     const float countdown = countdowns[n];
     const bool fire = countdown <= 0.0f;
     int bufpos = 0;
     // a full buffer (the host did not drain it in time) drops the sample instead of
     // writing past the end; the position keeps counting so the host can tell
     if (fire) bufpos = bufpositions[n];
-    if (fire && bufpos < desc[n].capacity) {
-        const ProbeDesc d = desc[n];
+    if (fire && bufpos < d.capacity) {
         const int n_dims = d.shape0 * d.shape1;
         const float* x = X + d.x_start;
         float* y = Y + d.y_start + (size_t)bufpos * n_dims;
-        for (int ij = threadIdx.x; ij < n_dims; ij += NHIP_WG) {
+        for (int ij = tid; ij < n_dims; ij += NHIP_WG) {
             const int i = ij / d.shape1, j = ij - i * d.shape1;
             y[ij] = x[(size_t)i * d.stride0 + (size_t)j * d.stride1];
         }
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (tid == 0) {
         if (fire) {
             countdowns[n] = countdown + periods[n] - 1.0f;
             bufpositions[n] = bufpos + 1;
@@ -269,9 +307,122 @@ __global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __rest
     }
 }
 
+__global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __restrict__ desc,
+                                                         float* countdowns, int* bufpositions,
+                                                         const float* __restrict__ periods,
+                                                         const float* X, float* Y) {
+    probes_block(desc[blockIdx.x], countdowns, bufpositions, periods, X, Y, blockIdx.x, threadIdx.x);
+}
+
 __global__ __launch_bounds__(NHIP_WG) void fill_i32_kernel(int* dst, int n, int value) {
     const int i = blockIdx.x * NHIP_WG + threadIdx.x;
     if (i < n) dst[i] = value;
+}
+
+// ---------------------------------------------------------------- sequence
+// Several small operations of a timestep in one launch.  A kernel that moves a few
+// hundred floats costs about as much as its launch and the first cold memory
+// accesses (4-5 us each, one after the other); here one 256-thread group runs
+// the blocks of each operation in turn, a group barrier between operations, so a run
+// of such operations costs one launch.  The operation records and every row of
+// their work lists are fetched into LDS up front, side by side, so that only the
+// data accesses of each operation remain one after the other.  Every block function
+// is the one the plain kernels use, so results are identical.  Data pointers are
+// never marked restrict or read-only: an operation may read what the one before it
+// wrote, and the barrier (which orders global memory at work-group scope) makes
+// that visible.
+constexpr int SEQ_MAX_OPS = 16;
+constexpr int SEQ_MAX_ROWS = 32;
+constexpr int SEQ_ROW_WORDS = 16;  // the widest work-list row: 64 bytes
+
+__device__ __forceinline__ int seq_row_words(int kind) {
+    switch (kind) {
+        case NHIP_SEQ_RESET: return 4;
+        case NHIP_SEQ_DIRECT_UNARY: return 4;
+        case NHIP_SEQ_ELEMENTWISE_INC: return 16;
+        case NHIP_SEQ_LINEARFILTER: return 16;
+        case NHIP_SEQ_TIMEUPDATE: return 0;
+        default: return 8;
+    }
+}
+
+__global__ __launch_bounds__(NHIP_WG) void sequence_kernel(const NhipSeqOp* __restrict__ ops,
+                                                           int n_ops) {
+    __shared__ NhipSeqOp s_ops[SEQ_MAX_OPS];
+    __shared__ __attribute__((aligned(16))) int s_rows[SEQ_MAX_ROWS][SEQ_ROW_WORDS];
+    const int tid = threadIdx.x;
+    {   // operation records: 22 words each
+        const int* src = reinterpret_cast<const int*>(ops);
+        int* dst = reinterpret_cast<int*>(s_ops);
+        const int n_words = n_ops * (int)(sizeof(NhipSeqOp) / sizeof(int));
+        for (int w = tid; w < n_words; w += NHIP_WG) dst[w] = src[w];
+    }
+    __syncthreads();
+    {   // work-list rows: 16 threads per row, one word each
+        const int row = tid >> 4, word = tid & 15;
+        for (int r0 = 0; r0 < SEQ_MAX_ROWS; r0 += NHIP_WG / 16) {
+            int r = r0 + row, k = 0;
+            while (k < n_ops && r >= s_ops[k].n_blocks) r -= s_ops[k++].n_blocks;
+            if (k < n_ops) {
+                const int words = seq_row_words(s_ops[k].kind);
+                if (word < words)
+                    s_rows[r0 + row][word] =
+                        reinterpret_cast<const int*>(s_ops[k].p[0])[r * words + word];
+            }
+        }
+    }
+    __syncthreads();
+    int row = 0;
+    for (int k = 0; k < n_ops; ++k) {
+        const NhipSeqOp& op = s_ops[k];
+#define SEQ_P(i, T) reinterpret_cast<T>(op.p[i])
+#define SEQ_ROW(T) (*reinterpret_cast<const T*>(s_rows[row]))
+        for (int b = 0; b < op.n_blocks; ++b, ++row) {
+            switch (op.kind) {
+                case NHIP_SEQ_RESET:
+                    reset_block(SEQ_ROW(int4), SEQ_P(1, float*), tid);
+                    break;
+                case NHIP_SEQ_COPY:
+                    copy_block(SEQ_ROW(CopyDesc), SEQ_P(1, const float*), SEQ_P(2, float*), tid);
+                    break;
+                case NHIP_SEQ_SLICEDCOPY:
+                    slicedcopy_block(SEQ_ROW(SlicedDesc), SEQ_P(1, const float*), SEQ_P(2, float*),
+                                     SEQ_P(3, const int*), SEQ_P(4, const int*), tid);
+                    break;
+                case NHIP_SEQ_ELEMENTWISE_INC:
+                    elementwise_inc_block(SEQ_ROW(EwDesc), SEQ_P(1, const float*),
+                                          SEQ_P(2, const float*), SEQ_P(3, float*), tid);
+                    break;
+                case NHIP_SEQ_LINEARFILTER:
+                    linearfilter_block(SEQ_ROW(LfDesc), SEQ_P(1, int2*), SEQ_P(2, const float*),
+                                       SEQ_P(3, float*), SEQ_P(4, const float*),
+                                       SEQ_P(5, const float*), SEQ_P(6, float*), SEQ_P(7, float*),
+                                       b, tid);
+                    break;
+                case NHIP_SEQ_TIMEUPDATE:
+                    timeupdate_block(SEQ_P(0, float*), SEQ_P(1, float*), op.d0, tid);
+                    break;
+                case NHIP_SEQ_PRESENTINPUT:
+                    presentinput_block(SEQ_ROW(PiDesc), (float)op.d0, SEQ_P(1, float*),
+                                       SEQ_P(2, const float*), SEQ_P(3, const float*), tid);
+                    break;
+                case NHIP_SEQ_DIRECT_UNARY:
+                    direct_unary_block(op.i0, SEQ_ROW(int4), SEQ_P(1, const float*),
+                                       SEQ_P(2, float*), tid);
+                    break;
+                case NHIP_SEQ_PROBES:
+                    probes_block(SEQ_ROW(ProbeDesc), SEQ_P(1, float*), SEQ_P(2, int*),
+                                 SEQ_P(3, const float*), SEQ_P(4, const float*), SEQ_P(5, float*),
+                                 b, tid);
+                    break;
+                default:
+                    break;
+            }
+            __syncthreads();  // blocks of one operation may share state (ring positions)
+        }
+#undef SEQ_P
+#undef SEQ_ROW
+    }
 }
 
 }  // namespace
@@ -374,6 +525,16 @@ extern "C" int nhip_fill_i32(void* stream, int* dst, int n, int value) {
     if (n < 0 || !dst) return NHIP_E_BADARG;
     hipLaunchKernelGGL(fill_i32_kernel, dim3((n + NHIP_WG - 1) / NHIP_WG), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), dst, n, value);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_sequence(void* stream, const void* ops, int n_ops, int n_rows) {
+    if (n_ops == 0) return 0;
+    if (n_ops < 0 || n_ops > SEQ_MAX_OPS || n_rows < n_ops || n_rows > SEQ_MAX_ROWS || !ops)
+        return NHIP_E_BADARG;
+    hipLaunchKernelGGL(sequence_kernel, dim3(1), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const NhipSeqOp*>(ops), n_ops);
     NHIP_LAUNCH_CHECK();
     return 0;
 }

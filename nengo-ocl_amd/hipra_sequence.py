@@ -1,0 +1,154 @@
+"""Runs of small plans of a timestep, bound into one launch each.
+
+The reference launches every plan separately (plan.py:137-149).  On this device a
+kernel that moves a few hundred floats costs what its launch and its first cold
+memory accesses cost (4-5 us, strictly one after the other), so the clock update,
+input playback, small copies and filters and the probe gather of a step cost more
+than their work.  `merge_small_plans` moves such plans next to each other where the
+memory they touch allows it and binds each run to one ``nhip_sequence`` launch, in
+which a single work-group executes them in order -- the same device functions, the
+same results.
+"""
+
+import ctypes
+
+import numpy as np
+
+from .hipraggedarray import to_device
+from .plan import Plan
+
+# kinds of include/nengo_hip.h
+SEQ_RESET, SEQ_COPY, SEQ_SLICEDCOPY, SEQ_ELEMENTWISE_INC, SEQ_LINEARFILTER = 1, 2, 3, 4, 5
+SEQ_TIMEUPDATE, SEQ_PRESENTINPUT, SEQ_DIRECT_UNARY, SEQ_PROBES = 6, 7, 8, 9
+
+SEQ_OP_DTYPE = np.dtype([("kind", "<i4"), ("n_blocks", "<i4"), ("i0", "<i4"), ("reserved", "<i4"),
+                         ("d0", "<f8"), ("p", "<u8", (8,))])
+assert SEQ_OP_DTYPE.itemsize == 88
+
+# one work-group runs the blocks one after the other: only operations this short,
+# and only so many per launch (limits of the kernel's LDS staging)
+MAX_BLOCKS_PER_OP = 4
+MAX_OPS = 16
+MAX_ROWS = 32
+
+
+def _addr(pointer, byte_offset=0):
+    if pointer is None:
+        return 0
+    value = pointer.value if isinstance(pointer, ctypes.c_void_p) else int(pointer)
+    return (value or 0) + byte_offset
+
+
+def sequence_op(plan):
+    """(kind, n_blocks, i0, d0, pointers) of a device plan, or None if its kernel has
+    no counterpart in the sequence kernel."""
+    name = getattr(getattr(plan, "kern", None), "__name__", None)
+    a = getattr(plan, "args", ())
+    if name == "nhip_reset":
+        table, n, Y = a
+        return SEQ_RESET, n, 0, 0.0, [table, Y]
+    if name == "nhip_copy":
+        desc, n, X, Y = a
+        return SEQ_COPY, n, 0, 0.0, [desc, X, Y]
+    if name == "nhip_slicedcopy":
+        desc, n, X, Y, XI, YI = a
+        return SEQ_SLICEDCOPY, n, 0, 0.0, [desc, X, Y, XI, YI]
+    if name == "nhip_elementwise_inc":
+        desc, n, A, X, Y = a
+        return SEQ_ELEMENTWISE_INC, n, 0, 0.0, [desc, A, X, Y]
+    if name == "nhip_linearfilter":
+        desc, pos, n, X, Y, A, B, Xbuf, Ybuf = a
+        return SEQ_LINEARFILTER, n, 0, 0.0, [desc, pos, X, Y, A, B, Xbuf, Ybuf]
+    if name == "nhip_timeupdate":
+        step, step_start, time, time_start, dt = a
+        return SEQ_TIMEUPDATE, 1, 0, float(dt), [_addr(step, 4 * step_start),
+                                                 _addr(time, 4 * time_start)]
+    if name == "nhip_presentinput":
+        desc, n, dt, Y, T, S = a
+        # the entry point takes dt as a float: round it the same way
+        return SEQ_PRESENTINPUT, n, 0, float(np.float32(dt)), [desc, Y, T, S]
+    if name == "nhip_direct_unary":
+        opcode, desc, n, X, Y = a
+        return SEQ_DIRECT_UNARY, n, int(opcode), 0.0, [desc, X, Y]
+    if name == "nhip_probes":
+        desc, n, countdowns, bufpositions, periods, X, Y = a
+        return SEQ_PROBES, n, 0, 0.0, [desc, countdowns, bufpositions, periods, X, Y]
+    return None
+
+
+def is_small(plan):
+    op = sequence_op(plan)
+    return op is not None and 0 < op[1] <= MAX_BLOCKS_PER_OP
+
+
+def _conflict(p, q):
+    rp, wp = getattr(p, "reads_mem", None), getattr(p, "writes_mem", None)
+    rq, wq = getattr(q, "reads_mem", None), getattr(q, "writes_mem", None)
+    if rp is None or wp is None or rq is None or wq is None:
+        return True
+    return bool((wp & rq) or (wp & wq) or (rp & wq))
+
+
+def plan_sequence(queue, plans):
+    """One launch that runs `plans` (all small, see `is_small`) in order."""
+    table = np.zeros(len(plans), dtype=SEQ_OP_DTYPE)
+    for row, plan in zip(table, plans):
+        kind, n, i0, d0, pointers = sequence_op(plan)
+        row["kind"], row["n_blocks"], row["i0"], row["d0"] = kind, n, i0, d0
+        for k, ptr in enumerate(pointers):
+            row["p"][k] = _addr(ptr)
+    n_rows = int(table["n_blocks"].sum())
+    assert len(plans) <= MAX_OPS and n_rows <= MAX_ROWS
+    dev_table = to_device(queue, table.view(np.int32))
+    merged = Plan(queue, queue.lib.nhip_sequence, (dev_table.ptr, len(plans), n_rows), gsize=(256,),
+                  lsize=(256,), full_args=(dev_table,) + tuple(plans), name="hip_sequence",
+                  tag="+".join(p.name.replace("hip_", "") for p in plans))
+    merged.members = list(plans)
+    bws = [p.bw_per_call for p in plans if p.bw_per_call]
+    merged.bw_per_call = sum(bws) if bws else None
+    reads = [getattr(p, "reads_mem", None) for p in plans]
+    writes = [getattr(p, "writes_mem", None) for p in plans]
+    if all(r is not None for r in reads) and all(w is not None for w in writes):
+        merged.reads_mem = set().union(*reads)
+        merged.writes_mem = set().union(*writes)
+    return merged
+
+
+def merge_small_plans(plans):
+    """The plan list with every run of two or more small plans bound into one launch.
+
+    First every small plan sinks past the large plans behind it that touch different
+    memory (the list order stays a valid execution order), so that small plans
+    separated only by unrelated large ones meet; then runs are merged.
+    """
+    plans = list(plans)
+    small = [hasattr(p, "enqueue") and is_small(p) for p in plans]
+    for i in range(len(plans) - 2, -1, -1):
+        if not small[i]:
+            continue
+        j = i
+        while (j + 1 < len(plans) and not small[j + 1] and hasattr(plans[j + 1], "enqueue")
+               and not _conflict(plans[j], plans[j + 1])):
+            plans[j], plans[j + 1] = plans[j + 1], plans[j]
+            small[j], small[j + 1] = small[j + 1], small[j]
+            j += 1
+    out, run = [], []
+
+    def close():
+        if len(run) >= 2:
+            out.append(plan_sequence(run[0].queue, run))
+        else:
+            out.extend(run)
+        del run[:]
+
+    for plan, s in zip(plans, small):
+        if s:
+            rows = sum(sequence_op(p)[1] for p in run) + sequence_op(plan)[1]
+            if len(run) == MAX_OPS or rows > MAX_ROWS:
+                close()
+            run.append(plan)
+        else:
+            close()
+            out.append(plan)
+    close()
+    return out

@@ -69,6 +69,9 @@ class HipBackend:
             setattr(self, name, getattr(hipra_nonlinearities, name))
         self.plan_block_gemv = hipra_gemv.plan_block_gemv
         self._fuse_lif = hipra_gemv.fuse_lif
+        from . import hipra_sequence
+
+        self.merge_small_plans = hipra_sequence.merge_small_plans
 
     def fuse_gemv_neurons(self, gemv_plans, neuron_plans):
         """Plans replacing ``gemv_plans + neuron_plans`` by launches that update the
@@ -193,15 +196,19 @@ class Simulator:
     (the CPU oracle used by the tests plugs in there); ``use_graph=False`` runs
     the plan list as an eager launch loop; ``fuse=False`` keeps vector copies and
     resets as separate operators instead of folding them into the GEMVs
-    (`operators.fuse_into_multidotinc`); ``branches=False`` records the timestep as
-    one chain of kernels instead of a graph in which kernels that touch different
-    memory run side by side.
+    (`operators.fuse_into_multidotinc`) and the neuron update as a separate launch
+    instead of the epilogue of the GEMV that computes the input currents;
+    ``branches=True`` records the timestep as a graph in which kernels that touch
+    different memory run side by side instead of one chain of kernels (slower on
+    current drivers, off by default); ``merge_small=False`` keeps every short
+    operation (clock, inputs, small copies and filters, probes) as a launch of its
+    own instead of binding runs of them into one launch.
     """
 
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
                  n_prealloc_probes=32, profiling=None, if_python_code="none",
                  planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
-                 fuse=True, branches=False):
+                 fuse=True, branches=False, merge_small=True):
         self.closed = False
         self.model = None
 
@@ -318,7 +325,15 @@ class Simulator:
                     del plans[len(plans) - len(previous[1]):]
                     group_plans = fused
             for plan in group_plans:
-                plan.reads_mem, plan.writes_mem = reads, writes
+                own = getattr(plan, "planned_ops", None)
+                if own is None:
+                    plan.reads_mem, plan.writes_mem = reads, writes
+                else:  # a plan that covers only part of the group
+                    skip = set(getattr(plan, "unread_signals", ()))  # declared, not touched
+                    plan.reads_mem = {sig.base for op in own
+                                      for sig in list(op.reads) + list(op.incs) if sig not in skip}
+                    plan.writes_mem = {sig.base for op in own
+                                       for sig in list(op.sets) + list(op.incs) + list(op.updates)}
             plans.extend(group_plans)
             previous = (op_type, group_plans)
         probe_plans = self._plan_probes()
@@ -326,6 +341,8 @@ class Simulator:
             plan.reads_mem = {self.model.sig[p]["in"].base for p in self.model.probes}
             plan.writes_mem = set()
         plans.extend(probe_plans)
+        if merge_small and hasattr(self.backend, "merge_small_plans"):
+            plans = self.backend.merge_small_plans(plans)
         logger.info("Plans in %0.3f s", _time.time() - t0)
 
         self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches)
@@ -775,7 +792,11 @@ class Simulator:
                     break
             else:
                 python_ops.extend(ops)
-        plans = [p for attr, ops in plan_groups.items() for p in getattr(self, attr)(ops)]
+        plans = []
+        for attr, ops in plan_groups.items():
+            for p in getattr(self, attr)(ops):
+                p.planned_ops = ops  # each process class touches its own signals only
+                plans.append(p)
         plans += [p for op in python_ops for p in self._plan_python_process(op)]
         return plans
 
@@ -829,6 +850,7 @@ class Simulator:
             pos = getattr(p, "bufpos", None)
             if pos is not None:
                 self._filter_positions.extend(pos if isinstance(pos, tuple) else [pos])
+            p.unread_signals = [op.t for op in ops]  # a filter step does not look at the clock
         return plans
 
     _plan_Lowpass = _plan_LinearFilter

@@ -265,3 +265,46 @@ def test_plan_dependencies():
     assert deps[3] == {0, 2} and deps[4] == {3} and deps[5] == {3}
     plans = [P("", "x"), P("", "x"), P("x", "")]  # two writers of x stay in order
     assert plan_dependencies(plans) == [set(), {0}, {1}]
+
+
+def test_small_plans_sink_and_merge(monkeypatch):
+    """Short plans move behind unrelated long ones until they meet, runs of two or more
+    are merged, conflicts and host callbacks stop the move, order of conflicting plans
+    is kept."""
+    from nengo_ocl_amd import hipra_sequence as hs
+
+    class K:
+        def __init__(self, name):
+            self.__name__ = name
+
+    class P:
+        def __init__(self, label, kern, n_blocks, reads, writes):
+            self.label, self.kern, self.name = label, K(kern), kern
+            self.args = (None, n_blocks, None, None) if kern == "nhip_copy" else ()
+            self.reads_mem, self.writes_mem = set(reads), set(writes)
+            self.queue = None
+
+        def enqueue(self):
+            pass
+
+    class Host:  # a host callback plan: no enqueue
+        label = "host"
+
+    def small(label, reads, writes):
+        return P(label, "nhip_copy", 1, reads, writes)
+
+    def big(label, reads, writes):
+        return P(label, "nhip_gemv", 0, reads, writes)
+
+    monkeypatch.setattr(hs, "plan_sequence",
+                        lambda queue, run: type("M", (), {"label": "+".join(p.label for p in run)})())
+    plans = [small("clock", "", "t"), small("bias", "b", "j"), big("sum", "f", "x"),
+             big("enc", "xj", "js"), big("dec", "s", "d"), small("input", "t", "n"),
+             big("filter", "d", "f"), small("nfilter", "n", "m"), small("probe", "f", "")]
+    labels = [p.label for p in hs.merge_small_plans(plans)]
+    assert labels == ["sum", "clock+bias", "enc", "dec", "filter", "input+nfilter+probe"]
+    # a copy of 5 blocks is not small; a host callback is never passed
+    plans = [small("a", "", "p"), Host(), big("g", "q", "r"), small("b", "", "s"),
+             P("wide", "nhip_copy", 5, "", "u"), small("c", "", "v")]
+    labels = [p.label for p in hs.merge_small_plans(plans)]
+    assert labels == ["a", "host", "g", "wide", "b+c"]

@@ -223,15 +223,17 @@ def _graph_cases():
 @pytest.mark.parametrize("case", ["c2", "c1", "c4", "c3"])
 def test_graph_replay_equals_eager(queue, case):
     """The recorded graph -- with independent kernels as side-by-side branches, and as
-    one chain -- and the eager launch loop give bit-identical state, also when the
-    graph is replayed in several batches with host work in between."""
+    one chain, short operations bound into sequence launches -- and the eager loop of
+    one launch per operation give bit-identical state, also when the graph is
+    replayed in several batches with host work in between."""
     from nengo_ocl_amd.simulator import Simulator
 
     results = []
-    for use_graph, branches in ((True, True), (True, False), (False, False)):
+    for use_graph, branches, merge in ((True, True, True), (True, False, True), (False, False, False)):
         net, probes, _ = _graph_cases()[case]()
-        with Simulator(net, seed=1, use_graph=use_graph, branches=branches,
+        with Simulator(net, seed=1, use_graph=use_graph, branches=branches, merge_small=merge,
                        n_prealloc_probes=8) as sim:
+            assert any(p.name == "hip_sequence" for p in sim._plans) == merge
             for chunk in (3, 8, 21, 1, 40):
                 sim.run_steps(chunk)
                 _ = sim.signals[sim.model.time]
