@@ -310,12 +310,16 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     // neuron r of the item's population, which is updated on the spot
     LifPop pop = {};
     if (LIF) pop = lif.pops[task.item];
+    // an item without dot products that would copy Y onto itself unchanged is only
+    // there for its epilogue (a constant input current): nothing to store
+    const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
+                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
 #pragma unroll
     for (int k = 0; k < ROW_SLOTS; ++k) {
         const int r = lane + k * NHIP_WAVE;
         if (r < n_rows) {
             const float y = sum[k] + cf.z;
-            Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
+            if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
             if (LIF && pop.enabled) lif_epilogue(lif, pop, task.row0 + r, y);
         }
     }
@@ -540,12 +544,16 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     wave_sync();
     LifPop pop = {};
     if (LIF) pop = lif.pops[task.item];
+    // an item without dot products that would copy Y onto itself unchanged is only
+    // there for its epilogue (a constant input current): nothing to store
+    const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
+                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
 #pragma unroll
     for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
         const int r = lane + k * NHIP_WAVE;
         if (r < n_rows) {
             const float y = ys[r] + cf.z;
-            Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
+            if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
             if (LIF && pop.enabled) lif_epilogue(lif, pop, task.row0 + r, y);
         }
     }

@@ -317,6 +317,51 @@ def fuse_into_multidotinc(operators):
     return fused
 
 
+def neurons_read_constant_input(operators, keep=()):
+    """Neurons whose input current is only ever a copy of a constant (an ensemble
+    without incoming connections: J = bias every step) read that constant directly,
+    and the copy goes away.
+
+    Applies to ``Copy(src -> J)`` (whole vectors, not an increment) when nothing else
+    writes J, nothing writes src, and the neuron operator is the only reader of J;
+    signals in `keep` (probed ones) are left alone.  The neuron update sees the same
+    values, so results do not change; J itself is no longer refreshed.
+    """
+    import copy as _copy
+
+    written = {}
+    readers = {}
+    for op in operators:
+        for sig in list(op.sets) + list(op.incs) + list(op.updates):
+            written.setdefault(sig.base, []).append(op)
+        for sig in list(op.reads) + list(op.incs):
+            readers.setdefault(sig.base, []).append(op)
+    keep_bases = {sig.base for sig in keep}
+    drop, replace = set(), {}
+    for op in operators:
+        if not _is(op, "SimNeurons") or not hasattr(op, "J"):
+            continue
+        J = op.J
+        if J.base in keep_bases or getattr(J, "is_view", False):
+            continue
+        writers = written.get(J.base, [])
+        if len(writers) != 1 or len(readers.get(J.base, [])) != 1:
+            continue
+        cp = writers[0]
+        if not (_is(cp, "Copy") and not cp.inc and cp.src_slice is None and cp.dst_slice is None
+                and cp.dst is J and cp.src.shape == J.shape and cp.src.base not in written
+                and not getattr(cp.src, "is_view", False)):
+            continue
+        new = _copy.copy(op)
+        new.J = cp.src
+        new.reads = [cp.src if sig is J else sig for sig in op.reads]
+        replace[op] = new
+        drop.add(cp)
+    if not replace:
+        return operators
+    return [replace.get(op, op) for op in operators if op not in drop]
+
+
 def simplify_operators(operators):
     """Apply every function in ``simplifications`` in turn."""
     for simplification in simplifications:

@@ -168,26 +168,33 @@ class _GraphSegment:
     """
 
     MAX_SIDE_STREAMS = 7
+    MAX_UNROLL = 16        # timesteps recorded back to back into the long graph
+    MAX_GRAPH_NODES = 1024
 
     def __init__(self, queue, plans, deps=None):
         self.queue = queue
         self.plans = list(plans)
         self.deps = deps
-        self.exec = None
+        self.execs = {}  # timesteps per graph -> executable graph
+        self.unroll = max(1, min(self.MAX_UNROLL, self.MAX_GRAPH_NODES // max(1, len(self.plans))))
         self._side_streams = []
         self.n_streams_used = 1
 
-    def capture(self):
+    def capture(self, n_steps=1):
+        """Record `n_steps` consecutive timesteps into one executable graph.  Between two
+        graph launches the device idles for several microseconds; a graph that holds
+        many steps pays that once."""
         lib = self.queue.lib
         _lib.check(lib.nhip_capture_begin(self.queue.handle), "graph capture begin")
         err = None
         events = []
         try:
-            if self.deps is None:
-                for plan in self.plans:
-                    plan.enqueue()
-            else:
-                self._record_branches(events)
+            for _ in range(n_steps):
+                if self.deps is None:
+                    for plan in self.plans:
+                        plan.enqueue()
+                else:
+                    self._record_branches(events)
         except Exception as e:  # close the capture before re-raising
             err = e
         handle = ctypes.c_void_p()
@@ -197,7 +204,11 @@ class _GraphSegment:
         if err is not None:
             raise err
         _lib.check(rc, "graph capture end")
-        self.exec = handle
+        self.execs[n_steps] = handle
+
+    @property
+    def exec(self):
+        return self.execs.get(1)
 
     def _record_branches(self, events):
         lib = self.queue.lib
@@ -250,14 +261,19 @@ class _GraphSegment:
         self.n_streams_used = len(streams)
 
     def launch(self, n):
-        if self.exec is None:
-            self.capture()
-        _lib.check(self.queue.lib.nhip_graph_launch(self.exec, self.queue.handle, n), "graph launch")
+        lib = self.queue.lib
+        long_runs, rest = (n // self.unroll, n % self.unroll) if self.unroll > 1 else (0, n)
+        for n_steps, times in ((self.unroll, long_runs), (1, rest)):
+            if times:
+                if n_steps not in self.execs:
+                    self.capture(n_steps)
+                _lib.check(lib.nhip_graph_launch(self.execs[n_steps], self.queue.handle, times),
+                           "graph launch")
 
     def destroy(self):
-        if self.exec is not None:
-            self.queue.lib.nhip_graph_destroy(self.exec)
-            self.exec = None
+        for handle in self.execs.values():
+            self.queue.lib.nhip_graph_destroy(handle)
+        self.execs = {}
         for s in self._side_streams:
             self.queue.lib.nhip_stream_destroy(s)
         self._side_streams = []

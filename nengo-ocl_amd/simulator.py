@@ -191,7 +191,8 @@ class Simulator:
 
     Parameters follow the reference (simulator.py:145-190): ``network, dt, seed,
     model, context, n_prealloc_probes, profiling, if_python_code, planner,
-    progress_bar``.  ``context`` is the HIP device index here.  Not in the
+    progress_bar``.  ``context`` is the HIP device index here; ``n_prealloc_probes``
+    defaults to what fits 64 MiB (32 to 4096 rows) instead of 32.  Not in the
     reference: ``backend`` replaces the device side of the ``plan_*`` boundary
     (the CPU oracle used by the tests plugs in there); ``use_graph=False`` runs
     the plan list as an eager launch loop; ``fuse=False`` keeps vector copies and
@@ -206,7 +207,7 @@ class Simulator:
     """
 
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
-                 n_prealloc_probes=32, profiling=None, if_python_code="none",
+                 n_prealloc_probes=None, profiling=None, if_python_code="none",
                  planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
                  fuse=True, branches=False, merge_small=True):
         self.closed = False
@@ -245,6 +246,8 @@ class Simulator:
         operators = list(map(MultiDotInc.convert_to, operators))
         if fuse:
             operators = ops_mod.fuse_into_multidotinc(operators)
+            operators = ops_mod.neurons_read_constant_input(
+                operators, keep=[self.model.sig[p]["in"] for p in self.model.probes])
         operators = MultiDotInc.compress(operators)
         op_groups = planner(operators)
         assert len([t for t, _ in op_groups if t.__name__ == "Reset"]) < 2, \
@@ -579,13 +582,22 @@ class Simulator:
         return self.dt * steps[steps % period < 1]
 
     # ------------------------------------------------------------- planning
+    # probe rows buffered on the device when `n_prealloc_probes` is None: as many as fit
+    # this many bytes, between the reference's 32 and 4096 (draining means a device
+    # sync and several host copies, which cost tens of steps of a fast model)
+    PROBE_BUFFER_BYTES = 64 * 1024 * 1024
+
     def _plan_probes(self):
-        if len(self.model.probes) == 0:
+        probes = self.model.probes
+        if self.n_prealloc_probes is None:
+            row_bytes = 4 * sum(self.model.sig[p]["in"].size for p in probes)
+            rows = self.PROBE_BUFFER_BYTES // max(row_bytes, 1)
+            self.n_prealloc_probes = int(min(4096, max(32, rows - rows % 32)))
+        if len(probes) == 0:
             self._max_steps_between_probes = self.n_prealloc_probes
             self._probe_plan = None
             return []
         n_prealloc = self.n_prealloc_probes
-        probes = self.model.probes
         periods = [max(1 if p.sample_every is None else p.sample_every / self.dt, 1)
                    for p in probes]
         X = self.all_data[[self.sidx[self.model.sig[p]["in"]] for p in probes]]

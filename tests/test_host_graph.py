@@ -176,7 +176,7 @@ def test_probe_sample_every():
     net, _, _ = configs.c4_pes(n_triples=1, n_neurons=50, dims=2, solver="lstsq", sample_every=0.01)
     p_fast = net.Probe(net.ensembles[0], synapse=0.01)
     p_slow = net.probes[0]
-    with OracleSimulator(net, seed=1) as sim:
+    with OracleSimulator(net, seed=1, n_prealloc_probes=32) as sim:
         assert sim._max_steps_between_probes == 32  # 32 buffer rows x the shortest period (1 step)
         sim.run_steps(95)
         assert len(sim.data[p_fast]) == 95 and len(sim.data[p_slow]) == 9
@@ -308,3 +308,32 @@ def test_small_plans_sink_and_merge(monkeypatch):
              P("wide", "nhip_copy", 5, "", "u"), small("c", "", "v")]
     labels = [p.label for p in hs.merge_small_plans(plans)]
     assert labels == ["a", "host", "g", "wide", "b+c"]
+
+
+def test_neurons_without_input_read_their_bias():
+    """An ensemble without incoming connections: the copy of its bias into J goes away
+    (the neurons read the bias directly); spikes are unchanged."""
+    def make():
+        net = minibuilder.Network(seed=2)
+        node = net.Node(minibuilder.WhiteSignal(1.0, 5.0, seed=0), size_out=1)
+        driven, idle = net.Ensemble(40, 1), net.Ensemble(40, 1)
+        net.Connection(node, driven, synapse=None)
+        probes = [net.Probe(driven.neurons), net.Probe(idle.neurons)]
+        return net, probes
+
+    def n_copies(sim):
+        return sum(type(op).__name__ == "Copy" for op in sim.operators)
+
+    net, probes = make()
+    plain = OracleSimulator(net, seed=1, fuse=False)
+    net2, probes2 = make()
+    fused = OracleSimulator(net2, seed=1, fuse=True)
+    assert n_copies(fused) < n_copies(plain)
+    idle_op = [op for op in fused.operators if type(op).__name__ == "SimNeurons"
+               and "bias" in (op.J.name or "")]
+    assert len(idle_op) == 1
+    plain.run_steps(300)
+    fused.run_steps(300)
+    for a, b in zip(probes, probes2):
+        assert np.array_equal(plain.data[a], fused.data[b])
+    assert plain.data[probes[1]].sum() > 0
