@@ -115,6 +115,22 @@ int nhip_gemv_tile_lif(void *stream, int vec, int pow2_cols, int blk_words, cons
                        const int *pops, double dt, int upsample, float *V, float *W, float *S,
                        const float *TAU, const float *REF, const float *AMP);
 
+/* nhip_gemv_tile followed by the step of first-order filters on its outputs, in one
+ * launch: replaces `plan_block_gemv` (clra_gemv.py:1193-1195) + the simple case of
+ * `plan_linearfilter` (clra_nonlinearities.py:577-803, one numerator and at most one
+ * denominator coefficient: a decoded value and the synapses of the connections
+ * that carry it).  Row r of item b is the new input of element r of each of the
+ * item's filters:
+ *   item_targets : int32[n_items][2] {first target, number of targets}
+ *   targets      : int32[n][4] {y_start, a0 bits, b0 bits, na}
+ *   F[y_start + r] = b0 * y - a0 * F[y_start + r]   (na == 1)   or   b0 * y   (na == 0)
+ * Y is still written.  The filter outputs must not overlap anything the launch reads
+ * through A, X or Yin.  Results are bit-identical to the two separate calls. */
+int nhip_gemv_tile_filter(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
+                          const float *coefs, const int *dots, const int *tasks, int n_tasks,
+                          const float *A, const float *X, const float *Yin, float *Y,
+                          const int *item_targets, const int *targets, float *F);
+
 /* ---- neurons -----------------------------------------------------------
  * LIF with refractory state and spike-time interpolation.
  * replaces: clra_nonlinearities.py `plan_lif` (:1028-1146, non-adaptive,

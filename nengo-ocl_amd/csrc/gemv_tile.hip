@@ -33,6 +33,8 @@
 #include "gemv_types.h"
 #include "neuron_math.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int TILE = 128;          // columns per tile of the reference kernel
@@ -101,12 +103,12 @@ struct Stage {
     GemvDot dot;
 };
 
-template <int VEC, bool LIF>
+template <int VEC, int EPI>
 __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
-    float* Y, LifArgs lif)
+    float* Y, EpilogueArgs epi)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
@@ -306,10 +308,13 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
         sb = sd;
     }
 
-    // the finished rows; with LIF, row r of the item is also the input current of
-    // neuron r of the item's population, which is updated on the spot
+    // the finished rows; with the LIF epilogue, row r of the item is also the input
+    // current of neuron r of the item's population, which is updated on the spot; with
+    // the filter epilogue it is the new input of element r of the item's filters
     LifPop pop = {};
-    if (LIF) pop = lif.pops[task.item];
+    int2 filters = make_int2(0, 0);
+    if (EPI == EPI_LIF) pop = epi.lif.pops[task.item];
+    if (EPI == EPI_FILTER) filters = epi.filter.item_targets[task.item];
     // an item without dot products that would copy Y onto itself unchanged is only
     // there for its epilogue (a constant input current): nothing to store
     const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
@@ -320,7 +325,8 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
         if (r < n_rows) {
             const float y = sum[k] + cf.z;
             if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
-            if (LIF && pop.enabled) lif_epilogue(lif, pop, task.row0 + r, y);
+            if (EPI == EPI_LIF && pop.enabled) lif_epilogue(epi.lif, pop, task.row0 + r, y);
+            if (EPI == EPI_FILTER) filter_epilogue(epi.filter, filters, task.row0 + r, y);
         }
     }
 }
@@ -349,12 +355,12 @@ struct P2Stage {
     GemvDot dot;  // p0 = rows per block, p1 = log2(columns)
 };
 
-template <bool LIF>
+template <int EPI>
 __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
-    float* Y, LifArgs lif)
+    float* Y, EpilogueArgs epi)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
@@ -543,7 +549,9 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
 
     wave_sync();
     LifPop pop = {};
-    if (LIF) pop = lif.pops[task.item];
+    int2 filters = make_int2(0, 0);
+    if (EPI == EPI_LIF) pop = epi.lif.pops[task.item];
+    if (EPI == EPI_FILTER) filters = epi.filter.item_targets[task.item];
     // an item without dot products that would copy Y onto itself unchanged is only
     // there for its epilogue (a constant input current): nothing to store
     const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
@@ -554,7 +562,8 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
         if (r < n_rows) {
             const float y = ys[r] + cf.z;
             if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
-            if (LIF && pop.enabled) lif_epilogue(lif, pop, task.row0 + r, y);
+            if (EPI == EPI_LIF && pop.enabled) lif_epilogue(epi.lif, pop, task.row0 + r, y);
+            if (EPI == EPI_FILTER) filter_epilogue(epi.filter, filters, task.row0 + r, y);
         }
     }
 }
@@ -572,7 +581,7 @@ namespace {
 
 int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* items,
                 const float* coefs, const int* dots, const int* tasks, int n_tasks, const float* A,
-                const float* X, const float* Yin, float* Y, const LifArgs* lif) {
+                const float* X, const float* Yin, float* Y, int epilogue, const EpilogueArgs& args) {
     if (n_tasks == 0) return 0;
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
@@ -586,7 +595,6 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
     const int n_groups = (n_tasks + waves - 1) / waves;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const LifArgs args = lif ? *lif : LifArgs{};
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
                            reinterpret_cast<const GemvItem*>(items),
@@ -595,15 +603,15 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
                            reinterpret_cast<const GemvTask*>(tasks), n_tasks, blk_words, A, X, Yin,
                            Y, args);
     };
-    if (lif) {
-        if (pow2_cols) launch(gemv_tile_p2_kernel<true>);
-        else if (vec == 4) launch(gemv_tile_kernel<4, true>);
-        else launch(gemv_tile_kernel<1, true>);
-    } else {
-        if (pow2_cols) launch(gemv_tile_p2_kernel<false>);
-        else if (vec == 4) launch(gemv_tile_kernel<4, false>);
-        else launch(gemv_tile_kernel<1, false>);
-    }
+    auto launch_epi = [&](auto epi_tag) {
+        constexpr int E = decltype(epi_tag)::value;
+        if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
+        else if (vec == 4) launch(gemv_tile_kernel<4, E>);
+        else launch(gemv_tile_kernel<1, E>);
+    };
+    if (epilogue == EPI_LIF) launch_epi(std::integral_constant<int, EPI_LIF>{});
+    else if (epilogue == EPI_FILTER) launch_epi(std::integral_constant<int, EPI_FILTER>{});
+    else launch_epi(std::integral_constant<int, EPI_NONE>{});
     NHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -615,7 +623,7 @@ extern "C" int nhip_gemv_tile(void* stream, int vec, int pow2_cols, int blk_word
                               const int* tasks, int n_tasks, const float* A, const float* X,
                               const float* Yin, float* Y) {
     return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
-                       Yin, Y, nullptr);
+                       Yin, Y, EPI_NONE, EpilogueArgs{});
 }
 
 extern "C" int nhip_gemv_tile_lif(void* stream, int vec, int pow2_cols, int blk_words,
@@ -625,7 +633,8 @@ extern "C" int nhip_gemv_tile_lif(void* stream, int vec, int pow2_cols, int blk_
                                   int upsample, float* V, float* W, float* S, const float* TAU,
                                   const float* REF, const float* AMP) {
     if (!pops || !V || !W || !S || upsample < 1 || !(dt > 0.0)) return NHIP_E_BADARG;
-    LifArgs lif;
+    EpilogueArgs args{};
+    LifArgs& lif = args.lif;
     lif.pops = reinterpret_cast<const LifPop*>(pops);
     lif.dtu = (float)(dt / (double)upsample);  // formed in double and rounded once, as in nhip_lif
     lif.dt_inv = (float)(1.0 / dt);
@@ -637,5 +646,19 @@ extern "C" int nhip_gemv_tile_lif(void* stream, int vec, int pow2_cols, int blk_
     lif.REF = REF;
     lif.AMP = AMP;
     return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
-                       Yin, Y, &lif);
+                       Yin, Y, EPI_LIF, args);
+}
+
+extern "C" int nhip_gemv_tile_filter(void* stream, int vec, int pow2_cols, int blk_words,
+                                     const int* items, const float* coefs, const int* dots,
+                                     const int* tasks, int n_tasks, const float* A, const float* X,
+                                     const float* Yin, float* Y, const int* item_targets,
+                                     const int* targets, float* F) {
+    if (!item_targets || !targets || !F) return NHIP_E_BADARG;
+    EpilogueArgs args{};
+    args.filter.item_targets = reinterpret_cast<const int2*>(item_targets);
+    args.filter.targets = reinterpret_cast<const FilterTarget*>(targets);
+    args.filter.F = F;
+    return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
+                       Yin, Y, EPI_FILTER, args);
 }

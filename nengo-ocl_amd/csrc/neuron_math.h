@@ -1,4 +1,4 @@
-// Per-neuron update rules shared by the neuron kernels and by GEMV epilogues.
+// Per-element update rules shared by the neuron / filter kernels and by GEMV epilogues.
 #pragma once
 
 #include "nhip_common.h"
@@ -70,3 +70,32 @@ __device__ __forceinline__ void lif_epilogue(const LifArgs& a, const LifPop& p, 
     a.W[(size_t)p.w_start + i] = w;
     a.S[(size_t)p.s_start + i] = spiked ? __fmul_rn(amp, a.dt_inv) : 0.0f;
 }
+
+// First-order filters fed by one output item of a GEMV (a decoded value and the
+// synapses of the connections that carry it): y = b0 x - a0 y, or y = b0 x.
+struct FilterTarget { int y_start, a_bits, b_bits, na; };
+
+struct FilterArgs {
+    const int2* item_targets;     // per GEMV item: {first target, number of targets}
+    const FilterTarget* targets;
+    float* F;                     // buffer that holds the filter outputs
+};
+
+// Filter step of element i of every target of a GEMV item whose fresh output is x
+// (the arithmetic of the simple case of the linear-filter kernel,
+// clra_nonlinearities.py:630-650: rounded products, rounded subtract).
+__device__ __forceinline__ void filter_epilogue(const FilterArgs& a, int2 range, int i, float x) {
+    for (int q = 0; q < range.y; ++q) {
+        const FilterTarget t = a.targets[range.x + q];
+        float* f = a.F + (size_t)t.y_start + i;
+        const float bx = __fmul_rn(nhip_bits(t.b_bits), x);
+        *f = t.na ? __fsub_rn(bx, __fmul_rn(nhip_bits(t.a_bits), *f)) : bx;
+    }
+}
+
+// What a GEMV launch does with a finished output row besides storing it.
+enum { EPI_NONE = 0, EPI_LIF = 1, EPI_FILTER = 2 };
+struct EpilogueArgs {
+    LifArgs lif;
+    FilterArgs filter;
+};

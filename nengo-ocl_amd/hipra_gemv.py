@@ -513,3 +513,109 @@ def fuse_lif(prog, lif_plan):
                             _subset_param(spec["amp"], rest), upsample=spec["upsample"],
                             tag=lif_plan.tag))
     return out
+
+
+def _read_spans(prog, ptr_value):
+    """Element intervals a GEMV reads through A, X and a Y_in that is not its Y, in
+    the device buffer at `ptr_value`."""
+    read = []
+    for g in prog.geometry:
+        for d in g["dots"]:
+            if prog.A.ptr.value == ptr_value:
+                read.append(_span(prog.A, d["a_j"]))
+            if prog.X.ptr.value == ptr_value:
+                read.append(_span(prog.X, d["x_j"]))
+    if prog.Y_in.ptr.value == ptr_value:
+        for b in range(len(prog.Y)):
+            if (int(prog.Y_in.starts[b]) != int(prog.Y.starts[b])
+                    or prog.Y_in.ptr.value != prog.Y.ptr.value):
+                read.append(_span(prog.Y_in, b))
+    return [iv for iv in read if iv]
+
+
+def fuse_linearfilter(gemv_plans, lf_plan):
+    """Fewer launches for "Y = GEMV(...); filter step on Y" (clra_gemv.py
+    `plan_block_gemv` followed by clra_nonlinearities.py `plan_linearfilter`): the
+    reference-order kernel for large items steps the first-order filters whose input
+    is one of its output items as soon as a row is final.
+
+    `gemv_plans` are the plans of one GEMV (one `gemv_prog`).  A filter item is fused
+    when it has one numerator and at most one denominator coefficient, its input is
+    exactly the output of a large item in a plan without another epilogue, and both
+    vectors are contiguous.  Returns ``(plans replacing gemv_plans, plans replacing
+    [lf_plan])`` -- the second list holds a filter launch for the items that were not
+    fused, or is empty -- or None when nothing can be fused.
+    """
+    from .hipra_nonlinearities import plan_linearfilter
+
+    spec = getattr(lf_plan, "lf_spec", None)
+    if spec is None or not gemv_plans:
+        return None
+    prog = gemv_plans[0].prog
+    queue, lib = prog.queue, prog.queue.lib
+    X, F, A, B = spec["X"], spec["Y"], spec["A"], spec["B"]
+    Y = prog.Y
+    if X.ptr.value != Y.ptr.value:
+        return None
+    large = {}
+    for plan in gemv_plans:
+        if plan.name == "hipra_gemv.tile" and plan.kernel_class[0] == 3:
+            for b in plan.members:
+                if int(Y.stride0s[b]) == 1:
+                    large[(int(Y.starts[b]), int(Y.shape0s[b]))] = b
+    if not large:
+        return None
+    a_host, b_host = A.to_host(), B.to_host()
+    targets_of = defaultdict(list)
+    rest = []
+    for i in range(len(X)):
+        simple = int(B.shape0s[i]) == 1 and int(A.shape0s[i]) <= 1
+        vector = (int(X.shape1s[i]) == 1 and int(X.stride0s[i]) == 1
+                  and int(F.shape1s[i]) == 1 and int(F.stride0s[i]) == 1)
+        b = large.get((int(X.starts[i]), int(X.shape0s[i]))) if simple and vector else None
+        if b is None:
+            rest.append(i)
+            continue
+        na = int(A.shape0s[i])
+        a0 = np.float32(a_host[i][0, 0]) if na else np.float32(0)
+        b0 = np.float32(b_host[i][0, 0])
+        targets_of[b].append((int(F.starts[i]), int(a0.view(np.int32)), int(b0.view(np.int32)), na))
+    if not targets_of:
+        return None
+    fused_filters = [i for i in range(len(X)) if i not in set(rest)]
+    written = [iv for iv in (_span(F, i) for i in fused_filters) if iv]
+    if _overlaps(written, _read_spans(prog, F.ptr.value)):
+        return None
+    if F.ptr.value == Y.ptr.value and _overlaps(
+            written, [iv for iv in (_span(Y, b) for b in range(len(Y))) if iv]):
+        return None
+
+    item_targets = np.zeros((len(Y), 2), dtype=np.int32)
+    target_rows = []
+    for b, rows in sorted(targets_of.items()):
+        item_targets[b] = (len(target_rows), len(rows))
+        target_rows.extend(rows)
+    dev_items = to_device(queue, item_targets)
+    dev_targets = to_device(queue, np.array(target_rows, dtype=np.int32))
+    extra = (dev_items.ptr, dev_targets.ptr, F.ptr)
+    out = []
+    for plan in gemv_plans:
+        if plan.name != "hipra_gemv.tile" or not any(b in targets_of for b in plan.members):
+            out.append(plan)
+            continue
+        f_bytes = sum(8 * int(Y.shape0s[b]) * len(targets_of[b]) for b in plan.members
+                      if b in targets_of)  # filter state in and out
+        fused = Plan(queue, lib.nhip_gemv_tile_filter, plan.args + extra, gsize=plan.gsize,
+                     lsize=plan.lsize, full_args=plan.full_args + (dev_items, dev_targets, F.dev_buf),
+                     name="hipra_gemv.tile_filter", tag=plan.tag,
+                     bw_per_call=plan.bw_per_call + f_bytes, flops_per_call=plan.flops_per_call)
+        fused.description = plan.description
+        fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
+        fused.members, fused.prog = plan.members, prog
+        fused.gemv_bytes = plan.bw_per_call
+        out.append(fused)
+    residual = []
+    if rest:
+        residual = plan_linearfilter(queue, X[rest], F[rest], A[rest], B[rest],
+                                     spec["Xbuf"][rest], spec["Ybuf"][rest], tag=lf_plan.tag)
+    return out, residual

@@ -265,6 +265,8 @@ def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
     plan.bw_per_call = (X.nbytes + Y.nbytes + A.nbytes + B.nbytes + Xbuf.nbytes + Ybuf.nbytes)
     plan.description = _description(Y)
     plan.bufpos = pos  # zeroed again by Simulator.reset()
+    # what a GEMV that produces X needs to run simple filters as its epilogue
+    plan.lf_spec = dict(X=X, Y=Y, A=A, B=B, Xbuf=Xbuf, Ybuf=Ybuf)
     return [plan]
 
 

@@ -72,6 +72,8 @@ class HipBackend:
         from . import hipra_sequence
 
         self.merge_small_plans = hipra_sequence.merge_small_plans
+        self.plans_conflict = hipra_sequence._conflict
+        self.fuse_gemv_filter = hipra_gemv.fuse_linearfilter
 
     def fuse_gemv_neurons(self, gemv_plans, neuron_plans):
         """Plans replacing ``gemv_plans + neuron_plans`` by launches that update the
@@ -344,6 +346,8 @@ class Simulator:
             plan.reads_mem = {self.model.sig[p]["in"].base for p in self.model.probes}
             plan.writes_mem = set()
         plans.extend(probe_plans)
+        if fuse and hasattr(self.backend, "fuse_gemv_filter"):
+            plans = self._fuse_filter_epilogues(plans)
         if merge_small and hasattr(self.backend, "merge_small_plans"):
             plans = self.backend.merge_small_plans(plans)
         logger.info("Plans in %0.3f s", _time.time() - t0)
@@ -351,6 +355,44 @@ class Simulator:
         self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches)
         self.rng = None
         self._reset_probes()
+
+    def _fuse_filter_epilogues(self, plans):
+        """Synapse filters whose input is the output of a large GEMV item become the
+        epilogue of that GEMV (`hipra_gemv.fuse_linearfilter`), when no plan between
+        the two touches what the filter reads or writes."""
+        plans = list(plans)
+        j = 0
+        while j < len(plans):
+            lf = plans[j]
+            j += 1
+            if getattr(lf, "lf_spec", None) is None:
+                continue
+            i = j - 2
+            while i >= 0 and not hasattr(plans[i], "prog"):
+                if not hasattr(plans[i], "enqueue") or self.backend.plans_conflict(lf, plans[i]):
+                    i = -1
+                    break
+                i -= 1
+            if i < 0:
+                continue
+            lo = i
+            while lo > 0 and getattr(plans[lo - 1], "prog", None) is plans[i].prog:
+                lo -= 1
+            result = self.backend.fuse_gemv_filter(plans[lo:i + 1], lf)
+            if result is None:
+                continue
+            fused, residual = result
+            for new, old in zip(fused, plans[lo:i + 1]):
+                new.reads_mem = old.reads_mem | lf.reads_mem
+                new.writes_mem = old.writes_mem | lf.writes_mem
+            for p in residual:
+                p.reads_mem, p.writes_mem = lf.reads_mem, lf.writes_mem
+                if getattr(p, "bufpos", None) is not None:
+                    self._filter_positions.append(p.bufpos)
+            plans[j - 1:j] = residual
+            plans[lo:i + 1] = fused
+            j += len(residual) - 1
+        return plans
 
     # ------------------------------------------------------------ build help
     @staticmethod

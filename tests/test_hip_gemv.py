@@ -449,3 +449,70 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     assert g.fuse_lif(prog3, lif3) is None
     prog4 = g.plan_block_gemv(queue, 1.0, dev, [A_js[1]], dev, [X_js[1]], 1.0, dev[[iJ[1]]])
     assert g.fuse_lif(prog4, lif3) is not None
+
+
+def test_gemv_with_filter_epilogue(queue):
+    """GEMV + first-order filters in one launch: every decoded vector and every filter
+    output equals the oracle's GEMV followed by its filter step bit for bit over
+    several steps -- several filters per GEMV item, a pure gain, a filter fed by a
+    small item and a second-order filter (both keep a launch of their own)."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from nengo_ocl_amd import hipra_nonlinearities as nl
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(5)
+    shapes = [(64, 4096), (64, 2048), (100, 300), (16, 8)]
+    n = len(shapes)
+    mats = [rng.normal(scale=0.1, size=s) for s in shapes]
+    xs = [rng.normal(size=s[1]) for s in shapes]
+    outs = [np.zeros(s[0]) for s in shapes]
+    # (GEMV item, denominator, numerator)
+    lowpass = lambda tau: (np.array([-np.exp(-0.001 / tau)]), np.array([1 - np.exp(-0.001 / tau)]))
+    filters = [(0,) + lowpass(0.005), (0,) + lowpass(0.1), (0,) + lowpass(0.02),
+               (1, np.zeros(0), np.array([0.5])), (2,) + lowpass(0.01), (3,) + lowpass(0.01),
+               (0, np.array([-1.2, 0.4]), np.array([0.1, 0.1]))]
+    f_out = [rng.normal(size=shapes[b][0]) for b, _, _ in filters]
+    R = RA(mats + xs + outs + f_out, align=True)
+    iA, iX, iY = (list(range(k * n, (k + 1) * n)) for k in range(3))
+    iF = list(range(3 * n, 3 * n + len(filters)))
+    A_js = [np.array([i], dtype=np.int32) for i in iA]
+    X_js = [np.array([i], dtype=np.int32) for i in iX]
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    # an empty denominator (a pure gain) is a ragged item of shape (0, 1)
+    den = RaggedArray([np.asarray(f[1], dtype=np.float32).reshape(-1, 1) if f[1].size
+                       else np.zeros((0, 1), dtype=np.float32) for f in filters], dtype=np.float32)
+    num = RaggedArray([np.asarray(f[2], dtype=np.float32).reshape(-1, 1) for f in filters],
+                      dtype=np.float32)
+    fx = [iY[b] for b, _, _ in filters]
+    xbuf = RaggedArray([np.zeros((f[2].size, shapes[f[0]][0]), dtype=np.float32) for f in filters],
+                       dtype=np.float32)
+    ybuf = RaggedArray([np.zeros((f[1].size, shapes[f[0]][0]), dtype=np.float32) for f in filters],
+                       dtype=np.float32)
+
+    def build(ra, mod_gemv, mod_nl, q, up):
+        prog = mod_gemv.plan_block_gemv(q, 1.0, ra, A_js, ra, X_js, 0.0, ra[iY])
+        lf = mod_nl.plan_linearfilter(q, ra[fx], ra[iF], up(den), up(num), up(clone(xbuf)),
+                                      up(clone(ybuf)))
+        return prog, lf
+
+    host = clone(R)
+    dev = to_dev(queue, R)
+    prog, lf = build(dev, g, nl, queue, lambda a: to_dev(queue, a))
+    result = g.fuse_linearfilter(prog.plans, lf[0])
+    assert result is not None
+    fused, residual = result
+    assert sorted(p.name for p in fused) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_filter",
+                                              "hipra_gemv.wave_ref"]
+    assert [p.name for p in residual] == ["hip_linearfilter"]
+    oprog, olf = build(host, orc, orc, None, lambda a: a)
+    for step in range(4):
+        for i in iX:  # new inputs every step
+            v = rng.normal(size=R.shape0s[i])
+            dev[i] = v
+            host[i] = v[:, None]
+        for p in fused + residual:
+            p()
+        for p in oprog.plans + olf:
+            p()
+        assert np.array_equal(dev.to_host().buf, host.buf), step

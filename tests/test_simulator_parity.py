@@ -156,6 +156,8 @@ def test_c3_large_reduced_spiking(queue, share):
         # the neurons are updated by the GEMV that computes their input current
         assert any(p.name == "hipra_gemv.tile_lif" for p in gpu._plans)
         assert not any(p.name == "hip_lif" for p in gpu._plans)
+        # and the synapse filters by the GEMV that decodes their input
+        assert any(p.name == "hipra_gemv.tile_filter" for p in gpu._plans)
         check_spiking(gpu, cpu, pg["spikes"], pc["spikes"], 1000, "c3 reduced (8 x 1024 x 64-D)")
 
 
