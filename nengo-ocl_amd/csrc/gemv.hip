@@ -179,7 +179,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
 {
     constexpr int RPP = NHIP_WAVE / LPR;
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
-    const int t = blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6);
+    const int t = blockIdx.x * (NHIP_WG / NHIP_WAVE) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (t >= n_tasks) return;  // wave-uniform; this kernel has no barrier
 
     const GemvTask task = tasks[t];
@@ -235,6 +235,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_ref_kernel(
     const float* __restrict__ A, const float* __restrict__ X, const float* Yin, float* Y)
 {
     constexpr int TILE = 128;
+    constexpr int BATCH = 4;  // dot products whose operands are fetched together
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int t = blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6);
     if (t >= n_tasks) return;  // wave-uniform; this kernel has no barrier
@@ -250,18 +251,52 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_ref_kernel(
         const bool valid = r0 + sub < row_end;
         const int r = valid ? r0 + sub : row_end - 1;
         float sum = cf.y * Yin[it.yin_start + (size_t)r * it.yin_stride0];
-        for (int d = 0; d < it.n_dots; ++d) {
-            const GemvDot dot = dots[it.dot_begin + d];
-            const float* arow = A + dot.a_start + (size_t)r * dot.a_stride0;
-            const float* xg = X + dot.x_start;
-            const size_t xs = (size_t)dot.x_stride0;
-            for (int c0 = 0; c0 < dot.N; c0 += TILE) {
-                const int c1 = min(c0 + TILE, dot.N);
-                float s = 0.0f;
-                for (int c = c0 + lir; c < c1; c += 4) s = fmaf(arow[c], xg[(size_t)c * xs], s);
-                s = s + __shfl_xor(s, 2, NHIP_WAVE);
-                s = s + __shfl_xor(s, 1, NHIP_WAVE);
-                sum = sum + cf.x * s;
+        for (int d0 = 0; d0 < it.n_dots; d0 += BATCH) {
+            // These items are latency bound (a handful of short dot products per row):
+            // the records of a batch are read together, and when every dot product of
+            // the batch has at most four columns -- one element per lane, the common
+            // "scalar times vector" increments -- so are all their operands, before the
+            // sums are formed in the usual order.
+            GemvDot dot[BATCH];
+            bool tiny = true;
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                dot[k] = dots[it.dot_begin + min(d0 + k, it.n_dots - 1)];
+                tiny = tiny && dot[k].N <= 4;
+            }
+            if (tiny) {
+                float a[BATCH], x[BATCH];
+#pragma unroll
+                for (int k = 0; k < BATCH; ++k) {
+                    const bool live = d0 + k < it.n_dots && lir < dot[k].N;
+                    a[k] = live ? A[dot[k].a_start + (size_t)r * dot[k].a_stride0 + lir] : 0.0f;
+                    x[k] = live ? X[dot[k].x_start + (size_t)lir * dot[k].x_stride0] : 0.0f;
+                }
+#pragma unroll
+                for (int k = 0; k < BATCH; ++k) {
+                    if (d0 + k < it.n_dots) {  // uniform
+                        float s = lir < dot[k].N ? fmaf(a[k], x[k], 0.0f) : 0.0f;
+                        s = s + __shfl_xor(s, 2, NHIP_WAVE);
+                        s = s + __shfl_xor(s, 1, NHIP_WAVE);
+                        sum = sum + cf.x * s;
+                    }
+                }
+                continue;
+            }
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {  // static indices keep the records in registers
+                if (d0 + k >= it.n_dots) break;
+                const float* arow = A + dot[k].a_start + (size_t)r * dot[k].a_stride0;
+                const float* xg = X + dot[k].x_start;
+                const size_t xs = (size_t)dot[k].x_stride0;
+                for (int c0 = 0; c0 < dot[k].N; c0 += TILE) {
+                    const int c1 = min(c0 + TILE, dot[k].N);
+                    float s = 0.0f;
+                    for (int c = c0 + lir; c < c1; c += 4) s = fmaf(arow[c], xg[(size_t)c * xs], s);
+                    s = s + __shfl_xor(s, 2, NHIP_WAVE);
+                    s = s + __shfl_xor(s, 1, NHIP_WAVE);
+                    sum = sum + cf.x * s;
+                }
             }
         }
         if (lir == 0 && valid) Y[it.y_start + (size_t)r * it.y_stride0] = sum + cf.z;
