@@ -4,15 +4,18 @@
 ``python bench.py --gpus 1 --steps K --warmup W`` builds the large
 bandwidth-bound network (256 ensembles x 4096 LIF neurons x 64-D, 1,048,576
 neurons; `nengo_ocl_amd.configs.c3_large`), runs W untimed steps, then times
-exactly K steps of ``Simulator.run_steps`` (graph replay, probes drained every
-32 steps) between stream synchronisations and prints ONE JSON line:
+exactly K steps of ``Simulator.run_steps`` (replays of a recorded graph that holds
+16 steps; probe buffers are drained when full, here every 4096 steps) between
+stream synchronisations and prints ONE JSON line:
 
 * ``value``: simulator steps per second (inputs resident in HBM);
 * ``roofline``: for the dominant kernel (the ragged gather-GEMV launch with the
   largest share of the step), algorithmic bytes per launch (the reference's own
-  accounting: A + X per dot, Y_in, Y) divided by its average duration, measured
-  with HIP events on the simulator's stream in a separate eager pass over the
-  same state, against the 8 TB/s HBM peak;
+  accounting: A + X per dot, Y_in, Y; plus the state its epilogue reads and
+  writes) divided by its average duration, measured with HIP events on the
+  simulator's stream in a separate eager pass over the same state, against the
+  8 TB/s HBM peak; ``traffic`` is the HBM traffic per launch the hardware
+  counters showed for that kernel (profiles/c3_shared_step.txt);
 * ``cpu_baseline``: the CPU oracle (C restatement of the reference kernels,
   OpenMP) stepping the same network on the host cores for a bounded sample.
 
@@ -73,6 +76,22 @@ def gemv_summary(sim, profile_steps):
                              bytes=p.bw_per_call,
                              gbs=(1e-9 * p.bw_per_call / avg) if p.bw_per_call and avg > 0 else None))
     return rows
+
+
+def measured_traffic(plan_name):
+    """HBM bytes per launch of the dominant kernel, from the counter runs summarised in
+    profiles/c3_shared_step.txt (FETCH_SIZE and WRITE_SIZE, scaled by what the same
+    counters read for a plain copy of known size).  None for other workloads."""
+    kernel = {"hipra_gemv.tile_lif": "gemv_tile_p2_kernel<1>",
+              "hipra_gemv.tile_filter": "gemv_tile_p2_kernel<2>"}.get(plan_name)
+    path = os.path.join(ROOT, "profiles", "c3_shared_step.txt")
+    if kernel is None or not os.path.exists(path):
+        return None
+    for line in open(path):
+        parts = line.split()
+        if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == kernel:
+            return float(parts[2])
+    return None
 
 
 def cpu_baseline(config, variant, scale, budget_s, dt_gpu_step):
@@ -170,8 +189,11 @@ def main():
     gemv_us = sum(r["avg_us"] for r in gemv_rows)
     roofline = None
     if dom is not None:
+        traffic = None
+        if args.config == "c3" and args.variant == "shared" and args.scale == 1.0:
+            traffic = measured_traffic(dom["name"])
         roofline = dict(bound="hbm", achieved=dom["gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
-                        frac=dom["gbs"] / HBM_PEAK_GBS, traffic=None, kernel=dom["plan"],
+                        frac=dom["gbs"] / HBM_PEAK_GBS, traffic=traffic, kernel=dom["plan"],
                         avg_us=dom["avg_us"], bytes_per_launch=dom["bytes"])
 
     out = {
