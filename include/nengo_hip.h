@@ -103,9 +103,14 @@ int nhip_gemv_tile_rows(int n_cols, int blk_words);
  * `plan_block_gemv` (clra_gemv.py:1193-1195) + `plan_lif`
  * (clra_nonlinearities.py:1028-1146) when the GEMV output is the neurons' input
  * current.  Row r of item b is the current of neuron r of population b:
- *   pops : int32[n_items][8] {v_start, w_start, s_start, enabled, tau, ref, amp, pflags}
+ *   pops : int32[n_items][8] {v_start, w_start, s_start, decay, tau, ref, amp, pflags}
  * (tau / ref / amp: float bits, or with bit 0/1/2 of pflags set the element offset
- * of a per-neuron vector in TAU / REF / AMP; items with enabled == 0 only get Y).
+ * of a per-neuron vector in TAU / REF / AMP; bit 8 of pflags: the item has a
+ * population -- items without it only get Y; bit 9: `decay` holds the float bits of
+ * -expm1(-dt / tau) formed as the kernel would (float quotient, expm1 in double,
+ * rounded once to float), allowed when tau is a scalar and upsample == 1: the
+ * launch then evaluates transcendental functions only for the few neurons that
+ * leave their refractory period or spike in this step).
  * Y is still written.  V, W, S must not overlap anything the launch reads through
  * A, X or Yin; dt, upsample as for nhip_lif.  Results are bit-identical to the two
  * separate calls. */

@@ -46,6 +46,8 @@ constexpr int MAX_CHAIN = TILE / 4;  // elements of one partial sum: 32
 constexpr int X_PF = STAGE_COLS / NHIP_WAVE;  // gathered X elements per lane and column stage
 constexpr int XBLK_WORDS = (STAGE_COLS / TILE) * TILE_LDS;  // X block of a wave in LDS
 constexpr int ROW_SLOTS = 4;       // row sums per lane: a task covers <= 256 rows
+constexpr int MAX_TASK_ROWS = ROW_SLOTS * NHIP_WAVE;
+constexpr int LIF_QUEUE_WORDS = 7 * MAX_TASK_ROWS;  // LDS words of lif_task_compacted's queues
 
 typedef float tile_f4 __attribute__((ext_vector_type(4)));
 
@@ -325,7 +327,11 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
         if (r < n_rows) {
             const float y = sum[k] + cf.z;
             if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
-            if (EPI == EPI_LIF && pop.enabled) lif_epilogue(epi.lif, pop, task.row0 + r, y);
+            if (EPI == EPI_LIF && (pop.pflags & LIF_POP_ENABLED)) {
+                const int i = task.row0 + r;
+                lif_epilogue(epi.lif, pop, i, y, epi.lif.V[(size_t)pop.v_start + i],
+                             epi.lif.W[(size_t)pop.w_start + i]);
+            }
             if (EPI == EPI_FILTER) filter_epilogue(epi.filter, filters, task.row0 + r, y);
         }
     }
@@ -337,6 +343,107 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
 // mask of wave-uniform values, stages and tiles are always full, and a block is at
 // most 8 loads per lane.  This is the streaming path of the big encoder / decoder
 // matrices; its instruction count per byte is a fraction of the general kernel's.
+// LIF update of all rows of a task by one wave, for a population with one time
+// constant and no sub-steps.  The update of a neuron needs a transcendental function
+// only in two rare cases: expm1 when the neuron leaves its refractory period inside
+// the step (the integration time is then neither the whole step, whose decay factor
+// comes precomputed with the population, nor zero), and log1p when it spikes.  A
+// wave executes a branch for all 64 lanes as soon as one lane takes it, and with a
+// few per cent of the neurons in each case almost every wave would pay for both
+// double-precision evaluations.  So the rare cases of the whole task are queued in
+// LDS (`queue`: the wave's stage block, free by now) and evaluated densely
+// afterwards.  Operation by operation this is `lif_step` (same inputs, same rounded
+// operations), so the results are identical.
+__device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPop& p, int row0,
+                                                   int n_rows, const float* ys, float gamma,
+                                                   float* y_out, int y_stride0, float* queue,
+                                                   int lane, const float (&v_in)[ROW_SLOTS],
+                                                   const float (&w_in)[ROW_SLOTS]) {
+    const float tau = nhip_bits(p.tau);
+    const float decay = nhip_bits(p.decay);
+    const float dtu = a.dtu;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    float* leaving = queue;                     // {neuron, integration time, j, v} x n_rows
+    float* spiking = queue + 4 * MAX_TASK_ROWS;  // {neuron, j, v} x n_rows
+    int n_leaving = 0, n_spiking = 0;           // wave-uniform
+
+    auto push_spike = [&](bool want, int i, float j, float v) {
+        const unsigned long long m = __ballot(want);
+        if (want) {
+            float* e = spiking + 3 * (n_spiking + __popcll(m & below));
+            e[0] = __int_as_float(i);
+            e[1] = j;
+            e[2] = v;
+        }
+        n_spiking += __popcll(m);
+    };
+    // voltage step with a known decay factor; queues the neuron if it spikes
+    auto integrate = [&](bool live, int i, float j, float v, float factor) {
+        const float dv = __fmul_rn(factor, j - v);
+        v = __fadd_rn(v, dv);
+        const bool fired = live && v > 1.0f;
+        push_spike(fired, i, j, v);
+        if (live && !fired) {
+            a.V[(size_t)p.v_start + i] = v < 0.0f ? 0.0f : v;
+            a.S[(size_t)p.s_start + i] = 0.0f;
+        }
+    };
+
+#pragma unroll
+    for (int k = 0; k < ROW_SLOTS; ++k) {
+        if (k * NHIP_WAVE >= n_rows) break;  // uniform
+        const int r = k * NHIP_WAVE + lane;
+        const bool live = r < n_rows;
+        const int i = row0 + (live ? r : 0);
+        float j = 0.0f, v = 0.0f, w = 0.0f;
+        if (live) {
+            j = ys[r] + gamma;
+            if (y_out) y_out[(size_t)i * y_stride0] = j;
+            v = v_in[k];
+            w = w_in[k] - dtu;
+        }
+        const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
+        const bool whole = delta_t == dtu, none = delta_t == 0.0f;
+        const bool partial = live && !whole && !none;
+        const unsigned long long m = __ballot(partial);
+        if (partial) {
+            float* e = leaving + 4 * (n_leaving + __popcll(m & below));
+            e[0] = __int_as_float(i);
+            e[1] = delta_t;
+            e[2] = j;
+            e[3] = v;
+        }
+        n_leaving += __popcll(m);
+        if (live) a.W[(size_t)p.w_start + i] = w;  // a spike overwrites it below
+        // integration over no time leaves the voltage as it is (the factor is +0)
+        if (live && none) a.S[(size_t)p.s_start + i] = 0.0f;
+        integrate(live && whole, i, j, v, decay);
+    }
+    wave_sync();
+    for (int e0 = 0; e0 < n_leaving; e0 += NHIP_WAVE) {
+        const bool live = e0 + lane < n_leaving;
+        const float* e = leaving + 4 * (live ? e0 + lane : 0);
+        const int i = __float_as_int(e[0]);
+        const float factor = -(float)expm1((double)__fdiv_rn(-e[1], tau));
+        integrate(live, i, e[2], e[3], factor);
+    }
+    wave_sync();
+    for (int e0 = 0; e0 < n_spiking; e0 += NHIP_WAVE) {
+        if (e0 + lane < n_spiking) {
+            const float* e = spiking + 3 * (e0 + lane);
+            const int i = __float_as_int(e[0]);
+            const float j = e[1], v = e[2];
+            const float ref = lif_param(p.ref, p.pflags & 2, a.REF, i);
+            const float amp = lif_param(p.amp, p.pflags & 4, a.AMP, i);
+            const float t_spike = __fadd_rn(
+                dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
+            a.V[(size_t)p.v_start + i] = 0.0f;
+            a.W[(size_t)p.w_start + i] = ref + t_spike;
+            a.S[(size_t)p.s_start + i] = __fmul_rn(amp, a.dt_inv);
+        }
+    }
+}
+
 constexpr int P2_PF = 8;         // 16-byte loads per lane and block
 constexpr int YSUM_WORDS = 256;  // running sums of the task's rows, in LDS
 
@@ -385,6 +492,24 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
         const int r = lane + k * NHIP_WAVE;
         if (r < n_rows)
             ys[r] = cf.y * Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0];
+    }
+    // What the epilogue will need of the item besides its sums is requested now, so
+    // that it has arrived when the last block is done (read at the end, these loads
+    // would stall the wave for a memory round trip with nothing else in flight).
+    LifPop pop = {};
+    float v_in[ROW_SLOTS] = {}, w_in[ROW_SLOTS] = {};
+    if (EPI == EPI_LIF) {
+        pop = epi.lif.pops[task.item];
+        if (pop.pflags & LIF_POP_ENABLED) {
+#pragma unroll
+            for (int k = 0; k < ROW_SLOTS; ++k) {
+                const int r = lane + k * NHIP_WAVE;
+                if (r < n_rows) {
+                    v_in[k] = epi.lif.V[(size_t)pop.v_start + task.row0 + r];
+                    w_in[k] = epi.lif.W[(size_t)pop.w_start + task.row0 + r];
+                }
+            }
+        }
     }
 
     auto first_stage = [&]() {
@@ -548,21 +673,25 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     }
 
     wave_sync();
-    LifPop pop = {};
     int2 filters = make_int2(0, 0);
-    if (EPI == EPI_LIF) pop = epi.lif.pops[task.item];
     if (EPI == EPI_FILTER) filters = epi.filter.item_targets[task.item];
     // an item without dot products that would copy Y onto itself unchanged is only
     // there for its epilogue (a constant input current): nothing to store
     const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
                            it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
+    if (EPI == EPI_LIF && (pop.pflags & LIF_POP_DECAY)) {
+        lif_task_compacted(epi.lif, pop, task.row0, n_rows, ys, cf.z,
+                           store_y ? Y + it.y_start : nullptr, it.y_stride0, ab, lane, v_in, w_in);
+        return;
+    }
 #pragma unroll
     for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
         const int r = lane + k * NHIP_WAVE;
         if (r < n_rows) {
             const float y = ys[r] + cf.z;
             if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
-            if (EPI == EPI_LIF && pop.enabled) lif_epilogue(epi.lif, pop, task.row0 + r, y);
+            if (EPI == EPI_LIF && (pop.pflags & LIF_POP_ENABLED))
+                lif_epilogue(epi.lif, pop, task.row0 + r, y, v_in[k], w_in[k]);
             if (EPI == EPI_FILTER) filter_epilogue(epi.filter, filters, task.row0 + r, y);
         }
     }
@@ -593,6 +722,9 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     const size_t wave_words = (size_t)blk_words + TSUM_WORDS + XBLK_WORDS + (pow2_cols ? YSUM_WORDS : 0);
     const size_t lds_bytes = sizeof(float) * waves * wave_words;
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
+    // the LIF epilogue queues its rare cases in the stage block and what follows it
+    if (epilogue == EPI_LIF && pow2_cols && blk_words + TSUM_WORDS + XBLK_WORDS < LIF_QUEUE_WORDS)
+        return NHIP_E_BADARG;
     const int n_groups = (n_tasks + waves - 1) / waves;
     hipStream_t s = static_cast<hipStream_t>(stream);
     auto launch = [&](auto kernel) {

@@ -7,9 +7,12 @@
 // offsets of its state, and its parameters as float bits or (pflags bit set) as the
 // element offset of a per-neuron vector.
 struct LifPop {
-    int v_start, w_start, s_start, enabled;
+    int v_start, w_start, s_start;
+    int decay;                  // float bits of -expm1(-dtu / tau), valid with LIF_POP_DECAY
     int tau, ref, amp, pflags;  // bit 0/1/2 of pflags: tau/ref/amp is a per-neuron vector
 };
+constexpr int LIF_POP_ENABLED = 1 << 8;  // pflags: the item has a population at all
+constexpr int LIF_POP_DECAY = 1 << 9;    // pflags: `decay` is set (one tau, upsample == 1)
 
 // State arrays and constants of a fused LIF update (all populations of a launch).
 struct LifArgs {
@@ -58,10 +61,10 @@ __device__ __forceinline__ bool lif_step(float j, float& v, float& w, float tau,
     return spiked;
 }
 
-// LIF update of neuron i of population p with input current j (GEMV epilogue)
-__device__ __forceinline__ void lif_epilogue(const LifArgs& a, const LifPop& p, int i, float j) {
-    float v = a.V[(size_t)p.v_start + i];
-    float w = a.W[(size_t)p.w_start + i];
+// LIF update of neuron i of population p with input current j (GEMV epilogue);
+// v and w are the neuron's voltage and refractory time, read earlier
+__device__ __forceinline__ void lif_epilogue(const LifArgs& a, const LifPop& p, int i, float j,
+                                             float v, float w) {
     const float tau = lif_param(p.tau, p.pflags & 1, a.TAU, i);
     const float ref = lif_param(p.ref, p.pflags & 2, a.REF, i);
     const float amp = lif_param(p.amp, p.pflags & 4, a.AMP, i);

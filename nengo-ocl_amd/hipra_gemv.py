@@ -37,6 +37,8 @@ MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
 WG, WAVE = 256, 64
+LIF_POP_ENABLED, LIF_POP_DECAY = 1 << 8, 1 << 9  # flag bits of a population row
+LIF_COMPACT = os.environ.get("NENGO_HIP_LIF_COMPACT", "1") != "0"
 
 
 def flops_from_geometry(geometry, items):
@@ -484,8 +486,20 @@ def fuse_lif(prog, lif_plan):
     cols, pptrs, keep = lif_population_table(queue, spec)
     table = np.zeros((len(Y), 8), dtype=np.int32)
     for p, b in matched:
-        table[b] = (cols["v_start"][p], cols["w_start"][p], cols["s_start"][p], 1,
-                    cols["tau"][p], cols["ref"][p], cols["amp"][p], cols["pflags"][p])
+        flags = int(cols["pflags"][p]) | LIF_POP_ENABLED
+        decay_bits = 0
+        if not (flags & 1) and spec["upsample"] == 1 and LIF_COMPACT:
+            # one time constant and no sub-steps: the decay factor of a whole step,
+            # -expm1(-dt / tau) with the kernel's roundings (float quotient, expm1 in
+            # double, rounded once), is the same for every neuron that is not refractory
+            tau = np.int32(cols["tau"][p]).view(np.float32)
+            dtu = np.float32(spec["dt"] / float(spec["upsample"]))
+            quotient = np.float32(-dtu) / tau
+            decay = np.float32(-np.float32(np.expm1(np.float64(quotient))))
+            decay_bits = int(decay.view(np.int32))
+            flags |= LIF_POP_DECAY
+        table[b] = (cols["v_start"][p], cols["w_start"][p], cols["s_start"][p], decay_bits,
+                    cols["tau"][p], cols["ref"][p], cols["amp"][p], flags)
     dev_pops = to_device(queue, table)
     lif_args = (dev_pops.ptr, spec["dt"], spec["upsample"], V.ptr, W.ptr, S.ptr,
                 pptrs[0], pptrs[1], pptrs[2])
