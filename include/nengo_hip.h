@@ -151,6 +151,33 @@ int nhip_lif(void *stream, const int *desc, int n_blocks, double dt, int upsampl
  *   desc : int32[n_blocks][8] {j_start, r_start, count, tau, ref, amp, pflags, 0} */
 int nhip_lif_rate(void *stream, const int *desc, int n_blocks, const float *J, float *R,
                   const float *TAU, const float *REF, const float *AMP);
+/* The other neuron types share one work-list row per block of one population:
+ *   desc : int32[n_blocks][16] {j_start, out_start, v_start, w_start, n_start, count,
+ *                               pflags, 0, p0, p1, p2, p3, p4, 0, 0, 0}
+ * p0.. are the type's parameters in the order of its pointer arguments, as float
+ * bits or (bit k of pflags set) element offsets of per-neuron vectors; offsets of
+ * arrays a type does not use are ignored.
+ * Adaptive LIF: the LIF update on J - N, then N += (dt / tau_n) (inc_n S - N);
+ * parameters tau, ref, amp, tau_n, inc_n.  replaces: `plan_lif` with N, tau_n, inc_n
+ * (:1028-1146). */
+int nhip_alif(void *stream, const int *desc, int n_blocks, double dt, int upsample,
+              const float *J, float *V, float *W, float *S, float *N, const float *TAU,
+              const float *REF, const float *AMP, const float *TAU_N, const float *INC_N);
+/* Adaptive LIF rate.  replaces: `plan_lif_rate` with N, tau_n, inc_n (:1149-1197). */
+int nhip_alif_rate(void *stream, const int *desc, int n_blocks, double dt, const float *J,
+                   float *R, float *N, const float *TAU, const float *REF, const float *AMP,
+                   const float *TAU_N, const float *INC_N);
+/* R = amp max(J, 0).  replaces: `plan_rectified_linear` (:1238-1258). */
+int nhip_relu(void *stream, const int *desc, int n_blocks, const float *J, float *R,
+              const float *AMP);
+/* V += dt max(J, 0); spikes = floor(V); V -= spikes; S = amp spikes / dt.
+ * replaces: `plan_spiking_rectified_linear` (:1200-1235). */
+int nhip_spiking_relu(void *stream, const int *desc, int n_blocks, double dt, const float *J,
+                      float *V, float *S, const float *AMP);
+/* R = 1 / (ref (1 + exp(-J))), 0 below J = -88, 1 / ref above J = 15.
+ * replaces: `plan_sigmoid` (:1261-1283). */
+int nhip_sigmoid(void *stream, const int *desc, int n_blocks, const float *J, float *R,
+                 const float *REF);
 
 /* ---- synapses ----------------------------------------------------------
  * Direct-form linear filter step  y <- sum_p b[p] x[n-p] - sum_p a[p] y[n-1-p]

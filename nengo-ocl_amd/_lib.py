@@ -34,6 +34,11 @@ SIGNATURES = {
     "nhip_gemv_tile_rows": [c_int, c_int],
     "nhip_lif": [P, P, c_int, c_double, c_int, P, P, P, P, P, P, P],
     "nhip_lif_rate": [P, P, c_int, P, P, P, P, P],
+    "nhip_alif": [P, P, c_int, c_double, c_int, P, P, P, P, P, P, P, P, P, P],
+    "nhip_alif_rate": [P, P, c_int, c_double, P, P, P, P, P, P, P, P],
+    "nhip_relu": [P, P, c_int, P, P, P],
+    "nhip_spiking_relu": [P, P, c_int, c_double, P, P, P, P],
+    "nhip_sigmoid": [P, P, c_int, P, P, P],
     "nhip_linearfilter": [P, P, P, c_int, P, P, P, P, P, P],
     "nhip_elementwise_inc": [P, P, c_int, P, P, P],
     "nhip_copy": [P, P, c_int, P, P],

@@ -395,7 +395,9 @@ def _check_vectors(ras):
 def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, N=None, tau_n=None, inc_n=None,
              upsample=1, fastlif=False, tag=None, **kwargs):
     if N is not None or tau_n is not None or inc_n is not None:
-        raise NotImplementedError("adaptive LIF")
+        if fastlif:
+            raise NotImplementedError("fastlif approximation")
+        return _plan_alif(queue, dt, J, V, W, outS, ref, tau, amp, N, tau_n, inc_n, upsample, tag)
     if fastlif:
         raise NotImplementedError("fastlif approximation")
     assert J.ctype == "float"
@@ -442,7 +444,7 @@ def lif_population_table(queue, spec):
 def plan_lif_rate(queue, dt, J, R, ref, tau, amp, N=None, tau_n=None, inc_n=None, tag=None,
                   **kwargs):
     if N is not None or tau_n is not None or inc_n is not None:
-        raise NotImplementedError("adaptive LIF rate")
+        return _plan_alif_rate(queue, dt, J, R, ref, tau, amp, N, tau_n, inc_n, tag)
     assert J.ctype == "float"
     assert R.ctype == J.ctype
     _check_vectors([J, R])
@@ -458,6 +460,108 @@ def plan_lif_rate(queue, dt, J, R, ref, tau, amp, N=None, tau_n=None, inc_n=None
                 full_args=(table, J.dev_buf, R.dev_buf) + tuple(keep), name="hip_lif_rate",
                 tag=tag)
     plan.bw_per_call = J.nbytes + R.nbytes + bin(pflags).count("1") * J.nbytes
+    plan.description = _description(J)
+    return plan
+
+
+# ---------------------------------------------------------------- further neuron types
+def _neuron_table(queue, J, out, params, V=None, W=None, N=None):
+    """Work list {j, out, v, w, n offsets, count, pflags, 0, p0..p4, 0, 0, 0} of the neuron
+    kernels that share `NeuronDesc` (one row per block of <= 512 neurons)."""
+    inds, offsets, counts = blockify(J.shape0s, 2 * WG)
+    pcols, pflags, pptrs, keep = _neuron_params(queue, params, J.shape0s, inds, offsets)
+    zeros = np.zeros(len(inds), dtype=np.int32)
+    start = lambda ra: zeros if ra is None else ra.starts[inds] + offsets
+    columns = [start(J), start(out), start(V), start(W), start(N), counts,
+               np.full(len(inds), pflags, dtype=np.int32), zeros]
+    columns += pcols + [zeros] * (8 - len(pcols))
+    table, n = _dev_table(queue, columns, 16)
+    n_vec = bin(pflags).count("1")
+    return table, n, pptrs, keep, n_vec
+
+
+def _plan_alif(queue, dt, J, V, W, outS, ref, tau, amp, N, tau_n, inc_n, upsample, tag):
+    """Adaptive LIF (clra_nonlinearities.py `plan_lif` with N, tau_n, inc_n, :1028-1146)."""
+    assert all(x is not None for x in [N, tau_n, inc_n])
+    assert J.ctype == "float"
+    for x in [V, W, outS, N]:
+        assert x.ctype == J.ctype
+    _check_vectors([J, V, W, outS, N])
+    _check(("J", J), ("V", V), ("W", W), ("outS", outS), ("N", N), ("tau", tau), ("ref", ref),
+           ("amp", amp), ("tau_n", tau_n), ("inc_n", inc_n))
+    table, n, pp, keep, n_vec = _neuron_table(queue, J, outS, [tau, ref, amp, tau_n, inc_n],
+                                              V=V, W=W, N=N)
+    args = (table.ptr, n, float(dt), int(upsample), J.ptr, V.ptr, W.ptr, outS.ptr, N.ptr,
+            pp[0], pp[1], pp[2], pp[3], pp[4])
+    plan = Plan(queue, queue.lib.nhip_alif, args, gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, J.dev_buf, V.dev_buf, W.dev_buf, outS.dev_buf, N.dev_buf)
+                + tuple(keep), name="hip_alif", tag=tag)
+    plan.bw_per_call = (J.nbytes + 2 * V.nbytes + 2 * W.nbytes + 2 * N.nbytes + outS.nbytes
+                        + n_vec * J.nbytes)
+    plan.description = _description(J)
+    return plan
+
+
+def _plan_alif_rate(queue, dt, J, R, ref, tau, amp, N, tau_n, inc_n, tag):
+    """Adaptive LIF rate (`plan_lif_rate` with N, tau_n, inc_n, :1149-1197)."""
+    assert all(x is not None for x in [N, tau_n, inc_n])
+    assert J.ctype == "float" and R.ctype == J.ctype and N.ctype == J.ctype
+    _check_vectors([J, R, N])
+    _check(("J", J), ("R", R), ("N", N), ("tau", tau), ("ref", ref), ("amp", amp),
+           ("tau_n", tau_n), ("inc_n", inc_n))
+    table, n, pp, keep, n_vec = _neuron_table(queue, J, R, [tau, ref, amp, tau_n, inc_n], N=N)
+    args = (table.ptr, n, float(dt), J.ptr, R.ptr, N.ptr, pp[0], pp[1], pp[2], pp[3], pp[4])
+    plan = Plan(queue, queue.lib.nhip_alif_rate, args, gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, J.dev_buf, R.dev_buf, N.dev_buf) + tuple(keep),
+                name="hip_alif_rate", tag=tag)
+    plan.bw_per_call = J.nbytes + R.nbytes + 2 * N.nbytes + n_vec * J.nbytes
+    plan.description = _description(J)
+    return plan
+
+
+def plan_rectified_linear(queue, J, R, amp, tag=None, **kwargs):
+    """``R = amp * max(J, 0)`` (clra_nonlinearities.py:1238-1258)."""
+    assert J.ctype == "float" and R.ctype == J.ctype
+    _check_vectors([J, R])
+    _check(("J", J), ("R", R), ("amp", amp))
+    table, n, pp, keep, n_vec = _neuron_table(queue, J, R, [amp])
+    plan = Plan(queue, queue.lib.nhip_relu, (table.ptr, n, J.ptr, R.ptr, pp[0]),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, J.dev_buf, R.dev_buf) + tuple(keep), name="hip_relu", tag=tag)
+    plan.bw_per_call = J.nbytes + R.nbytes + n_vec * J.nbytes
+    plan.description = _description(J)
+    return plan
+
+
+def plan_spiking_rectified_linear(queue, dt, J, V, outS, amp, tag=None, **kwargs):
+    """``V += dt * max(J, 0); n = floor(V); V -= n; S = amp * n / dt``
+    (clra_nonlinearities.py:1200-1235)."""
+    assert J.ctype == "float"
+    for x in [V, outS]:
+        assert x.ctype == J.ctype
+    _check_vectors([J, V, outS])
+    _check(("J", J), ("V", V), ("outS", outS), ("amp", amp))
+    table, n, pp, keep, n_vec = _neuron_table(queue, J, outS, [amp], V=V)
+    plan = Plan(queue, queue.lib.nhip_spiking_relu,
+                (table.ptr, n, float(dt), J.ptr, V.ptr, outS.ptr, pp[0]),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, J.dev_buf, V.dev_buf, outS.dev_buf) + tuple(keep),
+                name="hip_spikingrelu", tag=tag)
+    plan.bw_per_call = J.nbytes + 2 * V.nbytes + outS.nbytes + n_vec * J.nbytes
+    plan.description = _description(J)
+    return plan
+
+
+def plan_sigmoid(queue, J, R, ref, tag=None, **kwargs):
+    """``R = 1 / (ref * (1 + exp(-J)))`` with the cut-offs of clra_nonlinearities.py:1261-1283."""
+    assert J.ctype == "float" and R.ctype == J.ctype
+    _check_vectors([J, R])
+    _check(("J", J), ("R", R), ("ref", ref))
+    table, n, pp, keep, n_vec = _neuron_table(queue, J, R, [ref])
+    plan = Plan(queue, queue.lib.nhip_sigmoid, (table.ptr, n, J.ptr, R.ptr, pp[0]),
+                gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=(table, J.dev_buf, R.dev_buf) + tuple(keep), name="hip_sigmoid", tag=tag)
+    plan.bw_per_call = J.nbytes + R.nbytes + n_vec * J.nbytes
     plan.description = _description(J)
     return plan
 

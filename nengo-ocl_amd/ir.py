@@ -281,6 +281,64 @@ class LIF(LIFRate):
         self.min_voltage = min_voltage
 
 
+class AdaptiveLIFRate(LIFRate):
+    """LIF rate with an adaptation state N: J_eff = J - N, N += (dt/tau_n)(inc_n r - N)."""
+
+    def __init__(self, tau_n=1.0, inc_n=0.01, tau_rc=0.02, tau_ref=0.002, amplitude=1.0):
+        super().__init__(tau_rc, tau_ref, amplitude)
+        self.tau_n, self.inc_n = float(tau_n), float(inc_n)
+
+
+class AdaptiveLIF(LIF):
+    def __init__(self, tau_n=1.0, inc_n=0.01, tau_rc=0.02, tau_ref=0.002, min_voltage=0,
+                 amplitude=1.0):
+        super().__init__(tau_rc, tau_ref, min_voltage, amplitude)
+        self.tau_n, self.inc_n = float(tau_n), float(inc_n)
+
+
+class RectifiedLinear(LIFRate):
+    """r = amplitude * max(J, 0); silent at the intercept, max_rate at x = 1."""
+
+    def __init__(self, amplitude=1.0):
+        self.amplitude = float(amplitude)
+
+    def rates_from_current(self, J):
+        return self.amplitude * np.maximum(np.asarray(J, dtype=np.float64), 0.0)
+
+    def gain_bias(self, max_rates, intercepts):
+        max_rates = np.asarray(max_rates, dtype=np.float64)
+        intercepts = np.asarray(intercepts, dtype=np.float64)
+        gain = max_rates / (1 - intercepts)
+        bias = -intercepts * gain
+        return gain, bias
+
+
+class SpikingRectifiedLinear(RectifiedLinear):
+    """Integrates max(J, 0) and emits floor(V) spikes per step."""
+
+
+class Sigmoid(LIFRate):
+    """r = 1 / (tau_ref (1 + exp(-J))); the intercept is the inflection point."""
+
+    def __init__(self, tau_ref=0.0025):
+        self.tau_ref = float(tau_ref)
+        self.amplitude = 1.0
+
+    def rates_from_current(self, J):
+        return 1.0 / (self.tau_ref * (1.0 + np.exp(-np.asarray(J, dtype=np.float64))))
+
+    def gain_bias(self, max_rates, intercepts):
+        max_rates = np.asarray(max_rates, dtype=np.float64)
+        intercepts = np.asarray(intercepts, dtype=np.float64)
+        lim = 1.0 / self.tau_ref
+        if np.any(max_rates >= lim):
+            raise ValueError("max_rates must be below 1/tau_ref")
+        inverse = -np.log(lim / max_rates - 1.0)
+        gain = inverse / (1.0 - intercepts)
+        bias = inverse - gain
+        return gain, bias
+
+
 # ============================================================== processes
 class Process:
     seed = None

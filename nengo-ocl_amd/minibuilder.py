@@ -28,7 +28,9 @@ and one filter (what a passthrough node after the ensemble gives in nengo).
 import numpy as np
 
 from . import ir
-from .ir import LIF, Alpha, LIFRate, LinearFilter, Lowpass, PresentInput, WhiteSignal  # noqa: F401
+from .ir import (LIF, AdaptiveLIF, AdaptiveLIFRate, Alpha, LIFRate, LinearFilter,  # noqa: F401
+                 Lowpass, PresentInput, RectifiedLinear, Sigmoid, SpikingRectifiedLinear,
+                 WhiteSignal)
 
 
 class _Sliceable:
@@ -222,11 +224,12 @@ class Network:
         model.add_op(ir.Reset(sig["in"]))
         model.add_op(ir.Copy(nsig["bias"], nsig["in"]))
         model.add_op(ir.DotInc(sig["encoders"], sig["in"], nsig["in"], tag="%s encoding" % name))
-        if type(ens.neuron_type).__name__ == "LIF":
-            state = {"voltage": ir.Signal(np.zeros(n), name="%s.voltage" % name),
-                     "refractory_time": ir.Signal(np.zeros(n), name="%s.refractory_time" % name)}
-        else:
-            state = {}
+        state_names = {"LIF": ("voltage", "refractory_time"),
+                       "AdaptiveLIF": ("voltage", "refractory_time", "adaptation"),
+                       "AdaptiveLIFRate": ("adaptation",),
+                       "SpikingRectifiedLinear": ("voltage",)}
+        state = {key: ir.Signal(np.zeros(n), name="%s.%s" % (name, key))
+                 for key in state_names.get(type(ens.neuron_type).__name__, ())}
         model.add_op(ir.SimNeurons(ens.neuron_type, nsig["in"], nsig["out"], state=state))
 
     def _build_node(self, model, node, rng):

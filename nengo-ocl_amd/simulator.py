@@ -65,7 +65,8 @@ class HipBackend:
         self._ra = hipraggedarray
         for name in ("plan_timeupdate", "plan_reset", "plan_copy", "plan_slicedcopy",
                      "plan_elementwise_inc", "plan_linearfilter", "plan_probes", "plan_direct",
-                     "plan_lif", "plan_lif_rate", "plan_presentinput"):
+                     "plan_lif", "plan_lif_rate", "plan_presentinput", "plan_rectified_linear",
+                     "plan_spiking_rectified_linear", "plan_sigmoid"):
             setattr(self, name, getattr(hipra_nonlinearities, name))
         self.plan_block_gemv = hipra_gemv.plan_block_gemv
         self._fuse_lif = hipra_gemv.fuse_lif
@@ -833,6 +834,49 @@ class Simulator:
         tau = np.array([op.neurons.tau_rc for op in ops], dtype=np.float32)
         amp = np.array([op.neurons.amplitude for op in ops], dtype=np.float32)
         return [self.backend.plan_lif_rate(self.queue, self.model.dt, J, R, ref, tau, amp)]
+
+    def _per_population(self, ops, attr):
+        return np.array([getattr(op.neurons, attr) for op in ops], dtype=np.float32)
+
+    def _plan_AdaptiveLIF(self, ops):
+        if not all(getattr(op.neurons, "min_voltage", 0) == 0 for op in ops):
+            raise NotImplementedError("LIF min voltage")
+        J = self.all_data[[self.sidx[op.J] for op in ops]]
+        V = self.all_data[[self.sidx[op.state["voltage"]] for op in ops]]
+        W = self.all_data[[self.sidx[op.state["refractory_time"]] for op in ops]]
+        N = self.all_data[[self.sidx[op.state["adaptation"]] for op in ops]]
+        S = self.all_data[[self.sidx[op.output] for op in ops]]
+        par = lambda name: self._per_population(ops, name)
+        return [self.backend.plan_lif(self.queue, self.model.dt, J, V, W, S, par("tau_ref"),
+                                      par("tau_rc"), par("amplitude"), N=N, tau_n=par("tau_n"),
+                                      inc_n=par("inc_n"))]
+
+    def _plan_AdaptiveLIFRate(self, ops):
+        J = self.all_data[[self.sidx[op.J] for op in ops]]
+        R = self.all_data[[self.sidx[op.output] for op in ops]]
+        N = self.all_data[[self.sidx[op.state["adaptation"]] for op in ops]]
+        par = lambda name: self._per_population(ops, name)
+        return [self.backend.plan_lif_rate(self.queue, self.model.dt, J, R, par("tau_ref"),
+                                           par("tau_rc"), par("amplitude"), N=N,
+                                           tau_n=par("tau_n"), inc_n=par("inc_n"))]
+
+    def _plan_RectifiedLinear(self, ops):
+        J = self.all_data[[self.sidx[op.J] for op in ops]]
+        R = self.all_data[[self.sidx[op.output] for op in ops]]
+        return [self.backend.plan_rectified_linear(self.queue, J, R,
+                                                   self._per_population(ops, "amplitude"))]
+
+    def _plan_SpikingRectifiedLinear(self, ops):
+        J = self.all_data[[self.sidx[op.J] for op in ops]]
+        V = self.all_data[[self.sidx[op.state["voltage"]] for op in ops]]
+        S = self.all_data[[self.sidx[op.output] for op in ops]]
+        return [self.backend.plan_spiking_rectified_linear(
+            self.queue, self.model.dt, J, V, S, self._per_population(ops, "amplitude"))]
+
+    def _plan_Sigmoid(self, ops):
+        J = self.all_data[[self.sidx[op.J] for op in ops]]
+        R = self.all_data[[self.sidx[op.output] for op in ops]]
+        return [self.backend.plan_sigmoid(self.queue, J, R, self._per_population(ops, "tau_ref"))]
 
     # --- processes
     def _plan_SimProcess(self, all_ops):

@@ -132,9 +132,22 @@ plan_ragged_gather_gemv = plan_block_gemv
 
 
 # ------------------------------------------------------------------ neurons
-def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, upsample=1, tag=None, **kwargs):
-    assert not kwargs.get("fastlif") and kwargs.get("N") is None
+def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, N=None, tau_n=None, inc_n=None,
+             upsample=1, tag=None, **kwargs):
+    assert not kwargs.get("fastlif")
     n = len(J)
+    if N is not None:
+        args = [_i32(J.shape0s), _i32(J.starts), _i32(V.starts), _i32(W.starts),
+                _i32(outS.starts), _i32(N.starts), _param_per_item(tau, n),
+                _param_per_item(ref, n), _param_per_item(amp, n), _param_per_item(tau_n, n),
+                _param_per_item(inc_n, n)]
+        fn = lib().orc_alif
+
+        def step():
+            fn(ctypes.c_int(n), *[_p(a) for a in args], ctypes.c_double(dt),
+               ctypes.c_int(upsample), _p(J.buf), _p(V.buf), _p(W.buf), _p(outS.buf), _p(N.buf))
+
+        return _plan(step, "oracle_alif", args, tag)
     args = [_i32(J.shape0s), _i32(J.starts), _i32(V.starts), _i32(W.starts), _i32(outS.starts),
             _param_per_item(tau, n), _param_per_item(ref, n), _param_per_item(amp, n)]
     fn = lib().orc_lif
@@ -146,9 +159,20 @@ def plan_lif(queue, dt, J, V, W, outS, ref, tau, amp, upsample=1, tag=None, **kw
     return _plan(step, "oracle_lif", args, tag)
 
 
-def plan_lif_rate(queue, dt, J, R, ref, tau, amp, tag=None, **kwargs):
-    assert kwargs.get("N") is None
+def plan_lif_rate(queue, dt, J, R, ref, tau, amp, N=None, tau_n=None, inc_n=None, tag=None,
+                  **kwargs):
     n = len(J)
+    if N is not None:
+        args = [_i32(J.shape0s), _i32(J.starts), _i32(R.starts), _i32(N.starts),
+                _param_per_item(tau, n), _param_per_item(ref, n), _param_per_item(amp, n),
+                _param_per_item(tau_n, n), _param_per_item(inc_n, n)]
+        fn = lib().orc_alif_rate
+
+        def step():
+            fn(ctypes.c_int(n), *[_p(a) for a in args], ctypes.c_double(dt), _p(J.buf), _p(R.buf),
+               _p(N.buf))
+
+        return _plan(step, "oracle_alif_rate", args, tag)
     args = [_i32(J.shape0s), _i32(J.starts), _i32(R.starts), _param_per_item(tau, n),
             _param_per_item(ref, n), _param_per_item(amp, n)]
     fn = lib().orc_lif_rate
@@ -157,6 +181,32 @@ def plan_lif_rate(queue, dt, J, R, ref, tau, amp, tag=None, **kwargs):
         fn(ctypes.c_int(n), *[_p(a) for a in args], _p(J.buf), _p(R.buf))
 
     return _plan(step, "oracle_lif_rate", args, tag)
+
+
+def _plan_simple_neurons(kind, name, dt, J, out, param, V=None, tag=None):
+    n = len(J)
+    args = [_i32(J.shape0s), _i32(J.starts), _i32(out.starts),
+            _i32(V.starts if V is not None else np.zeros(n)), _param_per_item(param, n)]
+    fn = lib().orc_simple_neurons
+    vbuf = V.buf if V is not None else out.buf
+
+    def step():
+        fn(ctypes.c_int(kind), ctypes.c_int(n), *[_p(a) for a in args], ctypes.c_double(dt),
+           _p(J.buf), _p(out.buf), _p(vbuf))
+
+    return _plan(step, name, args, tag)
+
+
+def plan_rectified_linear(queue, J, R, amp, tag=None, **kwargs):
+    return _plan_simple_neurons(0, "oracle_relu", 1.0, J, R, amp, tag=tag)
+
+
+def plan_spiking_rectified_linear(queue, dt, J, V, outS, amp, tag=None, **kwargs):
+    return _plan_simple_neurons(1, "oracle_spikingrelu", dt, J, outS, amp, V=V, tag=tag)
+
+
+def plan_sigmoid(queue, J, R, ref, tag=None, **kwargs):
+    return _plan_simple_neurons(2, "oracle_sigmoid", 1.0, J, R, ref, tag=tag)
 
 
 # ----------------------------------------------------------------- synapses

@@ -136,6 +136,101 @@ void orc_lif(int n_items, const int *sizes, const int *j_starts, const int *v_st
     }
 }
 
+/* Adaptive LIF: clra_nonlinearities.py `plan_lif` with N, tau_n, inc_n (:1086-1133): the
+ * voltage step uses J - N - V, the spike time the unadapted J, and afterwards
+ * N += (dt / tau_n) * (inc_n * S - N).  All constants are float (`const ${type}`). */
+void orc_alif(int n_items, const int *sizes, const int *j_starts, const int *v_starts,
+              const int *w_starts, const int *s_starts, const int *n_starts, const float *taus,
+              const float *refs, const float *amps, const float *tau_ns, const float *inc_ns,
+              double dt, int upsample, const float *J, float *V, float *W, float *S, float *N) {
+    const float dtf = (float)dt;
+    const float dtu = (float)(dt / (double)upsample);
+    const float dt_inv = (float)(1.0 / dt);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int k = 0; k < n_items; ++k) {
+        const float tau = taus[k], ref = refs[k], amp = amps[k];
+        for (int i = 0; i < sizes[k]; ++i) {
+            const float j = J[(size_t)j_starts[k] + i];
+            const float n = N[(size_t)n_starts[k] + i];
+            float v = V[(size_t)v_starts[k] + i];
+            float w = W[(size_t)w_starts[k] + i];
+            int spiked = 0;
+            for (int u = 0; u < upsample; ++u) {
+                w = w - dtu;
+                const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
+                const float dv = -(float)expm1((double)(-delta_t / tau)) * ((j - n) - v);
+                v = v + dv;
+                if (v > 1.0f) {
+                    const float t_spike = dtu + tau * (float)log1p((double)(-(v - 1.0f) / (j - 1.0f)));
+                    w = ref + t_spike;
+                    v = 0.0f;
+                    spiked = 1;
+                } else if (v < 0.0f) {
+                    v = 0.0f;
+                }
+            }
+            const float s = spiked ? amp * dt_inv : 0.0f;
+            V[(size_t)v_starts[k] + i] = v;
+            W[(size_t)w_starts[k] + i] = w;
+            S[(size_t)s_starts[k] + i] = s;
+            N[(size_t)n_starts[k] + i] = n + (dtf / tau_ns[k]) * (inc_ns[k] * s - n);
+        }
+    }
+}
+
+/* Adaptive LIF rate: `plan_lif_rate` with N, tau_n, inc_n (:1174-1188). */
+void orc_alif_rate(int n_items, const int *sizes, const int *j_starts, const int *r_starts,
+                   const int *n_starts, const float *taus, const float *refs, const float *amps,
+                   const float *tau_ns, const float *inc_ns, double dt, const float *J, float *R,
+                   float *N) {
+    const float dtf = (float)dt;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int k = 0; k < n_items; ++k) {
+        for (int i = 0; i < sizes[k]; ++i) {
+            const float n = N[(size_t)n_starts[k] + i];
+            float j = (J[(size_t)j_starts[k] + i] - n) - 1.0f;
+            j = (j > 0.0f) ? j : 0.0f;
+            const float r = amps[k] / (refs[k] + taus[k] * (float)log1p((double)(1.0f / j)));
+            R[(size_t)r_starts[k] + i] = r;
+            N[(size_t)n_starts[k] + i] = n + (dtf / tau_ns[k]) * (inc_ns[k] * r - n);
+        }
+    }
+}
+
+/* kind 0: rectified linear `R = amp*max(J, c0)` (:1244-1245); kind 1: spiking rectified
+ * linear (:1217-1223) `V += (J > 0) ? dt*J : 0; n = floor(V); outV = V - n;
+ * outS = amp * n * dt_inv`; kind 2: sigmoid (:1267-1268)
+ * `R = J < t0 ? c0 : J > t1 ? c1/ref : c1 / (ref * (c1 + exp(-J)))`, t0 = -88, t1 = 15,
+ * exp evaluated in double and rounded once. */
+void orc_simple_neurons(int kind, int n_items, const int *sizes, const int *j_starts,
+                        const int *out_starts, const int *v_starts, const float *params, double dt,
+                        const float *J, float *OUT, float *V) {
+    const float dtf = (float)dt;
+    const float dt_inv = (float)(1.0 / dt);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int k = 0; k < n_items; ++k) {
+        const float p = params[k];
+        for (int i = 0; i < sizes[k]; ++i) {
+            const float j = J[(size_t)j_starts[k] + i];
+            float out;
+            if (kind == 0) {
+                out = p * ((j > 0.0f) ? j : 0.0f);
+            } else if (kind == 1) {
+                float v = V[(size_t)v_starts[k] + i];
+                v = v + ((j > 0.0f) ? dtf * j : 0.0f);
+                const float n_spikes = floorf(v);
+                V[(size_t)v_starts[k] + i] = v - n_spikes;
+                out = (p * n_spikes) * dt_inv;
+            } else {
+                out = (j < -88.0f) ? 0.0f
+                      : (j > 15.0f) ? 1.0f / p
+                                    : 1.0f / (p * (1.0f + (float)exp((double)-j)));
+            }
+            OUT[(size_t)out_starts[k] + i] = out;
+        }
+    }
+}
+
 /* LIF rate curve: clra_nonlinearities.py `plan_lif_rate` :1174-1184. */
 void orc_lif_rate(int n_items, const int *sizes, const int *j_starts, const int *r_starts,
                   const float *taus, const float *refs, const float *amps, const float *J,

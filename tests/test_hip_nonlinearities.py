@@ -347,3 +347,86 @@ def test_probes(queue, rng):
     assert list(pos) == [30, 12, 3]
     assert np.array_equal(plan.dev_countdowns.get(), oplan.countdowns)
     assert np.array_equal(dYp.buf, Yh.buf)
+
+
+@pytest.mark.parametrize("upsample", [1, 3])
+def test_adaptive_lif_and_rate(queue, rng, upsample):
+    """Adaptive LIF (state V, W, N) and adaptive LIF rate against the oracle, several
+    steps, one parameter set per population: bit for bit."""
+    dt = 1e-3
+    sizes = [1000, 2345, 17]
+    J = RA([rng.normal(loc=1.5, scale=1.5, size=n) for n in sizes])
+    V = RA([rng.uniform(0, 1, size=n) for n in sizes])
+    W = RA([rng.uniform(-3 * dt, 3 * dt, size=n) for n in sizes])
+    N = RA([rng.uniform(0, 0.3, size=n) for n in sizes])
+    S = RA([np.zeros(n) for n in sizes])
+    tau = np.float32([0.02, 0.03, 0.05])
+    ref = np.float32([0.002, 0.001, 0.003])
+    amp = np.float32([1.0, 0.5, 2.0])
+    tau_n = np.float32([0.1, 0.5, 1.0])
+    inc_n = np.float32([0.01, 0.1, 0.05])
+    dV, dW, dN, dS, dJ = (to_dev(queue, x) for x in (V, W, N, S, J))
+    plan = nl().plan_lif(queue, dt, dJ, dV, dW, dS, ref, tau, amp, N=dN, tau_n=tau_n, inc_n=inc_n,
+                         upsample=upsample)
+    Vo, Wo, No, So = clone(V), clone(W), clone(N), clone(S)
+    oplan = orc().plan_lif(None, dt, J, Vo, Wo, So, ref, tau, amp, N=No, tau_n=tau_n, inc_n=inc_n,
+                           upsample=upsample)
+    total = 0.0
+    for _ in range(20):
+        plan()
+        oplan()
+        total += So.buf.sum()
+        for got, want in ((dV, Vo), (dW, Wo), (dN, No), (dS, So)):
+            assert np.array_equal(got.buf, want.buf)
+    assert total > 0
+
+    R, Nr = RA([np.zeros(n) for n in sizes]), clone(N)
+    dR, dNr = to_dev(queue, R), to_dev(queue, Nr)
+    plan = nl().plan_lif_rate(queue, dt, dJ, dR, ref, tau, amp, N=dNr, tau_n=tau_n, inc_n=inc_n)
+    oplan = orc().plan_lif_rate(None, dt, J, R, ref, tau, amp, N=Nr, tau_n=tau_n, inc_n=inc_n)
+    for _ in range(20):
+        plan()
+        oplan()
+        assert np.array_equal(dR.buf, R.buf) and np.array_equal(dNr.buf, Nr.buf)
+    assert R.buf.sum() > 0
+
+
+def test_relu_spiking_relu_sigmoid(queue, rng):
+    """The one-line neuron types against the oracle (bit for bit), with one parameter
+    per population and, for the rectified linear type, per neuron."""
+    dt = 1e-3
+    sizes = [3000, 777, 5]
+    J = RA([rng.normal(scale=s, size=n) for n, s in zip(sizes, (2, 40, 400))])
+    amp = np.float32([1.0, 0.25, 3.0])
+    dJ = to_dev(queue, J)
+
+    R = RA([np.zeros(n) for n in sizes])
+    dR = to_dev(queue, R)
+    nl().plan_rectified_linear(queue, dJ, dR, amp)()
+    orc().plan_rectified_linear(None, J, R, amp)()
+    assert np.array_equal(dR.buf, R.buf) and R.buf.max() > 0
+
+    amps = RA([rng.uniform(0.5, 2, size=n) for n in sizes])
+    dR2 = to_dev(queue, RA([np.zeros(n) for n in sizes]))
+    nl().plan_rectified_linear(queue, dJ, dR2, to_dev(queue, amps))()
+    got = dR2.to_host()
+    for i in range(len(sizes)):
+        assert np.array_equal(got[i], amps[i] * np.maximum(J[i], 0))
+
+    V, S = RA([rng.uniform(0, 1, size=n) for n in sizes]), RA([np.zeros(n) for n in sizes])
+    dV, dS = to_dev(queue, V), to_dev(queue, S)
+    plan = nl().plan_spiking_rectified_linear(queue, dt, dJ, dV, dS, amp)
+    oplan = orc().plan_spiking_rectified_linear(None, dt, J, V, S, amp)
+    for _ in range(30):
+        plan()
+        oplan()
+        assert np.array_equal(dV.buf, V.buf) and np.array_equal(dS.buf, S.buf)
+    assert S.buf.max() > 0
+
+    Rs = RA([np.zeros(n) for n in sizes])
+    dRs = to_dev(queue, Rs)
+    ref = np.float32([0.0025, 0.002, 0.01])
+    nl().plan_sigmoid(queue, dJ, dRs, ref)()
+    orc().plan_sigmoid(None, J, Rs, ref)()
+    assert np.array_equal(dRs.buf, Rs.buf)
+    assert (Rs.buf == 0).any() and (Rs[2] == 1 / ref[2]).any()  # both cut-offs are reached

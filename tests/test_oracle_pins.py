@@ -332,3 +332,110 @@ def test_direct_unary():
     x, y = RA([[0.731], [2.5]]), RA([[0.0], [0.0]])
     orc.plan_direct_unary(None, "sin", x, y)()
     np.testing.assert_allclose(y.buf, np.sin(np.float32([0.731, 2.5])), rtol=1e-6)
+
+
+# ------------------------------------------------------- further neuron types
+def test_adaptive_lif_reduces_to_lif_and_adapts():
+    """With inc_n = 0 and N = 0 adaptive LIF is LIF bit for bit; a constant N with a
+    very slow tau_n shifts the sub-threshold voltage exactly like a smaller current;
+    without spikes N decays as N0 (1 - dt/tau_n)^k; with spikes N approaches
+    inc_n * rate and the rate drops below the unadapted one."""
+    rng = np.random.RandomState(11)
+    dt, n = 1e-3, 300
+    J = RA([rng.uniform(-1, 4, size=n)])
+    V0, W0 = RA([rng.uniform(0, 1, size=n)]), RA([rng.uniform(-dt, 2 * dt, size=n)])
+    # (i) inc_n = 0, N = 0: identical to LIF
+    Va, Wa, Sa, Na = clone(V0), clone(W0), RA([np.zeros(n)]), RA([np.zeros(n)])
+    Vl, Wl, Sl = clone(V0), clone(W0), RA([np.zeros(n)])
+    alif = orc.plan_lif(None, dt, J, Va, Wa, Sa, 0.002, 0.02, 1.0, N=Na, tau_n=0.5, inc_n=0.0)
+    lif = orc.plan_lif(None, dt, J, Vl, Wl, Sl, 0.002, 0.02, 1.0)
+    for _ in range(50):
+        alif()
+        lif()
+    assert np.array_equal(Va.buf, Vl.buf) and np.array_equal(Wa.buf, Wl.buf)
+    assert np.array_equal(Sa.buf, Sl.buf) and Sa.buf.sum() > 0 and not Na.buf.any()
+    # (ii) sub-threshold: J - N - V with N held (tau_n huge) is LIF driven by J - N
+    Jq = RA([rng.uniform(-1, 0.9, size=n)])
+    Nq = RA([rng.uniform(0, 0.5, size=n)])
+    Jshift = RA([(Jq.buf - Nq.buf).astype(np.float32)])
+    Va, Wa, Sa = RA([np.zeros(n)]), RA([np.zeros(n)]), RA([np.zeros(n)])
+    Vl, Wl, Sl = RA([np.zeros(n)]), RA([np.zeros(n)]), RA([np.zeros(n)])
+    N_before = Nq.buf.copy()
+    orc.plan_lif(None, dt, Jq, Va, Wa, Sa, 0.002, 0.02, 1.0, N=Nq, tau_n=1e30, inc_n=0.0)()
+    orc.plan_lif(None, dt, Jshift, Vl, Wl, Sl, 0.002, 0.02, 1.0)()
+    assert np.array_equal(Va.buf, Vl.buf) and np.array_equal(Nq.buf, N_before)
+    # (iii) decay of N without spikes
+    Nd = RA([np.full(n, 0.3)])
+    step = orc.plan_lif(None, dt, RA([np.zeros(n)]), RA([np.zeros(n)]), RA([np.zeros(n)]),
+                        RA([np.zeros(n)]), 0.002, 0.02, 1.0, N=Nd, tau_n=0.05, inc_n=0.1)
+    for _ in range(100):
+        step()
+    np.testing.assert_allclose(Nd.buf, 0.3 * (1 - dt / 0.05) ** 100, rtol=1e-4)
+    # (iv) adaptation lowers the rate and N settles near inc_n * rate
+    Jc = RA([np.full(n, 3.0)])
+    Va, Wa, Sa, Na = (RA([np.zeros(n)]) for _ in range(4))
+    step = orc.plan_lif(None, dt, Jc, Va, Wa, Sa, 0.002, 0.02, 1.0, N=Na, tau_n=0.1, inc_n=0.01)
+    counts = np.zeros(n)
+    for k in range(3000):
+        step()
+        if k >= 2000:
+            counts += Sa.buf * dt
+    rate = counts.mean() / 1.0
+    unadapted = 1.0 / (0.002 + 0.02 * np.log1p(1.0 / (3.0 - 1.0)))
+    assert rate < 0.9 * unadapted
+    assert abs(Na.buf.mean() - 0.01 * rate) < 0.05 * 0.01 * rate + 0.02
+
+
+def test_adaptive_lif_rate_fixed_point():
+    """inc_n = 0: the LIF rate curve bit for bit; otherwise N converges to the solution of
+    N = inc_n * r(J - N)."""
+    rng = np.random.RandomState(12)
+    n, dt = 200, 1e-3
+    J = RA([rng.uniform(0, 6, size=n)])
+    Ra, Rl, N = RA([np.zeros(n)]), RA([np.zeros(n)]), RA([np.zeros(n)])
+    orc.plan_lif_rate(None, dt, J, Ra, 0.002, 0.02, 1.0, N=N, tau_n=0.1, inc_n=0.0)()
+    orc.plan_lif_rate(None, dt, J, Rl, 0.002, 0.02, 1.0)()
+    assert np.array_equal(Ra.buf, Rl.buf) and not N.buf.any()
+    step = orc.plan_lif_rate(None, dt, J, Ra, 0.002, 0.02, 1.0, N=N, tau_n=0.02, inc_n=0.01)
+    for _ in range(2000):
+        step()
+    rate = lambda j: np.where(j > 1, 1.0 / (0.002 + 0.02 * np.log1p(1.0 / np.maximum(j - 1, 1e-30))), 0)
+    j64 = J.buf.astype(np.float64)
+    ok = np.abs(j64 - N.buf - 1) > 0.05  # the curve is infinitely steep at threshold
+    assert ok.sum() > 150
+    np.testing.assert_allclose(N.buf[ok], 0.01 * rate(j64 - N.buf)[ok], rtol=2e-3, atol=1e-4)
+    np.testing.assert_allclose(Ra.buf[ok], rate(j64 - N.buf)[ok], rtol=2e-2, atol=1e-2)
+
+
+def test_relu_spiking_relu_sigmoid():
+    """Rectified linear against numpy (exact); spiking rectified linear: the spike count
+    over time is floor of the integrated current and the state stays in [0, 1);
+    sigmoid against float64 and at its cut-offs."""
+    rng = np.random.RandomState(13)
+    n, dt = 500, 1e-3
+    J = RA([rng.normal(scale=3, size=n), rng.normal(scale=30, size=n)])
+    amp = np.array([1.0, 0.5], dtype=np.float32)
+    R = RA([np.zeros(n), np.zeros(n)])
+    orc.plan_rectified_linear(None, J, R, amp)()
+    for i in range(2):
+        assert np.array_equal(R[i], amp[i] * np.maximum(J[i], 0))
+
+    V, S = RA([np.zeros(n), np.zeros(n)]), RA([np.zeros(n), np.zeros(n)])
+    Jc = RA([rng.uniform(-50, 900, size=n), rng.uniform(0, 2500, size=n)])
+    step = orc.plan_spiking_rectified_linear(None, dt, Jc, V, S, amp)
+    spikes = np.zeros(2 * n)
+    for _ in range(1000):
+        step()
+        spikes += S.buf * dt / np.repeat(amp, n)
+        assert np.all((V.buf >= 0) & (V.buf < 1))
+    expect = np.maximum(Jc.buf.astype(np.float64), 0) * dt * 1000
+    assert np.all(np.abs(spikes - expect) <= 1.0 + 1e-3 * expect)
+    assert np.all(np.abs(spikes + V.buf - expect) < 1e-2 + 1e-4 * expect)  # nothing is lost
+    assert spikes.max() > 2000  # several spikes per step occur
+
+    Js = RA([np.concatenate([rng.uniform(-30, 14, size=n - 4), [-100.0, -88.5, 15.5, 40.0]])])
+    Rs = RA([np.zeros(n)])
+    orc.plan_sigmoid(None, Js, Rs, 0.0025)()
+    j64 = Js.buf[:-4].astype(np.float64)
+    np.testing.assert_allclose(Rs.buf[:-4], 1.0 / (0.0025 * (1 + np.exp(-j64))), rtol=1e-6)
+    assert np.array_equal(Rs.buf[-4:], np.float32([0, 0, 1 / np.float32(0.0025), 1 / np.float32(0.0025)]))

@@ -291,3 +291,33 @@ def test_guards(queue):
         sim.run_steps(1)
     with pytest.raises(SimulatorClosed):
         sim.reset()
+
+
+@pytest.mark.parametrize("kind", ["AdaptiveLIF", "AdaptiveLIFRate", "RectifiedLinear",
+                                  "SpikingRectifiedLinear", "Sigmoid"])
+def test_other_neuron_types(queue, kind):
+    """A driven ensemble of every further neuron type, decoded and probed: all probe
+    samples and every signal equal the oracle simulator's bit for bit."""
+    from nengo_ocl_amd import minibuilder as mb
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    def make():
+        kwargs = dict(tau_n=0.2, inc_n=0.05) if kind.startswith("Adaptive") else {}
+        net = mb.Network(seed=4)
+        node = net.Node(mb.WhiteSignal(1.0, 5.0, seed=1), size_out=2)
+        ens = net.Ensemble(300, 2, neuron_type=getattr(mb, kind)(**kwargs))
+        out = net.Ensemble(50, 2)
+        net.Connection(node, ens, synapse=None)
+        net.Connection(ens, out, synapse=0.01)
+        return net, [net.Probe(ens.neurons), net.Probe(ens, synapse=0.02), net.Probe(out, synapse=0.02)]
+
+    net, probes = make()
+    net_o, probes_o = make()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        gpu.run_steps(400)
+        cpu.run_steps(400)
+        for a, b in zip(probes, probes_o):
+            assert np.array_equal(gpu.data[a], cpu.data[b])
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+        assert gpu.data[probes[0]].sum() > 0
