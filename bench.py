@@ -19,7 +19,7 @@ stream synchronisations and prints ONE JSON line:
 * ``cpu_baseline``: the CPU oracle (C restatement of the reference kernels,
   OpenMP) stepping the same network on the host cores for a bounded sample.
 
-Other configurations: ``--config c0|c1|c2|c4``; ``--variant per-connection``
+Other configurations: ``--config c0|c1|c2|c4|c5``; ``--variant per-connection``
 gives c3 with one decoder matrix per connection.
 """
 
@@ -56,6 +56,10 @@ def make_network(config, variant, scale):
     if config == "c4":
         n = max(1, int(round(64 * scale)))
         return configs.c4_pes(n_triples=n), "c4: PES, %d triples x 2000 LIF x 32-D" % n
+    if config == "c5":
+        n = max(1000, int(round(1000000 * scale)))
+        return (configs.c5_sparse_recurrent(n_neurons=n),
+                "c5: %d LIF neurons, recurrent sparse weights, 100 per row" % n)
     raise SystemExit("unknown config %r" % config)
 
 

@@ -136,6 +136,21 @@ int nhip_gemv_tile_filter(void *stream, int vec, int pow2_cols, int blk_words, c
                           const float *A, const float *X, const float *Yin, float *Y,
                           const int *item_targets, const int *targets, float *F);
 
+/* ---- sparse matrix-vector products -----------------------------------------
+ * Y[b] (=|+=) A[b] @ X[b] for many sparse matrices in one launch.
+ * replaces: `plan_sparse_dot_inc` / `spmv_csr_impl` / `spmv_ellpack_impl`
+ * (clra_gemv.py:1494-1646, :1649-1755, :1919-1948), which run one launch per
+ * matrix.  Layout: sliced ELLPACK with slices of 64 rows; element k of row r of a
+ * slice is at data_start + 64 k + r in `cols` (column index) and `vals`, rows padded
+ * to the slice's longest row; row r of a slice has row_len[len_start + r] elements.
+ *   slices : int32[n_slices][8] {data_start, width, len_start, n_rows (<= 64),
+ *                                x_start, y_start (of the slice's first row), inc, 0}
+ * X and Y items are contiguous vectors.  Each row is summed in column order with one
+ * fused multiply-add per element (starting from the old y when inc), like the
+ * reference's CSR kernel. */
+int nhip_spmv_sell(void *stream, const int *slices, int n_slices, const int *row_len,
+                   const int *cols, const float *vals, const float *X, float *Y);
+
 /* ---- neurons -----------------------------------------------------------
  * LIF with refractory state and spike-time interpolation.
  * replaces: clra_nonlinearities.py `plan_lif` (:1028-1146, non-adaptive,

@@ -22,7 +22,7 @@ c4     PES learning: 64 (pre, post, error) triples of 2000-neuron 32-D ensembles
 
 import numpy as np
 
-from .minibuilder import LIF, PES, Lowpass, Network, WhiteSignal
+from .minibuilder import LIF, PES, Lowpass, Network, Sparse, WhiteSignal
 
 
 def c0_readme(seed=0, n_neurons=100, neuron_type=None):
@@ -190,10 +190,46 @@ def c4_pes(seed=0, n_triples=64, n_neurons=2000, dims=32, learning_rate=1e-4,
     return net, probes, {}
 
 
+def sparse_ring_weights(n, fan_outs, rewire_frac, rng, scale=1.0):
+    """Sparse n x n weights of the shape the reference's sparse benchmark builds
+    (examples/benchmark_wattsstrogatz.py:154-172): a directed ring in which every row
+    holds `fan_outs` consecutive neighbours (wrapping around), a fraction of the column
+    indices redrawn at random (duplicates inside a row may occur and stay separate
+    entries); values normal(0, scale) instead of the reference's ones."""
+    import scipy.sparse
+
+    offsets = list(range(1, fan_outs + 1))
+    offsets += [off - n for off in offsets]
+    mat = scipy.sparse.diags(np.ones((len(offsets), n), dtype=np.float32), offsets=offsets,
+                             shape=(n, n), format="csr")
+    n_edges = mat.data.size
+    rewire = np.nonzero(rng.random_sample(n_edges) < rewire_frac)[0]
+    mat.indices[rewire] = rng.randint(n, size=rewire.size)
+    mat.data[:] = rng.normal(scale=scale, size=n_edges)
+    return mat
+
+
+def c5_sparse_recurrent(seed=9, n_neurons=100000, fan_outs=100, rewire_frac=0.2,
+                        weight_scale=2e-4, probe_neurons=64):
+    """One population whose neurons are connected to each other through a sparse
+    weight matrix (the reference's own sparse benchmark, examples/
+    benchmark_wattsstrogatz.py:66-84): LIF with tau_ref 1 ms, recurrent synapse 0.1 s.
+    The reference probes every neuron; here a slice of `probe_neurons` is probed."""
+    rng = np.random.RandomState(seed)
+    net = Network(seed=seed, label="c5-sparse-%d" % n_neurons)
+    ens = net.Ensemble(n_neurons, 1, neuron_type=LIF(tau_ref=0.001), label="pop")
+    weights = sparse_ring_weights(n_neurons, fan_outs, rewire_frac, rng, scale=weight_scale)
+    net.Connection(ens.neurons, ens.neurons, transform=Sparse((n_neurons, n_neurons), weights),
+                   synapse=Lowpass(0.1))
+    probes = {"spikes": net.Probe(ens.neurons[:probe_neurons], synapse=0.03)}
+    return net, probes, {"nnz": int(weights.nnz)}
+
+
 CONFIGS = {
     "c0": c0_readme,
     "c1": c1_circconv,
     "c2": c2_watts_strogatz,
     "c3": c3_large,
     "c4": c4_pes,
+    "c5": c5_sparse_recurrent,
 }

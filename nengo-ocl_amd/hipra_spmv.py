@@ -1,0 +1,116 @@
+"""Sparse matrix-vector products: host side of ``nhip_spmv_sell``.
+
+Counterpart of the reference's ``plan_sparse_dot_inc`` (clra_gemv.py:1919-1948) and
+its ``spmv_prog`` family (:1249-1567), which keep every matrix in CSR or ELLPACK on
+the device and launch one kernel per matrix.  Here any number of matrices share one
+launch: their rows are cut into slices of 64 (the wave width) and stored slice by
+slice, element k of every row of a slice side by side, so that a wave reads values
+and column indices in contiguous runs while each lane sums its row in column order.
+"""
+
+import numpy as np
+
+from .hipraggedarray import to_device
+from .plan import Plan
+
+WG, WAVE = 256, 64
+
+
+class HostSparseMatrix:
+    """A sparse matrix on the host in CSR form (reference clra_gemv.py:1242-1247)."""
+
+    def __init__(self, matrix):
+        import scipy.sparse
+
+        csr = matrix.csr if hasattr(matrix, "csr") else matrix
+        self.csr = scipy.sparse.csr_matrix(csr)
+        self.csr.sort_indices()
+        self.shape = self.csr.shape
+
+
+def sell_layout(matrices):
+    """Sliced-ELLPACK arrays of a list of CSR matrices.
+
+    Returns ``(slice_rows, row_len, cols, vals)``: ``slice_rows[k] = (item, data_start,
+    width, len_start, n_rows, row0)``; ``row_len`` padded to 64 per slice; ``cols`` /
+    ``vals`` with element j of row r of slice k at ``data_start + 64 j + r``.
+    """
+    slice_rows, lens, cols, vals = [], [], [], []
+    data_start = 0
+    for item, m in enumerate(matrices):
+        csr = m.csr
+        indptr = np.asarray(csr.indptr, dtype=np.int64)
+        indices = np.asarray(csr.indices, dtype=np.int32)
+        data = np.asarray(csr.data, dtype=np.float32)
+        row_counts = np.diff(indptr).astype(np.int32)
+        for row0 in range(0, csr.shape[0], WAVE):
+            n_rows = min(WAVE, csr.shape[0] - row0)
+            counts = row_counts[row0:row0 + n_rows]
+            width = int(counts.max()) if n_rows else 0
+            block_c = np.zeros((width, WAVE), dtype=np.int32)
+            block_v = np.zeros((width, WAVE), dtype=np.float32)
+            # scatter the slice's elements: position inside its row, row inside the slice
+            lo, hi = int(indptr[row0]), int(indptr[row0 + n_rows])
+            r = np.repeat(np.arange(n_rows), counts)
+            j = np.arange(lo, hi) - np.repeat(indptr[row0:row0 + n_rows], counts)
+            block_c[j, r] = indices[lo:hi]
+            block_v[j, r] = data[lo:hi]
+            padded = np.zeros(WAVE, dtype=np.int32)
+            padded[:n_rows] = counts
+            slice_rows.append((item, data_start, width, len(lens) * WAVE, n_rows, row0))
+            lens.append(padded)
+            cols.append(block_c.ravel())
+            vals.append(block_v.ravel())
+            data_start += width * WAVE
+    cat = lambda parts, dtype: (np.concatenate(parts) if parts else np.zeros(0, dtype)).astype(dtype)
+    return slice_rows, cat(lens, np.int32), cat(cols, np.int32), cat(vals, np.float32)
+
+
+class plan_sparse_dot_inc:
+    """``Y[b] (=|+=) A[b] @ X[b]``; ``.plans`` holds the one launch.
+
+    ``hA`` is a `HostSparseMatrix` (with X, Y of length 1: the reference's signature,
+    clra_gemv.py:1919) or a list of them with one X and one Y item each.  ``inc``
+    defaults to False like the reference's (whose Simulator thereby *sets* Y); the
+    Simulator here passes True, the meaning of the operator.
+    """
+
+    def __init__(self, queue, hA, X, Y, inc=False, tag=None, algorithm=None):
+        matrices = list(hA) if isinstance(hA, (list, tuple)) else [hA]
+        matrices = [m if isinstance(m, HostSparseMatrix) else HostSparseMatrix(m) for m in matrices]
+        if not (len(matrices) == len(X) == len(Y)):
+            raise ValueError("need one X and one Y item per matrix")
+        for arr, name in ((X, "X"), (Y, "Y")):
+            arr.check_bounds(name)
+            if not ((arr.shape1s == 1).all() and (arr.stride0s == 1).all()):
+                raise NotImplementedError("sparse products are matrix-vector only")
+        for b, m in enumerate(matrices):
+            if m.shape != (int(Y.shape0s[b]), int(X.shape0s[b])):
+                raise ValueError("matrix %d is %s, Y has %d and X %d elements"
+                                 % (b, m.shape, Y.shape0s[b], X.shape0s[b]))
+            if m.csr.nnz and (m.csr.indices.min() < 0 or m.csr.indices.max() >= m.shape[1]):
+                raise ValueError("matrix %d has column indices outside X" % b)
+        incs = np.broadcast_to(np.asarray(inc, dtype=np.int32), (len(matrices),))
+        slice_rows, row_len, cols, vals = sell_layout(matrices)
+        table = np.zeros((max(len(slice_rows), 1), 8), dtype=np.int32)
+        for k, (item, data_start, width, len_start, n_rows, row0) in enumerate(slice_rows):
+            table[k] = (data_start, width, len_start, n_rows, int(X.starts[item]),
+                        int(Y.starts[item]) + row0, int(incs[item]), 0)
+        if vals.size >= 2 ** 31:
+            raise ValueError("more than 2^31 stored elements")
+        n = len(slice_rows)
+        dev = [to_device(queue, a) for a in (table, row_len if row_len.size else np.zeros(1, np.int32),
+                                             cols if cols.size else np.zeros(1, np.int32),
+                                             vals if vals.size else np.zeros(1, np.float32))]
+        args = (dev[0].ptr, n, dev[1].ptr, dev[2].ptr, dev[3].ptr, X.ptr, Y.ptr)
+        n_groups = max(1, -(-n // (WG // WAVE)))
+        plan = Plan(queue, queue.lib.nhip_spmv_sell, args, gsize=(WG * n_groups,), lsize=(WG,),
+                    full_args=tuple(dev) + (X.dev_buf, Y.dev_buf), name="hip_spmv", tag=tag)
+        nnz = int(sum(m.csr.nnz for m in matrices))
+        plan.flops_per_call = 2 * nnz
+        # reference accounting (clra_gemv.py:1552-1560): values, indices, row pointers, X, Y
+        plan.bw_per_call = 8 * nnz + 4 * sum(m.shape[0] + 1 for m in matrices) + X.nbytes + Y.nbytes
+        plan.stored_bytes = 8 * int(vals.size)
+        plan.description = "groups: %d; nonzeros: %d; stored: %d" % (len(matrices), nnz, vals.size)
+        self.plans = [plan]
+        self.matrices = matrices

@@ -115,6 +115,36 @@ class Signal:
         return "Signal(name=%s, shape=%s)" % (self.name, self.shape)
 
 
+class SparseSignal(Signal):
+    """A constant sparse matrix (scipy CSR); never sliced or reshaped.  nengo's
+    counterpart is a Signal whose initial value is a ``SparseMatrix`` (``sig.sparse``)."""
+
+    sparse = True
+
+    def __init__(self, matrix, name=None):
+        import scipy.sparse
+
+        self._csr = scipy.sparse.csr_matrix(matrix, dtype=np.float64)
+        self._csr.sort_indices()
+        self._base = None
+        self.name = name
+        self._readonly = True
+
+    initial_value = property(lambda self: self._csr)
+    dtype = property(lambda self: self._csr.dtype)
+    shape = property(lambda self: self._csr.shape)
+    ndim = property(lambda self: 2)
+    size = property(lambda self: self._csr.nnz)
+
+    def may_share_memory(self, other):
+        return other is self
+
+    def __getitem__(self, item):
+        raise ValueError("sparse signals have no views")
+
+    reshape = __getitem__
+
+
 # ============================================================= operators
 class Operator:
     """Base class: lists of signals set / incremented / read / updated this step.
@@ -181,6 +211,19 @@ class DotInc(Operator):
         self.A, self.X, self.Y = A, X, Y
         self.reads = [A, X]
         self.incs = [Y]
+
+
+class SparseDotInc(Operator):
+    """``Y += A @ X`` with a sparse matrix signal A (nengo's SparseDotInc)."""
+
+    def __init__(self, A, X, Y, tag=None):
+        super().__init__(tag)
+        if not getattr(A, "sparse", False):
+            raise ValueError("A must be a sparse signal")
+        if A.shape != (Y.size, X.size):
+            raise ValueError("shape mismatch: %s @ %s -> %s" % (A.shape, X.shape, Y.shape))
+        self.A, self.X, self.Y = A, X, Y
+        self.incs, self.reads = [Y], [A, X]
 
 
 class ElementwiseInc(Operator):

@@ -98,6 +98,18 @@ class Probe(ir.Probe):
         self.synapse = Lowpass(synapse) if isinstance(synapse, (int, float)) else synapse
 
 
+class Sparse:
+    """A sparse transform (nengo.transforms.Sparse): ``shape`` and a scipy sparse ``init``."""
+
+    def __init__(self, shape, init):
+        import scipy.sparse
+
+        self.shape = tuple(shape)
+        self.init = scipy.sparse.csr_matrix(init)
+        if self.init.shape != self.shape:
+            raise ValueError("init has shape %s, not %s" % (self.init.shape, self.shape))
+
+
 def _uniform(rng, spec, n):
     if np.ndim(spec) == 1 and len(spec) == 2 and not isinstance(spec, np.ndarray):
         return rng.uniform(spec[0], spec[1], size=n)
@@ -310,7 +322,9 @@ class Network:
         post, post_slice = self._split(conn.post)
         crng = np.random.RandomState(rng.randint(2 ** 31 - 1))
         name = conn.label or "conn%d" % len(model.sig)
-        transform = None if conn.transform is None else np.asarray(conn.transform, dtype=np.float64)
+        sparse = conn.transform if isinstance(conn.transform, Sparse) else None
+        transform = (None if conn.transform is None or sparse is not None
+                     else np.asarray(conn.transform, dtype=np.float64))
 
         if isinstance(pre, Ensemble):
             if pre_slice is not None:
@@ -353,6 +367,21 @@ class Network:
             signal = model.sig[pre]["out"]
             if pre_slice is not None:
                 signal = signal[pre_slice]
+            if sparse is not None or (transform is not None and transform.ndim == 2):
+                # weights between neurons: weighted = W @ activities, then the synapse
+                n_out = sparse.shape[0] if sparse is not None else transform.shape[0]
+                weighted = ir.Signal(np.zeros(n_out), name="%s.weighted" % name)
+                model.add_op(ir.Reset(weighted))
+                if sparse is not None:
+                    wsig = ir.SparseSignal(sparse.init, name="%s.weights" % name)
+                    model.add_op(ir.SparseDotInc(wsig, signal, weighted, tag="%s.weights" % name))
+                else:
+                    wsig = ir.Signal(transform, name="%s.weights" % name, readonly=True)
+                    model.add_op(ir.DotInc(wsig, signal, weighted, tag="%s.weights" % name))
+                model.sig[conn] = {"weights": wsig}
+                signal = weighted
+            elif transform is not None:
+                raise NotImplementedError("scalar / diagonal transforms between neurons")
             signal = self._apply_synapse(model, signal, conn.synapse, name)
         elif isinstance(pre, Node):
             signal = model.sig[pre]["out"]

@@ -72,6 +72,9 @@ class HipBackend:
         self._fuse_lif = hipra_gemv.fuse_lif
         from . import hipra_sequence
 
+        from . import hipra_spmv
+
+        self.plan_sparse_dot_inc = hipra_spmv.plan_sparse_dot_inc
         self.merge_small_plans = hipra_sequence.merge_small_plans
         self.plans_conflict = hipra_sequence._conflict
         self.fuse_gemv_filter = hipra_gemv.fuse_linearfilter
@@ -265,9 +268,15 @@ class Simulator:
         all_signals = stable_unique(sig for op in all_operators + operators
                                     for sig in op.all_signals)
         all_bases = stable_unique(sig.base for sig in all_signals)
-        if any(getattr(s, "sparse", False) for s in all_signals):
-            raise NotImplementedError("sparse signals")
-        values = self._initial_values(all_operators, all_bases)
+        # sparse matrices are constants of the sparse products: they stay on the host
+        # until `_plan_SparseDotInc` lays them out (reference simulator.py:281-329)
+        sparse_bases = [b for b in all_bases if getattr(b, "sparse", False)]
+        if any(getattr(s, "sparse", False) and s.base is not s for s in all_signals):
+            raise NotImplementedError("views of sparse signals")
+        all_bases = [b for b in all_bases if not getattr(b, "sparse", False)]
+        all_values = self._initial_values(all_operators, all_bases + sparse_bases)
+        self.sparse_data = {b: all_values[b] for b in sparse_bases}
+        values = {b: all_values[b] for b in all_bases}
 
         self.base_reshapes = {}
         dense = []
@@ -686,6 +695,17 @@ class Simulator:
         prog = self.backend.plan_block_gemv(self.queue, alpha, all_data, A_js, all_data, X_js,
                                             beta, Y, Y_in=Y_in, gamma=gamma, tag=tag)
         return prog.plans
+
+    def _plan_SparseDotInc(self, ops):
+        """All sparse products of the group in one launch (the reference plans one
+        launch per operator, simulator.py:877-892)."""
+        matrices = []
+        for op in ops:
+            value = self.sparse_data[op.A]
+            matrices.append(value.csr if hasattr(value, "csr") else value)
+        X = self.all_data[[self.sidx[op.X] for op in ops]]
+        Y = self.all_data[[self.sidx[op.Y] for op in ops]]
+        return self.backend.plan_sparse_dot_inc(self.queue, matrices, X, Y, inc=True).plans
 
     def _plan_TimeUpdate(self, ops):
         (op,) = ops

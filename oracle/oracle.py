@@ -209,6 +209,40 @@ def plan_sigmoid(queue, J, R, ref, tag=None, **kwargs):
     return _plan_simple_neurons(2, "oracle_sigmoid", 1.0, J, R, ref, tag=tag)
 
 
+# ------------------------------------------------------------------ sparse
+class plan_sparse_dot_inc:
+    """``Y[b] (=|+=) A[b] @ X[b]`` from CSR, rows summed in column order
+    (clra_gemv.py `spmv_csr_impl` :1570-1646)."""
+
+    def __init__(self, queue, hA, X, Y, inc=False, tag=None, algorithm=None):
+        import scipy.sparse
+
+        mats = list(hA) if isinstance(hA, (list, tuple)) else [hA]
+        csrs = []
+        for m in mats:
+            c = scipy.sparse.csr_matrix(m.csr if hasattr(m, "csr") else m)
+            c.sort_indices()
+            csrs.append(c)
+        n = len(csrs)
+        assert n == len(X) == len(Y)
+        starts = np.cumsum([0] + [c.nnz for c in csrs])
+        # each item's row pointers index the concatenated data: shift them by its offset
+        indptr = np.concatenate([np.asarray(c.indptr, dtype=np.int64) + s
+                                 for c, s in zip(csrs, starts)]).astype(np.int32)
+        ptr_starts = np.cumsum([0] + [c.shape[0] + 1 for c in csrs])[:-1]
+        args = [_i32([c.shape[0] for c in csrs]), _i32(ptr_starts), _i32(X.starts), _i32(Y.starts),
+                _i32(np.broadcast_to(np.asarray(inc, dtype=np.int32), (n,))), indptr,
+                _i32(np.concatenate([c.indices for c in csrs]) if n else []),
+                np.ascontiguousarray(np.concatenate([c.data for c in csrs]) if n else [],
+                                     dtype=np.float32)]
+        fn = lib().orc_spmv_csr
+
+        def step():
+            fn(ctypes.c_int(n), *[_p(a) for a in args], _p(X.buf), _p(Y.buf))
+
+        self.plans = [_plan(step, "oracle_spmv", args, tag)]
+
+
 # ----------------------------------------------------------------- synapses
 def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
     n = len(X)

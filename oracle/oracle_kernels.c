@@ -462,3 +462,22 @@ void orc_direct_unary(int opcode, int n_items, const int *x_starts, const int *y
         Y[y_starts[n]] = y;
     }
 }
+
+/* Sparse matrix-vector product in CSR form: clra_gemv.py `spmv_csr_impl` :1588-1617
+ * (`y[irow] = 0` unless inc, then `y[irow] += A_data[k] * x[A_indices[k]]` for k in row
+ * order; one fused multiply-add per element, see orc_gemv_block). */
+void orc_spmv_csr(int n_items, const int *n_rows, const int *indptr_starts,
+                  const int *x_starts, const int *y_starts, const int *incs, const int *indptr,
+                  const int *indices, const float *data, const float *X, float *Y) {
+    for (int n = 0; n < n_items; ++n) {
+        const int *ptr = indptr + indptr_starts[n];
+        const float *x = X + x_starts[n];
+        float *y = Y + y_starts[n];
+#pragma omp parallel for schedule(static)
+        for (int r = 0; r < n_rows[n]; ++r) {
+            float acc = incs[n] ? y[r] : 0.0f;
+            for (int k = ptr[r]; k < ptr[r + 1]; ++k) acc = fmaf(data[k], x[indices[k]], acc);
+            y[r] = acc;
+        }
+    }
+}

@@ -516,3 +516,49 @@ def test_gemv_with_filter_epilogue(queue):
         for p in oprog.plans + olf:
             p()
         assert np.array_equal(dev.to_host().buf, host.buf), step
+
+
+def test_sparse_products(queue):
+    """Many sparse matrices in one launch (64-row slices, rows summed in column order):
+    bit-identical to the oracle's CSR product for row counts that are no multiple of
+    64, empty rows and empty matrices, duplicate entries, rows much longer than their
+    neighbours, incrementing and setting items side by side; the layout is checked
+    against the matrices it came from."""
+    import scipy.sparse as sp
+
+    from nengo_ocl_amd import hipra_spmv
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(8)
+    shapes = [(1000, 700), (64, 64), (65, 10), (1, 300), (300, 1), (130, 4000), (40, 40)]
+    mats = [sp.random(m, n, density=d, random_state=rng, format="csr", dtype=np.float32)
+            for (m, n), d in zip(shapes, (0.05, 0.5, 0.3, 0.9, 0.5, 0.02, 0.0))]
+    long_row = sp.lil_matrix(mats[5].shape, dtype=np.float32)
+    long_row[7, :] = rng.normal(size=4000)          # one full row among sparse ones
+    mats[5] = sp.csr_matrix(mats[5] + long_row.tocsr())
+    mats[1].indices[:] = rng.randint(64, size=mats[1].nnz)  # unsorted, with duplicates
+    X = RA([rng.normal(size=n) for m, n in shapes], align=True)
+    Y = RA([rng.normal(size=m) for m, n in shapes], align=True)
+    inc = [1, 0, 1, 0, 1, 0, 1]
+
+    slice_rows, row_len, cols, vals = hipra_spmv.sell_layout([hipra_spmv.HostSparseMatrix(m) for m in mats])
+    k = [r for r in slice_rows if r[0] == 0][3]     # fourth slice of the first matrix
+    _, start, width, len_start, n_rows, row0 = k
+    csr = hipra_spmv.HostSparseMatrix(mats[0]).csr
+    for r in (0, 17, 63):
+        n = row_len[len_start + r]
+        lo = csr.indptr[row0 + r]
+        assert n == csr.indptr[row0 + r + 1] - lo
+        assert np.array_equal(cols[start + 64 * np.arange(n) + r], csr.indices[lo:lo + n])
+        assert np.array_equal(vals[start + 64 * np.arange(n) + r], csr.data[lo:lo + n])
+
+    Yo = clone(Y)
+    oplan = orc.plan_sparse_dot_inc(None, mats, X, Yo, inc=inc).plans[0]
+    dX, dY = to_dev(queue, X), to_dev(queue, Y)
+    plan = hipra_spmv.plan_sparse_dot_inc(queue, mats, dX, dY, inc=inc).plans[0]
+    for _ in range(3):  # the incrementing items accumulate
+        plan()
+        oplan()
+        assert np.array_equal(dY.to_host().buf, Yo.buf)
+    with pytest.raises(ValueError):
+        hipra_spmv.plan_sparse_dot_inc(queue, mats[:2], dX[[0, 2]], dY[[0, 1]])

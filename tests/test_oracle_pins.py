@@ -439,3 +439,34 @@ def test_relu_spiking_relu_sigmoid():
     j64 = Js.buf[:-4].astype(np.float64)
     np.testing.assert_allclose(Rs.buf[:-4], 1.0 / (0.0025 * (1 + np.exp(-j64))), rtol=1e-6)
     assert np.array_equal(Rs.buf[-4:], np.float32([0, 0, 1 / np.float32(0.0025), 1 / np.float32(0.0025)]))
+
+
+# ------------------------------------------------------------------ sparse
+def test_spmv_against_scipy():
+    """The CSR product against scipy: exact for small integers (any order gives the same
+    sums), float64 closeness otherwise; duplicate entries add up, empty rows give 0 (or
+    keep y when incrementing), several matrices per call, increment and set."""
+    import scipy.sparse as sp
+
+    rng = np.random.RandomState(21)
+    shapes = [(70, 50), (1, 9), (200, 200), (5, 3)]
+    mats = [sp.random(m, n, density=0.2, random_state=rng, format="csr") for m, n in shapes]
+    mats[2].data[:] = rng.randint(-4, 5, size=mats[2].nnz)            # integers: exact
+    dup = sp.csr_matrix((np.float32([1, 2, 3]), np.int32([2, 2, 0]), np.int32([0, 2, 2, 3, 3, 3])),
+                        shape=(5, 3))                                  # duplicate column, empty rows
+    mats[3] = dup
+    X = RA([rng.randint(-3, 4, size=n) if i == 2 else rng.normal(size=n) for i, (m, n) in enumerate(shapes)])
+    Y0 = RA([rng.normal(size=m) for m, n in shapes])
+    for inc in (False, True, [1, 0, 1, 0]):
+        Y = clone(Y0)
+        orc.plan_sparse_dot_inc(None, mats, X, Y, inc=inc).plans[0]()
+        incs = np.broadcast_to(np.asarray(inc, dtype=bool), (4,))
+        for i, mat in enumerate(mats):
+            want = mat.astype(np.float64) @ X[i][:, 0].astype(np.float64) + (Y0[i][:, 0] if incs[i] else 0)
+            if i == 2 and not incs[i]:
+                assert np.array_equal(Y[i][:, 0], want.astype(np.float32))
+            else:
+                np.testing.assert_allclose(Y[i][:, 0], want, rtol=1e-5, atol=1e-5)
+    Y = clone(Y0)
+    orc.plan_sparse_dot_inc(None, [dup], RA([[1.0, 10.0, 100.0]]), Y[[3]], inc=False).plans[0]()
+    assert np.array_equal(Y[3][:, 0], np.float32([300, 0, 3, 0, 0]))

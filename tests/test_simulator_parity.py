@@ -321,3 +321,25 @@ def test_other_neuron_types(queue, kind):
             assert np.array_equal(gpu.data[a], cpu.data[b])
         assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
         assert gpu.data[probes[0]].sum() > 0
+
+
+def test_sparse_recurrent_population(queue):
+    """A population recurrently connected through a sparse weight matrix (the shape of
+    the reference's sparse benchmark), 1 s: spikes and every signal bit-identical to the
+    oracle simulator."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    make = lambda: configs.c5_sparse_recurrent(n_neurons=3000, fan_outs=30, weight_scale=5e-4,
+                                               probe_neurons=3000)
+    net, probes, info = make()
+    net_o, probes_o, _ = make()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        assert any(p.name == "hip_spmv" for p in gpu._plans)
+        gpu.run_steps(1000)
+        cpu.run_steps(1000)
+        assert np.array_equal(gpu.data[probes["spikes"]], cpu.data[probes_o["spikes"]])
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+        rates = gpu.data[probes["spikes"]][-1]
+        assert rates.max() > 50 and rates.std() > 10  # the recurrence shapes the activity
