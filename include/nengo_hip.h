@@ -67,9 +67,11 @@ int nhip_device_info(int *n_cu, int *wave_size, int *lds_bytes, char *name, int 
  * `flavor` 0 = one work-group (256 threads) per task, X staged in LDS and
  * shared by the group's four waves; rows per task <= nhip_gemv_rows_per_task.
  * `flavor` 1 = one wave per task (four tasks per group), X read through L1;
- * for many tiny items.  `flavor` 2 = one wave per task in the summation order of
- * the reference's block kernel (four strided partial sums per 128-column tile,
- * tiles added in order; lpr must be 4 and vec 1): bit-identical to a float32
+ * for many tiny items.  `flavor` 2 = the summation order of the reference's block
+ * kernel (four strided partial sums per 128-column tile, tiles added in order) for
+ * small items: every task is ONE row (n_rows == 1), a wave takes 64 / lpr consecutive
+ * tasks of whatever items; lpr 4 (any widths) or 1 (every dot product of the launch
+ * has at most 4 columns), vec 1: bit-identical to a float32
  * restatement of that kernel.  `lpr` = lanes cooperating on one row (1,2,...,64, or
  * 256 for flavor 0); `vec` = 4 (16-byte loads; needs a_start % 4 == 0 and
  * a_stride0 % 4 == 0 for every dot of the launch) or 1.  `passes` (flavor 0) =

@@ -221,76 +221,90 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
     }
 }
 
-// Wave-per-task kernel in the summation order of the reference's block GEMV
-// (clra_gemv.py:1040-1058 and :1148-1153): per row and per 128-column tile, lane
-// j of four sums columns j, j+4, ... left to right (fused multiply-add, as an
-// OpenCL compiler contracts the reference's `+=`), the four partial sums combine as (s0+s2)+(s1+s3), and tile sums
-// are added one after the other onto beta*y_in; gamma comes last.  Used for the
-// small items of networks with thousands of tiny ensembles, where the order costs
-// nothing and makes the result bit-identical to a float32 restatement of the
-// reference; sixteen rows are in flight per wave.
-__global__ __launch_bounds__(NHIP_WG) void gemv_wave_ref_kernel(
+// ---------------------------------------------------------------- reference order, small items
+// One output row per task (task = {item, row, 1, 0}); a wave takes 64 / LPR
+// consecutive tasks, LPR lanes each, whatever items they belong to -- thousands of
+// one-row items (decoders of small populations) fill waves as well as a few tall ones.
+// Sums are formed in the order of the reference's block kernel (clra_gemv.py:1043-1058,
+// :1148-1153): per 128-column tile four strided partial sums, one fused multiply-add
+// per element, (s0+s2)+(s1+s3), tiles in order onto beta*y_in, gamma last.
+//   LPR = 4: lane j of a row carries partial sum j; any number of columns.
+//   LPR = 1: one lane per row, for items whose dot products all have <= 4 columns
+//            (vector sums, "scalar times vector" increments): the four partial sums are
+//            the (up to) four products themselves.
+// These launches are latency bound: the records of four dot products and, when those
+// have at most four columns, all their operands are fetched together before the sums
+// are formed in order.  Task, item and dot records are per-lane values on purpose
+// (different rows of a wave may belong to different items).
+template <int LPR>
+__global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     const float* __restrict__ A, const float* __restrict__ X, const float* Yin, float* Y)
 {
     constexpr int TILE = 128;
-    constexpr int BATCH = 4;  // dot products whose operands are fetched together
+    constexpr int BATCH = 4;             // dot products whose operands are fetched together
+    constexpr int ROWS = NHIP_WAVE / LPR;  // rows (tasks) per wave
+    constexpr int PER_LANE = 4 / LPR;    // elements of a <= 4 column dot product per lane
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
-    const int t = blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6);
-    if (t >= n_tasks) return;  // wave-uniform; this kernel has no barrier
-
-    const GemvTask task = tasks[t];
+    const int lir = lane % LPR;
+    const int slot = (blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6)) * ROWS + lane / LPR;
+    const bool valid = slot < n_tasks;
+    const GemvTask task = tasks[valid ? slot : n_tasks - 1];
     const GemvItem it = items[task.item];
     const float4 cf = coefs[task.item];
-    const int row_end = task.row0 + task.n_rows;
-    const int lir = lane & 3;
-    const int sub = lane >> 2;
+    const int r = task.row0;
+    const int n_dots = valid ? it.n_dots : 0;
+    float sum = cf.y * Yin[it.yin_start + (size_t)r * it.yin_stride0];
 
-    for (int r0 = task.row0; r0 < row_end; r0 += NHIP_WAVE / 4) {
-        const bool valid = r0 + sub < row_end;
-        const int r = valid ? r0 + sub : row_end - 1;
-        float sum = cf.y * Yin[it.yin_start + (size_t)r * it.yin_stride0];
-        for (int d0 = 0; d0 < it.n_dots; d0 += BATCH) {
-            // These items are latency bound (a handful of short dot products per row):
-            // the records of a batch are read together, and when every dot product of
-            // the batch has at most four columns -- one element per lane, the common
-            // "scalar times vector" increments -- so are all their operands, before the
-            // sums are formed in the usual order.
-            GemvDot dot[BATCH];
-            bool tiny = true;
+    for (int d0 = 0; __any(d0 < n_dots); d0 += BATCH) {
+        GemvDot dot[BATCH];
+        bool tiny = true;
+#pragma unroll
+        for (int k = 0; k < BATCH; ++k) {
+            dot[k] = dots[d0 + k < n_dots ? it.dot_begin + d0 + k : 0];
+            tiny = tiny && (d0 + k >= n_dots || dot[k].N <= 4);
+        }
+        if (LPR == 1 || __all(tiny)) {
+            float a[BATCH][PER_LANE], x[BATCH][PER_LANE];
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k)
+#pragma unroll
+                for (int e = 0; e < PER_LANE; ++e) {
+                    const int c = lir + e * LPR;
+                    const bool live = d0 + k < n_dots && c < dot[k].N;
+                    a[k][e] = live ? A[dot[k].a_start + (size_t)r * dot[k].a_stride0 + c] : 0.0f;
+                    x[k][e] = live ? X[dot[k].x_start + (size_t)c * dot[k].x_stride0] : 0.0f;
+                }
 #pragma unroll
             for (int k = 0; k < BATCH; ++k) {
-                dot[k] = dots[it.dot_begin + min(d0 + k, it.n_dots - 1)];
-                tiny = tiny && dot[k].N <= 4;
-            }
-            if (tiny) {
-                float a[BATCH], x[BATCH];
+                float s;
+                if (LPR == 4) {
+                    s = lir < dot[k].N ? fmaf(a[k][0], x[k][0], 0.0f) : 0.0f;
+                    s = s + __shfl_xor(s, 2, NHIP_WAVE);
+                    s = s + __shfl_xor(s, 1, NHIP_WAVE);
+                } else {
+                    float p[4];
 #pragma unroll
-                for (int k = 0; k < BATCH; ++k) {
-                    const bool live = d0 + k < it.n_dots && lir < dot[k].N;
-                    a[k] = live ? A[dot[k].a_start + (size_t)r * dot[k].a_stride0 + lir] : 0.0f;
-                    x[k] = live ? X[dot[k].x_start + (size_t)lir * dot[k].x_stride0] : 0.0f;
+                    for (int e = 0; e < 4; ++e)
+                        p[e] = e < dot[k].N ? fmaf(a[k][e % PER_LANE], x[k][e % PER_LANE], 0.0f) : 0.0f;
+                    s = (p[0] + p[2]) + (p[1] + p[3]);
                 }
-#pragma unroll
-                for (int k = 0; k < BATCH; ++k) {
-                    if (d0 + k < it.n_dots) {  // uniform
-                        float s = lir < dot[k].N ? fmaf(a[k], x[k], 0.0f) : 0.0f;
-                        s = s + __shfl_xor(s, 2, NHIP_WAVE);
-                        s = s + __shfl_xor(s, 1, NHIP_WAVE);
-                        sum = sum + cf.x * s;
-                    }
-                }
-                continue;
+                if (d0 + k < n_dots) sum = sum + cf.x * s;
             }
+            continue;
+        }
+        if (LPR == 4) {
 #pragma unroll
             for (int k = 0; k < BATCH; ++k) {  // static indices keep the records in registers
-                if (d0 + k >= it.n_dots) break;
+                if (!__any(d0 + k < n_dots)) break;
+                const bool have = d0 + k < n_dots;
+                const int n_cols = have ? dot[k].N : 0;
                 const float* arow = A + dot[k].a_start + (size_t)r * dot[k].a_stride0;
                 const float* xg = X + dot[k].x_start;
                 const size_t xs = (size_t)dot[k].x_stride0;
-                for (int c0 = 0; c0 < dot[k].N; c0 += TILE) {
-                    const int c1 = min(c0 + TILE, dot[k].N);
+                for (int c0 = 0; c0 < n_cols; c0 += TILE) {
+                    const int c1 = min(c0 + TILE, n_cols);
                     float s = 0.0f;
                     for (int c = c0 + lir; c < c1; c += 4) s = fmaf(arow[c], xg[(size_t)c * xs], s);
                     s = s + __shfl_xor(s, 2, NHIP_WAVE);
@@ -299,8 +313,8 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_ref_kernel(
                 }
             }
         }
-        if (lir == 0 && valid) Y[it.y_start + (size_t)r * it.y_stride0] = sum + cf.z;
     }
+    if (lir == 0 && valid) Y[it.y_start + (size_t)r * it.y_stride0] = sum + cf.z;
 }
 
 template <int LPR, int VEC, int P>
@@ -360,7 +374,7 @@ static int default_passes(int lpr) {
 
 extern "C" int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes) {
     if (vec != 1 && vec != 4) return 0;
-    if (flavor == 2) return (lpr == 4 && vec == 1) ? 0x7fffffff : 0;
+    if (flavor == 2) return ((lpr == 4 || lpr == 1) && vec == 1) ? 1 : 0;
     if (flavor == 1) {
         switch (lpr) { case 1: case 2: case 4: case 8: case 16: case 32: case 64: return 0x7fffffff; }
         return 0;
@@ -402,13 +416,21 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
             NHIP_WG_CASE(256)
         }
     } else if (flavor == 2) {
-        if (lpr != 4 || vec != 1) return NHIP_E_BADCLASS;
-        const int wpg = NHIP_WG / NHIP_WAVE;
-        hipLaunchKernelGGL(gemv_wave_ref_kernel, dim3((n_tasks + wpg - 1) / wpg), dim3(NHIP_WG), 0,
-                           s, reinterpret_cast<const GemvItem*>(items),
-                           reinterpret_cast<const float4*>(coefs),
-                           reinterpret_cast<const GemvDot*>(dots),
-                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
+        if ((lpr != 4 && lpr != 1) || vec != 1) return NHIP_E_BADCLASS;
+        const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
+        const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
+        if (lpr == 4)
+            hipLaunchKernelGGL(gemv_rows_ref_kernel<4>, grid, dim3(NHIP_WG), 0, s,
+                               reinterpret_cast<const GemvItem*>(items),
+                               reinterpret_cast<const float4*>(coefs),
+                               reinterpret_cast<const GemvDot*>(dots),
+                               reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
+        else
+            hipLaunchKernelGGL(gemv_rows_ref_kernel<1>, grid, dim3(NHIP_WG), 0, s,
+                               reinterpret_cast<const GemvItem*>(items),
+                               reinterpret_cast<const float4*>(coefs),
+                               reinterpret_cast<const GemvDot*>(dots),
+                               reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
         NHIP_LAUNCH_CHECK();
         return 0;
     } else if (flavor == 1) {

@@ -37,6 +37,7 @@ MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
 WG, WAVE = 256, 64
+THIN_MIN_ROWS, THIN_ROWS_FOR_LANE_PER_ROW = 32, 65536
 LIF_POP_ENABLED, LIF_POP_DECAY = 1 << 8, 1 << 9  # flag bits of a population row
 LIF_COMPACT = os.environ.get("NENGO_HIP_LIF_COMPACT", "1") != "0"
 
@@ -93,6 +94,7 @@ class gemv_prog:
                  tile_items=()):
         self.queue = queue
         self.tile_items = frozenset(tile_items)  # items that take the large-item kernel regardless
+        self._many_thin_rows = False
         self.A, self.A_js, self.X, self.X_js = A, A_js, X, X_js
         self.Y = Y
         self.Y_in = Y if Y_in is None else Y_in
@@ -196,6 +198,8 @@ class gemv_prog:
         if flavor is None:
             # default: the reference's summation order, bit for bit -- small items one
             # wave per task, large items staged through LDS by a work-group
+            if dots and n_max <= 4 and M >= THIN_MIN_ROWS and self._many_thin_rows:
+                return (2, 1, 1)  # a lane per row: vector sums, scalar-times-vector terms
             if M * n_sum <= SMALL_ITEM_ELEMS and n_max <= REF_ORDER_MAX_COLS:
                 return (2, 4, 1)
             pow2 = vec == 4 and all(
@@ -278,6 +282,17 @@ class gemv_prog:
                                  lib.nhip_gemv_tile_rows(n, TILE_STAGE_WORDS), log2_n, 0))
         dot_tab = np.array(dot_rows or [(0,) * 8], dtype=np.int32)
 
+        # Items whose dot products have at most four columns (sums of vectors, scalar
+        # times vector) can give every row a lane of its own: consecutive lanes then
+        # read consecutive elements and share the item's records.  That pays when there
+        # is enough of it to be a throughput problem (c2's 2048 x 100 encoders: 10.2 ->
+        # 6.7 us); a few thousand rows are latency bound and better spread over more
+        # waves, four lanes per row (c3's 254 x 64 input sums: 7.9 vs 8.8 us).
+        thin_rows = sum(geometry[b]["y_len"] for b in items
+                        if geometry[b]["dots"] and geometry[b]["y_len"] >= THIN_MIN_ROWS
+                        and max(d["a_shape1"] for d in geometry[b]["dots"]) <= 4)
+        self._many_thin_rows = thin_rows >= THIN_ROWS_FOR_LANE_PER_ROW
+
         by_class = defaultdict(list)
         for b in items:
             if geometry[b]["y_len"] > 0:
@@ -296,7 +311,7 @@ class gemv_prog:
             elif flavor == 0:
                 rows = lib.nhip_gemv_rows_per_task(flavor, lpr, vec, passes)
             elif flavor == 2:
-                rows = WAVE // lpr  # one pass: these items are latency bound, spread them
+                rows = 1  # a task is one row; a wave packs 64 / lpr of them, of any items
             else:
                 rows = (WAVE // lpr) * 4  # four passes of a wave
             if rows is not None and rows <= 0:
@@ -305,14 +320,26 @@ class gemv_prog:
                 task_rows = self._tile_tasks(members)
             else:
                 task_rows = []
-                for b in members:
+                for b in (members if flavor != 2 else ()):
                     M = geometry[b]["y_len"]
                     for r0 in range(0, M, rows):
                         task_rows.append((b, r0, min(rows, M - r0), 0))
+            if flavor == 2:  # built with numpy: there can be millions of rows
+                counts = np.array([geometry[b]["y_len"] for b in members], dtype=np.int64)
+                task_tab = np.zeros((int(counts.sum()), 4), dtype=np.int32)
+                task_tab[:, 0] = np.repeat(np.array(members, dtype=np.int32), counts)
+                task_tab[:, 1] = np.arange(int(counts.sum())) - np.repeat(np.cumsum(counts) - counts, counts)
+                task_tab[:, 2] = 1
+                task_rows = task_tab
             task_tab = np.array(task_rows, dtype=np.int32)
             dev_tasks = to_device(self.queue, task_tab)
             n_tasks = len(task_rows)
-            n_groups = n_tasks if flavor == 0 else -(-n_tasks // (WG // WAVE))
+            if flavor == 0:
+                n_groups = n_tasks
+            elif flavor == 2:
+                n_groups = -(-n_tasks // ((WG // WAVE) * (WAVE // lpr)))
+            else:
+                n_groups = -(-n_tasks // (WG // WAVE))
             tail = (dev_items.ptr, dev_coefs.ptr, dev_dots.ptr, dev_tasks.ptr, n_tasks, self.A.ptr,
                     self.X.ptr, self.Y_in.ptr, self.Y.ptr)
             if flavor == 3:

@@ -562,3 +562,31 @@ def test_sparse_products(queue):
         assert np.array_equal(dY.to_host().buf, Yo.buf)
     with pytest.raises(ValueError):
         hipra_spmv.plan_sparse_dot_inc(queue, mats[:2], dX[[0, 2]], dY[[0, 1]])
+
+
+def test_thin_items_lane_per_row(queue):
+    """Many rows of dot products with one to four columns take the lane-per-row class:
+    bit-identical to the oracle for sums of several such terms, strided operands and
+    a scalar X shared by all rows."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(17)
+    shapes = [(40000, 1), (30000, 4), (5000, 3), (33, 2)]
+    A = RA([rng.normal(size=s) for s in shapes] + [rng.normal(size=(40000, 1)) for _ in range(5)],
+           align=True)
+    X = RA([rng.normal(size=s[1]) for s in shapes] + [rng.normal(size=1) for _ in range(5)],
+           align=True)
+    Y = RA([rng.normal(size=s[0]) for s in shapes] + [rng.normal(size=40000)], align=True)
+    n = len(shapes)
+    js = [np.array([i], dtype=np.int32) for i in range(n)] + [np.arange(n, n + 5, dtype=np.int32)]
+    for beta, gamma in ((1.0, 0.0), (0.0, 0.25)):
+        Yo = clone(Y)
+        orc.plan_block_gemv(None, 1.0, A, js, X, js, beta, Yo, gamma=gamma).plans[0]()
+        dY = to_dev(queue, Y)
+        prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY,
+                                 gamma=gamma)
+        assert {p.kernel_class for p in prog.plans} == {(2, 1, 1)}
+        for plan in prog.plans:
+            plan()
+        assert np.array_equal(dY.buf, Yo.buf)
