@@ -25,6 +25,7 @@
 // + 4*LPR ...), so one load instruction of a wave covers contiguous memory.
 #include "nhip_common.h"
 #include "gemv_types.h"
+#include "gemv_rows.h"
 
 namespace {
 
@@ -222,99 +223,15 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
 }
 
 // ---------------------------------------------------------------- reference order, small items
-// One output row per task (task = {item, row, 1, 0}); a wave takes 64 / LPR
-// consecutive tasks, LPR lanes each, whatever items they belong to -- thousands of
-// one-row items (decoders of small populations) fill waves as well as a few tall ones.
-// Sums are formed in the order of the reference's block kernel (clra_gemv.py:1043-1058,
-// :1148-1153): per 128-column tile four strided partial sums, one fused multiply-add
-// per element, (s0+s2)+(s1+s3), tiles in order onto beta*y_in, gamma last.
-//   LPR = 4: lane j of a row carries partial sum j; any number of columns.
-//   LPR = 1: one lane per row, for items whose dot products all have <= 4 columns
-//            (vector sums, "scalar times vector" increments): the four partial sums are
-//            the (up to) four products themselves.
-// These launches are latency bound: the records of four dot products and, when those
-// have at most four columns, all their operands are fetched together before the sums
-// are formed in order.  Task, item and dot records are per-lane values on purpose
-// (different rows of a wave may belong to different items).
+// (the kernel body lives in gemv_rows.h, shared with the sequence kernel)
 template <int LPR>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
-    const float* __restrict__ A, const float* __restrict__ X, const float* Yin, float* Y)
+    const float* A, const float* X, const float* Yin, float* Y)
 {
-    constexpr int TILE = 128;
-    constexpr int BATCH = 4;             // dot products whose operands are fetched together
-    constexpr int ROWS = NHIP_WAVE / LPR;  // rows (tasks) per wave
-    constexpr int PER_LANE = 4 / LPR;    // elements of a <= 4 column dot product per lane
-    const int lane = threadIdx.x & (NHIP_WAVE - 1);
-    const int lir = lane % LPR;
-    const int slot = (blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6)) * ROWS + lane / LPR;
-    const bool valid = slot < n_tasks;
-    const GemvTask task = tasks[valid ? slot : n_tasks - 1];
-    const GemvItem it = items[task.item];
-    const float4 cf = coefs[task.item];
-    const int r = task.row0;
-    const int n_dots = valid ? it.n_dots : 0;
-    float sum = cf.y * Yin[it.yin_start + (size_t)r * it.yin_stride0];
-
-    for (int d0 = 0; __any(d0 < n_dots); d0 += BATCH) {
-        GemvDot dot[BATCH];
-        bool tiny = true;
-#pragma unroll
-        for (int k = 0; k < BATCH; ++k) {
-            dot[k] = dots[d0 + k < n_dots ? it.dot_begin + d0 + k : 0];
-            tiny = tiny && (d0 + k >= n_dots || dot[k].N <= 4);
-        }
-        if (LPR == 1 || __all(tiny)) {
-            float a[BATCH][PER_LANE], x[BATCH][PER_LANE];
-#pragma unroll
-            for (int k = 0; k < BATCH; ++k)
-#pragma unroll
-                for (int e = 0; e < PER_LANE; ++e) {
-                    const int c = lir + e * LPR;
-                    const bool live = d0 + k < n_dots && c < dot[k].N;
-                    a[k][e] = live ? A[dot[k].a_start + (size_t)r * dot[k].a_stride0 + c] : 0.0f;
-                    x[k][e] = live ? X[dot[k].x_start + (size_t)c * dot[k].x_stride0] : 0.0f;
-                }
-#pragma unroll
-            for (int k = 0; k < BATCH; ++k) {
-                float s;
-                if (LPR == 4) {
-                    s = lir < dot[k].N ? fmaf(a[k][0], x[k][0], 0.0f) : 0.0f;
-                    s = s + __shfl_xor(s, 2, NHIP_WAVE);
-                    s = s + __shfl_xor(s, 1, NHIP_WAVE);
-                } else {
-                    float p[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        p[e] = e < dot[k].N ? fmaf(a[k][e % PER_LANE], x[k][e % PER_LANE], 0.0f) : 0.0f;
-                    s = (p[0] + p[2]) + (p[1] + p[3]);
-                }
-                if (d0 + k < n_dots) sum = sum + cf.x * s;
-            }
-            continue;
-        }
-        if (LPR == 4) {
-#pragma unroll
-            for (int k = 0; k < BATCH; ++k) {  // static indices keep the records in registers
-                if (!__any(d0 + k < n_dots)) break;
-                const bool have = d0 + k < n_dots;
-                const int n_cols = have ? dot[k].N : 0;
-                const float* arow = A + dot[k].a_start + (size_t)r * dot[k].a_stride0;
-                const float* xg = X + dot[k].x_start;
-                const size_t xs = (size_t)dot[k].x_stride0;
-                for (int c0 = 0; c0 < n_cols; c0 += TILE) {
-                    const int c1 = min(c0 + TILE, n_cols);
-                    float s = 0.0f;
-                    for (int c = c0 + lir; c < c1; c += 4) s = fmaf(arow[c], xg[(size_t)c * xs], s);
-                    s = s + __shfl_xor(s, 2, NHIP_WAVE);
-                    s = s + __shfl_xor(s, 1, NHIP_WAVE);
-                    sum = sum + cf.x * s;
-                }
-            }
-        }
-    }
-    if (lir == 0 && valid) Y[it.y_start + (size_t)r * it.y_stride0] = sum + cf.z;
+    gemv_rows_ref_block<LPR>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y, blockIdx.x,
+                             threadIdx.x);
 }
 
 template <int LPR, int VEC, int P>

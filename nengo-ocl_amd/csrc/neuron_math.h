@@ -61,6 +61,49 @@ __device__ __forceinline__ bool lif_step(float j, float& v, float& w, float tau,
     return spiked;
 }
 
+// Work-list rows of the neuron kernels: a block of <= 512 neurons of one population.
+struct LifDesc {
+    int j_start, v_start, w_start, s_start;
+    int count, tau, ref, amp;  // tau/ref/amp: float bits, or element offsets (see pflags)
+    int pflags, p0, p1, p2;    // bit 0/1/2: tau/ref/amp is a per-neuron vector
+};
+struct RateDesc { int j_start, r_start, count, tau, ref, amp, pflags, pad; };
+
+// One thread per neuron; the update itself is `lif_step`.  dtu = dt / upsample.
+__device__ __forceinline__ void lif_block(const LifDesc d, float dtu, float dt_inv, int upsample,
+                                          const float* J, float* V, float* W, float* S,
+                                          const float* __restrict__ TAU,
+                                          const float* __restrict__ REF,
+                                          const float* __restrict__ AMP, int tid) {
+    for (int i = tid; i < d.count; i += NHIP_WG) {
+        const float j = J[(size_t)d.j_start + i];
+        float v = V[(size_t)d.v_start + i];
+        float w = W[(size_t)d.w_start + i];
+        const float tau = lif_param(d.tau, d.pflags & 1, TAU, i);
+        const float ref = lif_param(d.ref, d.pflags & 2, REF, i);
+        const float amp = lif_param(d.amp, d.pflags & 4, AMP, i);
+        const bool spiked = lif_step(j, v, w, tau, ref, dtu, upsample);
+        V[(size_t)d.v_start + i] = v;
+        W[(size_t)d.w_start + i] = w;
+        S[(size_t)d.s_start + i] = spiked ? __fmul_rn(amp, dt_inv) : 0.0f;
+    }
+}
+
+// clra_nonlinearities.py:1174-1184: J <= 1 gives 1/0 = inf, log1p(inf) = inf, amp/inf = 0.
+__device__ __forceinline__ void lif_rate_block(const RateDesc d, const float* J, float* R,
+                                               const float* __restrict__ TAU,
+                                               const float* __restrict__ REF,
+                                               const float* __restrict__ AMP, int tid) {
+    for (int i = tid; i < d.count; i += NHIP_WG) {
+        const float tau = lif_param(d.tau, d.pflags & 1, TAU, i);
+        const float ref = lif_param(d.ref, d.pflags & 2, REF, i);
+        const float amp = lif_param(d.amp, d.pflags & 4, AMP, i);
+        const float j = fmaxf(J[(size_t)d.j_start + i] - 1.0f, 0.0f);
+        const float denom = __fadd_rn(ref, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(1.0f, j))));
+        R[(size_t)d.r_start + i] = __fdiv_rn(amp, denom);
+    }
+}
+
 // LIF update of neuron i of population p with input current j (GEMV epilogue);
 // v and w are the neuron's voltage and refractory time, read earlier
 __device__ __forceinline__ void lif_epilogue(const LifArgs& a, const LifPop& p, int i, float j,

@@ -6,52 +6,23 @@
 
 namespace {
 
-struct LifDesc {
-    int j_start, v_start, w_start, s_start;
-    int count, tau, ref, amp;  // tau/ref/amp: float bits, or element offsets (see pflags)
-    int pflags, p0, p1, p2;    // bit 0/1/2: tau/ref/amp is a per-neuron vector
-};
-
-// One thread per neuron; the update itself is `lif_step` (neuron_math.h).
+// (LifDesc, RateDesc and the block functions lif_block / lif_rate_block live in
+// neuron_math.h: the sequence kernel runs them too)
 __global__ __launch_bounds__(NHIP_WG) void lif_kernel(const LifDesc* __restrict__ desc, float dt,
                                                       float dt_inv, int upsample, const float* J,
                                                       float* V, float* W, float* S,
                                                       const float* __restrict__ TAU,
                                                       const float* __restrict__ REF,
                                                       const float* __restrict__ AMP) {
-    const LifDesc d = desc[blockIdx.x];
-    const float dtu = dt;  // already divided by upsample on the host, in double
-    for (int i = threadIdx.x; i < d.count; i += NHIP_WG) {
-        const float j = J[(size_t)d.j_start + i];
-        float v = V[(size_t)d.v_start + i];
-        float w = W[(size_t)d.w_start + i];
-        const float tau = lif_param(d.tau, d.pflags & 1, TAU, i);
-        const float ref = lif_param(d.ref, d.pflags & 2, REF, i);
-        const float amp = lif_param(d.amp, d.pflags & 4, AMP, i);
-        const bool spiked = lif_step(j, v, w, tau, ref, dtu, upsample);
-        V[(size_t)d.v_start + i] = v;
-        W[(size_t)d.w_start + i] = w;
-        S[(size_t)d.s_start + i] = spiked ? __fmul_rn(amp, dt_inv) : 0.0f;
-    }
+    lif_block(desc[blockIdx.x], dt, dt_inv, upsample, J, V, W, S, TAU, REF, AMP, threadIdx.x);
 }
 
-struct RateDesc { int j_start, r_start, count, tau, ref, amp, pflags, pad; };
-
-// clra_nonlinearities.py:1174-1184: J <= 1 gives 1/0 = inf, log1p(inf) = inf, amp/inf = 0.
 __global__ __launch_bounds__(NHIP_WG) void lif_rate_kernel(const RateDesc* __restrict__ desc,
                                                            const float* J, float* R,
                                                            const float* __restrict__ TAU,
                                                            const float* __restrict__ REF,
                                                            const float* __restrict__ AMP) {
-    const RateDesc d = desc[blockIdx.x];
-    for (int i = threadIdx.x; i < d.count; i += NHIP_WG) {
-        const float tau = lif_param(d.tau, d.pflags & 1, TAU, i);
-        const float ref = lif_param(d.ref, d.pflags & 2, REF, i);
-        const float amp = lif_param(d.amp, d.pflags & 4, AMP, i);
-        const float j = fmaxf(J[(size_t)d.j_start + i] - 1.0f, 0.0f);
-        const float denom = __fadd_rn(ref, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(1.0f, j))));
-        R[(size_t)d.r_start + i] = __fdiv_rn(amp, denom);
-    }
+    lif_rate_block(desc[blockIdx.x], J, R, TAU, REF, AMP, threadIdx.x);
 }
 
 // ---------------------------------------------------------------- further neuron types

@@ -590,3 +590,39 @@ def test_thin_items_lane_per_row(queue):
         for plan in prog.plans:
             plan()
         assert np.array_equal(dY.buf, Yo.buf)
+
+
+@pytest.mark.parametrize("inc, long_row, sparsity, shape", [
+    (True, False, 0.02, 511), (False, False, 0.1, 511), (False, False, 0.02, 5000),
+    (False, True, 0.02, 5000), (True, False, 0.1, 5000), (False, False, 0.02, (2047, 5007)),
+    (True, True, 0.07, (2048, 5003)), (True, False, 0.02, (2057, 5981)),
+    (False, False, 0.02, (1, 4999)), (False, False, 0.02, (5001, 1))])
+def test_sparse_reference_cases(queue, rng, inc, long_row, sparsity, shape):
+    """The cases of the reference's test_sparse (tests/test_clra_gemv.py:383-462): random
+    masks, optionally ten rows with a run of 1025 entries, set and increment; checked
+    like there against scipy's product, and bit for bit against the oracle."""
+    import scipy.sparse as sp
+
+    from nengo_ocl_amd import hipra_spmv
+    from oracle import oracle as orc
+
+    shape = (shape, shape) if isinstance(shape, int) else shape
+    mask = rng.uniform(size=shape) < sparsity
+    if long_row:
+        rows = np.unique(rng.randint(0, shape[0], size=10))
+        mask[rows, :min(1025, shape[1])] = True
+    ii, jj = mask.nonzero()
+    assert len(ii) > 0
+    A = sp.coo_matrix((rng.uniform(0, 1, size=len(ii)), (ii, jj)), shape=shape)
+    X = RA([rng.uniform(0, 1, size=shape[1])])
+    Y = RA([rng.uniform(0, 1, size=shape[0])])
+    dX, dY = to_dev(queue, X), to_dev(queue, Y)
+    prog = hipra_spmv.plan_sparse_dot_inc(queue, hipra_spmv.HostSparseMatrix(A.tocsr()), dX, dY, inc=inc)
+    for plan in prog.plans:
+        plan()
+    ref = (Y[0][:, 0].astype(np.float64) if inc else 0) + A.astype(np.float64).dot(X[0][:, 0].astype(np.float64))
+    got = dY.to_host()[0][:, 0]
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5)
+    Yo = clone(Y)
+    orc.plan_sparse_dot_inc(None, A.tocsr(), X, Yo, inc=inc).plans[0]()
+    assert np.array_equal(got, Yo[0][:, 0])
