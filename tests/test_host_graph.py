@@ -15,17 +15,24 @@ from nengo_ocl_amd.planners import batching_planner, greedy_planner, operator_de
 from oracle.oracle_sim import OracleSimulator
 
 
+def golden(name):
+    import json
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                        "reference_test_vectors.json")
+    with open(path) as f:
+        return json.load(f)[name]
+
+
 def literal_model():
-    a = ir.Signal([0, 0], name="a")
-    b = ir.Signal([0, 0], name="b")
-    A = ir.Signal([[1, 2], [0, 1]], name="A")
-    B = ir.Signal([[2, 1], [-1, 1]], name="B")
-    x = ir.Signal([1, 1], name="x")
-    y = ir.Signal([1, -1], name="y")
+    """The operator graph of the fixture multidotinc_compress (tests/test_simulator.py:14-38)."""
+    g = golden("multidotinc_compress")
+    sig = {name: ir.Signal(value, name=name) for name, value in g["signals"].items()}
     m = ir.Model(dt=0.001)
-    m.operators += [ir.Reset(a), ir.DotInc(A, x, a), ir.DotInc(B, y, a)]
-    m.operators += [ir.DotInc(A, y, b), ir.DotInc(B, x, b)]
-    return m, a, b
+    for kind, *names in g["operators"]:
+        m.operators.append(getattr(ir, kind)(*[sig[n] for n in names]))
+    return m, sig["a"], sig["b"]
 
 
 @pytest.mark.parametrize("fuse", [True, False])
@@ -35,12 +42,10 @@ def test_multidotinc_compress_literal(fuse):
     with OracleSimulator(None, model=m, fuse=fuse) as sim:
         n_mdi = sum(isinstance(op, MultiDotInc) for op in sim.operators)
         assert n_mdi == 2  # four DotIncs folded onto two targets
-        sim.step()
-        assert np.allclose(sim.signals[a], [4, -1])
-        assert np.allclose(sim.signals[b], [2, -1])
-        sim.step()
-        assert np.allclose(sim.signals[a], [4, -1])
-        assert np.allclose(sim.signals[b], [4, -2])
+        for expect in golden("multidotinc_compress")["expected_after_step"]:
+            sim.step()
+            assert np.allclose(sim.signals[a], expect["a"])
+            assert np.allclose(sim.signals[b], expect["b"])
 
 
 def test_get_views_scalar_swap_and_shapes():

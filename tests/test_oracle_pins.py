@@ -15,16 +15,25 @@ from oracle import oracle as orc
 
 
 # ------------------------------------------------------------------ GEMV
+def golden(name):
+    import json
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                        "reference_test_vectors.json")
+    with open(path) as f:
+        return json.load(f)[name]
+
+
 def test_gemv_literal_vectors():
-    """nengo_ocl/tests/test_clra_gemv.py:60-93: Y0 = 4.5, Y1 = [3.3, 5.9]."""
-    A = RA([[[0.1, 0.2], [0.3, 0.4]], [[0.5, 0.6]]])
-    X = RA([[3, 5]])
-    Y = RA([[0.0], [2, 3]])
-    A_js = RA([[1], [0]], dtype=np.int32)
-    X_js = RA([[0], [0]], dtype=np.int32)
-    orc.plan_block_gemv(None, 1.0, A, A_js, X, X_js, 1.0, Y).plans[0]()
-    np.testing.assert_allclose(Y[0].ravel(), [4.5], rtol=1e-6)
-    np.testing.assert_allclose(Y[1].ravel(), [3.3, 5.9], rtol=1e-6)
+    """nengo_ocl/tests/test_clra_gemv.py:60-93 (fixture gemv_basic): Y0 = 4.5, Y1 = [3.3, 5.9]."""
+    g = golden("gemv_basic")
+    A, X, Y = RA(g["A"]), RA(g["X"]), RA(g["Y"])
+    A_js = RA(g["A_js"], dtype=np.int32)
+    X_js = RA(g["X_js"], dtype=np.int32)
+    orc.plan_block_gemv(None, g["alpha"], A, A_js, X, X_js, g["beta"], Y).plans[0]()
+    for i, want in enumerate(g["expected_Y"]):
+        np.testing.assert_allclose(Y[i].ravel(), want, rtol=1e-6)
 
 
 @pytest.mark.parametrize("k,p,m,n", [(4, 1, 10, 10), (10, 1, 550, 550), (4, 4, 10, 10),
