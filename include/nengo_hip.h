@@ -94,6 +94,11 @@ int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
  * bit-identical to a float32 restatement of that kernel while HBM is still read in
  * whole lines.  nhip_gemv_tile_rows(N, blk_words) = rows of a dot product with N
  * columns that fit one LDS block (a power of two; goes into the dots table).
+ * The task table of these entry points is wider than nhip_gemv's, so that a wave
+ * starts streaming after one read:
+ *   tasks : int32[n_tasks][24] {item, row0, n_rows, 0,  the item's row of `items` (8),
+ *                               alpha, beta, gamma (float bits), 0,
+ *                               the item's first row of `dots` (8; zeros without dots)}
  * `vec` as for nhip_gemv.  `pow2_cols` = 1 selects the streamlined kernel for
  * launches in which every dot product has a power-of-two column count >= 4
  * (log2_N set), vec == 4 and a_stride0 < 2^22; 0 = any shape. */

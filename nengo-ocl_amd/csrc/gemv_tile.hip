@@ -108,7 +108,7 @@ struct Stage {
 template <int VEC, int EPI>
 __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
-    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
     float* Y, EpilogueArgs epi)
 {
@@ -124,9 +124,10 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     const int t = nhip_xcd_remap(blockIdx.x, gridDim.x) * (NHIP_WG / NHIP_WAVE) + wave;
     if (t >= n_tasks) return;  // wave-uniform; the kernel has no group barrier
 
-    const GemvTask task = tasks[t];
-    const GemvItem it = items[task.item];
-    const float4 cf = coefs[task.item];
+    const GemvFatTask ft = tasks[t];
+    const GemvTask task = ft.task;
+    const GemvItem it = ft.item;
+    const float4 cf = make_float4(ft.alpha, ft.beta, ft.gamma, 0.0f);
     const int n_rows = task.n_rows;
 
     // lane l carries the running sums of rows l, l + 64, ... of the task
@@ -146,7 +147,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
         s.b = 0;
         s.rb = 1;
         if (s.d >= 0) {
-            s.dot = dots[it.dot_begin];
+            s.dot = ft.dot0;
             s.rb = s.dot.p0;
         }
         return s;
@@ -465,7 +466,7 @@ struct P2Stage {
 template <int EPI>
 __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
-    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int blk_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
     float* Y, EpilogueArgs epi)
 {
@@ -482,9 +483,10 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     const int t = nhip_xcd_remap(blockIdx.x, gridDim.x) * (NHIP_WG / NHIP_WAVE) + wave;
     if (t >= n_tasks) return;  // wave-uniform; the kernel has no group barrier
 
-    const GemvTask task = tasks[t];
-    const GemvItem it = items[task.item];
-    const float4 cf = coefs[task.item];
+    const GemvFatTask ft = tasks[t];
+    const GemvTask task = ft.task;
+    const GemvItem it = ft.item;
+    const float4 cf = make_float4(ft.alpha, ft.beta, ft.gamma, 0.0f);
     const int n_rows = task.n_rows;
 
 #pragma unroll
@@ -517,7 +519,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
         s.d = it.n_dots > 0 ? 0 : -1;
         s.c0 = 0;
         s.b = 0;
-        if (s.d >= 0) s.dot = dots[it.dot_begin];
+        if (s.d >= 0) s.dot = ft.dot0;
         return s;
     };
     auto next_stage = [&](const P2Stage& s) {
@@ -732,7 +734,7 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
                            reinterpret_cast<const GemvItem*>(items),
                            reinterpret_cast<const float4*>(coefs),
                            reinterpret_cast<const GemvDot*>(dots),
-                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, blk_words, A, X, Yin,
+                           reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, blk_words, A, X, Yin,
                            Y, args);
     };
     auto launch_epi = [&](auto epi_tag) {

@@ -5,3 +5,14 @@
 struct GemvItem { int y_start, y_stride0, yin_start, yin_stride0, dot_begin, n_dots, M, pad; };
 struct GemvDot { int a_start, a_stride0, N, x_start, x_stride0, p0, p1, p2; };
 struct GemvTask { int item, row0, n_rows, pad; };
+
+// Task record of the large-item kernels: everything a wave needs to start streaming
+// in ONE read -- the task, its item, the item's coefficients and the item's first dot
+// product (zeros if it has none).  Read one after the other from their own tables,
+// these are three dependent cold reads before the first matrix load can be issued.
+struct GemvFatTask {
+    GemvTask task;
+    GemvItem item;
+    float alpha, beta, gamma, pad;
+    GemvDot dot0;
+};

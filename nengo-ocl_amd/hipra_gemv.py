@@ -332,6 +332,17 @@ class gemv_prog:
                 task_tab[:, 2] = 1
                 task_rows = task_tab
             task_tab = np.array(task_rows, dtype=np.int32)
+            if flavor == 3:
+                # one record per task with its item, coefficients and first dot product
+                # inline: a wave starts streaming after one read instead of three
+                which = task_tab[:, 0]
+                fat = np.zeros((len(task_tab), 24), dtype=np.int32)
+                fat[:, 0:4] = task_tab
+                fat[:, 4:12] = item_tab[which]
+                fat[:, 12:16] = coef_tab[which].view(np.int32)
+                has_dots = item_tab[which, 5] > 0
+                fat[has_dots, 16:24] = dot_tab[item_tab[which[has_dots], 4]]
+                task_tab = fat
             dev_tasks = to_device(self.queue, task_tab)
             n_tasks = len(task_rows)
             if flavor == 0:
