@@ -113,6 +113,8 @@ def to_device(queue, array, dtype=None):
     """Upload a host array; returns a `DeviceArray` of the same shape."""
     torch = _torch()
     array = np.ascontiguousarray(array, dtype=dtype)
+    if not array.flags.writeable:  # read-only views (metadata rows): torch wants its own copy
+        array = array.copy()
     if array.dtype not in (np.dtype(np.float32), np.dtype(np.int32)):
         raise TypeError("device arrays are float32 or int32, got %s" % array.dtype)
     with queue.context():

@@ -343,3 +343,28 @@ def test_sparse_recurrent_population(queue):
         assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
         rates = gpu.data[probes["spikes"]][-1]
         assert rates.max() > 50 and rates.std() > 10  # the recurrence shapes the activity
+
+
+def test_profiling_and_plan_listing(queue, capsys):
+    """`profiling=True` times every launch with events (one row per plan: calls, seconds,
+    GF/s, GB/s), `print_plans` lists the launches of a step; results are unchanged."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+
+    make = lambda: configs.c3_large(n_ens=4, n_neurons=512, dims=32, fan_out=2, solver="lstsq")
+    net, probes, _ = make()
+    net2, probes2, _ = make()
+    with Simulator(net, seed=1, profiling=True) as prof, Simulator(net2, seed=1) as plain:
+        prof.run_steps(40)
+        plain.run_steps(40)
+        for k in probes:
+            assert np.array_equal(prof.data[probes[k]], plain.data[probes2[k]])
+        table = prof.profiling_table()
+        assert len(table) == len(prof._plans)
+        assert all(row[0] == 40 and row[1] > 0 for row in table)
+        gemv_rows = [row for row in table if "hipra_gemv.tile" in row[4]]
+        assert gemv_rows and all(row[3] > 0 for row in gemv_rows)  # GB/s is reported
+        prof.print_profiling(sort=1)
+        prof.print_plans()
+        out = capsys.readouterr().out
+        assert "Profiling" in out and "hipra_gemv.tile_lif" in out and "totals:" in out
