@@ -222,6 +222,65 @@ int nhip_linearfilter(void *stream, const int *desc, int *pos, int n_blocks, con
  *          count, alpha_bits, flags(bit0 outer, bit1 inc), 0} */
 int nhip_elementwise_inc(void *stream, const int *desc, int n_blocks, const float *A,
                          const float *X, float *Y);
+/* Weight-update rules that write a delta matrix per connection (row i = post
+ * neuron, column j = pre element; delta rows are contiguous):
+ *   BCM  delta[i,j] = alpha * post[i] * (post[i] - theta[i]) * pre[j]
+ *   OJA  delta[i,j] = alpha * post[i] * (pre[j] - beta * weights[i,j] * post[i])
+ *   VOJA delta[i,j] = alpha * learn * post[i] * (scale[i] * pre[j] - enc[i,j])
+ * each product and difference rounded separately, left to right.
+ * replaces: `plan_bcm` (:2082-2169), `plan_oja` (:2172-2277), `plan_voja`
+ * (:2280-2405).  AUX is theta (vector), weights or encoders (matrix, rows
+ * contiguous); LEARN and SCALE are read by VOJA only.
+ *   desc : int32[n_blocks][16] {pre_start, pre_stride0, post_start, post_stride0,
+ *          aux_start, aux_stride0, delta_start, delta_stride0, shape1, offset,
+ *          count, alpha_bits, beta_bits, learn_start, scale_start, scale_stride0} */
+#define NHIP_RULE_BCM 1
+#define NHIP_RULE_OJA 2
+#define NHIP_RULE_VOJA 3
+int nhip_learning_rule(void *stream, int rule, const int *desc, int n_blocks, const float *PRE,
+                       const float *POST, const float *AUX, float *DELTA, const float *LEARN,
+                       const float *SCALE);
+/* ---- convolution, pooling -------------------------------------------------
+ * Y = conv2d(X, F) over one image signal (Y is set, not incremented, like the
+ * reference's kernel), or local filtering (one filter bank per output pixel).
+ * replaces: `plan_conv2d` (:1762-1969; biases unsupported there too).
+ *   geom : HOST int32[21] {nxi, nxj, nc, nyi, nyj, nf, si, sj, sti, stj, pi, pj,
+ *          x_start, y_start, f_start, channels_last, local, tile_i, tile_j,
+ *          tile_f, c_chunk}
+ * X is (nxi, nxj, nc) with channels last, else (nc, nxi, nxj); Y likewise with nf;
+ * F is (si, sj, nc, nf), or for local filtering (nf, nc, si, sj, nyi, nyj).  A group
+ * computes tile_i x tile_j output pixels x tile_f filters (product <= 256) and
+ * stages c_chunk channels of the input patch in LDS at a time (<= 48 KiB).  Each
+ * output is accumulated over channel, kernel row, kernel column in that order with
+ * one fused multiply-add per term. */
+int nhip_conv2d(void *stream, const int *geom, const float *X, const float *F, float *Y);
+/* Average pooling, channels first; window elements outside the image (bottom /
+ * right edge) and NaN inputs are left out of the mean.
+ * replaces: `plan_pool2d` (:1972-2079).
+ *   geom : HOST int32[11] {nc, nyi, nyj, nxi, nxj, si, sj, sti, stj, x_start, y_start} */
+int nhip_pool2d(void *stream, const int *geom, const float *X, float *Y);
+
+/* ---- white noise -----------------------------------------------------------
+ * Y[item] (=|+=) a fresh sample per element, from Uniform(p0, p1) or
+ * Gaussian(mean p0, std p1), times sqrt_dt_inv where flagged.
+ * replaces: `plan_whitenoise`, `init_rngs`, `create_rngs` (:1486-1675).  The
+ * reference draws from RANLUX states in device memory; this library uses the
+ * counter-based Philox4x32-10 generator: the block of four 32-bit words for
+ * elements 4q..4q+3 of call n is philox(counter {q, n, 0, 0}, key {seed, 0}), so
+ * the sample streams are not the reference's (whose streams are not nengo's
+ * either), and the only state is the per-item call count.
+ *   desc     : int32[n_items][8] {y_start, count, dist, p0_bits, p1_bits,
+ *                                 flags(bit0 scale, bit1 inc), seed, 0}
+ *   counters : int32[n_items], read and advanced by one per call (zero them to
+ *              restart the streams) */
+#define NHIP_DIST_UNIFORM 0
+#define NHIP_DIST_GAUSSIAN 1
+int nhip_whitenoise(void *stream, const int *desc, int n_items, int *counters,
+                    double sqrt_dt_inv, float *Y);
+/* out[t] = philox4x32_10(counter = in[t][0..3], key = in[t][4..5]) for n blocks
+ * (known-answer testing of the generator). */
+int nhip_philox4x32(void *stream, const unsigned *counters_keys, unsigned *out, int n);
+
 /* 2-D strided Y (=|+=) X.  replaces: `plan_copy` (:217-304).
  *   desc : int32[n_blocks][8] {x_start, y_start, shape1, x_stride0, y_stride0,
  *                              offset, count, inc} */

@@ -595,3 +595,240 @@ def plan_presentinput(queue, Y, t, signals, dt, pres_t=None, tag=None):
                 name="hip_presentinput", tag=tag)
     plan.description = _description(Y)
     return plan
+
+
+# ---------------------------------------------------------------- learning rules
+RULE_BCM, RULE_OJA, RULE_VOJA = 1, 2, 3
+
+
+def _plan_rule(queue, rule, name, pre, post, aux, delta, alpha, beta=None, learn=None,
+               scale=None, flops_per_element=4, tag=None):
+    N = len(pre)
+    alpha = _host(alpha).astype(np.float32).reshape(-1)
+    beta = np.zeros(N, dtype=np.float32) if beta is None else _host(beta).astype(
+        np.float32).reshape(-1)
+    assert alpha.size == N and beta.size == N
+    operands = [("pre", pre), ("post", post), ("aux", aux), ("delta", delta)]
+    if rule == RULE_VOJA:
+        operands += [("learn", learn), ("scale", scale)]
+    _check(*operands)
+
+    inds, offsets, counts = blockify(delta.sizes)
+    zeros = np.zeros(len(inds), dtype=np.int32)
+    table, n = _dev_table(queue, [
+        pre.starts[inds], pre.stride0s[inds], post.starts[inds], post.stride0s[inds],
+        aux.starts[inds], aux.stride0s[inds], delta.starts[inds], delta.stride0s[inds],
+        delta.shape1s[inds], offsets, counts, _bits(alpha[inds]),
+        _bits(beta[inds]),
+        learn.starts[inds] if learn is not None else zeros,
+        scale.starts[inds] if scale is not None else zeros,
+        scale.stride0s[inds] if scale is not None else zeros], 16)
+    args = (rule, table.ptr, n, pre.ptr, post.ptr, aux.ptr, delta.ptr,
+            learn.ptr if learn is not None else None, scale.ptr if scale is not None else None)
+    keep = [table, pre.dev_buf, post.dev_buf, aux.dev_buf, delta.dev_buf]
+    keep += [ra.dev_buf for ra in (learn, scale) if ra is not None]
+    plan = Plan(queue, queue.lib.nhip_learning_rule, args, gsize=(WG * max(n, 1),), lsize=(WG,),
+                full_args=tuple(keep), name=name, tag=tag)
+    plan.flops_per_call = flops_per_element * int(delta.sizes.sum())
+    plan.bw_per_call = (sum(ra.nbytes for _, ra in operands) + alpha.nbytes
+                        + (beta.nbytes if rule == RULE_OJA else 0))
+    plan.description = _description(delta)
+    return plan
+
+
+def plan_bcm(queue, pre, post, theta, delta, alpha, tag=None):
+    """``delta = alpha * post * (post - theta) (outer) pre`` per connection
+    (reference ``plan_bcm`` :2082-2169)."""
+    assert len(pre) == len(post) == len(theta) == len(delta) == np.size(_host(alpha))
+    for arr in (pre, post, theta):  # vectors
+        assert (arr.shape1s == 1).all()
+    assert (delta.stride1s == 1).all()
+    assert (post.shape0s == delta.shape0s).all()
+    assert (pre.shape0s == delta.shape1s).all()
+    assert (post.shape0s == theta.shape0s).all()
+    assert pre.ctype == post.ctype == theta.ctype == delta.ctype == "float"
+    return _plan_rule(queue, RULE_BCM, "hip_bcm", pre, post, theta, delta, alpha,
+                      flops_per_element=4, tag=tag)
+
+
+def plan_oja(queue, pre, post, weights, delta, alpha, beta, tag=None):
+    """``delta = alpha * post * (pre - beta * weights * post)`` per connection
+    (reference ``plan_oja`` :2172-2277)."""
+    assert (len(pre) == len(post) == len(weights) == len(delta) == np.size(_host(alpha))
+            == np.size(_host(beta)))
+    for arr in (pre, post):  # vectors
+        assert (arr.shape1s == 1).all()
+    for arr in (delta, weights):  # matrices
+        assert (arr.stride1s == 1).all()
+    assert (post.shape0s == weights.shape0s).all()
+    assert (pre.shape0s == weights.shape1s).all()
+    assert (weights.shape0s == delta.shape0s).all()
+    assert (weights.shape1s == delta.shape1s).all()
+    assert pre.ctype == post.ctype == weights.ctype == delta.ctype == "float"
+    return _plan_rule(queue, RULE_OJA, "hip_oja", pre, post, weights, delta, alpha, beta=beta,
+                      flops_per_element=6, tag=tag)
+
+
+def plan_voja(queue, pre, post, enc, delta, learn, scale, alpha, tag=None):
+    """``delta = alpha * learn * post * (scale * pre - enc)`` per connection
+    (reference ``plan_voja`` :2280-2405)."""
+    assert (len(pre) == len(post) == len(enc) == len(delta) == len(learn)
+            == np.size(_host(alpha)) == len(scale))
+    assert (learn.shape0s == 1).all() and (learn.shape1s == 1).all()
+    for arr in (pre, post, scale):  # vectors
+        assert (arr.shape1s == 1).all()
+    for arr in (enc, delta):  # matrices
+        assert (arr.stride1s == 1).all()
+    assert (post.shape0s == enc.shape0s).all()
+    assert (pre.shape0s == enc.shape1s).all()
+    assert (enc.shape0s == delta.shape0s).all()
+    assert (enc.shape1s == delta.shape1s).all()
+    assert (scale.shape0s == enc.shape0s).all()
+    assert (pre.ctype == post.ctype == enc.ctype == delta.ctype == learn.ctype
+            == scale.ctype == "float")
+    return _plan_rule(queue, RULE_VOJA, "hip_voja", pre, post, enc, delta, alpha, learn=learn,
+                      scale=scale, flops_per_element=5, tag=tag)
+
+
+# ---------------------------------------------------------------- convolution, pooling
+def _single_contiguous(ra, what):
+    """(start, size) of a one-item ragged view whose item is one contiguous run."""
+    assert len(ra) == 1, "%s: one signal expected" % what
+    m, n = int(ra.shape0s[0]), int(ra.shape1s[0])
+    assert ra.stride1s[0] == 1 or n == 1, "%s: not contiguous" % what
+    assert ra.stride0s[0] == n or m == 1, "%s: not contiguous" % what
+    return int(ra.starts[0]), m * n
+
+
+def conv2d_tiles(shape_out_ijf, kernel_shape, strides, nc, channels_last):
+    """Output tile (rows, columns, filters) of one work-group and the number of input
+    channels staged in LDS at a time."""
+    nyi, nyj, nf = shape_out_ijf
+    si, sj = kernel_shape
+    sti, stj = strides
+    tile_f = 1
+    if channels_last:  # filters run fastest over the lanes: take up to a wave of them
+        while tile_f < min(nf, 64):
+            tile_f *= 2
+    tile_j = 1
+    while tile_j * 2 * tile_f <= WG and tile_j < nyj:
+        tile_j *= 2
+    tile_j = min(tile_j, 32)
+    tile_i = max(1, min(WG // (tile_j * tile_f), nyi))
+    patch = ((tile_i - 1) * sti + si) * ((tile_j - 1) * stj + sj)
+    c_chunk = max(1, min(nc, (32 * 1024 // 4) // patch))
+    assert patch * 4 <= 48 * 1024, "convolution window too large for one LDS patch"
+    return tile_i, tile_j, tile_f, c_chunk
+
+
+def plan_conv2d(queue, X, Y, filters, shape_in, shape_out, kernel_shape, conv=True, biases=None,
+                padding=(0, 0), strides=(1, 1), channels_last=True, tag=None, transposed=False):
+    """``Y = conv2d(X, filters)`` (``conv``) or local filtering of one image signal;
+    X, Y and filters are one-item views (reference ``plan_conv2d`` :1762-1969).
+
+    filters: ``(size_i, size_j, channels, n_filters)``; for local filtering
+    ``(n_filters, channels, size_i, size_j, out_i, out_j)``."""
+    assert biases is None, "Not tested with biases (strides may be wrong)"
+    si, sj = (int(v) for v in kernel_shape)
+    sti, stj = (int(v) for v in strides)
+    if channels_last:
+        nxi, nxj, nc = (int(v) for v in shape_in)
+        nyi, nyj, nf = (int(v) for v in shape_out)
+    else:
+        nc, nxi, nxj = (int(v) for v in shape_in)
+        nf, nyi, nyj = (int(v) for v in shape_out)
+    if padding == "valid":
+        pi, pj = 0, 0
+    elif padding == "same":
+        pi, pj = (si - 1) // 2, (sj - 1) // 2
+    elif isinstance(padding, (tuple, list)) and len(padding) == 2:
+        pi, pj = (int(v) for v in padding)
+    else:
+        raise ValueError("Unsupported padding (must be 'same', 'valid', or 2-tuple)")
+    for ra in (X, Y, filters):
+        assert ra.ctype == "float"
+    _check(("X", X), ("Y", Y), ("filters", filters))
+    x_start, x_size = _single_contiguous(X, "X")
+    y_start, y_size = _single_contiguous(Y, "Y")
+    f_start, f_size = _single_contiguous(filters, "filters")
+    assert x_size == nxi * nxj * nc, "X does not have shape_in's size"
+    assert y_size == nyi * nyj * nf, "Y does not have shape_out's size"
+    assert f_size == si * sj * nc * nf * (1 if conv else nyi * nyj), "filters have the wrong size"
+    # every output pixel's window must start inside the padded image
+    assert (nyi - 1) * sti - pi < nxi and (nyj - 1) * stj - pj < nxj
+
+    tile_i, tile_j, tile_f, c_chunk = conv2d_tiles((nyi, nyj, nf), (si, sj), (sti, stj), nc,
+                                                   channels_last)
+    geom = np.array([nxi, nxj, nc, nyi, nyj, nf, si, sj, sti, stj, pi, pj, x_start, y_start,
+                     f_start, int(bool(channels_last)), int(not conv), tile_i, tile_j, tile_f,
+                     c_chunk], dtype=np.int32)
+    n_groups = (-(-nyi // tile_i)) * (-(-nyj // tile_j)) * (-(-nf // tile_f))
+    plan = Plan(queue, queue.lib.nhip_conv2d, (geom.ctypes.data, X.ptr, filters.ptr, Y.ptr),
+                gsize=(WG * n_groups,), lsize=(WG,),
+                full_args=(geom, X.dev_buf, filters.dev_buf, Y.dev_buf), name="hip_conv2d", tag=tag)
+    plan.flops_per_call = 2 * nyi * nyj * nf * nc * si * sj
+    plan.bw_per_call = 4 * (x_size + f_size + y_size)
+    plan.description = "shape_in=%s, shape_out=%s, kernel=%s, conv=%s" % (
+        tuple(shape_in), tuple(shape_out), tuple(kernel_shape), conv)
+    return plan
+
+
+def plan_pool2d(queue, X, Y, shape, pool_size, strides, tag=None):
+    """Average pooling of a channels-first image; ``shape = (channels, out_i, out_j,
+    in_i, in_j)`` (reference ``plan_pool2d`` :1972-2079)."""
+    nc, nyi, nyj, nxi, nxj = (int(v) for v in shape)
+    si, sj = (int(v) for v in pool_size)
+    sti, stj = (int(v) for v in strides)
+    assert X.ctype == Y.ctype == "float"
+    _check(("X", X), ("Y", Y))
+    x_start, x_size = _single_contiguous(X, "X")
+    y_start, y_size = _single_contiguous(Y, "Y")
+    assert x_size == nc * nxi * nxj and y_size == nc * nyi * nyj
+    geom = np.array([nc, nyi, nyj, nxi, nxj, si, sj, sti, stj, x_start, y_start], dtype=np.int32)
+    n_groups = -(-(nc * nyi * nyj) // WG)
+    plan = Plan(queue, queue.lib.nhip_pool2d, (geom.ctypes.data, X.ptr, Y.ptr),
+                gsize=(WG * n_groups,), lsize=(WG,), full_args=(geom, X.dev_buf, Y.dev_buf),
+                name="hip_pool2d", tag=tag)
+    plan.flops_per_call = x_size
+    plan.bw_per_call = 4 * (x_size + y_size)
+    return plan
+
+
+# ---------------------------------------------------------------- white noise
+DIST_UNIFORM, DIST_GAUSSIAN = 0, 1
+
+
+def plan_whitenoise(queue, Y, dist_enums, dist_params, scale, inc, dt, seeds, tag=None):
+    """``Y[k] (=|+=) samples of distribution k``, scaled by ``1/sqrt(dt)`` where
+    ``scale[k]`` (reference ``plan_whitenoise`` :1578-1675).
+
+    ``dist_enums[k]`` is 0 (uniform; params low, high) or 1 (Gaussian; params mean,
+    std) and ``seeds[k]`` the seed of process k (the reference takes a ragged array
+    of generator states made by ``create_rngs`` / ``init_rngs`` in this place).  The
+    plan owns one call counter per process; ``plan.reset_streams()`` zeroes them,
+    which restarts every stream from its first sample."""
+    N = len(Y)
+    enums = np.asarray(_host(dist_enums), dtype=np.int32).reshape(-1)
+    params = np.asarray(_host(dist_params), dtype=np.float32).reshape(N, 2)
+    scale = np.asarray(_host(scale)).astype(bool).reshape(-1)
+    inc = np.asarray(_host(inc)).astype(bool).reshape(-1)
+    seeds = np.asarray(seeds, dtype=np.int64).reshape(-1)
+    assert N == enums.size == scale.size == inc.size == seeds.size
+    assert np.isin(enums, (DIST_UNIFORM, DIST_GAUSSIAN)).all()
+    assert (Y.shape1s == 1).all() and (Y.stride0s == 1).all() and (Y.stride1s == 1).all()
+    assert Y.ctype == "float"
+    _check(("Y", Y))
+    table, n = _dev_table(queue, [
+        Y.starts, Y.shape0s, enums, _bits(params[:, 0]), _bits(params[:, 1]),
+        scale.astype(np.int32) | (inc.astype(np.int32) << 1),
+        (seeds & 0xFFFFFFFF).astype(np.uint32).view(np.int32)], 8)
+    counters = to_device(queue, np.zeros(max(N, 1), dtype=np.int32))
+    plan = Plan(queue, queue.lib.nhip_whitenoise,
+                (table.ptr, n, counters.ptr, 1.0 / np.sqrt(dt), Y.ptr),
+                gsize=(WG * max(n, 1),), lsize=(WG,), full_args=(table, counters, Y.dev_buf),
+                name="hip_whitenoise", tag=tag)
+    plan.counters = counters
+    plan.reset_streams = lambda: counters.fill(0)
+    plan.bw_per_call = Y.nbytes
+    plan.description = _description(Y)
+    return plan

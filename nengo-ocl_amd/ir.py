@@ -285,6 +285,100 @@ class SimPES(Operator):
         self.updates = [delta]
 
 
+class SimBCM(Operator):
+    """``delta = learning_rate * dt * post_filtered * (post_filtered - theta) (outer) pre_filtered``."""
+
+    def __init__(self, pre_filtered, post_filtered, theta, delta, learning_rate, tag=None):
+        super().__init__(tag)
+        self.pre_filtered, self.post_filtered, self.theta = pre_filtered, post_filtered, theta
+        self.delta, self.learning_rate = delta, float(learning_rate)
+        self.reads = [pre_filtered, post_filtered, theta]
+        self.updates = [delta]
+
+
+class SimOja(Operator):
+    """``delta = learning_rate * dt * post * (pre - beta * weights * post)`` (Hebbian term
+    minus the forgetting term that bounds the weights)."""
+
+    def __init__(self, pre_filtered, post_filtered, weights, delta, learning_rate, beta, tag=None):
+        super().__init__(tag)
+        self.pre_filtered, self.post_filtered, self.weights = pre_filtered, post_filtered, weights
+        self.delta, self.learning_rate, self.beta = delta, float(learning_rate), float(beta)
+        self.reads = [pre_filtered, post_filtered, weights]
+        self.updates = [delta]
+
+
+class SimVoja(Operator):
+    """``delta = learning_rate * dt * learning_signal * post_filtered *
+    (scale * pre_decoded - scaled_encoders)``: encoders of active neurons move towards
+    the decoded input."""
+
+    def __init__(self, pre_decoded, post_filtered, scaled_encoders, delta, scale, learning_signal,
+                 learning_rate, tag=None):
+        super().__init__(tag)
+        self.pre_decoded, self.post_filtered = pre_decoded, post_filtered
+        self.scaled_encoders, self.delta = scaled_encoders, delta
+        self.scale = np.asarray(scale, dtype=np.float64)
+        self.learning_signal, self.learning_rate = learning_signal, float(learning_rate)
+        self.reads = [pre_decoded, post_filtered, scaled_encoders, learning_signal]
+        self.updates = [delta]
+
+
+class ConvSpec:
+    """Geometry of a convolution transform (what the operator's ``conv`` attribute holds
+    in nengo: ``nengo.Convolution``)."""
+
+    def __init__(self, n_filters, input_shape, kernel_size=(3, 3), strides=(1, 1),
+                 padding="valid", channels_last=True):
+        self.n_filters = int(n_filters)
+        self.kernel_size = tuple(int(k) for k in kernel_size)
+        self.strides = tuple(int(s) for s in strides)
+        self.padding = padding
+        self.channels_last = bool(channels_last)
+        self.dimensions = len(self.kernel_size)
+        self.input_shape = ImageShape(input_shape, channels_last)
+        spatial = self.input_shape.spatial_shape
+        if padding.lower() == "same":
+            out = [-(-n // s) for n, s in zip(spatial, self.strides)]
+        else:
+            out = [(n - k) // s + 1 for n, k, s in zip(spatial, self.kernel_size, self.strides)]
+        shape = tuple(out) + (self.n_filters,) if channels_last else (self.n_filters,) + tuple(out)
+        self.output_shape = ImageShape(shape, channels_last)
+
+    @property
+    def kernel_shape(self):
+        return self.kernel_size + (self.input_shape.n_channels, self.n_filters)
+
+
+class ImageShape:
+    def __init__(self, shape, channels_last=True):
+        self.shape = tuple(int(s) for s in shape)
+        self.channels_last = bool(channels_last)
+
+    @property
+    def spatial_shape(self):
+        return self.shape[:-1] if self.channels_last else self.shape[1:]
+
+    @property
+    def n_channels(self):
+        return self.shape[-1] if self.channels_last else self.shape[0]
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape))
+
+
+class ConvInc(Operator):
+    """``Y = conv(X, W)`` for one image signal (the reference's kernel sets Y,
+    simulator.py:1290-1332)."""
+
+    def __init__(self, W, X, Y, conv, tag=None):
+        super().__init__(tag)
+        self.W, self.X, self.Y, self.conv = W, X, Y, conv
+        self.reads = [W, X]
+        self.incs = [Y]
+
+
 # =========================================================== neuron types
 class LIFRate:
     def __init__(self, tau_rc=0.02, tau_ref=0.002, amplitude=1.0):
@@ -449,6 +543,24 @@ class WhiteSignal(Process):
         power = np.sqrt(np.mean(sig ** 2, axis=0))
         power[power == 0] = 1
         return sig * (self.rms / power)
+
+
+class Uniform:
+    def __init__(self, low, high):
+        self.low, self.high = float(low), float(high)
+
+
+class Gaussian:
+    def __init__(self, mean, std):
+        self.mean, self.std = float(mean), float(std)
+
+
+class WhiteNoise(Process):
+    """Independent samples of ``dist`` every step, times ``1/sqrt(dt)`` if ``scale``."""
+
+    def __init__(self, dist=None, scale=True, seed=None):
+        self.dist = Gaussian(0.0, 1.0) if dist is None else dist
+        self.scale, self.seed = bool(scale), seed
 
 
 class PresentInput(Process):

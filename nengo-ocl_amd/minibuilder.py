@@ -28,9 +28,9 @@ and one filter (what a passthrough node after the ensemble gives in nengo).
 import numpy as np
 
 from . import ir
-from .ir import (LIF, AdaptiveLIF, AdaptiveLIFRate, Alpha, LIFRate, LinearFilter,  # noqa: F401
-                 Lowpass, PresentInput, RectifiedLinear, Sigmoid, SpikingRectifiedLinear,
-                 WhiteSignal)
+from .ir import (LIF, AdaptiveLIF, AdaptiveLIFRate, Alpha, Gaussian, LIFRate,  # noqa: F401
+                 LinearFilter, Lowpass, PresentInput, RectifiedLinear, Sigmoid,
+                 SpikingRectifiedLinear, Uniform, WhiteNoise, WhiteSignal)
 
 
 class _Sliceable:
@@ -67,11 +67,11 @@ class Neurons(_Sliceable):
 
 class Ensemble(_Sliceable):
     def __init__(self, n_neurons, dimensions, radius=1.0, neuron_type=None, max_rates=(200, 400),
-                 intercepts=(-1, 1), encoders=None, label=None, seed=None):
+                 intercepts=(-1, 1), encoders=None, label=None, seed=None, noise=None):
         self.n_neurons, self.dimensions, self.radius = int(n_neurons), int(dimensions), radius
         self.neuron_type = LIF() if neuron_type is None else neuron_type
         self.max_rates, self.intercepts, self.encoders = max_rates, intercepts, encoders
-        self.label, self.seed = label, seed
+        self.label, self.seed, self.noise = label, seed, noise
         self.neurons = Neurons(self)
         self.size_in = self.size_out = self.dimensions
 
@@ -80,6 +80,56 @@ class PES:
     def __init__(self, learning_rate=1e-4, pre_synapse=Lowpass(0.005)):
         self.learning_rate, self.pre_synapse = learning_rate, pre_synapse
         self.connection = None
+
+
+class BCM:
+    """Bienenstock-Cooper-Munro rule on weights between neurons."""
+
+    def __init__(self, learning_rate=1e-9, pre_synapse=Lowpass(0.005), post_synapse=None,
+                 theta_synapse=Lowpass(1.0)):
+        self.learning_rate, self.pre_synapse = learning_rate, pre_synapse
+        self.post_synapse = pre_synapse if post_synapse is None else post_synapse
+        self.theta_synapse = theta_synapse
+        self.connection = None
+        self.size_in = 0
+
+
+class Oja:
+    """Oja's rule (Hebbian with a forgetting term) on weights between neurons."""
+
+    def __init__(self, learning_rate=1e-6, pre_synapse=Lowpass(0.005), post_synapse=None,
+                 beta=1.0):
+        self.learning_rate, self.pre_synapse, self.beta = learning_rate, pre_synapse, beta
+        self.post_synapse = pre_synapse if post_synapse is None else post_synapse
+        self.connection = None
+        self.size_in = 0
+
+
+class Voja:
+    """Vector Oja rule: moves the post ensemble's encoders towards the decoded input;
+    its one-dimensional input scales the learning (0 switches it off)."""
+
+    def __init__(self, learning_rate=1e-2, post_synapse=Lowpass(0.005)):
+        self.learning_rate, self.post_synapse = learning_rate, post_synapse
+        self.connection = None
+        self.size_in = 1
+
+
+class Convolution:
+    """A convolution transform (nengo.Convolution): ``init`` has shape
+    ``kernel_size + (input channels, n_filters)``."""
+
+    def __init__(self, n_filters, input_shape, kernel_size=(3, 3), strides=(1, 1),
+                 padding="valid", channels_last=True, init=None, seed=None):
+        self.spec = ir.ConvSpec(n_filters, input_shape, kernel_size, strides, padding,
+                                channels_last)
+        if init is None:
+            rng = np.random.RandomState(seed)
+            fan_in = np.prod(self.spec.kernel_size) * self.spec.input_shape.n_channels
+            init = rng.uniform(-1, 1, size=self.spec.kernel_shape) * np.sqrt(3.0 / fan_in)
+        self.init = np.asarray(init, dtype=np.float64).reshape(self.spec.kernel_shape)
+        self.size_in = self.spec.input_shape.size
+        self.size_out = self.spec.output_shape.size
 
 
 class Connection:
@@ -188,6 +238,8 @@ class Network:
         rng = np.random.RandomState(self.seed)
         self._decoded_cache = {}
         self._decoder_values = {}
+        self._voja_targets = {(c.post.obj if isinstance(c.post, ObjView) else c.post)
+                              for c in self.connections if isinstance(c.learning_rule, Voja)}
         for ens in self.ensembles:
             self._build_ensemble(model, ens, rng)
         for node in self.nodes:
@@ -197,8 +249,15 @@ class Network:
             if conn.learning_rule is not None:
                 rule = conn.learning_rule
                 post_obj = conn.post.obj if isinstance(conn.post, ObjView) else conn.post
-                model.sig[rule] = {"in": ir.Signal(np.zeros(post_obj.size_in), name="PES:error")}
-                model.add_op(ir.Reset(model.sig[rule]["in"]))
+                if isinstance(rule, PES):
+                    model.sig[rule] = {"in": ir.Signal(np.zeros(post_obj.size_in),
+                                                       name="PES:error")}
+                    model.add_op(ir.Reset(model.sig[rule]["in"]))
+                elif isinstance(rule, Voja):  # learning signal: 1 unless something drives it
+                    model.sig[rule] = {"in": ir.Signal(np.zeros(1), name="Voja:learning")}
+                    model.add_op(ir.Reset(model.sig[rule]["in"], value=1.0))
+                else:
+                    model.sig[rule] = {"in": None}
         for conn in self.connections:
             self._build_connection(model, conn, rng)
         for probe in self.probes:
@@ -223,7 +282,8 @@ class Network:
         name = ens.label or "ens%d" % len(model.sig)
         sig = {
             "in": ir.Signal(np.zeros(d), name="%s.signal" % name),
-            "encoders": ir.Signal(scaled_encoders, name="%s.scaled_encoders" % name, readonly=True),
+            "encoders": ir.Signal(scaled_encoders, name="%s.scaled_encoders" % name,
+                                  readonly=ens not in self._voja_targets),
         }
         nsig = {
             "in": ir.Signal(np.zeros(n), name="%s.neuron_in" % name),
@@ -242,6 +302,8 @@ class Network:
                        "SpikingRectifiedLinear": ("voltage",)}
         state = {key: ir.Signal(np.zeros(n), name="%s.%s" % (name, key))
                  for key in state_names.get(type(ens.neuron_type).__name__, ())}
+        if ens.noise is not None:  # injected into the input current
+            model.add_op(ir.SimProcess(ens.noise, None, nsig["in"], model.time, mode="inc"))
         model.add_op(ir.SimNeurons(ens.neuron_type, nsig["in"], nsig["out"], state=state))
 
     def _build_node(self, model, node, rng):
@@ -323,8 +385,12 @@ class Network:
         crng = np.random.RandomState(rng.randint(2 ** 31 - 1))
         name = conn.label or "conn%d" % len(model.sig)
         sparse = conn.transform if isinstance(conn.transform, Sparse) else None
-        transform = (None if conn.transform is None or sparse is not None
+        convolution = conn.transform if isinstance(conn.transform, Convolution) else None
+        transform = (None if conn.transform is None or sparse is not None or convolution is not None
                      else np.asarray(conn.transform, dtype=np.float64))
+        rule = conn.learning_rule
+        if convolution is not None and not isinstance(pre, (Neurons, Node)):
+            raise NotImplementedError("convolution transforms on decoded connections")
 
         if isinstance(pre, Ensemble):
             if pre_slice is not None:
@@ -333,7 +399,9 @@ class Network:
                 function = (lambda x, f=base_fn, s=sel: (x if f is None else np.atleast_1d(f(x)))[s])
             else:
                 function = conn.function
-            learned = conn.learning_rule is not None
+            learned = isinstance(rule, PES)
+            if rule is not None and not isinstance(rule, (PES, Voja)):
+                raise NotImplementedError("%s on a decoded connection" % type(rule).__name__)
             key = (pre, conn.function, None if transform is None else transform.tobytes(),
                    repr(pre_slice), self._synapse_key(conn.synapse))
             cached = self._decoded_cache.get(key) if (self.share_decoded and not learned) else None
@@ -363,11 +431,20 @@ class Network:
                     self._decoded_cache[key] = signal
                 if learned:
                     self._build_pes(model, conn, pre, wsig, name)
+            if isinstance(rule, Voja):
+                self._build_voja(model, conn, post, signal, name)
         elif isinstance(pre, Neurons):
             signal = model.sig[pre]["out"]
             if pre_slice is not None:
                 signal = signal[pre_slice]
-            if sparse is not None or (transform is not None and transform.ndim == 2):
+            if rule is not None and not (isinstance(rule, (BCM, Oja)) and transform is not None
+                                         and transform.ndim == 2 and isinstance(post, Neurons)
+                                         and pre_slice is None and post_slice is None):
+                raise NotImplementedError("%s needs full weights between two neuron "
+                                          "populations" % type(rule).__name__)
+            if convolution is not None:
+                signal = self._build_convolution(model, convolution, signal, name)
+            elif sparse is not None or (transform is not None and transform.ndim == 2):
                 # weights between neurons: weighted = W @ activities, then the synapse
                 n_out = sparse.shape[0] if sparse is not None else transform.shape[0]
                 weighted = ir.Signal(np.zeros(n_out), name="%s.weighted" % name)
@@ -376,9 +453,11 @@ class Network:
                     wsig = ir.SparseSignal(sparse.init, name="%s.weights" % name)
                     model.add_op(ir.SparseDotInc(wsig, signal, weighted, tag="%s.weights" % name))
                 else:
-                    wsig = ir.Signal(transform, name="%s.weights" % name, readonly=True)
+                    wsig = ir.Signal(transform, name="%s.weights" % name, readonly=rule is None)
                     model.add_op(ir.DotInc(wsig, signal, weighted, tag="%s.weights" % name))
                 model.sig[conn] = {"weights": wsig}
+                if rule is not None:
+                    self._build_hebbian(model, conn, pre, post, wsig, name)
                 signal = weighted
             elif transform is not None:
                 raise NotImplementedError("scalar / diagonal transforms between neurons")
@@ -389,7 +468,11 @@ class Network:
                 signal = signal[pre_slice]
             if conn.function is not None:
                 raise NotImplementedError("functions on node connections")
-            if transform is not None:
+            if rule is not None:
+                raise NotImplementedError("learning rules on connections from nodes")
+            if convolution is not None:
+                signal = self._build_convolution(model, convolution, signal, name)
+            elif transform is not None:
                 if transform.ndim == 0:
                     tsig = ir.Signal(transform, name="%s.transform" % name, readonly=True)
                     weighted = ir.Signal(np.zeros(signal.shape), name="%s.weighted" % name)
@@ -417,7 +500,7 @@ class Network:
             if post.output is not None:
                 raise NotImplementedError("connections into function nodes")
             target = model.sig[post]["in"]
-        elif isinstance(post, PES):
+        elif isinstance(post, (PES, Voja)):
             target = model.sig[post]["in"]
         else:
             raise TypeError("cannot connect to %r" % (post,))
@@ -440,6 +523,50 @@ class Network:
         model.add_op(ir.SimPES(pre_filtered, model.sig[rule]["in"], delta, rule.learning_rate))
         model.add_op(ir.Copy(delta, wsig, inc=True, tag="%s += delta" % name))
         model.sig[rule]["delta"] = delta
+
+    def _build_hebbian(self, model, conn, pre, post, wsig, name):
+        """BCM / Oja on weights between two neuron populations: filtered activities on
+        both sides, the delta written by the rule, then added to the weights."""
+        rule = conn.learning_rule
+        pre_acts, post_acts = model.sig[pre]["out"], model.sig[post]["out"]
+        pre_filtered = self._apply_synapse(model, pre_acts, rule.pre_synapse, "%s.rule_pre" % name)
+        post_filtered = self._apply_synapse(model, post_acts, rule.post_synapse,
+                                            "%s.rule_post" % name)
+        delta = ir.Signal(np.zeros(wsig.shape), name="%s.Delta" % name)
+        if isinstance(rule, BCM):
+            theta = self._apply_synapse(model, post_acts, rule.theta_synapse, "%s.theta" % name)
+            model.add_op(ir.SimBCM(pre_filtered, post_filtered, theta, delta, rule.learning_rate))
+        else:
+            model.add_op(ir.SimOja(pre_filtered, post_filtered, wsig, delta, rule.learning_rate,
+                                   rule.beta))
+        model.add_op(ir.Copy(delta, wsig, inc=True, tag="%s += delta" % name))
+        model.sig[rule]["delta"] = delta
+
+    def _build_voja(self, model, conn, post, pre_decoded, name):
+        rule = conn.learning_rule
+        if not isinstance(post, Ensemble):
+            raise NotImplementedError("Voja needs an ensemble as the connection's target")
+        if pre_decoded.size != post.dimensions:
+            raise ValueError("Voja: the connection must deliver the ensemble's full input")
+        post_filtered = self._apply_synapse(model, model.sig[post.neurons]["out"],
+                                            rule.post_synapse, "%s.voja_post" % name)
+        encoders = model.sig[post]["encoders"]
+        delta = ir.Signal(np.zeros(encoders.shape), name="%s.Delta" % name)
+        scale = model.params[post]["gain"] / post.radius
+        model.add_op(ir.SimVoja(pre_decoded, post_filtered, encoders, delta, scale,
+                                model.sig[rule]["in"], rule.learning_rate))
+        model.add_op(ir.Copy(delta, encoders, inc=True, tag="%s encoders += delta" % name))
+        model.sig[rule]["delta"] = delta
+
+    def _build_convolution(self, model, convolution, signal, name):
+        if signal.size != convolution.size_in:
+            raise ValueError("%s: %d values into a convolution over %s" % (
+                name, signal.size, convolution.spec.input_shape.shape))
+        wsig = ir.Signal(convolution.init, name="%s.kernel" % name, readonly=True)
+        weighted = ir.Signal(np.zeros(convolution.size_out), name="%s.weighted" % name)
+        model.add_op(ir.Reset(weighted))
+        model.add_op(ir.ConvInc(wsig, signal, weighted, convolution.spec, tag="%s.conv" % name))
+        return weighted
 
     # --- probes
     def _build_probe(self, model, probe, rng):

@@ -66,7 +66,8 @@ class HipBackend:
         for name in ("plan_timeupdate", "plan_reset", "plan_copy", "plan_slicedcopy",
                      "plan_elementwise_inc", "plan_linearfilter", "plan_probes", "plan_direct",
                      "plan_lif", "plan_lif_rate", "plan_presentinput", "plan_rectified_linear",
-                     "plan_spiking_rectified_linear", "plan_sigmoid"):
+                     "plan_spiking_rectified_linear", "plan_sigmoid", "plan_bcm", "plan_oja",
+                     "plan_voja", "plan_conv2d", "plan_pool2d", "plan_whitenoise"):
             setattr(self, name, getattr(hipra_nonlinearities, name))
         self.plan_block_gemv = hipra_gemv.plan_block_gemv
         self._fuse_lif = hipra_gemv.fuse_lif
@@ -320,6 +321,7 @@ class Simulator:
         t0 = _time.time()
         self._raggedarrays_to_reset = []  # (device ragged, host initial)
         self._filter_positions = []
+        self._noise_plans = []
         self._python_rngs = {}
         plans = []
         previous = None  # (type, plans) of the group planned last
@@ -580,6 +582,8 @@ class Simulator:
             self.backend.write_all(dev, host.buf)
         for pos in self._filter_positions:
             self.backend.fill_array(pos, 0)
+        for plan in self._noise_plans:
+            plan.reset_streams()
         for rng, state in self._python_rngs.items():
             rng.set_state(state)
         self._reset_probes()
@@ -1012,6 +1016,96 @@ class Simulator:
                           for op in ops])
         return [self.backend.plan_elementwise_inc(self.queue, error, pre, delta, alpha=alpha,
                                                   outer=True, inc=False)]
+
+    def _plan_SimBCM(self, ops):
+        pre = self.all_data[[self.sidx[op.pre_filtered] for op in ops]]
+        post = self.all_data[[self.sidx[op.post_filtered] for op in ops]]
+        theta = self.all_data[[self.sidx[op.theta] for op in ops]]
+        delta = self.all_data[[self.sidx[op.delta] for op in ops]]
+        alpha = np.array([op.learning_rate * self.model.dt for op in ops])
+        return [self.backend.plan_bcm(self.queue, pre, post, theta, delta, alpha)]
+
+    def _plan_SimOja(self, ops):
+        pre = self.all_data[[self.sidx[op.pre_filtered] for op in ops]]
+        post = self.all_data[[self.sidx[op.post_filtered] for op in ops]]
+        weights = self.all_data[[self.sidx[op.weights] for op in ops]]
+        delta = self.all_data[[self.sidx[op.delta] for op in ops]]
+        alpha = np.array([op.learning_rate * self.model.dt for op in ops])
+        beta = np.array([op.beta for op in ops])
+        return [self.backend.plan_oja(self.queue, pre, post, weights, delta, alpha, beta)]
+
+    def _plan_SimRLS(self, ops):
+        raise NotImplementedError("RLS learning rule not yet supported")
+
+    def _plan_SimVoja(self, ops):
+        pre = self.all_data[[self.sidx[op.pre_decoded] for op in ops]]
+        post = self.all_data[[self.sidx[op.post_filtered] for op in ops]]
+        encoders = self.all_data[[self.sidx[op.scaled_encoders] for op in ops]]
+        delta = self.all_data[[self.sidx[op.delta] for op in ops]]
+        learning_signal = self.all_data[[self.sidx[op.learning_signal] for op in ops]]
+        scale = self.RaggedArray([np.asarray(op.scale).reshape(-1) for op in ops],
+                                 dtype=np.float32)
+        alpha = np.array([op.learning_rate * self.model.dt for op in ops])
+        return [self.backend.plan_voja(self.queue, pre, post, encoders, delta, learning_signal,
+                                       scale, alpha)]
+
+    # --- convolution
+    def _plan_ConvInc(self, ops):
+        plans = []
+        for op in ops:
+            conv = op.conv
+            assert conv.dimensions in (1, 2)
+            channels_last = conv.channels_last
+            assert channels_last == conv.input_shape.channels_last
+            assert channels_last == conv.output_shape.channels_last
+            shape_in, shape_out = tuple(conv.input_shape.shape), tuple(conv.output_shape.shape)
+            kernel_shape, strides = tuple(conv.kernel_size), tuple(conv.strides)
+            if conv.dimensions == 1:  # a 1-D convolution is a 2-D one over a single row
+                assert len(shape_in) == len(shape_out) == 2
+                kernel_shape, strides = (1,) + kernel_shape, (1,) + strides
+                if channels_last:
+                    shape_in, shape_out = (1,) + shape_in, (1,) + shape_out
+                else:
+                    shape_in = (shape_in[0], 1, shape_in[1])
+                    shape_out = (shape_out[0], 1, shape_out[1])
+            plan = self.backend.plan_conv2d(
+                self.queue, X=self.all_data[[self.sidx[op.X]]], Y=self.all_data[[self.sidx[op.Y]]],
+                filters=self.all_data[[self.sidx[op.W]]], biases=None, shape_in=shape_in,
+                shape_out=shape_out, kernel_shape=kernel_shape, padding=conv.padding.lower(),
+                strides=strides, channels_last=channels_last, conv=True)
+            plan.planned_ops = [op]
+            plans.append(plan)
+        return plans
+
+    # --- noise
+    def _plan_WhiteNoise(self, ops):
+        assert all(op.input is None for op in ops)
+        seeds = [self.rng.randint(2 ** 31 - 1) if op.process.seed is None else op.process.seed
+                 for op in ops]
+        Y = self.all_data[[self.sidx[op.output] for op in ops]]
+        scale = [bool(op.process.scale) for op in ops]
+        inc = [op.mode == "inc" for op in ops]
+        enums, params = [], []
+        for op in ops:
+            dist = op.process.dist
+            kind = type(dist).__name__
+            if kind == "Uniform":
+                enums.append(0)
+                params.append((dist.low, dist.high))
+            elif kind == "Gaussian":
+                enums.append(1)
+                params.append((dist.mean, dist.std))
+            else:
+                raise NotImplementedError("white noise with distribution %r" % kind)
+        plan = self.backend.plan_whitenoise(self.queue, Y, np.array(enums, dtype=np.int32),
+                                            np.array(params, dtype=np.float32), scale, inc,
+                                            self.model.dt, seeds)
+        self._noise_plans.append(plan)
+        plan.unread_signals = [op.t for op in ops]
+        return [plan]
+
+    def _plan_FilteredNoise(self, ops):
+        raise NotImplementedError()
 
     # ------------------------------------------------------------- reporting
     def print_plans(self):

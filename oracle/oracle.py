@@ -376,3 +376,103 @@ def plan_probes(queue, periods, X, Y, tag=None):
     plan.periods = periods
     plan.Y = Y
     return plan
+
+
+# ------------------------------------------------- learning rules, convolution, noise
+def _plan_rule(rule, name, pre, post, aux, delta, alpha, beta=None, learn=None, scale=None,
+               tag=None):
+    n = len(pre)
+    alphas = _per_item(alpha, n, np.float32)
+    betas = _per_item(0.0 if beta is None else beta, n, np.float32)
+    zeros = np.zeros(n, dtype=np.int32)
+    args = [_i32(delta.shape0s), _i32(delta.shape1s), _i32(pre.starts), _i32(pre.stride0s),
+            _i32(post.starts), _i32(post.stride0s), _i32(aux.starts), _i32(aux.stride0s),
+            _i32(delta.starts), _i32(delta.stride0s), alphas, betas,
+            zeros if learn is None else _i32(learn.starts),
+            zeros if scale is None else _i32(scale.starts),
+            zeros if scale is None else _i32(scale.stride0s)]
+    fn = lib().orc_learning_rule
+
+    def step():
+        fn(ctypes.c_int(rule), ctypes.c_int(n), *[_p(a) for a in args], _p(pre.buf), _p(post.buf),
+           _p(aux.buf), _p(delta.buf), None if learn is None else _p(learn.buf),
+           None if scale is None else _p(scale.buf))
+
+    return _plan(step, name, args, tag)
+
+
+def plan_bcm(queue, pre, post, theta, delta, alpha, tag=None):
+    return _plan_rule(1, "oracle_bcm", pre, post, theta, delta, alpha, tag=tag)
+
+
+def plan_oja(queue, pre, post, weights, delta, alpha, beta, tag=None):
+    return _plan_rule(2, "oracle_oja", pre, post, weights, delta, alpha, beta=beta, tag=tag)
+
+
+def plan_voja(queue, pre, post, enc, delta, learn, scale, alpha, tag=None):
+    return _plan_rule(3, "oracle_voja", pre, post, enc, delta, alpha, learn=learn, scale=scale,
+                      tag=tag)
+
+
+def plan_conv2d(queue, X, Y, filters, shape_in, shape_out, kernel_shape, conv=True, biases=None,
+                padding=(0, 0), strides=(1, 1), channels_last=True, tag=None, transposed=False):
+    assert biases is None
+    si, sj = kernel_shape
+    if channels_last:
+        nxi, nxj, nc = shape_in
+        nyi, nyj, nf = shape_out
+    else:
+        nc, nxi, nxj = shape_in
+        nf, nyi, nyj = shape_out
+    if padding == "valid":
+        pi, pj = 0, 0
+    elif padding == "same":
+        pi, pj = (si - 1) // 2, (sj - 1) // 2
+    else:
+        pi, pj = padding
+    geom = _i32([nxi, nxj, nc, nyi, nyj, nf, si, sj, strides[0], strides[1], pi, pj,
+                 X.starts[0], Y.starts[0], filters.starts[0], bool(channels_last), not conv])
+    fn = lib().orc_conv2d
+
+    def step():
+        fn(_p(geom), _p(X.buf), _p(filters.buf), _p(Y.buf))
+
+    return _plan(step, "oracle_conv2d", [geom], tag)
+
+
+def plan_pool2d(queue, X, Y, shape, pool_size, strides, tag=None):
+    geom = _i32(list(shape) + list(pool_size) + list(strides) + [X.starts[0], Y.starts[0]])
+    fn = lib().orc_pool2d
+
+    def step():
+        fn(_p(geom), _p(X.buf), _p(Y.buf))
+
+    return _plan(step, "oracle_pool2d", [geom], tag)
+
+
+def philox4x32(counters_keys):
+    """Philox4x32-10 of ``(n, 6)`` uint32 rows (counter words 0-3, key words 0-1)."""
+    rows = np.ascontiguousarray(counters_keys, dtype=np.uint32).reshape(-1, 6)
+    out = np.zeros((len(rows), 4), dtype=np.uint32)
+    lib().orc_philox4x32(_p(rows), _p(out), ctypes.c_int(len(rows)))
+    return out
+
+
+def plan_whitenoise(queue, Y, dist_enums, dist_params, scale, inc, dt, seeds, tag=None):
+    n = len(Y)
+    params = np.asarray(dist_params, dtype=np.float32).reshape(n, 2)
+    args = [_i32(Y.starts), _i32(Y.shape0s), _i32(np.asarray(dist_enums).reshape(-1)),
+            _f32(params[:, 0]), _f32(params[:, 1]), _i32(np.asarray(scale).astype(bool)),
+            _i32(np.asarray(inc).astype(bool)),
+            np.ascontiguousarray(np.asarray(seeds, dtype=np.int64) & 0xFFFFFFFF, dtype=np.uint32)]
+    counters = np.zeros(max(n, 1), dtype=np.int32)
+    fn = lib().orc_whitenoise
+
+    def step():
+        fn(ctypes.c_int(n), *[_p(a) for a in args], _p(counters),
+           ctypes.c_double(1.0 / np.sqrt(dt)), _p(Y.buf))
+
+    plan = _plan(step, "oracle_whitenoise", args, tag)
+    plan.counters = counters
+    plan.reset_streams = lambda: counters.fill(0)
+    return plan

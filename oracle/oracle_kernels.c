@@ -481,3 +481,173 @@ void orc_spmv_csr(int n_items, const int *n_rows, const int *indptr_starts,
         }
     }
 }
+
+/* ------------------------------------------------------------------------
+ * Learning rules that write a delta matrix (clra_nonlinearities.py:2082-2405).
+ * rule 1 BCM  :2130-2131  delta = alpha * post * (post - theta) * pre
+ * rule 2 Oja  :2237-2238  delta = alpha * post * (pre - beta * weight * post)
+ * rule 3 Voja :2349-2350  delta = alpha * learn * post * (scale * pre - enc)
+ * C evaluates these left to right, every product and difference rounded to
+ * float32 on its own (no contraction in this build). */
+void orc_learning_rule(int rule, int n_items, const int *shape0s, const int *shape1s,
+                       const int *pre_starts, const int *pre_stride0s, const int *post_starts,
+                       const int *post_stride0s, const int *aux_starts, const int *aux_stride0s,
+                       const int *delta_starts, const int *delta_stride0s, const float *alphas,
+                       const float *betas, const int *learn_starts, const int *scale_starts,
+                       const int *scale_stride0s, const float *PRE, const float *POST,
+                       const float *AUX, float *DELTA, const float *LEARN, const float *SCALE) {
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int k = 0; k < n_items; ++k) {
+        const float alpha = alphas[k];
+        for (int i = 0; i < shape0s[k]; ++i) {
+            const float post = POST[post_starts[k] + (size_t)i * post_stride0s[k]];
+            for (int j = 0; j < shape1s[k]; ++j) {
+                const float pre = PRE[pre_starts[k] + (size_t)j * pre_stride0s[k]];
+                float out;
+                if (rule == 1) {
+                    const float theta = AUX[aux_starts[k] + (size_t)i * aux_stride0s[k]];
+                    out = alpha * post * (post - theta) * pre;
+                } else if (rule == 2) {
+                    const float weight = AUX[aux_starts[k] + (size_t)i * aux_stride0s[k] + j];
+                    const float beta = betas[k];
+                    out = alpha * post * (pre - beta * weight * post);
+                } else {
+                    const float enc = AUX[aux_starts[k] + (size_t)i * aux_stride0s[k] + j];
+                    const float learn = LEARN[learn_starts[k]];
+                    const float scale = SCALE[scale_starts[k] + (size_t)i * scale_stride0s[k]];
+                    out = alpha * learn * post * (scale * pre - enc);
+                }
+                DELTA[delta_starts[k] + (size_t)i * delta_stride0s[k] + j] = out;
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------
+ * 2-D convolution / local filtering of one image (clra_nonlinearities.py:1812-1849):
+ * out = 0, then for channel c, kernel row ii, kernel column jj in that order
+ * out += filter * x (zero outside the image), here one fused multiply-add per term
+ * (an OpenCL compiler may contract the `+=` line; this restatement fixes that choice,
+ * like the GEMV's).  geom as the HIP library takes it. */
+void orc_conv2d(const int *g, const float *X, const float *F, float *Y) {
+    const int nxi = g[0], nxj = g[1], nc = g[2], nyi = g[3], nyj = g[4], nf = g[5];
+    const int si = g[6], sj = g[7], sti = g[8], stj = g[9], pi = g[10], pj = g[11];
+    const int channels_last = g[15], local = g[16];
+    const float *x = X + g[12];
+    float *y = Y + g[13];
+    const float *f = F + g[14];
+    const size_t xs_i = (size_t)nxj * (channels_last ? nc : 1), xs_j = channels_last ? nc : 1;
+    const size_t xs_c = channels_last ? 1 : (size_t)nxi * nxj;
+    const size_t ys_i = (size_t)nyj * (channels_last ? nf : 1), ys_j = channels_last ? nf : 1;
+    const size_t ys_f = channels_last ? 1 : (size_t)nyi * nyj;
+#pragma omp parallel for schedule(static)
+    for (int k = 0; k < nf; ++k) {
+        for (int i = 0; i < nyi; ++i) {
+            for (int j = 0; j < nyj; ++j) {
+                float out = 0.0f;
+                for (int c = 0; c < nc; ++c) {
+                    for (int ii = 0; ii < si; ++ii) {
+                        for (int jj = 0; jj < sj; ++jj) {
+                            const int r = i * sti - pi + ii, q = j * stj - pj + jj;
+                            const float xv = (r >= 0 && r < nxi && q >= 0 && q < nxj)
+                                                 ? x[c * xs_c + r * xs_i + q * xs_j] : 0.0f;
+                            const float w = local
+                                ? f[((size_t)(k * nc + c) * si * sj + ii * sj + jj) * nyi * nyj
+                                    + i * nyj + j]
+                                : f[((size_t)(ii * sj + jj) * nc + c) * nf + k];
+                            out = fmaf(w, xv, out);
+                        }
+                    }
+                }
+                y[k * ys_f + i * ys_i + j * ys_j] = out;
+            }
+        }
+    }
+}
+
+/* Average pooling, channels first (clra_nonlinearities.py:2012-2041): mean of the
+ * window's in-range inputs that are not NaN, summed row by row. */
+void orc_pool2d(const int *g, const float *X, float *Y) {
+    const int nc = g[0], nyi = g[1], nyj = g[2], nxi = g[3], nxj = g[4];
+    const int si = g[5], sj = g[6], sti = g[7], stj = g[8];
+    const float *x = X + g[9];
+    float *y = Y + g[10];
+    for (int c = 0; c < nc; ++c)
+        for (int i = 0; i < nyi; ++i)
+            for (int j = 0; j < nyj; ++j) {
+                float out = 0.0f;
+                int n = 0;
+                for (int ii = 0; ii < si; ++ii)
+                    for (int jj = 0; jj < sj; ++jj) {
+                        const int r = i * sti + ii, q = j * stj + jj;
+                        if (r < nxi && q < nxj) {
+                            const float v = x[((size_t)c * nxi + r) * nxj + q];
+                            if (!isnan(v)) {
+                                out += v;
+                                n++;
+                            }
+                        }
+                    }
+                y[((size_t)c * nyi + i) * nyj + j] = out / n;
+            }
+}
+
+/* ------------------------------------------------------------------------
+ * White noise.  The reference samples from pyopencl's RANLUX states
+ * (clra_nonlinearities.py:1486-1675); pyopencl is a third-party module that is not
+ * part of the reference's sources, and its stream is not nengo's either, so the
+ * build defines its own stream: Philox4x32-10 (Salmon, Moraes, Dror, Shaw, SC'11),
+ * block {q, n, 0, 0} under key {seed, 0} for elements 4q..4q+3 of call n.
+ * The distribution formulas follow :1553-1562 (low + (high-low)*u; mean + std*z);
+ * the unit samples u, z are this build's own (24-bit uniform, Box-Muller). */
+static void orc_philox_block(uint32_t c[4], uint32_t k0, uint32_t k1) {
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        c[0] = n0; c[1] = (uint32_t)p1; c[2] = n2; c[3] = (uint32_t)p0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+void orc_philox4x32(const uint32_t *in, uint32_t *out, int n) {
+    for (int t = 0; t < n; ++t) {
+        uint32_t c[4] = {in[6 * t], in[6 * t + 1], in[6 * t + 2], in[6 * t + 3]};
+        orc_philox_block(c, in[6 * t + 4], in[6 * t + 5]);
+        memcpy(out + 4 * t, c, sizeof c);
+    }
+}
+
+void orc_whitenoise(int n_items, const int *y_starts, const int *counts, const int *dists,
+                    const float *p0s, const float *p1s, const int *scales, const int *incs,
+                    const uint32_t *seeds, int *counters, double sqrt_dt_inv, float *Y) {
+    for (int k = 0; k < n_items; ++k) {
+        float *y = Y + y_starts[k];
+        const uint32_t call = (uint32_t)counters[k];
+        for (int i = 0; i < counts[k]; ++i) {
+            uint32_t c[4] = {(uint32_t)(i >> 2), call, 0u, 0u};
+            orc_philox_block(c, seeds[k], 0u);
+            const int lane = i & 3;
+            float sample;
+            if (dists[k] == 0) {
+                const float u = (float)(c[lane] >> 8) * 0x1p-24f;
+                const float span = p1s[k] - p0s[k];
+                const float t = span * u;
+                sample = p0s[k] + t;
+            } else {
+                const uint32_t wa = c[lane & 2], wb = c[(lane & 2) + 1];
+                const double u1 = (double)((wa >> 8) + 1u) * 0x1p-24;
+                const double phi = 6.283185307179586476925 * ((double)(wb >> 8) * 0x1p-24);
+                const double r = sqrt(-2.0 * log(u1));
+                const float z = (float)((lane & 1) ? r * sin(phi) : r * cos(phi));
+                const float t = p1s[k] * z;
+                sample = p0s[k] + t;
+            }
+            if (scales[k]) sample = (float)((double)sample * sqrt_dt_inv);
+            y[i] = incs[k] ? y[i] + sample : sample;
+        }
+        counters[k] = (int)(call + 1u);
+    }
+}

@@ -26,7 +26,9 @@ class OracleBackend:
         for name in ("plan_timeupdate", "plan_reset", "plan_copy", "plan_slicedcopy",
                      "plan_elementwise_inc", "plan_linearfilter", "plan_lif", "plan_lif_rate",
                      "plan_presentinput", "plan_block_gemv", "plan_rectified_linear",
-                     "plan_spiking_rectified_linear", "plan_sigmoid", "plan_sparse_dot_inc"):
+                     "plan_spiking_rectified_linear", "plan_sigmoid", "plan_sparse_dot_inc",
+                     "plan_bcm", "plan_oja", "plan_voja", "plan_conv2d", "plan_pool2d",
+                     "plan_whitenoise"):
             setattr(self, name, getattr(oracle, name))
 
     @staticmethod

@@ -430,3 +430,211 @@ def test_relu_spiking_relu_sigmoid(queue, rng):
     orc().plan_sigmoid(None, J, Rs, ref)()
     assert np.array_equal(dRs.buf, Rs.buf)
     assert (Rs.buf == 0).any() and (Rs[2] == 1 / ref[2]).any()  # both cut-offs are reached
+
+
+# ------------------------------------------------------------------ learning rules
+@pytest.mark.parametrize("rule", ["bcm", "oja", "voja"])
+def test_learning_rules(queue, rng, rule):
+    """Delta matrices of many connections of different shapes in one launch, bit for bit
+    (every product and difference is rounded separately on both sides)."""
+    shapes = [(7, 5), (1, 9), (300, 70), (64, 1), (1000, 513), (33, 1100)]
+    k = len(shapes)
+    pre = RA([rng.uniform(0, 200, size=n) for m, n in shapes])
+    post = RA([rng.uniform(0, 200, size=m) for m, n in shapes])
+    theta = RA([rng.uniform(0, 200, size=m) for m, n in shapes])
+    mat = RA([rng.normal(scale=0.01, size=(m, n)) for m, n in shapes])
+    delta = RA([rng.normal(size=(m, n)) for m, n in shapes])
+    learn = RA([[rng.uniform(0, 1)] for _ in shapes])
+    scale = RA([rng.uniform(1, 30, size=m) for m, n in shapes])
+    alpha = rng.uniform(1e-6, 1e-4, size=k).astype(np.float32)
+    beta = rng.uniform(0.5, 2, size=k).astype(np.float32)
+
+    d = {name: to_dev(queue, x) for name, x in dict(pre=pre, post=post, theta=theta, mat=mat,
+                                                    delta=delta, learn=learn, scale=scale).items()}
+    want = clone(delta)
+    if rule == "bcm":
+        plan = nl().plan_bcm(queue, d["pre"], d["post"], d["theta"], d["delta"], alpha)
+        orc().plan_bcm(None, pre, post, theta, want, alpha)()
+    elif rule == "oja":
+        plan = nl().plan_oja(queue, d["pre"], d["post"], d["mat"], d["delta"], alpha, beta)
+        orc().plan_oja(None, pre, post, mat, want, alpha, beta)()
+    else:
+        plan = nl().plan_voja(queue, d["pre"], d["post"], d["mat"], d["delta"], d["learn"],
+                              d["scale"], alpha)
+        orc().plan_voja(None, pre, post, mat, want, learn, scale, alpha)()
+    plan()
+    got = d["delta"].to_host()
+    assert np.abs(want.buf).max() > 0
+    assert np.array_equal(got.buf, want.buf)
+    for name, host in (("pre", pre), ("post", post), ("mat", mat)):
+        assert np.array_equal(d[name].buf, host.buf), "%s was modified" % name
+
+
+def test_learning_rule_on_views(queue, rng):
+    """Operands that are strided views of one buffer (what the simulator passes): rows of
+    a wider matrix as delta / weights, every other element as pre."""
+    m, n = 40, 24
+    big = RA([rng.normal(size=(m, 2 * n)), rng.normal(size=(m, 2 * n)), rng.uniform(0, 9, size=2 * n),
+              rng.uniform(0, 9, size=m)])
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    s = big.starts
+    host = lambda start, s0, s1, st0: RaggedArray.from_buffer(big.buf, [start], [s0], [s1], [st0], [1])
+    dbig = to_dev(queue, big)
+    from nengo_ocl_amd.hipraggedarray import HIPRaggedArray
+
+    dev = lambda start, s0, s1, st0: HIPRaggedArray.from_buffer(
+        queue, dbig.dev_buf, np.int32([start]), np.int32([s0]), np.int32([s1]), np.int32([st0]),
+        np.int32([1]))
+    specs = dict(delta=(s[0] + n, m, n, 2 * n), weights=(s[1], m, n, 2 * n), pre=(s[2], n, 1, 2),
+                 post=(s[3], m, 1, 1))
+    h = {k: host(*v) for k, v in specs.items()}
+    g = {k: dev(*v) for k, v in specs.items()}
+    alpha, beta = np.float32([1e-3]), np.float32([1.5])
+    orc().plan_oja(None, h["pre"], h["post"], h["weights"], h["delta"], alpha, beta)()
+    nl().plan_oja(queue, g["pre"], g["post"], g["weights"], g["delta"], alpha, beta)()
+    assert np.array_equal(dbig.buf, big.buf)
+
+
+# ------------------------------------------------------------------ convolution, pooling
+CONV_CASES = [
+    # shape_in (i, j, c), n_filters, kernel, strides, padding
+    ((28, 28, 1), 32, (3, 3), (1, 1), "valid"),
+    ((14, 14, 32), 64, (3, 3), (2, 2), "same"),
+    ((9, 11, 3), 4, (3, 5), (2, 3), "same"),
+    ((1, 100, 6), 5, (1, 7), (1, 2), "valid"),       # a 1-D convolution as the simulator poses it
+    ((33, 17, 70), 3, (5, 5), (1, 1), (2, 1)),       # more channels than one LDS chunk holds
+    ((6, 6, 2), 300, (6, 6), (1, 1), "valid"),       # one output pixel, many filters
+]
+
+
+@pytest.mark.parametrize("channels_last", [True, False])
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d(queue, rng, case, channels_last):
+    """Bit-identical to the oracle: per output the same fused multiply-adds in the same
+    order (channel, kernel row, kernel column), whatever the tiling."""
+    (nxi, nxj, nc), nf, (si, sj), (sti, stj), padding = case
+    if padding == "valid":
+        pi, pj = 0, 0
+    elif padding == "same":
+        pi, pj = (si - 1) // 2, (sj - 1) // 2
+    else:
+        pi, pj = padding
+    nyi, nyj = (nxi + 2 * pi - si) // sti + 1, (nxj + 2 * pj - sj) // stj + 1
+    shape_in = (nxi, nxj, nc) if channels_last else (nc, nxi, nxj)
+    shape_out = (nyi, nyj, nf) if channels_last else (nf, nyi, nyj)
+    # the image and kernel sit between other signals of one buffer, as in the simulator
+    data = RA([rng.normal(size=5), rng.normal(size=nxi * nxj * nc),
+               rng.normal(size=si * sj * nc * nf), rng.normal(size=nyi * nyj * nf),
+               rng.normal(size=3)])
+    dev = to_dev(queue, data)
+    nl().plan_conv2d(queue, dev[[1]], dev[[3]], dev[[2]], shape_in, shape_out, (si, sj),
+                     padding=padding, strides=(sti, stj), channels_last=channels_last)()
+    orc().plan_conv2d(None, data[[1]], data[[3]], data[[2]], shape_in, shape_out, (si, sj),
+                      padding=padding, strides=(sti, stj), channels_last=channels_last)()
+    assert np.array_equal(dev.buf, data.buf)
+
+
+def test_local_filtering(queue, rng):
+    nxi, nxj, nc, nf, si, sj = 12, 10, 3, 5, 3, 2
+    nyi, nyj = nxi - si + 1, nxj - sj + 1
+    for channels_last in (True, False):
+        data = RA([rng.normal(size=nxi * nxj * nc), rng.normal(size=nf * nc * si * sj * nyi * nyj),
+                   np.zeros(nf * nyi * nyj)])
+        dev = to_dev(queue, data)
+        shape_in = (nxi, nxj, nc) if channels_last else (nc, nxi, nxj)
+        shape_out = (nyi, nyj, nf) if channels_last else (nf, nyi, nyj)
+        nl().plan_conv2d(queue, dev[[0]], dev[[2]], dev[[1]], shape_in, shape_out, (si, sj),
+                         conv=False, channels_last=channels_last)()
+        orc().plan_conv2d(None, data[[0]], data[[2]], data[[1]], shape_in, shape_out, (si, sj),
+                          conv=False, channels_last=channels_last)()
+        assert np.abs(data[2]).max() > 0
+        assert np.array_equal(dev.buf, data.buf)
+
+
+def test_conv2d_rejects_bad_arguments(queue, rng):
+    data = RA([np.zeros(50), np.zeros(9), np.zeros(18)])
+    dev = to_dev(queue, data)
+    with pytest.raises(AssertionError):  # X is not the size shape_in says
+        nl().plan_conv2d(queue, dev[[0]], dev[[2]], dev[[1]], (5, 5, 1), (3, 3, 2), (3, 3))
+    with pytest.raises(ValueError):
+        nl().plan_conv2d(queue, dev[[0]], dev[[2]], dev[[1]], (5, 10, 1), (3, 6, 1), (3, 3),
+                         padding="full")
+    with pytest.raises(AssertionError):  # biases are not supported, as in the reference
+        nl().plan_conv2d(queue, dev[[0]], dev[[2]], dev[[1]], (5, 10, 1), (3, 6, 1), (3, 3),
+                         biases=dev[[1]])
+
+
+@pytest.mark.parametrize("shape,pool,strides", [((3, 4, 4, 8, 12), (2, 3), (2, 3)),
+                                                ((1, 3, 3, 5, 5), (2, 2), (2, 2)),
+                                                ((16, 14, 14, 28, 28), (2, 2), (2, 2)),
+                                                ((5, 9, 7, 20, 15), (3, 3), (2, 2))])
+def test_pool2d(queue, rng, shape, pool, strides):
+    nc, nyi, nyj, nxi, nxj = shape
+    img = rng.normal(size=nc * nxi * nxj)
+    img[rng.randint(0, img.size, size=5)] = np.nan  # skipped by the mean
+    data = RA([np.zeros(3), img, np.zeros(nc * nyi * nyj)])
+    dev = to_dev(queue, data)
+    nl().plan_pool2d(queue, dev[[1]], dev[[2]], shape, pool, strides)()
+    orc().plan_pool2d(None, data[[1]], data[[2]], shape, pool, strides)()
+    assert np.array_equal(dev.buf, data.buf, equal_nan=True)
+
+
+# ------------------------------------------------------------------ noise
+def test_philox_known_answers(queue):
+    """The generator's published test vectors, on the device."""
+    import ctypes
+
+    from nengo_ocl_amd import _lib
+    from nengo_ocl_amd.hipraggedarray import to_device
+    from helpers import PHILOX_KNOWN_ANSWERS
+
+    rows = np.array([c + k for c, k, _ in PHILOX_KNOWN_ANSWERS], dtype=np.uint32)
+    want = np.array([o for _, _, o in PHILOX_KNOWN_ANSWERS], dtype=np.uint32)
+    extra = np.random.RandomState(0).randint(0, 2 ** 32, size=(500, 6), dtype=np.uint64).astype(np.uint32)
+    rows = np.concatenate([rows, extra])
+    d_in = to_device(queue, rows.view(np.int32))
+    d_out = to_device(queue, np.zeros((len(rows), 4), dtype=np.int32))
+    _lib.check(queue.lib.nhip_philox4x32(queue.handle, d_in.ptr, d_out.ptr, len(rows)))
+    queue.finish()
+    got = d_out.get().view(np.uint32)
+    assert np.array_equal(got[:3], want)
+    assert np.array_equal(got, orc().philox4x32(rows))
+
+
+def test_whitenoise(queue):
+    """Same streams as the oracle: uniform samples bit for bit; Gaussian samples go through
+    double-precision log / sqrt / sin / cos of two math libraries and one final rounding,
+    so they agree to the last float32 bit except where the double result lies within an
+    ulp of a rounding boundary (tolerance: 1 float32 ulp, mismatches reported)."""
+    dt = 1e-3
+    sizes = [20000, 7, 1, 3000, 257]
+    enums = [1, 0, 1, 0, 1]
+    params = [(0.0, 1.0), (-2.0, 3.0), (1.5, 0.5), (0.0, 1.0), (0.0, 2.0)]
+    scale, inc, seeds = [1, 0, 0, 1, 0], [0, 0, 1, 1, 0], [11, 12, 13, 14, 2 ** 31 + 5]
+    Y = RA([np.full(n, 0.25) for n in sizes])
+    dev = to_dev(queue, Y)
+    gplan = nl().plan_whitenoise(queue, dev, np.int32(enums), np.float32(params), scale, inc, dt,
+                                 seeds)
+    oplan = orc().plan_whitenoise(None, Y, enums, params, scale, inc, dt, seeds)
+    for call in range(3):
+        gplan()
+        oplan()
+        got = dev.to_host()
+        for i, e in enumerate(enums):
+            if e == 0:
+                assert np.array_equal(got[i], Y[i])
+            else:
+                ulp = np.spacing(np.abs(Y[i]))
+                assert np.all(np.abs(got[i] - Y[i]) <= ulp)
+                mismatch = np.mean(got[i] != Y[i])
+                assert mismatch < 1e-3, "Gaussian samples differing in the last bit: %g" % mismatch
+        dev.dev_buf.set(Y.buf)  # same starting point for the incrementing items
+    assert np.array_equal(gplan.counters.get()[:len(sizes)], np.full(len(sizes), 3))
+    gplan.reset_streams()
+    oplan.reset_streams()
+    Y.buf[:] = 0.25
+    dev.dev_buf.set(Y.buf)
+    gplan()
+    oplan()
+    assert np.allclose(dev.buf, Y.buf, rtol=1e-6, atol=0)

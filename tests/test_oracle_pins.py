@@ -10,7 +10,7 @@ compare the HIP kernels with the oracle.
 import numpy as np
 import pytest
 
-from helpers import RA, clone
+from helpers import PHILOX_KNOWN_ANSWERS, RA, clone
 from oracle import oracle as orc
 
 
@@ -479,3 +479,194 @@ def test_spmv_against_scipy():
     Y = clone(Y0)
     orc.plan_sparse_dot_inc(None, [dup], RA([[1.0, 10.0, 100.0]]), Y[[3]], inc=False).plans[0]()
     assert np.array_equal(Y[3][:, 0], np.float32([300, 0, 3, 0, 0]))
+
+
+# ------------------------------------------------------------------ learning rules
+def _rule_operands(rng, shapes):
+    pre = RA([rng.uniform(0, 200, size=n) for m, n in shapes])
+    post = RA([rng.uniform(0, 200, size=m) for m, n in shapes])
+    theta = RA([rng.uniform(0, 200, size=m) for m, n in shapes])
+    mat = RA([rng.normal(scale=0.01, size=(m, n)) for m, n in shapes])
+    delta = RA([rng.normal(size=(m, n)) for m, n in shapes])  # stale values must be overwritten
+    return pre, post, theta, mat, delta
+
+
+def test_learning_rules_against_float64_outer_forms():
+    """BCM, Oja and Voja deltas against their matrix forms in float64: a swapped index,
+    a wrong sign or a dropped factor changes the matrices far beyond rounding."""
+    rng = np.random.RandomState(5)
+    shapes = [(7, 5), (1, 9), (33, 70), (64, 1)]
+    pre, post, theta, mat, delta = _rule_operands(rng, shapes)
+    k = len(shapes)
+    alpha = rng.uniform(1e-6, 1e-4, size=k).astype(np.float32)
+    beta = rng.uniform(0.5, 2, size=k).astype(np.float32)
+    f64 = lambda ra, i: ra[i].astype(np.float64)
+
+    orc.plan_bcm(None, pre, post, theta, delta, alpha)()
+    for i in range(k):
+        po, th, pr = f64(post, i)[:, 0], f64(theta, i)[:, 0], f64(pre, i)[:, 0]
+        np.testing.assert_allclose(delta[i], alpha[i] * np.outer(po * (po - th), pr), rtol=1e-5,
+                                   atol=1e-12)
+
+    orc.plan_oja(None, pre, post, mat, delta, alpha, beta)()
+    for i in range(k):
+        po, pr, w = f64(post, i)[:, 0], f64(pre, i)[:, 0], f64(mat, i)
+        want = alpha[i] * (np.outer(po, pr) - beta[i] * w * (po ** 2)[:, None])
+        np.testing.assert_allclose(delta[i], want, rtol=1e-4, atol=1e-9)
+
+    learn = RA([[rng.uniform(0, 1)] for _ in shapes])
+    scale = RA([rng.uniform(1, 30, size=m) for m, n in shapes])
+    orc.plan_voja(None, pre, post, mat, delta, learn, scale, alpha)()
+    for i in range(k):
+        po, pr, enc = f64(post, i)[:, 0], f64(pre, i)[:, 0], f64(mat, i)
+        want = alpha[i] * learn[i][0, 0] * po[:, None] * (np.outer(f64(scale, i)[:, 0], pr) - enc)
+        np.testing.assert_allclose(delta[i], want, rtol=1e-4, atol=1e-9)
+
+
+def test_learning_rule_fixed_points():
+    """What the rules are for: BCM's delta vanishes where post == theta and changes sign
+    there; Oja's vanishes for a unit-norm weight row aligned with the input (post = w.pre);
+    Voja's vanishes where the encoder already equals the scaled input, and with a zero
+    learning signal."""
+    pre = RA([[1.0, 2.0, 3.0]])
+    post = RA([[4.0, 6.0, 8.0]])
+    theta = RA([[4.0, 7.0, 5.0]])
+    delta = RA([np.ones((3, 3))])
+    orc.plan_bcm(None, pre, post, theta, delta, np.float32([0.5]))()
+    assert np.all(delta[0][0] == 0) and np.all(delta[0][1] < 0) and np.all(delta[0][2] > 0)
+
+    x = np.float32([0.6, 0.8])  # unit norm
+    w = RA([np.float32([x, 2 * x])])
+    pre, post = RA([x]), RA([np.float32([x @ x, 2 * x @ x])])
+    delta = RA([np.ones((2, 2))])
+    orc.plan_oja(None, pre, post, w, delta, np.float32([1.0]), np.float32([1.0]))()
+    np.testing.assert_allclose(delta[0][0], 0, atol=1e-7)       # |w| = 1: fixed point
+    assert np.all(delta[0][1] * x < 0)                           # |w| = 2: pulled back
+
+    enc = RA([np.float32([[2.0, 4.0], [1.0, 1.0]])])
+    pre, post = RA([[1.0, 2.0]]), RA([[3.0, 3.0]])
+    scale = RA([[2.0, 2.0]])
+    for learn, moves in ((1.0, True), (0.0, False)):
+        delta = RA([np.ones((2, 2))])
+        orc.plan_voja(None, pre, post, enc, delta, RA([[learn]]), scale, np.float32([0.1]))()
+        assert np.all(delta[0][0] == 0)
+        assert np.all(delta[0][1] > 0) if moves else np.all(delta[0] == 0)
+
+
+# ------------------------------------------------------------------ convolution, pooling
+@pytest.mark.parametrize("channels_last", [True, False])
+@pytest.mark.parametrize("padding,strides", [("valid", (1, 1)), ("same", (1, 1)), ("same", (2, 3)),
+                                             ("valid", (2, 2)), ((2, 1), (1, 1))])
+def test_conv2d_against_scipy(channels_last, padding, strides):
+    """Convolution against scipy.signal.correlate2d per (channel, filter) pair: a zero-padded
+    full correlation subsampled by the strides."""
+    from scipy.signal import correlate2d
+
+    rng = np.random.RandomState(8)
+    nxi, nxj, nc, nf, si, sj = 9, 11, 3, 4, 3, 5
+    sti, stj = strides
+    if padding == "valid":
+        pi, pj = 0, 0
+    elif padding == "same":
+        pi, pj = (si - 1) // 2, (sj - 1) // 2
+    else:
+        pi, pj = padding
+    nyi, nyj = (nxi + 2 * pi - si) // sti + 1, (nxj + 2 * pj - sj) // stj + 1
+    img = rng.normal(size=(nxi, nxj, nc))
+    filt = rng.normal(size=(si, sj, nc, nf))
+    X = RA([(img if channels_last else img.transpose(2, 0, 1)).ravel()])
+    F = RA([filt.ravel()])
+    Y = RA([np.full(nyi * nyj * nf, 7.0)])
+    shape_in = (nxi, nxj, nc) if channels_last else (nc, nxi, nxj)
+    shape_out = (nyi, nyj, nf) if channels_last else (nf, nyi, nyj)
+    orc.plan_conv2d(None, X, Y, F, shape_in, shape_out, (si, sj), padding=padding,
+                    strides=strides, channels_last=channels_last)()
+    got = Y[0].reshape(shape_out)
+    if not channels_last:
+        got = got.transpose(1, 2, 0)
+    padded = np.pad(img, ((pi, pi), (pj, pj), (0, 0)))
+    for k in range(nf):
+        want = sum(correlate2d(padded[:, :, c], filt[:, :, c, k], mode="valid") for c in range(nc))
+        want = want[::sti, ::stj][:nyi, :nyj]
+        np.testing.assert_allclose(got[:, :, k], want, rtol=1e-5, atol=1e-5)
+
+
+def test_local_filtering_brute_force():
+    rng = np.random.RandomState(9)
+    nxi, nxj, nc, nf, si, sj = 5, 6, 2, 3, 2, 3
+    nyi, nyj = nxi - si + 1, nxj - sj + 1
+    img = rng.normal(size=(nc, nxi, nxj))
+    filt = rng.normal(size=(nf, nc, si, sj, nyi, nyj))
+    X, F, Y = RA([img.ravel()]), RA([filt.ravel()]), RA([np.zeros(nf * nyi * nyj)])
+    orc.plan_conv2d(None, X, Y, F, (nc, nxi, nxj), (nf, nyi, nyj), (si, sj), conv=False,
+                    channels_last=False)()
+    want = np.zeros((nf, nyi, nyj))
+    for k in range(nf):
+        for i in range(nyi):
+            for j in range(nyj):
+                want[k, i, j] = np.sum(filt[k, :, :, :, i, j] * img[:, i:i + si, j:j + sj])
+    np.testing.assert_allclose(Y[0].reshape(nf, nyi, nyj), want, rtol=1e-5, atol=1e-5)
+
+
+def test_pool2d_block_means_and_edges():
+    rng = np.random.RandomState(10)
+    nc, nxi, nxj = 3, 8, 12
+    img = rng.normal(size=(nc, nxi, nxj)).astype(np.float32)
+    X, Y = RA([img.ravel()]), RA([np.zeros(nc * 4 * 4)])
+    orc.plan_pool2d(None, X, Y, (nc, 4, 4, nxi, nxj), (2, 3), (2, 3))()
+    want = img.reshape(nc, 4, 2, 4, 3).mean(axis=(2, 4))
+    np.testing.assert_allclose(Y[0].reshape(nc, 4, 4), want, rtol=1e-6, atol=1e-6)
+    # windows hanging over the bottom / right edge average what is inside; NaNs are skipped
+    img2 = np.arange(25, dtype=np.float32).reshape(1, 5, 5)
+    img2[0, 0, 1] = np.nan
+    X, Y = RA([img2.ravel()]), RA([np.zeros(9)])
+    orc.plan_pool2d(None, X, Y, (1, 3, 3, 5, 5), (2, 2), (2, 2))()
+    got = Y[0].reshape(3, 3)
+    assert got[0, 0] == np.float32((0 + 5 + 6) / 3)
+    assert got[2, 2] == 24 and got[0, 2] == np.float32((4 + 9) / 2)
+    assert got[2, 0] == np.float32((20 + 21) / 2)
+
+
+# ------------------------------------------------------------------ noise
+def test_philox_known_answers():
+    rows = np.array([c + k for c, k, _ in PHILOX_KNOWN_ANSWERS], dtype=np.uint32)
+    want = np.array([o for _, _, o in PHILOX_KNOWN_ANSWERS], dtype=np.uint32)
+    assert np.array_equal(orc.philox4x32(rows), want)
+
+
+def test_whitenoise_distributions_and_streams():
+    """Uniform and Gaussian samples against their distributions (Kolmogorov-Smirnov),
+    the 1/sqrt(dt) scaling, increment mode, independence between calls, elements and
+    seeds, and the restart of the streams."""
+    from scipy import stats
+
+    n, dt = 20000, 1e-3
+    Y = RA([np.zeros(n), np.zeros(n), np.zeros(n), np.ones(5)])
+    enums = [0, 1, 1, 0]
+    params = [(-2.0, 3.0), (1.5, 0.5), (0.0, 1.0), (0.0, 1.0)]
+    plan = orc.plan_whitenoise(None, Y, enums, params, [0, 0, 1, 0], [0, 0, 0, 1], dt,
+                               [1, 2, 3, 4])
+    plan()
+    first = np.array(Y.buf)
+    assert stats.kstest(Y[0][:, 0], stats.uniform(-2, 5).cdf).pvalue > 1e-3
+    assert Y[0].min() >= -2 and Y[0].max() < 3
+    assert stats.kstest(Y[1][:, 0], stats.norm(1.5, 0.5).cdf).pvalue > 1e-3
+    assert stats.kstest(Y[2][:, 0], stats.norm(0, np.sqrt(1 / dt)).cdf).pvalue > 1e-3
+    assert np.all((Y[3] >= 1) & (Y[3] < 2))  # incremented, not set
+    # neighbouring elements (which share a generator block) and consecutive calls are
+    # uncorrelated
+    z = (Y[1][:, 0] - 1.5) / 0.5
+    for lag in (1, 2, 3, 4):
+        assert abs(np.mean(z[:-lag] * z[lag:])) < 4 / np.sqrt(n)
+    plan()
+    z2 = (Y[1][:, 0] - 1.5) / 0.5
+    assert abs(np.mean(z * z2)) < 4 / np.sqrt(n)
+    assert not np.array_equal(first[:n], Y.buf[:n])
+    # restart: same samples again; another seed: other samples
+    plan.reset_streams()
+    Y.buf[-5:] = 1
+    plan()
+    assert np.array_equal(Y.buf, first)
+    Y2 = RA([np.zeros(n)])
+    orc.plan_whitenoise(None, Y2, [0], [(-2.0, 3.0)], [0], [0], dt, [99])()
+    assert abs(np.corrcoef(Y2[0][:, 0], first[:n])[0, 1]) < 4 / np.sqrt(n)

@@ -368,3 +368,80 @@ def test_profiling_and_plan_listing(queue, capsys):
         prof.print_plans()
         out = capsys.readouterr().out
         assert "Profiling" in out and "hipra_gemv.tile_lif" in out and "totals:" in out
+
+
+def _pair_equal(make, steps, check=None):
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    made_g, made_c = make(), make()
+    with Simulator(made_g[0], seed=1) as gpu, OracleSimulator(made_c[0], seed=1) as cpu:
+        gpu.run_steps(steps)
+        cpu.run_steps(steps)
+        for a, b in zip(made_g[-1], made_c[-1]):
+            assert np.array_equal(gpu.data[a], cpu.data[b])
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+        if check is not None:
+            check(gpu, made_g)
+        return [p.name for p in gpu._plans]
+
+
+@pytest.mark.parametrize("rule_type", ["BCM", "Oja"])
+def test_hebbian_learning_network(queue, rule_type):
+    """Weights between two populations learned with BCM / Oja for 400 steps: weights,
+    deltas, spikes and every other signal bit-identical to the oracle simulator."""
+    from nengo_ocl_amd import minibuilder as mb
+    from test_builder_extras import hebbian_network
+
+    make = lambda: hebbian_network(mb.BCM(learning_rate=1e-9) if rule_type == "BCM"
+                                   else mb.Oja(learning_rate=1e-6))
+
+    def check(gpu, made):
+        w = np.array(gpu.signals[gpu.model.sig[made[1]]["weights"]])
+        assert np.abs(w).max() > 5e-3  # started at ~3e-3: they were learned
+
+    names = _pair_equal(make, 400, check)
+    assert "hip_" + rule_type.lower() in names
+
+
+def test_voja_learning_network(queue):
+    from test_builder_extras import voja_network
+
+    names = _pair_equal(lambda: voja_network(), 400)
+    assert "hip_voja" in names
+
+
+def test_noise_network(queue):
+    """White-noise nodes and noise injected into neurons.  Uniform streams are equal bit
+    for bit; Gaussian ones to the last bit except for rare rounding-boundary cases, and a
+    single differing sample can move a spike, so this compares samples within one ulp and
+    spike counts within the spiking criterion (99.9 %)."""
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+    from test_builder_extras import noise_network
+
+    (net, probes), (net_o, probes_o) = noise_network(), noise_network()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        assert "hip_whitenoise" in [p.name for p in gpu._plans]
+        gpu.run_steps(1000)
+        cpu.run_steps(1000)
+        g = [np.array(gpu.data[p]) for p in probes]
+        c = [np.array(cpu.data[p]) for p in probes_o]
+        assert np.array_equal(g[1], c[1])                                 # uniform
+        assert np.all(np.abs(g[0] - c[0]) <= np.spacing(np.abs(c[0])))    # Gaussian
+        print("Gaussian samples equal: %.5f %%" % (100 * np.mean(g[0] == c[0])))
+        counts_g, counts_c = g[2].sum(axis=0) * 1e-3, c[2].sum(axis=0) * 1e-3
+        assert np.mean(np.round(counts_g) == np.round(counts_c)) >= 0.999
+        assert np.array_equal(g[3], c[3])                                 # the quiet twin
+        first = g[0]
+        gpu.reset()
+        gpu.run_steps(1000)
+        assert np.array_equal(first, gpu.data[probes[0]])                 # streams restart
+
+
+@pytest.mark.parametrize("channels_last", [True, False])
+def test_convolution_network(queue, channels_last):
+    from test_builder_extras import conv_network
+
+    names = _pair_equal(lambda: conv_network(channels_last), 5)
+    assert "hip_conv2d" in names
