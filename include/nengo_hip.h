@@ -37,6 +37,7 @@ extern "C" {
 
 #define NHIP_E_BADARG (-1)   /* null pointer / negative count / unknown mode   */
 #define NHIP_E_BADCLASS (-2) /* GEMV class (lanes-per-row, vector width) unknown */
+#define NHIP_E_RTC (-3)      /* run-time compilation failed (see the log)          */
 
 /* ---- library ---------------------------------------------------------- */
 int nhip_abi_version(void);
@@ -353,6 +354,27 @@ typedef struct NhipSeqOp {
 /* at most 16 operations with at most 32 work-list rows in all; n_rows = the sum of
  * n_blocks over `ops` (the library cannot read the device table to check it) */
 int nhip_sequence(void *stream, const void *ops, int n_ops, int n_rows);
+
+/* ---- function nodes compiled at run time ----------------------------------
+ * replaces: `plan_direct` (:954-1025), which builds an OpenCL program from the
+ * translated body of a Python function.  `source` is HIP source text holding
+ *     extern "C" __global__ void <kernel_name>(int n, const int *t_starts,
+ *         const float *T, const int *x_starts, const float *X,
+ *         const int *y_starts, float *Y)
+ * in which thread k < n computes instance k: it reads its time at T + t_starts[k]
+ * and its input vector at X + x_starts[k] (either may be unused and NULL) and
+ * writes its output vector at Y + y_starts[k].
+ * nhip_rtc_compile compiles for `arch` (NULL: gfx950) and needs no device; the
+ * compiler's messages are copied into `log`.  nhip_rtc_load loads the code on the
+ * current device (once per program) and looks the kernel up; nhip_rtc_destroy
+ * unloads and frees (no launch of the program may be pending or recorded). */
+int nhip_rtc_compile(const char *source, const char *arch, void **program_out, char *log,
+                     int log_len);
+int nhip_rtc_load(void *program, const char *kernel_name, void **function_out);
+int nhip_rtc_destroy(void *program);
+int nhip_rtc_launch_direct(void *stream, void *function, int n, const int *t_starts,
+                           const float *T, const int *x_starts, const float *X,
+                           const int *y_starts, float *Y);
 
 /* ---- executor ----------------------------------------------------------
  * replaces the Python launch loop of `Plans.enqueue_n_times` (plan.py:137-149):

@@ -47,6 +47,11 @@ SIGNATURES = {
     "nhip_pool2d": [P, P, P, P],
     "nhip_whitenoise": [P, P, c_int, P, c_double, P],
     "nhip_philox4x32": [P, P, P, c_int],
+    "nhip_rtc_compile": [ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(c_void_p),
+                         ctypes.c_char_p, c_int],
+    "nhip_rtc_load": [P, ctypes.c_char_p, ctypes.POINTER(c_void_p)],
+    "nhip_rtc_destroy": [P],
+    "nhip_rtc_launch_direct": [P, P, c_int, P, P, P, P, P, P],
     "nhip_copy": [P, P, c_int, P, P],
     "nhip_slicedcopy": [P, P, c_int, P, P, P, P],
     "nhip_reset": [P, P, c_int, P],

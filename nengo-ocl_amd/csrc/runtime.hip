@@ -15,6 +15,7 @@ extern "C" const char* nhip_error_string(int err) {
         case 0: return "success";
         case NHIP_E_BADARG: return "nengo_hip: bad argument (null pointer, negative count or unknown mode)";
         case NHIP_E_BADCLASS: return "nengo_hip: unknown GEMV kernel class (flavor, lanes per row, vector width)";
+        case NHIP_E_RTC: return "nengo_hip: run-time compilation of a function node failed (see its log)";
     }
     return hipGetErrorString(static_cast<hipError_t>(err));
 }

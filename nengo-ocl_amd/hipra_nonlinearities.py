@@ -313,30 +313,101 @@ _DIRECT_RE = re.compile(
 
 
 def plan_direct(queue, code, init, input_names, inputs, output, tag=None):
-    """Function nodes whose translated code is ``OUTPUT__[0] = f(name[0]);`` with f in
-    the unary table.  Anything else raises NotImplementedError, on which the
-    Simulator falls back to a host callback, as the reference does when its
-    translator fails (simulator.py:955-964)."""
+    """A function node on the device: ``code`` (C statements assigning ``OUTPUT__[i]``
+    from the inputs ``name[i]``, after the declarations in ``init``) runs once per
+    output item, one thread each (reference ``plan_direct`` :954-1025).
+
+    ``OUTPUT__[0] = f(name[0]);`` with f in the unary table goes to a precompiled kernel
+    (which can share a launch with other short operations); any other code is compiled
+    at run time.  Compilation errors raise NotImplementedError, on which the Simulator
+    falls back to a host callback, as the reference does when its translator fails
+    (simulator.py:955-964)."""
     assert len(input_names) == len(inputs)
     for x in inputs:
         assert len(x) == len(output)
     for x in list(inputs) + [output]:
         assert (x.shape1s == 1).all() and (x.stride1s == 1).all()
         assert (x.stride0s == 1).all()
+        assert x.ctype == "float"
+    _check(*([("input", x) for x in inputs] + [("output", output)]))
     m = _DIRECT_RE.match(code or "")
-    if (init or "").strip() or m is None or m.group("fn") not in UNARY_OPCODES:
-        raise NotImplementedError("only single unary functions run on the device: %r" % code)
-    if m.group("arg") not in input_names:
-        raise NotImplementedError("unknown input %r" % m.group("arg"))
-    x = inputs[list(input_names).index(m.group("arg"))]
-    assert (x.shape0s == 1).all() and (output.shape0s == 1).all()
-    _check(("input", x), ("output", output))
+    if (not (init or "").strip() and m is not None and m.group("fn") in UNARY_OPCODES
+            and m.group("arg") in input_names):
+        x = inputs[list(input_names).index(m.group("arg"))]
+        assert (x.shape0s == 1).all() and (output.shape0s == 1).all()
+        table, n = _dev_table(queue, [x.starts, output.starts, np.ones(len(output), np.int32)], 4)
+        plan = Plan(queue, queue.lib.nhip_direct_unary,
+                    (UNARY_OPCODES[m.group("fn")], table.ptr, n, x.ptr, output.ptr),
+                    gsize=(WG * max(n, 1),), lsize=(WG,),
+                    full_args=(table, x.dev_buf, output.dev_buf), name="hip_direct", tag=tag)
+        plan.description = _description(output)
+        return plan
+    return _plan_direct_compiled(queue, code, init, input_names, inputs, output, tag)
 
-    table, n = _dev_table(queue, [x.starts, output.starts, np.ones(len(output), np.int32)], 4)
-    plan = Plan(queue, queue.lib.nhip_direct_unary,
-                (UNARY_OPCODES[m.group("fn")], table.ptr, n, x.ptr, output.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,),
-                full_args=(table, x.dev_buf, output.dev_buf), name="hip_direct", tag=tag)
+
+DIRECT_KERNEL = """\
+extern "C" __global__ void direct(int n__, const int* in0_starts__, const float* in0_data__,
+                                  const int* in1_starts__, const float* in1_data__,
+                                  const int* out_starts__, float* out_data__) {
+    const int k__ = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k__ >= n__) return;
+%(inputs)s
+    float* OUTPUT__ = out_data__ + out_starts__[k__];
+%(init)s
+%(code)s
+}
+"""
+
+
+def direct_kernel_source(code, init, input_names):
+    """HIP source of the kernel ``plan_direct`` compiles for this code."""
+    if len(input_names) > 2:
+        raise NotImplementedError("function nodes take at most two inputs (time, vector)")
+    lines = ["    const float* %s = in%d_data__ + in%d_starts__[k__];" % (name, i, i)
+             for i, name in enumerate(input_names)]
+    indent = lambda text: "\n".join("    " + line for line in (text or "").splitlines())
+    return DIRECT_KERNEL % dict(inputs="\n".join(lines), init=indent(init), code=indent(code))
+
+
+_compiled_programs = {}  # source text -> compiled program (kept for the life of the process)
+
+
+def compile_direct(lib, source):
+    """Compile (or look up) a function-node kernel; raises NotImplementedError with the
+    compiler's messages if the source does not compile.  Needs no device."""
+    import ctypes
+
+    program = _compiled_programs.get(source)
+    if program is None:
+        handle = ctypes.c_void_p()
+        log = ctypes.create_string_buffer(8192)
+        err = lib.nhip_rtc_compile(source.encode(), b"gfx950", ctypes.byref(handle), log, len(log))
+        if err != 0:
+            raise NotImplementedError("the function's kernel does not compile:\n%s"
+                                      % log.value.decode(errors="replace"))
+        program = _compiled_programs[source] = handle
+    return program
+
+
+def _plan_direct_compiled(queue, code, init, input_names, inputs, output, tag):
+    import ctypes
+
+    source = direct_kernel_source(code, init, list(input_names))
+    program = compile_direct(queue.lib, source)
+    function = ctypes.c_void_p()
+    _lib.check(queue.lib.nhip_rtc_load(program, b"direct", ctypes.byref(function)),
+               "loading a function-node kernel")
+    n = len(output)
+    starts = [to_device(queue, np.ascontiguousarray(x.starts, dtype=np.int32)) for x in inputs]
+    out_starts = to_device(queue, np.ascontiguousarray(output.starts, dtype=np.int32))
+    pairs = [(s.ptr, x.ptr) for s, x in zip(starts, inputs)] + [(None, None)] * (2 - len(inputs))
+    args = (function, n, pairs[0][0], pairs[0][1], pairs[1][0], pairs[1][1], out_starts.ptr,
+            output.ptr)
+    plan = Plan(queue, queue.lib.nhip_rtc_launch_direct, args, gsize=(64 * max(-(-n // 64), 1),),
+                lsize=(64,), full_args=tuple(starts) + (out_starts, output.dev_buf, function)
+                + tuple(x.dev_buf for x in inputs), name="hip_direct_compiled", tag=tag)
+    plan.source = source
+    plan.bw_per_call = output.nbytes + sum(x.nbytes for x in inputs)
     plan.description = _description(output)
     return plan
 

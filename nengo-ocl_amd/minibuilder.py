@@ -313,8 +313,15 @@ class Network:
             model.sig[node] = {"in": sig_in, "out": sig_in}
             model.add_op(ir.Reset(sig_in))
             return
-        if node.size_in:
-            raise NotImplementedError("nodes with both input and output function")
+        if node.size_in:  # out = f(t, in)
+            if not callable(node.output) or isinstance(node.output, ir.Process):
+                raise NotImplementedError("nodes with input need a function as output")
+            sig_in = ir.Signal(np.zeros(node.size_in), name="<Node %s>.in" % name)
+            out = ir.Signal(np.zeros(node.size_out), name="<Node %s>.out" % name)
+            model.sig[node] = {"in": sig_in, "out": out}
+            model.add_op(ir.Reset(sig_in))
+            model.add_op(ir.SimPyFunc(out, node.output, model.time, sig_in))
+            return
         if isinstance(node.output, np.ndarray):
             out = ir.Signal(node.output, name="<Node %s>.out" % name)
             model.sig[node] = {"in": None, "out": out}
@@ -497,8 +504,8 @@ class Network:
         elif isinstance(post, Neurons):
             target = model.sig[post]["in"]
         elif isinstance(post, Node):
-            if post.output is not None:
-                raise NotImplementedError("connections into function nodes")
+            if not post.size_in:
+                raise ValueError("%s: the target node takes no input" % name)
             target = model.sig[post]["in"]
         elif isinstance(post, (PES, Voja)):
             target = model.sig[post]["in"]

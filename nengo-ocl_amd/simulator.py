@@ -796,17 +796,35 @@ class Simulator:
         return plans
 
     def _plan_fn_on_device(self, fn, tt, xx, yy, fn_name):
-        """Functions of time alone from the unary table (``Node(np.sin)``)."""
+        """The function as a kernel: single unary functions of time from the precompiled
+        table (``Node(np.sin)``), everything else traced and compiled at run time
+        (reference ``_plan_fn_in_ocl``, simulator.py:968-1009)."""
+        from . import fn_trace
+
+        t_in, x_in = tt[0] is not None, xx[0] is not None
+        x_dim = xx[0].size if x_in else None
+        y_dim = yy[0].size
+        assert all((x.size if x is not None else None) == x_dim for x in xx)
+        assert all(y.size == y_dim for y in yy)
+        vector = lambda s: s.ndim == 1 or (s.ndim == 2 and s.shape[1] == 1)
+        if not all(vector(s) for s in list(yy) + (list(xx) if x_in else [])):
+            raise NotImplementedError("function nodes on matrix signals")
         try:
             known = _DIRECT_FUNCTIONS.get(fn)
         except TypeError:
             known = None
-        if known is None or tt[0] is None or xx[0] is not None or yy[0].size != 1:
-            raise NotImplementedError("not a single unary function of time")
-        inputs = [self.all_data[[self.sidx[t] for t in tt]]]
+        if known is not None and t_in and not x_in and y_dim == 1:
+            code, init, names = "OUTPUT__[0] = %s(t[0]);" % known, "", ["t"]
+        else:
+            traced = fn_trace.trace(fn, t_in, x_dim, y_dim)
+            code, init, names = traced.code, traced.init, traced.input_names
+        inputs = []
+        if t_in:
+            inputs.append(self.all_data[[self.sidx[t] for t in tt]])
+        if x_in:
+            inputs.append(self.all_data[[self.sidx[x] for x in xx]])
         output = self.all_data[[self.sidx[y] for y in yy]]
-        code = "OUTPUT__[0] = %s(t[0]);" % known
-        return self.backend.plan_direct(self.queue, code, "", ["t"], inputs, output, tag=fn_name)
+        return self.backend.plan_direct(self.queue, code, init, names, inputs, output, tag=fn_name)
 
     def _plan_fn_in_python(self, fn, tt, xx, yy, fn_name):
         t_in = tt[0] is not None

@@ -638,3 +638,48 @@ def test_whitenoise(queue):
     gplan()
     oplan()
     assert np.allclose(dev.buf, Y.buf, rtol=1e-6, atol=0)
+
+
+# ------------------------------------------------------------------ compiled function nodes
+def test_plan_direct_compiled_functions(queue, rng):
+    """Traced functions compiled at run time and launched over many node instances: the
+    device's float32 result against the Python function in double precision (rtol 1e-5 /
+    atol 2e-6: float32 evaluation of up to a dozen operations and library functions; the
+    reference's own check of translated functions allows rtol 1e-5 / atol 2e-7 on single
+    functions, tests/test_ast_conversion.py:198-200)."""
+    from nengo_ocl_amd import fn_trace as ft
+    from test_fn_trace import CASES
+
+    n = 300  # instances: several waves
+    skip_discontinuous = {20, 31}  # floor / mod / round: a float32 input next to a step
+    for case, (fn, t_in, x_dim, out_dim) in enumerate(CASES):
+        traced = ft.trace(fn, t_in, x_dim, out_dim)
+        T = RA([[rng.uniform(0, 2)] for _ in range(n)])
+        X = RA([rng.uniform(-3, 4, size=x_dim or 1) for _ in range(n)])
+        Y = RA([np.zeros(out_dim) for _ in range(n)])
+        dT, dX, dY = (to_dev(queue, a) for a in (T, X, Y))
+        inputs = ([dT] if t_in else []) + ([dX] if x_dim else [])
+        plan = nl().plan_direct(queue, traced.code, traced.init, traced.input_names, inputs, dY)
+        assert plan.name == "hip_direct_compiled"
+        plan()
+        got = dY.to_host()
+        if case in skip_discontinuous:
+            continue
+        for k in range(n):
+            args = ([float(T[k][0, 0])] if t_in else []) + ([X[k][:, 0].astype(np.float64)] if x_dim else [])
+            want = np.asarray(fn(*args), dtype=np.float64).ravel()
+            np.testing.assert_allclose(got[k][:, 0], want, rtol=1e-5, atol=2e-6,
+                                       err_msg="case %d instance %d" % (case, k))
+        assert np.array_equal(dX.buf, X.buf) and np.array_equal(dT.buf, T.buf)
+
+
+def test_plan_direct_unary_table_still_precompiled(queue):
+    T = RA([[0.3], [1.2]])
+    Y = RA([[0.0], [0.0]])
+    dT, dY = to_dev(queue, T), to_dev(queue, Y)
+    plan = nl().plan_direct(queue, "OUTPUT__[0] = sin(t[0]);", "", ["t"], [dT], dY)
+    assert plan.name == "hip_direct"
+    plan()
+    np.testing.assert_allclose(dY.buf, np.sin(np.float32([0.3, 1.2])), rtol=1e-6)
+    with pytest.raises(NotImplementedError, match="does not compile"):
+        nl().plan_direct(queue, "OUTPUT__[0] = undefined_function(t[0]);", "", ["t"], [dT], dY)

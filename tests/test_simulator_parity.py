@@ -445,3 +445,41 @@ def test_convolution_network(queue, channels_last):
 
     names = _pair_equal(lambda: conv_network(channels_last), 5)
     assert "hip_conv2d" in names
+
+
+def function_node_network(seed=3):
+    from nengo_ocl_amd import minibuilder as mb
+
+    net = mb.Network(seed=seed)
+    stim = net.Node(lambda t: [np.sin(6 * t), np.cos(3 * t) * np.exp(-t)], size_out=2)
+    ens = net.Ensemble(200, 2, neuron_type=mb.LIFRate())
+    net.Connection(stim, ens, synapse=None)
+    # a node computing on decoded values: product, a rectification and a saturating gain
+    calc = net.Node(lambda t, x: [x[0] * x[1], max(x[0], 0.0), np.tanh(3 * x[1]) if t > 0.1005 else 0.0],
+                    size_in=2, size_out=3)
+    net.Connection(ens, calc, synapse=0.01)
+    out = net.Ensemble(100, 3, neuron_type=mb.LIFRate())
+    net.Connection(calc, out, synapse=0.01)
+    return net, [net.Probe(stim), net.Probe(calc), net.Probe(out, synapse=0.02)]
+
+
+def test_function_nodes_run_on_the_device(queue):
+    """Function nodes (of time, and of time and input) are compiled into the step: no host
+    callback is left (`if_python_code="error"` would raise), the whole step is one graph,
+    and the probes follow the oracle simulator, which calls the Python functions on the
+    host, within the rate-neuron tolerance."""
+    from nengo_ocl_amd.plan import PythonPlan
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    (net, probes), (net_o, probes_o) = function_node_network(), function_node_network()
+    with Simulator(net, seed=1, if_python_code="error") as gpu, \
+            OracleSimulator(net_o, seed=1) as cpu:
+        assert not any(isinstance(p, PythonPlan) for p in gpu._plans)
+        assert sum(p.name == "hip_direct_compiled" for p in gpu._plans) == 2
+        assert any(isinstance(p, PythonPlan) for p in cpu._plans)
+        gpu.run_steps(500)
+        cpu.run_steps(500)
+        for a, b in zip(probes, probes_o):
+            np.testing.assert_allclose(gpu.data[a], cpu.data[b], rtol=1e-4, atol=1e-5)
+        assert np.abs(gpu.data[probes[1]]).max() > 0.1
