@@ -14,10 +14,14 @@ plan_slicedcopy        plan_slicedcopy :307-411                       nhip_slice
 plan_elementwise_inc   plan_elementwise_inc :414-574                  nhip_elementwise_inc
 plan_linearfilter      plan_linearfilter :577-803                     nhip_linearfilter
 plan_probes            plan_probes :806-951                           nhip_probes
-plan_direct            plan_direct :954-1025 (unary table only)       nhip_direct_unary
-plan_lif               plan_lif :1028-1146 (non-adaptive)             nhip_lif
-plan_lif_rate          plan_lif_rate :1149-1197 (non-adaptive)        nhip_lif_rate
+plan_direct            plan_direct :954-1025                          nhip_direct_unary, nhip_rtc_*
+plan_lif               plan_lif :1028-1146                            nhip_lif, nhip_alif
+plan_lif_rate          plan_lif_rate :1149-1197                       nhip_lif_rate, nhip_alif_rate
+plan_rectified_linear  :1238-1258 (and spiking :1200-1235, sigmoid)   nhip_relu, ...
+plan_whitenoise        plan_whitenoise :1578-1675 (own generator)     nhip_whitenoise
 plan_presentinput      plan_presentinput :1678-1759                   nhip_presentinput
+plan_conv2d / pool2d   plan_conv2d :1762-1969, plan_pool2d :1972-2079  nhip_conv2d, nhip_pool2d
+plan_bcm / oja / voja  :2082-2169, :2172-2277, :2280-2405             nhip_learning_rule
 =====================  =============================================  ==========
 
 Where the reference's kernels index ``*_starts[n]`` device arrays, these build
