@@ -212,16 +212,22 @@ int nhip_sigmoid(void *stream, const int *desc, int n_blocks, const float *J, fl
  *          y_stride0, y_stride1, shape1, offset, count, na, nb, a_start,
  *          b_start, xbuf_start, ybuf_start, size}
  *   pos  : int32[n_blocks][2]  {xbuf_pos, ybuf_pos}   (read and advanced) */
-int nhip_linearfilter(void *stream, const int *desc, int *pos, int n_blocks, const float *X,
-                      float *Y, const float *A, const float *B, float *Xbuf, float *Ybuf);
+int nhip_linearfilter(void *stream, const int *desc, int *pos, int n_blocks, int lanes,
+                      const float *X, float *Y, const float *A, const float *B, float *Xbuf,
+                      float *Ybuf);
 
-/* ---- element-wise ------------------------------------------------------ */
+/* ---- element-wise ------------------------------------------------------
+ * `lanes` (here and for the synapse filter above, the inputs and the probes below) =
+ * threads that work on one row of the work list: 256 (one group per row, for long
+ * rows) or a power of two from 1 to 64 (a group then takes 256 / lanes rows side by
+ * side, for models with very many very short signals).  The host picks it per launch from the
+ * row lengths; results do not depend on it. */
 /* Y (=|+=) alpha * A * X with scalar/row/column broadcasting, or outer product.
  * replaces: `plan_elementwise_inc` (:414-574).
  *   desc : int32[n_blocks][16] {a_start, a_shape0, a_shape1, a_stride0, x_start,
  *          x_shape0, x_shape1, x_stride0, y_start, y_shape1, y_stride0, offset,
  *          count, alpha_bits, flags(bit0 outer, bit1 inc), 0} */
-int nhip_elementwise_inc(void *stream, const int *desc, int n_blocks, const float *A,
+int nhip_elementwise_inc(void *stream, const int *desc, int n_blocks, int lanes, const float *A,
                          const float *X, float *Y);
 /* Weight-update rules that write a delta matrix per connection (row i = post
  * neuron, column j = pre element; delta rows are contiguous):
@@ -285,15 +291,15 @@ int nhip_philox4x32(void *stream, const unsigned *counters_keys, unsigned *out, 
 /* 2-D strided Y (=|+=) X.  replaces: `plan_copy` (:217-304).
  *   desc : int32[n_blocks][8] {x_start, y_start, shape1, x_stride0, y_stride0,
  *                              offset, count, inc} */
-int nhip_copy(void *stream, const int *desc, int n_blocks, const float *X, float *Y);
+int nhip_copy(void *stream, const int *desc, int n_blocks, int lanes, const float *X, float *Y);
 /* gather/scatter  Y[yi[k]*ys] (=|+=) X[xi[k]*xs].  replaces: `plan_slicedcopy` (:307-411).
  *   desc : int32[n_blocks][8] {x_start, x_stride0, y_start, y_stride0, xi_start,
  *                              yi_start, count, inc} */
-int nhip_slicedcopy(void *stream, const int *desc, int n_blocks, const float *X, float *Y,
-                    const int *XI, const int *YI);
+int nhip_slicedcopy(void *stream, const int *desc, int n_blocks, int lanes, const float *X,
+                    float *Y, const int *XI, const int *YI);
 /* constant fill.  replaces: `plan_reset` (:147-214).
  *   blocks : int32[n_blocks][4] {start, count, value_bits, 0} */
-int nhip_reset(void *stream, const int *blocks, int n_blocks, float *Y);
+int nhip_reset(void *stream, const int *blocks, int n_blocks, int lanes, float *Y);
 /* step += 1; time = dt * step (dt in double, rounded once).
  * replaces: `plan_timeupdate` (:113-144). */
 int nhip_timeupdate(void *stream, float *step_data, int step_start, float *time_data,
@@ -302,20 +308,21 @@ int nhip_timeupdate(void *stream, float *step_data, int step_start, float *time_
 /* ---- inputs and outputs ------------------------------------------------ */
 /* table playback  y = S[row(step) , :].  replaces: `plan_presentinput` (:1678-1759).
  *   desc : int32[n][8] {y_start, m, t_start, s_start, nt, pt_bits, has_pt, 0} */
-int nhip_presentinput(void *stream, const int *desc, int n, float dt, float *Y, const float *T,
-                      const float *S);
+int nhip_presentinput(void *stream, const int *desc, int n, int lanes, float dt, float *Y,
+                      const float *T, const float *S);
 /* y[k] = f(x[k]) for a fixed table of unary functions (opcode: 0 identity, 1 sin,
  * 2 cos, 3 tanh, 4 exp, 5 square).  replaces the generated `direct` kernel of
  * `plan_direct` (:954-1025) for the expressions the function translator
  * reduces to one of these.
  *   desc : int32[n][4] {x_start, y_start, count, 0} */
-int nhip_direct_unary(void *stream, int opcode, const int *desc, int n, const float *X, float *Y);
+int nhip_direct_unary(void *stream, int opcode, const int *desc, int n, int lanes, const float *X,
+                      float *Y);
 /* probe gather with per-probe float countdown.  replaces: `plan_probes` (:806-951).
  *   desc : int32[n][8] {x_start, shape0, shape1, stride0, stride1, y_start, capacity, 0}
  * `capacity` = rows of Y[i]; a sample that would land beyond it is dropped (the
  * position still advances), so an undrained buffer can never be overrun. */
-int nhip_probes(void *stream, const int *desc, int n, float *countdowns, int *bufpositions,
-                const float *periods, const float *X, float *Y);
+int nhip_probes(void *stream, const int *desc, int n, int lanes, float *countdowns,
+                int *bufpositions, const float *periods, const float *X, float *Y);
 /* fill an int32 device array (used to zero probe buffer positions without a
  * memset node, so that it may also be recorded into a graph) */
 int nhip_fill_i32(void *stream, int *dst, int n, int value);
@@ -347,13 +354,15 @@ typedef struct NhipSeqOp {
     int kind;                /* NHIP_SEQ_* */
     int n_blocks;            /* rows of the operation's work list (1 for TIMEUPDATE) */
     int i0;                  /* DIRECT_UNARY: opcode */
-    int reserved;
+    int lanes;               /* threads per work-list row, as for the matching entry point */
     double d0;               /* TIMEUPDATE, PRESENTINPUT: dt */
     unsigned long long p[8]; /* device pointers, see above */
 } NhipSeqOp;                 /* 88 bytes */
-/* at most 16 operations with at most 32 work-list rows in all; n_rows = the sum of
- * n_blocks over `ops` (the library cannot read the device table to check it) */
-int nhip_sequence(void *stream, const void *ops, int n_ops, int n_rows);
+/* at most 16 operations; `lanes` of every record as for the matching entry point
+ * (256 for TIMEUPDATE).  n_staged = the sum of n_blocks over the operations with
+ * lanes == 256, at most 128: their rows are staged in LDS (the library cannot read
+ * the device table to check it). */
+int nhip_sequence(void *stream, const void *ops, int n_ops, int n_staged);
 
 /* ---- function nodes compiled at run time ----------------------------------
  * replaces: `plan_direct` (:954-1025), which builds an OpenCL program from the

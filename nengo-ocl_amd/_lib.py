@@ -40,8 +40,8 @@ SIGNATURES = {
     "nhip_relu": [P, P, c_int, P, P, P],
     "nhip_spiking_relu": [P, P, c_int, c_double, P, P, P, P],
     "nhip_sigmoid": [P, P, c_int, P, P, P],
-    "nhip_linearfilter": [P, P, P, c_int, P, P, P, P, P, P],
-    "nhip_elementwise_inc": [P, P, c_int, P, P, P],
+    "nhip_linearfilter": [P, P, P, c_int, c_int, P, P, P, P, P, P],
+    "nhip_elementwise_inc": [P, P, c_int, c_int, P, P, P],
     "nhip_learning_rule": [P, c_int, P, c_int, P, P, P, P, P, P],
     "nhip_conv2d": [P, P, P, P, P],
     "nhip_pool2d": [P, P, P, P],
@@ -52,13 +52,13 @@ SIGNATURES = {
     "nhip_rtc_load": [P, ctypes.c_char_p, ctypes.POINTER(c_void_p)],
     "nhip_rtc_destroy": [P],
     "nhip_rtc_launch_direct": [P, P, c_int, P, P, P, P, P, P],
-    "nhip_copy": [P, P, c_int, P, P],
-    "nhip_slicedcopy": [P, P, c_int, P, P, P, P],
-    "nhip_reset": [P, P, c_int, P],
+    "nhip_copy": [P, P, c_int, c_int, P, P],
+    "nhip_slicedcopy": [P, P, c_int, c_int, P, P, P, P],
+    "nhip_reset": [P, P, c_int, c_int, P],
     "nhip_timeupdate": [P, P, c_int, P, c_int, c_double],
-    "nhip_presentinput": [P, P, c_int, c_float, P, P, P],
-    "nhip_direct_unary": [P, c_int, P, c_int, P, P],
-    "nhip_probes": [P, P, c_int, P, P, P, P, P],
+    "nhip_presentinput": [P, P, c_int, c_int, c_float, P, P, P],
+    "nhip_direct_unary": [P, c_int, P, c_int, c_int, P, P],
+    "nhip_probes": [P, P, c_int, c_int, P, P, P, P, P],
     "nhip_fill_i32": [P, P, c_int, c_int],
     "nhip_sequence": [P, P, c_int, c_int],
     "nhip_capture_begin": [P],

@@ -3,40 +3,64 @@
 // unary function nodes and probe gather.  All of them are one pass over
 // float32 data described by int32 block work lists: a "block" is a run of at
 // most a few thousand consecutive logical elements of one ragged item, handled
-// by one 256-thread group with a strided loop (consecutive threads touch
-// consecutive elements, so accesses coalesce whenever the item is contiguous).
+// by `lanes` threads with a strided loop (consecutive threads touch consecutive
+// elements, so accesses coalesce whenever the item is contiguous).  `lanes` is
+// 256 (a whole group per block, for long items) or 64, 16, 4, 1 (a group then
+// handles 256 / lanes blocks side by side), chosen per launch by the host from the
+// item sizes: a model with twenty thousand one-element synapses gets one thread,
+// not one group, per synapse.
 #include "nhip_common.h"
 
 namespace {
 
-// Every operation is written as a "block" function: what one 256-thread group does
-// for one row of its work list.  The plain kernels below run one block per group;
-// the sequence kernel at the end of this file runs the blocks of several small
-// operations one after the other inside a single group.
+// Every operation is written as a "block" function: what `L` threads (`lane` = 0..L-1)
+// do for one row of its work list.  The plain kernels below run 256 / L blocks per
+// group; the sequence kernel at the end of this file runs the blocks of several small
+// operations one after the other inside a single group.  Block functions synchronise
+// only when L is the whole group; smaller L divide a wave, whose lanes run in step.
+
+// Runs CALL for this thread's row of a launch with L lanes per row (L a power of two),
+// with `row`, `lane` and `LL` (= L) in scope.  The whole-group case is spelled out so
+// that its loops are compiled with a constant stride.
+#define NHIP_FOR_MY_ROW(L, n_rows, CALL)                                          \
+    if ((L) == NHIP_WG) {                                                          \
+        const int row = blockIdx.x, lane = threadIdx.x;                            \
+        constexpr int LL = NHIP_WG;                                                \
+        CALL;                                                                      \
+    } else {                                                                       \
+        const int lane = threadIdx.x & ((L) - 1);                                  \
+        const int row = blockIdx.x * (NHIP_WG / (L)) + threadIdx.x / (L);          \
+        const int LL = (L);                                                        \
+        if (row < (n_rows)) {                                                      \
+            CALL;                                                                  \
+        }                                                                          \
+    }
 
 // ---------------------------------------------------------------- reset
 // clra_nonlinearities.py:154-172 fills 16-element chunks; here a block is up to
 // 4096 elements of one contiguous item.
-__device__ __forceinline__ void reset_block(const int4 b, float* Y, int tid) {
+__device__ __forceinline__ void reset_block(const int4 b, float* Y, int lane, int L) {
     // b = {start, count, value_bits, 0}
     const float v = nhip_bits(b.z);
     float* y = Y + b.x;
-    for (int i = tid; i < b.y; i += NHIP_WG) y[i] = v;
+    for (int i = lane; i < b.y; i += L) y[i] = v;
 }
 
-__global__ __launch_bounds__(NHIP_WG) void reset_kernel(const int4* __restrict__ blocks, float* Y) {
-    reset_block(blocks[blockIdx.x], Y, threadIdx.x);
+__global__ __launch_bounds__(NHIP_WG) void reset_kernel(const int4* __restrict__ blocks, int n_rows,
+                                                        int L, float* Y) {
+    NHIP_FOR_MY_ROW(L, n_rows, reset_block(blocks[row], Y, lane, LL));
 }
 
 // ---------------------------------------------------------------- copy
 // 2-D strided Y (=|+=) X (clra_nonlinearities.py:225-262).
 struct CopyDesc { int x_start, y_start, shape1, x_stride0, y_stride0, offset, count, inc; };
 
-__device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, float* Y, int tid) {
+__device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, float* Y, int lane,
+                                           int L) {
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const bool flat = (d.x_stride0 == d.shape1) && (d.y_stride0 == d.shape1);
-    for (int k = tid; k < d.count; k += NHIP_WG) {
+    for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
         size_t xo, yo;
         if (flat) {
@@ -52,8 +76,9 @@ __device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, flo
 }
 
 __global__ __launch_bounds__(NHIP_WG) void copy_kernel(const CopyDesc* __restrict__ desc,
-                                                       const float* X, float* Y) {
-    copy_block(desc[blockIdx.x], X, Y, threadIdx.x);
+                                                       int n_rows, int L, const float* X,
+                                                       float* Y) {
+    NHIP_FOR_MY_ROW(L, n_rows, copy_block(desc[row], X, Y, lane, LL));
 }
 
 // ---------------------------------------------------------------- sliced copy
@@ -63,12 +88,12 @@ struct SlicedDesc { int x_start, x_stride0, y_start, y_stride0, xi_start, yi_sta
 
 __device__ __forceinline__ void slicedcopy_block(const SlicedDesc d, const float* X, float* Y,
                                                  const int* __restrict__ XI,
-                                                 const int* __restrict__ YI, int tid) {
+                                                 const int* __restrict__ YI, int lane, int L) {
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const int* xi = XI + d.xi_start;
     const int* yi = YI + d.yi_start;
-    for (int k = tid; k < d.count; k += NHIP_WG) {
+    for (int k = lane; k < d.count; k += L) {
         const float v = x[(size_t)xi[k] * d.x_stride0];
         float* dst = y + (size_t)yi[k] * d.y_stride0;
         if (d.inc) *dst += v;
@@ -77,10 +102,10 @@ __device__ __forceinline__ void slicedcopy_block(const SlicedDesc d, const float
 }
 
 __global__ __launch_bounds__(NHIP_WG) void slicedcopy_kernel(const SlicedDesc* __restrict__ desc,
-                                                             const float* X, float* Y,
-                                                             const int* __restrict__ XI,
+                                                             int n_rows, int L, const float* X,
+                                                             float* Y, const int* __restrict__ XI,
                                                              const int* __restrict__ YI) {
-    slicedcopy_block(desc[blockIdx.x], X, Y, XI, YI, threadIdx.x);
+    NHIP_FOR_MY_ROW(L, n_rows, slicedcopy_block(desc[row], X, Y, XI, YI, lane, LL));
 }
 
 // ---------------------------------------------------------------- elementwise inc
@@ -102,13 +127,13 @@ __device__ __forceinline__ float ew_element(const float* data, int shape0, int s
 }
 
 __device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const float* A,
-                                                      const float* X, float* Y, int tid) {
+                                                      const float* X, float* Y, int lane, int L) {
     const float* a = A + d.a_start;
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const float alpha = nhip_bits(d.alpha_bits);
     const bool outer = d.flags & 1, inc = d.flags & 2;
-    for (int k = tid; k < d.count; k += NHIP_WG) {
+    for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
         const int i = ij / d.y_shape1, j = ij - i * d.y_shape1;
         float aa, xx;
@@ -129,9 +154,10 @@ __device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const floa
 }
 
 __global__ __launch_bounds__(NHIP_WG) void elementwise_inc_kernel(const EwDesc* __restrict__ desc,
+                                                                  int n_rows, int L,
                                                                   const float* A, const float* X,
                                                                   float* Y) {
-    elementwise_inc_block(desc[blockIdx.x], A, X, Y, threadIdx.x);
+    NHIP_FOR_MY_ROW(L, n_rows, elementwise_inc_block(desc[row], A, X, Y, lane, LL));
 }
 
 // ---------------------------------------------------------------- linear filter
@@ -147,7 +173,7 @@ struct LfDesc {
 __device__ __forceinline__ void linearfilter_block(const LfDesc d, int2* pos, const float* X,
                                                    float* Y, const float* __restrict__ A,
                                                    const float* __restrict__ B, float* Xbuf,
-                                                   float* Ybuf, int block, int tid) {
+                                                   float* Ybuf, int block, int lane, int L) {
     const float* a = A + d.a_start;
     const float* b = B + d.b_start;
     const int na = d.na, nb = d.nb;
@@ -158,7 +184,7 @@ __device__ __forceinline__ void linearfilter_block(const LfDesc d, int2* pos, co
         ix = p.x;
         iy = p.y;
     }
-    for (int k = tid; k < d.count; k += NHIP_WG) {
+    for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
         const int i = ij / d.shape1, j = ij - i * d.shape1;
         const size_t xij = (size_t)d.x_start + (size_t)i * d.x_stride0 + (size_t)j * d.x_stride1;
@@ -190,26 +216,28 @@ __device__ __forceinline__ void linearfilter_block(const LfDesc d, int2* pos, co
         }
     }
     if (general) {
-        // every thread has read its position before anyone moves it
-        __syncthreads();
-        if (tid == 0)
+        // every thread has read its position before anyone moves it (lanes of a divided
+        // wave run in step and have all consumed the value by now)
+        if (L == NHIP_WG) __syncthreads();
+        if (lane == 0)
             pos[block] = make_int2((ix > 0) ? ix - 1 : nb - 1, (iy > 0) ? iy - 1 : na - 1);
     }
 }
 
 __global__ __launch_bounds__(NHIP_WG) void linearfilter_kernel(const LfDesc* __restrict__ desc,
-                                                               int2* pos, const float* X, float* Y,
+                                                               int2* pos, int n_rows, int L,
+                                                               const float* X, float* Y,
                                                                const float* __restrict__ A,
                                                                const float* __restrict__ B,
                                                                float* Xbuf, float* Ybuf) {
-    linearfilter_block(desc[blockIdx.x], pos, X, Y, A, B, Xbuf, Ybuf, blockIdx.x, threadIdx.x);
+    NHIP_FOR_MY_ROW(L, n_rows, linearfilter_block(desc[row], pos, X, Y, A, B, Xbuf, Ybuf, row, lane, LL));
 }
 
 // ---------------------------------------------------------------- time update
 // clra_nonlinearities.py:119-133: the step counter is a float32 signal;
 // time = (float)(dt * (double)step) with dt a double literal.
-__device__ __forceinline__ void timeupdate_block(float* step, float* time, double dt, int tid) {
-    if (tid == 0) {
+__device__ __forceinline__ void timeupdate_block(float* step, float* time, double dt, int lane) {
+    if (lane == 0) {
         const float s = step[0] + 1.0f;
         step[0] = s;
         time[0] = (float)(dt * (double)s);
@@ -226,7 +254,7 @@ struct PiDesc { int y_start, m, t_start, s_start, nt, pt_bits, has_pt, pad; };
 
 __device__ __forceinline__ void presentinput_block(const PiDesc d, float dt, float* Y,
                                                    const float* T, const float* __restrict__ S,
-                                                   int tid) {
+                                                   int lane, int L) {
     const int it = (int)T[d.t_start];
     int ti;
     if (d.has_pt) {
@@ -237,20 +265,21 @@ __device__ __forceinline__ void presentinput_block(const PiDesc d, float dt, flo
     }
     float* y = Y + d.y_start;
     const float* s = S + d.s_start + (size_t)d.m * ti;
-    for (int i = tid; i < d.m; i += NHIP_WG) y[i] = s[i];
+    for (int i = lane; i < d.m; i += L) y[i] = s[i];
 }
 
 __global__ __launch_bounds__(NHIP_WG) void presentinput_kernel(const PiDesc* __restrict__ desc,
-                                                               float dt, float* Y, const float* T,
+                                                               int n_rows, int L, float dt, float* Y,
+                                                               const float* T,
                                                                const float* __restrict__ S) {
-    presentinput_block(desc[blockIdx.x], dt, Y, T, S, threadIdx.x);
+    NHIP_FOR_MY_ROW(L, n_rows, presentinput_block(desc[row], dt, Y, T, S, lane, LL));
 }
 
 // ---------------------------------------------------------------- unary function nodes
 __device__ __forceinline__ void direct_unary_block(int opcode, const int4 d, const float* X,
-                                                   float* Y, int tid) {
+                                                   float* Y, int lane, int L) {
     // d = {x_start, y_start, count, 0}
-    for (int i = tid; i < d.z; i += NHIP_WG) {
+    for (int i = lane; i < d.z; i += L) {
         const float x = X[d.x + i];
         float y;
         switch (opcode) {
@@ -267,19 +296,21 @@ __device__ __forceinline__ void direct_unary_block(int opcode, const int4 d, con
 
 __global__ __launch_bounds__(NHIP_WG) void direct_unary_kernel(int opcode,
                                                                const int4* __restrict__ desc,
-                                                               const float* X, float* Y) {
-    direct_unary_block(opcode, desc[blockIdx.x], X, Y, threadIdx.x);
+                                                               int n_rows, int L, const float* X,
+                                                               float* Y) {
+    NHIP_FOR_MY_ROW(L, n_rows, direct_unary_block(opcode, desc[row], X, Y, lane, LL));
 }
 
 // ---------------------------------------------------------------- probes
 // clra_nonlinearities.py:831-902 (plus a capacity guard).  One block per probe; the
 // float32 countdown and the buffer position are read by every thread before the
-// barrier and written by thread 0 after it.
+// barrier (or, in a divided wave, before the lanes reach the update together) and
+// written by lane 0 after it.
 struct ProbeDesc { int x_start, shape0, shape1, stride0, stride1, y_start, capacity, p1; };
 
 __device__ __forceinline__ void probes_block(const ProbeDesc d, float* countdowns,
                                              int* bufpositions, const float* __restrict__ periods,
-                                             const float* X, float* Y, int block, int tid) {
+                                             const float* X, float* Y, int block, int lane, int L) {
     const int n = block;
     const float countdown = countdowns[n];
     const bool fire = countdown <= 0.0f;
@@ -291,13 +322,13 @@ __device__ __forceinline__ void probes_block(const ProbeDesc d, float* countdown
         const int n_dims = d.shape0 * d.shape1;
         const float* x = X + d.x_start;
         float* y = Y + d.y_start + (size_t)bufpos * n_dims;
-        for (int ij = tid; ij < n_dims; ij += NHIP_WG) {
+        for (int ij = lane; ij < n_dims; ij += L) {
             const int i = ij / d.shape1, j = ij - i * d.shape1;
             y[ij] = x[(size_t)i * d.stride0 + (size_t)j * d.stride1];
         }
     }
-    __syncthreads();
-    if (tid == 0) {
+    if (L == NHIP_WG) __syncthreads();
+    if (lane == 0) {
         if (fire) {
             countdowns[n] = countdown + periods[n] - 1.0f;
             bufpositions[n] = bufpos + 1;
@@ -308,10 +339,11 @@ __device__ __forceinline__ void probes_block(const ProbeDesc d, float* countdown
 }
 
 __global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __restrict__ desc,
-                                                         float* countdowns, int* bufpositions,
+                                                         int n_rows, int L, float* countdowns,
+                                                         int* bufpositions,
                                                          const float* __restrict__ periods,
                                                          const float* X, float* Y) {
-    probes_block(desc[blockIdx.x], countdowns, bufpositions, periods, X, Y, blockIdx.x, threadIdx.x);
+    NHIP_FOR_MY_ROW(L, n_rows, probes_block(desc[row], countdowns, bufpositions, periods, X, Y, row, lane, LL));
 }
 
 __global__ __launch_bounds__(NHIP_WG) void fill_i32_kernel(int* dst, int n, int value) {
@@ -326,13 +358,15 @@ __global__ __launch_bounds__(NHIP_WG) void fill_i32_kernel(int* dst, int n, int 
 // the blocks of each operation in turn, a group barrier between operations, so a run
 // of such operations costs one launch.  The operation records and every row of
 // their work lists are fetched into LDS up front, side by side, so that only the
-// data accesses of each operation remain one after the other.  Every block function
+// data accesses of each operation remain one after the other (rows of operations
+// with fewer than 256 lanes per row are handled many at a time and are read where
+// they are).  Every block function
 // is the one the plain kernels use, so results are identical.  Data pointers are
 // never marked restrict or read-only: an operation may read what the one before it
 // wrote, and the barrier (which orders global memory at work-group scope) makes
 // that visible.
 constexpr int SEQ_MAX_OPS = 16;
-constexpr int SEQ_MAX_ROWS = 32;
+constexpr int SEQ_MAX_ROWS = 128;
 constexpr int SEQ_ROW_WORDS = 16;  // the widest work-list row: 64 bytes
 
 __device__ __forceinline__ int seq_row_words(int kind) {
@@ -347,7 +381,7 @@ __device__ __forceinline__ int seq_row_words(int kind) {
 }
 
 __global__ __launch_bounds__(NHIP_WG) void sequence_kernel(const NhipSeqOp* __restrict__ ops,
-                                                           int n_ops) {
+                                                           int n_ops, int n_staged) {
     __shared__ NhipSeqOp s_ops[SEQ_MAX_OPS];
     __shared__ __attribute__((aligned(16))) int s_rows[SEQ_MAX_ROWS][SEQ_ROW_WORDS];
     const int tid = threadIdx.x;
@@ -358,68 +392,82 @@ __global__ __launch_bounds__(NHIP_WG) void sequence_kernel(const NhipSeqOp* __re
         for (int w = tid; w < n_words; w += NHIP_WG) dst[w] = src[w];
     }
     __syncthreads();
-    {   // work-list rows: 16 threads per row, one word each
-        const int row = tid >> 4, word = tid & 15;
-        for (int r0 = 0; r0 < SEQ_MAX_ROWS; r0 += NHIP_WG / 16) {
-            int r = r0 + row, k = 0;
-            while (k < n_ops && r >= s_ops[k].n_blocks) r -= s_ops[k++].n_blocks;
+    {   // work-list rows of the operations with a whole group per row: 16 threads per
+        // row, one word each
+        const int sub = tid >> 4, word = tid & 15;
+        for (int r0 = 0; r0 < n_staged; r0 += NHIP_WG / 16) {
+            int r = r0 + sub, k = 0;
+            while (k < n_ops && (s_ops[k].lanes != NHIP_WG || r >= s_ops[k].n_blocks)) {
+                if (s_ops[k].lanes == NHIP_WG) r -= s_ops[k].n_blocks;
+                ++k;
+            }
             if (k < n_ops) {
                 const int words = seq_row_words(s_ops[k].kind);
                 if (word < words)
-                    s_rows[r0 + row][word] =
+                    s_rows[r0 + sub][word] =
                         reinterpret_cast<const int*>(s_ops[k].p[0])[r * words + word];
             }
         }
     }
     __syncthreads();
-    int row = 0;
+    int first_row = 0;
     for (int k = 0; k < n_ops; ++k) {
         const NhipSeqOp& op = s_ops[k];
+        const int L = op.lanes;                 // lanes per row: 256 or a power of two <= 64
+        const int lane = tid & (L - 1);
+        const int per_pass = NHIP_WG / L;       // rows handled side by side
 #define SEQ_P(i, T) reinterpret_cast<T>(op.p[i])
-#define SEQ_ROW(T) (*reinterpret_cast<const T*>(s_rows[row]))
-        for (int b = 0; b < op.n_blocks; ++b, ++row) {
-            switch (op.kind) {
-                case NHIP_SEQ_RESET:
-                    reset_block(SEQ_ROW(int4), SEQ_P(1, float*), tid);
-                    break;
-                case NHIP_SEQ_COPY:
-                    copy_block(SEQ_ROW(CopyDesc), SEQ_P(1, const float*), SEQ_P(2, float*), tid);
-                    break;
-                case NHIP_SEQ_SLICEDCOPY:
-                    slicedcopy_block(SEQ_ROW(SlicedDesc), SEQ_P(1, const float*), SEQ_P(2, float*),
-                                     SEQ_P(3, const int*), SEQ_P(4, const int*), tid);
-                    break;
-                case NHIP_SEQ_ELEMENTWISE_INC:
-                    elementwise_inc_block(SEQ_ROW(EwDesc), SEQ_P(1, const float*),
-                                          SEQ_P(2, const float*), SEQ_P(3, float*), tid);
-                    break;
-                case NHIP_SEQ_LINEARFILTER:
-                    linearfilter_block(SEQ_ROW(LfDesc), SEQ_P(1, int2*), SEQ_P(2, const float*),
-                                       SEQ_P(3, float*), SEQ_P(4, const float*),
-                                       SEQ_P(5, const float*), SEQ_P(6, float*), SEQ_P(7, float*),
-                                       b, tid);
-                    break;
-                case NHIP_SEQ_TIMEUPDATE:
-                    timeupdate_block(SEQ_P(0, float*), SEQ_P(1, float*), op.d0, tid);
-                    break;
-                case NHIP_SEQ_PRESENTINPUT:
-                    presentinput_block(SEQ_ROW(PiDesc), (float)op.d0, SEQ_P(1, float*),
-                                       SEQ_P(2, const float*), SEQ_P(3, const float*), tid);
-                    break;
-                case NHIP_SEQ_DIRECT_UNARY:
-                    direct_unary_block(op.i0, SEQ_ROW(int4), SEQ_P(1, const float*),
-                                       SEQ_P(2, float*), tid);
-                    break;
-                case NHIP_SEQ_PROBES:
-                    probes_block(SEQ_ROW(ProbeDesc), SEQ_P(1, float*), SEQ_P(2, int*),
-                                 SEQ_P(3, const float*), SEQ_P(4, const float*), SEQ_P(5, float*),
-                                 b, tid);
-                    break;
-                default:
-                    break;
+#define SEQ_ROW(T) \
+    (L == NHIP_WG ? *reinterpret_cast<const T*>(s_rows[first_row + b]) : SEQ_P(0, const T*)[b])
+        for (int b0 = 0; b0 < op.n_blocks; b0 += per_pass) {
+            const int b = b0 + tid / L;
+            if (b < op.n_blocks) {  // uniform over the group when L is the whole group
+                switch (op.kind) {
+                    case NHIP_SEQ_RESET:
+                        reset_block(SEQ_ROW(int4), SEQ_P(1, float*), lane, L);
+                        break;
+                    case NHIP_SEQ_COPY:
+                        copy_block(SEQ_ROW(CopyDesc), SEQ_P(1, const float*), SEQ_P(2, float*),
+                                   lane, L);
+                        break;
+                    case NHIP_SEQ_SLICEDCOPY:
+                        slicedcopy_block(SEQ_ROW(SlicedDesc), SEQ_P(1, const float*),
+                                         SEQ_P(2, float*), SEQ_P(3, const int*),
+                                         SEQ_P(4, const int*), lane, L);
+                        break;
+                    case NHIP_SEQ_ELEMENTWISE_INC:
+                        elementwise_inc_block(SEQ_ROW(EwDesc), SEQ_P(1, const float*),
+                                              SEQ_P(2, const float*), SEQ_P(3, float*), lane, L);
+                        break;
+                    case NHIP_SEQ_LINEARFILTER:
+                        linearfilter_block(SEQ_ROW(LfDesc), SEQ_P(1, int2*), SEQ_P(2, const float*),
+                                           SEQ_P(3, float*), SEQ_P(4, const float*),
+                                           SEQ_P(5, const float*), SEQ_P(6, float*),
+                                           SEQ_P(7, float*), b, lane, L);
+                        break;
+                    case NHIP_SEQ_TIMEUPDATE:
+                        timeupdate_block(SEQ_P(0, float*), SEQ_P(1, float*), op.d0, tid);
+                        break;
+                    case NHIP_SEQ_PRESENTINPUT:
+                        presentinput_block(SEQ_ROW(PiDesc), (float)op.d0, SEQ_P(1, float*),
+                                           SEQ_P(2, const float*), SEQ_P(3, const float*), lane, L);
+                        break;
+                    case NHIP_SEQ_DIRECT_UNARY:
+                        direct_unary_block(op.i0, SEQ_ROW(int4), SEQ_P(1, const float*),
+                                           SEQ_P(2, float*), lane, L);
+                        break;
+                    case NHIP_SEQ_PROBES:
+                        probes_block(SEQ_ROW(ProbeDesc), SEQ_P(1, float*), SEQ_P(2, int*),
+                                     SEQ_P(3, const float*), SEQ_P(4, const float*),
+                                     SEQ_P(5, float*), b, lane, L);
+                        break;
+                    default:
+                        break;
+                }
             }
             __syncthreads();  // blocks of one operation may share state (ring positions)
         }
+        if (L == NHIP_WG) first_row += op.n_blocks;
 #undef SEQ_P
 #undef SEQ_ROW
     }
@@ -429,52 +477,69 @@ __global__ __launch_bounds__(NHIP_WG) void sequence_kernel(const NhipSeqOp* __re
 
 #define NHIP_STREAM(s) static_cast<hipStream_t>(s)
 
-extern "C" int nhip_reset(void* stream, const int* blocks, int n_blocks, float* Y) {
+namespace {
+// lanes per work-list row: the whole group, or a power-of-two share of a wave
+bool lanes_ok(int lanes) {
+    return lanes == NHIP_WG || (lanes >= 1 && lanes <= NHIP_WAVE && (lanes & (lanes - 1)) == 0);
+}
+dim3 row_grid(int n_rows, int lanes) {
+    const int per_group = NHIP_WG / lanes;
+    return dim3((unsigned)((n_rows + per_group - 1) / per_group));
+}
+}  // namespace
+
+extern "C" int nhip_reset(void* stream, const int* blocks, int n_blocks, int lanes, float* Y) {
     if (n_blocks == 0) return 0;
-    if (n_blocks < 0 || !blocks || !Y) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(reset_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const int4*>(blocks), Y);
+    if (n_blocks < 0 || !lanes_ok(lanes) || !blocks || !Y) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(reset_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), reinterpret_cast<const int4*>(blocks), n_blocks, lanes,
+                       Y);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
 
-extern "C" int nhip_copy(void* stream, const int* desc, int n_blocks, const float* X, float* Y) {
+extern "C" int nhip_copy(void* stream, const int* desc, int n_blocks, int lanes, const float* X,
+                         float* Y) {
     if (n_blocks == 0) return 0;
-    if (n_blocks < 0 || !desc || !X || !Y) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(copy_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const CopyDesc*>(desc), X, Y);
+    if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !X || !Y) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(copy_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), reinterpret_cast<const CopyDesc*>(desc), n_blocks,
+                       lanes, X, Y);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
 
-extern "C" int nhip_slicedcopy(void* stream, const int* desc, int n_blocks, const float* X,
-                               float* Y, const int* XI, const int* YI) {
+extern "C" int nhip_slicedcopy(void* stream, const int* desc, int n_blocks, int lanes,
+                               const float* X, float* Y, const int* XI, const int* YI) {
     if (n_blocks == 0) return 0;
-    if (n_blocks < 0 || !desc || !X || !Y || !XI || !YI) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(slicedcopy_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const SlicedDesc*>(desc), X, Y, XI, YI);
+    if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !X || !Y || !XI || !YI) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(slicedcopy_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), reinterpret_cast<const SlicedDesc*>(desc), n_blocks,
+                       lanes, X, Y, XI, YI);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
 
-extern "C" int nhip_elementwise_inc(void* stream, const int* desc, int n_blocks, const float* A,
-                                    const float* X, float* Y) {
+extern "C" int nhip_elementwise_inc(void* stream, const int* desc, int n_blocks, int lanes,
+                                    const float* A, const float* X, float* Y) {
     if (n_blocks == 0) return 0;
-    if (n_blocks < 0 || !desc || !A || !X || !Y) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(elementwise_inc_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
-                       NHIP_STREAM(stream), reinterpret_cast<const EwDesc*>(desc), A, X, Y);
+    if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !A || !X || !Y) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(elementwise_inc_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), reinterpret_cast<const EwDesc*>(desc), n_blocks, lanes,
+                       A, X, Y);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
 
-extern "C" int nhip_linearfilter(void* stream, const int* desc, int* pos, int n_blocks,
+extern "C" int nhip_linearfilter(void* stream, const int* desc, int* pos, int n_blocks, int lanes,
                                  const float* X, float* Y, const float* A, const float* B,
                                  float* Xbuf, float* Ybuf) {
     if (n_blocks == 0) return 0;
-    if (n_blocks < 0 || !desc || !pos || !X || !Y || !B) return NHIP_E_BADARG;  // A, Xbuf, Ybuf may be empty
-    hipLaunchKernelGGL(linearfilter_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const LfDesc*>(desc), reinterpret_cast<int2*>(pos), X, Y, A,
-                       B, Xbuf, Ybuf);
+    // A, Xbuf, Ybuf may be empty
+    if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !pos || !X || !Y || !B) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(linearfilter_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), reinterpret_cast<const LfDesc*>(desc),
+                       reinterpret_cast<int2*>(pos), n_blocks, lanes, X, Y, A, B, Xbuf, Ybuf);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -488,34 +553,37 @@ extern "C" int nhip_timeupdate(void* stream, float* step_data, int step_start, f
     return 0;
 }
 
-extern "C" int nhip_presentinput(void* stream, const int* desc, int n, float dt, float* Y,
-                                 const float* T, const float* S) {
+extern "C" int nhip_presentinput(void* stream, const int* desc, int n, int lanes, float dt,
+                                 float* Y, const float* T, const float* S) {
     if (n == 0) return 0;
-    if (n < 0 || !desc || !Y || !T || !S) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(presentinput_kernel, dim3(n), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const PiDesc*>(desc), dt, Y, T, S);
+    if (n < 0 || !lanes_ok(lanes) || !desc || !Y || !T || !S) return NHIP_E_BADARG;
+    hipLaunchKernelGGL(presentinput_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), reinterpret_cast<const PiDesc*>(desc), n, lanes, dt, Y,
+                       T, S);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
 
-extern "C" int nhip_direct_unary(void* stream, int opcode, const int* desc, int n, const float* X,
-                                 float* Y) {
+extern "C" int nhip_direct_unary(void* stream, int opcode, const int* desc, int n, int lanes,
+                                 const float* X, float* Y) {
     if (n == 0) return 0;
-    if (n < 0 || !desc || !X || !Y || opcode < 0 || opcode > 5) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(direct_unary_kernel, dim3(n), dim3(NHIP_WG), 0, NHIP_STREAM(stream), opcode,
-                       reinterpret_cast<const int4*>(desc), X, Y);
+    if (n < 0 || !lanes_ok(lanes) || !desc || !X || !Y || opcode < 0 || opcode > 5)
+        return NHIP_E_BADARG;
+    hipLaunchKernelGGL(direct_unary_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0,
+                       NHIP_STREAM(stream), opcode, reinterpret_cast<const int4*>(desc), n, lanes,
+                       X, Y);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
 
-extern "C" int nhip_probes(void* stream, const int* desc, int n, float* countdowns,
+extern "C" int nhip_probes(void* stream, const int* desc, int n, int lanes, float* countdowns,
                            int* bufpositions, const float* periods, const float* X, float* Y) {
     if (n == 0) return 0;
-    if (n < 0 || !desc || !countdowns || !bufpositions || !periods || !X || !Y)
+    if (n < 0 || !lanes_ok(lanes) || !desc || !countdowns || !bufpositions || !periods || !X || !Y)
         return NHIP_E_BADARG;
-    hipLaunchKernelGGL(probes_kernel, dim3(n), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const ProbeDesc*>(desc), countdowns, bufpositions, periods,
-                       X, Y);
+    hipLaunchKernelGGL(probes_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const ProbeDesc*>(desc), n, lanes, countdowns,
+                       bufpositions, periods, X, Y);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -529,12 +597,12 @@ extern "C" int nhip_fill_i32(void* stream, int* dst, int n, int value) {
     return 0;
 }
 
-extern "C" int nhip_sequence(void* stream, const void* ops, int n_ops, int n_rows) {
+extern "C" int nhip_sequence(void* stream, const void* ops, int n_ops, int n_staged) {
     if (n_ops == 0) return 0;
-    if (n_ops < 0 || n_ops > SEQ_MAX_OPS || n_rows < n_ops || n_rows > SEQ_MAX_ROWS || !ops)
+    if (n_ops < 0 || n_ops > SEQ_MAX_OPS || n_staged < 0 || n_staged > SEQ_MAX_ROWS || !ops)
         return NHIP_E_BADARG;
     hipLaunchKernelGGL(sequence_kernel, dim3(1), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const NhipSeqOp*>(ops), n_ops);
+                       reinterpret_cast<const NhipSeqOp*>(ops), n_ops, n_staged);
     NHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -61,6 +61,37 @@ def blockify(sizes, max_size=BLOCK):
     return inds.astype(np.int32), offsets.astype(np.int32), counts.astype(np.int32)
 
 
+def lanes_for(size):
+    """Threads that share one work-list row of `size` elements: the next power of two up
+    to a wave (64), beyond that a whole group (256)."""
+    lanes = 1
+    while lanes < size and lanes < 64:
+        lanes *= 2
+    return lanes if size <= lanes else WG
+
+
+def rows_for(sizes, max_size=BLOCK):
+    """`blockify` with the row length fitted to the items: the lanes per row follow the
+    median item size (one element per lane; longer items are cut into several rows), so
+    that models with very many very short signals get a few lanes -- not a 256-thread
+    group -- per signal, and a group works on 256 / lanes rows side by side.  Items
+    longer than a group keep rows of `max_size` elements.
+    Returns ``(item index, offset, count, lanes)``."""
+    sizes = np.asarray(sizes, dtype=np.int64).reshape(-1)
+    used = sizes[sizes > 0]
+    lanes = lanes_for(int(np.median(used))) if used.size else WG
+    return blockify(sizes, max_size if lanes == WG else lanes) + (lanes,)
+
+
+def _row_iterations(counts, lanes):
+    """Elements the busiest lane handles one after the other."""
+    return int(-(-int(np.max(counts)) // lanes)) if len(counts) else 1
+
+
+def _gsize(n_rows, lanes):
+    return (WG * max(-(-n_rows // (WG // lanes)), 1),)
+
+
 def _check(*named):
     """Bounds-check ragged operands on the host before any kernel is bound to them."""
     for name, ra in named:
@@ -116,13 +147,14 @@ def plan_reset(queue, Y, values, tag=None):
     assert Y.ctype == "float"
     _check(("Y", Y))
 
-    inds, offsets, counts = blockify(Y.sizes, 4 * BLOCK)
+    inds, offsets, counts, lanes = rows_for(Y.sizes, 4 * BLOCK)
     table, n = _dev_table(queue, [Y.starts[inds] + offsets, counts, _bits(values[inds])], 4)
-    plan = Plan(queue, queue.lib.nhip_reset, (table.ptr, n, Y.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,), full_args=(table, Y.dev_buf),
+    plan = Plan(queue, queue.lib.nhip_reset, (table.ptr, n, lanes, Y.ptr),
+                gsize=_gsize(n, lanes), lsize=(WG,), full_args=(table, Y.dev_buf),
                 name="hip_reset", tag=tag)
     plan.bw_per_call = Y.nbytes + values.nbytes + table.nbytes
     plan.description = _description(Y)
+    plan.row_iterations = _row_iterations(counts, lanes)
     return plan
 
 
@@ -138,15 +170,16 @@ def plan_copy(queue, X, Y, incs, tag=None):
     assert incs.shape == (len(X),)
     _check(("X", X), ("Y", Y))
 
-    inds, offsets, counts = blockify(Y.sizes)
+    inds, offsets, counts, lanes = rows_for(Y.sizes)
     table, n = _dev_table(queue, [X.starts[inds], Y.starts[inds], X.shape1s[inds],
                                   X.stride0s[inds], Y.stride0s[inds], offsets, counts,
                                   incs[inds]], 8)
-    plan = Plan(queue, queue.lib.nhip_copy, (table.ptr, n, X.ptr, Y.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,),
+    plan = Plan(queue, queue.lib.nhip_copy, (table.ptr, n, lanes, X.ptr, Y.ptr),
+                gsize=_gsize(n, lanes), lsize=(WG,),
                 full_args=(table, X.dev_buf, Y.dev_buf), name="hip_copy", tag=tag)
     plan.bw_per_call = X.nbytes + Y.nbytes
     plan.description = _description(X)
+    plan.row_iterations = _row_iterations(counts, lanes)
     return plan
 
 
@@ -170,17 +203,18 @@ def plan_slicedcopy(queue, X, Y, Xinds, Yinds, incs, tag=None):
             assert 0 <= xi_host[k].min() and xi_host[k].max() < X.shape0s[k], "Xinds[%d] out of range" % k
             assert 0 <= yi_host[k].min() and yi_host[k].max() < Y.shape0s[k], "Yinds[%d] out of range" % k
 
-    inds, offsets, counts = blockify(Xinds.shape0s)
+    inds, offsets, counts, lanes = rows_for(Xinds.shape0s)
     table, n = _dev_table(queue, [X.starts[inds], X.stride0s[inds], Y.starts[inds],
                                   Y.stride0s[inds], Xinds.starts[inds] + offsets,
                                   Yinds.starts[inds] + offsets, counts, incs[inds]], 8)
     plan = Plan(queue, queue.lib.nhip_slicedcopy,
-                (table.ptr, n, X.ptr, Y.ptr, Xinds.ptr, Yinds.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,),
+                (table.ptr, n, lanes, X.ptr, Y.ptr, Xinds.ptr, Yinds.ptr),
+                gsize=_gsize(n, lanes), lsize=(WG,),
                 full_args=(table, X.dev_buf, Y.dev_buf, Xinds.dev_buf, Yinds.dev_buf),
                 name="hip_slicedcopy", tag=tag)
     plan.bw_per_call = 2 * (Xinds.nbytes + int(Xinds.sizes.sum()) * X.dtype.itemsize)
     plan.description = _description(Xinds)
+    plan.row_iterations = _row_iterations(counts, lanes)
     return plan
 
 
@@ -211,20 +245,21 @@ def plan_elementwise_inc(queue, A, X, Y, alpha=None, outer=False, inc=True, tag=
         alphas = np.ones(len(Y), dtype=np.float32)
     _check(("A", A), ("X", X), ("Y", Y))
 
-    inds, offsets, counts = blockify(Y.sizes)
+    inds, offsets, counts, lanes = rows_for(Y.sizes)
     flags = np.full(len(inds), (1 if outer else 0) | (2 if inc else 0), dtype=np.int32)
     table, n = _dev_table(queue, [
         A.starts[inds], A.shape0s[inds], A.shape1s[inds], A.stride0s[inds],
         X.starts[inds], X.shape0s[inds], X.shape1s[inds], X.stride0s[inds],
         Y.starts[inds], Y.shape1s[inds], Y.stride0s[inds], offsets,
         counts, _bits(alphas[inds]), flags], 16)
-    plan = Plan(queue, queue.lib.nhip_elementwise_inc, (table.ptr, n, A.ptr, X.ptr, Y.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,),
+    plan = Plan(queue, queue.lib.nhip_elementwise_inc, (table.ptr, n, lanes, A.ptr, X.ptr, Y.ptr),
+                gsize=_gsize(n, lanes), lsize=(WG,),
                 full_args=(table, A.dev_buf, X.dev_buf, Y.dev_buf),
                 name="hip_elementwise_inc", tag=tag)
     plan.flops_per_call = 2 * int(Y.sizes.sum())
     plan.bw_per_call = A.nbytes + X.nbytes + Y.nbytes + (0 if alpha is None else alphas.nbytes)
     plan.description = _description(Y)
+    plan.row_iterations = _row_iterations(counts, lanes)
     return plan
 
 
@@ -253,7 +288,7 @@ def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
     assert Y.ctype == Ybuf.ctype
     _check(("X", X), ("Y", Y), ("A", A), ("B", B), ("Xbuf", Xbuf), ("Ybuf", Ybuf))
 
-    inds, offsets, counts = blockify(X.sizes)
+    inds, offsets, counts, lanes = rows_for(X.sizes)
     table, n = _dev_table(queue, [
         X.starts[inds], X.stride0s[inds], X.stride1s[inds], Y.starts[inds],
         Y.stride0s[inds], Y.stride1s[inds], X.shape1s[inds], offsets,
@@ -261,13 +296,14 @@ def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
         B.starts[inds], Xbuf.starts[inds], Ybuf.starts[inds], X.sizes[inds]], 16)
     pos = to_device(queue, np.zeros((max(n, 1), 2), dtype=np.int32))
     plan = Plan(queue, queue.lib.nhip_linearfilter,
-                (table.ptr, pos.ptr, n, X.ptr, Y.ptr, A.ptr, B.ptr, Xbuf.ptr, Ybuf.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,),
+                (table.ptr, pos.ptr, n, lanes, X.ptr, Y.ptr, A.ptr, B.ptr, Xbuf.ptr, Ybuf.ptr),
+                gsize=_gsize(n, lanes), lsize=(WG,),
                 full_args=(table, pos, X.dev_buf, Y.dev_buf, A.dev_buf, B.dev_buf,
                            Xbuf.dev_buf, Ybuf.dev_buf),
                 name="hip_linearfilter", tag=tag)
     plan.bw_per_call = (X.nbytes + Y.nbytes + A.nbytes + B.nbytes + Xbuf.nbytes + Ybuf.nbytes)
     plan.description = _description(Y)
+    plan.row_iterations = _row_iterations(counts, lanes)
     plan.bufpos = pos  # zeroed again by Simulator.reset()
     # what a GEMV that produces X needs to run simple filters as its epilogue
     plan.lf_spec = dict(X=X, Y=Y, A=A, B=B, Xbuf=Xbuf, Ybuf=Ybuf)
@@ -293,10 +329,12 @@ def plan_probes(queue, periods, X, Y, tag=None):
     dev_bufpositions = to_device(queue, np.zeros(N, dtype=np.int32))
     table, n = _dev_table(queue, [X.starts, X.shape0s, X.shape1s, X.stride0s, X.stride1s,
                                   Y.starts, Y.shape0s], 8)
+    widest = int((X.shape0s * X.shape1s).max()) if N else 1
+    lanes = lanes_for(widest)  # a probe is one row
     plan = Plan(queue, queue.lib.nhip_probes,
-                (table.ptr, n, dev_countdowns.ptr, dev_bufpositions.ptr, dev_periods.ptr,
+                (table.ptr, n, lanes, dev_countdowns.ptr, dev_bufpositions.ptr, dev_periods.ptr,
                  X.ptr, Y.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,),
+                gsize=_gsize(n, lanes), lsize=(WG,),
                 full_args=(table, dev_countdowns, dev_bufpositions, dev_periods, X.dev_buf,
                            Y.dev_buf), name="hip_probes", tag=tag)
     plan.dev_bufpositions = dev_bufpositions
@@ -304,6 +342,7 @@ def plan_probes(queue, periods, X, Y, tag=None):
     plan.dev_countdowns = dev_countdowns
     plan.periods = periods
     plan.Y = Y
+    plan.row_iterations = -(-widest // lanes)
     plan.bw_per_call = (2 * X.nbytes + dev_periods.nbytes + dev_countdowns.nbytes
                         + dev_bufpositions.nbytes)
     plan.description = _description(X)
@@ -341,8 +380,8 @@ def plan_direct(queue, code, init, input_names, inputs, output, tag=None):
         assert (x.shape0s == 1).all() and (output.shape0s == 1).all()
         table, n = _dev_table(queue, [x.starts, output.starts, np.ones(len(output), np.int32)], 4)
         plan = Plan(queue, queue.lib.nhip_direct_unary,
-                    (UNARY_OPCODES[m.group("fn")], table.ptr, n, x.ptr, output.ptr),
-                    gsize=(WG * max(n, 1),), lsize=(WG,),
+                    (UNARY_OPCODES[m.group("fn")], table.ptr, n, 1, x.ptr, output.ptr),
+                    gsize=_gsize(n, 1), lsize=(WG,),
                     full_args=(table, x.dev_buf, output.dev_buf), name="hip_direct", tag=tag)
         plan.description = _description(output)
         return plan
@@ -663,11 +702,14 @@ def plan_presentinput(queue, Y, t, signals, dt, pres_t=None, tag=None):
         Y.starts, Y.shape0s, t.starts, signals.starts, signals.shape0s,
         np.zeros(N, np.int32) if pres is None else _bits(pres),
         np.full(N, 0 if pres is None else 1, dtype=np.int32)], 8)
+    widest = int(Y.shape0s.max()) if N else 1
+    lanes = lanes_for(widest)  # an input signal is one row
     plan = Plan(queue, queue.lib.nhip_presentinput,
-                (table.ptr, n, float(np.float32(dt)), Y.ptr, t.ptr, signals.ptr),
-                gsize=(WG * max(n, 1),), lsize=(WG,),
+                (table.ptr, n, lanes, float(np.float32(dt)), Y.ptr, t.ptr, signals.ptr),
+                gsize=_gsize(n, lanes), lsize=(WG,),
                 full_args=(table, Y.dev_buf, t.dev_buf, signals.dev_buf),
                 name="hip_presentinput", tag=tag)
+    plan.row_iterations = -(-widest // lanes)
     plan.description = _description(Y)
     return plan
 

@@ -21,15 +21,17 @@ from .plan import Plan
 SEQ_RESET, SEQ_COPY, SEQ_SLICEDCOPY, SEQ_ELEMENTWISE_INC, SEQ_LINEARFILTER = 1, 2, 3, 4, 5
 SEQ_TIMEUPDATE, SEQ_PRESENTINPUT, SEQ_DIRECT_UNARY, SEQ_PROBES = 6, 7, 8, 9
 
-SEQ_OP_DTYPE = np.dtype([("kind", "<i4"), ("n_blocks", "<i4"), ("i0", "<i4"), ("reserved", "<i4"),
+SEQ_OP_DTYPE = np.dtype([("kind", "<i4"), ("n_blocks", "<i4"), ("i0", "<i4"), ("lanes", "<i4"),
                          ("d0", "<f8"), ("p", "<u8", (8,))])
 assert SEQ_OP_DTYPE.itemsize == 88
 
-# one work-group runs the blocks one after the other: only operations this short,
-# and only so many per launch (limits of the kernel's LDS staging)
-MAX_BLOCKS_PER_OP = 4
+# one work-group runs the rows of an operation in passes of 256 / lanes rows, one pass
+# after the other, and a lane its elements one after the other: only operations this
+# short (passes x elements per lane), and only so many operations per launch and rows of
+# whole-group operations (they are staged in LDS)
+MAX_STEPS_PER_OP = 4
 MAX_OPS = 16
-MAX_ROWS = 32
+MAX_STAGED_ROWS = 128
 
 
 def _addr(pointer, byte_offset=0):
@@ -40,45 +42,54 @@ def _addr(pointer, byte_offset=0):
 
 
 def sequence_op(plan):
-    """(kind, n_blocks, i0, d0, pointers) of a device plan, or None if its kernel has
+    """(kind, n_rows, lanes, i0, d0, pointers) of a device plan, or None if its kernel has
     no counterpart in the sequence kernel."""
     name = getattr(getattr(plan, "kern", None), "__name__", None)
     a = getattr(plan, "args", ())
     if name == "nhip_reset":
-        table, n, Y = a
-        return SEQ_RESET, n, 0, 0.0, [table, Y]
+        table, n, lanes, Y = a
+        return SEQ_RESET, n, lanes, 0, 0.0, [table, Y]
     if name == "nhip_copy":
-        desc, n, X, Y = a
-        return SEQ_COPY, n, 0, 0.0, [desc, X, Y]
+        desc, n, lanes, X, Y = a
+        return SEQ_COPY, n, lanes, 0, 0.0, [desc, X, Y]
     if name == "nhip_slicedcopy":
-        desc, n, X, Y, XI, YI = a
-        return SEQ_SLICEDCOPY, n, 0, 0.0, [desc, X, Y, XI, YI]
+        desc, n, lanes, X, Y, XI, YI = a
+        return SEQ_SLICEDCOPY, n, lanes, 0, 0.0, [desc, X, Y, XI, YI]
     if name == "nhip_elementwise_inc":
-        desc, n, A, X, Y = a
-        return SEQ_ELEMENTWISE_INC, n, 0, 0.0, [desc, A, X, Y]
+        desc, n, lanes, A, X, Y = a
+        return SEQ_ELEMENTWISE_INC, n, lanes, 0, 0.0, [desc, A, X, Y]
     if name == "nhip_linearfilter":
-        desc, pos, n, X, Y, A, B, Xbuf, Ybuf = a
-        return SEQ_LINEARFILTER, n, 0, 0.0, [desc, pos, X, Y, A, B, Xbuf, Ybuf]
+        desc, pos, n, lanes, X, Y, A, B, Xbuf, Ybuf = a
+        return SEQ_LINEARFILTER, n, lanes, 0, 0.0, [desc, pos, X, Y, A, B, Xbuf, Ybuf]
     if name == "nhip_timeupdate":
         step, step_start, time, time_start, dt = a
-        return SEQ_TIMEUPDATE, 1, 0, float(dt), [_addr(step, 4 * step_start),
-                                                 _addr(time, 4 * time_start)]
+        return SEQ_TIMEUPDATE, 1, 256, 0, float(dt), [_addr(step, 4 * step_start),
+                                                      _addr(time, 4 * time_start)]
     if name == "nhip_presentinput":
-        desc, n, dt, Y, T, S = a
+        desc, n, lanes, dt, Y, T, S = a
         # the entry point takes dt as a float: round it the same way
-        return SEQ_PRESENTINPUT, n, 0, float(np.float32(dt)), [desc, Y, T, S]
+        return SEQ_PRESENTINPUT, n, lanes, 0, float(np.float32(dt)), [desc, Y, T, S]
     if name == "nhip_direct_unary":
-        opcode, desc, n, X, Y = a
-        return SEQ_DIRECT_UNARY, n, int(opcode), 0.0, [desc, X, Y]
+        opcode, desc, n, lanes, X, Y = a
+        return SEQ_DIRECT_UNARY, n, lanes, int(opcode), 0.0, [desc, X, Y]
     if name == "nhip_probes":
-        desc, n, countdowns, bufpositions, periods, X, Y = a
-        return SEQ_PROBES, n, 0, 0.0, [desc, countdowns, bufpositions, periods, X, Y]
+        desc, n, lanes, countdowns, bufpositions, periods, X, Y = a
+        return SEQ_PROBES, n, lanes, 0, 0.0, [desc, countdowns, bufpositions, periods, X, Y]
     return None
+
+
+def _staged_rows(op):
+    return op[1] if op[2] == 256 else 0
 
 
 def is_small(plan):
     op = sequence_op(plan)
-    return op is not None and 0 < op[1] <= MAX_BLOCKS_PER_OP
+    if op is None:
+        return False
+    n_rows, lanes = op[1], op[2]
+    passes = -(-n_rows // (256 // lanes))
+    return (n_rows > 0 and passes * getattr(plan, "row_iterations", 1) <= MAX_STEPS_PER_OP
+            and _staged_rows(op) <= MAX_STAGED_ROWS)
 
 
 def _conflict(p, q):
@@ -93,14 +104,14 @@ def plan_sequence(queue, plans):
     """One launch that runs `plans` (all small, see `is_small`) in order."""
     table = np.zeros(len(plans), dtype=SEQ_OP_DTYPE)
     for row, plan in zip(table, plans):
-        kind, n, i0, d0, pointers = sequence_op(plan)
-        row["kind"], row["n_blocks"], row["i0"], row["d0"] = kind, n, i0, d0
+        kind, n, lanes, i0, d0, pointers = sequence_op(plan)
+        row["kind"], row["n_blocks"], row["lanes"], row["i0"], row["d0"] = kind, n, lanes, i0, d0
         for k, ptr in enumerate(pointers):
             row["p"][k] = _addr(ptr)
-    n_rows = int(table["n_blocks"].sum())
-    assert len(plans) <= MAX_OPS and n_rows <= MAX_ROWS
+    n_staged = int(table["n_blocks"][table["lanes"] == 256].sum())
+    assert len(plans) <= MAX_OPS and n_staged <= MAX_STAGED_ROWS
     dev_table = to_device(queue, table.view(np.int32))
-    merged = Plan(queue, queue.lib.nhip_sequence, (dev_table.ptr, len(plans), n_rows), gsize=(256,),
+    merged = Plan(queue, queue.lib.nhip_sequence, (dev_table.ptr, len(plans), n_staged), gsize=(256,),
                   lsize=(256,), full_args=(dev_table,) + tuple(plans), name="hip_sequence",
                   tag="+".join(p.name.replace("hip_", "") for p in plans))
     merged.members = list(plans)
@@ -143,8 +154,8 @@ def merge_small_plans(plans):
 
     for plan, s in zip(plans, small):
         if s:
-            rows = sum(sequence_op(p)[1] for p in run) + sequence_op(plan)[1]
-            if len(run) == MAX_OPS or rows > MAX_ROWS:
+            rows = sum(_staged_rows(sequence_op(p)) for p in run + [plan])
+            if len(run) == MAX_OPS or rows > MAX_STAGED_ROWS:
                 close()
             run.append(plan)
         else:

@@ -683,3 +683,80 @@ def test_plan_direct_unary_table_still_precompiled(queue):
     np.testing.assert_allclose(dY.buf, np.sin(np.float32([0.3, 1.2])), rtol=1e-6)
     with pytest.raises(NotImplementedError, match="does not compile"):
         nl().plan_direct(queue, "OUTPUT__[0] = undefined_function(t[0]);", "", ["t"], [dT], dY)
+
+
+# ------------------------------------------------------------------ many short signals
+@pytest.mark.parametrize("size,lanes", [(1, 1), (2, 2), (3, 4), (6, 8), (11, 16), (25, 32),
+                                        (50, 64), (200, 256), (2000, 256)])
+def test_many_short_items_every_lane_width(queue, rng, size, lanes):
+    """Models with very many very short signals: rows are handled by 1, 2, ... 64 lanes
+    each instead of a 256-thread group (the width follows the median item size; longer
+    items are cut into several rows).  Every element-wise operation, the
+    filters (all three forms, several steps, so that ring positions advance), input
+    playback, probes and unary functions against the oracle, bit for bit."""
+    n_items = 700 if size <= 200 else 5
+    sizes = np.maximum(1, rng.randint(size - size // 4, size + size // 4 + 1, size=n_items))
+    sizes[1] = size          # (the median stays `size`)
+    sizes[0] = 9 * size + 1  # one long item among them: cut into several rows
+    vec = lambda: RA([rng.normal(size=n) for n in sizes])
+    plans = []  # (device plan, oracle plan)
+
+    # reset / copy / sliced copy / elementwise
+    Y1 = vec(); dY1 = to_dev(queue, Y1)
+    values = rng.normal(size=n_items).astype(np.float32)
+    plans.append((nl().plan_reset(queue, dY1, values), orc().plan_reset(None, Y1, values)))
+    X2, Y2 = vec(), vec(); dX2, dY2 = to_dev(queue, X2), to_dev(queue, Y2)
+    incs = rng.randint(0, 2, size=n_items).astype(np.int32)
+    plans.append((nl().plan_copy(queue, dX2, dY2, incs), orc().plan_copy(None, X2, Y2, incs)))
+    XI = RA([rng.permutation(n)[: max(1, n // 2)] for n in sizes], dtype=np.int32)
+    YI = RA([rng.permutation(n)[: max(1, n // 2)] for n in sizes], dtype=np.int32)
+    X3, Y3 = vec(), vec(); dX3, dY3 = to_dev(queue, X3), to_dev(queue, Y3)
+    plans.append((nl().plan_slicedcopy(queue, dX3, dY3, to_dev(queue, XI), to_dev(queue, YI), incs),
+                  orc().plan_slicedcopy(None, X3, Y3, XI, YI, incs)))
+    A4 = RA([[rng.normal()] for _ in sizes]); X4, Y4 = vec(), vec()
+    dY4 = to_dev(queue, Y4)
+    plans.append((nl().plan_elementwise_inc(queue, to_dev(queue, A4), to_dev(queue, X4), dY4),
+                  orc().plan_elementwise_inc(None, A4, X4, Y4)))
+
+    # filters: gain, lowpass and second-order items mixed
+    kinds = [("gain", "lowpass", "alpha")[k % 3] for k in range(n_items)]
+    coefs = [_filter_coefficients(k) for k in kinds]
+    A5, B5 = RA([den for _, den in coefs]), RA([num for num, _ in coefs])
+    X5, Y5 = vec(), RA([np.zeros(n) for n in sizes])
+    Xbuf, Ybuf = RA([np.zeros(s) for s in zip(B5.sizes, X5.sizes)]), RA(
+        [np.zeros(s) for s in zip(A5.sizes, Y5.sizes)])
+    dX5, dY5 = to_dev(queue, X5), to_dev(queue, Y5)
+    gf = nl().plan_linearfilter(queue, dX5, dY5, to_dev(queue, A5), to_dev(queue, B5),
+                                to_dev(queue, Xbuf), to_dev(queue, Ybuf))
+    of = orc().plan_linearfilter(None, X5, Y5, A5, B5, Xbuf, Ybuf)
+    plans += list(zip(gf, of[:len(gf)]))
+    extra_oracle = of[len(gf):]  # the oracle's separate position update, if any
+
+    # input playback and probes: rows cannot be cut, the width follows the largest item
+    small = np.minimum(sizes, 300)
+    tables = [rng.normal(size=(7, n)) for n in small]
+    S6, Y6 = RA(tables), RA([np.zeros(n) for n in small])
+    T6 = RA([[3.0]] * n_items)
+    dY6 = to_dev(queue, Y6)
+    plans.append((nl().plan_presentinput(queue, dY6, to_dev(queue, T6), to_dev(queue, S6), 1e-3),
+                  orc().plan_presentinput(None, Y6, T6, S6, 1e-3)))
+    n_buf = 6
+    P7 = RA([np.zeros((n_buf, n)) for n in sizes]); dP7 = to_dev(queue, P7)
+    periods = rng.choice([1.0, 2.0, 2.5], size=n_items)
+    gp, op = nl().plan_probes(queue, periods, dX5, dP7), orc().plan_probes(None, periods, X5, P7)
+    plans.append((gp, op))
+
+    widths = {p.name: p.args[{"hip_linearfilter": 3}.get(p.name, 2)] for p, _ in plans}
+    assert widths["hip_reset"] == widths["hip_copy"] == widths["hip_linearfilter"] == lanes, widths
+    for step in range(4):
+        x_new = rng.normal(size=X5.buf.size).astype(np.float32)
+        X5.buf[:] = x_new
+        dX5.dev_buf.set(x_new)
+        for g, o in plans:
+            g()
+            o()
+        for o in extra_oracle:
+            o()
+        for dev, host in ((dY1, Y1), (dY2, Y2), (dY3, Y3), (dY4, Y4), (dY5, Y5), (dY6, Y6), (dP7, P7)):
+            assert np.array_equal(dev.buf, host.buf), "step %d" % step
+    assert np.array_equal(gp.dev_bufpositions.get(), op.bufpositions)

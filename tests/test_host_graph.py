@@ -285,7 +285,7 @@ def test_small_plans_sink_and_merge(monkeypatch):
     class P:
         def __init__(self, label, kern, n_blocks, reads, writes):
             self.label, self.kern, self.name = label, K(kern), kern
-            self.args = (None, n_blocks, None, None) if kern == "nhip_copy" else ()
+            self.args = (None, n_blocks, 256, None, None) if kern == "nhip_copy" else ()
             self.reads_mem, self.writes_mem = set(reads), set(writes)
             self.queue = None
 
@@ -313,6 +313,15 @@ def test_small_plans_sink_and_merge(monkeypatch):
              P("wide", "nhip_copy", 5, "", "u"), small("c", "", "v")]
     labels = [p.label for p in hs.merge_small_plans(plans)]
     assert labels == ["a", "host", "g", "wide", "b+c"]
+    # 1000 rows at one lane per row are four passes of a group: small; 100 rows at 64
+    # lanes per row are 25 passes: not small; one pass in which a lane handles eight
+    # elements one after the other: not small; more whole-group rows than are staged: not
+    narrow, wider, deep, many = (P(k, "nhip_copy", 100, "", k) for k in "nwdm")
+    narrow.args, wider.args = (None, 1000, 1, None, None), (None, 100, 64, None, None)
+    deep.args, deep.row_iterations = (None, 1, 256, None, None), 8
+    many.args = (None, 200, 256, None, None)
+    assert hs.is_small(narrow)
+    assert not hs.is_small(wider) and not hs.is_small(deep) and not hs.is_small(many)
 
 
 def test_neurons_without_input_read_their_bias():
