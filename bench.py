@@ -151,6 +151,8 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
     ap.add_argument("--no-fuse", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--learn-in-place", action="store_true",
+                    help="learning rules add their change to the weights in one pass (c4)")
     ap.add_argument("--branches", action="store_true",
                     help="record kernels that touch different memory as side-by-side graph "
                          "branches instead of one chain")
@@ -171,7 +173,7 @@ def main():
     t0 = time.time()
     (net, probes, _), workload = make_network(args.config, args.variant, args.scale)
     sim = Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph,
-                    branches=args.branches)
+                    branches=args.branches, learn_in_place=args.learn_in_place)
     build_s = time.time() - t0
     n_plans = len(sim._plans)
 
@@ -215,7 +217,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": workload, "neurons": net.n_neurons, "plans_per_step": n_plans,
                    "dt": 0.001, "graph": not args.no_graph, "graph_branches": args.branches,
-                   "fused_copies": not args.no_fuse},
+                   "fused_copies": not args.no_fuse, "learn_in_place": args.learn_in_place},
         "roofline": roofline,
         "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,
                      "gbs": 1e-3 * gemv_bytes / gemv_us if gemv_us else None,

@@ -237,16 +237,19 @@ int nhip_elementwise_inc(void *stream, const int *desc, int n_blocks, int lanes,
  * each product and difference rounded separately, left to right.
  * replaces: `plan_bcm` (:2082-2169), `plan_oja` (:2172-2277), `plan_voja`
  * (:2280-2405).  AUX is theta (vector), weights or encoders (matrix, rows
- * contiguous); LEARN and SCALE are read by VOJA only.
+ * contiguous); LEARN and SCALE are read by VOJA only.  With `inc` the change is added
+ * to DELTA instead of stored (DELTA may then be the weight / encoder matrix itself,
+ * also when it is AUX: the learning step and the `Copy(delta -> weights, inc)` that
+ * follows it in the reference's graph in one pass).
  *   desc : int32[n_blocks][16] {pre_start, pre_stride0, post_start, post_stride0,
  *          aux_start, aux_stride0, delta_start, delta_stride0, shape1, offset,
  *          count, alpha_bits, beta_bits, learn_start, scale_start, scale_stride0} */
 #define NHIP_RULE_BCM 1
 #define NHIP_RULE_OJA 2
 #define NHIP_RULE_VOJA 3
-int nhip_learning_rule(void *stream, int rule, const int *desc, int n_blocks, const float *PRE,
-                       const float *POST, const float *AUX, float *DELTA, const float *LEARN,
-                       const float *SCALE);
+int nhip_learning_rule(void *stream, int rule, int inc, const int *desc, int n_blocks,
+                       const float *PRE, const float *POST, const float *AUX, float *DELTA,
+                       const float *LEARN, const float *SCALE);
 /* ---- convolution, pooling -------------------------------------------------
  * Y = conv2d(X, F) over one image signal (Y is set, not incremented, like the
  * reference's kernel), or local filtering (one filter bank per output pixel).

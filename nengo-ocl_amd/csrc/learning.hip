@@ -22,9 +22,9 @@ struct LearnDesc {
 // :2349-2350 (Voja), left to right.
 template <int RULE>
 __global__ __launch_bounds__(NHIP_WG) void learning_kernel(const LearnDesc* __restrict__ desc,
-                                                           const float* PRE, const float* POST,
-                                                           const float* AUX, float* DELTA,
-                                                           const float* LEARN,
+                                                           int inc, const float* PRE,
+                                                           const float* POST, const float* AUX,
+                                                           float* DELTA, const float* LEARN,
                                                            const float* SCALE) {
     const LearnDesc d = desc[blockIdx.x];
     const float alpha = nhip_bits(d.alpha_bits);
@@ -53,13 +53,17 @@ __global__ __launch_bounds__(NHIP_WG) void learning_kernel(const LearnDesc* __re
             out = __fmul_rn(__fmul_rn(__fmul_rn(alpha, learn), y),
                             __fsub_rn(__fmul_rn(scale, x), enc));
         }
-        delta[(size_t)i * d.delta_stride0 + j] = out;
+        // inc: the change is added to the matrix DELTA points at (which may be the
+        // weights or encoders AUX was just read from: each element is read, then written,
+        // by this thread only)
+        float* dst = delta + (size_t)i * d.delta_stride0 + j;
+        *dst = inc ? __fadd_rn(*dst, out) : out;
     }
 }
 
 }  // namespace
 
-extern "C" int nhip_learning_rule(void* stream, int rule, const int* desc, int n_blocks,
+extern "C" int nhip_learning_rule(void* stream, int rule, int inc, const int* desc, int n_blocks,
                                   const float* PRE, const float* POST, const float* AUX,
                                   float* DELTA, const float* LEARN, const float* SCALE) {
     if (n_blocks == 0) return 0;
@@ -69,16 +73,16 @@ extern "C" int nhip_learning_rule(void* stream, int rule, const int* desc, int n
     switch (rule) {
     case NHIP_RULE_BCM:
         hipLaunchKernelGGL(learning_kernel<NHIP_RULE_BCM>, grid, block, 0, NHIP_STREAM(stream), d,
-                           PRE, POST, AUX, DELTA, LEARN, SCALE);
+                           inc, PRE, POST, AUX, DELTA, LEARN, SCALE);
         break;
     case NHIP_RULE_OJA:
         hipLaunchKernelGGL(learning_kernel<NHIP_RULE_OJA>, grid, block, 0, NHIP_STREAM(stream), d,
-                           PRE, POST, AUX, DELTA, LEARN, SCALE);
+                           inc, PRE, POST, AUX, DELTA, LEARN, SCALE);
         break;
     case NHIP_RULE_VOJA:
         if (!LEARN || !SCALE) return NHIP_E_BADARG;
         hipLaunchKernelGGL(learning_kernel<NHIP_RULE_VOJA>, grid, block, 0, NHIP_STREAM(stream),
-                           d, PRE, POST, AUX, DELTA, LEARN, SCALE);
+                           d, inc, PRE, POST, AUX, DELTA, LEARN, SCALE);
         break;
     default:
         return NHIP_E_BADARG;

@@ -719,7 +719,7 @@ RULE_BCM, RULE_OJA, RULE_VOJA = 1, 2, 3
 
 
 def _plan_rule(queue, rule, name, pre, post, aux, delta, alpha, beta=None, learn=None,
-               scale=None, flops_per_element=4, tag=None):
+               scale=None, inc=False, flops_per_element=4, tag=None):
     N = len(pre)
     alpha = _host(alpha).astype(np.float32).reshape(-1)
     beta = np.zeros(N, dtype=np.float32) if beta is None else _host(beta).astype(
@@ -740,7 +740,7 @@ def _plan_rule(queue, rule, name, pre, post, aux, delta, alpha, beta=None, learn
         learn.starts[inds] if learn is not None else zeros,
         scale.starts[inds] if scale is not None else zeros,
         scale.stride0s[inds] if scale is not None else zeros], 16)
-    args = (rule, table.ptr, n, pre.ptr, post.ptr, aux.ptr, delta.ptr,
+    args = (rule, int(bool(inc)), table.ptr, n, pre.ptr, post.ptr, aux.ptr, delta.ptr,
             learn.ptr if learn is not None else None, scale.ptr if scale is not None else None)
     keep = [table, pre.dev_buf, post.dev_buf, aux.dev_buf, delta.dev_buf]
     keep += [ra.dev_buf for ra in (learn, scale) if ra is not None]
@@ -748,14 +748,16 @@ def _plan_rule(queue, rule, name, pre, post, aux, delta, alpha, beta=None, learn
                 full_args=tuple(keep), name=name, tag=tag)
     plan.flops_per_call = flops_per_element * int(delta.sizes.sum())
     plan.bw_per_call = (sum(ra.nbytes for _, ra in operands) + alpha.nbytes
-                        + (beta.nbytes if rule == RULE_OJA else 0))
+                        + (beta.nbytes if rule == RULE_OJA else 0) + (delta.nbytes if inc else 0))
     plan.description = _description(delta)
     return plan
 
 
-def plan_bcm(queue, pre, post, theta, delta, alpha, tag=None):
+def plan_bcm(queue, pre, post, theta, delta, alpha, inc=False, tag=None):
     """``delta = alpha * post * (post - theta) (outer) pre`` per connection
-    (reference ``plan_bcm`` :2082-2169)."""
+    (reference ``plan_bcm`` :2082-2169).  ``inc`` (here and for the two rules below, not
+    in the reference): add the change to ``delta`` -- which may then be the learned
+    matrix itself -- instead of storing it."""
     assert len(pre) == len(post) == len(theta) == len(delta) == np.size(_host(alpha))
     for arr in (pre, post, theta):  # vectors
         assert (arr.shape1s == 1).all()
@@ -764,11 +766,11 @@ def plan_bcm(queue, pre, post, theta, delta, alpha, tag=None):
     assert (pre.shape0s == delta.shape1s).all()
     assert (post.shape0s == theta.shape0s).all()
     assert pre.ctype == post.ctype == theta.ctype == delta.ctype == "float"
-    return _plan_rule(queue, RULE_BCM, "hip_bcm", pre, post, theta, delta, alpha,
+    return _plan_rule(queue, RULE_BCM, "hip_bcm", pre, post, theta, delta, alpha, inc=inc,
                       flops_per_element=4, tag=tag)
 
 
-def plan_oja(queue, pre, post, weights, delta, alpha, beta, tag=None):
+def plan_oja(queue, pre, post, weights, delta, alpha, beta, inc=False, tag=None):
     """``delta = alpha * post * (pre - beta * weights * post)`` per connection
     (reference ``plan_oja`` :2172-2277)."""
     assert (len(pre) == len(post) == len(weights) == len(delta) == np.size(_host(alpha))
@@ -783,10 +785,10 @@ def plan_oja(queue, pre, post, weights, delta, alpha, beta, tag=None):
     assert (weights.shape1s == delta.shape1s).all()
     assert pre.ctype == post.ctype == weights.ctype == delta.ctype == "float"
     return _plan_rule(queue, RULE_OJA, "hip_oja", pre, post, weights, delta, alpha, beta=beta,
-                      flops_per_element=6, tag=tag)
+                      inc=inc, flops_per_element=6, tag=tag)
 
 
-def plan_voja(queue, pre, post, enc, delta, learn, scale, alpha, tag=None):
+def plan_voja(queue, pre, post, enc, delta, learn, scale, alpha, inc=False, tag=None):
     """``delta = alpha * learn * post * (scale * pre - enc)`` per connection
     (reference ``plan_voja`` :2280-2405)."""
     assert (len(pre) == len(post) == len(enc) == len(delta) == len(learn)
@@ -804,7 +806,7 @@ def plan_voja(queue, pre, post, enc, delta, learn, scale, alpha, tag=None):
     assert (pre.ctype == post.ctype == enc.ctype == delta.ctype == learn.ctype
             == scale.ctype == "float")
     return _plan_rule(queue, RULE_VOJA, "hip_voja", pre, post, enc, delta, alpha, learn=learn,
-                      scale=scale, flops_per_element=5, tag=tag)
+                      scale=scale, inc=inc, flops_per_element=5, tag=tag)
 
 
 # ---------------------------------------------------------------- convolution, pooling

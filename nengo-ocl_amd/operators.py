@@ -362,6 +362,64 @@ def neurons_read_constant_input(operators, keep=()):
     return [replace.get(op, op) for op in operators if op not in drop]
 
 
+LEARNING_RULES = ("SimPES", "SimBCM", "SimOja", "SimVoja")
+
+
+def apply_learning_in_place(operators, keep=()):
+    """Learning rules whose delta matrix only exists to be added to the learned matrix
+    add their change to that matrix directly.
+
+    The builder emits ``rule(... -> delta)`` (an update: its result is first seen in the
+    next step) and ``Copy(delta -> target, inc=True)``.  The copy of step n+1 adds what
+    the rule computed at the end of step n, and nothing can see the target in between,
+    so adding the change at the end of step n gives every reader the same values -- in
+    one pass over the matrix instead of a pass that writes the delta and another that
+    reads delta and target and writes the target.  Rewritten when the copy is the only
+    writer of the target and the only reader of the delta, both are whole signals (no
+    views, no slices), and neither is in `keep` (probed signals; a probe samples at the
+    very end of a step and would see the change one step early): the rule gets
+    ``delta = target`` and ``apply_inc = True``, the copy goes away.  Sums are formed as
+    before (change rounded, then added), so everything computed inside the simulation
+    is bit-identical.  What differs: the delta signal is no longer written, and a host
+    read of the target *between* steps already includes the change of the step just
+    finished.
+    """
+    import copy as _copy
+
+    writers, readers = {}, {}
+    for op in operators:
+        for sig in list(op.sets) + list(op.incs) + list(op.updates):
+            writers.setdefault(sig.base, []).append(op)
+        for sig in list(op.reads) + list(op.incs):
+            readers.setdefault(sig.base, []).append(op)
+    keep_bases = {sig.base for sig in keep}
+    whole = lambda sig: not getattr(sig, "is_view", False)
+    drop, replace = set(), {}
+    for op in operators:
+        if type(op).__name__ not in LEARNING_RULES or getattr(op, "apply_inc", False):
+            continue
+        delta = op.delta
+        if not whole(delta) or delta.base in keep_bases or writers.get(delta.base) != [op]:
+            continue
+        users = readers.get(delta.base, [])
+        if len(users) != 1:
+            continue
+        cp = users[0]
+        if not (_is(cp, "Copy") and cp.inc and cp.src is delta and cp.src_slice is None
+                and cp.dst_slice is None and whole(cp.dst) and cp.dst.shape == delta.shape
+                and cp.dst.base not in keep_bases and writers.get(cp.dst.base) == [cp]):
+            continue
+        new = _copy.copy(op)
+        new.delta, new.apply_inc = cp.dst, True
+        new.updates = [cp.dst]
+        new.reads = list(op.reads)
+        replace[op] = new
+        drop.add(cp)
+    if not replace:
+        return operators
+    return [replace.get(op, op) for op in operators if op not in drop]
+
+
 def simplify_operators(operators):
     """Apply every function in ``simplifications`` in turn."""
     for simplification in simplifications:

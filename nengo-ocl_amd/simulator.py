@@ -210,13 +210,18 @@ class Simulator:
     different memory run side by side instead of one chain of kernels (slower on
     current drivers, off by default); ``merge_small=False`` keeps every short
     operation (clock, inputs, small copies and filters, probes) as a launch of its
-    own instead of binding runs of them into one launch.
+    own instead of binding runs of them into one launch; ``learn_in_place=True`` (with
+    ``fuse``) lets learning rules add their change to the learned matrix directly instead
+    of writing a delta matrix that a copy adds in the next step: one pass over the matrix
+    instead of two, identical values inside the simulation and in all probe data, but the
+    delta signals are not written and ``sim.signals[weights]`` read between steps already
+    holds the change of the last step (`operators.apply_learning_in_place`).
     """
 
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
                  n_prealloc_probes=None, profiling=None, if_python_code="none",
                  planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
-                 fuse=True, branches=False, merge_small=True):
+                 fuse=True, branches=False, merge_small=True, learn_in_place=False):
         self.closed = False
         self.model = None
 
@@ -253,8 +258,10 @@ class Simulator:
         operators = list(map(MultiDotInc.convert_to, operators))
         if fuse:
             operators = ops_mod.fuse_into_multidotinc(operators)
-            operators = ops_mod.neurons_read_constant_input(
-                operators, keep=[self.model.sig[p]["in"] for p in self.model.probes])
+            probed = [self.model.sig[p]["in"] for p in self.model.probes]
+            operators = ops_mod.neurons_read_constant_input(operators, keep=probed)
+            if learn_in_place:
+                operators = ops_mod.apply_learning_in_place(operators, keep=probed)
         operators = MultiDotInc.compress(operators)
         op_groups = planner(operators)
         assert len([t for t, _ in op_groups if t.__name__ == "Reset"]) < 2, \
@@ -1027,35 +1034,67 @@ class Simulator:
 
     # --- learning
     def _plan_SimPES(self, ops):
+        return self._plan_learning(ops, self._plan_pes_group)
+
+    def _plan_pes_group(self, ops):
         pre = self.all_data[[self.sidx[op.pre_filtered] for op in ops]]
         error = self.all_data[[self.sidx[op.error] for op in ops]]
         delta = self.all_data[[self.sidx[op.delta] for op in ops]]
         alpha = np.array([-op.learning_rate * self.model.dt / op.pre_filtered.shape[0]
                           for op in ops])
         return [self.backend.plan_elementwise_inc(self.queue, error, pre, delta, alpha=alpha,
-                                                  outer=True, inc=False)]
+                                                  outer=True, inc=ops[0].apply_inc)]
+
+    @staticmethod
+    def _by_application(ops):
+        """Learning operators split into those that store their change and those that
+        add it to the learned matrix (`operators.apply_learning_in_place`)."""
+        for op in ops:
+            if not hasattr(op, "apply_inc"):
+                op.apply_inc = False
+        groups = [[op for op in ops if op.apply_inc == flag] for flag in (False, True)]
+        return [g for g in groups if g]
+
+    def _plan_learning(self, ops, plan_group):
+        plans = []
+        for group in self._by_application(ops):
+            for plan in plan_group(group):
+                plan.planned_ops = group
+                plans.append(plan)
+        return plans
 
     def _plan_SimBCM(self, ops):
+        return self._plan_learning(ops, self._plan_bcm_group)
+
+    def _plan_bcm_group(self, ops):
         pre = self.all_data[[self.sidx[op.pre_filtered] for op in ops]]
         post = self.all_data[[self.sidx[op.post_filtered] for op in ops]]
         theta = self.all_data[[self.sidx[op.theta] for op in ops]]
         delta = self.all_data[[self.sidx[op.delta] for op in ops]]
         alpha = np.array([op.learning_rate * self.model.dt for op in ops])
-        return [self.backend.plan_bcm(self.queue, pre, post, theta, delta, alpha)]
+        return [self.backend.plan_bcm(self.queue, pre, post, theta, delta, alpha,
+                                      inc=ops[0].apply_inc)]
 
     def _plan_SimOja(self, ops):
+        return self._plan_learning(ops, self._plan_oja_group)
+
+    def _plan_oja_group(self, ops):
         pre = self.all_data[[self.sidx[op.pre_filtered] for op in ops]]
         post = self.all_data[[self.sidx[op.post_filtered] for op in ops]]
         weights = self.all_data[[self.sidx[op.weights] for op in ops]]
         delta = self.all_data[[self.sidx[op.delta] for op in ops]]
         alpha = np.array([op.learning_rate * self.model.dt for op in ops])
         beta = np.array([op.beta for op in ops])
-        return [self.backend.plan_oja(self.queue, pre, post, weights, delta, alpha, beta)]
+        return [self.backend.plan_oja(self.queue, pre, post, weights, delta, alpha, beta,
+                                      inc=ops[0].apply_inc)]
 
     def _plan_SimRLS(self, ops):
         raise NotImplementedError("RLS learning rule not yet supported")
 
     def _plan_SimVoja(self, ops):
+        return self._plan_learning(ops, self._plan_voja_group)
+
+    def _plan_voja_group(self, ops):
         pre = self.all_data[[self.sidx[op.pre_decoded] for op in ops]]
         post = self.all_data[[self.sidx[op.post_filtered] for op in ops]]
         encoders = self.all_data[[self.sidx[op.scaled_encoders] for op in ops]]
@@ -1065,7 +1104,7 @@ class Simulator:
                                  dtype=np.float32)
         alpha = np.array([op.learning_rate * self.model.dt for op in ops])
         return [self.backend.plan_voja(self.queue, pre, post, encoders, delta, learning_signal,
-                                       scale, alpha)]
+                                       scale, alpha, inc=ops[0].apply_inc)]
 
     # --- convolution
     def _plan_ConvInc(self, ops):

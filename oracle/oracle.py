@@ -380,7 +380,7 @@ def plan_probes(queue, periods, X, Y, tag=None):
 
 # ------------------------------------------------- learning rules, convolution, noise
 def _plan_rule(rule, name, pre, post, aux, delta, alpha, beta=None, learn=None, scale=None,
-               tag=None):
+               inc=False, tag=None):
     n = len(pre)
     alphas = _per_item(alpha, n, np.float32)
     betas = _per_item(0.0 if beta is None else beta, n, np.float32)
@@ -394,24 +394,26 @@ def _plan_rule(rule, name, pre, post, aux, delta, alpha, beta=None, learn=None, 
     fn = lib().orc_learning_rule
 
     def step():
-        fn(ctypes.c_int(rule), ctypes.c_int(n), *[_p(a) for a in args], _p(pre.buf), _p(post.buf),
+        fn(ctypes.c_int(rule), ctypes.c_int(bool(inc)), ctypes.c_int(n), *[_p(a) for a in args],
+           _p(pre.buf), _p(post.buf),
            _p(aux.buf), _p(delta.buf), None if learn is None else _p(learn.buf),
            None if scale is None else _p(scale.buf))
 
     return _plan(step, name, args, tag)
 
 
-def plan_bcm(queue, pre, post, theta, delta, alpha, tag=None):
-    return _plan_rule(1, "oracle_bcm", pre, post, theta, delta, alpha, tag=tag)
+def plan_bcm(queue, pre, post, theta, delta, alpha, inc=False, tag=None):
+    return _plan_rule(1, "oracle_bcm", pre, post, theta, delta, alpha, inc=inc, tag=tag)
 
 
-def plan_oja(queue, pre, post, weights, delta, alpha, beta, tag=None):
-    return _plan_rule(2, "oracle_oja", pre, post, weights, delta, alpha, beta=beta, tag=tag)
-
-
-def plan_voja(queue, pre, post, enc, delta, learn, scale, alpha, tag=None):
-    return _plan_rule(3, "oracle_voja", pre, post, enc, delta, alpha, learn=learn, scale=scale,
+def plan_oja(queue, pre, post, weights, delta, alpha, beta, inc=False, tag=None):
+    return _plan_rule(2, "oracle_oja", pre, post, weights, delta, alpha, beta=beta, inc=inc,
                       tag=tag)
+
+
+def plan_voja(queue, pre, post, enc, delta, learn, scale, alpha, inc=False, tag=None):
+    return _plan_rule(3, "oracle_voja", pre, post, enc, delta, alpha, learn=learn, scale=scale,
+                      inc=inc, tag=tag)
 
 
 def plan_conv2d(queue, X, Y, filters, shape_in, shape_out, kernel_shape, conv=True, biases=None,

@@ -489,7 +489,7 @@ void orc_spmv_csr(int n_items, const int *n_rows, const int *indptr_starts,
  * rule 3 Voja :2349-2350  delta = alpha * learn * post * (scale * pre - enc)
  * C evaluates these left to right, every product and difference rounded to
  * float32 on its own (no contraction in this build). */
-void orc_learning_rule(int rule, int n_items, const int *shape0s, const int *shape1s,
+void orc_learning_rule(int rule, int inc, int n_items, const int *shape0s, const int *shape1s,
                        const int *pre_starts, const int *pre_stride0s, const int *post_starts,
                        const int *post_stride0s, const int *aux_starts, const int *aux_stride0s,
                        const int *delta_starts, const int *delta_stride0s, const float *alphas,
@@ -517,7 +517,10 @@ void orc_learning_rule(int rule, int n_items, const int *shape0s, const int *sha
                     const float scale = SCALE[scale_starts[k] + (size_t)i * scale_stride0s[k]];
                     out = alpha * learn * post * (scale * pre - enc);
                 }
-                DELTA[delta_starts[k] + (size_t)i * delta_stride0s[k] + j] = out;
+                /* inc: the step and the Copy(delta -> target, inc=True) that follows it
+                 * in the operator graph, applied to the target directly */
+                float *dst = DELTA + delta_starts[k] + (size_t)i * delta_stride0s[k] + j;
+                *dst = inc ? *dst + out : out;
             }
         }
     }

@@ -150,3 +150,59 @@ def test_unsupported_combinations_raise():
     net.Connection(a.neurons, b, transform=np.ones((1, 10)), learning_rule=mb.Oja())
     with pytest.raises(NotImplementedError):
         net.build_model()
+
+
+@pytest.mark.parametrize("rule_type", ["PES", "BCM", "Oja", "Voja"])
+def test_learning_in_place_gives_the_same_simulation(rule_type):
+    """`learn_in_place=True`: the rule adds its change to the learned matrix itself (no
+    delta matrix, no copy).  Probe data of every step are bit-identical to the two-pass
+    form; the matrix read from the host after n steps equals the two-pass matrix after its
+    next copy, i.e. with the last step's delta added."""
+    from nengo_ocl_amd import configs
+
+    def make():
+        if rule_type == "PES":
+            net, probes, _ = configs.c4_pes(n_triples=2, n_neurons=60, dims=3, solver="lstsq",
+                                            learning_rate=3e-4, sample_every=None)
+            return net, list(probes.values())
+        if rule_type == "Voja":
+            net, conn, post, probes = voja_network()
+            return net, probes
+        rule = mb.BCM(learning_rate=1e-9) if rule_type == "BCM" else mb.Oja(learning_rate=1e-6)
+        net, conn, probes = hebbian_network(rule)
+        return net, probes
+
+    def learned(sim):
+        """(learned matrix, delta matrix or None) per learning operator of the model."""
+        rules = [op for op in sim.model.operators
+                 if type(op).__name__ in ("SimPES", "SimBCM", "SimOja", "SimVoja")]
+        copies = {op.src: op.dst for op in sim.model.operators if type(op).__name__ == "Copy"}
+        return [(copies[op.delta], op.delta) for op in rules]
+
+    (net_a, probes_a), (net_b, probes_b) = make(), make()
+    with OracleSimulator(net_a, seed=1) as two_pass, \
+            OracleSimulator(net_b, seed=1, learn_in_place=True) as in_place:
+        kinds = lambda sim: [type(op).__name__ for op in sim.operators]
+        assert kinds(in_place).count("Copy") < kinds(two_pass).count("Copy")
+        assert any(getattr(op, "apply_inc", False) for op in in_place.operators)
+        for n in (1, 50, 150):
+            two_pass.run_steps(n)
+            in_place.run_steps(n)
+            for (w_a, d_a), (w_b, _) in zip(learned(two_pass), learned(in_place)):
+                want = np.array(two_pass.signals[w_a]) + np.array(two_pass.signals[d_a])
+                assert np.array_equal(np.array(in_place.signals[w_b]), want)
+        for a, b in zip(probes_a, probes_b):
+            assert np.array_equal(two_pass.data[a], in_place.data[b])
+        assert any(np.abs(np.array(two_pass.signals[d])).max() > 0 for _, d in learned(two_pass))
+
+
+def test_learning_in_place_leaves_probed_matrices_alone():
+    rule = mb.Oja(learning_rate=1e-6)
+    net, conn, probes = hebbian_network(rule)
+    model = net.build_model()
+    wsig = model.sig[conn]["weights"]
+    probe = ir.Probe(None)
+    model.probes.append(probe)
+    model.sig[probe] = {"in": wsig}
+    with OracleSimulator(None, model=model, seed=1, learn_in_place=True) as sim:
+        assert not any(getattr(op, "apply_inc", False) for op in sim.operators)

@@ -483,3 +483,52 @@ def test_function_nodes_run_on_the_device(queue):
         for a, b in zip(probes, probes_o):
             np.testing.assert_allclose(gpu.data[a], cpu.data[b], rtol=1e-4, atol=1e-5)
         assert np.abs(gpu.data[probes[1]]).max() > 0.1
+
+
+def test_c4_pes_learning_in_place(queue):
+    """The PES network with `learn_in_place=True` (the rule adds its change to the decoders
+    in one pass): the device follows the oracle simulator bit for bit, and both reproduce
+    the probe data of the two-pass form exactly."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    make = lambda: configs.c4_pes(n_triples=3, n_neurons=300, dims=8, solver="lstsq",
+                                  learning_rate=3e-4, sample_every=None)
+    nets = [make() for _ in range(3)]
+    with Simulator(nets[0][0], seed=1, learn_in_place=True) as gpu, \
+            OracleSimulator(nets[1][0], seed=1, learn_in_place=True) as cpu, \
+            Simulator(nets[2][0], seed=1) as two_pass:
+        assert sum(p.name == "hip_copy" for p in gpu._plans) < sum(
+            p.name == "hip_copy" for p in two_pass._plans)
+        for sim in (gpu, cpu, two_pass):
+            sim.run_steps(400)
+        for key in nets[0][1]:
+            assert np.array_equal(gpu.data[nets[0][1][key]], cpu.data[nets[1][1][key]])
+            assert np.array_equal(gpu.data[nets[0][1][key]], two_pass.data[nets[2][1][key]])
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+        assert np.abs(gpu.data[nets[0][1]["post0"]][-1]).max() > 0.05  # something was learned
+
+
+@pytest.mark.parametrize("rule_type", ["BCM", "Oja", "Voja"])
+def test_other_rules_learning_in_place(queue, rule_type):
+    from nengo_ocl_amd import minibuilder as mb
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+    from test_builder_extras import hebbian_network, voja_network
+
+    def make():
+        if rule_type == "Voja":
+            return voja_network()
+        return hebbian_network(mb.BCM(learning_rate=1e-9) if rule_type == "BCM"
+                               else mb.Oja(learning_rate=1e-6))
+
+    made_g, made_c = make(), make()
+    with Simulator(made_g[0], seed=1, learn_in_place=True) as gpu, \
+            OracleSimulator(made_c[0], seed=1, learn_in_place=True) as cpu:
+        assert any(getattr(op, "apply_inc", False) for op in gpu.operators)
+        gpu.run_steps(300)
+        cpu.run_steps(300)
+        for a, b in zip(made_g[-1], made_c[-1]):
+            assert np.array_equal(gpu.data[a], cpu.data[b])
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
