@@ -154,8 +154,8 @@ def main():
     ap.add_argument("--learn-in-place", action="store_true",
                     help="learning rules add their change to the weights in one pass (c4)")
     ap.add_argument("--branches", action="store_true",
-                    help="record kernels that touch different memory as side-by-side graph "
-                         "branches instead of one chain")
+                    help="(switched off in the library: raises) record kernels that touch "
+                         "different memory as side-by-side graph branches instead of one chain")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run the plain copy kernel on 256 MiB (1 GiB of traffic per 2 "
                          "launches) 20 times: the known-size reference for HBM counters")

@@ -144,6 +144,20 @@ int nhip_gemv_tile_filter(void *stream, int vec, int pow2_cols, int blk_words, c
                           const float *A, const float *X, const float *Yin, float *Y,
                           const int *item_targets, const int *targets, float *F);
 
+/* The same two epilogues for launches of small items (nhip_gemv with flavor 2, whose
+ * `items`, `coefs`, `dots` and 4-int `tasks` tables these take; `lpr` 4 or 1): the
+ * neuron update / filter step of a row runs in the lane that holds the row's sum.
+ * `pops`, `item_targets`, `targets` and the other arguments as above. */
+int nhip_gemv_rows_lif(void *stream, int lpr, const int *items, const float *coefs,
+                       const int *dots, const int *tasks, int n_tasks, const float *A,
+                       const float *X, const float *Yin, float *Y, const int *pops, double dt,
+                       int upsample, float *V, float *W, float *S, const float *TAU,
+                       const float *REF, const float *AMP);
+int nhip_gemv_rows_filter(void *stream, int lpr, const int *items, const float *coefs,
+                          const int *dots, const int *tasks, int n_tasks, const float *A,
+                          const float *X, const float *Yin, float *Y, const int *item_targets,
+                          const int *targets, float *F);
+
 /* ---- sparse matrix-vector products -----------------------------------------
  * Y[b] (=|+=) A[b] @ X[b] for many sparse matrices in one launch.
  * replaces: `plan_sparse_dot_inc` / `spmv_csr_impl` / `spmv_ellpack_impl`

@@ -234,6 +234,44 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
                              threadIdx.x);
 }
 
+// the same with an epilogue per finished row (A, X, Yin are not marked read-only
+// here either: the epilogue writes neuron state / filter outputs into the same buffer)
+template <int LPR, int EPI>
+__global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_epi_kernel(
+    const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
+    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    const float* A, const float* X, const float* Yin, float* Y, const EpilogueArgs epi)
+{
+    gemv_rows_ref_block<LPR, EPI>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y, blockIdx.x,
+                                  threadIdx.x, &epi);
+}
+
+template <int EPI>
+int launch_rows_epi(hipStream_t s, int lpr, const int* items, const float* coefs, const int* dots,
+                    const int* tasks, int n_tasks, const float* A, const float* X,
+                    const float* Yin, float* Y, const EpilogueArgs& epi) {
+    if (n_tasks == 0) return 0;
+    if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
+        return NHIP_E_BADARG;
+    if (lpr != 4 && lpr != 1) return NHIP_E_BADCLASS;
+    const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
+    const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
+    if (lpr == 4)
+        hipLaunchKernelGGL((gemv_rows_ref_epi_kernel<4, EPI>), grid, dim3(NHIP_WG), 0, s,
+                           reinterpret_cast<const GemvItem*>(items),
+                           reinterpret_cast<const float4*>(coefs),
+                           reinterpret_cast<const GemvDot*>(dots),
+                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi);
+    else
+        hipLaunchKernelGGL((gemv_rows_ref_epi_kernel<1, EPI>), grid, dim3(NHIP_WG), 0, s,
+                           reinterpret_cast<const GemvItem*>(items),
+                           reinterpret_cast<const float4*>(coefs),
+                           reinterpret_cast<const GemvDot*>(dots),
+                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
 template <int LPR, int VEC, int P>
 int launch_wg_p(hipStream_t s, const int* items, const float* coefs, const int* dots,
                 const int* tasks, int n_tasks, const float* A, const float* X, const float* Yin,
@@ -362,4 +400,39 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
         }
     }
     return NHIP_E_BADCLASS;
+}
+
+extern "C" int nhip_gemv_rows_lif(void* stream, int lpr, const int* items, const float* coefs,
+                                  const int* dots, const int* tasks, int n_tasks, const float* A,
+                                  const float* X, const float* Yin, float* Y, const int* pops,
+                                  double dt, int upsample, float* V, float* W, float* S,
+                                  const float* TAU, const float* REF, const float* AMP) {
+    if (!pops || !V || !W || !S || upsample < 1 || !(dt > 0.0)) return NHIP_E_BADARG;
+    EpilogueArgs args{};
+    LifArgs& lif = args.lif;
+    lif.pops = reinterpret_cast<const LifPop*>(pops);
+    lif.dtu = (float)(dt / (double)upsample);  // formed in double and rounded once, as in nhip_lif
+    lif.dt_inv = (float)(1.0 / dt);
+    lif.upsample = upsample;
+    lif.V = V;
+    lif.W = W;
+    lif.S = S;
+    lif.TAU = TAU;
+    lif.REF = REF;
+    lif.AMP = AMP;
+    return launch_rows_epi<EPI_LIF>(static_cast<hipStream_t>(stream), lpr, items, coefs, dots,
+                                    tasks, n_tasks, A, X, Yin, Y, args);
+}
+
+extern "C" int nhip_gemv_rows_filter(void* stream, int lpr, const int* items, const float* coefs,
+                                     const int* dots, const int* tasks, int n_tasks,
+                                     const float* A, const float* X, const float* Yin, float* Y,
+                                     const int* item_targets, const int* targets, float* F) {
+    if (!item_targets || !targets || !F) return NHIP_E_BADARG;
+    EpilogueArgs args{};
+    args.filter.item_targets = reinterpret_cast<const int2*>(item_targets);
+    args.filter.targets = reinterpret_cast<const FilterTarget*>(targets);
+    args.filter.F = F;
+    return launch_rows_epi<EPI_FILTER>(static_cast<hipStream_t>(stream), lpr, items, coefs, dots,
+                                       tasks, n_tasks, A, X, Yin, Y, args);
 }

@@ -5,6 +5,7 @@
 
 #include "nhip_common.h"
 #include "gemv_types.h"
+#include "neuron_math.h"
 
 // ---------------------------------------------------------------- reference order, small items
 // One output row per task (task = {item, row, 1, 0}); a wave takes 64 / LPR
@@ -21,11 +22,16 @@
 // have at most four columns, all their operands are fetched together before the sums
 // are formed in order.  Task, item and dot records are per-lane values on purpose
 // (different rows of a wave may belong to different items).
-template <int LPR>
+// EPI: what happens to a finished row besides being stored -- nothing, the LIF update
+// of the neuron whose input current the row is, or the step of the first-order filters
+// fed by the row (the same epilogues as the kernel for large items has; small
+// populations and low-dimensional decoded values save a launch the same way).
+template <int LPR, int EPI = EPI_NONE>
 __device__ __forceinline__ void gemv_rows_ref_block(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
-    const float* A, const float* X, const float* Yin, float* Y, int block, int tid)
+    const float* A, const float* X, const float* Yin, float* Y, int block, int tid,
+    const EpilogueArgs* epi = nullptr)
 {
     constexpr int TILE = 128;
     constexpr int BATCH = 4;             // dot products whose operands are fetched together
@@ -99,5 +105,18 @@ __device__ __forceinline__ void gemv_rows_ref_block(
             }
         }
     }
-    if (lir == 0 && valid) Y[it.y_start + (size_t)r * it.y_stride0] = sum + cf.z;
+    if (lir == 0 && valid) {
+        const float y = sum + cf.z;
+        Y[it.y_start + (size_t)r * it.y_stride0] = y;
+        if (EPI == EPI_LIF) {
+            const LifPop pop = epi->lif.pops[task.item];
+            if (pop.pflags & LIF_POP_ENABLED) {
+                const float v = epi->lif.V[(size_t)pop.v_start + r];
+                const float w = epi->lif.W[(size_t)pop.w_start + r];
+                lif_epilogue(epi->lif, pop, r, y, v, w);
+            }
+        }
+        if (EPI == EPI_FILTER)
+            filter_epilogue(epi->filter, epi->filter.item_targets[task.item], r, y);
+    }
 }

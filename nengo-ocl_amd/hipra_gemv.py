@@ -445,16 +445,31 @@ def _subset_param(param, idx):
     return param
 
 
+def _takes_epilogue(plan):
+    """Reference-order launches (large or small items) that do not have an epilogue yet."""
+    return (plan.name in ("hipra_gemv.tile", "hipra_gemv.wave_ref")
+            and getattr(plan, "kernel_class", (None,))[0] in (2, 3))
+
+
+def _epilogue_call(lib, plan, kind):
+    """Entry point and leading arguments of `plan`'s launch with an epilogue."""
+    if plan.kernel_class[0] == 3:
+        return getattr(lib, "nhip_gemv_tile_" + kind), plan.args
+    # nhip_gemv's (flavor, lpr, vec, passes, tables...) -> (lpr, tables...)
+    return getattr(lib, "nhip_gemv_rows_" + kind), (plan.args[1],) + tuple(plan.args[4:])
+
+
 def fuse_lif(prog, lif_plan):
     """Fewer launches for "J = GEMV(...); LIF(J)" (clra_gemv.py `plan_block_gemv` followed
-    by clra_nonlinearities.py `plan_lif`): the reference-order kernel for large items
-    updates the neurons of a row block as soon as its currents are final, so the
-    currents are not read back and the neuron kernel is not launched.
+    by clra_nonlinearities.py `plan_lif`): the reference-order kernels update the neurons
+    of a row (block) as soon as its currents are final, so the currents are not read
+    back and the neuron kernel is not launched.
 
-    A population is fused when its J is exactly the output of one large item of
-    `prog`.  Populations whose J no item of `prog` writes (neurons without input
-    connections) ride along as items without dot products.  Populations fed by small
-    items keep a neuron launch of their own.  Nothing is fused when a state the
+    A population is fused when its J is exactly the output of one item of a
+    reference-order launch of `prog` (large or small items).  Populations whose J no
+    item of `prog` writes (neurons without input connections) ride along as items
+    without dot products.  Populations fed by launches of another kind keep a neuron
+    launch of their own.  Nothing is fused when a state the
     update writes (voltage, refractory time, spikes) is read by a dot product of
     `prog`.  Returns the plans that replace ``prog.plans + [lif_plan]`` (same results
     bit for bit), or None.
@@ -471,7 +486,7 @@ def fuse_lif(prog, lif_plan):
         return None  # different device buffers: nothing to match offsets against
     large = {}
     for plan in prog.plans:
-        if plan.kernel_class[0] == 3:
+        if _takes_epilogue(plan):
             for b in plan.members:
                 if int(Y.stride0s[b]) == 1:
                     large[(int(Y.starts[b]), int(Y.shape0s[b]))] = b
@@ -544,14 +559,15 @@ def fuse_lif(prog, lif_plan):
     pop_of = {b: p for p, b in matched}
     out = []
     for plan in prog.plans:
-        if plan.kernel_class[0] != 3 or not any(b in pop_of for b in plan.members):
+        if not _takes_epilogue(plan) or not any(b in pop_of for b in plan.members):
             out.append(plan)
             continue
         lif_bytes = sum(4 * int(J.shape0s[pop_of[b]]) for b in plan.members if b in pop_of)
-        fused = Plan(queue, lib.nhip_gemv_tile_lif, plan.args + lif_args, gsize=plan.gsize,
+        entry, args = _epilogue_call(lib, plan, "lif")
+        fused = Plan(queue, entry, args + lif_args, gsize=plan.gsize,
                      lsize=plan.lsize,
                      full_args=plan.full_args + (dev_pops, V.dev_buf, W.dev_buf, S.dev_buf) + tuple(keep),
-                     name="hipra_gemv.tile_lif", tag=plan.tag,
+                     name=plan.name + "_lif", tag=plan.tag,
                      bw_per_call=plan.bw_per_call + 5 * lif_bytes,  # V and W in and out, spikes out
                      flops_per_call=plan.flops_per_call)
         fused.description = plan.description
@@ -588,15 +604,16 @@ def _read_spans(prog, ptr_value):
 def fuse_linearfilter(gemv_plans, lf_plan):
     """Fewer launches for "Y = GEMV(...); filter step on Y" (clra_gemv.py
     `plan_block_gemv` followed by clra_nonlinearities.py `plan_linearfilter`): the
-    reference-order kernel for large items steps the first-order filters whose input
-    is one of its output items as soon as a row is final.
+    reference-order kernels step the first-order filters whose input is one of their
+    output items as soon as a row is final.
 
     `gemv_plans` are the plans of one GEMV (one `gemv_prog`).  A filter item is fused
     when it has one numerator and at most one denominator coefficient, its input is
-    exactly the output of a large item in a plan without another epilogue, and both
-    vectors are contiguous.  Returns ``(plans replacing gemv_plans, plans replacing
-    [lf_plan])`` -- the second list holds a filter launch for the items that were not
-    fused, or is empty -- or None when nothing can be fused.
+    exactly the output of an item of a reference-order launch without another
+    epilogue, and both vectors are contiguous.  Returns ``(plans replacing gemv_plans,
+    plans replacing [lf_plan])`` -- the second list holds a filter launch for the items
+    that were not fused (their indices in `lf_plan`: its ``unfused_items``), or is empty
+    -- or None when nothing can be fused.
     """
     from .hipra_nonlinearities import plan_linearfilter
 
@@ -611,7 +628,7 @@ def fuse_linearfilter(gemv_plans, lf_plan):
         return None
     large = {}
     for plan in gemv_plans:
-        if plan.name == "hipra_gemv.tile" and plan.kernel_class[0] == 3:
+        if _takes_epilogue(plan):
             for b in plan.members:
                 if int(Y.stride0s[b]) == 1:
                     large[(int(Y.starts[b]), int(Y.shape0s[b]))] = b
@@ -652,14 +669,15 @@ def fuse_linearfilter(gemv_plans, lf_plan):
     extra = (dev_items.ptr, dev_targets.ptr, F.ptr)
     out = []
     for plan in gemv_plans:
-        if plan.name != "hipra_gemv.tile" or not any(b in targets_of for b in plan.members):
+        if not _takes_epilogue(plan) or not any(b in targets_of for b in plan.members):
             out.append(plan)
             continue
         f_bytes = sum(8 * int(Y.shape0s[b]) * len(targets_of[b]) for b in plan.members
                       if b in targets_of)  # filter state in and out
-        fused = Plan(queue, lib.nhip_gemv_tile_filter, plan.args + extra, gsize=plan.gsize,
+        entry, args = _epilogue_call(lib, plan, "filter")
+        fused = Plan(queue, entry, args + extra, gsize=plan.gsize,
                      lsize=plan.lsize, full_args=plan.full_args + (dev_items, dev_targets, F.dev_buf),
-                     name="hipra_gemv.tile_filter", tag=plan.tag,
+                     name=plan.name + "_filter", tag=plan.tag,
                      bw_per_call=plan.bw_per_call + f_bytes, flops_per_call=plan.flops_per_call)
         fused.description = plan.description
         fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
@@ -670,4 +688,5 @@ def fuse_linearfilter(gemv_plans, lf_plan):
     if rest:
         residual = plan_linearfilter(queue, X[rest], F[rest], A[rest], B[rest],
                                      spec["Xbuf"][rest], spec["Ybuf"][rest], tag=lf_plan.tag)
+        residual[0].unfused_items = list(rest)
     return out, residual

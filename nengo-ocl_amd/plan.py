@@ -188,6 +188,7 @@ class _GraphSegment:
         _lib.check(lib.nhip_capture_begin(self.queue.handle), "graph capture begin")
         err = None
         events = []
+        self._recording_sides = []  # side streams that have joined this recording
         try:
             for _ in range(n_steps):
                 if self.deps is None:
@@ -197,11 +198,22 @@ class _GraphSegment:
                     self._record_branches(events)
         except Exception as e:  # close the capture before re-raising
             err = e
+            # side streams that joined the recording must be led back into the recording
+            # stream first: ending a capture with unjoined streams is an error the
+            # runtime does not survive
+            for side in self._recording_sides:
+                ev = ctypes.c_void_p()
+                if lib.nhip_event_create(ctypes.byref(ev)) == 0:
+                    events.append(ev)
+                    if lib.nhip_event_record(ev, side) == 0:
+                        lib.nhip_stream_wait_event(self.queue.handle, ev)
         handle = ctypes.c_void_p()
         rc = lib.nhip_capture_end(self.queue.handle, ctypes.byref(handle))
         for ev in events:
             lib.nhip_event_destroy(ev)
         if err is not None:
+            if rc == 0 and handle:
+                lib.nhip_graph_destroy(handle)
             raise err
         _lib.check(rc, "graph capture end")
         self.execs[n_steps] = handle
@@ -247,6 +259,8 @@ class _GraphSegment:
                     si = side_stream()
                     tail[si] = None
                     _lib.check(lib.nhip_stream_wait_event(streams[si], fork), "fork")
+                    if streams[si] not in self._recording_sides:
+                        self._recording_sides.append(streams[si])
                 else:  # out of streams: queue behind the oldest tail (an extra, harmless edge)
                     si = min(tail, key=lambda k: -1 if tail[k] is None else tail[k])
             for d in deps:
@@ -282,7 +296,15 @@ class _GraphSegment:
 class Plans:
     """The ordered plan list of one timestep and its executor."""
 
-    def __init__(self, planlist, profiling, use_graph=True, branches=True):
+    def __init__(self, planlist, profiling, use_graph=True, branches=False):
+        if branches and use_graph:
+            # Switched off: ending a multi-stream recording crashed inside the HIP runtime
+            # (segmentation fault in the call that ends the capture) for a step whose
+            # branches depend on each other back and forth (stream 1 -> 2 -> 1), and the
+            # mode was slower than the single chain on this driver in every measurement.
+            raise NotImplementedError(
+                "recording independent kernels as parallel graph branches is switched off "
+                "(the runtime did not survive ending such a recording); use branches=False")
         self.plans = list(planlist)
         self.profiling = profiling
         self.use_graph = use_graph

@@ -206,9 +206,11 @@ class Simulator:
     resets as separate operators instead of folding them into the GEMVs
     (`operators.fuse_into_multidotinc`) and the neuron update as a separate launch
     instead of the epilogue of the GEMV that computes the input currents;
-    ``branches=True`` records the timestep as a graph in which kernels that touch
-    different memory run side by side instead of one chain of kernels (slower on
-    current drivers, off by default); ``merge_small=False`` keeps every short
+    ``branches=True`` (record the timestep as a graph in which kernels that touch
+    different memory run side by side instead of one chain of kernels) is switched off
+    and raises NotImplementedError: it was slower than the chain, and ending such a
+    multi-stream recording crashed inside the runtime for one step shape;
+    ``merge_small=False`` keeps every short
     operation (clock, inputs, small copies and filters, probes) as a launch of its
     own instead of binding runs of them into one launch; ``learn_in_place=True`` (with
     ``fuse``) lets learning rules add their change to the learned matrix directly instead
@@ -401,11 +403,20 @@ class Simulator:
             if result is None:
                 continue
             fused, residual = result
+            # memory of the filters that moved into the GEMV / of those that stayed behind
+            ops = getattr(lf, "planned_ops", None)
+            rest = set(residual[0].unfused_items) if residual else set()
+            if ops is not None and len(ops) == len(lf.lf_spec["X"]):
+                mem = lambda sel: ({op.input.base for k, op in enumerate(ops) if sel(k)},
+                                   {op.output.base for k, op in enumerate(ops) if sel(k)})
+                (fr, fw), (rr, rw) = mem(lambda k: k not in rest), mem(lambda k: k in rest)
+            else:
+                (fr, fw), (rr, rw) = (lf.reads_mem, lf.writes_mem), (lf.reads_mem, lf.writes_mem)
             for new, old in zip(fused, plans[lo:i + 1]):
-                new.reads_mem = old.reads_mem | lf.reads_mem
-                new.writes_mem = old.writes_mem | lf.writes_mem
+                new.reads_mem = old.reads_mem | fr
+                new.writes_mem = old.writes_mem | fw
             for p in residual:
-                p.reads_mem, p.writes_mem = lf.reads_mem, lf.writes_mem
+                p.reads_mem, p.writes_mem = rr, rw
                 if getattr(p, "bufpos", None) is not None:
                     self._filter_positions.append(p.bufpos)
             plans[j - 1:j] = residual

@@ -408,10 +408,10 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     fused = g.fuse_lif(prog, lif)
     assert fused is not None
     names = sorted(p.name for p in fused)
-    # three large-item classes (the input-less population joins the power-of-two one),
-    # the small item's wave kernel, and the neuron launch of the population it feeds
-    assert names == ["hip_lif", "hipra_gemv.tile_lif", "hipra_gemv.tile_lif",
-                     "hipra_gemv.tile_lif", "hipra_gemv.wave_ref"]
+    # three large-item classes (the input-less population joins the power-of-two one)
+    # and the small item's launch, each updating the neurons it feeds: no neuron launch
+    assert names == ["hipra_gemv.tile_lif", "hipra_gemv.tile_lif", "hipra_gemv.tile_lif",
+                     "hipra_gemv.wave_ref_lif"]
     assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_lif"} == {
         (3, 1, 4), (3, 0, 4), (3, 0, 1)}
     for step in range(3):
@@ -455,7 +455,8 @@ def test_gemv_with_filter_epilogue(queue):
     """GEMV + first-order filters in one launch: every decoded vector and every filter
     output equals the oracle's GEMV followed by its filter step bit for bit over
     several steps -- several filters per GEMV item, a pure gain, a filter fed by a
-    small item and a second-order filter (both keep a launch of their own)."""
+    small item (epilogue of the small-item launch) and a second-order filter (keeps a
+    launch of its own)."""
     from nengo_ocl_amd import hipra_gemv as g
     from nengo_ocl_amd import hipra_nonlinearities as nl
     from oracle import oracle as orc
@@ -503,7 +504,7 @@ def test_gemv_with_filter_epilogue(queue):
     assert result is not None
     fused, residual = result
     assert sorted(p.name for p in fused) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_filter",
-                                              "hipra_gemv.wave_ref"]
+                                              "hipra_gemv.wave_ref_filter"]
     assert [p.name for p in residual] == ["hip_linearfilter"]
     oprog, olf = build(host, orc, orc, None, lambda a: a)
     for step in range(4):

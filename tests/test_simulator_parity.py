@@ -222,16 +222,28 @@ def _graph_cases():
     }
 
 
+BRANCHES_OFF = ("recording a step as parallel graph branches is switched off: the call that "
+                "ends such a multi-stream recording crashed inside the HIP runtime for the c4 "
+                "step (host segmentation fault, no device fault); Simulator(branches=True) "
+                "raises NotImplementedError")
+
+
 @pytest.mark.parametrize("case", ["c2", "c1", "c4", "c3"])
-def test_graph_replay_equals_eager(queue, case):
-    """The recorded graph -- with independent kernels as side-by-side branches, and as
-    one chain, short operations bound into sequence launches -- and the eager loop of
-    one launch per operation give bit-identical state, also when the graph is
-    replayed in several batches with host work in between."""
+@pytest.mark.parametrize("with_branches", [False, pytest.param(True, marks=pytest.mark.skip(
+    reason=BRANCHES_OFF))], ids=["chain", "branches"])
+def test_graph_replay_equals_eager(queue, case, with_branches):
+    """The recorded graph -- one chain of kernels, short operations bound into sequence
+    launches (and, when that mode is available, independent kernels as side-by-side
+    branches) -- and the eager loop of one launch per operation give bit-identical
+    state, also when the graph is replayed in several batches with host work in
+    between."""
     from nengo_ocl_amd.simulator import Simulator
 
     results = []
-    for use_graph, branches, merge in ((True, True, True), (True, False, True), (False, False, False)):
+    variants = [(True, False, True), (False, False, False)]
+    if with_branches:
+        variants.insert(0, (True, True, True))
+    for use_graph, branches, merge in variants:
         net, probes, _ = _graph_cases()[case]()
         with Simulator(net, seed=1, use_graph=use_graph, branches=branches, merge_small=merge,
                        n_prealloc_probes=8) as sim:
@@ -532,3 +544,12 @@ def test_other_rules_learning_in_place(queue, rule_type):
         for a, b in zip(made_g[-1], made_c[-1]):
             assert np.array_equal(gpu.data[a], cpu.data[b])
         assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+
+
+def test_graph_branches_are_switched_off(queue):
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+
+    net, _, _ = configs.c0_readme(n_neurons=20)
+    with pytest.raises(NotImplementedError, match="switched off"):
+        Simulator(net, seed=1, branches=True)
