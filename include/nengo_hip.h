@@ -421,6 +421,14 @@ int nhip_stream_create(void **stream_out); /* non-blocking, default priority */
 int nhip_stream_destroy(void *stream);
 int nhip_stream_wait_event(void *stream, void *event);
 
+/* The next kernel launched by the calling thread through this library carries
+ * `start` and `stop` itself: their difference is the kernel's own duration, without
+ * the dispatch latency and end-of-kernel cache maintenance that events recorded
+ * around a launch include (the figure a kernel trace shows).  Both NULL cancels.
+ * Not for launches that are being recorded into a graph, and not for
+ * nhip_rtc_launch_direct (which launches through the module API). */
+int nhip_time_next_launch(void *start, void *stop);
+
 /* events on `stream` (for per-plan and whole-run timing) */
 int nhip_event_create(void **event_out);
 int nhip_event_record(void *event, void *stream);

@@ -72,6 +72,7 @@ SIGNATURES = {
     "nhip_stream_create": [ctypes.POINTER(c_void_p)],
     "nhip_stream_destroy": [P],
     "nhip_stream_wait_event": [P, P],
+    "nhip_time_next_launch": [P, P],
     "nhip_event_create": [ctypes.POINTER(c_void_p)],
     "nhip_event_record": [P, P],
     "nhip_event_elapsed_ms": [P, P, ctypes.POINTER(c_float)],

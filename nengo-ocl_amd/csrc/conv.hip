@@ -164,7 +164,7 @@ extern "C" int nhip_conv2d(void* stream, const int* geom, const float* X, const 
     const size_t lds = (size_t)g.c_chunk * g.nipatch * g.njpatch * sizeof(float);
     if (lds > 48 * 1024) return NHIP_E_BADARG;
     const dim3 grid(g.tiles_j * tiles_i, (g.nf + g.tile_f - 1) / g.tile_f);
-    hipLaunchKernelGGL(conv2d_kernel, grid, dim3(NHIP_WG), lds, NHIP_STREAM(stream), g, X, F, Y);
+    NHIP_LAUNCH(conv2d_kernel, grid, dim3(NHIP_WG), lds, NHIP_STREAM(stream), g, X, F, Y);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -180,7 +180,7 @@ extern "C" int nhip_pool2d(void* stream, const int* geom, const float* X, float*
         return NHIP_E_BADARG;
     const long long n = (long long)g.nc * g.nyi * g.nyj;
     if (n > 0x7fffffffLL) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(pool2d_kernel, dim3((unsigned)((n + NHIP_WG - 1) / NHIP_WG)),
+    NHIP_LAUNCH(pool2d_kernel, dim3((unsigned)((n + NHIP_WG - 1) / NHIP_WG)),
                        dim3(NHIP_WG), 0, NHIP_STREAM(stream), g, X, Y);
     NHIP_LAUNCH_CHECK();
     return 0;

@@ -491,7 +491,7 @@ dim3 row_grid(int n_rows, int lanes) {
 extern "C" int nhip_reset(void* stream, const int* blocks, int n_blocks, int lanes, float* Y) {
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !lanes_ok(lanes) || !blocks || !Y) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(reset_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(reset_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), reinterpret_cast<const int4*>(blocks), n_blocks, lanes,
                        Y);
     NHIP_LAUNCH_CHECK();
@@ -502,7 +502,7 @@ extern "C" int nhip_copy(void* stream, const int* desc, int n_blocks, int lanes,
                          float* Y) {
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !X || !Y) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(copy_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(copy_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), reinterpret_cast<const CopyDesc*>(desc), n_blocks,
                        lanes, X, Y);
     NHIP_LAUNCH_CHECK();
@@ -513,7 +513,7 @@ extern "C" int nhip_slicedcopy(void* stream, const int* desc, int n_blocks, int 
                                const float* X, float* Y, const int* XI, const int* YI) {
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !X || !Y || !XI || !YI) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(slicedcopy_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(slicedcopy_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), reinterpret_cast<const SlicedDesc*>(desc), n_blocks,
                        lanes, X, Y, XI, YI);
     NHIP_LAUNCH_CHECK();
@@ -524,7 +524,7 @@ extern "C" int nhip_elementwise_inc(void* stream, const int* desc, int n_blocks,
                                     const float* A, const float* X, float* Y) {
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !A || !X || !Y) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(elementwise_inc_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(elementwise_inc_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), reinterpret_cast<const EwDesc*>(desc), n_blocks, lanes,
                        A, X, Y);
     NHIP_LAUNCH_CHECK();
@@ -537,7 +537,7 @@ extern "C" int nhip_linearfilter(void* stream, const int* desc, int* pos, int n_
     if (n_blocks == 0) return 0;
     // A, Xbuf, Ybuf may be empty
     if (n_blocks < 0 || !lanes_ok(lanes) || !desc || !pos || !X || !Y || !B) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(linearfilter_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(linearfilter_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), reinterpret_cast<const LfDesc*>(desc),
                        reinterpret_cast<int2*>(pos), n_blocks, lanes, X, Y, A, B, Xbuf, Ybuf);
     NHIP_LAUNCH_CHECK();
@@ -547,7 +547,7 @@ extern "C" int nhip_linearfilter(void* stream, const int* desc, int* pos, int n_
 extern "C" int nhip_timeupdate(void* stream, float* step_data, int step_start, float* time_data,
                                int time_start, double dt) {
     if (!step_data || !time_data || step_start < 0 || time_start < 0) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(timeupdate_kernel, dim3(1), dim3(NHIP_WAVE), 0, NHIP_STREAM(stream),
+    NHIP_LAUNCH(timeupdate_kernel, dim3(1), dim3(NHIP_WAVE), 0, NHIP_STREAM(stream),
                        step_data + step_start, time_data + time_start, dt);
     NHIP_LAUNCH_CHECK();
     return 0;
@@ -557,7 +557,7 @@ extern "C" int nhip_presentinput(void* stream, const int* desc, int n, int lanes
                                  float* Y, const float* T, const float* S) {
     if (n == 0) return 0;
     if (n < 0 || !lanes_ok(lanes) || !desc || !Y || !T || !S) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(presentinput_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(presentinput_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), reinterpret_cast<const PiDesc*>(desc), n, lanes, dt, Y,
                        T, S);
     NHIP_LAUNCH_CHECK();
@@ -569,7 +569,7 @@ extern "C" int nhip_direct_unary(void* stream, int opcode, const int* desc, int 
     if (n == 0) return 0;
     if (n < 0 || !lanes_ok(lanes) || !desc || !X || !Y || opcode < 0 || opcode > 5)
         return NHIP_E_BADARG;
-    hipLaunchKernelGGL(direct_unary_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(direct_unary_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), opcode, reinterpret_cast<const int4*>(desc), n, lanes,
                        X, Y);
     NHIP_LAUNCH_CHECK();
@@ -581,7 +581,7 @@ extern "C" int nhip_probes(void* stream, const int* desc, int n, int lanes, floa
     if (n == 0) return 0;
     if (n < 0 || !lanes_ok(lanes) || !desc || !countdowns || !bufpositions || !periods || !X || !Y)
         return NHIP_E_BADARG;
-    hipLaunchKernelGGL(probes_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+    NHIP_LAUNCH(probes_kernel, row_grid(n, lanes), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
                        reinterpret_cast<const ProbeDesc*>(desc), n, lanes, countdowns,
                        bufpositions, periods, X, Y);
     NHIP_LAUNCH_CHECK();
@@ -591,7 +591,7 @@ extern "C" int nhip_probes(void* stream, const int* desc, int n, int lanes, floa
 extern "C" int nhip_fill_i32(void* stream, int* dst, int n, int value) {
     if (n == 0) return 0;
     if (n < 0 || !dst) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(fill_i32_kernel, dim3((n + NHIP_WG - 1) / NHIP_WG), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(fill_i32_kernel, dim3((n + NHIP_WG - 1) / NHIP_WG), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), dst, n, value);
     NHIP_LAUNCH_CHECK();
     return 0;
@@ -601,7 +601,7 @@ extern "C" int nhip_sequence(void* stream, const void* ops, int n_ops, int n_sta
     if (n_ops == 0) return 0;
     if (n_ops < 0 || n_ops > SEQ_MAX_OPS || n_staged < 0 || n_staged > SEQ_MAX_ROWS || !ops)
         return NHIP_E_BADARG;
-    hipLaunchKernelGGL(sequence_kernel, dim3(1), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+    NHIP_LAUNCH(sequence_kernel, dim3(1), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
                        reinterpret_cast<const NhipSeqOp*>(ops), n_ops, n_staged);
     NHIP_LAUNCH_CHECK();
     return 0;

@@ -257,13 +257,13 @@ int launch_rows_epi(hipStream_t s, int lpr, const int* items, const float* coefs
     const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
     const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
     if (lpr == 4)
-        hipLaunchKernelGGL((gemv_rows_ref_epi_kernel<4, EPI>), grid, dim3(NHIP_WG), 0, s,
+        NHIP_LAUNCH((gemv_rows_ref_epi_kernel<4, EPI>), grid, dim3(NHIP_WG), 0, s,
                            reinterpret_cast<const GemvItem*>(items),
                            reinterpret_cast<const float4*>(coefs),
                            reinterpret_cast<const GemvDot*>(dots),
                            reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi);
     else
-        hipLaunchKernelGGL((gemv_rows_ref_epi_kernel<1, EPI>), grid, dim3(NHIP_WG), 0, s,
+        NHIP_LAUNCH((gemv_rows_ref_epi_kernel<1, EPI>), grid, dim3(NHIP_WG), 0, s,
                            reinterpret_cast<const GemvItem*>(items),
                            reinterpret_cast<const float4*>(coefs),
                            reinterpret_cast<const GemvDot*>(dots),
@@ -276,7 +276,7 @@ template <int LPR, int VEC, int P>
 int launch_wg_p(hipStream_t s, const int* items, const float* coefs, const int* dots,
                 const int* tasks, int n_tasks, const float* A, const float* X, const float* Yin,
                 float* Y) {
-    hipLaunchKernelGGL((gemv_wg_kernel<LPR, VEC, P>), dim3(n_tasks), dim3(NHIP_WG), 0, s,
+    NHIP_LAUNCH((gemv_wg_kernel<LPR, VEC, P>), dim3(n_tasks), dim3(NHIP_WG), 0, s,
                        reinterpret_cast<const GemvItem*>(items),
                        reinterpret_cast<const float4*>(coefs),
                        reinterpret_cast<const GemvDot*>(dots),
@@ -302,7 +302,7 @@ int launch_wave(hipStream_t s, const int* items, const float* coefs, const int* 
                 const int* tasks, int n_tasks, const float* A, const float* X,
                 const float* Yin, float* Y) {
     const int wpg = NHIP_WG / NHIP_WAVE;
-    hipLaunchKernelGGL((gemv_wave_kernel<LPR, VEC>), dim3((n_tasks + wpg - 1) / wpg),
+    NHIP_LAUNCH((gemv_wave_kernel<LPR, VEC>), dim3((n_tasks + wpg - 1) / wpg),
                        dim3(NHIP_WG), 0, s, reinterpret_cast<const GemvItem*>(items),
                        reinterpret_cast<const float4*>(coefs),
                        reinterpret_cast<const GemvDot*>(dots),
@@ -375,13 +375,13 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
         const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
         const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
         if (lpr == 4)
-            hipLaunchKernelGGL(gemv_rows_ref_kernel<4>, grid, dim3(NHIP_WG), 0, s,
+            NHIP_LAUNCH(gemv_rows_ref_kernel<4>, grid, dim3(NHIP_WG), 0, s,
                                reinterpret_cast<const GemvItem*>(items),
                                reinterpret_cast<const float4*>(coefs),
                                reinterpret_cast<const GemvDot*>(dots),
                                reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
         else
-            hipLaunchKernelGGL(gemv_rows_ref_kernel<1>, grid, dim3(NHIP_WG), 0, s,
+            NHIP_LAUNCH(gemv_rows_ref_kernel<1>, grid, dim3(NHIP_WG), 0, s,
                                reinterpret_cast<const GemvItem*>(items),
                                reinterpret_cast<const float4*>(coefs),
                                reinterpret_cast<const GemvDot*>(dots),

@@ -730,7 +730,7 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     const int n_groups = (n_tasks + waves - 1) / waves;
     hipStream_t s = static_cast<hipStream_t>(stream);
     auto launch = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+        NHIP_LAUNCH(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
                            reinterpret_cast<const GemvItem*>(items),
                            reinterpret_cast<const float4*>(coefs),
                            reinterpret_cast<const GemvDot*>(dots),

@@ -72,16 +72,16 @@ extern "C" int nhip_learning_rule(void* stream, int rule, int inc, const int* de
     const dim3 grid(n_blocks), block(NHIP_WG);
     switch (rule) {
     case NHIP_RULE_BCM:
-        hipLaunchKernelGGL(learning_kernel<NHIP_RULE_BCM>, grid, block, 0, NHIP_STREAM(stream), d,
+        NHIP_LAUNCH(learning_kernel<NHIP_RULE_BCM>, grid, block, 0, NHIP_STREAM(stream), d,
                            inc, PRE, POST, AUX, DELTA, LEARN, SCALE);
         break;
     case NHIP_RULE_OJA:
-        hipLaunchKernelGGL(learning_kernel<NHIP_RULE_OJA>, grid, block, 0, NHIP_STREAM(stream), d,
+        NHIP_LAUNCH(learning_kernel<NHIP_RULE_OJA>, grid, block, 0, NHIP_STREAM(stream), d,
                            inc, PRE, POST, AUX, DELTA, LEARN, SCALE);
         break;
     case NHIP_RULE_VOJA:
         if (!LEARN || !SCALE) return NHIP_E_BADARG;
-        hipLaunchKernelGGL(learning_kernel<NHIP_RULE_VOJA>, grid, block, 0, NHIP_STREAM(stream),
+        NHIP_LAUNCH(learning_kernel<NHIP_RULE_VOJA>, grid, block, 0, NHIP_STREAM(stream),
                            d, inc, PRE, POST, AUX, DELTA, LEARN, SCALE);
         break;
     default:

@@ -153,7 +153,7 @@ extern "C" int nhip_lif(void* stream, const int* desc, int n_blocks, double dt, 
     // reference's rendered literals are
     const float dtu = (float)(dt / (double)upsample);
     const float dt_inv = (float)(1.0 / dt);
-    hipLaunchKernelGGL(lif_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(lif_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),
                        reinterpret_cast<const LifDesc*>(desc), dtu, dt_inv, upsample, J, V, W, S,
                        TAU, REF, AMP);
@@ -165,7 +165,7 @@ extern "C" int nhip_lif_rate(void* stream, const int* desc, int n_blocks, const 
                              const float* TAU, const float* REF, const float* AMP) {
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !desc || !J || !R) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(lif_rate_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(lif_rate_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),
                        reinterpret_cast<const RateDesc*>(desc), J, R, TAU, REF, AMP);
     NHIP_LAUNCH_CHECK();
@@ -179,7 +179,7 @@ extern "C" int nhip_alif(void* stream, const int* desc, int n_blocks, double dt,
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !desc || !J || !V || !W || !S || !N || upsample < 1 || !(dt > 0.0))
         return NHIP_E_BADARG;
-    hipLaunchKernelGGL(alif_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(alif_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),
                        reinterpret_cast<const NeuronDesc*>(desc), (float)dt,
                        (float)(dt / (double)upsample), (float)(1.0 / dt), upsample, J, V, W, S, N,
@@ -194,7 +194,7 @@ extern "C" int nhip_alif_rate(void* stream, const int* desc, int n_blocks, doubl
                               const float* INC_N) {
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !desc || !J || !R || !N || !(dt > 0.0)) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(alif_rate_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(alif_rate_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),
                        reinterpret_cast<const NeuronDesc*>(desc), (float)dt, J, R, N, TAU, REF, AMP,
                        TAU_N, INC_N);
@@ -208,7 +208,7 @@ int launch_simple(void* stream, int kind, const int* desc, int n_blocks, double 
     if (n_blocks == 0) return 0;
     if (n_blocks < 0 || !desc || !J || !OUT || (kind == 1 && (!V || !(dt > 0.0))))
         return NHIP_E_BADARG;
-    hipLaunchKernelGGL(simple_neuron_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(simple_neuron_kernel, dim3(n_blocks), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream), kind,
                        reinterpret_cast<const NeuronDesc*>(desc), (float)dt,
                        kind == 1 ? (float)(1.0 / dt) : 0.0f, J, OUT, V, P);

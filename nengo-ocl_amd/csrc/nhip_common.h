@@ -2,12 +2,32 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include "../../include/nengo_hip.h"
 
 #define NHIP_WG 256    // threads per work-group: four wave64
 #define NHIP_WAVE 64
 #define NHIP_NXCD 8    // MI355X: 8 accelerator dies, each with its own L2
+
+// Every kernel of the library is launched through NHIP_LAUNCH.  Normally that is a
+// plain launch.  After nhip_time_next_launch(start, stop) the next launch of the
+// calling thread carries the two events itself, so that their difference is the
+// kernel's own duration (first wave to last wave), without the dispatch latency and
+// end-of-kernel cache maintenance that events recorded around a launch include.
+struct NhipLaunchEvents { hipEvent_t start, stop; };
+extern thread_local NhipLaunchEvents nhip_launch_events;
+#define NHIP_LAUNCH(kernel, grid, block, lds, stream, ...)                                   \
+    do {                                                                                     \
+        if (nhip_launch_events.start) {                                                      \
+            const NhipLaunchEvents ev_ = nhip_launch_events;                                 \
+            nhip_launch_events = NhipLaunchEvents{nullptr, nullptr};                         \
+            hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, ev_.start, ev_.stop, 0,  \
+                                  __VA_ARGS__);                                              \
+        } else {                                                                             \
+            hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);               \
+        }                                                                                    \
+    } while (0)
 
 #define NHIP_LAUNCH_CHECK()                 \
     do {                                    \

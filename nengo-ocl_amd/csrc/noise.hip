@@ -90,7 +90,7 @@ extern "C" int nhip_whitenoise(void* stream, const int* desc, int n_items, int* 
                                double sqrt_dt_inv, float* Y) {
     if (n_items == 0) return 0;
     if (n_items < 0 || !desc || !counters || !Y) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(whitenoise_kernel, dim3(n_items), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+    NHIP_LAUNCH(whitenoise_kernel, dim3(n_items), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
                        reinterpret_cast<const NoiseDesc*>(desc), counters, sqrt_dt_inv, Y);
     NHIP_LAUNCH_CHECK();
     return 0;
@@ -100,7 +100,7 @@ extern "C" int nhip_philox4x32(void* stream, const unsigned* counters_keys, unsi
                                int n) {
     if (n == 0) return 0;
     if (n < 0 || !counters_keys || !out) return NHIP_E_BADARG;
-    hipLaunchKernelGGL(philox_test_kernel, dim3((n + 63) / 64), dim3(64), 0, NHIP_STREAM(stream),
+    NHIP_LAUNCH(philox_test_kernel, dim3((n + 63) / 64), dim3(64), 0, NHIP_STREAM(stream),
                        counters_keys, out, n);
     NHIP_LAUNCH_CHECK();
     return 0;

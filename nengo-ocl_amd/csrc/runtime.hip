@@ -8,7 +8,16 @@
 
 #include "nhip_common.h"
 
+thread_local NhipLaunchEvents nhip_launch_events = {nullptr, nullptr};
+
 extern "C" int nhip_abi_version(void) { return NHIP_ABI_VERSION; }
+
+extern "C" int nhip_time_next_launch(void* start, void* stop) {
+    if ((start == nullptr) != (stop == nullptr)) return NHIP_E_BADARG;
+    nhip_launch_events = NhipLaunchEvents{static_cast<hipEvent_t>(start),
+                                          static_cast<hipEvent_t>(stop)};
+    return 0;
+}
 
 extern "C" const char* nhip_error_string(int err) {
     switch (err) {

@@ -68,7 +68,7 @@ extern "C" int nhip_spmv_sell(void* stream, const int* slices, int n_slices, con
     if (n_slices == 0) return 0;
     if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y) return NHIP_E_BADARG;
     const int wpg = NHIP_WG / NHIP_WAVE;
-    hipLaunchKernelGGL(spmv_sell_kernel, dim3((n_slices + wpg - 1) / wpg), dim3(NHIP_WG), 0,
+    NHIP_LAUNCH(spmv_sell_kernel, dim3((n_slices + wpg - 1) / wpg), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),
                        reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X,
                        Y);

@@ -66,6 +66,8 @@ class Plan(BasePlan):
     not free them.
     """
 
+    LAUNCHES_WITHOUT_EVENTS = ("nhip_rtc_launch_direct",)
+
     def __init__(self, queue, kern, args, gsize, lsize=None, full_args=(), **kwargs):
         super().__init__(**kwargs)
         self.queue = queue
@@ -92,10 +94,19 @@ class Plan(BasePlan):
             ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
             _lib.check(lib.nhip_event_create(ctypes.byref(ev0)))
             _lib.check(lib.nhip_event_create(ctypes.byref(ev1)))
-            _lib.check(lib.nhip_event_record(ev0, handle))
+            # the kernel carries its own start / stop events where the entry point
+            # launches through the runtime API; otherwise events around the launch
+            own = getattr(self.kern, "__name__", "") not in self.LAUNCHES_WITHOUT_EVENTS
+            if own:
+                _lib.check(lib.nhip_time_next_launch(ev0, ev1))
+            else:
+                _lib.check(lib.nhip_event_record(ev0, handle))
         _lib.check(self.kern(handle, *self.args), self.name)
         if profiling:
-            _lib.check(lib.nhip_event_record(ev1, handle))
+            if own:
+                _lib.check(lib.nhip_time_next_launch(None, None))  # in case nothing was launched
+            else:
+                _lib.check(lib.nhip_event_record(ev1, handle))
             self._events_to_profile.append((ev0, ev1))
         return self
 
