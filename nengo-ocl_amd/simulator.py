@@ -434,8 +434,10 @@ class Simulator:
             raise ImportError(
                 "building a nengo Network needs the `nengo` package (>= 3.1); without it "
                 "pass a minibuilder.Network or a ready ir.Model") from e
+        from .builder import Builder
+
         model = Model(dt=float(dt), label="%s, dt=%f" % (network, dt),
-                      decoder_cache=get_default_decoder_cache())
+                      decoder_cache=get_default_decoder_cache(), builder=Builder())
         model.build(network)
         return model
 
