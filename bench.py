@@ -139,6 +139,77 @@ def calibrate_copy(n_floats=64 * 1024 * 1024, repeats=20):
                       "read_bytes_per_launch": 4 * n_floats, "write_bytes_per_launch": 4 * n_floats}))
 
 
+def micro_benchmarks(repeats=50):
+    """Kernels that no benchmark network exercises, each on one representative problem:
+    one JSON line per kernel with its average duration (start / stop events carried by
+    the launch) and the rate of its algorithmic bytes."""
+    import numpy as np
+
+    from nengo_ocl_amd import fn_trace
+    from nengo_ocl_amd import hipra_nonlinearities as nl
+    from nengo_ocl_amd.hipraggedarray import HIPRaggedArray, Queue
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    queue = Queue(0)
+    rng = np.random.RandomState(0)
+    dev = lambda arrays, **kw: HIPRaggedArray(queue, RaggedArray(arrays, dtype=np.float32, **kw))
+    cases = []
+
+    n_conn, m, n = 64, 2000, 2000  # 64 learned 2000 x 2000 weight matrices
+    pre, post = dev([rng.rand(n) for _ in range(n_conn)]), dev([rng.rand(m) for _ in range(n_conn)])
+    theta = dev([rng.rand(m) for _ in range(n_conn)])
+    W, delta = (dev([rng.normal(size=(m, n)) for _ in range(n_conn)]) for _ in range(2))
+    alpha, beta = np.full(n_conn, 1e-6, np.float32), np.ones(n_conn, np.float32)
+    what = "%d x (%d x %d)" % (n_conn, m, n)
+    cases.append(("bcm", what, nl.plan_bcm(queue, pre, post, theta, delta, alpha)))
+    cases.append(("oja", what, nl.plan_oja(queue, pre, post, W, delta, alpha, beta)))
+    cases.append(("oja, in place", what, nl.plan_oja(queue, pre, post, W, W, alpha, beta, inc=True)))
+    err = dev([rng.rand(m) for _ in range(n_conn)])
+    cases.append(("pes (outer product)", what,
+                  nl.plan_elementwise_inc(queue, err, pre, delta, alpha=alpha, outer=True, inc=False)))
+
+    for shape_in, nf, kernel, strides in (((28, 28, 1), 32, (3, 3), (1, 1)),
+                                          ((26, 26, 32), 64, (3, 3), (2, 2)),
+                                          ((224, 224, 3), 64, (7, 7), (2, 2))):
+        nyi = (shape_in[0] - kernel[0]) // strides[0] + 1
+        nyj = (shape_in[1] - kernel[1]) // strides[1] + 1
+        data = dev([rng.rand(int(np.prod(shape_in))),
+                    rng.normal(size=kernel[0] * kernel[1] * shape_in[2] * nf),
+                    np.zeros(nyi * nyj * nf)])
+        plan = nl.plan_conv2d(queue, data[[0]], data[[2]], data[[1]], shape_in, (nyi, nyj, nf), kernel,
+                              strides=strides, channels_last=True)
+        cases.append(("conv2d", "%s -> %s, kernel %s, stride %s" % (
+            shape_in, (nyi, nyj, nf), kernel, strides), plan))
+
+    Y = dev([np.zeros(1000000), np.zeros(64)])
+    cases.append(("whitenoise (Gaussian)", "1,000,000 + 64 samples",
+                  nl.plan_whitenoise(queue, Y, np.int32([1, 1]), np.float32([[0, 1], [0, 1]]),
+                                     [1, 1], [0, 0], 1e-3, [1, 2])))
+    n_nodes = 100000
+    traced = fn_trace.trace(lambda t, x: [np.sin(t) * x[0] + x[1] ** 2, np.tanh(x[0] - x[1])],
+                            True, 2, 2)
+    T, X2, Y2 = dev([[0.5]] * n_nodes), dev([rng.rand(2) for _ in range(n_nodes)]), dev(
+        [np.zeros(2)] * n_nodes)
+    plan = nl.plan_direct(queue, traced.code, traced.init, traced.input_names, [T, X2], Y2)
+    cases.append(("compiled function node", "%d instances of a 2 -> 2 function" % n_nodes, plan))
+
+    for name, what, plan in cases:
+        for _ in range(3):
+            plan()
+        for _ in range(repeats):
+            plan.enqueue(profiling=True)
+        queue.finish()
+        plan.update_profiling()
+        avg = sum(plan.ctimes) / len(plan.ctimes)
+        print(json.dumps({"kernel": name, "problem": what, "avg_us": round(1e6 * avg, 2),
+                          "algorithmic_bytes": plan.bw_per_call,
+                          "gbs": round(1e-9 * plan.bw_per_call / avg, 1) if plan.bw_per_call else None,
+                          "gflops": round(1e-9 * plan.flops_per_call / avg, 1)
+                          if plan.flops_per_call else None,
+                          "timing": "events carried by the launch" if name != "compiled function node"
+                          else "events around the launch"}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,9 +230,14 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run the plain copy kernel on 256 MiB (1 GiB of traffic per 2 "
                          "launches) 20 times: the known-size reference for HBM counters")
+    ap.add_argument("--micro", action="store_true",
+                    help="only time the kernels no benchmark network uses (learning rules, "
+                         "convolution, noise, compiled function nodes), one JSON line each")
     args = ap.parse_args()
     if args.calibrate_copy:
         return calibrate_copy()
+    if args.micro:
+        return micro_benchmarks()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the timestep of one simulator runs on a single "
                          "MI355X and nothing here uses a second device (got --gpus %d)" % args.gpus)

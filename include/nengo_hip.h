@@ -274,7 +274,8 @@ int nhip_learning_rule(void *stream, int rule, int inc, const int *desc, int n_b
  * X is (nxi, nxj, nc) with channels last, else (nc, nxi, nxj); Y likewise with nf;
  * F is (si, sj, nc, nf), or for local filtering (nf, nc, si, sj, nyi, nyj).  A group
  * computes tile_i x tile_j output pixels x tile_f filters (product <= 256) and
- * stages c_chunk channels of the input patch in LDS at a time (<= 48 KiB).  Each
+ * stages c_chunk channels of the input patch and of its filters' taps in LDS at a
+ * time (<= 64 KiB).  Each
  * output is accumulated over channel, kernel row, kernel column in that order with
  * one fused multiply-add per term. */
 int nhip_conv2d(void *stream, const int *geom, const float *X, const float *F, float *Y);
@@ -292,14 +293,16 @@ int nhip_pool2d(void *stream, const int *geom, const float *X, float *Y);
  * counter-based Philox4x32-10 generator: the block of four 32-bit words for
  * elements 4q..4q+3 of call n is philox(counter {q, n, 0, 0}, key {seed, 0}), so
  * the sample streams are not the reference's (whose streams are not nengo's
- * either), and the only state is the per-item call count.
- *   desc     : int32[n_items][8] {y_start, count, dist, p0_bits, p1_bits,
- *                                 flags(bit0 scale, bit1 inc), seed, 0}
- *   counters : int32[n_items], read and advanced by one per call (zero them to
+ * either), and the only state is the call count.  An item is cut into blocks of
+ * elements [offset, offset + count), offset a multiple of 4; every block carries its
+ * own copy of the call count.
+ *   desc     : int32[n_blocks][8] {y_start (of the item), count, dist, p0_bits,
+ *                                  p1_bits, flags(bit0 scale, bit1 inc), seed, offset}
+ *   counters : int32[n_blocks], read and advanced by one per call (zero them to
  *              restart the streams) */
 #define NHIP_DIST_UNIFORM 0
 #define NHIP_DIST_GAUSSIAN 1
-int nhip_whitenoise(void *stream, const int *desc, int n_items, int *counters,
+int nhip_whitenoise(void *stream, const int *desc, int n_blocks, int *counters,
                     double sqrt_dt_inv, float *Y);
 /* out[t] = philox4x32_10(counter = in[t][0..3], key = in[t][4..5]) for n blocks
  * (known-answer testing of the generator). */

@@ -1,9 +1,9 @@
 // 2-D convolution / local filtering and average pooling of one image signal.
 //
 // Convolution: a group owns a tile of output pixels x a tile of filters.  For one
-// chunk of input channels at a time it stages the input patch under its pixels in
-// LDS, then every thread accumulates its (pixel, filter) output over the chunk's
-// channels and the kernel taps.  The accumulation order per output element is
+// chunk of input channels at a time it stages the input patch under its pixels and
+// the taps of its filters in LDS, then every thread accumulates its (pixel, filter)
+// output over the chunk's channels and the kernel taps from LDS alone.  The accumulation order per output element is
 // channel, kernel row, kernel column, one fused multiply-add each, as in the loop
 // of clra_nonlinearities.py:1812-1845; channel chunks are visited in order, so
 // chunking does not change it.  With channels last the filter index runs fastest
@@ -14,6 +14,9 @@
 namespace {
 
 #define NHIP_STREAM(s) static_cast<hipStream_t>(s)
+
+constexpr int STAGE_PF = 8;   // loads in flight per lane while staging the patch
+constexpr int FILT_PF = 16;   // ... and the filter taps
 
 struct ConvGeom {
     int nxi, nxj, nc, nyi, nyj, nf;
@@ -26,12 +29,20 @@ struct ConvGeom {
 
 __global__ __launch_bounds__(NHIP_WG) void conv2d_kernel(const ConvGeom g, const float* X,
                                                          const float* F, float* Y) {
-    extern __shared__ float patch[];  // [c_chunk][nipatch][njpatch]
+    // [c_chunk][nipatch][njpatch] input patch, then (convolution only) the filter taps
+    // of the group's filters [taps][channels of the chunk][tile_f], then the patch offset
+    // of every tap
+    extern __shared__ float lds[];
     const int tid = threadIdx.x;
     const int tile = blockIdx.x;
     const int i_base = (tile / g.tiles_j) * g.tile_i;
     const int j_base = (tile % g.tiles_j) * g.tile_j;
     const int k_base = blockIdx.y * g.tile_f;
+    const int npatch = g.nipatch * g.njpatch;
+    const int taps = g.si * g.sj;
+    float* patch = lds;
+    float* filt = patch + g.c_chunk * npatch;
+    int* tap_off = reinterpret_cast<int*>(filt + (g.local ? 0 : g.c_chunk * taps * g.tile_f));
 
     const int n_pix = g.tile_i * g.tile_j;
     int pix, kf;
@@ -49,45 +60,108 @@ __global__ __launch_bounds__(NHIP_WG) void conv2d_kernel(const ConvGeom g, const
 
     const int i0 = i_base * g.sti - g.pi;
     const int j0 = j_base * g.stj - g.pj;
-    const int npatch = g.nipatch * g.njpatch;
     const float* x = X + g.x_start;
     const float* f = F + g.f_start;
-    const int taps = g.si * g.sj;
+    for (int tap = tid; tap < taps; tap += NHIP_WG)
+        tap_off[tap] = (tap / g.sj) * g.njpatch + tap % g.sj;
 
     float out = 0.0f;
     for (int c0 = 0; c0 < g.nc; c0 += g.c_chunk) {
         const int cc = min(g.c_chunk, g.nc - c0);
-        for (int idx = tid; idx < cc * npatch; idx += NHIP_WG) {
-            int c, kij;
-            if (g.f_fast) {  // channels last: channel is the unit-stride axis of X
-                c = idx % cc;
-                kij = idx / cc;
-            } else {
-                kij = idx % npatch;
-                c = idx / npatch;
+        // staging: STAGE_PF independent global loads per lane are issued before the
+        // first of them is stored (few groups run, so nothing else hides the latency)
+        for (int base = tid; base < cc * npatch; base += NHIP_WG * STAGE_PF) {
+            float v[STAGE_PF];
+            int where[STAGE_PF];
+#pragma unroll
+            for (int u = 0; u < STAGE_PF; ++u) {
+                const int idx = base + u * NHIP_WG;
+                v[u] = 0.0f;
+                where[u] = -1;
+                if (idx < cc * npatch) {
+                    int c, kij;
+                    if (g.f_fast) {  // channels last: channel is the unit-stride axis of X
+                        c = idx % cc;
+                        kij = idx / cc;
+                    } else {
+                        kij = idx % npatch;
+                        c = idx / npatch;
+                    }
+                    const int ki = kij / g.njpatch, kj = kij - ki * g.njpatch;
+                    const int ii = i0 + ki, jj = j0 + kj;
+                    where[u] = c * npatch + kij;
+                    if (ii >= 0 && ii < g.nxi && jj >= 0 && jj < g.nxj)
+                        v[u] = x[(size_t)(c0 + c) * g.xs_c + (size_t)ii * g.xs_i +
+                                 (size_t)jj * g.xs_j];
+                }
             }
-            const int ki = kij / g.njpatch, kj = kij - ki * g.njpatch;
-            const int ii = i0 + ki, jj = j0 + kj;
-            float v = 0.0f;
-            if (ii >= 0 && ii < g.nxi && jj >= 0 && jj < g.nxj)
-                v = x[(size_t)(c0 + c) * g.xs_c + (size_t)ii * g.xs_i + (size_t)jj * g.xs_j];
-            patch[c * npatch + kij] = v;
+#pragma unroll
+            for (int u = 0; u < STAGE_PF; ++u)
+                if (where[u] >= 0) patch[where[u]] = v[u];
+        }
+        if (!g.local) {
+            // filters are (tap, channel, filter) in memory, filter index at unit stride;
+            // the LDS copy is [tap][channel of the chunk][filter of the tile].  All loads
+            // of a lane are in flight before the first is stored; tile_f is a power of two.
+            const int lg_f = __ffs(g.tile_f) - 1;
+            const int total = (taps * cc) << lg_f;
+            const float inv_cc = __frcp_rn((float)cc);
+            for (int base = tid; base < total; base += NHIP_WG * FILT_PF) {
+                float v[FILT_PF];
+#pragma unroll
+                for (int u = 0; u < FILT_PF; ++u) {
+                    const int idx = base + u * NHIP_WG;
+                    v[u] = 0.0f;
+                    if (idx < total) {
+                        const int q = idx & (g.tile_f - 1), r = idx >> lg_f;  // r = tap * cc + c
+                        int tap = (int)((float)r * inv_cc);
+                        if ((tap + 1) * cc <= r) ++tap;
+                        if (tap * cc > r) --tap;
+                        const int c = r - tap * cc;
+                        if (k_base + q < g.nf)
+                            v[u] = f[((size_t)tap * g.nc + (c0 + c)) * g.nf + k_base + q];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < FILT_PF; ++u)
+                    if (base + u * NHIP_WG < total) filt[base + u * NHIP_WG] = v[u];
+            }
         }
         __syncthreads();
         if (active) {
-            for (int c = 0; c < cc; ++c) {
-                const float* p = patch + c * npatch + (g.sti * ti) * g.njpatch + g.stj * tj;
-                const int ch = c0 + c;
-                for (int ii = 0; ii < g.si; ++ii) {
-                    for (int jj = 0; jj < g.sj; ++jj) {
-                        const int tap = ii * g.sj + jj;
-                        float w;
-                        if (g.local)
-                            w = f[((size_t)(k * g.nc + ch) * taps + tap) * (g.nyi * g.nyj) +
-                                  i * g.nyj + j];
-                        else
-                            w = f[((size_t)tap * g.nc + ch) * g.nf + k];
-                        out = fmaf(w, p[ii * g.njpatch + jj], out);
+            const float* p = patch + (g.sti * ti) * g.njpatch + g.stj * tj;
+            if (g.local) {
+                for (int c = 0; c < cc; ++c)
+                    for (int tap = 0; tap < taps; ++tap) {
+                        const float w = f[((size_t)(k * g.nc + c0 + c) * taps + tap) *
+                                              (g.nyi * g.nyj) + i * g.nyj + j];
+                        out = fmaf(w, p[c * npatch + tap_off[tap]], out);
+                    }
+            } else {
+                // A lane's output is one chain of fused multiply-adds in a fixed order, and
+                // small problems leave one wave per SIMD: the LDS reads of up to four
+                // taps of a kernel row are issued together, ahead of their chain links.
+                const float* w = filt + kf;
+                for (int c = 0; c < cc; ++c) {
+                    for (int ii = 0; ii < g.si; ++ii) {
+                        const float* pr = p + c * npatch + ii * g.njpatch;
+                        const float* wr = w + (ii * g.sj * cc + c) * g.tile_f;
+                        for (int jj = 0; jj < g.sj; jj += 4) {
+                            // no branches between the loads: past the row's end the last
+                            // tap is read again and its chain link discarded
+                            float pv[4], wv[4];
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                const int jq = min(jj + q, g.sj - 1);
+                                pv[q] = pr[jq];
+                                wv[q] = wr[jq * cc * g.tile_f];
+                            }
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                const float next = fmaf(wv[q], pv[q], out);
+                                out = (jj + q < g.sj) ? next : out;
+                            }
+                        }
                     }
                 }
             }
@@ -161,8 +235,10 @@ extern "C" int nhip_conv2d(void* stream, const int* geom, const float* X, const 
     g.njpatch = (g.tile_j - 1) * g.stj + g.sj;
     g.tiles_j = (g.nyj + g.tile_j - 1) / g.tile_j;
     const int tiles_i = (g.nyi + g.tile_i - 1) / g.tile_i;
-    const size_t lds = (size_t)g.c_chunk * g.nipatch * g.njpatch * sizeof(float);
-    if (lds > 48 * 1024) return NHIP_E_BADARG;
+    const size_t taps = (size_t)g.si * g.sj;
+    const size_t lds = ((size_t)g.c_chunk * (g.nipatch * g.njpatch + (g.local ? 0 : taps * g.tile_f)) +
+                        taps) * sizeof(float);
+    if (lds > 64 * 1024) return NHIP_E_BADARG;
     const dim3 grid(g.tiles_j * tiles_i, (g.nf + g.tile_f - 1) / g.tile_f);
     NHIP_LAUNCH(conv2d_kernel, grid, dim3(NHIP_WG), lds, NHIP_STREAM(stream), g, X, F, Y);
     NHIP_LAUNCH_CHECK();

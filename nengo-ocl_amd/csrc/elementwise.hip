@@ -60,13 +60,15 @@ __device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, flo
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const bool flat = (d.x_stride0 == d.shape1) && (d.y_stride0 == d.shape1);
+    const int i0 = d.offset / d.shape1, j0 = d.offset - i0 * d.shape1;  // once per block
     for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
         size_t xo, yo;
         if (flat) {
             xo = yo = (size_t)ij;
         } else {
-            const int i = ij / d.shape1, j = ij - i * d.shape1;
+            int i, j;
+            nhip_row_col(i0, j0, k, d.shape1, d.count, i, j);
             xo = (size_t)i * d.x_stride0 + j;
             yo = (size_t)i * d.y_stride0 + j;
         }
@@ -133,9 +135,10 @@ __device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const floa
     float* y = Y + d.y_start;
     const float alpha = nhip_bits(d.alpha_bits);
     const bool outer = d.flags & 1, inc = d.flags & 2;
+    const int i0 = d.offset / d.y_shape1, j0 = d.offset - i0 * d.y_shape1;  // once per block
     for (int k = lane; k < d.count; k += L) {
-        const int ij = d.offset + k;
-        const int i = ij / d.y_shape1, j = ij - i * d.y_shape1;
+        int i, j;
+        nhip_row_col(i0, j0, k, d.y_shape1, d.count, i, j);
         float aa, xx;
         if (outer) {
             aa = ew_element(a, d.a_shape0, 1, d.a_stride0, i, 0);
@@ -184,9 +187,11 @@ __device__ __forceinline__ void linearfilter_block(const LfDesc d, int2* pos, co
         ix = p.x;
         iy = p.y;
     }
+    const int i0 = d.offset / d.shape1, j0 = d.offset - i0 * d.shape1;  // once per block
     for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
-        const int i = ij / d.shape1, j = ij - i * d.shape1;
+        int i, j;
+        nhip_row_col(i0, j0, k, d.shape1, d.count, i, j);
         const size_t xij = (size_t)d.x_start + (size_t)i * d.x_stride0 + (size_t)j * d.x_stride1;
         const size_t yij = (size_t)d.y_start + (size_t)i * d.y_stride0 + (size_t)j * d.y_stride1;
         if (!general) {

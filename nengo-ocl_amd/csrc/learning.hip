@@ -32,9 +32,10 @@ __global__ __launch_bounds__(NHIP_WG) void learning_kernel(const LearnDesc* __re
     const float* post = POST + d.post_start;
     const float* aux = AUX + d.aux_start;
     float* delta = DELTA + d.delta_start;
+    const int i0 = d.offset / d.shape1, j0 = d.offset - i0 * d.shape1;  // once per block
     for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
-        const int ij = d.offset + k;
-        const int i = ij / d.shape1, j = ij - i * d.shape1;
+        int i, j;
+        nhip_row_col(i0, j0, k, d.shape1, d.count, i, j);
         const float x = pre[(size_t)j * d.pre_stride0];
         const float y = post[(size_t)i * d.post_stride0];
         float out;

@@ -50,3 +50,25 @@ __device__ __forceinline__ int nhip_xcd_remap(int bid, int n_groups) {
 }
 
 __device__ __forceinline__ float nhip_bits(int b) { return __int_as_float(b); }
+
+// Row and column of element `offset + k` of a row-major matrix with `cols` columns,
+// for the k-th element (k < count <= 8192) of a block that starts at row i0, column j0
+// (= offset / cols, offset % cols, formed once per block on the scalar unit).  An
+// integer division per element costs more instructions than the rest of a streaming
+// kernel's loop body: here it is a comparison when a block is no longer than a row,
+// and otherwise (cols < count <= 8192) a float reciprocal with a correction step, exact
+// for these magnitudes.
+__device__ __forceinline__ void nhip_row_col(int i0, int j0, int k, int cols, int count, int& i,
+                                             int& j) {
+    const int t = j0 + k;  // < cols + count
+    int q;
+    if (cols >= count) {   // uniform over the block
+        q = t >= cols ? 1 : 0;
+    } else {
+        q = (int)((float)t * __frcp_rn((float)cols));
+        if ((q + 1) * cols <= t) ++q;
+        if (q * cols > t) --q;
+    }
+    i = i0 + q;
+    j = t - q * cols;
+}

@@ -3,9 +3,10 @@
 // memory (clra_nonlinearities.py:1486-1675); here the generator is the counter-based
 // Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3",
 // SC'11): sample (item, call n, element i) is a pure function of the item's seed
-// and (n, i), so the only state is one call counter per item, no two lanes share
-// generator state, and a signal of any length is filled by as many lanes as it has
-// elements.
+// and (n, i), so the only state is a call counter, no two lanes share generator
+// state, and a signal of any length is filled by as many lanes as it has elements:
+// an item is cut into blocks (rows of the work list), one group each, and every
+// block keeps its own copy of the call counter, which it alone reads and advances.
 //
 // Block of four 32-bit words for elements 4q..4q+3 of call n of an item:
 //     philox4x32_10(counter = {q, n, 0, 0}, key = {seed, 0})
@@ -20,8 +21,8 @@ namespace {
 #define NHIP_STREAM(s) static_cast<hipStream_t>(s)
 
 struct NoiseDesc {
-    int y_start, count, dist, p0_bits;
-    int p1_bits, flags, seed, pad;
+    int y_start, count, dist, p0_bits;   // y_start: of the item; count: elements of the block
+    int p1_bits, flags, seed, offset;    // offset: first element of the block (a multiple of 4)
 };
 
 __device__ __forceinline__ void philox_round(unsigned (&c)[4], unsigned k0, unsigned k1) {
@@ -43,8 +44,8 @@ __device__ __forceinline__ void philox4x32_10(unsigned (&c)[4], unsigned k0, uns
     }
 }
 
-// One group per item (a strided loop over its elements), so that the group can read
-// the item's call counter, use it, and advance it without another group racing.
+// One group per block: it reads the block's call counter, uses it, and advances it
+// without another group racing.
 __global__ __launch_bounds__(NHIP_WG) void whitenoise_kernel(const NoiseDesc* __restrict__ desc,
                                                              int* counters, double sqrt_dt_inv,
                                                              float* Y) {
@@ -53,7 +54,8 @@ __global__ __launch_bounds__(NHIP_WG) void whitenoise_kernel(const NoiseDesc* __
     __syncthreads();
     float* y = Y + d.y_start;
     const float p0 = nhip_bits(d.p0_bits), p1 = nhip_bits(d.p1_bits);
-    for (int i = threadIdx.x; i < d.count; i += NHIP_WG) {
+    for (int k = threadIdx.x; k < d.count; k += NHIP_WG) {
+        const int i = d.offset + k;  // element of the item
         unsigned c[4] = {(unsigned)(i >> 2), call, 0u, 0u};
         philox4x32_10(c, (unsigned)d.seed, 0u);
         const int lane = i & 3;
@@ -86,11 +88,11 @@ __global__ void philox_test_kernel(const unsigned* in, unsigned* out, int n) {
 
 }  // namespace
 
-extern "C" int nhip_whitenoise(void* stream, const int* desc, int n_items, int* counters,
+extern "C" int nhip_whitenoise(void* stream, const int* desc, int n_blocks, int* counters,
                                double sqrt_dt_inv, float* Y) {
-    if (n_items == 0) return 0;
-    if (n_items < 0 || !desc || !counters || !Y) return NHIP_E_BADARG;
-    NHIP_LAUNCH(whitenoise_kernel, dim3(n_items), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+    if (n_blocks == 0) return 0;
+    if (n_blocks < 0 || !desc || !counters || !Y) return NHIP_E_BADARG;
+    NHIP_LAUNCH(whitenoise_kernel, dim3(n_blocks), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
                        reinterpret_cast<const NoiseDesc*>(desc), counters, sqrt_dt_inv, Y);
     NHIP_LAUNCH_CHECK();
     return 0;

@@ -834,9 +834,10 @@ def conv2d_tiles(shape_out_ijf, kernel_shape, strides, nc, channels_last):
         tile_j *= 2
     tile_j = min(tile_j, 32)
     tile_i = max(1, min(WG // (tile_j * tile_f), nyi))
-    patch = ((tile_i - 1) * sti + si) * ((tile_j - 1) * stj + sj)
-    c_chunk = max(1, min(nc, (32 * 1024 // 4) // patch))
-    assert patch * 4 <= 48 * 1024, "convolution window too large for one LDS patch"
+    # LDS words per staged channel: the input patch and the taps of the group's filters
+    per_channel = ((tile_i - 1) * sti + si) * ((tile_j - 1) * stj + sj) + si * sj * tile_f
+    c_chunk = max(1, min(nc, (32 * 1024 // 4) // per_channel))
+    assert (per_channel + si * sj) * 4 <= 60 * 1024, "convolution window too large for LDS"
     return tile_i, tile_j, tile_f, c_chunk
 
 
@@ -937,11 +938,12 @@ def plan_whitenoise(queue, Y, dist_enums, dist_params, scale, inc, dt, seeds, ta
     assert (Y.shape1s == 1).all() and (Y.stride0s == 1).all() and (Y.stride1s == 1).all()
     assert Y.ctype == "float"
     _check(("Y", Y))
+    inds, offsets, counts = blockify(Y.shape0s, 4 * BLOCK)  # blocks start at multiples of 4
+    flags = scale.astype(np.int32) | (inc.astype(np.int32) << 1)
     table, n = _dev_table(queue, [
-        Y.starts, Y.shape0s, enums, _bits(params[:, 0]), _bits(params[:, 1]),
-        scale.astype(np.int32) | (inc.astype(np.int32) << 1),
-        (seeds & 0xFFFFFFFF).astype(np.uint32).view(np.int32)], 8)
-    counters = to_device(queue, np.zeros(max(N, 1), dtype=np.int32))
+        Y.starts[inds], counts, enums[inds], _bits(params[inds, 0]), _bits(params[inds, 1]),
+        flags[inds], (seeds & 0xFFFFFFFF).astype(np.uint32).view(np.int32)[inds], offsets], 8)
+    counters = to_device(queue, np.zeros(max(n, 1), dtype=np.int32))  # one per block
     plan = Plan(queue, queue.lib.nhip_whitenoise,
                 (table.ptr, n, counters.ptr, 1.0 / np.sqrt(dt), Y.ptr),
                 gsize=(WG * max(n, 1),), lsize=(WG,), full_args=(table, counters, Y.dev_buf),
