@@ -362,6 +362,74 @@ def neurons_read_constant_input(operators, keep=()):
     return [replace.get(op, op) for op in operators if op not in drop]
 
 
+def propagate_vector_copies(operators, keep=()):
+    """Vectors that are only ever a copy of another vector are not copied: their readers
+    read the source.
+
+    After `fuse_into_multidotinc` and `MultiDotInc.compress`, ``Reset(y); Copy(x -> y,
+    inc=True)`` -- what a passthrough node or an ensemble with a single unweighted input
+    leaves in the graph -- is one operator ``y = 0*y + 0 + 1*x``.  When that operator is
+    the only writer of ``y``, ``y`` is a whole signal that is not in `keep` (probed
+    signals), and every reader of ``y`` is a MultiDotInc that uses it as a vector
+    operand, those readers take ``x`` instead and the copy goes away: one launch less per
+    link of such a chain (the reference runs each link as a GEMV of its own,
+    simulator.py:746-816).  The planner orders the readers after the writers of ``x``
+    and before its updates, which is when the copy read it.  Values are unchanged except
+    that a copy turns -0.0 into +0.0, so a sum downstream may be -0.0 where it was +0.0.
+    The copied signal is no longer part of the simulation (``sim.signals`` does not hold
+    it), like the signals the reference's own simplifications remove.  The operators
+    passed in are left as they are (readers are replaced by modified copies), so that the
+    caller can keep the original list if the rewritten one does not plan better.
+    """
+    import copy as _copy
+
+    keep_bases = {sig.base for sig in keep}
+    ops = list(operators)
+    # positions of the operators that write / read each base signal; kept current while
+    # readers are redirected (a dropped operator leaves None at its position)
+    writers, readers = {}, {}
+    for pos, op in enumerate(ops):
+        for sig in list(op.sets) + list(op.incs) + list(op.updates):
+            writers.setdefault(sig.base, []).append(pos)
+        for sig in op.reads:
+            readers.setdefault(sig.base, []).append(pos)
+    mine = set()  # positions holding copies made here (safe to modify)
+
+    for pos in range(len(ops)):
+        op = ops[pos]
+        if not isinstance(op, MultiDotInc):
+            continue
+        if (op._incs_Y or op._signal_beta is not None or op._float_beta != 0 or op.gamma != 0
+                or len(op.As) != 1):
+            continue
+        A, X, Y = op.As[0], op.Xs[0], op.Y
+        base = Y.base
+        if (getattr(Y, "is_view", False) or base in keep_bases or X.shape != Y.shape
+                or X.base is base or A.size != 1 or not getattr(A, "readonly", False)
+                or writers.get(A.base) or float(np.asarray(A.initial_value).ravel()[0]) != 1.0):
+            continue
+        if writers.get(base) != [pos]:
+            continue
+        users = sorted({q for q in readers.get(base, []) if q != pos and ops[q] is not None})
+        if not users or not all(
+                isinstance(ops[q], MultiDotInc) and any(x is Y for x in ops[q].Xs)
+                and all(a is not Y for a in ops[q].As) and ops[q].Y_in is not Y
+                and ops[q]._signal_beta is not Y for q in users):
+            continue
+        for q in users:
+            if q not in mine:
+                new = _copy.copy(ops[q])
+                new.As, new.Xs = list(new.As), list(new.Xs)
+                ops[q] = new
+                mine.add(q)
+            ops[q].Xs = [X if x is Y else x for x in ops[q].Xs]
+            readers.setdefault(X.base, []).append(q)
+        ops[pos] = None
+        writers[base] = []
+        readers[base] = []
+    return [op for op in ops if op is not None]
+
+
 LEARNING_RULES = ("SimPES", "SimBCM", "SimOja", "SimVoja")
 
 

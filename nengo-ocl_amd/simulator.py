@@ -266,6 +266,15 @@ class Simulator:
                 operators = ops_mod.apply_learning_in_place(operators, keep=probed)
         operators = MultiDotInc.compress(operators)
         op_groups = planner(operators)
+        if fuse:
+            # cutting vector copies out of the graph saves launches in chains of small
+            # operators, but it can also split a group of like operators whose members no
+            # longer depend on the same things: keep it only where the step gets shorter
+            shorter = ops_mod.propagate_vector_copies(operators, keep=probed)
+            if len(shorter) < len(operators):
+                shorter_groups = planner(shorter)
+                if len(shorter_groups) < len(op_groups):
+                    operators, op_groups = shorter, shorter_groups
         assert len([t for t, _ in op_groups if t.__name__ == "Reset"]) < 2, \
             "All resets not planned together"
         self.operators = operators

@@ -351,3 +351,60 @@ def test_neurons_without_input_read_their_bias():
     for a, b in zip(probes, probes2):
         assert np.array_equal(plain.data[a], fused.data[b])
     assert plain.data[probes[1]].sum() > 0
+
+
+def test_vector_copies_are_propagated():
+    """Chains of vector copies (passthrough nodes, ensembles with one unweighted input) are
+    cut out of the step: the readers take the source, probe data stay equal to the
+    unfused simulator's (a copy's only effect, -0.0 -> +0.0, compares equal), and copies
+    that are probed, partial, weighted or read by other operators stay."""
+    from nengo_ocl_amd.operators import MultiDotInc, propagate_vector_copies
+
+    def is_copy(op):
+        return (isinstance(op, MultiDotInc) and not op._incs_Y and op._float_beta == 0
+                and op.gamma == 0 and len(op.As) == 1 and op.As[0].size == 1)
+
+    for make, steps in ((lambda: configs.c1_circconv(dims=8, n_per_dim=30), 300),
+                        (lambda: configs.c0_readme(n_neurons=50), 300)):
+        sims = []
+        for fuse in (True, False):
+            net, probes, _ = make()
+            sim = OracleSimulator(net, seed=1, fuse=fuse)
+            sim.run_steps(steps)
+            sims.append((sim, probes))
+        (fused, pf), (plain, pp) = sims
+        for k in pf:
+            assert np.array_equal(fused.data[pf[k]], plain.data[pp[k]])
+        # what is left of the copies in the fused graph is read by something other than a GEMV
+        # (probes) or not a whole signal
+        for op in fused.operators:
+            if is_copy(op) and not op.Y.is_view and op.Xs[0].shape == op.Y.shape:
+                users = [r for r in fused.operators if r is not op and any(s.base is op.Y.base for s in r.reads)]
+                assert not users or not all(isinstance(r, MultiDotInc) for r in users)
+
+    # unit cases on a hand-made graph: y = x feeds z = A @ y; a probed copy stays
+    one = ir.Signal(np.array(1.0), name="one", readonly=True)
+    x = ir.Signal(np.ones(3), name="x")
+    y = ir.Signal(np.zeros(3), name="y")
+    z = ir.Signal(np.zeros(2), name="z")
+    A = ir.Signal(np.ones((2, 3)), name="A", readonly=True)
+
+    def graph():
+        copy = MultiDotInc(y, y, beta=0, gamma=0)
+        copy.add_AX(one, x)
+        user = MultiDotInc(z, z, beta=0, gamma=0)
+        user.add_AX(A, y)
+        return [copy, user]
+
+    ops = propagate_vector_copies(graph())
+    assert len(ops) == 1 and ops[0].Xs == [x]
+    assert len(propagate_vector_copies(graph(), keep=[y])) == 2       # probed
+    ops = graph()
+    ops[0].gamma = 0.5                                                # not a plain copy
+    assert len(propagate_vector_copies(ops)) == 2
+    ops = graph() + [ir.Copy(y, ir.Signal(np.zeros(3), name="w"))]    # another kind of reader
+    assert len(propagate_vector_copies(ops)) == 3
+    two = ir.Signal(np.array(2.0), name="two", readonly=True)
+    ops = graph()
+    ops[0].As = [two]                                                 # a scaled copy
+    assert len(propagate_vector_copies(ops)) == 2
