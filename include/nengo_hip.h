@@ -138,7 +138,11 @@ int nhip_gemv_tile_lif(void *stream, int vec, int pow2_cols, int blk_words, cons
  *   targets      : int32[n][4] {y_start, a0 bits, b0 bits, na}
  *   F[y_start + r] = b0 * y - a0 * F[y_start + r]   (na == 1)   or   b0 * y   (na == 0)
  * Y is still written.  The filter outputs must not overlap anything the launch reads
- * through A, X or Yin.  Results are bit-identical to the two separate calls. */
+ * through A, X or Yin.  Results are bit-identical to the two separate calls.
+ * The kernels of this entry point read an item's range of targets from its task
+ * records, so that a wave needs no further read before it can start: tasks[t][3] =
+ * first target and tasks[t][11] = number of targets of the task's item, i.e. the
+ * item's row of `item_targets` (which nhip_gemv_rows_filter reads). */
 int nhip_gemv_tile_filter(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
                           const float *coefs, const int *dots, const int *tasks, int n_tasks,
                           const float *A, const float *X, const float *Yin, float *Y,

@@ -317,7 +317,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     LifPop pop = {};
     int2 filters = make_int2(0, 0);
     if (EPI == EPI_LIF) pop = epi.lif.pops[task.item];
-    if (EPI == EPI_FILTER) filters = epi.filter.item_targets[task.item];
+    if (EPI == EPI_FILTER) filters = make_int2(task.pad, it.pad);  // rides in the task record
     // an item without dot products that would copy Y onto itself unchanged is only
     // there for its epilogue (a constant input current): nothing to store
     const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
@@ -447,6 +447,7 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
 
 constexpr int P2_PF = 8;         // 16-byte loads per lane and block
 constexpr int YSUM_WORDS = 256;  // running sums of the task's rows, in LDS
+constexpr int F_SLOTS = 2;       // (filter target, row) pairs per lane whose old values are fetched ahead
 
 __device__ __forceinline__ float quad_xor(float v, int ctrl_sel) {
     // lanes exchange inside groups of four: xor 2 = [2,3,0,1], xor 1 = [1,0,3,2]
@@ -454,6 +455,66 @@ __device__ __forceinline__ float quad_xor(float v, int ctrl_sel) {
         ? __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true)
         : __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true);
     return __int_as_float(r);
+}
+
+// What a task does with its finished sums `ys` (row r of the task at ys[r], gamma not
+// yet added): store them, and run the launch's epilogue on them.  `block` is the
+// wave's LDS block, free by now.
+struct FilterPrefetch {
+    int2 range;                    // the item's {first target, number of targets}
+    int n_pairs;                   // (target, row) pairs of the task
+    FilterTarget target[F_SLOTS];  // this lane's pairs: target record, row, old filter value
+    int row[F_SLOTS];
+    float old[F_SLOTS];
+};
+
+template <int EPI>
+__device__ __forceinline__ void finish_task(const GemvTask& task, const GemvItem& it,
+                                            const float4& cf, const float* ys, float* ab,
+                                            const float* Yin, float* Y, const EpilogueArgs& epi,
+                                            const LifPop& pop, const float (&v_in)[ROW_SLOTS],
+                                            const float (&w_in)[ROW_SLOTS],
+                                            const FilterPrefetch& fp, int lane) {
+    const int n_rows = task.n_rows;
+    const int2 filters = fp.range;
+    const int n_pairs = fp.n_pairs;
+    wave_sync();
+    // an item without dot products that would copy Y onto itself unchanged is only
+    // there for its epilogue (a constant input current): nothing to store
+    const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
+                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
+    if (EPI == EPI_LIF && (pop.pflags & LIF_POP_DECAY)) {
+        lif_task_compacted(epi.lif, pop, task.row0, n_rows, ys, cf.z,
+                           store_y ? Y + it.y_start : nullptr, it.y_stride0, ab, lane, v_in, w_in);
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
+        const int r = lane + k * NHIP_WAVE;
+        if (r < n_rows) {
+            const float y = ys[r] + cf.z;
+            if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
+            if (EPI == EPI_LIF && (pop.pflags & LIF_POP_ENABLED))
+                lif_epilogue(epi.lif, pop, task.row0 + r, y, v_in[k], w_in[k]);
+        }
+    }
+    if (EPI == EPI_FILTER) {
+        // y = b0 x - a0 y, or y = b0 x: the arithmetic of filter_epilogue
+        auto step = [&](const FilterTarget& t, int r, float old_value) {
+            const float bx = __fmul_rn(nhip_bits(t.b_bits), ys[r] + cf.z);
+            epi.filter.F[(size_t)t.y_start + task.row0 + r] =
+                t.na ? __fsub_rn(bx, __fmul_rn(nhip_bits(t.a_bits), old_value)) : bx;
+        };
+#pragma unroll
+        for (int k = 0; k < F_SLOTS; ++k)
+            if (lane + k * NHIP_WAVE < n_pairs) step(fp.target[k], fp.row[k], fp.old[k]);
+        for (int e = lane + F_SLOTS * NHIP_WAVE; e < n_pairs; e += NHIP_WAVE) {
+            const int q = small_div(e, n_rows);
+            const int r = e - q * n_rows;
+            const FilterTarget t = epi.filter.targets[filters.x + q];
+            step(t, r, epi.filter.F[(size_t)t.y_start + task.row0 + r]);
+        }
+    }
 }
 
 struct P2Stage {
@@ -489,28 +550,36 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     const float4 cf = make_float4(ft.alpha, ft.beta, ft.gamma, 0.0f);
     const int n_rows = task.n_rows;
 
+    // The old Y values are requested now and used once the first matrix loads have
+    // been issued.  A lane without a row reads the task's last row: loads without a
+    // branch around them do not make the compiler wait for each one before it issues
+    // the next.
+    float y_old[ROW_SLOTS];
 #pragma unroll
-    for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
-        const int r = lane + k * NHIP_WAVE;
-        if (r < n_rows)
-            ys[r] = cf.y * Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0];
+    for (int k = 0; k < ROW_SLOTS; ++k) {
+        const int r = min(lane + k * NHIP_WAVE, n_rows - 1);
+        y_old[k] = Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0];
     }
-    // What the epilogue will need of the item besides its sums is requested now, so
-    // that it has arrived when the last block is done (read at the end, these loads
-    // would stall the wave for a memory round trip with nothing else in flight).
-    LifPop pop = {};
-    float v_in[ROW_SLOTS] = {}, w_in[ROW_SLOTS] = {};
-    if (EPI == EPI_LIF) {
-        pop = epi.lif.pops[task.item];
-        if (pop.pflags & LIF_POP_ENABLED) {
+
+    // Filter epilogue: the task's (target, row) pairs are spread over the lanes, and
+    // each lane's target record is requested now; the old filter values follow once
+    // the first matrix loads are on their way.  Pairs beyond F_SLOTS * 64 are read at
+    // the end instead.
+    int2 filters = make_int2(0, 0);
+    int n_pairs = 0;
+    FilterTarget f_target[F_SLOTS];
+    float f_old[F_SLOTS];
+    int f_row[F_SLOTS];
+    if (EPI == EPI_FILTER) {
+        filters = make_int2(task.pad, it.pad);  // the item's range of targets rides in the task record
+        n_pairs = filters.y * n_rows;
+        // no branch around the loads: an item without targets reads the table's first record
 #pragma unroll
-            for (int k = 0; k < ROW_SLOTS; ++k) {
-                const int r = lane + k * NHIP_WAVE;
-                if (r < n_rows) {
-                    v_in[k] = epi.lif.V[(size_t)pop.v_start + task.row0 + r];
-                    w_in[k] = epi.lif.W[(size_t)pop.w_start + task.row0 + r];
-                }
-            }
+        for (int k = 0; k < F_SLOTS; ++k) {
+            const int e = max(0, min(lane + k * NHIP_WAVE, n_pairs - 1));
+            const int q = small_div(e, n_rows);
+            f_row[k] = e - q * n_rows;
+            f_target[k] = epi.filter.targets[filters.x + q];
         }
     }
 
@@ -519,7 +588,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
         s.d = it.n_dots > 0 ? 0 : -1;
         s.c0 = 0;
         s.b = 0;
-        if (s.d >= 0) s.dot = ft.dot0;
+        s.dot = ft.dot0;  // all zero for an item without dot products
         return s;
     };
     auto next_stage = [&](const P2Stage& s) {
@@ -545,7 +614,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
 #define P2_GEOMETRY(s)                                                              \
     const int lgn = (s).dot.p1;                                                     \
     const int lgc = lgn < 9 ? lgn : 9;               /* log2 columns of the stage */ \
-    const int lgq = lgc - 2 < 6 ? lgc - 2 : 6;                                      \
+    const int lgq = lgc < 2 ? 0 : lgc - 2 < 6 ? lgc - 2 : 6;  /* (< 2: no stage) */  \
     const int lg_lpr = lgc - 2 - lgq;                                               \
     const int rpl = NHIP_WAVE >> lgq;                                               \
     const int lgt = lgc > 7 ? lgc - 7 : 0;           /* log2 tiles of the stage */  \
@@ -555,33 +624,41 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     const int lane_r = lane >> lgq;                                                 \
     const int lane_q = lane & ((1 << lgq) - 1);
 
+    // Every call issues exactly P2_PF vector loads of the matrix, whatever the stage
+    // looks like (a lane without an element of its own reads the block's first
+    // bytes instead, and so does every lane when the stage does not exist: then that
+    // is the first block of the task's last dot product): the
+    // compiler can then count how many loads are younger than the ones a block
+    // waits for, and waits for the older register set only, with the younger one
+    // still in flight.  Loads under a branch would make it wait for everything.
+    // The same holds for the X loads: always X_PF of them, from the stage's first
+    // element where a lane has nothing to fetch.
     auto load_stage = [&](tile_f4 (&pf)[P2_PF], float (&xq)[X_PF], const P2Stage& s) {
         P2_GEOMETRY(s)
         (void)lgt; (void)roww;
+        const bool exists = s.d >= 0;
+        {   // the gathered X of a column stage travels with the stage's first row block
+            const int ncs = (exists && s.b == 0) ? 1 << lgc : 0;
+            const float* xg = X + s.dot.x_start + (size_t)s.c0 * s.dot.x_stride0;
+            const int lane_x = lane * s.dot.x_stride0;
+#pragma unroll
+            for (int i = 0; i < X_PF; ++i) {
+                const float* p = xg + (size_t)i * NHIP_WAVE * s.dot.x_stride0 + lane_x;
+                xq[i] = *(lane + i * NHIP_WAVE < ncs ? p : xg);
+            }
+        }
         const char* base = reinterpret_cast<const char*>(
             A + s.dot.a_start + (size_t)(task.row0 + s.b * rb) * s.dot.a_stride0 + s.c0);
+        const char* safe = base;  // a line this wave reads anyway, not one all waves would share
         const unsigned lane_off = 4u * (unsigned)(lane_r * s.dot.a_stride0 + 4 * lane_q);
         const size_t load_pitch = (size_t)rpl * s.dot.a_stride0 * 4u;  // bytes between loads
+        const int my_rows = exists ? rows - lane_r : 0;  // loads with ri < my_rows are this lane's
 #pragma unroll
         for (int i = 0; i < P2_PF; ++i) {
             const int ri = (i >> lg_lpr) * rpl;                  // uniform
             const int part = i & ((1 << lg_lpr) - 1);            // uniform: which 256 columns
-            if (ri < rows) {                                     // uniform
-                if (ri + lane_r < rows)
-                    pf[i] = load_nt4(reinterpret_cast<const float*>(
-                        base + ((size_t)(i >> lg_lpr) * load_pitch + (size_t)part * 1024u) + lane_off));
-            }
-        }
-        if (s.b == 0) {  // first row block of a column stage: its gathered X travels along
-            const int ncs = 1 << lgc;
-            const float* xg = X + s.dot.x_start + (size_t)s.c0 * s.dot.x_stride0;
-            const int lane_x = lane * s.dot.x_stride0;
-#pragma unroll
-            for (int i = 0; i < X_PF; ++i)
-                if (i * NHIP_WAVE < ncs) {                       // uniform
-                    if (lane + i * NHIP_WAVE < ncs)
-                        xq[i] = xg[(size_t)i * NHIP_WAVE * s.dot.x_stride0 + lane_x];
-                }
+            const char* p = base + ((size_t)(i >> lg_lpr) * load_pitch + (size_t)part * 1024u) + lane_off;
+            pf[i] = load_nt4(reinterpret_cast<const float*>(ri < my_rows ? p : safe));
         }
     };
 
@@ -653,50 +730,346 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
     tile_f4 pf0[P2_PF], pf1[P2_PF];
     float xq0[X_PF], xq1[X_PF];
 #pragma unroll
-    for (int i = 0; i < P2_PF; ++i) pf0[i] = pf1[i] = tile_f4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
     for (int i = 0; i < X_PF; ++i) xq0[i] = xq1[i] = 0.0f;
     P2Stage sa = first_stage();
     P2Stage sb = next_stage(sa);
-    if (sa.d >= 0) load_stage(pf0, xq0, sa);
-    if (sb.d >= 0) load_stage(pf1, xq1, sb);
-    while (sa.d >= 0) {
-        store_stage(pf0, xq0, sa);
-        const P2Stage sc = next_stage(sb);
-        if (sc.d >= 0) load_stage(pf0, xq0, sc);
-        sum_stage(sa);
-        if (sb.d < 0) break;
-        store_stage(pf1, xq1, sb);
-        const P2Stage sd = next_stage(sc);
-        if (sd.d >= 0) load_stage(pf1, xq1, sd);
-        sum_stage(sb);
-        sa = sc;
-        sb = sd;
-    }
-
-    wave_sync();
-    int2 filters = make_int2(0, 0);
-    if (EPI == EPI_FILTER) filters = epi.filter.item_targets[task.item];
-    // an item without dot products that would copy Y onto itself unchanged is only
-    // there for its epilogue (a constant input current): nothing to store
-    const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
-                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
-    if (EPI == EPI_LIF && (pop.pflags & LIF_POP_DECAY)) {
-        lif_task_compacted(epi.lif, pop, task.row0, n_rows, ys, cf.z,
-                           store_y ? Y + it.y_start : nullptr, it.y_stride0, ab, lane, v_in, w_in);
-        return;
+    load_stage(pf0, xq0, sa);
+    load_stage(pf1, xq1, sb);
+    // What the epilogue will need of the item besides its sums is requested now, so
+    // that it has arrived when the last block is done (read at the end, these loads
+    // would stall the wave for a memory round trip with nothing else in flight; read
+    // before the matrix loads, the population record would hold those back).
+    LifPop pop = {};
+    float v_in[ROW_SLOTS] = {}, w_in[ROW_SLOTS] = {};
+    if (EPI == EPI_LIF) {
+        pop = epi.lif.pops[task.item];
+        if (pop.pflags & LIF_POP_ENABLED) {
+#pragma unroll
+            for (int k = 0; k < ROW_SLOTS; ++k) {
+                const int r = min(lane + k * NHIP_WAVE, n_rows - 1);
+                v_in[k] = epi.lif.V[(size_t)pop.v_start + task.row0 + r];
+                w_in[k] = epi.lif.W[(size_t)pop.w_start + task.row0 + r];
+            }
+        }
     }
 #pragma unroll
     for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
         const int r = lane + k * NHIP_WAVE;
-        if (r < n_rows) {
-            const float y = ys[r] + cf.z;
-            if (store_y) Y[it.y_start + (size_t)(task.row0 + r) * it.y_stride0] = y;
-            if (EPI == EPI_LIF && (pop.pflags & LIF_POP_ENABLED))
-                lif_epilogue(epi.lif, pop, task.row0 + r, y, v_in[k], w_in[k]);
-            if (EPI == EPI_FILTER) filter_epilogue(epi.filter, filters, task.row0 + r, y);
+        if (r < n_rows) ys[r] = cf.y * y_old[k];
+    }
+    if (EPI == EPI_FILTER) {
+#pragma unroll
+        for (int k = 0; k < F_SLOTS; ++k)
+            f_old[k] = epi.filter.F[(size_t)f_target[k].y_start + (n_pairs > 0 ? task.row0 + f_row[k] : 0)];
+    }
+    // no way out of the middle of the loop: with one, the compiler no longer sees
+    // that a register set always has the other set's loads behind it
+    while (sa.d >= 0) {
+        store_stage(pf0, xq0, sa);
+        const P2Stage sc = next_stage(sb);
+        load_stage(pf0, xq0, sc);
+        sum_stage(sa);
+        const P2Stage sd = next_stage(sc);
+        if (sb.d >= 0) store_stage(pf1, xq1, sb);
+        load_stage(pf1, xq1, sd);
+        if (sb.d >= 0) sum_stage(sb);
+        sa = sc;
+        sb = sd;
+    }
+
+    FilterPrefetch fp;
+    fp.range = filters;
+    fp.n_pairs = n_pairs;
+#pragma unroll
+    for (int k = 0; k < F_SLOTS; ++k) {
+        fp.target[k] = f_target[k];
+        fp.row[k] = f_row[k];
+        fp.old[k] = f_old[k];
+    }
+    finish_task<EPI>(task, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
+}
+
+
+// ---------------------------------------------------------------------------
+// The streamlined kernel once more, with the shape of a dot product known at compile
+// time.  The kernels above spend several hundred scalar and vector instructions per
+// 8 KiB block on bookkeeping (the shape of every stage is worked out again from the
+// dot record, every load has its own 64-bit address arithmetic and predicate), and
+// with three or four waves per SIMD that, not HBM, is what bounds them.  Here the
+// column count of a stage is a template parameter (32, 64, or 512 for every power
+// of two from 512 up): all LDS addresses are immediates, a block's loads share one
+// scalar base and per-lane offsets that are set up once per dot product, tile sums
+// go from the lanes that hold them straight onto the running row sums, and the loop
+// over the stages of a dot product is written so that the loads of the register set
+// that is NOT being waited for are never under a branch (the compiler then waits for
+// the older set only).  Same sums in the same order: bit-identical results.
+template <int LGC>
+struct StreamGeo {
+    static constexpr int LG_COLS = LGC;
+    static constexpr int NCS = 1 << LGC;                    // columns of a stage
+    static constexpr int LGQ = LGC - 2 < 6 ? LGC - 2 : 6;   // log2 of the lanes side by side in a row
+    static constexpr int LG_LPR = LGC - 2 - LGQ;            // log2 of the loads that cover a row
+    static constexpr int RPL = NHIP_WAVE >> LGQ;            // rows one load instruction covers
+    static constexpr int LGT = LGC > 7 ? LGC - 7 : 0;       // log2 of the tiles of a stage
+    static constexpr int TILES = 1 << LGT;
+    static constexpr int ROWW = LGC >= 7 ? (TILE_LDS << LGT) : NCS + 4;  // LDS words of a row
+    static constexpr int RB = LGC >= 7 ? 16 >> LGT : 32;    // rows of a block
+    static constexpr int NL = (RB / RPL) << LG_LPR;         // loads per lane and block
+    static constexpr int CHAIN = LGC >= 7 ? MAX_CHAIN : NCS / 4;  // elements of a partial sum
+    static constexpr int XL = NCS >= NHIP_WAVE ? NCS / NHIP_WAVE : 1;  // X loads per lane and stage
+    static constexpr bool WIDE = LGC >= 9;                  // several column stages: X travels with them
+    static constexpr int PASSES = (RB * TILES + 15) / 16;   // (row, tile) pairs come 16 at a time
+    static constexpr int PASS_WORDS = (16 >> LGT) * ROWW;
+    static_assert(NL >= 1 && NL <= P2_PF && RB * ROWW <= 2176 && RB * TILES <= TSUM_WORDS, "block shape");
+};
+
+constexpr int STREAM_BLK_WORDS = 2176;  // the LDS block these shapes are made for
+
+// lane i receives the value of lane i + n of its row of 16 lanes
+template <int N>
+__device__ __forceinline__ float row_from_right(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x100 + N, 0xF, 0xF, true));
+}
+
+template <int EPI>
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4))) void gemv_stream_kernel(
+    const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
+    int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
+    float* Y, EpilogueArgs epi)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float* ab = lds + wave * (STREAM_BLK_WORDS + xb_words + YSUM_WORDS);  // the wave's block
+    float* xb = ab + STREAM_BLK_WORDS;  // gathered X of the current column stage, tiles padded
+    float* ys = xb + xb_words;          // running sum of row r of the task
+
+    const int t = nhip_xcd_remap(blockIdx.x, gridDim.x) * (NHIP_WG / NHIP_WAVE) + wave;
+    if (t >= n_tasks) return;  // wave-uniform; the kernel has no group barrier
+
+    const GemvFatTask ft = tasks[t];
+    const GemvTask task = ft.task;
+    const GemvItem it = ft.item;
+    const float4 cf = make_float4(ft.alpha, ft.beta, ft.gamma, 0.0f);
+    const int n_rows = task.n_rows;
+
+    // old Y values and the filter targets: requested now, used after the first matrix
+    // loads have been issued (no branch around the loads, see gemv_tile_p2_kernel)
+    float y_old[ROW_SLOTS];
+#pragma unroll
+    for (int k = 0; k < ROW_SLOTS; ++k) {
+        const int r = min(lane + k * NHIP_WAVE, n_rows - 1);
+        y_old[k] = Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0];
+    }
+    FilterPrefetch fp;
+    fp.range = make_int2(0, 0);
+    fp.n_pairs = 0;
+    if (EPI == EPI_FILTER) {
+        fp.range = make_int2(task.pad, it.pad);  // rides in the task record
+        fp.n_pairs = fp.range.y * n_rows;
+#pragma unroll
+        for (int k = 0; k < F_SLOTS; ++k) {
+            const int e = max(0, min(lane + k * NHIP_WAVE, fp.n_pairs - 1));
+            const int q = small_div(e, n_rows);
+            fp.row[k] = e - q * n_rows;
+            fp.target[k] = epi.filter.targets[fp.range.x + q];
         }
     }
+    LifPop pop = {};
+    float v_in[ROW_SLOTS], w_in[ROW_SLOTS];
+    // runs once, behind the first matrix loads of the task
+    auto after_first_loads = [&]() {
+        if (EPI == EPI_LIF) {
+            pop = epi.lif.pops[task.item];
+            const bool enabled = pop.pflags & LIF_POP_ENABLED;  // else: the buffers' first element
+#pragma unroll
+            for (int k = 0; k < ROW_SLOTS; ++k) {
+                const int i = task.row0 + min(lane + k * NHIP_WAVE, n_rows - 1);
+                v_in[k] = epi.lif.V[enabled ? (size_t)pop.v_start + i : 0];
+                w_in[k] = epi.lif.W[enabled ? (size_t)pop.w_start + i : 0];
+            }
+        }
+        if (EPI == EPI_FILTER) {
+#pragma unroll
+            for (int k = 0; k < F_SLOTS; ++k)
+                fp.old[k] = epi.filter.F[(size_t)fp.target[k].y_start +
+                                         (fp.n_pairs > 0 ? task.row0 + fp.row[k] : 0)];
+        }
+#pragma unroll
+        for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
+            const int r = lane + k * NHIP_WAVE;
+            if (r < n_rows) ys[r] = cf.y * y_old[k];
+        }
+    };
+
+    // all stages of one dot product: column stages outside, row blocks inside
+    auto dot_pass = [&](auto lgc_tag, auto first_tag, const GemvDot& dot) {
+        using G = StreamGeo<decltype(lgc_tag)::value>;
+        const int nb = (n_rows + G::RB - 1) / G::RB;            // row blocks of the task
+        const int n_stages = nb * (G::WIDE ? dot.N >> G::LG_COLS : 1);
+        const unsigned stride4 = 4u * (unsigned)dot.a_stride0;  // bytes between rows
+        const char* const a0 = reinterpret_cast<const char*>(
+            A + dot.a_start + (size_t)task.row0 * dot.a_stride0);
+        const float* const x0 = X + dot.x_start;
+        const int lane_r = lane >> G::LGQ;
+        const int lane_q = lane & ((1 << G::LGQ) - 1);
+        // byte offset of this lane's quad in the first load of a block; load i is
+        // (i >> LG_LPR) * RPL rows and (i & (LPR - 1)) * 1024 bytes further, which is the
+        // same for all lanes and goes into the scalar base
+        const unsigned lane_off = (unsigned)lane_r * stride4 + 16u * (unsigned)lane_q;
+        const unsigned row0_off = 16u * (unsigned)lane_q;  // ... if it were in the block's first row
+        // LDS: where this lane's quads go, where its partial sum starts
+        float* const wp = ab + lane_r * G::ROWW + (lane_q >> 5) * TILE_LDS + ((lane_q & 31) << 2);
+        const int j = lane & 3;
+        const int rt = lane >> 2;
+        const int tl = rt & (G::TILES - 1);
+        const float* const ap = ab + (rt >> G::LGT) * G::ROWW + tl * TILE_LDS + j;
+        const float* const xp = xb + tl * TILE_LDS + j;
+
+        // the loader walks the stages two ahead of the sums
+        int l_b = 0;                 // row block of the next stage to load
+        int l_c0 = 0;                // its first column
+        const char* l_ptr = a0;      // its first byte
+        auto load_block = [&](tile_f4 (&pf)[G::NL], float (&xq)[G::XL]) {
+            if (G::WIDE) {
+                const float* xg = x0 + (size_t)l_c0 * dot.x_stride0;
+#pragma unroll
+                for (int i = 0; i < G::XL; ++i)
+                    xq[i] = xg[(size_t)(lane + i * NHIP_WAVE) * dot.x_stride0];
+            }
+            const int rows = min(G::RB, n_rows - l_b * G::RB);
+            if (rows == G::RB) {
+#pragma unroll
+                for (int i = 0; i < G::NL; ++i) {
+                    const char* row = l_ptr + (size_t)((i >> G::LG_LPR) * G::RPL) * stride4 +
+                                      (i & ((1 << G::LG_LPR) - 1)) * 1024;
+                    pf[i] = load_nt4(reinterpret_cast<const float*>(row + lane_off));
+                }
+            } else {  // the task's last rows: a lane without a row reads the block's first row
+#pragma unroll
+                for (int i = 0; i < G::NL; ++i) {
+                    const bool mine = lane_r + (i >> G::LG_LPR) * G::RPL < rows;
+                    const char* row = l_ptr + (i & ((1 << G::LG_LPR) - 1)) * 1024;
+                    const unsigned off = (unsigned)(lane_r + (i >> G::LG_LPR) * G::RPL) * stride4 +
+                                         16u * (unsigned)lane_q;
+                    pf[i] = load_nt4(reinterpret_cast<const float*>(row + (mine ? off : row0_off)));
+                }
+            }
+            if (++l_b == nb) {
+                l_b = 0;
+                l_c0 += G::NCS;
+                l_ptr = a0 + 4u * (unsigned)l_c0;
+            } else {
+                l_ptr += (size_t)G::RB * stride4;
+            }
+        };
+        auto store_block = [&](const tile_f4 (&pf)[G::NL], const float (&xq)[G::XL], bool with_x) {
+            wave_sync();  // every lane is done reading the previous block
+#pragma unroll
+            for (int i = 0; i < G::NL; ++i)  // rows the task does not have get whatever was read
+                *reinterpret_cast<tile_f4*>(wp + (i >> G::LG_LPR) * G::RPL * G::ROWW +
+                                            (i & ((1 << G::LG_LPR) - 1)) * (2 * TILE_LDS)) = pf[i];
+            if (with_x) {
+#pragma unroll
+                for (int i = 0; i < G::XL; ++i)
+                    if (G::NCS >= NHIP_WAVE || lane < G::NCS)
+                        xb[lane + (i >> 1) * TILE_LDS + (i & 1) * NHIP_WAVE] = xq[i];
+            }
+            wave_sync();
+        };
+        auto sum_block = [&](int b) {
+            const int n_rt = min(G::RB, n_rows - b * G::RB) << G::LGT;  // (row, tile) pairs
+#pragma unroll
+            for (int p = 0; p < G::PASSES; ++p) {
+                if (p * 16 < n_rt) {  // uniform
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int m = 0; m < G::CHAIN; ++m)
+                        acc = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
+                    acc = acc + quad_xor(acc, 2);
+                    acc = acc + quad_xor(acc, 1);
+                    // tile sums, in order, onto the running sum of the row
+                    float t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+                    if (G::TILES >= 2) t1 = row_from_right<4>(acc);
+                    if (G::TILES == 4) {
+                        t2 = row_from_right<8>(acc);
+                        t3 = row_from_right<12>(acc);
+                    }
+                    if (j == 0 && tl == 0 && p * 16 + rt < n_rt) {
+                        float* yp = ys + b * G::RB + ((p * 16 + rt) >> G::LGT);
+                        float v = *yp;
+                        v = v + cf.x * acc;
+                        if (G::TILES >= 2) v = v + cf.x * t1;
+                        if (G::TILES == 4) {
+                            v = v + cf.x * t2;
+                            v = v + cf.x * t3;
+                        }
+                        *yp = v;
+                    }
+                }
+            }
+        };
+
+        tile_f4 pf0[G::NL], pf1[G::NL];
+        float xq0[G::XL], xq1[G::XL];
+        load_block(pf0, xq0);
+        if (n_stages == 1) {  // the second set's first loads are never under a branch
+            l_b = 0;
+            l_c0 = 0;
+            l_ptr = a0;
+        }
+        load_block(pf1, xq1);
+        if (!G::WIDE) {  // one column stage: its X is fetched once
+#pragma unroll
+            for (int i = 0; i < G::XL; ++i)
+                xq0[i] = x0[(size_t)min(lane + i * NHIP_WAVE, G::NCS - 1) * dot.x_stride0];
+        }
+        if (decltype(first_tag)::value) after_first_loads();
+        int k = 0;   // stage whose block is in pf0
+        int b = 0;   // its row block
+        auto next_b = [&](int v) { return v + 1 == nb ? 0 : v + 1; };
+        // stages k + 2 and k + 3 exist: both register sets are refilled without a branch
+        while (k + 3 < n_stages) {
+            const int b1 = next_b(b);
+            store_block(pf0, xq0, G::WIDE ? b == 0 : k == 0);
+            load_block(pf0, xq0);
+            sum_block(b);
+            store_block(pf1, xq1, G::WIDE && b1 == 0);
+            load_block(pf1, xq1);
+            sum_block(b1);
+            b = next_b(b1);
+            k += 2;
+        }
+        // at most three stages left; k and k + 1 are loaded, k + 2 is not
+        {
+            const int b1 = next_b(b);
+            const int b2 = next_b(b1);
+            store_block(pf0, xq0, G::WIDE ? b == 0 : k == 0);
+            if (k + 2 < n_stages) load_block(pf0, xq0);
+            sum_block(b);
+            if (k + 1 < n_stages) {
+                store_block(pf1, xq1, G::WIDE && b1 == 0);
+                sum_block(b1);
+            }
+            if (k + 2 < n_stages) {
+                store_block(pf0, xq0, G::WIDE && b2 == 0);
+                sum_block(b2);
+            }
+        }
+    };
+
+    auto dot_of_width = [&](auto first_tag, const GemvDot& dot) {
+        if (dot.p1 == 5) dot_pass(std::integral_constant<int, 5>{}, first_tag, dot);
+        else if (dot.p1 == 6) dot_pass(std::integral_constant<int, 6>{}, first_tag, dot);
+        else dot_pass(std::integral_constant<int, 9>{}, first_tag, dot);
+    };
+    if (it.n_dots == 0) {
+        after_first_loads();
+    } else {
+        dot_of_width(std::true_type{}, ft.dot0);
+        for (int d = 1; d < it.n_dots; ++d) dot_of_width(std::false_type{}, dots[it.dot_begin + d]);
+    }
+    finish_task<EPI>(task, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
 }
 
 }  // namespace
@@ -717,15 +1090,18 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
-    if (pow2_cols != 0 && (pow2_cols != 1 || vec != 4)) return NHIP_E_BADCLASS;
+    if (pow2_cols != 0 && ((pow2_cols != 1 && pow2_cols != 2) || vec != 4)) return NHIP_E_BADCLASS;
+    if (pow2_cols == 2 && blk_words != STREAM_BLK_WORDS) return NHIP_E_BADARG;
     if (blk_words < (STAGE_COLS / TILE) * TILE_LDS || (blk_words & 3)) return NHIP_E_BADARG;
     if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
     const int waves = NHIP_WG / NHIP_WAVE;
-    const size_t wave_words = (size_t)blk_words + TSUM_WORDS + XBLK_WORDS + (pow2_cols ? YSUM_WORDS : 0);
+    const size_t wave_words = pow2_cols == 2
+        ? (size_t)STREAM_BLK_WORDS + XBLK_WORDS + YSUM_WORDS
+        : (size_t)blk_words + TSUM_WORDS + XBLK_WORDS + (pow2_cols ? YSUM_WORDS : 0);
     const size_t lds_bytes = sizeof(float) * waves * wave_words;
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
     // the LIF epilogue queues its rare cases in the stage block and what follows it
-    if (epilogue == EPI_LIF && pow2_cols && blk_words + TSUM_WORDS + XBLK_WORDS < LIF_QUEUE_WORDS)
+    if (epilogue == EPI_LIF && pow2_cols == 1 && blk_words + TSUM_WORDS + XBLK_WORDS < LIF_QUEUE_WORDS)
         return NHIP_E_BADARG;
     const int n_groups = (n_tasks + waves - 1) / waves;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -739,7 +1115,12 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     };
     auto launch_epi = [&](auto epi_tag) {
         constexpr int E = decltype(epi_tag)::value;
-        if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
+        if (pow2_cols == 2) {
+            NHIP_LAUNCH(gemv_stream_kernel<E>, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+                        reinterpret_cast<const GemvDot*>(dots),
+                        reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, (int)XBLK_WORDS, A, X,
+                        Yin, Y, args);
+        } else if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
         else if (vec == 4) launch(gemv_tile_kernel<4, E>);
         else launch(gemv_tile_kernel<1, E>);
     };

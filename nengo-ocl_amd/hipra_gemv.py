@@ -36,6 +36,9 @@ TILE_STAGE_WORDS = int(os.environ.get("NENGO_HIP_TILE_WORDS", 2176))
 MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
+# dot products the large-item kernel with compile-time shapes takes: these widths, and
+# every power of two from STREAM_MIN_WIDE up; its LDS block has STREAM_STAGE_WORDS words
+STREAM_WIDTHS, STREAM_MIN_WIDE, STREAM_STAGE_WORDS = (32, 64), 512, 2176
 WG, WAVE = 256, 64
 THIN_MIN_ROWS, THIN_ROWS_FOR_LANE_PER_ROW = 32, 65536
 LIF_POP_ENABLED, LIF_POP_DECAY = 1 << 8, 1 << 9  # flag bits of a population row
@@ -205,7 +208,11 @@ class gemv_prog:
             pow2 = vec == 4 and all(
                 d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0
                 and d["a_stride0"] < 2 ** 22 for d in dots)
-            return (3, int(pow2), vec)  # second entry: 1 = every column count a power of two
+            # second entry: 1 = every column count a power of two, 2 = ... and one of the
+            # widths the kernel with compile-time shapes is built for
+            stream = pow2 and TILE_STAGE_WORDS == STREAM_STAGE_WORDS and all(
+                d["a_shape1"] in STREAM_WIDTHS or d["a_shape1"] >= STREAM_MIN_WIDE for d in dots)
+            return (3, 2 if stream else int(pow2), vec)
         if flavor == 0:
             # Matrix loads are non-temporal, so one wave instruction should take whole
             # 128-byte lines of a row: at least 8 lanes x 16 bytes per row, each lane then
@@ -298,6 +305,15 @@ class gemv_prog:
             if geometry[b]["y_len"] > 0:
                 by_class[self._item_class(geometry[b])].append(b)
 
+        # items without dot products (class (3, 1, 4)) ride with the launch of the
+        # compile-time-shape kernel when there is one
+        if (3, 2, 4) in by_class and (3, 1, 4) in by_class:
+            bare = [b for b in by_class[(3, 1, 4)] if not geometry[b]["dots"]]
+            by_class[(3, 2, 4)] = sorted(by_class[(3, 2, 4)] + bare)
+            by_class[(3, 1, 4)] = [b for b in by_class[(3, 1, 4)] if geometry[b]["dots"]]
+            if not by_class[(3, 1, 4)]:
+                del by_class[(3, 1, 4)]
+
         dev_items = to_device(self.queue, item_tab)
         dev_coefs = to_device(self.queue, coef_tab)
         dev_dots = to_device(self.queue, dot_tab)
@@ -371,6 +387,7 @@ class gemv_prog:
             plan.n_tasks = n_tasks
             plan.members = list(members)
             plan.prog = self
+            plan.host_tasks = task_tab if flavor == 3 else None
             plans.append(plan)
         return plans
 
@@ -675,8 +692,20 @@ def fuse_linearfilter(gemv_plans, lf_plan):
         f_bytes = sum(8 * int(Y.shape0s[b]) * len(targets_of[b]) for b in plan.members
                       if b in targets_of)  # filter state in and out
         entry, args = _epilogue_call(lib, plan, "filter")
+        keep = ()
+        if plan.kernel_class[0] == 3:
+            # the large-item kernel finds an item's range of targets in the spare
+            # fields of its task records (one read less before it can start)
+            tasks = plan.host_tasks.copy()
+            tasks[:, 3] = item_targets[tasks[:, 0], 0]
+            tasks[:, 11] = item_targets[tasks[:, 0], 1]
+            dev_tasks = to_device(queue, tasks)
+            at = 6  # (vec, pow2, words, items, coefs, dots, tasks, ...)
+            args = tuple(args[:at]) + (dev_tasks.ptr,) + tuple(args[at + 1:])
+            keep = (dev_tasks,)
         fused = Plan(queue, entry, args + extra, gsize=plan.gsize,
-                     lsize=plan.lsize, full_args=plan.full_args + (dev_items, dev_targets, F.dev_buf),
+                     lsize=plan.lsize,
+                     full_args=plan.full_args + (dev_items, dev_targets, F.dev_buf) + keep,
                      name=plan.name + "_filter", tag=plan.tag,
                      bw_per_call=plan.bw_per_call + f_bytes, flops_per_call=plan.flops_per_call)
         fused.description = plan.description

@@ -140,7 +140,7 @@ def test_ensemble_shapes(queue, pi):
     thin), decoders (d x n, short and wide), per-neuron scalars, single dots."""
     rng = np.random.RandomState(7)
     shapes = [(4096, 64), (64, 4096), (100, 1), (1, 100), (100, 2), (2, 100), (2000, 32),
-              (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000)]
+              (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000), (600, 128)]
     A = RA([rng.normal(size=s) for s in shapes], align=True)
     X = RA([rng.normal(size=s[1]) for s in shapes], align=True)
     Y = RA([rng.normal(size=s[0]) for s in shapes], align=True)
@@ -148,7 +148,8 @@ def test_ensemble_shapes(queue, pi):
     prog = run_case(queue, planners()[pi], 1.0, 1.0, 0.0, A, X, Y, js, js)
     if pi == 0:
         classes = {p.kernel_class for p in prog.plans}
-        assert classes == {(3, 1, 4), (3, 0, 4), (2, 4, 1)}  # power-of-two widths, any width, small
+        # widths 32 / 64 / >= 512 (compile-time shapes), other powers of two, any width, small
+        assert classes == {(3, 2, 4), (3, 1, 4), (3, 0, 4), (2, 4, 1)}
 
 
 def test_strided_views_and_yin(queue):
@@ -332,7 +333,7 @@ def test_pow2_items_bit_exact(queue, beta):
     orc.plan_block_gemv(None, 1.0, A, js, X, js, beta, Yo).plans[0]()
     dY = to_dev(queue, Y)
     prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY)
-    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4)}
+    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4), (3, 2, 4)}
     for plan in prog.plans:
         plan()
     got = dY.to_host()
@@ -359,6 +360,69 @@ def test_pow2_items_bit_exact(queue, beta):
     assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("beta", [1.0, 0.5])
+def test_compile_time_shape_items_bit_exact(queue, beta):
+    """Widths 32, 64 and powers of two from 512 up take the kernel whose stage shapes
+    are compile-time constants: row counts that leave partial row blocks, tasks of one
+    to many stages, outputs that sum dot products of several such widths, a Y_in
+    different from Y, and views with a row stride larger than the width and a strided
+    X -- bit-identical to the oracle."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(31337)
+    shapes = [(999, 32), (513, 32), (8200, 32), (4096, 64), (777, 64), (2049, 64), (129, 64),
+              (67, 512), (17, 512), (33, 1024), (64, 4096), (6, 4096), (9, 8192), (1, 16384),
+              (257, 2048), (3, 32768)]
+    multi = (64, 1024, 32, 512, 64)
+    mats = [rng.normal(size=s) for s in shapes] + [rng.normal(size=(300, n)) for n in multi]
+    A = RA(mats, align=True)
+    X = RA([rng.normal(size=m.shape[1]) for m in mats], align=True)
+    Y = RA([rng.normal(size=s[0]) for s in shapes] + [rng.normal(size=300)], align=True)
+    Yin = RA([rng.normal(size=s[0]) for s in shapes] + [rng.normal(size=300)], align=True)
+    n = len(shapes)
+    js = [np.array([i], dtype=np.int32) for i in range(n)] + [np.arange(n, n + len(multi), dtype=np.int32)]
+    for use_yin in (False, True):
+        Yo = clone(Y)
+        orc.plan_block_gemv(None, 0.75, A, js, X, js, beta, Yo, Y_in=clone(Yin) if use_yin else None,
+                            gamma=0.125).plans[0]()
+        dY = to_dev(queue, Y)
+        prog = g.plan_block_gemv(queue, 0.75, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY,
+                                 Y_in=to_dev(queue, Yin) if use_yin else None, gamma=0.125)
+        assert {p.kernel_class for p in prog.plans} == {(3, 2, 4)}
+        for plan in prog.plans:
+            plan()
+        got = dY.to_host()
+        for i in range(len(Y)):
+            assert np.array_equal(got[i], Yo[i]), (i, use_yin)
+
+    # column blocks of a wider matrix (row stride 1200: widths 64, 512 and 32) times
+    # every second / third element of longer vectors
+    wide = rng.normal(size=(700, 1200)).astype(np.float32)
+    Aw = RA([wide], align=True)
+    Av = Aw[[0]]  # shares the buffer
+    s0 = int(Aw.starts[0])
+    Av.add_views([s0, s0 + 64, s0 + 576], [700, 700, 700], [64, 512, 32], [1200] * 3, [1] * 3)
+    xs = [rng.normal(size=64 * 2), rng.normal(size=512 * 3), rng.normal(size=32)]
+    Xw = RA(xs, align=True)
+    Xv = Xw[[0]]
+    Xv.add_views([int(Xw.starts[0]), int(Xw.starts[1]), int(Xw.starts[2])], [64, 512, 32], [1] * 3,
+                 [2, 3, 1], [1] * 3)
+    Yw = RA([rng.normal(size=700)], align=True)
+    jA, jX = [np.array([1, 2, 3], dtype=np.int32)], [np.array([1, 2, 3], dtype=np.int32)]
+    Yo = clone(Yw)
+    orc.plan_block_gemv(None, 1.0, Av, jA, Xv, jX, beta, Yo).plans[0]()
+    dY = to_dev(queue, Yw)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, Av), jA, to_dev(queue, Xv), jX, beta, dY)
+    assert {p.kernel_class for p in prog.plans} == {(3, 2, 4)}
+    for plan in prog.plans:
+        plan()
+    assert np.array_equal(dY.to_host()[0], Yo[0])
+    expect = (beta * Yw[0][:, 0] + wide[:, :64] @ xs[0][::2] + wide[:, 64:576] @ xs[1][::3]
+              + wide[:, 576:608] @ xs[2])
+    assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
+
+
 @pytest.mark.parametrize("tau_kind", ["per-population", "per-neuron"])
 def test_gemv_with_lif_epilogue(queue, tau_kind):
     """GEMV + LIF in one launch: the currents, voltages, refractory times and spikes
@@ -374,7 +438,7 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     rng = np.random.RandomState(31)
     dt = 1e-3
     # GEMV items: four large ones with neurons, a small one with neurons, a large one without
-    shapes = [(4096, 64), (1000, 64), (3000, 48), (520, 130), (60, 8), (300, 64)]
+    shapes = [(4096, 64), (1000, 128), (3000, 48), (520, 130), (60, 8), (300, 64)]
     pop_sizes = [4096, 1000, 3000, 520, 60, 700]  # the last population has no input item
     n, n_pop = len(shapes), len(pop_sizes)
     mats = [rng.normal(scale=0.4, size=s) for s in shapes]
@@ -408,12 +472,12 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     fused = g.fuse_lif(prog, lif)
     assert fused is not None
     names = sorted(p.name for p in fused)
-    # three large-item classes (the input-less population joins the power-of-two one)
-    # and the small item's launch, each updating the neurons it feeds: no neuron launch
-    assert names == ["hipra_gemv.tile_lif", "hipra_gemv.tile_lif", "hipra_gemv.tile_lif",
-                     "hipra_gemv.wave_ref_lif"]
+    # four large-item classes (the input-less population joins the one with compile-time
+    # shapes) and the small item's launch, each updating the neurons it feeds: no neuron
+    # launch
+    assert names == ["hipra_gemv.tile_lif"] * 4 + ["hipra_gemv.wave_ref_lif"]
     assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_lif"} == {
-        (3, 1, 4), (3, 0, 4), (3, 0, 1)}
+        (3, 2, 4), (3, 1, 4), (3, 0, 4), (3, 0, 1)}
     for step in range(3):
         for p in fused:
             p()
@@ -462,7 +526,7 @@ def test_gemv_with_filter_epilogue(queue):
     from oracle import oracle as orc
 
     rng = np.random.RandomState(5)
-    shapes = [(64, 4096), (64, 2048), (100, 300), (16, 8)]
+    shapes = [(64, 4096), (64, 2048), (100, 300), (16, 8), (80, 128)]
     n = len(shapes)
     mats = [rng.normal(scale=0.1, size=s) for s in shapes]
     xs = [rng.normal(size=s[1]) for s in shapes]
@@ -471,7 +535,8 @@ def test_gemv_with_filter_epilogue(queue):
     lowpass = lambda tau: (np.array([-np.exp(-0.001 / tau)]), np.array([1 - np.exp(-0.001 / tau)]))
     filters = [(0,) + lowpass(0.005), (0,) + lowpass(0.1), (0,) + lowpass(0.02),
                (1, np.zeros(0), np.array([0.5])), (2,) + lowpass(0.01), (3,) + lowpass(0.01),
-               (0, np.array([-1.2, 0.4]), np.array([0.1, 0.1]))]
+               (0, np.array([-1.2, 0.4]), np.array([0.1, 0.1])), (4,) + lowpass(0.03),
+               (4,) + lowpass(0.002)]
     f_out = [rng.normal(size=shapes[b][0]) for b, _, _ in filters]
     R = RA(mats + xs + outs + f_out, align=True)
     iA, iX, iY = (list(range(k * n, (k + 1) * n)) for k in range(3))
@@ -503,8 +568,11 @@ def test_gemv_with_filter_epilogue(queue):
     result = g.fuse_linearfilter(prog.plans, lf[0])
     assert result is not None
     fused, residual = result
-    assert sorted(p.name for p in fused) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_filter",
-                                              "hipra_gemv.wave_ref_filter"]
+    # compile-time shapes (4096, 2048), another power of two (128), any width (300), small
+    assert sorted(p.name for p in fused) == ["hipra_gemv.tile_filter"] * 3 + [
+        "hipra_gemv.wave_ref_filter"]
+    assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_filter"} == {
+        (3, 2, 4), (3, 1, 4), (3, 0, 4)}
     assert [p.name for p in residual] == ["hip_linearfilter"]
     oprog, olf = build(host, orc, orc, None, lambda a: a)
     for step in range(4):
