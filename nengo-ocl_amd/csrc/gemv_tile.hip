@@ -824,6 +824,7 @@ struct StreamGeo {
 };
 
 constexpr int STREAM_BLK_WORDS = 2176;  // the LDS block these shapes are made for
+constexpr int STREAM_NARROW_XB_WORDS = 72;  // X block of a launch whose widest dot product has 64 columns
 
 // lane i receives the value of lane i + n of its row of 16 lanes
 template <int N>
@@ -831,7 +832,9 @@ __device__ __forceinline__ float row_from_right(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x100 + N, 0xF, 0xF, true));
 }
 
-template <int EPI>
+// WIDE: the launch has dot products of 512 columns or more (more registers and a
+// larger X block in LDS: three waves per SIMD instead of four).
+template <int EPI, bool WIDE>
 __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4))) void gemv_stream_kernel(
     const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
@@ -1060,7 +1063,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4)))
 
     auto dot_of_width = [&](auto first_tag, const GemvDot& dot) {
         if (dot.p1 == 5) dot_pass(std::integral_constant<int, 5>{}, first_tag, dot);
-        else if (dot.p1 == 6) dot_pass(std::integral_constant<int, 6>{}, first_tag, dot);
+        else if (!WIDE || dot.p1 == 6) dot_pass(std::integral_constant<int, 6>{}, first_tag, dot);
         else dot_pass(std::integral_constant<int, 9>{}, first_tag, dot);
     };
     if (it.n_dots == 0) {
@@ -1090,13 +1093,14 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
-    if (pow2_cols != 0 && ((pow2_cols != 1 && pow2_cols != 2) || vec != 4)) return NHIP_E_BADCLASS;
-    if (pow2_cols == 2 && blk_words != STREAM_BLK_WORDS) return NHIP_E_BADARG;
+    if (pow2_cols != 0 && (pow2_cols < 1 || pow2_cols > 3 || vec != 4)) return NHIP_E_BADCLASS;
+    if (pow2_cols >= 2 && blk_words != STREAM_BLK_WORDS) return NHIP_E_BADARG;
+    const int stream_xb = pow2_cols == 3 ? STREAM_NARROW_XB_WORDS : XBLK_WORDS;
     if (blk_words < (STAGE_COLS / TILE) * TILE_LDS || (blk_words & 3)) return NHIP_E_BADARG;
     if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
     const int waves = NHIP_WG / NHIP_WAVE;
-    const size_t wave_words = pow2_cols == 2
-        ? (size_t)STREAM_BLK_WORDS + XBLK_WORDS + YSUM_WORDS
+    const size_t wave_words = pow2_cols >= 2
+        ? (size_t)STREAM_BLK_WORDS + stream_xb + YSUM_WORDS
         : (size_t)blk_words + TSUM_WORDS + XBLK_WORDS + (pow2_cols ? YSUM_WORDS : 0);
     const size_t lds_bytes = sizeof(float) * waves * wave_words;
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
@@ -1116,10 +1120,15 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     auto launch_epi = [&](auto epi_tag) {
         constexpr int E = decltype(epi_tag)::value;
         if (pow2_cols == 2) {
-            NHIP_LAUNCH(gemv_stream_kernel<E>, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+            NHIP_LAUNCH((gemv_stream_kernel<E, true>), dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
                         reinterpret_cast<const GemvDot*>(dots),
-                        reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, (int)XBLK_WORDS, A, X,
-                        Yin, Y, args);
+                        reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, stream_xb, A, X, Yin,
+                        Y, args);
+        } else if (pow2_cols == 3) {
+            NHIP_LAUNCH((gemv_stream_kernel<E, false>), dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+                        reinterpret_cast<const GemvDot*>(dots),
+                        reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, stream_xb, A, X, Yin,
+                        Y, args);
         } else if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
         else if (vec == 4) launch(gemv_tile_kernel<4, E>);
         else launch(gemv_tile_kernel<1, E>);

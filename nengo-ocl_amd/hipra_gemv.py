@@ -209,10 +209,13 @@ class gemv_prog:
                 d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0
                 and d["a_stride0"] < 2 ** 22 for d in dots)
             # second entry: 1 = every column count a power of two, 2 = ... and one of the
-            # widths the kernel with compile-time shapes is built for
+            # widths the kernel with compile-time shapes is built for, 3 = ... and none
+            # of them wide (more waves fit a compute unit then)
             stream = pow2 and TILE_STAGE_WORDS == STREAM_STAGE_WORDS and all(
                 d["a_shape1"] in STREAM_WIDTHS or d["a_shape1"] >= STREAM_MIN_WIDE for d in dots)
-            return (3, 2 if stream else int(pow2), vec)
+            if stream:
+                return (3, 3 if all(d["a_shape1"] in STREAM_WIDTHS for d in dots) else 2, vec)
+            return (3, int(pow2), vec)
         if flavor == 0:
             # Matrix loads are non-temporal, so one wave instruction should take whole
             # 128-byte lines of a row: at least 8 lanes x 16 bytes per row, each lane then
@@ -307,9 +310,13 @@ class gemv_prog:
 
         # items without dot products (class (3, 1, 4)) ride with the launch of the
         # compile-time-shape kernel when there is one
-        if (3, 2, 4) in by_class and (3, 1, 4) in by_class:
+        # ... whose narrow items join the wide ones when both kinds are there
+        if (3, 2, 4) in by_class and (3, 3, 4) in by_class:
+            by_class[(3, 2, 4)] = sorted(by_class[(3, 2, 4)] + by_class.pop((3, 3, 4)))
+        stream = (3, 2, 4) if (3, 2, 4) in by_class else (3, 3, 4)
+        if stream in by_class and (3, 1, 4) in by_class:
             bare = [b for b in by_class[(3, 1, 4)] if not geometry[b]["dots"]]
-            by_class[(3, 2, 4)] = sorted(by_class[(3, 2, 4)] + bare)
+            by_class[stream] = sorted(by_class[stream] + bare)
             by_class[(3, 1, 4)] = [b for b in by_class[(3, 1, 4)] if geometry[b]["dots"]]
             if not by_class[(3, 1, 4)]:
                 del by_class[(3, 1, 4)]

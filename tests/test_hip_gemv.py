@@ -148,7 +148,8 @@ def test_ensemble_shapes(queue, pi):
     prog = run_case(queue, planners()[pi], 1.0, 1.0, 0.0, A, X, Y, js, js)
     if pi == 0:
         classes = {p.kernel_class for p in prog.plans}
-        # widths 32 / 64 / >= 512 (compile-time shapes), other powers of two, any width, small
+        # widths 32 / 64 / >= 512 (compile-time shapes; 2: some of them wide), other powers of
+        # two, any width, small
         assert classes == {(3, 2, 4), (3, 1, 4), (3, 0, 4), (2, 4, 1)}
 
 
@@ -477,7 +478,7 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     # launch
     assert names == ["hipra_gemv.tile_lif"] * 4 + ["hipra_gemv.wave_ref_lif"]
     assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_lif"} == {
-        (3, 2, 4), (3, 1, 4), (3, 0, 4), (3, 0, 1)}
+        (3, 3, 4), (3, 1, 4), (3, 0, 4), (3, 0, 1)}
     for step in range(3):
         for p in fused:
             p()
