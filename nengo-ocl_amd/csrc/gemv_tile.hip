@@ -355,11 +355,12 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
 // LDS (`queue`: the wave's stage block, free by now) and evaluated densely
 // afterwards.  Operation by operation this is `lif_step` (same inputs, same rounded
 // operations), so the results are identical.
+template <int SLOTS>
 __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPop& p, int row0,
                                                    int n_rows, const float* ys, float gamma,
                                                    float* y_out, int y_stride0, float* queue,
-                                                   int lane, const float (&v_in)[ROW_SLOTS],
-                                                   const float (&w_in)[ROW_SLOTS]) {
+                                                   int lane, const float (&v_in)[SLOTS],
+                                                   const float (&w_in)[SLOTS]) {
     const float tau = nhip_bits(p.tau);
     const float decay = nhip_bits(p.decay);
     const float dtu = a.dtu;
@@ -391,7 +392,7 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
     };
 
 #pragma unroll
-    for (int k = 0; k < ROW_SLOTS; ++k) {
+    for (int k = 0; k < SLOTS; ++k) {
         if (k * NHIP_WAVE >= n_rows) break;  // uniform
         const int r = k * NHIP_WAVE + lane;
         const bool live = r < n_rows;
@@ -468,12 +469,12 @@ struct FilterPrefetch {
     float old[F_SLOTS];
 };
 
-template <int EPI>
+template <int EPI, int SLOTS>
 __device__ __forceinline__ void finish_task(const GemvTask& task, const GemvItem& it,
                                             const float4& cf, const float* ys, float* ab,
                                             const float* Yin, float* Y, const EpilogueArgs& epi,
-                                            const LifPop& pop, const float (&v_in)[ROW_SLOTS],
-                                            const float (&w_in)[ROW_SLOTS],
+                                            const LifPop& pop, const float (&v_in)[SLOTS],
+                                            const float (&w_in)[SLOTS],
                                             const FilterPrefetch& fp, int lane) {
     const int n_rows = task.n_rows;
     const int2 filters = fp.range;
@@ -484,12 +485,12 @@ __device__ __forceinline__ void finish_task(const GemvTask& task, const GemvItem
     const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
                            it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
     if (EPI == EPI_LIF && (pop.pflags & LIF_POP_DECAY)) {
-        lif_task_compacted(epi.lif, pop, task.row0, n_rows, ys, cf.z,
+        lif_task_compacted<SLOTS>(epi.lif, pop, task.row0, n_rows, ys, cf.z,
                            store_y ? Y + it.y_start : nullptr, it.y_stride0, ab, lane, v_in, w_in);
         return;
     }
 #pragma unroll
-    for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
+    for (int k = 0; k < SLOTS; ++k) {
         const int r = lane + k * NHIP_WAVE;
         if (r < n_rows) {
             const float y = ys[r] + cf.z;
@@ -786,7 +787,7 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
         fp.row[k] = f_row[k];
         fp.old[k] = f_old[k];
     }
-    finish_task<EPI>(task, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
+    finish_task<EPI, ROW_SLOTS>(task, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
 }
 
 
@@ -825,6 +826,7 @@ struct StreamGeo {
 
 constexpr int STREAM_BLK_WORDS = 2176;  // the LDS block these shapes are made for
 constexpr int STREAM_NARROW_XB_WORDS = 72;  // X block of a launch whose widest dot product has 64 columns
+constexpr int STREAM_NARROW_SLOTS = 2;      // ... and row sums per lane: its tasks cover <= 128 rows
 
 // lane i receives the value of lane i + n of its row of 16 lanes
 template <int N>
@@ -835,7 +837,7 @@ __device__ __forceinline__ float row_from_right(float v) {
 // WIDE: the launch has dot products of 512 columns or more (more registers and a
 // larger X block in LDS: three waves per SIMD instead of four).
 template <int EPI, bool WIDE>
-__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4))) void gemv_stream_kernel(
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 3 : 4, 4))) void gemv_stream_kernel(
     const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
     float* Y, EpilogueArgs epi)
@@ -843,7 +845,9 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4)))
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    float* ab = lds + wave * (STREAM_BLK_WORDS + xb_words + YSUM_WORDS);  // the wave's block
+    // a launch without wide dot products keeps its tasks to 128 rows (fewer registers)
+    constexpr int SLOTS = WIDE ? ROW_SLOTS : STREAM_NARROW_SLOTS;
+    float* ab = lds + wave * (STREAM_BLK_WORDS + xb_words + SLOTS * NHIP_WAVE);  // the wave's block
     float* xb = ab + STREAM_BLK_WORDS;  // gathered X of the current column stage, tiles padded
     float* ys = xb + xb_words;          // running sum of row r of the task
 
@@ -856,14 +860,8 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4)))
     const float4 cf = make_float4(ft.alpha, ft.beta, ft.gamma, 0.0f);
     const int n_rows = task.n_rows;
 
-    // old Y values and the filter targets: requested now, used after the first matrix
-    // loads have been issued (no branch around the loads, see gemv_tile_p2_kernel)
-    float y_old[ROW_SLOTS];
-#pragma unroll
-    for (int k = 0; k < ROW_SLOTS; ++k) {
-        const int r = min(lane + k * NHIP_WAVE, n_rows - 1);
-        y_old[k] = Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0];
-    }
+    // the filter targets: requested now, used after the first matrix loads have been
+    // issued (no branch around the loads, see gemv_tile_p2_kernel)
     FilterPrefetch fp;
     fp.range = make_int2(0, 0);
     fp.n_pairs = 0;
@@ -879,14 +877,20 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4)))
         }
     }
     LifPop pop = {};
-    float v_in[ROW_SLOTS], w_in[ROW_SLOTS];
+    float v_in[SLOTS], w_in[SLOTS];
     // runs once, behind the first matrix loads of the task
     auto after_first_loads = [&]() {
+        float y_old[SLOTS];
+#pragma unroll
+        for (int k = 0; k < SLOTS; ++k) {
+            const int r = min(lane + k * NHIP_WAVE, n_rows - 1);
+            y_old[k] = Yin[it.yin_start + (size_t)(task.row0 + r) * it.yin_stride0];
+        }
         if (EPI == EPI_LIF) {
             pop = epi.lif.pops[task.item];
             const bool enabled = pop.pflags & LIF_POP_ENABLED;  // else: the buffers' first element
 #pragma unroll
-            for (int k = 0; k < ROW_SLOTS; ++k) {
+            for (int k = 0; k < SLOTS; ++k) {
                 const int i = task.row0 + min(lane + k * NHIP_WAVE, n_rows - 1);
                 v_in[k] = epi.lif.V[enabled ? (size_t)pop.v_start + i : 0];
                 w_in[k] = epi.lif.W[enabled ? (size_t)pop.w_start + i : 0];
@@ -899,7 +903,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4)))
                                          (fp.n_pairs > 0 ? task.row0 + fp.row[k] : 0)];
         }
 #pragma unroll
-        for (int k = 0; k < YSUM_WORDS / NHIP_WAVE; ++k) {
+        for (int k = 0; k < SLOTS; ++k) {
             const int r = lane + k * NHIP_WAVE;
             if (r < n_rows) ys[r] = cf.y * y_old[k];
         }
@@ -984,6 +988,9 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4)))
             const int n_rt = min(G::RB, n_rows - b * G::RB) << G::LGT;  // (row, tile) pairs
 #pragma unroll
             for (int p = 0; p < G::PASSES; ++p) {
+                // the passes one after the other: all their LDS reads at once would need
+                // more registers than four waves per SIMD leave
+                if (p > 0) __builtin_amdgcn_sched_barrier(0);
                 if (p * 16 < n_rt) {  // uniform
                     float acc = 0.0f;
 #pragma unroll
@@ -1072,7 +1079,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(3, 4)))
         dot_of_width(std::true_type{}, ft.dot0);
         for (int d = 1; d < it.n_dots; ++d) dot_of_width(std::false_type{}, dots[it.dot_begin + d]);
     }
-    finish_task<EPI>(task, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
+    finish_task<EPI, SLOTS>(task, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
 }
 
 }  // namespace
@@ -1100,7 +1107,7 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
     const int waves = NHIP_WG / NHIP_WAVE;
     const size_t wave_words = pow2_cols >= 2
-        ? (size_t)STREAM_BLK_WORDS + stream_xb + YSUM_WORDS
+        ? (size_t)STREAM_BLK_WORDS + stream_xb + (pow2_cols == 3 ? STREAM_NARROW_SLOTS * NHIP_WAVE : YSUM_WORDS)
         : (size_t)blk_words + TSUM_WORDS + XBLK_WORDS + (pow2_cols ? YSUM_WORDS : 0);
     const size_t lds_bytes = sizeof(float) * waves * wave_words;
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit

@@ -39,6 +39,7 @@ TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
 # dot products the large-item kernel with compile-time shapes takes: these widths, and
 # every power of two from STREAM_MIN_WIDE up; its LDS block has STREAM_STAGE_WORDS words
 STREAM_WIDTHS, STREAM_MIN_WIDE, STREAM_STAGE_WORDS = (32, 64), 512, 2176
+STREAM_NARROW_MAX_ROWS = 128
 WG, WAVE = 256, 64
 THIN_MIN_ROWS, THIN_ROWS_FOR_LANE_PER_ROW = 32, 65536
 LIF_POP_ENABLED, LIF_POP_DECAY = 1 << 8, 1 << 9  # flag bits of a population row
@@ -233,7 +234,7 @@ class gemv_prog:
             lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         return (flavor, lpr, vec)
 
-    def _tile_tasks(self, members):
+    def _tile_tasks(self, members, max_rows=256):
         """Tasks (item, first row, rows, 0) of the reference-order kernel for large items.
 
         A task is the rows one wave carries through all columns, a few row blocks of
@@ -251,7 +252,7 @@ class gemv_prog:
             out = []
             for b in members:
                 M = geometry[b]["y_len"]
-                item_rows = max(1, min(int(blk[b] * per_task), 256))
+                item_rows = max(1, min(int(blk[b] * per_task), max_rows))
                 if M > item_rows:
                     item_rows = _balanced_rows(M, item_rows)
                     if item_rows >= 2 * blk[b]:
@@ -340,7 +341,9 @@ class gemv_prog:
             if rows is not None and rows <= 0:
                 raise _lib.HipError("unknown GEMV class %r" % (cls,))
             if flavor == 3:
-                task_rows = self._tile_tasks(members)
+                # launches without wide dot products keep tasks to 128 rows (the kernel
+                # then needs fewer registers and a fourth wave fits each SIMD)
+                task_rows = self._tile_tasks(members, STREAM_NARROW_MAX_ROWS if lpr == 3 else 256)
             else:
                 task_rows = []
                 for b in (members if flavor != 2 else ()):
