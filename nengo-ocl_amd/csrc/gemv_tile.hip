@@ -47,7 +47,7 @@ constexpr int X_PF = STAGE_COLS / NHIP_WAVE;  // gathered X elements per lane an
 constexpr int XBLK_WORDS = (STAGE_COLS / TILE) * TILE_LDS;  // X block of a wave in LDS
 constexpr int ROW_SLOTS = 4;       // row sums per lane: a task covers <= 256 rows
 constexpr int MAX_TASK_ROWS = ROW_SLOTS * NHIP_WAVE;
-constexpr int LIF_QUEUE_WORDS = 7 * MAX_TASK_ROWS;  // LDS words of lif_task_compacted's queues
+constexpr int LIF_QUEUE_WORDS = 10 * MAX_TASK_ROWS;  // LDS words of lif_task_compacted's queues and results
 
 typedef float tile_f4 __attribute__((ext_vector_type(4)));
 
@@ -361,34 +361,39 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
                                                    float* y_out, int y_stride0, float* queue,
                                                    int lane, const float (&v_in)[SLOTS],
                                                    const float (&w_in)[SLOTS]) {
+    constexpr int MAXR = SLOTS * NHIP_WAVE;
     const float tau = nhip_bits(p.tau);
     const float decay = nhip_bits(p.decay);
     const float dtu = a.dtu;
     const unsigned long long below = (1ull << lane) - 1ull;
-    float* leaving = queue;                     // {neuron, integration time, j, v} x n_rows
-    float* spiking = queue + 4 * MAX_TASK_ROWS;  // {neuron, j, v} x n_rows
-    int n_leaving = 0, n_spiking = 0;           // wave-uniform
+    float* leaving = queue;             // {row, integration time, j, v} x rows
+    float* spiking = queue + 4 * MAXR;  // {row, j, v} x rows
+    // The new state of row r.  Every lane files its common-case result here, the dense
+    // passes overwrite the rows they handle, and the state then leaves in whole-wave
+    // stores: written from the passes directly it would be scattered four-byte stores
+    // and several partial stores per cache line.
+    float* new_v = queue + 7 * MAXR;
+    float* new_w = new_v + MAXR;
+    float* new_s = new_w + MAXR;
+    int n_leaving = 0, n_spiking = 0;   // wave-uniform
 
-    auto push_spike = [&](bool want, int i, float j, float v) {
+    auto push_spike = [&](bool want, int r, float j, float v) {
         const unsigned long long m = __ballot(want);
         if (want) {
             float* e = spiking + 3 * (n_spiking + __popcll(m & below));
-            e[0] = __int_as_float(i);
+            e[0] = __int_as_float(r);
             e[1] = j;
             e[2] = v;
         }
         n_spiking += __popcll(m);
     };
     // voltage step with a known decay factor; queues the neuron if it spikes
-    auto integrate = [&](bool live, int i, float j, float v, float factor) {
+    auto integrate = [&](bool live, int r, float j, float v, float factor) {
         const float dv = __fmul_rn(factor, j - v);
         v = __fadd_rn(v, dv);
         const bool fired = live && v > 1.0f;
-        push_spike(fired, i, j, v);
-        if (live && !fired) {
-            a.V[(size_t)p.v_start + i] = v < 0.0f ? 0.0f : v;
-            a.S[(size_t)p.s_start + i] = 0.0f;
-        }
+        push_spike(fired, r, j, v);
+        if (live && !fired) new_v[r] = v < 0.0f ? 0.0f : v;
     };
 
 #pragma unroll
@@ -396,11 +401,10 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
         if (k * NHIP_WAVE >= n_rows) break;  // uniform
         const int r = k * NHIP_WAVE + lane;
         const bool live = r < n_rows;
-        const int i = row0 + (live ? r : 0);
         float j = 0.0f, v = 0.0f, w = 0.0f;
         if (live) {
             j = ys[r] + gamma;
-            if (y_out) y_out[(size_t)i * y_stride0] = j;
+            if (y_out) y_out[(size_t)(row0 + r) * y_stride0] = j;
             v = v_in[k];
             w = w_in[k] - dtu;
         }
@@ -410,38 +414,51 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
         const unsigned long long m = __ballot(partial);
         if (partial) {
             float* e = leaving + 4 * (n_leaving + __popcll(m & below));
-            e[0] = __int_as_float(i);
+            e[0] = __int_as_float(r);
             e[1] = delta_t;
             e[2] = j;
             e[3] = v;
         }
         n_leaving += __popcll(m);
-        if (live) a.W[(size_t)p.w_start + i] = w;  // a spike overwrites it below
-        // integration over no time leaves the voltage as it is (the factor is +0)
-        if (live && none) a.S[(size_t)p.s_start + i] = 0.0f;
-        integrate(live && whole, i, j, v, decay);
+        if (live) {
+            new_w[r] = w;     // a spike overwrites these two below
+            new_s[r] = 0.0f;
+            // integration over no time leaves the voltage as it is (the factor is +0)
+            if (!whole) new_v[r] = v;
+        }
+        integrate(live && whole, r, j, v, decay);
     }
     wave_sync();
     for (int e0 = 0; e0 < n_leaving; e0 += NHIP_WAVE) {
         const bool live = e0 + lane < n_leaving;
         const float* e = leaving + 4 * (live ? e0 + lane : 0);
-        const int i = __float_as_int(e[0]);
+        const int r = __float_as_int(e[0]);
         const float factor = -(float)expm1((double)__fdiv_rn(-e[1], tau));
-        integrate(live, i, e[2], e[3], factor);
+        integrate(live, r, e[2], e[3], factor);
     }
     wave_sync();
     for (int e0 = 0; e0 < n_spiking; e0 += NHIP_WAVE) {
         if (e0 + lane < n_spiking) {
             const float* e = spiking + 3 * (e0 + lane);
-            const int i = __float_as_int(e[0]);
+            const int r = __float_as_int(e[0]);
             const float j = e[1], v = e[2];
-            const float ref = lif_param(p.ref, p.pflags & 2, a.REF, i);
-            const float amp = lif_param(p.amp, p.pflags & 4, a.AMP, i);
+            const float ref = lif_param(p.ref, p.pflags & 2, a.REF, row0 + r);
+            const float amp = lif_param(p.amp, p.pflags & 4, a.AMP, row0 + r);
             const float t_spike = __fadd_rn(
                 dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
-            a.V[(size_t)p.v_start + i] = 0.0f;
-            a.W[(size_t)p.w_start + i] = ref + t_spike;
-            a.S[(size_t)p.s_start + i] = __fmul_rn(amp, a.dt_inv);
+            new_v[r] = 0.0f;
+            new_w[r] = ref + t_spike;
+            new_s[r] = __fmul_rn(amp, a.dt_inv);
+        }
+    }
+    wave_sync();
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const int r = k * NHIP_WAVE + lane;
+        if (r < n_rows) {
+            a.V[(size_t)p.v_start + row0 + r] = new_v[r];
+            a.W[(size_t)p.w_start + row0 + r] = new_w[r];
+            a.S[(size_t)p.s_start + row0 + r] = new_s[r];
         }
     }
 }
@@ -924,7 +941,6 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         // (i >> LG_LPR) * RPL rows and (i & (LPR - 1)) * 1024 bytes further, which is the
         // same for all lanes and goes into the scalar base
         const unsigned lane_off = (unsigned)lane_r * stride4 + 16u * (unsigned)lane_q;
-        const unsigned row0_off = 16u * (unsigned)lane_q;  // ... if it were in the block's first row
         // LDS: where this lane's quads go, where its partial sum starts
         float* const wp = ab + lane_r * G::ROWW + (lane_q >> 5) * TILE_LDS + ((lane_q & 31) << 2);
         const int j = lane & 3;
@@ -952,14 +968,14 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
                                       (i & ((1 << G::LG_LPR) - 1)) * 1024;
                     pf[i] = load_nt4(reinterpret_cast<const float*>(row + lane_off));
                 }
-            } else {  // the task's last rows: a lane without a row reads the block's first row
+            } else {  // the task's last rows: a lane without a row reads the block's first bytes
 #pragma unroll
                 for (int i = 0; i < G::NL; ++i) {
                     const bool mine = lane_r + (i >> G::LG_LPR) * G::RPL < rows;
                     const char* row = l_ptr + (i & ((1 << G::LG_LPR) - 1)) * 1024;
                     const unsigned off = (unsigned)(lane_r + (i >> G::LG_LPR) * G::RPL) * stride4 +
                                          16u * (unsigned)lane_q;
-                    pf[i] = load_nt4(reinterpret_cast<const float*>(row + (mine ? off : row0_off)));
+                    pf[i] = load_nt4(reinterpret_cast<const float*>(row + (mine ? off : 0u)));
                 }
             }
             if (++l_b == nb) {
