@@ -930,7 +930,11 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
     auto dot_pass = [&](auto lgc_tag, auto first_tag, const GemvDot& dot) {
         using G = StreamGeo<decltype(lgc_tag)::value>;
         const int nb = (n_rows + G::RB - 1) / G::RB;            // row blocks of the task
-        const int n_stages = nb * (G::WIDE ? dot.N >> G::LG_COLS : 1);
+        // wide dot products: any column count that is a multiple of 4; the last column
+        // stage then has last_cols < NCS columns
+        const int n_col = G::WIDE ? (dot.N + G::NCS - 1) >> G::LG_COLS : 1;
+        const int last_cols = G::WIDE ? dot.N - (n_col - 1) * G::NCS : G::NCS;
+        const int n_stages = nb * n_col;
         const unsigned stride4 = 4u * (unsigned)dot.a_stride0;  // bytes between rows
         const char* const a0 = reinterpret_cast<const char*>(
             A + dot.a_start + (size_t)task.row0 * dot.a_stride0);
@@ -954,24 +958,33 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         int l_c0 = 0;                // its first column
         const char* l_ptr = a0;      // its first byte
         auto load_block = [&](tile_f4 (&pf)[G::NL], float (&xq)[G::XL]) {
+            const int cols = G::WIDE ? min(G::NCS, dot.N - l_c0) : G::NCS;
             if (G::WIDE) {
                 const float* xg = x0 + (size_t)l_c0 * dot.x_stride0;
+                if (cols == G::NCS) {
 #pragma unroll
-                for (int i = 0; i < G::XL; ++i)
-                    xq[i] = xg[(size_t)(lane + i * NHIP_WAVE) * dot.x_stride0];
+                    for (int i = 0; i < G::XL; ++i)
+                        xq[i] = xg[(size_t)(lane + i * NHIP_WAVE) * dot.x_stride0];
+                } else {  // the last columns: lanes past the end read the last element
+#pragma unroll
+                    for (int i = 0; i < G::XL; ++i)
+                        xq[i] = xg[(size_t)min(lane + i * NHIP_WAVE, cols - 1) * dot.x_stride0];
+                }
             }
             const int rows = min(G::RB, n_rows - l_b * G::RB);
-            if (rows == G::RB) {
+            if (rows == G::RB && cols == G::NCS) {
 #pragma unroll
                 for (int i = 0; i < G::NL; ++i) {
                     const char* row = l_ptr + (size_t)((i >> G::LG_LPR) * G::RPL) * stride4 +
                                       (i & ((1 << G::LG_LPR) - 1)) * 1024;
                     pf[i] = load_nt4(reinterpret_cast<const float*>(row + lane_off));
                 }
-            } else {  // the task's last rows: a lane without a row reads the block's first bytes
+            } else {  // the task's last rows, the last columns: a lane without an element
+                      // reads the block's first bytes
 #pragma unroll
                 for (int i = 0; i < G::NL; ++i) {
-                    const bool mine = lane_r + (i >> G::LG_LPR) * G::RPL < rows;
+                    const bool mine = lane_r + (i >> G::LG_LPR) * G::RPL < rows &&
+                                      (i & ((1 << G::LG_LPR) - 1)) * 256 + 4 * lane_q < cols;
                     const char* row = l_ptr + (i & ((1 << G::LG_LPR) - 1)) * 1024;
                     const unsigned off = (unsigned)(lane_r + (i >> G::LG_LPR) * G::RPL) * stride4 +
                                          16u * (unsigned)lane_q;
@@ -989,7 +1002,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         auto store_block = [&](const tile_f4 (&pf)[G::NL], const float (&xq)[G::XL], bool with_x) {
             wave_sync();  // every lane is done reading the previous block
 #pragma unroll
-            for (int i = 0; i < G::NL; ++i)  // rows the task does not have get whatever was read
+            for (int i = 0; i < G::NL; ++i)  // rows and columns that do not exist get whatever was read
                 *reinterpret_cast<tile_f4*>(wp + (i >> G::LG_LPR) * G::RPL * G::ROWW +
                                             (i & ((1 << G::LG_LPR) - 1)) * (2 * TILE_LDS)) = pf[i];
             if (with_x) {
@@ -1000,8 +1013,13 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
             }
             wave_sync();
         };
-        auto sum_block = [&](int b) {
+        auto sum_block = [&](int b, int cols) {
             const int n_rt = min(G::RB, n_rows - b * G::RB) << G::LGT;  // (row, tile) pairs
+            // tiles of the stage, and elements of this lane's partial sum (the last tile
+            // of the last column stage may be narrower, later tiles are missing)
+            const int tiles_s = (cols + TILE - 1) >> 7;
+            const int in_tile = cols - tl * TILE;
+            const int count = in_tile >= TILE ? MAX_CHAIN : in_tile <= j ? 0 : (in_tile - j + 3) >> 2;
 #pragma unroll
             for (int p = 0; p < G::PASSES; ++p) {
                 // the passes one after the other: all their LDS reads at once would need
@@ -1009,9 +1027,17 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
                 if (p > 0) __builtin_amdgcn_sched_barrier(0);
                 if (p * 16 < n_rt) {  // uniform
                     float acc = 0.0f;
+                    if (!G::WIDE || cols == G::NCS) {
 #pragma unroll
-                    for (int m = 0; m < G::CHAIN; ++m)
-                        acc = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
+                        for (int m = 0; m < G::CHAIN; ++m)
+                            acc = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
+                    } else {
+#pragma unroll
+                        for (int m = 0; m < G::CHAIN; ++m) {
+                            const float next = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
+                            acc = m < count ? next : acc;
+                        }
+                    }
                     acc = acc + quad_xor(acc, 2);
                     acc = acc + quad_xor(acc, 1);
                     // tile sums, in order, onto the running sum of the row
@@ -1025,10 +1051,10 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
                         float* yp = ys + b * G::RB + ((p * 16 + rt) >> G::LGT);
                         float v = *yp;
                         v = v + cf.x * acc;
-                        if (G::TILES >= 2) v = v + cf.x * t1;
+                        if (G::TILES >= 2 && tiles_s > 1) v = v + cf.x * t1;
                         if (G::TILES == 4) {
-                            v = v + cf.x * t2;
-                            v = v + cf.x * t3;
+                            if (tiles_s > 2) v = v + cf.x * t2;
+                            if (tiles_s > 3) v = v + cf.x * t3;
                         }
                         *yp = v;
                     }
@@ -1054,15 +1080,17 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         int k = 0;   // stage whose block is in pf0
         int b = 0;   // its row block
         auto next_b = [&](int v) { return v + 1 == nb ? 0 : v + 1; };
+        // columns of stage q: only the stages of the last column stage can have fewer
+        auto cols_of = [&](int q) { return q >= n_stages - nb ? last_cols : G::NCS; };
         // stages k + 2 and k + 3 exist: both register sets are refilled without a branch
         while (k + 3 < n_stages) {
             const int b1 = next_b(b);
             store_block(pf0, xq0, G::WIDE ? b == 0 : k == 0);
             load_block(pf0, xq0);
-            sum_block(b);
+            sum_block(b, cols_of(k));
             store_block(pf1, xq1, G::WIDE && b1 == 0);
             load_block(pf1, xq1);
-            sum_block(b1);
+            sum_block(b1, cols_of(k + 1));
             b = next_b(b1);
             k += 2;
         }
@@ -1072,14 +1100,14 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
             const int b2 = next_b(b1);
             store_block(pf0, xq0, G::WIDE ? b == 0 : k == 0);
             if (k + 2 < n_stages) load_block(pf0, xq0);
-            sum_block(b);
+            sum_block(b, cols_of(k));
             if (k + 1 < n_stages) {
                 store_block(pf1, xq1, G::WIDE && b1 == 0);
-                sum_block(b1);
+                sum_block(b1, cols_of(k + 1));
             }
             if (k + 2 < n_stages) {
                 store_block(pf0, xq0, G::WIDE && b2 == 0);
-                sum_block(b2);
+                sum_block(b2, cols_of(k + 2));
             }
         }
     };

@@ -37,7 +37,7 @@ MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
 # dot products the large-item kernel with compile-time shapes takes: these widths, and
-# every power of two from STREAM_MIN_WIDE up; its LDS block has STREAM_STAGE_WORDS words
+# every multiple of 4 from STREAM_MIN_WIDE up; its LDS block has STREAM_STAGE_WORDS words
 STREAM_WIDTHS, STREAM_MIN_WIDE, STREAM_STAGE_WORDS = (32, 64), 512, 2176
 STREAM_NARROW_MAX_ROWS = 128
 WG, WAVE = 256, 64
@@ -209,11 +209,13 @@ class gemv_prog:
             pow2 = vec == 4 and all(
                 d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0
                 and d["a_stride0"] < 2 ** 22 for d in dots)
-            # second entry: 1 = every column count a power of two, 2 = ... and one of the
-            # widths the kernel with compile-time shapes is built for, 3 = ... and none
-            # of them wide (more waves fit a compute unit then)
-            stream = pow2 and TILE_STAGE_WORDS == STREAM_STAGE_WORDS and all(
-                d["a_shape1"] in STREAM_WIDTHS or d["a_shape1"] >= STREAM_MIN_WIDE for d in dots)
+            # second entry: 1 = every column count a power of two; 2 = every column count
+            # one the kernel with compile-time shapes is built for (32, 64, or a multiple
+            # of 4 from 512 up); 3 = ... and none of them wide (more waves fit a compute
+            # unit then)
+            stream = (vec == 4 and TILE_STAGE_WORDS == STREAM_STAGE_WORDS and dots and all(
+                d["a_stride0"] < 2 ** 22 and (d["a_shape1"] in STREAM_WIDTHS or (
+                    d["a_shape1"] >= STREAM_MIN_WIDE and d["a_shape1"] % 4 == 0)) for d in dots))
             if stream:
                 return (3, 3 if all(d["a_shape1"] in STREAM_WIDTHS for d in dots) else 2, vec)
             return (3, int(pow2), vec)

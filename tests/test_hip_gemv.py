@@ -363,19 +363,22 @@ def test_pow2_items_bit_exact(queue, beta):
 
 @pytest.mark.parametrize("beta", [1.0, 0.5])
 def test_compile_time_shape_items_bit_exact(queue, beta):
-    """Widths 32, 64 and powers of two from 512 up take the kernel whose stage shapes
-    are compile-time constants: row counts that leave partial row blocks, tasks of one
-    to many stages, outputs that sum dot products of several such widths, a Y_in
-    different from Y, and views with a row stride larger than the width and a strided
-    X -- bit-identical to the oracle."""
+    """Widths 32, 64 and multiples of 4 from 512 up take the kernel whose stage shapes
+    are compile-time constants: row counts that leave partial row blocks, widths that
+    leave a narrower last column stage, tasks of one to many stages, outputs that sum
+    dot products of several such widths, a Y_in different from Y, and views with a
+    row stride larger than the width and a strided X -- bit-identical to the oracle."""
     from nengo_ocl_amd import hipra_gemv as g
     from oracle import oracle as orc
 
     rng = np.random.RandomState(31337)
     shapes = [(999, 32), (513, 32), (8200, 32), (4096, 64), (777, 64), (2049, 64), (129, 64),
               (67, 512), (17, 512), (33, 1024), (64, 4096), (6, 4096), (9, 8192), (1, 16384),
-              (257, 2048), (3, 32768)]
-    multi = (64, 1024, 32, 512, 64)
+              (257, 2048), (3, 32768),
+              # wide, not a power of two: last column stages of 4 ... 508 columns
+              (32, 2000), (300, 9000), (5, 5000), (64, 516), (9, 1028), (40, 700), (7, 520),
+              (21, 1660), (130, 1020)]
+    multi = (64, 1024, 32, 512, 64, 2000, 644)
     mats = [rng.normal(size=s) for s in shapes] + [rng.normal(size=(300, n)) for n in multi]
     A = RA(mats, align=True)
     X = RA([rng.normal(size=m.shape[1]) for m in mats], align=True)
@@ -397,17 +400,17 @@ def test_compile_time_shape_items_bit_exact(queue, beta):
         for i in range(len(Y)):
             assert np.array_equal(got[i], Yo[i]), (i, use_yin)
 
-    # column blocks of a wider matrix (row stride 1200: widths 64, 512 and 32) times
+    # column blocks of a wider matrix (row stride 1200: widths 64, 600 and 32) times
     # every second / third element of longer vectors
     wide = rng.normal(size=(700, 1200)).astype(np.float32)
     Aw = RA([wide], align=True)
     Av = Aw[[0]]  # shares the buffer
     s0 = int(Aw.starts[0])
-    Av.add_views([s0, s0 + 64, s0 + 576], [700, 700, 700], [64, 512, 32], [1200] * 3, [1] * 3)
-    xs = [rng.normal(size=64 * 2), rng.normal(size=512 * 3), rng.normal(size=32)]
+    Av.add_views([s0, s0 + 64, s0 + 664], [700, 700, 700], [64, 600, 32], [1200] * 3, [1] * 3)
+    xs = [rng.normal(size=64 * 2), rng.normal(size=600 * 3), rng.normal(size=32)]
     Xw = RA(xs, align=True)
     Xv = Xw[[0]]
-    Xv.add_views([int(Xw.starts[0]), int(Xw.starts[1]), int(Xw.starts[2])], [64, 512, 32], [1] * 3,
+    Xv.add_views([int(Xw.starts[0]), int(Xw.starts[1]), int(Xw.starts[2])], [64, 600, 32], [1] * 3,
                  [2, 3, 1], [1] * 3)
     Yw = RA([rng.normal(size=700)], align=True)
     jA, jX = [np.array([1, 2, 3], dtype=np.int32)], [np.array([1, 2, 3], dtype=np.int32)]
@@ -419,8 +422,8 @@ def test_compile_time_shape_items_bit_exact(queue, beta):
     for plan in prog.plans:
         plan()
     assert np.array_equal(dY.to_host()[0], Yo[0])
-    expect = (beta * Yw[0][:, 0] + wide[:, :64] @ xs[0][::2] + wide[:, 64:576] @ xs[1][::3]
-              + wide[:, 576:608] @ xs[2])
+    expect = (beta * Yw[0][:, 0] + wide[:, :64] @ xs[0][::2] + wide[:, 64:664] @ xs[1][::3]
+              + wide[:, 664:696] @ xs[2])
     assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
 
 
