@@ -100,9 +100,14 @@ int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
  *   tasks : int32[n_tasks][24] {item, row0, n_rows, 0,  the item's row of `items` (8),
  *                               alpha, beta, gamma (float bits), 0,
  *                               the item's first row of `dots` (8; zeros without dots)}
- * `vec` as for nhip_gemv.  `pow2_cols` = 1 selects the streamlined kernel for
- * launches in which every dot product has a power-of-two column count >= 4
- * (log2_N set), vec == 4 and a_stride0 < 2^22; 0 = any shape. */
+ * `vec` as for nhip_gemv.  `pow2_cols` selects the kernel: 0 = any shape; 1 = every
+ * dot product of the launch has a power-of-two column count >= 4 (log2_N set),
+ * vec == 4 and a_stride0 < 2^22; 2 = every dot product has 32 or 64 columns
+ * (log2_N = 5 / 6) or a multiple of 4 from 512 up (any other log2_N), vec == 4,
+ * a_stride0 < 2^22 and blk_words == 2176: the kernel whose stage shapes are
+ * compile-time constants (fewest instructions per byte); 3 = as 2, but no dot
+ * product has more than 64 columns and no task more than 128 rows (a smaller LDS
+ * footprint and fewer registers: four waves per SIMD). */
 int nhip_gemv_tile(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
                    const float *coefs, const int *dots, const int *tasks, int n_tasks,
                    const float *A, const float *X, const float *Yin, float *Y);

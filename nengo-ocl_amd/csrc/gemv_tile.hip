@@ -814,8 +814,9 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
 // 8 KiB block on bookkeeping (the shape of every stage is worked out again from the
 // dot record, every load has its own 64-bit address arithmetic and predicate), and
 // with three or four waves per SIMD that, not HBM, is what bounds them.  Here the
-// column count of a stage is a template parameter (32, 64, or 512 for every power
-// of two from 512 up): all LDS addresses are immediates, a block's loads share one
+// column count of a stage is a template parameter (32, 64, or 512 for every column
+// count from 512 up that is a multiple of 4; the last column stage of such a dot
+// product may be narrower): all LDS addresses are immediates, a block's loads share one
 // scalar base and per-lane offsets that are set up once per dot product, tile sums
 // go from the lanes that hold them straight onto the running row sums, and the loop
 // over the stages of a dot product is written so that the loads of the register set
