@@ -876,7 +876,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
     const GemvTask task = ft.task;
     const GemvItem it = ft.item;
     const float4 cf = make_float4(ft.alpha, ft.beta, ft.gamma, 0.0f);
-    const int n_rows = task.n_rows;
+    const int n_rows = min(task.n_rows, SLOTS * NHIP_WAVE);  // the host keeps tasks within this
 
     // the filter targets: requested now, used after the first matrix loads have been
     // issued (no branch around the loads, see gemv_tile_p2_kernel)
@@ -1124,7 +1124,9 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         dot_of_width(std::true_type{}, ft.dot0);
         for (int d = 1; d < it.n_dots; ++d) dot_of_width(std::false_type{}, dots[it.dot_begin + d]);
     }
-    finish_task<EPI, SLOTS>(task, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
+    GemvTask done = task;
+    done.n_rows = n_rows;
+    finish_task<EPI, SLOTS>(done, it, cf, ys, ab, Yin, Y, epi, pop, v_in, w_in, fp, lane);
 }
 
 }  // namespace
