@@ -392,6 +392,15 @@ typedef struct NhipSeqOp {
  * lanes == 256, at most 128: their rows are staged in LDS (the library cannot read
  * the device table to check it). */
 int nhip_sequence(void *stream, const void *ops, int n_ops, int n_staged);
+/* The same with up to NHIP_SEQ_MAX_CHAINS chains side by side, a work-group each:
+ * `ops` holds the chains one after the other, chain c has chain_ops[c] operations
+ * (1 ... 16) and chain_staged[c] staged rows (HOST arrays).  Operations of different
+ * chains must not touch the same memory unless both only read it; inside a chain the
+ * order of `ops` holds.  No counterpart in the reference, which runs every plan as a
+ * launch of its own (plan.py:128-135). */
+#define NHIP_SEQ_MAX_CHAINS 4
+int nhip_sequence_chains(void *stream, const void *ops, const int *chain_ops,
+                         const int *chain_staged, int n_chains);
 
 /* ---- function nodes compiled at run time ----------------------------------
  * replaces: `plan_direct` (:954-1025), which builds an OpenCL program from the

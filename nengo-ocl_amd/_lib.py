@@ -64,6 +64,7 @@ SIGNATURES = {
     "nhip_probes": [P, P, c_int, c_int, P, P, P, P, P],
     "nhip_fill_i32": [P, P, c_int, c_int],
     "nhip_sequence": [P, P, c_int, c_int],
+    "nhip_sequence_chains": [P, P, P, P, c_int],
     "nhip_capture_begin": [P],
     "nhip_capture_end": [P, ctypes.POINTER(c_void_p)],
     "nhip_graph_launch": [P, P, c_int],

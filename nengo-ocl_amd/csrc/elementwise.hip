@@ -385,8 +385,19 @@ __device__ __forceinline__ int seq_row_words(int kind) {
     }
 }
 
-__global__ __launch_bounds__(NHIP_WG) void sequence_kernel(const NhipSeqOp* __restrict__ ops,
-                                                           int n_ops, int n_staged) {
+// Operations of a launch that touch different memory need not wait for each other:
+// the host sorts them into chains (operations that conflict share a chain, in their
+// order), and every chain gets a group of its own.
+struct SeqChains {
+    int first_op[NHIP_SEQ_MAX_CHAINS + 1];  // chain c runs ops[first_op[c] .. first_op[c + 1])
+    int n_staged[NHIP_SEQ_MAX_CHAINS];      // its rows staged in LDS
+};
+
+__global__ __launch_bounds__(NHIP_WG) void sequence_kernel(const NhipSeqOp* __restrict__ all_ops,
+                                                           SeqChains chains) {
+    const NhipSeqOp* ops = all_ops + chains.first_op[blockIdx.x];
+    const int n_ops = chains.first_op[blockIdx.x + 1] - chains.first_op[blockIdx.x];
+    const int n_staged = chains.n_staged[blockIdx.x];
     __shared__ NhipSeqOp s_ops[SEQ_MAX_OPS];
     __shared__ __attribute__((aligned(16))) int s_rows[SEQ_MAX_ROWS][SEQ_ROW_WORDS];
     const int tid = threadIdx.x;
@@ -602,12 +613,26 @@ extern "C" int nhip_fill_i32(void* stream, int* dst, int n, int value) {
     return 0;
 }
 
-extern "C" int nhip_sequence(void* stream, const void* ops, int n_ops, int n_staged) {
-    if (n_ops == 0) return 0;
-    if (n_ops < 0 || n_ops > SEQ_MAX_OPS || n_staged < 0 || n_staged > SEQ_MAX_ROWS || !ops)
+extern "C" int nhip_sequence_chains(void* stream, const void* ops, const int* chain_ops,
+                                    const int* chain_staged, int n_chains) {
+    if (n_chains == 0) return 0;
+    if (n_chains < 0 || n_chains > NHIP_SEQ_MAX_CHAINS || !ops || !chain_ops || !chain_staged)
         return NHIP_E_BADARG;
-    NHIP_LAUNCH(sequence_kernel, dim3(1), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
-                       reinterpret_cast<const NhipSeqOp*>(ops), n_ops, n_staged);
+    SeqChains chains = {};
+    for (int c = 0; c < n_chains; ++c) {
+        if (chain_ops[c] < 1 || chain_ops[c] > SEQ_MAX_OPS || chain_staged[c] < 0 ||
+            chain_staged[c] > SEQ_MAX_ROWS)
+            return NHIP_E_BADARG;
+        chains.first_op[c + 1] = chains.first_op[c] + chain_ops[c];
+        chains.n_staged[c] = chain_staged[c];
+    }
+    NHIP_LAUNCH(sequence_kernel, dim3(n_chains), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                       reinterpret_cast<const NhipSeqOp*>(ops), chains);
     NHIP_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int nhip_sequence(void* stream, const void* ops, int n_ops, int n_staged) {
+    if (n_ops == 0) return 0;
+    return nhip_sequence_chains(stream, ops, &n_ops, &n_staged, 1);
 }

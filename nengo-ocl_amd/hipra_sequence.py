@@ -100,8 +100,41 @@ def _conflict(p, q):
     return bool((wp & rq) or (wp & wq) or (rp & wq))
 
 
+MAX_CHAINS = 4
+
+
+def chains_of(plans):
+    """`plans` sorted into chains: plans that conflict (one writes what the other reads
+    or writes) share a chain and keep their order; chains are independent of each other
+    and can run side by side.  At most MAX_CHAINS: the shortest ones are joined."""
+    parent = list(range(len(plans)))
+
+    def find(i):
+        while parent[i] != i:
+            parent[i] = parent[parent[i]]
+            i = parent[i]
+        return i
+
+    for j in range(len(plans)):
+        for i in range(j):
+            if _conflict(plans[i], plans[j]):
+                parent[find(j)] = find(i)
+    groups = {}
+    for i in range(len(plans)):
+        groups.setdefault(find(i), []).append(i)
+    chains = sorted(groups.values(), key=lambda c: c[0])
+    while len(chains) > MAX_CHAINS:
+        chains.sort(key=len)
+        chains[0:2] = [sorted(chains[0] + chains[1])]
+        chains.sort(key=lambda c: c[0])
+    return [[plans[i] for i in chain] for chain in chains]
+
+
 def plan_sequence(queue, plans):
-    """One launch that runs `plans` (all small, see `is_small`) in order."""
+    """One launch that runs `plans` (all small, see `is_small`): in order where they
+    depend on each other, independent chains of them side by side (a group each)."""
+    chains = chains_of(plans)
+    plans = [p for chain in chains for p in chain]
     table = np.zeros(len(plans), dtype=SEQ_OP_DTYPE)
     for row, plan in zip(table, plans):
         kind, n, lanes, i0, d0, pointers = sequence_op(plan)
@@ -111,9 +144,14 @@ def plan_sequence(queue, plans):
     n_staged = int(table["n_blocks"][table["lanes"] == 256].sum())
     assert len(plans) <= MAX_OPS and n_staged <= MAX_STAGED_ROWS
     dev_table = to_device(queue, table.view(np.int32))
-    merged = Plan(queue, queue.lib.nhip_sequence, (dev_table.ptr, len(plans), n_staged), gsize=(256,),
-                  lsize=(256,), full_args=(dev_table,) + tuple(plans), name="hip_sequence",
-                  tag="+".join(p.name.replace("hip_", "") for p in plans))
+    chain_ops = (ctypes.c_int * len(chains))(*[len(c) for c in chains])
+    chain_staged = (ctypes.c_int * len(chains))(
+        *[sum(_staged_rows(sequence_op(p)) for p in c) for c in chains])
+    merged = Plan(queue, queue.lib.nhip_sequence_chains,
+                  (dev_table.ptr, chain_ops, chain_staged, len(chains)), gsize=(256 * len(chains),),
+                  lsize=(256,), full_args=(dev_table, chain_ops, chain_staged) + tuple(plans),
+                  name="hip_sequence",
+                  tag=" | ".join("+".join(p.name.replace("hip_", "") for p in c) for c in chains))
     merged.members = list(plans)
     bws = [p.bw_per_call for p in plans if p.bw_per_call]
     merged.bw_per_call = sum(bws) if bws else None

@@ -324,6 +324,38 @@ def test_small_plans_sink_and_merge(monkeypatch):
     assert not hs.is_small(wider) and not hs.is_small(deep) and not hs.is_small(many)
 
 
+def test_sequence_chains():
+    """The operations of a sequence launch are sorted into chains: conflicting ones
+    share a chain and keep their order, independent ones get chains of their own, and
+    more chains than the launch has groups for are joined."""
+    from nengo_ocl_amd import hipra_sequence as hs
+
+    class P:
+        def __init__(self, label, reads, writes):
+            self.label, self.reads_mem, self.writes_mem = label, set(reads), set(writes)
+
+    def labels(plans):
+        return [[p.label for p in chain] for chain in hs.chains_of(plans)]
+
+    clock, play, filt, probe = P("clock", "", "t"), P("play", "t", "n"), P("filter", "n", "m"), P("probe", "f", "p")
+    assert labels([clock, play, filt, probe]) == [["clock", "play", "filter"], ["probe"]]
+    # a later plan that touches two chains joins them; order inside the chain is the list's
+    both = P("both", "mp", "z")
+    assert labels([clock, probe, play, filt, both]) == [["clock", "probe", "play", "filter", "both"]]
+    # readers of the same memory do not conflict; two writers do
+    assert labels([P("a", "x", "u"), P("b", "x", "v"), P("c", "", "u")]) == [["a", "c"], ["b"]]
+    # six independent plans: four chains at most, every plan still there exactly once
+    many = [P(str(k), "", "abcdef"[k]) for k in range(6)]
+    chains = labels(many)
+    assert len(chains) == hs.MAX_CHAINS
+    assert sorted(l for c in chains for l in c) == [str(k) for k in range(6)]
+    assert all(c == sorted(c) for c in chains)
+    # a plan without memory sets conflicts with everything
+    class U:
+        label = "unknown"
+    assert labels([clock, U(), probe]) == [["clock", "unknown", "probe"]]
+
+
 def test_neurons_without_input_read_their_bias():
     """An ensemble without incoming connections: the copy of its bias into J goes away
     (the neurons read the bias directly); spikes are unchanged."""
