@@ -18,10 +18,14 @@
 //   LPR = 1: one lane per row, for items whose dot products all have <= 4 columns
 //            (vector sums, "scalar times vector" increments): the four partial sums are
 //            the (up to) four products themselves.
-// These launches are latency bound: the records of four dot products and, when those
-// have at most four columns, all their operands are fetched together before the sums
-// are formed in order.  Task, item and dot records are per-lane values on purpose
-// (different rows of a wave may belong to different items).
+// These launches are latency bound (a wave or two per SIMD, each a chain of dependent
+// reads): the records of four dot products and, when those have at most four columns,
+// all their operands are fetched together before the sums are formed in order; wider
+// dot products fetch the operands of 8 steps of a partial sum at a time; and what the
+// epilogue needs (population record, old neuron state, first filter target and its old
+// value) is requested as soon as the task is known, not after the sums.  Task, item and
+// dot records are per-lane values on purpose (different rows of a wave may belong to
+// different items).
 // EPI: what happens to a finished row besides being stored -- nothing, the LIF update
 // of the neuron whose input current the row is, or the step of the first-order filters
 // fed by the row (the same epilogues as the kernel for large items has; small
@@ -35,6 +39,7 @@ __device__ __forceinline__ void gemv_rows_ref_block(
 {
     constexpr int TILE = 128;
     constexpr int BATCH = 4;             // dot products whose operands are fetched together
+    constexpr int CHUNK = 8;             // steps of a partial sum whose operands are fetched together
     constexpr int ROWS = NHIP_WAVE / LPR;  // rows (tasks) per wave
     constexpr int PER_LANE = 4 / LPR;    // elements of a <= 4 column dot product per lane
     const int lane = tid & (NHIP_WAVE - 1);
@@ -46,6 +51,24 @@ __device__ __forceinline__ void gemv_rows_ref_block(
     const float4 cf = coefs[task.item];
     const int r = task.row0;
     const int n_dots = valid ? it.n_dots : 0;
+    // epilogue operands, fetched ahead (no branch around the loads: a row without a
+    // population or a target reads the first element of the buffer instead)
+    LifPop pop = {};
+    float v_old = 0.0f, w_old = 0.0f;
+    int2 f_range = make_int2(0, 0);
+    FilterTarget f_first = {};
+    float f_old = 0.0f;
+    if (EPI == EPI_LIF) {
+        pop = epi->lif.pops[task.item];
+        const bool enabled = pop.pflags & LIF_POP_ENABLED;
+        v_old = epi->lif.V[enabled ? (size_t)pop.v_start + r : 0];
+        w_old = epi->lif.W[enabled ? (size_t)pop.w_start + r : 0];
+    }
+    if (EPI == EPI_FILTER) {
+        f_range = epi->filter.item_targets[task.item];
+        f_first = epi->filter.targets[f_range.y > 0 ? f_range.x : 0];
+        f_old = epi->filter.F[f_range.y > 0 ? (size_t)f_first.y_start + r : 0];
+    }
     float sum = cf.y * Yin[it.yin_start + (size_t)r * it.yin_stride0];
 
     for (int d0 = 0; __any(d0 < n_dots); d0 += BATCH) {
@@ -97,7 +120,20 @@ __device__ __forceinline__ void gemv_rows_ref_block(
                 for (int c0 = 0; c0 < n_cols; c0 += TILE) {
                     const int c1 = min(c0 + TILE, n_cols);
                     float s = 0.0f;
-                    for (int c = c0 + lir; c < c1; c += 4) s = fmaf(arow[c], xg[(size_t)c * xs], s);
+                    // partial sum `lir`: columns c0 + lir, + 4, ... below c1, CHUNK of them
+                    // fetched at a time (past the end: the last column again, not used)
+                    for (int cb = c0 + lir; cb < c1; cb += 4 * CHUNK) {
+                        float av[CHUNK], xv[CHUNK];
+#pragma unroll
+                        for (int e = 0; e < CHUNK; ++e) {
+                            const int c = min(cb + 4 * e, c1 - 1);
+                            av[e] = arow[c];
+                            xv[e] = xg[(size_t)c * xs];
+                        }
+#pragma unroll
+                        for (int e = 0; e < CHUNK; ++e)
+                            if (cb + 4 * e < c1) s = fmaf(av[e], xv[e], s);
+                    }
                     s = s + __shfl_xor(s, 2, NHIP_WAVE);
                     s = s + __shfl_xor(s, 1, NHIP_WAVE);
                     sum = sum + cf.x * s;
@@ -108,15 +144,15 @@ __device__ __forceinline__ void gemv_rows_ref_block(
     if (lir == 0 && valid) {
         const float y = sum + cf.z;
         Y[it.y_start + (size_t)r * it.y_stride0] = y;
-        if (EPI == EPI_LIF) {
-            const LifPop pop = epi->lif.pops[task.item];
-            if (pop.pflags & LIF_POP_ENABLED) {
-                const float v = epi->lif.V[(size_t)pop.v_start + r];
-                const float w = epi->lif.W[(size_t)pop.w_start + r];
-                lif_epilogue(epi->lif, pop, r, y, v, w);
-            }
+        if (EPI == EPI_LIF && (pop.pflags & LIF_POP_ENABLED))
+            lif_epilogue(epi->lif, pop, r, y, v_old, w_old);
+        if (EPI == EPI_FILTER && f_range.y > 0) {
+            // the first target with what was fetched ahead (the arithmetic of
+            // filter_epilogue), further targets of the item from memory
+            const float bx = __fmul_rn(nhip_bits(f_first.b_bits), y);
+            epi->filter.F[(size_t)f_first.y_start + r] =
+                f_first.na ? __fsub_rn(bx, __fmul_rn(nhip_bits(f_first.a_bits), f_old)) : bx;
+            filter_epilogue(epi->filter, make_int2(f_range.x + 1, f_range.y - 1), r, y);
         }
-        if (EPI == EPI_FILTER)
-            filter_epilogue(epi->filter, epi->filter.item_targets[task.item], r, y);
     }
 }
