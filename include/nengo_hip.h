@@ -77,8 +77,9 @@ int nhip_device_info(int *n_cu, int *wave_size, int *lds_bytes, char *name, int 
  * 256 for flavor 0); `vec` = 4 (16-byte loads; needs a_start % 4 == 0 and
  * a_stride0 % 4 == 0 for every dot of the launch) or 1.  `passes` (flavor 0) =
  * rows each lane accumulates at once, i.e. independent loads in flight: 2, 4, 8,
- * or 0 for the class default.  The host validates these preconditions; the
- * kernel trusts them. */
+ * or 0 for the class default; (flavor 2) = 16 when the task records are the 16-word
+ * ones described with nhip_gemv_rows_lif, else 0.  The host validates these
+ * preconditions; the kernel trusts them. */
 int nhip_gemv(void *stream, int flavor, int lpr, int vec, int passes, const int *items,
               const float *coefs, const int *dots, const int *tasks, int n_tasks,
               const float *A, const float *X, const float *Yin, float *Y);
@@ -154,16 +155,26 @@ int nhip_gemv_tile_filter(void *stream, int vec, int pow2_cols, int blk_words, c
                           const int *item_targets, const int *targets, float *F);
 
 /* The same two epilogues for launches of small items (nhip_gemv with flavor 2, whose
- * `items`, `coefs`, `dots` and 4-int `tasks` tables these take; `lpr` 4 or 1): the
+ * `items`, `coefs`, `dots` and `tasks` tables these take; `lpr` 4 or 1): the
  * neuron update / filter step of a row runs in the lane that holds the row's sum.
- * `pops`, `item_targets`, `targets` and the other arguments as above. */
-int nhip_gemv_rows_lif(void *stream, int lpr, const int *items, const float *coefs,
+ * `pops`, `item_targets`, `targets` and the other arguments as above.
+ * `task_words` = 4: tasks as for nhip_gemv.  = 16: every task record also holds its
+ * item and coefficients (a launch of a few thousand rows is a chain of dependent
+ * reads, and this takes one out of it; nhip_gemv takes such tables for flavor 2
+ * with `passes` = 16):
+ *   tasks : int32[n_tasks][16] {item, row0, 1, e0,  the item's row of `items` with its
+ *                               last word = e1,  alpha, beta, gamma (float bits), e2}
+ * e0, e1, e2 let the epilogue start its own reads at once: nhip_gemv_rows_lif
+ * v_start, w_start, pflags of the item's row of `pops`; nhip_gemv_rows_filter first
+ * target, number of targets, 0; nhip_gemv 0, 0, 0. */
+int nhip_gemv_rows_lif(void *stream, int lpr, int task_words, const int *items, const float *coefs,
                        const int *dots, const int *tasks, int n_tasks, const float *A,
                        const float *X, const float *Yin, float *Y, const int *pops, double dt,
                        int upsample, float *V, float *W, float *S, const float *TAU,
                        const float *REF, const float *AMP);
-int nhip_gemv_rows_filter(void *stream, int lpr, const int *items, const float *coefs,
-                          const int *dots, const int *tasks, int n_tasks, const float *A,
+int nhip_gemv_rows_filter(void *stream, int lpr, int task_words, const int *items,
+                          const float *coefs, const int *dots, const int *tasks, int n_tasks,
+                          const float *A,
                           const float *X, const float *Yin, float *Y, const int *item_targets,
                           const int *targets, float *F);
 

@@ -223,51 +223,49 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
 }
 
 // ---------------------------------------------------------------- reference order, small items
-// (the kernel body lives in gemv_rows.h, shared with the sequence kernel)
-template <int LPR>
+// (the kernel body lives in gemv_rows.h)
+template <int LPR, bool WIDE>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     const float* A, const float* X, const float* Yin, float* Y)
 {
-    gemv_rows_ref_block<LPR>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y, blockIdx.x,
-                             threadIdx.x);
+    gemv_rows_ref_block<LPR, EPI_NONE, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
+                                             blockIdx.x, threadIdx.x);
 }
 
 // the same with an epilogue per finished row (A, X, Yin are not marked read-only
 // here either: the epilogue writes neuron state / filter outputs into the same buffer)
-template <int LPR, int EPI>
+template <int LPR, int EPI, bool WIDE>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_epi_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     const float* A, const float* X, const float* Yin, float* Y, const EpilogueArgs epi)
 {
-    gemv_rows_ref_block<LPR, EPI>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y, blockIdx.x,
-                                  threadIdx.x, &epi);
+    gemv_rows_ref_block<LPR, EPI, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
+                                        blockIdx.x, threadIdx.x, &epi);
 }
 
 template <int EPI>
-int launch_rows_epi(hipStream_t s, int lpr, const int* items, const float* coefs, const int* dots,
-                    const int* tasks, int n_tasks, const float* A, const float* X,
+int launch_rows_epi(hipStream_t s, int lpr, int task_words, const int* items, const float* coefs,
+                    const int* dots, const int* tasks, int n_tasks, const float* A, const float* X,
                     const float* Yin, float* Y, const EpilogueArgs& epi) {
     if (n_tasks == 0) return 0;
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (lpr != 4 && lpr != 1) return NHIP_E_BADCLASS;
+    if (task_words != 4 && task_words != 16) return NHIP_E_BADARG;
     const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
     const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
-    if (lpr == 4)
-        NHIP_LAUNCH((gemv_rows_ref_epi_kernel<4, EPI>), grid, dim3(NHIP_WG), 0, s,
-                           reinterpret_cast<const GemvItem*>(items),
-                           reinterpret_cast<const float4*>(coefs),
-                           reinterpret_cast<const GemvDot*>(dots),
-                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi);
-    else
-        NHIP_LAUNCH((gemv_rows_ref_epi_kernel<1, EPI>), grid, dim3(NHIP_WG), 0, s,
-                           reinterpret_cast<const GemvItem*>(items),
-                           reinterpret_cast<const float4*>(coefs),
-                           reinterpret_cast<const GemvDot*>(dots),
-                           reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi);
+    auto launch = [&](auto kernel) {
+        NHIP_LAUNCH(kernel, grid, dim3(NHIP_WG), 0, s, reinterpret_cast<const GemvItem*>(items),
+                    reinterpret_cast<const float4*>(coefs), reinterpret_cast<const GemvDot*>(dots),
+                    reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi);
+    };
+    if (lpr == 4 && task_words == 16) launch(gemv_rows_ref_epi_kernel<4, EPI, true>);
+    else if (lpr == 4) launch(gemv_rows_ref_epi_kernel<4, EPI, false>);
+    else if (task_words == 16) launch(gemv_rows_ref_epi_kernel<1, EPI, true>);
+    else launch(gemv_rows_ref_epi_kernel<1, EPI, false>);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -372,20 +370,19 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
         }
     } else if (flavor == 2) {
         if ((lpr != 4 && lpr != 1) || vec != 1) return NHIP_E_BADCLASS;
+        if (passes != 0 && passes != 16) return NHIP_E_BADARG;  // words of a task record
         const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
         const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
-        if (lpr == 4)
-            NHIP_LAUNCH(gemv_rows_ref_kernel<4>, grid, dim3(NHIP_WG), 0, s,
-                               reinterpret_cast<const GemvItem*>(items),
-                               reinterpret_cast<const float4*>(coefs),
-                               reinterpret_cast<const GemvDot*>(dots),
-                               reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
-        else
-            NHIP_LAUNCH(gemv_rows_ref_kernel<1>, grid, dim3(NHIP_WG), 0, s,
-                               reinterpret_cast<const GemvItem*>(items),
-                               reinterpret_cast<const float4*>(coefs),
-                               reinterpret_cast<const GemvDot*>(dots),
-                               reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
+        auto launch = [&](auto kernel) {
+            NHIP_LAUNCH(kernel, grid, dim3(NHIP_WG), 0, s, reinterpret_cast<const GemvItem*>(items),
+                        reinterpret_cast<const float4*>(coefs),
+                        reinterpret_cast<const GemvDot*>(dots),
+                        reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
+        };
+        if (lpr == 4 && passes == 16) launch(gemv_rows_ref_kernel<4, true>);
+        else if (lpr == 4) launch(gemv_rows_ref_kernel<4, false>);
+        else if (passes == 16) launch(gemv_rows_ref_kernel<1, true>);
+        else launch(gemv_rows_ref_kernel<1, false>);
         NHIP_LAUNCH_CHECK();
         return 0;
     } else if (flavor == 1) {
@@ -402,8 +399,9 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
     return NHIP_E_BADCLASS;
 }
 
-extern "C" int nhip_gemv_rows_lif(void* stream, int lpr, const int* items, const float* coefs,
-                                  const int* dots, const int* tasks, int n_tasks, const float* A,
+extern "C" int nhip_gemv_rows_lif(void* stream, int lpr, int task_words, const int* items,
+                                  const float* coefs, const int* dots, const int* tasks,
+                                  int n_tasks, const float* A,
                                   const float* X, const float* Yin, float* Y, const int* pops,
                                   double dt, int upsample, float* V, float* W, float* S,
                                   const float* TAU, const float* REF, const float* AMP) {
@@ -420,12 +418,13 @@ extern "C" int nhip_gemv_rows_lif(void* stream, int lpr, const int* items, const
     lif.TAU = TAU;
     lif.REF = REF;
     lif.AMP = AMP;
-    return launch_rows_epi<EPI_LIF>(static_cast<hipStream_t>(stream), lpr, items, coefs, dots,
-                                    tasks, n_tasks, A, X, Yin, Y, args);
+    return launch_rows_epi<EPI_LIF>(static_cast<hipStream_t>(stream), lpr, task_words, items, coefs,
+                                    dots, tasks, n_tasks, A, X, Yin, Y, args);
 }
 
-extern "C" int nhip_gemv_rows_filter(void* stream, int lpr, const int* items, const float* coefs,
-                                     const int* dots, const int* tasks, int n_tasks,
+extern "C" int nhip_gemv_rows_filter(void* stream, int lpr, int task_words, const int* items,
+                                     const float* coefs, const int* dots, const int* tasks,
+                                     int n_tasks,
                                      const float* A, const float* X, const float* Yin, float* Y,
                                      const int* item_targets, const int* targets, float* F) {
     if (!item_targets || !targets || !F) return NHIP_E_BADARG;
@@ -433,6 +432,6 @@ extern "C" int nhip_gemv_rows_filter(void* stream, int lpr, const int* items, co
     args.filter.item_targets = reinterpret_cast<const int2*>(item_targets);
     args.filter.targets = reinterpret_cast<const FilterTarget*>(targets);
     args.filter.F = F;
-    return launch_rows_epi<EPI_FILTER>(static_cast<hipStream_t>(stream), lpr, items, coefs, dots,
-                                       tasks, n_tasks, A, X, Yin, Y, args);
+    return launch_rows_epi<EPI_FILTER>(static_cast<hipStream_t>(stream), lpr, task_words, items,
+                                       coefs, dots, tasks, n_tasks, A, X, Yin, Y, args);
 }

@@ -30,7 +30,8 @@
 // of the neuron whose input current the row is, or the step of the first-order filters
 // fed by the row (the same epilogues as the kernel for large items has; small
 // populations and low-dimensional decoded values save a launch the same way).
-template <int LPR, int EPI = EPI_NONE>
+// WIDE: the task table holds GemvRowTask records.
+template <int LPR, int EPI = EPI_NONE, bool WIDE = false>
 __device__ __forceinline__ void gemv_rows_ref_block(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
@@ -46,9 +47,21 @@ __device__ __forceinline__ void gemv_rows_ref_block(
     const int lir = lane % LPR;
     const int slot = (block * (NHIP_WG / NHIP_WAVE) + (tid >> 6)) * ROWS + lane / LPR;
     const bool valid = slot < n_tasks;
-    const GemvTask task = tasks[valid ? slot : n_tasks - 1];
-    const GemvItem it = items[task.item];
-    const float4 cf = coefs[task.item];
+    GemvTask task;
+    GemvItem it;
+    float4 cf;
+    int wide_pad = 0;
+    if (WIDE) {
+        const GemvRowTask rt = reinterpret_cast<const GemvRowTask*>(tasks)[valid ? slot : n_tasks - 1];
+        task = rt.task;
+        it = rt.item;
+        cf = make_float4(rt.alpha, rt.beta, rt.gamma, 0.0f);
+        wide_pad = rt.pad;
+    } else {
+        task = tasks[valid ? slot : n_tasks - 1];
+        it = items[task.item];
+        cf = coefs[task.item];
+    }
     const int r = task.row0;
     const int n_dots = valid ? it.n_dots : 0;
     // epilogue operands, fetched ahead (no branch around the loads: a row without a
@@ -60,12 +73,14 @@ __device__ __forceinline__ void gemv_rows_ref_block(
     float f_old = 0.0f;
     if (EPI == EPI_LIF) {
         pop = epi->lif.pops[task.item];
-        const bool enabled = pop.pflags & LIF_POP_ENABLED;
-        v_old = epi->lif.V[enabled ? (size_t)pop.v_start + r : 0];
-        w_old = epi->lif.W[enabled ? (size_t)pop.w_start + r : 0];
+        // where the neuron's state is: from the task record if it says so (the state is
+        // then requested together with the population record, not after it)
+        const bool enabled = (WIDE ? wide_pad : pop.pflags) & LIF_POP_ENABLED;
+        v_old = epi->lif.V[enabled ? (size_t)(WIDE ? task.pad : pop.v_start) + r : 0];
+        w_old = epi->lif.W[enabled ? (size_t)(WIDE ? it.pad : pop.w_start) + r : 0];
     }
     if (EPI == EPI_FILTER) {
-        f_range = epi->filter.item_targets[task.item];
+        f_range = WIDE ? make_int2(task.pad, it.pad) : epi->filter.item_targets[task.item];
         f_first = epi->filter.targets[f_range.y > 0 ? f_range.x : 0];
         f_old = epi->filter.F[f_range.y > 0 ? (size_t)f_first.y_start + r : 0];
     }

@@ -16,3 +16,16 @@ struct GemvFatTask {
     float alpha, beta, gamma, pad;
     GemvDot dot0;
 };
+
+// Task record of the small-item kernel when a launch is short enough to be latency
+// bound (the host decides): the task with its item and coefficients inline, one read
+// instead of two dependent ones.  The spare fields carry what an epilogue needs to
+// start its own reads at once: with the LIF epilogue task.pad = v_start, item.pad =
+// w_start, pad = pflags of the item's population; with the filter epilogue task.pad =
+// first target, item.pad = number of targets.
+struct GemvRowTask {
+    GemvTask task;
+    GemvItem item;
+    float alpha, beta, gamma;
+    int pad;
+};

@@ -40,6 +40,9 @@ TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
 # every multiple of 4 from STREAM_MIN_WIDE up; its LDS block has STREAM_STAGE_WORDS words
 STREAM_WIDTHS, STREAM_MIN_WIDE, STREAM_STAGE_WORDS = (32, 64), 512, 2176
 STREAM_NARROW_MAX_ROWS = 128
+# small-item launches of at most this many rows get task records with the item and its
+# coefficients inline (they are chains of dependent reads; larger ones are about traffic)
+WIDE_TASK_MAX_ROWS = 65536
 WG, WAVE = 256, 64
 THIN_MIN_ROWS, THIN_ROWS_FOR_LANE_PER_ROW = 32, 65536
 LIF_POP_ENABLED, LIF_POP_DECAY = 1 << 8, 1 << 9  # flag bits of a population row
@@ -360,6 +363,15 @@ class gemv_prog:
                 task_tab[:, 2] = 1
                 task_rows = task_tab
             task_tab = np.array(task_rows, dtype=np.int32)
+            if flavor == 2 and 0 < len(task_tab) <= WIDE_TASK_MAX_ROWS:
+                which = task_tab[:, 0]
+                wide = np.zeros((len(task_tab), 16), dtype=np.int32)
+                wide[:, 0:4] = task_tab
+                wide[:, 4:12] = item_tab[which]
+                wide[:, 12:16] = coef_tab[which].view(np.int32)
+                wide[:, 15] = 0
+                task_tab = wide
+                passes = 16  # nhip_gemv: words of a task record
             if flavor == 3:
                 # one record per task with its item, coefficients and first dot product
                 # inline: a wave starts streaming after one read instead of three
@@ -399,7 +411,7 @@ class gemv_prog:
             plan.n_tasks = n_tasks
             plan.members = list(members)
             plan.prog = self
-            plan.host_tasks = task_tab if flavor == 3 else None
+            plan.host_tasks = task_tab if flavor == 3 or task_tab.shape[1] == 16 else None
             plans.append(plan)
         return plans
 
@@ -480,12 +492,23 @@ def _takes_epilogue(plan):
             and getattr(plan, "kernel_class", (None,))[0] in (2, 3))
 
 
-def _epilogue_call(lib, plan, kind):
-    """Entry point and leading arguments of `plan`'s launch with an epilogue."""
+def _epilogue_call(lib, plan, kind, extras=None):
+    """Entry point, leading arguments and device arrays to keep alive of `plan`'s launch
+    with an epilogue.  `extras(item indices) -> int32[n, 3]`: what the epilogue wants to
+    find in the spare words 3, 11, 15 of 16-word task records (small-item launches)."""
     if plan.kernel_class[0] == 3:
-        return getattr(lib, "nhip_gemv_tile_" + kind), plan.args
-    # nhip_gemv's (flavor, lpr, vec, passes, tables...) -> (lpr, tables...)
-    return getattr(lib, "nhip_gemv_rows_" + kind), (plan.args[1],) + tuple(plan.args[4:])
+        return getattr(lib, "nhip_gemv_tile_" + kind), plan.args, ()
+    # nhip_gemv's (flavor, lpr, vec, passes, items, coefs, dots, tasks, ...)
+    #   -> (lpr, task_words, items, coefs, dots, tasks, ...)
+    tables, keep = tuple(plan.args[4:]), ()
+    task_words = 16 if plan.host_tasks is not None else 4
+    if task_words == 16:
+        tasks = plan.host_tasks.copy()
+        tasks[:, [3, 11, 15]] = extras(tasks[:, 0])
+        dev_tasks = to_device(plan.queue, tasks)
+        tables = tables[:3] + (dev_tasks.ptr,) + tables[4:]
+        keep = (dev_tasks,)
+    return getattr(lib, "nhip_gemv_rows_" + kind), (plan.args[1], task_words) + tables, keep
 
 
 def fuse_lif(prog, lif_plan):
@@ -592,10 +615,11 @@ def fuse_lif(prog, lif_plan):
             out.append(plan)
             continue
         lif_bytes = sum(4 * int(J.shape0s[pop_of[b]]) for b in plan.members if b in pop_of)
-        entry, args = _epilogue_call(lib, plan, "lif")
+        entry, args, kept = _epilogue_call(lib, plan, "lif", lambda items: table[items][:, [0, 1, 7]])
         fused = Plan(queue, entry, args + lif_args, gsize=plan.gsize,
                      lsize=plan.lsize,
-                     full_args=plan.full_args + (dev_pops, V.dev_buf, W.dev_buf, S.dev_buf) + tuple(keep),
+                     full_args=(plan.full_args + (dev_pops, V.dev_buf, W.dev_buf, S.dev_buf)
+                                + tuple(keep) + kept),
                      name=plan.name + "_lif", tag=plan.tag,
                      bw_per_call=plan.bw_per_call + 5 * lif_bytes,  # V and W in and out, spikes out
                      flops_per_call=plan.flops_per_call)
@@ -703,8 +727,9 @@ def fuse_linearfilter(gemv_plans, lf_plan):
             continue
         f_bytes = sum(8 * int(Y.shape0s[b]) * len(targets_of[b]) for b in plan.members
                       if b in targets_of)  # filter state in and out
-        entry, args = _epilogue_call(lib, plan, "filter")
-        keep = ()
+        entry, args, keep = _epilogue_call(
+            lib, plan, "filter",
+            lambda items: np.column_stack([item_targets[items], np.zeros(len(items), np.int32)]))
         if plan.kernel_class[0] == 3:
             # the large-item kernel finds an item's range of targets in the spare
             # fields of its task records (one read less before it can start)
