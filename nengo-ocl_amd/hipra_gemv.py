@@ -28,6 +28,10 @@ from .utils import next_pow2
 
 # items with at most this many matrix elements go to the wave-per-task kernel
 SMALL_ITEM_ELEMS = 8192
+# ... and so do items of few rows up to four times that size: the large-item kernel
+# would give them a handful of waves that walk whole rows one after the other
+SHORT_ITEM_ROWS = int(os.environ.get("NENGO_HIP_SHORT_ITEM_ROWS", 128))
+SHORT_ITEM_ELEMS = 4 * SMALL_ITEM_ELEMS
 # ... and among those, rows up to this length use the reference-order wave kernel
 REF_ORDER_MAX_COLS = 512
 # float32 words of one wave's LDS block in the reference-order kernel for large items
@@ -207,7 +211,8 @@ class gemv_prog:
             # wave per task, large items staged through LDS by a work-group
             if dots and n_max <= 4 and M >= THIN_MIN_ROWS and self._many_thin_rows:
                 return (2, 1, 1)  # a lane per row: vector sums, scalar-times-vector terms
-            if M * n_sum <= SMALL_ITEM_ELEMS and n_max <= REF_ORDER_MAX_COLS:
+            if n_max <= REF_ORDER_MAX_COLS and (M * n_sum <= SMALL_ITEM_ELEMS or (
+                    M <= SHORT_ITEM_ROWS and M * n_sum <= SHORT_ITEM_ELEMS)):
                 return (2, 4, 1)
             pow2 = vec == 4 and all(
                 d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0

@@ -140,7 +140,8 @@ def test_ensemble_shapes(queue, pi):
     thin), decoders (d x n, short and wide), per-neuron scalars, single dots."""
     rng = np.random.RandomState(7)
     shapes = [(4096, 64), (64, 4096), (100, 1), (1, 100), (100, 2), (2, 100), (2000, 32),
-              (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000), (600, 128)]
+              (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000), (600, 128),
+              (300, 132)]
     A = RA([rng.normal(size=s) for s in shapes], align=True)
     X = RA([rng.normal(size=s[1]) for s in shapes], align=True)
     Y = RA([rng.normal(size=s[0]) for s in shapes], align=True)
@@ -373,7 +374,7 @@ def test_compile_time_shape_items_bit_exact(queue, beta):
 
     rng = np.random.RandomState(31337)
     shapes = [(999, 32), (513, 32), (8200, 32), (4096, 64), (777, 64), (2049, 64), (129, 64),
-              (67, 512), (17, 512), (33, 1024), (64, 4096), (6, 4096), (9, 8192), (1, 16384),
+              (67, 512), (131, 512), (33, 1024), (64, 4096), (6, 4096), (9, 8192), (1, 16384),
               (257, 2048), (3, 32768),
               # wide, not a power of two: last column stages of 4 ... 508 columns
               (32, 2000), (300, 9000), (5, 5000), (64, 516), (9, 1028), (40, 700), (7, 520),
@@ -530,7 +531,7 @@ def test_gemv_with_filter_epilogue(queue):
     from oracle import oracle as orc
 
     rng = np.random.RandomState(5)
-    shapes = [(64, 4096), (64, 2048), (100, 300), (16, 8), (80, 128)]
+    shapes = [(64, 4096), (64, 2048), (140, 300), (16, 8), (130, 128)]
     n = len(shapes)
     mats = [rng.normal(scale=0.1, size=s) for s in shapes]
     xs = [rng.normal(size=s[1]) for s in shapes]
