@@ -30,7 +30,7 @@ from .utils import next_pow2
 SMALL_ITEM_ELEMS = 8192
 # ... and so do items of few rows up to four times that size: the large-item kernel
 # would give them a handful of waves that walk whole rows one after the other
-SHORT_ITEM_ROWS = int(os.environ.get("NENGO_HIP_SHORT_ITEM_ROWS", 128))
+SHORT_ITEM_ROWS = int(os.environ.get("NENGO_HIP_SHORT_ITEM_ROWS", 256))
 SHORT_ITEM_ELEMS = 4 * SMALL_ITEM_ELEMS
 # ... and among those, rows up to this length use the reference-order wave kernel
 REF_ORDER_MAX_COLS = 512

@@ -373,7 +373,7 @@ def test_compile_time_shape_items_bit_exact(queue, beta):
     from oracle import oracle as orc
 
     rng = np.random.RandomState(31337)
-    shapes = [(999, 32), (513, 32), (8200, 32), (4096, 64), (777, 64), (2049, 64), (129, 64),
+    shapes = [(999, 32), (513, 32), (8200, 32), (4096, 64), (777, 64), (2049, 64), (257, 64),
               (67, 512), (131, 512), (33, 1024), (64, 4096), (6, 4096), (9, 8192), (1, 16384),
               (257, 2048), (3, 32768),
               # wide, not a power of two: last column stages of 4 ... 508 columns
@@ -531,7 +531,7 @@ def test_gemv_with_filter_epilogue(queue):
     from oracle import oracle as orc
 
     rng = np.random.RandomState(5)
-    shapes = [(64, 4096), (64, 2048), (140, 300), (16, 8), (130, 128)]
+    shapes = [(64, 4096), (64, 2048), (140, 300), (16, 8), (260, 128)]
     n = len(shapes)
     mats = [rng.normal(scale=0.1, size=s) for s in shapes]
     xs = [rng.normal(size=s[1]) for s in shapes]
