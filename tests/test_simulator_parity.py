@@ -161,6 +161,59 @@ def test_c3_large_reduced_spiking(queue, share):
         check_spiking(gpu, cpu, pg["spikes"], pc["spikes"], 1000, "c3 reduced (8 x 1024 x 64-D)")
 
 
+def test_c3_full_size_state_bit_exact(queue):
+    """The benchmark network at its full size (256 ensembles x 4096 LIF x 64-D, the
+    configuration the throughput is quoted on, surrogate decoders as in the benchmark):
+    after 40 steps every signal -- currents, voltages, refractory times, spikes, decoded
+    and filtered values -- and every probe sample is bit-identical to the oracle's, and
+    the step runs as the four launches the benchmark times."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    net, probes, _ = configs.c3_large()
+    net_o, probes_o, _ = configs.c3_large()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        names = [p.name for p in gpu._plans]
+        assert sorted(names) == ["hip_sequence", "hipra_gemv.tile_filter", "hipra_gemv.tile_lif",
+                                 "hipra_gemv.wave_ref"]
+        classes = {p.name: p.kernel_class for p in gpu._plans if hasattr(p, "kernel_class")}
+        assert classes["hipra_gemv.tile_lif"] == (3, 3, 4)     # compile-time shapes, narrow
+        assert classes["hipra_gemv.tile_filter"] == (3, 2, 4)  # compile-time shapes, wide
+        gpu.run_steps(40)
+        cpu.run_steps(40)
+        for key in probes:
+            assert np.array_equal(gpu.data[probes[key]], cpu.data[probes_o[key]]), key
+        got, want = np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf)
+        assert got.shape == want.shape and got.size > 140e6
+        assert np.array_equal(got, want)
+        assert all(np.any(gpu.data[probes[key]] != 0) for key in probes)  # something happened
+
+
+@pytest.mark.parametrize("case", ["c2", "c3-per-connection", "c4", "c5"])
+def test_other_configurations_full_size_state_bit_exact(queue, case):
+    """The other benchmark configurations at their full sizes (2048 ensembles on a
+    small-world graph; the 1.37 GB variant of the large network; 64 PES-learning
+    triples; one million neurons with sparse recurrent weights): every signal and
+    every probe sample bit-identical to the oracle's after 30 steps."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    make = {"c2": configs.c2_watts_strogatz,
+            "c3-per-connection": lambda: configs.c3_large(share_decoded=False),
+            "c4": configs.c4_pes,
+            "c5": lambda: configs.c5_sparse_recurrent(n_neurons=1000000)}[case]
+    net, probes, _ = make()
+    net_o, probes_o, _ = make()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        gpu.run_steps(30)
+        cpu.run_steps(30)
+        for key in probes:
+            assert np.array_equal(gpu.data[probes[key]], cpu.data[probes_o[key]]), key
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+
+
 def test_c4_pes_reduced(queue):
     """PES learning: weights after 1 s agree with the oracle's, and learning happened."""
     from nengo_ocl_amd import configs
