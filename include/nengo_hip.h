@@ -58,9 +58,10 @@ int nhip_device_info(int *n_cu, int *wave_size, int *lds_bytes, char *name, int 
  *                               dot_begin, n_dots, M, 0}
  *   coefs : float[n_items][4]  {alpha, beta, gamma, 0}
  *   dots  : int32[n_dots][8]   {a_start, a_stride0, N, x_start, x_stride0,
- *                               tile_rows, log2_N, 0}
+ *                               tile_rows, log2_N, stage}
  *                               (A rows are contiguous: a_stride1 == 1; the last
- *                               two are read by nhip_gemv_tile only: tile_rows =
+ *                               three are read by nhip_gemv_tile only (stage: with
+ *                               pow2_cols >= 2, see there): tile_rows =
  *                               nhip_gemv_tile_rows(N, blk_words), log2_N = the
  *                               exponent when N is a power of two, else -1)
  *   tasks : int32[n_tasks][4]  {item, row0, n_rows, 0}
@@ -103,12 +104,15 @@ int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
  *                               the item's first row of `dots` (8; zeros without dots)}
  * `vec` as for nhip_gemv.  `pow2_cols` selects the kernel: 0 = any shape; 1 = every
  * dot product of the launch has a power-of-two column count >= 4 (log2_N set),
- * vec == 4 and a_stride0 < 2^22; 2 = every dot product has 32 or 64 columns
- * (log2_N = 5 / 6) or a multiple of 4 from 512 up (any other log2_N), vec == 4,
- * a_stride0 < 2^22 and blk_words == 2176: the kernel whose stage shapes are
- * compile-time constants (fewest instructions per byte); 3 = as 2, but no dot
- * product has more than 64 columns and no task more than 128 rows (a smaller LDS
- * footprint and fewer registers: four waves per SIMD). */
+ * vec == 4 and a_stride0 < 2^22; 2 = every dot product has a multiple of 4 columns
+ * from 32 up, vec == 4, a_stride0 < 2^22 and blk_words == 2176: the kernel whose
+ * stage shapes are compile-time constants (fewest instructions per byte); the last
+ * word of a dots row then says which: 5 (N <= 32: stages of 32 columns, blocks of
+ * 32 rows), 6 (N <= 64: 64 columns, 32 rows), 7 (N < 512: 128 columns, 16 rows) or
+ * 9 (512 columns, 4 rows); tasks should be whole blocks.  The kernel comes in three
+ * instances: 3 = no dot product has more than 64 columns and no task more than 128
+ * rows (a smaller LDS footprint and fewer registers: four waves per SIMD); 2 = no
+ * stage 7; 4 = any. */
 int nhip_gemv_tile(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
                    const float *coefs, const int *dots, const int *tasks, int n_tasks,
                    const float *A, const float *X, const float *Yin, float *Y);

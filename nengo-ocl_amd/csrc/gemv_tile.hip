@@ -814,9 +814,10 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
 // 8 KiB block on bookkeeping (the shape of every stage is worked out again from the
 // dot record, every load has its own 64-bit address arithmetic and predicate), and
 // with three or four waves per SIMD that, not HBM, is what bounds them.  Here the
-// column count of a stage is a template parameter (32, 64, or 512 for every column
-// count from 512 up that is a multiple of 4; the last column stage of such a dot
-// product may be narrower): all LDS addresses are immediates, a block's loads share one
+// column count of a stage is a template parameter (32, 64, 128 or 512; the host picks
+// the smallest that holds the dot product, 128 for 68 ... 508 columns, 512 from there
+// up; the last or only column stage may be narrower, any multiple of 4): all LDS
+// addresses are immediates, a block's loads share one
 // scalar base and per-lane offsets that are set up once per dot product, tile sums
 // go from the lanes that hold them straight onto the running row sums, and the loop
 // over the stages of a dot product is written so that the loads of the register set
@@ -836,7 +837,7 @@ struct StreamGeo {
     static constexpr int NL = (RB / RPL) << LG_LPR;         // loads per lane and block
     static constexpr int CHAIN = LGC >= 7 ? MAX_CHAIN : NCS / 4;  // elements of a partial sum
     static constexpr int XL = NCS >= NHIP_WAVE ? NCS / NHIP_WAVE : 1;  // X loads per lane and stage
-    static constexpr bool WIDE = LGC >= 9;                  // several column stages: X travels with them
+    static constexpr bool MULTI = LGC >= 7;                 // several column stages: X travels with them
     static constexpr int PASSES = (RB * TILES + 15) / 16;   // (row, tile) pairs come 16 at a time
     static constexpr int PASS_WORDS = (16 >> LGT) * ROWW;
     static_assert(NL >= 1 && NL <= P2_PF && RB * ROWW <= 2176 && RB * TILES <= TSUM_WORDS, "block shape");
@@ -852,14 +853,17 @@ __device__ __forceinline__ float row_from_right(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x100 + N, 0xF, 0xF, true));
 }
 
-// WIDE: the launch has dot products of 512 columns or more (more registers and a
-// larger X block in LDS: three waves per SIMD instead of four).
-template <int EPI, bool WIDE>
-__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 3 : 4, 4))) void gemv_stream_kernel(
+// SET: the stage widths the launch needs -- 0: 32 and 64 columns only; 1: also 512
+// (more registers and a larger X block in LDS: three waves per SIMD instead of four);
+// 2: also 128.  An instance that holds fewer shapes needs fewer registers, and the
+// large matrices of the benchmark networks need only 0 and 1.
+template <int EPI, int SET>
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(SET ? 3 : 4, 4))) void gemv_stream_kernel(
     const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
     float* Y, EpilogueArgs epi)
 {
+    constexpr bool WIDE = SET >= 1;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -928,13 +932,16 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
     };
 
     // all stages of one dot product: column stages outside, row blocks inside
-    auto dot_pass = [&](auto lgc_tag, auto first_tag, const GemvDot& dot) {
+    // ragged_tag: the column count is not a multiple of the stage width (the last or
+    // only column stage is narrower); without it no column is ever tested
+    auto dot_pass = [&](auto lgc_tag, auto first_tag, auto ragged_tag, const GemvDot& dot) {
         using G = StreamGeo<decltype(lgc_tag)::value>;
+        constexpr bool RAGGED = decltype(ragged_tag)::value;
         const int nb = (n_rows + G::RB - 1) / G::RB;            // row blocks of the task
-        // wide dot products: any column count that is a multiple of 4; the last column
-        // stage then has last_cols < NCS columns
-        const int n_col = G::WIDE ? (dot.N + G::NCS - 1) >> G::LG_COLS : 1;
-        const int last_cols = G::WIDE ? dot.N - (n_col - 1) * G::NCS : G::NCS;
+        // any column count that is a multiple of 4: the last (or only) column stage has
+        // last_cols <= NCS columns
+        const int n_col = G::MULTI ? (dot.N + G::NCS - 1) >> G::LG_COLS : 1;
+        const int last_cols = RAGGED ? dot.N - (n_col - 1) * G::NCS : G::NCS;
         const int n_stages = nb * n_col;
         const unsigned stride4 = 4u * (unsigned)dot.a_stride0;  // bytes between rows
         const char* const a0 = reinterpret_cast<const char*>(
@@ -959,8 +966,8 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         int l_c0 = 0;                // its first column
         const char* l_ptr = a0;      // its first byte
         auto load_block = [&](tile_f4 (&pf)[G::NL], float (&xq)[G::XL]) {
-            const int cols = G::WIDE ? min(G::NCS, dot.N - l_c0) : G::NCS;
-            if (G::WIDE) {
+            const int cols = RAGGED ? min(G::NCS, dot.N - l_c0) : G::NCS;
+            if (G::MULTI) {
                 const float* xg = x0 + (size_t)l_c0 * dot.x_stride0;
                 if (cols == G::NCS) {
 #pragma unroll
@@ -1014,7 +1021,8 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
             }
             wave_sync();
         };
-        auto sum_block = [&](int b, int cols) {
+        auto sum_block = [&](int b, int cols_in) {
+            const int cols = RAGGED ? cols_in : G::NCS;
             const int n_rt = min(G::RB, n_rows - b * G::RB) << G::LGT;  // (row, tile) pairs
             // tiles of the stage, and elements of this lane's partial sum (the last tile
             // of the last column stage may be narrower, later tiles are missing)
@@ -1028,13 +1036,19 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
                 if (p > 0) __builtin_amdgcn_sched_barrier(0);
                 if (p * 16 < n_rt) {  // uniform
                     float acc = 0.0f;
-                    if (!G::WIDE || cols == G::NCS) {
+                    if (cols == G::NCS) {
 #pragma unroll
-                        for (int m = 0; m < G::CHAIN; ++m)
+                        for (int m = 0; m < G::CHAIN; ++m) {
+                            // 128-column stages: the operands in two batches (registers)
+                            if (G::LG_COLS == 7 && m == G::CHAIN / 2) __builtin_amdgcn_sched_barrier(0);
                             acc = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
+                        }
                     } else {
 #pragma unroll
                         for (int m = 0; m < G::CHAIN; ++m) {
+                            // (eight steps at a time: this path is rare and must not be
+                            // what sets the kernel's register count)
+                            if (m % 8 == 0 && m > 0) __builtin_amdgcn_sched_barrier(0);
                             const float next = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
                             acc = m < count ? next : acc;
                         }
@@ -1072,10 +1086,10 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
             l_ptr = a0;
         }
         load_block(pf1, xq1);
-        if (!G::WIDE) {  // one column stage: its X is fetched once
+        if (!G::MULTI) {  // one column stage: its X is fetched once
 #pragma unroll
             for (int i = 0; i < G::XL; ++i)
-                xq0[i] = x0[(size_t)min(lane + i * NHIP_WAVE, G::NCS - 1) * dot.x_stride0];
+                xq0[i] = x0[(size_t)min(lane + i * NHIP_WAVE, last_cols - 1) * dot.x_stride0];
         }
         if (decltype(first_tag)::value) after_first_loads();
         int k = 0;   // stage whose block is in pf0
@@ -1086,10 +1100,10 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         // stages k + 2 and k + 3 exist: both register sets are refilled without a branch
         while (k + 3 < n_stages) {
             const int b1 = next_b(b);
-            store_block(pf0, xq0, G::WIDE ? b == 0 : k == 0);
+            store_block(pf0, xq0, G::MULTI ? b == 0 : k == 0);
             load_block(pf0, xq0);
             sum_block(b, cols_of(k));
-            store_block(pf1, xq1, G::WIDE && b1 == 0);
+            store_block(pf1, xq1, G::MULTI && b1 == 0);
             load_block(pf1, xq1);
             sum_block(b1, cols_of(k + 1));
             b = next_b(b1);
@@ -1099,30 +1113,37 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(WIDE ? 
         {
             const int b1 = next_b(b);
             const int b2 = next_b(b1);
-            store_block(pf0, xq0, G::WIDE ? b == 0 : k == 0);
+            store_block(pf0, xq0, G::MULTI ? b == 0 : k == 0);
             if (k + 2 < n_stages) load_block(pf0, xq0);
             sum_block(b, cols_of(k));
             if (k + 1 < n_stages) {
-                store_block(pf1, xq1, G::WIDE && b1 == 0);
+                store_block(pf1, xq1, G::MULTI && b1 == 0);
                 sum_block(b1, cols_of(k + 1));
             }
             if (k + 2 < n_stages) {
-                store_block(pf0, xq0, G::WIDE && b2 == 0);
+                store_block(pf0, xq0, G::MULTI && b2 == 0);
                 sum_block(b2, cols_of(k + 2));
             }
         }
     };
 
-    auto dot_of_width = [&](auto first_tag, const GemvDot& dot) {
-        if (dot.p1 == 5) dot_pass(std::integral_constant<int, 5>{}, first_tag, dot);
-        else if (!WIDE || dot.p1 == 6) dot_pass(std::integral_constant<int, 6>{}, first_tag, dot);
-        else dot_pass(std::integral_constant<int, 9>{}, first_tag, dot);
+    // dot.p2: the stage width the host chose for the dot product (log2: 5, 6, 7 or 9)
+    auto dot_of_width = [&](auto first_tag, auto ragged_tag, const GemvDot& dot) {
+        if (dot.p2 == 5) dot_pass(std::integral_constant<int, 5>{}, first_tag, ragged_tag, dot);
+        else if (!WIDE || dot.p2 == 6) dot_pass(std::integral_constant<int, 6>{}, first_tag, ragged_tag, dot);
+        else if (SET == 2 && dot.p2 == 7) dot_pass(std::integral_constant<int, 7>{}, first_tag, ragged_tag, dot);
+        else dot_pass(std::integral_constant<int, 9>{}, first_tag, ragged_tag, dot);
     };
+    // column count a multiple of its stage width (the stage width is 1 << p2)
+    auto whole_stages = [&](const GemvDot& dot) { return (dot.N & ((1 << dot.p2) - 1)) == 0; };
     if (it.n_dots == 0) {
         after_first_loads();
     } else {
-        dot_of_width(std::true_type{}, ft.dot0);
-        for (int d = 1; d < it.n_dots; ++d) dot_of_width(std::false_type{}, dots[it.dot_begin + d]);
+        if (whole_stages(ft.dot0)) dot_of_width(std::true_type{}, std::false_type{}, ft.dot0);
+        else dot_of_width(std::true_type{}, std::true_type{}, ft.dot0);
+        // further dot products of an item: the general form
+        for (int d = 1; d < it.n_dots; ++d)
+            dot_of_width(std::false_type{}, std::true_type{}, dots[it.dot_begin + d]);
     }
     GemvTask done = task;
     done.n_rows = n_rows;
@@ -1147,7 +1168,7 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
-    if (pow2_cols != 0 && (pow2_cols < 1 || pow2_cols > 3 || vec != 4)) return NHIP_E_BADCLASS;
+    if (pow2_cols != 0 && (pow2_cols < 1 || pow2_cols > 4 || vec != 4)) return NHIP_E_BADCLASS;
     if (pow2_cols >= 2 && blk_words != STREAM_BLK_WORDS) return NHIP_E_BADARG;
     const int stream_xb = pow2_cols == 3 ? STREAM_NARROW_XB_WORDS : XBLK_WORDS;
     if (blk_words < (STAGE_COLS / TILE) * TILE_LDS || (blk_words & 3)) return NHIP_E_BADARG;
@@ -1173,17 +1194,16 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     };
     auto launch_epi = [&](auto epi_tag) {
         constexpr int E = decltype(epi_tag)::value;
-        if (pow2_cols == 2) {
-            NHIP_LAUNCH((gemv_stream_kernel<E, true>), dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+        auto launch_stream = [&](auto kernel) {
+            NHIP_LAUNCH(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
                         reinterpret_cast<const GemvDot*>(dots),
                         reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, stream_xb, A, X, Yin,
                         Y, args);
-        } else if (pow2_cols == 3) {
-            NHIP_LAUNCH((gemv_stream_kernel<E, false>), dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
-                        reinterpret_cast<const GemvDot*>(dots),
-                        reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, stream_xb, A, X, Yin,
-                        Y, args);
-        } else if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
+        };
+        if (pow2_cols == 2) launch_stream(gemv_stream_kernel<E, 1>);
+        else if (pow2_cols == 3) launch_stream(gemv_stream_kernel<E, 0>);
+        else if (pow2_cols == 4) launch_stream(gemv_stream_kernel<E, 2>);
+        else if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
         else if (vec == 4) launch(gemv_tile_kernel<4, E>);
         else launch(gemv_tile_kernel<1, E>);
     };

@@ -40,10 +40,23 @@ TILE_STAGE_WORDS = int(os.environ.get("NENGO_HIP_TILE_WORDS", 2176))
 MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
-# dot products the large-item kernel with compile-time shapes takes: these widths, and
-# every multiple of 4 from STREAM_MIN_WIDE up; its LDS block has STREAM_STAGE_WORDS words
-STREAM_WIDTHS, STREAM_MIN_WIDE, STREAM_STAGE_WORDS = (32, 64), 512, 2176
+# The large-item kernel with compile-time shapes takes dot products whose column count
+# is a multiple of 4 from STREAM_MIN_COLS up; its LDS block has STREAM_STAGE_WORDS words.
+STREAM_MIN_COLS, STREAM_STAGE_WORDS = 32, 2176
 STREAM_NARROW_MAX_ROWS = 128
+
+
+def stream_stage(n_cols):
+    """(log2 of the stage width, rows of a block) the kernel with compile-time shapes
+    uses for a dot product of `n_cols` columns: the smallest stage that holds it, 128
+    columns wide from 68 to 508 columns, 512 from there up."""
+    if n_cols <= 32:
+        return 5, 32
+    if n_cols <= 64:
+        return 6, 32
+    if n_cols < 512:
+        return 7, 16
+    return 9, 4
 # small-item launches of at most this many rows get task records with the item and its
 # coefficients inline (they are chains of dependent reads; larger ones are about traffic)
 WIDE_TASK_MAX_ROWS = 65536
@@ -217,15 +230,16 @@ class gemv_prog:
             pow2 = vec == 4 and all(
                 d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0
                 and d["a_stride0"] < 2 ** 22 for d in dots)
-            # second entry: 1 = every column count a power of two; 2 = every column count
-            # one the kernel with compile-time shapes is built for (32, 64, or a multiple
-            # of 4 from 512 up); 3 = ... and none of them wide (more waves fit a compute
-            # unit then)
+            # second entry: 1 = every column count a power of two; 2, 3, 4 = every column
+            # count a multiple of 4 from 32 up (the kernel with compile-time shapes): 3 =
+            # none above 64 (more waves fit a compute unit then), 2 = none from 68 to 508,
+            # 4 = any
             stream = (vec == 4 and TILE_STAGE_WORDS == STREAM_STAGE_WORDS and dots and all(
-                d["a_stride0"] < 2 ** 22 and (d["a_shape1"] in STREAM_WIDTHS or (
-                    d["a_shape1"] >= STREAM_MIN_WIDE and d["a_shape1"] % 4 == 0)) for d in dots))
+                d["a_stride0"] < 2 ** 22 and d["a_shape1"] >= STREAM_MIN_COLS
+                and d["a_shape1"] % 4 == 0 for d in dots))
             if stream:
-                return (3, 3 if all(d["a_shape1"] in STREAM_WIDTHS for d in dots) else 2, vec)
+                stages = {stream_stage(d["a_shape1"])[0] for d in dots}
+                return (3, 4 if 7 in stages else 2 if 9 in stages else 3, vec)
             return (3, int(pow2), vec)
         if flavor == 0:
             # Matrix loads are non-temporal, so one wave instruction should take whole
@@ -244,7 +258,7 @@ class gemv_prog:
             lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         return (flavor, lpr, vec)
 
-    def _tile_tasks(self, members, max_rows=256):
+    def _tile_tasks(self, members, max_rows=256, stream=False):
         """Tasks (item, first row, rows, 0) of the reference-order kernel for large items.
 
         A task is the rows one wave carries through all columns, a few row blocks of
@@ -255,7 +269,8 @@ class gemv_prog:
         give enough tasks, the one with the least uneven spread wins.
         """
         lib, geometry = self.queue.lib, self.geometry
-        blk = {b: min([lib.nhip_gemv_tile_rows(dd["a_shape1"], TILE_STAGE_WORDS)
+        blk = {b: min([stream_stage(dd["a_shape1"])[1] if stream else
+                       lib.nhip_gemv_tile_rows(dd["a_shape1"], TILE_STAGE_WORDS)
                        for dd in geometry[b]["dots"]] or [WAVE]) for b in members}
 
         def tasks_for(per_task):
@@ -300,7 +315,8 @@ class gemv_prog:
                 n = d["a_shape1"]
                 log2_n = n.bit_length() - 1 if n > 0 and n & (n - 1) == 0 else -1
                 dot_rows.append((d["a_start"], d["a_stride0"], n, d["x_start"], d["x_stride0"],
-                                 lib.nhip_gemv_tile_rows(n, TILE_STAGE_WORDS), log2_n, 0))
+                                 lib.nhip_gemv_tile_rows(n, TILE_STAGE_WORDS), log2_n,
+                                 stream_stage(n)[0]))
         dot_tab = np.array(dot_rows or [(0,) * 8], dtype=np.int32)
 
         # Items whose dot products have at most four columns (sums of vectors, scalar
@@ -321,10 +337,13 @@ class gemv_prog:
 
         # items without dot products (class (3, 1, 4)) ride with the launch of the
         # compile-time-shape kernel when there is one
-        # ... whose narrow items join the wide ones when both kinds are there
-        if (3, 2, 4) in by_class and (3, 3, 4) in by_class:
-            by_class[(3, 2, 4)] = sorted(by_class[(3, 2, 4)] + by_class.pop((3, 3, 4)))
-        stream = (3, 2, 4) if (3, 2, 4) in by_class else (3, 3, 4)
+        # ... and the launch of the instance that holds more stage widths takes the items
+        # of the ones that hold fewer, when several are there
+        for wider, narrower in (((3, 4, 4), (3, 2, 4)), ((3, 4, 4), (3, 3, 4)),
+                                ((3, 2, 4), (3, 3, 4))):
+            if wider in by_class and narrower in by_class:
+                by_class[wider] = sorted(by_class[wider] + by_class.pop(narrower))
+        stream = next((c for c in ((3, 4, 4), (3, 2, 4), (3, 3, 4)) if c in by_class), (3, 3, 4))
         if stream in by_class and (3, 1, 4) in by_class:
             bare = [b for b in by_class[(3, 1, 4)] if not geometry[b]["dots"]]
             by_class[stream] = sorted(by_class[stream] + bare)
@@ -353,7 +372,8 @@ class gemv_prog:
             if flavor == 3:
                 # launches without wide dot products keep tasks to 128 rows (the kernel
                 # then needs fewer registers and a fourth wave fits each SIMD)
-                task_rows = self._tile_tasks(members, STREAM_NARROW_MAX_ROWS if lpr == 3 else 256)
+                task_rows = self._tile_tasks(members, STREAM_NARROW_MAX_ROWS if lpr == 3 else 256,
+                                             stream=lpr >= 2)
             else:
                 task_rows = []
                 for b in (members if flavor != 2 else ()):

@@ -140,8 +140,8 @@ def test_ensemble_shapes(queue, pi):
     thin), decoders (d x n, short and wide), per-neuron scalars, single dots."""
     rng = np.random.RandomState(7)
     shapes = [(4096, 64), (64, 4096), (100, 1), (1, 100), (100, 2), (2, 100), (2000, 32),
-              (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000), (600, 128),
-              (300, 132)]
+              (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000), (600, 16),
+              (600, 20)]
     A = RA([rng.normal(size=s) for s in shapes], align=True)
     X = RA([rng.normal(size=s[1]) for s in shapes], align=True)
     Y = RA([rng.normal(size=s[0]) for s in shapes], align=True)
@@ -149,8 +149,8 @@ def test_ensemble_shapes(queue, pi):
     prog = run_case(queue, planners()[pi], 1.0, 1.0, 0.0, A, X, Y, js, js)
     if pi == 0:
         classes = {p.kernel_class for p in prog.plans}
-        # widths 32 / 64 / >= 512 (compile-time shapes; 2: some of them wide), other powers of
-        # two, any width, small
+        # multiples of 4 from 32 up (compile-time shapes; 2: none from 68 to 508 columns),
+        # smaller powers of two, any width, small
         assert classes == {(3, 2, 4), (3, 1, 4), (3, 0, 4), (2, 4, 1)}
 
 
@@ -335,7 +335,7 @@ def test_pow2_items_bit_exact(queue, beta):
     orc.plan_block_gemv(None, 1.0, A, js, X, js, beta, Yo).plans[0]()
     dY = to_dev(queue, Y)
     prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY)
-    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4), (3, 2, 4)}
+    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4), (3, 4, 4)}
     for plan in prog.plans:
         plan()
     got = dY.to_host()
@@ -354,7 +354,7 @@ def test_pow2_items_bit_exact(queue, beta):
     orc.plan_block_gemv(None, 1.0, Av, jA, Xw, jX, beta, Yo).plans[0]()
     dY = to_dev(queue, Yw)
     prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, Av), jA, to_dev(queue, Xw), jX, beta, dY)
-    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4)}
+    assert {p.kernel_class for p in prog.plans} == {(3, 4, 4)}
     for plan in prog.plans:
         plan()
     assert np.array_equal(dY.to_host()[0], Yo[0])
@@ -363,23 +363,32 @@ def test_pow2_items_bit_exact(queue, beta):
 
 
 @pytest.mark.parametrize("beta", [1.0, 0.5])
-def test_compile_time_shape_items_bit_exact(queue, beta):
-    """Widths 32, 64 and multiples of 4 from 512 up take the kernel whose stage shapes
-    are compile-time constants: row counts that leave partial row blocks, widths that
-    leave a narrower last column stage, tasks of one to many stages, outputs that sum
-    dot products of several such widths, a Y_in different from Y, and views with a
-    row stride larger than the width and a strided X -- bit-identical to the oracle."""
+@pytest.mark.parametrize("widths", ["to-64", "to-64-and-from-512", "all"])
+def test_compile_time_shape_items_bit_exact(queue, beta, widths):
+    """Column counts that are multiples of 4 from 32 up take the kernel whose stage
+    shapes are compile-time constants (stages of 32, 64, 128 or 512 columns; one
+    instance per set of stage widths a launch needs): row counts that leave partial
+    row blocks, widths that leave a narrower last or only column stage, tasks of one to
+    many stages, outputs that sum dot products of several such widths, a Y_in different
+    from Y -- bit-identical to the oracle."""
     from nengo_ocl_amd import hipra_gemv as g
     from oracle import oracle as orc
 
     rng = np.random.RandomState(31337)
-    shapes = [(999, 32), (513, 32), (8200, 32), (4096, 64), (777, 64), (2049, 64), (257, 64),
-              (67, 512), (131, 512), (33, 1024), (64, 4096), (6, 4096), (9, 8192), (1, 16384),
-              (257, 2048), (3, 32768),
-              # wide, not a power of two: last column stages of 4 ... 508 columns
-              (32, 2000), (300, 9000), (5, 5000), (64, 516), (9, 1028), (40, 700), (7, 520),
-              (21, 1660), (130, 1020)]
-    multi = (64, 1024, 32, 512, 64, 2000, 644)
+    narrow = [(999, 32), (513, 32), (8200, 32), (4096, 64), (777, 64), (2049, 64), (257, 64),
+              (1000, 36), (700, 48), (4100, 60), (300, 52), (2000, 44)]
+    wide = [(67, 512), (131, 512), (33, 1024), (64, 4096), (6, 4096), (9, 8192), (1, 16384),
+            (257, 2048), (3, 32768),
+            # not a power of two: last column stages of 4 ... 508 columns
+            (32, 2000), (300, 9000), (5, 5000), (64, 516), (9, 1028), (40, 700), (7, 520),
+            (21, 1660), (130, 1020)]
+    middle = [(301, 128), (130, 256), (700, 100), (300, 132), (260, 300), (1000, 500), (90, 508),
+              (513, 68), (400, 260)]
+    shapes, multi, expected = {
+        "to-64": (narrow, (64, 32, 48, 64, 36), (3, 3, 4)),
+        "to-64-and-from-512": (narrow + wide, (64, 1024, 32, 512, 64, 2000, 644, 40), (3, 2, 4)),
+        "all": (narrow + wide + middle, (64, 1024, 300, 32, 512, 128, 2000, 68), (3, 4, 4)),
+    }[widths]
     mats = [rng.normal(size=s) for s in shapes] + [rng.normal(size=(300, n)) for n in multi]
     A = RA(mats, align=True)
     X = RA([rng.normal(size=m.shape[1]) for m in mats], align=True)
@@ -394,13 +403,21 @@ def test_compile_time_shape_items_bit_exact(queue, beta):
         dY = to_dev(queue, Y)
         prog = g.plan_block_gemv(queue, 0.75, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY,
                                  Y_in=to_dev(queue, Yin) if use_yin else None, gamma=0.125)
-        assert {p.kernel_class for p in prog.plans} == {(3, 2, 4)}
+        assert {p.kernel_class for p in prog.plans} == {expected}
         for plan in prog.plans:
             plan()
         got = dY.to_host()
         for i in range(len(Y)):
             assert np.array_equal(got[i], Yo[i]), (i, use_yin)
 
+
+@pytest.mark.parametrize("beta", [1.0, 0.5])
+def test_compile_time_shape_views_bit_exact(queue, beta):
+    """Matrix views with a row stride larger than the width and strided X vectors."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(4711)
     # column blocks of a wider matrix (row stride 1200: widths 64, 600 and 32) times
     # every second / third element of longer vectors
     wide = rng.normal(size=(700, 1200)).astype(np.float32)
@@ -443,7 +460,7 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     rng = np.random.RandomState(31)
     dt = 1e-3
     # GEMV items: four large ones with neurons, a small one with neurons, a large one without
-    shapes = [(4096, 64), (1000, 128), (3000, 48), (520, 130), (60, 8), (300, 64)]
+    shapes = [(4096, 64), (1000, 16), (3000, 28), (520, 130), (60, 8), (300, 64)]
     pop_sizes = [4096, 1000, 3000, 520, 60, 700]  # the last population has no input item
     n, n_pop = len(shapes), len(pop_sizes)
     mats = [rng.normal(scale=0.4, size=s) for s in shapes]
@@ -531,7 +548,7 @@ def test_gemv_with_filter_epilogue(queue):
     from oracle import oracle as orc
 
     rng = np.random.RandomState(5)
-    shapes = [(64, 4096), (64, 2048), (140, 300), (16, 8), (260, 128)]
+    shapes = [(64, 4096), (64, 2048), (300, 28), (16, 8), (600, 16)]
     n = len(shapes)
     mats = [rng.normal(scale=0.1, size=s) for s in shapes]
     xs = [rng.normal(size=s[1]) for s in shapes]
@@ -573,7 +590,7 @@ def test_gemv_with_filter_epilogue(queue):
     result = g.fuse_linearfilter(prog.plans, lf[0])
     assert result is not None
     fused, residual = result
-    # compile-time shapes (4096, 2048), another power of two (128), any width (300), small
+    # compile-time shapes (4096, 2048), a small power of two (16), any width (28), small
     assert sorted(p.name for p in fused) == ["hipra_gemv.tile_filter"] * 3 + [
         "hipra_gemv.wave_ref_filter"]
     assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_filter"} == {
