@@ -104,8 +104,9 @@ int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
  *                               the item's first row of `dots` (8; zeros without dots)}
  * `vec` as for nhip_gemv.  `pow2_cols` selects the kernel: 0 = any shape; 1 = every
  * dot product of the launch has a power-of-two column count >= 4 (log2_N set),
- * vec == 4 and a_stride0 < 2^22; 2 = every dot product has a multiple of 4 columns
- * from 32 up, vec == 4, a_stride0 < 2^22 and blk_words == 2176: the kernel whose
+ * vec == 4 and a_stride0 < 2^22; 2 = every dot product has 32 columns or more (a
+ * row whose length is no multiple of 4 followed by readable memory up to the next
+ * one), vec == 4, a_stride0 < 2^22 and blk_words == 2176: the kernel whose
  * stage shapes are compile-time constants (fewest instructions per byte); the last
  * word of a dots row then says which: 5 (N <= 32: stages of 32 columns, blocks of
  * 32 rows), 6 (N <= 64: 64 columns, 32 rows), 7 (N < 512: 128 columns, 16 rows) or

@@ -40,8 +40,8 @@ TILE_STAGE_WORDS = int(os.environ.get("NENGO_HIP_TILE_WORDS", 2176))
 MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
-# The large-item kernel with compile-time shapes takes dot products whose column count
-# is a multiple of 4 from STREAM_MIN_COLS up; its LDS block has STREAM_STAGE_WORDS words.
+# The large-item kernel with compile-time shapes takes dot products of STREAM_MIN_COLS
+# columns or more whose rows are 16-byte aligned; its LDS block has STREAM_STAGE_WORDS words.
 STREAM_MIN_COLS, STREAM_STAGE_WORDS = 32, 2176
 STREAM_NARROW_MAX_ROWS = 128
 
@@ -231,12 +231,23 @@ class gemv_prog:
                 d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0
                 and d["a_stride0"] < 2 ** 22 for d in dots)
             # second entry: 1 = every column count a power of two; 2, 3, 4 = every column
-            # count a multiple of 4 from 32 up (the kernel with compile-time shapes): 3 =
+            # count from 32 up (the kernel with compile-time shapes): 3 =
             # none above 64 (more waves fit a compute unit then), 2 = none from 68 to 508,
             # 4 = any
+            # (vec == 4: rows start on 16-byte boundaries; a row whose length is no multiple
+            # of 4 must be followed by readable memory up to the next one: a column block
+            # of a wider matrix)
+            a_size = int(self.A.dev_buf.size)
+
+            def quads_readable(d):  # 16-byte loads may run up to three columns past a row
+                n4 = -(-d["a_shape1"] // 4) * 4
+                return (d["a_shape1"] == n4 or (
+                    M > 1 and d["a_stride0"] >= n4
+                    and d["a_start"] + (M - 1) * d["a_stride0"] + n4 <= a_size))
+
             stream = (vec == 4 and TILE_STAGE_WORDS == STREAM_STAGE_WORDS and dots and all(
                 d["a_stride0"] < 2 ** 22 and d["a_shape1"] >= STREAM_MIN_COLS
-                and d["a_shape1"] % 4 == 0 for d in dots))
+                and quads_readable(d) for d in dots))
             if stream:
                 stages = {stream_stage(d["a_shape1"])[0] for d in dots}
                 return (3, 4 if 7 in stages else 2 if 9 in stages else 3, vec)

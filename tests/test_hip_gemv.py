@@ -445,6 +445,45 @@ def test_compile_time_shape_views_bit_exact(queue, beta):
     assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
 
 
+def test_compile_time_shape_odd_width_views_bit_exact(queue):
+    """Column blocks of a wider matrix whose widths are no multiple of 4 (50, 333 and 601
+    columns at a row stride of 1200, rows 16-byte aligned) take the same kernel: the
+    16-byte loads run into the columns next to the block, which are not summed."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(99)
+    wide = rng.normal(size=(700, 1200)).astype(np.float32)
+    Aw = RA([wide], align=True)
+    Av = Aw[[0]]
+    s0 = int(Aw.starts[0])
+    Av.add_views([s0, s0 + 52, s0 + 388], [700, 700, 700], [50, 333, 601], [1200] * 3, [1] * 3)
+    xs = [rng.normal(size=50), rng.normal(size=333), rng.normal(size=601)]
+    Xw = RA(xs, align=True)
+    Yw = RA([rng.normal(size=700), rng.normal(size=700)], align=True)
+    jA = [np.array([1, 2, 3], dtype=np.int32), np.array([1], dtype=np.int32)]
+    jX = [np.array([0, 1, 2], dtype=np.int32), np.array([0], dtype=np.int32)]
+    Yo = clone(Yw)
+    orc.plan_block_gemv(None, 1.0, Av, jA, Xw, jX, 0.5, Yo).plans[0]()
+    dY = to_dev(queue, Yw)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, Av), jA, to_dev(queue, Xw), jX, 0.5, dY)
+    assert {p.kernel_class for p in prog.plans} == {(3, 4, 4)}
+    for plan in prog.plans:
+        plan()
+    got = dY.to_host()
+    assert np.array_equal(got[0], Yo[0]) and np.array_equal(got[1], Yo[1])
+    expect = (0.5 * Yw[0][:, 0] + wide[:, :50] @ xs[0] + wide[:, 52:385] @ xs[1]
+              + wide[:, 388:989] @ xs[2])
+    assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
+    # a contiguous matrix of such a width has nothing readable behind its last row: general kernel
+    A = RA([rng.normal(size=(700, 50))], align=True)
+    X = RA([rng.normal(size=50)], align=True)
+    Y = RA([rng.normal(size=700)], align=True)
+    js = [np.array([0], dtype=np.int32)]
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, 0.0, to_dev(queue, Y))
+    assert {p.kernel_class for p in prog.plans} == {(3, 0, 1)}
+
+
 @pytest.mark.parametrize("tau_kind", ["per-population", "per-neuron"])
 def test_gemv_with_lif_epilogue(queue, tau_kind):
     """GEMV + LIF in one launch: the currents, voltages, refractory times and spikes
