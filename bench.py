@@ -86,8 +86,8 @@ def measured_traffic(plan_name):
     """HBM bytes per launch of the dominant kernel, from the counter runs summarised in
     profiles/c3_shared_step.txt (FETCH_SIZE and WRITE_SIZE, scaled by what the same
     counters read for a plain copy of known size).  None for other workloads."""
-    kernel = {"hipra_gemv.tile_lif": "gemv_stream_kernel<1,false>",
-              "hipra_gemv.tile_filter": "gemv_stream_kernel<2,true>"}.get(plan_name)
+    kernel = {"hipra_gemv.tile_lif": "gemv_stream_kernel<1,0>",
+              "hipra_gemv.tile_filter": "gemv_stream_kernel<2,4>"}.get(plan_name)
     path = os.path.join(ROOT, "profiles", "c3_shared_step.txt")
     if kernel is None or not os.path.exists(path):
         return None

@@ -104,16 +104,18 @@ int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
  *                               the item's first row of `dots` (8; zeros without dots)}
  * `vec` as for nhip_gemv.  `pow2_cols` selects the kernel: 0 = any shape; 1 = every
  * dot product of the launch has a power-of-two column count >= 4 (log2_N set),
- * vec == 4 and a_stride0 < 2^22; 2 = every dot product has 32 columns or more (a
+ * vec == 4 and a_stride0 < 2^22; 2 = every dot product has 5 columns or more (a
  * row whose length is no multiple of 4 followed by readable memory up to the next
  * one), vec == 4, a_stride0 < 2^22 and blk_words == 2176: the kernel whose
  * stage shapes are compile-time constants (fewest instructions per byte); the last
- * word of a dots row then says which: 5 (N <= 32: stages of 32 columns, blocks of
- * 32 rows), 6 (N <= 64: 64 columns, 32 rows), 7 (N < 512: 128 columns, 16 rows) or
- * 9 (512 columns, 4 rows); tasks should be whole blocks.  The kernel comes in three
- * instances: 3 = no dot product has more than 64 columns and no task more than 128
- * rows (a smaller LDS footprint and fewer registers: four waves per SIMD); 2 = no
- * stage 7; 4 = any. */
+ * word of a dots row then says which: 3 (N <= 8: stages of 8 columns, blocks of 128
+ * rows), 4 (N <= 16: 16 columns, 64 rows), 5 (N <= 32: 32 columns, 32 rows), 6 (N <=
+ * 64: 64 columns, 32 rows), 7 (N < 512: 128 columns, 16 rows) or
+ * 9 (512 columns, 4 rows); tasks should be whole blocks.  The kernel comes in five
+ * instances, by the stages the launch may hold (each stage a launch does not need
+ * costs the others registers): 3 = stages 5 and 6 only, and no task of more than 128
+ * rows (a smaller LDS footprint and fewer registers: four waves per SIMD); 5 = the
+ * same with stages 3 and 4 too; 2 = stages 5, 6, 9; 4 = stages 5, 6, 7, 9; 6 = any. */
 int nhip_gemv_tile(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
                    const float *coefs, const int *dots, const int *tasks, int n_tasks,
                    const float *A, const float *X, const float *Yin, float *Y);

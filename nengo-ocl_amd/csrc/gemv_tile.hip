@@ -814,10 +814,10 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_p2_kernel(
 // 8 KiB block on bookkeeping (the shape of every stage is worked out again from the
 // dot record, every load has its own 64-bit address arithmetic and predicate), and
 // with three or four waves per SIMD that, not HBM, is what bounds them.  Here the
-// column count of a stage is a template parameter (32, 64, 128 or 512; the host picks
-// the smallest that holds the dot product, 128 for 68 ... 508 columns, 512 from there
-// up; the last or only column stage may be narrower, any multiple of 4): all LDS
-// addresses are immediates, a block's loads share one
+// column count of a stage is a template parameter (8, 16, 32, 64, 128 or 512; the host
+// picks the smallest that holds the dot product, 128 for 65 ... 511 columns, 512 from
+// there up; the last or only column stage may be narrower): all LDS addresses are
+// immediates, a block's loads share one
 // scalar base and per-lane offsets that are set up once per dot product, tile sums
 // go from the lanes that hold them straight onto the running row sums, and the loop
 // over the stages of a dot product is written so that the loads of the register set
@@ -833,14 +833,14 @@ struct StreamGeo {
     static constexpr int LGT = LGC > 7 ? LGC - 7 : 0;       // log2 of the tiles of a stage
     static constexpr int TILES = 1 << LGT;
     static constexpr int ROWW = LGC >= 7 ? (TILE_LDS << LGT) : NCS + 4;  // LDS words of a row
-    static constexpr int RB = LGC >= 7 ? 16 >> LGT : 32;    // rows of a block
+    static constexpr int RB = LGC >= 7 ? 16 >> LGT : LGC >= 5 ? 32 : LGC == 4 ? 64 : 128;  // rows of a block
     static constexpr int NL = (RB / RPL) << LG_LPR;         // loads per lane and block
     static constexpr int CHAIN = LGC >= 7 ? MAX_CHAIN : NCS / 4;  // elements of a partial sum
     static constexpr int XL = NCS >= NHIP_WAVE ? NCS / NHIP_WAVE : 1;  // X loads per lane and stage
     static constexpr bool MULTI = LGC >= 7;                 // several column stages: X travels with them
     static constexpr int PASSES = (RB * TILES + 15) / 16;   // (row, tile) pairs come 16 at a time
     static constexpr int PASS_WORDS = (16 >> LGT) * ROWW;
-    static_assert(NL >= 1 && NL <= P2_PF && RB * ROWW <= 2176 && RB * TILES <= TSUM_WORDS, "block shape");
+    static_assert(NL >= 1 && NL <= P2_PF && RB * ROWW <= 2176 && LGC >= 3, "block shape");
 };
 
 constexpr int STREAM_BLK_WORDS = 2176;  // the LDS block these shapes are made for
@@ -853,17 +853,18 @@ __device__ __forceinline__ float row_from_right(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x100 + N, 0xF, 0xF, true));
 }
 
-// SET: the stage widths the launch needs -- 0: 32 and 64 columns only; 1: also 512
-// (more registers and a larger X block in LDS: three waves per SIMD instead of four);
-// 2: also 128.  An instance that holds fewer shapes needs fewer registers, and the
-// large matrices of the benchmark networks need only 0 and 1.
+// SET: the stage widths the launch needs besides 32 and 64 columns, as bits -- 1: 8 and
+// 16 columns; 2: 128; 4: 512 (with 2 or 4: more registers and a larger X block in LDS,
+// three waves per SIMD instead of four).  An instance that holds fewer shapes needs
+// fewer registers, and the large matrices of the benchmark networks need only 0 and 4.
+constexpr int SET_TINY = 1, SET_MID = 2, SET_WIDE = 4;
 template <int EPI, int SET>
-__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(SET ? 3 : 4, 4))) void gemv_stream_kernel(
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 6) ? 3 : 4, 4))) void gemv_stream_kernel(
     const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
     float* Y, EpilogueArgs epi)
 {
-    constexpr bool WIDE = SET >= 1;
+    constexpr bool WIDE = (SET & (SET_MID | SET_WIDE)) != 0;  // the large LDS layout
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1127,12 +1128,14 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu(SET ? 3
         }
     };
 
-    // dot.p2: the stage width the host chose for the dot product (log2: 5, 6, 7 or 9)
+    // dot.p2: the stage width the host chose for the dot product (log2: 3 ... 7 or 9)
     auto dot_of_width = [&](auto first_tag, auto ragged_tag, const GemvDot& dot) {
-        if (dot.p2 == 5) dot_pass(std::integral_constant<int, 5>{}, first_tag, ragged_tag, dot);
+        if ((SET & SET_TINY) && dot.p2 == 3) dot_pass(std::integral_constant<int, 3>{}, first_tag, ragged_tag, dot);
+        else if ((SET & SET_TINY) && dot.p2 == 4) dot_pass(std::integral_constant<int, 4>{}, first_tag, ragged_tag, dot);
+        else if (dot.p2 == 5) dot_pass(std::integral_constant<int, 5>{}, first_tag, ragged_tag, dot);
         else if (!WIDE || dot.p2 == 6) dot_pass(std::integral_constant<int, 6>{}, first_tag, ragged_tag, dot);
-        else if (SET == 2 && dot.p2 == 7) dot_pass(std::integral_constant<int, 7>{}, first_tag, ragged_tag, dot);
-        else dot_pass(std::integral_constant<int, 9>{}, first_tag, ragged_tag, dot);
+        else if ((SET & SET_MID) && dot.p2 == 7) dot_pass(std::integral_constant<int, 7>{}, first_tag, ragged_tag, dot);
+        else if (SET & SET_WIDE) dot_pass(std::integral_constant<int, 9>{}, first_tag, ragged_tag, dot);
     };
     // column count a multiple of its stage width (the stage width is 1 << p2)
     auto whole_stages = [&](const GemvDot& dot) { return (dot.N & ((1 << dot.p2) - 1)) == 0; };
@@ -1168,14 +1171,15 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
-    if (pow2_cols != 0 && (pow2_cols < 1 || pow2_cols > 4 || vec != 4)) return NHIP_E_BADCLASS;
+    if (pow2_cols != 0 && (pow2_cols < 1 || pow2_cols > 6 || vec != 4)) return NHIP_E_BADCLASS;
     if (pow2_cols >= 2 && blk_words != STREAM_BLK_WORDS) return NHIP_E_BADARG;
-    const int stream_xb = pow2_cols == 3 ? STREAM_NARROW_XB_WORDS : XBLK_WORDS;
+    const bool stream_small = pow2_cols == 3 || pow2_cols == 5;  // no stage above 64 columns
+    const int stream_xb = stream_small ? STREAM_NARROW_XB_WORDS : XBLK_WORDS;
     if (blk_words < (STAGE_COLS / TILE) * TILE_LDS || (blk_words & 3)) return NHIP_E_BADARG;
     if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
     const int waves = NHIP_WG / NHIP_WAVE;
     const size_t wave_words = pow2_cols >= 2
-        ? (size_t)STREAM_BLK_WORDS + stream_xb + (pow2_cols == 3 ? STREAM_NARROW_SLOTS * NHIP_WAVE : YSUM_WORDS)
+        ? (size_t)STREAM_BLK_WORDS + stream_xb + (stream_small ? STREAM_NARROW_SLOTS * NHIP_WAVE : YSUM_WORDS)
         : (size_t)blk_words + TSUM_WORDS + XBLK_WORDS + (pow2_cols ? YSUM_WORDS : 0);
     const size_t lds_bytes = sizeof(float) * waves * wave_words;
     if (lds_bytes > 64 * 1024) return NHIP_E_BADARG;  // stays within the default dynamic LDS limit
@@ -1200,9 +1204,11 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
                         reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, stream_xb, A, X, Yin,
                         Y, args);
         };
-        if (pow2_cols == 2) launch_stream(gemv_stream_kernel<E, 1>);
+        if (pow2_cols == 2) launch_stream(gemv_stream_kernel<E, SET_WIDE>);
         else if (pow2_cols == 3) launch_stream(gemv_stream_kernel<E, 0>);
-        else if (pow2_cols == 4) launch_stream(gemv_stream_kernel<E, 2>);
+        else if (pow2_cols == 4) launch_stream(gemv_stream_kernel<E, SET_WIDE | SET_MID>);
+        else if (pow2_cols == 5) launch_stream(gemv_stream_kernel<E, SET_TINY>);
+        else if (pow2_cols == 6) launch_stream(gemv_stream_kernel<E, SET_WIDE | SET_MID | SET_TINY>);
         else if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
         else if (vec == 4) launch(gemv_tile_kernel<4, E>);
         else launch(gemv_tile_kernel<1, E>);

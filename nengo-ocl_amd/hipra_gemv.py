@@ -42,14 +42,33 @@ TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
 # The large-item kernel with compile-time shapes takes dot products of STREAM_MIN_COLS
 # columns or more whose rows are 16-byte aligned; its LDS block has STREAM_STAGE_WORDS words.
-STREAM_MIN_COLS, STREAM_STAGE_WORDS = 32, 2176
+STREAM_MIN_COLS, STREAM_STAGE_WORDS = 5, 2176
 STREAM_NARROW_MAX_ROWS = 128
+
+
+def stream_class(stages):
+    """The instance of the kernel with compile-time shapes (the `pow2_cols` argument of
+    nhip_gemv_tile) that holds the stage widths `stages` (log2): 3 = 32 and 64 columns
+    only (more waves fit a compute unit then), 5 = also 8 and 16, 2 = also 512, 4 = also
+    128 and 512, 6 = all."""
+    tiny, mid, wide = bool(stages & {3, 4}), 7 in stages, 9 in stages
+    if tiny:
+        return 6 if mid or wide else 5
+    return 4 if mid else 2 if wide else 3
+
+
+STREAM_CLASS_STAGES = {3: {5, 6}, 5: {3, 4, 5, 6}, 2: {5, 6, 9}, 4: {5, 6, 7, 9},
+                       6: {3, 4, 5, 6, 7, 9}}
 
 
 def stream_stage(n_cols):
     """(log2 of the stage width, rows of a block) the kernel with compile-time shapes
     uses for a dot product of `n_cols` columns: the smallest stage that holds it, 128
-    columns wide from 68 to 508 columns, 512 from there up."""
+    columns wide from 65 to 511 columns, 512 from there up."""
+    if n_cols <= 8:
+        return 3, 128
+    if n_cols <= 16:
+        return 4, 64
     if n_cols <= 32:
         return 5, 32
     if n_cols <= 64:
@@ -230,10 +249,8 @@ class gemv_prog:
             pow2 = vec == 4 and all(
                 d["a_shape1"] >= 4 and d["a_shape1"] & (d["a_shape1"] - 1) == 0
                 and d["a_stride0"] < 2 ** 22 for d in dots)
-            # second entry: 1 = every column count a power of two; 2, 3, 4 = every column
-            # count from 32 up (the kernel with compile-time shapes): 3 =
-            # none above 64 (more waves fit a compute unit then), 2 = none from 68 to 508,
-            # 4 = any
+            # second entry: 1 = every column count a power of two; 2 ... 6 = the kernel with
+            # compile-time shapes, by the stage widths needed (`stream_class`)
             # (vec == 4: rows start on 16-byte boundaries; a row whose length is no multiple
             # of 4 must be followed by readable memory up to the next one: a column block
             # of a wider matrix)
@@ -249,8 +266,7 @@ class gemv_prog:
                 d["a_stride0"] < 2 ** 22 and d["a_shape1"] >= STREAM_MIN_COLS
                 and quads_readable(d) for d in dots))
             if stream:
-                stages = {stream_stage(d["a_shape1"])[0] for d in dots}
-                return (3, 4 if 7 in stages else 2 if 9 in stages else 3, vec)
+                return (3, stream_class({stream_stage(d["a_shape1"])[0] for d in dots}), vec)
             return (3, int(pow2), vec)
         if flavor == 0:
             # Matrix loads are non-temporal, so one wave instruction should take whole
@@ -346,15 +362,15 @@ class gemv_prog:
             if geometry[b]["y_len"] > 0:
                 by_class[self._item_class(geometry[b])].append(b)
 
-        # items without dot products (class (3, 1, 4)) ride with the launch of the
-        # compile-time-shape kernel when there is one
-        # ... and the launch of the instance that holds more stage widths takes the items
-        # of the ones that hold fewer, when several are there
-        for wider, narrower in (((3, 4, 4), (3, 2, 4)), ((3, 4, 4), (3, 3, 4)),
-                                ((3, 2, 4), (3, 3, 4))):
-            if wider in by_class and narrower in by_class:
-                by_class[wider] = sorted(by_class[wider] + by_class.pop(narrower))
-        stream = next((c for c in ((3, 4, 4), (3, 2, 4), (3, 3, 4)) if c in by_class), (3, 3, 4))
+        # the one instance of the compile-time-shape kernel that holds the stage widths of
+        # all of them takes the items of several instances
+        present = [c for c in by_class if c[0] == 3 and c[1] >= 2]
+        stream = (3, 3, 4)
+        if present:
+            stream = (3, stream_class(set().union(
+                *(STREAM_CLASS_STAGES[c[1]] for c in present))), 4)
+            by_class[stream] = sorted(b for c in present for b in by_class.pop(c))
+        # ... and items without dot products (class (3, 1, 4)) ride with that launch
         if stream in by_class and (3, 1, 4) in by_class:
             bare = [b for b in by_class[(3, 1, 4)] if not geometry[b]["dots"]]
             by_class[stream] = sorted(by_class[stream] + bare)
@@ -383,8 +399,8 @@ class gemv_prog:
             if flavor == 3:
                 # launches without wide dot products keep tasks to 128 rows (the kernel
                 # then needs fewer registers and a fourth wave fits each SIMD)
-                task_rows = self._tile_tasks(members, STREAM_NARROW_MAX_ROWS if lpr == 3 else 256,
-                                             stream=lpr >= 2)
+                task_rows = self._tile_tasks(
+                    members, STREAM_NARROW_MAX_ROWS if lpr in (3, 5) else 256, stream=lpr >= 2)
             else:
                 task_rows = []
                 for b in (members if flavor != 2 else ()):

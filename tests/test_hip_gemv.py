@@ -141,7 +141,7 @@ def test_ensemble_shapes(queue, pi):
     rng = np.random.RandomState(7)
     shapes = [(4096, 64), (64, 4096), (100, 1), (1, 100), (100, 2), (2, 100), (2000, 32),
               (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000), (600, 16),
-              (600, 20)]
+              (600, 20), (3000, 4), (700, 50)]
     A = RA([rng.normal(size=s) for s in shapes], align=True)
     X = RA([rng.normal(size=s[1]) for s in shapes], align=True)
     Y = RA([rng.normal(size=s[0]) for s in shapes], align=True)
@@ -149,9 +149,9 @@ def test_ensemble_shapes(queue, pi):
     prog = run_case(queue, planners()[pi], 1.0, 1.0, 0.0, A, X, Y, js, js)
     if pi == 0:
         classes = {p.kernel_class for p in prog.plans}
-        # multiples of 4 from 32 up (compile-time shapes; 2: none from 68 to 508 columns),
-        # smaller powers of two, any width, small
-        assert classes == {(3, 2, 4), (3, 1, 4), (3, 0, 4), (2, 4, 1)}
+        # compile-time shapes (6: stages of 8 / 16 as well as of 512 columns), 4 columns
+        # (a power of two), rows that are not 16-byte aligned, small
+        assert classes == {(3, 6, 4), (3, 1, 4), (3, 0, 1), (2, 4, 1)}
 
 
 def test_strided_views_and_yin(queue):
@@ -314,10 +314,11 @@ def test_large_items_bit_exact(queue, beta):
 
 @pytest.mark.parametrize("beta", [1.0, 0.5])
 def test_pow2_items_bit_exact(queue, beta):
-    """Power-of-two column counts take the streamlined staged kernel: every width from
-    4 to 8192, row counts that leave partial row blocks and partial tasks, outputs that
-    sum dot products of different power-of-two widths, and matrix views with a row
-    stride larger than the width -- bit-identical to the oracle."""
+    """Power-of-two column counts: every width from 4 to 16384, row counts that leave
+    partial row blocks and partial tasks, outputs that sum dot products of different
+    power-of-two widths, and matrix views with a row stride larger than the width --
+    bit-identical to the oracle.  Items with a 4-column dot product take the staged
+    kernel for powers of two, the others the one with compile-time shapes."""
     from nengo_ocl_amd import hipra_gemv as g
     from oracle import oracle as orc
 
@@ -335,7 +336,7 @@ def test_pow2_items_bit_exact(queue, beta):
     orc.plan_block_gemv(None, 1.0, A, js, X, js, beta, Yo).plans[0]()
     dY = to_dev(queue, Y)
     prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY)
-    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4), (3, 4, 4)}
+    assert {p.kernel_class for p in prog.plans} == {(3, 1, 4), (3, 6, 4)}
     for plan in prog.plans:
         plan()
     got = dY.to_host()
@@ -363,10 +364,10 @@ def test_pow2_items_bit_exact(queue, beta):
 
 
 @pytest.mark.parametrize("beta", [1.0, 0.5])
-@pytest.mark.parametrize("widths", ["to-64", "to-64-and-from-512", "all"])
+@pytest.mark.parametrize("widths", ["to-64", "to-64-and-from-512", "from-32", "from-8-to-64", "all"])
 def test_compile_time_shape_items_bit_exact(queue, beta, widths):
-    """Column counts that are multiples of 4 from 32 up take the kernel whose stage
-    shapes are compile-time constants (stages of 32, 64, 128 or 512 columns; one
+    """Column counts that are multiples of 4 from 8 up take the kernel whose stage
+    shapes are compile-time constants (stages of 8, 16, 32, 64, 128 or 512 columns; one
     instance per set of stage widths a launch needs): row counts that leave partial
     row blocks, widths that leave a narrower last or only column stage, tasks of one to
     many stages, outputs that sum dot products of several such widths, a Y_in different
@@ -384,10 +385,15 @@ def test_compile_time_shape_items_bit_exact(queue, beta, widths):
             (21, 1660), (130, 1020)]
     middle = [(301, 128), (130, 256), (700, 100), (300, 132), (260, 300), (1000, 500), (90, 508),
               (513, 68), (400, 260)]
+    tiny = [(4096, 16), (4096, 8), (3000, 24), (5000, 12), (1037, 8), (999, 16), (2000, 28),
+            (515, 20), (8300, 8), (2057, 12), (1029, 16), (7000, 16)]
     shapes, multi, expected = {
         "to-64": (narrow, (64, 32, 48, 64, 36), (3, 3, 4)),
         "to-64-and-from-512": (narrow + wide, (64, 1024, 32, 512, 64, 2000, 644, 40), (3, 2, 4)),
-        "all": (narrow + wide + middle, (64, 1024, 300, 32, 512, 128, 2000, 68), (3, 4, 4)),
+        "from-32": (narrow + wide + middle, (64, 1024, 300, 32, 512, 128, 2000, 68), (3, 4, 4)),
+        "from-8-to-64": (tiny + narrow, (16, 64, 8, 32, 12, 48, 16, 8, 24), (3, 5, 4)),
+        "all": (tiny + narrow[:6] + wide[::3] + middle[::2],
+                (8, 1024, 300, 16, 512, 12, 128, 2000, 68, 8, 32), (3, 6, 4)),
     }[widths]
     mats = [rng.normal(size=s) for s in shapes] + [rng.normal(size=(300, n)) for n in multi]
     A = RA(mats, align=True)
@@ -475,6 +481,29 @@ def test_compile_time_shape_odd_width_views_bit_exact(queue):
     expect = (0.5 * Yw[0][:, 0] + wide[:, :50] @ xs[0] + wide[:, 52:385] @ xs[1]
               + wide[:, 388:989] @ xs[2])
     assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
+    # widths from 5 up: 5, 9, 14 and 17 columns of a matrix with 48
+    slim = rng.normal(size=(3000, 48)).astype(np.float32)
+    As = RA([slim], align=True)
+    Av = As[[0]]
+    s0 = int(As.starts[0])
+    cols, widths = [0, 8, 20, 28], [5, 9, 14, 17]
+    Av.add_views([s0 + c for c in cols], [3000] * 4, widths, [48] * 4, [1] * 4)
+    xs = [rng.normal(size=w) for w in widths]
+    Xs = RA(xs, align=True)
+    Ys = RA([rng.normal(size=3000), rng.normal(size=3000)], align=True)
+    jA = [np.array([1, 2, 3, 4], dtype=np.int32), np.array([2], dtype=np.int32)]
+    jX = [np.array([0, 1, 2, 3], dtype=np.int32), np.array([1], dtype=np.int32)]
+    Yo = clone(Ys)
+    orc.plan_block_gemv(None, 1.0, Av, jA, Xs, jX, 0.5, Yo).plans[0]()
+    dY = to_dev(queue, Ys)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, Av), jA, to_dev(queue, Xs), jX, 0.5, dY)
+    assert {p.kernel_class for p in prog.plans} == {(3, 5, 4)}
+    for plan in prog.plans:
+        plan()
+    got = dY.to_host()
+    assert np.array_equal(got[0], Yo[0]) and np.array_equal(got[1], Yo[1])
+    expect = 0.5 * Ys[0][:, 0] + sum(slim[:, c:c + w] @ x for c, w, x in zip(cols, widths, xs))
+    assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
     # a contiguous matrix of such a width has nothing readable behind its last row: general kernel
     A = RA([rng.normal(size=(700, 50))], align=True)
     X = RA([rng.normal(size=50)], align=True)
@@ -499,8 +528,8 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     rng = np.random.RandomState(31)
     dt = 1e-3
     # GEMV items: four large ones with neurons, a small one with neurons, a large one without
-    shapes = [(4096, 64), (1000, 16), (3000, 28), (520, 130), (60, 8), (300, 64)]
-    pop_sizes = [4096, 1000, 3000, 520, 60, 700]  # the last population has no input item
+    shapes = [(4096, 64), (3000, 4), (3000, 12), (520, 130), (60, 8), (300, 64)]
+    pop_sizes = [4096, 3000, 3000, 520, 60, 700]  # the last population has no input item
     n, n_pop = len(shapes), len(pop_sizes)
     mats = [rng.normal(scale=0.4, size=s) for s in shapes]
     xs = [rng.normal(size=s[1]) for s in shapes]
@@ -533,12 +562,12 @@ def test_gemv_with_lif_epilogue(queue, tau_kind):
     fused = g.fuse_lif(prog, lif)
     assert fused is not None
     names = sorted(p.name for p in fused)
-    # four large-item classes (the input-less population joins the one with compile-time
+    # three large-item classes (the input-less population joins the one with compile-time
     # shapes) and the small item's launch, each updating the neurons it feeds: no neuron
     # launch
-    assert names == ["hipra_gemv.tile_lif"] * 4 + ["hipra_gemv.wave_ref_lif"]
+    assert names == ["hipra_gemv.tile_lif"] * 3 + ["hipra_gemv.wave_ref_lif"]
     assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_lif"} == {
-        (3, 3, 4), (3, 1, 4), (3, 0, 4), (3, 0, 1)}
+        (3, 5, 4), (3, 1, 4), (3, 0, 1)}
     for step in range(3):
         for p in fused:
             p()
@@ -587,7 +616,7 @@ def test_gemv_with_filter_epilogue(queue):
     from oracle import oracle as orc
 
     rng = np.random.RandomState(5)
-    shapes = [(64, 4096), (64, 2048), (300, 28), (16, 8), (600, 16)]
+    shapes = [(64, 4096), (64, 2048), (3000, 12), (16, 8), (2500, 4), (300, 30)]
     n = len(shapes)
     mats = [rng.normal(scale=0.1, size=s) for s in shapes]
     xs = [rng.normal(size=s[1]) for s in shapes]
@@ -597,7 +626,7 @@ def test_gemv_with_filter_epilogue(queue):
     filters = [(0,) + lowpass(0.005), (0,) + lowpass(0.1), (0,) + lowpass(0.02),
                (1, np.zeros(0), np.array([0.5])), (2,) + lowpass(0.01), (3,) + lowpass(0.01),
                (0, np.array([-1.2, 0.4]), np.array([0.1, 0.1])), (4,) + lowpass(0.03),
-               (4,) + lowpass(0.002)]
+               (4,) + lowpass(0.002), (5,) + lowpass(0.02)]
     f_out = [rng.normal(size=shapes[b][0]) for b, _, _ in filters]
     R = RA(mats + xs + outs + f_out, align=True)
     iA, iX, iY = (list(range(k * n, (k + 1) * n)) for k in range(3))
@@ -629,11 +658,11 @@ def test_gemv_with_filter_epilogue(queue):
     result = g.fuse_linearfilter(prog.plans, lf[0])
     assert result is not None
     fused, residual = result
-    # compile-time shapes (4096, 2048), a small power of two (16), any width (28), small
+    # compile-time shapes (4096, 2048, 12), 4 columns, rows not 16-byte aligned (30), small
     assert sorted(p.name for p in fused) == ["hipra_gemv.tile_filter"] * 3 + [
         "hipra_gemv.wave_ref_filter"]
     assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_filter"} == {
-        (3, 2, 4), (3, 1, 4), (3, 0, 4)}
+        (3, 6, 4), (3, 1, 4), (3, 0, 1)}
     assert [p.name for p in residual] == ["hip_linearfilter"]
     oprog, olf = build(host, orc, orc, None, lambda a: a)
     for step in range(4):
