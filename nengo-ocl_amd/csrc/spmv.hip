@@ -27,7 +27,7 @@ struct SpmvSlice {
     int pad;
 };
 
-constexpr int SPMV_UNROLL = 4;  // independent loads in flight per lane
+constexpr int SPMV_UNROLL = 4;  // elements of a row whose operands are fetched together
 
 __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
     const SpmvSlice* __restrict__ slices, int n_slices, const int* __restrict__ row_len,
@@ -43,20 +43,35 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
     float acc = (live && sl.inc) ? Y[(size_t)sl.y_start + lane] : 0.0f;
     const int* c = cols + (size_t)sl.data_start + lane;
     const float* v = vals + (size_t)sl.data_start + lane;
+    // values and column indices of the next SPMV_UNROLL elements are requested before
+    // the gathers from X of the current ones (past the end: the last again, unused)
+    int ci[SPMV_UNROLL];
+    float vi[SPMV_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SPMV_UNROLL; ++u) {
+        const int k = min(u, sl.width - 1);
+        ci[u] = sl.width > 0 ? __builtin_nontemporal_load(c + (size_t)k * NHIP_WAVE) : 0;
+        vi[u] = sl.width > 0 ? __builtin_nontemporal_load(v + (size_t)k * NHIP_WAVE) : 0.0f;
+    }
     for (int k0 = 0; k0 < sl.width; k0 += SPMV_UNROLL) {
-        int ci[SPMV_UNROLL];
-        float vi[SPMV_UNROLL], xi[SPMV_UNROLL];
+        int cn[SPMV_UNROLL];
+        float vn[SPMV_UNROLL], xi[SPMV_UNROLL];
 #pragma unroll
         for (int u = 0; u < SPMV_UNROLL; ++u) {
-            const bool in = k0 + u < sl.width;  // uniform
-            ci[u] = in ? __builtin_nontemporal_load(c + (size_t)(k0 + u) * NHIP_WAVE) : 0;
-            vi[u] = in ? __builtin_nontemporal_load(v + (size_t)(k0 + u) * NHIP_WAVE) : 0.0f;
+            const int k = min(k0 + SPMV_UNROLL + u, sl.width - 1);
+            cn[u] = __builtin_nontemporal_load(c + (size_t)k * NHIP_WAVE);
+            vn[u] = __builtin_nontemporal_load(v + (size_t)k * NHIP_WAVE);
         }
 #pragma unroll
         for (int u = 0; u < SPMV_UNROLL; ++u) xi[u] = (k0 + u < len) ? x[ci[u]] : 0.0f;
 #pragma unroll
         for (int u = 0; u < SPMV_UNROLL; ++u)
             if (k0 + u < len) acc = fmaf(vi[u], xi[u], acc);
+#pragma unroll
+        for (int u = 0; u < SPMV_UNROLL; ++u) {
+            ci[u] = cn[u];
+            vi[u] = vn[u];
+        }
     }
     if (live) Y[(size_t)sl.y_start + lane] = acc;
 }
