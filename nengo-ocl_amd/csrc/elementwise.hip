@@ -60,6 +60,20 @@ __device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, flo
     const float* x = X + d.x_start;
     float* y = Y + d.y_start;
     const bool flat = (d.x_stride0 == d.shape1) && (d.y_stride0 == d.shape1);
+    if (flat && !((d.x_start | d.y_start | d.offset | d.count) & 3)) {
+        // contiguous on both sides and made of whole aligned quads: 16 bytes per access
+        const float4* x4 = reinterpret_cast<const float4*>(x + d.offset);
+        float4* y4 = reinterpret_cast<float4*>(y + d.offset);
+        for (int q = lane; q < (d.count >> 2); q += L) {
+            float4 v = x4[q];
+            if (d.inc) {
+                const float4 w = y4[q];
+                v = make_float4(w.x + v.x, w.y + v.y, w.z + v.z, w.w + v.w);
+            }
+            y4[q] = v;
+        }
+        return;
+    }
     const int i0 = d.offset / d.shape1, j0 = d.offset - i0 * d.shape1;  // once per block
     for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
@@ -136,6 +150,28 @@ __device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const floa
     const float alpha = nhip_bits(d.alpha_bits);
     const bool outer = d.flags & 1, inc = d.flags & 2;
     const int i0 = d.offset / d.y_shape1, j0 = d.offset - i0 * d.y_shape1;  // once per block
+    if (outer && !((d.y_start | d.y_shape1 | d.y_stride0 | d.offset | d.count) & 3)) {
+        // outer product whose rows are made of whole aligned quads: four elements of one
+        // row per lane, 16 bytes per access to Y (the same products and sums)
+        for (int k = 4 * lane; k < d.count; k += 4 * L) {
+            int i, j;
+            nhip_row_col(i0, j0, k, d.y_shape1, d.count, i, j);
+            const float aa = __fmul_rn(alpha, ew_element(a, d.a_shape0, 1, d.a_stride0, i, 0));
+            float xx[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) xx[e] = ew_element(x, d.x_shape0, 1, d.x_stride0, j + e, 0);
+            float4* dst = reinterpret_cast<float4*>(y + (size_t)i * d.y_stride0 + j);
+            float4 v = make_float4(__fmul_rn(aa, xx[0]), __fmul_rn(aa, xx[1]),
+                                   __fmul_rn(aa, xx[2]), __fmul_rn(aa, xx[3]));
+            if (inc) {
+                const float4 w = *dst;
+                v = make_float4(__fadd_rn(w.x, v.x), __fadd_rn(w.y, v.y), __fadd_rn(w.z, v.z),
+                                __fadd_rn(w.w, v.w));
+            }
+            *dst = v;
+        }
+        return;
+    }
     for (int k = lane; k < d.count; k += L) {
         int i, j;
         nhip_row_col(i0, j0, k, d.y_shape1, d.count, i, j);
