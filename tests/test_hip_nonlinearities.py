@@ -96,11 +96,14 @@ def test_lif_rate(queue, rng):
     assert np.array_equal(got.buf, Ro.buf)  # log1p correctly rounded on both sides: bit-exact
 
 
-def test_copy(queue, rng):
-    sizes = [(10, 1), (40, 64), (457, 342), (1, 100), (3000, 1)]
-    X = RA([rng.normal(size=s) for s in sizes])
-    Y0 = RA([rng.normal(size=s) for s in sizes])
-    incs = np.array([0, 1, 1, 0, 1], dtype=np.int32)
+@pytest.mark.parametrize("align", [False, True])
+def test_copy(queue, rng, align):
+    """`align`: items start on 64-byte boundaries, so those made of whole quads take the
+    16-byte path (with blocks of 1024 elements: whole, short and ragged last blocks)."""
+    sizes = [(10, 1), (40, 64), (457, 342), (1, 100), (3000, 1), (2000, 32), (8, 1), (1, 1028)]
+    X = RA([rng.normal(size=s) for s in sizes], align=align)
+    Y0 = RA([rng.normal(size=s) for s in sizes], align=align)
+    incs = np.array([0, 1, 1, 0, 1, 1, 1, 0], dtype=np.int32)
     dX, dY = to_dev(queue, X), to_dev(queue, Y0)
     nl().plan_copy(queue, dX, dY, incs)()
     Yo = clone(Y0)
@@ -154,13 +157,16 @@ def test_elementwise_inc(queue, rng, inc, use_alpha):
         assert np.array_equal(got[k], Y[k] + ax if inc else ax), k
 
 
-def test_elementwise_inc_outer(queue, rng):
-    Xsizes = [3, 9, 15, 432]
-    Asizes = [9, 42, 10, 124]
+@pytest.mark.parametrize("align", [False, True])
+def test_elementwise_inc_outer(queue, rng, align):
+    """`align`: items start on 64-byte boundaries, so products whose rows are whole quads
+    take the 16-byte path (rows shorter and longer than a block of 1024 elements)."""
+    Xsizes = [3, 9, 15, 432, 2000, 16, 4]
+    Asizes = [9, 42, 10, 124, 32, 8, 700]
     alpha = rng.normal(size=len(Xsizes)).astype(np.float32)
-    A = RA([rng.normal(size=s) for s in Asizes])
-    X = RA([rng.normal(size=s) for s in Xsizes])
-    Y = RA([rng.normal(size=(a, x)) for a, x in zip(Asizes, Xsizes)])
+    A = RA([rng.normal(size=s) for s in Asizes], align=align)
+    X = RA([rng.normal(size=s) for s in Xsizes], align=align)
+    Y = RA([rng.normal(size=(a, x)) for a, x in zip(Asizes, Xsizes)], align=align)
     for inc in (True, False):
         dY = to_dev(queue, Y)
         nl().plan_elementwise_inc(queue, to_dev(queue, A), to_dev(queue, X), dY, alpha=alpha,
