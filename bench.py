@@ -193,6 +193,7 @@ def micro_benchmarks(repeats=50):
     plan = nl.plan_direct(queue, traced.code, traced.init, traced.input_names, [T, X2], Y2)
     cases.append(("compiled function node", "%d instances of a 2 -> 2 function" % n_nodes, plan))
 
+    gemv_micro(queue, rng, repeats)
     for name, what, plan in cases:
         for _ in range(3):
             plan()
@@ -208,6 +209,51 @@ def micro_benchmarks(repeats=50):
                           if plan.flops_per_call else None,
                           "timing": "events carried by the launch" if name != "compiled function node"
                           else "events around the launch"}), flush=True)
+
+
+def gemv_micro(queue, rng, repeats):
+    """The ragged GEMV alone on matrices of one shape: two sets of about 268 MB each
+    (more than the caches hold), launched in turn; one JSON line per shape."""
+    import numpy as np
+
+    from nengo_ocl_amd import hipra_gemv
+    from nengo_ocl_amd.hipraggedarray import HIPRaggedArray
+    from nengo_ocl_amd.raggedarray import RaggedArray
+
+    for m, n in ((4096, 8), (4096, 16), (4096, 28), (4096, 48), (4096, 64), (4096, 100),
+                 (2048, 200), (64, 4096), (300, 9000)):
+        n_items = max(1, int(round(268e6 / (4.0 * m * n))))
+        progs = []
+        for _ in range(2):
+            block = rng.standard_normal(size=(m, n)).astype(np.float32)
+            ra = lambda arrays: HIPRaggedArray(queue, RaggedArray(arrays, dtype=np.float32, align=True))
+            A = ra([block] * n_items)
+            X = ra([rng.standard_normal(size=n).astype(np.float32)] * n_items)
+            Y = ra([np.zeros(m, dtype=np.float32)] * n_items)
+            js = [np.array([i], dtype=np.int32) for i in range(n_items)]
+            progs.append(hipra_gemv.plan_block_gemv(queue, 1.0, A, js, X, js, 0.0, Y))
+        plans = [p for prog in progs for p in prog.plans]
+        for _ in range(3):
+            for p in plans:
+                p()
+        for _ in range(repeats // 2):
+            for p in plans:
+                p.enqueue(profiling=True)
+        queue.finish()
+        total, calls, nbytes = 0.0, 0, 0
+        for p in plans:
+            p.update_profiling()
+            total += sum(p.ctimes)
+            calls += len(p.ctimes)
+            nbytes += p.bw_per_call
+        avg = total / calls * len(plans) / 2.0  # per set
+        print(json.dumps({"kernel": "ragged GEMV, " + ", ".join(sorted({p.name for p in plans})),
+                          "problem": "%d x (%d x %d), two sets in turn" % (n_items, m, n),
+                          "class": sorted({str(p.kernel_class) for p in plans}),
+                          "avg_us": round(1e6 * avg, 2), "algorithmic_bytes": nbytes // 2,
+                          "gbs": round(1e-9 * (nbytes / 2.0) / avg, 1),
+                          "timing": "events carried by the launch"}), flush=True)
+        del progs, plans
 
 
 def main():

@@ -39,7 +39,8 @@ TILE_STAGE_WORDS = int(os.environ.get("NENGO_HIP_TILE_WORDS", 2176))
 # the reference-order kernel wants at least this many (wave) tasks per launch
 MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
-    "NENGO_HIP_TILE_TASK_BLOCKS", "4,2,1.5,1").split(","))  # row blocks per task, tried in order
+    "NENGO_HIP_TILE_TASK_BLOCKS", "4,3.5,3,2.5,2,1.5,1").split(","))  # row blocks per task, tried in order
+TASK_OVERHEAD_BYTES = 8192.0  # what starting and finishing a task costs, in streamed bytes
 # The large-item kernel with compile-time shapes takes dot products of STREAM_MIN_COLS
 # columns or more whose rows are 16-byte aligned; its LDS block has STREAM_STAGE_WORDS words.
 STREAM_MIN_COLS, STREAM_STAGE_WORDS = 5, 2176
@@ -289,11 +290,14 @@ class gemv_prog:
         """Tasks (item, first row, rows, 0) of the reference-order kernel for large items.
 
         A task is the rows one wave carries through all columns, a few row blocks of
-        what fits its LDS stage.  Larger tasks reuse the gathered X more often; but all
-        groups of a launch are resident at once (up to three per compute unit) and take
-        about as long as the launch itself, so the device is only busy to the end when
-        the groups spread evenly over the compute units.  Among the task sizes that
-        give enough tasks, the one with the least uneven spread wins.
+        what fits its LDS stage.  Larger tasks reuse the gathered X more often and pay
+        the start of a task (its record, the first loads, the epilogue: about what
+        TASK_OVERHEAD_BYTES of streaming cost) less often; but the groups of a launch
+        spread over the compute units in whole groups, and a launch of few groups (all
+        resident at once, each lasting about as long as the launch) is only busy to the
+        end when they spread evenly.  Among the task sizes that give enough tasks, the
+        one with the smallest (groups per compute unit, rounded up) x (bytes of a task +
+        overhead) wins.
         """
         lib, geometry = self.queue.lib, self.geometry
         blk = {b: min([stream_stage(dd["a_shape1"])[1] if stream else
@@ -315,12 +319,14 @@ class gemv_prog:
 
         n_cu = self.queue.n_compute_units
         best = None
+        row_bytes = {b: 4.0 * sum(dd["a_shape1"] for dd in geometry[b]["dots"]) for b in members}
         for per_task in TILE_TASK_BLOCKS:
             tasks = tasks_for(per_task)
-            rounds = -(-len(tasks) // (WG // WAVE)) / float(n_cu)  # groups per compute unit
-            uneven = -(-rounds // 1) / rounds
+            groups = -(-len(tasks) // (WG // WAVE))
+            task_bytes = sum(row_bytes[b] * n for b, _, n, _ in tasks) / max(len(tasks), 1)
+            cost = -(-groups // n_cu) * (task_bytes + TASK_OVERHEAD_BYTES)
             enough = len(tasks) >= MIN_TILE_TASKS
-            key = (not enough, round(uneven, 2))
+            key = (not enough, cost)
             if best is None or key < best[0]:
                 best = (key, tasks)
         return best[1]
