@@ -440,3 +440,37 @@ def test_vector_copies_are_propagated():
     ops = graph()
     ops[0].As = [two]                                                 # a scaled copy
     assert len(propagate_vector_copies(ops)) == 2
+
+
+def test_large_item_task_sizes():
+    """Rows per task of the large-item GEMV: a launch of many groups takes the largest
+    tasks (the start of a task is paid less often), a launch of few groups the size that
+    spreads its groups evenly over the compute units, and a size that leaves too few
+    tasks is not taken while another gives enough."""
+    from types import SimpleNamespace
+
+    from nengo_ocl_amd import hipra_gemv as g
+
+    def tasks_of(n_items, rows, cols, max_rows, n_cu=256):
+        prog = g.gemv_prog.__new__(g.gemv_prog)
+        prog.queue = SimpleNamespace(lib=None, n_compute_units=n_cu)
+        prog.geometry = [{"y_len": rows, "dots": [{"a_shape1": cols}]} for _ in range(n_items)]
+        tasks = prog._tile_tasks(list(range(n_items)), max_rows, stream=True)
+        # every row of every item exactly once, in order
+        for b in range(n_items):
+            mine = [(r0, n) for i, r0, n, _ in tasks if i == b]
+            assert mine[0][0] == 0 and sum(n for _, n in mine) == rows
+            assert all(mine[k][0] + mine[k][1] == mine[k + 1][0] for k in range(len(mine) - 1))
+        return tasks
+
+    # 584 matrices of 4096 x 28 (18,688 tasks of 128 rows): many groups per compute unit
+    assert {n for _, _, n, _ in tasks_of(584, 4096, 28, 128)} == {128}
+    # 256 matrices of 4096 x 64: 128 rows, 8 groups per compute unit
+    assert {n for _, _, n, _ in tasks_of(256, 4096, 64, 128)} == {128}
+    # 258 matrices of 64 x 4096 (blocks of 4 rows): 8-row tasks would leave 516 groups for
+    # 256 compute units, 6-row tasks (the last of an item: 4) give 710 groups, under 3 each
+    assert {n for _, _, n, _ in tasks_of(258, 64, 4096, 256)} == {6, 4}
+    # 192 matrices of 2000 x 32 (blocks of 32 rows): 96 rows = 1008 groups, under 4 each
+    assert max(n for _, _, n, _ in tasks_of(192, 2000, 32, 128)) == 96
+    # 64 x 4096 on a device of 64 compute units: 16-row tasks would be too few (1032)
+    assert max(n for _, _, n, _ in tasks_of(258, 64, 4096, 256, n_cu=64)) < 16
