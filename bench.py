@@ -221,13 +221,13 @@ def gemv_micro(queue, rng, repeats):
     from nengo_ocl_amd.raggedarray import RaggedArray
 
     for m, n in ((4096, 8), (4096, 16), (4096, 28), (4096, 48), (4096, 64), (4096, 100),
-                 (2048, 200), (64, 4096), (300, 9000)):
+                 (2048, 200), (64, 4096), (300, 9000), (4096, 10), (4096, 50)):
         n_items = max(1, int(round(268e6 / (4.0 * m * n))))
         progs = []
         for _ in range(2):
             block = rng.standard_normal(size=(m, n)).astype(np.float32)
             ra = lambda arrays: HIPRaggedArray(queue, RaggedArray(arrays, dtype=np.float32, align=True))
-            A = ra([block] * n_items)
+            A = ra([block] * n_items + [np.zeros(4, dtype=np.float32)])  # (readable behind the last)
             X = ra([rng.standard_normal(size=n).astype(np.float32)] * n_items)
             Y = ra([np.zeros(m, dtype=np.float32)] * n_items)
             js = [np.array([i], dtype=np.int32) for i in range(n_items)]

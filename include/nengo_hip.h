@@ -115,7 +115,11 @@ int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
  * instances, by the stages the launch may hold (each stage a launch does not need
  * costs the others registers): 3 = stages 5 and 6 only, and no task of more than 128
  * rows (a smaller LDS footprint and fewer registers: four waves per SIMD); 5 = the
- * same with stages 3 and 4 too; 2 = stages 5, 6, 9; 4 = stages 5, 6, 7, 9; 6 = any. */
+ * same with stages 3 and 4 too; 2 = stages 5, 6, 9; 4 = stages 5, 6, 7, 9; 6 = any;
+ * 7 = stages 3 to 6 for matrices whose rows lie back to back (a_stride0 == N <= 64, any
+ * value: rows need not be 16-byte aligned) from a_start % 4 == 0, with every task
+ * starting at a row that is a multiple of 4 and 12 readable bytes behind each matrix: a
+ * row block is then one aligned run of memory and is read in 16-byte quads. */
 int nhip_gemv_tile(void *stream, int vec, int pow2_cols, int blk_words, const int *items,
                    const float *coefs, const int *dots, const int *tasks, int n_tasks,
                    const float *A, const float *X, const float *Yin, float *Y);

@@ -857,14 +857,21 @@ __device__ __forceinline__ float row_from_right(float v) {
 // 16 columns; 2: 128; 4: 512 (with 2 or 4: more registers and a larger X block in LDS,
 // three waves per SIMD instead of four).  An instance that holds fewer shapes needs
 // fewer registers, and the large matrices of the benchmark networks need only 0 and 4.
-constexpr int SET_TINY = 1, SET_MID = 2, SET_WIDE = 4;
+// 8 (with 1, without 2 and 4): the rows of every matrix of the launch lie back to back
+// (row stride = column count, at most 64, any value) from a 16-byte boundary, every task
+// starts at a row that is a multiple of 4, and the 12 bytes behind a matrix can be read:
+// a row block is then one aligned run of memory, read in quads and laid out in LDS as it
+// lies in memory, although single rows are not 16-byte aligned.
+constexpr int SET_TINY = 1, SET_MID = 2, SET_WIDE = 4, SET_FLAT = 8;
 template <int EPI, int SET>
-__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 6) ? 3 : 4, 4))) void gemv_stream_kernel(
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 14) ? 3 : 4, 4))) void gemv_stream_kernel(
     const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
     float* Y, EpilogueArgs epi)
 {
     constexpr bool WIDE = (SET & (SET_MID | SET_WIDE)) != 0;  // the large LDS layout
+    constexpr bool FLAT = (SET & SET_FLAT) != 0;
+    static_assert(!(FLAT && WIDE), "back-to-back rows: single-stage widths only");
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -959,7 +966,10 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
         const int j = lane & 3;
         const int rt = lane >> 2;
         const int tl = rt & (G::TILES - 1);
-        const float* const ap = ab + (rt >> G::LGT) * G::ROWW + tl * TILE_LDS + j;
+        // (rows back to back: a row of the block has dot.N words, a pass 16 rows)
+        const float* const ap = FLAT ? ab + rt * dot.N + j
+                                     : ab + (rt >> G::LGT) * G::ROWW + tl * TILE_LDS + j;
+        const int pass_words = FLAT ? 16 * dot.N : G::PASS_WORDS;
         const float* const xp = xb + tl * TILE_LDS + j;
 
         // the loader walks the stages two ahead of the sums
@@ -981,7 +991,14 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                 }
             }
             const int rows = min(G::RB, n_rows - l_b * G::RB);
-            if (rows == G::RB && cols == G::NCS) {
+            if (FLAT) {  // the block is one run of rows * N words; lanes past it read its start
+                const unsigned n_bytes = 4u * (unsigned)(rows * dot.N);
+#pragma unroll
+                for (int i = 0; i < G::NL; ++i) {
+                    const unsigned off = 16u * (unsigned)(lane + i * NHIP_WAVE);
+                    pf[i] = load_nt4(reinterpret_cast<const float*>(l_ptr + (off < n_bytes ? off : 0u)));
+                }
+            } else if (rows == G::RB && cols == G::NCS) {
 #pragma unroll
                 for (int i = 0; i < G::NL; ++i) {
                     const char* row = l_ptr + (size_t)((i >> G::LG_LPR) * G::RPL) * stride4 +
@@ -1011,9 +1028,13 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
         auto store_block = [&](const tile_f4 (&pf)[G::NL], const float (&xq)[G::XL], bool with_x) {
             wave_sync();  // every lane is done reading the previous block
 #pragma unroll
-            for (int i = 0; i < G::NL; ++i)  // rows and columns that do not exist get whatever was read
-                *reinterpret_cast<tile_f4*>(wp + (i >> G::LG_LPR) * G::RPL * G::ROWW +
-                                            (i & ((1 << G::LG_LPR) - 1)) * (2 * TILE_LDS)) = pf[i];
+            for (int i = 0; i < G::NL; ++i) {  // rows and columns that do not exist get whatever was read
+                if (FLAT)
+                    *reinterpret_cast<tile_f4*>(ab + 4 * (lane + i * NHIP_WAVE)) = pf[i];
+                else
+                    *reinterpret_cast<tile_f4*>(wp + (i >> G::LG_LPR) * G::RPL * G::ROWW +
+                                                (i & ((1 << G::LG_LPR) - 1)) * (2 * TILE_LDS)) = pf[i];
+            }
             if (with_x) {
 #pragma unroll
                 for (int i = 0; i < G::XL; ++i)
@@ -1042,7 +1063,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                         for (int m = 0; m < G::CHAIN; ++m) {
                             // 128-column stages: the operands in two batches (registers)
                             if (G::LG_COLS == 7 && m == G::CHAIN / 2) __builtin_amdgcn_sched_barrier(0);
-                            acc = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
+                            acc = fmaf(ap[p * pass_words + 4 * m], xp[4 * m], acc);
                         }
                     } else {
 #pragma unroll
@@ -1050,7 +1071,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                             // (eight steps at a time: this path is rare and must not be
                             // what sets the kernel's register count)
                             if (m % 8 == 0 && m > 0) __builtin_amdgcn_sched_barrier(0);
-                            const float next = fmaf(ap[p * G::PASS_WORDS + 4 * m], xp[4 * m], acc);
+                            const float next = fmaf(ap[p * pass_words + 4 * m], xp[4 * m], acc);
                             acc = m < count ? next : acc;
                         }
                     }
@@ -1171,9 +1192,9 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
-    if (pow2_cols != 0 && (pow2_cols < 1 || pow2_cols > 6 || vec != 4)) return NHIP_E_BADCLASS;
+    if (pow2_cols != 0 && (pow2_cols < 1 || pow2_cols > 7 || vec != 4)) return NHIP_E_BADCLASS;
     if (pow2_cols >= 2 && blk_words != STREAM_BLK_WORDS) return NHIP_E_BADARG;
-    const bool stream_small = pow2_cols == 3 || pow2_cols == 5;  // no stage above 64 columns
+    const bool stream_small = pow2_cols == 3 || pow2_cols == 5 || pow2_cols == 7;  // no stage above 64 columns
     const int stream_xb = stream_small ? STREAM_NARROW_XB_WORDS : XBLK_WORDS;
     if (blk_words < (STAGE_COLS / TILE) * TILE_LDS || (blk_words & 3)) return NHIP_E_BADARG;
     if (vec == 4 && (reinterpret_cast<uintptr_t>(A) & 15u)) return NHIP_E_BADARG;
@@ -1209,6 +1230,7 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
         else if (pow2_cols == 4) launch_stream(gemv_stream_kernel<E, SET_WIDE | SET_MID>);
         else if (pow2_cols == 5) launch_stream(gemv_stream_kernel<E, SET_TINY>);
         else if (pow2_cols == 6) launch_stream(gemv_stream_kernel<E, SET_WIDE | SET_MID | SET_TINY>);
+        else if (pow2_cols == 7) launch_stream(gemv_stream_kernel<E, SET_TINY | SET_FLAT>);
         else if (pow2_cols) launch(gemv_tile_p2_kernel<E>);
         else if (vec == 4) launch(gemv_tile_kernel<4, E>);
         else launch(gemv_tile_kernel<1, E>);

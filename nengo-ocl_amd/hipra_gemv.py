@@ -45,6 +45,10 @@ TASK_OVERHEAD_BYTES = 8192.0  # what starting and finishing a task costs, in str
 # columns or more whose rows are 16-byte aligned; its LDS block has STREAM_STAGE_WORDS words.
 STREAM_MIN_COLS, STREAM_STAGE_WORDS = 5, 2176
 STREAM_NARROW_MAX_ROWS = 128
+# instance of that kernel (`pow2_cols`) for matrices of at most FLAT_MAX_COLS columns
+# whose rows are not 16-byte aligned but lie back to back: blocks of rows are read as
+# aligned runs of memory
+STREAM_FLAT, FLAT_MAX_COLS = 7, 64
 
 
 def stream_class(stages):
@@ -268,6 +272,14 @@ class gemv_prog:
                 and quads_readable(d) for d in dots))
             if stream:
                 return (3, stream_class({stream_stage(d["a_shape1"])[0] for d in dots}), vec)
+            # rows that are not 16-byte aligned but lie back to back, at most 64 columns: row
+            # blocks are aligned runs of memory when tasks start at multiples of 4 rows
+            # (the last quad of a matrix may reach 12 bytes past it)
+            if (vec == 1 and TILE_STAGE_WORDS == STREAM_STAGE_WORDS and dots and all(
+                    d["a_start"] % 4 == 0 and d["a_stride0"] == d["a_shape1"]
+                    and STREAM_MIN_COLS <= d["a_shape1"] <= FLAT_MAX_COLS
+                    and d["a_start"] + M * d["a_shape1"] + 3 <= a_size for d in dots)):
+                return (3, STREAM_FLAT, 4)
             return (3, int(pow2), vec)
         if flavor == 0:
             # Matrix loads are non-temporal, so one wave instruction should take whole
@@ -286,7 +298,7 @@ class gemv_prog:
             lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         return (flavor, lpr, vec)
 
-    def _tile_tasks(self, members, max_rows=256, stream=False):
+    def _tile_tasks(self, members, max_rows=256, stream=False, row_multiple=1):
         """Tasks (item, first row, rows, 0) of the reference-order kernel for large items.
 
         A task is the rows one wave carries through all columns, a few row blocks of
@@ -313,6 +325,8 @@ class gemv_prog:
                     item_rows = _balanced_rows(M, item_rows)
                     if item_rows >= 2 * blk[b]:
                         item_rows -= item_rows % blk[b]
+                    # (tasks that must start at a multiple of so many rows)
+                    item_rows = min(-(-item_rows // row_multiple) * row_multiple, max_rows)
                 for r0 in range(0, M, item_rows):
                     out.append((b, r0, min(item_rows, M - r0), 0))
             return out
@@ -370,7 +384,7 @@ class gemv_prog:
 
         # the one instance of the compile-time-shape kernel that holds the stage widths of
         # all of them takes the items of several instances
-        present = [c for c in by_class if c[0] == 3 and c[1] >= 2]
+        present = [c for c in by_class if c[0] == 3 and c[1] in STREAM_CLASS_STAGES]
         stream = (3, 3, 4)
         if present:
             stream = (3, stream_class(set().union(
@@ -406,7 +420,8 @@ class gemv_prog:
                 # launches without wide dot products keep tasks to 128 rows (the kernel
                 # then needs fewer registers and a fourth wave fits each SIMD)
                 task_rows = self._tile_tasks(
-                    members, STREAM_NARROW_MAX_ROWS if lpr in (3, 5) else 256, stream=lpr >= 2)
+                    members, STREAM_NARROW_MAX_ROWS if lpr in (3, 5, STREAM_FLAT) else 256,
+                    stream=lpr >= 2, row_multiple=4 if lpr == STREAM_FLAT else 1)
             else:
                 task_rows = []
                 for b in (members if flavor != 2 else ()):

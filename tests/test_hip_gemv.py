@@ -141,7 +141,7 @@ def test_ensemble_shapes(queue, pi):
     rng = np.random.RandomState(7)
     shapes = [(4096, 64), (64, 4096), (100, 1), (1, 100), (100, 2), (2, 100), (2000, 32),
               (32, 2000), (132, 64), (64, 132), (5, 5000), (3, 7), (1, 1), (300, 9000), (600, 16),
-              (600, 20), (3000, 4), (700, 50)]
+              (600, 20), (3000, 4), (700, 50), (700, 130)]
     A = RA([rng.normal(size=s) for s in shapes], align=True)
     X = RA([rng.normal(size=s[1]) for s in shapes], align=True)
     Y = RA([rng.normal(size=s[0]) for s in shapes], align=True)
@@ -150,8 +150,9 @@ def test_ensemble_shapes(queue, pi):
     if pi == 0:
         classes = {p.kernel_class for p in prog.plans}
         # compile-time shapes (6: stages of 8 / 16 as well as of 512 columns), 4 columns
-        # (a power of two), rows that are not 16-byte aligned, small
-        assert classes == {(3, 6, 4), (3, 1, 4), (3, 0, 1), (2, 4, 1)}
+        # (a power of two), rows that are not 16-byte aligned (back to back with at most 64
+        # columns: read in quads all the same; otherwise 4-byte loads), small
+        assert classes == {(3, 6, 4), (3, 1, 4), (3, 7, 4), (3, 0, 1), (2, 4, 1)}
 
 
 def test_strided_views_and_yin(queue):
@@ -504,13 +505,72 @@ def test_compile_time_shape_odd_width_views_bit_exact(queue):
     assert np.array_equal(got[0], Yo[0]) and np.array_equal(got[1], Yo[1])
     expect = 0.5 * Ys[0][:, 0] + sum(slim[:, c:c + w] @ x for c, w, x in zip(cols, widths, xs))
     assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
-    # a contiguous matrix of such a width has nothing readable behind its last row: general kernel
+    # a contiguous matrix of such a width at the very end of its buffer has nothing readable
+    # behind its last row: general kernel
     A = RA([rng.normal(size=(700, 50))], align=True)
     X = RA([rng.normal(size=50)], align=True)
     Y = RA([rng.normal(size=700)], align=True)
     js = [np.array([0], dtype=np.int32)]
     prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, 0.0, to_dev(queue, Y))
     assert {p.kernel_class for p in prog.plans} == {(3, 0, 1)}
+
+
+@pytest.mark.parametrize("beta", [1.0, 0.5])
+def test_back_to_back_rows_bit_exact(queue, beta):
+    """Matrices of at most 64 columns whose rows are not 16-byte aligned but lie back to
+    back (10, 50, 30, 5, 6, 13, 63 columns) are read in 16-byte quads block by block: row
+    counts that leave partial blocks, partial last quads and short last tasks, outputs
+    that sum several such dot products (one of them with aligned rows), a Y_in different
+    from Y -- bit-identical to the oracle.  Wider ones, and a column block of a wider
+    matrix with such a width, stay on 4-byte loads."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(2718)
+    shapes = [(4096, 10), (4097, 50), (1001, 30), (2500, 5), (333, 63), (5003, 6), (999, 37),
+              (1026, 13), (300, 62), (8190, 9)]
+    multi = (10, 50, 64, 7, 62)
+    mats = [rng.normal(size=s) for s in shapes] + [rng.normal(size=(1030, n)) for n in multi]
+    mats.append(np.zeros((1, 8)))  # something readable behind the last matrix
+    A = RA(mats, align=True)
+    X = RA([rng.normal(size=m.shape[1]) for m in mats], align=True)
+    Y = RA([rng.normal(size=s[0]) for s in shapes] + [rng.normal(size=1030)], align=True)
+    Yin = RA([rng.normal(size=s[0]) for s in shapes] + [rng.normal(size=1030)], align=True)
+    n = len(shapes)
+    js = [np.array([i], dtype=np.int32) for i in range(n)] + [np.arange(n, n + len(multi), dtype=np.int32)]
+    for use_yin in (False, True):
+        Yo = clone(Y)
+        orc.plan_block_gemv(None, 0.75, A, js, X, js, beta, Yo, Y_in=clone(Yin) if use_yin else None,
+                            gamma=0.125).plans[0]()
+        dY = to_dev(queue, Y)
+        prog = g.plan_block_gemv(queue, 0.75, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY,
+                                 Y_in=to_dev(queue, Yin) if use_yin else None, gamma=0.125)
+        assert {p.kernel_class for p in prog.plans} == {(3, 7, 4)}
+        for plan in prog.plans:
+            plan()
+        got = dY.to_host()
+        for i in range(len(Y)):
+            assert np.array_equal(got[i], Yo[i]), (i, use_yin)
+    expect = 0.75 * (mats[0].astype(np.float32) @ X[0][:, 0]) + beta * Yin[0][:, 0] + 0.125
+    assert np.allclose(Yo[0][:, 0], expect, rtol=1e-4, atol=1e-3)
+
+    # 50 columns of a matrix with 70 whose block starts at column 2: neither aligned rows
+    # nor rows back to back
+    wide = rng.normal(size=(700, 70)).astype(np.float32)
+    Aw = RA([wide], align=True)
+    Av = Aw[[0]]
+    Av.add_views([int(Aw.starts[0]) + 2], [700], [50], [70], [1])
+    Xw = RA([rng.normal(size=50)], align=True)
+    Yw = RA([rng.normal(size=700)], align=True)
+    jA, jX = [np.array([1], dtype=np.int32)], [np.array([0], dtype=np.int32)]
+    Yo = clone(Yw)
+    orc.plan_block_gemv(None, 1.0, Av, jA, Xw, jX, beta, Yo).plans[0]()
+    dY = to_dev(queue, Yw)
+    prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, Av), jA, to_dev(queue, Xw), jX, beta, dY)
+    assert {p.kernel_class for p in prog.plans} == {(3, 0, 1)}
+    for plan in prog.plans:
+        plan()
+    assert np.array_equal(dY.to_host()[0], Yo[0])
 
 
 @pytest.mark.parametrize("tau_kind", ["per-population", "per-neuron"])
@@ -658,11 +718,12 @@ def test_gemv_with_filter_epilogue(queue):
     result = g.fuse_linearfilter(prog.plans, lf[0])
     assert result is not None
     fused, residual = result
-    # compile-time shapes (4096, 2048, 12), 4 columns, rows not 16-byte aligned (30), small
+    # compile-time shapes (4096, 2048, 12), 4 columns, rows not 16-byte aligned but back to
+    # back (30), small
     assert sorted(p.name for p in fused) == ["hipra_gemv.tile_filter"] * 3 + [
         "hipra_gemv.wave_ref_filter"]
     assert {p.kernel_class for p in fused if p.name == "hipra_gemv.tile_filter"} == {
-        (3, 6, 4), (3, 1, 4), (3, 0, 1)}
+        (3, 6, 4), (3, 1, 4), (3, 7, 4)}
     assert [p.name for p in residual] == ["hip_linearfilter"]
     oprog, olf = build(host, orc, orc, None, lambda a: a)
     for step in range(4):
