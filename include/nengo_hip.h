@@ -193,9 +193,13 @@ int nhip_gemv_rows_filter(void *stream, int lpr, int task_words, const int *item
  * Y[b] (=|+=) A[b] @ X[b] for many sparse matrices in one launch.
  * replaces: `plan_sparse_dot_inc` / `spmv_csr_impl` / `spmv_ellpack_impl`
  * (clra_gemv.py:1494-1646, :1649-1755, :1919-1948), which run one launch per
- * matrix.  Layout: sliced ELLPACK with slices of 64 rows; element k of row r of a
- * slice is at data_start + 64 k + r in `cols` (column index) and `vals`, rows padded
- * to the slice's longest row; row r of a slice has row_len[len_start + r] elements.
+ * matrix.  Layout: sliced ELLPACK with slices of 64 rows, four elements of a row per
+ * 16 bytes: element k of row r of a slice is at data_start + 256 (k / 4) + 4 r + k % 4
+ * in `cols` (column index) and `vals`; rows are padded to `width`, the slice's longest
+ * row rounded up to a multiple of 4; row r of a slice has row_len[len_start + r]
+ * elements.  `cols` and `vals` are 16-byte aligned and every data_start is a multiple
+ * of 4 (NHIP_E_BADARG otherwise; the table is not read on the host, so a data_start
+ * or width that is no multiple of 4 is the caller's error).
  *   slices : int32[n_slices][8] {data_start, width, len_start, n_rows (<= 64),
  *                                x_start, y_start (of the slice's first row), inc, 0}
  * X and Y items are contiguous vectors.  Each row is summed in column order with one

@@ -4,10 +4,12 @@
 // The reference keeps each matrix in CSR or ELLPACK and launches one kernel per
 // matrix with one work-item per row (clra_gemv.py:1570-1646, :1649-1755).  Here all
 // matrices of a step share one launch and one layout made for 64-wide waves:
-// rows are cut into slices of 64, and inside a slice element k of row r sits at
-// slice_start + 64 k + r (sliced ELLPACK with slice height 64), padded to the longest
-// row of the slice.  A wave owns a slice, lane r owns row r: every load of values
-// and column indices is one contiguous 256-byte run, and each row is still summed
+// rows are cut into slices of 64 and padded to the longest row of the slice, rounded
+// up to a multiple of 4; inside a slice elements 4q .. 4q+3 of row r sit side by side
+// at slice_start + 256 q + 4 r (sliced ELLPACK with slice height 64, four elements of
+// a row per 16 bytes).  A wave owns a slice, lane r owns row r: a load of values or
+// column indices is one 16-byte access per lane and one contiguous 1-KiB run per wave
+// (a quarter of the address work of 4-byte accesses), and each row is still summed
 // strictly in column order (one fused multiply-add per stored element, starting from
 // the old y when incrementing), which is the order of the reference's CSR kernel, so
 // results are bit-identical to a sequential float32 restatement.  Only the gather
@@ -18,7 +20,7 @@ namespace {
 
 struct SpmvSlice {
     int data_start;  // offset of the slice in `cols` / `vals`
-    int width;       // stored elements per row of the slice (longest row)
+    int width;       // stored elements per row of the slice (longest row, rounded up to 4)
     int len_start;   // offset of the slice's row lengths in `row_len`
     int n_rows;      // rows in the slice (<= 64)
     int x_start;     // element offsets of the item's X and of the slice's first Y row
@@ -27,7 +29,8 @@ struct SpmvSlice {
     int pad;
 };
 
-constexpr int SPMV_UNROLL = 4;  // elements of a row whose operands are fetched together
+typedef int spmv_i4 __attribute__((ext_vector_type(4)));
+typedef float spmv_f4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
     const SpmvSlice* __restrict__ slices, int n_slices, const int* __restrict__ row_len,
@@ -41,36 +44,28 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
     const int len = live ? row_len[sl.len_start + lane] : 0;
     const float* x = X + sl.x_start;
     float acc = (live && sl.inc) ? Y[(size_t)sl.y_start + lane] : 0.0f;
-    const int* c = cols + (size_t)sl.data_start + lane;
-    const float* v = vals + (size_t)sl.data_start + lane;
-    // values and column indices of the next SPMV_UNROLL elements are requested before
-    // the gathers from X of the current ones (past the end: the last again, unused)
-    int ci[SPMV_UNROLL];
-    float vi[SPMV_UNROLL];
+    const int n_quads = sl.width >> 2;  // the host pads the width to a multiple of 4
+    if (n_quads > 0) {
+        const spmv_i4* c = reinterpret_cast<const spmv_i4*>(cols + (size_t)sl.data_start) + lane;
+        const spmv_f4* v = reinterpret_cast<const spmv_f4*>(vals + (size_t)sl.data_start) + lane;
+        // values and column indices of the next two quads are requested before the
+        // gathers from X of the current one (past the end: the last again, unused)
+        const int q1 = min(1, n_quads - 1);
+        spmv_i4 ci = __builtin_nontemporal_load(c), ci1 = __builtin_nontemporal_load(c + (size_t)q1 * NHIP_WAVE);
+        spmv_f4 vi = __builtin_nontemporal_load(v), vi1 = __builtin_nontemporal_load(v + (size_t)q1 * NHIP_WAVE);
+        for (int q = 0; q < n_quads; ++q) {
+            const int qn = min(q + 2, n_quads - 1);
+            const spmv_i4 cn = __builtin_nontemporal_load(c + (size_t)qn * NHIP_WAVE);
+            const spmv_f4 vn = __builtin_nontemporal_load(v + (size_t)qn * NHIP_WAVE);
+            const int k0 = 4 * q;
+            float xi[4];
 #pragma unroll
-    for (int u = 0; u < SPMV_UNROLL; ++u) {
-        const int k = min(u, sl.width - 1);
-        ci[u] = sl.width > 0 ? __builtin_nontemporal_load(c + (size_t)k * NHIP_WAVE) : 0;
-        vi[u] = sl.width > 0 ? __builtin_nontemporal_load(v + (size_t)k * NHIP_WAVE) : 0.0f;
-    }
-    for (int k0 = 0; k0 < sl.width; k0 += SPMV_UNROLL) {
-        int cn[SPMV_UNROLL];
-        float vn[SPMV_UNROLL], xi[SPMV_UNROLL];
+            for (int u = 0; u < 4; ++u) xi[u] = (k0 + u < len) ? x[ci[u]] : 0.0f;
 #pragma unroll
-        for (int u = 0; u < SPMV_UNROLL; ++u) {
-            const int k = min(k0 + SPMV_UNROLL + u, sl.width - 1);
-            cn[u] = __builtin_nontemporal_load(c + (size_t)k * NHIP_WAVE);
-            vn[u] = __builtin_nontemporal_load(v + (size_t)k * NHIP_WAVE);
-        }
-#pragma unroll
-        for (int u = 0; u < SPMV_UNROLL; ++u) xi[u] = (k0 + u < len) ? x[ci[u]] : 0.0f;
-#pragma unroll
-        for (int u = 0; u < SPMV_UNROLL; ++u)
-            if (k0 + u < len) acc = fmaf(vi[u], xi[u], acc);
-#pragma unroll
-        for (int u = 0; u < SPMV_UNROLL; ++u) {
-            ci[u] = cn[u];
-            vi[u] = vn[u];
+            for (int u = 0; u < 4; ++u)
+                if (k0 + u < len) acc = fmaf(vi[u], xi[u], acc);
+            ci = ci1; vi = vi1;
+            ci1 = cn; vi1 = vn;
         }
     }
     if (live) Y[(size_t)sl.y_start + lane] = acc;
@@ -82,6 +77,8 @@ extern "C" int nhip_spmv_sell(void* stream, const int* slices, int n_slices, con
                               const int* cols, const float* vals, const float* X, float* Y) {
     if (n_slices == 0) return 0;
     if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y) return NHIP_E_BADARG;
+    // the kernel reads `cols` and `vals` 16 bytes at a time
+    if ((reinterpret_cast<uintptr_t>(cols) | reinterpret_cast<uintptr_t>(vals)) & 15) return NHIP_E_BADARG;
     const int wpg = NHIP_WG / NHIP_WAVE;
     NHIP_LAUNCH(spmv_sell_kernel, dim3((n_slices + wpg - 1) / wpg), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),

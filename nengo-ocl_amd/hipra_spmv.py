@@ -4,8 +4,9 @@ Counterpart of the reference's ``plan_sparse_dot_inc`` (clra_gemv.py:1919-1948) 
 its ``spmv_prog`` family (:1249-1567), which keep every matrix in CSR or ELLPACK on
 the device and launch one kernel per matrix.  Here any number of matrices share one
 launch: their rows are cut into slices of 64 (the wave width) and stored slice by
-slice, element k of every row of a slice side by side, so that a wave reads values
-and column indices in contiguous runs while each lane sums its row in column order.
+slice, four consecutive elements of every row of a slice side by side, so that a lane
+reads values and column indices 16 bytes at a time, a wave in contiguous 1-KiB runs,
+while each lane sums its row in column order.
 """
 
 import numpy as np
@@ -14,6 +15,14 @@ from .hipraggedarray import to_device
 from .plan import Plan
 
 WG, WAVE = 256, 64
+QUAD = 4  # elements of a row stored side by side (one 16-byte access)
+
+
+def sell_index(data_start, r, j):
+    """Position in ``cols`` / ``vals`` of element ``j`` of row ``r`` of the slice that
+    starts at ``data_start`` (``j`` may be an array)."""
+    j = np.asarray(j)
+    return data_start + WAVE * QUAD * (j // QUAD) + QUAD * r + j % QUAD
 
 
 class HostSparseMatrix:
@@ -32,8 +41,10 @@ def sell_layout(matrices):
     """Sliced-ELLPACK arrays of a list of CSR matrices.
 
     Returns ``(slice_rows, row_len, cols, vals)``: ``slice_rows[k] = (item, data_start,
-    width, len_start, n_rows, row0)``; ``row_len`` padded to 64 per slice; ``cols`` /
-    ``vals`` with element j of row r of slice k at ``data_start + 64 j + r``.
+    width, len_start, n_rows, row0)``; ``width`` is the longest row of the slice rounded
+    up to a multiple of 4, ``row_len`` is padded to 64 per slice; ``cols`` / ``vals``
+    hold element j of row r of slice k at ``data_start + 256 (j // 4) + 4 r + j % 4``
+    (see `sell_index`).
     """
     slice_rows, lens, cols, vals = [], [], [], []
     data_start = 0
@@ -46,15 +57,15 @@ def sell_layout(matrices):
         for row0 in range(0, csr.shape[0], WAVE):
             n_rows = min(WAVE, csr.shape[0] - row0)
             counts = row_counts[row0:row0 + n_rows]
-            width = int(counts.max()) if n_rows else 0
-            block_c = np.zeros((width, WAVE), dtype=np.int32)
-            block_v = np.zeros((width, WAVE), dtype=np.float32)
+            width = -(-(int(counts.max()) if n_rows else 0) // QUAD) * QUAD
+            block_c = np.zeros((width // QUAD, WAVE, QUAD), dtype=np.int32)
+            block_v = np.zeros((width // QUAD, WAVE, QUAD), dtype=np.float32)
             # scatter the slice's elements: position inside its row, row inside the slice
             lo, hi = int(indptr[row0]), int(indptr[row0 + n_rows])
             r = np.repeat(np.arange(n_rows), counts)
             j = np.arange(lo, hi) - np.repeat(indptr[row0:row0 + n_rows], counts)
-            block_c[j, r] = indices[lo:hi]
-            block_v[j, r] = data[lo:hi]
+            block_c[j // QUAD, r, j % QUAD] = indices[lo:hi]
+            block_v[j // QUAD, r, j % QUAD] = data[lo:hi]
             padded = np.zeros(WAVE, dtype=np.int32)
             padded[:n_rows] = counts
             slice_rows.append((item, data_start, width, len(lens) * WAVE, n_rows, row0))

@@ -769,8 +769,8 @@ def test_sparse_products(queue):
         n = row_len[len_start + r]
         lo = csr.indptr[row0 + r]
         assert n == csr.indptr[row0 + r + 1] - lo
-        assert np.array_equal(cols[start + 64 * np.arange(n) + r], csr.indices[lo:lo + n])
-        assert np.array_equal(vals[start + 64 * np.arange(n) + r], csr.data[lo:lo + n])
+        assert np.array_equal(cols[hipra_spmv.sell_index(start, r, np.arange(n))], csr.indices[lo:lo + n])
+        assert np.array_equal(vals[hipra_spmv.sell_index(start, r, np.arange(n))], csr.data[lo:lo + n])
 
     Yo = clone(Y)
     oplan = orc.plan_sparse_dot_inc(None, mats, X, Yo, inc=inc).plans[0]
