@@ -201,7 +201,10 @@ int nhip_gemv_rows_filter(void *stream, int lpr, int task_words, const int *item
  * of 4 (NHIP_E_BADARG otherwise; the table is not read on the host, so a data_start
  * or width that is no multiple of 4 is the caller's error).
  *   slices : int32[n_slices][8] {data_start, width, len_start, n_rows (<= 64),
- *                                x_start, y_start (of the slice's first row), inc, 0}
+ *                                x_start, y_start (of the slice's first row), inc, window}
+ * window >= 0 (a multiple of 4, with x_start a multiple of 4 and X 16-byte aligned): the
+ * 1024 elements of the item's X from `window` on are copied to LDS first and read from
+ * there (they must lie inside X); window < 0: none.  Results do not depend on it.
  * X and Y items are contiguous vectors.  Each row is summed in column order with one
  * fused multiply-add per element (starting from the old y when inc), like the
  * reference's CSR kernel. */

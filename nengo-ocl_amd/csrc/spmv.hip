@@ -13,7 +13,11 @@
 // strictly in column order (one fused multiply-add per stored element, starting from
 // the old y when incrementing), which is the order of the reference's CSR kernel, so
 // results are bit-identical to a sequential float32 restatement.  Only the gather
-// from X is irregular; X is a few MB at most and stays in cache.
+// from X is irregular; X is a few MB at most and stays in cache.  Where the host found
+// a run of SPMV_WINDOW consecutive elements of X that holds a good part of a slice's
+// column indices (band matrices, rings), the wave first copies that run into LDS and
+// takes the elements inside it from there: only the lanes whose column lies outside
+// go to the cache, which spares it one look-up per line and instruction.
 #include "nhip_common.h"
 
 namespace {
@@ -26,8 +30,10 @@ struct SpmvSlice {
     int x_start;     // element offsets of the item's X and of the slice's first Y row
     int y_start;
     int inc;         // 1: Y += A X, 0: Y = A X
-    int pad;
+    int window;      // first element (relative to x_start, multiple of 4) of the run of X kept in LDS; < 0: none
 };
+
+constexpr int SPMV_WINDOW = 1024;  // elements of X a wave keeps in LDS (4 KiB)
 
 typedef int spmv_i4 __attribute__((ext_vector_type(4)));
 typedef float spmv_f4 __attribute__((ext_vector_type(4)));
@@ -38,8 +44,21 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
 {
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int s = blockIdx.x * (NHIP_WG / NHIP_WAVE) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (s >= n_slices) return;  // wave-uniform; the kernel has no barrier
-    const SpmvSlice sl = slices[s];
+    __shared__ __attribute__((aligned(16))) float s_x[NHIP_WG / NHIP_WAVE][SPMV_WINDOW];
+    // waves past the last slice have no work but still meet the group barrier below
+    const bool has_slice = s < n_slices;
+    SpmvSlice sl = slices[has_slice ? s : 0];
+    if (!has_slice) { sl.n_rows = 0; sl.width = 0; sl.window = -1; }
+    float* wx = s_x[__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)];
+    if (sl.window >= 0) {
+        const spmv_f4* src = reinterpret_cast<const spmv_f4*>(X + sl.x_start + sl.window) + lane;
+#pragma unroll
+        for (int i = 0; i < SPMV_WINDOW / (4 * NHIP_WAVE); ++i)
+            reinterpret_cast<spmv_f4*>(wx)[i * NHIP_WAVE + lane] = src[i * NHIP_WAVE];
+    }
+    __syncthreads();  // every wave of the group arrives here exactly once
+    const unsigned win_lo = sl.window >= 0 ? (unsigned)sl.window : 0u;
+    const unsigned win_n = sl.window >= 0 ? (unsigned)SPMV_WINDOW : 0u;
     const bool live = lane < sl.n_rows;
     const int len = live ? row_len[sl.len_start + lane] : 0;
     const float* x = X + sl.x_start;
@@ -60,7 +79,10 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
             const int k0 = 4 * q;
             float xi[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) xi[u] = (k0 + u < len) ? x[ci[u]] : 0.0f;
+            for (int u = 0; u < 4; ++u) {
+                const unsigned w = (unsigned)ci[u] - win_lo;  // position inside the run kept in LDS
+                xi[u] = (k0 + u < len) ? (w < win_n ? wx[w] : x[ci[u]]) : 0.0f;
+            }
 #pragma unroll
             for (int u = 0; u < 4; ++u)
                 if (k0 + u < len) acc = fmaf(vi[u], xi[u], acc);
@@ -68,7 +90,7 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
             ci1 = cn; vi1 = vn;
         }
     }
-    if (live) Y[(size_t)sl.y_start + lane] = acc;
+    if (live) Y[(size_t)sl.y_start + lane] = acc;  // no wave without a slice is live
 }
 
 }  // namespace
@@ -77,8 +99,10 @@ extern "C" int nhip_spmv_sell(void* stream, const int* slices, int n_slices, con
                               const int* cols, const float* vals, const float* X, float* Y) {
     if (n_slices == 0) return 0;
     if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y) return NHIP_E_BADARG;
-    // the kernel reads `cols` and `vals` 16 bytes at a time
-    if ((reinterpret_cast<uintptr_t>(cols) | reinterpret_cast<uintptr_t>(vals)) & 15) return NHIP_E_BADARG;
+    // the kernel reads `cols`, `vals` and the runs of X it keeps in LDS 16 bytes at a time
+    if ((reinterpret_cast<uintptr_t>(cols) | reinterpret_cast<uintptr_t>(vals) |
+         reinterpret_cast<uintptr_t>(X)) & 15)
+        return NHIP_E_BADARG;
     const int wpg = NHIP_WG / NHIP_WAVE;
     NHIP_LAUNCH(spmv_sell_kernel, dim3((n_slices + wpg - 1) / wpg), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),

@@ -16,6 +16,20 @@ from .plan import Plan
 
 WG, WAVE = 256, 64
 QUAD = 4  # elements of a row stored side by side (one 16-byte access)
+WINDOW = 1024  # consecutive elements of X a wave can keep in LDS (SPMV_WINDOW in csrc/spmv.hip)
+
+
+def slice_window(columns, n_cols, x_start):
+    """First element of the run of `WINDOW` consecutive elements of X that a wave keeps
+    in LDS for a slice with the given column indices, or -1 for none: the run is centred
+    on the median column, starts on a multiple of 4 (16-byte reads; X itself must start
+    on one) and lies inside X; it is used when it holds at least a quarter of the indices."""
+    if columns.size == 0 or n_cols < WINDOW or x_start % QUAD:
+        return -1
+    lo = int(np.median(columns)) - WINDOW // 2
+    lo = max(0, min(lo, n_cols - WINDOW)) // QUAD * QUAD
+    inside = np.count_nonzero((columns >= lo) & (columns < lo + WINDOW))
+    return lo if 4 * inside >= columns.size else -1
 
 
 def sell_index(data_start, r, j):
@@ -105,8 +119,11 @@ class plan_sparse_dot_inc:
         slice_rows, row_len, cols, vals = sell_layout(matrices)
         table = np.zeros((max(len(slice_rows), 1), 8), dtype=np.int32)
         for k, (item, data_start, width, len_start, n_rows, row0) in enumerate(slice_rows):
+            csr = matrices[item].csr
+            window = slice_window(csr.indices[csr.indptr[row0]:csr.indptr[row0 + n_rows]],
+                                  csr.shape[1], int(X.starts[item]))
             table[k] = (data_start, width, len_start, n_rows, int(X.starts[item]),
-                        int(Y.starts[item]) + row0, int(incs[item]), 0)
+                        int(Y.starts[item]) + row0, int(incs[item]), window)
         if vals.size >= 2 ** 31:
             raise ValueError("more than 2^31 stored elements")
         n = len(slice_rows)

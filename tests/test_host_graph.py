@@ -474,3 +474,26 @@ def test_large_item_task_sizes():
     assert max(n for _, _, n, _ in tasks_of(192, 2000, 32, 128)) == 96
     # 64 x 4096 on a device of 64 compute units: 16-row tasks would be too few (1032)
     assert max(n for _, _, n, _ in tasks_of(258, 64, 4096, 256, n_cu=64)) < 16
+
+
+def test_sparse_slice_window():
+    """The run of X a wave keeps in LDS for a slice: centred on the median column, a
+    multiple of 4, inside X; none for short or misaligned X, and none when it would hold
+    less than a quarter of the slice's column indices."""
+    from nengo_ocl_amd import hipra_spmv as h
+
+    band = np.arange(5000, 5164).repeat(3)
+    lo = h.slice_window(band, 100000, 64)
+    assert lo % 4 == 0 and lo <= 5000 and lo + h.WINDOW >= 5164
+    assert h.slice_window(band, 100000, 62) == -1            # X does not start on 16 bytes
+    assert h.slice_window(np.arange(10), 500, 0) == -1       # X shorter than the window
+    assert h.slice_window(np.zeros(0, dtype=np.int32), 100000, 0) == -1
+    assert h.slice_window(np.arange(99990, 100000), 100000, 0) == 100000 - h.WINDOW
+    assert h.slice_window(np.arange(0, 10), 100001, 0) == 0
+    end = h.slice_window(np.arange(99995, 100001), 100001, 0)
+    assert end % 4 == 0 and end + h.WINDOW <= 100001 and end <= 99995
+    scattered = np.random.RandomState(0).randint(100000, size=6400)
+    assert h.slice_window(scattered, 100000, 0) == -1
+    mixed = np.sort(np.concatenate([band, scattered[:band.size // 4]]))  # four fifths in the band
+    lo = h.slice_window(mixed, 100000, 0)
+    assert lo >= 0 and lo <= 5000 and lo + h.WINDOW >= 5164
