@@ -38,6 +38,7 @@ extern "C" {
 #define NHIP_E_BADARG (-1)   /* null pointer / negative count / unknown mode   */
 #define NHIP_E_BADCLASS (-2) /* GEMV class (lanes-per-row, vector width) unknown */
 #define NHIP_E_RTC (-3)      /* run-time compilation failed (see the log)          */
+#define NHIP_E_TOOBIG (-4)   /* the request does not fit the workspace it was given */
 
 /* ---- library ---------------------------------------------------------- */
 int nhip_abi_version(void);
@@ -381,6 +382,27 @@ int nhip_direct_unary(void *stream, int opcode, const int *desc, int n, int lane
  * position still advances), so an undrained buffer can never be overrun. */
 int nhip_probes(void *stream, const int *desc, int n, int lanes, float *countdowns,
                 int *bufpositions, const float *periods, const float *X, float *Y);
+/* End-of-batch drain of the probe buffers in one device-to-host transfer.
+ * replaces: the host loop of `Simulator._probe` (simulator.py:499-520: one transfer
+ * of `bufpositions`, one whole-buffer transfer per probe, a fill, two `finish()`),
+ * and the reads of the step counter and clock behind `sim.n_steps` / `sim.time`.
+ * A kernel packs into `staging` (device workspace of `staging_words` floats), in words:
+ *   [0] signals[step_start], [1] signals[time_start], [2 .. 2+n) bufpositions (int bits),
+ *   zero padding up to NHIP_DRAIN_HEADER(n); then for probe i its first
+ *   min(bufpositions[i], capacity_i, rows_bound) rows at
+ *   NHIP_DRAIN_HEADER(n) + rows_bound * wprefix_i (row-major, width_i words per row);
+ * then bufpositions is zeroed, the first NHIP_DRAIN_HEADER(n) + rows_bound * total_width
+ * words are copied to `host_out` (HOST memory of at least that size; pinned memory makes
+ * the copy a single DMA) and the stream is synchronised: on return `host_out` is valid.
+ *   desc : int32[n][4] {y_start, width, wprefix, capacity}, wprefix_i = sum of width_j, j < i
+ *   total_width = sum of widths, max_width = the largest; rows_bound = the caller's upper
+ *   bound on rows buffered since the last drain (rows beyond it are not transferred; the
+ *   reported counts still tell).  NHIP_E_TOOBIG if the block does not fit `staging`. */
+#define NHIP_DRAIN_HEADER(n) ((((n) + 2) + 63) / 64 * 64)
+int nhip_probes_drain(void *stream, const int *desc, int n_probes, int total_width,
+                      int max_width, int rows_bound, int *bufpositions, const float *Y,
+                      const float *signals, int step_start, int time_start, float *staging,
+                      long long staging_words, float *host_out);
 /* fill an int32 device array (used to zero probe buffer positions without a
  * memset node, so that it may also be recorded into a graph) */
 int nhip_fill_i32(void *stream, int *dst, int n, int value);
@@ -458,19 +480,12 @@ int nhip_rtc_launch_direct(void *stream, void *function, int n, const int *t_sta
  * stream into a graph and replayed. */
 int nhip_capture_begin(void *stream);
 int nhip_capture_end(void *stream, void **graph_exec_out);
+/* Hands an instantiated graph to the device ahead of its first launch (nothing is
+ * executed), so that the first launch costs what every later one costs. */
+int nhip_graph_upload(void *graph_exec, void *stream);
 int nhip_graph_launch(void *graph_exec, void *stream, int n_times);
 int nhip_graph_destroy(void *graph_exec);
 int nhip_stream_sync(void *stream);
-/* Branches of a timestep that do not depend on each other (the reference runs its
- * plans strictly in order on one in-order queue, plan.py:137-149) are recorded on
- * side streams: a side stream joins the recording by waiting on an event recorded
- * on a stream that is already being captured, and the capturing stream waits on
- * an event of every side stream before nhip_capture_end.  The graph keeps only
- * these dependencies; replays run independent kernels side by side. */
-int nhip_stream_create(void **stream_out); /* non-blocking, default priority */
-int nhip_stream_destroy(void *stream);
-int nhip_stream_wait_event(void *stream, void *event);
-
 /* The next kernel launched by the calling thread through this library carries
  * `start` and `stop` itself: their difference is the kernel's own duration, without
  * the dispatch latency and end-of-kernel cache maintenance that events recorded
@@ -478,6 +493,9 @@ int nhip_stream_wait_event(void *stream, void *event);
  * Not for launches that are being recorded into a graph, and not for
  * nhip_rtc_launch_direct (which launches through the module API). */
 int nhip_time_next_launch(void *start, void *stop);
+/* 1 while events armed by nhip_time_next_launch wait for a launch (an entry point
+ * that returned without launching, e.g. on an empty work list, leaves them so), else 0. */
+int nhip_launch_events_pending(void);
 
 /* events on `stream` (for per-plan and whole-run timing) */
 int nhip_event_create(void **event_out);

@@ -62,18 +62,19 @@ SIGNATURES = {
     "nhip_presentinput": [P, P, c_int, c_int, c_float, P, P, P],
     "nhip_direct_unary": [P, c_int, P, c_int, c_int, P, P],
     "nhip_probes": [P, P, c_int, c_int, P, P, P, P, P],
+    "nhip_probes_drain": [P, P, c_int, c_int, c_int, c_int, P, P, P, c_int, c_int, P,
+                          ctypes.c_longlong, P],
     "nhip_fill_i32": [P, P, c_int, c_int],
     "nhip_sequence": [P, P, c_int, c_int],
     "nhip_sequence_chains": [P, P, P, P, c_int],
     "nhip_capture_begin": [P],
     "nhip_capture_end": [P, ctypes.POINTER(c_void_p)],
+    "nhip_graph_upload": [P, P],
     "nhip_graph_launch": [P, P, c_int],
     "nhip_graph_destroy": [P],
     "nhip_stream_sync": [P],
-    "nhip_stream_create": [ctypes.POINTER(c_void_p)],
-    "nhip_stream_destroy": [P],
-    "nhip_stream_wait_event": [P, P],
     "nhip_time_next_launch": [P, P],
+    "nhip_launch_events_pending": [],
     "nhip_event_create": [ctypes.POINTER(c_void_p)],
     "nhip_event_record": [P, P],
     "nhip_event_elapsed_ms": [P, P, ctypes.POINTER(c_float)],

@@ -387,6 +387,41 @@ __global__ __launch_bounds__(NHIP_WG) void probes_kernel(const ProbeDesc* __rest
     NHIP_FOR_MY_ROW(L, n_rows, probes_block(desc[row], countdowns, bufpositions, periods, X, Y, row, lane, LL));
 }
 
+// ---------------------------------------------------------------- probe drain
+// What the host needs at the end of a batch of steps -- the step counter, the clock, how
+// many rows every probe buffered, and those rows -- packed into one contiguous block so
+// that a single device-to-host copy fetches it (the reference reads every probe buffer
+// whole, one transfer per probe, simulator.py:499-520).  Layout of the block, in words:
+// [0] step, [1] time, [2 .. 2+n) row counts (int bits), padded to `header` words; then for
+// probe i `rows_bound` rows of `width_i` words at header + rows_bound * wprefix_i.
+// blockIdx.y = probe, blockIdx.x = run of 1024 words of its region.
+struct DrainDesc { int y_start, width, wprefix, capacity; };
+
+__global__ __launch_bounds__(NHIP_WG) void probes_pack_kernel(
+    const DrainDesc* __restrict__ desc, int n_probes, const int* __restrict__ bufpositions,
+    const float* __restrict__ Y, const float* __restrict__ signals, int step_start,
+    int time_start, int rows_bound, int header, float* __restrict__ out) {
+    const int probe = blockIdx.y;
+    if (blockIdx.x == 0 && probe == 0 && threadIdx.x == 0) {
+        out[0] = signals[step_start];
+        out[1] = signals[time_start];
+    }
+    if (probe >= n_probes) return;  // a launch without probes still packs the clock
+    const DrainDesc d = desc[probe];
+    const int count = bufpositions[probe];
+    if (blockIdx.x == 0 && threadIdx.x == 0) out[2 + probe] = __int_as_float(count);
+    const int rows = min(min(count, d.capacity), rows_bound);
+    const int n_words = rows * d.width;
+    const float* src = Y + d.y_start;
+    float* dst = out + header + (size_t)rows_bound * d.wprefix;
+    const int w0 = blockIdx.x * 1024;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int w = w0 + k * NHIP_WG + threadIdx.x;
+        if (w < n_words) dst[w] = src[w];
+    }
+}
+
 __global__ __launch_bounds__(NHIP_WG) void fill_i32_kernel(int* dst, int n, int value) {
     const int i = blockIdx.x * NHIP_WG + threadIdx.x;
     if (i < n) dst[i] = value;
@@ -647,6 +682,37 @@ extern "C" int nhip_fill_i32(void* stream, int* dst, int n, int value) {
                        NHIP_STREAM(stream), dst, n, value);
     NHIP_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int nhip_probes_drain(void* stream, const int* desc, int n_probes, int total_width,
+                                 int max_width, int rows_bound, int* bufpositions, const float* Y,
+                                 const float* signals, int step_start, int time_start,
+                                 float* staging, long long staging_words, float* host_out) {
+    if (n_probes < 0 || total_width < 0 || max_width < 0 || max_width > total_width ||
+        rows_bound < 0 || (n_probes > 0 && (!desc || !bufpositions || !Y)) || !signals ||
+        step_start < 0 || time_start < 0 || !staging || !host_out)
+        return NHIP_E_BADARG;
+    const long long header = NHIP_DRAIN_HEADER(n_probes);
+    const long long words = header + (long long)rows_bound * total_width;
+    if (words > staging_words) return NHIP_E_TOOBIG;
+    const long long widest = (long long)rows_bound * max_width;
+    if (widest > (1LL << 30)) return NHIP_E_TOOBIG;
+    const dim3 grid((unsigned)((widest + 1023) / 1024 > 0 ? (widest + 1023) / 1024 : 1),
+                    (unsigned)(n_probes > 0 ? n_probes : 1));
+    hipStream_t s = NHIP_STREAM(stream);
+    NHIP_LAUNCH(probes_pack_kernel, grid, dim3(NHIP_WG), 0, s,
+                reinterpret_cast<const DrainDesc*>(desc), n_probes, bufpositions, Y, signals,
+                step_start, time_start, rows_bound, (int)header, staging);
+    NHIP_LAUNCH_CHECK();
+    if (n_probes > 0) {
+        hipLaunchKernelGGL(fill_i32_kernel, dim3((n_probes + NHIP_WG - 1) / NHIP_WG), dim3(NHIP_WG),
+                           0, s, bufpositions, n_probes, 0);
+        NHIP_LAUNCH_CHECK();
+    }
+    hipError_t e = hipMemcpyAsync(host_out, staging, (size_t)words * sizeof(float),
+                                  hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return (int)e;
+    return (int)hipStreamSynchronize(s);
 }
 
 extern "C" int nhip_sequence_chains(void* stream, const void* ops, const int* chain_ops,

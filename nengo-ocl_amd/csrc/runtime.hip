@@ -19,11 +19,16 @@ extern "C" int nhip_time_next_launch(void* start, void* stop) {
     return 0;
 }
 
+extern "C" int nhip_launch_events_pending(void) {
+    return nhip_launch_events.start != nullptr ? 1 : 0;
+}
+
 extern "C" const char* nhip_error_string(int err) {
     switch (err) {
         case 0: return "success";
         case NHIP_E_BADARG: return "nengo_hip: bad argument (null pointer, negative count or unknown mode)";
         case NHIP_E_BADCLASS: return "nengo_hip: unknown GEMV kernel class (flavor, lanes per row, vector width)";
+        case NHIP_E_TOOBIG: return "nengo_hip: the request is larger than the workspace it was given";
         case NHIP_E_RTC: return "nengo_hip: run-time compilation of a function node failed (see its log)";
     }
     return hipGetErrorString(static_cast<hipError_t>(err));
@@ -68,6 +73,12 @@ extern "C" int nhip_capture_end(void* stream, void** graph_exec_out) {
     return 0;
 }
 
+extern "C" int nhip_graph_upload(void* graph_exec, void* stream) {
+    if (!graph_exec) return NHIP_E_BADARG;
+    return (int)hipGraphUpload(static_cast<hipGraphExec_t>(graph_exec),
+                               static_cast<hipStream_t>(stream));
+}
+
 extern "C" int nhip_graph_launch(void* graph_exec, void* stream, int n_times) {
     if (!graph_exec || n_times < 0) return NHIP_E_BADARG;
     for (int i = 0; i < n_times; ++i) {
@@ -85,28 +96,6 @@ extern "C" int nhip_graph_destroy(void* graph_exec) {
 
 extern "C" int nhip_stream_sync(void* stream) {
     return (int)hipStreamSynchronize(static_cast<hipStream_t>(stream));
-}
-
-// Side streams carry the branches of a timestep that do not depend on each other
-// while the step is recorded; the recorded graph keeps only the dependencies.
-extern "C" int nhip_stream_create(void** stream_out) {
-    if (!stream_out) return NHIP_E_BADARG;
-    hipStream_t s = nullptr;
-    hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);  // default priority
-    if (e != hipSuccess) return (int)e;
-    *stream_out = s;
-    return 0;
-}
-
-extern "C" int nhip_stream_destroy(void* stream) {
-    if (!stream) return 0;
-    return (int)hipStreamDestroy(static_cast<hipStream_t>(stream));
-}
-
-extern "C" int nhip_stream_wait_event(void* stream, void* event) {
-    if (!stream || !event) return NHIP_E_BADARG;
-    return (int)hipStreamWaitEvent(static_cast<hipStream_t>(stream),
-                                   static_cast<hipEvent_t>(event), 0);
 }
 
 extern "C" int nhip_event_create(void** event_out) {

@@ -35,7 +35,7 @@ import re
 import numpy as np
 
 from . import _lib
-from .hipraggedarray import DeviceArray, HIPRaggedArray, to_device
+from .hipraggedarray import DeviceArray, HIPRaggedArray, _torch, to_device
 from .plan import Plan
 from .utils import f32_bits, is_number
 
@@ -347,6 +347,79 @@ def plan_probes(queue, periods, X, Y, tag=None):
                         + dev_bufpositions.nbytes)
     plan.description = _description(X)
     return plan
+
+
+class ProbeDrain:
+    """End-of-batch transfer of the step counter, the clock and the buffered probe rows
+    in one device-to-host copy (`nhip_probes_drain`); what `Simulator._probe` does in the
+    reference with one transfer per probe (simulator.py:499-520).
+
+    ``probe_plan`` is the plan returned by `plan_probes` (or None for a model without
+    probes: the drain then fetches the clock only); ``signals`` the ragged array holding
+    the step counter (item ``step_idx``) and the clock (``time_idx``)."""
+
+    STAGING_BYTES = 16 * 1024 * 1024  # larger drains are read buffer by buffer
+
+    def __init__(self, queue, probe_plan, signals, step_idx, time_idx):
+        import ctypes
+
+        torch = _torch()
+        self.queue, self.plan, self.signals = queue, probe_plan, signals
+        self.step_start = int(signals.starts[step_idx])
+        self.time_start = int(signals.starts[time_idx])
+        if probe_plan is not None:
+            Y = probe_plan.Y
+            widths = np.asarray(Y.shape1s, dtype=np.int64)
+            self.capacities = np.asarray(Y.shape0s, dtype=np.int64)
+            self.n = len(Y)
+        else:
+            widths = np.zeros(0, dtype=np.int64)
+            self.capacities = np.zeros(0, dtype=np.int64)
+            self.n = 0
+        self.widths = widths
+        self.wprefix = np.concatenate([[0], np.cumsum(widths)[:-1]]).astype(np.int64) if self.n else widths
+        self.total_width = int(widths.sum())
+        self.max_width = int(widths.max()) if self.n else 0
+        self.header = (self.n + 2 + 63) // 64 * 64
+        full = self.header + int(self.capacities.max() if self.n else 0) * self.total_width
+        self.words = int(min(full, max(self.STAGING_BYTES // 4, self.header + self.total_width)))
+        if self.n:
+            self.table, _ = _dev_table(queue, [Y.starts, widths, self.wprefix, self.capacities], 4)
+        else:
+            self.table = None
+        with queue.context():
+            self.staging = torch.zeros(self.words, dtype=torch.float32, device=queue.device)
+        self.host = torch.zeros(self.words, dtype=torch.float32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self._p = ctypes.c_void_p
+
+    def max_rows(self):
+        """Most rows per probe one transfer can carry."""
+        if not self.n:
+            return 0
+        return (self.words - self.header) // max(self.total_width, 1)
+
+    def __call__(self, rows_bound):
+        """Returns ``(step, time, counts, rows)``: ``rows[i]`` is an array of shape
+        ``(min(counts[i], rows_bound), width_i)`` (a copy).  Buffer positions are zero
+        afterwards."""
+        p = self._p
+        rows_bound = int(min(rows_bound, self.capacities.max())) if self.n else 0
+        plan = self.plan
+        _lib.check(self.queue.lib.nhip_probes_drain(
+            self.queue.handle, self.table.ptr if self.n else None, self.n, self.total_width,
+            self.max_width, rows_bound, plan.dev_bufpositions.ptr if self.n else None,
+            plan.Y.ptr if self.n else None, self.signals.ptr, self.step_start, self.time_start,
+            p(self.staging.data_ptr()), self.words, p(self.host.data_ptr())), "probe drain")
+        out = self.host_np
+        counts = out[2:2 + self.n].view(np.int32).copy()
+        rows = []
+        for i in range(self.n):
+            k = int(min(counts[i], rows_bound, self.capacities[i]))
+            w = int(self.widths[i])
+            a = self.header + rows_bound * int(self.wprefix[i])
+            rows.append(out[a:a + k * w].reshape(k, w).copy())
+        return float(out[0]), float(out[1]), counts, rows
 
 
 # ---------------------------------------------------------------- function nodes

@@ -85,17 +85,17 @@ class Plan(BasePlan):
             raise ValueError("launch sizes must be positive, got %r" % (size,))
         return size
 
-    def enqueue(self, wait_for=None, profiling=False, stream=None):
-        """Put the launch on the queue's stream (or on `stream`, a raw handle, while a
-        timestep with independent branches is being recorded); returns immediately."""
+    def enqueue(self, wait_for=None, profiling=False):
+        """Put the launch on the queue's stream; returns immediately."""
         lib = self.queue.lib
-        handle = self.queue.handle if stream is None else stream
+        handle = self.queue.handle
         if profiling:
             ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
             _lib.check(lib.nhip_event_create(ctypes.byref(ev0)))
             _lib.check(lib.nhip_event_create(ctypes.byref(ev1)))
             # the kernel carries its own start / stop events where the entry point
-            # launches through the runtime API; otherwise events around the launch
+            # launches through the runtime API; otherwise events around the launch.  An
+            # entry point that issues several launches times its first one only.
             own = getattr(self.kern, "__name__", "") not in self.LAUNCHES_WITHOUT_EVENTS
             if own:
                 _lib.check(lib.nhip_time_next_launch(ev0, ev1))
@@ -103,9 +103,14 @@ class Plan(BasePlan):
                 _lib.check(lib.nhip_event_record(ev0, handle))
         _lib.check(self.kern(handle, *self.args), self.name)
         if profiling:
-            if own:
-                _lib.check(lib.nhip_time_next_launch(None, None))  # in case nothing was launched
-            else:
+            if own and lib.nhip_launch_events_pending():
+                # the entry point returned without launching (an empty work list): the
+                # events were never recorded and there is nothing to time
+                _lib.check(lib.nhip_time_next_launch(None, None))
+                lib.nhip_event_destroy(ev0)
+                lib.nhip_event_destroy(ev1)
+                return self
+            if not own:
                 _lib.check(lib.nhip_event_record(ev1, handle))
             self._events_to_profile.append((ev0, ev1))
         return self
@@ -169,59 +174,50 @@ def plan_dependencies(plans):
 
 
 class _GraphSegment:
-    """A run of consecutive device plans recorded into one executable graph.
+    """A run of consecutive device plans recorded into executable graphs.
 
-    With `deps` (see `plan_dependencies`) the plans are recorded on several streams so
-    that the graph holds their true dependencies only: kernels of one timestep that
-    do not touch the same memory run side by side when the graph is replayed, which
-    takes the short launch-latency-bound kernels (clock, inputs, filters, probes)
-    off the critical path of the long ones.
+    Between two graph launches the device idles for several microseconds, so the run is
+    recorded several times: as a long graph holding `unroll` consecutive timesteps, and
+    as graphs of unroll/2, ..., 2, 1 timesteps for what is left over (n steps are then
+    n // unroll launches of the long graph plus at most one launch of each shorter one).
+    All of them are recorded, instantiated and uploaded to the device by `prepare`,
+    before the first step runs, so that no call of `launch` ever records anything.
     """
 
-    MAX_SIDE_STREAMS = 7
     MAX_UNROLL = 16        # timesteps recorded back to back into the long graph
     MAX_GRAPH_NODES = 1024
 
-    def __init__(self, queue, plans, deps=None):
+    def __init__(self, queue, plans):
         self.queue = queue
         self.plans = list(plans)
-        self.deps = deps
         self.execs = {}  # timesteps per graph -> executable graph
-        self.unroll = max(1, min(self.MAX_UNROLL, self.MAX_GRAPH_NODES // max(1, len(self.plans))))
-        self._side_streams = []
-        self.n_streams_used = 1
+        unroll = 1
+        while unroll * 2 <= self.MAX_UNROLL and unroll * 2 * len(self.plans) <= self.MAX_GRAPH_NODES:
+            unroll *= 2
+        self.unroll = unroll  # a power of two
+
+    @property
+    def sizes(self):
+        """Timesteps per recorded graph, longest first."""
+        out, n = [], self.unroll
+        while n >= 1:
+            out.append(n)
+            n //= 2
+        return out
 
     def capture(self, n_steps=1):
-        """Record `n_steps` consecutive timesteps into one executable graph.  Between two
-        graph launches the device idles for several microseconds; a graph that holds
-        many steps pays that once."""
+        """Record `n_steps` consecutive timesteps into one executable graph."""
         lib = self.queue.lib
         _lib.check(lib.nhip_capture_begin(self.queue.handle), "graph capture begin")
         err = None
-        events = []
-        self._recording_sides = []  # side streams that have joined this recording
         try:
             for _ in range(n_steps):
-                if self.deps is None:
-                    for plan in self.plans:
-                        plan.enqueue()
-                else:
-                    self._record_branches(events)
+                for plan in self.plans:
+                    plan.enqueue()
         except Exception as e:  # close the capture before re-raising
             err = e
-            # side streams that joined the recording must be led back into the recording
-            # stream first: ending a capture with unjoined streams is an error the
-            # runtime does not survive
-            for side in self._recording_sides:
-                ev = ctypes.c_void_p()
-                if lib.nhip_event_create(ctypes.byref(ev)) == 0:
-                    events.append(ev)
-                    if lib.nhip_event_record(ev, side) == 0:
-                        lib.nhip_stream_wait_event(self.queue.handle, ev)
         handle = ctypes.c_void_p()
         rc = lib.nhip_capture_end(self.queue.handle, ctypes.byref(handle))
-        for ev in events:
-            lib.nhip_event_destroy(ev)
         if err is not None:
             if rc == 0 and handle:
                 lib.nhip_graph_destroy(handle)
@@ -229,79 +225,35 @@ class _GraphSegment:
         _lib.check(rc, "graph capture end")
         self.execs[n_steps] = handle
 
+    def prepare(self):
+        """Record every graph `launch` can ask for and hand each to the device ahead of
+        its first launch; nothing is executed."""
+        for n_steps in self.sizes:
+            if n_steps not in self.execs:
+                self.capture(n_steps)
+                _lib.check(self.queue.lib.nhip_graph_upload(self.execs[n_steps], self.queue.handle),
+                           "graph upload")
+
     @property
     def exec(self):
         return self.execs.get(1)
 
-    def _record_branches(self, events):
-        lib = self.queue.lib
-        streams = [self.queue.handle]
-
-        def new_event(stream):
-            ev = ctypes.c_void_p()
-            _lib.check(lib.nhip_event_create(ctypes.byref(ev)), "event create")
-            events.append(ev)
-            _lib.check(lib.nhip_event_record(ev, stream), "event record")
-            return ev
-
-        def side_stream():
-            k = len(streams) - 1
-            if k == len(self._side_streams):
-                s = ctypes.c_void_p()
-                _lib.check(lib.nhip_stream_create(ctypes.byref(s)), "stream create")
-                self._side_streams.append(s)
-            streams.append(self._side_streams[k])
-            return len(streams) - 1
-
-        fork = new_event(streams[0])  # start of the step: what a branch without inputs waits for
-        tail = {0: None}   # stream -> plan recorded last on it
-        where, done = {}, {}
-        for i, plan in enumerate(self.plans):
-            deps = self.deps[i]
-            si = None
-            for d in sorted(deps, reverse=True):  # continue the stream of a dependency
-                if tail[where[d]] == d:
-                    si = where[d]
-                    break
-            if si is None:
-                if tail[0] is None and not deps:
-                    si = 0
-                elif len(streams) <= self.MAX_SIDE_STREAMS:
-                    si = side_stream()
-                    tail[si] = None
-                    _lib.check(lib.nhip_stream_wait_event(streams[si], fork), "fork")
-                    if streams[si] not in self._recording_sides:
-                        self._recording_sides.append(streams[si])
-                else:  # out of streams: queue behind the oldest tail (an extra, harmless edge)
-                    si = min(tail, key=lambda k: -1 if tail[k] is None else tail[k])
-            for d in deps:
-                if where[d] != si:
-                    _lib.check(lib.nhip_stream_wait_event(streams[si], done[d]), "join")
-            plan.enqueue(stream=streams[si])
-            done[i] = new_event(streams[si])
-            tail[si], where[i] = i, si
-        for k, last in tail.items():
-            if k != 0 and last is not None:
-                _lib.check(lib.nhip_stream_wait_event(streams[0], done[last]), "join")
-        self.n_streams_used = len(streams)
-
     def launch(self, n):
         lib = self.queue.lib
-        long_runs, rest = (n // self.unroll, n % self.unroll) if self.unroll > 1 else (0, n)
-        for n_steps, times in ((self.unroll, long_runs), (1, rest)):
-            if times:
-                if n_steps not in self.execs:
-                    self.capture(n_steps)
-                _lib.check(lib.nhip_graph_launch(self.execs[n_steps], self.queue.handle, times),
+        self.prepare()
+        times, rest = divmod(n, self.unroll)
+        if times:
+            _lib.check(lib.nhip_graph_launch(self.execs[self.unroll], self.queue.handle, times),
+                       "graph launch")
+        for n_steps in self.sizes[1:]:
+            if rest & n_steps:
+                _lib.check(lib.nhip_graph_launch(self.execs[n_steps], self.queue.handle, 1),
                            "graph launch")
 
     def destroy(self):
         for handle in self.execs.values():
             self.queue.lib.nhip_graph_destroy(handle)
         self.execs = {}
-        for s in self._side_streams:
-            self.queue.lib.nhip_stream_destroy(s)
-        self._side_streams = []
 
 
 class Plans:
@@ -319,7 +271,6 @@ class Plans:
         self.plans = list(planlist)
         self.profiling = profiling
         self.use_graph = use_graph
-        self.branches = branches  # record independent plans as parallel graph branches
         self._segments = None  # list of _GraphSegment | PythonPlan
 
     def __call__(self):
@@ -345,8 +296,7 @@ class Plans:
 
         def close_run():
             if run:
-                deps = plan_dependencies(run) if self.branches else None
-                segments.append(_GraphSegment(run[0].queue, run, deps))
+                segments.append(_GraphSegment(run[0].queue, run))
 
         for plan in self.plans:
             if hasattr(plan, "enqueue"):
@@ -357,6 +307,21 @@ class Plans:
                 segments.append(plan)
         close_run()
         self._segments = segments
+
+    def prepare(self):
+        """Record all graphs of the executor now (the Simulator calls this once its plan
+        list is complete), so that the first `run_steps` -- of any length -- only
+        launches.  Does nothing for eager execution."""
+        if self.profiling or not self.use_graph:
+            return
+        if self._segments is None:
+            self._build_segments()
+        for seg in self._segments:
+            if isinstance(seg, _GraphSegment):
+                seg.prepare()
+        queue = self._queue()
+        if queue is not None:
+            queue.finish()
 
     def call_n_times(self, n):
         """Run the whole plan sequence ``n`` times and wait for it to finish."""

@@ -91,6 +91,13 @@ class HipBackend:
     def upload(self, host_ragged):
         return self._ra.HIPRaggedArray(self.queue, host_ragged)
 
+    def probe_drain(self, probe_plan, signals, step_idx, time_idx):
+        """Callable ``drain(rows_bound) -> (step, time, counts, rows)`` that fetches the
+        clock and the buffered probe rows in one transfer and zeroes the positions."""
+        from .hipra_nonlinearities import ProbeDrain
+
+        return ProbeDrain(self.queue, probe_plan, signals, step_idx, time_idx)
+
     def array(self, values, dtype=np.float32):
         return self._ra.to_device(self.queue, np.asarray(values, dtype=dtype))
 
@@ -384,7 +391,13 @@ class Simulator:
 
         self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches)
         self.rng = None
+        self._drain = None
+        if hasattr(self.backend, "probe_drain"):
+            self._drain = self.backend.probe_drain(self._probe_plan, self.all_data,
+                                                   self.sidx[self.model.step],
+                                                   self.sidx[self.model.time])
         self._reset_probes()
+        self._plans.prepare()  # record the step graphs now, not inside the first run
 
     def _fuse_filter_epilogues(self, plans):
         """Synapse filters whose input is the output of a large GEMV item become the
@@ -566,12 +579,49 @@ class Simulator:
         self._plans = None
         self._raggedarrays_to_reset = None
         self._probe_plan = None
+        self._drain = None
 
     # ---------------------------------------------------------------- probes
-    def _probe(self):
-        """Drain the device probe buffers into ``sim.data``."""
-        self._probe_step_time()
+    def _probe(self, steps_since_drain=None):
+        """Drain the device probe buffers into ``sim.data`` and refresh ``n_steps`` /
+        ``time``.  ``steps_since_drain`` bounds the rows a probe can have buffered."""
         plan = self._probe_plan
+        drain = self._drain
+        if drain is not None:
+            if plan is None:
+                self._n_steps, self._time = (lambda r: (int(r[0]), r[1]))(drain(0))
+                return
+            if steps_since_drain is None:
+                bound = int(plan.Y.shape0s.max())
+            else:
+                bound = int(steps_since_drain // max(int(self._min_period), 1)) + 1
+            if bound <= drain.max_rows():
+                step, time, counts, rows = drain(bound)
+                self._n_steps, self._time = int(step), time
+                complete = True
+                for i, probe in enumerate(self.model.probes):
+                    cap = int(plan.Y.shape0s[i])
+                    if counts[i] > cap:
+                        raise RuntimeError("probe buffer %d overran: %d samples for %d rows"
+                                           % (i, counts[i], cap))
+                    complete = complete and counts[i] == len(rows[i])
+                if complete:
+                    for i, probe in enumerate(self.model.probes):
+                        shape = self.model.sig[probe]["in"].shape
+                        if len(rows[i]):
+                            self._probe_outputs[probe].extend(
+                                rows[i].reshape((len(rows[i]),) + shape))
+                    return
+                # more rows than the bound (cannot happen with the bound above): the rows
+                # are still in the buffers, only the positions were zeroed
+                for i, probe in enumerate(self.model.probes):
+                    shape = self.model.sig[probe]["in"].shape
+                    n_buffered = int(counts[i])
+                    if n_buffered:
+                        got = self.backend.read_rows(plan.Y, i, n_buffered)
+                        self._probe_outputs[probe].extend(got.reshape((n_buffered,) + shape))
+                return
+        self._probe_step_time()
         if plan is None:
             return
         self.backend.finish()
@@ -598,6 +648,7 @@ class Simulator:
         for probe in self.model.probes:
             self._probe_outputs[probe] = []
         self.data.reset()
+        self._probes_drained = True
         self._probe_step_time()
 
     def reset(self, seed=None):
@@ -639,14 +690,15 @@ class Simulator:
             raise ValueError("Cannot handle more than 2**24 steps")
         if steps < 0:
             raise ValueError("Cannot run for negative steps (got %r)" % (steps,))
-        if self._probe_plan is not None:
-            bufpositions = self.backend.get_array(self._probe_plan.dev_bufpositions)
-            assert np.all(bufpositions == 0)
+        # every path that runs steps drains afterwards, so the buffers are empty here
+        assert self._probes_drained
 
         while steps > 0:
             B = min(steps, self._max_steps_between_probes)
+            self._probes_drained = False
             self._plans.call_n_times(B)
-            self._probe()
+            self._probe(B)
+            self._probes_drained = True
             steps -= B
 
         if self.profiling > 1:
@@ -690,6 +742,7 @@ class Simulator:
                               for p in probes], dtype=np.float32)
         plan = self.backend.plan_probes(self.queue, periods, X, Y)
         self._max_steps_between_probes = n_prealloc * int(min(periods))
+        self._min_period = int(min(periods))
         self._probe_plan = plan
         assert self._max_steps_between_probes >= 1
         return [plan]
