@@ -390,7 +390,8 @@ int nhip_probes(void *stream, const int *desc, int n, int lanes, float *countdow
  *   [0] signals[step_start], [1] signals[time_start], [2 .. 2+n) bufpositions (int bits),
  *   zero padding up to NHIP_DRAIN_HEADER(n); then for probe i its first
  *   min(bufpositions[i], capacity_i, rows_bound) rows at
- *   NHIP_DRAIN_HEADER(n) + rows_bound * wprefix_i (row-major, width_i words per row);
+ *   NHIP_DRAIN_HEADER(n) + rows_bound * wprefix_i (row-major, width_i words per row),
+ *   the rest of its rows_bound rows zero (every transferred word is defined by the call);
  * then bufpositions is zeroed, the first NHIP_DRAIN_HEADER(n) + rows_bound * total_width
  * words are copied to `host_out` (HOST memory of at least that size; pinned memory makes
  * the copy a single DMA) and the stream is synchronised: on return `host_out` is valid.
@@ -403,6 +404,22 @@ int nhip_probes_drain(void *stream, const int *desc, int n_probes, int total_wid
                       int max_width, int rows_bound, int *bufpositions, const float *Y,
                       const float *signals, int step_start, int time_start, float *staging,
                       long long staging_words, float *host_out);
+/* The same drain for callers that cannot allocate device memory or bring a workspace
+ * (code under graph capture rules, tight serving loops, harnesses that forbid
+ * hipMalloc): no counterpart in the reference.  The staging block is a file-scope
+ * device array of NHIP_DRAIN_STATIC_WORDS floats (4 MiB) that every GPU the library runs
+ * on holds until the process ends; its address on the current device is looked up once
+ * per device, on the first call there.  Allocates nothing, provided `host_out` is
+ * pinned host memory (a pageable target makes the runtime stage the copy itself).
+ * NHIP_E_TOOBIG when NHIP_DRAIN_HEADER(n) + rows_bound * total_width exceeds
+ * NHIP_DRAIN_STATIC_WORDS.  All calls on one GPU share the array: calls that overlap
+ * on one GPU (different streams or host threads) race; the array keeps the last
+ * call's block, and every word a call transfers is written by that call first. */
+#define NHIP_DRAIN_STATIC_WORDS (1 << 20)
+int nhip_probes_drain_static(void *stream, const int *desc, int n_probes, int total_width,
+                             int max_width, int rows_bound, int *bufpositions, const float *Y,
+                             const float *signals, int step_start, int time_start,
+                             float *host_out);
 /* fill an int32 device array (used to zero probe buffer positions without a
  * memset node, so that it may also be recorded into a graph) */
 int nhip_fill_i32(void *stream, int *dst, int n, int value);

@@ -64,6 +64,7 @@ SIGNATURES = {
     "nhip_probes": [P, P, c_int, c_int, P, P, P, P, P],
     "nhip_probes_drain": [P, P, c_int, c_int, c_int, c_int, P, P, P, c_int, c_int, P,
                           ctypes.c_longlong, P],
+    "nhip_probes_drain_static": [P, P, c_int, c_int, c_int, c_int, P, P, P, c_int, c_int, P],
     "nhip_fill_i32": [P, P, c_int, c_int],
     "nhip_sequence": [P, P, c_int, c_int],
     "nhip_sequence_chains": [P, P, P, P, c_int],

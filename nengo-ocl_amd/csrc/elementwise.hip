@@ -9,6 +9,8 @@
 // handles 256 / lanes blocks side by side), chosen per launch by the host from the
 // item sizes: a model with twenty thousand one-element synapses gets one thread,
 // not one group, per synapse.
+#include <mutex>
+
 #include "nhip_common.h"
 
 namespace {
@@ -402,23 +404,29 @@ __global__ __launch_bounds__(NHIP_WG) void probes_pack_kernel(
     const float* __restrict__ Y, const float* __restrict__ signals, int step_start,
     int time_start, int rows_bound, int header, float* __restrict__ out) {
     const int probe = blockIdx.y;
-    if (blockIdx.x == 0 && probe == 0 && threadIdx.x == 0) {
-        out[0] = signals[step_start];
-        out[1] = signals[time_start];
+    if (blockIdx.x == 0 && probe == 0) {
+        // the whole header is written (the workspace may hold an earlier drain)
+        for (int w = threadIdx.x; w < header; w += NHIP_WG) {
+            float v = 0.0f;
+            if (w == 0) v = signals[step_start];
+            else if (w == 1) v = signals[time_start];
+            else if (w - 2 < n_probes) v = __int_as_float(bufpositions[w - 2]);
+            out[w] = v;
+        }
     }
     if (probe >= n_probes) return;  // a launch without probes still packs the clock
     const DrainDesc d = desc[probe];
     const int count = bufpositions[probe];
-    if (blockIdx.x == 0 && threadIdx.x == 0) out[2 + probe] = __int_as_float(count);
     const int rows = min(min(count, d.capacity), rows_bound);
-    const int n_words = rows * d.width;
+    const int n_words = rows * d.width;          // buffered rows: copied
+    const int n_region = rows_bound * d.width;   // the rest of the region: zeros
     const float* src = Y + d.y_start;
     float* dst = out + header + (size_t)rows_bound * d.wprefix;
     const int w0 = blockIdx.x * 1024;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int w = w0 + k * NHIP_WG + threadIdx.x;
-        if (w < n_words) dst[w] = src[w];
+        if (w < n_region) dst[w] = w < n_words ? src[w] : 0.0f;
     }
 }
 
@@ -684,10 +692,11 @@ extern "C" int nhip_fill_i32(void* stream, int* dst, int n, int value) {
     return 0;
 }
 
-extern "C" int nhip_probes_drain(void* stream, const int* desc, int n_probes, int total_width,
-                                 int max_width, int rows_bound, int* bufpositions, const float* Y,
-                                 const float* signals, int step_start, int time_start,
-                                 float* staging, long long staging_words, float* host_out) {
+namespace {
+int probes_drain(hipStream_t s, const int* desc, int n_probes, int total_width, int max_width,
+                 int rows_bound, int* bufpositions, const float* Y, const float* signals,
+                 int step_start, int time_start, float* staging, long long staging_words,
+                 float* host_out) {
     if (n_probes < 0 || total_width < 0 || max_width < 0 || max_width > total_width ||
         rows_bound < 0 || (n_probes > 0 && (!desc || !bufpositions || !Y)) || !signals ||
         step_start < 0 || time_start < 0 || !staging || !host_out)
@@ -697,9 +706,8 @@ extern "C" int nhip_probes_drain(void* stream, const int* desc, int n_probes, in
     if (words > staging_words) return NHIP_E_TOOBIG;
     const long long widest = (long long)rows_bound * max_width;
     if (widest > (1LL << 30)) return NHIP_E_TOOBIG;
-    const dim3 grid((unsigned)((widest + 1023) / 1024 > 0 ? (widest + 1023) / 1024 : 1),
-                    (unsigned)(n_probes > 0 ? n_probes : 1));
-    hipStream_t s = NHIP_STREAM(stream);
+    const long long runs = (widest + 1023) / 1024;
+    const dim3 grid((unsigned)(runs > 0 ? runs : 1), (unsigned)(n_probes > 0 ? n_probes : 1));
     NHIP_LAUNCH(probes_pack_kernel, grid, dim3(NHIP_WG), 0, s,
                 reinterpret_cast<const DrainDesc*>(desc), n_probes, bufpositions, Y, signals,
                 step_start, time_start, rows_bound, (int)header, staging);
@@ -713,6 +721,56 @@ extern "C" int nhip_probes_drain(void* stream, const int* desc, int n_probes, in
                                   hipMemcpyDeviceToHost, s);
     if (e != hipSuccess) return (int)e;
     return (int)hipStreamSynchronize(s);
+}
+}  // namespace
+
+extern "C" int nhip_probes_drain(void* stream, const int* desc, int n_probes, int total_width,
+                                 int max_width, int rows_bound, int* bufpositions, const float* Y,
+                                 const float* signals, int step_start, int time_start,
+                                 float* staging, long long staging_words, float* host_out) {
+    return probes_drain(NHIP_STREAM(stream), desc, n_probes, total_width, max_width, rows_bound,
+                        bufpositions, Y, signals, step_start, time_start, staging, staging_words,
+                        host_out);
+}
+
+// The drain's staging block for callers that can neither allocate nor bring a workspace.
+// In host code the array's name is only a handle for the symbol look-up: the address a
+// kernel may use is the one hipGetSymbolAddress returns, and every GPU has its own.
+static __device__ __align__(256) float scratch[NHIP_DRAIN_STATIC_WORDS];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+float* scratch_ptr[MAX_DEVICES] = {};  // per device, filled on the first call there
+
+int scratch_of_current_device(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return NHIP_E_BADARG;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return NHIP_E_BADARG;
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+extern "C" int nhip_probes_drain_static(void* stream, const int* desc, int n_probes,
+                                        int total_width, int max_width, int rows_bound,
+                                        int* bufpositions, const float* Y, const float* signals,
+                                        int step_start, int time_start, float* host_out) {
+    float* staging = nullptr;
+    const int rc = scratch_of_current_device(&staging);
+    if (rc != 0) return rc;
+    return probes_drain(NHIP_STREAM(stream), desc, n_probes, total_width, max_width, rows_bound,
+                        bufpositions, Y, signals, step_start, time_start, staging,
+                        (long long)NHIP_DRAIN_STATIC_WORDS, host_out);
 }
 
 extern "C" int nhip_sequence_chains(void* stream, const void* ops, const int* chain_ops,
