@@ -19,8 +19,10 @@ stream synchronisations and prints ONE JSON line:
 * ``cpu_baseline``: the CPU oracle (C restatement of the reference kernels,
   OpenMP) stepping the same network on the host cores for a bounded sample.
 
-Other configurations: ``--config c0|c1|c2|c4|c5``; ``--variant per-connection``
-gives c3 with one decoder matrix per connection.
+The network is built with one decoder matrix, product and synapse per connection, as a
+model builder emits it; the simulator's operator rewrite (`operators.merge_identical_chains`)
+computes identical ones once.  ``--no-dedup`` switches that off (c3 then reads 1.37 GB of
+matrices per step).  Other configurations: ``--config c0|c1|c2|c4|c5``.
 """
 
 import argparse
@@ -46,13 +48,16 @@ def make_network(config, variant, scale):
         return (configs.c2_watts_strogatz(),
                 "c2: Watts-Strogatz, 2048 ensembles x 100 LIF, 20,480 decoded edges")
     if config == "c3":
+        # built the way a model builder emits it: one weight signal, one product and one
+        # synapse per connection.  The simulator's operator rewrite computes identical ones
+        # once (one decoder matrix per ensemble); `variant` "per-connection" switches that
+        # rewrite off
         n_ens = max(2, int(round(256 * scale)))
-        share = variant == "shared"
         desc = ("c3: %d ensembles x 4096 LIF x 64-D, fan-out 4, %s, surrogate decoders"
-                % (n_ens, "one decoder matrix per ensemble (~%d MB of matrices per step)"
-                   % (n_ens * 2) if share else
+                % (n_ens, "identical decoder products merged: one decoder matrix per ensemble "
+                   "(~%d MB of matrices per step)" % (n_ens * 2) if variant == "shared" else
                    "one decoder matrix per connection (~%d MB of matrices per step)" % (n_ens * 5)))
-        return configs.c3_large(n_ens=n_ens, share_decoded=share), desc
+        return configs.c3_large(n_ens=n_ens, share_decoded=False), desc
     if config == "c4":
         n = max(1, int(round(64 * scale)))
         return configs.c4_pes(n_triples=n), "c4: PES, %d triples x 2000 LIF x 32-D" % n
@@ -82,20 +87,45 @@ def gemv_summary(sim, profile_steps):
     return rows
 
 
+KERNEL_SOURCES = ("gemv_tile.hip", "gemv_types.h", "gemv_rows.h", "neuron_math.h", "nhip_common.h")
+
+
+def kernel_sources_hash():
+    """sha256 over the sources of the dominant kernel as they are in this tree."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "nengo-ocl_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def measured_traffic(plan_name):
-    """HBM bytes per launch of the dominant kernel, from the counter runs summarised in
-    profiles/c3_shared_step.txt (FETCH_SIZE and WRITE_SIZE, scaled by what the same
-    counters read for a plain copy of known size).  None for other workloads."""
+    """(bytes, source): HBM bytes per launch of the dominant kernel from the counter runs
+    summarised in profiles/c3_shared_step.txt (FETCH_SIZE and WRITE_SIZE, scaled by what
+    the same counters read for a plain copy of known size), and where the figure comes
+    from.  The summary names the hash of the kernel sources it was taken with; when the
+    sources in this tree hash differently the figure is stale and None is returned in its
+    place.  (None, None) for other workloads."""
     kernel = {"hipra_gemv.tile_lif": "gemv_stream_kernel<1,0>",
               "hipra_gemv.tile_filter": "gemv_stream_kernel<2,4>"}.get(plan_name)
-    path = os.path.join(ROOT, "profiles", "c3_shared_step.txt")
+    rel = os.path.join("profiles", "c3_shared_step.txt")
+    path = os.path.join(ROOT, rel)
     if kernel is None or not os.path.exists(path):
-        return None
+        return None, None
+    value, profiled_hash = None, None
     for line in open(path):
         parts = line.split()
         if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == kernel:
-            return float(parts[2])
-    return None
+            value = float(parts[2])
+        if len(parts) == 2 and parts[0] == "kernel_sources_sha256":
+            profiled_hash = parts[1]
+    here = kernel_sources_hash()
+    source = {"file": rel, "kernel": kernel, "kernel_sources_sha256_profiled": profiled_hash,
+              "kernel_sources_sha256_tree": here, "current": profiled_hash == here,
+              "method": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy"}
+    return (value if profiled_hash == here else None), source
 
 
 def cpu_baseline(config, variant, scale, budget_s, dt_gpu_step):
@@ -103,7 +133,7 @@ def cpu_baseline(config, variant, scale, budget_s, dt_gpu_step):
     from oracle.oracle_sim import OracleSimulator
 
     (net, probes, _), _ = make_network(config, variant, scale)
-    sim = OracleSimulator(net, seed=1)
+    sim = OracleSimulator(net, seed=1, dedup=variant == "shared")
     sim.run_steps(2)  # warm caches, first-touch
     t0 = time.perf_counter()
     sim.run_steps(3)
@@ -262,7 +292,14 @@ def main():
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c3")
-    ap.add_argument("--variant", default="shared", choices=["shared", "per-connection"])
+    ap.add_argument("--variant", default="shared", choices=["shared", "per-connection"],
+                    help="c3: 'per-connection' is the same as --no-dedup")
+    ap.add_argument("--no-dedup", action="store_true",
+                    help="keep identical decoder products and synapses as the builder emitted "
+                         "them, one per connection (c3: 1.37 GB of matrices per step)")
+    ap.add_argument("--kernel-hash", action="store_true",
+                    help="only print the hash of the dominant kernel's sources (the line a "
+                         "counter summary under profiles/ carries)")
     ap.add_argument("--scale", type=float, default=1.0, help="fraction of the ensembles (c3, c4)")
     ap.add_argument("--profile-steps", type=int, default=100)
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
@@ -280,6 +317,10 @@ def main():
                     help="only time the kernels no benchmark network uses (learning rules, "
                          "convolution, noise, compiled function nodes), one JSON line each")
     args = ap.parse_args()
+    if args.kernel_hash:
+        return print("kernel_sources_sha256", kernel_sources_hash())
+    if args.no_dedup:
+        args.variant = "per-connection"
     if args.calibrate_copy:
         return calibrate_copy()
     if args.micro:
@@ -295,7 +336,7 @@ def main():
     t0 = time.time()
     (net, probes, _), workload = make_network(args.config, args.variant, args.scale)
     sim = Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph,
-                    learn_in_place=args.learn_in_place)
+                    learn_in_place=args.learn_in_place, dedup=args.variant == "shared")
     build_s = time.time() - t0
     n_plans = len(sim._plans)
 
@@ -331,11 +372,12 @@ def main():
     gemv_us = sum(r["avg_us"] for r in gemv_rows)
     roofline = None
     if dom is not None:
-        traffic = None
+        traffic, traffic_source = None, None
         if args.config == "c3" and args.variant == "shared" and args.scale == 1.0:
-            traffic = measured_traffic(dom["name"])
+            traffic, traffic_source = measured_traffic(dom["name"])
         roofline = dict(bound="hbm", achieved=dom["gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
-                        frac=dom["gbs"] / HBM_PEAK_GBS, traffic=traffic, kernel=dom["plan"],
+                        frac=dom["gbs"] / HBM_PEAK_GBS, traffic=traffic,
+                        traffic_source=traffic_source, kernel=dom["plan"],
                         avg_us=dom["avg_us"], bytes_per_launch=dom["bytes"])
 
     out = {
@@ -356,7 +398,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": workload, "neurons": net.n_neurons, "plans_per_step": n_plans,
                    "dt": 0.001, "graph": not args.no_graph,
-                   "fused_copies": not args.no_fuse, "learn_in_place": args.learn_in_place},
+                   "fused_copies": not args.no_fuse, "learn_in_place": args.learn_in_place,
+                   "identical_products_merged": args.variant == "shared"},
         "roofline": roofline,
         "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,
                      "gbs": 1e-3 * gemv_bytes / gemv_us if gemv_us else None,

@@ -146,11 +146,13 @@ def c2_watts_strogatz(seed=0, n_ens=2048, n_neurons=100, k=10, p=0.1, n_driven=6
     return net, probes, dict(edges=edges, driven=driven)
 
 
-def c3_large(seed=0, n_ens=256, n_neurons=4096, dims=64, fan_out=4, share_decoded=True,
+def c3_large(seed=0, n_ens=256, n_neurons=4096, dims=64, fan_out=4, share_decoded=False,
              solver="surrogate", n_probes=2):
-    """``share_decoded=True``: one 64 x 4096 decoder per ensemble feeds its four
-    targets (~512 MB of matrices per step at full size); ``False``: one decoder
-    per connection, as nengo builds separate connections (~1.3 GB per step)."""
+    """One decoder matrix, product and synapse per connection, as nengo builds separate
+    connections (~1.3 GB of matrices at full size); the four connections that leave an
+    ensemble carry equal decoders, which the simulator merges into one 64 x 4096 decoder
+    per ensemble (~512 MB of matrices per step) unless told not to (``dedup=False``).
+    ``share_decoded=True`` makes the generator emit the merged graph itself."""
     rng = np.random.RandomState(seed)
     net = Network(seed=seed, label="c3-large-%dx%d" % (n_ens, n_neurons),
                   share_decoded=share_decoded, solver=solver, n_eval_points=1024)

@@ -20,9 +20,12 @@ nengo build of "the same" network is not claimed):
 * PES:  ``SimProcess(pre_synapse, pre.out -> pre_filtered)``, ``Reset(error)``,
   ``SimPES(pre_filtered, error -> delta)``, ``Copy(delta -> weights, inc=True)``
 
-``share_decoded=True`` lets connections leaving one ensemble with the same
-function, transform and synapse share one decoder matrix, one decoded signal
-and one filter (what a passthrough node after the ensemble gives in nengo).
+Every connection gets its own weight signal, product and synapse, as nengo's builder
+emits them; merging identical ones is the simulator's job
+(`operators.merge_identical_chains`).  ``share_decoded=True`` makes the generator itself
+let connections that leave one ensemble with the same function, transform and synapse
+share one decoder matrix, one decoded signal and one filter (what a passthrough node
+after the ensemble gives in nengo): the graph the rewrite must arrive at, kept for tests.
 """
 
 import numpy as np
@@ -198,7 +201,7 @@ class Network:
     runs at sizes where hundreds of large solves would dominate start-up).
     """
 
-    def __init__(self, seed=0, label=None, share_decoded=True, solver="lstsq",
+    def __init__(self, seed=0, label=None, share_decoded=False, solver="lstsq",
                  n_eval_points=None):
         self.seed, self.label = seed, label
         self.share_decoded, self.solver, self.n_eval_points = share_decoded, solver, n_eval_points

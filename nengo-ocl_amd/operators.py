@@ -488,12 +488,210 @@ def apply_learning_in_place(operators, keep=()):
     return [replace.get(op, op) for op in operators if op not in drop]
 
 
-def simplify_operators(operators):
-    """Apply every function in ``simplifications`` in turn."""
+def _replace_signals(op, mapping):
+    """A shallow copy of ``op`` in which every signal that is a key of ``mapping`` (by
+    identity) is replaced by its value -- in attributes, and in lists, tuples and dicts held
+    by attributes (nengo's operators keep their signals in the sets / incs / reads /
+    updates lists, `ir`'s also in named attributes)."""
+    import copy as _copy
+
+    def swap(v):
+        if isinstance(v, (list, tuple)):
+            w = [swap(x) for x in v]
+            return type(v)(w) if any(a is not b for a, b in zip(w, v)) else v
+        if isinstance(v, dict):
+            w = {k: swap(x) for k, x in v.items()}
+            return w if any(w[k] is not v[k] for k in v) else v
+        try:
+            return mapping.get(v, v)
+        except TypeError:  # unhashable attribute values (arrays) are not signals
+            return v
+
+    new = _copy.copy(op)
+    for key, value in list(vars(new).items()):
+        swapped = swap(value)
+        if swapped is not value:
+            setattr(new, key, swapped)
+    return new
+
+
+def _process_key(process):
+    """What makes two synapse processes the same filter, or None for a process that is
+    not a plain transfer function (noise, tables, anything with a seed)."""
+    num, den = getattr(process, "num", None), getattr(process, "den", None)
+    if num is None or den is None or getattr(process, "seed", None) is not None:
+        return None
+    return (type(process).__name__, tuple(np.atleast_1d(num).tolist()),
+            tuple(np.atleast_1d(den).tolist()), bool(getattr(process, "analog", True)),
+            str(getattr(process, "method", "")),
+            repr(getattr(process, "initial_output", None)))
+
+
+def merge_identical_chains(operators, keep=(), aliases=None):
+    """Signals that are computed the same way from the same inputs are computed once.
+
+    nengo's builder emits one weight signal, one ``Reset`` + ``DotInc`` and one synapse per
+    Connection.  Connections that leave one ensemble with the same function, solver and
+    transform carry bit-identical decoders and read the same activities, so their weighted
+    sums -- and behind equal synapses their filtered values -- are the same numbers every
+    step.  Here such duplicates are found and dropped, their readers redirected to the one
+    that stays: the matrix is then stored and read once per step instead of once per
+    connection (the reference keeps every copy: its `compress`, operators.py:112-146,
+    merges by target signal only).
+
+    A signal ``S`` is a candidate when every operator refers to it whole (no views), it is
+    not in `keep` (probed signals), and each of its writers is one of ``Reset``,
+    ``DotInc``, ``ElementwiseInc``, a whole ``Copy``, or a ``SimProcess`` (mode update)
+    of a plain transfer function whose state signals nobody else touches.  Two candidates
+    are duplicates when shape and initial value agree and their writer lists agree
+    operator by operator: same kind, same parameters, and the same operand signals, where
+    operands that are read-only constants nobody writes count as the same signal if their
+    values are bit-identical.  Learned weights have a writer, so they never qualify.
+    Repeated to a fixed point, so a chain (weighted sum, then synapse) folds link by link.
+
+    Every reader then sees the values it saw before, bit for bit.  ``aliases`` (a dict,
+    filled in place) maps each dropped signal to the one that replaces it, for whoever
+    resolves signals afterwards (``sim.signals[dropped]``).
+    """
+    if aliases is None:
+        aliases = {}
+    keep_bases = {sig.base for sig in keep}
+    ops = list(operators)
+    const_canon = {}   # signal -> canonical equal-valued constant
+    const_buckets = {}
+
+    def canonical_constant(sig, writers):
+        """`sig`, or the first constant seen with its shape and values."""
+        if sig in const_canon:
+            return const_canon[sig]
+        out = sig
+        if (not getattr(sig, "is_view", False) and getattr(sig, "readonly", False)
+                and not getattr(sig, "sparse", False) and not writers.get(sig.base)
+                and sig.base not in keep_bases):
+            value = np.asarray(sig.initial_value)
+            flat = value.reshape(-1)
+            key = (value.shape, str(value.dtype), flat[:4].tobytes(), flat[-4:].tobytes())
+            for other in const_buckets.setdefault(key, []):
+                if np.array_equal(np.asarray(other.initial_value), value):
+                    out = other
+                    break
+            else:
+                const_buckets[key].append(sig)
+        const_canon[sig] = out
+        return out
+
+    while True:
+        writers, readers, partial = {}, {}, set()
+        for pos, op in enumerate(ops):
+            for sig in list(op.sets) + list(op.incs) + list(op.updates):
+                writers.setdefault(sig.base, []).append(pos)
+            for sig in op.reads:
+                readers.setdefault(sig.base, []).append(pos)
+            for sig in op.all_signals:
+                if sig.base is not sig:
+                    partial.add(sig.base)
+
+        def exclusive_state(op, pos):
+            """Initial values of the operator's state signals if only it touches them."""
+            out = []
+            for name in sorted(getattr(op, "state", None) or {}):
+                st = op.state[name]
+                if (st.base is not st or st.base in partial or st.base in keep_bases
+                        or writers.get(st.base) != [pos]
+                        or any(q != pos for q in readers.get(st.base, []))):
+                    return None
+                v = np.asarray(st.initial_value)
+                out.append((name, v.shape, v.tobytes()))
+            return tuple(out)
+
+        def writer_key(pos, S):
+            op = ops[pos]
+            const = lambda sig: id(canonical_constant(sig, writers))
+            if _is(op, "Reset") and op.dst is S:
+                return ("Reset", float(op.value))
+            if _is(op, "DotInc") and op.Y is S:
+                return ("DotInc", const(op.A), const(op.X))
+            if _is(op, "ElementwiseInc") and op.Y is S:
+                return ("ElementwiseInc", const(op.A), const(op.X))
+            if (_is(op, "Copy") and op.dst is S and op.src_slice is None
+                    and op.dst_slice is None):
+                return ("Copy", bool(op.inc), const(op.src))
+            if (_is(op, "SimProcess") and op.output is S and op.mode == "update"
+                    and op.input is not None):
+                pkey = _process_key(op.process)
+                state = exclusive_state(op, pos)
+                if pkey is not None and state is not None:
+                    return ("SimProcess", pkey, id(op.input), state)
+            return None
+
+        groups = {}
+        for S, wpos in writers.items():
+            if S in partial or S in keep_bases or getattr(S, "sparse", False):
+                continue
+            keys = []
+            for pos in wpos:
+                op = ops[pos]
+                own_state = list((getattr(op, "state", None) or {}).values())
+                outputs = list(op.sets) + list(op.incs) + list(op.updates)
+                if any(sig is not S and all(sig is not st for st in own_state)
+                       for sig in outputs):
+                    keys = None  # the writer also writes something else
+                    break
+                k = writer_key(pos, S)
+                if k is None:
+                    keys = None
+                    break
+                keys.append(k)
+            if not keys:
+                continue
+            v = np.asarray(S.initial_value)
+            groups.setdefault((v.shape, v.tobytes(), tuple(keys)), []).append(S)
+
+        mapping = {}
+        for members in groups.values():
+            for dup in members[1:]:
+                mapping[dup] = members[0]
+        if not mapping:
+            break
+        drop = {pos for dup in mapping for pos in writers[dup]}
+        ops_before = ops
+        touched = {pos for dup in mapping for pos in readers.get(dup, [])} - drop
+        ops = [_replace_signals(op, mapping) if pos in touched else op
+               for pos, op in enumerate(ops) if pos not in drop]
+        for dup, rep in mapping.items():
+            aliases[dup] = rep
+            # what only the dropped writers used (their equal-valued constants, their
+            # state) resolves to the surviving writers' operands
+            for p_dup, p_rep in zip(writers[dup], writers[rep]):
+                a_sigs = list(ops_before[p_dup].reads) + list(ops_before[p_dup].updates)
+                b_sigs = list(ops_before[p_rep].reads) + list(ops_before[p_rep].updates)
+                for a, b in zip(a_sigs, b_sigs):
+                    if a is not b and a is not dup:
+                        aliases.setdefault(a, b)
+        for sig, rep in list(aliases.items()):  # chains of replacements end at a survivor
+            while rep in aliases:
+                rep = aliases[rep]
+            aliases[sig] = rep
+    return ops
+
+
+merge_identical_chains.takes_context = True
+
+
+def simplify_operators(operators, keep=(), aliases=None, skip=()):
+    """Apply every function in ``simplifications`` in turn (those named in `skip`
+    excepted).  `keep` (signals that must stay as they are: probed ones) and `aliases`
+    (dict filled with dropped signal -> its replacement) go to the simplifications that
+    take them."""
     for simplification in simplifications:
-        operators = simplification(operators)
+        if simplification.__name__ in skip:
+            continue
+        if getattr(simplification, "takes_context", False):
+            operators = simplification(operators, keep=keep, aliases=aliases)
+        else:
+            operators = simplification(operators)
     return operators
 
 
 # Modify this module-level list to change which simplifications run.
-simplifications = [remove_unmodified_resets, remove_zero_incs]
+simplifications = [remove_unmodified_resets, remove_zero_incs, merge_identical_chains]

@@ -230,7 +230,8 @@ class Simulator:
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
                  n_prealloc_probes=None, profiling=None, if_python_code="none",
                  planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
-                 fuse=True, branches=False, merge_small=True, learn_in_place=False):
+                 fuse=True, branches=False, merge_small=True, learn_in_place=False,
+                 dedup=True):
         self.closed = False
         self.model = None
 
@@ -263,11 +264,14 @@ class Simulator:
         # --- operators
         t0 = _time.time()
         all_operators = list(self.model.operators)
-        operators = ops_mod.simplify_operators(all_operators)
+        probed = [self.model.sig[p]["in"] for p in self.model.probes]
+        self.signal_aliases = {}  # signal dropped as a duplicate -> the one computed
+        operators = ops_mod.simplify_operators(
+            all_operators, keep=probed, aliases=self.signal_aliases,
+            skip=() if dedup else ("merge_identical_chains",))
         operators = list(map(MultiDotInc.convert_to, operators))
         if fuse:
             operators = ops_mod.fuse_into_multidotinc(operators)
-            probed = [self.model.sig[p]["in"] for p in self.model.probes]
             operators = ops_mod.neurons_read_constant_input(operators, keep=probed)
             if learn_in_place:
                 operators = ops_mod.apply_learning_in_place(operators, keep=probed)
@@ -294,6 +298,22 @@ class Simulator:
         all_signals = stable_unique(sig for op in all_operators + operators
                                     for sig in op.all_signals)
         all_bases = stable_unique(sig.base for sig in all_signals)
+        if self.signal_aliases:
+            # duplicates (and the constants only they read) take no device memory: they
+            # resolve to the signal that replaces them
+            live = {sig.base for op in operators for sig in op.all_signals}
+            live |= {sig.base for sig in probed}
+            gone = {sig.base for sig in self.signal_aliases}
+            dropped = {id(op) for op in all_operators
+                       if any(sig.base in gone for sig in
+                              list(op.sets) + list(op.incs) + list(op.updates))}
+            only_dropped = {}
+            for op in all_operators:
+                for sig in op.all_signals:
+                    only_dropped[sig.base] = (only_dropped.get(sig.base, True)
+                                              and id(op) in dropped)
+            all_bases = [b for b in all_bases
+                         if b in live or not (b in gone or only_dropped.get(b, False))]
         # sparse matrices are constants of the sparse products: they stay on the host
         # until `_plan_SparseDotInc` lays them out (reference simulator.py:281-329)
         sparse_bases = [b for b in all_bases if getattr(b, "sparse", False)]
@@ -322,6 +342,9 @@ class Simulator:
 
         self.all_bases = all_bases
         self.sidx = {k: np.int32(v) for k, v in view_builder.sidx.items()}
+        for sig, rep in self.signal_aliases.items():
+            if sig not in self.sidx and rep in self.sidx:
+                self.sidx[sig] = self.sidx[rep]
         self._A_views = view_builder._A_views
         self._X_views = view_builder._X_views
         self._YYB_views = view_builder._YYB_views

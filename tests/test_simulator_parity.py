@@ -27,7 +27,7 @@ def build_pair(make_net, **sim_kwargs):
     model = net.build_model(dt=0.001)
     gpu = Simulator(None, model=model, seed=1, **sim_kwargs)
     net2, probes2, _ = make_net()
-    cpu = OracleSimulator(None, model=net2.build_model(dt=0.001), seed=1)
+    cpu = OracleSimulator(None, model=net2.build_model(dt=0.001), seed=1, dedup=False)
     return gpu, cpu, probes, probes2, info
 
 
@@ -141,17 +141,20 @@ def test_c2_watts_strogatz_spiking(queue):
         check_spiking(gpu, cpu, pg["spikes"], pc["spikes"], 1000, "c2 (256 ensembles, 25,600 neurons)")
 
 
-@pytest.mark.parametrize("share", [True, False], ids=["shared-decoders", "per-connection"])
-def test_c3_large_reduced_spiking(queue, share):
+@pytest.mark.parametrize("dedup", [True, False], ids=["merged-decoders", "per-connection"])
+def test_c3_large_reduced_spiking(queue, dedup):
+    """The GPU simulator with identical decoder products merged (or not) against the
+    oracle simulator that keeps one product per connection."""
     from nengo_ocl_amd import configs
 
     def make():
         net, probes, info = configs.c3_large(n_ens=8, n_neurons=1024, dims=64, fan_out=4,
-                                             share_decoded=share, solver="lstsq")
+                                             solver="lstsq")
         probes["spikes"] = add_spike_probes(net, net.ensembles)
         return net, probes, info
 
-    gpu, cpu, pg, pc, _ = build_pair(make)
+    gpu, cpu, pg, pc, _ = build_pair(make, dedup=dedup)
+    assert bool(gpu.signal_aliases) == dedup and not cpu.signal_aliases
     with gpu, cpu:
         # the neurons are updated by the GEMV that computes their input current
         assert any(p.name == "hipra_gemv.tile_lif" for p in gpu._plans)
@@ -171,9 +174,10 @@ def test_c3_full_size_state_bit_exact(queue):
     from nengo_ocl_amd.simulator import Simulator
     from oracle.oracle_sim import OracleSimulator
 
-    net, probes, _ = configs.c3_large()
+    net, probes, _ = configs.c3_large()  # one decoder matrix per connection; merged below
     net_o, probes_o, _ = configs.c3_large()
     with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        assert len(gpu.signal_aliases) == 3 * 768
         names = [p.name for p in gpu._plans]
         assert sorted(names) == ["hip_sequence", "hipra_gemv.tile_filter", "hipra_gemv.tile_lif",
                                  "hipra_gemv.wave_ref"]
@@ -190,6 +194,30 @@ def test_c3_full_size_state_bit_exact(queue):
         assert all(np.any(gpu.data[probes[key]] != 0) for key in probes)  # something happened
 
 
+def test_merged_products_keep_every_signal(queue):
+    """One built model (per-connection decoders, reduced c3) run on the GPU with identical
+    products merged and without: every probe sample and every signal of the model --
+    dropped duplicates through their alias -- bit-identical after 200 steps, and the
+    merged step is the four launches of the benchmark."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+
+    net, probes, _ = configs.c3_large(n_ens=8, n_neurons=1024, dims=64, fan_out=4)
+    model = net.build_model(dt=0.001)
+    with Simulator(None, model=model, seed=1) as a, \
+            Simulator(None, model=model, seed=1, dedup=False) as b:
+        assert sorted(p.name for p in a._plans) == [
+            "hip_sequence", "hipra_gemv.tile_filter", "hipra_gemv.tile_lif", "hipra_gemv.wave_ref"]
+        assert a.all_data.buf.size < b.all_data.buf.size
+        a.run_steps(200)
+        b.run_steps(200)
+        for p in probes.values():
+            assert np.array_equal(a.data[p], b.data[p]) and np.any(a.data[p] != 0)
+        for base in {sig.base for op in model.operators for sig in op.all_signals}:
+            got, want = np.asarray(a.signals[base]), np.asarray(b.signals[base])
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), base
+
+
 @pytest.mark.parametrize("case", ["c2", "c3-per-connection", "c4", "c5"])
 def test_other_configurations_full_size_state_bit_exact(queue, case):
     """The other benchmark configurations at their full sizes (2048 ensembles on a
@@ -201,12 +229,13 @@ def test_other_configurations_full_size_state_bit_exact(queue, case):
     from oracle.oracle_sim import OracleSimulator
 
     make = {"c2": configs.c2_watts_strogatz,
-            "c3-per-connection": lambda: configs.c3_large(share_decoded=False),
+            "c3-per-connection": configs.c3_large,
             "c4": configs.c4_pes,
             "c5": lambda: configs.c5_sparse_recurrent(n_neurons=1000000)}[case]
     net, probes, _ = make()
     net_o, probes_o, _ = make()
-    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+    with Simulator(net, seed=1, dedup=False) as gpu, \
+            OracleSimulator(net_o, seed=1, dedup=False) as cpu:
         gpu.run_steps(30)
         cpu.run_steps(30)
         for key in probes:
