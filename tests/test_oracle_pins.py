@@ -337,10 +337,22 @@ def test_probe_schedule_matches_trange_rule():
         assert np.array_equal(Y[i][: len(fired[i]), 0], fired[i])  # the sampled values, in order
 
 
-def test_direct_unary():
-    x, y = RA([[0.731], [2.5]]), RA([[0.0], [0.0]])
-    orc.plan_direct_unary(None, "sin", x, y)()
-    np.testing.assert_allclose(y.buf, np.sin(np.float32([0.731, 2.5])), rtol=1e-6)
+UNARY = {"identity": lambda v: v, "sin": np.sin, "cos": np.cos, "tanh": np.tanh, "exp": np.exp,
+         "square": np.square}
+
+
+@pytest.mark.parametrize("name", sorted(UNARY))
+def test_direct_unary(name):
+    """Every opcode of the single-function node kernel against numpy in float64 (the
+    functions differ pairwise at these points, so a swapped opcode fails)."""
+    points = np.float32([0.731, 2.5, -1.25])
+    x, y = RA([[v] for v in points]), RA([[0.0]] * 3)
+    orc.plan_direct_unary(None, name, x, y)()
+    want = UNARY[name](points.astype(np.float64))
+    np.testing.assert_allclose(y.buf[[int(s) for s in y.starts]], want, rtol=3e-7)
+    for other, fn in UNARY.items():
+        if other != name:
+            assert np.abs(fn(points.astype(np.float64)) - want).max() > 1e-2, other
 
 
 # ------------------------------------------------------- further neuron types
