@@ -494,7 +494,10 @@ class Simulator:
             sigdict = SignalDict()
             for op in all_operators:
                 op.init_signals(sigdict)
-            return {b: sigdict[b] for b in all_bases}
+            # signals that only the rewritten operator list knows (the constant one of the
+            # fused copies) are not among nengo's operators: their own initial value
+            return {b: sigdict[b] if b in sigdict else np.array(b.initial_value)
+                    for b in all_bases}
         return {b: b.initial_value for b in all_bases}
 
     def RaggedArray(self, listofarrays, **kwargs):

@@ -11,6 +11,7 @@ import os as _os
 _pkg_dir = _os.path.join(_os.path.dirname(_os.path.abspath(__file__)), "nengo-ocl_amd")
 __path__ = [_pkg_dir]
 __file__ = _os.path.join(_pkg_dir, "__init__.py")
+__package__ = __name__  # relative imports inside the package's __init__ resolve against it
 if __spec__ is not None:
     __spec__.submodule_search_locations = __path__
 

@@ -1,0 +1,199 @@
+"""The simulator's nengo path run without nengo: operators, signals, processes, neuron
+types, a Model and a Builder registry of nengo's *family* (stand-ins in `nengo_standin`,
+modules named like nengo's) go through `Simulator(network)` -- `_nengo_build`, the
+backend's `Builder`, `SignalDict` initial values, the state-space -> transfer-function
+conversion of synapses, the table pulled out of a process's step closure, dispatch by class
+name -- and must give the numbers of the same graph written with `ir`'s classes.
+Reference paths mirrored: nengo_ocl/simulator.py:230-243, 266-276, 1196-1227, 1263-1277;
+nengo_ocl/builder.py:11-51."""
+
+import types
+
+import numpy as np
+import pytest
+
+import nengo_standin
+from nengo_ocl_amd import ir
+from oracle.oracle_sim import OracleSimulator
+
+IR = types.SimpleNamespace(
+    Signal=ir.Signal, Reset=ir.Reset, Copy=ir.Copy, DotInc=ir.DotInc,
+    ElementwiseInc=ir.ElementwiseInc, SimPyFunc=ir.SimPyFunc, SimNeurons=ir.SimNeurons,
+    SimProcess=ir.SimProcess, LIF=ir.LIF, Lowpass=ir.Lowpass, WhiteSignal=ir.WhiteSignal,
+    Model=ir.Model, family="ir")
+
+
+class ToyNetwork:
+    """What the toy build function below turns into operators."""
+    seed = 3
+
+    def __init__(self, n_neurons=80, dims=3):
+        self.n_neurons, self.dims = n_neurons, dims
+
+
+class ToyProbe:
+    def __init__(self, sample_every=None):
+        self.sample_every = sample_every
+        self.label = None
+
+
+def emit(model, net, F):
+    """sin(t) and a band-limited table -> two LIF populations chained through decoders
+    and lowpass synapses, with a scaled feedback; probes on the filtered outputs and on
+    the spikes.  `F` supplies the classes (nengo's family or `ir`'s)."""
+    rng = np.random.RandomState(11)
+    n, d = net.n_neurons, net.dims
+    t = model.time
+    sin_out = F.Signal(np.zeros(1), name="sin.out")
+    model.add_op(F.SimPyFunc(sin_out, lambda t: np.sin(8 * t), t, None))
+    noise_out = F.Signal(np.zeros(d), name="noise.out")
+    model.add_op(F.SimProcess(F.WhiteSignal(0.2, high=10.0, seed=5), None, noise_out, t, mode="set"))
+    gain_sig = F.Signal(np.array(0.5), name="half", readonly=True)
+    probes = {}
+    previous = None
+    for k in range(2):
+        x_in = F.Signal(np.zeros(d), name="e%d.in" % k)
+        model.add_op(F.Reset(x_in))
+        model.add_op(F.Copy(noise_out, x_in, inc=True))
+        model.add_op(F.Copy(sin_out, x_in, dst_slice=slice(0, 1), inc=True))
+        if previous is not None:
+            model.add_op(F.Copy(previous, x_in, inc=True))
+        enc = F.Signal(rng.normal(size=(n, d)) * 3, name="e%d.encoders" % k, readonly=True)
+        bias = F.Signal(rng.uniform(0.5, 2.0, size=n), name="e%d.bias" % k, readonly=True)
+        J = F.Signal(np.zeros(n), name="e%d.J" % k)
+        model.add_op(F.Copy(bias, J))
+        model.add_op(F.DotInc(enc, x_in, J))
+        out = F.Signal(np.zeros(n), name="e%d.out" % k)
+        state = {"voltage": F.Signal(np.zeros(n), name="e%d.voltage" % k),
+                 "refractory_time": F.Signal(np.zeros(n), name="e%d.refractory_time" % k)}
+        model.add_op(F.SimNeurons(F.LIF(tau_rc=0.02 + 0.01 * k), J, out, state=state))
+        dec = F.Signal(rng.normal(size=(d, n)) / (50.0 * n), name="e%d.decoders" % k, readonly=True)
+        weighted = F.Signal(np.zeros(d), name="e%d.weighted" % k)
+        model.add_op(F.Reset(weighted))
+        model.add_op(F.DotInc(dec, out, weighted))
+        filtered = F.Signal(np.zeros(d), name="e%d.filtered" % k)
+        model.add_op(F.SimProcess(F.Lowpass(0.005 * (k + 1)), weighted, filtered, t, mode="update"))
+        scaled = F.Signal(np.zeros(d), name="e%d.scaled" % k)
+        model.add_op(F.Reset(scaled))
+        model.add_op(F.ElementwiseInc(gain_sig, filtered, scaled))
+        previous = scaled
+        for name, sig, every in (("filtered%d" % k, filtered, None), ("spikes%d" % k, out, 0.005)):
+            p = ToyProbe(sample_every=every)
+            model.probes.append(p)
+            model.sig[p] = {"in": sig}
+            model.params[p] = []
+            probes[name] = p
+    return probes
+
+
+def test_nengo_family_graph_runs_like_the_ir_graph(monkeypatch):
+    N = nengo_standin.install(monkeypatch)
+    net = ToyNetwork()
+    built = {}
+
+    @N.Builder.register(ToyNetwork)  # nengo's own registry: the fallback of the backend's
+    def build_toy(model, network):
+        built["probes"] = emit(model, network, N)
+
+    with OracleSimulator(net, dt=0.001) as sim:  # -> _nengo_build -> backend Builder -> fallback
+        assert type(sim.model) is N.Model and sim.model.dt == 0.001
+        assert type(sim.model.builder).__module__ == "nengo_ocl_amd.builder"
+        assert all(type(op).__module__.startswith("nengo.") for op in sim.model.operators)
+        ref_model = ir.Model(dt=0.001)
+        ref_probes = emit(ref_model, net, IR)
+        with OracleSimulator(None, model=ref_model, seed=net.seed + 1) as ref:
+            assert [t.__name__ for t, _ in sim.op_groups] == [t.__name__ for t, _ in ref.op_groups]
+            assert [p.name for p in sim._plans] == [p.name for p in ref._plans]
+            sim.run_steps(300)
+            ref.run_steps(300)
+            for key in ref_probes:
+                got, want = sim.data[built["probes"][key]], ref.data[ref_probes[key]]
+                assert got.shape == want.shape and np.any(want != 0), key
+                assert np.array_equal(got, want), (key, np.abs(got - want).max())
+            assert np.array_equal(np.asarray(sim.all_data.buf), np.asarray(ref.all_data.buf))
+            assert sim.data[built["probes"]["spikes0"]].shape == (60, net.n_neurons)
+
+
+def test_backend_registry_comes_before_nengos(monkeypatch):
+    N = nengo_standin.install(monkeypatch)
+    from nengo_ocl_amd.builder import Builder
+
+    calls = []
+    N.Builder.register(ToyNetwork)(lambda model, obj: calls.append("nengo"))
+    model = N.Model(builder=Builder())
+    model.build(ToyNetwork())
+    assert calls == ["nengo"]  # nothing registered here: nengo's build function runs
+    Builder.builders[ToyNetwork] = lambda model, obj: calls.append("backend")
+    try:
+        model.build(ToyNetwork())
+        assert calls == ["nengo", "backend"]
+        assert ToyNetwork not in N.Builder.builders or N.Builder.builders[ToyNetwork] is not \
+            Builder.builders[ToyNetwork]  # registering here leaves nengo's registry alone
+        with pytest.raises(N.BuildError):
+            model.build(object())
+    finally:
+        Builder.builders.pop(ToyNetwork, None)
+
+
+def test_synapse_coefficients_from_state_space(monkeypatch):
+    """A nengo-family Lowpass / second-order filter reaches the filter kernel with the
+    coefficients the `ir` process gives directly (reference :1196-1227)."""
+    N = nengo_standin.install(monkeypatch)
+    from nengo_ocl_amd.simulator import Simulator
+
+    fake = types.SimpleNamespace(model=types.SimpleNamespace(dt=0.001))
+    x, y = ir.Signal(np.zeros(4)), ir.Signal(np.zeros(4))
+    for theirs, ours in ((N.Lowpass(0.005), ir.Lowpass(0.005)),
+                         (nengo_standin.LinearFilter([1.0], [0.01 ** 2, 0.02, 1.0]), ir.Alpha(0.01))):
+        op = types.SimpleNamespace(process=theirs, input=x, output=y)
+        num, den = Simulator._filter_tf(fake, op)
+        want_num, want_den = ours.discrete_tf(0.001)
+        np.testing.assert_allclose(num, want_num, rtol=1e-9, atol=1e-15)
+        np.testing.assert_allclose(den, want_den, rtol=1e-9, atol=1e-15)
+        assert np.array_equal(np.float32(num), np.float32(want_num))
+        assert np.array_equal(np.float32(den), np.float32(want_den))
+
+
+def test_backend_entry_point_and_test_loader():
+    """The `nengo.backends` entry point (reference setup.py:72-76) names something that
+    imports, and the loader for nengo's test suite (reference tests/__init__.py:6-17)
+    hands out this backend's Simulator with the progress bar off."""
+    import configparser
+    import importlib
+    import os
+
+    import tomli
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "pyproject.toml"), "rb") as f:
+        meta = tomli.load(f)
+    target = meta["project"]["entry-points"]["nengo.backends"]["hip"]
+    module, _, attr = target.partition(":")
+    from nengo_ocl_amd.simulator import Simulator
+
+    assert getattr(importlib.import_module(module), attr) is Simulator
+    cfg = configparser.ConfigParser()
+    cfg.read(os.path.join(root, "nengo-ocl_amd", "nengo_tests.cfg"))
+    loader = cfg["pytest"]["nengo_simloader"]
+    module, _, attr = loader.rpartition(".")
+    factory = getattr(importlib.import_module(module), attr)(request=None)
+    seen = {}
+
+    class Recorder(Simulator):
+        def __init__(self, net, **kwargs):
+            seen.update(kwargs, net=net)
+
+    import nengo_ocl_amd
+
+    original = nengo_ocl_amd.__dict__.get("Simulator")
+    nengo_ocl_amd.Simulator = Recorder
+    try:
+        factory("a network", dt=0.002)
+    finally:
+        if original is None:
+            del nengo_ocl_amd.Simulator
+        else:
+            nengo_ocl_amd.Simulator = original
+    assert seen == {"net": "a network", "dt": 0.002, "progress_bar": False}
+    unsupported = cfg["pytest"]["nengo_test_unsupported"]
+    assert "test_lif_min_voltage" in unsupported and "test_pickle_sim" in unsupported
