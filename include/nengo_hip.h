@@ -145,6 +145,27 @@ int nhip_gemv_tile_lif(void *stream, int vec, int pow2_cols, int blk_words, cons
                        const float *A, const float *X, const float *Yin, float *Y,
                        const int *pops, double dt, int upsample, float *V, float *W, float *S,
                        const float *TAU, const float *REF, const float *AMP);
+/* The same launch when the vector operand of an item's first dot product is itself a sum
+ * of vectors that a small-item GEMV launch would form just before (the decoded inputs of
+ * an ensemble added up: `_plan_MultiDotInc` on the `in` signal, simulator.py:746-816,
+ * followed by the encoders' GEMV and `plan_lif`): the launch forms the sum itself,
+ *   x[c] = (...(0 + v_0[c] * s_0) + v_1[c] * s_1) + ...,   every product rounded on its own,
+ * which is what that GEMV gives for Y = 0 * Y + sum_k v_k * s_k (one-column dot products,
+ * alpha = 1, beta = 0, gamma = 0) as long as the old Y is finite, and stores it where that
+ * launch would have: at the operand's own place (x_start of the dot product, stride 1).
+ *   parts : int32[n][2] {start of vector v_k, start of scalar s_k}, offsets into X
+ * An item with such an operand names its parts in the spare words of its task records:
+ * task.pad = first part, item.pad = number of parts (0: the operand is read as usual);
+ * its first dot product must have at most 64 columns.  X and Y must be the same buffer,
+ * the launch one of the compile-time-shape kernel (pow2_cols >= 2), and no part may
+ * overlap an operand that the launch writes.  Results are bit-identical to the separate
+ * launches. */
+int nhip_gemv_tile_lif_sums(void *stream, int vec, int pow2_cols, int blk_words,
+                            const int *items, const float *coefs, const int *dots,
+                            const int *tasks, int n_tasks, const float *A, const float *X,
+                            const float *Yin, float *Y, const int *pops, double dt,
+                            int upsample, float *V, float *W, float *S, const float *TAU,
+                            const float *REF, const float *AMP, const int *parts);
 
 /* nhip_gemv_tile followed by the step of first-order filters on its outputs, in one
  * launch: replaces `plan_block_gemv` (clra_gemv.py:1193-1195) + the simple case of

@@ -1112,6 +1112,22 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
 #pragma unroll
             for (int i = 0; i < G::XL; ++i)
                 xq0[i] = x0[(size_t)min(lane + i * NHIP_WAVE, last_cols - 1) * dot.x_stride0];
+            if (EPI == EPI_LIF && decltype(first_tag)::value && G::XL == 1 && it.pad > 0) {
+                // X is a sum of vectors that this launch forms itself, element c =
+                // (...(0 + v_0[c] * s_0) + v_1[c] * s_1) + ..., every product rounded on
+                // its own and added in order: what the small-item kernel computes for
+                // Y = 0 * Y + sum_k v_k * s_k (one-column dot products, alpha = 1,
+                // gamma = 0).  The wave that has the item's first rows also stores the sum
+                // where the separate launch would have (the X operand's own place).
+                const int c = min(lane, last_cols - 1);
+                float s = 0.0f;
+                for (int q = 0; q < it.pad; ++q) {
+                    const int2 part = epi.lif.parts[task.pad + q];
+                    s = s + fmaf(X[(size_t)part.x + c], X[part.y], 0.0f);
+                }
+                xq0[0] = s;
+                if (task.row0 == 0 && lane < last_cols) Y[(size_t)dot.x_start + lane] = s;
+            }
         }
         if (decltype(first_tag)::value) after_first_loads();
         int k = 0;   // stage whose block is in pf0
@@ -1162,6 +1178,20 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
     auto whole_stages = [&](const GemvDot& dot) { return (dot.N & ((1 << dot.p2) - 1)) == 0; };
     if (it.n_dots == 0) {
         after_first_loads();
+        if (EPI == EPI_LIF && it.pad > 0) {
+            // an item that is nothing but a sum of vectors times scalars (see the single
+            // column stage of a dot product below): row r = (...(0 + v_0[r] s_0) + ...)
+#pragma unroll
+            for (int k = 0; k < SLOTS; ++k) {
+                const int r = lane + k * NHIP_WAVE;
+                float s = 0.0f;
+                for (int q = 0; q < it.pad; ++q) {
+                    const int2 part = epi.lif.parts[task.pad + q];
+                    s = s + fmaf(X[(size_t)part.x + task.row0 + min(r, n_rows - 1)], X[part.y], 0.0f);
+                }
+                if (r < n_rows) ys[r] = s;
+            }
+        }
     } else {
         if (whole_stages(ft.dot0)) dot_of_width(std::true_type{}, std::false_type{}, ft.dot0);
         else dot_of_width(std::true_type{}, std::true_type{}, ft.dot0);
@@ -1271,6 +1301,34 @@ extern "C" int nhip_gemv_tile_lif(void* stream, int vec, int pow2_cols, int blk_
     lif.TAU = TAU;
     lif.REF = REF;
     lif.AMP = AMP;
+    return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
+                       Yin, Y, EPI_LIF, args);
+}
+
+extern "C" int nhip_gemv_tile_lif_sums(void* stream, int vec, int pow2_cols, int blk_words,
+                                       const int* items, const float* coefs, const int* dots,
+                                       const int* tasks, int n_tasks, const float* A,
+                                       const float* X, const float* Yin, float* Y, const int* pops,
+                                       double dt, int upsample, float* V, float* W, float* S,
+                                       const float* TAU, const float* REF, const float* AMP,
+                                       const int* parts) {
+    if (!pops || !V || !W || !S || upsample < 1 || !(dt > 0.0) || !parts) return NHIP_E_BADARG;
+    // the sums are stored through Y at offsets of X: one buffer; and only the kernel with
+    // compile-time shapes forms them
+    if (static_cast<const float*>(Y) != X || pow2_cols < 2) return NHIP_E_BADARG;
+    EpilogueArgs args{};
+    LifArgs& lif = args.lif;
+    lif.pops = reinterpret_cast<const LifPop*>(pops);
+    lif.dtu = (float)(dt / (double)upsample);
+    lif.dt_inv = (float)(1.0 / dt);
+    lif.upsample = upsample;
+    lif.V = V;
+    lif.W = W;
+    lif.S = S;
+    lif.TAU = TAU;
+    lif.REF = REF;
+    lif.AMP = AMP;
+    lif.parts = reinterpret_cast<const int2*>(parts);
     return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
                        Yin, Y, EPI_LIF, args);
 }

@@ -25,6 +25,11 @@ struct LifArgs {
     const float* TAU;
     const float* REF;
     const float* AMP;
+    // input sums formed by the launch itself (large-item kernel with compile-time shapes):
+    // the vector operand of an item's first dot product is the sum of `n` vectors times
+    // scalars, parts[begin .. begin + n) = {vector start, scalar start} in the X buffer;
+    // begin / n ride in the spare words of the task record.  Null: no item has one.
+    const int2* parts;
 };
 
 __device__ __forceinline__ float lif_param(int word, bool is_vector, const float* data, int i) {

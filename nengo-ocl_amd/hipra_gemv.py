@@ -700,6 +700,10 @@ def fuse_lif(prog, lif_plan):
         fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
         fused.members, fused.prog = plan.members, prog
         fused.gemv_bytes = plan.bw_per_call
+        if plan.kernel_class[0] == 3:
+            fused.host_tasks = plan.host_tasks
+            fused.host_pops = table
+            fused.lif_written = [V, W, S]
         out.append(fused)
     if rest:
         out.append(plan_lif(queue, spec["dt"], J[rest], V[rest], W[rest], S[rest],
@@ -707,6 +711,118 @@ def fuse_lif(prog, lif_plan):
                             _subset_param(spec["amp"], rest), upsample=spec["upsample"],
                             tag=lif_plan.tag))
     return out
+
+
+def fuse_input_sums(sum_plan, lif_plan):
+    """One launch less for "x = sum of vectors; J = E x; LIF(J)": the large-item launch with
+    the LIF epilogue (`fuse_lif`) forms the vector operands it needs itself, when the
+    small-item launch `sum_plan` right before it does nothing but form them.
+
+    Fused when every item of `sum_plan` is ``Y = 0 * Y + 0 + sum_k v_k * s_k`` (one-column
+    dot products: vectors times scalars, alpha = 1) of at most 64 elements with stride 1,
+    is the vector operand of the FIRST dot product of an item of `lif_plan` (a launch of the
+    compile-time-shape kernel) and of nothing else in that GEMV, and no part ``v_k`` / ``s_k``
+    is something either launch writes; all in one device buffer.  The sums are formed with
+    the roundings and in the order of the small-item kernel and stored where it stores them,
+    so results are bit-identical as long as the sums' old values are finite (the 0 * Y
+    term is not formed).  Returns the plan that replaces ``[sum_plan, lif_plan]``, or None.
+    """
+    S, E = getattr(sum_plan, "prog", None), getattr(lif_plan, "prog", None)
+    if (S is None or E is None or sum_plan.name != "hipra_gemv.wave_ref"
+            or lif_plan.name != "hipra_gemv.tile_lif" or getattr(lif_plan, "host_tasks", None) is None
+            or lif_plan.kernel_class[0] != 3 or lif_plan.kernel_class[1] < 2):
+        return None
+    queue, lib = E.queue, E.queue.lib
+    buf = E.X.ptr.value
+    if any(ra.ptr.value != buf for ra in (S.A, S.X, S.Y, S.Y_in, E.Y)):
+        return None
+    # the sums: start -> (length, parts)
+    sums = {}
+    for b in sum_plan.members:
+        g = S.geometry[b]
+        if (S.alpha[b] != 1 or S.beta[b] != 0 or S.gamma[b] != 0 or g["y_stride0"] != 1
+                or g["y_in_start"] != g["y_start"] or not 1 <= g["y_len"] <= 64
+                or not g["dots"] or g["y_start"] in sums):
+            return None
+        if any(d["a_shape1"] != 1 or (d["a_stride0"] != 1 and g["y_len"] > 1) for d in g["dots"]):
+            return None
+        sums[g["y_start"]] = (g["y_len"], [(d["a_start"], d["x_start"]) for d in g["dots"]])
+    sum_spans = sorted((lo, lo + n) for lo, (n, _) in sums.items())
+    # every dot product of the GEMV that touches a sum is the first one of an item of this
+    # launch, reads the whole sum with stride 1, and has a single column stage
+    used = set()
+    members = set(lif_plan.members)
+    for g in E.geometry:
+        for k, d in enumerate(g["dots"]):
+            span = (d["x_start"], d["x_start"] + (d["a_shape1"] - 1) * d["x_stride0"] + 1)
+            if not _overlaps([span], sum_spans):
+                continue
+            want = sums.get(d["x_start"])
+            if (k != 0 or g["index"] not in members or want is None or want[0] != d["a_shape1"]
+                    or d["x_stride0"] != 1 or stream_stage(d["a_shape1"])[0] > 6):
+                return None
+            used.add(d["x_start"])
+        # (matrices and old outputs that overlap a sum would be read while it is written)
+        if _overlaps([(g["y_in_start"], g["y_in_start"] + (g["y_len"] - 1) * g["y_in_stride0"] + 1)],
+                     sum_spans) and E.Y_in.ptr.value == buf:
+            return None
+    spare = sorted(set(sums) - used)  # sums nothing here reads: tasks of their own, below
+    if not used:
+        return None
+    if E.A.ptr.value == buf and _overlaps(
+            [iv for g in E.geometry for d in g["dots"] for iv in [_span(E.A, d["a_j"])] if iv],
+            sum_spans):
+        return None
+    # no part is written by either launch
+    written = list(sum_spans) + [iv for iv in (_span(E.Y, b) for b in lif_plan.members) if iv]
+    for ra in getattr(lif_plan, "lif_written", ()):
+        if ra.ptr.value == buf:
+            written += [iv for iv in (_span(ra, p) for p in range(len(ra))) if iv]
+    part_spans = [(a, a + n) for n, parts in sums.values() for a, _ in parts]
+    part_spans += [(x, x + 1) for _, parts in sums.values() for _, x in parts]
+    if _overlaps(part_spans, written):
+        return None
+
+    part_rows, where = [], {}
+    for start, (_, parts) in sums.items():
+        where[start] = (len(part_rows), len(parts))
+        part_rows.extend(parts)
+    tasks = lif_plan.host_tasks.copy()  # 24-word records: task, item, coefficients, first dot
+    for row in tasks:
+        if row[9] > 0 and int(row[19]) in where:  # the item has dot products; x_start of the first
+            row[3], row[11] = where[int(row[19])]
+    args = tuple(lif_plan.args)
+    keep = ()
+    if spare:
+        # one task each, of an item without dot products and without neurons: Y = the sum
+        pops = np.concatenate([lif_plan.host_pops, np.zeros((1, 8), dtype=np.int32)])
+        extra = np.zeros((len(spare), 24), dtype=np.int32)
+        for row, start in zip(extra, spare):
+            first, count = where[start]
+            row[0:4] = (len(pops) - 1, 0, sums[start][0], first)
+            row[4:12] = (start, 1, start, 1, 0, 0, sums[start][0], count)
+            row[12:16] = np.array([1.0, 0.0, 0.0, 0.0], dtype=np.float32).view(np.int32)
+        tasks = np.concatenate([tasks, extra])
+        dev_pops = to_device(queue, pops)
+        args = args[:12] + (dev_pops.ptr,) + args[13:]
+        keep = (dev_pops,)
+    dev_tasks = to_device(queue, tasks)
+    dev_parts = to_device(queue, np.array(part_rows, dtype=np.int32))
+    n_groups = -(-len(tasks) // (WG // WAVE))
+    args = args[:6] + (dev_tasks.ptr, len(tasks)) + args[8:] + (dev_parts.ptr,)
+    sum_bytes = sum_plan.bw_per_call or 0
+    fused = Plan(queue, lib.nhip_gemv_tile_lif_sums, args, gsize=(WG * n_groups,), lsize=lif_plan.lsize,
+                 full_args=tuple(lif_plan.full_args) + (dev_tasks, dev_parts) + keep,
+                 name=lif_plan.name, tag=lif_plan.tag,
+                 bw_per_call=lif_plan.bw_per_call + sum_bytes,
+                 flops_per_call=(lif_plan.flops_per_call or 0) + (sum_plan.flops_per_call or 0))
+    fused.description = lif_plan.description + "; input sums: " + sum_plan.description
+    fused.kernel_class, fused.n_tasks = lif_plan.kernel_class, len(tasks)
+    fused.members, fused.prog = lif_plan.members, E
+    fused.gemv_bytes = getattr(lif_plan, "gemv_bytes", lif_plan.bw_per_call)
+    fused.host_tasks = tasks
+    fused.input_sums = len(sums)
+    return fused
 
 
 def _read_spans(prog, ptr_value):

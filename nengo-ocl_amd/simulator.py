@@ -71,6 +71,9 @@ class HipBackend:
             setattr(self, name, getattr(hipra_nonlinearities, name))
         self.plan_block_gemv = hipra_gemv.plan_block_gemv
         self._fuse_lif = hipra_gemv.fuse_lif
+        self._gemv = hipra_gemv
+        # switch for measurements: False keeps input sums a launch of their own
+        self.input_sums_in_launch = os.environ.get("NENGO_HIP_INPUT_SUMS", "1") != "0"
         from . import hipra_sequence
 
         from . import hipra_spmv
@@ -79,6 +82,13 @@ class HipBackend:
         self.merge_small_plans = hipra_sequence.merge_small_plans
         self.plans_conflict = hipra_sequence._conflict
         self.fuse_gemv_filter = hipra_gemv.fuse_linearfilter
+
+    def fuse_input_sums(self, sum_plan, lif_plan):
+        """The plan replacing ``[sum_plan, lif_plan]`` when the first only forms vector
+        operands of the second, or None."""
+        if self.input_sums_in_launch and hasattr(sum_plan, "prog") and hasattr(lif_plan, "prog"):
+            return self._gemv.fuse_input_sums(sum_plan, lif_plan)
+        return None
 
     def fuse_gemv_neurons(self, gemv_plans, neuron_plans):
         """Plans replacing ``gemv_plans + neuron_plans`` by launches that update the
@@ -408,6 +418,8 @@ class Simulator:
         plans.extend(probe_plans)
         if fuse and hasattr(self.backend, "fuse_gemv_filter"):
             plans = self._fuse_filter_epilogues(plans)
+        if fuse and hasattr(self.backend, "fuse_input_sums"):
+            plans = self._fuse_input_sums(plans)
         if merge_small and hasattr(self.backend, "merge_small_plans"):
             plans = self.backend.merge_small_plans(plans)
         logger.info("Plans in %0.3f s", _time.time() - t0)
@@ -421,6 +433,21 @@ class Simulator:
                                                    self.sidx[self.model.time])
         self._reset_probes()
         self._plans.prepare()  # record the step graphs now, not inside the first run
+
+    def _fuse_input_sums(self, plans):
+        """A launch that only adds up the decoded inputs of ensembles, right before the
+        launch that encodes them and updates the neurons, becomes part of that launch
+        (`hipra_gemv.fuse_input_sums`)."""
+        out = []
+        for plan in plans:
+            fused = self.backend.fuse_input_sums(out[-1], plan) if out else None
+            if fused is None:
+                out.append(plan)
+                continue
+            fused.reads_mem = out[-1].reads_mem | plan.reads_mem
+            fused.writes_mem = out[-1].writes_mem | plan.writes_mem
+            out[-1] = fused
+        return out
 
     def _fuse_filter_epilogues(self, plans):
         """Synapse filters whose input is the output of a large GEMV item become the

@@ -846,3 +846,104 @@ def test_sparse_reference_cases(queue, rng, inc, long_row, sparsity, shape):
     Yo = clone(Y)
     orc.plan_sparse_dot_inc(None, A.tocsr(), X, Yo, inc=inc).plans[0]()
     assert np.array_equal(got, Yo[0][:, 0])
+
+
+def test_gemv_lif_forms_its_input_sums(queue):
+    """Sums of vectors -> encoders -> LIF in one launch: inputs that are sums of one to
+    eleven vectors times scalars (64, 40 and 8 elements), an ensemble whose input is a
+    plain vector in the same launch, and two sums that nothing in the launch reads; the
+    sums, currents and neuron states equal the oracle's three separate kernels bit for bit
+    over several steps in which the summed vectors change."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from nengo_ocl_amd import hipra_nonlinearities as nl
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(77)
+    dt = 1e-3
+    dims = [64, 64, 40, 8, 64]        # input dimension of the five ensembles
+    n_neurons = [4096, 1000, 2048, 2048, 300]
+    fan_in = [4, 11, 1, 3, 0]         # the last ensemble reads its input vector as it is
+    spare = [64, 5]                   # sums that no encoder reads (probe inputs)
+    srcs = [rng.normal(size=64) for _ in range(12)]
+    scal = [np.array([v]) for v in (1.0, 1.0, 0.5, -2.0)]
+    ins = [rng.normal(size=d) for d in dims] + [rng.normal(size=d) for d in spare]
+    enc = [rng.normal(scale=0.5, size=(m, d)) for m, d in zip(n_neurons, dims)]
+    bias = [rng.normal(loc=1.0, size=m) for m in n_neurons]
+    J = [np.zeros(m) for m in n_neurons]
+    V = [rng.uniform(0, 1, size=m) for m in n_neurons]
+    W = [rng.uniform(-2 * dt, 2 * dt, size=m) for m in n_neurons]
+    S = [np.zeros(m) for m in n_neurons]
+    R = RA(srcs + scal + ins + enc + bias + J + V + W + S, align=True)
+    n_e = len(dims)
+    i_src = list(range(12))
+    i_scal = list(range(12, 16))
+    i_in = list(range(16, 16 + n_e + 2))
+    at = 16 + n_e + 2
+    i_enc, i_bias, i_J, i_V, i_W, i_S = (list(range(at + k * n_e, at + (k + 1) * n_e))
+                                         for k in range(6))
+    # which vectors each sum adds up (a source longer than the sum is used through a view)
+    picks = [rng.choice(12, size=f, replace=False) for f in fan_in[:4]] + [
+        rng.choice(12, size=2, replace=False), rng.choice(12, size=3, replace=False)]
+    sum_items = [0, 1, 2, 3, 5, 6]    # positions in `ins` that are sums
+    sum_lens = [dims[0], dims[1], dims[2], dims[3]] + spare
+
+    def build(ra, mg, mn, q, second_reader=False):
+        # A of the sums: the first n elements of each source as an n x 1 matrix
+        views, A_js, X_js = [], [], []
+        for length, pk in zip(sum_lens, picks):
+            a_idx = []
+            for src in pk:
+                views.append((int(ra.starts[i_src[src]]), length))
+                a_idx.append(len(views) - 1)
+            A_js.append(np.array(a_idx, dtype=np.int32))
+            X_js.append(np.array([i_scal[k % 4] for k in range(len(pk))], dtype=np.int32))
+        from_buffer = type(ra).from_buffer
+        buf = ra.dev_buf if hasattr(ra, "dev_buf") else ra.buf
+        mk = (lambda *m: from_buffer(q, buf, *m)) if hasattr(ra, "dev_buf") else (
+            lambda *m: from_buffer(buf, *m))
+        starts = np.array([v[0] for v in views])
+        lens = np.array([v[1] for v in views])
+        ones = np.ones(len(views), dtype=int)
+        A_sum = mk(starts, lens, ones, ones, ones)
+        Y_sum = ra[[i_in[k] for k in sum_items]]
+        sums = mg.plan_block_gemv(q, 1.0, A_sum, A_js, ra, X_js, 0.0, Y_sum)
+        e_A = [np.array([i], dtype=np.int32) for i in i_enc]
+        e_X = [np.array([i_in[k]], dtype=np.int32) for k in range(n_e)]
+        if second_reader:  # the last ensemble also reads the first one's input sum
+            e_A[4] = np.array([i_enc[4], i_enc[4]], dtype=np.int32)
+            e_X[4] = np.array([i_in[4], i_in[0]], dtype=np.int32)
+        encs = mg.plan_block_gemv(q, 1.0, ra, e_A, ra, e_X, 1.0, ra[i_J], Y_in=ra[i_bias])
+        lif = mn.plan_lif(q, dt, ra[i_J], ra[i_V], ra[i_W], ra[i_S], 0.002,
+                          np.float32([0.02, 0.03, 0.02, 0.05, 0.02]), 1.0)
+        return sums, encs, lif
+
+    host = clone(R)
+    dev = to_dev(queue, R)
+    sums, encs, lif = build(dev, g, nl, queue)
+    assert [p.name for p in sums.plans] == ["hipra_gemv.wave_ref"]
+    with_lif = g.fuse_lif(encs, lif)
+    assert [p.name for p in with_lif] == ["hipra_gemv.tile_lif"]
+    fused = g.fuse_input_sums(sums.plans[0], with_lif[0])
+    assert fused is not None and fused.input_sums == 6
+    assert fused.n_tasks == with_lif[0].n_tasks + 2   # the two sums nothing reads
+    osums, oencs, olif = build(host, orc, orc, None)
+    for step in range(4):
+        fused()
+        for p in osums.plans + oencs.plans:
+            p()
+        olif()
+        got = dev.to_host()
+        assert np.array_equal(got.buf, host.buf), step
+        # new source vectors for the next step, the same on both sides
+        for i in i_src:
+            v = rng.normal(size=64)
+            host[i] = v[:, None]
+            dev[i] = v
+    assert host.buf[int(host.starts[i_S[0]]):][:4096].any()
+
+    # refused: a sum that a second dot product of the launch reads as well
+    dev2 = to_dev(queue, R)
+    sums2, encs2, lif2 = build(dev2, g, nl, queue, second_reader=True)
+    with_lif2 = g.fuse_lif(encs2, lif2)
+    assert with_lif2 is not None
+    assert all(g.fuse_input_sums(sums2.plans[0], p) is None for p in with_lif2)
