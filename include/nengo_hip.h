@@ -490,6 +490,17 @@ int nhip_sequence(void *stream, const void *ops, int n_ops, int n_staged);
 #define NHIP_SEQ_MAX_CHAINS 4
 int nhip_sequence_chains(void *stream, const void *ops, const int *chain_ops,
                          const int *chain_staged, int n_chains);
+/* The same chains without a launch of their own: they ride in the calling thread's NEXT
+ * large-item GEMV launch (nhip_gemv_tile_lif, nhip_gemv_tile_lif_sums or
+ * nhip_gemv_tile_filter with pow2_cols >= 2), one extra work-group per chain that runs
+ * beside the groups of the GEMV.  For chains that touch nothing that launch reads or
+ * writes (unless both only read it).  This call only records its arguments (`ops` must stay
+ * valid until that launch has run; the host arrays are copied); the launch consumes them,
+ * and fails with NHIP_E_BADARG if it cannot carry them (another kernel class, no epilogue,
+ * an empty task list).  n_chains = 0 disarms.  No counterpart in the reference
+ * (plan.py:128-149 runs every plan as a launch of its own). */
+int nhip_gemv_tile_carry(const void *ops, const int *chain_ops, const int *chain_staged,
+                         int n_chains);
 
 /* ---- function nodes compiled at run time ----------------------------------
  * replaces: `plan_direct` (:954-1025), which builds an OpenCL program from the

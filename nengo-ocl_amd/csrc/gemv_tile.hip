@@ -32,6 +32,7 @@
 #include "nhip_common.h"
 #include "gemv_types.h"
 #include "neuron_math.h"
+#include "sequence_ops.h"
 
 #include <type_traits>
 
@@ -863,16 +864,39 @@ __device__ __forceinline__ float row_from_right(float v) {
 // a row block is then one aligned run of memory, read in quads and laid out in LDS as it
 // lies in memory, although single rows are not 16-byte aligned.
 constexpr int SET_TINY = 1, SET_MID = 2, SET_WIDE = 4, SET_FLAT = 8;
+// A sequence of short streaming operations (sequence_ops.h) that rides in a launch of the
+// kernel below, one extra group per chain behind the groups of the GEMV: the operations of
+// a step that touch nothing the launch touches (clock, input playback, small filters, probe
+// gather) then cost no launch of their own.
+struct SeqSide {
+    const NhipSeqOp* ops;
+    SeqChains chains;
+    int n_chains;       // 0: none
+    int n_gemv_groups;  // groups of the GEMV itself (the grid has n_chains more)
+};
+
 template <int EPI, int SET>
 __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 14) ? 3 : 4, 4))) void gemv_stream_kernel(
     const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
     int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
-    float* Y, EpilogueArgs epi)
+    float* Y, EpilogueArgs epi, SeqSide side)
 {
     constexpr bool WIDE = (SET & (SET_MID | SET_WIDE)) != 0;  // the large LDS layout
     constexpr bool FLAT = (SET & SET_FLAT) != 0;
     static_assert(!(FLAT && WIDE), "back-to-back rows: single-stage widths only");
     extern __shared__ __attribute__((aligned(16))) float lds[];
+    if (EPI != EPI_NONE && side.n_chains > 0 && (int)blockIdx.x >= side.n_gemv_groups) {
+        // (uniform over the group: all of its threads run the chain and its barriers)
+        const int c = blockIdx.x - side.n_gemv_groups;
+        NhipSeqOp* s_ops = reinterpret_cast<NhipSeqOp*>(lds);
+        int (*s_rows)[SEQ_ROW_WORDS] = reinterpret_cast<int (*)[SEQ_ROW_WORDS]>(
+            lds + SEQ_MAX_OPS * sizeof(NhipSeqOp) / sizeof(float));
+        sequence_chain(side.ops + side.chains.first_op[c],
+                       side.chains.first_op[c + 1] - side.chains.first_op[c],
+                       side.chains.n_staged[c], s_ops, s_rows, threadIdx.x);
+        return;
+    }
+    const int n_gemv_groups = (EPI != EPI_NONE && side.n_chains > 0) ? side.n_gemv_groups : gridDim.x;
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // a launch without wide dot products keeps its tasks to 128 rows (fewer registers)
@@ -881,7 +905,7 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
     float* xb = ab + STREAM_BLK_WORDS;  // gathered X of the current column stage, tiles padded
     float* ys = xb + xb_words;          // running sum of row r of the task
 
-    const int t = nhip_xcd_remap(blockIdx.x, gridDim.x) * (NHIP_WG / NHIP_WAVE) + wave;
+    const int t = nhip_xcd_remap(blockIdx.x, n_gemv_groups) * (NHIP_WG / NHIP_WAVE) + wave;
     if (t >= n_tasks) return;  // wave-uniform; the kernel has no group barrier
 
     const GemvFatTask ft = tasks[t];
@@ -1215,10 +1239,22 @@ extern "C" int nhip_gemv_tile_rows(int n_cols, int blk_words) {
 
 namespace {
 
+// what nhip_gemv_tile_carry armed for the calling thread's next launch
+struct Carried {
+    const NhipSeqOp* ops = nullptr;
+    SeqChains chains = {};
+    int n_chains = 0;
+};
+thread_local Carried carried;
+
 int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* items,
                 const float* coefs, const int* dots, const int* tasks, int n_tasks, const float* A,
                 const float* X, const float* Yin, float* Y, int epilogue, const EpilogueArgs& args) {
-    if (n_tasks == 0) return 0;
+    if (n_tasks == 0) {
+        const bool armed = carried.n_chains > 0;
+        carried = Carried{};
+        return armed ? NHIP_E_BADARG : 0;  // an empty launch cannot carry a sequence
+    }
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
@@ -1239,6 +1275,18 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
         return NHIP_E_BADARG;
     const int n_groups = (n_tasks + waves - 1) / waves;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // a sequence armed by nhip_gemv_tile_carry rides in this launch
+    SeqSide side{};
+    side.n_gemv_groups = n_groups;
+    if (carried.n_chains > 0) {
+        side.ops = carried.ops;
+        side.chains = carried.chains;
+        side.n_chains = carried.n_chains;
+        carried = Carried{};
+        if (pow2_cols < 2 || epilogue == EPI_NONE ||
+            lds_bytes < SEQ_MAX_OPS * sizeof(NhipSeqOp) + sizeof(int) * SEQ_MAX_ROWS * SEQ_ROW_WORDS)
+            return NHIP_E_BADARG;  // only launches of the compile-time-shape kernel with an epilogue
+    }
     auto launch = [&](auto kernel) {
         NHIP_LAUNCH(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
                            reinterpret_cast<const GemvItem*>(items),
@@ -1250,10 +1298,10 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     auto launch_epi = [&](auto epi_tag) {
         constexpr int E = decltype(epi_tag)::value;
         auto launch_stream = [&](auto kernel) {
-            NHIP_LAUNCH(kernel, dim3(n_groups), dim3(NHIP_WG), lds_bytes, s,
+            NHIP_LAUNCH(kernel, dim3(n_groups + side.n_chains), dim3(NHIP_WG), lds_bytes, s,
                         reinterpret_cast<const GemvDot*>(dots),
                         reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, stream_xb, A, X, Yin,
-                        Y, args);
+                        Y, args, side);
         };
         if (pow2_cols == 2) launch_stream(gemv_stream_kernel<E, SET_WIDE>);
         else if (pow2_cols == 3) launch_stream(gemv_stream_kernel<E, 0>);
@@ -1345,4 +1393,26 @@ extern "C" int nhip_gemv_tile_filter(void* stream, int vec, int pow2_cols, int b
     args.filter.F = F;
     return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
                        Yin, Y, EPI_FILTER, args);
+}
+
+extern "C" int nhip_gemv_tile_carry(const void* ops, const int* chain_ops, const int* chain_staged,
+                                    int n_chains) {
+    if (n_chains == 0) {
+        carried = Carried{};
+        return 0;
+    }
+    if (n_chains < 0 || n_chains > NHIP_SEQ_MAX_CHAINS || !ops || !chain_ops || !chain_staged)
+        return NHIP_E_BADARG;
+    Carried c;
+    c.ops = static_cast<const NhipSeqOp*>(ops);
+    c.n_chains = n_chains;
+    for (int k = 0; k < n_chains; ++k) {
+        if (chain_ops[k] < 1 || chain_ops[k] > SEQ_MAX_OPS || chain_staged[k] < 0 ||
+            chain_staged[k] > SEQ_MAX_ROWS)
+            return NHIP_E_BADARG;
+        c.chains.first_op[k + 1] = c.chains.first_op[k] + chain_ops[k];
+        c.chains.n_staged[k] = chain_staged[k];
+    }
+    carried = c;
+    return 0;
 }

@@ -201,3 +201,47 @@ def merge_small_plans(plans):
             out.append(plan)
     close()
     return out
+
+
+def _can_carry(plan):
+    """Launches of the large-item GEMV kernel with compile-time shapes and an epilogue."""
+    cls = getattr(plan, "kernel_class", None)
+    return (getattr(plan, "name", "") in ("hipra_gemv.tile_lif", "hipra_gemv.tile_filter")
+            and cls is not None and cls[0] == 3 and cls[1] >= 2 and plan.prelude is None
+            and getattr(plan, "n_tasks", 0) > 0)
+
+
+def carry_sequences(plans):
+    """Sequence launches (and single small plans) next to a large-item GEMV launch that
+    touches none of their memory ride in that launch, in work-groups of their own
+    (``nhip_gemv_tile_carry``): the launch before them if it can take them, else the one
+    after.  The plan list loses those launches; results are unchanged."""
+    plans = list(plans)
+    k = 0
+    while k < len(plans):
+        seq = plans[k]
+        rides = getattr(seq, "name", "") == "hip_sequence" or (
+            hasattr(seq, "enqueue") and is_small(seq))
+        if not rides:
+            k += 1
+            continue
+        for j in (k - 1, k + 1):
+            if 0 <= j < len(plans) and _can_carry(plans[j]) and not _conflict(seq, plans[j]):
+                break
+        else:
+            k += 1
+            continue
+        if seq.name != "hip_sequence":
+            seq = plan_sequence(seq.queue, [seq])
+        carrier = plans[j]
+        carrier.prelude = (seq.queue.lib.nhip_gemv_tile_carry, seq.args)
+        carrier.full_args = carrier.full_args + (seq,)
+        carrier.carried = seq
+        carrier.tag = "%s + %s" % (carrier.tag, seq.tag)
+        carrier.gsize = (carrier.gsize[0] + seq.gsize[0],)
+        if carrier.bw_per_call and seq.bw_per_call:
+            carrier.bw_per_call += seq.bw_per_call
+        carrier.reads_mem = carrier.reads_mem | seq.reads_mem
+        carrier.writes_mem = carrier.writes_mem | seq.writes_mem
+        del plans[k]
+    return plans

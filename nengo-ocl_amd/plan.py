@@ -77,6 +77,9 @@ class Plan(BasePlan):
         self.lsize = self._format_size(lsize) if lsize is not None else None
         self.full_args = tuple(full_args)
         self._events_to_profile = []
+        # (function, arguments) of a call that prepares the launch and launches nothing
+        # itself, made right before it (a sequence the launch carries)
+        self.prelude = None
 
     @staticmethod
     def _format_size(size):
@@ -101,6 +104,8 @@ class Plan(BasePlan):
                 _lib.check(lib.nhip_time_next_launch(ev0, ev1))
             else:
                 _lib.check(lib.nhip_event_record(ev0, handle))
+        if self.prelude is not None:
+            _lib.check(self.prelude[0](*self.prelude[1]), self.name)
         _lib.check(self.kern(handle, *self.args), self.name)
         if profiling:
             if own and lib.nhip_launch_events_pending():

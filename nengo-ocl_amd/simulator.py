@@ -80,6 +80,8 @@ class HipBackend:
 
         self.plan_sparse_dot_inc = hipra_spmv.plan_sparse_dot_inc
         self.merge_small_plans = hipra_sequence.merge_small_plans
+        if os.environ.get("NENGO_HIP_CARRY_SEQUENCES", "1") != "0":  # switch for measurements
+            self.carry_sequences = hipra_sequence.carry_sequences
         self.plans_conflict = hipra_sequence._conflict
         self.fuse_gemv_filter = hipra_gemv.fuse_linearfilter
 
@@ -422,6 +424,8 @@ class Simulator:
             plans = self._fuse_input_sums(plans)
         if merge_small and hasattr(self.backend, "merge_small_plans"):
             plans = self.backend.merge_small_plans(plans)
+            if fuse and hasattr(self.backend, "carry_sequences"):
+                plans = self.backend.carry_sequences(plans)
         logger.info("Plans in %0.3f s", _time.time() - t0)
 
         self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches)

@@ -169,7 +169,7 @@ def test_c3_full_size_state_bit_exact(queue):
     configuration the throughput is quoted on, surrogate decoders as in the benchmark):
     after 40 steps every signal -- currents, voltages, refractory times, spikes, decoded
     and filtered values -- and every probe sample is bit-identical to the oracle's, and
-    the step runs as the three launches the benchmark times."""
+    the step runs as the two launches the benchmark times."""
     from nengo_ocl_amd import configs
     from nengo_ocl_amd.simulator import Simulator
     from oracle.oracle_sim import OracleSimulator
@@ -179,8 +179,11 @@ def test_c3_full_size_state_bit_exact(queue):
     with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
         assert len(gpu.signal_aliases) == 3 * 768
         names = [p.name for p in gpu._plans]
-        # input sums + encoders + neurons, decoders + synapses, clock / input / probes
-        assert sorted(names) == ["hip_sequence", "hipra_gemv.tile_filter", "hipra_gemv.tile_lif"]
+        # input sums + encoders + neurons; decoders + synapses, with clock / input / probes
+        # riding in groups of their own
+        assert sorted(names) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_lif"]
+        assert [p.carried.name for p in gpu._plans if p.name == "hipra_gemv.tile_filter"] == [
+            "hip_sequence"]
         assert [p.input_sums for p in gpu._plans if p.name == "hipra_gemv.tile_lif"] == [254]
         classes = {p.name: p.kernel_class for p in gpu._plans if hasattr(p, "kernel_class")}
         assert classes["hipra_gemv.tile_lif"] == (3, 3, 4)     # compile-time shapes, narrow
@@ -199,7 +202,7 @@ def test_merged_products_keep_every_signal(queue):
     """One built model (per-connection decoders, reduced c3) run on the GPU with identical
     products merged and without: every probe sample and every signal of the model --
     dropped duplicates through their alias -- bit-identical after 200 steps, and the
-    merged step is the three launches of the benchmark."""
+    merged step is the two launches of the benchmark."""
     from nengo_ocl_amd import configs
     from nengo_ocl_amd.simulator import Simulator
 
@@ -207,8 +210,7 @@ def test_merged_products_keep_every_signal(queue):
     model = net.build_model(dt=0.001)
     with Simulator(None, model=model, seed=1) as a, \
             Simulator(None, model=model, seed=1, dedup=False) as b:
-        assert sorted(p.name for p in a._plans) == [
-            "hip_sequence", "hipra_gemv.tile_filter", "hipra_gemv.tile_lif"]
+        assert sorted(p.name for p in a._plans) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_lif"]
         assert a.all_data.buf.size < b.all_data.buf.size
         a.run_steps(200)
         b.run_steps(200)
@@ -217,6 +219,42 @@ def test_merged_products_keep_every_signal(queue):
         for base in {sig.base for op in model.operators for sig in op.all_signals}:
             got, want = np.asarray(a.signals[base]), np.asarray(b.signals[base])
             assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), base
+
+
+def test_launch_fusions_change_nothing(queue, monkeypatch):
+    """Input sums formed inside the encoder launch and the short operations of a step
+    carried by the decoder launch, against the same model with each as a launch of its
+    own: four launches per step become two, every signal and probe sample stays
+    bit-identical (eager and as a recorded graph), and a failed carry is reported."""
+    from nengo_ocl_amd import _lib, configs
+    from nengo_ocl_amd.simulator import Simulator
+
+    net, probes, _ = configs.c3_large(n_ens=8, n_neurons=1024, dims=64, fan_out=4)
+    model = net.build_model(dt=0.001)
+    sims = []
+    for sums, carry, graph in (("1", "1", True), ("1", "1", False), ("0", "0", True)):
+        monkeypatch.setenv("NENGO_HIP_INPUT_SUMS", sums)
+        monkeypatch.setenv("NENGO_HIP_CARRY_SEQUENCES", carry)
+        sims.append(Simulator(None, model=model, seed=1, use_graph=graph))
+    a, eager, plain = sims
+    with a, eager, plain:
+        assert [len(s._plans) for s in sims] == [2, 2, 4]
+        for s in sims:
+            s.run_steps(100)
+        for other in (eager, plain):
+            for p in probes.values():
+                assert np.array_equal(a.data[p], other.data[p]) and np.any(a.data[p] != 0)
+            assert np.array_equal(np.asarray(a.all_data.buf), np.asarray(other.all_data.buf))
+        # a launch that cannot carry a sequence says so instead of dropping it
+        lib = queue.lib
+        carrier = [p for p in a._plans if getattr(p, "carried", None) is not None][0]
+        fn, args = carrier.prelude
+        _lib.check(fn(*args))
+        small = [p for p in plain._plans if p.name == "hipra_gemv.wave_ref"][0]
+        big = [p for p in plain._plans if p.name == "hipra_gemv.tile_lif"][0]
+        assert lib.nhip_gemv_tile(queue.handle, *big.args[:7], 0, *big.args[8:12]) == -1
+        _lib.check(fn(args[0], args[1], args[2], 0))  # disarmed
+        small()
 
 
 @pytest.mark.parametrize("case", ["c2", "c3-per-connection", "c4", "c5"])
