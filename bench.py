@@ -305,8 +305,9 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
     ap.add_argument("--no-fuse", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--learn-in-place", action="store_true",
-                    help="learning rules add their change to the weights in one pass (c4)")
+    ap.add_argument("--two-pass-learning", action="store_true",
+                    help="learning rules write a delta matrix that a copy adds to the weights in "
+                         "the next step, as the builder emits it (c4); default: one pass")
     ap.add_argument("--max-regions", type=int, default=25,
                     help="a timed region of K steps shorter than 50 ms is repeated up to this "
                          "many times; the median region is reported")
@@ -336,7 +337,7 @@ def main():
     t0 = time.time()
     (net, probes, _), workload = make_network(args.config, args.variant, args.scale)
     sim = Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph,
-                    learn_in_place=args.learn_in_place, dedup=args.variant == "shared")
+                    learn_in_place=not args.two_pass_learning, dedup=args.variant == "shared")
     build_s = time.time() - t0
     n_plans = len(sim._plans)
 
@@ -398,7 +399,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": workload, "neurons": net.n_neurons, "plans_per_step": n_plans,
                    "dt": 0.001, "graph": not args.no_graph,
-                   "fused_copies": not args.no_fuse, "learn_in_place": args.learn_in_place,
+                   "fused_copies": not args.no_fuse, "learn_in_place": not args.two_pass_learning,
                    "identical_products_merged": args.variant == "shared"},
         "roofline": roofline,
         "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,

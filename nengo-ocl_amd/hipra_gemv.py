@@ -44,7 +44,7 @@ TASK_OVERHEAD_BYTES = 8192.0  # what starting and finishing a task costs, in str
 # The large-item kernel with compile-time shapes takes dot products of STREAM_MIN_COLS
 # columns or more whose rows are 16-byte aligned; its LDS block has STREAM_STAGE_WORDS words.
 STREAM_MIN_COLS, STREAM_STAGE_WORDS = 5, 2176
-STREAM_NARROW_MAX_ROWS = 128
+STREAM_NARROW_MAX_ROWS = int(os.environ.get("NENGO_HIP_NARROW_ROWS", 128))
 # instance of that kernel (`pow2_cols`) for matrices of at most FLAT_MAX_COLS columns
 # whose rows are not 16-byte aligned but lie back to back: blocks of rows are read as
 # aligned runs of memory

@@ -225,10 +225,19 @@ def carry_sequences(plans):
         if not rides:
             k += 1
             continue
-        for j in (k - 1, k + 1):
-            if 0 <= j < len(plans) and _can_carry(plans[j]) and not _conflict(seq, plans[j]):
+        # the nearest launch that can take it, backwards then forwards, over plans that touch
+        # none of its memory (moving past those changes nothing)
+        j = None
+        for step in (-1, 1):
+            q = k + step
+            while 0 <= q < len(plans) and hasattr(plans[q], "enqueue") and not _conflict(seq, plans[q]):
+                if _can_carry(plans[q]):
+                    j = q
+                    break
+                q += step
+            if j is not None:
                 break
-        else:
+        if j is None:
             k += 1
             continue
         if seq.name != "hip_sequence":
@@ -243,5 +252,5 @@ def carry_sequences(plans):
             carrier.bw_per_call += seq.bw_per_call
         carrier.reads_mem = carrier.reads_mem | seq.reads_mem
         carrier.writes_mem = carrier.writes_mem | seq.writes_mem
-        del plans[k]
+        del plans[k]  # (the same index now holds the next plan)
     return plans

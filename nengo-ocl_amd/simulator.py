@@ -231,18 +231,22 @@ class Simulator:
     multi-stream recording crashed inside the runtime for one step shape;
     ``merge_small=False`` keeps every short
     operation (clock, inputs, small copies and filters, probes) as a launch of its
-    own instead of binding runs of them into one launch; ``learn_in_place=True`` (with
-    ``fuse``) lets learning rules add their change to the learned matrix directly instead
-    of writing a delta matrix that a copy adds in the next step: one pass over the matrix
-    instead of two, identical values inside the simulation and in all probe data, but the
-    delta signals are not written and ``sim.signals[weights]`` read between steps already
-    holds the change of the last step (`operators.apply_learning_in_place`).
+    own instead of binding runs of them into one launch; ``learn_in_place`` (on by
+    default, with ``fuse``) lets learning rules whose delta matrix nothing but the
+    builder's increment reads, and that is not probed, add their change to the learned
+    matrix directly instead of writing a delta matrix that a copy adds in the next step:
+    one pass over the matrix instead of two, identical values inside the simulation and
+    in all probe data, but the delta signals are not written and ``sim.signals[weights]``
+    read between steps already holds the change of the last step
+    (`operators.apply_learning_in_place`); ``learn_in_place=False`` keeps the two passes;
+    ``dedup=False`` keeps products and synapses that compute the same values from the same
+    inputs as separate operators (`operators.merge_identical_chains`).
     """
 
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
                  n_prealloc_probes=None, profiling=None, if_python_code="none",
                  planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
-                 fuse=True, branches=False, merge_small=True, learn_in_place=False,
+                 fuse=True, branches=False, merge_small=True, learn_in_place=True,
                  dedup=True):
         self.closed = False
         self.model = None
@@ -465,10 +469,12 @@ class Simulator:
             if getattr(lf, "lf_spec", None) is None:
                 continue
             i = j - 2
+            between = []  # plans the fused filters would move ahead of
             while i >= 0 and not hasattr(plans[i], "prog"):
-                if not hasattr(plans[i], "enqueue") or self.backend.plans_conflict(lf, plans[i]):
+                if not hasattr(plans[i], "enqueue"):
                     i = -1
                     break
+                between.append(plans[i])
                 i -= 1
             if i < 0:
                 continue
@@ -488,6 +494,12 @@ class Simulator:
                 (fr, fw), (rr, rw) = mem(lambda k: k not in rest), mem(lambda k: k in rest)
             else:
                 (fr, fw), (rr, rw) = (lf.reads_mem, lf.writes_mem), (lf.reads_mem, lf.writes_mem)
+            # only the filters that move must not touch what the plans in between touch
+            # (the others stay where they are): a learning rule that reads a filtered
+            # activity does not keep the synapses of decoded values out of the GEMV
+            moved = type("Moved", (), {"reads_mem": fr, "writes_mem": fw})
+            if any(self.backend.plans_conflict(moved, q) for q in between):
+                continue
             for new, old in zip(fused, plans[lo:i + 1]):
                 new.reads_mem = old.reads_mem | fr
                 new.writes_mem = old.writes_mem | fw

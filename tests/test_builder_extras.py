@@ -59,7 +59,7 @@ def conv_network(channels_last=True, seed=3):
 def test_hebbian_rules_change_weights(rule_type):
     rule = mb.BCM(learning_rate=1e-9) if rule_type == "BCM" else mb.Oja(learning_rate=1e-6)
     net, conn, probes = hebbian_network(rule)
-    with OracleSimulator(net, seed=1) as sim:
+    with OracleSimulator(net, seed=1, learn_in_place=False) as sim:  # (the delta is read below)
         kinds = [type(op).__name__ for op in sim.model.operators]
         assert "Sim" + rule_type in kinds
         wsig = sim.model.sig[conn]["weights"]
@@ -180,7 +180,7 @@ def test_learning_in_place_gives_the_same_simulation(rule_type):
         return [(copies[op.delta], op.delta) for op in rules]
 
     (net_a, probes_a), (net_b, probes_b) = make(), make()
-    with OracleSimulator(net_a, seed=1) as two_pass, \
+    with OracleSimulator(net_a, seed=1, learn_in_place=False) as two_pass, \
             OracleSimulator(net_b, seed=1, learn_in_place=True) as in_place:
         kinds = lambda sim: [type(op).__name__ for op in sim.operators]
         assert kinds(in_place).count("Copy") < kinds(two_pass).count("Copy")
