@@ -133,22 +133,36 @@ __device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const floa
     if (outer && !((d.y_start | d.y_shape1 | d.y_stride0 | d.offset | d.count) & 3)) {
         // outer product whose rows are made of whole aligned quads: four elements of one
         // row per lane, 16 bytes per access to Y (the same products and sums)
-        for (int k = 4 * lane; k < d.count; k += 4 * L) {
-            int i, j;
-            nhip_row_col(i0, j0, k, d.y_shape1, d.count, i, j);
-            const float aa = __fmul_rn(alpha, ew_element(a, d.a_shape0, 1, d.a_stride0, i, 0));
-            float xx[4];
+        // (four quads per lane at a time: their operands are requested together, so a lane
+        // waits for memory once per four stores, not once per store)
+        constexpr int U = 4;
+        for (int k0 = 4 * lane; k0 < d.count; k0 += U * 4 * L) {
+            float4* dst[U];
+            float4 w[U];
+            float aa[U], xx[U][4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) xx[e] = ew_element(x, d.x_shape0, 1, d.x_stride0, j + e, 0);
-            float4* dst = reinterpret_cast<float4*>(y + (size_t)i * d.y_stride0 + j);
-            float4 v = make_float4(__fmul_rn(aa, xx[0]), __fmul_rn(aa, xx[1]),
-                                   __fmul_rn(aa, xx[2]), __fmul_rn(aa, xx[3]));
-            if (inc) {
-                const float4 w = *dst;
-                v = make_float4(__fadd_rn(w.x, v.x), __fadd_rn(w.y, v.y), __fadd_rn(w.z, v.z),
-                                __fadd_rn(w.w, v.w));
+            for (int u = 0; u < U; ++u) {
+                const int k = min(k0 + u * 4 * L, d.count - 4);  // past the end: the last quad again
+                int i, j;
+                nhip_row_col(i0, j0, k, d.y_shape1, d.count, i, j);
+                dst[u] = reinterpret_cast<float4*>(y + (size_t)i * d.y_stride0 + j);
+                if (inc) w[u] = *dst[u];
+                aa[u] = ew_element(a, d.a_shape0, 1, d.a_stride0, i, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    xx[u][e] = ew_element(x, d.x_shape0, 1, d.x_stride0, j + e, 0);
             }
-            *dst = v;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (k0 + u * 4 * L >= d.count) break;
+                const float s = __fmul_rn(alpha, aa[u]);
+                float4 v = make_float4(__fmul_rn(s, xx[u][0]), __fmul_rn(s, xx[u][1]),
+                                       __fmul_rn(s, xx[u][2]), __fmul_rn(s, xx[u][3]));
+                if (inc)
+                    v = make_float4(__fadd_rn(w[u].x, v.x), __fadd_rn(w[u].y, v.y),
+                                    __fadd_rn(w[u].z, v.z), __fadd_rn(w[u].w, v.w));
+                *dst[u] = v;
+            }
         }
         return;
     }

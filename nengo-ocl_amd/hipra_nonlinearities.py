@@ -245,7 +245,10 @@ def plan_elementwise_inc(queue, A, X, Y, alpha=None, outer=False, inc=True, tag=
         alphas = np.ones(len(Y), dtype=np.float32)
     _check(("A", A), ("X", X), ("Y", Y))
 
-    inds, offsets, counts, lanes = rows_for(Y.sizes)
+    # large outer products (learning rules over whole weight matrices): rows of 4096
+    # elements, four 16-byte accesses per lane issued together
+    big = outer and int(Y.sizes.sum()) >= (1 << 20)
+    inds, offsets, counts, lanes = rows_for(Y.sizes, max_size=4 * BLOCK if big else BLOCK)
     flags = np.full(len(inds), (1 if outer else 0) | (2 if inc else 0), dtype=np.int32)
     table, n = _dev_table(queue, [
         A.starts[inds], A.shape0s[inds], A.shape1s[inds], A.stride0s[inds],
