@@ -87,7 +87,8 @@ def gemv_summary(sim, profile_steps):
     return rows
 
 
-KERNEL_SOURCES = ("gemv_tile.hip", "gemv_types.h", "gemv_rows.h", "neuron_math.h", "nhip_common.h")
+KERNEL_SOURCES = ("gemv_tile.hip", "gemv_types.h", "gemv_rows.h", "neuron_math.h", "nhip_common.h",
+                  "sequence_ops.h")
 
 
 def kernel_sources_hash():
