@@ -26,6 +26,7 @@
 #include "nhip_common.h"
 #include "gemv_types.h"
 #include "gemv_rows.h"
+#include "sequence_ops.h"
 
 namespace {
 
@@ -224,12 +225,46 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_wave_kernel(
 
 // ---------------------------------------------------------------- reference order, small items
 // (the kernel body lives in gemv_rows.h)
+// In `side.n_chains` extra groups behind those of the GEMV a launch can run a sequence of
+// short operations that touches nothing the launch touches (sequence_ops.h).
+struct RowsSide {
+    const NhipSeqOp* ops;
+    SeqChains chains;
+    int n_chains;
+    int n_gemv_groups;
+};
+
+// what nhip_gemv_tile_carry armed for this thread, taken over by the launch at hand
+__host__ inline bool take_carried(RowsSide& side) {
+    side = RowsSide{};
+    if (nhip_carried.n_chains <= 0) return false;
+    side.ops = static_cast<const NhipSeqOp*>(nhip_carried.ops);
+    for (int c = 0; c <= NHIP_SEQ_MAX_CHAINS; ++c) side.chains.first_op[c] = nhip_carried.first_op[c];
+    for (int c = 0; c < NHIP_SEQ_MAX_CHAINS; ++c) side.chains.n_staged[c] = nhip_carried.n_staged[c];
+    side.n_chains = nhip_carried.n_chains;
+    nhip_carried = NhipCarried{};
+    return true;
+}
+
+// a group behind the GEMV's runs its chain (uniform over the group)
+#define NHIP_ROWS_SIDE_GROUP(side)                                                          \
+    if ((side).n_chains > 0 && (int)blockIdx.x >= (side).n_gemv_groups) {                   \
+        __shared__ NhipSeqOp s_ops[SEQ_MAX_OPS];                                             \
+        __shared__ __attribute__((aligned(16))) int s_rows[SEQ_MAX_ROWS][SEQ_ROW_WORDS];     \
+        const int c = blockIdx.x - (side).n_gemv_groups;                                     \
+        sequence_chain((side).ops + (side).chains.first_op[c],                               \
+                       (side).chains.first_op[c + 1] - (side).chains.first_op[c],            \
+                       (side).chains.n_staged[c], s_ops, s_rows, threadIdx.x);               \
+        return;                                                                              \
+    }
+
 template <int LPR, bool WIDE>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
-    const float* A, const float* X, const float* Yin, float* Y)
+    const float* A, const float* X, const float* Yin, float* Y, const RowsSide side)
 {
+    NHIP_ROWS_SIDE_GROUP(side)
     gemv_rows_ref_block<LPR, EPI_NONE, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
                                              blockIdx.x, threadIdx.x);
 }
@@ -240,8 +275,10 @@ template <int LPR, int EPI, bool WIDE>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_epi_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
-    const float* A, const float* X, const float* Yin, float* Y, const EpilogueArgs epi)
+    const float* A, const float* X, const float* Yin, float* Y, const EpilogueArgs epi,
+    const RowsSide side)
 {
+    NHIP_ROWS_SIDE_GROUP(side)
     gemv_rows_ref_block<LPR, EPI, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
                                         blockIdx.x, threadIdx.x, &epi);
 }
@@ -250,17 +287,21 @@ template <int EPI>
 int launch_rows_epi(hipStream_t s, int lpr, int task_words, const int* items, const float* coefs,
                     const int* dots, const int* tasks, int n_tasks, const float* A, const float* X,
                     const float* Yin, float* Y, const EpilogueArgs& epi) {
+    // a sequence armed by nhip_gemv_tile_carry rides in this launch
+    RowsSide side;
+    if (take_carried(side) && n_tasks <= 0) return NHIP_E_BADARG;  // an empty launch cannot carry it
     if (n_tasks == 0) return 0;
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (lpr != 4 && lpr != 1) return NHIP_E_BADCLASS;
     if (task_words != 4 && task_words != 16) return NHIP_E_BADARG;
     const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
-    const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
+    side.n_gemv_groups = (n_tasks + rows_per_group - 1) / rows_per_group;
+    const dim3 grid(side.n_gemv_groups + side.n_chains);
     auto launch = [&](auto kernel) {
         NHIP_LAUNCH(kernel, grid, dim3(NHIP_WG), 0, s, reinterpret_cast<const GemvItem*>(items),
                     reinterpret_cast<const float4*>(coefs), reinterpret_cast<const GemvDot*>(dots),
-                    reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi);
+                    reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi, side);
     };
     if (lpr == 4 && task_words == 16) launch(gemv_rows_ref_epi_kernel<4, EPI, true>);
     else if (lpr == 4) launch(gemv_rows_ref_epi_kernel<4, EPI, false>);
@@ -351,6 +392,10 @@ extern "C" int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes)
 extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes, const int* items,
                          const float* coefs, const int* dots, const int* tasks, int n_tasks,
                          const float* A, const float* X, const float* Yin, float* Y) {
+    // a sequence armed by nhip_gemv_tile_carry: only small-item launches in the reference's
+    // order (flavor 2) can carry it
+    RowsSide side;
+    if (take_carried(side) && (n_tasks <= 0 || flavor != 2)) return NHIP_E_BADARG;
     if (n_tasks == 0) return 0;
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
@@ -372,12 +417,13 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
         if ((lpr != 4 && lpr != 1) || vec != 1) return NHIP_E_BADCLASS;
         if (passes != 0 && passes != 16) return NHIP_E_BADARG;  // words of a task record
         const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
-        const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
+        side.n_gemv_groups = (n_tasks + rows_per_group - 1) / rows_per_group;
+        const dim3 grid(side.n_gemv_groups + side.n_chains);
         auto launch = [&](auto kernel) {
             NHIP_LAUNCH(kernel, grid, dim3(NHIP_WG), 0, s, reinterpret_cast<const GemvItem*>(items),
                         reinterpret_cast<const float4*>(coefs),
                         reinterpret_cast<const GemvDot*>(dots),
-                        reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y);
+                        reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, side);
         };
         if (lpr == 4 && passes == 16) launch(gemv_rows_ref_kernel<4, true>);
         else if (lpr == 4) launch(gemv_rows_ref_kernel<4, false>);

@@ -1239,20 +1239,12 @@ extern "C" int nhip_gemv_tile_rows(int n_cols, int blk_words) {
 
 namespace {
 
-// what nhip_gemv_tile_carry armed for the calling thread's next launch
-struct Carried {
-    const NhipSeqOp* ops = nullptr;
-    SeqChains chains = {};
-    int n_chains = 0;
-};
-thread_local Carried carried;
-
 int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* items,
                 const float* coefs, const int* dots, const int* tasks, int n_tasks, const float* A,
                 const float* X, const float* Yin, float* Y, int epilogue, const EpilogueArgs& args) {
     if (n_tasks == 0) {
-        const bool armed = carried.n_chains > 0;
-        carried = Carried{};
+        const bool armed = nhip_carried.n_chains > 0;
+        nhip_carried = NhipCarried{};
         return armed ? NHIP_E_BADARG : 0;  // an empty launch cannot carry a sequence
     }
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
@@ -1278,11 +1270,12 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     // a sequence armed by nhip_gemv_tile_carry rides in this launch
     SeqSide side{};
     side.n_gemv_groups = n_groups;
-    if (carried.n_chains > 0) {
-        side.ops = carried.ops;
-        side.chains = carried.chains;
-        side.n_chains = carried.n_chains;
-        carried = Carried{};
+    if (nhip_carried.n_chains > 0) {
+        side.ops = static_cast<const NhipSeqOp*>(nhip_carried.ops);
+        for (int c = 0; c <= NHIP_SEQ_MAX_CHAINS; ++c) side.chains.first_op[c] = nhip_carried.first_op[c];
+        for (int c = 0; c < NHIP_SEQ_MAX_CHAINS; ++c) side.chains.n_staged[c] = nhip_carried.n_staged[c];
+        side.n_chains = nhip_carried.n_chains;
+        nhip_carried = NhipCarried{};
         if (pow2_cols < 2 || epilogue == EPI_NONE ||
             lds_bytes < SEQ_MAX_OPS * sizeof(NhipSeqOp) + sizeof(int) * SEQ_MAX_ROWS * SEQ_ROW_WORDS)
             return NHIP_E_BADARG;  // only launches of the compile-time-shape kernel with an epilogue
@@ -1395,24 +1388,26 @@ extern "C" int nhip_gemv_tile_filter(void* stream, int vec, int pow2_cols, int b
                        Yin, Y, EPI_FILTER, args);
 }
 
+thread_local NhipCarried nhip_carried;
+
 extern "C" int nhip_gemv_tile_carry(const void* ops, const int* chain_ops, const int* chain_staged,
                                     int n_chains) {
     if (n_chains == 0) {
-        carried = Carried{};
+        nhip_carried = NhipCarried{};
         return 0;
     }
     if (n_chains < 0 || n_chains > NHIP_SEQ_MAX_CHAINS || !ops || !chain_ops || !chain_staged)
         return NHIP_E_BADARG;
-    Carried c;
-    c.ops = static_cast<const NhipSeqOp*>(ops);
+    NhipCarried c;
+    c.ops = ops;
     c.n_chains = n_chains;
     for (int k = 0; k < n_chains; ++k) {
         if (chain_ops[k] < 1 || chain_ops[k] > SEQ_MAX_OPS || chain_staged[k] < 0 ||
             chain_staged[k] > SEQ_MAX_ROWS)
             return NHIP_E_BADARG;
-        c.chains.first_op[k + 1] = c.chains.first_op[k] + chain_ops[k];
-        c.chains.n_staged[k] = chain_staged[k];
+        c.first_op[k + 1] = c.first_op[k] + chain_ops[k];
+        c.n_staged[k] = chain_staged[k];
     }
-    carried = c;
+    nhip_carried = c;
     return 0;
 }

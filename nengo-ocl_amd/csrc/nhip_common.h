@@ -72,3 +72,14 @@ __device__ __forceinline__ void nhip_row_col(int i0, int j0, int k, int cols, in
     i = i0 + q;
     j = t - q * cols;
 }
+
+// A sequence of short operations armed by nhip_gemv_tile_carry for the calling thread's next
+// GEMV launch with an epilogue (large items, compile-time shapes; or small items): the
+// launch runs its chains in extra work-groups.  first_op / n_staged as in SeqChains.
+struct NhipCarried {
+    const void* ops = nullptr;
+    int first_op[NHIP_SEQ_MAX_CHAINS + 1] = {};
+    int n_staged[NHIP_SEQ_MAX_CHAINS] = {};
+    int n_chains = 0;
+};
+extern thread_local NhipCarried nhip_carried;  // defined with nhip_gemv_tile_carry
