@@ -23,6 +23,8 @@
 //          networks with thousands of small ensembles.
 // Lanes of a row own interleaved column quads (lane l: columns 4l..4l+3, then
 // + 4*LPR ...), so one load instruction of a wave covers contiguous memory.
+#include <type_traits>
+
 #include "nhip_common.h"
 #include "gemv_types.h"
 #include "gemv_rows.h"
@@ -258,27 +260,29 @@ __host__ inline bool take_carried(RowsSide& side) {
         return;                                                                              \
     }
 
-template <int LPR, bool WIDE>
+// (SIDE: the instance for launches that carry a sequence; the others are compiled without
+// that path and its LDS)
+template <int LPR, bool WIDE, bool SIDE>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     const float* A, const float* X, const float* Yin, float* Y, const RowsSide side)
 {
-    NHIP_ROWS_SIDE_GROUP(side)
+    if (SIDE) NHIP_ROWS_SIDE_GROUP(side)
     gemv_rows_ref_block<LPR, EPI_NONE, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
                                              blockIdx.x, threadIdx.x);
 }
 
 // the same with an epilogue per finished row (A, X, Yin are not marked read-only
 // here either: the epilogue writes neuron state / filter outputs into the same buffer)
-template <int LPR, int EPI, bool WIDE>
+template <int LPR, int EPI, bool WIDE, bool SIDE>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_epi_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     const float* A, const float* X, const float* Yin, float* Y, const EpilogueArgs epi,
     const RowsSide side)
 {
-    NHIP_ROWS_SIDE_GROUP(side)
+    if (SIDE) NHIP_ROWS_SIDE_GROUP(side)
     gemv_rows_ref_block<LPR, EPI, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
                                         blockIdx.x, threadIdx.x, &epi);
 }
@@ -303,10 +307,15 @@ int launch_rows_epi(hipStream_t s, int lpr, int task_words, const int* items, co
                     reinterpret_cast<const float4*>(coefs), reinterpret_cast<const GemvDot*>(dots),
                     reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, epi, side);
     };
-    if (lpr == 4 && task_words == 16) launch(gemv_rows_ref_epi_kernel<4, EPI, true>);
-    else if (lpr == 4) launch(gemv_rows_ref_epi_kernel<4, EPI, false>);
-    else if (task_words == 16) launch(gemv_rows_ref_epi_kernel<1, EPI, true>);
-    else launch(gemv_rows_ref_epi_kernel<1, EPI, false>);
+    auto pick = [&](auto side_tag) {
+        constexpr bool SD = decltype(side_tag)::value;
+        if (lpr == 4 && task_words == 16) launch(gemv_rows_ref_epi_kernel<4, EPI, true, SD>);
+        else if (lpr == 4) launch(gemv_rows_ref_epi_kernel<4, EPI, false, SD>);
+        else if (task_words == 16) launch(gemv_rows_ref_epi_kernel<1, EPI, true, SD>);
+        else launch(gemv_rows_ref_epi_kernel<1, EPI, false, SD>);
+    };
+    if (side.n_chains > 0) pick(std::true_type{});
+    else pick(std::false_type{});
     NHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -425,10 +434,15 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
                         reinterpret_cast<const GemvDot*>(dots),
                         reinterpret_cast<const GemvTask*>(tasks), n_tasks, A, X, Yin, Y, side);
         };
-        if (lpr == 4 && passes == 16) launch(gemv_rows_ref_kernel<4, true>);
-        else if (lpr == 4) launch(gemv_rows_ref_kernel<4, false>);
-        else if (passes == 16) launch(gemv_rows_ref_kernel<1, true>);
-        else launch(gemv_rows_ref_kernel<1, false>);
+        auto pick = [&](auto side_tag) {
+            constexpr bool SD = decltype(side_tag)::value;
+            if (lpr == 4 && passes == 16) launch(gemv_rows_ref_kernel<4, true, SD>);
+            else if (lpr == 4) launch(gemv_rows_ref_kernel<4, false, SD>);
+            else if (passes == 16) launch(gemv_rows_ref_kernel<1, true, SD>);
+            else launch(gemv_rows_ref_kernel<1, false, SD>);
+        };
+        if (side.n_chains > 0) pick(std::true_type{});
+        else pick(std::false_type{});
         NHIP_LAUNCH_CHECK();
         return 0;
     } else if (flavor == 1) {
