@@ -205,6 +205,21 @@ int nhip_gemv_rows_lif(void *stream, int lpr, int task_words, const int *items, 
                        const float *X, const float *Yin, float *Y, const int *pops, double dt,
                        int upsample, float *V, float *W, float *S, const float *TAU,
                        const float *REF, const float *AMP);
+/* nhip_gemv_rows_lif that forms input sums itself, as nhip_gemv_tile_lif_sums does for
+ * large items (replaces the same three reference steps): the vector operand of an item's
+ * first dot product -- every dot product of such an item has at most 4 columns -- or the
+ * rows of an item without dot products, is x[c] = (...(0 + v_0[c] s_0) + v_1[c] s_1) + ...
+ *   sum_ranges : int32[n_items][2] {first part, number of parts} (0 parts: none)
+ *   parts      : int32[n][2] {start of vector v_k, start of scalar s_k}, offsets into X
+ * The first row of an item stores the sum at the operand's place (x_start of the dot
+ * product, stride 1); X and Y must be the same buffer; no part may overlap anything the
+ * launch writes.  Bit-identical to the separate launches while the old sums are finite. */
+int nhip_gemv_rows_lif_sums(void *stream, int lpr, int task_words, const int *items,
+                            const float *coefs, const int *dots, const int *tasks, int n_tasks,
+                            const float *A, const float *X, const float *Yin, float *Y,
+                            const int *pops, double dt, int upsample, float *V, float *W,
+                            float *S, const float *TAU, const float *REF, const float *AMP,
+                            const int *sum_ranges, const int *parts);
 int nhip_gemv_rows_filter(void *stream, int lpr, int task_words, const int *items,
                           const float *coefs, const int *dots, const int *tasks, int n_tasks,
                           const float *A,

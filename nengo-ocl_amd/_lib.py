@@ -36,6 +36,8 @@ SIGNATURES = {
     "nhip_gemv_tile_rows": [c_int, c_int],
     "nhip_gemv_rows_lif": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
                            P, ctypes.c_double, c_int, P, P, P, P, P, P],
+    "nhip_gemv_rows_lif_sums": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
+                                P, ctypes.c_double, c_int, P, P, P, P, P, P, P, P],
     "nhip_gemv_rows_filter": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P, P, P, P],
     "nhip_spmv_sell": [P, P, c_int, P, P, P, P, P],
     "nhip_lif": [P, P, c_int, c_double, c_int, P, P, P, P, P, P, P],

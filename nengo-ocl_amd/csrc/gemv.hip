@@ -482,6 +482,34 @@ extern "C" int nhip_gemv_rows_lif(void* stream, int lpr, int task_words, const i
                                     dots, tasks, n_tasks, A, X, Yin, Y, args);
 }
 
+extern "C" int nhip_gemv_rows_lif_sums(void* stream, int lpr, int task_words, const int* items,
+                                       const float* coefs, const int* dots, const int* tasks,
+                                       int n_tasks, const float* A, const float* X,
+                                       const float* Yin, float* Y, const int* pops, double dt,
+                                       int upsample, float* V, float* W, float* S,
+                                       const float* TAU, const float* REF, const float* AMP,
+                                       const int* sum_ranges, const int* parts) {
+    if (!pops || !V || !W || !S || upsample < 1 || !(dt > 0.0) || !sum_ranges || !parts)
+        return NHIP_E_BADARG;
+    if (static_cast<const float*>(Y) != X) return NHIP_E_BADARG;  // the sums are stored through Y
+    EpilogueArgs args{};
+    LifArgs& lif = args.lif;
+    lif.pops = reinterpret_cast<const LifPop*>(pops);
+    lif.dtu = (float)(dt / (double)upsample);
+    lif.dt_inv = (float)(1.0 / dt);
+    lif.upsample = upsample;
+    lif.V = V;
+    lif.W = W;
+    lif.S = S;
+    lif.TAU = TAU;
+    lif.REF = REF;
+    lif.AMP = AMP;
+    lif.parts = reinterpret_cast<const int2*>(parts);
+    lif.sum_ranges = reinterpret_cast<const int2*>(sum_ranges);
+    return launch_rows_epi<EPI_LIF>(static_cast<hipStream_t>(stream), lpr, task_words, items, coefs,
+                                    dots, tasks, n_tasks, A, X, Yin, Y, args);
+}
+
 extern "C" int nhip_gemv_rows_filter(void* stream, int lpr, int task_words, const int* items,
                                      const float* coefs, const int* dots, const int* tasks,
                                      int n_tasks,

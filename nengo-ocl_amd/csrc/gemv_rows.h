@@ -85,6 +85,35 @@ __device__ __forceinline__ void gemv_rows_ref_block(
         f_old = epi->filter.F[f_range.y > 0 ? (size_t)f_first.y_start + r : 0];
     }
     float sum = cf.y * Yin[it.yin_start + (size_t)r * it.yin_stride0];
+    // LIF launches that form input sums themselves: the vector operand of the item's first
+    // dot product (at most 4 columns), or the whole row of an item without dot products, is
+    // (...(0 + v_0[c] s_0) + v_1[c] s_1) + ..., what this kernel computes for
+    // Y = 0 * Y + sum_k v_k s_k as a launch of its own
+    int2 sum_range = make_int2(0, 0);
+    if (EPI == EPI_LIF && epi->lif.sum_ranges != nullptr && valid)
+        sum_range = epi->lif.sum_ranges[task.item];
+    auto summed = [&](int c) {
+        // (the records of four parts, then their operands, are requested together: the
+        // launch is a chain of dependent reads, and this keeps it two links per four parts)
+        float s = 0.0f;
+        for (int q0 = 0; q0 < sum_range.y; q0 += 4) {
+            int2 part[4];
+            float v[4], w[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                part[u] = epi->lif.parts[sum_range.x + min(q0 + u, sum_range.y - 1)];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                v[u] = X[(size_t)part[u].x + c];
+                w[u] = X[part[u].y];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (q0 + u < sum_range.y) s = s + fmaf(v[u], w[u], 0.0f);
+        }
+        return s;
+    };
+    if (EPI == EPI_LIF && sum_range.y > 0 && n_dots == 0) sum = summed(r);
 
     for (int d0 = 0; __any(d0 < n_dots); d0 += BATCH) {
         GemvDot dot[BATCH];
@@ -104,6 +133,11 @@ __device__ __forceinline__ void gemv_rows_ref_block(
                     const bool live = d0 + k < n_dots && c < dot[k].N;
                     a[k][e] = live ? A[dot[k].a_start + (size_t)r * dot[k].a_stride0 + c] : 0.0f;
                     x[k][e] = live ? X[dot[k].x_start + (size_t)c * dot[k].x_stride0] : 0.0f;
+                    if (EPI == EPI_LIF && k == 0 && d0 == 0 && live && sum_range.y > 0) {
+                        x[k][e] = summed(c);
+                        // the item's first row also stores the sum in the operand's place
+                        if (r == 0) Y[(size_t)dot[k].x_start + c] = x[k][e];
+                    }
                 }
 #pragma unroll
             for (int k = 0; k < BATCH; ++k) {

@@ -1242,11 +1242,10 @@ namespace {
 int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* items,
                 const float* coefs, const int* dots, const int* tasks, int n_tasks, const float* A,
                 const float* X, const float* Yin, float* Y, int epilogue, const EpilogueArgs& args) {
-    if (n_tasks == 0) {
-        const bool armed = nhip_carried.n_chains > 0;
-        nhip_carried = NhipCarried{};
-        return armed ? NHIP_E_BADARG : 0;  // an empty launch cannot carry a sequence
-    }
+    // a sequence armed by nhip_gemv_tile_carry is this launch's, whatever becomes of it
+    const NhipCarried armed = nhip_carried;
+    nhip_carried = NhipCarried{};
+    if (n_tasks == 0) return armed.n_chains > 0 ? NHIP_E_BADARG : 0;  // nothing to ride in
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
     if (vec != 1 && vec != 4) return NHIP_E_BADCLASS;
@@ -1270,12 +1269,11 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
     // a sequence armed by nhip_gemv_tile_carry rides in this launch
     SeqSide side{};
     side.n_gemv_groups = n_groups;
-    if (nhip_carried.n_chains > 0) {
-        side.ops = static_cast<const NhipSeqOp*>(nhip_carried.ops);
-        for (int c = 0; c <= NHIP_SEQ_MAX_CHAINS; ++c) side.chains.first_op[c] = nhip_carried.first_op[c];
-        for (int c = 0; c < NHIP_SEQ_MAX_CHAINS; ++c) side.chains.n_staged[c] = nhip_carried.n_staged[c];
-        side.n_chains = nhip_carried.n_chains;
-        nhip_carried = NhipCarried{};
+    if (armed.n_chains > 0) {
+        side.ops = static_cast<const NhipSeqOp*>(armed.ops);
+        for (int c = 0; c <= NHIP_SEQ_MAX_CHAINS; ++c) side.chains.first_op[c] = armed.first_op[c];
+        for (int c = 0; c < NHIP_SEQ_MAX_CHAINS; ++c) side.chains.n_staged[c] = armed.n_staged[c];
+        side.n_chains = armed.n_chains;
         if (pow2_cols < 2 || epilogue == EPI_NONE ||
             lds_bytes < SEQ_MAX_OPS * sizeof(NhipSeqOp) + sizeof(int) * SEQ_MAX_ROWS * SEQ_ROW_WORDS)
             return NHIP_E_BADARG;  // only launches of the compile-time-shape kernel with an epilogue

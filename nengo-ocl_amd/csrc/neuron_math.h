@@ -30,6 +30,9 @@ struct LifArgs {
     // scalars, parts[begin .. begin + n) = {vector start, scalar start} in the X buffer;
     // begin / n ride in the spare words of the task record.  Null: no item has one.
     const int2* parts;
+    // the same for the small-item kernel, whose task records have no spare words: per GEMV
+    // item {first part, number of parts} (0 parts: the operand is read as usual).  Null: none.
+    const int2* sum_ranges;
 };
 
 __device__ __forceinline__ float lif_param(int word, bool is_vector, const float* data, int i) {

@@ -485,6 +485,7 @@ class gemv_prog:
             plan.members = list(members)
             plan.prog = self
             plan.host_tasks = task_tab if flavor == 3 or task_tab.shape[1] == 16 else None
+            plan.host_tables = (item_tab, coef_tab, task_tab)  # (for plans that extend the launch)
             plans.append(plan)
         return plans
 
@@ -581,6 +582,7 @@ def _epilogue_call(lib, plan, kind, extras=None):
         dev_tasks = to_device(plan.queue, tasks)
         tables = tables[:3] + (dev_tasks.ptr,) + tables[4:]
         keep = (dev_tasks,)
+        plan.epilogue_tasks = tasks
     return getattr(lib, "nhip_gemv_rows_" + kind), (plan.args[1], task_words) + tables, keep
 
 
@@ -700,10 +702,13 @@ def fuse_lif(prog, lif_plan):
         fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
         fused.members, fused.prog = plan.members, prog
         fused.gemv_bytes = plan.bw_per_call
+        fused.host_pops = table
+        fused.lif_written = [V, W, S]
         if plan.kernel_class[0] == 3:
             fused.host_tasks = plan.host_tasks
-            fused.host_pops = table
-            fused.lif_written = [V, W, S]
+        else:  # small items: 16-word records as the launch takes them, or the 4-word table
+            fused.host_tasks = getattr(plan, "epilogue_tasks", None)
+            fused.host_tables = plan.host_tables
         out.append(fused)
     if rest:
         out.append(plan_lif(queue, spec["dt"], J[rest], V[rest], W[rest], S[rest],
@@ -714,24 +719,33 @@ def fuse_lif(prog, lif_plan):
 
 
 def fuse_input_sums(sum_plan, lif_plan):
-    """One launch less for "x = sum of vectors; J = E x; LIF(J)": the large-item launch with
-    the LIF epilogue (`fuse_lif`) forms the vector operands it needs itself, when the
-    small-item launch `sum_plan` right before it does nothing but form them.
+    """One launch less for "x = sum of vectors; J = E x; LIF(J)": the launch with the LIF
+    epilogue (`fuse_lif`) forms the vector operands it needs itself, when the small-item
+    launch `sum_plan` right before it does nothing but form them.
 
     Fused when every item of `sum_plan` is ``Y = 0 * Y + 0 + sum_k v_k * s_k`` (one-column
     dot products: vectors times scalars, alpha = 1) of at most 64 elements with stride 1,
-    is the vector operand of the FIRST dot product of an item of `lif_plan` (a launch of the
-    compile-time-shape kernel) and of nothing else in that GEMV, and no part ``v_k`` / ``s_k``
-    is something either launch writes; all in one device buffer.  The sums are formed with
+    is the vector operand of the FIRST dot product of an item of `lif_plan` and of nothing
+    else in that GEMV, and no part ``v_k`` / ``s_k`` is something either launch writes; all
+    in one device buffer.  `lif_plan` is a launch of the large-item kernel with compile-time
+    shapes (a first dot product of at most 64 columns), or of the small-item kernel when no
+    dot product of the launch has more than 4 columns (ensembles of one to four
+    dimensions).  Sums that nothing in the launch reads become items without dot products.  The sums are formed with
     the roundings and in the order of the small-item kernel and stored where it stores them,
     so results are bit-identical as long as the sums' old values are finite (the 0 * Y
     term is not formed).  Returns the plan that replaces ``[sum_plan, lif_plan]``, or None.
     """
     S, E = getattr(sum_plan, "prog", None), getattr(lif_plan, "prog", None)
-    if (S is None or E is None or sum_plan.name != "hipra_gemv.wave_ref"
-            or lif_plan.name != "hipra_gemv.tile_lif" or getattr(lif_plan, "host_tasks", None) is None
-            or lif_plan.kernel_class[0] != 3 or lif_plan.kernel_class[1] < 2):
+    if S is None or E is None or sum_plan.name != "hipra_gemv.wave_ref":
         return None
+    large = (lif_plan.name == "hipra_gemv.tile_lif" and lif_plan.kernel_class[0] == 3
+             and lif_plan.kernel_class[1] >= 2 and getattr(lif_plan, "host_tasks", None) is not None)
+    small = (lif_plan.name == "hipra_gemv.wave_ref_lif" and lif_plan.kernel_class[0] == 2
+             and getattr(lif_plan, "host_tables", None) is not None)
+    if not (large or small):
+        return None
+    if small and any(d["a_shape1"] > 4 for b in lif_plan.members for d in E.geometry[b]["dots"]):
+        return None  # the small-item kernel forms sums on its path for narrow dot products only
     queue, lib = E.queue, E.queue.lib
     buf = E.X.ptr.value
     if any(ra.ptr.value != buf for ra in (S.A, S.X, S.Y, S.Y_in, E.Y)):
@@ -759,7 +773,8 @@ def fuse_input_sums(sum_plan, lif_plan):
                 continue
             want = sums.get(d["x_start"])
             if (k != 0 or g["index"] not in members or want is None or want[0] != d["a_shape1"]
-                    or d["x_stride0"] != 1 or stream_stage(d["a_shape1"])[0] > 6):
+                    or (d["x_stride0"] != 1 and d["a_shape1"] > 1)
+                    or stream_stage(d["a_shape1"])[0] > 6):
                 return None
             used.add(d["x_start"])
         # (matrices and old outputs that overlap a sum would be read while it is written)
@@ -787,32 +802,73 @@ def fuse_input_sums(sum_plan, lif_plan):
     for start, (_, parts) in sums.items():
         where[start] = (len(part_rows), len(parts))
         part_rows.extend(parts)
-    tasks = lif_plan.host_tasks.copy()  # 24-word records: task, item, coefficients, first dot
-    for row in tasks:
-        if row[9] > 0 and int(row[19]) in where:  # the item has dot products; x_start of the first
-            row[3], row[11] = where[int(row[19])]
-    args = tuple(lif_plan.args)
-    keep = ()
-    if spare:
-        # one task each, of an item without dot products and without neurons: Y = the sum
-        pops = np.concatenate([lif_plan.host_pops, np.zeros((1, 8), dtype=np.int32)])
-        extra = np.zeros((len(spare), 24), dtype=np.int32)
-        for row, start in zip(extra, spare):
-            first, count = where[start]
-            row[0:4] = (len(pops) - 1, 0, sums[start][0], first)
-            row[4:12] = (start, 1, start, 1, 0, 0, sums[start][0], count)
-            row[12:16] = np.array([1.0, 0.0, 0.0, 0.0], dtype=np.float32).view(np.int32)
-        tasks = np.concatenate([tasks, extra])
-        dev_pops = to_device(queue, pops)
-        args = args[:12] + (dev_pops.ptr,) + args[13:]
-        keep = (dev_pops,)
-    dev_tasks = to_device(queue, tasks)
     dev_parts = to_device(queue, np.array(part_rows, dtype=np.int32))
-    n_groups = -(-len(tasks) // (WG // WAVE))
-    args = args[:6] + (dev_tasks.ptr, len(tasks)) + args[8:] + (dev_parts.ptr,)
+    args = tuple(lif_plan.args)
     sum_bytes = sum_plan.bw_per_call or 0
-    fused = Plan(queue, lib.nhip_gemv_tile_lif_sums, args, gsize=(WG * n_groups,), lsize=lif_plan.lsize,
-                 full_args=tuple(lif_plan.full_args) + (dev_tasks, dev_parts) + keep,
+    one = np.array([1.0, 0.0, 0.0, 0.0], dtype=np.float32).view(np.int32)
+    if large:
+        tasks = lif_plan.host_tasks.copy()  # 24-word records: task, item, coefficients, first dot
+        for row in tasks:
+            if row[9] > 0 and int(row[19]) in where:  # has dot products; x_start of the first
+                row[3], row[11] = where[int(row[19])]
+        keep = ()
+        if spare:
+            # one task each, of an item without dot products and without neurons: Y = the sum
+            pops = np.concatenate([lif_plan.host_pops, np.zeros((1, 8), dtype=np.int32)])
+            extra = np.zeros((len(spare), 24), dtype=np.int32)
+            for row, start in zip(extra, spare):
+                first, count = where[start]
+                row[0:4] = (len(pops) - 1, 0, sums[start][0], first)
+                row[4:12] = (start, 1, start, 1, 0, 0, sums[start][0], count)
+                row[12:16] = one
+            tasks = np.concatenate([tasks, extra])
+            dev_pops = to_device(queue, pops)
+            args = args[:12] + (dev_pops.ptr,) + args[13:]
+            keep = (dev_pops,)
+        dev_tasks = to_device(queue, tasks)
+        n_groups = -(-len(tasks) // (WG // WAVE))
+        args = args[:6] + (dev_tasks.ptr, len(tasks)) + args[8:] + (dev_parts.ptr,)
+        entry = lib.nhip_gemv_tile_lif_sums
+        keep = keep + (dev_tasks, dev_parts)
+    else:
+        # (lpr, task words, items, coefs, dots, tasks, n_tasks, A, X, Yin, Y, pops, ...): the
+        # ranges of parts go by item; sums nothing reads become items without dot products
+        lpr, task_words = args[0], args[1]
+        item_tab, coef_tab, plain_tasks = lif_plan.host_tables
+        n_items = len(item_tab)
+        tasks = (lif_plan.host_tasks if task_words == 16 else plain_tasks).copy()
+        items = np.concatenate([item_tab, np.zeros((len(spare), 8), dtype=np.int32)])
+        coefs = np.concatenate([coef_tab, np.zeros((len(spare), 4), dtype=np.float32)])
+        pops = np.concatenate([lif_plan.host_pops[:n_items],
+                               np.zeros((len(spare), 8), dtype=np.int32)])
+        ranges = np.zeros((len(items), 2), dtype=np.int32)
+        for b in lif_plan.members:
+            dots = E.geometry[b]["dots"]
+            if dots and dots[0]["x_start"] in where:
+                ranges[b] = where[dots[0]["x_start"]]
+        extra = []
+        for k, start in enumerate(spare):
+            b, n = n_items + k, sums[start][0]
+            items[b] = (start, 1, start, 1, 0, 0, n, 0)
+            coefs[b] = (1.0, 0.0, 0.0, 0.0)
+            ranges[b] = where[start]
+            for r in range(n):
+                if task_words == 16:
+                    extra.append(np.concatenate([[b, r, 1, 0], items[b], one]).astype(np.int32))
+                    extra[-1][15] = 0
+                else:
+                    extra.append(np.array([b, r, 1, 0], dtype=np.int32))
+        if extra:
+            tasks = np.concatenate([tasks, np.array(extra, dtype=np.int32)])
+        dev = [to_device(queue, t) for t in (items, coefs, tasks, pops, ranges)]
+        rows_per_group = (WG // WAVE) * (WAVE // lpr)
+        n_groups = -(-len(tasks) // rows_per_group)
+        args = (lpr, task_words, dev[0].ptr, dev[1].ptr, args[4], dev[2].ptr, len(tasks)) + args[7:11] \
+            + (dev[3].ptr,) + args[12:] + (dev[4].ptr, dev_parts.ptr)
+        entry = lib.nhip_gemv_rows_lif_sums
+        keep = tuple(dev) + (dev_parts,)
+    fused = Plan(queue, entry, args, gsize=(WG * n_groups,), lsize=lif_plan.lsize,
+                 full_args=tuple(lif_plan.full_args) + keep,
                  name=lif_plan.name, tag=lif_plan.tag,
                  bw_per_call=lif_plan.bw_per_call + sum_bytes,
                  flops_per_call=(lif_plan.flops_per_call or 0) + (sum_plan.flops_per_call or 0))

@@ -947,3 +947,79 @@ def test_gemv_lif_forms_its_input_sums(queue):
     with_lif2 = g.fuse_lif(encs2, lif2)
     assert with_lif2 is not None
     assert all(g.fuse_input_sums(sums2.plans[0], p) is None for p in with_lif2)
+
+
+@pytest.mark.parametrize("n_ens", [24, 700], ids=["inline-task-records", "plain-task-records"])
+def test_small_item_lif_forms_its_input_sums(queue, n_ens):
+    """The same fusion for ensembles of 100 neurons with 1-D and 2-D inputs (the small-item
+    kernel; task records with the item inline for few rows, plain ones for many): sums of
+    one to twelve terms, a sum nothing reads, several steps with changing sources -- all
+    bit-identical to the oracle's three kernels."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from nengo_ocl_amd import hipra_nonlinearities as nl
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(5)
+    dt, n_neurons, n_src = 1e-3, 100, 40
+    dims = [1 + (k % 2) for k in range(n_ens)]
+    srcs = [rng.normal(size=2) for _ in range(n_src)]
+    scal = [np.array([v]) for v in (1.0, 0.25)]
+    ins = [rng.normal(size=d) for d in dims] + [rng.normal(size=2)]   # the last: read by nothing
+    enc = [rng.normal(scale=1.5, size=(n_neurons, d)) for d in dims]
+    bias = [rng.normal(loc=1.0, size=n_neurons) for _ in dims]
+    zeros = lambda: [np.zeros(n_neurons) for _ in dims]
+    V = [rng.uniform(0, 1, size=n_neurons) for _ in dims]
+    W = [rng.uniform(-2 * dt, 2 * dt, size=n_neurons) for _ in dims]
+    R = RA(srcs + scal + ins + enc + bias + zeros() + V + W + zeros(), align=True)
+    i_src = list(range(n_src))
+    i_scal = [n_src, n_src + 1]
+    i_in = list(range(n_src + 2, n_src + 2 + n_ens + 1))
+    at = i_in[-1] + 1
+    i_enc, i_bias, i_J, i_V, i_W, i_S = (list(range(at + k * n_ens, at + (k + 1) * n_ens))
+                                         for k in range(6))
+    sum_lens = dims + [2]
+    picks = [rng.choice(n_src, size=1 + (k * 5) % 12, replace=False) for k in range(n_ens + 1)]
+
+    def build(ra, mg, mn, q):
+        views, A_js, X_js = [], [], []
+        for length, pk in zip(sum_lens, picks):
+            a_idx = []
+            for src in pk:
+                views.append((int(ra.starts[i_src[src]]), length))
+                a_idx.append(len(views) - 1)
+            A_js.append(np.array(a_idx, dtype=np.int32))
+            X_js.append(np.array([i_scal[k % 2] for k in range(len(pk))], dtype=np.int32))
+        on_device = hasattr(ra, "dev_buf")
+        starts, lens = np.array([v[0] for v in views]), np.array([v[1] for v in views])
+        ones = np.ones(len(views), dtype=int)
+        A_sum = (type(ra).from_buffer(q, ra.dev_buf, starts, lens, ones, ones, ones) if on_device
+                 else type(ra).from_buffer(ra.buf, starts, lens, ones, ones, ones))
+        sums = mg.plan_block_gemv(q, 1.0, A_sum, A_js, ra, X_js, 0.0, ra[i_in])
+        e_A = [np.array([i], dtype=np.int32) for i in i_enc]
+        e_X = [np.array([i_in[k]], dtype=np.int32) for k in range(n_ens)]
+        encs = mg.plan_block_gemv(q, 1.0, ra, e_A, ra, e_X, 1.0, ra[i_J], Y_in=ra[i_bias])
+        lif = mn.plan_lif(q, dt, ra[i_J], ra[i_V], ra[i_W], ra[i_S], 0.002, 0.02, 1.0)
+        return sums, encs, lif
+
+    host = clone(R)
+    dev = to_dev(queue, R)
+    sums, encs, lif = build(dev, g, nl, queue)
+    assert [p.name for p in sums.plans] == ["hipra_gemv.wave_ref"]
+    with_lif = g.fuse_lif(encs, lif)
+    assert [p.name for p in with_lif] == ["hipra_gemv.wave_ref_lif"]
+    assert (with_lif[0].args[1] == 16) == (n_ens == 24)  # words of a task record
+    fused = g.fuse_input_sums(sums.plans[0], with_lif[0])
+    assert fused is not None and fused.input_sums == n_ens + 1
+    assert fused.n_tasks == with_lif[0].n_tasks + 2      # two rows of the sum nothing reads
+    osums, oencs, olif = build(host, orc, orc, None)
+    for step in range(3):
+        fused()
+        for p in osums.plans + oencs.plans:
+            p()
+        olif()
+        assert np.array_equal(dev.to_host().buf, host.buf), step
+        for i in i_src:
+            v = rng.normal(size=2)
+            host[i] = v[:, None]
+            dev[i] = v
+    assert any(host.buf[int(host.starts[i]):][:n_neurons].any() for i in i_S)
