@@ -1145,9 +1145,13 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                 // where the separate launch would have (the X operand's own place).
                 const int c = min(lane, last_cols - 1);
                 float s = 0.0f;
-                for (int q = 0; q < it.pad; ++q) {
-                    const int2 part = epi.lif.parts[task.pad + q];
-                    s = s + fmaf(X[(size_t)part.x + c], X[part.y], 0.0f);
+                for (int q0 = 0; q0 < it.pad; q0 += 2) {  // (two parts requested together)
+                    const int2 p0 = epi.lif.parts[task.pad + q0];
+                    const int2 p1 = epi.lif.parts[task.pad + min(q0 + 1, it.pad - 1)];
+                    const float v0 = X[(size_t)p0.x + c], w0 = X[p0.y];
+                    const float v1 = X[(size_t)p1.x + c], w1 = X[p1.y];
+                    s = s + fmaf(v0, w0, 0.0f);
+                    if (q0 + 1 < it.pad) s = s + fmaf(v1, w1, 0.0f);
                 }
                 xq0[0] = s;
                 if (task.row0 == 0 && lane < last_cols) Y[(size_t)dot.x_start + lane] = s;
