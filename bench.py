@@ -342,11 +342,11 @@ def main():
     build_s = time.time() - t0
     n_plans = len(sim._plans)
 
-    # W untimed steps, then one untimed launch of every recorded graph (16 + 8 + 4 + 2 + 1
+    # W untimed steps, then one untimed launch of every recorded graph (2^k + ... + 2 + 1
     # steps) so that no timed launch is a graph's first; the graphs themselves were
     # recorded and uploaded when the Simulator was constructed
     sim.run_steps(args.warmup)
-    sim.run_steps(31)
+    sim.run_steps(max(sim._plans.steps_of_every_graph(), 1))
     torch.cuda.synchronize()
 
     def timed_region():

@@ -189,8 +189,10 @@ class _GraphSegment:
     before the first step runs, so that no call of `launch` ever records anything.
     """
 
-    MAX_UNROLL = 16        # timesteps recorded back to back into the long graph
-    MAX_GRAPH_NODES = 1024
+    # timesteps recorded back to back into the long graph: as many as keep it within
+    # MAX_GRAPH_NODES kernel nodes (a step of two launches: 128 steps; of ten: 16)
+    MAX_UNROLL = 128
+    MAX_GRAPH_NODES = 256
 
     def __init__(self, queue, plans):
         self.queue = queue
@@ -229,6 +231,10 @@ class _GraphSegment:
             raise err
         _lib.check(rc, "graph capture end")
         self.execs[n_steps] = handle
+
+    def steps_of_every_graph(self):
+        """A step count whose run launches each recorded graph once."""
+        return sum(self.sizes)
 
     def prepare(self):
         """Record every graph `launch` can ask for and hand each to the device ahead of
@@ -312,6 +318,16 @@ class Plans:
                 segments.append(plan)
         close_run()
         self._segments = segments
+
+    def steps_of_every_graph(self):
+        """A step count whose run launches every recorded graph at least once (0 without
+        graphs)."""
+        if not self.use_graph:
+            return 0
+        if self._segments is None:
+            self._build_segments()
+        return max([seg.steps_of_every_graph() for seg in self._segments
+                    if isinstance(seg, _GraphSegment)] or [0])
 
     def prepare(self):
         """Record all graphs of the executor now (the Simulator calls this once its plan
