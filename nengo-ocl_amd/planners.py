@@ -21,14 +21,17 @@ def _share(a, b):
 
 
 def operator_dependency_graph(operators):
-    """``{op: set of ops that must run after it}`` for one timestep."""
+    """``{op: ops that must run after it}`` for one timestep.  The successors are kept in
+    the order the rules below find them (a dict used as an ordered set): a hash-ordered
+    set of operator objects would make the order in which operators become ready, and with
+    it the order of increments into views that overlap, vary from one run to the next."""
     by_base = defaultdict(lambda: ({}, {}, {}, {}))  # base -> (sets, incs, reads, updates)
     for op in operators:
         for kind, sigs in enumerate((op.sets, op.incs, op.reads, op.updates)):
             for sig in sigs:
                 by_base[sig.base][kind].setdefault(sig, []).append(op)
 
-    edges = {op: set() for op in operators}
+    edges = {op: {} for op in operators}
 
     def link(pre_table, post_table):
         for post_sig, post_ops in post_table.items():
@@ -37,7 +40,7 @@ def operator_dependency_graph(operators):
                     for pre in pre_ops:
                         for post in post_ops:
                             if pre is not post:
-                                edges[pre].add(post)
+                                edges[pre][post] = None
 
     for sets, incs, reads, updates in by_base.values():
         link(sets, incs)
@@ -78,7 +81,7 @@ def _plan(operators, completing):
     then greedily pick those of its operators whose written signals (sets
     against sets, incs against incs, updates against updates) do not overlap one
     another; they form one group.  Candidates are visited in the order they
-    became ready, so the result is deterministic.
+    became ready, which follows the operator list alone, so the result is deterministic.
     """
     edges = operator_dependency_graph(operators)
     n_waiting = {op: 0 for op in operators}

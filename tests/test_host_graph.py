@@ -497,3 +497,25 @@ def test_sparse_slice_window():
     mixed = np.sort(np.concatenate([band, scattered[:band.size // 4]]))  # four fifths in the band
     lo = h.slice_window(mixed, 100000, 0)
     assert lo >= 0 and lo <= 5000 and lo + h.WINDOW >= 5164
+
+
+@pytest.mark.parametrize("seed", [2, 3])
+def test_planning_is_reproducible(seed):
+    """Two simulators of one model schedule the operators identically (by position in the
+    operator list), also where several increments go into views that overlap and only the
+    planner decides their order."""
+    import gc
+
+    from random_networks import random_network
+
+    net, _ = random_network(seed, sliced=True)
+    model = net.build_model(dt=0.001)
+    schedules = []
+    junk = []
+    for k in range(3):
+        junk.append([object() for _ in range(1000 * k + 17)])  # shifts later addresses
+        with OracleSimulator(None, model=model, seed=1) as sim:
+            where = {op: i for i, op in enumerate(sim.operators)}
+            schedules.append([(t.__name__, [where[op] for op in ops]) for t, ops in sim.op_groups])
+        gc.collect()
+    assert schedules[0] == schedules[1] == schedules[2]
