@@ -43,17 +43,36 @@ def test_random_network_equals_one_operator_at_a_time(seed, sliced):
                 assert np.array_equal(got, naive.mem[base].reshape(-1)), base
 
 
+@pytest.mark.parametrize("seed", [31, 32, 33])
+def test_rich_random_network_merged_equals_unmerged(seed):
+    """Mixed neuron types, synapses of first and second order, learning rules, sparse and
+    dense links between neurons, noise: with identical products merged every probe gives
+    the numbers of the run that keeps one product per connection."""
+    net, probes = random_network(seed, sliced=False, rich=True)
+    model = net.build_model(dt=0.001)
+    with OracleSimulator(None, model=model, seed=1) as a, \
+            OracleSimulator(None, model=model, seed=1, dedup=False) as b:
+        a.run_steps(120)
+        b.run_steps(120)
+        for key, p in probes.items():
+            assert np.array_equal(a.data[p], b.data[p]), key
+            assert np.all(np.isfinite(a.data[p])), key
+        assert any(np.any(a.data[p] != 0) for p in probes.values())
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("seed,big,sliced", [
-    (1, False, True), (2, False, True), (3, False, False), (4, False, False),
-    (11, True, True), (12, True, False), (13, True, False)])
-def test_random_network_on_the_device(queue, seed, big, sliced):
+@pytest.mark.parametrize("seed,big,sliced,rich", [
+    (1, False, True, False), (2, False, True, False), (3, False, False, False),
+    (4, False, False, False), (11, True, True, False), (12, True, False, False),
+    (13, True, False, False), (21, False, True, True), (22, False, False, True),
+    (23, False, False, True), (24, True, True, True), (25, True, False, True)])
+def test_random_network_on_the_device(queue, seed, big, sliced, rich):
     """With slices among the targets the oracle simulator applies the same rewrites (the
     order of increments into overlapping views follows the operator list that is planned);
     without them it keeps one product per connection, so merging is checked as well."""
     from nengo_ocl_amd.simulator import Simulator
 
-    net, probes = random_network(seed, big=big, sliced=sliced)
+    net, probes = random_network(seed, big=big, sliced=sliced, rich=rich)
     model = net.build_model(dt=0.001)
     steps = 60 if big else 150
     with Simulator(None, model=model, seed=1) as gpu, \
