@@ -170,6 +170,53 @@ def calibrate_copy(n_floats=64 * 1024 * 1024, repeats=20):
                       "read_bytes_per_launch": 4 * n_floats, "write_bytes_per_launch": 4 * n_floats}))
 
 
+def traffic_floor(queue, n_rows, cols, n_reads=3, n_writes=4, repeats=60):
+    """Duration (microseconds, events carried by the launches) of the library's calibration
+    kernel on the traffic of a "GEMV + LIF" launch: `n_rows` x `cols` floats of matrix streamed
+    once, `n_reads` state vectors read and `n_writes` written per row (bias, voltage and
+    refractory time in; input current, voltage, refractory time and spikes out).  Two
+    matrices are streamed in turn so that nothing is left in the caches.  Returns a dict with
+    the duration without the writes, with ordinary and with non-temporal stores."""
+    import ctypes
+
+    import torch
+
+    from nengo_ocl_amd import _lib
+
+    lib = queue.lib
+    n_rows -= n_rows % 128
+    with torch.cuda.device(queue.device):
+        mats = [torch.zeros(n_rows * cols, dtype=torch.float32, device=queue.device) for _ in range(2)]
+        R = torch.zeros(max(n_reads, 1) * n_rows, dtype=torch.float32, device=queue.device)
+        W = torch.zeros(max(n_writes, 1) * n_rows, dtype=torch.float32, device=queue.device)
+    torch.cuda.synchronize()
+    ev = [ctypes.c_void_p() for _ in range(2)]
+    for e in ev:
+        _lib.check(lib.nhip_event_create(ctypes.byref(e)))
+    out = {}
+    for key, writes, nt in (("reads_only_us", 0, 0), ("us", n_writes, 0),
+                            ("nontemporal_stores_us", n_writes, 1)):
+        total = 0.0
+        for i in range(repeats + 4):
+            timed = i >= 4
+            if timed:
+                _lib.check(lib.nhip_time_next_launch(ev[0], ev[1]))
+            _lib.check(lib.nhip_calib_stream_mix(
+                queue.handle, ctypes.c_void_p(mats[i & 1].data_ptr()), n_rows, cols,
+                ctypes.c_void_p(R.data_ptr()), n_reads, ctypes.c_void_p(W.data_ptr()), writes, nt))
+            if timed:
+                ms = ctypes.c_float()
+                _lib.check(lib.nhip_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms)))
+                total += ms.value
+        out[key] = 1e3 * total / repeats
+    for e in ev:
+        lib.nhip_event_destroy(e)
+    queue.finish()
+    out["bytes"] = 4 * n_rows * (cols + n_reads + n_writes)
+    out["problem"] = "%d rows x %d columns, %d vectors read, %d written" % (n_rows, cols, n_reads, n_writes)
+    return out
+
+
 def micro_benchmarks(repeats=50):
     """Kernels that no benchmark network exercises, each on one representative problem:
     one JSON line per kernel with its average duration (start / stop events carried by
@@ -381,6 +428,23 @@ def main():
                         frac=dom["gbs"] / HBM_PEAK_GBS, traffic=traffic,
                         traffic_source=traffic_source, kernel=dom["plan"],
                         avg_us=dom["avg_us"], bytes_per_launch=dom["bytes"])
+        lif = next((p for p in sim._plans if str(p) == dom["plan"]
+                    and p.name == "hipra_gemv.tile_lif"), None)
+        if lif is not None:
+            # the same traffic through a kernel that does nothing else: rows = neurons of the
+            # launch, columns from its matrix bytes
+            geo = [lif.prog.geometry[b] for b in lif.members]
+            n_rows = sum(g["y_len"] for g in geo if g["dots"])
+            cols = sum(g["y_len"] * d["a_shape1"] for g in geo for d in g["dots"]) // max(n_rows, 1)
+            cols -= cols % 8
+            if n_rows >= 128 and cols >= 8:
+                floor = traffic_floor(sim.queue, n_rows, cols)
+                best = min(floor["us"], floor["nontemporal_stores_us"])
+                roofline["plain_kernel_same_traffic"] = dict(
+                    floor, frac_of_it=best / dom["avg_us"],
+                    note="calibration kernel of the library: streams the matrix rows, reads 3 "
+                         "and writes 4 vectors per row, keeps no summation order and updates "
+                         "no neurons")
 
     out = {
         "metric": "sim steps/sec + ragged-GEMV HBM GB/s (% peak), 1M-neuron LIF net, 1 MI355X",

@@ -567,6 +567,16 @@ int nhip_event_record(void *event, void *stream);
 int nhip_event_elapsed_ms(void *start, void *stop, float *ms_out); /* syncs on `stop` */
 int nhip_event_destroy(void *event);
 
+/* Calibration (no counterpart in the reference): what the device does with the traffic
+ * of a GEMV launch with a neuron epilogue when nothing else is asked of the kernel.  Every
+ * wave streams 128 rows x `cols` floats of the row-major `A` (n_rows x cols, 16-byte aligned,
+ * n_rows a multiple of 128, cols a multiple of 8), then reads `n_reads` and writes `n_writes`
+ * vectors of 128 floats at its rows (`R`: n_reads x n_rows, `W`: n_writes x n_rows floats,
+ * at least one float each); `nontemporal` != 0 writes with non-temporal stores.  Its
+ * duration is the floor against which bench.py reports the duration of the dominant launch. */
+int nhip_calib_stream_mix(void *stream, const float *A, long long n_rows, int cols,
+                          const float *R, int n_reads, float *W, int n_writes, int nontemporal);
+
 #ifdef __cplusplus
 }
 #endif

@@ -85,6 +85,7 @@ SIGNATURES = {
     "nhip_event_record": [P, P],
     "nhip_event_elapsed_ms": [P, P, ctypes.POINTER(c_float)],
     "nhip_event_destroy": [P],
+    "nhip_calib_stream_mix": [P, P, ctypes.c_longlong, c_int, P, c_int, P, c_int, c_int],
 }
 
 

@@ -3,6 +3,7 @@
 // never changes after construction (all device pointers and work lists are
 // fixed), so it is recorded once and replayed; this replaces the per-plan
 // Python launch loop of the reference executor (plan.py:137-149).
+#include <cstdint>
 #include <cstdio>
 #include <cstring>
 
@@ -123,4 +124,54 @@ extern "C" int nhip_event_elapsed_ms(void* start, void* stop, float* ms_out) {
 extern "C" int nhip_event_destroy(void* event) {
     if (!event) return 0;
     return (int)hipEventDestroy(static_cast<hipEvent_t>(event));
+}
+
+// ---------------------------------------------------------------- calibration
+// What this device does with the traffic of a "matrix rows in, a few state vectors in and
+// out" launch when nothing else is asked of the kernel: every wave streams a contiguous
+// block of `cols` x 128 floats (16-byte non-temporal loads, summed), then reads `n_reads`
+// and writes `n_writes` vectors of 128 floats at its rows.  No work list, no gather, no
+// summation order to keep: the duration is a floor for the GEMV launches with a neuron
+// epilogue, against which their own duration is reported.
+typedef float nhip_f4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(NHIP_WG) void calib_stream_mix_kernel(
+    const float* __restrict__ A, long long n_rows, int cols, const float* __restrict__ R, int n_reads,
+    float* W, int n_writes, int nontemporal)
+{
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    const long long t = (long long)blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6);  // 128 rows
+    if (t * 128 >= n_rows) return;
+    const nhip_f4* a = reinterpret_cast<const nhip_f4*>(A + t * 128 * cols);
+    const int n_loads = 128 * cols / (4 * NHIP_WAVE);
+    nhip_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 8
+    for (int i = 0; i < n_loads; ++i) acc += __builtin_nontemporal_load(a + i * NHIP_WAVE + lane);
+    float s = (acc.x + acc.y) + (acc.z + acc.w);
+    const long long r0 = t * 128;
+    for (int q = 0; q < n_reads; ++q)
+        for (int h = 0; h < 2; ++h) s += R[q * n_rows + r0 + h * NHIP_WAVE + lane];
+    for (int q = 0; q < n_writes; ++q)
+        for (int h = 0; h < 2; ++h) {
+            float* p = &W[q * n_rows + r0 + h * NHIP_WAVE + lane];
+            if (nontemporal) __builtin_nontemporal_store(s + q, p);
+            else *p = s + q;
+        }
+    if (n_writes == 0 && s == 12345.678f) W[0] = s;  // keeps the loads
+}
+
+extern "C" int nhip_calib_stream_mix(void* stream, const float* A, long long n_rows, int cols,
+                                     const float* R, int n_reads, float* W, int n_writes,
+                                     int nontemporal) {
+    if (!A || !R || !W || n_rows <= 0 || (n_rows % 128) || cols < 8 || (cols & 7) || n_reads < 0 ||
+        n_writes < 0)
+        return NHIP_E_BADARG;
+    if (reinterpret_cast<uintptr_t>(A) & 15u) return NHIP_E_BADARG;
+    const long long n_tasks = n_rows / 128;
+    const int waves = NHIP_WG / NHIP_WAVE;
+    NHIP_LAUNCH(calib_stream_mix_kernel, dim3((unsigned)((n_tasks + waves - 1) / waves)),
+                dim3(NHIP_WG), 0, static_cast<hipStream_t>(stream), A, n_rows, cols, R, n_reads, W, n_writes,
+                nontemporal);
+    NHIP_LAUNCH_CHECK();
+    return 0;
 }
