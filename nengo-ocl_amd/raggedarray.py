@@ -54,7 +54,13 @@ def allclose(a, b, atol=1e-3, rtol=1e-3):
 
 
 def _as_int32_row(values):
-    row = np.array(values, dtype=np.int32).reshape(-1)
+    """Offsets, shapes and strides are int32 element counts, as in the reference
+    (raggedarray.py:107-111): a buffer of 2^31 elements or more cannot be described."""
+    wide = np.asarray(values, dtype=np.int64).reshape(-1)
+    if wide.size and (wide.max() > np.iinfo(np.int32).max or wide.min() < np.iinfo(np.int32).min):
+        raise ValueError("a ragged array is limited to 2^31 - 1 elements (int32 offsets); "
+                         "got an offset, shape or stride of %d" % int(np.abs(wide).max()))
+    row = wide.astype(np.int32)
     row.setflags(write=False)
     return row
 
@@ -90,6 +96,9 @@ class RaggedArray:
             cursor = round_up(cursor, unit)
             starts.append(cursor)
             cursor += size
+        if cursor > np.iinfo(np.int32).max:
+            raise ValueError("a ragged array is limited to 2^31 - 1 elements (int32 offsets); "
+                             "these items need %d" % cursor)
 
         self._set_meta(
             starts,

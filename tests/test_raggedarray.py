@@ -79,3 +79,14 @@ def test_allclose_and_type_checks():
         RaggedArray([np.zeros(3, dtype=np.float64)])
     I = RA([[1, 2], [3]], dtype=np.int32)
     assert I.ctype == "int" and A.ctype == "float"
+
+
+def test_offsets_beyond_int32_are_refused():
+    """Offsets are int32 element counts (reference raggedarray.py:107-111): metadata that
+    does not fit is refused instead of wrapping around."""
+    buf = np.zeros(8, dtype=np.float32)
+    with pytest.raises(ValueError, match="2\\^31"):
+        RaggedArray.from_buffer(buf, [0, 2 ** 31], [1, 1], [1, 1], [1, 1], [1, 1])
+    with pytest.raises(ValueError, match="2\\^31"):
+        RaggedArray.from_buffer(buf, np.array([0, 2 ** 31 + 5], dtype=np.int64), [1, 1], [1, 1],
+                                [1, 1], [1, 1])
