@@ -248,6 +248,18 @@ int nhip_gemv_rows_filter(void *stream, int lpr, int task_words, const int *item
 int nhip_spmv_sell(void *stream, const int *slices, int n_slices, const int *row_len,
                    const int *cols, const float *vals, const float *X, float *Y);
 
+/* The same product for an X that is mostly zero (the spikes of a population; no
+ * counterpart in the reference, whose kernels multiply every stored element).  All slices
+ * read one X of `n_cols` elements at X + x_start (n_cols <= 1,179,648).  `mask` is a
+ * workspace of (n_cols + 127) / 128 * 4 words, 16-byte aligned, that the call fills with one
+ * bit per element of X ("is not +0.0") in a first launch; the second launch keeps it in LDS
+ * and takes the constant +0.0 instead of reading X where the bit is clear.  Bit-identical to
+ * nhip_spmv_sell whatever X and the matrices hold.  NHIP_E_TOOBIG when X is longer than the
+ * limit.  Events armed with nhip_time_next_launch time the first, short launch. */
+int nhip_spmv_sell_skip(void *stream, const int *slices, int n_slices, const int *row_len,
+                        const int *cols, const float *vals, const float *X, float *Y,
+                        int x_start, int n_cols, unsigned *mask);
+
 /* ---- neurons -----------------------------------------------------------
  * LIF with refractory state and spike-time interpolation.
  * replaces: clra_nonlinearities.py `plan_lif` (:1028-1146, non-adaptive,

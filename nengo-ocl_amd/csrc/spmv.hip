@@ -93,7 +93,140 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
     if (live) Y[(size_t)sl.y_start + lane] = acc;  // no wave without a slice is live
 }
 
+// ---- products whose X is mostly zero (spikes) -------------------------------------------
+// One bit per element of X ("is not +0.0"), made by a launch of its own, is kept in LDS by
+// every work-group; for a stored element whose bit is clear the operand is the constant +0.0
+// instead of a look-up in the cache.  The sum is formed as above, term by term, so the
+// result has the bits of the kernel above whatever X and the matrix hold.  Groups are
+// persistent: 16 waves per group take slices s, s + (waves of the grid), ... until none is
+// left; SPMV_SKIP_U quads of a row are in flight per lane while the previous ones are summed.
+constexpr int SPMV_SKIP_WG = 1024;
+constexpr int SPMV_MASK_WORDS = 36864;  // 144 KiB of LDS: X of up to 1,179,648 elements
+constexpr int SPMV_SKIP_U = 4;
+
+__global__ __launch_bounds__(NHIP_WG) void spmv_mask_kernel(const float* __restrict__ X, int n,
+                                                            unsigned* __restrict__ mask,
+                                                            int n_words) {
+    const int i = blockIdx.x * NHIP_WG + threadIdx.x;
+    const unsigned bits = i < n ? __float_as_uint(X[i]) : 0u;
+    const unsigned long long b = __ballot(bits != 0u);
+    if ((threadIdx.x & (NHIP_WAVE - 1)) == 0 && 2 * (i >> 6) < n_words) {
+        // (words past the last element of X, up to a multiple of 4, are written as zero)
+        mask[2 * (i >> 6)] = (unsigned)b;
+        mask[2 * (i >> 6) + 1] = (unsigned)(b >> 32);
+    }
+}
+
+__global__ __launch_bounds__(SPMV_SKIP_WG) void spmv_sell_skip_kernel(
+    const SpmvSlice* __restrict__ slices, int n_slices, const int* __restrict__ row_len,
+    const int* __restrict__ cols, const float* __restrict__ vals, const float* X, float* Y,
+    const unsigned* __restrict__ mask, int n_mask_quads)
+{
+    constexpr int U = SPMV_SKIP_U;
+    __shared__ __attribute__((aligned(16))) unsigned s_mask[SPMV_MASK_WORDS];
+    for (int i = threadIdx.x; i < n_mask_quads; i += SPMV_SKIP_WG)
+        reinterpret_cast<spmv_i4*>(s_mask)[i] = reinterpret_cast<const spmv_i4*>(mask)[i];
+    __syncthreads();  // the only barrier; every thread reaches it
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int stride = gridDim.x * (SPMV_SKIP_WG / NHIP_WAVE);
+    for (int s = blockIdx.x * (SPMV_SKIP_WG / NHIP_WAVE) + wave; s < n_slices; s += stride) {
+        const SpmvSlice sl = slices[s];
+        const bool live = lane < sl.n_rows;
+        const int len = live ? row_len[sl.len_start + lane] : 0;
+        const float* x = X + sl.x_start;
+        float acc = (live && sl.inc) ? Y[(size_t)sl.y_start + lane] : 0.0f;
+        const int n_quads = sl.width >> 2;
+        const spmv_i4* c = reinterpret_cast<const spmv_i4*>(cols + (size_t)sl.data_start) + lane;
+        const spmv_f4* v = reinterpret_cast<const spmv_f4*>(vals + (size_t)sl.data_start) + lane;
+        spmv_i4 ci[U];
+        spmv_f4 vi[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            ci[j] = spmv_i4{0, 0, 0, 0};
+            vi[j] = spmv_f4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (j < n_quads) {  // the same for all lanes
+                ci[j] = __builtin_nontemporal_load(c + (size_t)j * NHIP_WAVE);
+                vi[j] = __builtin_nontemporal_load(v + (size_t)j * NHIP_WAVE);
+            }
+        }
+        for (int q = 0; q < n_quads; q += U) {
+            // the next U quads are requested before the look-ups of the current ones
+            spmv_i4 cn[U];
+            spmv_f4 vn[U];
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                cn[j] = ci[j];
+                vn[j] = vi[j];
+                if (q + U + j < n_quads) {
+                    cn[j] = __builtin_nontemporal_load(c + (size_t)(q + U + j) * NHIP_WAVE);
+                    vn[j] = __builtin_nontemporal_load(v + (size_t)(q + U + j) * NHIP_WAVE);
+                }
+            }
+            float xi[U][4];
+#pragma unroll
+            for (int j = 0; j < U; ++j)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const unsigned col = (unsigned)ci[j][u];
+                    const bool set = (4 * (q + j) + u < len) && ((s_mask[col >> 5] >> (col & 31u)) & 1u);
+                    xi[j][u] = set ? x[col] : 0.0f;
+                }
+#pragma unroll
+            for (int j = 0; j < U; ++j)
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (4 * (q + j) + u < len) acc = fmaf(vi[j][u], xi[j][u], acc);
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                ci[j] = cn[j];
+                vi[j] = vn[j];
+            }
+        }
+        if (live) Y[(size_t)sl.y_start + lane] = acc;
+    }
+}
+
 }  // namespace
+
+// The product for an X that is mostly zero.  All slices must read the same X:
+// `n_cols` elements at X + x_start, n_cols <= 32 * SPMV_MASK_WORDS.  `mask` is a workspace
+// of (n_cols + 127) / 128 * 4 words that the call fills (one bit per element of X) and
+// then reads.  Two launches; events armed for the next launch time the first, short one.
+extern "C" int nhip_spmv_sell_skip(void* stream, const int* slices, int n_slices,
+                                   const int* row_len, const int* cols, const float* vals,
+                                   const float* X, float* Y, int x_start, int n_cols,
+                                   unsigned* mask) {
+    if (n_slices == 0) return 0;
+    if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y || !mask || x_start < 0 ||
+        n_cols <= 0)
+        return NHIP_E_BADARG;
+    if (n_cols > 32 * SPMV_MASK_WORDS) return NHIP_E_TOOBIG;
+    if ((reinterpret_cast<uintptr_t>(cols) | reinterpret_cast<uintptr_t>(vals) |
+         reinterpret_cast<uintptr_t>(mask)) & 15)
+        return NHIP_E_BADARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int n_mask_quads = (n_cols + 127) / 128;        // 128 bits per 16 bytes
+    const int n_mask_threads = n_mask_quads * 128;        // one thread per bit, whole quads
+    NHIP_LAUNCH(spmv_mask_kernel, dim3(n_mask_threads / NHIP_WG + (n_mask_threads % NHIP_WG != 0)),
+                dim3(NHIP_WG), 0, s, X + x_start, n_cols, mask, 4 * n_mask_quads);
+    NHIP_LAUNCH_CHECK();
+    static int n_cu = 0;
+    if (n_cu == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+            return NHIP_E_BADARG;
+        n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    const int wpg = SPMV_SKIP_WG / NHIP_WAVE;
+    const int n_groups = min(n_cu, (n_slices + wpg - 1) / wpg);
+    NHIP_LAUNCH(spmv_sell_skip_kernel, dim3(n_groups), dim3(SPMV_SKIP_WG), 0, s,
+                reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X, Y,
+                mask, n_mask_quads);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
 
 extern "C" int nhip_spmv_sell(void* stream, const int* slices, int n_slices, const int* row_len,
                               const int* cols, const float* vals, const float* X, float* Y) {

@@ -17,6 +17,7 @@ from .plan import Plan
 WG, WAVE = 256, 64
 QUAD = 4  # elements of a row stored side by side (one 16-byte access)
 WINDOW = 1024  # consecutive elements of X a wave can keep in LDS (SPMV_WINDOW in csrc/spmv.hip)
+SKIP_MAX_COLS = 32 * 36864  # longest X whose "is not zero" bits fit the LDS (SPMV_MASK_WORDS)
 
 
 def slice_window(columns, n_cols, x_start):
@@ -98,9 +99,16 @@ class plan_sparse_dot_inc:
     clra_gemv.py:1919) or a list of them with one X and one Y item each.  ``inc``
     defaults to False like the reference's (whose Simulator thereby *sets* Y); the
     Simulator here passes True, the meaning of the operator.
+
+    ``x_mostly_zero`` (one flag, or one per matrix) says that X is zero in most places
+    most of the time -- the spikes of a population.  When it holds for every matrix and all
+    read the same X of at most `SKIP_MAX_COLS` elements, the launch is
+    `nhip_spmv_sell_skip`: one bit per element of X ("is not +0.0") is made first and kept
+    in LDS, and where it is clear the operand is the constant instead of a look-up of X.
+    Same bits as the ordinary launch whatever X holds; only faster when X is mostly zero.
     """
 
-    def __init__(self, queue, hA, X, Y, inc=False, tag=None, algorithm=None):
+    def __init__(self, queue, hA, X, Y, inc=False, tag=None, algorithm=None, x_mostly_zero=False):
         matrices = list(hA) if isinstance(hA, (list, tuple)) else [hA]
         matrices = [m if isinstance(m, HostSparseMatrix) else HostSparseMatrix(m) for m in matrices]
         if not (len(matrices) == len(X) == len(Y)):
@@ -132,8 +140,21 @@ class plan_sparse_dot_inc:
                                              vals if vals.size else np.zeros(1, np.float32))]
         args = (dev[0].ptr, n, dev[1].ptr, dev[2].ptr, dev[3].ptr, X.ptr, Y.ptr)
         n_groups = max(1, -(-n // (WG // WAVE)))
-        plan = Plan(queue, queue.lib.nhip_spmv_sell, args, gsize=(WG * n_groups,), lsize=(WG,),
+        flags = np.broadcast_to(np.asarray(x_mostly_zero, dtype=bool), (len(matrices),))
+        same_x = len({(int(X.starts[b]), int(X.shape0s[b])) for b in range(len(matrices))}) == 1
+        skip = n > 0 and bool(flags.all()) and same_x and int(X.shape0s[0]) <= SKIP_MAX_COLS
+        if skip:
+            n_cols = int(X.shape0s[0])
+            mask = to_device(queue, np.zeros(-(-n_cols // 128) * 4, dtype=np.int32))
+            dev.append(mask)
+            entry = queue.lib.nhip_spmv_sell_skip
+            args = args + (int(X.starts[0]), n_cols, mask.ptr)
+            gsize, lsize = (1024 * min(queue.n_compute_units, -(-n // 16)),), (1024,)
+        else:
+            entry, gsize, lsize = queue.lib.nhip_spmv_sell, (WG * n_groups,), (WG,)
+        plan = Plan(queue, entry, args, gsize=gsize, lsize=lsize,
                     full_args=tuple(dev) + (X.dev_buf, Y.dev_buf), name="hip_spmv", tag=tag)
+        plan.skips_zero_x = skip
         nnz = int(sum(m.csr.nnz for m in matrices))
         plan.flops_per_call = 2 * nnz
         # reference accounting (clra_gemv.py:1552-1560): values, indices, row pointers, X, Y

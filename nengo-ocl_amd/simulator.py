@@ -79,6 +79,8 @@ class HipBackend:
         from . import hipra_spmv
 
         self.plan_sparse_dot_inc = hipra_spmv.plan_sparse_dot_inc
+        # switch for measurements: "0" multiplies every stored element of a sparse matrix
+        self.skips_zero_operands = os.environ.get("NENGO_HIP_SPMV_SKIP", "1") != "0"
         self.merge_small_plans = hipra_sequence.merge_small_plans
         if os.environ.get("NENGO_HIP_CARRY_SEQUENCES", "1") != "0":  # switch for measurements
             self.carry_sequences = hipra_sequence.carry_sequences
@@ -208,6 +210,9 @@ class ProbeData(Mapping):
 
 # numpy functions of time alone that the device runs without a host callback;
 # the translated code has the form the reference's translator emits for them
+# neuron types whose output is zero except in the steps a neuron spikes
+SPIKING_NEURON_TYPES = ("LIF", "AdaptiveLIF", "SpikingRectifiedLinear")
+
 _DIRECT_FUNCTIONS = {np.sin: "sin", np.cos: "cos", np.tanh: "tanh", np.exp: "exp",
                      np.square: "square"}
 
@@ -860,7 +865,14 @@ class Simulator:
             matrices.append(value.csr if hasattr(value, "csr") else value)
         X = self.all_data[[self.sidx[op.X] for op in ops]]
         Y = self.all_data[[self.sidx[op.Y] for op in ops]]
-        return self.backend.plan_sparse_dot_inc(self.queue, matrices, X, Y, inc=True).plans
+        extra = {}
+        if getattr(self.backend, "skips_zero_operands", False):
+            # vectors that are the spikes of a population are zero in most places
+            spikes = {op2.output.base for op2 in self.operators
+                      if type(op2).__name__ == "SimNeurons"
+                      and type(op2.neurons).__name__ in SPIKING_NEURON_TYPES}
+            extra["x_mostly_zero"] = [op.X.base in spikes for op in ops]
+        return self.backend.plan_sparse_dot_inc(self.queue, matrices, X, Y, inc=True, **extra).plans
 
     def _plan_TimeUpdate(self, ops):
         (op,) = ops

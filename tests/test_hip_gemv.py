@@ -848,6 +848,70 @@ def test_sparse_reference_cases(queue, rng, inc, long_row, sparsity, shape):
     assert np.array_equal(got, Yo[0][:, 0])
 
 
+@pytest.mark.parametrize("inc", [True, False])
+@pytest.mark.parametrize("density", [0.0, 0.06, 0.5, 1.0])
+def test_sparse_products_pass_over_zero_operands(queue, rng, inc, density):
+    """The launch for vectors that are mostly zero (spikes): several matrices reading one
+    X, rows longer than a slice is wide, an X with zeros, negative zeros and denormals in
+    it; bit-identical (signs of zero included) to the oracle's sequential product at every
+    density, also after X changes between two launches and with a stored value that is not
+    finite.  Matrices with different X take the ordinary launch."""
+    import scipy.sparse as sp
+
+    from nengo_ocl_amd import hipra_spmv
+    from oracle import oracle as orc
+
+    n_cols = 70001  # not a multiple of 128: the last mask words are partly used
+    shapes = [(3000, n_cols), (130, n_cols), (1, n_cols)]
+    mats = []
+    for m, n in shapes:
+        A = sp.random(m, n, density=0.002, random_state=rng, format="lil", dtype=np.float32)
+        A[min(5, m - 1), :3000] = rng.normal(size=3000)  # a long row among short ones
+        A = A.tocsr()
+        A.data[:] = rng.normal(size=A.nnz) * 10.0 ** rng.randint(-30, 5, size=A.nnz)
+        mats.append(A)
+
+    def draw_x():
+        x = np.where(rng.uniform(size=n_cols) < density, rng.normal(size=n_cols), 0.0).astype(np.float32)
+        x[rng.randint(0, n_cols, size=50)] = -0.0
+        x[rng.randint(0, n_cols, size=50)] = 1e-42  # denormal: not zero
+        return x
+
+    x = draw_x()
+    Xh = RA([x])
+    Y = RA([rng.normal(size=m) * (rng.uniform(size=m) < 0.5) for m, _ in shapes])
+    Yo = clone(Y)
+    dX, dY = to_dev(queue, Xh), to_dev(queue, Y)
+    idx = [0, 0, 0]
+    prog = hipra_spmv.plan_sparse_dot_inc(queue, mats, dX[idx], dY, inc=inc, x_mostly_zero=True)
+    assert prog.plans[0].skips_zero_x
+    oplan = orc.plan_sparse_dot_inc(None, mats, Xh[idx], Yo, inc=inc).plans[0]
+    for _ in range(3):
+        prog.plans[0]()
+        oplan()
+        got, want = dY.buf, Yo.buf
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        x = draw_x()
+        Xh[0] = x.reshape(-1, 1)
+        dX[0] = x.reshape(-1, 1)
+    # cases that keep the ordinary launch
+    two_x = to_dev(queue, RA([x, x]))
+    plain = hipra_spmv.plan_sparse_dot_inc(queue, mats[:2], two_x, dY[[0, 1]], x_mostly_zero=True)
+    assert not plain.plans[0].skips_zero_x
+    bad = mats[0].copy()
+    bad.data[3] = np.inf  # inf * 0 is not a number in both launches
+    outs = []
+    for flag in (True, False):
+        d = to_dev(queue, Y)
+        prog = hipra_spmv.plan_sparse_dot_inc(queue, [bad], dX, d[[0]], x_mostly_zero=flag)
+        assert prog.plans[0].skips_zero_x == flag
+        prog.plans[0]()
+        outs.append(d.to_host()[0])
+    assert np.array_equal(outs[0], outs[1], equal_nan=True)
+    plain = hipra_spmv.plan_sparse_dot_inc(queue, mats, dX[idx], dY, x_mostly_zero=[True, False, True])
+    assert not plain.plans[0].skips_zero_x
+
+
 def test_gemv_lif_forms_its_input_sums(queue):
     """Sums of vectors -> encoders -> LIF in one launch: inputs that are sums of one to
     eleven vectors times scalars (64, 40 and 8 elements), an ensemble whose input is a
