@@ -260,6 +260,21 @@ int nhip_spmv_sell_skip(void *stream, const int *slices, int n_slices, const int
                         const int *cols, const float *vals, const float *X, float *Y,
                         int x_start, int n_cols, unsigned *mask);
 
+/* Either product followed, row by row, by the first-order filters that read its output
+ * (`plan_sparse_dot_inc` followed by `plan_linearfilter`, clra_nonlinearities.py:577-803,
+ * simple case y = b0 x - a0 y or y = b0 x of :630-650): saves the filter launch and a pass
+ * over the product.
+ *   slice_epi : int32[n_slices][4] {first target, number of targets, first row of the slice
+ *               in its matrix, 0}
+ *   targets   : int32[][4] {y_start of the filter output, bits of a0, bits of b0, number of
+ *               denominator coefficients (0 or 1)}, as for nhip_gemv_tile_filter
+ *   F         : buffer of the filter outputs
+ * mask == NULL: the ordinary product (x_start, n_cols unused); else as nhip_spmv_sell_skip. */
+int nhip_spmv_sell_filter(void *stream, const int *slices, int n_slices, const int *row_len,
+                          const int *cols, const float *vals, const float *X, float *Y,
+                          const int *slice_epi, const int *targets, float *F, int x_start,
+                          int n_cols, unsigned *mask);
+
 /* ---- neurons -----------------------------------------------------------
  * LIF with refractory state and spike-time interpolation.
  * replaces: clra_nonlinearities.py `plan_lif` (:1028-1146, non-adaptive,

@@ -41,6 +41,7 @@ SIGNATURES = {
     "nhip_gemv_rows_filter": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P, P, P, P],
     "nhip_spmv_sell": [P, P, c_int, P, P, P, P, P],
     "nhip_spmv_sell_skip": [P, P, c_int, P, P, P, P, P, c_int, c_int, P],
+    "nhip_spmv_sell_filter": [P, P, c_int, P, P, P, P, P, P, P, P, c_int, c_int, P],
     "nhip_lif": [P, P, c_int, c_double, c_int, P, P, P, P, P, P, P],
     "nhip_lif_rate": [P, P, c_int, P, P, P, P, P],
     "nhip_alif": [P, P, c_int, c_double, c_int, P, P, P, P, P, P, P, P, P, P],

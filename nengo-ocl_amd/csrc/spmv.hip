@@ -19,8 +19,28 @@
 // takes the elements inside it from there: only the lanes whose column lies outside
 // go to the cache, which spares it one look-up per line and instruction.
 #include "nhip_common.h"
+#include "neuron_math.h"
 
 namespace {
+
+// First-order filters stepped on the fresh rows of a product (the synapse of a connection
+// through a sparse matrix): per slice {first target, number of targets, first row of the
+// slice in its matrix, 0}; targets as for the dense products.  slice_epi == nullptr: none.
+struct SpmvEpi {
+    const int4* slice_epi;
+    const FilterTarget* targets;
+    float* F;
+};
+
+__device__ __forceinline__ void spmv_filter_rows(const SpmvEpi& epi, int s, int lane, float y) {
+    const int4 e = epi.slice_epi[s];
+    for (int q = 0; q < e.y; ++q) {
+        const FilterTarget t = epi.targets[e.x + q];
+        float* f = epi.F + (size_t)t.y_start + e.z + lane;
+        const float bx = __fmul_rn(nhip_bits(t.b_bits), y);
+        *f = t.na ? __fsub_rn(bx, __fmul_rn(nhip_bits(t.a_bits), *f)) : bx;
+    }
+}
 
 struct SpmvSlice {
     int data_start;  // offset of the slice in `cols` / `vals`
@@ -40,7 +60,8 @@ typedef float spmv_f4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
     const SpmvSlice* __restrict__ slices, int n_slices, const int* __restrict__ row_len,
-    const int* __restrict__ cols, const float* __restrict__ vals, const float* X, float* Y)
+    const int* __restrict__ cols, const float* __restrict__ vals, const float* X, float* Y,
+    SpmvEpi epi)
 {
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int s = blockIdx.x * (NHIP_WG / NHIP_WAVE) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -90,7 +111,10 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
             ci1 = cn; vi1 = vn;
         }
     }
-    if (live) Y[(size_t)sl.y_start + lane] = acc;  // no wave without a slice is live
+    if (live) {  // no wave without a slice is live
+        Y[(size_t)sl.y_start + lane] = acc;
+        if (epi.slice_epi) spmv_filter_rows(epi, s, lane, acc);
+    }
 }
 
 // ---- products whose X is mostly zero (spikes) -------------------------------------------
@@ -120,7 +144,7 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_mask_kernel(const float* __restr
 __global__ __launch_bounds__(SPMV_SKIP_WG) void spmv_sell_skip_kernel(
     const SpmvSlice* __restrict__ slices, int n_slices, const int* __restrict__ row_len,
     const int* __restrict__ cols, const float* __restrict__ vals, const float* X, float* Y,
-    const unsigned* __restrict__ mask, int n_mask_quads)
+    const unsigned* __restrict__ mask, int n_mask_quads, SpmvEpi epi)
 {
     constexpr int U = SPMV_SKIP_U;
     __shared__ __attribute__((aligned(16))) unsigned s_mask[SPMV_MASK_WORDS];
@@ -183,20 +207,34 @@ __global__ __launch_bounds__(SPMV_SKIP_WG) void spmv_sell_skip_kernel(
                 vi[j] = vn[j];
             }
         }
-        if (live) Y[(size_t)sl.y_start + lane] = acc;
+        if (live) {
+            Y[(size_t)sl.y_start + lane] = acc;
+            if (epi.slice_epi) spmv_filter_rows(epi, s, lane, acc);
+        }
     }
 }
 
-}  // namespace
+int launch_plain(void* stream, const int* slices, int n_slices, const int* row_len,
+                 const int* cols, const float* vals, const float* X, float* Y, SpmvEpi epi) {
+    if (n_slices == 0) return 0;
+    if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y) return NHIP_E_BADARG;
+    // the kernel reads `cols`, `vals` and the runs of X it keeps in LDS 16 bytes at a time
+    if ((reinterpret_cast<uintptr_t>(cols) | reinterpret_cast<uintptr_t>(vals) |
+         reinterpret_cast<uintptr_t>(X)) & 15)
+        return NHIP_E_BADARG;
+    const int wpg = NHIP_WG / NHIP_WAVE;
+    NHIP_LAUNCH(spmv_sell_kernel, dim3((n_slices + wpg - 1) / wpg), dim3(NHIP_WG), 0,
+                       static_cast<hipStream_t>(stream),
+                       reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X,
+                       Y, epi);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
 
-// The product for an X that is mostly zero.  All slices must read the same X:
-// `n_cols` elements at X + x_start, n_cols <= 32 * SPMV_MASK_WORDS.  `mask` is a workspace
-// of (n_cols + 127) / 128 * 4 words that the call fills (one bit per element of X) and
-// then reads.  Two launches; events armed for the next launch time the first, short one.
-extern "C" int nhip_spmv_sell_skip(void* stream, const int* slices, int n_slices,
-                                   const int* row_len, const int* cols, const float* vals,
-                                   const float* X, float* Y, int x_start, int n_cols,
-                                   unsigned* mask) {
+// Two launches: the bits of X, then the product.
+int launch_skip(void* stream, const int* slices, int n_slices, const int* row_len,
+                const int* cols, const float* vals, const float* X, float* Y, int x_start,
+                int n_cols, unsigned* mask, SpmvEpi epi) {
     if (n_slices == 0) return 0;
     if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y || !mask || x_start < 0 ||
         n_cols <= 0)
@@ -223,24 +261,44 @@ extern "C" int nhip_spmv_sell_skip(void* stream, const int* slices, int n_slices
     const int n_groups = min(n_cu, (n_slices + wpg - 1) / wpg);
     NHIP_LAUNCH(spmv_sell_skip_kernel, dim3(n_groups), dim3(SPMV_SKIP_WG), 0, s,
                 reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X, Y,
-                mask, n_mask_quads);
+                mask, n_mask_quads, epi);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
 
+}  // namespace
+
 extern "C" int nhip_spmv_sell(void* stream, const int* slices, int n_slices, const int* row_len,
                               const int* cols, const float* vals, const float* X, float* Y) {
-    if (n_slices == 0) return 0;
-    if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y) return NHIP_E_BADARG;
-    // the kernel reads `cols`, `vals` and the runs of X it keeps in LDS 16 bytes at a time
-    if ((reinterpret_cast<uintptr_t>(cols) | reinterpret_cast<uintptr_t>(vals) |
-         reinterpret_cast<uintptr_t>(X)) & 15)
-        return NHIP_E_BADARG;
-    const int wpg = NHIP_WG / NHIP_WAVE;
-    NHIP_LAUNCH(spmv_sell_kernel, dim3((n_slices + wpg - 1) / wpg), dim3(NHIP_WG), 0,
-                       static_cast<hipStream_t>(stream),
-                       reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X,
-                       Y);
-    NHIP_LAUNCH_CHECK();
-    return 0;
+    return launch_plain(stream, slices, n_slices, row_len, cols, vals, X, Y, SpmvEpi{});
+}
+
+// The product for an X that is mostly zero.  All slices must read the same X:
+// `n_cols` elements at X + x_start, n_cols <= 32 * SPMV_MASK_WORDS.  `mask` is a workspace
+// of (n_cols + 127) / 128 * 4 words that the call fills (one bit per element of X) and
+// then reads.  Two launches; events armed for the next launch time the first, short one.
+extern "C" int nhip_spmv_sell_skip(void* stream, const int* slices, int n_slices,
+                                   const int* row_len, const int* cols, const float* vals,
+                                   const float* X, float* Y, int x_start, int n_cols,
+                                   unsigned* mask) {
+    return launch_skip(stream, slices, n_slices, row_len, cols, vals, X, Y, x_start, n_cols, mask,
+                       SpmvEpi{});
+}
+
+// Either product with first-order filters stepped on its fresh rows: `slice_epi` holds
+// {first target, number of targets, first row of the slice in its matrix, 0} per slice,
+// `targets` {y_start, a bits, b bits, number of denominator coefficients} as for the dense
+// products, `F` the buffer of the filter outputs.  mask == nullptr: the ordinary product.
+extern "C" int nhip_spmv_sell_filter(void* stream, const int* slices, int n_slices,
+                                     const int* row_len, const int* cols, const float* vals,
+                                     const float* X, float* Y, const int* slice_epi,
+                                     const int* targets, float* F, int x_start, int n_cols,
+                                     unsigned* mask) {
+    if (!slice_epi || !targets || !F) return NHIP_E_BADARG;
+    const SpmvEpi epi{reinterpret_cast<const int4*>(slice_epi),
+                      reinterpret_cast<const FilterTarget*>(targets), F};
+    if (mask)
+        return launch_skip(stream, slices, n_slices, row_len, cols, vals, X, Y, x_start, n_cols,
+                           mask, epi);
+    return launch_plain(stream, slices, n_slices, row_len, cols, vals, X, Y, epi);
 }

@@ -155,6 +155,11 @@ class plan_sparse_dot_inc:
         plan = Plan(queue, entry, args, gsize=gsize, lsize=lsize,
                     full_args=tuple(dev) + (X.dev_buf, Y.dev_buf), name="hip_spmv", tag=tag)
         plan.skips_zero_x = skip
+        # what `fuse_linearfilter` needs to rebuild the launch with filters behind its rows
+        plan.spmv = dict(X=X, Y=Y, slice_rows=slice_rows, dev=tuple(dev), n=n,
+                         mask=(mask if skip else None),
+                         x_start=int(X.starts[0]) if skip else 0,
+                         n_cols=int(X.shape0s[0]) if skip else 0)
         nnz = int(sum(m.csr.nnz for m in matrices))
         plan.flops_per_call = 2 * nnz
         # reference accounting (clra_gemv.py:1552-1560): values, indices, row pointers, X, Y
@@ -163,3 +168,81 @@ class plan_sparse_dot_inc:
         plan.description = "groups: %d; nonzeros: %d; stored: %d" % (len(matrices), nnz, vals.size)
         self.plans = [plan]
         self.matrices = matrices
+
+
+def fuse_linearfilter(spmv_plan, lf_plan):
+    """One launch less for "Y = A X (sparse); filter step on Y": the product steps the
+    first-order filters whose input is exactly one of its output vectors as soon as a row
+    is final (`nhip_spmv_sell_filter`), with the arithmetic of the filter kernel's simple
+    case.  Returns ``([plan replacing spmv_plan], plans replacing [lf_plan])`` -- the second
+    list holds a filter launch for the items that were not fused (their indices in
+    `lf_plan`: its ``unfused_items``), or is empty -- or None when nothing can be fused."""
+    from .hipra_gemv import _overlaps, _span
+    from .hipra_nonlinearities import plan_linearfilter
+
+    spec, sp = getattr(lf_plan, "lf_spec", None), getattr(spmv_plan, "spmv", None)
+    if spec is None or sp is None or sp["n"] == 0:
+        return None
+    queue = spmv_plan.queue
+    X, F, A, B = spec["X"], spec["Y"], spec["A"], spec["B"]
+    Y, SX = sp["Y"], sp["X"]
+    if X.ptr.value != Y.ptr.value:
+        return None
+    outputs = {(int(Y.starts[b]), int(Y.shape0s[b])): b for b in range(len(Y))}
+    a_host, b_host = A.to_host(), B.to_host()
+    targets_of, rest = {}, []
+    for i in range(len(X)):
+        simple = int(B.shape0s[i]) == 1 and int(A.shape0s[i]) <= 1
+        vector = (int(X.shape1s[i]) == 1 and int(X.stride0s[i]) == 1
+                  and int(F.shape1s[i]) == 1 and int(F.stride0s[i]) == 1)
+        b = outputs.get((int(X.starts[i]), int(X.shape0s[i]))) if simple and vector else None
+        if b is None:
+            rest.append(i)
+            continue
+        na = int(A.shape0s[i])
+        a0 = np.float32(a_host[i][0, 0]) if na else np.float32(0)
+        b0 = np.float32(b_host[i][0, 0])
+        targets_of.setdefault(b, []).append(
+            (int(F.starts[i]), int(a0.view(np.int32)), int(b0.view(np.int32)), na))
+    if not targets_of:
+        return None
+    # a fused filter's output must be nothing the product reads or writes
+    fused = [i for i in range(len(X)) if i not in set(rest)]
+    written = [iv for iv in (_span(F, i) for i in fused) if iv]
+    touched = []
+    if F.ptr.value == SX.ptr.value:
+        touched += [iv for iv in (_span(SX, b) for b in range(len(SX))) if iv]
+    if F.ptr.value == Y.ptr.value:
+        touched += [iv for iv in (_span(Y, b) for b in range(len(Y))) if iv]
+    if _overlaps(written, touched):
+        return None
+
+    first, target_rows = {}, []
+    for b, rows in sorted(targets_of.items()):
+        first[b] = (len(target_rows), len(rows))
+        target_rows.extend(rows)
+    slice_epi = np.zeros((sp["n"], 4), dtype=np.int32)
+    for k, (item, _, _, _, _, row0) in enumerate(sp["slice_rows"]):
+        if item in first:
+            slice_epi[k] = (first[item][0], first[item][1], row0, 0)
+    dev_epi = to_device(queue, slice_epi)
+    dev_targets = to_device(queue, np.array(target_rows, dtype=np.int32))
+    mask = sp["mask"]
+    args = tuple(spmv_plan.args[:7]) + (dev_epi.ptr, dev_targets.ptr, F.ptr, sp["x_start"],
+                                        sp["n_cols"], mask.ptr if mask is not None else None)
+    plan = Plan(queue, queue.lib.nhip_spmv_sell_filter, args, gsize=spmv_plan.gsize,
+                lsize=spmv_plan.lsize,
+                full_args=tuple(spmv_plan.full_args) + (dev_epi, dev_targets, F.dev_buf),
+                name="hip_spmv_filter", tag=spmv_plan.tag)
+    f_bytes = sum(8 * int(Y.shape0s[b]) * len(rows) for b, rows in targets_of.items())
+    plan.flops_per_call = spmv_plan.flops_per_call
+    plan.bw_per_call = spmv_plan.bw_per_call + f_bytes  # filter state in and out
+    plan.stored_bytes = spmv_plan.stored_bytes
+    plan.description = spmv_plan.description
+    plan.skips_zero_x = spmv_plan.skips_zero_x
+    residual = []
+    if rest:
+        residual = plan_linearfilter(queue, X[rest], F[rest], A[rest], B[rest],
+                                     spec["Xbuf"][rest], spec["Ybuf"][rest], tag=lf_plan.tag)
+        residual[0].unfused_items = list(rest)
+    return [plan], residual

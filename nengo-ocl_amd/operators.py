@@ -317,6 +317,38 @@ def fuse_into_multidotinc(operators):
     return fused
 
 
+class SparseDotSet(ir.Operator):
+    """``Y = A @ X`` with a sparse matrix signal A: what ``Reset(Y, 0)`` followed by a
+    ``SparseDotInc`` into Y is when nothing else writes Y."""
+
+    def __init__(self, A, X, Y, tag=None):
+        super().__init__(tag)
+        self.A, self.X, self.Y = A, X, Y
+        self.sets, self.reads = [Y], [A, X]
+
+
+def sparse_products_set_their_target(operators):
+    """``Reset(y, 0); SparseDotInc(y += A x)`` with no other writer of y becomes
+    `SparseDotSet` (``y = A x``): one launch and one pass over y less per step.  The sum of a
+    row starts from +0.0 either way, so the result has the same bits."""
+    sets, incs, _, updates = signal_io_dicts(operators)
+    drop, replace = set(), {}
+    for op in operators:
+        if not _is(op, "SparseDotInc") or op.Y.is_view:
+            continue
+        base = op.Y.base
+        resets = [w for w in sets[base] if _is(w, "Reset")]
+        if (len(sets[base]) != 1 or len(resets) != 1 or len(incs[base]) != 1
+                or incs[base][0] is not op or updates[base]):
+            continue
+        reset = resets[0]
+        if reset.dst.is_view or float(reset.value) != 0.0:
+            continue
+        drop.add(id(reset))
+        replace[id(op)] = SparseDotSet(op.A, op.X, op.Y, tag=getattr(op, "tag", None))
+    return [replace.get(id(op), op) for op in operators if id(op) not in drop]
+
+
 def neurons_read_constant_input(operators, keep=()):
     """Neurons whose input current is only ever a copy of a constant (an ensemble
     without incoming connections: J = bias every step) read that constant directly,

@@ -86,6 +86,7 @@ class HipBackend:
             self.carry_sequences = hipra_sequence.carry_sequences
         self.plans_conflict = hipra_sequence._conflict
         self.fuse_gemv_filter = hipra_gemv.fuse_linearfilter
+        self.fuse_spmv_filter = hipra_spmv.fuse_linearfilter
 
     def fuse_input_sums(self, sum_plan, lif_plan):
         """The plan replacing ``[sum_plan, lif_plan]`` when the first only forms vector
@@ -293,6 +294,7 @@ class Simulator:
         operators = list(map(MultiDotInc.convert_to, operators))
         if fuse:
             operators = ops_mod.fuse_into_multidotinc(operators)
+            operators = ops_mod.sparse_products_set_their_target(operators)
             operators = ops_mod.neurons_read_constant_input(operators, keep=probed)
             if learn_in_place:
                 operators = ops_mod.apply_learning_in_place(operators, keep=probed)
@@ -475,7 +477,9 @@ class Simulator:
                 continue
             i = j - 2
             between = []  # plans the fused filters would move ahead of
-            while i >= 0 and not hasattr(plans[i], "prog"):
+            producer = lambda p: hasattr(p, "prog") or (
+                hasattr(p, "spmv") and hasattr(self.backend, "fuse_spmv_filter"))
+            while i >= 0 and not producer(plans[i]):
                 if not hasattr(plans[i], "enqueue"):
                     i = -1
                     break
@@ -484,9 +488,12 @@ class Simulator:
             if i < 0:
                 continue
             lo = i
-            while lo > 0 and getattr(plans[lo - 1], "prog", None) is plans[i].prog:
-                lo -= 1
-            result = self.backend.fuse_gemv_filter(plans[lo:i + 1], lf)
+            if hasattr(plans[i], "spmv"):
+                result = self.backend.fuse_spmv_filter(plans[i], lf)
+            else:
+                while lo > 0 and getattr(plans[lo - 1], "prog", None) is plans[i].prog:
+                    lo -= 1
+                result = self.backend.fuse_gemv_filter(plans[lo:i + 1], lf)
             if result is None:
                 continue
             fused, residual = result
@@ -856,7 +863,10 @@ class Simulator:
                                             beta, Y, Y_in=Y_in, gamma=gamma, tag=tag)
         return prog.plans
 
-    def _plan_SparseDotInc(self, ops):
+    def _plan_SparseDotSet(self, ops):
+        return self._plan_SparseDotInc(ops, inc=False)
+
+    def _plan_SparseDotInc(self, ops, inc=True):
         """All sparse products of the group in one launch (the reference plans one
         launch per operator, simulator.py:877-892)."""
         matrices = []
@@ -872,7 +882,7 @@ class Simulator:
                       if type(op2).__name__ == "SimNeurons"
                       and type(op2.neurons).__name__ in SPIKING_NEURON_TYPES}
             extra["x_mostly_zero"] = [op.X.base in spikes for op in ops]
-        return self.backend.plan_sparse_dot_inc(self.queue, matrices, X, Y, inc=True, **extra).plans
+        return self.backend.plan_sparse_dot_inc(self.queue, matrices, X, Y, inc=inc, **extra).plans
 
     def _plan_TimeUpdate(self, ops):
         (op,) = ops

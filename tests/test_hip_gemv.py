@@ -912,6 +912,64 @@ def test_sparse_products_pass_over_zero_operands(queue, rng, inc, density):
     assert not plain.plans[0].skips_zero_x
 
 
+@pytest.mark.parametrize("mostly_zero", [False, True])
+def test_sparse_products_with_filter_epilogue(queue, mostly_zero):
+    """Sparse product + the first-order filters on its output in one launch, for both
+    sparse kernels: two matrices reading one X, two filters and a pure gain on the first
+    output, none on the second, a second-order filter that keeps a launch of its own; every
+    product and filter output equals the oracle's separate kernels bit for bit over steps."""
+    import scipy.sparse as sp
+
+    from nengo_ocl_amd import hipra_nonlinearities as nl
+    from nengo_ocl_amd import hipra_spmv
+    from nengo_ocl_amd.raggedarray import RaggedArray
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(11)
+    n_cols, rows = 5000, [3001, 257]
+    mats = [sp.random(m, n_cols, density=0.01, random_state=rng, format="csr", dtype=np.float32)
+            for m in rows]
+    lowpass = lambda tau: (np.array([-np.exp(-0.001 / tau)]), np.array([1 - np.exp(-0.001 / tau)]))
+    filters = [(0,) + lowpass(0.1), (0,) + lowpass(0.005), (0, np.zeros(0), np.array([0.25])),
+               (0, np.array([-1.2, 0.4]), np.array([0.1, 0.1]))]
+    f_out = [rng.normal(size=rows[b]) for b, _, _ in filters]
+    R = RA([np.zeros(n_cols)] + [np.zeros(m) for m in rows] + f_out, align=True)
+    iY, iF = [1, 2], list(range(3, 3 + len(filters)))
+    den = RaggedArray([np.asarray(f[1], dtype=np.float32).reshape(-1, 1) if f[1].size
+                       else np.zeros((0, 1), dtype=np.float32) for f in filters], dtype=np.float32)
+    num = RaggedArray([np.asarray(f[2], dtype=np.float32).reshape(-1, 1) for f in filters],
+                      dtype=np.float32)
+    xbuf = RaggedArray([np.zeros((f[2].size, rows[f[0]]), dtype=np.float32) for f in filters],
+                       dtype=np.float32)
+    ybuf = RaggedArray([np.zeros((f[1].size, rows[f[0]]), dtype=np.float32) for f in filters],
+                       dtype=np.float32)
+    fx = [iY[b] for b, _, _ in filters]
+
+    def build(ra, spmv, mod_nl, q, up, **kw):
+        prog = spmv(q, mats, ra[[0, 0]], ra[iY], inc=False, **kw)
+        lf = mod_nl.plan_linearfilter(q, ra[fx], ra[iF], up(den), up(num), up(clone(xbuf)),
+                                      up(clone(ybuf)))
+        return prog, lf
+
+    host, dev = clone(R), to_dev(queue, R)
+    prog, lf = build(dev, hipra_spmv.plan_sparse_dot_inc, nl, queue, lambda a: to_dev(queue, a),
+                     x_mostly_zero=mostly_zero)
+    assert prog.plans[0].skips_zero_x == mostly_zero
+    fused, residual = hipra_spmv.fuse_linearfilter(prog.plans[0], lf[0])
+    assert [p.name for p in fused] == ["hip_spmv_filter"]
+    assert [p.name for p in residual] == ["hip_linearfilter"] and residual[0].unfused_items == [3]
+    oprog, olf = build(host, orc.plan_sparse_dot_inc, orc, None, lambda a: a)
+    for step in range(4):
+        v = np.where(rng.uniform(size=n_cols) < 0.1, rng.normal(size=n_cols), 0.0)
+        dev[0] = v
+        host[0] = v[:, None]
+        for p in fused + residual:
+            p()
+        for p in oprog.plans + olf:
+            p()
+        assert np.array_equal(dev.to_host().buf.view(np.uint32), host.buf.view(np.uint32)), step
+
+
 def test_gemv_lif_forms_its_input_sums(queue):
     """Sums of vectors -> encoders -> LIF in one launch: inputs that are sums of one to
     eleven vectors times scalars (64, 40 and 8 elements), an ensemble whose input is a

@@ -519,3 +519,39 @@ def test_planning_is_reproducible(seed):
             schedules.append([(t.__name__, [where[op] for op in ops]) for t, ops in sim.op_groups])
         gc.collect()
     assert schedules[0] == schedules[1] == schedules[2]
+
+
+def test_sparse_product_sets_its_target():
+    """Reset + one sparse product into a vector become a product that sets it (same bits,
+    one operator group less); two products into one vector keep their Reset."""
+    import scipy.sparse
+
+    make = lambda: configs.c5_sparse_recurrent(n_neurons=2000, fan_outs=20, weight_scale=5e-4)
+    runs = []
+    for fuse in (True, False):
+        net, probes, _ = make()
+        with OracleSimulator(net, seed=1, fuse=fuse) as sim:
+            kinds = [type(op).__name__ for op in sim.operators]
+            assert ("SparseDotSet" in kinds) == fuse and ("SparseDotInc" in kinds) == (not fuse)
+            if fuse:
+                assert "Reset" not in kinds
+            sim.run_steps(300)
+            runs.append({k: np.array(sim.data[p]) for k, p in probes.items()})
+            runs[-1]["signals"] = {b.name: np.array(sim.signals[b]) for b in sim.all_bases
+                                   if b.name and b.name.endswith(".weighted")}
+    assert np.any(runs[0]["spikes"] != 0)
+    assert np.array_equal(runs[0]["spikes"], runs[1]["spikes"])
+    for name, value in runs[0]["signals"].items():
+        assert np.array_equal(value.view(np.uint32), runs[1]["signals"][name].view(np.uint32)), name
+
+    from nengo_ocl_amd import ir, operators
+
+    x, y = ir.Signal(np.ones(70), name="x"), ir.Signal(np.zeros(50), name="y")
+    mats = [ir.SparseSignal(scipy.sparse.random(50, 70, density=0.2, random_state=k), name="w%d" % k)
+            for k in range(2)]
+    two = [ir.Reset(y), ir.SparseDotInc(mats[0], x, y), ir.SparseDotInc(mats[1], x, y)]
+    assert operators.sparse_products_set_their_target(two) == two
+    one = operators.sparse_products_set_their_target(two[:2])
+    assert [type(op).__name__ for op in one] == ["SparseDotSet"]
+    half = [ir.Reset(y, value=0.5), ir.SparseDotInc(mats[0], x, y)]  # not a reset to zero
+    assert operators.sparse_products_set_their_target(half) == half

@@ -471,7 +471,10 @@ def test_sparse_recurrent_population(queue):
     net, probes, info = make()
     net_o, probes_o, _ = make()
     with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
-        assert any(p.name == "hip_spmv" for p in gpu._plans)
+        # the product passes over zero operands (spikes) and steps the synapse behind its rows
+        sparse = [p for p in gpu._plans if p.name == "hip_spmv_filter"]
+        assert len(sparse) == 1 and sparse[0].skips_zero_x
+        assert not any(p.name == "hip_reset" for p in gpu._plans)
         gpu.run_steps(1000)
         cpu.run_steps(1000)
         assert np.array_equal(gpu.data[probes["spikes"]], cpu.data[probes_o["spikes"]])
