@@ -462,7 +462,8 @@ class Sigmoid(LIFRate):
         self.amplitude = 1.0
 
     def rates_from_current(self, J):
-        return 1.0 / (self.tau_ref * (1.0 + np.exp(-np.asarray(J, dtype=np.float64))))
+        with np.errstate(over="ignore"):  # exp(-J) = inf for very negative J: a rate of 0
+            return 1.0 / (self.tau_ref * (1.0 + np.exp(-np.asarray(J, dtype=np.float64))))
 
     def gain_bias(self, max_rates, intercepts):
         max_rates = np.asarray(max_rates, dtype=np.float64)
