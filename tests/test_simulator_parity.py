@@ -340,6 +340,7 @@ def _graph_cases():
         "c1": lambda: configs.c1_circconv(dims=8, n_per_dim=30),
         "c4": lambda: configs.c4_pes(n_triples=3, n_neurons=100, dims=4),
         "c3": lambda: configs.c3_large(n_ens=6, n_neurons=256, dims=16, fan_out=2),
+        "c5": lambda: configs.c5_sparse_recurrent(n_neurons=3000, fan_outs=30, weight_scale=5e-4),
     }
 
 
@@ -349,7 +350,7 @@ BRANCHES_OFF = ("recording a step as parallel graph branches is switched off: th
                 "raises NotImplementedError")
 
 
-@pytest.mark.parametrize("case", ["c2", "c1", "c4", "c3"])
+@pytest.mark.parametrize("case", ["c2", "c1", "c4", "c3", "c5"])
 @pytest.mark.parametrize("with_branches", [False, pytest.param(True, marks=pytest.mark.skip(
     reason=BRANCHES_OFF))], ids=["chain", "branches"])
 def test_graph_replay_equals_eager(queue, case, with_branches):
