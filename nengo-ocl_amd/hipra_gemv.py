@@ -40,6 +40,8 @@ TILE_STAGE_WORDS = int(os.environ.get("NENGO_HIP_TILE_WORDS", 2176))
 MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,3.5,3,2.5,2,1.5,1").split(","))  # row blocks per task, tried in order
+# items of the launch that visits only the columns with x != 0 (csrc/gemv_events.hip)
+EVENT_MIN_COLS, EVENT_MAX_COLS, EVENT_MIN_ELEMS = 512, 4096, 16384
 TASK_OVERHEAD_BYTES = 8192.0  # what starting and finishing a task costs, in streamed bytes
 # The large-item kernel with compile-time shapes takes dot products of STREAM_MIN_COLS
 # columns or more whose rows are 16-byte aligned; its LDS block has STREAM_STAGE_WORDS words.
@@ -139,9 +141,13 @@ class gemv_prog:
     force_scalar = False  # one lane per output, 4-byte loads (the plain fallback)
 
     def __init__(self, queue, alpha, A, A_js, X, X_js, beta, Y, Y_in=None, gamma=0.0, tag=None,
-                 tile_items=()):
+                 tile_items=(), event_items=()):
         self.queue = queue
         self.tile_items = frozenset(tile_items)  # items that take the large-item kernel regardless
+        # items whose X is mostly zero (spikes) and whose A nothing ever writes: candidates
+        # for the launch that only visits the columns with x != 0 (`_event_item`)
+        self.event_items = frozenset(event_items)
+        self._host_A_cache = None
         self._many_thin_rows = False
         self.A, self.A_js, self.X, self.X_js = A, A_js, X, X_js
         self.Y = Y
@@ -239,6 +245,8 @@ class gemv_prog:
         n_sum = sum(d["a_shape1"] for d in dots)
         if self.force_scalar:
             return (1, 1, 1)
+        if self.force_flavor is None and self._event_item(g):
+            return (4, 0, 4)
         vec = 4
         if n_max < 4 or any(d["a_start"] % 4 or (d["a_stride0"] % 4 and M > 1) for d in dots):
             vec = 1
@@ -297,6 +305,65 @@ class gemv_prog:
         else:
             lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         return (flavor, lpr, vec)
+
+    def _event_item(self, g):
+        """Does item `g` take the launch that visits only the columns with x != 0?  One
+        dot product of `EVENT_MIN_COLS` to `EVENT_MAX_COLS` columns and at most 64 rows, a
+        contiguous X, enough elements to be a large item, and the caller's word that X is
+        mostly zero and A constant."""
+        if g["index"] not in self.event_items or len(g["dots"]) != 1:
+            return False
+        d = g["dots"][0]
+        return (1 <= g["y_len"] <= WAVE and EVENT_MIN_COLS <= d["a_shape1"] <= EVENT_MAX_COLS
+                and g["y_len"] * d["a_shape1"] >= EVENT_MIN_ELEMS
+                and (d["x_stride0"] == 1 or d["a_shape1"] == 1))
+
+    def _host_A(self):
+        if self._host_A_cache is None:
+            self._host_A_cache = self.A.to_host()
+        return self._host_A_cache
+
+    def _event_plan(self, members):
+        """The launch of `nhip_gemv_events` for `members`: their matrices transposed into a
+        device buffer of their own (column c of an item: `mp` consecutive floats)."""
+        queue, geometry = self.queue, self.geometry
+        host = self._host_A()
+        rows, parts, cursor = [], [], 0
+        for b in members:
+            g = geometry[b]
+            d = g["dots"][0]
+            M, N = g["y_len"], d["a_shape1"]
+            mp = -(-M // 16) * 16
+            block = np.asarray(host[d["a_j"]], dtype=np.float32).reshape(M, N)
+            t = np.zeros((N, mp), dtype=np.float32)
+            t[:, :M] = block.T
+            coefs = np.array([self.alpha[b], self.beta[b], self.gamma[b]], dtype=np.float32)
+            rows.append((cursor, mp, M, N, d["x_start"], g["y_start"], g["y_stride0"],
+                         g["y_in_start"], g["y_in_stride0"]) + tuple(coefs.view(np.int32).tolist())
+                        + (0, 0, 0, 0))
+            parts.append(t.ravel())
+            cursor += N * mp
+        if cursor >= 2 ** 31:
+            raise ValueError("more than 2^31 elements of transposed matrices")
+        table = np.array(rows, dtype=np.int32)
+        dev_items = to_device(queue, table)
+        dev_at = to_device(queue, np.concatenate(parts))
+        n = len(members)
+        args = (dev_items.ptr, n, dev_at.ptr, self.X.ptr, self.Y_in.ptr, self.Y.ptr, None, None)
+        plan = Plan(queue, queue.lib.nhip_gemv_events, args, gsize=(1024 * n,), lsize=(1024,),
+                    full_args=(dev_items, dev_at, self.X.dev_buf, self.Y_in.dev_buf, self.Y.dev_buf),
+                    name="hipra_gemv.events", tag="%s-events" % self.tag,
+                    bw_per_call=bw_from_geometry(geometry, members),
+                    flops_per_call=flops_from_geometry(geometry, members))
+        plan.description = self.geometry_summary(members)
+        plan.kernel_class = (4, 0, 4)
+        plan.n_tasks = n
+        plan.members = list(members)
+        plan.prog = self
+        plan.host_tasks = None
+        plan.event_table = table
+        plan.event_driven = True  # reads only the columns of A whose x is not zero
+        return plan
 
     def _tile_tasks(self, members, max_rows=256, stream=False, row_multiple=1):
         """Tasks (item, first row, rows, 0) of the reference-order kernel for large items.
@@ -405,6 +472,9 @@ class gemv_prog:
         plans = []
         for cls, members in sorted(by_class.items()):
             flavor, lpr, vec = cls[:3]
+            if flavor == 4:
+                plans.append(self._event_plan(members))
+                continue
             passes = cls[3] if len(cls) > 3 else 0  # 0 = the class default
             if flavor == 3:
                 rows = None  # per item, below
@@ -564,6 +634,12 @@ def _takes_epilogue(plan):
     """Reference-order launches (large or small items) that do not have an epilogue yet."""
     return (plan.name in ("hipra_gemv.tile", "hipra_gemv.wave_ref")
             and getattr(plan, "kernel_class", (None,))[0] in (2, 3))
+
+
+def _takes_filters(plan):
+    """Launches that can step first-order filters on their fresh rows."""
+    return _takes_epilogue(plan) or (plan.name == "hipra_gemv.events"
+                                     and getattr(plan, "kernel_class", (None,))[0] == 4)
 
 
 def _epilogue_call(lib, plan, kind, extras=None):
@@ -926,7 +1002,7 @@ def fuse_linearfilter(gemv_plans, lf_plan):
         return None
     large = {}
     for plan in gemv_plans:
-        if _takes_epilogue(plan):
+        if _takes_filters(plan):
             for b in plan.members:
                 if int(Y.stride0s[b]) == 1:
                     large[(int(Y.starts[b]), int(Y.shape0s[b]))] = b
@@ -967,11 +1043,32 @@ def fuse_linearfilter(gemv_plans, lf_plan):
     extra = (dev_items.ptr, dev_targets.ptr, F.ptr)
     out = []
     for plan in gemv_plans:
-        if not _takes_epilogue(plan) or not any(b in targets_of for b in plan.members):
+        if not _takes_filters(plan) or not any(b in targets_of for b in plan.members):
             out.append(plan)
             continue
         f_bytes = sum(8 * int(Y.shape0s[b]) * len(targets_of[b]) for b in plan.members
                       if b in targets_of)  # filter state in and out
+        if plan.kernel_class[0] == 4:
+            # the launch that visits only the columns with x != 0: an item's range of
+            # targets goes into its record
+            table = plan.event_table.copy()
+            table[:, 12:14] = item_targets[plan.members]
+            dev_table = to_device(queue, table)
+            fused = Plan(queue, lib.nhip_gemv_events,
+                         (dev_table.ptr,) + tuple(plan.args[1:6]) + (dev_targets.ptr, F.ptr),
+                         gsize=plan.gsize, lsize=plan.lsize,
+                         full_args=plan.full_args + (dev_table, dev_targets, F.dev_buf),
+                         name=plan.name + "_filter", tag=plan.tag,
+                         bw_per_call=plan.bw_per_call + f_bytes,
+                         flops_per_call=plan.flops_per_call)
+            fused.description = plan.description
+            fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
+            fused.members, fused.prog = plan.members, prog
+            fused.gemv_bytes = plan.bw_per_call
+            fused.event_table, fused.event_driven = table, True
+            fused.host_tasks = None
+            out.append(fused)
+            continue
         entry, args, keep = _epilogue_call(
             lib, plan, "filter",
             lambda items: np.column_stack([item_targets[items], np.zeros(len(items), np.int32)]))

@@ -204,14 +204,16 @@ def merge_small_plans(plans):
 
 
 def _can_carry(plan):
-    """GEMV launches with an epilogue: the large-item kernel with compile-time shapes, and
-    the small-item kernel."""
+    """GEMV launches with an epilogue: the large-item kernel with compile-time shapes, the
+    launch that visits only the columns with x != 0, and the small-item kernel."""
     cls = getattr(plan, "kernel_class", None)
     name = getattr(plan, "name", "")
     if cls is None or getattr(plan, "prelude", None) is not None or getattr(plan, "n_tasks", 0) <= 0:
         return False
     if name in ("hipra_gemv.tile_lif", "hipra_gemv.tile_filter"):
         return cls[0] == 3 and cls[1] >= 2
+    if name in ("hipra_gemv.events", "hipra_gemv.events_filter"):
+        return cls[0] == 4
     return name in ("hipra_gemv.wave_ref", "hipra_gemv.wave_ref_lif",
                     "hipra_gemv.wave_ref_filter") and cls[0] == 2
 

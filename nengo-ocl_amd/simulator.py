@@ -81,6 +81,8 @@ class HipBackend:
         self.plan_sparse_dot_inc = hipra_spmv.plan_sparse_dot_inc
         # switch for measurements: "0" multiplies every stored element of a sparse matrix
         self.skips_zero_operands = os.environ.get("NENGO_HIP_SPMV_SKIP", "1") != "0"
+        # switch for measurements: "0" multiplies every column of a matrix applied to spikes
+        self.event_driven_products = os.environ.get("NENGO_HIP_EVENT_GEMV", "1") != "0"
         self.merge_small_plans = hipra_sequence.merge_small_plans
         if os.environ.get("NENGO_HIP_CARRY_SEQUENCES", "1") != "0":  # switch for measurements
             self.carry_sequences = hipra_sequence.carry_sequences
@@ -840,16 +842,30 @@ class Simulator:
         constant_bs = [op for op in ops if op._float_beta is not None]
         if len(constant_bs) != len(ops):
             raise NotImplementedError("signal-valued beta")
+        extra = {}
+        if getattr(self.backend, "event_driven_products", False):
+            # products of a constant matrix with the spikes of a population: only the columns
+            # of the neurons that spiked need to be visited
+            spikes = {op2.output.base for op2 in self.operators
+                      if type(op2).__name__ == "SimNeurons"
+                      and type(op2.neurons).__name__ in SPIKING_NEURON_TYPES}
+            written = {s.base for op2 in self.operators
+                       for s in list(op2.sets) + list(op2.incs) + list(op2.updates)}
+            constant = lambda sig: getattr(sig.base, "readonly", False) and sig.base not in written
+            extra["event_items"] = [
+                k for k, op in enumerate(constant_bs)
+                if len(self._A_views[op]) == 1 and self._X_views[op][0].base in spikes
+                and constant(self._A_views[op][0])]
         return self._sig_gemv(
             constant_bs,
             lambda op: self._A_views[op], lambda op: self._X_views[op],
             lambda op: self._YYB_views[op][0], lambda op: self._YYB_views[op][1],
             beta=[op._float_beta for op in constant_bs],
             gamma=[op.gamma for op in constant_bs],
-            tag="c-beta-%d" % len(constant_bs))
+            tag="c-beta-%d" % len(constant_bs), **extra)
 
     def _sig_gemv(self, ops, A_js_fn, X_js_fn, Y_fn, Y_in_fn=None, alpha=1.0, beta=1.0,
-                  gamma=0.0, tag=None):
+                  gamma=0.0, tag=None, **extra):
         if len(ops) == 0:
             return []
         all_data, sidx = self.all_data, self.sidx
@@ -860,7 +876,7 @@ class Simulator:
         Y = all_data[[sidx[s] for s in Y_sigs]]
         Y_in = all_data[[sidx[s] for s in Y_in_sigs]]
         prog = self.backend.plan_block_gemv(self.queue, alpha, all_data, A_js, all_data, X_js,
-                                            beta, Y, Y_in=Y_in, gamma=gamma, tag=tag)
+                                            beta, Y, Y_in=Y_in, gamma=gamma, tag=tag, **extra)
         return prog.plans
 
     def _plan_SparseDotSet(self, ops):

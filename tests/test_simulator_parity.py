@@ -159,8 +159,9 @@ def test_c3_large_reduced_spiking(queue, dedup):
         # the neurons are updated by the GEMV that computes their input current
         assert any(p.name == "hipra_gemv.tile_lif" for p in gpu._plans)
         assert not any(p.name == "hip_lif" for p in gpu._plans)
-        # and the synapse filters by the GEMV that decodes their input
-        assert any(p.name == "hipra_gemv.tile_filter" for p in gpu._plans)
+        # and the synapse filters by the GEMV that decodes their input (the one that
+        # visits only the columns of the neurons that spiked)
+        assert any(p.name == "hipra_gemv.events_filter" for p in gpu._plans)
         check_spiking(gpu, cpu, pg["spikes"], pc["spikes"], 1000, "c3 reduced (8 x 1024 x 64-D)")
 
 
@@ -181,13 +182,13 @@ def test_c3_full_size_state_bit_exact(queue):
         names = [p.name for p in gpu._plans]
         # input sums + encoders + neurons; decoders + synapses, with clock / input / probes
         # riding in groups of their own
-        assert sorted(names) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_lif"]
-        assert [p.carried.name for p in gpu._plans if p.name == "hipra_gemv.tile_filter"] == [
+        assert sorted(names) == ["hipra_gemv.events_filter", "hipra_gemv.tile_lif"]
+        assert [p.carried.name for p in gpu._plans if p.name == "hipra_gemv.events_filter"] == [
             "hip_sequence"]
         assert [p.input_sums for p in gpu._plans if p.name == "hipra_gemv.tile_lif"] == [254]
         classes = {p.name: p.kernel_class for p in gpu._plans if hasattr(p, "kernel_class")}
         assert classes["hipra_gemv.tile_lif"] == (3, 3, 4)     # compile-time shapes, narrow
-        assert classes["hipra_gemv.tile_filter"] == (3, 2, 4)  # compile-time shapes, wide
+        assert classes["hipra_gemv.events_filter"] == (4, 0, 4)  # columns of spiking neurons only
         gpu.run_steps(40)
         cpu.run_steps(40)
         for key in probes:
@@ -210,7 +211,7 @@ def test_merged_products_keep_every_signal(queue):
     model = net.build_model(dt=0.001)
     with Simulator(None, model=model, seed=1) as a, \
             Simulator(None, model=model, seed=1, dedup=False) as b:
-        assert sorted(p.name for p in a._plans) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_lif"]
+        assert sorted(p.name for p in a._plans) == ["hipra_gemv.events_filter", "hipra_gemv.tile_lif"]
         assert a.all_data.buf.size < b.all_data.buf.size
         a.run_steps(200)
         b.run_steps(200)
@@ -224,24 +225,29 @@ def test_merged_products_keep_every_signal(queue):
 def test_launch_fusions_change_nothing(queue, monkeypatch):
     """Input sums formed inside the encoder launch and the short operations of a step
     carried by the decoder launch, against the same model with each as a launch of its
-    own: four launches per step become two, every signal and probe sample stays
-    bit-identical (eager and as a recorded graph), and a failed carry is reported."""
+    own, and decoders that visit only the columns of the neurons that spiked against decoders
+    that multiply every column: four launches per step become two, every signal and probe
+    sample stays bit-identical (eager and as a recorded graph), and a failed carry is
+    reported."""
     from nengo_ocl_amd import _lib, configs
     from nengo_ocl_amd.simulator import Simulator
 
     net, probes, _ = configs.c3_large(n_ens=8, n_neurons=1024, dims=64, fan_out=4)
     model = net.build_model(dt=0.001)
     sims = []
-    for sums, carry, graph in (("1", "1", True), ("1", "1", False), ("0", "0", True)):
+    for sums, carry, graph, events in (("1", "1", True, "1"), ("1", "1", False, "1"),
+                                       ("0", "0", True, "1"), ("1", "1", True, "0")):
         monkeypatch.setenv("NENGO_HIP_INPUT_SUMS", sums)
         monkeypatch.setenv("NENGO_HIP_CARRY_SEQUENCES", carry)
+        monkeypatch.setenv("NENGO_HIP_EVENT_GEMV", events)
         sims.append(Simulator(None, model=model, seed=1, use_graph=graph))
-    a, eager, plain = sims
-    with a, eager, plain:
-        assert [len(s._plans) for s in sims] == [2, 2, 4]
+    a, eager, plain, dense = sims
+    with a, eager, plain, dense:
+        assert [len(s._plans) for s in sims] == [2, 2, 4, 2]
+        assert sorted(p.name for p in dense._plans) == ["hipra_gemv.tile_filter", "hipra_gemv.tile_lif"]
         for s in sims:
             s.run_steps(100)
-        for other in (eager, plain):
+        for other in (eager, plain, dense):
             for p in probes.values():
                 assert np.array_equal(a.data[p], other.data[p]) and np.any(a.data[p] != 0)
             assert np.array_equal(np.asarray(a.all_data.buf), np.asarray(other.all_data.buf))
