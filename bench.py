@@ -217,6 +217,42 @@ def traffic_floor(queue, n_rows, cols, n_reads=3, n_writes=4, repeats=60):
     return out
 
 
+def event_driven_report(sim, event_rows, steps_per_s, make_sim, args):
+    """What the launches that visit only the columns with x != 0 were given to do: the
+    fraction of neurons that spiked in the last step, their algorithmic bytes (which they do
+    not read), and the same simulation with every column multiplied, timed briefly."""
+    import numpy as np
+
+    spiking = [op.output for op in sim.operators if type(op).__name__ == "SimNeurons"]
+    n = sum(int(np.asarray(sim.signals[s]).size) for s in spiking)
+    nz = sum(int(np.count_nonzero(np.asarray(sim.signals[s]))) for s in spiking)
+    out = {"plans": [r["plan"] for r in event_rows],
+           "avg_us": sum(r["avg_us"] for r in event_rows),
+           "algorithmic_bytes_per_step": sum(r["bytes"] for r in event_rows),
+           "note": "these launches read only the columns of their matrices whose x is not zero "
+                   "(results bit-identical to the dense product); their algorithmic bytes are "
+                   "not traffic and are left out of gemv_all",
+           "neurons_that_spiked_in_the_last_step": nz / max(n, 1)}
+    os.environ["NENGO_HIP_EVENT_GEMV"] = "0"
+    try:
+        dense = make_sim()
+        steps = min(max(args.steps, 20), 400)
+        dense.run_steps(args.warmup)
+        dense.run_steps(max(dense._plans.steps_of_every_graph(), 1))
+        dense.queue.finish()
+        t0 = time.perf_counter()
+        dense.run_steps(steps)
+        dense.queue.finish()
+        dt = time.perf_counter() - t0
+        dense.close()
+        out["every_column_multiplied"] = {"steps_per_s": steps / dt, "ms_per_step": 1e3 * dt / steps,
+                                          "steps": steps, "flag": "--dense-decoders"}
+    finally:
+        os.environ.pop("NENGO_HIP_EVENT_GEMV", None)
+    out["speedup_over_every_column"] = steps_per_s / out["every_column_multiplied"]["steps_per_s"]
+    return out
+
+
 def micro_benchmarks(repeats=50):
     """Kernels that no benchmark network exercises, each on one representative problem:
     one JSON line per kernel with its average duration (start / stop events carried by
@@ -351,6 +387,9 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="fraction of the ensembles (c3, c4)")
     ap.add_argument("--profile-steps", type=int, default=100)
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
+    ap.add_argument("--dense-decoders", action="store_true",
+                    help="multiply every column of the matrices applied to spike vectors "
+                         "(default: only the columns of the neurons that spiked are visited)")
     ap.add_argument("--no-fuse", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--two-pass-learning", action="store_true",
@@ -382,10 +421,14 @@ def main():
 
     from nengo_ocl_amd.simulator import Simulator
 
+    if args.dense_decoders:
+        os.environ["NENGO_HIP_EVENT_GEMV"] = "0"
     t0 = time.time()
     (net, probes, _), workload = make_network(args.config, args.variant, args.scale)
-    sim = Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph,
-                    learn_in_place=not args.two_pass_learning, dedup=args.variant == "shared")
+    make_sim = lambda: Simulator(net, seed=1, fuse=not args.no_fuse, use_graph=not args.no_graph,
+                                 learn_in_place=not args.two_pass_learning,
+                                 dedup=args.variant == "shared")
+    sim = make_sim()
     build_s = time.time() - t0
     n_plans = len(sim._plans)
 
@@ -414,7 +457,17 @@ def main():
     steps_per_s = args.steps / elapsed
 
     rows = gemv_summary(sim, args.profile_steps)
-    gemv_rows = [r for r in rows if r["name"].startswith("hipra_gemv") and r["bytes"]]
+    # launches that visit only the columns of the neurons that spiked do not read their
+    # algorithmic bytes: they are reported apart, without a rate
+    event_plans = {str(p) for p in sim._plans if getattr(p, "event_driven", False)}
+    event_rows = [r for r in rows if r["plan"] in event_plans]
+    for r in event_rows:
+        r["gbs"] = None
+    gemv_rows = [r for r in rows if r["name"].startswith("hipra_gemv") and r["bytes"]
+                 and r["plan"] not in event_plans]
+    if event_rows:
+        workload += ("; matrices applied to spikes are read only in the columns of the neurons "
+                     "that spiked (--dense-decoders reads them whole)")
     dom = max(gemv_rows, key=lambda r: r["avg_us"]) if gemv_rows else None
     step_us_kernels = sum(r["avg_us"] for r in rows)
     gemv_bytes = sum(r["bytes"] for r in gemv_rows)
@@ -465,11 +518,14 @@ def main():
         "config": {"workload": workload, "neurons": net.n_neurons, "plans_per_step": n_plans,
                    "dt": 0.001, "graph": not args.no_graph,
                    "fused_copies": not args.no_fuse, "learn_in_place": not args.two_pass_learning,
-                   "identical_products_merged": args.variant == "shared"},
+                   "identical_products_merged": args.variant == "shared",
+                   "products_with_spikes_visit_active_columns_only": bool(event_rows)},
         "roofline": roofline,
         "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,
                      "gbs": 1e-3 * gemv_bytes / gemv_us if gemv_us else None,
                      "frac_of_peak": (1e-3 * gemv_bytes / gemv_us / HBM_PEAK_GBS) if gemv_us else None},
+        "event_driven": event_driven_report(sim, event_rows, steps_per_s, make_sim, args)
+        if event_rows else None,
         "kernels": [{"plan": r["plan"], "avg_us": round(r["avg_us"], 2),
                      "gbs": None if r["gbs"] is None else round(r["gbs"], 1)} for r in rows],
         "kernel_us_per_step": step_us_kernels,

@@ -42,6 +42,7 @@ TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,3.5,3,2.5,2,1.5,1").split(","))  # row blocks per task, tried in order
 # items of the launch that visits only the columns with x != 0 (csrc/gemv_events.hip)
 EVENT_MIN_COLS, EVENT_MAX_COLS, EVENT_MIN_ELEMS = 512, 4096, 16384
+EVENT_MIN_SPLIT_BYTES = 64 << 20  # matrix bytes that pay for a launch next to a dense one
 TASK_OVERHEAD_BYTES = 8192.0  # what starting and finishing a task costs, in streamed bytes
 # The large-item kernel with compile-time shapes takes dot products of STREAM_MIN_COLS
 # columns or more whose rows are 16-byte aligned; its LDS block has STREAM_STAGE_WORDS words.
@@ -147,6 +148,7 @@ class gemv_prog:
         # items whose X is mostly zero (spikes) and whose A nothing ever writes: candidates
         # for the launch that only visits the columns with x != 0 (`_event_item`)
         self.event_items = frozenset(event_items)
+        self._events_off = False
         self._host_A_cache = None
         self._many_thin_rows = False
         self.A, self.A_js, self.X, self.X_js = A, A_js, X, X_js
@@ -311,7 +313,7 @@ class gemv_prog:
         dot product of `EVENT_MIN_COLS` to `EVENT_MAX_COLS` columns and at most 64 rows, a
         contiguous X, enough elements to be a large item, and the caller's word that X is
         mostly zero and A constant."""
-        if g["index"] not in self.event_items or len(g["dots"]) != 1:
+        if self._events_off or g["index"] not in self.event_items or len(g["dots"]) != 1:
             return False
         d = g["dots"][0]
         return (1 <= g["y_len"] <= WAVE and EVENT_MIN_COLS <= d["a_shape1"] <= EVENT_MAX_COLS
@@ -448,6 +450,19 @@ class gemv_prog:
         for b in items:
             if geometry[b]["y_len"] > 0:
                 by_class[self._item_class(geometry[b])].append(b)
+        # visiting only the columns with x != 0 is a launch of its own: next to a launch of
+        # large items that stays anyway it must save more than it costs
+        events = by_class.get((4, 0, 4), [])
+        if events and any(c[0] == 3 for c in by_class) and 4 * sum(
+                geometry[b]["y_len"] * geometry[b]["dots"][0]["a_shape1"]
+                for b in events) < EVENT_MIN_SPLIT_BYTES:
+            del by_class[(4, 0, 4)]
+            self._events_off = True
+            for b in events:
+                by_class[self._item_class(geometry[b])].append(b)
+            self._events_off = False
+            for members in by_class.values():
+                members.sort()
 
         # the one instance of the compile-time-shape kernel that holds the stage widths of
         # all of them takes the items of several instances

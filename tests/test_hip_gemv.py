@@ -971,7 +971,7 @@ def test_sparse_products_with_filter_epilogue(queue, mostly_zero):
 
 
 @pytest.mark.parametrize("activity", [0.0, 0.08, 1.0])
-def test_products_with_spike_vectors_visit_active_columns_only(queue, activity):
+def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, monkeypatch):
     """Items flagged as "X mostly zero, A constant" take the launch that reads only the
     columns of A whose x is not zero (matrices transposed on the device): 64 x 4096,
     32 x 2000 (columns no multiple of the tile), 64 x 512, 19 x 1000, with coefficients;
@@ -1002,6 +1002,11 @@ def test_products_with_spike_vectors_visit_active_columns_only(queue, activity):
     flagged = [0, 1, 2, 3, 4, 5, 6]
 
     host, dev = clone(R), to_dev(queue, R)
+    # a few MB of matrices next to a dense launch that stays: not worth a launch of its own
+    prog = g.plan_block_gemv(queue, alpha, dev, A_js, dev, X_js, beta, dev[iY], gamma=gamma,
+                             event_items=flagged)
+    assert not any(p.name == "hipra_gemv.events" for p in prog.plans)
+    monkeypatch.setattr(g, "EVENT_MIN_SPLIT_BYTES", 0)
     prog = g.plan_block_gemv(queue, alpha, dev, A_js, dev, X_js, beta, dev[iY], gamma=gamma,
                              event_items=flagged)
     events = [p for p in prog.plans if p.name == "hipra_gemv.events"]
