@@ -290,6 +290,7 @@ class Simulator:
         all_operators = list(self.model.operators)
         probed = [self.model.sig[p]["in"] for p in self.model.probes]
         self.signal_aliases = {}  # signal dropped as a duplicate -> the one computed
+        self._copied_constants = set()  # constants that launches read from a copy of their own
         operators = ops_mod.simplify_operators(
             all_operators, keep=probed, aliases=self.signal_aliases,
             skip=() if dedup else ("merge_identical_chains",))
@@ -627,6 +628,11 @@ class Simulator:
 
             def __setitem__(self, item, val):
                 incoming = np.asarray(val)
+                if item.base in sim._copied_constants:
+                    raise ValueError(
+                        "%s is a constant whose device copy in another layout would go stale; "
+                        "build the simulator with NENGO_HIP_EVENT_GEMV=0 to change it at run "
+                        "time" % (item,))
                 if item.ndim == 0:
                     assert incoming.size == 1
                     sim.all_data[sim.sidx[item]] = incoming
@@ -877,6 +883,11 @@ class Simulator:
         Y_in = all_data[[sidx[s] for s in Y_in_sigs]]
         prog = self.backend.plan_block_gemv(self.queue, alpha, all_data, A_js, all_data, X_js,
                                             beta, Y, Y_in=Y_in, gamma=gamma, tag=tag, **extra)
+        for plan in prog.plans:
+            if getattr(plan, "event_driven", False):
+                # these matrices have a second, transposed copy on the device
+                self._copied_constants.update(
+                    sig.base for b in plan.members for sig in A_js_fn(ops[b]))
         return prog.plans
 
     def _plan_SparseDotSet(self, ops):

@@ -686,3 +686,26 @@ def test_graph_branches_are_switched_off(queue):
     net, _, _ = configs.c0_readme(n_neurons=20)
     with pytest.raises(NotImplementedError, match="switched off"):
         Simulator(net, seed=1, branches=True)
+
+
+@pytest.mark.gpu
+def test_constants_with_a_transposed_copy_cannot_be_set(queue, monkeypatch):
+    """Decoders that the device also keeps transposed (for the launch that visits only the
+    columns of the neurons that spiked) refuse to be overwritten from the host; without that
+    launch they can be."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+
+    net, probes, _ = configs.c3_large(n_ens=4, n_neurons=1024, dims=16, fan_out=2)
+    model = net.build_model(dt=0.001)
+    with Simulator(None, model=model, seed=1) as sim:
+        assert any(getattr(p, "event_driven", False) for p in sim._plans)
+        weights = sorted(sim._copied_constants, key=lambda s: str(s.name))[0]
+        with pytest.raises(ValueError, match="another layout"):
+            sim.signals[weights] = np.zeros(weights.shape)
+    monkeypatch.setenv("NENGO_HIP_EVENT_GEMV", "0")
+    with Simulator(None, model=model, seed=1) as sim:
+        assert not sim._copied_constants
+        sim.signals[weights] = np.zeros(weights.shape)
+        sim.run_steps(20)
+        assert not np.any(np.asarray(sim.signals[weights]))
