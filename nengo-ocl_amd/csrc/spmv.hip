@@ -20,6 +20,7 @@
 // go to the cache, which spares it one look-up per line and instruction.
 #include "nhip_common.h"
 #include "neuron_math.h"
+#include "sequence_ops.h"
 
 namespace {
 
@@ -31,6 +32,27 @@ struct SpmvEpi {
     const FilterTarget* targets;
     float* F;
 };
+
+// A sequence armed with nhip_gemv_tile_carry rides in extra work-groups behind those of the
+// product (256 threads run a chain; further waves of such a group end at once: a barrier
+// waits for the waves that are still running).
+struct SpmvSide {
+    const NhipSeqOp* ops;
+    SeqChains chains;
+    int n_chains;       // 0: none
+    int n_groups;       // groups of the product itself
+};
+
+__device__ __forceinline__ void spmv_side_chain(const SpmvSide& side, void* lds) {
+    if (threadIdx.x >= NHIP_WG) return;
+    const int c = blockIdx.x - side.n_groups;
+    NhipSeqOp* s_ops = reinterpret_cast<NhipSeqOp*>(lds);
+    int (*s_rows)[SEQ_ROW_WORDS] = reinterpret_cast<int (*)[SEQ_ROW_WORDS]>(
+        reinterpret_cast<char*>(lds) + SEQ_MAX_OPS * sizeof(NhipSeqOp));
+    sequence_chain(side.ops + side.chains.first_op[c],
+                   side.chains.first_op[c + 1] - side.chains.first_op[c], side.chains.n_staged[c],
+                   s_ops, s_rows, threadIdx.x);
+}
 
 __device__ __forceinline__ void spmv_filter_rows(const SpmvEpi& epi, int s, int lane, float y) {
     const int4 e = epi.slice_epi[s];
@@ -61,11 +83,14 @@ typedef float spmv_f4 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(NHIP_WG) void spmv_sell_kernel(
     const SpmvSlice* __restrict__ slices, int n_slices, const int* __restrict__ row_len,
     const int* __restrict__ cols, const float* __restrict__ vals, const float* X, float* Y,
-    SpmvEpi epi)
+    SpmvEpi epi, SpmvSide side)
 {
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int s = blockIdx.x * (NHIP_WG / NHIP_WAVE) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     __shared__ __attribute__((aligned(16))) float s_x[NHIP_WG / NHIP_WAVE][SPMV_WINDOW];
+    static_assert(sizeof(s_x) >= SEQ_MAX_OPS * sizeof(NhipSeqOp) + sizeof(int) * SEQ_MAX_ROWS * SEQ_ROW_WORDS,
+                  "a carried sequence stages its records in the same LDS");
+    if (side.n_chains > 0 && (int)blockIdx.x >= side.n_groups) return spmv_side_chain(side, s_x);
     // waves past the last slice have no work but still meet the group barrier below
     const bool has_slice = s < n_slices;
     SpmvSlice sl = slices[has_slice ? s : 0];
@@ -144,16 +169,17 @@ __global__ __launch_bounds__(NHIP_WG) void spmv_mask_kernel(const float* __restr
 __global__ __launch_bounds__(SPMV_SKIP_WG) void spmv_sell_skip_kernel(
     const SpmvSlice* __restrict__ slices, int n_slices, const int* __restrict__ row_len,
     const int* __restrict__ cols, const float* __restrict__ vals, const float* X, float* Y,
-    const unsigned* __restrict__ mask, int n_mask_quads, SpmvEpi epi)
+    const unsigned* __restrict__ mask, int n_mask_quads, SpmvEpi epi, SpmvSide side)
 {
     constexpr int U = SPMV_SKIP_U;
     __shared__ __attribute__((aligned(16))) unsigned s_mask[SPMV_MASK_WORDS];
+    if (side.n_chains > 0 && (int)blockIdx.x >= side.n_groups) return spmv_side_chain(side, s_mask);
     for (int i = threadIdx.x; i < n_mask_quads; i += SPMV_SKIP_WG)
         reinterpret_cast<spmv_i4*>(s_mask)[i] = reinterpret_cast<const spmv_i4*>(mask)[i];
     __syncthreads();  // the only barrier; every thread reaches it
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int stride = gridDim.x * (SPMV_SKIP_WG / NHIP_WAVE);
+    const int stride = side.n_groups * (SPMV_SKIP_WG / NHIP_WAVE);
     for (int s = blockIdx.x * (SPMV_SKIP_WG / NHIP_WAVE) + wave; s < n_slices; s += stride) {
         const SpmvSlice sl = slices[s];
         const bool live = lane < sl.n_rows;
@@ -214,19 +240,35 @@ __global__ __launch_bounds__(SPMV_SKIP_WG) void spmv_sell_skip_kernel(
     }
 }
 
+// a sequence armed by nhip_gemv_tile_carry is the calling launch's, whatever becomes of it
+SpmvSide take_side() {
+    SpmvSide side{};
+    const NhipCarried armed = nhip_carried;
+    nhip_carried = NhipCarried{};
+    if (armed.n_chains > 0) {
+        side.ops = static_cast<const NhipSeqOp*>(armed.ops);
+        for (int c = 0; c <= NHIP_SEQ_MAX_CHAINS; ++c) side.chains.first_op[c] = armed.first_op[c];
+        for (int c = 0; c < NHIP_SEQ_MAX_CHAINS; ++c) side.chains.n_staged[c] = armed.n_staged[c];
+        side.n_chains = armed.n_chains;
+    }
+    return side;
+}
+
 int launch_plain(void* stream, const int* slices, int n_slices, const int* row_len,
                  const int* cols, const float* vals, const float* X, float* Y, SpmvEpi epi) {
-    if (n_slices == 0) return 0;
+    SpmvSide side = take_side();
+    if (n_slices == 0) return side.n_chains > 0 ? NHIP_E_BADARG : 0;  // nothing to ride in
     if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y) return NHIP_E_BADARG;
     // the kernel reads `cols`, `vals` and the runs of X it keeps in LDS 16 bytes at a time
     if ((reinterpret_cast<uintptr_t>(cols) | reinterpret_cast<uintptr_t>(vals) |
          reinterpret_cast<uintptr_t>(X)) & 15)
         return NHIP_E_BADARG;
     const int wpg = NHIP_WG / NHIP_WAVE;
-    NHIP_LAUNCH(spmv_sell_kernel, dim3((n_slices + wpg - 1) / wpg), dim3(NHIP_WG), 0,
+    side.n_groups = (n_slices + wpg - 1) / wpg;
+    NHIP_LAUNCH(spmv_sell_kernel, dim3(side.n_groups + side.n_chains), dim3(NHIP_WG), 0,
                        static_cast<hipStream_t>(stream),
                        reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X,
-                       Y, epi);
+                       Y, epi, side);
     NHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -235,7 +277,8 @@ int launch_plain(void* stream, const int* slices, int n_slices, const int* row_l
 int launch_skip(void* stream, const int* slices, int n_slices, const int* row_len,
                 const int* cols, const float* vals, const float* X, float* Y, int x_start,
                 int n_cols, unsigned* mask, SpmvEpi epi) {
-    if (n_slices == 0) return 0;
+    SpmvSide side = take_side();
+    if (n_slices == 0) return side.n_chains > 0 ? NHIP_E_BADARG : 0;  // nothing to ride in
     if (n_slices < 0 || !slices || !row_len || !cols || !vals || !X || !Y || !mask || x_start < 0 ||
         n_cols <= 0)
         return NHIP_E_BADARG;
@@ -258,10 +301,10 @@ int launch_skip(void* stream, const int* slices, int n_slices, const int* row_le
         n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     }
     const int wpg = SPMV_SKIP_WG / NHIP_WAVE;
-    const int n_groups = min(n_cu, (n_slices + wpg - 1) / wpg);
-    NHIP_LAUNCH(spmv_sell_skip_kernel, dim3(n_groups), dim3(SPMV_SKIP_WG), 0, s,
+    side.n_groups = min(n_cu, (n_slices + wpg - 1) / wpg);
+    NHIP_LAUNCH(spmv_sell_skip_kernel, dim3(side.n_groups + side.n_chains), dim3(SPMV_SKIP_WG), 0, s,
                 reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X, Y,
-                mask, n_mask_quads, epi);
+                mask, n_mask_quads, epi, side);
     NHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -205,9 +205,12 @@ def merge_small_plans(plans):
 
 def _can_carry(plan):
     """GEMV launches with an epilogue: the large-item kernel with compile-time shapes, the
-    launch that visits only the columns with x != 0, and the small-item kernel."""
+    launch that visits only the columns with x != 0, the small-item kernel, and the sparse
+    products."""
     cls = getattr(plan, "kernel_class", None)
     name = getattr(plan, "name", "")
+    if name in ("hip_spmv", "hip_spmv_filter"):  # the sparse products (one or more slices)
+        return getattr(plan, "prelude", None) is None and getattr(plan, "spmv", {}).get("n", 0) > 0
     if cls is None or getattr(plan, "prelude", None) is not None or getattr(plan, "n_tasks", 0) <= 0:
         return False
     if name in ("hipra_gemv.tile_lif", "hipra_gemv.tile_filter"):

@@ -240,6 +240,7 @@ def fuse_linearfilter(spmv_plan, lf_plan):
     plan.stored_bytes = spmv_plan.stored_bytes
     plan.description = spmv_plan.description
     plan.skips_zero_x = spmv_plan.skips_zero_x
+    plan.spmv = spmv_plan.spmv
     residual = []
     if rest:
         residual = plan_linearfilter(queue, X[rest], F[rest], A[rest], B[rest],
