@@ -249,8 +249,8 @@ int nhip_spmv_sell(void *stream, const int *slices, int n_slices, const int *row
                    const int *cols, const float *vals, const float *X, float *Y);
 
 /* Y[b] = beta[b] Y_in[b] + alpha[b] A[b] X[b] + gamma[b] for items with one dot product,
- * at most 64 rows and at most 4096 columns whose X is mostly zero (decoders applied to the
- * spikes of a population): `plan_block_gemv` (clra_gemv.py:861-1175) restricted to such
+ * and at most 64 rows whose X is mostly zero (decoders applied to the spikes of a
+ * population): `plan_block_gemv` (clra_gemv.py:861-1175) restricted to such
  * items, visiting only the columns whose x is not zero -- in the reference's order, with its
  * operations, so the result is that of nhip_gemv_tile (a running sum that underflows to -0
  * aside) -- and reading only those columns of A.  For that the matrices are handed over
@@ -261,9 +261,12 @@ int nhip_spmv_sell(void *stream, const int *slices, int n_slices, const int *row
  *   AT    : the transposed matrices; X, Yin, Y: the buffers the offsets refer to
  *   targets, F : first-order filters stepped on the fresh y, as for nhip_gemv_tile_filter
  *           (both NULL: none); an item's range of targets is in its record
- * One work-group per item.  A sequence armed with nhip_gemv_tile_carry rides in the launch. */
+ * max_cols: the largest N of the items (when it says 4096 or less, only the first 4096
+ * columns of every item are visited).  One work-group per item.  A sequence armed with nhip_gemv_tile_carry rides in
+ * the launch. */
 int nhip_gemv_events(void *stream, const int *items, int n_items, const float *AT,
-                     const float *X, const float *Yin, float *Y, const int *targets, float *F);
+                     const float *X, const float *Yin, float *Y, const int *targets, float *F,
+                     int max_cols);
 
 /* The same product for an X that is mostly zero (the spikes of a population; no
  * counterpart in the reference, whose kernels multiply every stored element).  All slices

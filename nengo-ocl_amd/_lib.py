@@ -39,7 +39,7 @@ SIGNATURES = {
     "nhip_gemv_rows_lif_sums": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
                                 P, ctypes.c_double, c_int, P, P, P, P, P, P, P, P],
     "nhip_gemv_rows_filter": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P, P, P, P],
-    "nhip_gemv_events": [P, P, c_int, P, P, P, P, P, P],
+    "nhip_gemv_events": [P, P, c_int, P, P, P, P, P, P, c_int],
     "nhip_spmv_sell": [P, P, c_int, P, P, P, P, P],
     "nhip_spmv_sell_skip": [P, P, c_int, P, P, P, P, P, c_int, c_int, P],
     "nhip_spmv_sell_filter": [P, P, c_int, P, P, P, P, P, P, P, P, c_int, c_int, P],

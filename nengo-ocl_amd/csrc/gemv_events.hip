@@ -14,11 +14,13 @@
 // kept transposed in a buffer of their own: column c of an item is `mp` consecutive floats
 // (one per row), so a wave reads a column with one coalesced load, lane r holding row r.
 //
-// One work-group per item.  Each of its sixteen waves takes a share of the tiles: it lists the
+// One work-group per item, 4096 columns at a time (almost always the whole item).  Each of
+// its sixteen waves takes a share of the tiles: it lists the
 // columns of its range with x != 0 in LDS (ballot and prefix count, so the list is in
 // column order), then walks the list EV_BATCH columns at a time -- the loads of a batch are
 // issued together -- and leaves alpha * tile sum of every tile in LDS.  After a barrier the
-// first wave adds the tiles in order, stores y and steps the filters that read it.
+// first wave adds the tiles in order; after the last run of columns it stores y and steps the
+// filters that read it.
 // A sequence armed with nhip_gemv_tile_carry rides in extra work-groups, as in the other
 // GEMV launches with an epilogue.
 #include "nhip_common.h"
@@ -28,7 +30,7 @@
 
 namespace {
 
-constexpr int EV_MAX_COLS = 4096;   // columns of an item (the lists of a group: 32 KiB of LDS)
+constexpr int EV_MAX_COLS = 4096;   // columns taken at a time (the lists of a group: 32 KiB of LDS)
 constexpr int EV_TILE = 128;        // the reference's tile width
 constexpr int EV_WG = 1024;         // sixteen waves per item: a wave's list is short, its loads few
 constexpr int EV_WAVES = EV_WG / NHIP_WAVE;
@@ -39,7 +41,7 @@ constexpr int EV_BATCH = 32;
 struct EvItem {  // 16 words
     int at_start;      // column c of the transposed matrix: AT[at_start + c * mp + row]
     int mp;            // floats between columns (>= M)
-    int M, N;          // rows (<= 64), columns (<= EV_MAX_COLS)
+    int M, N;          // rows (<= 64), columns
     int x_start;       // X is contiguous
     int y_start, y_stride0, yin_start, yin_stride0;
     float alpha, beta, gamma;
@@ -60,6 +62,8 @@ struct EvLds {
     float tile[EV_MAX_TILES][NHIP_WAVE];
 };
 
+// MULTI: some item of the launch has more than EV_MAX_COLS columns
+template <bool MULTI>
 __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
     const EvItem* __restrict__ items, int n_items, const float* __restrict__ AT, const float* X,
     const float* Yin, float* Y, FilterArgs filter, EvSide side)
@@ -84,13 +88,6 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
     const int lane = threadIdx.x & (NHIP_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const EvItem it = items[blockIdx.x];
-    const int n_tiles = (it.N + EV_TILE - 1) / EV_TILE;
-    const int tiles_per_wave = (n_tiles + EV_WAVES - 1) / EV_WAVES;
-    const int t_lo = min(wave * tiles_per_wave, n_tiles);
-    const int t_hi = min(t_lo + tiles_per_wave, n_tiles);
-    const int c_lo = t_lo * EV_TILE, c_hi = min(t_hi * EV_TILE, it.N);
-    const float empty_tile = it.alpha * ((0.0f + 0.0f) + (0.0f + 0.0f));
-    for (int t = t_lo; t < t_hi; ++t) lds.tile[t][lane] = empty_tile;
     // what the first wave needs at the end is requested now: the old y and the state of the
     // first filter (no branch around the loads: a lane without a row reads the first one's)
     const int row = min(lane, it.M - 1);
@@ -103,91 +100,108 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
             f_old = filter.F[(size_t)f_first.y_start + row];
         }
     }
-
-    // the columns of this wave's range whose x is not zero, in column order
+    const float empty_tile = it.alpha * ((0.0f + 0.0f) + (0.0f + 0.0f));
+    const float* x = X + it.x_start;
+    const float* at = AT + it.at_start + row;
     int* col = lds.col[wave];
     float* xs = lds.x[wave];
-    int count = 0;
-    const float* x = X + it.x_start;
-    for (int c0 = c_lo; c0 < c_hi; c0 += 4 * NHIP_WAVE) {
-        float xv[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int c = c0 + u * NHIP_WAVE + lane;
-            xv[u] = c < c_hi ? x[c] : 0.0f;
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const bool nz = (__float_as_uint(xv[u]) & 0x7fffffffu) != 0u;
-            const unsigned long long b = __ballot(nz);
-            const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(b >> 32),
-                                                         __builtin_amdgcn_mbcnt_lo((unsigned)b, 0));
-            if (nz) {
-                col[count + before] = c0 + u * NHIP_WAVE + lane;
-                xs[count + before] = xv[u];
-            }
-            count += __popcll(b);
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float sum = it.beta * y_old;  // (the first wave's; the tiles are added onto it in order)
 
-    // walk the list: the loads of EV_BATCH columns together, then their multiply-adds in order
-    const float* at = AT + it.at_start + row;
-    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
-    int cur = -1;  // the tile the running sums belong to
-    for (int k = 0; k < count; k += EV_BATCH) {
-        float a[EV_BATCH];
-        int cc[EV_BATCH];
+    // EV_MAX_COLS columns at a time: almost always the whole item
+    int base = 0;
+    do {
+        const int n_cols = min(it.N - base, EV_MAX_COLS);
+        const int n_tiles = (n_cols + EV_TILE - 1) / EV_TILE;
+        const int tiles_per_wave = (n_tiles + EV_WAVES - 1) / EV_WAVES;
+        const int t_lo = min(wave * tiles_per_wave, n_tiles);
+        const int t_hi = min(t_lo + tiles_per_wave, n_tiles);
+        const int c_lo = t_lo * EV_TILE, c_hi = min(t_hi * EV_TILE, n_cols);  // relative to base
+        for (int t = t_lo; t < t_hi; ++t) lds.tile[t][lane] = empty_tile;
+
+        // the columns of this wave's range whose x is not zero, in column order
+        int count = 0;
+        for (int c0 = c_lo; c0 < c_hi; c0 += 4 * NHIP_WAVE) {
+            float xv[4];
 #pragma unroll
-        for (int u = 0; u < EV_BATCH; ++u) {
-            cc[u] = col[min(k + u, count - 1)];
-            a[u] = at[(size_t)cc[u] * it.mp];
-        }
+            for (int u = 0; u < 4; ++u) {
+                const int c = c0 + u * NHIP_WAVE + lane;
+                xv[u] = c < c_hi ? x[base + c] : 0.0f;
+            }
 #pragma unroll
-        for (int u = 0; u < EV_BATCH; ++u) {
-            if (k + u < count) {  // the same for all lanes
-                const int c = __builtin_amdgcn_readfirstlane(cc[u]);
-                const float xv = xs[k + u];
-                const int t = c >> 7;
-                if (t != cur) {
-                    if (cur >= 0) lds.tile[cur][lane] = it.alpha * ((s0 + s2) + (s1 + s3));
-                    cur = t;
-                    s0 = s1 = s2 = s3 = 0.0f;
+            for (int u = 0; u < 4; ++u) {
+                const bool nz = (__float_as_uint(xv[u]) & 0x7fffffffu) != 0u;
+                const unsigned long long b = __ballot(nz);
+                const int before = __builtin_amdgcn_mbcnt_hi(
+                    (unsigned)(b >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b, 0));
+                if (nz) {
+                    col[count + before] = c0 + u * NHIP_WAVE + lane;
+                    xs[count + before] = xv[u];
                 }
-                switch (c & 3) {
-                    case 0: s0 = fmaf(a[u], xv, s0); break;
-                    case 1: s1 = fmaf(a[u], xv, s1); break;
-                    case 2: s2 = fmaf(a[u], xv, s2); break;
-                    default: s3 = fmaf(a[u], xv, s3); break;
-                }
+                count += __popcll(b);
             }
         }
-    }
-    if (cur >= 0) lds.tile[cur][lane] = it.alpha * ((s0 + s2) + (s1 + s3));
-    __syncthreads();  // every thread of an item's group arrives here exactly once
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-    if (wave == 0) {
-        float tv[EV_MAX_TILES];
+        // walk the list: the loads of EV_BATCH columns together, then their multiply-adds
+        // in order
+        float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+        int cur = -1;  // the tile the running sums belong to
+        for (int k = 0; k < count; k += EV_BATCH) {
+            float a[EV_BATCH];
+            int cc[EV_BATCH];
 #pragma unroll
-        for (int t = 0; t < EV_MAX_TILES; ++t) tv[t] = lds.tile[t][lane];  // (all reads at once)
-        float sum = it.beta * y_old;
+            for (int u = 0; u < EV_BATCH; ++u) {
+                cc[u] = col[min(k + u, count - 1)];
+                a[u] = at[(size_t)(base + cc[u]) * it.mp];
+            }
 #pragma unroll
-        for (int t = 0; t < EV_MAX_TILES; ++t)
-            if (t < n_tiles) sum = sum + tv[t];
+            for (int u = 0; u < EV_BATCH; ++u) {
+                if (k + u < count) {  // the same for all lanes
+                    const int c = __builtin_amdgcn_readfirstlane(cc[u]);
+                    const float xv = xs[k + u];
+                    const int t = c >> 7;
+                    if (t != cur) {
+                        if (cur >= 0) lds.tile[cur][lane] = it.alpha * ((s0 + s2) + (s1 + s3));
+                        cur = t;
+                        s0 = s1 = s2 = s3 = 0.0f;
+                    }
+                    switch (c & 3) {
+                        case 0: s0 = fmaf(a[u], xv, s0); break;
+                        case 1: s1 = fmaf(a[u], xv, s1); break;
+                        case 2: s2 = fmaf(a[u], xv, s2); break;
+                        default: s3 = fmaf(a[u], xv, s3); break;
+                    }
+                }
+            }
+        }
+        if (cur >= 0) lds.tile[cur][lane] = it.alpha * ((s0 + s2) + (s1 + s3));
+        __syncthreads();  // the tiles of this run of columns are in LDS
+
+        if (wave == 0) {
+            float tv[EV_MAX_TILES];
+#pragma unroll
+            for (int t = 0; t < EV_MAX_TILES; ++t) tv[t] = lds.tile[t][lane];  // (all reads at once)
+#pragma unroll
+            for (int t = 0; t < EV_MAX_TILES; ++t)
+                if (t < n_tiles) sum = sum + tv[t];
+        }
+        base += EV_MAX_COLS;
+        if (MULTI && base < it.N) __syncthreads();  // ... and read, before the next run
+    } while (MULTI && base < it.N);
+
+    if (wave == 0 && lane < it.M) {
         const float y = sum + it.gamma;
-        if (lane < it.M) {
-            Y[(size_t)it.y_start + (size_t)lane * it.y_stride0] = y;
-            if (it.n_targets > 0) {
-                // the first filter from what was requested at the start, the others as usual
-                // (the arithmetic of filter_epilogue: rounded products, rounded subtract)
-                const float bx = __fmul_rn(nhip_bits(f_first.b_bits), y);
-                filter.F[(size_t)f_first.y_start + lane] =
-                    f_first.na ? __fsub_rn(bx, __fmul_rn(nhip_bits(f_first.a_bits), f_old)) : bx;
-                if (it.n_targets > 1)
-                    filter_epilogue(filter, make_int2(it.first_target + 1, it.n_targets - 1), lane, y);
-            }
+        Y[(size_t)it.y_start + (size_t)lane * it.y_stride0] = y;
+        if (it.n_targets > 0) {
+            // the first filter from what was requested at the start, the others as usual
+            // (the arithmetic of filter_epilogue: rounded products, rounded subtract)
+            const float bx = __fmul_rn(nhip_bits(f_first.b_bits), y);
+            filter.F[(size_t)f_first.y_start + lane] =
+                f_first.na ? __fsub_rn(bx, __fmul_rn(nhip_bits(f_first.a_bits), f_old)) : bx;
+            if (it.n_targets > 1)
+                filter_epilogue(filter, make_int2(it.first_target + 1, it.n_targets - 1), lane, y);
         }
     }
 }
@@ -196,12 +210,12 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
 
 extern "C" int nhip_gemv_events(void* stream, const int* items, int n_items, const float* AT,
                                 const float* X, const float* Yin, float* Y,
-                                const int* targets, float* F) {
+                                const int* targets, float* F, int max_cols) {
     // a sequence armed by nhip_gemv_tile_carry is this launch's, whatever becomes of it
     const NhipCarried armed = nhip_carried;
     nhip_carried = NhipCarried{};
     if (n_items == 0) return armed.n_chains > 0 ? NHIP_E_BADARG : 0;  // nothing to ride in
-    if (n_items < 0 || !items || !AT || !X || !Yin || !Y) return NHIP_E_BADARG;
+    if (n_items < 0 || !items || !AT || !X || !Yin || !Y || max_cols <= 0) return NHIP_E_BADARG;
     if ((targets == nullptr) != (F == nullptr)) return NHIP_E_BADARG;
     EvSide side{};
     if (armed.n_chains > 0) {
@@ -213,9 +227,13 @@ extern "C" int nhip_gemv_events(void* stream, const int* items, int n_items, con
     FilterArgs filter{};
     filter.targets = reinterpret_cast<const FilterTarget*>(targets);
     filter.F = F;
-    NHIP_LAUNCH(gemv_events_kernel, dim3(n_items + side.n_chains), dim3(EV_WG), 0,
-                static_cast<hipStream_t>(stream), reinterpret_cast<const EvItem*>(items), n_items,
-                AT, X, Yin, Y, filter, side);
+    auto launch = [&](auto kernel) {
+        NHIP_LAUNCH(kernel, dim3(n_items + side.n_chains), dim3(EV_WG), 0,
+                    static_cast<hipStream_t>(stream), reinterpret_cast<const EvItem*>(items),
+                    n_items, AT, X, Yin, Y, filter, side);
+    };
+    if (max_cols > EV_MAX_COLS) launch(gemv_events_kernel<true>);
+    else launch(gemv_events_kernel<false>);
     NHIP_LAUNCH_CHECK();
     return 0;
 }

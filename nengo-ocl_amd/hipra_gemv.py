@@ -41,7 +41,7 @@ MIN_TILE_TASKS = int(os.environ.get("NENGO_HIP_TILE_MIN_TASKS", 2048))
 TILE_TASK_BLOCKS = tuple(float(v) for v in os.environ.get(
     "NENGO_HIP_TILE_TASK_BLOCKS", "4,3.5,3,2.5,2,1.5,1").split(","))  # row blocks per task, tried in order
 # items of the launch that visits only the columns with x != 0 (csrc/gemv_events.hip)
-EVENT_MIN_COLS, EVENT_MAX_COLS, EVENT_MIN_ELEMS = 512, 4096, 16384
+EVENT_MIN_COLS, EVENT_MAX_COLS, EVENT_MIN_ELEMS = 512, 1 << 20, 16384
 EVENT_MIN_SPLIT_BYTES = 64 << 20  # matrix bytes that pay for a launch next to a dense one
 TASK_OVERHEAD_BYTES = 8192.0  # what starting and finishing a task costs, in streamed bytes
 # The large-item kernel with compile-time shapes takes dot products of STREAM_MIN_COLS
@@ -351,7 +351,8 @@ class gemv_prog:
         dev_items = to_device(queue, table)
         dev_at = to_device(queue, np.concatenate(parts))
         n = len(members)
-        args = (dev_items.ptr, n, dev_at.ptr, self.X.ptr, self.Y_in.ptr, self.Y.ptr, None, None)
+        args = (dev_items.ptr, n, dev_at.ptr, self.X.ptr, self.Y_in.ptr, self.Y.ptr, None, None,
+                int(table[:, 3].max()))
         plan = Plan(queue, queue.lib.nhip_gemv_events, args, gsize=(1024 * n,), lsize=(1024,),
                     full_args=(dev_items, dev_at, self.X.dev_buf, self.Y_in.dev_buf, self.Y.dev_buf),
                     name="hipra_gemv.events", tag="%s-events" % self.tag,
@@ -1070,7 +1071,8 @@ def fuse_linearfilter(gemv_plans, lf_plan):
             table[:, 12:14] = item_targets[plan.members]
             dev_table = to_device(queue, table)
             fused = Plan(queue, lib.nhip_gemv_events,
-                         (dev_table.ptr,) + tuple(plan.args[1:6]) + (dev_targets.ptr, F.ptr),
+                         (dev_table.ptr,) + tuple(plan.args[1:6]) + (dev_targets.ptr, F.ptr,
+                                                                      plan.args[8]),
                          gsize=plan.gsize, lsize=plan.lsize,
                          full_args=plan.full_args + (dev_table, dev_targets, F.dev_buf),
                          name=plan.name + "_filter", tag=plan.tag,

@@ -974,7 +974,8 @@ def test_sparse_products_with_filter_epilogue(queue, mostly_zero):
 def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, monkeypatch):
     """Items flagged as "X mostly zero, A constant" take the launch that reads only the
     columns of A whose x is not zero (matrices transposed on the device): 64 x 4096,
-    32 x 2000 (columns no multiple of the tile), 64 x 512, 19 x 1000, with coefficients;
+    32 x 2000 (columns no multiple of the tile), 64 x 512, 19 x 1000, 16 x 10000 (three runs of
+    columns), with coefficients;
     bit-identical to the oracle's dense product at every activity, with negative zeros and
     denormals in X, over steps in which X changes.  Flagged items that do not fit (more than
     64 rows, two dot products, few columns) and unflagged ones keep the dense kernels, in
@@ -983,7 +984,8 @@ def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, 
     from oracle import oracle as orc
 
     rng = np.random.RandomState(23)
-    shapes = [(64, 4096), (32, 2000), (64, 512), (19, 1000), (100, 4096), (64, 4096), (16, 300)]
+    shapes = [(64, 4096), (32, 2000), (64, 512), (19, 1000), (100, 4096), (64, 4096), (16, 300),
+              (16, 10000)]
     n = len(shapes)
     mats = [rng.normal(scale=0.01, size=s) for s in shapes] + [rng.normal(size=(64, 4096))]
     xs = [np.zeros(s[1]) for s in shapes] + [np.zeros(4096)]
@@ -996,10 +998,10 @@ def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, 
     X_js = [np.array([i], dtype=np.int32) for i in iX[:n]]
     A_js[5] = np.array([iA[5], iA[n]], dtype=np.int32)  # two dot products: stays dense
     X_js[5] = np.array([iX[5], iX[n]], dtype=np.int32)
-    alpha = [1.0, 0.5, 1.0, -2.0, 1.0, 1.0, 1.0]
-    beta = [0.0, 1.0, 0.25, 0.0, 1.0, 0.0, 1.0]
-    gamma = [0.0, 0.0, 0.125, 0.0, 0.0, 0.0, 0.0]
-    flagged = [0, 1, 2, 3, 4, 5, 6]
+    alpha = [1.0, 0.5, 1.0, -2.0, 1.0, 1.0, 1.0, 0.75]
+    beta = [0.0, 1.0, 0.25, 0.0, 1.0, 0.0, 1.0, 1.0]
+    gamma = [0.0, 0.0, 0.125, 0.0, 0.0, 0.0, 0.0, 0.0]
+    flagged = [0, 1, 2, 3, 4, 5, 6, 7]
 
     host, dev = clone(R), to_dev(queue, R)
     # a few MB of matrices next to a dense launch that stays: not worth a launch of its own
@@ -1010,7 +1012,7 @@ def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, 
     prog = g.plan_block_gemv(queue, alpha, dev, A_js, dev, X_js, beta, dev[iY], gamma=gamma,
                              event_items=flagged)
     events = [p for p in prog.plans if p.name == "hipra_gemv.events"]
-    assert len(events) == 1 and events[0].members == [0, 1, 2, 3]
+    assert len(events) == 1 and events[0].members == [0, 1, 2, 3, 7]
     assert sorted(b for p in prog.plans if p.name != "hipra_gemv.events" for b in p.members) == [4, 5, 6]
     oprog = orc.plan_block_gemv(None, alpha, host, A_js, host, X_js, beta, host[iY], gamma=gamma)
     for step in range(3):
