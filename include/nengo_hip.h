@@ -249,20 +249,21 @@ int nhip_spmv_sell(void *stream, const int *slices, int n_slices, const int *row
                    const int *cols, const float *vals, const float *X, float *Y);
 
 /* Y[b] = beta[b] Y_in[b] + alpha[b] A[b] X[b] + gamma[b] for items with one dot product,
- * and at most 64 rows whose X is mostly zero (decoders applied to the spikes of a
- * population): `plan_block_gemv` (clra_gemv.py:861-1175) restricted to such
+ * whose X is mostly zero (decoders and weights applied to the spikes of a population): `plan_block_gemv` (clra_gemv.py:861-1175) restricted to such
  * items, visiting only the columns whose x is not zero -- in the reference's order, with its
  * operations, so the result is that of nhip_gemv_tile (a running sum that underflows to -0
  * aside) -- and reading only those columns of A.  For that the matrices are handed over
  * transposed, in a buffer of their own:
  *   items : int32[n_items][16] {at_start, mp, M, N, x_start, y_start, y_stride0, yin_start,
- *           yin_stride0, bits of alpha, beta, gamma, first_target, n_targets, 0, 0}
- *           column c of item b is AT[at_start + c * mp + row], row < M <= mp
+ *           yin_stride0, bits of alpha, beta, gamma, first_target, n_targets, row0, 0}
+ *           a record stands for rows row0 .. row0 + M - 1 (M <= 64) of a matrix whose
+ *           column c is AT[at_start + c * mp + row]; y_start / yin_start are those of the
+ *           matrix's row 0; a matrix of more than 64 rows is several records
  *   AT    : the transposed matrices; X, Yin, Y: the buffers the offsets refer to
  *   targets, F : first-order filters stepped on the fresh y, as for nhip_gemv_tile_filter
  *           (both NULL: none); an item's range of targets is in its record
  * max_cols: the largest N of the items (when it says 4096 or less, only the first 4096
- * columns of every item are visited).  One work-group per item.  A sequence armed with nhip_gemv_tile_carry rides in
+ * columns of every item are visited).  One work-group per record.  A sequence armed with nhip_gemv_tile_carry rides in
  * the launch. */
 int nhip_gemv_events(void *stream, const int *items, int n_items, const float *AT,
                      const float *X, const float *Yin, float *Y, const int *targets, float *F,

@@ -1,5 +1,5 @@
 // Matrix-vector products whose vector is mostly zero: Y = beta Y_in + alpha A X + gamma for
-// items with one dot product, at most 64 rows and a vector of spikes (decoders: what a
+// items with one dot product and a vector of spikes (decoders: what a
 // population sends on is D s with s zero for every neuron that did not spike in the step).
 //
 // The reference's block kernel (clra_gemv.py:1010-1060 with the reduce kernel :1122-1155)
@@ -14,7 +14,8 @@
 // kept transposed in a buffer of their own: column c of an item is `mp` consecutive floats
 // (one per row), so a wave reads a column with one coalesced load, lane r holding row r.
 //
-// One work-group per item, 4096 columns at a time (almost always the whole item).  Each of
+// One work-group per 64 rows of an item, 4096 columns at a time (almost always the whole
+// item).  Each of
 // its sixteen waves takes a share of the tiles: it lists the
 // columns of its range with x != 0 in LDS (ballot and prefix count, so the list is in
 // column order), then walks the list EV_BATCH columns at a time -- the loads of a batch are
@@ -41,12 +42,13 @@ constexpr int EV_BATCH = 32;
 struct EvItem {  // 16 words
     int at_start;      // column c of the transposed matrix: AT[at_start + c * mp + row]
     int mp;            // floats between columns (>= M)
-    int M, N;          // rows (<= 64), columns
+    int M, N;          // rows of this record (<= 64), columns
     int x_start;       // X is contiguous
-    int y_start, y_stride0, yin_start, yin_stride0;
+    int y_start, y_stride0, yin_start, yin_stride0;  // of the item's first row
     float alpha, beta, gamma;
     int first_target, n_targets;  // filters fed by y (none: 0, 0)
-    int pad0, pad1;
+    int row0;          // first row of this record in its item (items of more than 64 rows
+    int pad1;          // are several records; at_start is that of row 0)
 };
 static_assert(sizeof(EvItem) == 64, "item records are 16 words");
 
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
     const EvItem it = items[blockIdx.x];
     // what the first wave needs at the end is requested now: the old y and the state of the
     // first filter (no branch around the loads: a lane without a row reads the first one's)
-    const int row = min(lane, it.M - 1);
+    const int row = it.row0 + min(lane, it.M - 1);
     float y_old = 0.0f, f_old = 0.0f;
     FilterTarget f_first = {};
     if (wave == 0) {
@@ -193,15 +195,15 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
 
     if (wave == 0 && lane < it.M) {
         const float y = sum + it.gamma;
-        Y[(size_t)it.y_start + (size_t)lane * it.y_stride0] = y;
+        Y[(size_t)it.y_start + (size_t)row * it.y_stride0] = y;
         if (it.n_targets > 0) {
             // the first filter from what was requested at the start, the others as usual
             // (the arithmetic of filter_epilogue: rounded products, rounded subtract)
             const float bx = __fmul_rn(nhip_bits(f_first.b_bits), y);
-            filter.F[(size_t)f_first.y_start + lane] =
+            filter.F[(size_t)f_first.y_start + row] =
                 f_first.na ? __fsub_rn(bx, __fmul_rn(nhip_bits(f_first.a_bits), f_old)) : bx;
             if (it.n_targets > 1)
-                filter_epilogue(filter, make_int2(it.first_target + 1, it.n_targets - 1), lane, y);
+                filter_epilogue(filter, make_int2(it.first_target + 1, it.n_targets - 1), row, y);
         }
     }
 }

@@ -308,16 +308,15 @@ class gemv_prog:
             lpr = min(WAVE, next_pow2(-(-n_max // vec)))
         return (flavor, lpr, vec)
 
-    def _event_item(self, g):
+    def _event_item(self, g, any_size=False):
         """Does item `g` take the launch that visits only the columns with x != 0?  One
-        dot product of `EVENT_MIN_COLS` to `EVENT_MAX_COLS` columns and at most 64 rows, a
-        contiguous X, enough elements to be a large item, and the caller's word that X is
+        dot product of `EVENT_MIN_COLS` to `EVENT_MAX_COLS` columns, a contiguous X, enough elements to be a large item, and the caller's word that X is
         mostly zero and A constant."""
         if self._events_off or g["index"] not in self.event_items or len(g["dots"]) != 1:
             return False
         d = g["dots"][0]
-        return (1 <= g["y_len"] <= WAVE and EVENT_MIN_COLS <= d["a_shape1"] <= EVENT_MAX_COLS
-                and g["y_len"] * d["a_shape1"] >= EVENT_MIN_ELEMS
+        return (g["y_len"] >= 1 and EVENT_MIN_COLS <= d["a_shape1"] <= EVENT_MAX_COLS
+                and (any_size or g["y_len"] * d["a_shape1"] >= EVENT_MIN_ELEMS)
                 and (d["x_stride0"] == 1 or d["a_shape1"] == 1))
 
     def _host_A(self):
@@ -330,7 +329,7 @@ class gemv_prog:
         device buffer of their own (column c of an item: `mp` consecutive floats)."""
         queue, geometry = self.queue, self.geometry
         host = self._host_A()
-        rows, parts, cursor = [], [], 0
+        rows, parts, cursor, record_item = [], [], 0, []
         for b in members:
             g = geometry[b]
             d = g["dots"][0]
@@ -340,9 +339,11 @@ class gemv_prog:
             t = np.zeros((N, mp), dtype=np.float32)
             t[:, :M] = block.T
             coefs = np.array([self.alpha[b], self.beta[b], self.gamma[b]], dtype=np.float32)
-            rows.append((cursor, mp, M, N, d["x_start"], g["y_start"], g["y_stride0"],
-                         g["y_in_start"], g["y_in_stride0"]) + tuple(coefs.view(np.int32).tolist())
-                        + (0, 0, 0, 0))
+            for row0 in range(0, M, WAVE):  # a work-group per 64 rows
+                rows.append((cursor, mp, min(WAVE, M - row0), N, d["x_start"], g["y_start"],
+                             g["y_stride0"], g["y_in_start"], g["y_in_stride0"])
+                            + tuple(coefs.view(np.int32).tolist()) + (0, 0, row0, 0))
+                record_item.append(b)
             parts.append(t.ravel())
             cursor += N * mp
         if cursor >= 2 ** 31:
@@ -350,7 +351,7 @@ class gemv_prog:
         table = np.array(rows, dtype=np.int32)
         dev_items = to_device(queue, table)
         dev_at = to_device(queue, np.concatenate(parts))
-        n = len(members)
+        n = len(rows)
         args = (dev_items.ptr, n, dev_at.ptr, self.X.ptr, self.Y_in.ptr, self.Y.ptr, None, None,
                 int(table[:, 3].max()))
         plan = Plan(queue, queue.lib.nhip_gemv_events, args, gsize=(1024 * n,), lsize=(1024,),
@@ -365,6 +366,7 @@ class gemv_prog:
         plan.prog = self
         plan.host_tasks = None
         plan.event_table = table
+        plan.event_record_item = np.array(record_item, dtype=np.int64)  # Y item of each record
         plan.event_driven = True  # reads only the columns of A whose x is not zero
         return plan
 
@@ -454,6 +456,17 @@ class gemv_prog:
         # visiting only the columns with x != 0 is a launch of its own: next to a launch of
         # large items that stays anyway it must save more than it costs
         events = by_class.get((4, 0, 4), [])
+        if events:
+            # where that launch exists, candidates too small to ask for it join it rather
+            # than keep a launch of large items alive
+            for cls in [c for c in by_class if c[0] == 3]:
+                join = [b for b in by_class[cls] if self._event_item(geometry[b], any_size=True)]
+                if join:
+                    events.extend(join)
+                    by_class[cls] = [b for b in by_class[cls] if b not in set(join)]
+                    if not by_class[cls]:
+                        del by_class[cls]
+            events.sort()
         if events and any(c[0] == 3 for c in by_class) and 4 * sum(
                 geometry[b]["y_len"] * geometry[b]["dots"][0]["a_shape1"]
                 for b in events) < EVENT_MIN_SPLIT_BYTES:
@@ -1068,7 +1081,7 @@ def fuse_linearfilter(gemv_plans, lf_plan):
             # the launch that visits only the columns with x != 0: an item's range of
             # targets goes into its record
             table = plan.event_table.copy()
-            table[:, 12:14] = item_targets[plan.members]
+            table[:, 12:14] = item_targets[plan.event_record_item]
             dev_table = to_device(queue, table)
             fused = Plan(queue, lib.nhip_gemv_events,
                          (dev_table.ptr,) + tuple(plan.args[1:6]) + (dev_targets.ptr, F.ptr,
@@ -1083,6 +1096,7 @@ def fuse_linearfilter(gemv_plans, lf_plan):
             fused.members, fused.prog = plan.members, prog
             fused.gemv_bytes = plan.bw_per_call
             fused.event_table, fused.event_driven = table, True
+            fused.event_record_item = plan.event_record_item
             fused.host_tasks = None
             out.append(fused)
             continue

@@ -977,9 +977,9 @@ def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, 
     32 x 2000 (columns no multiple of the tile), 64 x 512, 19 x 1000, 16 x 10000 (three runs of
     columns), with coefficients;
     bit-identical to the oracle's dense product at every activity, with negative zeros and
-    denormals in X, over steps in which X changes.  Flagged items that do not fit (more than
-    64 rows, two dot products, few columns) and unflagged ones keep the dense kernels, in
-    the same program."""
+    denormals in X, over steps in which X changes; 100 x 4096 as two groups of rows.  Flagged
+    items that do not fit (two dot products, few columns) keep the dense kernels, in the same
+    program."""
     from nengo_ocl_amd import hipra_gemv as g
     from oracle import oracle as orc
 
@@ -1012,8 +1012,9 @@ def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, 
     prog = g.plan_block_gemv(queue, alpha, dev, A_js, dev, X_js, beta, dev[iY], gamma=gamma,
                              event_items=flagged)
     events = [p for p in prog.plans if p.name == "hipra_gemv.events"]
-    assert len(events) == 1 and events[0].members == [0, 1, 2, 3, 7]
-    assert sorted(b for p in prog.plans if p.name != "hipra_gemv.events" for b in p.members) == [4, 5, 6]
+    assert len(events) == 1 and events[0].members == [0, 1, 2, 3, 4, 7]
+    assert events[0].n_tasks == 7  # 100 rows are two records
+    assert sorted(b for p in prog.plans if p.name != "hipra_gemv.events" for b in p.members) == [5, 6]
     oprog = orc.plan_block_gemv(None, alpha, host, A_js, host, X_js, beta, host[iY], gamma=gamma)
     for step in range(3):
         for i in iX:

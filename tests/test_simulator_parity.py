@@ -709,3 +709,38 @@ def test_constants_with_a_transposed_copy_cannot_be_set(queue, monkeypatch):
         sim.signals[weights] = np.zeros(weights.shape)
         sim.run_steps(20)
         assert not np.any(np.asarray(sim.signals[weights]))
+
+
+@pytest.mark.gpu
+def test_constant_weights_between_neurons_visit_active_columns_only(queue):
+    """A constant weight matrix from 1024 neurons onto 160 neurons (more than 64 rows: several
+    groups of rows), with and without a synapse: the products read only the columns of the
+    neurons that spiked, the neurons they drive are updated as usual, and everything equals
+    the oracle simulator bit for bit."""
+    from nengo_ocl_amd import minibuilder as mb
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    def make():
+        rng = np.random.RandomState(4)
+        net = mb.Network(seed=7)
+        stim = net.Node(mb.WhiteSignal(period=0.5, high=6.0, seed=3), size_out=2)
+        a = net.Ensemble(1024, 2, label="a")
+        b = net.Ensemble(160, 1, label="b")
+        c = net.Ensemble(96, 1, label="c")
+        net.Connection(stim, a, synapse=None)
+        net.Connection(a.neurons, b.neurons, transform=rng.normal(scale=2e-3, size=(160, 1024)),
+                       synapse=None)
+        net.Connection(a.neurons, c.neurons, transform=rng.normal(scale=2e-3, size=(96, 1024)),
+                       synapse=mb.Lowpass(0.01))
+        return net, [net.Probe(b.neurons), net.Probe(c.neurons), net.Probe(a, synapse=0.01)]
+
+    (net, probes), (net_o, probes_o) = make(), make()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        events = [p for p in gpu._plans if getattr(p, "event_driven", False)]
+        assert events and sum(p.n_tasks for p in events) >= 3 + 2  # 160 and 96 rows
+        gpu.run_steps(300)
+        cpu.run_steps(300)
+        for p, q in zip(probes, probes_o):
+            assert np.array_equal(gpu.data[p], cpu.data[q]) and np.any(gpu.data[p] != 0)
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
