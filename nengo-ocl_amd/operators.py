@@ -462,6 +462,112 @@ def propagate_vector_copies(operators, keep=()):
     return [op for op in ops if op is not None]
 
 
+def _exactly_disjoint(a, b):
+    """Views of one signal that share no element (interleaved slices pass a test of their
+    bounds and are still disjoint)."""
+    if not a.may_share_memory(b):
+        return True
+    try:
+        return not np.shares_memory(a.initial_value, b.initial_value, max_work=100000)
+    except Exception:  # too hard to decide: assume the worst
+        return False
+
+
+def products_write_their_target(operators, keep=(), ahead=None):
+    """``w = gamma + A x`` followed by ``v += 1 * w`` becomes ``v = gamma + A x``.
+
+    A transform whose result is then added into a part ``v`` of a node's or ensemble's
+    input leaves three operators behind: ``Reset(B)``, the product into its own vector
+    ``w``, and the copy ``v += w`` (after `fuse_into_multidotinc`: a MultiDotInc with the
+    constant one as its matrix).  When the views written that way are pairwise disjoint and
+    together make up the whole of ``B``, nothing else writes ``B``, and each ``w`` is a whole
+    signal outside `keep` that only its product writes and only its copy reads, the products
+    write the views themselves and the copies and the Reset go: two operator groups less in
+    a chain like "transform -> interleave -> ensembles" (the reference runs each link as a
+    launch, simulator.py:746-816).  The same holds for a ``w`` that a process updates at the
+    end of every step (the synapse of a connection into a part of a node's input: what an
+    ensemble array's output node collects): the process writes ``v`` itself, unless ``B`` is
+    in `keep` (a probe reads after the updates of a step).  Every operator then reads what it
+    read before; only the host, looking at ``B`` between two steps, sees the value the next
+    step will read where the reference shows the one the last step read -- such ``B`` are
+    added to the set `ahead`.  Values are unchanged except that the copy turned -0.0 into
+    +0.0.  The vectors ``w`` are no longer part of the simulation.  The operators
+    passed in are left as they are.
+    """
+    import copy as _copy
+
+    keep_bases = {sig.base for sig in keep}
+    ops = list(operators)
+    writers, readers = {}, {}
+    for pos, op in enumerate(ops):
+        for sig in list(op.sets) + list(op.incs) + list(op.updates):
+            writers.setdefault(sig.base, []).append(pos)
+        for sig in op.reads:
+            readers.setdefault(sig.base, []).append(pos)
+
+    def is_one(A):
+        return (A.size == 1 and getattr(A, "readonly", False) and not writers.get(A.base)
+                and float(np.asarray(A.initial_value).ravel()[0]) == 1.0)
+
+    copies_into = {}
+    for pos, op in enumerate(ops):
+        if (isinstance(op, MultiDotInc) and op._incs_Y and op.gamma == 0 and len(op.As) == 1
+                and is_one(op.As[0])):
+            w = op.Xs[0]
+            if (not getattr(w, "is_view", False) and w.base not in keep_bases
+                    and w.shape == op.Y.shape and w.base is not op.Y.base):
+                copies_into.setdefault(op.Y.base, []).append(pos)
+
+    for base, copies in copies_into.items():
+        resets = [q for q in writers.get(base, []) if _is(ops[q], "Reset")]
+        if (len(resets) != 1 or float(ops[resets[0]].value) != 0.0
+                or getattr(ops[resets[0]].dst, "is_view", False)
+                or sorted(writers[base]) != sorted(resets + copies)):
+            continue
+        views = [ops[q].Y for q in copies]
+        if sum(v.size for v in views) != base.size or not all(
+                _exactly_disjoint(a, b) for i, a in enumerate(views) for b in views[i + 1:]):
+            continue
+        pairs = []
+        for q in copies:
+            w = ops[q].Xs[0]
+            made_by = writers.get(w.base, [])
+            producer = ops[made_by[0]] if len(made_by) == 1 else None
+            if producer is None or readers.get(w.base, []) != [q]:
+                break
+            product = (isinstance(producer, MultiDotInc) and not producer._incs_Y
+                       and producer.Y is w and producer._signal_beta is None
+                       and producer._float_beta == 0
+                       and not any(sig.base is base for sig in producer.reads))
+            # a process that updates w at the end of a step (a synapse): what the copy adds
+            # at the start of the next step is what the process can leave in v itself
+            process = (_is(producer, "SimProcess") and getattr(producer, "mode", None) == "update"
+                       and getattr(producer, "output", None) is w and base not in keep_bases
+                       and not any(sig.base is base for sig in producer.all_signals))
+            if not (product or process):
+                break
+            pairs.append((made_by[0], q, product))
+        if len(pairs) != len(copies):
+            continue
+        for ppos, q, product in pairs:
+            if product:
+                new = _copy.copy(ops[ppos])
+                new.As, new.Xs = list(new.As), list(new.Xs)
+                new.Y = new.Y_in = ops[q].Y
+                if getattr(ops[q], "tag", None) is not None:
+                    new.tag = ops[q].tag
+            else:
+                w = ops[q].Xs[0]
+                new = _replace_signals(ops[ppos], {w: ops[q].Y})
+                _overwrite_initial_value(ops[q].Y, np.asarray(w.initial_value).reshape(ops[q].Y.shape))
+                if ahead is not None:
+                    ahead.add(base)
+            ops[ppos] = new
+            ops[q] = None
+        ops[resets[0]] = None
+    return [op for op in ops if op is not None]
+
+
 LEARNING_RULES = ("SimPES", "SimBCM", "SimOja", "SimVoja")
 
 

@@ -15,9 +15,20 @@ number of launches per step.
 
 from collections import defaultdict
 
+import numpy as np
+
 
 def _share(a, b):
-    return a is b or a.may_share_memory(b)
+    """Do two signals have an element in common?  Views whose bounds overlap are looked at
+    exactly: interleaved slices of one vector are disjoint."""
+    if a is b:
+        return True
+    if not a.may_share_memory(b):
+        return False
+    try:
+        return bool(np.shares_memory(a.initial_value, b.initial_value, max_work=100000))
+    except Exception:  # too hard to decide, or a signal without a host array
+        return True
 
 
 def operator_dependency_graph(operators):

@@ -291,6 +291,7 @@ class Simulator:
         probed = [self.model.sig[p]["in"] for p in self.model.probes]
         self.signal_aliases = {}  # signal dropped as a duplicate -> the one computed
         self._copied_constants = set()  # constants that launches read from a copy of their own
+        self.signals_a_step_ahead = set()
         operators = ops_mod.simplify_operators(
             all_operators, keep=probed, aliases=self.signal_aliases,
             skip=() if dedup else ("merge_identical_chains",))
@@ -308,10 +309,14 @@ class Simulator:
             # operators, but it can also split a group of like operators whose members no
             # longer depend on the same things: keep it only where the step gets shorter
             shorter = ops_mod.propagate_vector_copies(operators, keep=probed)
+            ahead = set()
+            shorter = ops_mod.products_write_their_target(shorter, keep=probed, ahead=ahead)
             if len(shorter) < len(operators):
                 shorter_groups = planner(shorter)
                 if len(shorter_groups) < len(op_groups):
                     operators, op_groups = shorter, shorter_groups
+                    # signals that hold, between two steps, what the next step will read
+                    self.signals_a_step_ahead = ahead
         assert len([t for t, _ in op_groups if t.__name__ == "Reset"]) < 2, \
             "All resets not planned together"
         self.operators = operators
