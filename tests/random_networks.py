@@ -133,3 +133,25 @@ def _learning_and_neuron_links(net, rng, ens, stim, probes, big):
                     size_out=1, label="hiss")
     net.Connection(hiss, noisy, synapse=mb.Lowpass(0.005))
     probes["noisy"] = net.Probe(noisy.neurons, sample_every=0.002)
+
+
+def ensemble_array_network(probe_node=False):
+    """Three ensembles whose filtered outputs a node collects, that node and the stimulus
+    interleaved by two transforms into a second node, which drives an ensemble."""
+    rng = np.random.RandomState(2)
+    net = mb.Network(seed=5)
+    stim = net.Node(mb.WhiteSignal(period=0.4, high=7.0, seed=2), size_out=3)
+    parts = [net.Ensemble(60, 1, label="part%d" % k) for k in range(3)]
+    out = net.Node(None, size_in=3, label="collect")
+    mix = net.Node(None, size_in=6, label="interleave")
+    for k, ens in enumerate(parts):
+        net.Connection(stim[k:k + 1], ens, synapse=None)
+        net.Connection(ens, out[k:k + 1], synapse=mb.Lowpass(0.005))
+    net.Connection(out, mix[0::2], transform=rng.normal(size=(3, 3)), synapse=None)
+    net.Connection(stim, mix[1::2], transform=rng.normal(size=(3, 3)), synapse=None)
+    post = net.Ensemble(120, 6, label="post")
+    net.Connection(mix, post, synapse=None)
+    probes = {"post": net.Probe(post, synapse=0.01)}
+    if probe_node:
+        probes["collect"] = net.Probe(out)
+    return net, probes

@@ -555,3 +555,35 @@ def test_sparse_product_sets_its_target():
     assert [type(op).__name__ for op in one] == ["SparseDotSet"]
     half = [ir.Reset(y, value=0.5), ir.SparseDotInc(mats[0], x, y)]  # not a reset to zero
     assert operators.sparse_products_set_their_target(half) == half
+
+
+def test_synapses_write_the_node_input_they_feed():
+    """An ensemble array: three ensembles whose filtered outputs are collected by a node, and
+    two transforms interleaved into another node.  The synapses and the transforms write their
+    part of the node's input themselves (no Reset, no copies); probes equal the
+    operator-at-a-time interpreter bit for bit, and the collected input holds, between steps,
+    what the next step reads.  A probed node input is left alone."""
+    from naive_interpreter import NaiveInterpreter
+    from random_networks import ensemble_array_network as make
+
+    net, probes = make(probe_node=False)
+    model = net.build_model(dt=0.001)
+    naive = NaiveInterpreter(model)
+    with OracleSimulator(None, model=model, seed=1) as sim:
+        names = {b.name for b in sim.signals_a_step_ahead}
+        assert names == {"<Node collect>.in"}
+        kinds = [type(op).__name__ for op in sim.operators]
+        assert "Reset" not in kinds
+        sim.run_steps(200)
+        naive.run_steps(200)
+        assert np.array_equal(sim.data[probes["post"]], naive.data(probes["post"]))
+        assert np.any(sim.data[probes["post"]] != 0)
+    net, probes = make(probe_node=True)
+    model = net.build_model(dt=0.001)
+    naive = NaiveInterpreter(model)
+    with OracleSimulator(None, model=model, seed=1) as sim:
+        assert not sim.signals_a_step_ahead
+        sim.run_steps(100)
+        naive.run_steps(100)
+        for key, p in probes.items():
+            assert np.array_equal(sim.data[p], naive.data(p)), key

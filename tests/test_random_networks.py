@@ -88,3 +88,24 @@ def test_random_network_on_the_device(queue, seed, big, sliced, rich):
                 got = np.asarray(gpu.signals[base]).reshape(-1)
                 want = np.asarray(cpu.signals[base]).reshape(-1)
                 assert np.array_equal(got, want), base
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("probe_node", [False, True])
+def test_ensemble_array_on_the_device(queue, probe_node):
+    """Synapses and transforms that write their part of a node's input (strided and
+    one-element views as outputs of the GEMV and filter launches): the device equals the
+    oracle simulator bit for bit, in every signal."""
+    from nengo_ocl_amd.simulator import Simulator
+    from random_networks import ensemble_array_network
+
+    net, probes = ensemble_array_network(probe_node)
+    model = net.build_model(dt=0.001)
+    with Simulator(None, model=model, seed=1) as gpu, \
+            OracleSimulator(None, model=model, seed=1) as cpu:
+        assert bool(gpu.signals_a_step_ahead) == (not probe_node)
+        gpu.run_steps(200)
+        cpu.run_steps(200)
+        for key, p in probes.items():
+            assert np.array_equal(gpu.data[p], cpu.data[p]) and np.any(gpu.data[p] != 0), key
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
