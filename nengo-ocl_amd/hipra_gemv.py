@@ -388,7 +388,7 @@ class gemv_prog:
                        lib.nhip_gemv_tile_rows(dd["a_shape1"], TILE_STAGE_WORDS)
                        for dd in geometry[b]["dots"]] or [WAVE]) for b in members}
 
-        def tasks_for(per_task):
+        def tasks_for(per_task, whole_blocks_up):
             out = []
             for b in members:
                 M = geometry[b]["y_len"]
@@ -396,7 +396,12 @@ class gemv_prog:
                 if M > item_rows:
                     item_rows = _balanced_rows(M, item_rows)
                     if item_rows >= 2 * blk[b]:
-                        item_rows -= item_rows % blk[b]
+                        # whole row blocks: fewer rows per task, or more (fewer tasks, the
+                        # last one of an item shorter); the cost below decides
+                        if whole_blocks_up:
+                            item_rows = min(-(-item_rows // blk[b]) * blk[b], max_rows)
+                        else:
+                            item_rows -= item_rows % blk[b]
                     # (tasks that must start at a multiple of so many rows)
                     item_rows = min(-(-item_rows // row_multiple) * row_multiple, max_rows)
                 for r0 in range(0, M, item_rows):
@@ -406,8 +411,8 @@ class gemv_prog:
         n_cu = self.queue.n_compute_units
         best = None
         row_bytes = {b: 4.0 * sum(dd["a_shape1"] for dd in geometry[b]["dots"]) for b in members}
-        for per_task in TILE_TASK_BLOCKS:
-            tasks = tasks_for(per_task)
+        for per_task, up in [(p, u) for p in TILE_TASK_BLOCKS for u in (False, True)]:
+            tasks = tasks_for(per_task, up)
             groups = -(-len(tasks) // (WG // WAVE))
             task_bytes = sum(row_bytes[b] * n for b, _, n, _ in tasks) / max(len(tasks), 1)
             cost = -(-groups // n_cu) * (task_bytes + TASK_OVERHEAD_BYTES)

@@ -470,8 +470,10 @@ def test_large_item_task_sizes():
     # 258 matrices of 64 x 4096 (blocks of 4 rows): 8-row tasks would leave 516 groups for
     # 256 compute units, 6-row tasks (the last of an item: 4) give 710 groups, under 3 each
     assert {n for _, _, n, _ in tasks_of(258, 64, 4096, 256)} == {6, 4}
-    # 192 matrices of 2000 x 32 (blocks of 32 rows): 96 rows = 1008 groups, under 4 each
-    assert max(n for _, _, n, _ in tasks_of(192, 2000, 32, 128)) == 96
+    # 192 matrices of 2000 x 32 (blocks of 32 rows): 96-row tasks are 1008 groups, just under
+    # 4 per compute unit; whole blocks rounded up instead, 128 rows (the last of an item:
+    # 80), are 768 groups, 3 each, and fewer task starts
+    assert {n for _, _, n, _ in tasks_of(192, 2000, 32, 128)} == {128, 80}
     # 64 x 4096 on a device of 64 compute units: 16-row tasks would be too few (1032)
     assert max(n for _, _, n, _ in tasks_of(258, 64, 4096, 256, n_cu=64)) < 16
 
