@@ -233,6 +233,8 @@ def event_driven_report(sim, event_rows, steps_per_s, make_sim, args):
                    "(results bit-identical to the dense product); their algorithmic bytes are "
                    "not traffic and are left out of gemv_all",
            "neurons_that_spiked_in_the_last_step": nz / max(n, 1)}
+    if args.no_dense_comparison:
+        return out
     os.environ["NENGO_HIP_EVENT_GEMV"] = "0"
     try:
         dense = make_sim()
@@ -390,6 +392,9 @@ def main():
     ap.add_argument("--dense-decoders", action="store_true",
                     help="multiply every column of the matrices applied to spike vectors "
                          "(default: only the columns of the neurons that spiked are visited)")
+    ap.add_argument("--no-dense-comparison", action="store_true",
+                    help="do not time the every-column variant next to the default one "
+                         "(kernel traces then hold the default launches only)")
     ap.add_argument("--no-fuse", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--two-pass-learning", action="store_true",
