@@ -88,7 +88,7 @@ def gemv_summary(sim, profile_steps):
 
 
 KERNEL_SOURCES = ("gemv_tile.hip", "gemv_types.h", "gemv_rows.h", "neuron_math.h", "nhip_common.h",
-                  "sequence_ops.h")
+                  "sequence_ops.h", "small_arg_math.h")
 
 
 def kernel_sources_hash():

@@ -434,7 +434,7 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
         const bool live = e0 + lane < n_leaving;
         const float* e = leaving + 4 * (live ? e0 + lane : 0);
         const int r = __float_as_int(e[0]);
-        const float factor = -(float)expm1((double)__fdiv_rn(-e[1], tau));
+        const float factor = -(float)nhip_expm1((double)__fdiv_rn(-e[1], tau));
         integrate(live, r, e[2], e[3], factor);
     }
     wave_sync();
@@ -446,7 +446,7 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
             const float ref = lif_param(p.ref, p.pflags & 2, a.REF, row0 + r);
             const float amp = lif_param(p.amp, p.pflags & 4, a.AMP, row0 + r);
             const float t_spike = __fadd_rn(
-                dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
+                dtu, __fmul_rn(tau, (float)nhip_log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
             new_v[r] = 0.0f;
             new_w[r] = ref + t_spike;
             new_s[r] = __fmul_rn(amp, a.dt_inv);

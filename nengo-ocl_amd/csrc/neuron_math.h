@@ -2,6 +2,7 @@
 #pragma once
 
 #include "nhip_common.h"
+#include "small_arg_math.h"
 
 // One population of LIF neurons driven by one output item of a GEMV: element
 // offsets of its state, and its parameters as float bits or (pflags bit set) as the
@@ -47,18 +48,20 @@ __device__ __forceinline__ float lif_param(int word, bool is_vector, const float
 // expm1 and log1p are evaluated in double and rounded once to float: that is the
 // correctly rounded float32 value (the best any float implementation can return),
 // so every conforming host or device math library gives the same bits and spike
-// decisions do not depend on the library.  Returns whether the neuron spiked.
+// decisions do not depend on the library.  Their arguments are small here (at most
+// dt / tau in magnitude), which `nhip_expm1` / `nhip_log1p` use: a short series for
+// |x| <= 1/16, the library routine otherwise.  Returns whether the neuron spiked.
 __device__ __forceinline__ bool lif_step(float j, float& v, float& w, float tau, float ref,
                                          float dtu, int upsample) {
     bool spiked = false;
     for (int u = 0; u < upsample; ++u) {
         w -= dtu;
         const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
-        const float dv = __fmul_rn(-(float)expm1((double)__fdiv_rn(-delta_t, tau)), j - v);
+        const float dv = __fmul_rn(-(float)nhip_expm1((double)__fdiv_rn(-delta_t, tau)), j - v);
         v = __fadd_rn(v, dv);
         if (v > 1.0f) {
             const float t_spike =
-                __fadd_rn(dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
+                __fadd_rn(dtu, __fmul_rn(tau, (float)nhip_log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
             w = ref + t_spike;
             v = 0.0f;
             spiked = true;
@@ -107,7 +110,7 @@ __device__ __forceinline__ void lif_rate_block(const RateDesc d, const float* J,
         const float ref = lif_param(d.ref, d.pflags & 2, REF, i);
         const float amp = lif_param(d.amp, d.pflags & 4, AMP, i);
         const float j = fmaxf(J[(size_t)d.j_start + i] - 1.0f, 0.0f);
-        const float denom = __fadd_rn(ref, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(1.0f, j))));
+        const float denom = __fadd_rn(ref, __fmul_rn(tau, (float)nhip_log1p((double)__fdiv_rn(1.0f, j))));
         R[(size_t)d.r_start + i] = __fdiv_rn(amp, denom);
     }
 }

@@ -62,12 +62,12 @@ __global__ __launch_bounds__(NHIP_WG) void alif_kernel(const NeuronDesc* __restr
             w -= dtu;
             const float delta_t = (w > dtu) ? 0.0f : (w < 0.0f) ? dtu : dtu - w;
             const float dv =
-                __fmul_rn(-(float)expm1((double)__fdiv_rn(-delta_t, tau)), (j - n) - v);
+                __fmul_rn(-(float)nhip_expm1((double)__fdiv_rn(-delta_t, tau)), (j - n) - v);
             v = __fadd_rn(v, dv);
             if (v > 1.0f) {
                 // the spike time interpolates with the unadapted current, as the reference does
                 const float t_spike = __fadd_rn(
-                    dtu, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
+                    dtu, __fmul_rn(tau, (float)nhip_log1p((double)__fdiv_rn(-(v - 1.0f), j - 1.0f))));
                 w = ref + t_spike;
                 v = 0.0f;
                 spiked = true;
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(NHIP_WG) void alif_rate_kernel(const NeuronDesc* __
         const float inc_n = lif_param(d.p[4], d.pflags & 16, INC_N, i);
         const float n = N[(size_t)d.n_start + i];
         const float j = fmaxf((J[(size_t)d.j_start + i] - n) - 1.0f, 0.0f);
-        const float denom = __fadd_rn(ref, __fmul_rn(tau, (float)log1p((double)__fdiv_rn(1.0f, j))));
+        const float denom = __fadd_rn(ref, __fmul_rn(tau, (float)nhip_log1p((double)__fdiv_rn(1.0f, j))));
         const float r = __fdiv_rn(amp, denom);
         R[(size_t)d.out_start + i] = r;
         N[(size_t)d.n_start + i] =

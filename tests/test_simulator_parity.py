@@ -199,6 +199,69 @@ def test_c3_full_size_state_bit_exact(queue):
         assert all(np.any(gpu.data[probes[key]] != 0) for key in probes)  # something happened
 
 
+def _spike_reader(sim, signals):
+    """A function that returns the current spike vector of every population, read in one
+    device-to-host copy when the signals lie close together in the simulator's buffer."""
+    idx = [int(sim.sidx[s]) for s in signals]
+    starts = [int(sim.all_data.starts[i]) for i in idx]
+    sizes = [int(s.size) for s in signals]
+    lo, hi = min(starts), max(a + n for a, n in zip(starts, sizes))
+    dev_buf = getattr(sim.all_data, "dev_buf", None)
+    if dev_buf is None or hi - lo > 4 * sum(sizes):
+        return lambda: np.concatenate([np.asarray(sim.signals[s]).ravel() for s in signals])
+
+    def read():
+        span = dev_buf.get_span(lo, hi - lo)
+        return np.concatenate([span[a - lo: a - lo + n] for a, n in zip(starts, sizes)])
+    return read
+
+
+def test_c3_full_size_spike_counts_over_one_second(queue):
+    """The acceptance criterion at the size the throughput is quoted on: 1000 steps (1 s) of
+    the full benchmark network (1,048,576 LIF neurons, the two launches per step that the
+    benchmark times, no extra probes), the spike vector of every population read after every
+    step on both sides; at least 99.9 % of the per-neuron spike counts must be equal (they
+    all are: the test prints the figures), and the final state is bit-identical."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    net, probes, _ = configs.c3_large()
+    net_o, probes_o, _ = configs.c3_large()
+    model, model_o = net.build_model(dt=0.001), net_o.build_model(dt=0.001)
+    with Simulator(None, model=model, seed=1) as gpu, \
+            OracleSimulator(None, model=model_o, seed=1) as cpu:
+        assert sorted(p.name for p in gpu._plans) == ["hipra_gemv.events_filter",
+                                                      "hipra_gemv.tile_lif"]
+        spikes_g = [model.sig[e.neurons]["out"] for e in net.ensembles]
+        spikes_c = [model_o.sig[e.neurons]["out"] for e in net_o.ensembles]
+        read_g, read_c = _spike_reader(gpu, spikes_g), _spike_reader(cpu, spikes_c)
+        n = sum(int(s.size) for s in spikes_g)
+        assert n == 1048576
+        counts_g, counts_c = np.zeros(n, dtype=np.int64), np.zeros(n, dtype=np.int64)
+        steps_that_differ = 0
+        for step in range(1000):
+            gpu.run_steps(1)
+            cpu.run_steps(1)
+            g, c = read_g() != 0, read_c() != 0
+            counts_g += g
+            counts_c += c
+            steps_that_differ += int(np.any(g != c))
+            if step % 100 == 99:
+                print("step %d: %d spikes so far (oracle %d)" % (
+                    step + 1, counts_g.sum(), counts_c.sum()), flush=True)
+        equal = int((counts_g == counts_c).sum())
+        print("c3 full size, 1 s: %d of %d per-neuron spike counts equal (%.4f %%), largest "
+              "difference %d spikes, %d spikes in total (mean rate %.1f Hz), %d steps with any "
+              "difference" % (equal, n, 100.0 * equal / n, int(np.abs(counts_g - counts_c).max()),
+                              int(counts_c.sum()), counts_c.sum() / n, steps_that_differ))
+        assert equal / n >= 0.999
+        assert counts_c.sum() > 50 * n  # the network is active: tens of Hz per neuron
+        for key in probes:
+            assert np.array_equal(gpu.data[probes[key]], cpu.data[probes_o[key]]), key
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+
+
 def test_merged_products_keep_every_signal(queue):
     """One built model (per-connection decoders, reduced c3) run on the GPU with identical
     products merged and without: every probe sample and every signal of the model --
