@@ -366,6 +366,24 @@ int nhip_linearfilter(void *stream, const int *desc, int *pos, int n_blocks, int
  *          count, alpha_bits, flags(bit0 outer, bit1 inc), 0} */
 int nhip_elementwise_inc(void *stream, const int *desc, int n_blocks, int lanes, const float *A,
                          const float *X, float *Y);
+/* Outer-product increment Y (=|+=) (alpha a) (x) x and, in the same launch, the step of
+ * the first-order filters that produce its column operands: a record's work-group owns
+ * all rows of up to 128 columns of one matrix, so it is the only reader of those elements
+ * of the filter output and steps them once its part of the matrix is written.
+ * replaces: `plan_elementwise_inc` with outer=True (:414-574) followed by
+ * `plan_linearfilter` (:577-803, its cases (na,nb) = (0,1) and (1,1)) on the vector the
+ * outer product has just read -- the end of a PES step.  Element by element the same
+ * rounded operations as the two kernels.
+ *   desc : int32[n_records][16] {a_start, a_stride0 (0: one value for all rows),
+ *          x_start, x_stride0 (0: one value for all columns), y_start, y_stride0,
+ *          rows (<= 256), col0, ncols (<= 128), alpha_bits,
+ *          flags (bit0 inc, bit1 filter present, bit2 filter has a0, bit3 no outer
+ *          product: the record only steps a filter), s_start, f_start (filter input /
+ *          output; column c of the record at *_start + c), a0_bits, b0_bits, 0};
+ *          y_start, y_stride0, col0 and ncols are multiples of 4 (16-byte accesses)
+ *   A, X, Y : buffers of the outer product;  S, F : of the filters (F may be X). */
+int nhip_outer_filter(void *stream, const int *desc, int n_records, const float *A,
+                      const float *X, float *Y, const float *S, float *F);
 /* Weight-update rules that write a delta matrix per connection (row i = post
  * neuron, column j = pre element; delta rows are contiguous):
  *   BCM  delta[i,j] = alpha * post[i] * (post[i] - theta[i]) * pre[j]

@@ -52,6 +52,7 @@ SIGNATURES = {
     "nhip_sigmoid": [P, P, c_int, P, P, P],
     "nhip_linearfilter": [P, P, P, c_int, c_int, P, P, P, P, P, P],
     "nhip_elementwise_inc": [P, P, c_int, c_int, P, P, P],
+    "nhip_outer_filter": [P, P, c_int, P, P, P, P, P],
     "nhip_learning_rule": [P, c_int, c_int, P, c_int, P, P, P, P, P, P],
     "nhip_conv2d": [P, P, P, P, P],
     "nhip_pool2d": [P, P, P, P],

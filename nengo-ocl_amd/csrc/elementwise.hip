@@ -42,6 +42,90 @@ __global__ __launch_bounds__(NHIP_WG) void elementwise_inc_kernel(const EwDesc* 
     NHIP_FOR_MY_ROW(L, n_rows, elementwise_inc_block(desc[row], A, X, Y, lane, LL));
 }
 
+// Outer-product increment and the filter of its column operand in one launch.
+// A learning rule like PES ends a step with W += (alpha a) (x) f  (plan_elementwise_inc with
+// outer=True, clra_nonlinearities.py:449-525) followed by the filter step that produces the
+// next f from the spikes (plan_linearfilter, simple case :630-650): two launches, the second
+// one a few hundred kilobytes that cost a launch's latency.  The filter may not run before
+// every element of W that uses the old f has been formed.  Here a work-group owns all rows
+// of up to 128 columns of one matrix: it is the only reader of those elements of f, so it
+// steps them itself once its part of W is done -- the same rounded operations in both
+// parts, element by element, as the two kernels.  Filters that feed no outer product of the
+// launch, and outer products whose column operand is not filtered here, ride as records
+// with one half only.
+struct OuterFilterDesc {  // 16 words
+    int a_start, a_stride0;  // row operand (stride 0: one value for all rows)
+    int x_start, x_stride0;  // column operand (stride 0: one value for all columns)
+    int y_start, y_stride0;  // first element of the matrix, words between its rows
+    int rows, col0, ncols;   // the record's tile: all rows of columns col0 .. col0 + ncols
+    int alpha_bits;
+    int flags;               // OF_INC, OF_FILTER, OF_FILTER_HAS_A, OF_NO_OUTER
+    int s_start, f_start;    // filter input and output: element col0 + t at *_start + col0 + t
+    int fa_bits, fb_bits;    // y = b0 x - a0 y (or y = b0 x)
+    int pad;
+};
+static_assert(sizeof(OuterFilterDesc) == 64, "records are 16 words");
+constexpr int OF_INC = 1, OF_FILTER = 2, OF_FILTER_HAS_A = 4, OF_NO_OUTER = 8;
+
+__global__ __launch_bounds__(NHIP_WG) void outer_filter_kernel(
+    const OuterFilterDesc* __restrict__ desc, const float* A, const float* X, float* Y,
+    const float* S, float* F)
+{
+    const OuterFilterDesc d = desc[blockIdx.x];
+    const int tid = threadIdx.x;
+    if (!(d.flags & OF_NO_OUTER)) {
+        // four elements of a row per lane and access (the host has checked that rows, tiles
+        // and the matrix start on 16-byte boundaries), four such quads per lane requested
+        // together; (alpha a) x then the sum, each rounded, as in elementwise_inc_block
+        const float alpha = nhip_bits(d.alpha_bits);
+        const bool inc = d.flags & OF_INC;
+        const float* a = A + d.a_start;
+        const float* x = X + d.x_start;
+        float* y = Y + d.y_start + d.col0;
+        const int qpr = d.ncols >> 2;  // quads per row of the tile, <= 32
+        const int n_quads = d.rows * qpr;
+        const float qpr_inv = __frcp_rn((float)qpr);
+        constexpr int U = 4;
+        for (int k0 = tid; k0 < n_quads; k0 += U * NHIP_WG) {
+            float4* dst[U];
+            float4 w[U];
+            float aa[U], xx[U][4];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int k = min(k0 + u * NHIP_WG, n_quads - 1);  // past the end: the last quad again
+                int i = (int)((float)k * qpr_inv);  // k < 8192: exact after one correction
+                if ((i + 1) * qpr <= k) ++i;
+                if (i * qpr > k) --i;
+                const int j = 4 * (k - i * qpr);
+                dst[u] = reinterpret_cast<float4*>(y + (size_t)i * d.y_stride0 + j);
+                if (inc) w[u] = *dst[u];
+                aa[u] = a[(size_t)i * d.a_stride0];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) xx[u][e] = x[(size_t)(d.col0 + j + e) * d.x_stride0];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (k0 + u * NHIP_WG >= n_quads) break;
+                const float s = __fmul_rn(alpha, aa[u]);
+                float4 v = make_float4(__fmul_rn(s, xx[u][0]), __fmul_rn(s, xx[u][1]),
+                                       __fmul_rn(s, xx[u][2]), __fmul_rn(s, xx[u][3]));
+                if (inc)
+                    v = make_float4(__fadd_rn(w[u].x, v.x), __fadd_rn(w[u].y, v.y),
+                                    __fadd_rn(w[u].z, v.z), __fadd_rn(w[u].w, v.w));
+                *dst[u] = v;
+            }
+        }
+    }
+    // every lane of the group has read its column operands: the filter may overwrite them
+    __syncthreads();
+    if ((d.flags & OF_FILTER) && tid < d.ncols) {
+        const size_t c = (size_t)d.col0 + tid;
+        const float bx = __fmul_rn(nhip_bits(d.fb_bits), S[d.s_start + c]);
+        float* f = F + d.f_start + c;
+        *f = (d.flags & OF_FILTER_HAS_A) ? __fsub_rn(bx, __fmul_rn(nhip_bits(d.fa_bits), *f)) : bx;
+    }
+}
+
 __global__ __launch_bounds__(NHIP_WG) void linearfilter_kernel(const LfDesc* __restrict__ desc,
                                                                int2* pos, int n_rows, int L,
                                                                const float* X, float* Y,
@@ -201,6 +285,16 @@ extern "C" int nhip_linearfilter(void* stream, const int* desc, int* pos, int n_
     NHIP_LAUNCH(linearfilter_kernel, row_grid(n_blocks, lanes), dim3(NHIP_WG), 0,
                        NHIP_STREAM(stream), reinterpret_cast<const LfDesc*>(desc),
                        reinterpret_cast<int2*>(pos), n_blocks, lanes, X, Y, A, B, Xbuf, Ybuf);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int nhip_outer_filter(void* stream, const int* desc, int n_records, const float* A,
+                                 const float* X, float* Y, const float* S, float* F) {
+    if (n_records == 0) return 0;
+    if (n_records < 0 || !desc || !A || !X || !Y || !S || !F) return NHIP_E_BADARG;
+    NHIP_LAUNCH(outer_filter_kernel, dim3(n_records), dim3(NHIP_WG), 0, NHIP_STREAM(stream),
+                reinterpret_cast<const OuterFilterDesc*>(desc), A, X, Y, S, F);
     NHIP_LAUNCH_CHECK();
     return 0;
 }

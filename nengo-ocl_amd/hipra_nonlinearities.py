@@ -30,6 +30,7 @@ item) at plan time; argument checks raise the same exception types the
 reference's asserts / raises produce (AssertionError, NotImplementedError).
 """
 
+import logging
 import re
 
 import numpy as np
@@ -38,6 +39,8 @@ from . import _lib
 from .hipraggedarray import DeviceArray, HIPRaggedArray, _torch, to_device
 from .plan import Plan
 from .utils import f32_bits, is_number
+
+logger = logging.getLogger(__name__)
 
 WG = 256
 BLOCK = 1024  # elements of one item handled by one work-group
@@ -263,6 +266,143 @@ def plan_elementwise_inc(queue, A, X, Y, alpha=None, outer=False, inc=True, tag=
     plan.bw_per_call = A.nbytes + X.nbytes + Y.nbytes + (0 if alpha is None else alphas.nbytes)
     plan.description = _description(Y)
     plan.row_iterations = _row_iterations(counts, lanes)
+    # what `fuse_outer_filter` needs to run the filters of the column operands in this launch
+    plan.ew_spec = dict(A=A, X=X, Y=Y, alphas=alphas, outer=outer, inc=inc)
+    return plan
+
+
+# ---------------------------------------------------------------- outer product + filter
+OF_INC, OF_FILTER, OF_FILTER_HAS_A, OF_NO_OUTER = 1, 2, 4, 8  # flags of csrc/elementwise.hip
+OF_MAX_COLS, OF_MAX_ROWS = 128, 256
+
+
+def _interval(ra, i):
+    """[first, last + 1) element of item i of a ragged array (empty items: None)."""
+    n0, n1 = int(ra.shape0s[i]), int(ra.shape1s[i])
+    if n0 == 0 or n1 == 0:
+        return None
+    first = int(ra.starts[i])
+    return first, first + (n0 - 1) * int(ra.stride0s[i]) + (n1 - 1) * int(ra.stride1s[i]) + 1
+
+
+def _apart(reason):
+    logger.debug("outer product and filter stay launches of their own: %s", reason)
+    return None
+
+
+def _touch(iv, others):
+    return iv is not None and any(o is not None and iv[0] < o[1] and o[0] < iv[1] for o in others)
+
+
+def fuse_outer_filter(ew_plan, lf_plan):
+    """One launch for "W (+)= (alpha a) (x) f; f <- filter(s)" (clra_nonlinearities.py
+    `plan_elementwise_inc` with outer=True followed by `plan_linearfilter`): the end of a
+    PES step, where the filter of the pre-synaptic activities may only run once the weight
+    update has read their old values.  A work-group of `nhip_outer_filter` owns all rows of
+    up to 128 columns of a matrix and steps the filter elements of those columns after
+    writing them.
+
+    Fused when every outer product has at most 256 rows and 16-byte aligned rows, every
+    filter has one numerator and at most one denominator coefficient over contiguous
+    vectors, and each filter output is either the column operand of exactly one outer
+    product (same start and length) or touched by none of them; nothing the filters write
+    may be a row operand or another operand of the launch.  Returns the plan that replaces
+    both, or None.
+    """
+    ew, lf = getattr(ew_plan, "ew_spec", None), getattr(lf_plan, "lf_spec", None)
+    if ew is None or lf is None or not ew["outer"]:
+        return _apart("no outer product or no simple filter plan")
+    A, X, Y, alphas, inc = ew["A"], ew["X"], ew["Y"], ew["alphas"], ew["inc"]
+    S, F, FA, FB = lf["X"], lf["Y"], lf["A"], lf["B"]
+    queue = ew_plan.queue
+    n_outer, n_filters = len(Y), len(F)
+    if n_outer == 0 or n_filters == 0:
+        return _apart("nothing to fuse")
+    # shapes the kernel takes
+    for i in range(n_outer):
+        rows, cols = int(Y.shape0s[i]), int(Y.shape1s[i])
+        if rows > OF_MAX_ROWS or rows == 0 or cols == 0:
+            return _apart("an outer product with more than 256 rows or an empty one")
+        if (int(Y.starts[i]) | int(Y.stride0s[i]) | cols) & 3:
+            return _apart("rows of an outer product are not whole aligned quads")
+    for k in range(n_filters):
+        simple = int(FB.shape0s[k]) == 1 and int(FA.shape0s[k]) <= 1
+        vector = all(int(r.shape1s[k]) == 1 and int(r.stride0s[k]) == 1 for r in (S, F))
+        if not (simple and vector and int(S.shape0s[k]) == int(F.shape0s[k])):
+            return _apart("a filter of higher order or over strided vectors")
+    same = lambda p, q: p.ptr.value == q.ptr.value
+    f_iv = [_interval(F, k) for k in range(n_filters)]
+    x_iv = [_interval(X, i) for i in range(n_outer)]
+    a_iv = [_interval(A, i) for i in range(n_outer)]
+    y_iv = [_interval(Y, i) for i in range(n_outer)]
+    s_iv = [_interval(S, k) for k in range(n_filters)]
+    # filter outputs: the column operand of exactly one outer product, or of none
+    owner = {}  # filter -> outer product
+    for k in range(n_filters):
+        users = [i for i in range(n_outer) if same(F, X) and _touch(f_iv[k], [x_iv[i]])]
+        if same(F, A) and _touch(f_iv[k], a_iv):
+            return _apart("a filter output is a row operand of the launch")
+        if same(F, Y) and _touch(f_iv[k], y_iv):
+            return _apart("a filter output overlaps a matrix of the launch")
+        if same(F, S) and _touch(f_iv[k], [s_iv[q] for q in range(n_filters) if q != k]):
+            return _apart("a filter output is another filter's input")
+        if not users:
+            continue
+        i = users[0]
+        exact = (len(users) == 1 and int(X.shape0s[i]) == int(Y.shape1s[i])
+                 and int(X.stride0s[i]) == 1 and x_iv[i] == f_iv[k])
+        if not exact:
+            return _apart("a filter output is not exactly the column operand of one outer product")
+        owner[k] = i
+    if len(set(owner.values())) != len(owner):
+        return _apart("two filters feed the column operand of one outer product")
+    if same(S, Y) and any(_touch(iv, y_iv) for iv in s_iv):
+        return _apart("a filter input overlaps a matrix of the launch")
+    if not owner:
+        return _apart("no filter output is a column operand of the launch")
+    filter_of = {i: k for k, i in owner.items()}
+
+    a_host, b_host = FA.to_host(), FB.to_host()
+
+    def filter_words(k):
+        na = int(FA.shape0s[k])
+        a0 = np.float32(a_host[k][0, 0]) if na else np.float32(0)
+        b0 = np.float32(b_host[k][0, 0])
+        flags = OF_FILTER | (OF_FILTER_HAS_A if na else 0)
+        return flags, int(S.starts[k]), int(F.starts[k]), int(a0.view(np.int32)), int(b0.view(np.int32))
+
+    records = []
+    for i in range(n_outer):
+        rows, cols = int(Y.shape0s[i]), int(Y.shape1s[i])
+        a_stride = 0 if int(A.shape0s[i]) == 1 else int(A.stride0s[i])
+        x_stride = 0 if int(X.shape0s[i]) == 1 else int(X.stride0s[i])
+        alpha_bits = int(np.float32(alphas[i]).view(np.int32))
+        flags, s0, f0, fa, fb = (0, 0, 0, 0, 0)
+        if i in filter_of:
+            flags, s0, f0, fa, fb = filter_words(filter_of[i])
+        for col0 in range(0, cols, OF_MAX_COLS):
+            records.append((int(A.starts[i]), a_stride, int(X.starts[i]), x_stride,
+                            int(Y.starts[i]), int(Y.stride0s[i]), rows, col0,
+                            min(OF_MAX_COLS, cols - col0), alpha_bits,
+                            flags | (OF_INC if inc else 0), s0, f0, fa, fb, 0))
+    for k in range(n_filters):
+        if k in owner:
+            continue
+        flags, s0, f0, fa, fb = filter_words(k)
+        for col0 in range(0, int(F.shape0s[k]), OF_MAX_COLS):
+            records.append((0, 0, 0, 0, 0, 0, 0, col0, min(OF_MAX_COLS, int(F.shape0s[k]) - col0),
+                            0, flags | OF_NO_OUTER, s0, f0, fa, fb, 0))
+    table = to_device(queue, np.array(records, dtype=np.int32).reshape(-1, 16))
+    n = len(records)
+    plan = Plan(queue, queue.lib.nhip_outer_filter,
+                (table.ptr, n, A.ptr, X.ptr, Y.ptr, S.ptr, F.ptr),
+                gsize=(n * WG,), lsize=(WG,),
+                full_args=tuple(ew_plan.full_args) + tuple(lf_plan.full_args) + (table,),
+                name="hip_outer_filter", tag=ew_plan.tag)
+    plan.flops_per_call = (ew_plan.flops_per_call or 0) + (lf_plan.flops_per_call or 0)
+    plan.bw_per_call = (ew_plan.bw_per_call or 0) + (lf_plan.bw_per_call or 0)
+    plan.description = ew_plan.description
+    plan.fused_filters = sorted(owner)
     return plan
 
 

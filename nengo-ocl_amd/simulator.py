@@ -89,6 +89,8 @@ class HipBackend:
         self.plans_conflict = hipra_sequence._conflict
         self.fuse_gemv_filter = hipra_gemv.fuse_linearfilter
         self.fuse_spmv_filter = hipra_spmv.fuse_linearfilter
+        if os.environ.get("NENGO_HIP_OUTER_FILTER", "1") != "0":  # switch for measurements
+            self.fuse_outer_filter = hipra_nonlinearities.fuse_outer_filter
 
     def fuse_input_sums(self, sum_plan, lif_plan):
         """The plan replacing ``[sum_plan, lif_plan]`` when the first only forms vector
@@ -439,6 +441,8 @@ class Simulator:
         plans.extend(probe_plans)
         if fuse and hasattr(self.backend, "fuse_gemv_filter"):
             plans = self._fuse_filter_epilogues(plans)
+        if fuse and hasattr(self.backend, "fuse_outer_filter"):
+            plans = self._fuse_outer_filters(plans)
         if fuse and hasattr(self.backend, "fuse_input_sums"):
             plans = self._fuse_input_sums(plans)
         if merge_small and hasattr(self.backend, "merge_small_plans"):
@@ -471,6 +475,43 @@ class Simulator:
             fused.writes_mem = out[-1].writes_mem | plan.writes_mem
             out[-1] = fused
         return out
+
+    def _fuse_outer_filters(self, plans):
+        """An outer-product update (a learning rule's weight increment) and the launch behind
+        it that filters its column operands become one launch
+        (`hipra_nonlinearities.fuse_outer_filter`), when the plans between the two touch
+        nothing that the one that moves reads or writes."""
+        plans = list(plans)
+        conflict = self.backend.plans_conflict
+        j = 0
+        while j < len(plans):
+            lf = plans[j]
+            j += 1
+            if getattr(lf, "lf_spec", None) is None:
+                continue
+            i = j - 2
+            while i >= 0 and not (getattr(plans[i], "ew_spec", None) or {}).get("outer"):
+                i -= 1
+            if i < 0:
+                continue
+            ew, between = plans[i], plans[i + 1:j - 1]
+            # the filters move up to the outer product, or the outer product down to them
+            if not any(conflict(lf, q) for q in between):
+                at = i
+            elif not any(conflict(ew, q) for q in between):
+                at = j - 2
+            else:
+                continue
+            fused = self.backend.fuse_outer_filter(ew, lf)
+            if fused is None:
+                continue
+            fused.reads_mem = ew.reads_mem | lf.reads_mem
+            fused.writes_mem = ew.writes_mem | lf.writes_mem
+            del plans[j - 1]
+            del plans[i]
+            plans.insert(at, fused)
+            j -= 1
+        return plans
 
     def _fuse_filter_epilogues(self, plans):
         """Synapse filters whose input is the output of a large GEMV item become the

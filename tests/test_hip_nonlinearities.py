@@ -12,7 +12,7 @@ not depend on the math library.
 import numpy as np
 import pytest
 
-from helpers import RA, clone, to_dev
+from helpers import RA, clone, run_plans, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -175,6 +175,106 @@ def test_elementwise_inc_outer(queue, rng, align):
         for k in range(len(Y)):
             ax = np.outer(alpha[k] * A[k].ravel(), X[k].ravel())
             assert np.array_equal(got[k], Y[k] + ax if inc else ax)
+
+
+def _outer_filter_case(queue, rng, shapes, broadcast_row=None, extra_filters=(), unfiltered=()):
+    """Device arrays and plans for "W += (alpha a) (x) f; f <- filter(s)": item k of `vec` is
+    the filter output f_k and the column operand of outer product k (products listed in
+    `unfiltered` have a column operand that no filter writes); `extra_filters` are lengths of
+    further filters that feed no product."""
+    n = len(shapes)
+    cols = [c for _, c in shapes]
+    vec = RA([rng.normal(size=c) for c in cols] + [rng.normal(size=m) for m in extra_filters],
+             align=True)
+    spikes = RA([rng.normal(size=c) for c in cols] + [rng.normal(size=m) for m in extra_filters],
+                align=True)
+    rows = [1 if k == broadcast_row else r for k, (r, _) in enumerate(shapes)]
+    A = RA([rng.normal(size=r) for r in rows], align=True)
+    W = RA([rng.normal(size=s) for s in shapes], align=True)
+    alpha = rng.normal(size=n).astype(np.float32)
+    filtered = [k for k in range(n) if k not in unfiltered] + list(range(n, n + len(extra_filters)))
+    kinds = ["lowpass" if k % 3 else "gain" for k in range(len(filtered))]
+    coefs = [_filter_coefficients(kind) for kind in kinds]
+    FA, FB = RA([den for _, den in coefs]), RA([num for num, _ in coefs])
+    sizes = [vec.sizes[k] for k in filtered]
+    Xbuf = RA([np.zeros((1, m)) for m in sizes])
+    Ybuf = RA([np.zeros((len(den), m)) for (_, den), m in zip(coefs, sizes)])
+    return dict(vec=vec, spikes=spikes, A=A, W=W, alpha=alpha, FA=FA, FB=FB, Xbuf=Xbuf, Ybuf=Ybuf,
+                filtered=filtered, n=n)
+
+
+def _outer_filter_plans(queue, case, where):
+    """(weights, vectors, spikes, [outer-product plan, filter plan]) on the device
+    (`where` = the device module) or on the host (the oracle module)."""
+    c, n, filtered = case, case["n"], case["filtered"]
+    if where is nl():
+        put = lambda ra: to_dev(queue, ra)
+        q = queue
+    else:
+        put, q = clone, None
+    vec, spikes, W = put(c["vec"]), put(c["spikes"]), put(c["W"])
+    A, FA, FB = put(c["A"]), put(c["FA"]), put(c["FB"])
+    ew = where.plan_elementwise_inc(q, A, vec[list(range(n))], W, alpha=c["alpha"], outer=True,
+                                    inc=True)
+    lf = where.plan_linearfilter(q, spikes[filtered], vec[filtered], FA, FB, put(c["Xbuf"]),
+                                 put(c["Ybuf"]))
+    return W, vec, spikes, [ew] + list(lf)
+
+
+def test_outer_product_with_the_filter_of_its_column_operand(queue, rng):
+    """`nhip_outer_filter`: the weight update of a learning rule and the filter step of the
+    activities it has just read, in one launch, against the two launches it replaces and
+    against the oracle's two kernels -- bit for bit over several calls with fresh filter
+    inputs.  Shapes: the benchmark's 32 x 2000, tiles that are not full, a single row, a row
+    operand that is one value for all rows, a product whose column operand nothing filters,
+    filters that feed no product."""
+    shapes = [(32, 2000), (8, 128), (256, 4), (1, 260), (17, 64), (5, 388)]
+    case = _outer_filter_case(queue, rng, shapes, broadcast_row=4, extra_filters=(300, 5),
+                              unfiltered=(1,))
+    W1, vec1, spikes1, two = _outer_filter_plans(queue, case, nl())
+    W2, vec2, spikes2, pair = _outer_filter_plans(queue, case, nl())
+    Wo, veco, spikeso, oplans = _outer_filter_plans(queue, case, orc())
+    fused = nl().fuse_outer_filter(pair[0], pair[1])
+    assert fused is not None and fused.name == "hip_outer_filter"
+    assert fused.fused_filters == [0, 1, 2, 3, 4]  # the filters of products 0, 2, 3, 4, 5
+    for call in range(4):
+        for k in range(len(case["spikes"])):
+            fresh = rng.normal(size=case["spikes"].sizes[k]).astype(np.float32)
+            spikes1[k] = fresh
+            spikes2[k] = fresh
+            spikeso[k] = fresh[:, None]
+        run_plans(two)
+        fused()
+        run_plans(oplans)
+        assert np.array_equal(W2.buf, W1.buf) and np.array_equal(vec2.buf, vec1.buf), call
+        assert np.array_equal(W2.buf, Wo.buf) and np.array_equal(vec2.buf, veco.buf), call
+    assert not np.array_equal(W2.buf, case["W"].buf)
+
+
+def test_outer_product_and_filter_stay_apart_where_the_launch_cannot_take_them(queue, rng):
+    # a filter output read by two outer products: neither work-group may overwrite it
+    case = _outer_filter_case(queue, rng, [(8, 64), (8, 64)])
+    W, vec, spikes, (ew, lf) = _outer_filter_plans(queue, case, nl())
+    A = to_dev(queue, case["A"])
+    shared = nl().plan_elementwise_inc(queue, A, vec[[0, 0]], W, alpha=case["alpha"], outer=True)
+    assert nl().fuse_outer_filter(shared, lf) is None
+    assert nl().fuse_outer_filter(ew, lf) is not None
+    # more rows than a work-group's tile takes; rows that are not whole quads
+    for shapes in ([(300, 64)], [(8, 66)]):
+        case = _outer_filter_case(queue, rng, shapes)
+        _, _, _, (ew, lf) = _outer_filter_plans(queue, case, nl())
+        assert nl().fuse_outer_filter(ew, lf) is None
+    # a second-order filter
+    case = _outer_filter_case(queue, rng, [(8, 64)])
+    num, den = _filter_coefficients("alpha")
+    case["FA"], case["FB"] = RA([den]), RA([num])
+    case["Xbuf"], case["Ybuf"] = RA([np.zeros((len(num), 64))]), RA([np.zeros((len(den), 64))])
+    _, _, _, (ew, lf) = _outer_filter_plans(queue, case, nl())
+    assert nl().fuse_outer_filter(ew, lf) is None
+    # an element-wise product that is no outer product
+    d = to_dev(queue, RA([rng.normal(size=(4, 8))] * 3))
+    plain = nl().plan_elementwise_inc(queue, d[[0]], d[[1]], d[[2]])
+    assert nl().fuse_outer_filter(plain, lf) is None
 
 
 def test_reset(queue, rng):

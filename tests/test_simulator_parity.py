@@ -344,6 +344,10 @@ def test_other_configurations_full_size_state_bit_exact(queue, case):
     net_o, probes_o, _ = make()
     with Simulator(net, seed=1, dedup=False) as gpu, \
             OracleSimulator(net_o, seed=1, dedup=False) as cpu:
+        if case == "c4":
+            # the weight update runs together with the filter of the activities it reads
+            names = [p.name for p in gpu._plans]
+            assert "hip_outer_filter" in names and "hip_elementwise_inc" not in names
         gpu.run_steps(30)
         cpu.run_steps(30)
         for key in probes:
@@ -693,7 +697,7 @@ def test_function_nodes_run_on_the_device(queue):
         assert np.abs(gpu.data[probes[1]]).max() > 0.1
 
 
-def test_c4_pes_learning_in_place(queue):
+def test_c4_pes_learning_in_place(queue, monkeypatch):
     """The PES network with `learn_in_place=True` (the rule adds its change to the decoders
     in one pass): the device follows the oracle simulator bit for bit, and both reproduce
     the probe data of the two-pass form exactly."""
@@ -703,14 +707,23 @@ def test_c4_pes_learning_in_place(queue):
 
     make = lambda: configs.c4_pes(n_triples=3, n_neurons=300, dims=8, solver="lstsq",
                                   learning_rate=3e-4, sample_every=None)
-    nets = [make() for _ in range(3)]
+    nets = [make() for _ in range(4)]
+    monkeypatch.setenv("NENGO_HIP_OUTER_FILTER", "0")
+    apart = Simulator(nets[3][0], seed=1, learn_in_place=True)
+    monkeypatch.delenv("NENGO_HIP_OUTER_FILTER")
     with Simulator(nets[0][0], seed=1, learn_in_place=True) as gpu, \
             OracleSimulator(nets[1][0], seed=1, learn_in_place=True) as cpu, \
-            Simulator(nets[2][0], seed=1, learn_in_place=False) as two_pass:
+            Simulator(nets[2][0], seed=1, learn_in_place=False) as two_pass, apart:
         assert sum(p.name == "hip_copy" for p in gpu._plans) < sum(
             p.name == "hip_copy" for p in two_pass._plans)
-        for sim in (gpu, cpu, two_pass):
+        # the weight update runs the filter of the activities it has read; switched off,
+        # the two are launches of their own: one launch more, the same bits
+        assert any(p.name == "hip_outer_filter" for p in gpu._plans)
+        assert not any(p.name == "hip_outer_filter" for p in apart._plans)
+        assert len(apart._plans) == len(gpu._plans) + 1
+        for sim in (gpu, cpu, two_pass, apart):
             sim.run_steps(400)
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(apart.all_data.buf))
         for key in nets[0][1]:
             assert np.array_equal(gpu.data[nets[0][1][key]], cpu.data[nets[1][1][key]])
             assert np.array_equal(gpu.data[nets[0][1][key]], two_pass.data[nets[2][1][key]])
