@@ -1156,15 +1156,30 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                 // Y = 0 * Y + sum_k v_k * s_k (one-column dot products, alpha = 1,
                 // gamma = 0).  The wave that has the item's first rows also stores the sum
                 // where the separate launch would have (the X operand's own place).
+                // Two dependent reads for up to four parts (records, then operands), one more
+                // per further four: lane k fetches the record and the scalar of part k (one
+                // coalesced read each), the vectors' addresses reach the other lanes through
+                // readlane, and the vector elements of four parts are requested together.
                 const int c = min(lane, last_cols - 1);
                 float s = 0.0f;
-                for (int q0 = 0; q0 < it.pad; q0 += 2) {  // (two parts requested together)
-                    const int2 p0 = epi.lif.parts[task.pad + q0];
-                    const int2 p1 = epi.lif.parts[task.pad + min(q0 + 1, it.pad - 1)];
-                    const float v0 = X[(size_t)p0.x + c], w0 = X[p0.y];
-                    const float v1 = X[(size_t)p1.x + c], w1 = X[p1.y];
-                    s = s + fmaf(v0, w0, 0.0f);
-                    if (q0 + 1 < it.pad) s = s + fmaf(v1, w1, 0.0f);
+                for (int q0 = 0; q0 < it.pad; q0 += NHIP_WAVE) {
+                    const int m = min(it.pad - q0, NHIP_WAVE);  // uniform
+                    const int2 mine = epi.lif.parts[task.pad + q0 + min(lane, m - 1)];
+                    const float my_w = X[mine.y];
+                    for (int k0 = 0; k0 < m; k0 += 4) {
+                        float v[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int px = __builtin_amdgcn_readlane(mine.x, min(k0 + u, m - 1));
+                            v[u] = X[(size_t)px + c];
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const float w = __int_as_float(__builtin_amdgcn_readlane(
+                                __float_as_int(my_w), min(k0 + u, m - 1)));
+                            if (k0 + u < m) s = s + fmaf(v[u], w, 0.0f);
+                        }
+                    }
                 }
                 xq0[0] = s;
                 if (task.row0 == 0 && lane < last_cols) Y[(size_t)dot.x_start + lane] = s;
