@@ -75,7 +75,10 @@ int nhip_device_info(int *n_cu, int *wave_size, int *lds_bytes, char *name, int 
  * small items: every task is ONE row (n_rows == 1), a wave takes 64 / lpr consecutive
  * tasks of whatever items; lpr 4 (any widths) or 1 (every dot product of the launch
  * has at most 4 columns), vec 1: bit-identical to a float32
- * restatement of that kernel.  `lpr` = lanes cooperating on one row (1,2,...,64, or
+ * restatement of that kernel.  With lpr 64 (and 16-word task records) the launch is the
+ * lpr 1 one with tasks of up to 64 consecutive rows of one item (n_rows <= 64) that a wave
+ * takes whole, lane l the row row0 + l: the records are then read once per wave instead
+ * of once per row, and the parts of an input sum are fetched by the lanes side by side.  `lpr` = lanes cooperating on one row (1,2,...,64, or
  * 256 for flavor 0); `vec` = 4 (16-byte loads; needs a_start % 4 == 0 and
  * a_stride0 % 4 == 0 for every dot of the launch) or 1.  `passes` (flavor 0) =
  * rows each lane accumulates at once, i.e. independent loads in flight: 2, 4, 8,
@@ -188,14 +191,14 @@ int nhip_gemv_tile_filter(void *stream, int vec, int pow2_cols, int blk_words, c
                           const int *item_targets, const int *targets, float *F);
 
 /* The same two epilogues for launches of small items (nhip_gemv with flavor 2, whose
- * `items`, `coefs`, `dots` and `tasks` tables these take; `lpr` 4 or 1): the
+ * `items`, `coefs`, `dots` and `tasks` tables these take; `lpr` 4, 1 or 64): the
  * neuron update / filter step of a row runs in the lane that holds the row's sum.
  * `pops`, `item_targets`, `targets` and the other arguments as above.
  * `task_words` = 4: tasks as for nhip_gemv.  = 16: every task record also holds its
  * item and coefficients (a launch of a few thousand rows is a chain of dependent
  * reads, and this takes one out of it; nhip_gemv takes such tables for flavor 2
  * with `passes` = 16):
- *   tasks : int32[n_tasks][16] {item, row0, 1, e0,  the item's row of `items` with its
+ *   tasks : int32[n_tasks][16] {item, row0, 1 (lpr 64: n_rows), e0,  the item's row of `items` with its
  *                               last word = e1,  alpha, beta, gamma (float bits), e2}
  * e0, e1, e2 let the epilogue start its own reads at once: nhip_gemv_rows_lif
  * v_start, w_start, pflags of the item's row of `pops`; nhip_gemv_rows_filter first

@@ -262,20 +262,20 @@ __host__ inline bool take_carried(RowsSide& side) {
 
 // (SIDE: the instance for launches that carry a sequence; the others are compiled without
 // that path and its LDS)
-template <int LPR, bool WIDE, bool SIDE>
+template <int LPR, bool WIDE, bool SIDE, bool WAVE_TASK = false>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     const float* A, const float* X, const float* Yin, float* Y, const RowsSide side)
 {
     if (SIDE) NHIP_ROWS_SIDE_GROUP(side)
-    gemv_rows_ref_block<LPR, EPI_NONE, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
-                                             blockIdx.x, threadIdx.x);
+    gemv_rows_ref_block<LPR, EPI_NONE, WIDE, WAVE_TASK>(items, coefs, dots, tasks, n_tasks, A, X, Yin,
+                                                    Y, blockIdx.x, threadIdx.x);
 }
 
 // the same with an epilogue per finished row (A, X, Yin are not marked read-only
 // here either: the epilogue writes neuron state / filter outputs into the same buffer)
-template <int LPR, int EPI, bool WIDE, bool SIDE>
+template <int LPR, int EPI, bool WIDE, bool SIDE, bool WAVE_TASK = false>
 __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_epi_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
@@ -283,8 +283,8 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_epi_kernel(
     const RowsSide side)
 {
     if (SIDE) NHIP_ROWS_SIDE_GROUP(side)
-    gemv_rows_ref_block<LPR, EPI, WIDE>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
-                                        blockIdx.x, threadIdx.x, &epi);
+    gemv_rows_ref_block<LPR, EPI, WIDE, WAVE_TASK>(items, coefs, dots, tasks, n_tasks, A, X, Yin, Y,
+                                               blockIdx.x, threadIdx.x, &epi);
 }
 
 template <int EPI>
@@ -297,8 +297,9 @@ int launch_rows_epi(hipStream_t s, int lpr, int task_words, const int* items, co
     if (n_tasks == 0) return 0;
     if (n_tasks < 0 || !items || !coefs || !dots || !tasks || !A || !X || !Yin || !Y)
         return NHIP_E_BADARG;
-    if (lpr != 4 && lpr != 1) return NHIP_E_BADCLASS;
+    if (lpr != 4 && lpr != 1 && lpr != NHIP_WAVE) return NHIP_E_BADCLASS;
     if (task_words != 4 && task_words != 16) return NHIP_E_BADARG;
+    if (lpr == NHIP_WAVE && task_words != 16) return NHIP_E_BADARG;  // tasks of up to 64 rows
     const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
     side.n_gemv_groups = (n_tasks + rows_per_group - 1) / rows_per_group;
     const dim3 grid(side.n_gemv_groups + side.n_chains);
@@ -309,7 +310,8 @@ int launch_rows_epi(hipStream_t s, int lpr, int task_words, const int* items, co
     };
     auto pick = [&](auto side_tag) {
         constexpr bool SD = decltype(side_tag)::value;
-        if (lpr == 4 && task_words == 16) launch(gemv_rows_ref_epi_kernel<4, EPI, true, SD>);
+        if (lpr == NHIP_WAVE) launch(gemv_rows_ref_epi_kernel<1, EPI, true, SD, true>);
+        else if (lpr == 4 && task_words == 16) launch(gemv_rows_ref_epi_kernel<4, EPI, true, SD>);
         else if (lpr == 4) launch(gemv_rows_ref_epi_kernel<4, EPI, false, SD>);
         else if (task_words == 16) launch(gemv_rows_ref_epi_kernel<1, EPI, true, SD>);
         else launch(gemv_rows_ref_epi_kernel<1, EPI, false, SD>);
@@ -423,8 +425,9 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
             NHIP_WG_CASE(256)
         }
     } else if (flavor == 2) {
-        if ((lpr != 4 && lpr != 1) || vec != 1) return NHIP_E_BADCLASS;
+        if ((lpr != 4 && lpr != 1 && lpr != NHIP_WAVE) || vec != 1) return NHIP_E_BADCLASS;
         if (passes != 0 && passes != 16) return NHIP_E_BADARG;  // words of a task record
+        if (lpr == NHIP_WAVE && passes != 16) return NHIP_E_BADARG;  // tasks of up to 64 rows
         const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / lpr);
         side.n_gemv_groups = (n_tasks + rows_per_group - 1) / rows_per_group;
         const dim3 grid(side.n_gemv_groups + side.n_chains);
@@ -436,7 +439,8 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
         };
         auto pick = [&](auto side_tag) {
             constexpr bool SD = decltype(side_tag)::value;
-            if (lpr == 4 && passes == 16) launch(gemv_rows_ref_kernel<4, true, SD>);
+            if (lpr == NHIP_WAVE) launch(gemv_rows_ref_kernel<1, true, SD, true>);
+            else if (lpr == 4 && passes == 16) launch(gemv_rows_ref_kernel<4, true, SD>);
             else if (lpr == 4) launch(gemv_rows_ref_kernel<4, false, SD>);
             else if (passes == 16) launch(gemv_rows_ref_kernel<1, true, SD>);
             else launch(gemv_rows_ref_kernel<1, false, SD>);

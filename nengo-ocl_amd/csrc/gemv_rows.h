@@ -31,7 +31,13 @@
 // fed by the row (the same epilogues as the kernel for large items has; small
 // populations and low-dimensional decoded values save a launch the same way).
 // WIDE: the task table holds GemvRowTask records.
-template <int LPR, int EPI = EPI_NONE, bool WIDE = false>
+// WAVE_TASK (with LPR = 1 and WIDE): a task is up to 64 consecutive rows of one item (n_rows) and
+// takes a whole wave, lane l the row row0 + l.  Launches of very many thin rows (hundreds of
+// thousands of neurons of one- to four-dimensional populations) otherwise read a record per
+// row; here the record is the wave's: every lane reads the same addresses for the task, the
+// item's dot products, its population and its input sum, and the parts of an input sum are
+// fetched by the lanes side by side instead of in rounds.
+template <int LPR, int EPI = EPI_NONE, bool WIDE = false, bool WAVE_TASK = false>
 __device__ __forceinline__ void gemv_rows_ref_block(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
@@ -43,10 +49,12 @@ __device__ __forceinline__ void gemv_rows_ref_block(
     constexpr int CHUNK = 8;             // steps of a partial sum whose operands are fetched together
     constexpr int ROWS = NHIP_WAVE / LPR;  // rows (tasks) per wave
     constexpr int PER_LANE = 4 / LPR;    // elements of a <= 4 column dot product per lane
+    static_assert(!WAVE_TASK || (LPR == 1 && WIDE), "tasks of several rows: one lane per row, wide records");
     const int lane = tid & (NHIP_WAVE - 1);
     const int lir = lane % LPR;
-    const int slot = (block * (NHIP_WG / NHIP_WAVE) + (tid >> 6)) * ROWS + lane / LPR;
-    const bool valid = slot < n_tasks;
+    const int wave_slot = block * (NHIP_WG / NHIP_WAVE) + __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slot = WAVE_TASK ? wave_slot : wave_slot * ROWS + lane / LPR;
+    bool valid = slot < n_tasks;
     GemvTask task;
     GemvItem it;
     float4 cf;
@@ -62,7 +70,11 @@ __device__ __forceinline__ void gemv_rows_ref_block(
         it = items[task.item];
         cf = coefs[task.item];
     }
-    const int r = task.row0;
+    int r = task.row0;
+    if (WAVE_TASK) {  // a lane past the task's rows keeps the last row's addresses and stores nothing
+        valid = valid && lane < task.n_rows;
+        r = task.row0 + min(lane, task.n_rows - 1);
+    }
     const int n_dots = valid ? it.n_dots : 0;
     // epilogue operands, fetched ahead (no branch around the loads: a row without a
     // population or a target reads the first element of the buffer instead)
@@ -90,12 +102,53 @@ __device__ __forceinline__ void gemv_rows_ref_block(
     // (...(0 + v_0[c] s_0) + v_1[c] s_1) + ..., what this kernel computes for
     // Y = 0 * Y + sum_k v_k s_k as a launch of its own
     int2 sum_range = make_int2(0, 0);
-    if (EPI == EPI_LIF && epi->lif.sum_ranges != nullptr && valid)
+    if (EPI == EPI_LIF && epi->lif.sum_ranges != nullptr && (WAVE_TASK ? slot < n_tasks : valid))
         sum_range = epi->lif.sum_ranges[task.item];
+    if (WAVE_TASK)  // the same for all lanes of the wave (the lanes past the task's rows take part)
+        sum_range = make_int2(__builtin_amdgcn_readfirstlane(sum_range.x),
+                              __builtin_amdgcn_readfirstlane(sum_range.y));
+    // WAVE_TASK: element c of the sum with c the same for all lanes (the vector operand of a dot
+    // product): lane k fetches the record, the scalar and element c of part k and forms
+    // their product -- two dependent reads however many parts there are -- and the products
+    // are added in order
+    auto summed_uniform = [&](int c) {
+        float s = 0.0f;
+        for (int q0 = 0; q0 < sum_range.y; q0 += NHIP_WAVE) {
+            const int m = min(sum_range.y - q0, NHIP_WAVE);
+            const int2 mine = epi->lif.parts[sum_range.x + q0 + min(lane, m - 1)];
+            const float p = fmaf(X[(size_t)mine.x + c], X[mine.y], 0.0f);
+            for (int k = 0; k < m; ++k)
+                s = s + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), k));
+        }
+        return s;
+    };
     auto summed = [&](int c) {
+        float s = 0.0f;
+        if (WAVE_TASK) {
+            // element c of the sum with c the lane's own (rows of an item that is a sum):
+            // lane k fetches the record and the scalar of part k, the vector elements of
+            // four parts are requested together
+            for (int q0 = 0; q0 < sum_range.y; q0 += NHIP_WAVE) {
+                const int m = min(sum_range.y - q0, NHIP_WAVE);
+                const int2 mine = epi->lif.parts[sum_range.x + q0 + min(lane, m - 1)];
+                const float my_w = X[mine.y];
+                for (int k0 = 0; k0 < m; k0 += 4) {
+                    float v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        v[u] = X[(size_t)__builtin_amdgcn_readlane(mine.x, min(k0 + u, m - 1)) + c];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float w = __int_as_float(__builtin_amdgcn_readlane(
+                            __float_as_int(my_w), min(k0 + u, m - 1)));
+                        if (k0 + u < m) s = s + fmaf(v[u], w, 0.0f);
+                    }
+                }
+            }
+            return s;
+        }
         // (the records of four parts, then their operands, are requested together: the
         // launch is a chain of dependent reads, and this keeps it two links per four parts)
-        float s = 0.0f;
         for (int q0 = 0; q0 < sum_range.y; q0 += 4) {
             int2 part[4];
             float v[4], w[4];
@@ -113,7 +166,9 @@ __device__ __forceinline__ void gemv_rows_ref_block(
         }
         return s;
     };
-    if (EPI == EPI_LIF && sum_range.y > 0 && n_dots == 0) sum = summed(r);
+    // (WAVE_TASK: the whole wave forms the sum, also the lanes past the task's rows, whose reads
+    // the others use; the condition is the same for all of them)
+    if (EPI == EPI_LIF && sum_range.y > 0 && (WAVE_TASK ? it.n_dots == 0 : n_dots == 0)) sum = summed(r);
 
     for (int d0 = 0; __any(d0 < n_dots); d0 += BATCH) {
         GemvDot dot[BATCH];
@@ -133,7 +188,15 @@ __device__ __forceinline__ void gemv_rows_ref_block(
                     const bool live = d0 + k < n_dots && c < dot[k].N;
                     a[k][e] = live ? A[dot[k].a_start + (size_t)r * dot[k].a_stride0 + c] : 0.0f;
                     x[k][e] = live ? X[dot[k].x_start + (size_t)c * dot[k].x_stride0] : 0.0f;
-                    if (EPI == EPI_LIF && k == 0 && d0 == 0 && live && sum_range.y > 0) {
+                    if (WAVE_TASK && EPI == EPI_LIF && k == 0 && d0 == 0 && sum_range.y > 0 &&
+                        __any(live)) {
+                        // (all lanes of the wave run the sum: its reads are spread over them)
+                        const float xs = summed_uniform(c);
+                        if (live) {
+                            x[k][e] = xs;
+                            if (r == 0) Y[(size_t)dot[k].x_start + c] = xs;
+                        }
+                    } else if (EPI == EPI_LIF && k == 0 && d0 == 0 && live && sum_range.y > 0) {
                         x[k][e] = summed(c);
                         // the item's first row also stores the sum in the operand's place
                         if (r == 0) Y[(size_t)dot[k].x_start + c] = x[k][e];

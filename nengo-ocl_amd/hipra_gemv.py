@@ -87,6 +87,9 @@ def stream_stage(n_cols):
 # small-item launches of at most this many rows get task records with the item and its
 # coefficients inline (they are chains of dependent reads; larger ones are about traffic)
 WIDE_TASK_MAX_ROWS = 65536
+# launches with a lane per row: a wave takes a task of up to 64 rows of one item (switch for
+# measurements: "0" keeps a task record per row)
+WAVE_TASKS = os.environ.get("NENGO_HIP_WAVE_TASKS", "1") != "0"
 WG, WAVE = 256, 64
 THIN_MIN_ROWS, THIN_ROWS_FOR_LANE_PER_ROW = 32, 65536
 LIF_POP_ENABLED, LIF_POP_DECAY = 1 << 8, 1 << 9  # flag bits of a population row
@@ -532,7 +535,16 @@ class gemv_prog:
                     M = geometry[b]["y_len"]
                     for r0 in range(0, M, rows):
                         task_rows.append((b, r0, min(rows, M - r0), 0))
-            if flavor == 2:  # built with numpy: there can be millions of rows
+            lpr_arg = lpr
+            if flavor == 2 and lpr == 1 and WAVE_TASKS:
+                # a lane per row: tasks of up to 64 consecutive rows of an item that a wave
+                # takes whole, so that the records are the wave's and not each row's
+                lpr_arg = WAVE
+                task_rows = np.array([(b, r0, min(WAVE, geometry[b]["y_len"] - r0), 0)
+                                      for b in members
+                                      for r0 in range(0, geometry[b]["y_len"], WAVE)],
+                                     dtype=np.int32).reshape(-1, 4)
+            elif flavor == 2:  # built with numpy: there can be millions of rows
                 counts = np.array([geometry[b]["y_len"] for b in members], dtype=np.int64)
                 task_tab = np.zeros((int(counts.sum()), 4), dtype=np.int32)
                 task_tab[:, 0] = np.repeat(np.array(members, dtype=np.int32), counts)
@@ -540,7 +552,7 @@ class gemv_prog:
                 task_tab[:, 2] = 1
                 task_rows = task_tab
             task_tab = np.array(task_rows, dtype=np.int32)
-            if flavor == 2 and 0 < len(task_tab) <= WIDE_TASK_MAX_ROWS:
+            if flavor == 2 and (0 < len(task_tab) <= WIDE_TASK_MAX_ROWS or lpr_arg == WAVE):
                 which = task_tab[:, 0]
                 wide = np.zeros((len(task_tab), 16), dtype=np.int32)
                 wide[:, 0:4] = task_tab
@@ -565,7 +577,7 @@ class gemv_prog:
             if flavor == 0:
                 n_groups = n_tasks
             elif flavor == 2:
-                n_groups = -(-n_tasks // ((WG // WAVE) * (WAVE // lpr)))
+                n_groups = -(-n_tasks // ((WG // WAVE) * (WAVE // lpr_arg)))
             else:
                 n_groups = -(-n_tasks // (WG // WAVE))
             tail = (dev_items.ptr, dev_coefs.ptr, dev_dots.ptr, dev_tasks.ptr, n_tasks, self.A.ptr,
@@ -573,7 +585,7 @@ class gemv_prog:
             if flavor == 3:
                 kern, args = lib.nhip_gemv_tile, (vec, lpr, TILE_STAGE_WORDS) + tail
             else:
-                kern, args = lib.nhip_gemv, (flavor, lpr, vec, passes) + tail
+                kern, args = lib.nhip_gemv, (flavor, lpr_arg, vec, passes) + tail
             plan = Plan(
                 self.queue, kern, args, gsize=(WG * n_groups,), lsize=(WG,),
                 full_args=(dev_items, dev_coefs, dev_dots, dev_tasks, self.A.dev_buf,
@@ -962,6 +974,10 @@ def fuse_input_sums(sum_plan, lif_plan):
             items[b] = (start, 1, start, 1, 0, 0, n, 0)
             coefs[b] = (1.0, 0.0, 0.0, 0.0)
             ranges[b] = where[start]
+            if lpr == WAVE:  # a wave takes a task of up to 64 rows: the whole sum
+                extra.append(np.concatenate([[b, 0, n, 0], items[b], one]).astype(np.int32))
+                extra[-1][15] = 0
+                continue
             for r in range(n):
                 if task_words == 16:
                     extra.append(np.concatenate([[b, r, 1, 0], items[b], one]).astype(np.int32))

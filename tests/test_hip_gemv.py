@@ -784,12 +784,15 @@ def test_sparse_products(queue):
         hipra_spmv.plan_sparse_dot_inc(queue, mats[:2], dX[[0, 2]], dY[[0, 1]])
 
 
-def test_thin_items_lane_per_row(queue):
-    """Many rows of dot products with one to four columns take the lane-per-row class:
-    bit-identical to the oracle for sums of several such terms, strided operands and
-    a scalar X shared by all rows."""
+@pytest.mark.parametrize("wave_tasks", [True, False], ids=["wave-tasks", "row-tasks"])
+def test_thin_items_lane_per_row(queue, monkeypatch, wave_tasks):
+    """Many rows of dot products with one to four columns take the lane-per-row class (a
+    wave per task of up to 64 rows, or a task record per row): bit-identical to the oracle
+    for sums of several such terms, strided operands and a scalar X shared by all rows."""
     from nengo_ocl_amd import hipra_gemv as g
     from oracle import oracle as orc
+
+    monkeypatch.setattr(g, "WAVE_TASKS", wave_tasks)
 
     rng = np.random.RandomState(17)
     shapes = [(40000, 1), (30000, 4), (5000, 3), (33, 2)]
@@ -807,6 +810,7 @@ def test_thin_items_lane_per_row(queue):
         prog = g.plan_block_gemv(queue, 1.0, to_dev(queue, A), js, to_dev(queue, X), js, beta, dY,
                                  gamma=gamma)
         assert {p.kernel_class for p in prog.plans} == {(2, 1, 1)}
+        assert {p.args[1] for p in prog.plans} == {64 if wave_tasks else 1}
         for plan in prog.plans:
             plan()
         assert np.array_equal(dY.buf, Yo.buf)
@@ -1133,13 +1137,17 @@ def test_gemv_lif_forms_its_input_sums(queue):
     assert all(g.fuse_input_sums(sums2.plans[0], p) is None for p in with_lif2)
 
 
-@pytest.mark.parametrize("n_ens", [24, 700], ids=["inline-task-records", "plain-task-records"])
-def test_small_item_lif_forms_its_input_sums(queue, n_ens):
+@pytest.mark.parametrize("n_ens, wave_tasks", [(24, True), (700, True), (700, False)],
+                         ids=["inline-task-records", "wave-tasks", "plain-task-records"])
+def test_small_item_lif_forms_its_input_sums(queue, monkeypatch, n_ens, wave_tasks):
     """The same fusion for ensembles of 100 neurons with 1-D and 2-D inputs (the small-item
-    kernel; task records with the item inline for few rows, plain ones for many): sums of
-    one to twelve terms, a sum nothing reads, several steps with changing sources -- all
-    bit-identical to the oracle's three kernels."""
+    kernel; a row per task with the item inline in its record for few rows; for many rows a
+    lane per row, with tasks of up to 64 rows that a wave takes whole or, that switched off,
+    a plain record per row): sums of one to twelve terms, a sum nothing reads, several steps
+    with changing sources -- all bit-identical to the oracle's three kernels."""
     from nengo_ocl_amd import hipra_gemv as g
+
+    monkeypatch.setattr(g, "WAVE_TASKS", wave_tasks)
     from nengo_ocl_amd import hipra_nonlinearities as nl
     from oracle import oracle as orc
 
@@ -1191,10 +1199,17 @@ def test_small_item_lif_forms_its_input_sums(queue, n_ens):
     assert [p.name for p in sums.plans] == ["hipra_gemv.wave_ref"]
     with_lif = g.fuse_lif(encs, lif)
     assert [p.name for p in with_lif] == ["hipra_gemv.wave_ref_lif"]
-    assert (with_lif[0].args[1] == 16) == (n_ens == 24)  # words of a task record
+    lanes, task_words = with_lif[0].args[:2]
+    if n_ens == 24:
+        assert (lanes, task_words) == (4, 16)
+    else:  # a lane per row: 64 rows per task with the item inline, or a plain record per row
+        assert with_lif[0].kernel_class == (2, 1, 1)
+        assert (lanes, task_words) == ((64, 16) if wave_tasks else (1, 4))
+        assert with_lif[0].n_tasks == (2 * n_ens if wave_tasks else 100 * n_ens)
     fused = g.fuse_input_sums(sums.plans[0], with_lif[0])
     assert fused is not None and fused.input_sums == n_ens + 1
-    assert fused.n_tasks == with_lif[0].n_tasks + 2      # two rows of the sum nothing reads
+    # the sum nothing reads: two rows of their own, or one task of two rows
+    assert fused.n_tasks == with_lif[0].n_tasks + (1 if lanes == 64 else 2)
     osums, oencs, olif = build(host, orc, orc, None)
     for step in range(3):
         fused()
