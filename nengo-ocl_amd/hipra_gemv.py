@@ -540,10 +540,14 @@ class gemv_prog:
                 # a lane per row: tasks of up to 64 consecutive rows of an item that a wave
                 # takes whole, so that the records are the wave's and not each row's
                 lpr_arg = WAVE
-                task_rows = np.array([(b, r0, min(WAVE, geometry[b]["y_len"] - r0), 0)
-                                      for b in members
-                                      for r0 in range(0, geometry[b]["y_len"], WAVE)],
-                                     dtype=np.int32).reshape(-1, 4)
+                lens = np.array([geometry[b]["y_len"] for b in members], dtype=np.int64)
+                per_item = -(-lens // WAVE)  # (built with numpy: there can be millions of rows)
+                first = np.cumsum(per_item) - per_item
+                row0 = (np.arange(int(per_item.sum())) - np.repeat(first, per_item)) * WAVE
+                task_rows = np.zeros((len(row0), 4), dtype=np.int32)
+                task_rows[:, 0] = np.repeat(np.array(members, dtype=np.int32), per_item)
+                task_rows[:, 1] = row0
+                task_rows[:, 2] = np.minimum(WAVE, np.repeat(lens, per_item) - row0)
             elif flavor == 2:  # built with numpy: there can be millions of rows
                 counts = np.array([geometry[b]["y_len"] for b in members], dtype=np.int64)
                 task_tab = np.zeros((int(counts.sum()), 4), dtype=np.int32)
