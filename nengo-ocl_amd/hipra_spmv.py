@@ -9,6 +9,8 @@ reads values and column indices 16 bytes at a time, a wave in contiguous 1-KiB r
 while each lane sums its row in column order.
 """
 
+import os
+
 import numpy as np
 
 from .hipraggedarray import to_device
@@ -109,6 +111,13 @@ class plan_sparse_dot_inc:
     """
 
     def __init__(self, queue, hA, X, Y, inc=False, tag=None, algorithm=None, x_mostly_zero=False):
+        # `algorithm` / NENGO_OCL_SPMV_ALGORITHM name one of the reference's planners
+        # (clra_gemv.py:1937-1948); an unknown name is an error as there, a known one
+        # changes nothing: they all are this launch
+        if algorithm is None:
+            algorithm = os.environ.get("NENGO_OCL_SPMV_ALGORITHM", None)
+        if algorithm is not None and algorithm not in algostr_to_planner:
+            raise KeyError(algorithm)
         matrices = list(hA) if isinstance(hA, (list, tuple)) else [hA]
         matrices = [m if isinstance(m, HostSparseMatrix) else HostSparseMatrix(m) for m in matrices]
         if not (len(matrices) == len(X) == len(Y)):
@@ -168,6 +177,64 @@ class plan_sparse_dot_inc:
         plan.description = "groups: %d; nonzeros: %d; stored: %d" % (len(matrices), nnz, vals.size)
         self.plans = [plan]
         self.matrices = matrices
+
+
+# The reference's planner classes (clra_gemv.py:1249-1567) differ in the storage format of
+# the matrix (CSR, ELLPACK) and in how a row's products are reduced (one lane per row, a tree
+# in LDS, two steps through global memory); its `plan_sparse_dot_inc` picks one from the
+# ELLPACK footprint (padding every row to the longest can cost many times the CSR arrays).
+# The sliced layout here pads a row only to the longest of its 64-row slice, so there is no
+# such trade-off to decide and every name takes the same launch -- same constructor, same
+# results (each row summed in column order); the names are kept so that code and tests
+# written against the reference's planners run unchanged.
+class spmv_prog(plan_sparse_dot_inc):
+    """Reference constructor ``(queue, hA, X, Y, inc=False, tag=None)`` (clra_gemv.py:1271-1279)."""
+
+    def __init__(self, queue, hA, X, Y, inc=False, tag=None):
+        super().__init__(queue, hA, X, Y, inc=inc, tag=tag)
+
+
+class plan_csr(spmv_prog):
+    """clra_gemv.py:1494-1567."""
+
+
+class plan_ellpack(spmv_prog):
+    """clra_gemv.py:1322-1408."""
+
+
+class plan_ellpack_tree(plan_ellpack):
+    """clra_gemv.py:1411-1443 (there: rows of at most one work-group's length; no such limit here)."""
+
+
+class plan_ellpack_twostep(plan_ellpack):
+    """clra_gemv.py:1446-1491."""
+
+
+#: names of `algorithm` / the NENGO_OCL_SPMV_ALGORITHM environment variable (clra_gemv.py:1991-1997)
+algostr_to_planner = {
+    "ELLPACK": plan_ellpack,
+    "ELLPACK-tree": plan_ellpack_tree,
+    "ELLPACK-twostep": plan_ellpack_twostep,
+    "CSR": plan_csr,
+}
+
+
+def spmv_algorithm_heuristic(queue, hA, footprint_hard_limit=0.8, footprint_soft_limit=0.05,
+                             soft_limit_ratio=0.1):
+    """The reference's choice between "CSR" and "ELLPACK" from the footprint of the ELLPACK
+    arrays relative to the device's memory (clra_gemv.py:1951-1988, the same rule): above the
+    hard limit CSR, below the soft limit ELLPACK, in between CSR when it is smaller than
+    `soft_limit_ratio` of ELLPACK.  Reported for callers that ask; the launch is the same."""
+    csr = hA.csr
+    ellwidth = max(np.diff(csr.indptr))
+    ell_bytes = 2 * 4 * int(ellwidth) * csr.shape[1]
+    csr_bytes = 2 * 4 * csr.nnz
+    ell_device_ratio = ell_bytes / queue.global_mem_size
+    if ell_device_ratio > footprint_hard_limit:
+        return "CSR"
+    if ell_device_ratio < footprint_soft_limit:
+        return "ELLPACK"
+    return "CSR" if csr_bytes / ell_bytes < soft_limit_ratio else "ELLPACK"
 
 
 def fuse_linearfilter(spmv_plan, lf_plan):

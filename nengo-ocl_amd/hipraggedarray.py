@@ -50,6 +50,7 @@ class Queue:
                                                  ctypes.byref(lds), name, 64), "device info")
         self.n_compute_units = max(1, n_cu.value)
         self.arch = name.value.decode()
+        self.global_mem_size = int(torch.cuda.get_device_properties(self.device).total_memory)
 
     def finish(self):
         _lib.check(self.lib.nhip_stream_sync(self.handle), "stream sync")

@@ -1137,6 +1137,43 @@ def test_gemv_lif_forms_its_input_sums(queue):
     assert all(g.fuse_input_sums(sums2.plans[0], p) is None for p in with_lif2)
 
 
+@pytest.mark.parametrize("planner", ["plan_csr", "plan_ellpack", "plan_ellpack_tree",
+                                     "plan_ellpack_twostep", "spmv_prog"])
+def test_sparse_planner_names_of_the_reference(queue, rng, planner, monkeypatch):
+    """The reference's sparse planner classes (its test_sparse is run over plan_ellpack and
+    plan_csr, tests/test_clra_gemv.py:40-49, 383-462) exist with its constructor and give
+    the oracle's product bit for bit -- also for rows longer than a work-group, which the
+    reference's tree planner refuses; `algorithm` strings are checked like there."""
+    import scipy.sparse as sp
+
+    from nengo_ocl_amd import hipra_spmv
+    from oracle import oracle as orc
+
+    shape = (2057, 5981)
+    mask = rng.uniform(size=shape) < 0.02
+    mask[rng.randint(0, shape[0], size=5), :1025] = True
+    ii, jj = mask.nonzero()
+    A = sp.coo_matrix((rng.uniform(0, 1, size=len(ii)), (ii, jj)), shape=shape).tocsr()
+    X, Y = RA([rng.uniform(0, 1, size=shape[1])]), RA([rng.uniform(0, 1, size=shape[0])])
+    hA = hipra_spmv.HostSparseMatrix(A)
+    for inc in (False, True):
+        dX, dY = to_dev(queue, X), to_dev(queue, Y)
+        prog = getattr(hipra_spmv, planner)(queue, hA, dX, dY, inc=inc)
+        for plan in prog.plans:
+            plan()
+        Yo = clone(Y)
+        orc.plan_sparse_dot_inc(None, A, X, Yo, inc=inc).plans[0]()
+        assert np.array_equal(dY.to_host()[0][:, 0], Yo[0][:, 0])
+    dX, dY = to_dev(queue, X), to_dev(queue, Y)
+    assert hipra_spmv.spmv_algorithm_heuristic(queue, hA) == "ELLPACK"
+    hipra_spmv.plan_sparse_dot_inc(queue, hA, dX, dY, algorithm="CSR")
+    with pytest.raises(KeyError):
+        hipra_spmv.plan_sparse_dot_inc(queue, hA, dX, dY, algorithm="COO")
+    monkeypatch.setenv("NENGO_OCL_SPMV_ALGORITHM", "nonsense")
+    with pytest.raises(KeyError):
+        hipra_spmv.plan_sparse_dot_inc(queue, hA, dX, dY)
+
+
 @pytest.mark.parametrize("n_ens, wave_tasks", [(24, True), (700, True), (700, False)],
                          ids=["inline-task-records", "wave-tasks", "plain-task-records"])
 def test_small_item_lif_forms_its_input_sums(queue, monkeypatch, n_ens, wave_tasks):

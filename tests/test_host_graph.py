@@ -589,3 +589,34 @@ def test_synapses_write_the_node_input_they_feed():
         naive.run_steps(100)
         for key, p in probes.items():
             assert np.array_equal(sim.data[p], naive.data(p)), key
+
+
+def test_sparse_planner_choice_follows_the_reference_rule():
+    """`spmv_algorithm_heuristic`: the cases of the reference's test_spmv_impl_heuristic
+    (tests/test_clra_gemv.py:465-492) with their answers -- an identity matrix and one with a
+    full column fit ELLPACK, one full row makes ELLPACK pad every row to the full width and
+    CSR is chosen, a small matrix is ELLPACK whatever its shape -- for a device of 8 GB; and
+    the planner names the reference's `algorithm` strings stand for."""
+    import scipy.sparse
+
+    from nengo_ocl_amd import hipra_spmv as sp
+
+    class FakeQueue:
+        global_mem_size = 8 << 30
+
+    testing_limit = 1e-7
+    bytes_limit = FakeQueue.global_mem_size * testing_limit
+    size = int(3 * (8 * bytes_limit))
+    best = scipy.sparse.eye(size, format="lil")
+    bad = best.copy()
+    bad[0, :] = 1
+    ok = best.copy()
+    ok[:, 0] = 1
+    small = scipy.sparse.eye(10, format="lil")
+    small[0, :] = 1
+    for matrix, answer in ((best, "ELLPACK"), (ok, "ELLPACK"), (bad, "CSR"), (small, "ELLPACK")):
+        hA = sp.HostSparseMatrix(matrix.tocsr())
+        assert sp.spmv_algorithm_heuristic(FakeQueue, hA, footprint_soft_limit=testing_limit) == answer
+    assert set(sp.algostr_to_planner) == {"ELLPACK", "ELLPACK-tree", "ELLPACK-twostep", "CSR"}
+    for cls in sp.algostr_to_planner.values():
+        assert issubclass(cls, sp.spmv_prog) and issubclass(cls, sp.plan_sparse_dot_inc)
