@@ -324,5 +324,21 @@ class HIPRaggedArray:
         return sio.getvalue()
 
 
+def to_host(queue, data, dtype, start, shape, elemstrides, is_blocking=True):
+    """One strided 2-D section of the device array `data` as a host array: the smallest
+    contiguous span that holds it is copied and viewed with the element strides (the
+    reference's helper of this name, clraggedarray.py:36-62; copies here always wait)."""
+    m, n = (int(v) for v in shape)
+    sm, sn = (int(v) for v in elemstrides)
+    if min(sm, sn) < 0:
+        raise NotImplementedError("negative strides")
+    dtype = np.dtype(dtype)
+    if m * n == 0:
+        return np.zeros((m, n), dtype=dtype)
+    span = data.get_span(int(start), (m - 1) * sm + (n - 1) * sn + 1)
+    isz = dtype.itemsize
+    return np.lib.stride_tricks.as_strided(span.view(dtype), shape=(m, n), strides=(sm * isz, sn * isz))
+
+
 # The reference's name for this class, so that code written against it reads the same.
 CLRaggedArray = HIPRaggedArray

@@ -2,8 +2,11 @@
 
 Counterparts of the helpers in the reference's ``nengo_ocl/utils.py`` that the
 timestep path needs (``round_up`` :48, ``split`` :56, ``stable_unique`` :69,
-``get_closures`` :40).  The benchmark ``SimRunner`` registry of that file is
-not part of the timestep path and is not provided.
+``get_closures`` :40, and the one-liners ``as_ascii`` :16, ``equal_strides`` :25,
+``nonelist`` :48, ``round_up_power_of_2`` :56 under their names; ``HostSparseMatrix``
+lives with the sparse products and is reachable from here as in the reference).  The
+benchmark ``SimRunner`` registry of that file is not part of the timestep path and is
+not provided.
 """
 
 import numpy as np
@@ -88,3 +91,40 @@ def f32_bits(value):
     them as raw bits and are re-read on the device with ``__int_as_float``.
     """
     return int(np.asarray(value, dtype=np.float32).view(np.int32))
+
+
+def as_ascii(text):
+    """``text`` as a str: bytes are decoded as ASCII, other objects go through ``str``."""
+    if isinstance(text, bytes):
+        return text.decode("ascii")
+    return text if isinstance(text, str) else str(text)
+
+
+def equal_strides(strides_a, strides_b, shape):
+    """Whether two stride tuples address an array of ``shape`` the same way: axes of
+    length one may differ, all others must agree, and the ranks must match."""
+    if not (len(strides_a) == len(strides_b) == len(shape)):
+        return False
+    return all(n == 1 or a == b for n, a, b in zip(shape, strides_a, strides_b))
+
+
+def nonelist(*args):
+    """The arguments that are not None, in order."""
+    return [a for a in args if a is not None]
+
+
+def round_up_power_of_2(x):
+    """The power of two at or above ``|x|`` with the sign of ``x`` (1 for ``|x| < 1``)."""
+    if abs(x) < 1:
+        return 1
+    magnitude = 2 ** int(np.ceil(np.log2(abs(x))))
+    return magnitude if x > 0 else -magnitude
+
+
+def __getattr__(name):
+    # (imported on demand: the sparse module imports this one)
+    if name == "HostSparseMatrix":
+        from .hipra_spmv import HostSparseMatrix
+
+        return HostSparseMatrix
+    raise AttributeError(name)

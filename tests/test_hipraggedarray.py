@@ -44,6 +44,26 @@ def test_getitem_and_getitems(queue, rng):
     assert sub.dev_buf is dA.dev_buf  # a view: same device memory
 
 
+def test_to_host_helper_and_reference_class_name(queue, rng):
+    """The module-level `to_host` (clraggedarray.py:36-62): a strided section of the device
+    buffer, bit for bit; `CLRaggedArray` is the device class under the reference's name."""
+    from nengo_ocl_amd import hipraggedarray as hra
+
+    A = random_ra(rng, 6, 2)
+    dA = to_dev(queue, A)
+    assert hra.CLRaggedArray is type(dA)
+    for i in range(len(A)):
+        got = hra.to_host(queue, dA.dev_buf, A.dtype, A.starts[i], (A.shape0s[i], A.shape1s[i]),
+                          (A.stride0s[i], A.stride1s[i]))
+        assert np.array_equal(got, A[i])
+    # every second column of an item
+    m, n = int(A.shape0s[2]), int(A.shape1s[2])
+    got = hra.to_host(queue, dA.dev_buf, A.dtype, A.starts[2], (m, (n + 1) // 2),
+                      (A.stride0s[2], 2 * A.stride1s[2]))
+    assert np.array_equal(got, A[2][:, ::2])
+    assert hra.to_host(queue, dA.dev_buf, A.dtype, 0, (0, 3), (3, 1)).shape == (0, 3)
+
+
 def test_setitem(queue, rng):
     A = random_ra(rng, 3, 2)
     dA = to_dev(queue, A)

@@ -90,3 +90,21 @@ def test_offsets_beyond_int32_are_refused():
     with pytest.raises(ValueError, match="2\\^31"):
         RaggedArray.from_buffer(buf, np.array([0, 2 ** 31 + 5], dtype=np.int64), [1, 1], [1, 1],
                                 [1, 1], [1, 1])
+
+
+def test_small_helpers_under_the_reference_names():
+    """nengo_ocl/utils.py:16-57: `as_ascii`, `equal_strides`, `nonelist`,
+    `round_up_power_of_2`; `HostSparseMatrix` is reachable from `utils` as there."""
+    from nengo_ocl_amd import utils
+
+    assert utils.as_ascii(b"abc") == "abc" and utils.as_ascii("x") == "x" and utils.as_ascii(3) == "3"
+    assert utils.equal_strides((8, 4), (8, 4), (3, 2))
+    assert utils.equal_strides((99, 4), (8, 4), (1, 2))      # an axis of length one may differ
+    assert not utils.equal_strides((16, 4), (8, 4), (3, 2))
+    assert not utils.equal_strides((8,), (8, 4), (3, 2))
+    assert utils.nonelist(1, None, "a", None) == [1, "a"]
+    assert [utils.round_up_power_of_2(v) for v in (0, 0.5, 1, 3, 4, 5, 1000, -3)] == [
+        1, 1, 1, 4, 4, 8, 1024, -4]
+    from nengo_ocl_amd.hipra_spmv import HostSparseMatrix
+
+    assert utils.HostSparseMatrix is HostSparseMatrix
