@@ -9,8 +9,9 @@ hand-written HIP for gfx950 in ``libnengo_hip.so``.
 
 import logging
 
+from .version import version as __version__
+
 ABI_VERSION = 1  # must equal NHIP_ABI_VERSION in include/nengo_hip.h
-__version__ = "0.1.0"
 
 logging.getLogger(__name__).addHandler(logging.NullHandler())
 

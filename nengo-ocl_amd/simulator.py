@@ -584,7 +584,11 @@ class Simulator:
                 "building a nengo Network needs the `nengo` package (>= 3.1); without it "
                 "pass a minibuilder.Network or a ready ir.Model") from e
         from .builder import Builder
+        from .version import check_nengo_version
 
+        import nengo
+
+        check_nengo_version(nengo)  # (the reference does this first, simulator.py:195-206)
         model = Model(dt=float(dt), label="%s, dt=%f" % (network, dt),
                       decoder_cache=get_default_decoder_cache(), builder=Builder())
         model.build(network)

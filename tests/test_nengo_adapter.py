@@ -197,3 +197,39 @@ def test_backend_entry_point_and_test_loader():
     assert seen == {"net": "a network", "dt": 0.002, "progress_bar": False}
     unsupported = cfg["pytest"]["nengo_test_unsupported"]
     assert "test_lif_min_voltage" in unsupported and "test_pickle_sim" in unsupported
+
+
+def test_nengo_version_is_checked_before_building(monkeypatch):
+    """Reference simulator.py:195-206: a nengo the backend cannot work with is refused when
+    the Simulator is constructed, a newer one than the last tested gets a warning (here:
+    older than 3.1 refused; stand-in modules carry the version under test)."""
+    import types
+    import warnings
+
+    import nengo_ocl_amd
+    from nengo_ocl_amd import version
+
+    assert nengo_ocl_amd.__version__ == version.version
+    N = nengo_standin.install(monkeypatch)
+
+    @N.Builder.register(ToyNetwork)
+    def build_toy(model, network):
+        emit(model, network, N)
+
+    import nengo
+
+    for info, outcome in (((3, 0, 0), "refused"), ((2, 8, 0), "refused"), ((3, 1, 0), "fine"),
+                          ((4, 0, 0), "warned")):
+        monkeypatch.setattr(nengo, "version", types.SimpleNamespace(version_info=info),
+                            raising=False)
+        monkeypatch.setattr(nengo, "__version__", ".".join(map(str, info)), raising=False)
+        with warnings.catch_warnings(record=True) as caught:
+            warnings.simplefilter("always")
+            if outcome == "refused":
+                with pytest.raises(ValueError, match="does not support Nengo version"):
+                    OracleSimulator(ToyNetwork(), dt=0.001)
+                continue
+            with OracleSimulator(ToyNetwork(), dt=0.001) as sim:
+                sim.run_steps(3)
+            untested = [w for w in caught if "has not been tested" in str(w.message)]
+            assert bool(untested) == (outcome == "warned")
