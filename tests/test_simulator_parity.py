@@ -355,6 +355,30 @@ def test_other_configurations_full_size_state_bit_exact(queue, case):
         assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
 
 
+@pytest.mark.parametrize("case", ["c2", "c4"])
+def test_other_configurations_full_size_over_one_second(queue, case):
+    """The small-world network and the PES-learning network at their full sizes over a
+    simulated second (1000 steps, run in batches as `run` does): every probe sample and every
+    signal -- the learned decoders included -- bit-identical to the oracle's at the end."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    make = {"c2": configs.c2_watts_strogatz, "c4": configs.c4_pes}[case]
+    net, probes, _ = make()
+    net_o, probes_o, _ = make()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        for _ in range(4):
+            gpu.run_steps(250)
+            cpu.run_steps(250)
+        assert gpu.n_steps == cpu.n_steps == 1000 and gpu.time == cpu.time
+        for key in probes:
+            got, want = gpu.data[probes[key]], cpu.data[probes_o[key]]
+            assert got.shape == want.shape and np.any(want != 0), key
+            assert np.array_equal(got, want), key
+        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+
+
 def test_c4_pes_reduced(queue):
     """PES learning: weights after 1 s agree with the oracle's, and learning happened."""
     from nengo_ocl_amd import configs
