@@ -43,7 +43,9 @@ def make_network(config, variant, scale):
     if config == "c0":
         return configs.c0_readme(), "c0: README two-ensemble net, 200 LIF neurons"
     if config == "c1":
-        return configs.c1_circconv(dims=64), "c1: circular convolution D=64, 13,200 LIF neurons"
+        dims = max(2, int(round(64 * scale)))  # (the reference's benchmark_circconv.py varies D)
+        return (configs.c1_circconv(dims=dims),
+                "c1: circular convolution D=%d, %d LIF neurons" % (dims, 100 * (2 * dims + 4)))
     if config == "c2":
         return (configs.c2_watts_strogatz(),
                 "c2: Watts-Strogatz, 2048 ensembles x 100 LIF, 20,480 decoded edges")
@@ -386,7 +388,7 @@ def main():
     ap.add_argument("--kernel-hash", action="store_true",
                     help="only print the hash of the dominant kernel's sources (the line a "
                          "counter summary under profiles/ carries)")
-    ap.add_argument("--scale", type=float, default=1.0, help="fraction of the ensembles (c3, c4)")
+    ap.add_argument("--scale", type=float, default=1.0, help="fraction of the ensembles (c3, c4), of the dimensions (c1), of the neurons (c5)")
     ap.add_argument("--profile-steps", type=int, default=100)
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds; 0 skips the CPU leg")
     ap.add_argument("--dense-decoders", action="store_true",
