@@ -65,7 +65,9 @@ def test_rich_random_network_merged_equals_unmerged(seed):
     (1, False, True, False), (2, False, True, False), (3, False, False, False),
     (4, False, False, False), (11, True, True, False), (12, True, False, False),
     (13, True, False, False), (21, False, True, True), (22, False, False, True),
-    (23, False, False, True), (24, True, True, True), (25, True, False, True)])
+    (23, False, False, True), (24, True, True, True), (25, True, False, True),
+    (100, True, True, True), (101, False, False, True), (104, False, True, True),
+    (105, True, False, False), (110, True, True, True), (115, True, False, True)])
 def test_random_network_on_the_device(queue, seed, big, sliced, rich):
     """With slices among the targets the oracle simulator applies the same rewrites (the
     order of increments into overlapping views follows the operator list that is planned);
