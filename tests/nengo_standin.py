@@ -27,10 +27,68 @@ def _module(name, **members):
 
 
 # ------------------------------------------------------------------ signals
+class SparseMatrix:
+    """nengo.transforms.SparseMatrix: `indices` (nnz x 2), `data`, `shape`, `ndim`, `size`,
+    `tocsr()`.  A Signal whose initial value is one has `sparse == True`."""
+
+    def __init__(self, indices, data, shape):
+        self.indices = np.asarray(indices, dtype=np.int64).reshape(-1, 2)
+        self.data = np.asarray(data, dtype=np.float64)
+        self.shape = tuple(shape)
+        self.ndim = 2
+        self.dtype = self.data.dtype
+
+    @property
+    def size(self):
+        return len(self.data)
+
+    def tocsr(self):
+        import scipy.sparse
+
+        m = scipy.sparse.csr_matrix((self.data, self.indices.T), shape=self.shape)
+        m.sort_indices()
+        return m
+
+
 class Signal(ir.Signal):
     """nengo.builder.signal.Signal: `base`, `is_view`, `initial_value`, `readonly`, `shape`,
     `ndim`, `size`, `elemoffset`, `elemstrides`, `may_share_memory`, `name`, `sparse`
-    (read at simulator.py:72-143, 266-300 of the reference)."""
+    (read at simulator.py:72-143, 266-300 of the reference).  With a `SparseMatrix` as its
+    initial value it is a sparse signal (reference simulator.py:281-286, 321-324)."""
+
+    def __init__(self, initial_value=None, **kwargs):
+        if isinstance(initial_value, SparseMatrix):
+            self._sparse_value = initial_value
+            self._base = None
+            self.name = kwargs.get("name")
+            self._readonly = True
+        else:
+            super().__init__(initial_value, **kwargs)
+
+    sparse = property(lambda self: hasattr(self, "_sparse_value"))
+
+    def _dense_or(name):  # noqa: N805 (a helper evaluated in the class body)
+        inherited = getattr(ir.Signal, name)
+
+        def get(self):
+            if self.sparse:
+                return getattr(self._sparse_value, name) if name != "initial_value" \
+                    else self._sparse_value
+            return inherited.fget(self)
+
+        return property(get)
+
+    initial_value = _dense_or("initial_value")
+    shape = _dense_or("shape")
+    ndim = _dense_or("ndim")
+    size = _dense_or("size")
+    dtype = _dense_or("dtype")
+    del _dense_or
+
+    def may_share_memory(self, other):
+        if self.sparse or getattr(other, "sparse", False):
+            return other is self
+        return super().may_share_memory(other)
 
 
 class SignalDict(dict):
@@ -39,7 +97,9 @@ class SignalDict(dict):
 
     def init(self, signal):
         if signal.base not in self:
-            dict.__setitem__(self, signal.base, np.array(signal.base.initial_value))
+            base = signal.base
+            value = base.initial_value.tocsr() if base.sparse else np.array(base.initial_value)
+            dict.__setitem__(self, base, value)
 
 
 # ------------------------------------------------------------------ operators
@@ -90,6 +150,23 @@ class DotInc(Operator):  # operators.py:51-66 of the reference: op.A, op.X, op.Y
         self.reads, self.incs = [A, X], [Y]
 
 
+class SparseDotInc(Operator):  # simulator.py:877-892 of the reference: op.A (sparse), op.X, op.Y
+    def __init__(self, A, X, Y, tag=None):
+        super().__init__(tag)
+        assert A.sparse
+        self.A, self.X, self.Y = A, X, Y
+        self.reads, self.incs = [A, X], [Y]
+
+
+class SimPES(Operator):  # simulator.py:1334-1345: pre_filtered, error, delta, learning_rate
+    def __init__(self, pre_filtered, error, delta, learning_rate, encoders=None, tag=None):
+        super().__init__(tag)
+        self.pre_filtered, self.error, self.delta = pre_filtered, error, delta
+        self.learning_rate, self.encoders = learning_rate, encoders
+        self.reads = [pre_filtered, error] + ([] if encoders is None else [encoders])
+        self.updates = [delta]
+
+
 class ElementwiseInc(Operator):  # simulator.py:871-875: op.A, op.X, op.Y
     def __init__(self, A, X, Y, tag=None):
         super().__init__(tag)
@@ -130,6 +207,12 @@ class LIF:  # simulator.py:1046-1063: tau_rc, tau_ref, amplitude, min_voltage
     def __init__(self, tau_rc=0.02, tau_ref=0.002, min_voltage=0, amplitude=1.0):
         self.tau_rc, self.tau_ref, self.min_voltage, self.amplitude = (
             tau_rc, tau_ref, min_voltage, amplitude)
+
+
+class AdaptiveLIF(LIF):  # clra_nonlinearities.py:1094-1132 through simulator.py:1080-1100
+    def __init__(self, tau_n=1.0, inc_n=0.01, **kwargs):
+        super().__init__(**kwargs)
+        self.tau_n, self.inc_n = tau_n, inc_n
 
 
 class Process:
@@ -254,14 +337,17 @@ def install(monkeypatch):
         "nengo.builder.builder": _module("nengo.builder.builder", Model=Model),
         "nengo.builder.operator": _module(
             "nengo.builder.operator", Operator=Operator, TimeUpdate=TimeUpdate, Reset=Reset,
-            Copy=Copy, DotInc=DotInc, ElementwiseInc=ElementwiseInc, SimPyFunc=SimPyFunc),
+            Copy=Copy, DotInc=DotInc, ElementwiseInc=ElementwiseInc, SimPyFunc=SimPyFunc,
+            SparseDotInc=SparseDotInc),
+        "nengo.builder.learning_rules": _module("nengo.builder.learning_rules", SimPES=SimPES),
+        "nengo.transforms": _module("nengo.transforms", SparseMatrix=SparseMatrix),
         "nengo.builder.neurons": _module("nengo.builder.neurons", SimNeurons=SimNeurons),
         "nengo.builder.processes": _module("nengo.builder.processes", SimProcess=SimProcess),
         "nengo.builder.signal": _module("nengo.builder.signal", Signal=Signal,
                                         SignalDict=SignalDict),
         "nengo.cache": _module("nengo.cache", get_default_decoder_cache=lambda: None),
         "nengo.exceptions": _module("nengo.exceptions", BuildError=BuildError),
-        "nengo.neurons": _module("nengo.neurons", LIF=LIF),
+        "nengo.neurons": _module("nengo.neurons", LIF=LIF, AdaptiveLIF=AdaptiveLIF),
         "nengo.synapses": _module("nengo.synapses", LinearFilter=LinearFilter, Lowpass=Lowpass),
         "nengo.processes": _module("nengo.processes", Process=Process, WhiteSignal=WhiteSignal),
         "nengo.utils": _module("nengo.utils"),
@@ -277,4 +363,11 @@ def install(monkeypatch):
         Signal=Signal, Reset=Reset, Copy=Copy, DotInc=DotInc, ElementwiseInc=ElementwiseInc,
         SimPyFunc=SimPyFunc, SimNeurons=SimNeurons, SimProcess=SimProcess, LIF=LIF,
         Lowpass=Lowpass, WhiteSignal=WhiteSignal, Model=Model, Builder=Builder,
-        BuildError=BuildError, family="nengo")
+        BuildError=BuildError, SparseDotInc=SparseDotInc, SimPES=SimPES, AdaptiveLIF=AdaptiveLIF,
+        sparse_signal=lambda matrix, name=None: Signal(_as_sparse_matrix(matrix), name=name),
+        family="nengo")
+
+
+def _as_sparse_matrix(matrix):
+    coo = matrix.tocoo()
+    return SparseMatrix(np.stack([coo.row, coo.col], axis=1), coo.data, coo.shape)

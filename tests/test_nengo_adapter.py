@@ -13,6 +13,7 @@ import numpy as np
 import pytest
 
 import nengo_standin
+from helpers import assert_same_signals
 from nengo_ocl_amd import ir
 from oracle.oracle_sim import OracleSimulator
 
@@ -20,15 +21,16 @@ IR = types.SimpleNamespace(
     Signal=ir.Signal, Reset=ir.Reset, Copy=ir.Copy, DotInc=ir.DotInc,
     ElementwiseInc=ir.ElementwiseInc, SimPyFunc=ir.SimPyFunc, SimNeurons=ir.SimNeurons,
     SimProcess=ir.SimProcess, LIF=ir.LIF, Lowpass=ir.Lowpass, WhiteSignal=ir.WhiteSignal,
-    Model=ir.Model, family="ir")
+    Model=ir.Model, SparseDotInc=ir.SparseDotInc, SimPES=ir.SimPES, AdaptiveLIF=ir.AdaptiveLIF,
+    sparse_signal=lambda matrix, name=None: ir.SparseSignal(matrix, name=name), family="ir")
 
 
 class ToyNetwork:
     """What the toy build function below turns into operators."""
     seed = 3
 
-    def __init__(self, n_neurons=80, dims=3):
-        self.n_neurons, self.dims = n_neurons, dims
+    def __init__(self, n_neurons=80, dims=3, fn=lambda t: np.sin(8 * t)):
+        self.n_neurons, self.dims, self.fn = n_neurons, dims, fn
 
 
 class ToyProbe:
@@ -45,7 +47,7 @@ def emit(model, net, F):
     n, d = net.n_neurons, net.dims
     t = model.time
     sin_out = F.Signal(np.zeros(1), name="sin.out")
-    model.add_op(F.SimPyFunc(sin_out, lambda t: np.sin(8 * t), t, None))
+    model.add_op(F.SimPyFunc(sin_out, net.fn, t, None))
     noise_out = F.Signal(np.zeros(d), name="noise.out")
     model.add_op(F.SimProcess(F.WhiteSignal(0.2, high=10.0, seed=5), None, noise_out, t, mode="set"))
     gain_sig = F.Signal(np.array(0.5), name="half", readonly=True)
@@ -84,6 +86,178 @@ def emit(model, net, F):
             model.params[p] = []
             probes[name] = p
     return probes
+
+
+class LearningNetwork:
+    """What `emit_learning` turns into operators."""
+    seed = 5
+
+    def __init__(self, n_pre=96, n_post=64, n_err=48, dims=4):
+        self.n_pre, self.n_post, self.n_err, self.dims = n_pre, n_post, n_err, dims
+
+
+def emit_learning(model, net, F):
+    """The operators nengo's builder emits for: a band-limited input into `pre` (LIF); a
+    decoded connection pre -> post (adaptive LIF) whose decoders PES learns from the error
+    that `err` (LIF) decodes as post - pre; a sparse weight matrix from pre's neurons onto
+    post's neurons behind a synapse.  Probes: the learned output, the error that reaches the
+    rule, and post's spikes every 5 ms.  `F` supplies the classes."""
+    import scipy.sparse
+
+    rng = np.random.RandomState(23)
+    d, t = net.dims, model.time
+    probes = {}
+
+    def probe(name, sig, every=None):
+        p = ToyProbe(sample_every=every)
+        model.probes.append(p)
+        model.sig[p] = {"in": sig}
+        model.params[p] = []
+        probes[name] = p
+
+    def lowpass(x, tau, name):
+        y = F.Signal(np.zeros(x.shape), name=name)
+        model.add_op(F.SimProcess(F.Lowpass(tau), x, y, t, mode="update"))
+        return y
+
+    def ensemble(name, n, neurons, state_names):
+        x_in = F.Signal(np.zeros(d), name=name + ".in")
+        model.add_op(F.Reset(x_in))
+        enc = F.Signal(rng.normal(size=(n, d)) * (2.0 / np.sqrt(d)), name=name + ".encoders",
+                       readonly=True)
+        bias = F.Signal(rng.uniform(0.6, 1.8, size=n), name=name + ".bias", readonly=True)
+        J = F.Signal(np.zeros(n), name=name + ".J")
+        model.add_op(F.Copy(bias, J))
+        model.add_op(F.DotInc(enc, x_in, J))
+        out = F.Signal(np.zeros(n), name=name + ".out")
+        state = {s: F.Signal(np.zeros(n), name="%s.%s" % (name, s)) for s in state_names}
+        model.add_op(F.SimNeurons(neurons, J, out, state=state))
+        return x_in, J, out
+
+    def decoded(out, n, name, scale=1.0, readonly=True):
+        dec = F.Signal(scale * rng.normal(size=(d, n)) / (40.0 * n), name=name + ".weights",
+                       readonly=readonly)
+        weighted = F.Signal(np.zeros(d), name=name + ".weighted")
+        model.add_op(F.Reset(weighted))
+        model.add_op(F.DotInc(dec, out, weighted))
+        return dec, lowpass(weighted, 0.005, name + ".filtered")
+
+    stim = F.Signal(np.zeros(d), name="stim.out")
+    model.add_op(F.SimProcess(F.WhiteSignal(0.3, high=8.0, seed=7), None, stim, t, mode="set"))
+    pre_in, _, pre_out = ensemble("pre", net.n_pre, F.LIF(), ("voltage", "refractory_time"))
+    post_in, post_J, post_out = ensemble(
+        "post", net.n_post, F.AdaptiveLIF(tau_n=0.5, inc_n=0.02),
+        ("voltage", "refractory_time", "adaptation"))
+    err_in, _, err_out = ensemble("err", net.n_err, F.LIF(tau_rc=0.03),
+                                  ("voltage", "refractory_time"))
+    model.add_op(F.Copy(stim, pre_in, inc=True))
+
+    # the learned connection and its rule
+    learned, learned_out = decoded(pre_out, net.n_pre, "learned", readonly=False)
+    model.add_op(F.Copy(learned_out, post_in, inc=True))
+    pre_filtered = lowpass(pre_out, 0.005, "pes.pre_filtered")
+    rule_in = F.Signal(np.zeros(d), name="pes.in")
+    model.add_op(F.Reset(rule_in))
+    delta = F.Signal(np.zeros((d, net.n_pre)), name="pes.delta")
+    model.add_op(F.SimPES(pre_filtered, rule_in, delta, 1e-4))
+    model.add_op(F.Copy(delta, learned, inc=True))
+
+    # err decodes post - pre and sends it to the rule
+    _, post_decoded = decoded(post_out, net.n_post, "post_to_err")
+    model.add_op(F.Copy(post_decoded, err_in, inc=True))
+    _, pre_decoded = decoded(pre_out, net.n_pre, "pre_to_err", scale=-1.0)
+    model.add_op(F.Copy(pre_decoded, err_in, inc=True))
+    _, err_decoded = decoded(err_out, net.n_err, "err_to_rule", scale=30.0)
+    model.add_op(F.Copy(err_decoded, rule_in, inc=True))
+
+    # a sparse matrix between the neurons of pre and post
+    matrix = scipy.sparse.random(net.n_post, net.n_pre, density=0.03, random_state=rng,
+                                 format="csr", data_rvs=lambda k: rng.normal(scale=2e-3, size=k))
+    A = F.sparse_signal(matrix, name="lateral.weights")
+    lateral = F.Signal(np.zeros(net.n_post), name="lateral.weighted")
+    model.add_op(F.Reset(lateral))
+    model.add_op(F.SparseDotInc(A, pre_out, lateral))
+    model.add_op(F.Copy(lowpass(lateral, 0.01, "lateral.filtered"), post_J, inc=True))
+
+    probe("learned", learned_out)
+    probe("error", rule_in)
+    probe("post_spikes", post_out, every=0.005)
+    return probes
+
+
+def _install_family(monkeypatch):
+    N = nengo_standin.install(monkeypatch)
+    built = {}
+    N.Builder.register(ToyNetwork)(
+        lambda model, network: built.__setitem__("toy", emit(model, network, N)))
+    N.Builder.register(LearningNetwork)(
+        lambda model, network: built.__setitem__("learning", emit_learning(model, network, N)))
+    return N, built
+
+
+def test_nengo_family_learning_graph_runs_like_the_ir_graph(monkeypatch):
+    """PES, a sparse product and adaptive LIF neurons out of nengo-family classes (sparse
+    signal = a Signal holding a SparseMatrix, initial values through SignalDict)."""
+    N, built = _install_family(monkeypatch)
+    net = LearningNetwork()
+    with OracleSimulator(net, dt=0.001) as sim:
+        kinds = {type(op).__name__ for op in sim.model.operators}
+        assert {"SimPES", "SparseDotInc", "SimNeurons"} <= kinds
+        assert all(type(op).__module__.startswith("nengo.") for op in sim.model.operators)
+        ref_model = ir.Model(dt=0.001)
+        ref_probes = emit_learning(ref_model, net, IR)
+        with OracleSimulator(None, model=ref_model, seed=net.seed + 1) as ref:
+            assert [p.name for p in sim._plans] == [p.name for p in ref._plans]
+            sim.run_steps(300)
+            ref.run_steps(300)
+            for key in ref_probes:
+                got, want = sim.data[built["learning"][key]], ref.data[ref_probes[key]]
+                assert got.shape == want.shape and np.any(want != 0), key
+                assert np.array_equal(got, want), (key, np.abs(got - want).max())
+            assert np.array_equal(np.asarray(sim.all_data.buf), np.asarray(ref.all_data.buf))
+            assert sim.data[built["learning"]["post_spikes"]].shape == (60, net.n_post)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", ["toy", "learning"])
+def test_nengo_family_graphs_on_the_device(monkeypatch, which):
+    """`Simulator(network)` on the HIP backend for graphs made of nengo-family classes: the
+    class-name keyed choices (spiking populations -> launches that visit active columns and
+    skip zero operands, neurons in the epilogue of the launch that forms their input,
+    synapses in the epilogue of the decoders) are taken, and probes and every signal equal
+    the oracle simulator's bit for bit after 300 steps (graph replay, all fusions on)."""
+    from nengo_ocl_amd.simulator import Simulator
+
+    N, built = _install_family(monkeypatch)
+    if which == "toy":
+        # (np.sin itself: both sides round the double-precision sine once, where a traced
+        # function is evaluated in float32 on the device and agrees to a tolerance only)
+        net = ToyNetwork(n_neurons=1024, dims=32, fn=np.sin)
+    else:
+        net = LearningNetwork(n_pre=1024, n_post=512, n_err=512, dims=32)
+    with Simulator(net, dt=0.001) as gpu:
+        gpu_probes = built[which]
+        assert type(gpu.model) is N.Model
+        assert all(type(op).__module__.startswith("nengo.") for op in gpu.model.operators)
+        names = [p.name for p in gpu._plans]
+        print(which, "plans per step:", names)
+        with OracleSimulator(net, dt=0.001) as cpu:
+            cpu_probes = built[which]
+            assert any(n in ("hipra_gemv.tile_lif", "hipra_gemv.rows_lif") or
+                       n.startswith("hipra_gemv.tile_lif") for n in names), names
+            assert any(n.startswith(("hipra_gemv.events_filter", "hipra_gemv.tile_filter",
+                                     "hipra_gemv.rows_filter")) for n in names), names
+            if which == "toy":
+                assert any(getattr(p, "event_driven", False) for p in gpu._plans), names
+            else:
+                assert any(hasattr(p, "spmv") for p in gpu._plans), names
+            gpu.run_steps(300)
+            cpu.run_steps(300)
+            for key in cpu_probes:
+                got, want = gpu.data[gpu_probes[key]], cpu.data[cpu_probes[key]]
+                assert got.shape == want.shape and np.any(want != 0), key
+                assert np.array_equal(got, want), (key, np.abs(got - want).max())
+            assert_same_signals(gpu, cpu)
 
 
 def test_nengo_family_graph_runs_like_the_ir_graph(monkeypatch):
