@@ -91,6 +91,19 @@ int nhip_gemv(void *stream, int flavor, int lpr, int vec, int passes, const int 
 /* rows one task of the given class covers at most (0 if the class is unknown) */
 int nhip_gemv_rows_per_task(int flavor, int lpr, int vec, int passes);
 
+/* The same operation in the reference's summation order for coefficients that the
+ * reference writes into its kernel text as double-precision literals (alpha, beta or
+ * gamma the same for every item: clra_gemv.py:20-34, used at :1058, :1148, :1153):
+ * alpha * (tile sum), beta * y_in and sum + gamma are formed in double and rounded to
+ * float32 once each.  Identical to nhip_gemv (flavor 2) whenever float32 holds the
+ * coefficients exactly; the host takes this entry point when it does not.
+ *   dcoefs : double[n_items][4] {alpha, beta, gamma, 0}
+ *   tasks  : int32[n_tasks][4] {item, row, 1, 0} -- one output row per task
+ * `items` and `dots` as for nhip_gemv. */
+int nhip_gemv_rows_literal(void *stream, const int *items, const double *dcoefs, const int *dots,
+                           const int *tasks, int n_tasks, const float *A, const float *X,
+                           const float *Yin, float *Y);
+
 /* The same operation and the same four tables, summed in the ORDER of the
  * reference's block kernel (clra_gemv.py:1043-1058, :1148-1153: four strided
  * partial sums per 128-column tile, one fused multiply-add per element,

@@ -27,6 +27,7 @@ SIGNATURES = {
     "nhip_device_info": [P, P, P, ctypes.c_char_p, c_int],
     "nhip_gemv": [P, c_int, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P],
     "nhip_gemv_rows_per_task": [c_int, c_int, c_int, c_int],
+    "nhip_gemv_rows_literal": [P, P, P, P, P, c_int, P, P, P, P],
     "nhip_gemv_tile": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P],
     "nhip_gemv_tile_lif": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
                            P, ctypes.c_double, c_int, P, P, P, P, P, P],

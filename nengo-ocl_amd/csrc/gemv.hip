@@ -463,6 +463,67 @@ extern "C" int nhip_gemv(void* stream, int flavor, int lpr, int vec, int passes,
     return NHIP_E_BADCLASS;
 }
 
+// ---------------------------------------------------------------- literal coefficients
+// The reference renders alpha, beta and gamma that are the same for every item into the
+// kernel text as double-precision literals (clra_gemv.py:20-34, :1058, :1148, :1153):
+// `ybuf = alpha * (s0 + s1)`, `sum = beta * yin`, `y = sum + gamma` are then formed in
+// double and rounded to float32 once each.  For coefficients that float32 holds exactly
+// (the Simulator's own: 1, 0) this equals the float32 arithmetic of the kernels above.
+// For others (0.1, 0.3) it does not, and such launches take this kernel: the small-item
+// kernel's decomposition (a task = one output row, four lanes per row, lane j the partial
+// sum j, reference order) with the three operations in double.  Coefficients that differ
+// from item to item are float32 arrays in the reference; the host passes them as the
+// doubles of their float32 values, for which the double operations round as the float32
+// ones do.
+__global__ __launch_bounds__(NHIP_WG) void gemv_rows_literal_kernel(
+    const GemvItem* __restrict__ items, const double* __restrict__ dcoefs,
+    const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
+    const float* A, const float* X, const float* Yin, float* Y)
+{
+    constexpr int TILE = 128;
+    const int lane = threadIdx.x & (NHIP_WAVE - 1);
+    const int lir = lane & 3;
+    const int slot = (blockIdx.x * (NHIP_WG / NHIP_WAVE) + (threadIdx.x >> 6)) * (NHIP_WAVE / 4) + lane / 4;
+    const bool valid = slot < n_tasks;
+    const GemvTask task = tasks[valid ? slot : n_tasks - 1];
+    const GemvItem it = items[task.item];
+    const double alpha = dcoefs[4 * task.item], beta = dcoefs[4 * task.item + 1];
+    const double gamma = dcoefs[4 * task.item + 2];
+    const int r = task.row0;
+    float sum = (float)(beta * (double)Yin[it.yin_start + (size_t)r * it.yin_stride0]);
+    for (int d = 0; d < it.n_dots; ++d) {
+        const GemvDot dot = dots[it.dot_begin + d];
+        const float* arow = A + dot.a_start + (size_t)r * dot.a_stride0;
+        const float* xg = X + dot.x_start;
+        for (int c0 = 0; c0 < dot.N; c0 += TILE) {
+            const int c1 = min(c0 + TILE, dot.N);
+            float s = 0.0f;
+            for (int c = c0 + lir; c < c1; c += 4) s = fmaf(arow[c], xg[(size_t)c * dot.x_stride0], s);
+            s = s + __shfl_xor(s, 2, NHIP_WAVE);  // lanes 0, 1 of the row: s0 + s2, s1 + s3
+            s = s + __shfl_xor(s, 1, NHIP_WAVE);  // lane 0: (s0 + s2) + (s1 + s3)
+            sum = sum + (float)(alpha * (double)s);
+        }
+    }
+    if (lir == 0 && valid)
+        Y[it.y_start + (size_t)r * it.y_stride0] = (float)((double)sum + gamma);
+}
+
+extern "C" int nhip_gemv_rows_literal(void* stream, const int* items, const double* dcoefs,
+                                      const int* dots, const int* tasks, int n_tasks,
+                                      const float* A, const float* X, const float* Yin, float* Y) {
+    if (n_tasks == 0) return 0;
+    if (n_tasks < 0 || !items || !dcoefs || !dots || !tasks || !A || !X || !Yin || !Y)
+        return NHIP_E_BADARG;
+    const int rows_per_group = (NHIP_WG / NHIP_WAVE) * (NHIP_WAVE / 4);
+    const dim3 grid((n_tasks + rows_per_group - 1) / rows_per_group);
+    NHIP_LAUNCH(gemv_rows_literal_kernel, grid, dim3(NHIP_WG), 0, static_cast<hipStream_t>(stream),
+                reinterpret_cast<const GemvItem*>(items), dcoefs,
+                reinterpret_cast<const GemvDot*>(dots), reinterpret_cast<const GemvTask*>(tasks),
+                n_tasks, A, X, Yin, Y);
+    NHIP_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" int nhip_gemv_rows_lif(void* stream, int lpr, int task_words, const int* items,
                                   const float* coefs, const int* dots, const int* tasks,
                                   int n_tasks, const float* A,

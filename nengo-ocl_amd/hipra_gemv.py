@@ -129,6 +129,18 @@ def _per_item_floats(arg, n, what):
     return vec
 
 
+def _literal_coefficient(arg, n):
+    """The double the reference writes into its kernel text for a coefficient that is the
+    same for every item (a Python float, or a list of equal values: clra_gemv.py:17-32), or
+    None for one that differs from item to item (a float32 array there)."""
+    v = np.asarray(arg, dtype=np.float64)
+    if v.ndim == 0:
+        return float(v)
+    if n and len(set(v.ravel().tolist())) == 1:
+        return float(v.ravel()[0])
+    return None
+
+
 def _balanced_rows(M, cap):
     """Rows per task so that the tasks of an item are equally full (M = 4096, cap = 128
     stays 128; M = 100, cap = 64 becomes 50 instead of 64 + 36)."""
@@ -153,6 +165,7 @@ class gemv_prog:
         self.event_items = frozenset(event_items)
         self._events_off = False
         self._host_A_cache = None
+        self._finite_cache = {}
         self._many_thin_rows = False
         self.A, self.A_js, self.X, self.X_js = A, A_js, X, X_js
         self.Y = Y
@@ -165,9 +178,17 @@ class gemv_prog:
         self.float_alpha = float(self.alpha[0]) if n and np.all(self.alpha == self.alpha[0]) else None
         self.float_beta = float(self.beta[0]) if n and np.all(self.beta == self.beta[0]) else None
         self.float_gamma = float(self.gamma[0]) if n and np.all(self.gamma == self.gamma[0]) else None
+        # coefficients the reference computes with as double literals; where float32 does not
+        # hold one of them exactly the launch takes the kernel that multiplies in double
+        # (the kernels in their own summation order agree to a tolerance only anyway)
+        self.literals = [_literal_coefficient(c, n) for c in (alpha, beta, gamma)]
+        self._literal_kernel = (
+            self.force_flavor is None and not self.force_scalar
+            and any(c is not None and float(np.float32(c)) != c for c in self.literals))
 
         self.geometry = self._geometry()
         self.plans = self.choose_plans()
+        self._host_A_cache = None  # (host copies of matrices: only needed while planning)
 
     # ------------------------------------------------------------ geometry
     def _geometry(self):
@@ -320,25 +341,37 @@ class gemv_prog:
         d = g["dots"][0]
         return (g["y_len"] >= 1 and EVENT_MIN_COLS <= d["a_shape1"] <= EVENT_MAX_COLS
                 and (any_size or g["y_len"] * d["a_shape1"] >= EVENT_MIN_ELEMS)
-                and (d["x_stride0"] == 1 or d["a_shape1"] == 1))
+                and (d["x_stride0"] == 1 or d["a_shape1"] == 1)
+                and self._finite_matrix(d["a_j"]))
 
-    def _host_A(self):
+    def _host_matrix(self, a_j):
+        """Matrix `a_j` of A on the host (one transfer of that matrix, kept: the launch
+        that visits active columns needs it again for its transposed copy)."""
         if self._host_A_cache is None:
-            self._host_A_cache = self.A.to_host()
-        return self._host_A_cache
+            self._host_A_cache = {}
+        if a_j not in self._host_A_cache:
+            self._host_A_cache[a_j] = np.array(self.A[int(a_j)], dtype=np.float32)
+        return self._host_A_cache[a_j]
+
+    def _finite_matrix(self, a_j):
+        """Skipping the columns whose x is zero equals the dense product only while no
+        skipped product would be 0 * inf or 0 * nan: matrices with a non-finite entry keep
+        the dense launch."""
+        if a_j not in self._finite_cache:
+            self._finite_cache[a_j] = bool(np.isfinite(self._host_matrix(a_j)).all())
+        return self._finite_cache[a_j]
 
     def _event_plan(self, members):
         """The launch of `nhip_gemv_events` for `members`: their matrices transposed into a
         device buffer of their own (column c of an item: `mp` consecutive floats)."""
         queue, geometry = self.queue, self.geometry
-        host = self._host_A()
         rows, parts, cursor, record_item = [], [], 0, []
         for b in members:
             g = geometry[b]
             d = g["dots"][0]
             M, N = g["y_len"], d["a_shape1"]
             mp = -(-M // 16) * 16
-            block = np.asarray(host[d["a_j"]], dtype=np.float32).reshape(M, N)
+            block = self._host_matrix(d["a_j"]).reshape(M, N)
             t = np.zeros((N, mp), dtype=np.float32)
             t[:, :M] = block.T
             coefs = np.array([self.alpha[b], self.beta[b], self.gamma[b]], dtype=np.float32)
@@ -456,6 +489,9 @@ class gemv_prog:
                         if geometry[b]["dots"] and geometry[b]["y_len"] >= THIN_MIN_ROWS
                         and max(d["a_shape1"] for d in geometry[b]["dots"]) <= 4)
         self._many_thin_rows = thin_rows >= THIN_ROWS_FOR_LANE_PER_ROW
+
+        if self._literal_kernel:
+            return self._literal_plans(items, item_tab, dot_tab)
 
         by_class = defaultdict(list)
         for b in items:
@@ -608,6 +644,41 @@ class gemv_prog:
             plan.host_tables = (item_tab, coef_tab, task_tab)  # (for plans that extend the launch)
             plans.append(plan)
         return plans
+
+    def _literal_plans(self, items, item_tab, dot_tab):
+        """One launch of `nhip_gemv_rows_literal` for all of `items`: a task per output row,
+        the coefficients as doubles (the literal where the reference writes one, else the
+        float32 value)."""
+        queue, geometry = self.queue, self.geometry
+        members = [b for b in items if geometry[b]["y_len"] > 0]
+        if not members:
+            return []
+        dcoefs = np.zeros((len(geometry), 4), dtype=np.float64)
+        for k, (lit, per_item) in enumerate(zip(self.literals, (self.alpha, self.beta, self.gamma))):
+            dcoefs[:, k] = per_item.astype(np.float64) if lit is None else lit
+        counts = np.array([geometry[b]["y_len"] for b in members], dtype=np.int64)
+        task_tab = np.zeros((int(counts.sum()), 4), dtype=np.int32)
+        task_tab[:, 0] = np.repeat(np.array(members, dtype=np.int32), counts)
+        task_tab[:, 1] = np.arange(int(counts.sum())) - np.repeat(np.cumsum(counts) - counts, counts)
+        task_tab[:, 2] = 1
+        # (device arrays are float32 or int32: the doubles travel as pairs of words)
+        dev = [to_device(queue, t) for t in (item_tab, dcoefs.view(np.int32), dot_tab, task_tab)]
+        n_tasks = len(task_tab)
+        args = tuple(d.ptr for d in dev) + (n_tasks, self.A.ptr, self.X.ptr, self.Y_in.ptr, self.Y.ptr)
+        plan = Plan(queue, queue.lib.nhip_gemv_rows_literal, args,
+                    gsize=(WG * -(-n_tasks // ((WG // WAVE) * (WAVE // 4))),), lsize=(WG,),
+                    full_args=tuple(dev) + (self.A.dev_buf, self.X.dev_buf, self.Y_in.dev_buf,
+                                            self.Y.dev_buf),
+                    name="hipra_gemv.wave_ref_literal", tag="%s-literal" % self.tag,
+                    bw_per_call=bw_from_geometry(geometry, members),
+                    flops_per_call=flops_from_geometry(geometry, members))
+        plan.description = self.geometry_summary(members)
+        plan.kernel_class = (5, 4, 1)
+        plan.n_tasks = n_tasks
+        plan.members = list(members)
+        plan.prog = self
+        plan.host_tasks = None
+        return [plan]
 
     def choose_plans(self):
         return self._build(list(range(len(self.Y))))

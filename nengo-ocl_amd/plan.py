@@ -194,10 +194,13 @@ class _GraphSegment:
     MAX_UNROLL = 128
     MAX_GRAPH_NODES = 256
 
-    def __init__(self, queue, plans):
+    def __init__(self, queue, plans, before_last=()):
         self.queue = queue
         self.plans = list(plans)
+        # plans that run once per `launch`, between its last timestep and the one before
+        self.before_last = list(before_last)
         self.execs = {}  # timesteps per graph -> executable graph
+        self.tail_execs = {}  # the same with `before_last` recorded ahead of the last step
         unroll = 1
         while unroll * 2 <= self.MAX_UNROLL and unroll * 2 * len(self.plans) <= self.MAX_GRAPH_NODES:
             unroll *= 2
@@ -212,13 +215,17 @@ class _GraphSegment:
             n //= 2
         return out
 
-    def capture(self, n_steps=1):
-        """Record `n_steps` consecutive timesteps into one executable graph."""
+    def capture(self, n_steps=1, tail=False):
+        """Record `n_steps` consecutive timesteps into one executable graph (`tail`: with
+        the `before_last` plans ahead of the last of them)."""
         lib = self.queue.lib
         _lib.check(lib.nhip_capture_begin(self.queue.handle), "graph capture begin")
         err = None
         try:
-            for _ in range(n_steps):
+            for k in range(n_steps):
+                if tail and k == n_steps - 1:
+                    for plan in self.before_last:
+                        plan.enqueue()
                 for plan in self.plans:
                     plan.enqueue()
         except Exception as e:  # close the capture before re-raising
@@ -230,7 +237,7 @@ class _GraphSegment:
                 lib.nhip_graph_destroy(handle)
             raise err
         _lib.check(rc, "graph capture end")
-        self.execs[n_steps] = handle
+        (self.tail_execs if tail else self.execs)[n_steps] = handle
 
     def steps_of_every_graph(self):
         """A step count whose run launches each recorded graph once."""
@@ -239,38 +246,46 @@ class _GraphSegment:
     def prepare(self):
         """Record every graph `launch` can ask for and hand each to the device ahead of
         its first launch; nothing is executed."""
-        for n_steps in self.sizes:
-            if n_steps not in self.execs:
-                self.capture(n_steps)
-                _lib.check(self.queue.lib.nhip_graph_upload(self.execs[n_steps], self.queue.handle),
-                           "graph upload")
+        for tail, execs in ((False, self.execs), (True, self.tail_execs)):
+            if tail and not self.before_last:
+                continue
+            for n_steps in self.sizes:
+                if n_steps not in execs:
+                    self.capture(n_steps, tail=tail)
+                    _lib.check(self.queue.lib.nhip_graph_upload(execs[n_steps], self.queue.handle),
+                               "graph upload")
 
     @property
     def exec(self):
         return self.execs.get(1)
 
-    def launch(self, n):
+    def launch(self, n, tail=True):
+        """Run `n` timesteps: n // unroll launches of the long graph plus the binary rest.
+        With `before_last` plans (and `tail`), the graph that holds the last timestep is the
+        variant with those plans recorded ahead of its last step."""
         lib = self.queue.lib
         self.prepare()
         times, rest = divmod(n, self.unroll)
-        if times:
-            _lib.check(lib.nhip_graph_launch(self.execs[self.unroll], self.queue.handle, times),
+        todo = [(self.unroll, times)] if times else []
+        todo += [(n_steps, 1) for n_steps in self.sizes[1:] if rest & n_steps]
+        if tail and self.before_last and todo:
+            n_steps, count = todo[-1]
+            todo[-1:] = ([(n_steps, count - 1)] if count > 1 else []) + [(n_steps, -1)]
+        for n_steps, count in todo:
+            execs = self.tail_execs if count < 0 else self.execs
+            _lib.check(lib.nhip_graph_launch(execs[n_steps], self.queue.handle, abs(count)),
                        "graph launch")
-        for n_steps in self.sizes[1:]:
-            if rest & n_steps:
-                _lib.check(lib.nhip_graph_launch(self.execs[n_steps], self.queue.handle, 1),
-                           "graph launch")
 
     def destroy(self):
-        for handle in self.execs.values():
+        for handle in list(self.execs.values()) + list(self.tail_execs.values()):
             self.queue.lib.nhip_graph_destroy(handle)
-        self.execs = {}
+        self.execs, self.tail_execs = {}, {}
 
 
 class Plans:
     """The ordered plan list of one timestep and its executor."""
 
-    def __init__(self, planlist, profiling, use_graph=True, branches=False):
+    def __init__(self, planlist, profiling, use_graph=True, branches=False, before_last=()):
         if branches and use_graph:
             # Switched off: ending a multi-stream recording crashed inside the HIP runtime
             # (segmentation fault in the call that ends the capture) for a step whose
@@ -280,6 +295,10 @@ class Plans:
                 "recording independent kernels as parallel graph branches is switched off "
                 "(the runtime did not survive ending such a recording); use branches=False")
         self.plans = list(planlist)
+        # device plans that every `call_n_times(n)` runs once, after timestep n - 1 and
+        # before timestep n (copies of what the host may ask for as it was before the last
+        # step); not part of a timestep, not listed among `plans`
+        self.before_last = list(before_last)
         self.profiling = profiling
         self.use_graph = use_graph
         self._segments = None  # list of _GraphSegment | PythonPlan
@@ -307,7 +326,7 @@ class Plans:
 
         def close_run():
             if run:
-                segments.append(_GraphSegment(run[0].queue, run))
+                segments.append(_GraphSegment(run[0].queue, run, before_last=self.before_last))
 
         for plan in self.plans:
             if hasattr(plan, "enqueue"):
@@ -358,7 +377,10 @@ class Plans:
         queue = self._queue()
         if self.profiling or not self.use_graph:
             # eager: one launch per plan, events around each when profiling
-            for _ in range(n):
+            for k in range(n):
+                if k == n - 1:
+                    for plan in self.before_last:
+                        plan.enqueue() if hasattr(plan, "enqueue") else plan()
                 for plan in self.plans:
                     if hasattr(plan, "enqueue"):
                         plan.enqueue(profiling=self.profiling)
@@ -372,10 +394,13 @@ class Plans:
         if len(self._segments) == 1 and isinstance(self._segments[0], _GraphSegment):
             self._segments[0].launch(n)  # the common case: n replays, one C call
             return
-        for _ in range(n):
+        for k in range(n):
+            if k == n - 1:
+                for plan in self.before_last:
+                    plan.enqueue()
             for seg in self._segments:
                 if isinstance(seg, _GraphSegment):
-                    seg.launch(1)
+                    seg.launch(1, tail=False)
                 else:
                     queue and queue.finish()
                     seg()

@@ -251,15 +251,31 @@ class Simulator:
     (`operators.apply_learning_in_place`); ``learn_in_place=False`` keeps the two passes;
     ``dedup=False`` keeps products and synapses that compute the same values from the same
     inputs as separate operators (`operators.merge_identical_chains`).
+
+    What the host sees through ``sim.signals`` follows the reference whatever rewrites are
+    on (`_host_state_rules`): a learned matrix that the rule updates in place and a node
+    input that synapses write directly are read from a copy taken before the last step of
+    every ``run_steps`` (the value the reference holds between two steps); signals that a
+    rewrite no longer computes (the delta matrix of such a rule, a vector whose copy was
+    cut out) raise ``ValueError`` when read instead of returning stale memory; writes to a
+    learned matrix updated in place, to a signal that merged connections share or to a
+    constant with a second device copy raise ``ValueError`` naming the constructor switch
+    that makes them possible.  ``reference_host_state=True`` switches ``learn_in_place``,
+    ``dedup``, the rewrites that move writes (``products_write_their_target``,
+    ``propagate_vector_copies``) and the second copies of constants off in one go: every
+    signal is then readable and writable as in the reference.
     """
 
     def __init__(self, network, dt=0.001, seed=None, model=None, context=None,
                  n_prealloc_probes=None, profiling=None, if_python_code="none",
                  planner=batching_planner, progress_bar=True, backend=None, use_graph=True,
                  fuse=True, branches=False, merge_small=True, learn_in_place=True,
-                 dedup=True):
+                 dedup=True, reference_host_state=False):
         self.closed = False
         self.model = None
+        if reference_host_state:
+            learn_in_place = dedup = False
+        self.reference_host_state = bool(reference_host_state)
 
         if profiling is None:
             profiling = int(os.getenv("NENGO_OCL_PROFILING", "0"))
@@ -301,12 +317,13 @@ class Simulator:
         if fuse:
             operators = ops_mod.fuse_into_multidotinc(operators)
             operators = ops_mod.sparse_products_set_their_target(operators)
-            operators = ops_mod.neurons_read_constant_input(operators, keep=probed)
+            if not reference_host_state:
+                operators = ops_mod.neurons_read_constant_input(operators, keep=probed)
             if learn_in_place:
                 operators = ops_mod.apply_learning_in_place(operators, keep=probed)
         operators = MultiDotInc.compress(operators)
         op_groups = planner(operators)
-        if fuse:
+        if fuse and not reference_host_state:
             # cutting vector copies out of the graph saves launches in chains of small
             # operators, but it can also split a group of like operators whose members no
             # longer depend on the same things: keep it only where the step gets shorter
@@ -331,6 +348,9 @@ class Simulator:
         all_signals = stable_unique(sig for op in all_operators + operators
                                     for sig in op.all_signals)
         all_bases = stable_unique(sig.base for sig in all_signals)
+        self._host_state_rules(all_operators, operators, probed)
+        if self._not_computed:  # nothing reads or writes them any more: no device memory
+            all_bases = [b for b in all_bases if b not in self._not_computed]
         if self.signal_aliases:
             # duplicates (and the constants only they read) take no device memory: they
             # resolve to the signal that replaces them
@@ -451,7 +471,8 @@ class Simulator:
                 plans = self.backend.carry_sequences(plans)
         logger.info("Plans in %0.3f s", _time.time() - t0)
 
-        self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches)
+        self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches,
+                            before_last=self._plan_host_view())
         self.rng = None
         self._drain = None
         if hasattr(self.backend, "probe_drain"):
@@ -460,6 +481,48 @@ class Simulator:
                                                    self.sidx[self.model.time])
         self._reset_probes()
         self._plans.prepare()  # record the step graphs now, not inside the first run
+
+    def _host_state_rules(self, all_operators, operators, probed):
+        """Which signals the host cannot read or write as they lie in device memory, given
+        the rewritten operator list (reference semantics of the accessor:
+        nengo_ocl/simulator.py:427-471).
+
+        ``_not_computed``: bases some operator of the model writes but no operator of the
+        rewritten list touches (and that are neither probed nor aliases of a survivor):
+        reading them raises.  ``_updated_in_place``: matrices a learning rule adds its
+        change to directly; with ``signals_a_step_ahead`` they make up ``_host_view``, the
+        bases read from a copy taken before the last step.  ``_shared``: bases that stand
+        for several signals of the model (survivors of a merge and what resolves to them)."""
+        written = lambda ops: {sig.base for op in ops
+                               for sig in list(op.sets) + list(op.incs) + list(op.updates)}
+        touched = {sig.base for op in operators for sig in op.all_signals}
+        touched |= {sig.base for sig in probed}
+        aliased = {sig.base for sig in self.signal_aliases}
+        self._not_computed = {b for b in written(all_operators)
+                              if b not in touched and b not in aliased}
+        self._updated_in_place = {
+            op.delta.base for op in operators
+            if type(op).__name__ in ops_mod.LEARNING_RULES and getattr(op, "apply_inc", False)}
+        self._shared = aliased | {sig.base for sig in self.signal_aliases.values()}
+        self._host_view = stable_unique(
+            [b for b in self._updated_in_place] + [b.base for b in self.signals_a_step_ahead])
+        self._host_view_index = {b: k for k, b in enumerate(self._host_view)}
+        self._host_view_copy = None
+
+    def _plan_host_view(self):
+        """The plan that copies every base of ``_host_view`` aside; the executor runs it
+        before the last timestep of each ``run_steps``."""
+        if not self._host_view:
+            return []
+        X = self.all_data[[self.sidx[b] for b in self._host_view]]
+        self._host_view_copy = self.RaggedArray(
+            [np.zeros((int(X.shape0s[k]), int(X.shape1s[k]))) for k in range(len(X))],
+            dtype=np.float32)
+        plan = self.backend.plan_copy(self.queue, X, self._host_view_copy,
+                                      np.zeros(len(X), dtype=np.int32))
+        self._host_view_plan = plan
+        plan()  # nothing has run yet: the copy holds the initial values
+        return [plan]
 
     def _fuse_input_sums(self, plans):
         """A launch that only adds up the decoded inputs of ensembles, right before the
@@ -667,7 +730,21 @@ class Simulator:
                 return len(sim.all_bases)
 
             def __getitem__(self, item):
-                raw = sim.all_data[sim.sidx[item]]
+                base = item.base
+                if base in sim._not_computed:
+                    raise ValueError(
+                        "%s is not computed by this simulator: a rewrite of the operator "
+                        "graph folded it into another operator (a learning rule that updates "
+                        "its matrix in place does not write its delta; a vector that was only "
+                        "a copy is read at its source).  Simulator(reference_host_state=True) "
+                        "keeps every signal of the model." % (item,))
+                if base in sim._host_view_index:
+                    # between two steps the reference holds what this signal was before
+                    # the last step's update of it
+                    full = np.array(sim._host_view_copy[sim._host_view_index[base]])
+                    raw = full if base is item else sim._view_of(item, full)
+                else:
+                    raw = sim.all_data[sim.sidx[item]]
                 if item.ndim == 0:
                     return raw[0, 0]
                 if item.ndim == 1:
@@ -678,11 +755,38 @@ class Simulator:
 
             def __setitem__(self, item, val):
                 incoming = np.asarray(val)
-                if item.base in sim._copied_constants:
+                base = item.base
+                if base in sim._shared:
+                    raise ValueError(
+                        "%s shares its memory with other signals of the model that compute "
+                        "the same values (merged connections): a write would change all of "
+                        "them.  Simulator(dedup=False) keeps them apart." % (item,))
+                resolved = sim.signal_aliases.get(base, base)
+                if base in sim._copied_constants or resolved in sim._copied_constants:
                     raise ValueError(
                         "%s is a constant whose device copy in another layout would go stale; "
-                        "build the simulator with NENGO_HIP_EVENT_GEMV=0 to change it at run "
-                        "time" % (item,))
+                        "build the simulator with NENGO_HIP_EVENT_GEMV=0 (or "
+                        "reference_host_state=True) to change it at run time" % (item,))
+                if base in sim._not_computed:
+                    raise ValueError(
+                        "%s is not computed by this simulator (see reading it); "
+                        "Simulator(reference_host_state=True) keeps every signal" % (item,))
+                if base in sim._updated_in_place:
+                    raise ValueError(
+                        "%s is updated in place by its learning rule: the change of the last "
+                        "step is already part of it and a write would lose it.  "
+                        "Simulator(learn_in_place=False) keeps the reference's two passes."
+                        % (item,))
+                if base in sim._host_view_index:
+                    # a node input that synapses write directly: the reference overwrites
+                    # it at the start of the next step, so a host write only changes what
+                    # the host reads back, not the simulation
+                    k = sim._host_view_index[base]
+                    full = np.array(sim._host_view_copy[k])
+                    window = sim._view_of(item, full)
+                    window[...] = incoming.reshape(window.shape)
+                    sim._host_view_copy[k] = full
+                    return
                 if item.ndim == 0:
                     assert incoming.size == 1
                     sim.all_data[sim.sidx[item]] = incoming
@@ -703,6 +807,17 @@ class Simulator:
 
         return Accessor()
 
+    def _view_of(self, sig, base_array):
+        """The window of ``base_array`` (the 2-D image of ``sig.base``) that ``sig`` covers,
+        in the 2-D shape the ragged index gives the view."""
+        i, b = self.sidx[sig], self.sidx[sig.base]
+        ra = self.all_data
+        offset = int(ra.starts[i]) - int(ra.starts[b])
+        flat = base_array.reshape(-1)
+        return np.lib.stride_tricks.as_strided(
+            flat[offset:], shape=(int(ra.shape0s[i]), int(ra.shape1s[i])),
+            strides=(4 * int(ra.stride0s[i]), 4 * int(ra.stride1s[i])))
+
     def clear_probes(self):
         for probe in self.model.probes:
             self._probe_outputs[probe] = []
@@ -719,6 +834,8 @@ class Simulator:
         self._raggedarrays_to_reset = None
         self._probe_plan = None
         self._drain = None
+        self._host_view_copy = None
+        self._host_view_plan = None
 
     # ---------------------------------------------------------------- probes
     def _probe(self, steps_since_drain=None):
@@ -805,6 +922,8 @@ class Simulator:
             plan.reset_streams()
         for rng, state in self._python_rngs.items():
             rng.set_state(state)
+        if self._host_view_copy is not None:
+            self._host_view_plan()
         self._reset_probes()
 
     # ------------------------------------------------------------------- run
@@ -899,7 +1018,7 @@ class Simulator:
         if len(constant_bs) != len(ops):
             raise NotImplementedError("signal-valued beta")
         extra = {}
-        if getattr(self.backend, "event_driven_products", False):
+        if getattr(self.backend, "event_driven_products", False) and not self.reference_host_state:
             # products of a constant matrix with the spikes of a population: only the columns
             # of the neurons that spiked need to be visited
             spikes = {op2.output.base for op2 in self.operators

@@ -90,6 +90,17 @@ def _plan(fn, name, keep, tag=None):
 
 
 # --------------------------------------------------------------------- GEMV
+def _gemv_coefficient(arg, n):
+    """alpha / beta / gamma per item as the doubles the reference's kernels compute with
+    (clra_gemv.py:17-32 `float_cl_clra`): a Python float, or a list whose values are all
+    equal, is written into the kernel text as a double literal; values that differ from
+    item to item become a float32 device array."""
+    v = np.asarray(arg, dtype=np.float64)
+    if v.ndim == 0 or len(set(v.ravel().tolist())) == 1:
+        return _per_item(v if v.ndim == 0 else v.ravel()[0], n, np.float64)
+    return _per_item(np.asarray(arg, dtype=np.float32), n, np.float64)
+
+
 class plan_block_gemv:
     """``Y = beta*Y_in + gamma + alpha * sum_j A[A_js[j]] @ X[X_js[j]]`` in the
     block order of clra_gemv.py:861-1175 (32x128 tiles, 4 strided partial sums)."""
@@ -116,8 +127,7 @@ class plan_block_gemv:
             _i32(Y.starts), _i32(Y.stride0s), _i32(Y.shape0s), _i32(Y_in.starts),
             _i32(Y_in.stride0s), _i32(dot_ptr), _i32(A.starts[a_idx]), _i32(A.stride0s[a_idx]),
             _i32(A.shape1s[a_idx]), _i32(X.starts[x_idx]), _i32(X.stride0s[x_idx]),
-            _per_item(alpha, n, np.float64), _per_item(beta, n, np.float64),
-            _per_item(gamma, n, np.float64),
+            _gemv_coefficient(alpha, n), _gemv_coefficient(beta, n), _gemv_coefficient(gamma, n),
         ]
         fn = lib().orc_gemv_block
 

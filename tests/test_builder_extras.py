@@ -156,8 +156,10 @@ def test_unsupported_combinations_raise():
 def test_learning_in_place_gives_the_same_simulation(rule_type):
     """`learn_in_place=True`: the rule adds its change to the learned matrix itself (no
     delta matrix, no copy).  Probe data of every step are bit-identical to the two-pass
-    form; the matrix read from the host after n steps equals the two-pass matrix after its
-    next copy, i.e. with the last step's delta added."""
+    form.  In device memory the matrix is a step ahead of the two-pass one (it already holds
+    the last step's change); what the host reads through `sim.signals` is the two-pass value
+    all the same (a copy taken before the last step), the delta matrix is gone and says so,
+    and a write to the matrix is refused."""
     from nengo_ocl_amd import configs
 
     def make():
@@ -188,9 +190,23 @@ def test_learning_in_place_gives_the_same_simulation(rule_type):
         for n in (1, 50, 150):
             two_pass.run_steps(n)
             in_place.run_steps(n)
-            for (w_a, d_a), (w_b, _) in zip(learned(two_pass), learned(in_place)):
-                want = np.array(two_pass.signals[w_a]) + np.array(two_pass.signals[d_a])
-                assert np.array_equal(np.array(in_place.signals[w_b]), want)
+            for (w_a, d_a), (w_b, d_b) in zip(learned(two_pass), learned(in_place)):
+                assert np.array_equal(np.array(in_place.signals[w_b]),
+                                      np.array(two_pass.signals[w_a]))
+                ahead = np.array(two_pass.signals[w_a]) + np.array(two_pass.signals[d_a])
+                assert np.array_equal(np.array(in_place.all_data[in_place.sidx[w_b]]), ahead)
+                with pytest.raises(ValueError, match="not computed"):
+                    in_place.signals[d_b]
+                with pytest.raises(ValueError, match="updated in place"):
+                    in_place.signals[w_b] = np.zeros(w_b.shape)
+        in_place.reset()
+        two_pass.reset()
+        for (w_a, _), (w_b, _) in zip(learned(two_pass), learned(in_place)):
+            assert np.array_equal(np.array(in_place.signals[w_b]), np.array(two_pass.signals[w_a]))
+        two_pass.run_steps(7)
+        in_place.run_steps(7)
+        for (w_a, _), (w_b, _) in zip(learned(two_pass), learned(in_place)):
+            assert np.array_equal(np.array(in_place.signals[w_b]), np.array(two_pass.signals[w_a]))
         for a, b in zip(probes_a, probes_b):
             assert np.array_equal(two_pass.data[a], in_place.data[b])
         assert any(np.abs(np.array(two_pass.signals[d])).max() > 0 for _, d in learned(two_pass))

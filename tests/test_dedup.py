@@ -27,6 +27,13 @@ def _same_everywhere(a, b, probes, steps):
         assert np.any(a.data[p] != 0)
     bases = {sig.base for op in model.operators for sig in op.all_signals
              if not getattr(sig, "sparse", False)}
+    # signals a rewrite folded into another operator (deltas of rules that update in place,
+    # vectors that were only copies) say so when read; which ones depends on the rewrites
+    for sim in (a, b):
+        for base in sim._not_computed:
+            with pytest.raises(ValueError, match="not computed"):
+                sim.signals[base]
+    bases -= a._not_computed | b._not_computed
     assert bases <= set(b.all_bases)
     for base in bases:  # every signal of the model, dropped ones through their alias
         got, want = np.asarray(a.signals[base]), np.asarray(b.signals[base])
@@ -168,3 +175,57 @@ def test_a_view_or_second_writer_blocks_the_merge():
     assert len(ops_mod.merge_identical_chains(viewed)) == len(viewed)
     extra = base + [ir.DotInc(W1, x, y2)]  # y2 gets one increment more than y1
     assert len(ops_mod.merge_identical_chains(extra)) == len(extra)
+
+
+def test_host_writes_to_shared_signals_are_refused():
+    """A write through `sim.signals` to a signal that merged connections share -- the dropped
+    duplicate or the survivor -- would change every one of them where the reference changes
+    one (reference accessor: simulator.py:451-463): it raises and names the switch; without
+    the merge the write lands in the one connection."""
+    kw = dict(n_ens=4, n_neurons=128, dims=8, fan_out=3, solver="lstsq")
+    net, probes, _ = configs.c3_large(share_decoded=False, **kw)
+    model, a, b = _pair(net)
+    with a, b:
+        decoders = [(dup, rep) for dup, rep in a.signal_aliases.items()
+                    if dup.ndim == 2 and getattr(dup, "readonly", False)]
+        assert decoders
+        dup, rep = decoders[0]
+        for sig in (dup, rep):
+            with pytest.raises(ValueError, match="dedup=False"):
+                a.signals[sig] = np.zeros(sig.shape)
+        assert np.array_equal(np.asarray(a.signals[dup]), np.asarray(b.signals[dup]))  # reads are fine
+        state = [d for d in a.signal_aliases if d.ndim == 1][0]
+        with pytest.raises(ValueError, match="dedup=False"):
+            a.signals[state] = np.zeros(state.shape)
+        before = np.array(b.signals[rep])
+        b.signals[dup] = np.zeros(dup.shape)  # unmerged: one connection changes
+        assert not np.any(np.asarray(b.signals[dup]))
+        assert np.array_equal(np.asarray(b.signals[rep]), before)
+        b.run_steps(5)
+
+
+@pytest.mark.parametrize("case", ["c1", "c4"])
+def test_reference_host_state_keeps_every_signal(case):
+    """`Simulator(reference_host_state=True)`: no rewrite that changes what lies in signal
+    memory between two steps -- every signal of the model reads as the one-operator-at-a-time
+    interpreter holds it, straight from the buffer, and every non-constant can be written."""
+    from naive_interpreter import NaiveInterpreter
+
+    if case == "c1":
+        net, probes, _ = configs.c1_circconv(dims=8, n_per_dim=20)
+    else:
+        net, probes, _ = configs.c4_pes(n_triples=2, n_neurons=60, dims=3, solver="lstsq")
+    model = net.build_model(dt=0.001)
+    naive = NaiveInterpreter(model)
+    with OracleSimulator(None, model=model, seed=1, reference_host_state=True) as sim:
+        assert not sim._not_computed and not sim._host_view and not sim.signal_aliases
+        assert not sim._updated_in_place and not sim.signals_a_step_ahead
+        sim.run_steps(60)
+        naive.run_steps(60)
+        for key, p in probes.items():
+            assert np.array_equal(sim.data[p], naive.data(p)), key
+        bases = {sig.base for op in model.operators for sig in op.all_signals}
+        for base in bases:
+            got = np.asarray(sim.all_data[sim.sidx[base]], dtype=np.float32).reshape(-1)
+            assert np.array_equal(got, naive.mem[base].reshape(-1)), base
+            sim.signals[base] = np.asarray(sim.signals[base])  # no signal refuses a write

@@ -1259,3 +1259,46 @@ def test_small_item_lif_forms_its_input_sums(queue, monkeypatch, n_ens, wave_tas
             host[i] = v[:, None]
             dev[i] = v
     assert any(host.buf[int(host.starts[i]):][:n_neurons].any() for i in i_S)
+
+
+@pytest.mark.parametrize("coefs", [(0.1, 0.3, 0.7), (0.1, [0.3, 0.25, 0.1, 1.0], 0.0),
+                                   ([0.5, 0.1, 0.2, 1.0], 0.6, [0.7, 0.0, 0.0, 0.1])],
+                         ids=["literals", "beta-per-item", "alpha-gamma-per-item"])
+def test_literal_coefficients_bit_exact(queue, coefs):
+    """Coefficients that float32 does not hold exactly and that are the same for every item
+    are double literals in the reference's kernel text (clra_gemv.py:17-32): the product of
+    alpha with a tile sum, of beta with y_in and the sum with gamma are double operations
+    rounded once.  Such launches take the kernel that does the same -- small and large items,
+    several dot products, strided y_in -- and equal the oracle bit for bit; coefficients
+    float32 holds keep the fast kernels."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(77)
+    shapes = [(7, 3), (300, 130), (64, 1024), (1000, 64)]
+    A = RA([rng.normal(size=s) for s in shapes] + [rng.normal(size=(300, 5))], align=True)
+    X = RA([rng.normal(size=s[1]) for s in shapes] + [rng.normal(size=5)])
+    Y = RA([rng.normal(size=s[0]) for s in shapes])
+    Yin = RA([rng.normal(size=s[0]) for s in shapes])
+    A_js = [np.array([0]), np.array([1, 4]), np.array([2]), np.array([3])]
+    X_js = [np.array([0]), np.array([1, 4]), np.array([2]), np.array([3])]
+    alpha, beta, gamma = coefs
+    Yo = clone(Y)
+    orc.plan_block_gemv(None, alpha, A, A_js, X, X_js, beta, Yo, Y_in=clone(Yin), gamma=gamma).plans[0]()
+    dY = to_dev(queue, Y)
+    prog = g.plan_block_gemv(queue, alpha, to_dev(queue, A), A_js, to_dev(queue, X), X_js, beta, dY,
+                             Y_in=to_dev(queue, Yin), gamma=gamma)
+    assert [p.name for p in prog.plans] == ["hipra_gemv.wave_ref_literal"]
+    for plan in prog.plans:
+        plan()
+    assert np.array_equal(dY.buf, Yo.buf)
+    # the same problem with coefficients float32 holds: the usual kernels, the same bits
+    Yo = clone(Y)
+    orc.plan_block_gemv(None, 0.5, A, A_js, X, X_js, 0.25, Yo, Y_in=clone(Yin), gamma=2.0).plans[0]()
+    dY = to_dev(queue, Y)
+    prog = g.plan_block_gemv(queue, 0.5, to_dev(queue, A), A_js, to_dev(queue, X), X_js, 0.25, dY,
+                             Y_in=to_dev(queue, Yin), gamma=2.0)
+    assert "hipra_gemv.wave_ref_literal" not in [p.name for p in prog.plans]
+    for plan in prog.plans:
+        plan()
+    assert np.array_equal(dY.buf, Yo.buf)

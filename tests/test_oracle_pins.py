@@ -95,6 +95,51 @@ def test_gemv_block_order_is_the_reference_order():
     assert Y[0][0, 0] == total
 
 
+@pytest.mark.parametrize("coefs", [(0.1, 0.3, 0.7), ([0.1, 0.1], [0.3, 0.25], [0.7, 0.7])],
+                         ids=["literals", "beta-per-item"])
+def test_gemv_coefficients_are_double_literals_or_float_arrays(coefs):
+    """`float_cl_clra` (clra_gemv.py:17-32): a coefficient that is the same for every item is
+    written into the kernel text as a double literal, so `alpha * (s0 + s1)` (:1058),
+    `beta * yin` (:1148) and `sum + gamma` (:1153) are double operations rounded to float32
+    once each; coefficients that differ between items are float32 arrays and the operations
+    float32.  Replayed in numpy with values float32 does not hold (0.1, 0.3, 0.7)."""
+    rng = np.random.RandomState(8)
+    n = 200  # two tiles
+    m = 40
+    A = [rng.normal(size=(m, n)).astype(np.float32) for _ in range(2)]
+    x = rng.normal(size=n).astype(np.float32)
+    y0 = [rng.normal(size=m).astype(np.float32) for _ in range(2)]
+    Y = RA(y0)
+    alpha, beta, gamma = coefs
+    orc.plan_block_gemv(None, alpha, RA(A), [np.array([0]), np.array([1])], RA([x]),
+                        [np.array([0]), np.array([0])], beta, Y, gamma=gamma).plans[0]()
+
+    def typed(c, b):  # the operand as the kernel sees it: double literal or float32 element
+        c = np.asarray(c, dtype=np.float64)
+        if c.ndim == 0 or len(set(c.tolist())) == 1:
+            return np.float64(c.ravel()[0])
+        return np.float32(c[b])
+
+    changed = False
+    for b in range(2):
+        al, be, ga = typed(alpha, b), typed(beta, b), typed(gamma, b)
+        for r in range(m):
+            total = np.float32(be * y0[b][r])  # numpy promotes float32 * float64 to float64
+            plain = np.float32(np.float32(be) * y0[b][r])
+            for c0 in range(0, n, 128):
+                s = np.zeros(4, dtype=np.float32)
+                for jj in range(min(128, n - c0)):
+                    s[jj % 4] = np.float32(np.longdouble(A[b][r, c0 + jj]) * np.longdouble(x[c0 + jj])
+                                           + np.longdouble(s[jj % 4]))
+                tile = np.float32(np.float32(s[0] + s[2]) + np.float32(s[1] + s[3]))
+                total = np.float32(total + np.float32(al * tile))
+                plain = np.float32(plain + np.float32(np.float32(al) * tile))
+            want = np.float32(total + ga)
+            changed |= want != np.float32(plain + np.float32(ga))
+            assert Y[b][r, 0] == want, (b, r)
+    assert changed  # float32 coefficients would have given other bits somewhere
+
+
 # ------------------------------------------------------------------- LIF
 def lif_step_float64(dt, J, V, W, tau_rc, tau_ref, amplitude=1.0):
     """nengo's LIF.step as the reference's test_lif_step (:35-91) runs it on the host:

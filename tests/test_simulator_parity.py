@@ -798,13 +798,15 @@ def test_constants_with_a_transposed_copy_cannot_be_set(queue, monkeypatch):
 
     net, probes, _ = configs.c3_large(n_ens=4, n_neurons=1024, dims=16, fan_out=2)
     model = net.build_model(dt=0.001)
-    with Simulator(None, model=model, seed=1) as sim:
+    # (dedup=False: every connection keeps its own matrix, so the only thing in the way of a
+    # write is the transposed copy)
+    with Simulator(None, model=model, seed=1, dedup=False) as sim:
         assert any(getattr(p, "event_driven", False) for p in sim._plans)
         weights = sorted(sim._copied_constants, key=lambda s: str(s.name))[0]
         with pytest.raises(ValueError, match="another layout"):
             sim.signals[weights] = np.zeros(weights.shape)
     monkeypatch.setenv("NENGO_HIP_EVENT_GEMV", "0")
-    with Simulator(None, model=model, seed=1) as sim:
+    with Simulator(None, model=model, seed=1, dedup=False) as sim:
         assert not sim._copied_constants
         sim.signals[weights] = np.zeros(weights.shape)
         sim.run_steps(20)
@@ -844,3 +846,99 @@ def test_constant_weights_between_neurons_visit_active_columns_only(queue):
         for p, q in zip(probes, probes_o):
             assert np.array_equal(gpu.data[p], cpu.data[q]) and np.any(gpu.data[p] != 0)
         assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+
+
+@pytest.mark.gpu
+def test_host_reads_follow_the_reference_under_the_rewrites(queue):
+    """What `sim.signals` returns between two steps, on the device, with every rewrite on:
+    learned decoders that the rule updates in place read as the two-pass simulator holds
+    them (device memory is a step ahead), node inputs that synapses write directly read as
+    the unrewritten simulator holds them, deltas say that they are not computed, writes to
+    in-place matrices are refused, and the copy behind this survives uneven `run_steps`
+    lengths (graphs of several sizes), single steps and `reset`."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    make = lambda: configs.c4_pes(n_triples=3, n_neurons=300, dims=8, solver="lstsq",
+                                  learning_rate=3e-4, sample_every=None)
+    (net_g, _, _), (net_c, _, _) = make(), make()
+    with Simulator(net_g, seed=1) as gpu, \
+            OracleSimulator(net_c, seed=1, reference_host_state=True) as ref:
+        assert gpu._updated_in_place and gpu._plans.before_last
+        pairs = []  # (learned matrix, delta) of the device model / of the reference model
+        for sim in (gpu, ref):
+            rules = [op for op in sim.model.operators if type(op).__name__ == "SimPES"]
+            copies = {op.src: op.dst for op in sim.model.operators if type(op).__name__ == "Copy"}
+            pairs.append([(copies[op.delta], op.delta) for op in rules])
+
+        def check():
+            for (w_g, d_g), (w_r, d_r) in zip(*pairs):
+                want = np.asarray(ref.signals[w_r])
+                assert np.array_equal(np.asarray(gpu.signals[w_g]), want)
+                ahead = want + np.asarray(ref.signals[d_r])
+                assert np.array_equal(np.asarray(gpu.all_data[gpu.sidx[w_g]]), ahead)
+                with pytest.raises(ValueError, match="not computed"):
+                    gpu.signals[d_g]
+                with pytest.raises(ValueError, match="updated in place"):
+                    gpu.signals[w_g] = want
+
+        check()  # nothing run yet: initial values
+        for n in (1, 1, 37, 300, 2):
+            gpu.run_steps(n)
+            ref.run_steps(n)
+            check()
+        gpu.reset()
+        ref.reset()
+        check()
+        gpu.run_steps(21)
+        ref.run_steps(21)
+        check()
+
+    (net_g, probes_g, _), (net_c, probes_c, _) = (configs.c1_circconv(dims=16) for _ in range(2))
+    model_g, model_c = net_g.build_model(dt=0.001), net_c.build_model(dt=0.001)
+    with Simulator(None, model=model_g, seed=1) as gpu, \
+            OracleSimulator(None, model=model_c, seed=1, reference_host_state=True) as ref:
+        assert gpu.signals_a_step_ahead and not ref.signals_a_step_ahead
+        by_name = {str(s.name): s for op in model_c.operators for s in op.all_signals}
+        for n in (1, 50, 13):
+            gpu.run_steps(n)
+            ref.run_steps(n)
+            for sig in gpu.signals_a_step_ahead:
+                got, want = np.asarray(gpu.signals[sig]), np.asarray(ref.signals[by_name[str(sig.name)]])
+                assert np.array_equal(got, want) and (n == 1 or np.any(want != 0)), sig
+        for key in probes_g:
+            assert np.array_equal(gpu.data[probes_g[key]], ref.data[probes_c[key]])
+
+
+@pytest.mark.gpu
+def test_writes_through_merged_signals_are_refused_on_the_device(queue):
+    """Decoders that four connections share after the merge and that the device also keeps
+    transposed: a write through the dropped duplicate or through the survivor raises (it
+    would change all four connections, and the transposed copy would go stale); with
+    `reference_host_state=True` the same write lands in one connection's matrix and the
+    simulation uses it."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+
+    net, probes, _ = configs.c3_large(n_ens=4, n_neurons=1024, dims=16, fan_out=2)
+    model = net.build_model(dt=0.001)
+    with Simulator(None, model=model, seed=1) as sim:
+        assert any(getattr(p, "event_driven", False) for p in sim._plans)
+        dups = [(d, r) for d, r in sim.signal_aliases.items() if d.ndim == 2]
+        assert dups
+        dup, rep = dups[0]
+        assert rep.base in sim._copied_constants and dup.base not in sim._copied_constants
+        for sig in (dup, rep):
+            with pytest.raises(ValueError, match="dedup=False|another layout"):
+                sim.signals[sig] = np.zeros(sig.shape)
+        sim.run_steps(10)
+        assert np.any(np.asarray(sim.signals[dup]))
+    with Simulator(None, model=model, seed=1, reference_host_state=True) as sim:
+        assert not sim.signal_aliases and not sim._copied_constants
+        assert not any(getattr(p, "event_driven", False) for p in sim._plans)
+        before = np.array(sim.signals[rep])
+        sim.signals[dup] = np.zeros(dup.shape)
+        sim.run_steps(10)
+        assert not np.any(np.asarray(sim.signals[dup]))
+        assert np.array_equal(np.asarray(sim.signals[rep]), before)
