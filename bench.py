@@ -23,6 +23,15 @@ The network is built with one decoder matrix, product and synapse per connection
 model builder emits it; the simulator's operator rewrite (`operators.merge_identical_chains`)
 computes identical ones once.  ``--no-dedup`` switches that off (c3 then reads 1.37 GB of
 matrices per step).  Other configurations: ``--config c0|c1|c2|c4|c5``.
+
+Next to ``value`` the line carries ``value_every_column`` (the same network with every
+column of the matrices applied to spikes multiplied, timed by the same rule: ``value``
+itself visits only the columns of the neurons that spiked, whose share is
+``spiking_fraction``), a ``configs`` block with the other benchmark configurations (each
+built, warmed up and timed for ``--config-steps`` steps with the same median rule: steps/s,
+launches per step, GEMV bytes per step and their rate against the 8 TB/s peak) and, in
+``cpu_baseline``, a second entry ``numpy``: the operator list of the same network evaluated
+one operator at a time with numpy in this process (``oracle/numpy_interpreter.py``).
 """
 
 import argparse
@@ -89,6 +98,98 @@ def gemv_summary(sim, profile_steps):
     return rows
 
 
+def timed_steps(sim, steps, max_regions, reserve_steps=0):
+    """Seconds of the median region of exactly `steps` steps of ``run_steps`` between stream
+    synchronisations; a region shorter than 50 ms is timed up to `max_regions` times over.
+    Returns (median, all regions)."""
+    import torch
+
+    def region():
+        sim.queue.finish()
+        t0 = time.perf_counter()
+        sim.run_steps(steps)  # exactly K steps, probe buffers drained at the end
+        sim.queue.finish()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    regions = [region()]
+    while sum(regions) < 0.05 * len(regions) and len(regions) < max_regions and (
+            sim.n_steps + steps + reserve_steps < 2 ** 24 - 1):
+        regions.append(region())
+    return sorted(regions)[len(regions) // 2], regions
+
+
+def warm_up(sim, warmup):
+    """W untimed steps, then one untimed launch of every recorded graph (2^k + ... + 2 + 1
+    steps) so that no timed launch is a graph's first; the graphs themselves were recorded
+    and uploaded when the Simulator was constructed."""
+    import torch
+
+    sim.run_steps(warmup)
+    sim.run_steps(max(sim._plans.steps_of_every_graph(), 1))
+    torch.cuda.synchronize()
+
+
+def split_rows(sim, rows):
+    """(GEMV rows with a rate, rows of launches that visit active columns only)."""
+    event_plans = {str(p) for p in sim._plans if getattr(p, "event_driven", False)}
+    event_rows = [r for r in rows if r["plan"] in event_plans]
+    for r in event_rows:
+        r["gbs"] = None
+    gemv_rows = [r for r in rows if r["name"].startswith("hipra_gemv") and r["bytes"]
+                 and r["plan"] not in event_plans]
+    return gemv_rows, event_rows
+
+
+def spiking_fraction(sim):
+    """Share of the neurons of spiking populations that spiked in the last step."""
+    import numpy as np
+
+    spiking = [op.output for op in sim.operators if type(op).__name__ == "SimNeurons"]
+    n = sum(int(np.asarray(sim.signals[s]).size) for s in spiking)
+    nz = sum(int(np.count_nonzero(np.asarray(sim.signals[s]))) for s in spiking)
+    return nz / max(n, 1)
+
+
+def config_summary(config, steps, warmup, profile_steps, max_regions):
+    """One of the other benchmark configurations at its full size through the same protocol:
+    built, warmed up, `steps` steps timed (median region), then an eager pass with events
+    for the per-launch durations."""
+    from nengo_ocl_amd.simulator import Simulator
+
+    t0 = time.time()
+    (net, probes, _), workload = make_network(config, "shared", 1.0)
+    sim = Simulator(net, seed=1)
+    build_s = time.time() - t0
+    warm_up(sim, warmup)
+    elapsed, regions = timed_steps(sim, steps, max_regions, reserve_steps=profile_steps)
+    rows = gemv_summary(sim, profile_steps)
+    gemv_rows, event_rows = split_rows(sim, rows)
+    gemv_bytes = sum(r["bytes"] for r in gemv_rows)
+    gemv_us = sum(r["avg_us"] for r in gemv_rows)
+    sparse_rows = [r for r in rows if r["name"].startswith("hip_spmv") and r["bytes"]]
+    out = {"workload": workload, "neurons": net.n_neurons, "steps": steps,
+           "steps_per_s": steps / elapsed, "ms_per_step": 1e3 * elapsed / steps,
+           "timed_regions": len(regions), "launches_per_step": len(sim._plans),
+           "plans": [p.name for p in sim._plans],
+           "kernel_us_per_step": sum(r["avg_us"] for r in rows),
+           "gemv_bytes_per_step": gemv_bytes, "gemv_us_per_step": gemv_us,
+           "gemv_gbs": 1e-3 * gemv_bytes / gemv_us if gemv_us else None,
+           "gemv_frac_of_peak": 1e-3 * gemv_bytes / gemv_us / HBM_PEAK_GBS if gemv_us else None,
+           "kernels": [{"plan": r["plan"], "avg_us": round(r["avg_us"], 2),
+                        "gbs": None if r["gbs"] is None else round(r["gbs"], 1)} for r in rows],
+           "build_s": build_s}
+    if event_rows:
+        out["launches_that_visit_active_columns_only"] = [r["plan"] for r in event_rows]
+        out["spiking_fraction"] = spiking_fraction(sim)
+    if sparse_rows:
+        b, us = sum(r["bytes"] for r in sparse_rows), sum(r["avg_us"] for r in sparse_rows)
+        out.update(sparse_bytes_per_step=b, sparse_gbs=1e-3 * b / us,
+                   sparse_frac_of_peak=1e-3 * b / us / HBM_PEAK_GBS)
+    sim.close()
+    return out
+
+
 KERNEL_SOURCES = ("gemv_tile.hip", "gemv_types.h", "gemv_rows.h", "neuron_math.h", "nhip_common.h",
                   "sequence_ops.h", "small_arg_math.h")
 
@@ -149,6 +250,35 @@ def cpu_baseline(config, variant, scale, budget_s, dt_gpu_step):
     return dict(value=n / elapsed, unit="steps/s", cores=oracle.num_threads(), kind="port",
                 sample="%d steps of the same network on the CPU oracle (C restatement of the "
                        "reference kernels, OpenMP over items), %.1f s" % (n, elapsed))
+
+
+def numpy_baseline(config, variant, scale, budget_s):
+    """The single-process NumPy leg: the operator list of the same network (one product per
+    connection, as the builder emits it) evaluated one operator at a time, one numpy
+    expression per operator, matrix-vector products through numpy's `@`."""
+    from oracle.numpy_interpreter import NaiveInterpreter
+
+    try:
+        from threadpoolctl import threadpool_info
+
+        threads = max([int(i.get("num_threads", 1)) for i in threadpool_info()
+                       if i.get("user_api") == "blas"] or [1])
+    except ImportError:
+        threads = None
+    (net, probes, _), _ = make_network(config, variant, scale)
+    sim = NaiveInterpreter(net.build_model(dt=0.001), blas=True)
+    sim.run_steps(1)
+    t0 = time.perf_counter()
+    sim.run_steps(2)
+    per_step = (time.perf_counter() - t0) / 2
+    n = int(max(3, min(2000, budget_s / max(per_step, 1e-6))))
+    t0 = time.perf_counter()
+    sim.run_steps(n)
+    elapsed = time.perf_counter() - t0
+    return dict(value=n / elapsed, unit="steps/s", cores=threads, kind="port",
+                sample="%d steps of the same network, operator by operator in numpy (float32, "
+                       "one process; matrix-vector products through numpy's BLAS, %s threads), "
+                       "%.1f s" % (n, threads, elapsed))
 
 
 def calibrate_copy(n_floats=64 * 1024 * 1024, repeats=20):
@@ -222,35 +352,27 @@ def traffic_floor(queue, n_rows, cols, n_reads=3, n_writes=4, repeats=60):
 def event_driven_report(sim, event_rows, steps_per_s, make_sim, args):
     """What the launches that visit only the columns with x != 0 were given to do: the
     fraction of neurons that spiked in the last step, their algorithmic bytes (which they do
-    not read), and the same simulation with every column multiplied, timed briefly."""
-    import numpy as np
-
-    spiking = [op.output for op in sim.operators if type(op).__name__ == "SimNeurons"]
-    n = sum(int(np.asarray(sim.signals[s]).size) for s in spiking)
-    nz = sum(int(np.count_nonzero(np.asarray(sim.signals[s]))) for s in spiking)
+    not read), and the same simulation with every column multiplied, timed by the same rule
+    as `value` (median of the same number of regions of K steps)."""
     out = {"plans": [r["plan"] for r in event_rows],
            "avg_us": sum(r["avg_us"] for r in event_rows),
            "algorithmic_bytes_per_step": sum(r["bytes"] for r in event_rows),
            "note": "these launches read only the columns of their matrices whose x is not zero "
                    "(results bit-identical to the dense product); their algorithmic bytes are "
                    "not traffic and are left out of gemv_all",
-           "neurons_that_spiked_in_the_last_step": nz / max(n, 1)}
+           "neurons_that_spiked_in_the_last_step": spiking_fraction(sim)}
     if args.no_dense_comparison:
         return out
     os.environ["NENGO_HIP_EVENT_GEMV"] = "0"
     try:
         dense = make_sim()
-        steps = min(max(args.steps, 20), 400)
-        dense.run_steps(args.warmup)
-        dense.run_steps(max(dense._plans.steps_of_every_graph(), 1))
-        dense.queue.finish()
-        t0 = time.perf_counter()
-        dense.run_steps(steps)
-        dense.queue.finish()
-        dt = time.perf_counter() - t0
+        warm_up(dense, args.warmup)
+        elapsed, regions = timed_steps(dense, args.steps, args.max_regions)
         dense.close()
-        out["every_column_multiplied"] = {"steps_per_s": steps / dt, "ms_per_step": 1e3 * dt / steps,
-                                          "steps": steps, "flag": "--dense-decoders"}
+        out["every_column_multiplied"] = {
+            "steps_per_s": args.steps / elapsed, "ms_per_step": 1e3 * elapsed / args.steps,
+            "steps": args.steps, "timed_regions": len(regions), "reported": "median",
+            "flag": "--dense-decoders"}
     finally:
         os.environ.pop("NENGO_HIP_EVENT_GEMV", None)
     out["speedup_over_every_column"] = steps_per_s / out["every_column_multiplied"]["steps_per_s"]
@@ -405,6 +527,14 @@ def main():
     ap.add_argument("--max-regions", type=int, default=25,
                     help="a timed region of K steps shorter than 50 ms is repeated up to this "
                          "many times; the median region is reported")
+    ap.add_argument("--config-steps", type=int, default=1000,
+                    help="timed steps of each of the other configurations in the `configs` "
+                         "block (the benchmark runs of these networks are 1000 steps)")
+    ap.add_argument("--other-configs", default="c0,c1,c2,c4,c5",
+                    help="configurations reported in the `configs` block of a c3 run at full "
+                         "size ('' for none)")
+    ap.add_argument("--numpy-budget", type=float, default=10.0,
+                    help="seconds for the single-process NumPy leg of the CPU baseline; 0 skips it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run the plain copy kernel on 256 MiB (1 GiB of traffic per 2 "
                          "launches) 20 times: the known-size reference for HBM counters")
@@ -439,39 +569,17 @@ def main():
     build_s = time.time() - t0
     n_plans = len(sim._plans)
 
-    # W untimed steps, then one untimed launch of every recorded graph (2^k + ... + 2 + 1
-    # steps) so that no timed launch is a graph's first; the graphs themselves were
-    # recorded and uploaded when the Simulator was constructed
-    sim.run_steps(args.warmup)
-    sim.run_steps(max(sim._plans.steps_of_every_graph(), 1))
-    torch.cuda.synchronize()
-
-    def timed_region():
-        sim.queue.finish()
-        t0 = time.perf_counter()
-        sim.run_steps(args.steps)  # exactly K steps, probe buffers drained at the end
-        sim.queue.finish()
-        torch.cuda.synchronize()
-        return time.perf_counter() - t0
-
+    warm_up(sim, args.warmup)
     # a region shorter than 50 ms is timed several times over (each region is exactly K
     # steps of the running simulation) and the median region is reported
-    regions = [timed_region()]
-    while sum(regions) < 0.05 * len(regions) and len(regions) < args.max_regions and (
-            sim.n_steps + args.steps + args.profile_steps < 2 ** 24 - 1):
-        regions.append(timed_region())
-    elapsed = sorted(regions)[len(regions) // 2]
+    elapsed, regions = timed_steps(sim, args.steps, args.max_regions,
+                                   reserve_steps=args.profile_steps)
     steps_per_s = args.steps / elapsed
 
     rows = gemv_summary(sim, args.profile_steps)
     # launches that visit only the columns of the neurons that spiked do not read their
     # algorithmic bytes: they are reported apart, without a rate
-    event_plans = {str(p) for p in sim._plans if getattr(p, "event_driven", False)}
-    event_rows = [r for r in rows if r["plan"] in event_plans]
-    for r in event_rows:
-        r["gbs"] = None
-    gemv_rows = [r for r in rows if r["name"].startswith("hipra_gemv") and r["bytes"]
-                 and r["plan"] not in event_plans]
+    gemv_rows, event_rows = split_rows(sim, rows)
     if event_rows:
         workload += ("; matrices applied to spikes are read only in the columns of the neurons "
                      "that spiked (--dense-decoders reads them whole)")
@@ -531,19 +639,39 @@ def main():
         "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,
                      "gbs": 1e-3 * gemv_bytes / gemv_us if gemv_us else None,
                      "frac_of_peak": (1e-3 * gemv_bytes / gemv_us / HBM_PEAK_GBS) if gemv_us else None},
-        "event_driven": event_driven_report(sim, event_rows, steps_per_s, make_sim, args)
-        if event_rows else None,
+        "event_driven": None,
         "kernels": [{"plan": r["plan"], "avg_us": round(r["avg_us"], 2),
                      "gbs": None if r["gbs"] is None else round(r["gbs"], 1)} for r in rows],
         "kernel_us_per_step": step_us_kernels,
         "build_s": build_s,
     }
+    if event_rows:
+        report = event_driven_report(sim, event_rows, steps_per_s, make_sim, args)
+        out["event_driven"] = report
+        # `value` depends on how many neurons spike; the figure that does not is the same
+        # network with every column multiplied, timed by the same rule
+        out["spiking_fraction"] = report["neurons_that_spiked_in_the_last_step"]
+        dense = report.get("every_column_multiplied")
+        out["value_every_column"] = dense["steps_per_s"] if dense else None
+    elif args.dense_decoders:
+        out["value_every_column"] = steps_per_s
+        out["spiking_fraction"] = spiking_fraction(sim)
     sim.close()
     del sim
+    full_size_default = (args.config == "c3" and args.variant == "shared" and args.scale == 1.0
+                         and not (args.no_fuse or args.no_graph or args.two_pass_learning))
+    if full_size_default and args.other_configs:
+        out["configs"] = {}
+        for name in args.other_configs.split(","):
+            out["configs"][name] = config_summary(name, args.config_steps, args.warmup,
+                                                  args.profile_steps, args.max_regions)
     if args.cpu_budget > 0:
         out["cpu_baseline"] = cpu_baseline(args.config, args.variant, args.scale, args.cpu_budget,
                                            elapsed / args.steps)
         out["cpu_baseline"]["host_cpu_count"] = os.cpu_count()
+        if args.numpy_budget > 0:
+            out["cpu_baseline"]["numpy"] = numpy_baseline(args.config, args.variant, args.scale,
+                                                          args.numpy_budget)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -29,6 +29,31 @@ extern thread_local NhipLaunchEvents nhip_launch_events;
         }                                                                                    \
     } while (0)
 
+// An entry point that issues two launches times both: its first launch carries the start
+// event, its last the stop event, so that their difference spans the entry point's work.
+#define NHIP_LAUNCH_FIRST(kernel, grid, block, lds, stream, ...)                             \
+    do {                                                                                     \
+        if (nhip_launch_events.start) {                                                      \
+            const hipEvent_t start_ = nhip_launch_events.start;                              \
+            nhip_launch_events.start = nullptr;                                              \
+            hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, start_, nullptr, 0,      \
+                                  __VA_ARGS__);                                              \
+        } else {                                                                             \
+            hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);               \
+        }                                                                                    \
+    } while (0)
+#define NHIP_LAUNCH_LAST(kernel, grid, block, lds, stream, ...)                              \
+    do {                                                                                     \
+        if (nhip_launch_events.stop) {                                                       \
+            const hipEvent_t stop_ = nhip_launch_events.stop;                                \
+            nhip_launch_events = NhipLaunchEvents{nullptr, nullptr};                         \
+            hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, nullptr, stop_, 0,       \
+                                  __VA_ARGS__);                                              \
+        } else {                                                                             \
+            hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);               \
+        }                                                                                    \
+    } while (0)
+
 #define NHIP_LAUNCH_CHECK()                 \
     do {                                    \
         hipError_t e_ = hipGetLastError();  \

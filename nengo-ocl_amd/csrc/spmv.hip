@@ -289,7 +289,7 @@ int launch_skip(void* stream, const int* slices, int n_slices, const int* row_le
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int n_mask_quads = (n_cols + 127) / 128;        // 128 bits per 16 bytes
     const int n_mask_threads = n_mask_quads * 128;        // one thread per bit, whole quads
-    NHIP_LAUNCH(spmv_mask_kernel, dim3(n_mask_threads / NHIP_WG + (n_mask_threads % NHIP_WG != 0)),
+    NHIP_LAUNCH_FIRST(spmv_mask_kernel, dim3(n_mask_threads / NHIP_WG + (n_mask_threads % NHIP_WG != 0)),
                 dim3(NHIP_WG), 0, s, X + x_start, n_cols, mask, 4 * n_mask_quads);
     NHIP_LAUNCH_CHECK();
     static int n_cu = 0;
@@ -302,7 +302,7 @@ int launch_skip(void* stream, const int* slices, int n_slices, const int* row_le
     }
     const int wpg = SPMV_SKIP_WG / NHIP_WAVE;
     side.n_groups = min(n_cu, (n_slices + wpg - 1) / wpg);
-    NHIP_LAUNCH(spmv_sell_skip_kernel, dim3(side.n_groups + side.n_chains), dim3(SPMV_SKIP_WG), 0, s,
+    NHIP_LAUNCH_LAST(spmv_sell_skip_kernel, dim3(side.n_groups + side.n_chains), dim3(SPMV_SKIP_WG), 0, s,
                 reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X, Y,
                 mask, n_mask_quads, epi, side);
     NHIP_LAUNCH_CHECK();

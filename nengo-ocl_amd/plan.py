@@ -98,7 +98,8 @@ class Plan(BasePlan):
             _lib.check(lib.nhip_event_create(ctypes.byref(ev1)))
             # the kernel carries its own start / stop events where the entry point
             # launches through the runtime API; otherwise events around the launch.  An
-            # entry point that issues several launches times its first one only.
+            # entry point that issues two launches puts the start event on its first and
+            # the stop event on its last.
             own = getattr(self.kern, "__name__", "") not in self.LAUNCHES_WITHOUT_EVENTS
             if own:
                 _lib.check(lib.nhip_time_next_launch(ev0, ev1))

@@ -1,4 +1,6 @@
-"""A model's operator list evaluated one operator at a time in numpy.  TEST INFRASTRUCTURE.
+"""A model's operator list evaluated one operator at a time in numpy.  TEST INFRASTRUCTURE
+(and, with ``blas=True``, the single-process NumPy leg of ``bench.py``'s CPU baseline); the
+product never imports it.
 
 Nothing here uses the simulator's operator rewrites, its planner, its view builder or its
 plan_* layer: every base signal is one float32 array, a view is a strided window onto it,
@@ -9,6 +11,11 @@ or batches operators must still produce these numbers.
 
 The fused multiply-add of the GEMV partial sums is emulated in extended precision (the
 product of two float32 is exact there; one rounding back to float32).
+
+``NaiveInterpreter(model, blas=True)`` forms matrix-vector products with ``A @ x`` instead
+(numpy's float32 product, its own summation order): the way a NumPy simulator of such a
+model computes a step (one array expression per operator), which is what the CPU baseline
+times.  Its results agree with the exact mode to rounding, not bit for bit.
 """
 
 import heapq
@@ -23,8 +30,9 @@ def _fma(a, b, c):
 
 
 class NaiveInterpreter:
-    def __init__(self, model):
+    def __init__(self, model, blas=False):
         self.model = model
+        self.blas = bool(blas)
         self.dt = model.dt
         self.ops = list(model.operators)
         self.mem = {}
@@ -88,6 +96,9 @@ class NaiveInterpreter:
         """y += A @ x the way the reference's block GEMV adds it (clra_gemv.py:1043-1058,
         :1148-1153): per tile of 128 columns four strided partial sums, fused
         multiply-adds, (s0 + s2) + (s1 + s3); tiles added onto y one after the other."""
+        if self.blas:
+            y += A @ x
+            return
         m, n = A.shape
         acc = y.copy()
         for c0 in range(0, n, 128):

@@ -209,7 +209,7 @@ def test_reference_host_state_keeps_every_signal(case):
     """`Simulator(reference_host_state=True)`: no rewrite that changes what lies in signal
     memory between two steps -- every signal of the model reads as the one-operator-at-a-time
     interpreter holds it, straight from the buffer, and every non-constant can be written."""
-    from naive_interpreter import NaiveInterpreter
+    from oracle.numpy_interpreter import NaiveInterpreter
 
     if case == "c1":
         net, probes, _ = configs.c1_circconv(dims=8, n_per_dim=20)

@@ -565,7 +565,7 @@ def test_synapses_write_the_node_input_they_feed():
     part of the node's input themselves (no Reset, no copies); probes equal the
     operator-at-a-time interpreter bit for bit, and the collected input holds, between steps,
     what the next step reads.  A probed node input is left alone."""
-    from naive_interpreter import NaiveInterpreter
+    from oracle.numpy_interpreter import NaiveInterpreter
     from random_networks import ensemble_array_network as make
 
     net, probes = make(probe_node=False)

@@ -1,6 +1,6 @@
 """The simulator's front half (operator rewrites, planner, view builder, probe logic)
 pinned without using any of it: an operator list evaluated one operator at a time by
-`naive_interpreter.NaiveInterpreter` must give the numbers `OracleSimulator` gives with
+`oracle.numpy_interpreter.NaiveInterpreter` must give the numbers `OracleSimulator` gives with
 all of its merging, fusing and batching switched on.  Graph shapes follow the reference's
 own fixtures (tests/test_operators.py:30,54,82, tests/test_planners.py:13-47) and the
 benchmark configurations at reduced sizes."""
@@ -8,7 +8,7 @@ benchmark configurations at reduced sizes."""
 import numpy as np
 import pytest
 
-from naive_interpreter import NaiveInterpreter
+from oracle.numpy_interpreter import NaiveInterpreter
 from nengo_ocl_amd import configs, ir
 from oracle.oracle_sim import OracleSimulator
 

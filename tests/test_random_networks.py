@@ -8,7 +8,7 @@ and the large-item kernels, input sums formed inside both, sequences carried by 
 import numpy as np
 import pytest
 
-from naive_interpreter import NaiveInterpreter
+from oracle.numpy_interpreter import NaiveInterpreter
 from oracle.oracle_sim import OracleSimulator
 from random_networks import random_network
 
