@@ -255,7 +255,8 @@ __device__ __forceinline__ void gemv_rows_ref_block(
     }
     if (lir == 0 && valid) {
         const float y = sum + cf.z;
-        Y[it.y_start + (size_t)r * it.y_stride0] = y;
+        if (!(EPI == EPI_LIF && (pop.pflags & LIF_POP_NO_J)))
+            Y[it.y_start + (size_t)r * it.y_stride0] = y;
         if (EPI == EPI_LIF && (pop.pflags & LIF_POP_ENABLED))
             lif_epilogue(epi->lif, pop, r, y, v_old, w_old);
         if (EPI == EPI_FILTER && f_range.y > 0) {

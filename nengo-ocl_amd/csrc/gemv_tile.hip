@@ -322,7 +322,8 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_tile_kernel(
     // an item without dot products that would copy Y onto itself unchanged is only
     // there for its epilogue (a constant input current): nothing to store
     const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
-                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
+                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0) &&
+                         !(EPI == EPI_LIF && (pop.pflags & LIF_POP_NO_J));
 #pragma unroll
     for (int k = 0; k < ROW_SLOTS; ++k) {
         const int r = lane + k * NHIP_WAVE;
@@ -514,7 +515,8 @@ __device__ __forceinline__ void finish_task(const GemvTask& task, const GemvItem
     // an item without dot products that would copy Y onto itself unchanged is only
     // there for its epilogue (a constant input current): nothing to store
     const bool store_y = !(it.n_dots == 0 && cf.y == 1.0f && cf.z == 0.0f && Y == Yin &&
-                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0);
+                           it.y_start == it.yin_start && it.y_stride0 == it.yin_stride0) &&
+                         !(EPI == EPI_LIF && (pop.pflags & LIF_POP_NO_J));
     if (EPI == EPI_LIF && (pop.pflags & LIF_POP_DECAY)) {
         lif_task_compacted<SLOTS>(epi.lif, pop, task.row0, n_rows, ys, cf.z,
                            store_y ? Y + it.y_start : nullptr, it.y_stride0, ab, lane, v_in, w_in);

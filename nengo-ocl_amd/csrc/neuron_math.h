@@ -14,6 +14,9 @@ struct LifPop {
 };
 constexpr int LIF_POP_ENABLED = 1 << 8;  // pflags: the item has a population at all
 constexpr int LIF_POP_DECAY = 1 << 9;    // pflags: `decay` is set (one tau, upsample == 1)
+// pflags: nothing but this epilogue reads the population's input current (the host's word),
+// so the launch does not store it; the host recomputes it when somebody asks
+constexpr int LIF_POP_NO_J = 1 << 10;
 
 // State arrays and constants of a fused LIF update (all populations of a launch).
 struct LifArgs {

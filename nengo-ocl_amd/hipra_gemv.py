@@ -92,7 +92,7 @@ WIDE_TASK_MAX_ROWS = 65536
 WAVE_TASKS = os.environ.get("NENGO_HIP_WAVE_TASKS", "1") != "0"
 WG, WAVE = 256, 64
 THIN_MIN_ROWS, THIN_ROWS_FOR_LANE_PER_ROW = 32, 65536
-LIF_POP_ENABLED, LIF_POP_DECAY = 1 << 8, 1 << 9  # flag bits of a population row
+LIF_POP_ENABLED, LIF_POP_DECAY, LIF_POP_NO_J = 1 << 8, 1 << 9, 1 << 10  # flag bits of a population row
 LIF_COMPACT = os.environ.get("NENGO_HIP_LIF_COMPACT", "1") != "0"
 
 
@@ -783,7 +783,7 @@ def _epilogue_call(lib, plan, kind, extras=None):
     return getattr(lib, "nhip_gemv_rows_" + kind), (plan.args[1], task_words) + tables, keep
 
 
-def fuse_lif(prog, lif_plan):
+def fuse_lif(prog, lif_plan, unread_currents=()):
     """Fewer launches for "J = GEMV(...); LIF(J)" (clra_gemv.py `plan_block_gemv` followed
     by clra_nonlinearities.py `plan_lif`): the reference-order kernels update the neurons
     of a row (block) as soon as its currents are final, so the currents are not read
@@ -797,6 +797,13 @@ def fuse_lif(prog, lif_plan):
     update writes (voltage, refractory time, spikes) is read by a dot product of
     `prog`.  Returns the plans that replace ``prog.plans + [lif_plan]`` (same results
     bit for bit), or None.
+
+    `unread_currents`: populations (indices into the neuron plan) whose input current the
+    caller knows nothing else reads.  Where such a current is formed from operands other
+    than itself (``J = bias + E x``, not ``J += ...``), the fused launch does not store it;
+    every fused plan carries ``lazy_currents = (those populations, a plain GEMV over their
+    items)``: running that GEMV puts the currents of the last step into their place, bit
+    for bit what the launch would have stored.
     """
     from .hipra_nonlinearities import lif_population_table, plan_lif
 
@@ -860,10 +867,29 @@ def fuse_lif(prog, lif_plan):
         matched = matched + [(p, n_old + k) for k, p in enumerate(idle)]
         Y = prog.Y
 
+    # currents nobody reads are not stored, when the product that forms them can be run
+    # again later with the same result: it must not read the current itself
+    unread = set(unread_currents)
+    lazy = [(p, b) for p, b in matched
+            if p in unread and prog.geometry[b]["dots"] and (
+                prog.beta[b] == 0 or _span(prog.Y_in, b) is None
+                or not _overlaps([_span(prog.Y_in, b)], [_span(Y, b)]))
+            and not any(_overlaps([_span(prog.X, d["x_j"])], [_span(Y, b)])
+                        for d in prog.geometry[b]["dots"])]
+    lazy_currents = None
+    if lazy:
+        sel = [b for _, b in lazy]
+        lazy_prog = plan_block_gemv(
+            queue, prog.alpha[sel], prog.A, [prog.A_js[b] for b in sel], prog.X,
+            [prog.X_js[b] for b in sel], prog.beta[sel], Y[sel], Y_in=prog.Y_in[sel],
+            gamma=prog.gamma[sel], tag="%s-currents-on-demand" % prog.tag)
+        lazy_currents = ([p for p, _ in lazy], lazy_prog)
+    no_store = {p for p, _ in lazy}
+
     cols, pptrs, keep = lif_population_table(queue, spec)
     table = np.zeros((len(Y), 8), dtype=np.int32)
     for p, b in matched:
-        flags = int(cols["pflags"][p]) | LIF_POP_ENABLED
+        flags = int(cols["pflags"][p]) | LIF_POP_ENABLED | (LIF_POP_NO_J if p in no_store else 0)
         decay_bits = 0
         if not (flags & 1) and spec["upsample"] == 1 and LIF_COMPACT:
             # one time constant and no sub-steps: the decay factor of a whole step,
@@ -887,20 +913,25 @@ def fuse_lif(prog, lif_plan):
             out.append(plan)
             continue
         lif_bytes = sum(4 * int(J.shape0s[pop_of[b]]) for b in plan.members if b in pop_of)
+        # (currents that are not stored are not traffic)
+        unstored = sum(4 * int(J.shape0s[pop_of[b]]) for b in plan.members
+                       if b in pop_of and pop_of[b] in no_store)
         entry, args, kept = _epilogue_call(lib, plan, "lif", lambda items: table[items][:, [0, 1, 7]])
         fused = Plan(queue, entry, args + lif_args, gsize=plan.gsize,
                      lsize=plan.lsize,
                      full_args=(plan.full_args + (dev_pops, V.dev_buf, W.dev_buf, S.dev_buf)
                                 + tuple(keep) + kept),
                      name=plan.name + "_lif", tag=plan.tag,
-                     bw_per_call=plan.bw_per_call + 5 * lif_bytes,  # V and W in and out, spikes out
+                     # V and W in and out, spikes out
+                     bw_per_call=plan.bw_per_call + 5 * lif_bytes - unstored,
                      flops_per_call=plan.flops_per_call)
         fused.description = plan.description
         fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
         fused.members, fused.prog = plan.members, prog
-        fused.gemv_bytes = plan.bw_per_call
+        fused.gemv_bytes = plan.bw_per_call - unstored
         fused.host_pops = table
         fused.lif_written = [V, W, S]
+        fused.lazy_currents = lazy_currents
         if plan.kernel_class[0] == 3:
             fused.host_tasks = plan.host_tasks
         else:  # small items: 16-word records as the launch takes them, or the 4-word table
@@ -1079,6 +1110,7 @@ def fuse_input_sums(sum_plan, lif_plan):
     fused.gemv_bytes = getattr(lif_plan, "gemv_bytes", lif_plan.bw_per_call)
     fused.host_tasks = tasks
     fused.input_sums = len(sums)
+    fused.lazy_currents = getattr(lif_plan, "lazy_currents", None)
     return fused
 
 

@@ -72,6 +72,8 @@ class HipBackend:
         self.plan_block_gemv = hipra_gemv.plan_block_gemv
         self._fuse_lif = hipra_gemv.fuse_lif
         self._gemv = hipra_gemv
+        # switch for measurements: "0" stores every input current
+        self.skip_unread_currents = os.environ.get("NENGO_HIP_SKIP_CURRENTS", "1") != "0"
         # switch for measurements: False keeps input sums a launch of their own
         self.input_sums_in_launch = os.environ.get("NENGO_HIP_INPUT_SUMS", "1") != "0"
         from . import hipra_sequence
@@ -99,13 +101,17 @@ class HipBackend:
             return self._gemv.fuse_input_sums(sum_plan, lif_plan)
         return None
 
-    def fuse_gemv_neurons(self, gemv_plans, neuron_plans):
+    def fuse_gemv_neurons(self, gemv_plans, neuron_plans, unread_currents=()):
         """Plans replacing ``gemv_plans + neuron_plans`` by launches that update the
-        neurons in the epilogue of the GEMV that produces their input, or None."""
+        neurons in the epilogue of the GEMV that produces their input, or None.
+        `unread_currents`: populations of the neuron plan whose input current nothing else
+        reads (the launch need not store it)."""
         progs = {id(getattr(p, "prog", None)) for p in gemv_plans}
         if len(neuron_plans) != 1 or len(progs) != 1 or not hasattr(gemv_plans[0], "prog"):
             return None
-        return self._fuse_lif(gemv_plans[0].prog, neuron_plans[0])
+        if not self.skip_unread_currents:
+            unread_currents = ()
+        return self._fuse_lif(gemv_plans[0].prog, neuron_plans[0], unread_currents=unread_currents)
 
     def upload(self, host_ragged):
         return self._ra.HIPRaggedArray(self.queue, host_ragged)
@@ -421,6 +427,8 @@ class Simulator:
         # --- plans
         t0 = _time.time()
         self._raggedarrays_to_reset = []  # (device ragged, host initial)
+        self._lazy_currents = {}  # signal base -> {"prog": GEMV that recomputes it, "at_step"}
+        self._n_steps = 0
         self._filter_positions = []
         self._noise_plans = []
         self._python_rngs = {}
@@ -436,8 +444,10 @@ class Simulator:
                     and previous[0].__name__ == "MultiDotInc" and previous[1]
                     and hasattr(self.backend, "fuse_gemv_neurons")):
                 # neurons right behind the GEMV that computes their input current
-                fused = self.backend.fuse_gemv_neurons(previous[1], group_plans)
+                fused = self.backend.fuse_gemv_neurons(
+                    previous[1], group_plans, unread_currents=self._unread_currents(op_list, probed))
                 if fused is not None:
+                    self._register_lazy_currents(fused, op_list)
                     reads = reads | previous[1][0].reads_mem
                     writes = writes | previous[1][0].writes_mem
                     del plans[len(plans) - len(previous[1]):]
@@ -481,6 +491,61 @@ class Simulator:
                                                    self.sidx[self.model.time])
         self._reset_probes()
         self._plans.prepare()  # record the step graphs now, not inside the first run
+
+    def _unread_currents(self, neuron_ops, probed):
+        """Indices of the neuron operators whose input current only they read and that can
+        be formed again after the step: a whole signal that is not probed, that no other
+        operator reads, increments or updates, that one operator sets, and whose operands
+        (matrices, vectors, the bias it starts from) nothing writes later in the step --
+        a vector that a synapse updates at the end of the step no longer holds what the
+        product read."""
+        if self.reference_host_state or len({type(op.neurons) for op in neuron_ops}) != 1:
+            return ()
+        probed_bases = {sig.base for sig in probed}
+        readers, writers = defaultdict(list), defaultdict(list)
+        when = {}  # operator -> index of its group in the step
+        for g, (_, ops) in enumerate(self.op_groups):
+            for op in ops:
+                when[id(op)] = g
+        for op in self.operators:
+            for sig in list(op.reads) + list(op.incs) + list(op.updates):
+                readers[sig.base].append(op)
+            for sig in list(op.sets) + list(op.incs) + list(op.updates):
+                writers[sig.base].append(op)
+        out = []
+        for k, op in enumerate(neuron_ops):
+            J = op.J
+            if not (J.base is J and J.base not in probed_bases and readers[J.base] == [op]
+                    and len(writers[J.base]) == 1 and J.base not in self._shared):
+                continue
+            product = writers[J.base][0]
+            if all(when[id(w)] < when[id(product)]
+                   for sig in product.reads for w in writers[sig.base]):
+                out.append(k)
+        return out
+
+    def _register_lazy_currents(self, plans, neuron_ops):
+        """Input currents the fused launches do not store: signal base -> the GEMV that
+        puts them into their place when the host asks for them."""
+        for plan in plans:
+            lazy = getattr(plan, "lazy_currents", None)
+            if lazy is None:
+                continue
+            populations, prog = lazy
+            group = {"prog": prog, "at_step": None}
+            for p in populations:
+                self._lazy_currents[neuron_ops[p].J.base] = group
+
+    def _refresh_lazy(self, base):
+        """Make a current that its launch does not store hold the last step's value (the
+        step counter tells whether that was done since the last step)."""
+        group = self._lazy_currents.get(base)
+        # (before the first step the signal holds its initial value, as in the reference)
+        if group is None or self._n_steps == 0 or group["at_step"] == self._n_steps:
+            return
+        for plan in group["prog"].plans:
+            plan()
+        group["at_step"] = self._n_steps
 
     def _host_state_rules(self, all_operators, operators, probed):
         """Which signals the host cannot read or write as they lie in device memory, given
@@ -744,6 +809,7 @@ class Simulator:
                     full = np.array(sim._host_view_copy[sim._host_view_index[base]])
                     raw = full if base is item else sim._view_of(item, full)
                 else:
+                    sim._refresh_lazy(base)
                     raw = sim.all_data[sim.sidx[item]]
                 if item.ndim == 0:
                     return raw[0, 0]
@@ -756,6 +822,7 @@ class Simulator:
             def __setitem__(self, item, val):
                 incoming = np.asarray(val)
                 base = item.base
+                sim._refresh_lazy(base)  # (a later read must not recompute over the write)
                 if base in sim._shared:
                     raise ValueError(
                         "%s shares its memory with other signals of the model that compute "
@@ -817,6 +884,21 @@ class Simulator:
         return np.lib.stride_tricks.as_strided(
             flat[offset:], shape=(int(ra.shape0s[i]), int(ra.shape1s[i])),
             strides=(4 * int(ra.stride0s[i]), 4 * int(ra.stride1s[i])))
+
+    def signal_buffer(self):
+        """A host copy of the whole signal buffer as the reference holds it between two
+        steps: currents that their launch does not store are brought up to date first, and
+        signals that device memory holds a step ahead are taken from the copy made before
+        the last step."""
+        for base in list(self._lazy_currents):
+            self._refresh_lazy(base)
+        buf = np.array(self.all_data.buf)
+        for base, k in self._host_view_index.items():
+            i = self.sidx[base]
+            start = int(self.all_data.starts[i])
+            flat = np.asarray(self._host_view_copy[k], dtype=np.float32).reshape(-1)
+            buf[start:start + flat.size] = flat
+        return buf
 
     def clear_probes(self):
         for probe in self.model.probes:
@@ -924,6 +1006,8 @@ class Simulator:
             rng.set_state(state)
         if self._host_view_copy is not None:
             self._host_view_plan()
+        for group in self._lazy_currents.values():
+            group["at_step"] = None
         self._reset_probes()
 
     # ------------------------------------------------------------------- run

@@ -8,6 +8,8 @@ benchmark configurations at reduced sizes."""
 import numpy as np
 import pytest
 
+from helpers import assert_same_signals
+
 from oracle.numpy_interpreter import NaiveInterpreter
 from nengo_ocl_amd import configs, ir
 from oracle.oracle_sim import OracleSimulator
@@ -94,4 +96,4 @@ def test_a_host_write_to_a_node_input_that_synapses_write_changes_no_step():
         untouched.run_steps(20)
         for p in probes.values():
             assert np.array_equal(sim.data[p], untouched.data[p])
-        assert np.array_equal(np.asarray(sim.all_data.buf), np.asarray(untouched.all_data.buf))
+        assert_same_signals(sim, untouched)

@@ -214,7 +214,7 @@ def test_nengo_family_learning_graph_runs_like_the_ir_graph(monkeypatch):
                 got, want = sim.data[built["learning"][key]], ref.data[ref_probes[key]]
                 assert got.shape == want.shape and np.any(want != 0), key
                 assert np.array_equal(got, want), (key, np.abs(got - want).max())
-            assert np.array_equal(np.asarray(sim.all_data.buf), np.asarray(ref.all_data.buf))
+            assert_same_signals(sim, ref)
             assert sim.data[built["learning"]["post_spikes"]].shape == (60, net.n_post)
 
 
@@ -284,7 +284,7 @@ def test_nengo_family_graph_runs_like_the_ir_graph(monkeypatch):
                 got, want = sim.data[built["probes"][key]], ref.data[ref_probes[key]]
                 assert got.shape == want.shape and np.any(want != 0), key
                 assert np.array_equal(got, want), (key, np.abs(got - want).max())
-            assert np.array_equal(np.asarray(sim.all_data.buf), np.asarray(ref.all_data.buf))
+            assert_same_signals(sim, ref)
             assert sim.data[built["probes"]["spikes0"]].shape == (60, net.n_neurons)
 
 

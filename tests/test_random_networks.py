@@ -8,6 +8,8 @@ and the large-item kernels, input sums formed inside both, sequences carried by 
 import numpy as np
 import pytest
 
+from helpers import assert_same_signals
+
 from oracle.numpy_interpreter import NaiveInterpreter
 from oracle.oracle_sim import OracleSimulator
 from random_networks import random_network
@@ -110,4 +112,4 @@ def test_ensemble_array_on_the_device(queue, probe_node):
         cpu.run_steps(200)
         for key, p in probes.items():
             assert np.array_equal(gpu.data[p], cpu.data[p]) and np.any(gpu.data[p] != 0), key
-        assert np.array_equal(np.asarray(gpu.all_data.buf), np.asarray(cpu.all_data.buf))
+        assert_same_signals(gpu, cpu)
