@@ -151,10 +151,11 @@ def spiking_fraction(sim):
     return nz / max(n, 1)
 
 
-def config_summary(config, steps, warmup, profile_steps, max_regions):
+def config_summary(config, steps, warmup, profile_steps, max_regions, cpu_budget=0.0,
+                   numpy_budget=0.0):
     """One of the other benchmark configurations at its full size through the same protocol:
     built, warmed up, `steps` steps timed (median region), then an eager pass with events
-    for the per-launch durations."""
+    for the per-launch durations; with budgets, the two CPU legs on a short sample."""
     from nengo_ocl_amd.simulator import Simulator
 
     t0 = time.time()
@@ -186,7 +187,12 @@ def config_summary(config, steps, warmup, profile_steps, max_regions):
         b, us = sum(r["bytes"] for r in sparse_rows), sum(r["avg_us"] for r in sparse_rows)
         out.update(sparse_bytes_per_step=b, sparse_gbs=1e-3 * b / us,
                    sparse_frac_of_peak=1e-3 * b / us / HBM_PEAK_GBS)
+    out["n_prealloc_probes"] = sim.n_prealloc_probes
     sim.close()
+    if cpu_budget > 0:
+        out["cpu_baseline"] = cpu_baseline(config, "shared", 1.0, cpu_budget, elapsed / steps)
+        if numpy_budget > 0:
+            out["cpu_baseline"]["numpy"] = numpy_baseline(config, "shared", 1.0, numpy_budget)
     return out
 
 
@@ -533,6 +539,8 @@ def main():
     ap.add_argument("--other-configs", default="c0,c1,c2,c4,c5",
                     help="configurations reported in the `configs` block of a c3 run at full "
                          "size ('' for none)")
+    ap.add_argument("--config-cpu-budget", type=float, default=2.0,
+                    help="seconds of each CPU leg for each of the other configurations")
     ap.add_argument("--numpy-budget", type=float, default=10.0,
                     help="seconds for the single-process NumPy leg of the CPU baseline; 0 skips it")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -634,6 +642,7 @@ def main():
                    "dt": 0.001, "graph": not args.no_graph,
                    "fused_copies": not args.no_fuse, "learn_in_place": not args.two_pass_learning,
                    "identical_products_merged": args.variant == "shared",
+                   "n_prealloc_probes": sim.n_prealloc_probes,
                    "products_with_spikes_visit_active_columns_only": bool(event_rows)},
         "roofline": roofline,
         "gemv_all": {"bytes_per_step": gemv_bytes, "us_per_step": gemv_us,
@@ -663,8 +672,10 @@ def main():
     if full_size_default and args.other_configs:
         out["configs"] = {}
         for name in args.other_configs.split(","):
-            out["configs"][name] = config_summary(name, args.config_steps, args.warmup,
-                                                  args.profile_steps, args.max_regions)
+            out["configs"][name] = config_summary(
+                name, args.config_steps, args.warmup, args.profile_steps, args.max_regions,
+                cpu_budget=min(args.cpu_budget, args.config_cpu_budget),
+                numpy_budget=min(args.numpy_budget, args.config_cpu_budget))
     if args.cpu_budget > 0:
         out["cpu_baseline"] = cpu_baseline(args.config, args.variant, args.scale, args.cpu_budget,
                                            elapsed / args.steps)

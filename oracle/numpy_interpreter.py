@@ -39,7 +39,10 @@ class NaiveInterpreter:
         for op in self.ops:
             for sig in op.all_signals:
                 if sig.base not in self.mem:
-                    self.mem[sig.base] = np.array(sig.base.initial_value, dtype=f32)
+                    if getattr(sig.base, "sparse", False):  # a constant scipy CSR matrix
+                        self.mem[sig.base] = sig.base.initial_value.astype(f32)
+                    else:
+                        self.mem[sig.base] = np.array(sig.base.initial_value, dtype=f32)
         self.order = self._step_order()
         self.tables = {}
         self.n_steps = 0
@@ -69,10 +72,13 @@ class NaiveInterpreter:
                     by_base.setdefault(sig.base, []).append((i, rank[kind], sig))
         after = {i: set() for i in range(len(self.ops))}
         for entries in by_base.values():
-            for i, ri, si in entries:
-                for j, rj, sj in entries:
-                    if ri < rj and i != j and si.may_share_memory(sj):
-                        after[j].add(i)
+            ranked = [[e for e in entries if e[1] == r] for r in range(4)]
+            for lo in range(4):  # only pairs of different kinds order each other
+                for hi in range(lo + 1, 4):
+                    for i, _, si in ranked[lo]:
+                        for j, _, sj in ranked[hi]:
+                            if i != j and (si is sj or si.may_share_memory(sj)):
+                                after[j].add(i)
         indegree = {i: len(after[i]) for i in after}
         users = {i: [] for i in after}
         for j, before in after.items():
@@ -114,6 +120,14 @@ class NaiveInterpreter:
             y[...] = y + (x * A.reshape(-1)[0]).reshape(y.shape)
         else:
             self._gemv_inc(A.reshape(y.size, x.size), x, y.reshape(-1))
+
+    def _SparseDotInc(self, op):
+        """clra_gemv.py:1590-1623 (`sparsedot_inc`): y += A x with A in CSR form.  Only in
+        the `blas` mode (scipy's product, its own summation order)."""
+        if not self.blas:
+            raise NotImplementedError("sparse products are not restated operation by operation")
+        y = self.view(op.Y)
+        y += (self.mem[op.A.base] @ self.view(op.X).reshape(-1)).reshape(y.shape)
 
     def _Reset(self, op):
         self.view(op.dst)[...] = f32(op.value)  # clra_nonlinearities.py:147-214
