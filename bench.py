@@ -366,7 +366,10 @@ def event_driven_report(sim, event_rows, steps_per_s, make_sim, args):
            "note": "these launches read only the columns of their matrices whose x is not zero "
                    "(results bit-identical to the dense product); their algorithmic bytes are "
                    "not traffic and are left out of gemv_all",
-           "neurons_that_spiked_in_the_last_step": spiking_fraction(sim)}
+           "neurons_that_spiked_in_the_last_step": spiking_fraction(sim),
+           # what the constructor's calibration run saw (populations that spike above the
+           # threshold per step would have been given dense products)
+           "calibration": sim.event_calibration}
     if args.no_dense_comparison:
         return out
     os.environ["NENGO_HIP_EVENT_GEMV"] = "0"
@@ -538,7 +541,7 @@ def main():
                          "block (the benchmark runs of these networks are 1000 steps)")
     ap.add_argument("--other-configs", default="c0,c1,c2,c4,c5",
                     help="configurations reported in the `configs` block of a c3 run at full "
-                         "size ('' for none)")
+                         "size ('none' for none)")
     ap.add_argument("--config-cpu-budget", type=float, default=2.0,
                     help="seconds of each CPU leg for each of the other configurations")
     ap.add_argument("--numpy-budget", type=float, default=10.0,
@@ -669,7 +672,7 @@ def main():
     del sim
     full_size_default = (args.config == "c3" and args.variant == "shared" and args.scale == 1.0
                          and not (args.no_fuse or args.no_graph or args.two_pass_learning))
-    if full_size_default and args.other_configs:
+    if full_size_default and args.other_configs not in ("", "none"):
         out["configs"] = {}
         for name in args.other_configs.split(","):
             out["configs"][name] = config_summary(

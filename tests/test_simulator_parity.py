@@ -1016,3 +1016,58 @@ def test_currents_nobody_reads_are_not_stored_and_read_back_exact(queue, monkeyp
             for Js, Jc in zip(currents(stored), currents(cpu)):
                 in_memory = np.array(stored.all_data[stored.sidx[Js]]).ravel()
                 assert np.array_equal(in_memory, np.asarray(cpu.signals[Jc]).ravel())
+
+
+@pytest.mark.gpu
+def test_populations_that_spike_densely_get_dense_products(queue):
+    """The launch that visits only the columns of the neurons that spiked loses to the dense
+    product when most neurons spike every step.  The constructor's calibration run sees a
+    population spiking above a quarter of its neurons per step and plans its products dense;
+    a population at ordinary rates keeps the launch; results equal the oracle simulator bit
+    for bit either way, and the calibration leaves no trace in the simulation (time, probes,
+    state)."""
+    from nengo_ocl_amd import minibuilder as mb
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    def make():
+        rng = np.random.RandomState(2)
+        net = mb.Network(seed=9)
+        stim = net.Node(mb.WhiteSignal(period=0.5, high=6.0, seed=3), size_out=2)
+        hot = net.Ensemble(1024, 2, label="hot", max_rates=(470, 495), intercepts=(-1.0, -0.97),
+                           neuron_type=mb.LIF(tau_rc=0.02, tau_ref=0.001))
+        cool = net.Ensemble(1024, 2, label="cool")
+        for ens in (hot, cool):
+            net.Connection(stim, ens, synapse=None)
+        targets = [net.Ensemble(128, 1, label="t%d" % k) for k in range(2)]
+        for ens, target in zip((hot, cool), targets):
+            net.Connection(ens.neurons, target.neurons, synapse=mb.Lowpass(0.01),
+                           transform=rng.normal(scale=5e-5, size=(128, 1024)))
+        return net, [net.Probe(t, synapse=0.01) for t in targets] + [net.Probe(hot.neurons)]
+
+    (net, probes), (net_o, probes_o) = make(), make()
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+        report = gpu.event_calibration
+        print("calibration:", report)
+        # (hot, cool and the two target populations, whose probe decoders join the launch)
+        assert report["populations"] == 4 and report["populations_switched_to_dense_products"] == 1
+        assert report["largest_share_spiking_per_step"] > 0.25
+        events = [p for p in gpu._plans if getattr(p, "event_driven", False)]
+        # hot's product is dense now (next to that launch the few small products left are not
+        # worth a launch of their own and may have joined it)
+        n_event_tasks = sum(p.n_tasks for p in events)
+        assert any(p.name.startswith("hipra_gemv.tile") for p in gpu._plans)
+        assert gpu.n_steps == 0 and gpu.time == 0.0 and len(gpu.data[probes[0]]) == 0
+        gpu.run_steps(200)
+        cpu.run_steps(200)
+        for p, q in zip(probes, probes_o):
+            assert np.array_equal(gpu.data[p], cpu.data[q]) and np.any(gpu.data[p] != 0)
+        share = np.count_nonzero(gpu.data[probes[2]]) / gpu.data[probes[2]].size
+        assert share > 0.25, share
+        assert_same_signals(gpu, cpu)
+    with Simulator(make()[0], seed=1, event_calibration_steps=0) as uncalibrated:
+        assert uncalibrated.event_calibration is None
+        # hot's 128 rows (two groups of 64) are in the launch that visits active columns
+        assert sum(p.n_tasks for p in uncalibrated._plans
+                   if getattr(p, "event_driven", False)) >= n_event_tasks + 2
+        assert not any(p.name.startswith("hipra_gemv.tile") for p in uncalibrated._plans)
