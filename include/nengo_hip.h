@@ -203,6 +203,47 @@ int nhip_gemv_tile_filter(void *stream, int vec, int pow2_cols, int blk_words, c
                           const float *A, const float *X, const float *Yin, float *Y,
                           const int *item_targets, const int *targets, float *F);
 
+/* A learning rule's outer-product update done by the launch that streams the learned
+ * matrices anyway (reference: `_plan_SimPES`, simulator.py:1334-1345, an outer-product
+ * `plan_elementwise_inc` of its own, clra_nonlinearities.py:414-574, and a `plan_copy` that
+ * adds the result to the weights).  nhip_gemv_tile_filter with one more table:
+ *   learn : int32[n_tasks][4] {e_start, f_start, alpha (float bits), flags}, one row per
+ *           TASK.  flags bit 0: the task's matrix (its item's only dot product, rows on
+ *           16-byte boundaries, a multiple of 4 columns, at most 64 rows in the task) is
+ *           learned: after a block of it has gone into the sums as it was read, element
+ *           (i, j) is written back as A[i][j] + (alpha * X[e_start + i]) * X[f_start + j],
+ *           every product and the sum rounded on their own -- the bits of the separate
+ *           launches.  Nothing in the launch may write X[e_start ..] or X[f_start ..];
+ *           f_start must be a multiple of 4.
+ * Only for pow2_cols = 2 (else NHIP_E_BADCLASS).  A is written: it is not const here. */
+int nhip_gemv_tile_filter_learn(void *stream, int vec, int pow2_cols, int blk_words,
+                                const int *items, const float *coefs, const int *dots,
+                                const int *tasks, int n_tasks, float *A, const float *X,
+                                const float *Yin, float *Y, const int *item_targets,
+                                const int *targets, float *F, const int *learn);
+
+/* nhip_gemv_tile_lif / nhip_gemv_tile_lif_sums (`parts` may be NULL: no input sums) that
+ * also steps first-order filters of the populations' spikes -- the pre-synaptic activities
+ * a learning rule reads (reference: the `plan_linearfilter` of the rule's pre-synaptic
+ * synapse, clra_nonlinearities.py:577-803, a launch at the end of the step).  The step is
+ * DEFERRED: the task that is about to replace the spikes of neurons [row0, row0 + n) with
+ * this step's first computes, from the spikes of the previous step,
+ *     Fdef[f_start + i] = b0 * S_old[i] - a0 * Fdef[f_start + i]     (or b0 * S_old[i])
+ * so that between two steps Fdef holds the filter output as it was BEFORE the previous
+ * step's update; whoever reads it from the host applies the pending step (the same two
+ * rounded operations).  With zero initial spikes and outputs the first such step changes
+ * nothing, as it must.
+ *   deferred : int32[n_items][4] {f_start, a0 (float bits), b0 (float bits), flags}; flags
+ *              bit 0: the item's population has such a filter, bit 1: it has a0.
+ * Only for pow2_cols = 3 (else NHIP_E_BADCLASS). */
+int nhip_gemv_tile_lif_deferred(void *stream, int vec, int pow2_cols, int blk_words,
+                                const int *items, const float *coefs, const int *dots,
+                                const int *tasks, int n_tasks, const float *A, const float *X,
+                                const float *Yin, float *Y, const int *pops, double dt,
+                                int upsample, float *V, float *W, float *S, const float *TAU,
+                                const float *REF, const float *AMP, const int *parts,
+                                const int *deferred, float *Fdef);
+
 /* The same two epilogues for launches of small items (nhip_gemv with flavor 2, whose
  * `items`, `coefs`, `dots` and `tasks` tables these take; `lpr` 4, 1 or 64): the
  * neuron update / filter step of a row runs in the lane that holds the row's sum.

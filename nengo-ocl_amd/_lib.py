@@ -34,6 +34,9 @@ SIGNATURES = {
     "nhip_gemv_tile_lif_sums": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
                                 P, ctypes.c_double, c_int, P, P, P, P, P, P, P],
     "nhip_gemv_tile_filter": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P, P, P, P],
+    "nhip_gemv_tile_filter_learn": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P, P, P, P, P],
+    "nhip_gemv_tile_lif_deferred": [P, c_int, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
+                                    P, ctypes.c_double, c_int, P, P, P, P, P, P, P, P, P],
     "nhip_gemv_tile_rows": [c_int, c_int],
     "nhip_gemv_rows_lif": [P, c_int, c_int, P, P, P, P, c_int, P, P, P, P,
                            P, ctypes.c_double, c_int, P, P, P, P, P, P],

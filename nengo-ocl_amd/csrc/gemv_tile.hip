@@ -890,14 +890,32 @@ struct SeqSide {
     int n_gemv_groups;  // groups of the GEMV itself (the grid has n_chains more)
 };
 
-template <int EPI, int SET>
-__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 14) ? 3 : 4, 4))) void gemv_stream_kernel(
+// VAR: what else the launch does while it has the data in hand (instances of their own, so
+// that the ordinary ones keep their registers) --
+// VAR_LEARN (with the filter epilogue): the matrices of some tasks are being learned by an
+//   outer-product rule, W += (alpha e) (x) f.  The task that streams a block of such a matrix
+//   forms its sums from the block as it was read and writes the block back with the change
+//   added, element by element the rounded operations of the outer-product kernel
+//   (elementwise_inc_block with `outer`): the matrix is read once per step instead of twice,
+//   and the update is no launch.  e and f are not written by the launch.
+// VAR_DEFER (with the LIF epilogue): first-order filters of the populations' spikes (the
+//   activities such a rule reads) are stepped HERE, on the spikes of the previous step, by the
+//   task that is about to replace them -- the filter step that closes the previous step,
+//   deferred to the one moment at which nobody else reads its output.
+constexpr int VAR_LEARN = 1, VAR_DEFER = 2;
+
+template <int EPI, int SET, int VAR = 0>
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((VAR & VAR_LEARN) ? 2 : (SET & 14) ? 3 : 4, 4))) void gemv_stream_kernel(
     const GemvDot* __restrict__ dots, const GemvFatTask* __restrict__ tasks, int n_tasks,
-    int xb_words, const float* __restrict__ A, const float* __restrict__ X, const float* Yin,
+    int xb_words, std::conditional_t<(VAR & VAR_LEARN) != 0, const float*, const float* __restrict__> A,
+    const float* __restrict__ X, const float* Yin,
     float* Y, EpilogueArgs epi, SeqSide side)
 {
     constexpr bool WIDE = (SET & (SET_MID | SET_WIDE)) != 0;  // the large LDS layout
     constexpr bool FLAT = (SET & SET_FLAT) != 0;
+    constexpr bool LEARN = EPI == EPI_FILTER && (VAR & VAR_LEARN) != 0;
+    constexpr bool DEFER = EPI == EPI_LIF && (VAR & VAR_DEFER) != 0;
+    static_assert(!(LEARN && FLAT), "learned matrices: rows on 16-byte boundaries");
     static_assert(!(FLAT && WIDE), "back-to-back rows: single-stage widths only");
     extern __shared__ __attribute__((aligned(16))) float lds[];
     if (EPI != EPI_NONE && side.n_chains > 0 && (int)blockIdx.x >= side.n_gemv_groups) {
@@ -945,6 +963,15 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
             fp.target[k] = epi.filter.targets[fp.range.x + q];
         }
     }
+    // a learned matrix: the task's record of the rule, and alpha * e of row `lane` of the
+    // task (learned tasks have at most 64 rows: the host's word), requested now
+    int4 lrn = make_int4(0, 0, 0, 0);
+    float ae_lane = 0.0f;
+    if (LEARN) {
+        lrn = epi.filter.learn[t];
+        ae_lane = __fmul_rn(nhip_bits(lrn.z),
+                            X[(lrn.w & 1) ? (size_t)lrn.x + task.row0 + min(lane, n_rows - 1) : 0]);
+    }
     LifPop pop = {};
     float v_in[SLOTS], w_in[SLOTS];
     // runs once, behind the first matrix loads of the task
@@ -963,6 +990,33 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                 const int i = task.row0 + min(lane + k * NHIP_WAVE, n_rows - 1);
                 v_in[k] = epi.lif.V[enabled ? (size_t)pop.v_start + i : 0];
                 w_in[k] = epi.lif.W[enabled ? (size_t)pop.w_start + i : 0];
+            }
+            if (DEFER) {
+                // The filter step that closes the previous step, on the spikes this task is
+                // about to replace: y = b0 x - a0 y, or y = b0 x -- the arithmetic of the
+                // filter kernel's simple case (clra_nonlinearities.py:630-650).  Done here, at
+                // the start of the task, while the first matrix blocks are on their way: its
+                // operands then occupy no registers during the streaming.  Nothing else in
+                // the launch reads the filter output.
+                const int4 dfr = epi.lif.deferred[task.item];
+                if (enabled && (dfr.w & 1)) {  // uniform
+                    float s_in[SLOTS], f_in[SLOTS];
+#pragma unroll
+                    for (int k = 0; k < SLOTS; ++k) {
+                        const int i = task.row0 + min(lane + k * NHIP_WAVE, n_rows - 1);
+                        s_in[k] = epi.lif.S[(size_t)pop.s_start + i];
+                        f_in[k] = epi.lif.Fdef[(size_t)dfr.x + i];
+                    }
+#pragma unroll
+                    for (int k = 0; k < SLOTS; ++k) {
+                        const int r = lane + k * NHIP_WAVE;
+                        if (r < n_rows) {
+                            const float bx = __fmul_rn(nhip_bits(dfr.z), s_in[k]);
+                            epi.lif.Fdef[(size_t)dfr.x + task.row0 + r] =
+                                (dfr.w & 2) ? __fsub_rn(bx, __fmul_rn(nhip_bits(dfr.y), f_in[k])) : bx;
+                        }
+                    }
+                }
             }
         }
         if (EPI == EPI_FILTER) {
@@ -1015,8 +1069,21 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
         int l_b = 0;                 // row block of the next stage to load
         int l_c0 = 0;                // its first column
         const char* l_ptr = a0;      // its first byte
-        auto load_block = [&](tile_f4 (&pf)[G::NL], float (&xq)[G::XL]) {
+        constexpr int NFQ = LEARN ? 1 << G::LG_LPR : 1;  // column quads of a lane per row
+        auto load_block = [&](tile_f4 (&pf)[G::NL], float (&xq)[G::XL], tile_f4 (&fq)[NFQ], int2& at) {
             const int cols = RAGGED ? min(G::NCS, dot.N - l_c0) : G::NCS;
+            if (LEARN) {
+                // where the block lies (row block, first column), for writing it back; and the
+                // column operand of the rule for this lane's quads (lanes past the end of a
+                // narrower last stage read the stage's first quad; their result is not stored)
+                at = make_int2(l_b, l_c0);
+#pragma unroll
+                for (int q = 0; q < NFQ; ++q) {
+                    const int c = q * 256 + 4 * lane_q;
+                    fq[q] = *reinterpret_cast<const tile_f4*>(
+                        X + (size_t)lrn.y + l_c0 + ((lrn.w & 1) && c < cols ? c : 0));
+                }
+            }
             if (G::MULTI) {
                 const float* xg = x0 + (size_t)l_c0 * dot.x_stride0;
                 if (cols == G::NCS) {
@@ -1064,7 +1131,8 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                 l_ptr += (size_t)G::RB * stride4;
             }
         };
-        auto store_block = [&](const tile_f4 (&pf)[G::NL], const float (&xq)[G::XL], bool with_x) {
+        auto store_block = [&](const tile_f4 (&pf)[G::NL], const float (&xq)[G::XL], bool with_x,
+                               const tile_f4 (&fq)[NFQ], int2 at) {
             wave_sync();  // every lane is done reading the previous block
 #pragma unroll
             for (int i = 0; i < G::NL; ++i) {  // rows and columns that do not exist get whatever was read
@@ -1073,6 +1141,30 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
                 else
                     *reinterpret_cast<tile_f4*>(wp + (i >> G::LG_LPR) * G::RPL * G::ROWW +
                                                 (i & ((1 << G::LG_LPR) - 1)) * (2 * TILE_LDS)) = pf[i];
+            }
+            if (LEARN && (lrn.w & 1)) {  // uniform
+                // the block goes back with (alpha e_i) f_j added, each product and each sum
+                // rounded on its own as in the outer-product kernel; the sums above use the
+                // block as it was read
+                const int rows = min(G::RB, n_rows - at.x * G::RB);
+                const int cols = RAGGED ? min(G::NCS, dot.N - at.y) : G::NCS;
+                float* const w0 = const_cast<float*>(A) + dot.a_start +
+                                  (size_t)(task.row0 + at.x * G::RB) * dot.a_stride0 + at.y;
+#pragma unroll
+                for (int i = 0; i < G::NL; ++i) {
+                    const int r = lane_r + (i >> G::LG_LPR) * G::RPL;
+                    const int q = i & ((1 << G::LG_LPR) - 1);
+                    const int c = q * 256 + 4 * lane_q;
+                    const float s = __shfl(ae_lane, at.x * G::RB + r, NHIP_WAVE);
+                    if (r < rows && c < cols) {
+                        tile_f4 v;
+                        v.x = __fadd_rn(pf[i].x, __fmul_rn(s, fq[q].x));
+                        v.y = __fadd_rn(pf[i].y, __fmul_rn(s, fq[q].y));
+                        v.z = __fadd_rn(pf[i].z, __fmul_rn(s, fq[q].z));
+                        v.w = __fadd_rn(pf[i].w, __fmul_rn(s, fq[q].w));
+                        *reinterpret_cast<tile_f4*>(w0 + (size_t)r * dot.a_stride0 + c) = v;
+                    }
+                }
             }
             if (with_x) {
 #pragma unroll
@@ -1140,13 +1232,15 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
 
         tile_f4 pf0[G::NL], pf1[G::NL];
         float xq0[G::XL], xq1[G::XL];
-        load_block(pf0, xq0);
+        tile_f4 fq0[NFQ], fq1[NFQ];  // (LEARN: the rule's column operand for the set's block)
+        int2 at0 = make_int2(0, 0), at1 = make_int2(0, 0);
+        load_block(pf0, xq0, fq0, at0);
         if (n_stages == 1) {  // the second set's first loads are never under a branch
             l_b = 0;
             l_c0 = 0;
             l_ptr = a0;
         }
-        load_block(pf1, xq1);
+        load_block(pf1, xq1, fq1, at1);
         if (!G::MULTI) {  // one column stage: its X is fetched once
 #pragma unroll
             for (int i = 0; i < G::XL; ++i)
@@ -1196,11 +1290,11 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
         // stages k + 2 and k + 3 exist: both register sets are refilled without a branch
         while (k + 3 < n_stages) {
             const int b1 = next_b(b);
-            store_block(pf0, xq0, G::MULTI ? b == 0 : k == 0);
-            load_block(pf0, xq0);
+            store_block(pf0, xq0, G::MULTI ? b == 0 : k == 0, fq0, at0);
+            load_block(pf0, xq0, fq0, at0);
             sum_block(b, cols_of(k));
-            store_block(pf1, xq1, G::MULTI && b1 == 0);
-            load_block(pf1, xq1);
+            store_block(pf1, xq1, G::MULTI && b1 == 0, fq1, at1);
+            load_block(pf1, xq1, fq1, at1);
             sum_block(b1, cols_of(k + 1));
             b = next_b(b1);
             k += 2;
@@ -1209,15 +1303,15 @@ __global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((SET & 
         {
             const int b1 = next_b(b);
             const int b2 = next_b(b1);
-            store_block(pf0, xq0, G::MULTI ? b == 0 : k == 0);
-            if (k + 2 < n_stages) load_block(pf0, xq0);
+            store_block(pf0, xq0, G::MULTI ? b == 0 : k == 0, fq0, at0);
+            if (k + 2 < n_stages) load_block(pf0, xq0, fq0, at0);
             sum_block(b, cols_of(k));
             if (k + 1 < n_stages) {
-                store_block(pf1, xq1, G::MULTI && b1 == 0);
+                store_block(pf1, xq1, G::MULTI && b1 == 0, fq1, at1);
                 sum_block(b1, cols_of(k + 1));
             }
             if (k + 2 < n_stages) {
-                store_block(pf0, xq0, G::MULTI && b2 == 0);
+                store_block(pf0, xq0, G::MULTI && b2 == 0, fq0, at0);
                 sum_block(b2, cols_of(k + 2));
             }
         }
@@ -1275,7 +1369,13 @@ namespace {
 
 int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* items,
                 const float* coefs, const int* dots, const int* tasks, int n_tasks, const float* A,
-                const float* X, const float* Yin, float* Y, int epilogue, const EpilogueArgs& args) {
+                const float* X, const float* Yin, float* Y, int epilogue, const EpilogueArgs& args,
+                int variant = 0) {
+    // the variants exist for the shapes they were built for: learned matrices in launches of
+    // the wide instance, deferred activity filters in launches of the narrow one
+    if (variant == VAR_LEARN && !(epilogue == EPI_FILTER && pow2_cols == 2)) return NHIP_E_BADCLASS;
+    if (variant == VAR_DEFER && !(epilogue == EPI_LIF && pow2_cols == 3)) return NHIP_E_BADCLASS;
+    if (variant != 0 && variant != VAR_LEARN && variant != VAR_DEFER) return NHIP_E_BADARG;
     // a sequence armed by nhip_gemv_tile_carry is this launch's, whatever becomes of it
     const NhipCarried armed = nhip_carried;
     nhip_carried = NhipCarried{};
@@ -1328,7 +1428,11 @@ int launch_tile(void* stream, int vec, int pow2_cols, int blk_words, const int* 
                         reinterpret_cast<const GemvFatTask*>(tasks), n_tasks, stream_xb, A, X, Yin,
                         Y, args, side);
         };
-        if (pow2_cols == 2) launch_stream(gemv_stream_kernel<E, SET_WIDE>);
+        if (variant == VAR_LEARN) {
+            if constexpr (E == EPI_FILTER) launch_stream(gemv_stream_kernel<E, SET_WIDE, VAR_LEARN>);
+        } else if (variant == VAR_DEFER) {
+            if constexpr (E == EPI_LIF) launch_stream(gemv_stream_kernel<E, 0, VAR_DEFER>);
+        } else if (pow2_cols == 2) launch_stream(gemv_stream_kernel<E, SET_WIDE>);
         else if (pow2_cols == 3) launch_stream(gemv_stream_kernel<E, 0>);
         else if (pow2_cols == 4) launch_stream(gemv_stream_kernel<E, SET_WIDE | SET_MID>);
         else if (pow2_cols == 5) launch_stream(gemv_stream_kernel<E, SET_TINY>);
@@ -1418,6 +1522,51 @@ extern "C" int nhip_gemv_tile_filter(void* stream, int vec, int pow2_cols, int b
     args.filter.F = F;
     return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
                        Yin, Y, EPI_FILTER, args);
+}
+
+extern "C" int nhip_gemv_tile_filter_learn(void* stream, int vec, int pow2_cols, int blk_words,
+                                           const int* items, const float* coefs, const int* dots,
+                                           const int* tasks, int n_tasks, float* A, const float* X,
+                                           const float* Yin, float* Y, const int* item_targets,
+                                           const int* targets, float* F, const int* learn) {
+    if (!item_targets || !targets || !F || !learn) return NHIP_E_BADARG;
+    EpilogueArgs args{};
+    args.filter.item_targets = reinterpret_cast<const int2*>(item_targets);
+    args.filter.targets = reinterpret_cast<const FilterTarget*>(targets);
+    args.filter.F = F;
+    args.filter.learn = reinterpret_cast<const int4*>(learn);
+    return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
+                       Yin, Y, EPI_FILTER, args, VAR_LEARN);
+}
+
+extern "C" int nhip_gemv_tile_lif_deferred(void* stream, int vec, int pow2_cols, int blk_words,
+                                           const int* items, const float* coefs, const int* dots,
+                                           const int* tasks, int n_tasks, const float* A,
+                                           const float* X, const float* Yin, float* Y,
+                                           const int* pops, double dt, int upsample, float* V,
+                                           float* W, float* S, const float* TAU, const float* REF,
+                                           const float* AMP, const int* parts, const int* deferred,
+                                           float* Fdef) {
+    if (!pops || !V || !W || !S || upsample < 1 || !(dt > 0.0) || !deferred || !Fdef)
+        return NHIP_E_BADARG;
+    if (parts && static_cast<const float*>(Y) != X) return NHIP_E_BADARG;  // (as nhip_gemv_tile_lif_sums)
+    EpilogueArgs args{};
+    LifArgs& lif = args.lif;
+    lif.pops = reinterpret_cast<const LifPop*>(pops);
+    lif.dtu = (float)(dt / (double)upsample);
+    lif.dt_inv = (float)(1.0 / dt);
+    lif.upsample = upsample;
+    lif.V = V;
+    lif.W = W;
+    lif.S = S;
+    lif.TAU = TAU;
+    lif.REF = REF;
+    lif.AMP = AMP;
+    lif.parts = reinterpret_cast<const int2*>(parts);
+    lif.deferred = reinterpret_cast<const int4*>(deferred);
+    lif.Fdef = Fdef;
+    return launch_tile(stream, vec, pow2_cols, blk_words, items, coefs, dots, tasks, n_tasks, A, X,
+                       Yin, Y, EPI_LIF, args, VAR_DEFER);
 }
 
 thread_local NhipCarried nhip_carried;

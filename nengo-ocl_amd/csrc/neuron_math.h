@@ -37,6 +37,15 @@ struct LifArgs {
     // the same for the small-item kernel, whose task records have no spare words: per GEMV
     // item {first part, number of parts} (0 parts: the operand is read as usual).  Null: none.
     const int2* sum_ranges;
+    // first-order filters of the populations' OLD spikes, stepped by the task that is about
+    // to overwrite those spikes (large-item kernel with compile-time shapes, the instance for
+    // it): per GEMV item {f_start, a0 bits, b0 bits, flags} -- flags bit 0: the item's
+    // population has such a filter, bit 1: it has a denominator coefficient; element i of the
+    // filter output is Fdef[f_start + i] = b0 * S_old[i] - a0 * Fdef[f_start + i].  This is the
+    // filter step that follows the neuron update of the PREVIOUS step, moved to where its
+    // input is about to be replaced (see nhip_gemv_tile_lif_deferred).  Null: none.
+    const int4* deferred;
+    float* Fdef;
 };
 
 __device__ __forceinline__ float lif_param(int word, bool is_vector, const float* data, int i) {
@@ -139,6 +148,12 @@ struct FilterArgs {
     const int2* item_targets;     // per GEMV item: {first target, number of targets}
     const FilterTarget* targets;
     float* F;                     // buffer that holds the filter outputs
+    // matrices a learning rule updates in place while the launch streams them (large-item
+    // kernel with compile-time shapes, the instance for it): per TASK {e_start, f_start,
+    // alpha bits, flags}; with flags bit 0 set, element (i, j) of the task's matrix becomes
+    // A + (alpha * X[e_start + i]) * X[f_start + j] after its old value has gone into the
+    // sums (see nhip_gemv_tile_filter_learn).  Null: none.
+    const int4* learn;
 };
 
 // Filter step of element i of every target of a GEMV item whose fresh output is x

@@ -16,6 +16,7 @@ signature, same ``.plans`` attribute; what differs is the work decomposition:
 For each item b:  ``Y[b] = beta[b]*Y_in[b] + gamma[b] + alpha[b] * sum_j A[A_js[b][j]] @ X[X_js[b][j]]``.
 """
 
+import logging
 import os
 from collections import defaultdict
 
@@ -25,6 +26,8 @@ from . import _lib
 from .hipraggedarray import HIPRaggedArray, to_device
 from .plan import Plan
 from .utils import next_pow2
+
+logger = logging.getLogger(__name__)
 
 # items with at most this many matrix elements go to the wave-per-task kernel
 SMALL_ITEM_ELEMS = 8192
@@ -1034,6 +1037,7 @@ def fuse_input_sums(sum_plan, lif_plan):
     args = tuple(lif_plan.args)
     sum_bytes = sum_plan.bw_per_call or 0
     one = np.array([1.0, 0.0, 0.0, 0.0], dtype=np.float32).view(np.int32)
+    new_pops = lif_plan.host_pops
     if large:
         tasks = lif_plan.host_tasks.copy()  # 24-word records: task, item, coefficients, first dot
         for row in tasks:
@@ -1051,6 +1055,7 @@ def fuse_input_sums(sum_plan, lif_plan):
                 row[12:16] = one
             tasks = np.concatenate([tasks, extra])
             dev_pops = to_device(queue, pops)
+            new_pops = pops
             args = args[:12] + (dev_pops.ptr,) + args[13:]
             keep = (dev_pops,)
         dev_tasks = to_device(queue, tasks)
@@ -1111,7 +1116,150 @@ def fuse_input_sums(sum_plan, lif_plan):
     fused.host_tasks = tasks
     fused.input_sums = len(sums)
     fused.lazy_currents = getattr(lif_plan, "lazy_currents", None)
+    fused.host_pops = new_pops if large else pops
     return fused
+
+
+def _learning_apart(which):
+    logger.debug("fuse_learning: check %d did not hold", which)
+    return None
+
+
+def fuse_learning(enc_plan, dec_plan, ew_plan, lf_plan):
+    """A step that ends with an outer-product learning rule -- ``W += (alpha e) (x) f`` and
+    then ``f <- filter(spikes)`` (the reference: `_plan_SimPES`, simulator.py:1334-1345, with
+    the copy that adds the result, and the `plan_linearfilter` of the rule's pre-synaptic
+    synapse) -- without a launch for either:
+
+    * the launch that decodes with the learned matrices (`dec_plan`, large items with the
+      filter epilogue) writes every block of such a matrix back with the change added once
+      the block has gone into its sums (``nhip_gemv_tile_filter_learn``): the matrix is read
+      once per step;
+    * the filters of the activities ``f`` are stepped by the NEXT step's launch that updates
+      the neurons (`enc_plan`, large items with the LIF epilogue,
+      ``nhip_gemv_tile_lif_deferred``), by the task that is about to replace the spikes they
+      read.  Between steps ``f`` then holds the value from before the pending filter step.
+
+    Fused when every outer product's matrix is the only matrix of an item of `dec_plan`
+    (same start, shape and row stride; tasks of at most 64 rows; whole aligned quads), its
+    row and column operands are contiguous vectors, every filter of `lf_plan` whose output is
+    such a column operand reads exactly the spikes of a population of `enc_plan` and has one
+    numerator and at most one denominator coefficient.  The caller checks what only it knows:
+    that nothing else reads ``f``, that ``f`` and the spikes start at zero, and that no plan in
+    between touches what moves.  Returns ``(new enc_plan, new dec_plan, plans for the filters
+    that stay, {f start: (spike start, a0 bits or None, b0 bits, length)})`` or None.
+    """
+    from .hipra_nonlinearities import plan_linearfilter
+
+    ew, lf = getattr(ew_plan, "ew_spec", None), getattr(lf_plan, "lf_spec", None)
+    if ew is None or lf is None or not ew.get("outer") or not ew.get("inc"):
+        return _learning_apart(1)
+    if (enc_plan.name != "hipra_gemv.tile_lif" or tuple(enc_plan.kernel_class) != (3, 3, 4)
+            or dec_plan.name != "hipra_gemv.tile_filter" or tuple(dec_plan.kernel_class) != (3, 2, 4)
+            or getattr(dec_plan, "host_tasks", None) is None
+            or getattr(enc_plan, "host_pops", None) is None):
+        return _learning_apart(2)
+    E, Fv, Wm, alphas = ew["A"], ew["X"], ew["Y"], ew["alphas"]
+    S, F, FA, FB = lf["X"], lf["Y"], lf["A"], lf["B"]
+    D = dec_plan.prog
+    queue, lib = D.queue, D.queue.lib
+    buf = D.A.ptr.value
+    if any(ra.ptr.value != buf for ra in (E, Fv, Wm, S, F, D.X, D.Y, enc_plan.prog.Y)):
+        return _learning_apart(3)
+    # the matrices: each the only dot product of one item of the decoding launch
+    by_matrix = {}
+    for b in dec_plan.members:
+        g = D.geometry[b]
+        if len(g["dots"]) == 1:
+            d = g["dots"][0]
+            by_matrix[(d["a_start"], g["y_len"], d["a_shape1"], d["a_stride0"])] = b
+    tasks = dec_plan.host_tasks
+    learn_of_item = {}
+    for i in range(len(Wm)):
+        rows, cols = int(Wm.shape0s[i]), int(Wm.shape1s[i])
+        key = (int(Wm.starts[i]), rows, cols, int(Wm.stride0s[i]) if rows > 1 else cols)
+        b = by_matrix.get(key)
+        if b is None or b in learn_of_item or int(Wm.stride1s[i]) != 1:
+            return _learning_apart(4)
+        if (key[0] | key[3] | cols) & 3 or cols < 512:  # aligned quads; the 512-column stages
+            return _learning_apart(5)
+        if not (int(E.shape0s[i]) == rows and (rows == 1 or int(E.stride0s[i]) == 1)
+                and int(E.shape1s[i]) == 1 and int(Fv.shape0s[i]) == cols
+                and int(Fv.stride0s[i]) == 1 and int(Fv.shape1s[i]) == 1
+                and int(Fv.starts[i]) % 4 == 0):
+            return _learning_apart(6)
+        alpha = np.float32(alphas[i])
+        learn_of_item[b] = (int(E.starts[i]), int(Fv.starts[i]), int(alpha.view(np.int32)), 1)
+    if not learn_of_item or int(tasks[np.isin(tasks[:, 0], list(learn_of_item)), 2].max()) > WAVE:
+        return _learning_apart(7)
+    learn = np.zeros((len(tasks), 4), dtype=np.int32)
+    for t, item in enumerate(tasks[:, 0]):
+        if int(item) in learn_of_item:
+            learn[t] = learn_of_item[int(item)]
+    # the filters: those whose output is a column operand move to the neuron launch
+    f_operands = {(int(Fv.starts[i]), int(Fv.shape0s[i])) for i in range(len(Wm))}
+    pops = enc_plan.host_pops
+    enc_geo = enc_plan.prog.geometry
+    by_spikes = {(int(pops[b][2]), enc_geo[b]["y_len"]): b for b in enc_plan.members
+                 if b < len(pops) and pops[b][7] & LIF_POP_ENABLED}
+    a_host, b_host = FA.to_host(), FB.to_host()
+    deferred = np.zeros((len(pops), 4), dtype=np.int32)
+    moved, rest, pending = [], [], {}
+    for k in range(len(F)):
+        out = (int(F.starts[k]), int(F.shape0s[k]))
+        if out not in f_operands:
+            rest.append(k)
+            continue
+        simple = int(FB.shape0s[k]) == 1 and int(FA.shape0s[k]) <= 1
+        vector = all(int(r.shape1s[k]) == 1 and int(r.stride0s[k]) == 1 for r in (S, F))
+        b = by_spikes.get((int(S.starts[k]), int(S.shape0s[k]))) if simple and vector else None
+        if b is None or deferred[b][3] or int(S.shape0s[k]) != out[1]:
+            return _learning_apart(8)
+        na = int(FA.shape0s[k])
+        a0 = np.float32(a_host[k][0, 0]) if na else np.float32(0)
+        b0 = np.float32(b_host[k][0, 0])
+        deferred[b] = (out[0], int(a0.view(np.int32)), int(b0.view(np.int32)), 1 | (2 if na else 0))
+        pending[out[0]] = (int(S.starts[k]), int(a0.view(np.int32)) if na else None,
+                           int(b0.view(np.int32)), out[1])
+        moved.append(k)
+    if len(moved) != len(f_operands):
+        return _learning_apart(9)  # a column operand that no filter of this plan produces: leave it all alone
+
+    dev_learn, dev_deferred = to_device(queue, learn), to_device(queue, deferred)
+    new_dec = Plan(queue, lib.nhip_gemv_tile_filter_learn, tuple(dec_plan.args) + (dev_learn.ptr,),
+                   gsize=dec_plan.gsize, lsize=dec_plan.lsize,
+                   full_args=tuple(dec_plan.full_args) + (dev_learn,) + tuple(ew_plan.full_args),
+                   name=dec_plan.name, tag="%s + learning" % dec_plan.tag,
+                   # the matrices are read by the decoding anyway: the update adds their write
+                   # and its two vectors
+                   bw_per_call=(dec_plan.bw_per_call or 0) + sum(
+                       4 * int(Wm.shape0s[i]) * int(Wm.shape1s[i]) + 4 * int(Wm.shape0s[i])
+                       + 4 * int(Wm.shape1s[i]) for i in range(len(Wm))),
+                   flops_per_call=(dec_plan.flops_per_call or 0) + (ew_plan.flops_per_call or 0))
+    enc_args = tuple(enc_plan.args)
+    if getattr(enc_plan.kern, "__name__", "") == "nhip_gemv_tile_lif":
+        enc_args += (None,)  # no input sums: no parts table
+    elif getattr(enc_plan.kern, "__name__", "") != "nhip_gemv_tile_lif_sums":
+        return _learning_apart(10)
+    new_enc = Plan(queue, lib.nhip_gemv_tile_lif_deferred, enc_args + (dev_deferred.ptr, F.ptr),
+                   gsize=enc_plan.gsize, lsize=enc_plan.lsize,
+                   full_args=tuple(enc_plan.full_args) + (dev_deferred, F.dev_buf),
+                   name=enc_plan.name, tag="%s + activity filters" % enc_plan.tag,
+                   bw_per_call=(enc_plan.bw_per_call or 0) + sum(12 * int(F.shape0s[k]) for k in moved),
+                   flops_per_call=enc_plan.flops_per_call)
+    for new, old in ((new_dec, dec_plan), (new_enc, enc_plan)):
+        for attr in ("description", "kernel_class", "n_tasks", "members", "prog", "gemv_bytes",
+                     "host_tasks", "host_pops", "lif_written", "lazy_currents", "input_sums"):
+            if hasattr(old, attr):
+                setattr(new, attr, getattr(old, attr))
+    new_dec.learned_matrices = len(learn_of_item)
+    new_enc.deferred_filters = len(moved)
+    residual = []
+    if rest:
+        residual = plan_linearfilter(queue, S[rest], F[rest], FA[rest], FB[rest],
+                                     lf["Xbuf"][rest], lf["Ybuf"][rest], tag=lf_plan.tag)
+        residual[0].unfused_items = list(rest)
+    return new_enc, new_dec, residual, pending
 
 
 def _read_spans(prog, ptr_value):
@@ -1250,6 +1398,8 @@ def fuse_linearfilter(gemv_plans, lf_plan):
         fused.kernel_class, fused.n_tasks = plan.kernel_class, plan.n_tasks
         fused.members, fused.prog = plan.members, prog
         fused.gemv_bytes = plan.bw_per_call
+        if plan.kernel_class[0] == 3:
+            fused.host_tasks = tasks
         out.append(fused)
     residual = []
     if rest:

@@ -93,6 +93,8 @@ class HipBackend:
         self.fuse_spmv_filter = hipra_spmv.fuse_linearfilter
         if os.environ.get("NENGO_HIP_OUTER_FILTER", "1") != "0":  # switch for measurements
             self.fuse_outer_filter = hipra_nonlinearities.fuse_outer_filter
+        if os.environ.get("NENGO_HIP_FOLD_LEARNING", "1") != "0":  # switch for measurements
+            self.fuse_learning = hipra_gemv.fuse_learning
 
     def fuse_input_sums(self, sum_plan, lif_plan):
         """The plan replacing ``[sum_plan, lif_plan]`` when the first only forms vector
@@ -448,6 +450,9 @@ class Simulator:
         self._raggedarrays_to_reset = []  # (device ragged, host initial)
         self._lazy_currents = {}  # signal base -> {"prog": GEMV that recomputes it, "at_step"}
         self._event_spike_sources = set()  # spike signals whose products may visit active columns
+        # filter outputs whose last step is pending in device memory (`_fuse_learning`):
+        # signal base -> (spike signal base, a0 or None, b0)
+        self._pending_filters = {}
         self._n_steps = 0
         self._filter_positions = []
         self._noise_plans = []
@@ -491,10 +496,12 @@ class Simulator:
         plans.extend(probe_plans)
         if fuse and hasattr(self.backend, "fuse_gemv_filter"):
             plans = self._fuse_filter_epilogues(plans)
-        if fuse and hasattr(self.backend, "fuse_outer_filter"):
-            plans = self._fuse_outer_filters(plans)
         if fuse and hasattr(self.backend, "fuse_input_sums"):
             plans = self._fuse_input_sums(plans)
+        if fuse and hasattr(self.backend, "fuse_learning"):
+            plans = self._fuse_learning(plans)
+        if fuse and hasattr(self.backend, "fuse_outer_filter"):
+            plans = self._fuse_outer_filters(plans)
         if merge_small and hasattr(self.backend, "merge_small_plans"):
             plans = self.backend.merge_small_plans(plans)
             if fuse and hasattr(self.backend, "carry_sequences"):
@@ -675,6 +682,97 @@ class Simulator:
             out[-1] = fused
         return out
 
+    def _fuse_learning(self, plans):
+        """An outer-product learning rule that updates its matrix in place, and the filter of
+        the activities it reads, without launches of their own (`hipra_gemv.fuse_learning`):
+        the update rides in the launch that decodes with the learned matrices, the filter step
+        in the next step's launch that updates the neurons.  Only where nothing else looks at
+        what moves: no plan between the decoding launch and the rule touches the rule's
+        operands or matrices, nothing but the rule reads the filtered activities (no probe, no
+        other operator), no plan from the filter to the end of the step or from its start to
+        the neuron launch touches them, and they and the spikes start at zero (the first
+        deferred filter step then changes nothing, as the step it stands for never ran)."""
+        plans = list(plans)
+        conflict = self.backend.plans_conflict
+        is_dec = lambda p: (getattr(p, "name", "") == "hipra_gemv.tile_filter"
+                            and tuple(getattr(p, "kernel_class", ())) == (3, 2, 4))
+        is_enc = lambda p: (getattr(p, "name", "") == "hipra_gemv.tile_lif"
+                            and tuple(getattr(p, "kernel_class", ())) == (3, 3, 4))
+        is_rule = lambda p: bool((getattr(p, "ew_spec", None) or {}).get("outer")
+                                 and (getattr(p, "ew_spec", None) or {}).get("inc"))
+        try:
+            j = next(k for k, p in enumerate(plans) if is_dec(p))
+            i = next(k for k in range(j - 1, -1, -1) if is_enc(plans[k]))
+            r = next(k for k in range(j + 1, len(plans)) if is_rule(plans[k]))
+            f = next(k for k in range(r + 1, len(plans)) if getattr(plans[k], "lf_spec", None))
+        except StopIteration:
+            return self._learning_apart(plans, 1)
+        enc, dec, rule, lf = plans[i], plans[j], plans[r], plans[f]
+        rule_ops = getattr(rule, "planned_ops", None)
+        lf_ops = getattr(lf, "planned_ops", None)
+        if not rule_ops or not lf_ops or len(lf_ops) != len(lf.lf_spec["X"]):
+            return self._learning_apart(plans, 2)
+        if any(conflict(rule, q) for q in plans[j + 1:r]):
+            return self._learning_apart(plans, 3)
+        activities = {op.pre_filtered.base for op in rule_ops if hasattr(op, "pre_filtered")}
+        if len(activities) != len(rule_ops):
+            return self._learning_apart(plans, 4)
+        moving = [op for op in lf_ops if op.output.base in activities]
+        probed = {self.model.sig[p]["in"].base for p in self.model.probes}
+        for op in moving:
+            out, spikes = op.output, op.input
+            readers = [q for q in self.operators if q is not op and any(
+                sig.base is out.base for sig in list(q.reads) + list(q.incs) + list(q.updates))]
+            if (out.base is not out or spikes.base is not spikes or out.base in probed
+                    or any(q not in rule_ops for q in readers) or out.base in self._shared
+                    or np.any(np.asarray(out.initial_value)) or np.any(np.asarray(spikes.initial_value))):
+                return self._learning_apart(plans, 5)
+        moved = type("Moved", (), {"reads_mem": {op.input.base for op in moving},
+                                   "writes_mem": {op.output.base for op in moving}})
+        if any(conflict(moved, q) for q in plans[f + 1:] + plans[:i]):
+            return self._learning_apart(plans, 6)
+        # neither launch may touch on its own what the other part relies on
+        if (dec.writes_mem & (rule.reads_mem | moved.writes_mem)) or (enc.reads_mem & moved.writes_mem):
+            return self._learning_apart(plans, 7)
+        result = self.backend.fuse_learning(enc, dec, rule, lf)
+        if result is None:
+            return self._learning_apart(plans, 8)
+        new_enc, new_dec, residual, pending = result
+        new_enc.reads_mem = enc.reads_mem | moved.reads_mem
+        new_enc.writes_mem = enc.writes_mem | moved.writes_mem
+        new_dec.reads_mem = dec.reads_mem | rule.reads_mem
+        new_dec.writes_mem = dec.writes_mem | rule.writes_mem
+        for p in residual:
+            rest = [op for op in lf_ops if op not in moving]
+            p.reads_mem = {op.input.base for op in rest}
+            p.writes_mem = {op.output.base for op in rest}
+            p.planned_ops = rest
+        for op in moving:
+            start = int(self.all_data.starts[self.sidx[op.output]])
+            spike_start, a_bits, b_bits, n = pending[start]
+            assert spike_start == int(self.all_data.starts[self.sidx[op.input]]) and n == op.output.size
+            bits = lambda v: None if v is None else np.int32(v).view(np.float32)
+            self._pending_filters[op.output.base] = (op.input.base, bits(a_bits), bits(b_bits))
+        plans[f:f + 1] = residual
+        del plans[r]
+        plans[j] = new_dec
+        plans[i] = new_enc
+        return plans
+
+    @staticmethod
+    def _learning_apart(plans, which):
+        logger.debug("learning rule and activity filters keep their launches (check %d of "
+                     "`_fuse_learning` did not hold)", which)
+        return plans
+
+    def _with_pending_filter(self, base, stored):
+        """The output of a filter whose last step is pending in device memory, as the
+        reference holds it: that step applied (the two rounded operations of the kernel)."""
+        spikes, a0, b0 = self._pending_filters[base]
+        x = np.asarray(self.all_data[self.sidx[spikes]], dtype=np.float32).reshape(stored.shape)
+        bx = np.float32(b0) * x
+        return bx if a0 is None else bx - np.float32(a0) * np.asarray(stored, dtype=np.float32)
+
     def _fuse_outer_filters(self, plans):
         """An outer-product update (a learning rule's weight increment) and the launch behind
         it that filters its column operands become one launch
@@ -765,6 +863,8 @@ class Simulator:
                 new.writes_mem = old.writes_mem | fw
             for p in residual:
                 p.reads_mem, p.writes_mem = rr, rw
+                if ops is not None and len(ops) == len(lf.lf_spec["X"]):
+                    p.planned_ops = [op for k, op in enumerate(ops) if k in rest]
                 if getattr(p, "bufpos", None) is not None:
                     self._filter_positions.append(p.bufpos)
             plans[j - 1:j] = residual
@@ -879,6 +979,9 @@ class Simulator:
                     # the last step's update of it
                     full = np.array(sim._host_view_copy[sim._host_view_index[base]])
                     raw = full if base is item else sim._view_of(item, full)
+                elif base in sim._pending_filters:
+                    full = sim._with_pending_filter(base, np.array(sim.all_data[sim.sidx[base]]))
+                    raw = full if base is item else sim._view_of(item, full)
                 else:
                     sim._refresh_lazy(base)
                     raw = sim.all_data[sim.sidx[item]]
@@ -909,6 +1012,14 @@ class Simulator:
                     raise ValueError(
                         "%s is not computed by this simulator (see reading it); "
                         "Simulator(reference_host_state=True) keeps every signal" % (item,))
+                deferred = set(sim._pending_filters) | {v[0] for v in sim._pending_filters.values()}
+                if base in deferred:
+                    raise ValueError(
+                        "%s belongs to a filter whose last step is still pending in device "
+                        "memory (it runs with the next step's neuron update): a write would be "
+                        "filtered once more or lost.  NENGO_HIP_FOLD_LEARNING=0 (or "
+                        "Simulator(reference_host_state=True)) keeps the filter a launch of the "
+                        "step it belongs to." % (item,))
                 if base in sim._updated_in_place:
                     raise ValueError(
                         "%s is updated in place by its learning rule: the change of the last "
@@ -964,6 +1075,10 @@ class Simulator:
         for base in list(self._lazy_currents):
             self._refresh_lazy(base)
         buf = np.array(self.all_data.buf)
+        for base in self._pending_filters:
+            i = self.sidx[base]
+            start, n = int(self.all_data.starts[i]), int(base.size)
+            buf[start:start + n] = self._with_pending_filter(base, buf[start:start + n]).reshape(-1)
         for base, k in self._host_view_index.items():
             i = self.sidx[base]
             start = int(self.all_data.starts[i])

@@ -358,9 +358,12 @@ def test_other_configurations_full_size_state_bit_exact(queue, case):
     with Simulator(net, seed=1, dedup=False) as gpu, \
             OracleSimulator(net_o, seed=1, dedup=False) as cpu:
         if case == "c4":
-            # the weight update runs together with the filter of the activities it reads
+            # the weight update rides in the launch that decodes with the learned matrices,
+            # the filter of the activities it reads in the launch that updates the neurons
             names = [p.name for p in gpu._plans]
-            assert "hip_outer_filter" in names and "hip_elementwise_inc" not in names
+            assert names[:2] == ["hipra_gemv.tile_lif", "hipra_gemv.tile_filter"]
+            assert "hip_outer_filter" not in names and "hip_elementwise_inc" not in names
+            assert gpu._plans[1].learned_matrices == 64 and gpu._plans[0].deferred_filters == 64
         gpu.run_steps(30)
         cpu.run_steps(30)
         for key in probes:
@@ -1071,3 +1074,63 @@ def test_populations_that_spike_densely_get_dense_products(queue):
         assert sum(p.n_tasks for p in uncalibrated._plans
                    if getattr(p, "event_driven", False)) >= n_event_tasks + 2
         assert not any(p.name.startswith("hipra_gemv.tile") for p in uncalibrated._plans)
+
+
+@pytest.mark.gpu
+def test_learning_rule_and_activity_filter_ride_in_the_two_launches(queue, monkeypatch):
+    """A PES step at sizes that take the large-item kernels: the outer-product update is done
+    by the launch that streams the learned decoders (each block written back with its change
+    once it has gone into the sums), and the filter of the pre-synaptic activities by the next
+    step's launch that updates the neurons (on the spikes it is about to replace).  Two
+    launches per step instead of three; every probe sample and every signal as the host reads
+    it -- the learned decoders, and the filtered activities whose last step is still pending
+    in device memory -- equal the oracle simulator bit for bit, over uneven `run_steps`
+    lengths, single steps and a reset; with the fold switched off the same numbers come from
+    three launches.  Writes to what is pending are refused."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    make = lambda: configs.c4_pes(n_triples=3, n_neurons=1024, dims=32, solver="lstsq",
+                                  learning_rate=3e-4, sample_every=None)
+    (net, probes, _), (net_o, probes_o, _), (net_u, probes_u, _) = make(), make(), make()
+    monkeypatch.setenv("NENGO_HIP_FOLD_LEARNING", "0")
+    unfolded = Simulator(net_u, seed=1)
+    monkeypatch.delenv("NENGO_HIP_FOLD_LEARNING")
+    with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu, unfolded:
+        assert [p.name for p in gpu._plans] == ["hipra_gemv.tile_lif", "hipra_gemv.tile_filter"]
+        assert [p.name for p in unfolded._plans] == ["hipra_gemv.tile_lif", "hipra_gemv.tile_filter",
+                                                     "hip_outer_filter"]
+        assert gpu._plans[1].learned_matrices == 3 and gpu._plans[0].deferred_filters == 3
+        assert len(gpu._pending_filters) == 3 and not unfolded._pending_filters
+        pending = list(gpu._pending_filters)
+
+        def check():
+            assert_same_signals(gpu, cpu)
+            assert_same_signals(gpu, unfolded)
+            for f in pending:  # the two simulators lay their signals out in the same order
+                same = cpu.all_bases[gpu.all_bases.index(f)]
+                assert np.array_equal(np.asarray(gpu.signals[f]), np.asarray(cpu.signals[same]))
+
+        check()  # before the first step
+        for n in (1, 1, 37, 200, 2):
+            for sim in (gpu, cpu, unfolded):
+                sim.run_steps(n)
+            check()
+        f = pending[0]
+        stored = np.asarray(gpu.all_data[gpu.sidx[f]]).ravel()
+        assert np.any(np.asarray(gpu.signals[f]) != 0)
+        assert not np.array_equal(stored, np.asarray(gpu.signals[f]).ravel())  # one step behind
+        for sig in (f, gpu._pending_filters[f][0]):
+            with pytest.raises(ValueError, match="pending"):
+                gpu.signals[sig] = np.zeros(sig.shape)
+        for sim in (gpu, cpu, unfolded):
+            sim.reset()
+        check()
+        for sim in (gpu, cpu, unfolded):
+            sim.run_steps(64)
+        check()
+        for key in probes:
+            assert np.array_equal(gpu.data[probes[key]], cpu.data[probes_o[key]]), key
+            assert np.array_equal(gpu.data[probes[key]], unfolded.data[probes_u[key]]), key
+        assert np.abs(gpu.data[probes["post0"]][-1]).max() > 0.01  # something was learned
