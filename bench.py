@@ -218,8 +218,8 @@ def measured_traffic(plan_name):
     from.  The summary names the hash of the kernel sources it was taken with; when the
     sources in this tree hash differently the figure is stale and None is returned in its
     place.  (None, None) for other workloads."""
-    kernel = {"hipra_gemv.tile_lif": "gemv_stream_kernel<1,0>",
-              "hipra_gemv.tile_filter": "gemv_stream_kernel<2,4>"}.get(plan_name)
+    kernel = {"hipra_gemv.tile_lif": "gemv_stream_kernel<1,0,0>",
+              "hipra_gemv.tile_filter": "gemv_stream_kernel<2,4,0>"}.get(plan_name)
     rel = os.path.join("profiles", "c3_shared_step.txt")
     path = os.path.join(ROOT, rel)
     if kernel is None or not os.path.exists(path):
@@ -617,13 +617,15 @@ def main():
             cols = sum(g["y_len"] * d["a_shape1"] for g in geo for d in g["dots"]) // max(n_rows, 1)
             cols -= cols % 8
             if n_rows >= 128 and cols >= 8:
-                floor = traffic_floor(sim.queue, n_rows, cols)
+                # (input currents that only the launch's own epilogue reads are not stored)
+                n_writes = 3 if getattr(lif, "lazy_currents", None) else 4
+                floor = traffic_floor(sim.queue, n_rows, cols, n_writes=n_writes)
                 best = min(floor["us"], floor["nontemporal_stores_us"])
                 roofline["plain_kernel_same_traffic"] = dict(
                     floor, frac_of_it=best / dom["avg_us"],
                     note="calibration kernel of the library: streams the matrix rows, reads 3 "
-                         "and writes 4 vectors per row, keeps no summation order and updates "
-                         "no neurons")
+                         "and writes %d vectors per row, keeps no summation order and updates "
+                         "no neurons" % n_writes)
 
     out = {
         "metric": "sim steps/sec + ragged-GEMV HBM GB/s (% peak), 1M-neuron LIF net, 1 MI355X",
