@@ -635,10 +635,15 @@ int nhip_sequence_chains(void *stream, const void *ops, const int *chain_ops,
  * writes (unless both only read it).  This call only records its arguments (`ops` must stay
  * valid until that launch has run; the host arrays are copied); the launch consumes them,
  * and fails with NHIP_E_BADARG if it cannot carry them (another kernel class, no epilogue,
- * an empty task list).  n_chains = 0 disarms.  No counterpart in the reference
+ * an empty task list).  n_chains = 0 disarms.  `needs` names the operations of the chains
+ * that not every carrying kernel holds (the library cannot read the device table): the
+ * launch that visits active columns only (nhip_gemv_events) runs on half the registers of
+ * the others and refuses chains that need any of them.  No counterpart in the reference
  * (plan.py:128-149 runs every plan as a launch of its own). */
+#define NHIP_SEQ_NEEDS_UNARY 1         /* an NHIP_SEQ_DIRECT_UNARY operation */
+#define NHIP_SEQ_NEEDS_HIGHER_ORDER 2  /* a linear filter with more than one coefficient on a side */
 int nhip_gemv_tile_carry(const void *ops, const int *chain_ops, const int *chain_staged,
-                         int n_chains);
+                         int n_chains, int needs);
 
 /* ---- function nodes compiled at run time ----------------------------------
  * replaces: `plan_direct` (:954-1025), which builds an OpenCL program from the

@@ -80,7 +80,7 @@ SIGNATURES = {
     "nhip_fill_i32": [P, P, c_int, c_int],
     "nhip_sequence": [P, P, c_int, c_int],
     "nhip_sequence_chains": [P, P, P, P, c_int],
-    "nhip_gemv_tile_carry": [P, P, P, c_int],
+    "nhip_gemv_tile_carry": [P, P, P, c_int, c_int],
     "nhip_capture_begin": [P],
     "nhip_capture_end": [P, ctypes.POINTER(c_void_p)],
     "nhip_graph_upload": [P, P],

@@ -15,8 +15,7 @@
 // (one per row), so a wave reads a column with one coalesced load, lane r holding row r.
 //
 // One work-group per 64 rows of an item, 4096 columns at a time (almost always the whole
-// item).  Each of
-// its sixteen waves takes a share of the tiles: it lists the
+// item).  Each of its eight waves takes a share of the tiles: it lists the
 // columns of its range with x != 0 in LDS (ballot and prefix count, so the list is in
 // column order), then walks the list EV_BATCH columns at a time -- the loads of a batch are
 // issued together -- and leaves alpha * tile sum of every tile in LDS.  After a barrier the
@@ -24,6 +23,13 @@
 // filters that read it.
 // A sequence armed with nhip_gemv_tile_carry rides in extra work-groups, as in the other
 // GEMV launches with an epilogue.
+// Group size and registers are chosen so that TWO groups fit a compute unit (512 threads,
+// at most 128 registers): a launch of a few groups more than the device has compute units
+// (one per 64 x 4096 decoder of 256 ensembles, two probes' decoders, two chains of a carried
+// sequence) then runs them all at once.  With groups of 1024 threads, one per compute unit,
+// the groups beyond the 256th waited for a compute unit to become free and the launch took
+// one and a half times as long as its groups.
+#define NHIP_SEQ_LEAN  // this kernel runs on 64 registers
 #include "nhip_common.h"
 #include "gemv_types.h"
 #include "neuron_math.h"
@@ -37,7 +43,9 @@ constexpr int EV_WG = 1024;         // sixteen waves per item: a wave's list is 
 constexpr int EV_WAVES = EV_WG / NHIP_WAVE;
 constexpr int EV_WAVE_COLS = EV_MAX_COLS / EV_WAVES;
 constexpr int EV_MAX_TILES = EV_MAX_COLS / EV_TILE;
-constexpr int EV_BATCH = 32;
+constexpr int EV_BATCH = 32;        // columns requested together: entry u of a batch is lane u's
+constexpr int EV_LIST_LOADS = EV_WAVE_COLS / NHIP_WAVE;  // x values a lane reads for the list
+static_assert(EV_BATCH <= NHIP_WAVE, "lane u of a wave holds entry u of the batch");
 
 struct EvItem {  // 16 words
     int at_start;      // column c of the transposed matrix: AT[at_start + c * mp + row]
@@ -65,8 +73,10 @@ struct EvLds {
 };
 
 // MULTI: some item of the launch has more than EV_MAX_COLS columns
-template <bool MULTI>
-__global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
+// CARRY: a sequence rides in extra groups (an instance of its own: the sequence's block
+// functions need more registers than the budget of 64, and spill; the products do not)
+template <bool MULTI, bool CARRY>
+__global__ __launch_bounds__(EV_WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void gemv_events_kernel(
     const EvItem* __restrict__ items, int n_items, const float* __restrict__ AT, const float* X,
     const float* Yin, float* Y, FilterArgs filter, EvSide side)
 {
@@ -74,7 +84,7 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
     static_assert(sizeof(EvLds) >= SEQ_MAX_OPS * sizeof(NhipSeqOp) +
                                        sizeof(int) * SEQ_MAX_ROWS * SEQ_ROW_WORDS,
                   "a carried sequence stages its records in the same LDS");
-    if (side.n_chains > 0 && (int)blockIdx.x >= n_items) {
+    if (CARRY && side.n_chains > 0 && (int)blockIdx.x >= n_items) {
         // a chain is run by 256 threads and their barriers: the other waves of the group
         // end here (a barrier waits for the waves that are still running)
         if (threadIdx.x >= NHIP_WG) return;
@@ -122,15 +132,15 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
 
         // the columns of this wave's range whose x is not zero, in column order
         int count = 0;
-        for (int c0 = c_lo; c0 < c_hi; c0 += 4 * NHIP_WAVE) {
-            float xv[4];
+        for (int c0 = c_lo; c0 < c_hi; c0 += EV_LIST_LOADS * NHIP_WAVE) {  // (once)
+            float xv[EV_LIST_LOADS];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < EV_LIST_LOADS; ++u) {
                 const int c = c0 + u * NHIP_WAVE + lane;
                 xv[u] = c < c_hi ? x[base + c] : 0.0f;
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < EV_LIST_LOADS; ++u) {
                 const bool nz = (__float_as_uint(xv[u]) & 0x7fffffffu) != 0u;
                 const unsigned long long b = __ballot(nz);
                 const int before = __builtin_amdgcn_mbcnt_hi(
@@ -151,18 +161,28 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
         float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
         int cur = -1;  // the tile the running sums belong to
         for (int k = 0; k < count; k += EV_BATCH) {
+            // lane u holds the column and the x of entry k + u; they reach the others
+            // through readlane, so a batch costs two LDS reads and no registers per entry
+            const int e = min(k + (lane & (EV_BATCH - 1)), count - 1);
+            const int col_e = col[e];
+            const float x_e = xs[e];
             float a[EV_BATCH];
-            int cc[EV_BATCH];
 #pragma unroll
-            for (int u = 0; u < EV_BATCH; ++u) {
-                cc[u] = col[min(k + u, count - 1)];
-                a[u] = at[(size_t)(base + cc[u]) * it.mp];
+            for (int g = 0; g < EV_BATCH; g += 16) {
+                if (k + g < count) {  // the same for all lanes
+#pragma unroll
+                    for (int u = g; u < g + 16; ++u) {
+                        const int c = __builtin_amdgcn_readlane(col_e, u);
+                        a[u] = at[(size_t)(base + c) * it.mp];
+                    }
+                }
             }
 #pragma unroll
             for (int u = 0; u < EV_BATCH; ++u) {
                 if (k + u < count) {  // the same for all lanes
-                    const int c = __builtin_amdgcn_readfirstlane(cc[u]);
-                    const float xv = xs[k + u];
+                    const int c = __builtin_amdgcn_readlane(col_e, u);
+                    const float xv = __builtin_bit_cast(
+                        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x_e), u));
                     const int t = c >> 7;
                     if (t != cur) {
                         if (cur >= 0) lds.tile[cur][lane] = it.alpha * ((s0 + s2) + (s1 + s3));
@@ -182,12 +202,15 @@ __global__ __launch_bounds__(EV_WG) void gemv_events_kernel(
         __syncthreads();  // the tiles of this run of columns are in LDS
 
         if (wave == 0) {
-            float tv[EV_MAX_TILES];
 #pragma unroll
-            for (int t = 0; t < EV_MAX_TILES; ++t) tv[t] = lds.tile[t][lane];  // (all reads at once)
+            for (int h = 0; h < EV_MAX_TILES; h += 16) {
+                float tv[16];
 #pragma unroll
-            for (int t = 0; t < EV_MAX_TILES; ++t)
-                if (t < n_tiles) sum = sum + tv[t];
+                for (int t = 0; t < 16; ++t) tv[t] = lds.tile[h + t][lane];  // (16 reads at once)
+#pragma unroll
+                for (int t = 0; t < 16; ++t)
+                    if (h + t < n_tiles) sum = sum + tv[t];
+            }
         }
         base += EV_MAX_COLS;
         if (MULTI && base < it.N) __syncthreads();  // ... and read, before the next run
@@ -217,6 +240,7 @@ extern "C" int nhip_gemv_events(void* stream, const int* items, int n_items, con
     const NhipCarried armed = nhip_carried;
     nhip_carried = NhipCarried{};
     if (n_items == 0) return armed.n_chains > 0 ? NHIP_E_BADARG : 0;  // nothing to ride in
+    if (armed.n_chains > 0 && armed.needs != 0) return NHIP_E_BADARG;  // (a lean sequence body)
     if (n_items < 0 || !items || !AT || !X || !Yin || !Y || max_cols <= 0) return NHIP_E_BADARG;
     if ((targets == nullptr) != (F == nullptr)) return NHIP_E_BADARG;
     EvSide side{};
@@ -234,8 +258,9 @@ extern "C" int nhip_gemv_events(void* stream, const int* items, int n_items, con
                     static_cast<hipStream_t>(stream), reinterpret_cast<const EvItem*>(items),
                     n_items, AT, X, Yin, Y, filter, side);
     };
-    if (max_cols > EV_MAX_COLS) launch(gemv_events_kernel<true>);
-    else launch(gemv_events_kernel<false>);
+    const bool carry = side.n_chains > 0;
+    if (max_cols > EV_MAX_COLS) carry ? launch(gemv_events_kernel<true, true>) : launch(gemv_events_kernel<true, false>);
+    else carry ? launch(gemv_events_kernel<false, true>) : launch(gemv_events_kernel<false, false>);
     NHIP_LAUNCH_CHECK();
     return 0;
 }

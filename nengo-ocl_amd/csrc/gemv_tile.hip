@@ -1572,7 +1572,7 @@ extern "C" int nhip_gemv_tile_lif_deferred(void* stream, int vec, int pow2_cols,
 thread_local NhipCarried nhip_carried;
 
 extern "C" int nhip_gemv_tile_carry(const void* ops, const int* chain_ops, const int* chain_staged,
-                                    int n_chains) {
+                                    int n_chains, int needs) {
     if (n_chains == 0) {
         nhip_carried = NhipCarried{};
         return 0;
@@ -1582,6 +1582,7 @@ extern "C" int nhip_gemv_tile_carry(const void* ops, const int* chain_ops, const
     NhipCarried c;
     c.ops = ops;
     c.n_chains = n_chains;
+    c.needs = needs;
     for (int k = 0; k < n_chains; ++k) {
         if (chain_ops[k] < 1 || chain_ops[k] > SEQ_MAX_OPS || chain_staged[k] < 0 ||
             chain_staged[k] > SEQ_MAX_ROWS)

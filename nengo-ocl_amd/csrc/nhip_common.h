@@ -106,5 +106,6 @@ struct NhipCarried {
     int first_op[NHIP_SEQ_MAX_CHAINS + 1] = {};
     int n_staged[NHIP_SEQ_MAX_CHAINS] = {};
     int n_chains = 0;
+    int needs = 0;  // NHIP_SEQ_NEEDS_*: operations that not every carrying kernel holds
 };
 extern thread_local NhipCarried nhip_carried;  // defined with nhip_gemv_tile_carry

@@ -4,6 +4,19 @@
 // whose launch can carry such a sequence in groups of its own.
 #pragma once
 
+// NHIP_SEQ_LEAN (defined by a kernel that carries sequences on a budget of 64 registers, before
+// it includes this file): an outer product keeps one quad per lane in flight instead of four,
+// the element loops stay rolled, and the two operations that need most registers -- unary
+// functions and linear filters of higher order (ring buffers) -- are left out; the host names
+// what a sequence needs (NHIP_SEQ_NEEDS_*) and such a kernel refuses one that needs them.
+#ifdef NHIP_SEQ_LEAN
+#define NHIP_SEQ_EW_QUADS 1
+#define NHIP_SEQ_LOOP _Pragma("unroll 1")
+#else
+#define NHIP_SEQ_EW_QUADS 4
+#define NHIP_SEQ_LOOP
+#endif
+
 #include "nhip_common.h"
 
 namespace {
@@ -38,6 +51,7 @@ __device__ __forceinline__ void reset_block(const int4 b, float* Y, int lane, in
     // b = {start, count, value_bits, 0}
     const float v = nhip_bits(b.z);
     float* y = Y + b.x;
+    NHIP_SEQ_LOOP
     for (int i = lane; i < b.y; i += L) y[i] = v;
 }
 
@@ -55,6 +69,7 @@ __device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, flo
         // contiguous on both sides and made of whole aligned quads: 16 bytes per access
         const float4* x4 = reinterpret_cast<const float4*>(x + d.offset);
         float4* y4 = reinterpret_cast<float4*>(y + d.offset);
+        NHIP_SEQ_LOOP
         for (int q = lane; q < (d.count >> 2); q += L) {
             float4 v = x4[q];
             if (d.inc) {
@@ -66,6 +81,7 @@ __device__ __forceinline__ void copy_block(const CopyDesc d, const float* X, flo
         return;
     }
     const int i0 = d.offset / d.shape1, j0 = d.offset - i0 * d.shape1;  // once per block
+    NHIP_SEQ_LOOP
     for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
         size_t xo, yo;
@@ -95,6 +111,7 @@ __device__ __forceinline__ void slicedcopy_block(const SlicedDesc d, const float
     float* y = Y + d.y_start;
     const int* xi = XI + d.xi_start;
     const int* yi = YI + d.yi_start;
+    NHIP_SEQ_LOOP
     for (int k = lane; k < d.count; k += L) {
         const float v = x[(size_t)xi[k] * d.x_stride0];
         float* dst = y + (size_t)yi[k] * d.y_stride0;
@@ -135,7 +152,8 @@ __device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const floa
         // row per lane, 16 bytes per access to Y (the same products and sums)
         // (four quads per lane at a time: their operands are requested together, so a lane
         // waits for memory once per four stores, not once per store)
-        constexpr int U = 4;
+        constexpr int U = NHIP_SEQ_EW_QUADS;
+        NHIP_SEQ_LOOP
         for (int k0 = 4 * lane; k0 < d.count; k0 += U * 4 * L) {
             float4* dst[U];
             float4 w[U];
@@ -166,6 +184,7 @@ __device__ __forceinline__ void elementwise_inc_block(const EwDesc d, const floa
         }
         return;
     }
+    NHIP_SEQ_LOOP
     for (int k = lane; k < d.count; k += L) {
         int i, j;
         nhip_row_col(i0, j0, k, d.y_shape1, d.count, i, j);
@@ -204,7 +223,11 @@ __device__ __forceinline__ void linearfilter_block(const LfDesc d, int2* pos, co
     const float* a = A + d.a_start;
     const float* b = B + d.b_start;
     const int na = d.na, nb = d.nb;
+#ifdef NHIP_SEQ_LEAN
+    const bool general = false;  // (such sequences are refused by the launch)
+#else
     const bool general = !(nb == 1 && na <= 1);
+#endif
     int ix = 0, iy = 0;
     if (general) {
         const int2 p = pos[block];
@@ -212,6 +235,7 @@ __device__ __forceinline__ void linearfilter_block(const LfDesc d, int2* pos, co
         iy = p.y;
     }
     const int i0 = d.offset / d.shape1, j0 = d.offset - i0 * d.shape1;  // once per block
+    NHIP_SEQ_LOOP
     for (int k = lane; k < d.count; k += L) {
         const int ij = d.offset + k;
         int i, j;
@@ -283,6 +307,7 @@ __device__ __forceinline__ void presentinput_block(const PiDesc d, float dt, flo
     }
     float* y = Y + d.y_start;
     const float* s = S + d.s_start + (size_t)d.m * ti;
+    NHIP_SEQ_LOOP
     for (int i = lane; i < d.m; i += L) y[i] = s[i];
 }
 
@@ -291,6 +316,7 @@ __device__ __forceinline__ void presentinput_block(const PiDesc d, float dt, flo
 __device__ __forceinline__ void direct_unary_block(int opcode, const int4 d, const float* X,
                                                    float* Y, int lane, int L) {
     // d = {x_start, y_start, count, 0}
+    NHIP_SEQ_LOOP
     for (int i = lane; i < d.z; i += L) {
         const float x = X[d.x + i];
         float y;
@@ -328,6 +354,7 @@ __device__ __forceinline__ void probes_block(const ProbeDesc d, float* countdown
         const int n_dims = d.shape0 * d.shape1;
         const float* x = X + d.x_start;
         float* y = Y + d.y_start + (size_t)bufpos * n_dims;
+        NHIP_SEQ_LOOP
         for (int ij = lane; ij < n_dims; ij += L) {
             const int i = ij / d.shape1, j = ij - i * d.shape1;
             y[ij] = x[(size_t)i * d.stride0 + (size_t)j * d.stride1];
@@ -392,12 +419,14 @@ __device__ __forceinline__ void sequence_chain(const NhipSeqOp* ops, int n_ops, 
         const int* src = reinterpret_cast<const int*>(ops);
         int* dst = reinterpret_cast<int*>(s_ops);
         const int n_words = n_ops * (int)(sizeof(NhipSeqOp) / sizeof(int));
+        NHIP_SEQ_LOOP
         for (int w = tid; w < n_words; w += NHIP_WG) dst[w] = src[w];
     }
     __syncthreads();
     {   // work-list rows of the operations with a whole group per row: 16 threads per
         // row, one word each
         const int sub = tid >> 4, word = tid & 15;
+        NHIP_SEQ_LOOP
         for (int r0 = 0; r0 < n_staged; r0 += NHIP_WG / 16) {
             int r = r0 + sub, k = 0;
             while (k < n_ops && (s_ops[k].lanes != NHIP_WG || r >= s_ops[k].n_blocks)) {
@@ -455,10 +484,12 @@ __device__ __forceinline__ void sequence_chain(const NhipSeqOp* ops, int n_ops, 
                         presentinput_block(SEQ_ROW(PiDesc), (float)op.d0, SEQ_P(1, float*),
                                            SEQ_P(2, const float*), SEQ_P(3, const float*), lane, L);
                         break;
+#ifndef NHIP_SEQ_LEAN
                     case NHIP_SEQ_DIRECT_UNARY:
                         direct_unary_block(op.i0, SEQ_ROW(int4), SEQ_P(1, const float*),
                                            SEQ_P(2, float*), lane, L);
                         break;
+#endif
                     case NHIP_SEQ_PROBES:
                         probes_block(SEQ_ROW(ProbeDesc), SEQ_P(1, float*), SEQ_P(2, int*),
                                      SEQ_P(3, const float*), SEQ_P(4, const float*),

@@ -448,6 +448,7 @@ def plan_linearfilter(queue, X, Y, A, B, Xbuf, Ybuf, tag=None):
     plan.description = _description(Y)
     plan.row_iterations = _row_iterations(counts, lanes)
     plan.bufpos = pos  # zeroed again by Simulator.reset()
+    plan.higher_order = bool(((A.shape0s > 1) | (B.shape0s > 1)).any())  # ring buffers in use
     # what a GEMV that produces X needs to run simple filters as its epilogue
     plan.lf_spec = dict(X=X, Y=Y, A=A, B=B, Xbuf=Xbuf, Ybuf=Ybuf)
     return [plan]

@@ -130,6 +130,13 @@ def chains_of(plans):
     return [[plans[i] for i in chain] for chain in chains]
 
 
+def sequence_needs(plans):
+    """What not every kernel that can carry a sequence of `plans` holds (NHIP_SEQ_NEEDS_*):
+    1 = a unary function, 2 = a linear filter of higher order (ring buffers)."""
+    return (1 if any(sequence_op(p)[0] == SEQ_DIRECT_UNARY for p in plans) else 0) | (
+        2 if any(getattr(p, "higher_order", False) for p in plans) else 0)
+
+
 def plan_sequence(queue, plans):
     """One launch that runs `plans` (all small, see `is_small`): in order where they
     depend on each other, independent chains of them side by side (a group each)."""
@@ -153,6 +160,7 @@ def plan_sequence(queue, plans):
                   name="hip_sequence",
                   tag=" | ".join("+".join(p.name.replace("hip_", "") for p in c) for c in chains))
     merged.members = list(plans)
+    merged.needs = sequence_needs(plans)
     bws = [p.bw_per_call for p in plans if p.bw_per_call]
     merged.bw_per_call = sum(bws) if bws else None
     reads = [getattr(p, "reads_mem", None) for p in plans]
@@ -203,10 +211,11 @@ def merge_small_plans(plans):
     return out
 
 
-def _can_carry(plan):
+def _can_carry(plan, needs=0):
     """GEMV launches with an epilogue: the large-item kernel with compile-time shapes, the
-    launch that visits only the columns with x != 0, the small-item kernel, and the sparse
-    products."""
+    launch that visits only the columns with x != 0 (which runs on half the registers of the
+    others and holds no unary functions and no higher-order filters: `needs`), the small-item
+    kernel, and the sparse products."""
     cls = getattr(plan, "kernel_class", None)
     name = getattr(plan, "name", "")
     if name in ("hip_spmv", "hip_spmv_filter"):  # the sparse products (one or more slices)
@@ -216,7 +225,7 @@ def _can_carry(plan):
     if name in ("hipra_gemv.tile_lif", "hipra_gemv.tile_filter"):
         return cls[0] == 3 and cls[1] >= 2
     if name in ("hipra_gemv.events", "hipra_gemv.events_filter"):
-        return cls[0] == 4
+        return cls[0] == 4 and needs == 0
     return name in ("hipra_gemv.wave_ref", "hipra_gemv.wave_ref_lif",
                     "hipra_gemv.wave_ref_filter") and cls[0] == 2
 
@@ -235,13 +244,14 @@ def carry_sequences(plans):
         if not rides:
             k += 1
             continue
+        needs = seq.needs if seq.name == "hip_sequence" else sequence_needs([seq])
         # the nearest launch that can take it, backwards then forwards, over plans that touch
         # none of its memory (moving past those changes nothing)
         j = None
         for step in (-1, 1):
             q = k + step
             while 0 <= q < len(plans) and hasattr(plans[q], "enqueue") and not _conflict(seq, plans[q]):
-                if _can_carry(plans[q]):
+                if _can_carry(plans[q], needs):
                     j = q
                     break
                 q += step
@@ -253,7 +263,7 @@ def carry_sequences(plans):
         if seq.name != "hip_sequence":
             seq = plan_sequence(seq.queue, [seq])
         carrier = plans[j]
-        carrier.prelude = (seq.queue.lib.nhip_gemv_tile_carry, seq.args)
+        carrier.prelude = (seq.queue.lib.nhip_gemv_tile_carry, tuple(seq.args) + (seq.needs,))
         carrier.full_args = carrier.full_args + (seq,)
         carrier.carried = seq
         carrier.tag = "%s + %s" % (carrier.tag, seq.tag)

@@ -335,8 +335,19 @@ def test_launch_fusions_change_nothing(queue, monkeypatch):
         small = [p for p in plain._plans if p.name == "hipra_gemv.wave_ref"][0]
         big = [p for p in plain._plans if p.name == "hipra_gemv.tile_lif"][0]
         assert lib.nhip_gemv_tile(queue.handle, *big.args[:7], 0, *big.args[8:12]) == -1
-        _lib.check(fn(args[0], args[1], args[2], 0))  # disarmed
+        _lib.check(fn(args[0], args[1], args[2], 0, 0))  # disarmed
         small()
+        # the launch that visits active columns runs on half the registers of the others and
+        # holds neither unary functions nor higher-order filters: a sequence said to need one
+        # is refused by it (and the planner does not offer it one)
+        from nengo_ocl_amd import hipra_sequence
+
+        assert carrier.name == "hipra_gemv.events_filter" and args[4] == 0
+        _lib.check(fn(args[0], args[1], args[2], args[3], 1))
+        assert lib.nhip_gemv_events(queue.handle, *carrier.args) == -1
+        bare = [p for p in plain._plans if p.name == "hipra_gemv.events_filter"][0]
+        assert hipra_sequence._can_carry(bare, 0) and not hipra_sequence._can_carry(bare, 1)
+        assert not hipra_sequence._can_carry(bare, 2)
 
 
 @pytest.mark.parametrize("case", ["c2", "c3-per-connection", "c4", "c5"])
