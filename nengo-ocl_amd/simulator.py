@@ -1145,10 +1145,10 @@ class Simulator:
                         got = self.backend.read_rows(plan.Y, i, n_buffered)
                         self._probe_outputs[probe].extend(got.reshape((n_buffered,) + shape))
                 return
+        self.backend.finish()
         self._probe_step_time()
         if plan is None:
             return
-        self.backend.finish()
         bufpositions = self.backend.get_array(plan.dev_bufpositions)
         for i, probe in enumerate(self.model.probes):
             shape = self.model.sig[probe]["in"].shape
@@ -1224,7 +1224,12 @@ class Simulator:
         while steps > 0:
             B = min(steps, self._max_steps_between_probes)
             self._probes_drained = False
-            self._plans.call_n_times(B)
+            if self._drain is not None and not self._plans.profiling:
+                # the drain is queued right behind the steps and waits for both: one host
+                # round trip per batch instead of two
+                self._plans.enqueue_n_times(B)
+            else:
+                self._plans.call_n_times(B)
             self._probe(B)
             self._probes_drained = True
             steps -= B
