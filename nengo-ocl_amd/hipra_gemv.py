@@ -144,6 +144,50 @@ def _literal_coefficient(arg, n):
     return None
 
 
+SPREAD_OVER_DIES = os.environ.get("NENGO_HIP_SPREAD_TASKS", "1") != "0"  # switch for measurements
+N_DIES = 8  # accelerator dies of the device: work-group g runs on die g % 8
+
+
+def spread_over_dies(tasks):
+    """The 24-word task records of a large-item launch in an order that gives every
+    accelerator die the same number of heavy tasks.
+
+    Work-groups go to the dies in turn, and the kernels map them so that a die works through
+    one contiguous range of the task list (`nhip_xcd_remap`).  Tasks without a matrix to stream
+    (sums nothing else reads, populations without input) sit at the end of the list as it is
+    built, so the last die got all of them and the first ones only heavy tasks: a launch of two
+    rounds of groups per die then ran a third round on some dies.  Here the light tasks are
+    dealt out over the ranges (at the end of each), so that the heavy ones divide evenly.
+    Tasks are independent of each other (each owns its rows), so any order gives the same
+    result."""
+    per_group = WG // WAVE
+    n = len(tasks)
+    groups = -(-n // per_group)
+    if not SPREAD_OVER_DIES or groups < 2 * N_DIES or tasks.shape[1] != 24:
+        return tasks
+    weight = tasks[:, 2].astype(np.int64) * np.maximum(tasks[:, 18], 1) * (tasks[:, 9] > 0)
+    heavy = weight >= 0.25 * max(int(weight.max()), 1)
+    if heavy.all() or not heavy.any():
+        return tasks
+    H, L = tasks[heavy], tasks[~heavy]
+    per, rem = divmod(groups, N_DIES)  # (the partition nhip_xcd_remap makes)
+    sizes = [(per + (1 if x < rem else 0)) * per_group for x in range(N_DIES)]
+    sizes[-1] -= groups * per_group - n
+    out, ih, il = [], 0, 0
+    for x, size in enumerate(sizes):
+        want = len(H) * (x + 1) // N_DIES
+        want -= want % per_group if x < N_DIES - 1 else 0  # whole groups of heavy tasks
+        h = max(0, min(want - ih, size, len(H) - ih))
+        l = min(size - h, len(L) - il)
+        h = min(size - l, len(H) - ih)  # (too few light tasks left: heavy ones fill the range)
+        out += [H[ih:ih + h], L[il:il + l]]
+        ih, il = ih + h, il + l
+    out += [H[ih:], L[il:]]
+    out = np.concatenate(out)
+    assert len(out) == n
+    return out
+
+
 def _balanced_rows(M, cap):
     """Rows per task so that the tasks of an item are equally full (M = 4096, cap = 128
     stays 128; M = 100, cap = 64 becomes 50 instead of 64 + 36)."""
@@ -614,7 +658,7 @@ class gemv_prog:
                 fat[:, 12:16] = coef_tab[which].view(np.int32)
                 has_dots = item_tab[which, 5] > 0
                 fat[has_dots, 16:24] = dot_tab[item_tab[which[has_dots], 4]]
-                task_tab = fat
+                task_tab = spread_over_dies(fat)
             dev_tasks = to_device(self.queue, task_tab)
             n_tasks = len(task_rows)
             if flavor == 0:
@@ -1058,6 +1102,7 @@ def fuse_input_sums(sum_plan, lif_plan):
             new_pops = pops
             args = args[:12] + (dev_pops.ptr,) + args[13:]
             keep = (dev_pops,)
+        tasks = spread_over_dies(tasks)
         dev_tasks = to_device(queue, tasks)
         n_groups = -(-len(tasks) // (WG // WAVE))
         args = args[:6] + (dev_tasks.ptr, len(tasks)) + args[8:] + (dev_parts.ptr,)

@@ -620,3 +620,34 @@ def test_sparse_planner_choice_follows_the_reference_rule():
     assert set(sp.algostr_to_planner) == {"ELLPACK", "ELLPACK-tree", "ELLPACK-twostep", "CSR"}
     for cls in sp.algostr_to_planner.values():
         assert issubclass(cls, sp.spmv_prog) and issubclass(cls, sp.plan_sparse_dot_inc)
+
+
+def test_heavy_tasks_divide_evenly_over_the_dies():
+    """Task records of a large-item launch are reordered so that every accelerator die (a
+    contiguous range of the list, `nhip_xcd_remap`) gets the same number of tasks that stream
+    a matrix; the light ones (no dot product) fill the ranges up.  Nothing is lost or
+    duplicated; lists of equal tasks and short lists stay as they are."""
+    from nengo_ocl_amd import hipra_gemv as g
+
+    t = np.zeros((8194, 24), dtype=np.int32)
+    t[:8064, 2], t[:8064, 9], t[:8064, 18] = 128, 1, 64
+    t[:8064, 0], t[:8064, 1] = np.arange(8064) // 32, (np.arange(8064) % 32) * 128
+    t[8064:, 2], t[8064:, 0] = 64, 300 + np.arange(130)
+    out = g.spread_over_dies(t)
+    assert sorted(map(tuple, out.tolist())) == sorted(map(tuple, t.tolist()))
+    groups = -(-len(t) // 4)
+    per, rem = divmod(groups, 8)
+    pos, heavy = 0, []
+    for x in range(8):
+        size = (per + (1 if x < rem else 0)) * 4
+        heavy.append(int((out[pos:pos + size, 9] > 0).sum()))
+        pos += size
+    assert heavy == [1008] * 8
+    # heavy tasks keep their order (rows of one matrix stay neighbours)
+    assert np.array_equal(out[out[:, 9] > 0], t[:8064])
+    assert g.spread_over_dies(t[:8064]) is t[:8064] or np.array_equal(g.spread_over_dies(t[:8064]), t[:8064])
+    assert np.array_equal(g.spread_over_dies(t[8000:8050]), t[8000:8050])  # 13 groups: left alone
+    # few light tasks: ranges are filled with heavy ones, nothing is dropped
+    few = np.concatenate([t[:8064], t[8064:8067]])
+    out = g.spread_over_dies(few)
+    assert sorted(map(tuple, out.tolist())) == sorted(map(tuple, few.tolist()))

@@ -350,6 +350,31 @@ def test_launch_fusions_change_nothing(queue, monkeypatch):
         assert not hipra_sequence._can_carry(bare, 2)
 
 
+def test_wide_populations_take_their_columns_in_runs(queue):
+    """Ensembles of more than 4096 neurons: the launch that visits active columns takes their
+    decoders 4096 columns at a time (its instance for such items, here with the step's short
+    operations riding in it); 64-D and 20-D values (rows of the transposed matrices padded to
+    16); every signal and probe sample equal the oracle simulator's bit for bit."""
+    from nengo_ocl_amd import configs
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    for dims in (64, 20):
+        make = lambda: configs.c3_large(n_ens=4, n_neurons=9000, dims=dims, fan_out=2)
+        (net, probes, _), (net_o, probes_o, _) = make(), make()
+        with Simulator(net, seed=1) as gpu, OracleSimulator(net_o, seed=1) as cpu:
+            ev = [p for p in gpu._plans if p.name.startswith("hipra_gemv.events")]
+            assert len(ev) == 1 and getattr(ev[0], "carried", None) is not None
+            assert int(ev[0].event_table[:, 3].max()) == 9000
+            for n in (1, 50, 49):
+                gpu.run_steps(n)
+                cpu.run_steps(n)
+                assert_same_signals(gpu, cpu)
+            for key in probes:
+                assert np.array_equal(gpu.data[probes[key]], cpu.data[probes_o[key]])
+                assert np.any(gpu.data[probes[key]] != 0)
+
+
 @pytest.mark.parametrize("case", ["c2", "c3-per-connection", "c4", "c5"])
 def test_other_configurations_full_size_state_bit_exact(queue, case):
     """The other benchmark configurations at their full sizes (2048 ensembles on a
