@@ -275,8 +275,12 @@ __global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_kernel(
 
 // the same with an epilogue per finished row (A, X, Yin are not marked read-only
 // here either: the epilogue writes neuron state / filter outputs into the same buffer)
+// (a launch of a wave per task without a carried sequence fits 96 registers: five waves per
+// SIMD instead of four, 1280 groups resident instead of 1024 -- a launch of a few groups more
+// than 1024, like 2048 ensembles of 100 neurons with their input sums, then runs in one round)
 template <int LPR, int EPI, bool WIDE, bool SIDE, bool WAVE_TASK = false>
-__global__ __launch_bounds__(NHIP_WG) void gemv_rows_ref_epi_kernel(
+__global__ __launch_bounds__(NHIP_WG) __attribute__((amdgpu_waves_per_eu((WAVE_TASK && !SIDE) ? 5 : 4)))
+void gemv_rows_ref_epi_kernel(
     const GemvItem* __restrict__ items, const float4* __restrict__ coefs,
     const GemvDot* __restrict__ dots, const GemvTask* __restrict__ tasks, int n_tasks,
     const float* A, const float* X, const float* Yin, float* Y, const EpilogueArgs epi,

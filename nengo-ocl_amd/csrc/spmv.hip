@@ -301,7 +301,10 @@ int launch_skip(void* stream, const int* slices, int n_slices, const int* row_le
         n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     }
     const int wpg = SPMV_SKIP_WG / NHIP_WAVE;
-    side.n_groups = min(n_cu, (n_slices + wpg - 1) / wpg);
+    // a group takes a whole compute unit (its LDS holds the bits of X), so the groups of a
+    // carried sequence need compute units of their own: with one product group per compute
+    // unit they would only start when the product is over
+    side.n_groups = min(n_cu > side.n_chains ? n_cu - side.n_chains : n_cu, (n_slices + wpg - 1) / wpg);
     NHIP_LAUNCH_LAST(spmv_sell_skip_kernel, dim3(side.n_groups + side.n_chains), dim3(SPMV_SKIP_WG), 0, s,
                 reinterpret_cast<const SpmvSlice*>(slices), n_slices, row_len, cols, vals, X, Y,
                 mask, n_mask_quads, epi, side);
