@@ -187,17 +187,13 @@ class _GraphSegment:
     as graphs of unroll/2, ..., 2, 1 timesteps for what is left over (n steps are then
     n // unroll launches of the long graph plus at most one launch of each shorter one).
     All of them are recorded, instantiated and uploaded to the device by `prepare`,
-    before the first step runs.  A caller that asks for the same number of steps twice in a
-    row (a control loop that advances the simulation a fixed interval at a time) gets one
-    more graph, of exactly that many steps, recorded at the second request: every further
-    request is then a single graph launch instead of one per binary digit.
+    before the first step runs, so that no call of `launch` ever records anything.
     """
 
     # timesteps recorded back to back into the long graph: as many as keep it within
     # MAX_GRAPH_NODES kernel nodes (a step of two launches: 128 steps; of ten: 16)
     MAX_UNROLL = 128
     MAX_GRAPH_NODES = 256
-    MAX_EXACT_GRAPHS = 4  # graphs of a repeated step count kept at a time
 
     def __init__(self, queue, plans, before_last=()):
         self.queue = queue
@@ -206,8 +202,6 @@ class _GraphSegment:
         self.before_last = list(before_last)
         self.execs = {}  # timesteps per graph -> executable graph
         self.tail_execs = {}  # the same with `before_last` recorded ahead of the last step
-        self.exact_execs = {}  # (timesteps, tail) -> graph of a step count asked for repeatedly
-        self._last_request = None
         unroll = 1
         while unroll * 2 <= self.MAX_UNROLL and unroll * 2 * len(self.plans) <= self.MAX_GRAPH_NODES:
             unroll *= 2
@@ -222,10 +216,9 @@ class _GraphSegment:
             n //= 2
         return out
 
-    def capture(self, n_steps=1, tail=False, exact=False):
+    def capture(self, n_steps=1, tail=False):
         """Record `n_steps` consecutive timesteps into one executable graph (`tail`: with
-        the `before_last` plans ahead of the last of them; `exact`: kept among the graphs of
-        repeated step counts)."""
+        the `before_last` plans ahead of the last of them)."""
         lib = self.queue.lib
         _lib.check(lib.nhip_capture_begin(self.queue.handle), "graph capture begin")
         err = None
@@ -245,10 +238,7 @@ class _GraphSegment:
                 lib.nhip_graph_destroy(handle)
             raise err
         _lib.check(rc, "graph capture end")
-        if exact:
-            self.exact_execs[(n_steps, tail)] = handle
-        else:
-            (self.tail_execs if tail else self.execs)[n_steps] = handle
+        (self.tail_execs if tail else self.execs)[n_steps] = handle
 
     def steps_of_every_graph(self):
         """A step count whose run launches each recorded graph once."""
@@ -276,11 +266,6 @@ class _GraphSegment:
         variant with those plans recorded ahead of its last step."""
         lib = self.queue.lib
         self.prepare()
-        tail = bool(tail and self.before_last)
-        exact = self._exact_graph(n, tail)
-        if exact is not None:
-            _lib.check(lib.nhip_graph_launch(exact, self.queue.handle, 1), "graph launch")
-            return
         times, rest = divmod(n, self.unroll)
         todo = [(self.unroll, times)] if times else []
         todo += [(n_steps, 1) for n_steps in self.sizes[1:] if rest & n_steps]
@@ -292,30 +277,10 @@ class _GraphSegment:
             _lib.check(lib.nhip_graph_launch(execs[n_steps], self.queue.handle, abs(count)),
                        "graph launch")
 
-    def _exact_graph(self, n, tail):
-        """The graph of exactly `n` timesteps if there is one; recorded when `n` is asked for
-        the second time in a row, takes more than one launch otherwise and fits a graph."""
-        key = (n, tail)
-        handle = self.exact_execs.get(key)
-        repeated, self._last_request = self._last_request == key, key
-        if handle is not None or not repeated:
-            return handle
-        nodes = n * len(self.plans) + len(self.before_last)
-        if n & (n - 1) == 0 or n <= 0 or nodes > self.MAX_GRAPH_NODES:
-            return None  # one launch already, or too long for one graph
-        while len(self.exact_execs) >= self.MAX_EXACT_GRAPHS:
-            self.queue.finish()  # (a graph must not be destroyed while it may still be running)
-            self.queue.lib.nhip_graph_destroy(self.exact_execs.pop(next(iter(self.exact_execs))))
-        self.capture(n, tail=tail, exact=True)
-        _lib.check(self.queue.lib.nhip_graph_upload(self.exact_execs[key], self.queue.handle),
-                   "graph upload")
-        return self.exact_execs[key]
-
     def destroy(self):
-        for handle in (list(self.execs.values()) + list(self.tail_execs.values())
-                       + list(self.exact_execs.values())):
+        for handle in list(self.execs.values()) + list(self.tail_execs.values()):
             self.queue.lib.nhip_graph_destroy(handle)
-        self.execs, self.tail_execs, self.exact_execs = {}, {}, {}
+        self.execs, self.tail_execs = {}, {}
 
 
 class Plans:
