@@ -196,6 +196,36 @@ def _not(a):
     return _node("not", a if a.is_bool else _apply("ne", a, 0.0))
 
 
+def _isnan(a):
+    return _apply("ne", a, a)
+
+
+def _isinf(a):
+    return _apply("eq", _apply("fabs", a), math.inf)
+
+
+def _isfinite(a):
+    return _apply("lt", _apply("fabs", a), math.inf)
+
+
+def _signbit(a):  # true for -0.0 as well
+    return _apply("lt", _apply("copysign", 1.0, a), 0.0)
+
+
+def _ldexp(a, b):
+    return _apply("mul", a, _apply("exp2", b))
+
+
+def _logaddexp(a, b):  # log(exp(a) + exp(b)) without overflow
+    return _apply("add", _apply("maximum", a, b),
+                  _apply("log1p", _apply("exp", _apply("neg", _apply("fabs", _apply("sub", a, b))))))
+
+
+def _logaddexp2(a, b):
+    return _apply("add", _apply("maximum", a, b),
+                  _apply("log2", _apply("add", 1.0, _apply("exp2", _apply("neg", _apply("fabs", _apply("sub", a, b)))))))
+
+
 def _logic(op):
     def fn(a, b):
         a, b = _wrap(a), _wrap(b)
@@ -230,6 +260,8 @@ _UFUNCS.update({
     "atan": lambda a: _apply("arctan", a), "asinh": lambda a: _apply("arcsinh", a),
     "acosh": lambda a: _apply("arccosh", a), "atanh": lambda a: _apply("arctanh", a),
     "atan2": lambda a, b: _apply("arctan2", a, b), "pow": _pow,
+    "isnan": _isnan, "isinf": _isinf, "isfinite": _isfinite, "signbit": _signbit,
+    "ldexp": _ldexp, "logaddexp": _logaddexp, "logaddexp2": _logaddexp2,
 })
 
 
@@ -362,7 +394,8 @@ class _MathShim:
               "sqrt": "sqrt", "pow": "pow", "fabs": "fabs", "floor": "floor", "ceil": "ceil",
               "trunc": "trunc", "fmod": "fmod", "hypot": "hypot", "copysign": "copysign",
               "degrees": "degrees", "radians": "radians", "erf": "erf", "erfc": "erfc",
-              "gamma": "gamma", "lgamma": "lgamma"}
+              "gamma": "gamma", "lgamma": "lgamma", "isnan": "isnan", "isinf": "isinf",
+              "isfinite": "isfinite", "ldexp": "ldexp"}
 
     def __getattr__(self, name):
         real = getattr(math, name)

@@ -606,6 +606,13 @@ def plan_direct(queue, code, init, input_names, inputs, output, tag=None):
 
 
 DIRECT_KERNEL = """\
+// (the run-time compiler's headers do not bring the C macros for these along)
+#ifndef INFINITY
+#define INFINITY __builtin_inff()
+#endif
+#ifndef NAN
+#define NAN __builtin_nanf("")
+#endif
 extern "C" __global__ void direct(int n__, const int* in0_starts__, const float* in0_data__,
                                   const int* in1_starts__, const float* in1_data__,
                                   const int* out_starts__, float* out_data__) {

@@ -87,6 +87,9 @@ CASES = [
     (lambda x: (x[0] ** 3, x[0] ** 0.5 if x[0] > 0 else 0.0, 2 ** x[1], x[1] ** -2), False, 2, 4),
     (lambda x: round(x[0]) + math.floor(x[1]) + math.ceil(x[0]) + np.trunc(x[1]), False, 2, 1),
     (lambda t: [1.0, 2.0], True, None, 2),
+    # (appended: the GPU test names earlier cases by position)
+    (lambda x: [np.logaddexp(x[0], x[1]), np.ldexp(x[0], 2), 1.0 if np.isfinite(x[1]) else 0.0,
+                2.0 if np.isnan(x[0]) else x[0], -1.0 if np.signbit(x[1]) else 1.0], False, 2, 5),
 ]
 
 
@@ -224,3 +227,31 @@ def test_generated_kernels_compile_for_gfx950():
         nl.compile_direct(lib, nl.direct_kernel_source("OUTPUT__[0] = nosuch(t[0]);", "", ["t"]))
     with pytest.raises(NotImplementedError):
         nl.direct_kernel_source("", "", ["a", "b", "c"])
+
+
+def test_classification_and_scaling_functions():
+    """isnan / isinf / isfinite / signbit, ldexp, logaddexp / logaddexp2 (the rest of the
+    reference translator's table, ast_conversion.py:103-105, 137, 164-171, 194): traced from
+    numpy and from math, against the functions themselves, special values included."""
+    special = [0.0, -0.0, 1.5, -2.25, np.inf, -np.inf, np.nan, 1e-40, 3e38]
+    for name in ("isnan", "isinf", "isfinite", "signbit"):
+        traced = ft.trace(lambda x, f=getattr(np, name): f(x[0]), False, 1, 1)
+        for v in special:
+            assert bool(traced(None, [v])[0]) == bool(getattr(np, name)(v)), (name, v)
+    for name in ("isnan", "isinf", "isfinite"):
+        traced = ft.trace(eval("lambda x: 1.0 if math.%s(x[0]) else 0.0" % name, {"math": math}),
+                          False, 1, 1)
+        for v in special:
+            assert bool(traced(None, [v])[0]) == bool(getattr(math, name)(v)), (name, v)
+    rng = np.random.RandomState(3)
+    two = {"ldexp": lambda a, b: np.ldexp(a, int(b)), "logaddexp": np.logaddexp,
+           "logaddexp2": np.logaddexp2}
+    for name, real in two.items():
+        fn = (lambda x: np.ldexp(x[0], 3)) if name == "ldexp" else (lambda x, f=real: f(x[0], x[1]))
+        traced = ft.trace(fn, False, 2, 1)
+        for a, b in rng.uniform(-30, 30, size=(50, 2)):
+            want = float(np.ldexp(a, 3)) if name == "ldexp" else float(real(a, b))
+            assert traced(None, [a, b])[0] == pytest.approx(want, rel=1e-12, abs=1e-12), name
+    big = ft.trace(lambda x: np.logaddexp(x[0], x[1]), False, 2, 1)
+    assert big(None, [1000.0, 999.0])[0] == pytest.approx(float(np.logaddexp(1000.0, 999.0)))
+    assert ft.trace(lambda x: math.ldexp(x[0], 2), False, 1, 1)(None, [1.5])[0] == 6.0
