@@ -651,3 +651,33 @@ def test_heavy_tasks_divide_evenly_over_the_dies():
     few = np.concatenate([t[:8064], t[8064:8067]])
     out = g.spread_over_dies(few)
     assert sorted(map(tuple, out.tolist())) == sorted(map(tuple, few.tolist()))
+
+
+def test_reset_restarts_the_random_streams_of_host_processes():
+    """The reference's test_reset (tests/test_simulator.py:62-87): a node driven by a process
+    whose step draws from the generator the simulator hands it gives the same samples again
+    after `reset()`."""
+    from nengo_ocl_amd import ir, minibuilder as mb
+    from oracle.oracle_sim import OracleSimulator
+
+    class CustomProcess(ir.Process):
+        def get_rng(self, rng):
+            return np.random.RandomState(rng.randint(2 ** 31 - 1) if self.seed is None else self.seed)
+
+        def make_state(self, shape_in, shape_out, dt, dtype=None):
+            return {}
+
+        def make_step(self, shape_in, shape_out, dt, rng, state):
+            return lambda t: rng.uniform(size=shape_out).ravel()
+
+    net = mb.Network(seed=3)
+    u = net.Node(CustomProcess(), size_out=2)
+    up = net.Probe(u)
+    with OracleSimulator(net, seed=3) as sim:
+        sim.run_steps(10)
+        ua = np.array(sim.data[up])
+        sim.reset()
+        sim.run_steps(10)
+        ub = np.array(sim.data[up])
+    assert ua.shape == (10, 2) and np.any(ua != 0) and len(np.unique(ua)) == 20
+    assert np.array_equal(ua, ub)
