@@ -69,3 +69,19 @@ def test_no_device_no_fallback():
 
     with pytest.raises(RuntimeError):
         Queue(0)
+
+
+def test_bench_command_line_contract():
+    """`bench.py --gpus N` with N above 1 exits with a message that says why (every box has one
+    GPU); `--kernel-hash` prints the hash that `profiles/c3_shared_step.txt` is compared with."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    two = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True, timeout=120)
+    assert two.returncode != 0 and "one GPU" in (two.stdout + two.stderr)
+    h = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--kernel-hash"],
+                       capture_output=True, text=True, timeout=120)
+    words = h.stdout.split()
+    assert h.returncode == 0 and words[0] == "kernel_sources_sha256" and len(words[1]) == 64
