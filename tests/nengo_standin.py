@@ -167,6 +167,33 @@ class SimPES(Operator):  # simulator.py:1334-1345: pre_filtered, error, delta, l
         self.updates = [delta]
 
 
+class SimBCM(Operator):  # simulator.py:1347-1353: pre_filtered, post_filtered, theta, delta, learning_rate
+    def __init__(self, pre_filtered, post_filtered, theta, delta, learning_rate, tag=None):
+        super().__init__(tag)
+        self.pre_filtered, self.post_filtered, self.theta = pre_filtered, post_filtered, theta
+        self.delta, self.learning_rate = delta, learning_rate
+        self.reads, self.updates = [pre_filtered, post_filtered, theta], [delta]
+
+
+class SimOja(Operator):  # simulator.py:1355-1365: ... weights, delta, learning_rate, beta
+    def __init__(self, pre_filtered, post_filtered, weights, delta, learning_rate, beta, tag=None):
+        super().__init__(tag)
+        self.pre_filtered, self.post_filtered, self.weights = pre_filtered, post_filtered, weights
+        self.delta, self.learning_rate, self.beta = delta, learning_rate, beta
+        self.reads, self.updates = [pre_filtered, post_filtered, weights], [delta]
+
+
+class SimVoja(Operator):  # simulator.py:1367-1386: pre_decoded, post_filtered, scaled_encoders, ...
+    def __init__(self, pre_decoded, post_filtered, scaled_encoders, delta, scale, learning_signal,
+                 learning_rate, tag=None):
+        super().__init__(tag)
+        self.pre_decoded, self.post_filtered = pre_decoded, post_filtered
+        self.scaled_encoders, self.delta, self.scale = scaled_encoders, delta, scale
+        self.learning_signal, self.learning_rate = learning_signal, learning_rate
+        self.reads = [pre_decoded, post_filtered, scaled_encoders, learning_signal]
+        self.updates = [delta]
+
+
 class ElementwiseInc(Operator):  # simulator.py:871-875: op.A, op.X, op.Y
     def __init__(self, A, X, Y, tag=None):
         super().__init__(tag)
@@ -213,6 +240,41 @@ class AdaptiveLIF(LIF):  # clra_nonlinearities.py:1094-1132 through simulator.py
     def __init__(self, tau_n=1.0, inc_n=0.01, **kwargs):
         super().__init__(**kwargs)
         self.tau_n, self.inc_n = tau_n, inc_n
+
+
+class LIFRate:  # simulator.py:1065-1078: tau_rc, tau_ref, amplitude
+    def __init__(self, tau_rc=0.02, tau_ref=0.002, amplitude=1.0):
+        self.tau_rc, self.tau_ref, self.amplitude = tau_rc, tau_ref, amplitude
+
+
+class AdaptiveLIFRate(LIFRate):  # simulator.py:1102-1121: + tau_n, inc_n
+    def __init__(self, tau_n=1.0, inc_n=0.01, **kwargs):
+        super().__init__(**kwargs)
+        self.tau_n, self.inc_n = tau_n, inc_n
+
+
+class RectifiedLinear:  # simulator.py:1123-1130: amplitude
+    def __init__(self, amplitude=1.0):
+        self.amplitude = amplitude
+
+
+class SpikingRectifiedLinear(RectifiedLinear):  # simulator.py:1132-1142: amplitude, state voltage
+    pass
+
+
+class Sigmoid:  # simulator.py:1144-1151: tau_ref
+    def __init__(self, tau_ref=0.0025):
+        self.tau_ref = tau_ref
+
+
+class Gaussian:  # clra_nonlinearities.py:1486-1510 (get_dist_enums_params): mean, std
+    def __init__(self, mean, std):
+        self.mean, self.std = mean, std
+
+
+class Uniform:  # the same: low, high
+    def __init__(self, low, high):
+        self.low, self.high = low, high
 
 
 class Process:
@@ -321,6 +383,12 @@ class Model:
         return self.builder.build(self, obj, *args, **kwargs)
 
 
+class WhiteNoise(Process):  # simulator.py:1245-1258: dist, scale, seed
+    def __init__(self, dist=None, scale=True, seed=None):
+        self.dist = Gaussian(0.0, 1.0) if dist is None else dist
+        self.scale, self.seed = scale, seed
+
+
 def ss2tf(A, B, C, D):
     """nengo.utils.filter_design.ss2tf is scipy's routine of the same name."""
     from scipy.signal import ss2tf as scipy_ss2tf
@@ -339,7 +407,9 @@ def install(monkeypatch):
             "nengo.builder.operator", Operator=Operator, TimeUpdate=TimeUpdate, Reset=Reset,
             Copy=Copy, DotInc=DotInc, ElementwiseInc=ElementwiseInc, SimPyFunc=SimPyFunc,
             SparseDotInc=SparseDotInc),
-        "nengo.builder.learning_rules": _module("nengo.builder.learning_rules", SimPES=SimPES),
+        "nengo.builder.learning_rules": _module("nengo.builder.learning_rules", SimPES=SimPES,
+                                                SimBCM=SimBCM, SimOja=SimOja, SimVoja=SimVoja),
+        "nengo.dists": _module("nengo.dists", Gaussian=Gaussian, Uniform=Uniform),
         "nengo.transforms": _module("nengo.transforms", SparseMatrix=SparseMatrix),
         "nengo.builder.neurons": _module("nengo.builder.neurons", SimNeurons=SimNeurons),
         "nengo.builder.processes": _module("nengo.builder.processes", SimProcess=SimProcess),
@@ -347,9 +417,12 @@ def install(monkeypatch):
                                         SignalDict=SignalDict),
         "nengo.cache": _module("nengo.cache", get_default_decoder_cache=lambda: None),
         "nengo.exceptions": _module("nengo.exceptions", BuildError=BuildError),
-        "nengo.neurons": _module("nengo.neurons", LIF=LIF, AdaptiveLIF=AdaptiveLIF),
+        "nengo.neurons": _module("nengo.neurons", LIF=LIF, AdaptiveLIF=AdaptiveLIF, LIFRate=LIFRate,
+                                 AdaptiveLIFRate=AdaptiveLIFRate, RectifiedLinear=RectifiedLinear,
+                                 SpikingRectifiedLinear=SpikingRectifiedLinear, Sigmoid=Sigmoid),
         "nengo.synapses": _module("nengo.synapses", LinearFilter=LinearFilter, Lowpass=Lowpass),
-        "nengo.processes": _module("nengo.processes", Process=Process, WhiteSignal=WhiteSignal),
+        "nengo.processes": _module("nengo.processes", Process=Process, WhiteSignal=WhiteSignal,
+                                   WhiteNoise=WhiteNoise),
         "nengo.utils": _module("nengo.utils"),
         "nengo.utils.filter_design": _module("nengo.utils.filter_design", ss2tf=ss2tf),
     }
@@ -364,6 +437,10 @@ def install(monkeypatch):
         SimPyFunc=SimPyFunc, SimNeurons=SimNeurons, SimProcess=SimProcess, LIF=LIF,
         Lowpass=Lowpass, WhiteSignal=WhiteSignal, Model=Model, Builder=Builder,
         BuildError=BuildError, SparseDotInc=SparseDotInc, SimPES=SimPES, AdaptiveLIF=AdaptiveLIF,
+        SimBCM=SimBCM, SimOja=SimOja, SimVoja=SimVoja, LIFRate=LIFRate,
+        AdaptiveLIFRate=AdaptiveLIFRate, RectifiedLinear=RectifiedLinear,
+        SpikingRectifiedLinear=SpikingRectifiedLinear, Sigmoid=Sigmoid, WhiteNoise=WhiteNoise,
+        Gaussian=Gaussian, Uniform=Uniform,
         sparse_signal=lambda matrix, name=None: Signal(_as_sparse_matrix(matrix), name=name),
         family="nengo")
 

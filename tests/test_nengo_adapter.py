@@ -22,6 +22,10 @@ IR = types.SimpleNamespace(
     ElementwiseInc=ir.ElementwiseInc, SimPyFunc=ir.SimPyFunc, SimNeurons=ir.SimNeurons,
     SimProcess=ir.SimProcess, LIF=ir.LIF, Lowpass=ir.Lowpass, WhiteSignal=ir.WhiteSignal,
     Model=ir.Model, SparseDotInc=ir.SparseDotInc, SimPES=ir.SimPES, AdaptiveLIF=ir.AdaptiveLIF,
+    SimBCM=ir.SimBCM, SimOja=ir.SimOja, SimVoja=ir.SimVoja, LIFRate=ir.LIFRate,
+    AdaptiveLIFRate=ir.AdaptiveLIFRate, RectifiedLinear=ir.RectifiedLinear,
+    SpikingRectifiedLinear=ir.SpikingRectifiedLinear, Sigmoid=ir.Sigmoid,
+    WhiteNoise=ir.WhiteNoise, Gaussian=ir.Gaussian, Uniform=ir.Uniform,
     sparse_signal=lambda matrix, name=None: ir.SparseSignal(matrix, name=name), family="ir")
 
 
@@ -185,6 +189,121 @@ def emit_learning(model, net, F):
     return probes
 
 
+class RulesNetwork:
+    """What `emit_rules` turns into operators."""
+    seed = 9
+
+    def __init__(self, n_a=96, n=64, dims=4):
+        self.n_a, self.n, self.dims = n_a, n, dims
+
+
+def emit_rules(model, net, F):
+    """The operators nengo's builder emits for: a band-limited input into `a` (LIF); weight
+    matrices from a's neurons onto `b` (spiking rectified linear) and `c` (LIF rate) that BCM
+    and Oja learn; `e` (sigmoid) whose encoders Voja moves towards its input; `f` (rectified
+    linear) with white noise added to its input current and `g` (adaptive LIF rate), both
+    behind decoders of a.  `F` supplies the classes."""
+    rng = np.random.RandomState(31)
+    d, t, n = net.dims, model.time, net.n
+    probes = {}
+
+    def probe(name, sig, every=None):
+        p = ToyProbe(sample_every=every)
+        model.probes.append(p)
+        model.sig[p] = {"in": sig}
+        model.params[p] = []
+        probes[name] = p
+
+    def lowpass(x, tau, name):
+        y = F.Signal(np.zeros(x.shape), name=name)
+        model.add_op(F.SimProcess(F.Lowpass(tau), x, y, t, mode="update"))
+        return y
+
+    def ensemble(name, n_neurons, neurons, state_names, encoded=True, learned_encoders=False,
+                 drive=1.0):
+        x_in = F.Signal(np.zeros(d), name=name + ".in")
+        model.add_op(F.Reset(x_in))
+        bias = F.Signal(drive * rng.uniform(0.6, 1.8, size=n_neurons), name=name + ".bias",
+                        readonly=True)
+        J = F.Signal(np.zeros(n_neurons), name=name + ".J")
+        model.add_op(F.Copy(bias, J))
+        enc = None
+        if encoded:
+            enc = F.Signal(rng.normal(size=(n_neurons, d)) * (2.0 / np.sqrt(d)),
+                           name=name + ".encoders", readonly=not learned_encoders)
+            model.add_op(F.DotInc(enc, x_in, J))
+        out = F.Signal(np.zeros(n_neurons), name=name + ".out")
+        state = {k: F.Signal(np.zeros(n_neurons), name="%s.%s" % (name, k)) for k in state_names}
+        model.add_op(F.SimNeurons(neurons, J, out, state=state))
+        return x_in, J, out, enc
+
+    def decoded_into(out, n_from, target, name):
+        dec = F.Signal(rng.normal(size=(d, n_from)) / (40.0 * n_from), name=name + ".weights",
+                       readonly=True)
+        weighted = F.Signal(np.zeros(d), name=name + ".weighted")
+        model.add_op(F.Reset(weighted))
+        model.add_op(F.DotInc(dec, out, weighted))
+        model.add_op(F.Copy(lowpass(weighted, 0.005, name + ".filtered"), target, inc=True))
+
+    def weights_onto(out, n_from, J_to, n_to, name):
+        W = F.Signal(rng.normal(scale=2e-3, size=(n_to, n_from)), name=name + ".weights")
+        weighted = F.Signal(np.zeros(n_to), name=name + ".weighted")
+        model.add_op(F.Reset(weighted))
+        model.add_op(F.DotInc(W, out, weighted))
+        model.add_op(F.Copy(lowpass(weighted, 0.005, name + ".filtered"), J_to, inc=True))
+        return W
+
+    stim = F.Signal(np.zeros(d), name="stim.out")
+    model.add_op(F.SimProcess(F.WhiteSignal(0.3, high=8.0, seed=11), None, stim, t, mode="set"))
+    a_in, _, a_out, _ = ensemble("a", net.n_a, F.LIF(), ("voltage", "refractory_time"))
+    model.add_op(F.Copy(stim, a_in, inc=True))
+    a_filtered = lowpass(a_out, 0.005, "a.filtered")
+
+    # BCM on the weights a -> b, Oja on a -> c
+    # (a current of about 100: a spike every ten steps or so)
+    _, b_J, b_out, _ = ensemble("b", n, F.SpikingRectifiedLinear(), ("voltage",), encoded=False,
+                                drive=100.0)
+    W_ab = weights_onto(a_out, net.n_a, b_J, n, "ab")
+    b_filtered = lowpass(b_out, 0.005, "b.filtered")
+    theta = lowpass(b_out, 0.1, "b.theta")
+    d_ab = F.Signal(np.zeros((n, net.n_a)), name="ab.delta")
+    model.add_op(F.SimBCM(a_filtered, b_filtered, theta, d_ab, 2e-10))
+    model.add_op(F.Copy(d_ab, W_ab, inc=True))
+    _, c_J, c_out, _ = ensemble("c", n, F.LIFRate(), (), encoded=False)
+    W_ac = weights_onto(a_out, net.n_a, c_J, n, "ac")
+    c_filtered = lowpass(c_out, 0.005, "c.filtered")
+    d_ac = F.Signal(np.zeros((n, net.n_a)), name="ac.delta")
+    model.add_op(F.SimOja(a_filtered, c_filtered, W_ac, d_ac, 1e-8, 1.0))
+    model.add_op(F.Copy(d_ac, W_ac, inc=True))
+
+    # Voja on the encoders of e
+    e_in, _, e_out, e_enc = ensemble("e", n, F.Sigmoid(), (), learned_encoders=True)
+    decoded_into(a_out, net.n_a, e_in, "a_to_e")
+    learning = F.Signal(np.ones(1), name="voja.learning", readonly=True)
+    d_e = F.Signal(np.zeros((n, d)), name="voja.delta")
+    scale = rng.uniform(0.5, 2.0, size=n)
+    model.add_op(F.SimVoja(e_in, lowpass(e_out, 0.005, "e.filtered"), e_enc, d_e, scale, learning, 1e-4))
+    model.add_op(F.Copy(d_e, e_enc, inc=True))
+
+    # two more neuron types; white noise into the input current of one
+    f_in, f_J, f_out, _ = ensemble("f", n, F.RectifiedLinear(), ())
+    decoded_into(a_out, net.n_a, f_in, "a_to_f")
+    noise = F.Signal(np.zeros(n), name="f.noise")
+    model.add_op(F.SimProcess(F.WhiteNoise(F.Gaussian(0.0, 0.01), scale=True, seed=5), None, noise, t,
+                              mode="set"))
+    model.add_op(F.Copy(noise, f_J, inc=True))
+    g_in, _, g_out, _ = ensemble("g", n, F.AdaptiveLIFRate(tau_n=0.2, inc_n=0.05), ("adaptation",))
+    decoded_into(a_out, net.n_a, g_in, "a_to_g")
+
+    probe("b", b_out)
+    probe("c", c_filtered)
+    probe("e", e_out, every=0.004)
+    probe("f", f_out)
+    probe("g", g_out)
+    probe("W_ab", W_ab, every=0.05)
+    return probes
+
+
 def _install_family(monkeypatch):
     N = nengo_standin.install(monkeypatch)
     built = {}
@@ -192,6 +311,8 @@ def _install_family(monkeypatch):
         lambda model, network: built.__setitem__("toy", emit(model, network, N)))
     N.Builder.register(LearningNetwork)(
         lambda model, network: built.__setitem__("learning", emit_learning(model, network, N)))
+    N.Builder.register(RulesNetwork)(
+        lambda model, network: built.__setitem__("rules", emit_rules(model, network, N)))
     return N, built
 
 
@@ -218,8 +339,35 @@ def test_nengo_family_learning_graph_runs_like_the_ir_graph(monkeypatch):
             assert sim.data[built["learning"]["post_spikes"]].shape == (60, net.n_post)
 
 
+def test_nengo_family_rules_graph_runs_like_the_ir_graph(monkeypatch):
+    """BCM, Oja and Voja, rate and rectified-linear neuron types and a white-noise process out
+    of nengo-family classes: the same numbers as the same graph in `ir` classes."""
+    N, built = _install_family(monkeypatch)
+    net = RulesNetwork()
+    with OracleSimulator(net, dt=0.001) as sim:
+        kinds = {type(op).__name__ for op in sim.model.operators}
+        assert {"SimBCM", "SimOja", "SimVoja", "SimNeurons", "SimProcess"} <= kinds
+        assert all(type(op).__module__.startswith("nengo.") for op in sim.model.operators)
+        assert {type(op.neurons).__name__ for op in sim.model.operators
+                if type(op).__name__ == "SimNeurons"} == {
+            "LIF", "SpikingRectifiedLinear", "LIFRate", "Sigmoid", "RectifiedLinear", "AdaptiveLIFRate"}
+        ref_model = ir.Model(dt=0.001)
+        ref_probes = emit_rules(ref_model, net, IR)
+        with OracleSimulator(None, model=ref_model, seed=net.seed + 1) as ref:
+            assert [p.name for p in sim._plans] == [p.name for p in ref._plans]
+            sim.run_steps(300)
+            ref.run_steps(300)
+            for key in ref_probes:
+                got, want = sim.data[built["rules"][key]], ref.data[ref_probes[key]]
+                assert got.shape == want.shape and np.any(want != 0), key
+                assert np.array_equal(got, want), (key, np.abs(got - want).max())
+            assert_same_signals(sim, ref)
+            w = sim.data[built["rules"]["W_ab"]]
+            assert np.any(w[-1] != w[0])  # the rule changed the weights
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("which", ["toy", "learning"])
+@pytest.mark.parametrize("which", ["toy", "learning", "rules"])
 def test_nengo_family_graphs_on_the_device(monkeypatch, which):
     """`Simulator(network)` on the HIP backend for graphs made of nengo-family classes: the
     class-name keyed choices (spiking populations -> launches that visit active columns and
@@ -233,8 +381,10 @@ def test_nengo_family_graphs_on_the_device(monkeypatch, which):
         # (np.sin itself: both sides round the double-precision sine once, where a traced
         # function is evaluated in float32 on the device and agrees to a tolerance only)
         net = ToyNetwork(n_neurons=1024, dims=32, fn=np.sin)
-    else:
+    elif which == "learning":
         net = LearningNetwork(n_pre=1024, n_post=512, n_err=512, dims=32)
+    else:
+        net = RulesNetwork(n_a=1024, n=512, dims=16)
     with Simulator(net, dt=0.001) as gpu:
         gpu_probes = built[which]
         assert type(gpu.model) is N.Model
@@ -243,14 +393,17 @@ def test_nengo_family_graphs_on_the_device(monkeypatch, which):
         print(which, "plans per step:", names)
         with OracleSimulator(net, dt=0.001) as cpu:
             cpu_probes = built[which]
-            assert any(n in ("hipra_gemv.tile_lif", "hipra_gemv.rows_lif") or
-                       n.startswith("hipra_gemv.tile_lif") for n in names), names
+            if which != "rules":  # (six neuron types in one step: no launch holds them all)
+                assert any(n in ("hipra_gemv.tile_lif", "hipra_gemv.rows_lif") or
+                           n.startswith("hipra_gemv.tile_lif") for n in names), names
             assert any(n.startswith(("hipra_gemv.events_filter", "hipra_gemv.tile_filter",
                                      "hipra_gemv.rows_filter")) for n in names), names
             if which == "toy":
                 assert any(getattr(p, "event_driven", False) for p in gpu._plans), names
-            else:
+            elif which == "learning":
                 assert any(hasattr(p, "spmv") for p in gpu._plans), names
+            else:
+                assert {"hip_bcm", "hip_oja", "hip_voja", "hip_whitenoise"} <= set(names), names
             gpu.run_steps(300)
             cpu.run_steps(300)
             for key in cpu_probes:
