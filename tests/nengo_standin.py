@@ -194,6 +194,38 @@ class SimVoja(Operator):  # simulator.py:1367-1386: pre_decoded, post_filtered, 
         self.updates = [delta]
 
 
+class ChannelShape:  # nengo.transforms.ChannelShape as simulator.py:1290-1332 reads it
+    def __init__(self, shape, channels_last=True):
+        self.shape, self.channels_last = tuple(shape), channels_last
+        self.spatial_shape = self.shape[:-1] if channels_last else self.shape[1:]
+        self.n_channels = self.shape[-1] if channels_last else self.shape[0]
+        self.size = int(np.prod(self.shape))
+        self.dimensions = len(self.spatial_shape)
+
+
+class Convolution:  # nengo.transforms.Convolution: the `conv` of a ConvInc (simulator.py:1290-1332)
+    def __init__(self, n_filters, input_shape, kernel_size=(3, 3), strides=(1, 1), padding="valid",
+                 channels_last=True):
+        self.n_filters, self.kernel_size, self.strides = n_filters, tuple(kernel_size), tuple(strides)
+        self.padding, self.channels_last = padding, channels_last
+        self.input_shape = ChannelShape(input_shape, channels_last)
+        self.dimensions = len(self.kernel_size)
+        spatial = self.input_shape.spatial_shape
+        if padding == "same":
+            out = [-(-n // s) for n, s in zip(spatial, self.strides)]
+        else:
+            out = [(n - k) // s + 1 for n, k, s in zip(spatial, self.kernel_size, self.strides)]
+        shape = tuple(out) + (n_filters,) if channels_last else (n_filters,) + tuple(out)
+        self.output_shape = ChannelShape(shape, channels_last)
+
+
+class ConvInc(Operator):  # simulator.py:1290-1332: op.W, op.X, op.Y, op.conv
+    def __init__(self, W, X, Y, conv, tag=None):
+        super().__init__(tag)
+        self.W, self.X, self.Y, self.conv = W, X, Y, conv
+        self.reads, self.incs = [W, X], [Y]
+
+
 class ElementwiseInc(Operator):  # simulator.py:871-875: op.A, op.X, op.Y
     def __init__(self, A, X, Y, tag=None):
         super().__init__(tag)
@@ -410,7 +442,9 @@ def install(monkeypatch):
         "nengo.builder.learning_rules": _module("nengo.builder.learning_rules", SimPES=SimPES,
                                                 SimBCM=SimBCM, SimOja=SimOja, SimVoja=SimVoja),
         "nengo.dists": _module("nengo.dists", Gaussian=Gaussian, Uniform=Uniform),
-        "nengo.transforms": _module("nengo.transforms", SparseMatrix=SparseMatrix),
+        "nengo.transforms": _module("nengo.transforms", SparseMatrix=SparseMatrix,
+                                    Convolution=Convolution, ChannelShape=ChannelShape),
+        "nengo.builder.transforms": _module("nengo.builder.transforms", ConvInc=ConvInc),
         "nengo.builder.neurons": _module("nengo.builder.neurons", SimNeurons=SimNeurons),
         "nengo.builder.processes": _module("nengo.builder.processes", SimProcess=SimProcess),
         "nengo.builder.signal": _module("nengo.builder.signal", Signal=Signal,
@@ -440,7 +474,7 @@ def install(monkeypatch):
         SimBCM=SimBCM, SimOja=SimOja, SimVoja=SimVoja, LIFRate=LIFRate,
         AdaptiveLIFRate=AdaptiveLIFRate, RectifiedLinear=RectifiedLinear,
         SpikingRectifiedLinear=SpikingRectifiedLinear, Sigmoid=Sigmoid, WhiteNoise=WhiteNoise,
-        Gaussian=Gaussian, Uniform=Uniform,
+        Gaussian=Gaussian, Uniform=Uniform, ConvInc=ConvInc, conv_spec=Convolution,
         sparse_signal=lambda matrix, name=None: Signal(_as_sparse_matrix(matrix), name=name),
         family="nengo")
 

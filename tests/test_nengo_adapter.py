@@ -25,7 +25,8 @@ IR = types.SimpleNamespace(
     SimBCM=ir.SimBCM, SimOja=ir.SimOja, SimVoja=ir.SimVoja, LIFRate=ir.LIFRate,
     AdaptiveLIFRate=ir.AdaptiveLIFRate, RectifiedLinear=ir.RectifiedLinear,
     SpikingRectifiedLinear=ir.SpikingRectifiedLinear, Sigmoid=ir.Sigmoid,
-    WhiteNoise=ir.WhiteNoise, Gaussian=ir.Gaussian, Uniform=ir.Uniform,
+    WhiteNoise=ir.WhiteNoise, Gaussian=ir.Gaussian, Uniform=ir.Uniform, ConvInc=ir.ConvInc,
+    conv_spec=ir.ConvSpec,
     sparse_signal=lambda matrix, name=None: ir.SparseSignal(matrix, name=name), family="ir")
 
 
@@ -295,7 +296,19 @@ def emit_rules(model, net, F):
     g_in, _, g_out, _ = ensemble("g", n, F.AdaptiveLIFRate(tau_n=0.2, inc_n=0.05), ("adaptation",))
     decoded_into(a_out, net.n_a, g_in, "a_to_g")
 
+    # a convolution of a constant image drives rectified-linear units, one per output pixel
+    conv = F.conv_spec(3, (6, 6, 2), kernel_size=(3, 3), strides=(1, 1), padding="valid",
+                       channels_last=True)
+    image = F.Signal(rng.uniform(size=6 * 6 * 2), name="image", readonly=True)
+    kernels = F.Signal(0.3 * rng.normal(size=(3, 3, 2, 3)), name="conv.weights", readonly=True)
+    conv_out = F.Signal(np.zeros(conv.output_shape.size), name="conv.out")
+    model.add_op(F.Reset(conv_out))
+    model.add_op(F.ConvInc(kernels, image, conv_out, conv))
+    _, h_J, h_out, _ = ensemble("h", conv.output_shape.size, F.RectifiedLinear(), (), encoded=False)
+    model.add_op(F.Copy(conv_out, h_J, inc=True))
+
     probe("b", b_out)
+    probe("h", h_out)
     probe("c", c_filtered)
     probe("e", e_out, every=0.004)
     probe("f", f_out)
@@ -346,7 +359,7 @@ def test_nengo_family_rules_graph_runs_like_the_ir_graph(monkeypatch):
     net = RulesNetwork()
     with OracleSimulator(net, dt=0.001) as sim:
         kinds = {type(op).__name__ for op in sim.model.operators}
-        assert {"SimBCM", "SimOja", "SimVoja", "SimNeurons", "SimProcess"} <= kinds
+        assert {"SimBCM", "SimOja", "SimVoja", "SimNeurons", "SimProcess", "ConvInc"} <= kinds
         assert all(type(op).__module__.startswith("nengo.") for op in sim.model.operators)
         assert {type(op.neurons).__name__ for op in sim.model.operators
                 if type(op).__name__ == "SimNeurons"} == {
@@ -403,7 +416,7 @@ def test_nengo_family_graphs_on_the_device(monkeypatch, which):
             elif which == "learning":
                 assert any(hasattr(p, "spmv") for p in gpu._plans), names
             else:
-                assert {"hip_bcm", "hip_oja", "hip_voja", "hip_whitenoise"} <= set(names), names
+                assert {"hip_bcm", "hip_oja", "hip_voja", "hip_whitenoise", "hip_conv2d"} <= set(names), names
             gpu.run_steps(300)
             cpu.run_steps(300)
             for key in cpu_probes:
