@@ -421,6 +421,11 @@ class WhiteNoise(Process):  # simulator.py:1245-1258: dist, scale, seed
         self.scale, self.seed = scale, seed
 
 
+class PresentInput(Process):  # simulator.py:1279-1288: inputs, presentation_time
+    def __init__(self, inputs, presentation_time):
+        self.inputs, self.presentation_time = np.asarray(inputs), presentation_time
+
+
 def ss2tf(A, B, C, D):
     """nengo.utils.filter_design.ss2tf is scipy's routine of the same name."""
     from scipy.signal import ss2tf as scipy_ss2tf
@@ -456,7 +461,7 @@ def install(monkeypatch):
                                  SpikingRectifiedLinear=SpikingRectifiedLinear, Sigmoid=Sigmoid),
         "nengo.synapses": _module("nengo.synapses", LinearFilter=LinearFilter, Lowpass=Lowpass),
         "nengo.processes": _module("nengo.processes", Process=Process, WhiteSignal=WhiteSignal,
-                                   WhiteNoise=WhiteNoise),
+                                   WhiteNoise=WhiteNoise, PresentInput=PresentInput),
         "nengo.utils": _module("nengo.utils"),
         "nengo.utils.filter_design": _module("nengo.utils.filter_design", ss2tf=ss2tf),
     }
@@ -475,6 +480,7 @@ def install(monkeypatch):
         AdaptiveLIFRate=AdaptiveLIFRate, RectifiedLinear=RectifiedLinear,
         SpikingRectifiedLinear=SpikingRectifiedLinear, Sigmoid=Sigmoid, WhiteNoise=WhiteNoise,
         Gaussian=Gaussian, Uniform=Uniform, ConvInc=ConvInc, conv_spec=Convolution,
+        PresentInput=PresentInput,
         sparse_signal=lambda matrix, name=None: Signal(_as_sparse_matrix(matrix), name=name),
         family="nengo")
 

@@ -26,7 +26,7 @@ IR = types.SimpleNamespace(
     AdaptiveLIFRate=ir.AdaptiveLIFRate, RectifiedLinear=ir.RectifiedLinear,
     SpikingRectifiedLinear=ir.SpikingRectifiedLinear, Sigmoid=ir.Sigmoid,
     WhiteNoise=ir.WhiteNoise, Gaussian=ir.Gaussian, Uniform=ir.Uniform, ConvInc=ir.ConvInc,
-    conv_spec=ir.ConvSpec,
+    conv_spec=ir.ConvSpec, PresentInput=ir.PresentInput,
     sparse_signal=lambda matrix, name=None: ir.SparseSignal(matrix, name=name), family="ir")
 
 
@@ -259,6 +259,11 @@ def emit_rules(model, net, F):
     a_in, _, a_out, _ = ensemble("a", net.n_a, F.LIF(), ("voltage", "refractory_time"))
     model.add_op(F.Copy(stim, a_in, inc=True))
     a_filtered = lowpass(a_out, 0.005, "a.filtered")
+    # a second input: five vectors shown for 20 ms each, in turn
+    shown = F.Signal(np.zeros(d), name="shown.out")
+    model.add_op(F.SimProcess(F.PresentInput(0.5 * rng.normal(size=(5, d)), 0.02), None, shown, t,
+                              mode="set"))
+    model.add_op(F.Copy(shown, a_in, inc=True))
 
     # BCM on the weights a -> b, Oja on a -> c
     # (a current of about 100: a spike every ten steps or so)
@@ -417,6 +422,8 @@ def test_nengo_family_graphs_on_the_device(monkeypatch, which):
                 assert any(hasattr(p, "spmv") for p in gpu._plans), names
             else:
                 assert {"hip_bcm", "hip_oja", "hip_voja", "hip_whitenoise", "hip_conv2d"} <= set(names), names
+                flat = " ".join(str(p) for p in gpu._plans)
+                assert "presentinput" in flat, flat  # (rides in a sequence launch)
             gpu.run_steps(300)
             cpu.run_steps(300)
             for key in cpu_probes:
