@@ -618,7 +618,12 @@ def main():
             cols -= cols % 8
             if n_rows >= 128 and cols >= 8:
                 # (input currents that only the launch's own epilogue reads are not stored)
+                # and spikes that only launches visiting active columns read leave as a bit each
                 n_writes = 3 if getattr(lif, "lazy_currents", None) else 4
+                import numpy as np
+                flags = np.asarray(lif.host_pops)[:, 7]
+                if np.any(flags & 0x100) and np.array_equal((flags & 0x800) != 0, (flags & 0x100) != 0):
+                    n_writes -= 1
                 floor = traffic_floor(sim.queue, n_rows, cols, n_writes=n_writes)
                 best = min(floor["us"], floor["nontemporal_stores_us"])
                 roofline["plain_kernel_same_traffic"] = dict(

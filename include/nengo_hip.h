@@ -152,7 +152,11 @@ int nhip_gemv_tile_rows(int n_cols, int blk_words);
  * -expm1(-dt / tau) formed as the kernel would (float quotient, expm1 in double,
  * rounded once to float), allowed when tau is a scalar and upsample == 1: the
  * launch then evaluates transcendental functions only for the few neurons that
- * leave their refractory period or spike in this step).
+ * leave their refractory period or spike in this step; bit 11, with bit 9, scalar amp,
+ * s_start even and every task of the item starting at a multiple of 32 rows: the launch
+ * leaves the spikes as one BIT per neuron -- bit r % 64 of the 64-bit word r / 64 at
+ * S + s_start, set where neuron r spiked -- and writes no float of S for the item; for
+ * spikes that only nhip_gemv_events reads, see its `x_bits`).
  * Y is still written.  V, W, S must not overlap anything the launch reads through
  * A, X or Yin; dt, upsample as for nhip_lif.  Results are bit-identical to the two
  * separate calls. */
@@ -312,10 +316,13 @@ int nhip_spmv_sell(void *stream, const int *slices, int n_slices, const int *row
  * aside) -- and reading only those columns of A.  For that the matrices are handed over
  * transposed, in a buffer of their own:
  *   items : int32[n_items][16] {at_start, mp, M, N, x_start, y_start, y_stride0, yin_start,
- *           yin_stride0, bits of alpha, beta, gamma, first_target, n_targets, row0, 0}
+ *           yin_stride0, bits of alpha, beta, gamma, first_target, n_targets, row0, x_bits}
  *           a record stands for rows row0 .. row0 + M - 1 (M <= 64) of a matrix whose
  *           column c is AT[at_start + c * mp + row]; y_start / yin_start are those of the
- *           matrix's row 0; a matrix of more than 64 rows is several records
+ *           matrix's row 0; a matrix of more than 64 rows is several records; x_bits != 0:
+ *           X + x_start (x_start even) holds one bit per column in 64-bit words, as
+ *           nhip_gemv_tile_lif leaves them with bit 11 of pflags, and x_bits is the float
+ *           bits of the value a set bit stands for (a clear bit: zero)
  *   AT    : the transposed matrices; X, Yin, Y: the buffers the offsets refer to
  *   targets, F : first-order filters stepped on the fresh y, as for nhip_gemv_tile_filter
  *           (both NULL: none); an item's range of targets is in its record

@@ -56,7 +56,11 @@ struct EvItem {  // 16 words
     float alpha, beta, gamma;
     int first_target, n_targets;  // filters fed by y (none: 0, 0)
     int row0;          // first row of this record in its item (items of more than 64 rows
-    int pad1;          // are several records; at_start is that of row 0)
+                       // are several records; at_start is that of row 0)
+    int x_bits;        // 0: X holds a float per column.  Else the bits of the one value a
+                       // column's x can have besides zero, and X + x_start holds one BIT per
+                       // column (64-bit words, x_start even): what the large-item launch leaves
+                       // of a population's spikes under LIF_POP_BITS
 };
 static_assert(sizeof(EvItem) == 64, "item records are 16 words");
 
@@ -132,6 +136,35 @@ __global__ __launch_bounds__(EV_WG) __attribute__((amdgpu_waves_per_eu(8, 8))) v
 
         // the columns of this wave's range whose x is not zero, in column order
         int count = 0;
+        if (it.x_bits != 0) {  // (the same for the whole group) a bit per column
+            const unsigned long long* words =
+                reinterpret_cast<const unsigned long long*>(X + it.x_start);
+            const float x_set = nhip_bits(it.x_bits);
+            static_assert(EV_LIST_LOADS * 16 == NHIP_WAVE, "sixteen lanes fetch each word");
+            for (int c0 = c_lo; c0 < c_hi; c0 += EV_LIST_LOADS * NHIP_WAVE) {  // (once)
+                // one load for the words of the whole range: lanes 16 u .. 16 u + 15 fetch
+                // the word of columns c0 + 64 u ...
+                const int c_mine = c0 + (lane >> 4) * NHIP_WAVE;
+                const uint2 mine = c_mine < c_hi
+                    ? *reinterpret_cast<const uint2*>(words + ((base + c_mine) >> 6))
+                    : make_uint2(0u, 0u);
+#pragma unroll
+                for (int u = 0; u < EV_LIST_LOADS; ++u) {
+                    const int c = c0 + u * NHIP_WAVE;
+                    unsigned long long b =
+                        (unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)mine.x, 16 * u) |
+                        ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)mine.y, 16 * u) << 32);
+                    if (c < c_hi && c_hi - c < NHIP_WAVE) b &= (1ull << (c_hi - c)) - 1ull;
+                    const int before = __builtin_amdgcn_mbcnt_hi(
+                        (unsigned)(b >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b, 0));
+                    if ((b >> lane) & 1ull) {
+                        col[count + before] = c + lane;
+                        xs[count + before] = x_set;
+                    }
+                    count += __popcll(b);
+                }
+            }
+        } else
         for (int c0 = c_lo; c0 < c_hi; c0 += EV_LIST_LOADS * NHIP_WAVE) {  // (once)
             float xv[EV_LIST_LOADS];
 #pragma unroll

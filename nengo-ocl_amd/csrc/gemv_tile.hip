@@ -454,6 +454,21 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
         }
     }
     wave_sync();
+    const bool as_bits = p.pflags & LIF_POP_BITS;  // uniform
+    if (as_bits) {
+        // one bit per neuron: the 64 rows of a slot are two 32-bit words (row0 is a multiple
+        // of 32, and so is the number of rows of every task but the item's last: a word
+        // belongs to one task)
+        unsigned* words = reinterpret_cast<unsigned*>(a.S + (size_t)p.s_start);
+#pragma unroll
+        for (int k = 0; k < SLOTS; ++k) {
+            if (k * NHIP_WAVE >= n_rows) break;  // uniform
+            const int r = k * NHIP_WAVE + lane;
+            const unsigned long long m = __ballot(r < n_rows && new_s[r] != 0.0f);
+            if (lane < 2 && k * NHIP_WAVE + 32 * lane < n_rows)
+                words[((row0 + k * NHIP_WAVE) >> 5) + lane] = (unsigned)(lane ? m >> 32 : m);
+        }
+    }
     // whole rows of four neurons per lane where the task's part of the state arrays is made
     // of aligned quads (16-byte stores: a quarter of the store instructions)
     if (((p.v_start | p.w_start | p.s_start | row0 | n_rows) & 3) == 0) {  // uniform
@@ -462,8 +477,9 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
                 *reinterpret_cast<const float4*>(new_v + r);
             *reinterpret_cast<float4*>(a.W + (size_t)p.w_start + row0 + r) =
                 *reinterpret_cast<const float4*>(new_w + r);
-            *reinterpret_cast<float4*>(a.S + (size_t)p.s_start + row0 + r) =
-                *reinterpret_cast<const float4*>(new_s + r);
+            if (!as_bits)
+                *reinterpret_cast<float4*>(a.S + (size_t)p.s_start + row0 + r) =
+                    *reinterpret_cast<const float4*>(new_s + r);
         }
         return;
     }
@@ -473,7 +489,7 @@ __device__ __forceinline__ void lif_task_compacted(const LifArgs& a, const LifPo
         if (r < n_rows) {
             a.V[(size_t)p.v_start + row0 + r] = new_v[r];
             a.W[(size_t)p.w_start + row0 + r] = new_w[r];
-            a.S[(size_t)p.s_start + row0 + r] = new_s[r];
+            if (!as_bits) a.S[(size_t)p.s_start + row0 + r] = new_s[r];
         }
     }
 }

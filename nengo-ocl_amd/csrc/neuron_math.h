@@ -17,6 +17,12 @@ constexpr int LIF_POP_DECAY = 1 << 9;    // pflags: `decay` is set (one tau, ups
 // pflags: nothing but this epilogue reads the population's input current (the host's word),
 // so the launch does not store it; the host recomputes it when somebody asks
 constexpr int LIF_POP_NO_J = 1 << 10;
+// pflags: nothing but launches that visit active columns reads the population's spikes (the
+// host's word), so the large-item launch stores them as one bit per neuron -- a 64-bit word
+// per 64 neurons, in the first words of the signal's own memory (s_start even, the rows of
+// every task starting at a multiple of 64) -- instead of a float each: a sixteenth of a
+// percent of the bytes, and writes next to a read stream cost about three times theirs
+constexpr int LIF_POP_BITS = 1 << 11;
 
 // State arrays and constants of a fused LIF update (all populations of a launch).
 struct LifArgs {

@@ -96,6 +96,7 @@ WAVE_TASKS = os.environ.get("NENGO_HIP_WAVE_TASKS", "1") != "0"
 WG, WAVE = 256, 64
 THIN_MIN_ROWS, THIN_ROWS_FOR_LANE_PER_ROW = 32, 65536
 LIF_POP_ENABLED, LIF_POP_DECAY, LIF_POP_NO_J = 1 << 8, 1 << 9, 1 << 10  # flag bits of a population row
+LIF_POP_BITS = 1 << 11  # spikes stored as a bit per neuron (see `store_spikes_as_bits`)
 LIF_COMPACT = os.environ.get("NENGO_HIP_LIF_COMPACT", "1") != "0"
 
 
@@ -449,6 +450,7 @@ class gemv_prog:
         plan.prog = self
         plan.host_tasks = None
         plan.event_table = table
+        plan.dev_event_table = dev_items
         plan.event_record_item = np.array(record_item, dtype=np.int64)  # Y item of each record
         plan.event_driven = True  # reads only the columns of A whose x is not zero
         return plan
@@ -977,6 +979,7 @@ def fuse_lif(prog, lif_plan, unread_currents=()):
         fused.members, fused.prog = plan.members, prog
         fused.gemv_bytes = plan.bw_per_call - unstored
         fused.host_pops = table
+        fused.dev_pops = dev_pops
         fused.lif_written = [V, W, S]
         fused.lazy_currents = lazy_currents
         if plan.kernel_class[0] == 3:
@@ -1162,12 +1165,48 @@ def fuse_input_sums(sum_plan, lif_plan):
     fused.input_sums = len(sums)
     fused.lazy_currents = getattr(lif_plan, "lazy_currents", None)
     fused.host_pops = new_pops if large else pops
+    # (the device copy of the table, where it is the one the launch reads: large items)
+    fused.dev_pops = (dev_pops if spare else getattr(lif_plan, "dev_pops", None)) if large else None
     return fused
 
 
 def _learning_apart(which):
     logger.debug("fuse_learning: check %d did not hold", which)
     return None
+
+
+def store_spikes_as_bits(enc_plan, items, event_records, dt):
+    """Populations of a `tile_lif` launch whose spikes only launches that visit active columns
+    read: the launch leaves one bit per neuron in the first words of the spike signal's memory
+    instead of a float per neuron (`LIF_POP_BITS`), and the records of the reading launches say
+    so (their `x_bits` word: the one value a spike has, amplitude / dt rounded as the neuron
+    update rounds it).  `items`: rows of the launch's population table; `event_records`:
+    ``{item: [(event plan, record index), ...]}``.  Returns ``{item: spike value}``.  The
+    caller has checked that nothing else reads those spikes."""
+    pops = enc_plan.host_pops
+    dt_inv = np.float32(1.0 / dt)
+    values = {}
+    touched = []
+    for b in items:
+        amp = np.array([pops[b, 6]], dtype=np.int32).view(np.float32)[0]
+        value = np.float32(amp * dt_inv)  # (__fmul_rn of two floats)
+        if not np.isfinite(value) or value == 0:
+            continue
+        pops[b, 7] |= LIF_POP_BITS
+        values[b] = value
+        for plan, k in event_records[b]:
+            plan.event_table[k, 15] = int(np.array([value], dtype=np.float32).view(np.int32)[0])
+            if plan not in touched:
+                touched.append(plan)
+        n = int(sum(int(row[2]) for row in enc_plan.host_tasks if row[0] == b))
+        if enc_plan.bw_per_call:
+            enc_plan.bw_per_call -= 4 * n - n // 8
+    if values:
+        enc_plan.dev_pops.set(pops.astype(np.int32).ravel())
+        for plan in touched:
+            plan.dev_event_table.set(plan.event_table.astype(np.int32).ravel())
+        enc_plan.tag = "%s + spikes as bits" % enc_plan.tag
+    return values
 
 
 def fuse_learning(enc_plan, dec_plan, ew_plan, lf_plan):
@@ -1294,7 +1333,8 @@ def fuse_learning(enc_plan, dec_plan, ew_plan, lf_plan):
                    flops_per_call=enc_plan.flops_per_call)
     for new, old in ((new_dec, dec_plan), (new_enc, enc_plan)):
         for attr in ("description", "kernel_class", "n_tasks", "members", "prog", "gemv_bytes",
-                     "host_tasks", "host_pops", "lif_written", "lazy_currents", "input_sums"):
+                     "host_tasks", "host_pops", "dev_pops", "lif_written", "lazy_currents",
+                     "input_sums"):
             if hasattr(old, attr):
                 setattr(new, attr, getattr(old, attr))
     new_dec.learned_matrices = len(learn_of_item)
@@ -1417,6 +1457,7 @@ def fuse_linearfilter(gemv_plans, lf_plan):
             fused.members, fused.prog = plan.members, prog
             fused.gemv_bytes = plan.bw_per_call
             fused.event_table, fused.event_driven = table, True
+            fused.dev_event_table = dev_table
             fused.event_record_item = plan.event_record_item
             fused.host_tasks = None
             out.append(fused)

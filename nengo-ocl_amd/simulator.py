@@ -74,6 +74,8 @@ class HipBackend:
         self._gemv = hipra_gemv
         # switch for measurements: "0" stores every input current
         self.skip_unread_currents = os.environ.get("NENGO_HIP_SKIP_CURRENTS", "1") != "0"
+        # spikes that only launches visiting active columns read: a bit per neuron
+        self.spikes_as_bits = os.environ.get("NENGO_HIP_SPIKE_BITS", "1") != "0"
         # switch for measurements: False keeps input sums a launch of their own
         self.input_sums_in_launch = os.environ.get("NENGO_HIP_INPUT_SUMS", "1") != "0"
         from . import hipra_sequence
@@ -102,6 +104,9 @@ class HipBackend:
         if self.input_sums_in_launch and hasattr(sum_plan, "prog") and hasattr(lif_plan, "prog"):
             return self._gemv.fuse_input_sums(sum_plan, lif_plan)
         return None
+
+    def store_spikes_as_bits(self, enc_plan, items, event_records, dt):
+        return self._gemv.store_spikes_as_bits(enc_plan, items, event_records, dt)
 
     def fuse_gemv_neurons(self, gemv_plans, neuron_plans, unread_currents=()):
         """Plans replacing ``gemv_plans + neuron_plans`` by launches that update the
@@ -268,10 +273,12 @@ class Simulator:
     cut out) raise ``ValueError`` when read instead of returning stale memory; writes to a
     learned matrix updated in place, to a signal that merged connections share or to a
     constant with a second device copy raise ``ValueError`` naming the constructor switch
-    that makes them possible.  ``reference_host_state=True`` switches ``learn_in_place``,
+    that makes them possible; spikes that only launches visiting active columns read are kept
+    as one bit per neuron (`_store_spikes_as_bits`): reads give the reference's floats,
+    writes raise ``ValueError``.  ``reference_host_state=True`` switches ``learn_in_place``,
     ``dedup``, the rewrites that move writes (``products_write_their_target``,
-    ``propagate_vector_copies``) and the second copies of constants off in one go: every
-    signal is then readable and writable as in the reference.
+    ``propagate_vector_copies``), the second copies of constants and the spike bits off in
+    one go: every signal is then readable and writable as in the reference.
 
     ``event_calibration_steps`` (default 32, 0 = off): products of a constant matrix with
     spikes visit only the columns of the neurons that spiked, which pays while few neurons
@@ -506,6 +513,7 @@ class Simulator:
             plans = self.backend.merge_small_plans(plans)
             if fuse and hasattr(self.backend, "carry_sequences"):
                 plans = self.backend.carry_sequences(plans)
+        self._store_spikes_as_bits(plans)
         logger.info("Plans in %0.3f s", _time.time() - t0)
 
         self._plans = Plans(plans, self.profiling, use_graph=use_graph, branches=branches,
@@ -549,7 +557,7 @@ class Simulator:
         for _ in range(0, n_steps, quarter):
             self.run_steps(quarter)
             for base in sources:
-                spikes = np.asarray(self.all_data[self.sidx[base]])
+                spikes = np.asarray(self.signals[base])
                 sources[base] = max(sources[base], float(np.count_nonzero(spikes)) / spikes.size)
         self.reset()
         for plan in plans:  # (the run leaves no trace in the profiling table either)
@@ -666,6 +674,88 @@ class Simulator:
         self._host_view_plan = plan
         plan()  # nothing has run yet: the copy holds the initial values
         return [plan]
+
+    def _store_spikes_as_bits(self, plans):
+        """Spike signals that nothing but launches visiting active columns reads -- no other
+        launch, no probe, no host copy; written by one large-item neuron launch in tasks that
+        start at multiples of 32 rows; one amplitude per population; zero at the start -- are
+        kept as one bit per neuron in the first words of their own memory
+        (`hipra_gemv.store_spikes_as_bits`): `_spike_bits` maps such a base to
+        (start, neurons, value of a spike).  The host reads them through `_spikes_from_bits`
+        and may not write them."""
+        self._spike_bits = {}
+        if self.reference_host_state or not getattr(self.backend, "spikes_as_bits", False):
+            return
+        encs = [p for p in plans if getattr(p, "name", "") == "hipra_gemv.tile_lif"
+                and getattr(p, "dev_pops", None) is not None
+                and getattr(p, "host_tasks", None) is not None]
+        events = [p for p in plans if getattr(p, "dev_event_table", None) is not None]
+        if not encs or not events:
+            return
+        ra = self.all_data
+        base_at = {int(ra.starts[self.sidx[b]]): b for b in self.all_bases}
+        records = defaultdict(list)  # (x_start, columns) -> [(plan, record)]
+        for q in events:
+            for k, row in enumerate(q.event_table):
+                records[(int(row[4]), int(row[3]))].append((q, k))
+        for enc in encs:
+            pops, tasks = enc.host_pops, enc.host_tasks
+            items, hits = [], {}
+            for b in sorted({int(t) for t in tasks[:, 0]}):
+                if b >= len(pops):
+                    continue
+                flags, start = int(pops[b, 7]), int(pops[b, 2])
+                if (flags & 0x304) != 0x300 or start % 2:  # a population, one decay, one amplitude
+                    continue
+                mine = tasks[tasks[:, 0] == b]
+                n = int(mine[:, 2].sum())
+                base = base_at.get(start)
+                checks = (base is not None and int(base.size) == n, (start, n) in records,
+                          not np.any(mine[:, 1] % 32),
+                          not np.any(self._initial_buf[start:start + n]),
+                          base not in self._host_view_index, base not in enc.reads_mem)
+                if not all(checks):
+                    logger.debug("spikes of item %d stay floats: %s", b, checks)
+                    continue
+                ok = True
+                for q in plans:
+                    carried = getattr(q, "carried", None)
+                    if carried is not None and base in getattr(carried, "reads_mem", {base}):
+                        ok = False
+                    if q is enc:
+                        continue
+                    if base in getattr(q, "writes_mem", {base}):
+                        ok = False
+                    if base in getattr(q, "reads_mem", {base}):
+                        if q not in events:
+                            ok = False
+                        else:  # every record of that launch that reads the span reads all of it
+                            for row in q.event_table:
+                                a, m = int(row[4]), int(row[3])
+                                if a < start + n and start < a + m and (a, m) != (start, n):
+                                    ok = False
+                if ok:
+                    items.append(b)
+                    hits[b] = records[(start, n)]
+                else:
+                    logger.debug("spikes of item %d stay floats: another launch reads or "
+                                 "writes them", b)
+            if not items:
+                continue
+            values = self.backend.store_spikes_as_bits(enc, items, hits, self.model.dt)
+            for b, value in values.items():
+                start = int(pops[b, 2])
+                base = base_at[start]
+                self._spike_bits[base] = (start, int(base.size), np.float32(value))
+
+    def _spikes_from_bits(self, base):
+        """The spike vector of a population whose spikes device memory holds as bits, as an
+        (n, 1) array: the value of a spike where the bit is set."""
+        start, n, value = self._spike_bits[base]
+        raw = np.ascontiguousarray(np.asarray(self.all_data[self.sidx[base]], dtype=np.float32))
+        words = raw.reshape(-1)[:2 * (-(-n // 64))]
+        bits = np.unpackbits(words.view(np.uint8), bitorder="little")[:n]
+        return (bits.astype(np.float32) * value).reshape(n, 1)
 
     def _fuse_input_sums(self, plans):
         """A launch that only adds up the decoded inputs of ensembles, right before the
@@ -982,6 +1072,9 @@ class Simulator:
                 elif base in sim._pending_filters:
                     full = sim._with_pending_filter(base, np.array(sim.all_data[sim.sidx[base]]))
                     raw = full if base is item else sim._view_of(item, full)
+                elif base in sim._spike_bits:
+                    full = sim._spikes_from_bits(base)
+                    raw = full if base is item else sim._view_of(item, full)
                 else:
                     sim._refresh_lazy(base)
                     raw = sim.all_data[sim.sidx[item]]
@@ -1020,6 +1113,12 @@ class Simulator:
                         "filtered once more or lost.  NENGO_HIP_FOLD_LEARNING=0 (or "
                         "Simulator(reference_host_state=True)) keeps the filter a launch of the "
                         "step it belongs to." % (item,))
+                if base in sim._spike_bits:
+                    raise ValueError(
+                        "%s is kept as one bit per neuron in device memory (only launches that "
+                        "visit the columns of the neurons that spiked read it).  "
+                        "NENGO_HIP_SPIKE_BITS=0 (or Simulator(reference_host_state=True)) keeps "
+                        "a float per neuron." % (item,))
                 if base in sim._updated_in_place:
                     raise ValueError(
                         "%s is updated in place by its learning rule: the change of the last "
@@ -1084,6 +1183,10 @@ class Simulator:
             start = int(self.all_data.starts[i])
             flat = np.asarray(self._host_view_copy[k], dtype=np.float32).reshape(-1)
             buf[start:start + flat.size] = flat
+        for base, (start, n, value) in self._spike_bits.items():
+            words = np.ascontiguousarray(buf[start:start + 2 * (-(-n // 64))])
+            bits = np.unpackbits(words.view(np.uint8), bitorder="little")[:n]
+            buf[start:start + n] = bits.astype(np.float32) * value
         return buf
 
     def clear_probes(self):

@@ -211,9 +211,18 @@ def _spike_reader(sim, signals):
     if dev_buf is None or hi - lo > 4 * sum(sizes):
         return lambda: np.concatenate([np.asarray(sim.signals[s]).ravel() for s in signals])
 
+    as_bits = getattr(sim, "_spike_bits", {})  # populations whose spikes the device keeps as bits
+
+    def part(span, s, a, n):
+        if s not in as_bits:
+            return span[a - lo: a - lo + n]
+        words = np.ascontiguousarray(span[a - lo: a - lo + 2 * (-(-n // 64))])
+        bits = np.unpackbits(words.view(np.uint8), bitorder="little")[:n]
+        return bits.astype(np.float32) * as_bits[s][2]
+
     def read():
         span = dev_buf.get_span(lo, hi - lo)
-        return np.concatenate([span[a - lo: a - lo + n] for a, n in zip(starts, sizes)])
+        return np.concatenate([part(span, s, a, n) for s, a, n in zip(signals, starts, sizes)])
     return read
 
 
@@ -1076,6 +1085,76 @@ def test_currents_nobody_reads_are_not_stored_and_read_back_exact(queue, monkeyp
             for Js, Jc in zip(currents(stored), currents(cpu)):
                 in_memory = np.array(stored.all_data[stored.sidx[Js]]).ravel()
                 assert np.array_equal(in_memory, np.asarray(cpu.signals[Jc]).ravel())
+
+
+@pytest.mark.gpu
+def test_spikes_only_event_launches_read_are_kept_as_bits(queue, monkeypatch):
+    """Spikes that nothing but launches visiting active columns reads are left in device
+    memory as one bit per neuron (populations whose size is no multiple of 64 included);
+    `sim.signals[S]` and `signal_buffer()` give back the oracle's floats, before the first
+    step zeros; writing them is refused; spikes that are probed stay floats; with
+    `NENGO_HIP_SPIKE_BITS=0` (and with `reference_host_state`) every spike is a float; the
+    probe data are the same bits either way."""
+    from nengo_ocl_amd import configs, ir
+    from nengo_ocl_amd.simulator import Simulator
+    from oracle.oracle_sim import OracleSimulator
+
+    def make():
+        net, probes, _ = configs.c3_large(n_ens=4, n_neurons=1000, dims=32, fan_out=2, solver="lstsq")
+        model = net.build_model(dt=0.001)
+        probe = ir.Probe(None)  # the spikes of one population, probed
+        model.probes.append(probe)
+        model.sig[probe] = {"in": model.sig[net.ensembles[1].neurons]["out"]}
+        probes["S1"] = probe
+        return model, probes, [model.sig[e.neurons]["out"] for e in net.ensembles]
+
+    (model, probes, spikes), (model_o, probes_o, spikes_o) = make(), make()
+    with Simulator(None, model=model, seed=1) as gpu, \
+            OracleSimulator(None, model=model_o, seed=1) as cpu:
+        kept = gpu._spike_bits
+        assert set(kept) == {s.base for s in spikes} - {spikes[1].base} and not cpu._spike_bits
+        assert any("spikes as bits" in p.tag for p in gpu._plans)
+        for s in spikes:  # before the first step: the initial value
+            assert not np.any(np.asarray(gpu.signals[s]))
+        for n in (1, 30, 7):
+            gpu.run_steps(n)
+            cpu.run_steps(n)
+            total = 0
+            for sg, sc in zip(spikes, spikes_o):
+                got, want = np.asarray(gpu.signals[sg]), np.asarray(cpu.signals[sc])
+                assert got.shape == want.shape and np.array_equal(got, want)
+                total += np.count_nonzero(want)
+                in_memory = np.array(gpu.all_data[gpu.sidx[sg]]).ravel()
+                if sg.base in kept:  # sixteen words of bits, the rest never written
+                    assert not np.any(in_memory[32:])
+                else:
+                    assert np.array_equal(in_memory, want.ravel())
+            assert n == 1 or total > 0
+            assert_same_signals(gpu, cpu)
+        with pytest.raises(ValueError, match="one bit per neuron"):
+            gpu.signals[spikes[0]] = np.zeros(spikes[0].shape, dtype=np.float32)
+        gpu.signals[spikes[1]] = np.asarray(gpu.signals[spikes[1]])  # floats: as ever
+        for key in probes:
+            assert np.array_equal(gpu.data[probes[key]], cpu.data[probes_o[key]]), key
+        gpu.reset()
+        cpu.reset()
+        for s in spikes:
+            assert not np.any(np.asarray(gpu.signals[s]))
+        gpu.run_steps(38)
+        cpu.run_steps(38)
+        assert_same_signals(gpu, cpu)
+        with Simulator(None, model=make()[0], seed=1, reference_host_state=True) as plain:
+            assert not plain._spike_bits
+        monkeypatch.setenv("NENGO_HIP_SPIKE_BITS", "0")
+        model_f, probes_f, spikes_f = make()
+        with Simulator(None, model=model_f, seed=1) as floats:
+            assert not floats._spike_bits
+            floats.run_steps(38)
+            for sf, sc in zip(spikes_f, spikes_o):
+                in_memory = np.array(floats.all_data[floats.sidx[sf]]).ravel()
+                assert np.array_equal(in_memory, np.asarray(cpu.signals[sc]).ravel())
+            for key in probes:
+                assert np.array_equal(floats.data[probes_f[key]], gpu.data[probes[key]]), key
 
 
 @pytest.mark.gpu
