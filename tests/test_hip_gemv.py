@@ -1036,6 +1036,60 @@ def test_products_with_spike_vectors_visit_active_columns_only(queue, activity, 
         assert np.array_equal(dev.to_host().buf.view(np.uint32), host.buf.view(np.uint32)), step
 
 
+@pytest.mark.parametrize("activity", [0.0, 0.08, 1.0])
+def test_active_columns_from_one_bit_per_column(queue, activity, monkeypatch):
+    """The same launch with X handed over as one bit per column (`x_bits` in the record: the
+    value of a set bit; 64-bit words at the start of the vector's memory): 64 x 4096,
+    32 x 2000 and 19 x 1000 (a partial last word), 100 x 4096 (two records), 16 x 10000 (three
+    runs of columns), with coefficients -- Y equals, bit for bit, the oracle's dense product
+    with the floats the bits stand for, over steps in which the bits change."""
+    from nengo_ocl_amd import hipra_gemv as g
+    from oracle import oracle as orc
+
+    rng = np.random.RandomState(29)
+    shapes = [(64, 4096), (32, 2000), (19, 1000), (100, 4096), (16, 10000)]
+    values = [1000.0, 500.0, 1000.0, 0.25, 1000.0]
+    n = len(shapes)
+    mats = [rng.normal(scale=0.01, size=s) for s in shapes]
+    xs = [np.zeros(s[1]) for s in shapes]
+    outs = [rng.normal(size=s[0]) for s in shapes]
+    R = RA(mats + xs + outs, align=True)
+    iA, iX, iY = list(range(n)), list(range(n, 2 * n)), list(range(2 * n, 3 * n))
+    A_js = [np.array([i], dtype=np.int32) for i in iA]
+    X_js = [np.array([i], dtype=np.int32) for i in iX]
+    alpha, beta = [1.0, 0.5, -2.0, 1.0, 0.75], [0.0, 1.0, 0.25, 1.0, 1.0]
+    gamma = [0.0, 0.0, 0.125, 0.0, 0.0]
+    host, dev = clone(R), to_dev(queue, R)
+    monkeypatch.setattr(g, "EVENT_MIN_SPLIT_BYTES", 0)
+    prog = g.plan_block_gemv(queue, alpha, dev, A_js, dev, X_js, beta, dev[iY], gamma=gamma,
+                             event_items=list(range(n)))
+    assert [p.name for p in prog.plans] == ["hipra_gemv.events"]
+    plan = prog.plans[0]
+    for k, b in enumerate(plan.event_record_item):
+        assert plan.event_table[k, 4] % 2 == 0  # 64-bit words
+        plan.event_table[k, 15] = int(np.array([values[b]], dtype=np.float32).view(np.int32)[0])
+    plan.dev_event_table.set(plan.event_table.astype(np.int32).ravel())
+    oprog = orc.plan_block_gemv(None, alpha, host, A_js, host, X_js, beta, host[iY], gamma=gamma)
+    for step in range(3):
+        for b, i in enumerate(iX):
+            m = R.shape0s[i]
+            active = rng.uniform(size=m) < activity
+            host[i] = np.where(active, values[b], 0.0)[:, None]
+            words = np.packbits(active, bitorder="little")
+            words = np.concatenate([words, np.zeros(-len(words) % 8, dtype=np.uint8)])
+            # the memory behind the words is never read: anything may be there
+            image = rng.normal(size=m).astype(np.float32)
+            image[:len(words) // 4] = words.view(np.float32)
+            dev[i] = image
+        plan()
+        for p in oprog.plans:
+            p()
+        got, want = dev.to_host(), host
+        for i in iY:
+            assert np.array_equal(np.asarray(got[i]).view(np.uint32),
+                                  np.asarray(want[i]).view(np.uint32)), (step, i)
+
+
 def test_gemv_lif_forms_its_input_sums(queue):
     """Sums of vectors -> encoders -> LIF in one launch: inputs that are sums of one to
     eleven vectors times scalars (64, 40 and 8 elements), an ensemble whose input is a
