@@ -681,3 +681,77 @@ def test_reset_restarts_the_random_streams_of_host_processes():
         ub = np.array(sim.data[up])
     assert ua.shape == (10, 2) and np.any(ua != 0) and len(np.unique(ua)) == 20
     assert np.array_equal(ua, ub)
+
+
+def test_which_spikes_are_kept_as_bits():
+    """`Simulator._store_spikes_as_bits` on stand-in plans: a population's spikes become bits
+    when one large-item neuron launch writes them (tasks at multiples of 32 rows, one
+    amplitude, one decay factor) and only whole-vector records of active-column launches
+    read them; a probe or any other reader, a record over a part of the vector, a carried
+    sequence that reads them, a host-visible copy, an initial value, an odd start or a
+    per-neuron amplitude keep the floats.  The tables are updated accordingly: flag bit 11 in
+    the population row, the value of a spike in word 15 of the reading records."""
+    from types import SimpleNamespace as NS
+    from nengo_ocl_amd import hipra_gemv as g
+    from nengo_ocl_amd.simulator import Simulator
+
+    class Table:
+        def __init__(self):
+            self.value = None
+
+        def set(self, array):
+            self.value = np.array(array)
+
+    class Base:
+        def __init__(self, name, size):
+            self.name, self.size = name, size
+
+    n_pops, n = 8, 200
+    bases = [Base("s%d" % p, n) for p in range(n_pops)]
+    starts = [1000 * p + (1 if p == 6 else 0) for p in range(n_pops)]  # population 6: odd start
+    extra = Base("other", 10)
+    amp_bits = int(np.array([2.0], dtype=np.float32).view(np.int32)[0])
+    pops = np.zeros((n_pops, 8), dtype=np.int32)
+    tasks = []
+    for p in range(n_pops):
+        pops[p] = (0, 0, starts[p], 1, 1, 1, amp_bits, 0x300 | (4 if p == 7 else 0))  # 7: amplitudes
+        tasks += [(p, 0, 128, 0), (p, 128, n - 128, 0)]
+    enc = NS(name="hipra_gemv.tile_lif", tag="enc", dev_pops=Table(), host_pops=pops,
+             host_tasks=np.array(tasks, dtype=np.int32), reads_mem=set(), writes_mem=set(bases),
+             bw_per_call=10 ** 6)
+    records = np.zeros((n_pops + 1, 16), dtype=np.int32)
+    for p in range(n_pops):
+        records[p, 3], records[p, 4] = n, starts[p]
+    records[n_pops, 3], records[n_pops, 4] = 100, starts[1] + 100  # a record over half of s1
+    events = NS(name="hipra_gemv.events_filter", tag="ev", dev_event_table=Table(),
+                event_table=records, reads_mem=set(bases), writes_mem={extra},
+                carried=NS(reads_mem={bases[2]}))  # a carried gather reads s2
+    probe = NS(name="hip_probes", reads_mem={bases[3]}, writes_mem=set())  # s3 is probed
+    initial = np.zeros(10000, dtype=np.float32)
+    initial[starts[4] + 5] = 1.0  # s4 starts with a spike
+    sim = NS(reference_host_state=False, model=NS(dt=0.001), _initial_buf=initial,
+             backend=NS(spikes_as_bits=True, store_spikes_as_bits=g.store_spikes_as_bits),
+             all_bases=bases + [extra], sidx={b: i for i, b in enumerate(bases + [extra])},
+             all_data=NS(starts=starts + [9000]), _host_view_index={bases[5]: 0})  # s5: host copy
+    Simulator._store_spikes_as_bits(sim, [enc, events, probe])
+    assert set(sim._spike_bits) == {bases[0]}
+    start, size, value = sim._spike_bits[bases[0]]
+    assert (start, size) == (0, n) and value == np.float32(2.0) * np.float32(1000.0)
+    assert [int(f) & g.LIF_POP_BITS for f in pops[:, 7]] == [g.LIF_POP_BITS] + [0] * 7
+    assert np.array_equal(enc.dev_pops.value.reshape(pops.shape), pops)
+    value_bits = int(np.array([2000.0], dtype=np.float32).view(np.int32)[0])
+    assert records[:, 15].tolist() == [value_bits] + [0] * n_pops
+    assert np.array_equal(events.dev_event_table.value.reshape(records.shape), records)
+    assert "spikes as bits" in enc.tag and enc.bw_per_call == 10 ** 6 - (4 * n - n // 8)
+
+    # tasks that start between multiples of 32 rows, and the switches
+    pops[:, 7] &= ~g.LIF_POP_BITS
+    records[:, 15] = 0
+    enc.host_tasks = np.array([(0, 0, 100, 0), (0, 100, 100, 0)], dtype=np.int32)
+    Simulator._store_spikes_as_bits(sim, [enc, events, probe])
+    assert not sim._spike_bits and not records[:, 15].any()
+    enc.host_tasks = np.array(tasks, dtype=np.int32)
+    for off in (dict(reference_host_state=True), dict(backend=NS(spikes_as_bits=False))):
+        quiet = NS(**{**vars(sim), **off})
+        Simulator._store_spikes_as_bits(quiet, [enc, events, probe])
+        assert quiet._spike_bits == {} and not records[:, 15].any()
