@@ -710,7 +710,7 @@ class Simulator:
                 mine = tasks[tasks[:, 0] == b]
                 n = int(mine[:, 2].sum())
                 base = base_at.get(start)
-                checks = (base is not None and int(base.size) == n, (start, n) in records,
+                checks = (base is not None and int(base.size) == n >= 64, (start, n) in records,
                           not np.any(mine[:, 1] % 32),
                           not np.any(self._initial_buf[start:start + n]),
                           base not in self._host_view_index, base not in enc.reads_mem)
