@@ -693,7 +693,11 @@ class Simulator:
         if not encs or not events:
             return
         ra = self.all_data
-        base_at = {int(ra.starts[self.sidx[b]]): b for b in self.all_bases}
+        base_at = {}  # start in the buffer -> the (largest) base signal that starts there
+        for b in self.all_bases:
+            start = int(ra.starts[self.sidx[b]])
+            if start not in base_at or int(b.size) > int(base_at[start].size):
+                base_at[start] = b
         records = defaultdict(list)  # (x_start, columns) -> [(plan, record)]
         for q in events:
             for k, row in enumerate(q.event_table):
@@ -705,7 +709,9 @@ class Simulator:
                 if b >= len(pops):
                     continue
                 flags, start = int(pops[b, 7]), int(pops[b, 2])
-                if (flags & 0x304) != 0x300 or start % 2:  # a population, one decay, one amplitude
+                # (bits of a population row: 4 = an amplitude per neuron, 0x100 = there is a
+                # population, 0x200 = one decay factor, which selects the code that can do this)
+                if (flags & 0x304) != 0x300 or start % 2:
                     continue
                 mine = tasks[tasks[:, 0] == b]
                 n = int(mine[:, 2].sum())
